@@ -1,0 +1,228 @@
+/*
+ * infr_hip.h — C ABI of the MI355X (gfx950) backend for infr's quantized-matmul path.
+ *
+ * The entry points are what an `infr-hip` crate would bind to implement infr-core's `Backend`
+ * trait (crates/infr-core/src/backend.rs:486-662) for the two ops on this path, `Op::Linear`
+ * (crates/infr-core/src/graph.rs:177-191) and `Op::MoeFfn` (graph.rs:911-1011). Plain pointers,
+ * sizes and opaque handles only; every call returns a status code and never throws or aborts
+ * across the boundary. One HIP stream per backend; calls on one backend must be externally
+ * serialised (the reference runner calls `execute` from one thread at a time,
+ * crates/infr-cpu/src/pool.rs:216-240).
+ *
+ * There is no CPU fallback: every compute entry point fails with INFR_HIP_ERR_BACKEND when no
+ * gfx950 device is usable.
+ */
+#ifndef INFR_HIP_H
+#define INFR_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Mirrors infr_core::error::Error (crates/infr-core/src/error.rs:5-25); 0 = Ok. */
+typedef enum {
+    INFR_HIP_OK = 0,
+    INFR_HIP_ERR_BACKEND = 1,     /* Error::Backend: device/runtime failure */
+    INFR_HIP_ERR_LOADER = 2,      /* Error::Loader */
+    INFR_HIP_ERR_MODEL = 3,       /* Error::Model */
+    INFR_HIP_ERR_UNSUPPORTED = 4, /* Error::Unsupported: dtype/shape this backend does not take */
+    INFR_HIP_ERR_ABORTED = 5,     /* Error::Aborted: shutdown latch was set */
+    INFR_HIP_ERR_IO = 6,          /* Error::Io */
+    INFR_HIP_ERR_OTHER = 7,       /* Error::Other */
+    INFR_HIP_ERR_INVALID = 8      /* programmer error the reference would panic on (unbound
+                                     buffer, size mismatch, misaligned w_off): reported, no abort */
+} infr_hip_status;
+
+/* Weight/activation element types, numbered as GGML type ids
+ * (crates/infr-gguf/src/lib.rs:330-354; crates/infr-core/src/tensor.rs:7-57). */
+typedef enum {
+    INFR_DTYPE_F32 = 0,
+    INFR_DTYPE_Q8_0 = 8,  /* 32 elems / 34 B:  [f16 d][i8 qs[32]]            decode_spec.rs:319-320 */
+    INFR_DTYPE_Q4_K = 12, /* 256 / 144 B: [f16 d][f16 dmin][u8 sc[12]][u8 qs[128]]        :326-327 */
+    INFR_DTYPE_Q6_K = 14, /* 256 / 210 B: [u8 ql[128]][u8 qh[64]][i8 sc[16]][f16 d]       :330-331 */
+    INFR_DTYPE_Q2_0 = 42  /* 64 / 18 B:   [f16 d][u8 qs[16]] ternary-style 2-bit codes    :357-358 */
+} infr_dtype;
+
+/* infr_core::backend::BufferUsage (crates/infr-core/src/backend.rs:358-380). Advisory: every
+ * class is device-local HBM here; upload/download stage through the copy engine. */
+typedef enum {
+    INFR_USAGE_WEIGHTS = 0,
+    INFR_USAGE_ACTIVATIONS = 1,
+    INFR_USAGE_KV_CACHE = 2,
+    INFR_USAGE_STAGING = 3,
+    INFR_USAGE_READBACK = 4,
+    INFR_USAGE_HOST_WEIGHTS = 5
+} infr_buffer_usage;
+
+typedef struct infr_hip infr_hip_t;               /* a Backend instance            */
+typedef struct infr_hip_buffer infr_hip_buffer_t; /* a Buffer (backend.rs:387-416) */
+typedef struct infr_hip_plan infr_hip_plan_t;     /* a Plan   (backend.rs:418-446) */
+
+/* Subset of infr_core::backend::Capabilities (backend.rs:43-213) this backend reports. */
+typedef struct {
+    int i8;                   /* int8 storage */
+    int i8_dot;               /* packed 4x int8 dot (v_dot4) */
+    int coopmat_i8_m, coopmat_i8_n, coopmat_i8_k; /* int8 MFMA tile */
+    int decode_replay;        /* execute() replays a recorded launch sequence */
+    int combined_gu, embed_gather, gpu_sample, argmax_rows, gated_rmsnorm; /* all 0: plain ops */
+    int graph_input_inplace;
+    int unified_memory;
+    uint64_t device_memory_bytes;
+    int compute_units;
+    char device_name[64];
+} infr_hip_caps_t;
+
+/* ---- lifetime (Backend construction; crates/infr-cpu/src/lib.rs:655-701 for the CPU peer) ---- */
+int infr_hip_create(int device, infr_hip_t **out);
+void infr_hip_destroy(infr_hip_t *be);
+/* Backend::name (backend.rs:487) */
+const char *infr_hip_name(const infr_hip_t *be);
+/* Backend::capabilities (backend.rs:488) */
+int infr_hip_capabilities(const infr_hip_t *be, infr_hip_caps_t *out);
+/* Message of the last failing call on this backend (Error's payload string). With be == NULL,
+ * the message of the last failing infr_hip_create on this thread. */
+const char *infr_hip_last_error(const infr_hip_t *be);
+
+/* ---- memory ---- */
+/* Backend::alloc (backend.rs:491-496): zero-initialised, calloc semantics. */
+int infr_hip_alloc(infr_hip_t *be, size_t bytes, int usage, infr_hip_buffer_t **out);
+/* Backend::alloc_uninit (backend.rs:497-503). */
+int infr_hip_alloc_uninit(infr_hip_t *be, size_t bytes, int usage, infr_hip_buffer_t **out);
+/* Adopt device memory owned by the caller (e.g. a framework tensor) as a Buffer; never freed by
+ * the backend. No reference counterpart: the reference's buffers are always backend-allocated. */
+int infr_hip_wrap(infr_hip_t *be, void *device_ptr, size_t bytes, infr_hip_buffer_t **out);
+/* Drop of Box<dyn Buffer>: the caller owns buffers and frees them. */
+void infr_hip_free(infr_hip_t *be, infr_hip_buffer_t *buf);
+/* Buffer::len_bytes / Buffer::device_addr (backend.rs:388-415). */
+size_t infr_hip_buffer_len(const infr_hip_buffer_t *buf);
+uint64_t infr_hip_buffer_device_addr(const infr_hip_buffer_t *buf);
+/* Backend::upload / download (backend.rs:504-510). `n` must not exceed the buffer. download
+ * observes every previously issued execute/linear on this backend. */
+int infr_hip_upload(infr_hip_t *be, infr_hip_buffer_t *dst, const void *src, size_t n);
+int infr_hip_download(infr_hip_t *be, const infr_hip_buffer_t *src, void *dst, size_t n);
+/* Same with a byte offset into the buffer (the reference slices host-side before uploading). */
+int infr_hip_upload_at(infr_hip_t *be, infr_hip_buffer_t *dst, size_t dst_off, const void *src, size_t n);
+int infr_hip_download_at(infr_hip_t *be, const infr_hip_buffer_t *src, size_t src_off, void *dst, size_t n);
+/* Backend::copy_buffer (backend.rs:547-558): oversize copies return an error, not a fault
+ * (check_copy_bytes, backend.rs:23-30). */
+int infr_hip_copy_buffer(infr_hip_t *be, const infr_hip_buffer_t *src, infr_hip_buffer_t *dst, size_t bytes);
+/* Backend::sync (backend.rs:606). */
+int infr_hip_sync(infr_hip_t *be);
+
+/* ---- the hot path, op by op ---- */
+
+/* Op::Linear (graph.rs:177-191; CPU arm crates/infr-cpu/src/lib.rs:985-1492):
+ *   dst[m, out_f] = x[m, in_f] . W^T, W row-major [rows, in_f] in raw GGUF blocks of `dtype`.
+ *   w        whole bound weight buffer; w_numel its declared element count (rows*in_f);
+ *   w_off    element offset of the first row (multiple of in_f) inside a concatenated weight;
+ *   x        f32 [m, in_f]; dst f32 [m, out_f], row-major.
+ * Activations are quantized on the device exactly as infr-cpu does (per-256 int8 + f32 scale for
+ * Q4_K/Q6_K/Q8_0, crates/infr-cpu/src/quant.rs:27-58; per-32 for Q2_0, quant.rs:97-117), the
+ * integer dot is exact, and the f32 epilogue follows the CPU kernels' expression per block.
+ * in_f must be a multiple of 256 (Q2_0: 64): a shorter tail is rejected, never truncated. */
+int infr_hip_linear(infr_hip_t *be, int dtype, const infr_hip_buffer_t *w, size_t w_numel,
+                    size_t w_off, const infr_hip_buffer_t *x, infr_hip_buffer_t *dst, size_t m,
+                    size_t in_f, size_t out_f);
+
+/* quantize_q8 (crates/infr-cpu/src/quant.rs:27-58) for m rows of k floats (k % 256 == 0):
+ *   qs i8 [m,k]; d f32 [m,k/256]; bsums i32 [m,k/32]; bsums16 i32 [m,k/16] (may be NULL).
+ * Exposes the integer stage so callers can check it bit-for-bit. */
+int infr_hip_quantize_q8(infr_hip_t *be, const infr_hip_buffer_t *x, size_t m, size_t k,
+                         infr_hip_buffer_t *qs, infr_hip_buffer_t *d, infr_hip_buffer_t *bsums,
+                         infr_hip_buffer_t *bsums16);
+/* quantize_q8_32 (quant.rs:97-117), k % 32 == 0: qs i8 [m,k]; d f32 [m,k/32]; bsum i32 [m,k/32]. */
+int infr_hip_quantize_q8_32(infr_hip_t *be, const infr_hip_buffer_t *x, size_t m, size_t k,
+                            infr_hip_buffer_t *qs, infr_hip_buffer_t *d, infr_hip_buffer_t *bsum);
+
+/* Per-block integer stages of Op::Linear for every (row r, output o), i32 [m][out_f][blocks]:
+ *   Q4_K: a = sd, b = sm per 256-block (crates/infr-cpu/src/kernels.rs:162-181);
+ *   Q6_K: a = isum per 256-block (kernels.rs:519-522);
+ *   Q8_0: a = iprod per 32-block (kernels.rs:1182); Q2_0: a = iprod per 32 sub-block (:5657-5662).
+ * b may be NULL unless dtype is Q4_K. Uses the same device code as infr_hip_linear. */
+int infr_hip_linear_int_stages(infr_hip_t *be, int dtype, const infr_hip_buffer_t *w,
+                               size_t w_numel, size_t w_off, const infr_hip_buffer_t *x, size_t m,
+                               size_t in_f, size_t out_f, infr_hip_buffer_t *a,
+                               infr_hip_buffer_t *b);
+
+/* Op::MoeFfn as qwen3moe emits it (graph.rs:911-1011; crates/infr-llama/src/seam/runner.rs:3971-3997):
+ * softmax gating, renormalised top-n_used weights x scale, split gate/up banks, SiLU, weights on
+ * the expert output. Expert e of a bank is its e-th equal byte slice. */
+typedef struct {
+    uint32_t ne, n_expert, n_used, n_ff_exp, rows;
+    float scale;
+    int router_dtype; /* INFR_DTYPE_F32 */
+    int gate_dtype, up_dtype, down_dtype;
+} infr_hip_moe_params_t;
+
+/* CPU arm: crates/infr-cpu/src/lib.rs:2264-2984, crates/infr-cpu/src/moe.rs. As there, rows == 1
+ * multiplies decoded f32 weights with the unquantized activation; rows >= 2 takes the int8 path.
+ * Only the selected experts' blocks are read. sel_idx (i32) / sel_w (f32), [rows, n_used], are
+ * optional outputs of the routing in descending-probability order. */
+int infr_hip_moe_ffn(infr_hip_t *be, const infr_hip_moe_params_t *p, const infr_hip_buffer_t *x,
+                     const infr_hip_buffer_t *router_x, const infr_hip_buffer_t *router,
+                     const infr_hip_buffer_t *gate_exps, const infr_hip_buffer_t *up_exps,
+                     const infr_hip_buffer_t *down_exps, infr_hip_buffer_t *dst,
+                     infr_hip_buffer_t *sel_idx, infr_hip_buffer_t *sel_w);
+
+/* ---- graph level: Backend::compile / execute (backend.rs:560-577) over a flat C mirror of
+ * infr_core::graph::Graph restricted to the ops of this path ---- */
+typedef enum { INFR_OP_LINEAR = 1, INFR_OP_MOE_FFN = 2 } infr_hip_op_kind;
+
+typedef struct {
+    int kind;      /* infr_hip_op_kind */
+    /* Op::Linear: tensor ids (indices into the bindings array) and shape */
+    uint32_t x, weight, dst;
+    uint32_t m, in_f, out_f;
+    uint64_t w_off;
+    uint64_t w_numel;
+    int w_dtype;
+    /* Op::MoeFfn */
+    uint32_t router_x, router, gate_exps, up_exps, down_exps;
+    infr_hip_moe_params_t moe;
+} infr_hip_op_t;
+
+/* Backend::compile: validates and stores the op list (the reference's GraphPlan clones the
+ * graph, backend.rs:424-446). */
+int infr_hip_compile(infr_hip_t *be, const infr_hip_op_t *ops, size_t n_ops, infr_hip_plan_t **out);
+void infr_hip_plan_free(infr_hip_t *be, infr_hip_plan_t *plan);
+/* Backend::execute: bindings[i] is the buffer bound to tensor id i (NULL = unbound;
+ * Bindings, backend.rs:448-483). With the same bindings as the previous call on this plan the
+ * recorded launch sequence is replayed (Capabilities::decode_replay, backend.rs:155-159).
+ * Asynchronous: results are visible after infr_hip_sync or a download. */
+int infr_hip_execute(infr_hip_t *be, infr_hip_plan_t *plan, infr_hip_buffer_t *const *bindings,
+                     size_t n_bindings);
+
+/* ---- shutdown latch (crates/infr-core/src/shutdown.rs:30-60): once requested, compute entry
+ * points enqueue nothing further and return INFR_HIP_ERR_ABORTED; work already enqueued drains.
+ * request_shutdown returns 1 if this call latched it, 0 if it was already set (signo != 0);
+ * shutdown_signal returns the latched signal or 0. */
+int infr_hip_request_shutdown(int signo);
+int infr_hip_shutdown_requested(void);
+int infr_hip_shutdown_signal(void);
+void infr_hip_reset_shutdown(void); /* tests only: the reference's latch is monotonic */
+
+/* ---- measurement: device-time of the work enqueued between begin and end on the backend's
+ * stream (the reference's per-op timing seam, crates/infr-core/src/prof.rs:1-80) ---- */
+int infr_hip_timer_begin(infr_hip_t *be);
+int infr_hip_timer_end(infr_hip_t *be, float *elapsed_ms); /* synchronises */
+
+/* ---- deterministic synthetic inputs (host side, no device work). The reference has no weight
+ * quantizer (it only reads GGUF) and its tests synthesize valid blocks
+ * (crates/infr-testkit/src/lib.rs:106-123); these encoders produce valid blocks from
+ * N(0, sigma^2) draws of a SplitMix64 + Box-Muller stream so every run sees identical bytes. ---- */
+/* f32 N(mean, sigma^2), n values from `seed`. */
+void infr_synth_normal_f32(uint64_t seed, float mean, float sigma, size_t n, float *out);
+/* Draw rows*in_f weights N(0, sigma^2) from `seed` and encode them in `dtype`
+ * (Q4_K/Q6_K/Q8_0: nearest-code encoders; Q2_0: codes uniform over {0,1,2} = {-1,0,+1} with
+ * per-64 scale |N(0, sigma^2)|). Returns bytes written (0 on bad arguments). */
+size_t infr_synth_weight(int dtype, uint64_t seed, float sigma, size_t rows, size_t in_f, uint8_t *out);
+/* Block geometry: elements and bytes per block; returns 0 on unknown dtype. */
+int infr_block_layout(int dtype, int *elems, int *bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* INFR_HIP_H */

@@ -1,0 +1,561 @@
+// C-ABI layer (include/infr_hip.h): buffers, stream, argument checking, op dispatch and the
+// plan/execute replay. Mirrors infr-core's Backend trait (crates/infr-core/src/backend.rs:486-662)
+// for Op::Linear and Op::MoeFfn. Nothing here computes on the host: with no usable gfx950 device
+// infr_hip_create fails and no other entry point can be reached.
+#include "../../include/infr_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "kernels.hpp"
+
+struct infr_hip_buffer {
+    void* ptr = nullptr;
+    size_t len = 0;
+    bool owned = false;
+};
+
+struct infr_hip_plan {
+    std::vector<infr_hip_op_t> ops;
+    uint32_t max_tensor = 0;
+    // decode replay: launch sequence recorded for one set of bound device addresses
+    hipGraphExec_t exec = nullptr;
+    std::vector<void*> bound;
+};
+
+struct infr_hip {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    hipDeviceProp_t props;
+    std::string err;
+    std::string name;
+    // Transient scratch for the quantized activation (TensorKind::Internal in the reference's
+    // terms: backend-allocated, graph.rs:109-122). Grow-only.
+    infr::ActQ8 act;
+    size_t act_cap_elems = 0;
+    // MoE scratch
+    void* moe_ws = nullptr;
+    size_t moe_ws_bytes = 0;
+};
+
+namespace {
+
+thread_local std::string g_create_err;
+std::atomic<int> g_shutdown_signo{0};
+
+int fail(infr_hip_t* be, int code, const std::string& msg) {
+    if (be) be->err = msg;
+    else g_create_err = msg;
+    return code;
+}
+
+#define HIP_TRY(be, expr)                                                                     \
+    do {                                                                                      \
+        hipError_t e__ = (expr);                                                              \
+        if (e__ != hipSuccess)                                                                \
+            return fail((be), INFR_HIP_ERR_BACKEND,                                           \
+                        std::string(#expr) + ": " + hipGetErrorString(e__));                 \
+    } while (0)
+
+bool is_quant(int dt) {
+    return dt == INFR_DTYPE_Q4_K || dt == INFR_DTYPE_Q6_K || dt == INFR_DTYPE_Q8_0 ||
+           dt == INFR_DTYPE_Q2_0;
+}
+// Which activation quantizer infr-cpu's dispatch pairs with the weight dtype
+// (crates/infr-cpu/src/lib.rs:1043-1076): per-32 only for Q2_0 among the formats carried here.
+bool act_per32(int dt) { return dt == INFR_DTYPE_Q2_0; }
+
+int ensure_act(infr_hip_t* be, size_t elems) {
+    if (elems <= be->act_cap_elems) return INFR_HIP_OK;
+    HIP_TRY(be, hipStreamSynchronize(be->stream));
+    if (be->act.qs) {
+        (void)hipFree(be->act.qs);
+        (void)hipFree(be->act.d);
+        (void)hipFree(be->act.bsums);
+        (void)hipFree(be->act.bsums16);
+        be->act = infr::ActQ8{};
+        be->act_cap_elems = 0;
+    }
+    const size_t cap = (elems + 4095) / 4096 * 4096;
+    HIP_TRY(be, hipMalloc((void**)&be->act.qs, cap));
+    HIP_TRY(be, hipMalloc((void**)&be->act.d, cap / 32 * sizeof(float)));
+    HIP_TRY(be, hipMalloc((void**)&be->act.bsums, cap / 32 * sizeof(int32_t)));
+    HIP_TRY(be, hipMalloc((void**)&be->act.bsums16, cap / 16 * sizeof(int32_t)));
+    be->act_cap_elems = cap;
+    return INFR_HIP_OK;
+}
+
+struct LinearArgs {
+    const uint8_t* wrows;  // first selected row
+    size_t bpr;
+};
+
+// Shape/size validation shared by linear and linear_int_stages
+// (crates/infr-cpu/src/lib.rs:1003-1008 for the row slicing).
+int check_linear(infr_hip_t* be, int dtype, const infr_hip_buffer_t* w, size_t w_numel,
+                 size_t w_off, const infr_hip_buffer_t* x, size_t m, size_t in_f, size_t out_f,
+                 LinearArgs* out) {
+    if (!w || !x) return fail(be, INFR_HIP_ERR_INVALID, "linear: unbound buffer");
+    if (!is_quant(dtype))
+        return fail(be, INFR_HIP_ERR_UNSUPPORTED,
+                    "linear: weight dtype " + std::to_string(dtype) + " has no kernel");
+    if (m == 0 || in_f == 0 || out_f == 0) return fail(be, INFR_HIP_ERR_INVALID, "linear: empty shape");
+    int qpb = 0, bpb = 0;
+    infr_block_layout(dtype, &qpb, &bpb);
+    // The per-256 activation quantizer drops a sub-256 tail (quant.rs:28); reject, never truncate.
+    const size_t need = act_per32(dtype) ? 64 : 256;
+    if (in_f % need != 0)
+        return fail(be, INFR_HIP_ERR_UNSUPPORTED,
+                    "linear: in_f " + std::to_string(in_f) + " is not a multiple of " +
+                        std::to_string(need) + " for dtype " + std::to_string(dtype));
+    if (w_numel == 0 || w_numel % in_f != 0 || w_off % in_f != 0)
+        return fail(be, INFR_HIP_ERR_INVALID, "linear: w_numel / w_off not row-aligned");
+    const size_t total_rows = w_numel / in_f;
+    const size_t bpr = in_f / (size_t)qpb * (size_t)bpb;
+    if (w->len < total_rows * bpr)
+        return fail(be, INFR_HIP_ERR_INVALID, "linear: weight buffer smaller than its declared shape");
+    const size_t row0 = w_off / in_f;
+    if (row0 + out_f > total_rows)
+        return fail(be, INFR_HIP_ERR_INVALID, "linear: w_off + out_f exceeds the weight's rows");
+    if (x->len < m * in_f * sizeof(float))
+        return fail(be, INFR_HIP_ERR_INVALID, "linear: x buffer too small");
+    if (in_f > 0x7FFFFFFFull || out_f > 0x7FFFFFFFull || m > 0x7FFFFFFFull)
+        return fail(be, INFR_HIP_ERR_UNSUPPORTED, "linear: dimension exceeds 2^31");
+    out->wrows = static_cast<const uint8_t*>(w->ptr) + row0 * bpr;
+    out->bpr = bpr;
+    return INFR_HIP_OK;
+}
+
+int enqueue_linear(infr_hip_t* be, int dtype, const LinearArgs& la, const float* x, float* y,
+                   size_t m, size_t in_f, size_t out_f, const infr::IntStages& st) {
+    infr::launch_quantize_q8(x, m, in_f, act_per32(dtype), be->act, be->stream);
+    bool ok;
+    if (m == 1)
+        ok = infr::launch_gemv(dtype, la.wrows, la.bpr, be->act, y, in_f, out_f, st, be->stream);
+    else
+        ok = infr::launch_mmq(dtype, la.wrows, la.bpr, be->act, y, m, in_f, out_f, st, be->stream);
+    if (!ok)
+        return fail(be, INFR_HIP_ERR_UNSUPPORTED,
+                    "linear: no kernel for dtype " + std::to_string(dtype) + " at in_f " +
+                        std::to_string(in_f) + ", m " + std::to_string(m));
+    HIP_TRY(be, hipGetLastError());
+    return INFR_HIP_OK;
+}
+
+int check_latch(infr_hip_t* be) {
+    if (g_shutdown_signo.load(std::memory_order_relaxed) != 0)
+        return fail(be, INFR_HIP_ERR_ABORTED, "shutdown requested");
+    return INFR_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int infr_hip_create(int device, infr_hip_t** out) {
+    if (!out) return fail(nullptr, INFR_HIP_ERR_INVALID, "create: out is null");
+    *out = nullptr;
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0)
+        return fail(nullptr, INFR_HIP_ERR_BACKEND,
+                    std::string("no HIP device: ") + (e != hipSuccess ? hipGetErrorString(e) : "count is 0"));
+    if (device < 0 || device >= n)
+        return fail(nullptr, INFR_HIP_ERR_INVALID, "create: device index out of range");
+    infr_hip_t* be = new (std::nothrow) infr_hip();
+    if (!be) return fail(nullptr, INFR_HIP_ERR_OTHER, "create: out of host memory");
+    be->device = device;
+    auto bail = [&](const char* what, hipError_t err) {
+        std::string msg = std::string(what) + ": " + hipGetErrorString(err);
+        infr_hip_destroy(be);
+        return fail(nullptr, INFR_HIP_ERR_BACKEND, msg);
+    };
+    if ((e = hipSetDevice(device)) != hipSuccess) return bail("hipSetDevice", e);
+    if ((e = hipGetDeviceProperties(&be->props, device)) != hipSuccess)
+        return bail("hipGetDeviceProperties", e);
+    if (std::strncmp(be->props.gcnArchName, "gfx950", 6) != 0) {
+        std::string msg = std::string("device is ") + be->props.gcnArchName +
+                          ", this library carries gfx950 code only";
+        infr_hip_destroy(be);
+        return fail(nullptr, INFR_HIP_ERR_UNSUPPORTED, msg);
+    }
+    if ((e = hipStreamCreateWithFlags(&be->stream, hipStreamNonBlocking)) != hipSuccess)
+        return bail("hipStreamCreate", e);
+    if ((e = hipEventCreate(&be->ev0)) != hipSuccess) return bail("hipEventCreate", e);
+    if ((e = hipEventCreate(&be->ev1)) != hipSuccess) return bail("hipEventCreate", e);
+    be->name = std::string("hip:") + be->props.gcnArchName;
+    *out = be;
+    return INFR_HIP_OK;
+}
+
+void infr_hip_destroy(infr_hip_t* be) {
+    if (!be) return;
+    (void)hipSetDevice(be->device);
+    if (be->stream) (void)hipStreamSynchronize(be->stream);
+    if (be->act.qs) {
+        (void)hipFree(be->act.qs);
+        (void)hipFree(be->act.d);
+        (void)hipFree(be->act.bsums);
+        (void)hipFree(be->act.bsums16);
+    }
+    if (be->moe_ws) (void)hipFree(be->moe_ws);
+    if (be->ev0) (void)hipEventDestroy(be->ev0);
+    if (be->ev1) (void)hipEventDestroy(be->ev1);
+    if (be->stream) (void)hipStreamDestroy(be->stream);
+    delete be;
+}
+
+const char* infr_hip_name(const infr_hip_t* be) { return be ? be->name.c_str() : "hip"; }
+
+int infr_hip_capabilities(const infr_hip_t* be, infr_hip_caps_t* out) {
+    if (!be || !out) return INFR_HIP_ERR_INVALID;
+    std::memset(out, 0, sizeof *out);
+    out->i8 = 1;
+    out->i8_dot = 1;
+    out->coopmat_i8_m = 32;
+    out->coopmat_i8_n = 32;
+    out->coopmat_i8_k = 32;
+    out->decode_replay = 1;
+    out->graph_input_inplace = 1;
+    out->unified_memory = 0;
+    out->device_memory_bytes = be->props.totalGlobalMem;
+    out->compute_units = be->props.multiProcessorCount;
+    std::snprintf(out->device_name, sizeof out->device_name, "%s", be->props.name);
+    return INFR_HIP_OK;
+}
+
+const char* infr_hip_last_error(const infr_hip_t* be) {
+    return be ? be->err.c_str() : g_create_err.c_str();
+}
+
+static int alloc_impl(infr_hip_t* be, size_t bytes, bool zero, infr_hip_buffer_t** out) {
+    if (!be || !out) return fail(be, INFR_HIP_ERR_INVALID, "alloc: null argument");
+    *out = nullptr;
+    infr_hip_buffer_t* b = new (std::nothrow) infr_hip_buffer();
+    if (!b) return fail(be, INFR_HIP_ERR_OTHER, "alloc: out of host memory");
+    const size_t n = bytes ? bytes : 4;  // the reference's harness allocs max(len, 4)
+    hipError_t e = hipMalloc(&b->ptr, n);
+    if (e != hipSuccess) {
+        delete b;
+        return fail(be, INFR_HIP_ERR_BACKEND,
+                    "hipMalloc(" + std::to_string(n) + "): " + hipGetErrorString(e));
+    }
+    if (zero) {
+        e = hipMemsetAsync(b->ptr, 0, n, be->stream);
+        if (e != hipSuccess) {
+            (void)hipFree(b->ptr);
+            delete b;
+            return fail(be, INFR_HIP_ERR_BACKEND, std::string("hipMemsetAsync: ") + hipGetErrorString(e));
+        }
+    }
+    b->len = bytes;
+    b->owned = true;
+    *out = b;
+    return INFR_HIP_OK;
+}
+
+int infr_hip_alloc(infr_hip_t* be, size_t bytes, int /*usage*/, infr_hip_buffer_t** out) {
+    return alloc_impl(be, bytes, true, out);
+}
+int infr_hip_alloc_uninit(infr_hip_t* be, size_t bytes, int /*usage*/, infr_hip_buffer_t** out) {
+    return alloc_impl(be, bytes, false, out);
+}
+
+int infr_hip_wrap(infr_hip_t* be, void* device_ptr, size_t bytes, infr_hip_buffer_t** out) {
+    if (!be || !out || !device_ptr) return fail(be, INFR_HIP_ERR_INVALID, "wrap: null argument");
+    infr_hip_buffer_t* b = new (std::nothrow) infr_hip_buffer();
+    if (!b) return fail(be, INFR_HIP_ERR_OTHER, "wrap: out of host memory");
+    b->ptr = device_ptr;
+    b->len = bytes;
+    b->owned = false;
+    *out = b;
+    return INFR_HIP_OK;
+}
+
+void infr_hip_free(infr_hip_t* be, infr_hip_buffer_t* buf) {
+    if (!buf) return;
+    if (buf->owned && buf->ptr) {
+        if (be && be->stream) (void)hipStreamSynchronize(be->stream);
+        (void)hipFree(buf->ptr);
+    }
+    delete buf;
+}
+
+size_t infr_hip_buffer_len(const infr_hip_buffer_t* buf) { return buf ? buf->len : 0; }
+uint64_t infr_hip_buffer_device_addr(const infr_hip_buffer_t* buf) {
+    return buf ? (uint64_t)(uintptr_t)buf->ptr : 0;
+}
+
+int infr_hip_upload_at(infr_hip_t* be, infr_hip_buffer_t* dst, size_t dst_off, const void* src,
+                       size_t n) {
+    if (!be || !dst || (!src && n)) return fail(be, INFR_HIP_ERR_INVALID, "upload: null argument");
+    if (dst_off > dst->len || n > dst->len - dst_off)
+        return fail(be, INFR_HIP_ERR_BACKEND,
+                    "upload of " + std::to_string(n) + " bytes at " + std::to_string(dst_off) +
+                        " exceeds the " + std::to_string(dst->len) + "-byte buffer");
+    if (n == 0) return INFR_HIP_OK;
+    HIP_TRY(be, hipMemcpyAsync(static_cast<uint8_t*>(dst->ptr) + dst_off, src, n,
+                               hipMemcpyHostToDevice, be->stream));
+    HIP_TRY(be, hipStreamSynchronize(be->stream));  // src may be reused as soon as we return
+    return INFR_HIP_OK;
+}
+int infr_hip_upload(infr_hip_t* be, infr_hip_buffer_t* dst, const void* src, size_t n) {
+    return infr_hip_upload_at(be, dst, 0, src, n);
+}
+
+int infr_hip_download_at(infr_hip_t* be, const infr_hip_buffer_t* src, size_t src_off, void* dst,
+                         size_t n) {
+    if (!be || !src || (!dst && n)) return fail(be, INFR_HIP_ERR_INVALID, "download: null argument");
+    if (src_off > src->len || n > src->len - src_off)
+        return fail(be, INFR_HIP_ERR_BACKEND,
+                    "download of " + std::to_string(n) + " bytes at " + std::to_string(src_off) +
+                        " exceeds the " + std::to_string(src->len) + "-byte buffer");
+    if (n) {
+        HIP_TRY(be, hipMemcpyAsync(dst, static_cast<const uint8_t*>(src->ptr) + src_off, n,
+                                   hipMemcpyDeviceToHost, be->stream));
+    }
+    HIP_TRY(be, hipStreamSynchronize(be->stream));
+    return INFR_HIP_OK;
+}
+int infr_hip_download(infr_hip_t* be, const infr_hip_buffer_t* src, void* dst, size_t n) {
+    return infr_hip_download_at(be, src, 0, dst, n);
+}
+
+int infr_hip_copy_buffer(infr_hip_t* be, const infr_hip_buffer_t* src, infr_hip_buffer_t* dst,
+                         size_t bytes) {
+    if (!be || !src || !dst) return fail(be, INFR_HIP_ERR_INVALID, "copy_buffer: null argument");
+    // check_copy_bytes (backend.rs:23-30): an oversize copy is an error, not a fault.
+    if (bytes > src->len || bytes > dst->len)
+        return fail(be, INFR_HIP_ERR_BACKEND,
+                    "copy_buffer: " + std::to_string(bytes) + " bytes exceeds src (" +
+                        std::to_string(src->len) + ") or dst (" + std::to_string(dst->len) + ")");
+    if (bytes)
+        HIP_TRY(be, hipMemcpyAsync(dst->ptr, src->ptr, bytes, hipMemcpyDeviceToDevice, be->stream));
+    return INFR_HIP_OK;
+}
+
+int infr_hip_sync(infr_hip_t* be) {
+    if (!be) return INFR_HIP_ERR_INVALID;
+    HIP_TRY(be, hipStreamSynchronize(be->stream));
+    return INFR_HIP_OK;
+}
+
+int infr_hip_linear(infr_hip_t* be, int dtype, const infr_hip_buffer_t* w, size_t w_numel,
+                    size_t w_off, const infr_hip_buffer_t* x, infr_hip_buffer_t* dst, size_t m,
+                    size_t in_f, size_t out_f) {
+    if (!be) return INFR_HIP_ERR_INVALID;
+    if (int rc = check_latch(be)) return rc;
+    LinearArgs la;
+    if (int rc = check_linear(be, dtype, w, w_numel, w_off, x, m, in_f, out_f, &la)) return rc;
+    if (!dst || dst->len < m * out_f * sizeof(float))
+        return fail(be, INFR_HIP_ERR_INVALID, "linear: dst buffer missing or too small");
+    if (int rc = ensure_act(be, m * in_f)) return rc;
+    return enqueue_linear(be, dtype, la, static_cast<const float*>(x->ptr),
+                          static_cast<float*>(dst->ptr), m, in_f, out_f, infr::IntStages{});
+}
+
+int infr_hip_linear_int_stages(infr_hip_t* be, int dtype, const infr_hip_buffer_t* w,
+                               size_t w_numel, size_t w_off, const infr_hip_buffer_t* x, size_t m,
+                               size_t in_f, size_t out_f, infr_hip_buffer_t* a,
+                               infr_hip_buffer_t* b) {
+    if (!be) return INFR_HIP_ERR_INVALID;
+    if (int rc = check_latch(be)) return rc;
+    LinearArgs la;
+    if (int rc = check_linear(be, dtype, w, w_numel, w_off, x, m, in_f, out_f, &la)) return rc;
+    const size_t blocks = (dtype == INFR_DTYPE_Q4_K || dtype == INFR_DTYPE_Q6_K) ? in_f / 256 : in_f / 32;
+    const size_t need = m * out_f * blocks * sizeof(int32_t);
+    if (!a || a->len < need) return fail(be, INFR_HIP_ERR_INVALID, "int_stages: buffer a too small");
+    if (dtype == INFR_DTYPE_Q4_K && (!b || b->len < need))
+        return fail(be, INFR_HIP_ERR_INVALID, "int_stages: Q4_K needs buffer b");
+    if (int rc = ensure_act(be, m * in_f)) return rc;
+    // y is not wanted here; use a transient output
+    float* y = nullptr;
+    HIP_TRY(be, hipMalloc((void**)&y, m * out_f * sizeof(float)));
+    infr::IntStages st;
+    st.a = static_cast<int32_t*>(a->ptr);
+    st.b = b ? static_cast<int32_t*>(b->ptr) : nullptr;
+    int rc = enqueue_linear(be, dtype, la, static_cast<const float*>(x->ptr), y, m, in_f, out_f, st);
+    (void)hipStreamSynchronize(be->stream);
+    (void)hipFree(y);
+    return rc;
+}
+
+static int quantize_impl(infr_hip_t* be, bool per32, const infr_hip_buffer_t* x, size_t m, size_t k,
+                         infr_hip_buffer_t* qs, infr_hip_buffer_t* d, infr_hip_buffer_t* bsums,
+                         infr_hip_buffer_t* bsums16) {
+    if (!be) return INFR_HIP_ERR_INVALID;
+    if (int rc = check_latch(be)) return rc;
+    if (!x || !qs || !d || !bsums) return fail(be, INFR_HIP_ERR_INVALID, "quantize: unbound buffer");
+    const size_t blk = per32 ? 32 : 256;
+    if (m == 0 || k == 0 || k % blk != 0)
+        return fail(be, INFR_HIP_ERR_UNSUPPORTED,
+                    "quantize: k " + std::to_string(k) + " is not a multiple of " + std::to_string(blk));
+    const size_t n = m * k;
+    if (x->len < n * 4 || qs->len < n || d->len < n / blk * 4 || bsums->len < n / 32 * 4 ||
+        (bsums16 && bsums16->len < n / 16 * 4))
+        return fail(be, INFR_HIP_ERR_INVALID, "quantize: a buffer is too small");
+    infr::ActQ8 out;
+    out.qs = static_cast<int8_t*>(qs->ptr);
+    out.d = static_cast<float*>(d->ptr);
+    out.bsums = static_cast<int32_t*>(bsums->ptr);
+    out.bsums16 = bsums16 ? static_cast<int32_t*>(bsums16->ptr) : nullptr;
+    infr::launch_quantize_q8(static_cast<const float*>(x->ptr), m, k, per32, out, be->stream);
+    HIP_TRY(be, hipGetLastError());
+    return INFR_HIP_OK;
+}
+
+int infr_hip_quantize_q8(infr_hip_t* be, const infr_hip_buffer_t* x, size_t m, size_t k,
+                         infr_hip_buffer_t* qs, infr_hip_buffer_t* d, infr_hip_buffer_t* bsums,
+                         infr_hip_buffer_t* bsums16) {
+    return quantize_impl(be, false, x, m, k, qs, d, bsums, bsums16);
+}
+int infr_hip_quantize_q8_32(infr_hip_t* be, const infr_hip_buffer_t* x, size_t m, size_t k,
+                            infr_hip_buffer_t* qs, infr_hip_buffer_t* d, infr_hip_buffer_t* bsum) {
+    return quantize_impl(be, true, x, m, k, qs, d, bsum, nullptr);
+}
+
+int infr_hip_moe_ffn(infr_hip_t* be, const infr_hip_moe_params_t*, const infr_hip_buffer_t*,
+                     const infr_hip_buffer_t*, const infr_hip_buffer_t*, const infr_hip_buffer_t*,
+                     const infr_hip_buffer_t*, const infr_hip_buffer_t*, infr_hip_buffer_t*,
+                     infr_hip_buffer_t*, infr_hip_buffer_t*) {
+    return fail(be, INFR_HIP_ERR_UNSUPPORTED, "moe_ffn: not built yet");
+}
+
+// ---- plan / execute ----
+
+int infr_hip_compile(infr_hip_t* be, const infr_hip_op_t* ops, size_t n_ops, infr_hip_plan_t** out) {
+    if (!be || !out || (!ops && n_ops)) return fail(be, INFR_HIP_ERR_INVALID, "compile: null argument");
+    *out = nullptr;
+    infr_hip_plan_t* p = new (std::nothrow) infr_hip_plan();
+    if (!p) return fail(be, INFR_HIP_ERR_OTHER, "compile: out of host memory");
+    p->ops.assign(ops, ops + n_ops);
+    size_t act_need = 0;
+    for (const auto& op : p->ops) {
+        if (op.kind == INFR_OP_LINEAR) {
+            if (!is_quant(op.w_dtype) || op.m == 0 || op.in_f == 0 || op.out_f == 0 ||
+                op.in_f % (act_per32(op.w_dtype) ? 64 : 256) != 0 || op.w_numel % op.in_f != 0 ||
+                op.w_off % op.in_f != 0) {
+                delete p;
+                return fail(be, INFR_HIP_ERR_UNSUPPORTED, "compile: Linear op with unsupported dtype/shape");
+            }
+            p->max_tensor = std::max({p->max_tensor, op.x, op.weight, op.dst});
+            act_need = std::max(act_need, (size_t)op.m * op.in_f);
+        } else {
+            delete p;
+            return fail(be, INFR_HIP_ERR_UNSUPPORTED, "compile: op kind " + std::to_string(op.kind));
+        }
+    }
+    // Scratch is sized here so that execute never allocates (it records launches for replay).
+    if (int rc = ensure_act(be, act_need)) {
+        delete p;
+        return rc;
+    }
+    *out = p;
+    return INFR_HIP_OK;
+}
+
+void infr_hip_plan_free(infr_hip_t* be, infr_hip_plan_t* plan) {
+    if (!plan) return;
+    if (plan->exec) {
+        if (be && be->stream) (void)hipStreamSynchronize(be->stream);
+        (void)hipGraphExecDestroy(plan->exec);
+    }
+    delete plan;
+}
+
+static int enqueue_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t* const* bindings) {
+    for (const auto& op : plan->ops) {
+        const infr_hip_buffer_t* w = bindings[op.weight];
+        const infr_hip_buffer_t* x = bindings[op.x];
+        infr_hip_buffer_t* dst = bindings[op.dst];
+        LinearArgs la;
+        if (int rc = check_linear(be, op.w_dtype, w, op.w_numel, op.w_off, x, op.m, op.in_f, op.out_f, &la))
+            return rc;
+        if (!dst || dst->len < (size_t)op.m * op.out_f * sizeof(float))
+            return fail(be, INFR_HIP_ERR_INVALID, "execute: dst buffer missing or too small");
+        if (int rc = enqueue_linear(be, op.w_dtype, la, static_cast<const float*>(x->ptr),
+                                    static_cast<float*>(dst->ptr), op.m, op.in_f, op.out_f,
+                                    infr::IntStages{}))
+            return rc;
+    }
+    return INFR_HIP_OK;
+}
+
+int infr_hip_execute(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t* const* bindings,
+                     size_t n_bindings) {
+    if (!be || !plan || (!bindings && n_bindings)) return fail(be, INFR_HIP_ERR_INVALID, "execute: null argument");
+    if (int rc = check_latch(be)) return rc;
+    if (!plan->ops.empty() && plan->max_tensor >= n_bindings)
+        return fail(be, INFR_HIP_ERR_INVALID, "execute: a tensor id has no binding slot");
+    // Replay when every bound device address is what the recording saw.
+    std::vector<void*> now(n_bindings);
+    for (size_t i = 0; i < n_bindings; ++i) now[i] = bindings[i] ? bindings[i]->ptr : nullptr;
+    if (plan->exec && now == plan->bound) {
+        HIP_TRY(be, hipGraphLaunch(plan->exec, be->stream));
+        return INFR_HIP_OK;
+    }
+    if (plan->exec) {
+        HIP_TRY(be, hipStreamSynchronize(be->stream));
+        (void)hipGraphExecDestroy(plan->exec);
+        plan->exec = nullptr;
+    }
+    // Validate everything before recording so a bad binding cannot leave a capture open.
+    for (const auto& op : plan->ops) {
+        LinearArgs la;
+        if (int rc = check_linear(be, op.w_dtype, bindings[op.weight], op.w_numel, op.w_off,
+                                  bindings[op.x], op.m, op.in_f, op.out_f, &la))
+            return rc;
+        if (!bindings[op.dst] || bindings[op.dst]->len < (size_t)op.m * op.out_f * sizeof(float))
+            return fail(be, INFR_HIP_ERR_INVALID, "execute: dst buffer missing or too small");
+    }
+    hipGraph_t graph = nullptr;
+    HIP_TRY(be, hipStreamBeginCapture(be->stream, hipStreamCaptureModeThreadLocal));
+    int rc = enqueue_plan(be, plan, bindings);
+    hipError_t e = hipStreamEndCapture(be->stream, &graph);
+    if (rc != INFR_HIP_OK) {
+        if (graph) (void)hipGraphDestroy(graph);
+        return rc;
+    }
+    if (e != hipSuccess) return fail(be, INFR_HIP_ERR_BACKEND, std::string("hipStreamEndCapture: ") + hipGetErrorString(e));
+    e = hipGraphInstantiate(&plan->exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) {
+        plan->exec = nullptr;
+        return fail(be, INFR_HIP_ERR_BACKEND, std::string("hipGraphInstantiate: ") + hipGetErrorString(e));
+    }
+    plan->bound = now;
+    HIP_TRY(be, hipGraphLaunch(plan->exec, be->stream));
+    return INFR_HIP_OK;
+}
+
+// ---- shutdown latch ----
+int infr_hip_request_shutdown(int signo) {
+    int expected = 0;
+    return g_shutdown_signo.compare_exchange_strong(expected, signo, std::memory_order_relaxed) ? 1 : 0;
+}
+int infr_hip_shutdown_requested(void) { return g_shutdown_signo.load(std::memory_order_relaxed) != 0; }
+int infr_hip_shutdown_signal(void) { return g_shutdown_signo.load(std::memory_order_relaxed); }
+void infr_hip_reset_shutdown(void) { g_shutdown_signo.store(0, std::memory_order_relaxed); }
+
+// ---- timing ----
+int infr_hip_timer_begin(infr_hip_t* be) {
+    if (!be) return INFR_HIP_ERR_INVALID;
+    HIP_TRY(be, hipEventRecord(be->ev0, be->stream));
+    return INFR_HIP_OK;
+}
+int infr_hip_timer_end(infr_hip_t* be, float* elapsed_ms) {
+    if (!be || !elapsed_ms) return INFR_HIP_ERR_INVALID;
+    HIP_TRY(be, hipEventRecord(be->ev1, be->stream));
+    HIP_TRY(be, hipEventSynchronize(be->ev1));
+    HIP_TRY(be, hipEventElapsedTime(elapsed_ms, be->ev0, be->ev1));
+    return INFR_HIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,85 @@
+// Shared device helpers for the gfx950 kernels: wave64 cross-lane primitives, f16 widening,
+// packed-int8 unpack helpers. Everything here is compiled with -ffp-contract=off: the f32
+// epilogues restate infr-cpu's expressions, which never fuse a multiply with an add unless the
+// CPU code calls mul_add (then __builtin_fmaf is written out here).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace infr {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+constexpr int kWave = 64;
+
+// half::f16::to_f32 (crates/infr-gguf/src/dequant.rs:68-70): exact widening, v_cvt_f32_f16.
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t bits16) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)bits16);
+}
+
+// 16-byte load from an address that is only 2-byte aligned (Q6_K / Q8_0 / Q2_0 block strides
+// are 2 mod 4). gfx950 global loads take any alignment in the HSA unaligned-access mode.
+__device__ __forceinline__ v4i load16_a2(const uint8_t* p) {
+    v4i v;
+    __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 16);
+    return v;
+}
+__device__ __forceinline__ v4i load16(const uint8_t* p) {
+    return *reinterpret_cast<const v4i*>(__builtin_assume_aligned(p, 16));
+}
+__device__ __forceinline__ uint32_t load_u16(const uint8_t* p) {
+    uint16_t v;
+    __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 2);
+    return v;
+}
+
+// signed int8x4 . int8x4 + acc  (v_dot4_i32_i8)
+__device__ __forceinline__ int dot4(int a, int b, int acc) {
+    return __builtin_amdgcn_sdot4(a, b, acc, false);
+}
+
+// DPP quad permutes: exchange with lane^1 / lane^2 inside each group of four lanes.
+__device__ __forceinline__ int quad_xor1(int v) {
+    return __builtin_amdgcn_mov_dpp(v, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+}
+__device__ __forceinline__ int quad_xor2(int v) {
+    return __builtin_amdgcn_mov_dpp(v, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+}
+// Sum over each aligned group of four lanes; every lane of the group gets the total.
+__device__ __forceinline__ int quad_sum(int v) {
+    v += quad_xor1(v);
+    v += quad_xor2(v);
+    return v;
+}
+
+__device__ __forceinline__ float readlane_f(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+// Butterfly sum over the 64 lanes (order fixed by the lane pairing, so runs are reproducible).
+__device__ __forceinline__ float wave_sum_f(float v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+__device__ __forceinline__ int wave_sum_i(int v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+// get_scale_min_k4 for all eight sub-blocks at once (crates/infr-gguf/src/dequant.rs:73-83):
+// s0,s1,s2 are the three little-endian words of scales[12]; on return sc8[0..1] hold the eight
+// 6-bit scales as bytes and mn8[0..1] the eight 6-bit mins.
+__device__ __forceinline__ void k4_all(uint32_t s0, uint32_t s1, uint32_t s2, uint32_t sc8[2],
+                                       uint32_t mn8[2]) {
+    sc8[0] = s0 & 0x3F3F3F3Fu;
+    mn8[0] = s1 & 0x3F3F3F3Fu;
+    sc8[1] = (s2 & 0x0F0F0F0Fu) | ((s0 >> 2) & 0x30303030u);
+    mn8[1] = ((s2 >> 4) & 0x0F0F0F0Fu) | ((s1 >> 2) & 0x30303030u);
+}
+
+}  // namespace infr

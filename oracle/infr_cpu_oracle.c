@@ -1,0 +1,839 @@
+/*
+ * CPU oracle: plain-C restatement of infr-cpu's quantized Op::Linear / Op::MoeFfn path.
+ * TEST INFRASTRUCTURE ONLY — see infr_cpu_oracle.h for scope, citations and pinning status.
+ * Build: gcc -O2 -ffp-contract=off -fno-fast-math -fopenmp (see Makefile).
+ */
+#include "infr_cpu_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+/* ───────────────────────────── block geometry ───────────────────────────── */
+
+/* crates/infr-core/src/decode_spec.rs:319-358: Q8_0 (32,34), Q4K (256,144), Q6K (256,210),
+ * Q2_0 (64,18). */
+int orc_block_layout(int dtype, int *elems, int *bytes) {
+    int e = 0, b = 0;
+    switch (dtype) {
+    case ORC_F32: e = 1; b = 4; break;
+    case ORC_F16: e = 1; b = 2; break;
+    case ORC_Q8_0: e = 32; b = 34; break;
+    case ORC_Q4_K: e = 256; b = 144; break;
+    case ORC_Q6_K: e = 256; b = 210; break;
+    case ORC_Q2_0: e = 64; b = 18; break;
+    default: return 0;
+    }
+    if (elems) *elems = e;
+    if (bytes) *bytes = b;
+    return 1;
+}
+
+/* ───────────────────────────── f16 ───────────────────────────── */
+
+/* half::f16::to_f32 — exact widening, subnormals included. */
+float orc_f16_bits_to_f32(uint16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1Fu;
+    uint32_t man = h & 0x3FFu;
+    uint32_t bits;
+    if (exp == 0) {
+        if (man == 0) {
+            bits = sign;
+        } else {
+            /* subnormal: value = man * 2^-24; normalise */
+            int shift = 0;
+            while ((man & 0x400u) == 0) {
+                man <<= 1;
+                shift++;
+            }
+            man &= 0x3FFu;
+            bits = sign | ((uint32_t)(127 - 15 - shift + 1) << 23) | (man << 13);
+        }
+    } else if (exp == 31) {
+        bits = sign | 0x7F800000u | (man << 13);
+    } else {
+        bits = sign | ((exp + (127 - 15)) << 23) | (man << 13);
+    }
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+
+float orc_rdf16(const uint8_t *b) {
+    return orc_f16_bits_to_f32((uint16_t)(b[0] | ((uint16_t)b[1] << 8)));
+}
+
+/* half::f16::from_f32 — round to nearest even, overflow to inf, gradual underflow. */
+uint16_t orc_f32_to_f16_bits(float f) {
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    uint32_t sign = (x >> 16) & 0x8000u;
+    uint32_t exp = (x >> 23) & 0xFFu;
+    uint32_t man = x & 0x7FFFFFu;
+    if (exp == 0xFF) { /* inf / nan */
+        return (uint16_t)(sign | 0x7C00u | (man ? (0x200u | (man >> 13)) : 0));
+    }
+    int e = (int)exp - 127 + 15;
+    if (e >= 31) return (uint16_t)(sign | 0x7C00u); /* overflow -> inf */
+    if (e <= 0) {
+        if (e < -10) return (uint16_t)sign; /* underflows to zero even after rounding */
+        man |= 0x800000u;                   /* implicit one */
+        int shift = 14 - e;                 /* 14..24 */
+        uint32_t half_man = man >> shift;
+        uint32_t rem = man & ((1u << shift) - 1);
+        uint32_t halfway = 1u << (shift - 1);
+        if (rem > halfway || (rem == halfway && (half_man & 1))) half_man++;
+        return (uint16_t)(sign | half_man); /* may carry into the exponent: correct */
+    }
+    uint32_t half_man = man >> 13;
+    uint32_t rem = man & 0x1FFFu;
+    uint16_t h = (uint16_t)(sign | ((uint32_t)e << 10) | half_man);
+    if (rem > 0x1000u || (rem == 0x1000u && (half_man & 1))) h++; /* carry may reach inf: correct */
+    return h;
+}
+
+/* ───────────────────────────── k4 ───────────────────────────── */
+
+/* crates/infr-gguf/src/dequant.rs:73-83 (llama.cpp get_scale_min_k4). */
+void orc_k4(int j, const uint8_t *q, uint32_t *sc, uint32_t *m) {
+    if (j < 4) {
+        *sc = q[j] & 63;
+        *m = q[j + 4] & 63;
+    } else {
+        *sc = (uint32_t)((q[j + 4] & 0x0F) | ((q[j - 4] >> 6) << 4));
+        *m = (uint32_t)((q[j + 4] >> 4) | ((q[j] >> 6) << 4));
+    }
+}
+
+/* ───────────────────────────── host decode ───────────────────────────── */
+
+/* crates/infr-gguf/src/dequant.rs:11-51: for affine quants the factored form is expanded as
+ *   sc = f32(d) * (f32)scm_sc;  mn = f32(dmin) * (f32)scm_m;  out = sc * (f32)code + mn
+ * (separate multiply and add). Factored arms: Q8_0 :209-219, Q4K :311-331, Q6K :361-385.
+ * Q2_0 is a codebook quant: (q-1) as f32 * d (:998-1018). */
+int orc_dequant_block(int dtype, const uint8_t *bytes, size_t nbytes, float *out) {
+    int qpb, bpb;
+    if (!orc_block_layout(dtype, &qpb, &bpb)) return -1;
+    size_t nblk = nbytes / (size_t)bpb;
+    switch (dtype) {
+    case ORC_F32:
+        memcpy(out, bytes, nblk * 4);
+        return 0;
+    case ORC_F16:
+        for (size_t i = 0; i < nblk; i++) out[i] = orc_rdf16(bytes + 2 * i);
+        return 0;
+    case ORC_Q8_0:
+        for (size_t b = 0; b < nblk; b++) {
+            const uint8_t *blk = bytes + b * 34;
+            float d = orc_rdf16(blk);
+            /* scm = (1, -128) for both 16-groups; code = q + 128 */
+            float sc = d * (float)1;
+            float mn = d * (float)(-128);
+            for (int i = 0; i < 32; i++) {
+                uint8_t code = (uint8_t)((int16_t)(int8_t)blk[2 + i] + 128);
+                out[b * 32 + i] = sc * (float)code + mn;
+            }
+        }
+        return 0;
+    case ORC_Q4_K:
+        for (size_t b = 0; b < nblk; b++) {
+            const uint8_t *blk = bytes + b * 144;
+            float d = orc_rdf16(blk);
+            float dmin = orc_rdf16(blk + 2);
+            const uint8_t *scales = blk + 4;
+            const uint8_t *qs = blk + 16;
+            float *o = out + b * 256;
+            for (int j = 0; j < 4; j++) {
+                uint32_t sc1, m1, sc2, m2;
+                orc_k4(2 * j, scales, &sc1, &m1);
+                orc_k4(2 * j + 1, scales, &sc2, &m2);
+                float fs1 = d * (float)(int16_t)sc1, fm1 = dmin * (float)(int16_t)(-(int16_t)m1);
+                float fs2 = d * (float)(int16_t)sc2, fm2 = dmin * (float)(int16_t)(-(int16_t)m2);
+                for (int l = 0; l < 32; l++) {
+                    uint8_t v = qs[j * 32 + l];
+                    o[j * 64 + l] = fs1 * (float)(v & 0xF) + fm1;
+                    o[j * 64 + 32 + l] = fs2 * (float)(v >> 4) + fm2;
+                }
+            }
+        }
+        return 0;
+    case ORC_Q6_K:
+        for (size_t b = 0; b < nblk; b++) {
+            const uint8_t *blk = bytes + b * 210;
+            const uint8_t *ql = blk, *qh = blk + 128, *scales = blk + 192;
+            float d = orc_rdf16(blk + 208);
+            float *o = out + b * 256;
+            for (int half = 0; half < 2; half++) {
+                int qlo = half * 64, qho = half * 32, sco = half * 8, base = half * 128;
+                for (int l = 0; l < 32; l++) {
+                    int is = l / 16;
+                    uint8_t c[4];
+                    c[0] = (uint8_t)((ql[qlo + l] & 0xF) | ((qh[qho + l] & 3) << 4));
+                    c[1] = (uint8_t)((ql[qlo + l + 32] & 0xF) | (((qh[qho + l] >> 2) & 3) << 4));
+                    c[2] = (uint8_t)((ql[qlo + l] >> 4) | (((qh[qho + l] >> 4) & 3) << 4));
+                    c[3] = (uint8_t)((ql[qlo + l + 32] >> 4) | (((qh[qho + l] >> 6) & 3) << 4));
+                    for (int k = 0; k < 4; k++) {
+                        int16_t s = (int16_t)(int8_t)scales[sco + is + 2 * k];
+                        float sc = d * (float)s;
+                        float mn = d * (float)(int16_t)(-32 * s);
+                        o[base + l + 32 * k] = sc * (float)c[k] + mn;
+                    }
+                }
+            }
+        }
+        return 0;
+    case ORC_Q2_0:
+        for (size_t b = 0; b < nblk; b++) {
+            const uint8_t *blk = bytes + b * 18;
+            float d = orc_rdf16(blk);
+            const uint8_t *qs = blk + 2;
+            for (int j = 0; j < 64; j++) {
+                int q = (qs[j / 4] >> ((j % 4) * 2)) & 3;
+                out[b * 64 + j] = (float)(q - 1) * d;
+            }
+        }
+        return 0;
+    default:
+        return -1;
+    }
+}
+
+/* ───────────────────────────── activation quantizers ───────────────────────────── */
+
+static inline int8_t quant_one(float v, float id) {
+    /* (v * id).round().clamp(-127.0, 127.0) as i8 — Rust f32::round is half away from zero */
+    float r = roundf(v * id);
+    if (r < -127.0f) r = -127.0f;
+    if (r > 127.0f) r = 127.0f;
+    return (int8_t)r;
+}
+
+/* crates/infr-cpu/src/quant.rs:27-58 */
+void orc_quantize_q8(const float *x, size_t len, int8_t *qs, float *d, int32_t *bsums,
+                     int32_t *bsums16) {
+    size_t nb = len / 256;
+    for (size_t b = 0; b < nb; b++) {
+        const float *blk = x + b * 256;
+        float amax = 0.0f;
+        for (int i = 0; i < 256; i++) {
+            float a = fabsf(blk[i]);
+            amax = a > amax ? a : amax; /* f32::max fold from 0 */
+        }
+        float dd = amax / 127.0f;
+        float id = dd > 0.0f ? 1.0f / dd : 0.0f;
+        d[b] = dd;
+        for (int i = 0; i < 256; i++) qs[b * 256 + i] = quant_one(blk[i], id);
+    }
+    for (size_t b = 0; b < nb; b++) {
+        int32_t s16[16];
+        for (int s = 0; s < 16; s++) {
+            int32_t acc = 0;
+            for (int i = 0; i < 16; i++) acc += qs[b * 256 + s * 16 + i];
+            s16[s] = acc;
+            if (bsums16) bsums16[b * 16 + s] = acc;
+        }
+        for (int s = 0; s < 8; s++) bsums[b * 8 + s] = s16[2 * s] + s16[2 * s + 1];
+    }
+}
+
+/* crates/infr-cpu/src/quant.rs:97-117 */
+void orc_quantize_q8_32(const float *x, size_t len, int8_t *qs, float *d, int32_t *bsum) {
+    size_t nb = len / 32;
+    for (size_t b = 0; b < nb; b++) {
+        const float *blk = x + b * 32;
+        float amax = 0.0f;
+        for (int i = 0; i < 32; i++) {
+            float a = fabsf(blk[i]);
+            amax = a > amax ? a : amax;
+        }
+        float dd = amax / 127.0f;
+        float id = dd > 0.0f ? 1.0f / dd : 0.0f;
+        d[b] = dd;
+        int32_t s = 0;
+        for (int i = 0; i < 32; i++) {
+            int8_t q = quant_one(blk[i], id);
+            qs[b * 32 + i] = q;
+            s += q;
+        }
+        bsum[b] = s;
+    }
+}
+
+/* ───────────────────────────── scalar dot kernels ───────────────────────────── */
+
+/* crates/infr-cpu/src/kernels.rs:151-184 (vec_dot_q4k_scalar); the batch scalar (:1458-1509)
+ * evaluates the same expression in the same order per activation row. */
+float orc_vec_dot_q4k(const uint8_t *row, const int8_t *qs8, const float *d8, const int32_t *bsums,
+                      size_t in_f, int32_t *sd_out, int32_t *sm_out) {
+    size_t nb = in_f / 256;
+    float sumf = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * 144;
+        float d = orc_rdf16(blk);
+        float dmin = orc_rdf16(blk + 2);
+        const uint8_t *scales = blk + 4;
+        const uint8_t *qs = blk + 16;
+        const int8_t *q8b = qs8 + b * 256;
+        int32_t sd = 0, sm = 0;
+        for (int s = 0; s < 8; s++) {
+            uint32_t sc, m;
+            orc_k4(s, scales, &sc, &m);
+            int half = s / 2, hi = (s % 2) == 1;
+            const uint8_t *qbyte = qs + half * 32;
+            const int8_t *q8s = q8b + s * 32;
+            int32_t iprod = 0;
+            for (int l = 0; l < 32; l++) {
+                int32_t q4 = hi ? (qbyte[l] >> 4) : (qbyte[l] & 0xF);
+                iprod += q4 * (int32_t)q8s[l];
+            }
+            int32_t isum = bsums[b * 8 + s];
+            sd += (int32_t)sc * iprod;
+            sm += (int32_t)m * isum;
+        }
+        if (sd_out) sd_out[b] = sd;
+        if (sm_out) sm_out[b] = sm;
+        sumf += d8[b] * (d * (float)sd - dmin * (float)sm);
+    }
+    return sumf;
+}
+
+/* crates/infr-cpu/src/kernels.rs:487-526 (vec_dot_q6k_scalar). */
+float orc_vec_dot_q6k(const uint8_t *row, const int8_t *qs8, const float *d8, size_t in_f,
+                      int32_t *isum_out) {
+    size_t nb = in_f / 256;
+    float sumf = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * 210;
+        const uint8_t *ql = blk, *qh = blk + 128, *scales = blk + 192;
+        float d = orc_rdf16(blk + 208);
+        const int8_t *q8b = qs8 + b * 256;
+        int32_t sumi[16] = {0}, bsum[16] = {0};
+        for (int half = 0; half < 2; half++) {
+            int qlo = half * 64, qho = half * 32, sco = half * 8, base = half * 128;
+            for (int l = 0; l < 32; l++) {
+                int is = l / 16;
+                int32_t q[4];
+                q[0] = (ql[qlo + l] & 0xF) | ((qh[qho + l] & 3) << 4);
+                q[1] = (ql[qlo + l + 32] & 0xF) | (((qh[qho + l] >> 2) & 3) << 4);
+                q[2] = (ql[qlo + l] >> 4) | (((qh[qho + l] >> 4) & 3) << 4);
+                q[3] = (ql[qlo + l + 32] >> 4) | (((qh[qho + l] >> 6) & 3) << 4);
+                for (int k = 0; k < 4; k++) {
+                    int sub = sco + is + 2 * k;
+                    int32_t v = q8b[base + l + 32 * k];
+                    sumi[sub] += q[k] * v;
+                    bsum[sub] += v;
+                }
+            }
+        }
+        int32_t isum = 0;
+        for (int sub = 0; sub < 16; sub++)
+            isum += (int32_t)(int8_t)scales[sub] * (sumi[sub] - 32 * bsum[sub]);
+        if (isum_out) isum_out[b] = isum;
+        sumf += d * d8[b] * (float)isum; /* (d * q8.d[b]) * (isum as f32) */
+    }
+    return sumf;
+}
+
+/* crates/infr-cpu/src/kernels.rs:1170-1187 (vec_dot_q8_0_scalar): weight blocks of 32 against the
+ * per-256 activation scale. */
+float orc_vec_dot_q8_0(const uint8_t *row, const int8_t *qs8, const float *d8, size_t in_f,
+                       int32_t *iprod_out) {
+    size_t nb_super = in_f / 256;
+    float sumf = 0.0f;
+    for (size_t b = 0; b < nb_super; b++) {
+        float dact = d8[b];
+        for (int s = 0; s < 8; s++) {
+            size_t wb = b * 8 + (size_t)s;
+            const uint8_t *blk = row + wb * 34;
+            float d_w = orc_rdf16(blk);
+            const int8_t *qw = (const int8_t *)(blk + 2);
+            const int8_t *qx = qs8 + b * 256 + s * 32;
+            int32_t iprod = 0;
+            for (int i = 0; i < 32; i++) iprod += (int32_t)qw[i] * (int32_t)qx[i];
+            if (iprod_out) iprod_out[wb] = iprod;
+            sumf += dact * d_w * (float)iprod; /* (d8 * d_w) * (iprod as f32) */
+        }
+    }
+    return sumf;
+}
+
+/* crates/infr-cpu/src/kernels.rs:5641-5668 (vec_dot_q2_0_batch_scalar, one activation row). */
+float orc_vec_dot_q2_0(const uint8_t *row, const int8_t *qs8, const float *d8, const int32_t *bsum,
+                       size_t in_f, int32_t *iprod_out) {
+    size_t nb = in_f / 64;
+    float sumf = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * 18;
+        const uint8_t *qs = blk + 2;
+        float d = orc_rdf16(blk);
+        for (int sub = 0; sub < 2; sub++) {
+            size_t s = 2 * b + (size_t)sub;
+            const int8_t *q8b = qs8 + s * 32;
+            int32_t iprod = 0;
+            for (int p = 0; p < 32; p++) {
+                int j = sub * 32 + p;
+                int32_t code = (qs[j / 4] >> ((j % 4) * 2)) & 3;
+                iprod += code * (int32_t)q8b[p];
+            }
+            if (iprod_out) iprod_out[s] = iprod;
+            sumf += d * d8[s] * ((float)iprod - (float)bsum[s]);
+        }
+    }
+    return sumf;
+}
+
+/* crates/infr-cpu/src/kernels.rs:6557-6573 */
+float orc_dot(const float *a, const float *b, size_t n) {
+    size_t chunks = n / 8;
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (size_t c = 0; c < chunks; c++) {
+        size_t base = c * 8;
+        for (int j = 0; j < 8; j++) acc[j] = fmaf(a[base + j], b[base + j], acc[j]);
+    }
+    float s = 0.0f; /* acc.iter().sum() */
+    for (int j = 0; j < 8; j++) s += acc[j];
+    for (size_t i = chunks * 8; i < n; i++) s = fmaf(a[i], b[i], s);
+    return s;
+}
+
+/* crates/infr-cpu/src/kernels.rs:6578-6585 (Activation::Silu) */
+float orc_silu(float g) { return g / (1.0f + expf(-g)); }
+
+/* ───────────────────────────── Op::Linear ───────────────────────────── */
+
+typedef struct {
+    int8_t *qs;
+    float *d;
+    int32_t *bsums;   /* per 32 */
+    int32_t *bsums16; /* per 16 (Q8 only) */
+} acts_t;
+
+static int is_q8_super(int dtype) {
+    return dtype == ORC_Q4_K || dtype == ORC_Q6_K || dtype == ORC_Q8_0;
+}
+
+static void acts_free(acts_t *a) {
+    free(a->qs);
+    free(a->d);
+    free(a->bsums);
+    free(a->bsums16);
+}
+
+/* Quantize m rows with the quantizer the dispatch picks: per-256 `Q8` for Q4K/Q6K/Q8_0
+ * (crates/infr-cpu/src/lib.rs:1043-1062,1186-1210), per-32 `Q8x32` for Q2_0 (:1064-1076,1406-1412). */
+static int acts_build(int dtype, const float *x, size_t m, size_t in_f, acts_t *a) {
+    memset(a, 0, sizeof *a);
+    a->qs = (int8_t *)malloc(m * in_f);
+    if (is_q8_super(dtype)) {
+        size_t nb = in_f / 256;
+        a->d = (float *)malloc(sizeof(float) * m * nb);
+        a->bsums = (int32_t *)malloc(sizeof(int32_t) * m * nb * 8);
+        a->bsums16 = (int32_t *)malloc(sizeof(int32_t) * m * nb * 16);
+#pragma omp parallel for schedule(static)
+        for (long r = 0; r < (long)m; r++)
+            orc_quantize_q8(x + r * in_f, in_f, a->qs + r * in_f, a->d + r * nb,
+                            a->bsums + r * nb * 8, a->bsums16 + r * nb * 16);
+    } else {
+        size_t nb = in_f / 32;
+        a->d = (float *)malloc(sizeof(float) * m * nb);
+        a->bsums = (int32_t *)malloc(sizeof(int32_t) * m * nb);
+#pragma omp parallel for schedule(static)
+        for (long r = 0; r < (long)m; r++)
+            orc_quantize_q8_32(x + r * in_f, in_f, a->qs + r * in_f, a->d + r * nb,
+                               a->bsums + r * nb);
+    }
+    return 0;
+}
+
+static float row_dot(int dtype, const uint8_t *row, const acts_t *a, size_t r, size_t in_f,
+                     int32_t *ia, int32_t *ib) {
+    switch (dtype) {
+    case ORC_Q4_K: {
+        size_t nb = in_f / 256;
+        return orc_vec_dot_q4k(row, a->qs + r * in_f, a->d + r * nb, a->bsums + r * nb * 8, in_f,
+                               ia, ib);
+    }
+    case ORC_Q6_K: {
+        size_t nb = in_f / 256;
+        return orc_vec_dot_q6k(row, a->qs + r * in_f, a->d + r * nb, in_f, ia);
+    }
+    case ORC_Q8_0: {
+        size_t nb = in_f / 256;
+        return orc_vec_dot_q8_0(row, a->qs + r * in_f, a->d + r * nb, in_f, ia);
+    }
+    case ORC_Q2_0: {
+        size_t nb = in_f / 32;
+        return orc_vec_dot_q2_0(row, a->qs + r * in_f, a->d + r * nb, a->bsums + r * nb, in_f, ia);
+    }
+    default:
+        return 0.0f;
+    }
+}
+
+static int linear_shape_ok(int dtype, size_t in_f) {
+    /* The restatement carries the arms the four formats take when in_f is block-aligned:
+     * Q4K/Q6K: 256-element weight blocks; Q8_0 with in_f % 256 != 0 would go to the per-32 kernel
+     * (lib.rs:1037-1042) which is not restated; Q2_0 needs in_f % 64 == 0 (lib.rs:1406). */
+    switch (dtype) {
+    case ORC_Q4_K:
+    case ORC_Q6_K:
+    case ORC_Q8_0: return in_f % 256 == 0;
+    case ORC_Q2_0: return in_f % 64 == 0;
+    case ORC_F32: return 1;
+    default: return 0;
+    }
+}
+
+int orc_max_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+int orc_linear(int dtype, const uint8_t *w, size_t wbytes, size_t w_numel, size_t w_off,
+               const float *x, float *y, size_t m, size_t in_f, size_t out_f, int reference_mode,
+               int threads) {
+    if (!w || !x || !y || in_f == 0 || w_numel % in_f != 0 || w_off % in_f != 0) return -2;
+    if (!linear_shape_ok(dtype, in_f)) return -1;
+    /* lib.rs:1003-1008 */
+    size_t total_rows = w_numel / in_f;
+    size_t bpr = wbytes / total_rows;
+    size_t row0 = w_off / in_f;
+    if (row0 + out_f > total_rows) return -2;
+    const uint8_t *wb = w + row0 * bpr;
+#ifdef _OPENMP
+    int nt = threads > 0 ? threads : omp_get_max_threads();
+#else
+    int nt = 1;
+    (void)threads;
+#endif
+    (void)nt;
+
+    if (dtype == ORC_F32 || reference_mode) {
+        /* lib.rs:1015-1031 (reference mode) / :1162,1443-1448 (F32 weights): decode row, dot(). */
+#pragma omp parallel num_threads(nt)
+        {
+            float *wf = (float *)malloc(sizeof(float) * in_f);
+#pragma omp for schedule(dynamic, 8)
+            for (long o = 0; o < (long)out_f; o++) {
+                orc_dequant_block(dtype, wb + (size_t)o * bpr, bpr, wf);
+                for (size_t r = 0; r < m; r++) y[r * out_f + (size_t)o] = orc_dot(wf, x + r * in_f, in_f);
+            }
+            free(wf);
+        }
+        return 0;
+    }
+
+    acts_t a;
+    acts_build(dtype, x, m, in_f, &a);
+    if (m == 1) {
+        /* lib.rs:1079: 16 output rows per claimed task */
+#pragma omp parallel for schedule(dynamic, 16) num_threads(nt)
+        for (long o = 0; o < (long)out_f; o++)
+            y[o] = row_dot(dtype, wb + (size_t)o * bpr, &a, 0, in_f, NULL, NULL);
+    } else {
+        /* lib.rs:1211-1489: o-major temp then transpose; per element identical to the single-row
+         * kernel (batch kernels are bit-identical, kernels.rs:9297-9405). 8-row groups. */
+        float *out_t = (float *)malloc(sizeof(float) * out_f * m);
+#pragma omp parallel for schedule(dynamic, 8) num_threads(nt)
+        for (long o = 0; o < (long)out_f; o++)
+            for (size_t r = 0; r < m; r++)
+                out_t[(size_t)o * m + r] = row_dot(dtype, wb + (size_t)o * bpr, &a, r, in_f, NULL, NULL);
+#pragma omp parallel for schedule(static) num_threads(nt)
+        for (long r = 0; r < (long)m; r++)
+            for (size_t o = 0; o < out_f; o++) y[(size_t)r * out_f + o] = out_t[o * m + (size_t)r];
+        free(out_t);
+    }
+    acts_free(&a);
+    return 0;
+}
+
+int orc_linear_int_stages(int dtype, const uint8_t *w, size_t wbytes, size_t w_numel, size_t w_off,
+                          const float *x, size_t m, size_t in_f, size_t out_f, int32_t *ia,
+                          int32_t *ib) {
+    if (!w || !x || !ia || in_f == 0 || w_numel % in_f != 0 || w_off % in_f != 0) return -2;
+    if (!linear_shape_ok(dtype, in_f) || dtype == ORC_F32) return -1;
+    size_t total_rows = w_numel / in_f;
+    size_t bpr = wbytes / total_rows;
+    size_t row0 = w_off / in_f;
+    if (row0 + out_f > total_rows) return -2;
+    const uint8_t *wb = w + row0 * bpr;
+    size_t blocks = (dtype == ORC_Q4_K || dtype == ORC_Q6_K) ? in_f / 256 : in_f / 32;
+    acts_t a;
+    acts_build(dtype, x, m, in_f, &a);
+#pragma omp parallel for schedule(dynamic, 8)
+    for (long o = 0; o < (long)out_f; o++)
+        for (size_t r = 0; r < m; r++) {
+            size_t off = (r * out_f + (size_t)o) * blocks;
+            row_dot(dtype, wb + (size_t)o * bpr, &a, r, in_f, ia + off, ib ? ib + off : NULL);
+        }
+    acts_free(&a);
+    return 0;
+}
+
+/* crates/infr-testkit/src/lib.rs:150-163 */
+void orc_ref_linear_f64(const float *x, const float *w, size_t m, size_t in_f, size_t out_f,
+                        float *out) {
+#pragma omp parallel for schedule(static)
+    for (long o = 0; o < (long)out_f; o++)
+        for (size_t r = 0; r < m; r++) {
+            double acc = 0.0;
+            for (size_t i = 0; i < in_f; i++)
+                acc += (double)x[r * in_f + i] * (double)w[(size_t)o * in_f + i];
+            out[r * out_f + (size_t)o] = (float)acc;
+        }
+}
+
+/* ───────────────────────────── Op::MoeFfn ───────────────────────────── */
+
+/* crates/infr-cpu/src/moe.rs:42-53 (restricted to the dtypes this restatement decodes). */
+int orc_expert_acts_kind(int dtype, size_t in_f, int int8_ok) {
+    if (int8_ok && (dtype == ORC_Q4_K || dtype == ORC_Q6_K || dtype == ORC_Q8_0) && in_f % 256 == 0)
+        return ORC_ACTS_SUPER;
+    if (int8_ok && dtype == ORC_Q8_0 && in_f % 32 == 0) return ORC_ACTS_BLK32;
+    return ORC_ACTS_RAW;
+}
+
+/* One expert bank applied to `count` activation rows: out_t[o*count + i], o-major
+ * (crates/infr-cpu/src/moe.rs:66-175). Super: per-256 int8 activations through the batch kernels
+ * (bit-identical to the single-row kernels); Raw: weight row decoded once, f32 dot(). */
+static int expert_gemm(const uint8_t *wbytes, size_t wlen, int dt, size_t in_f, size_t out_f,
+                       int kind, const float *xin, size_t count, float *out_t) {
+    size_t bpr = wlen / out_f;
+    if (kind == ORC_ACTS_SUPER) {
+        acts_t a;
+        acts_build(dt, xin, count, in_f, &a);
+        for (size_t o = 0; o < out_f; o++)
+            for (size_t i = 0; i < count; i++)
+                out_t[o * count + i] = row_dot(dt, wbytes + o * bpr, &a, i, in_f, NULL, NULL);
+        acts_free(&a);
+        return 0;
+    }
+    if (kind == ORC_ACTS_RAW) {
+        float *wf = (float *)malloc(sizeof(float) * in_f);
+        for (size_t o = 0; o < out_f; o++) {
+            if (orc_dequant_block(dt, wbytes + o * bpr, bpr, wf) != 0) {
+                free(wf);
+                return -1;
+            }
+            for (size_t i = 0; i < count; i++)
+                out_t[o * count + i] = orc_dot(wf, xin + i * in_f, in_f);
+        }
+        free(wf);
+        return 0;
+    }
+    return -1; /* Blk32 (Q8_0 with in_f % 256 != 0) is not restated */
+}
+
+int orc_moe_ffn(const orc_moe_params *p, const float *x, const float *router_x,
+                const uint8_t *router, size_t router_bytes, const uint8_t *gate, size_t gate_bytes,
+                const uint8_t *up, size_t up_bytes, const uint8_t *down, size_t down_bytes,
+                float *y, int32_t *sel_idx, float *sel_w, int threads) {
+    size_t ne = p->ne, n_expert = p->n_expert, n_used = p->n_used, nffx = p->n_ff_exp;
+    size_t rows = p->rows;
+    if (!ne || !n_expert || !n_used || !nffx || !rows || n_used > n_expert) return -2;
+#ifdef _OPENMP
+    int nt = threads > 0 ? threads : omp_get_max_threads();
+#else
+    int nt = 1;
+    (void)threads;
+#endif
+    (void)nt;
+    size_t gst = gate_bytes / n_expert, ust = up_bytes / n_expert, dst_ = down_bytes / n_expert;
+    /* lib.rs:2359 */
+    int int8_ok = rows >= 2 && !p->reference_mode;
+    int rc = 0;
+
+    /* Router GEMM over all rows (lib.rs:2364-2396). Its activations are router_x. */
+    float *lt = (float *)malloc(sizeof(float) * n_expert * rows);
+    int r_kind = orc_expert_acts_kind(p->router_dtype, ne, int8_ok);
+    if (expert_gemm(router, router_bytes, p->router_dtype, ne, n_expert, r_kind, router_x, rows, lt)) {
+        free(lt);
+        return -1;
+    }
+
+    /* Per-row softmax + stable top-k + renormalised weights (lib.rs:2421-2543). */
+    size_t *idx = (size_t *)malloc(sizeof(size_t) * rows * n_used);
+    float *wts = (float *)malloc(sizeof(float) * rows * n_used);
+    float *probs = (float *)malloc(sizeof(float) * n_expert);
+    char *taken = (char *)malloc(n_expert);
+    for (size_t r = 0; r < rows; r++) {
+        float maxl = -INFINITY;
+        for (size_t e = 0; e < n_expert; e++) {
+            float v = lt[e * rows + r];
+            maxl = v > maxl ? v : maxl;
+        }
+        float psum = 0.0f;
+        for (size_t e = 0; e < n_expert; e++) {
+            probs[e] = expf(lt[e * rows + r] - maxl);
+        }
+        for (size_t e = 0; e < n_expert; e++) psum += probs[e];
+        for (size_t e = 0; e < n_expert; e++) probs[e] /= psum;
+        /* stable descending sort, truncated: ties keep the lower expert index first */
+        memset(taken, 0, n_expert);
+        for (size_t k = 0; k < n_used; k++) {
+            size_t best = n_expert;
+            for (size_t e = 0; e < n_expert; e++) {
+                if (taken[e]) continue;
+                if (best == n_expert || probs[e] > probs[best]) best = e;
+            }
+            taken[best] = 1;
+            idx[r * n_used + k] = best;
+        }
+        float wsum = 0.0f;
+        for (size_t k = 0; k < n_used; k++) wsum += probs[idx[r * n_used + k]];
+        wsum = wsum > 1e-20f ? wsum : 1e-20f;
+        for (size_t k = 0; k < n_used; k++) {
+            wts[r * n_used + k] = probs[idx[r * n_used + k]] / wsum * p->scale;
+            if (sel_idx) sel_idx[r * n_used + k] = (int32_t)idx[r * n_used + k];
+            if (sel_w) sel_w[r * n_used + k] = wts[r * n_used + k];
+        }
+    }
+    free(probs);
+    free(taken);
+    free(lt);
+
+    /* Buckets: (row -> expert) pairs grouped by expert, rows ascending inside a bucket
+     * (lib.rs:2554-2587). */
+    size_t n_pairs = rows * n_used;
+    size_t *pair_row = (size_t *)malloc(sizeof(size_t) * n_pairs);
+    size_t *slot_pair = (size_t *)malloc(sizeof(size_t) * n_pairs); /* [r][rank] */
+    size_t *bucket_e = (size_t *)malloc(sizeof(size_t) * n_expert);
+    size_t *bucket_p0 = (size_t *)malloc(sizeof(size_t) * (n_expert + 1));
+    size_t n_buckets = 0, np = 0;
+    for (size_t e = 0; e < n_expert; e++) {
+        size_t p0 = np;
+        for (size_t r = 0; r < rows; r++)
+            for (size_t k = 0; k < n_used; k++)
+                if (idx[r * n_used + k] == e) {
+                    slot_pair[r * n_used + k] = np;
+                    pair_row[np++] = r;
+                }
+        if (np > p0) {
+            bucket_e[n_buckets] = e;
+            bucket_p0[n_buckets] = p0;
+            n_buckets++;
+        }
+    }
+    bucket_p0[n_buckets] = np;
+
+    int g_kind = orc_expert_acts_kind(p->gate_dtype, ne, int8_ok);
+    int u_kind = orc_expert_acts_kind(p->up_dtype, ne, int8_ok);
+    int d_kind = orc_expert_acts_kind(p->down_dtype, nffx, int8_ok);
+    float *y_pairs = (float *)calloc(n_pairs * ne, sizeof(float));
+
+    /* Stages A-D per bucket (lib.rs:2685-2946). The reference quantizes each distinct row once
+     * and clones it per pair; quantizing the pair's copy of the same row gives the same bytes. */
+#pragma omp parallel for schedule(dynamic, 1) num_threads(nt)
+    for (long b = 0; b < (long)n_buckets; b++) {
+        size_t e = bucket_e[b], p0 = bucket_p0[b], count = bucket_p0[b + 1] - p0;
+        float *xin = (float *)malloc(sizeof(float) * count * ne);
+        for (size_t i = 0; i < count; i++)
+            memcpy(xin + i * ne, x + pair_row[p0 + i] * ne, sizeof(float) * ne);
+        float *gt = (float *)malloc(sizeof(float) * nffx * count);
+        float *ut = (float *)malloc(sizeof(float) * nffx * count);
+        float *act = (float *)malloc(sizeof(float) * count * nffx);
+        float *dt_ = (float *)malloc(sizeof(float) * ne * count);
+        int e1 = expert_gemm(gate + e * gst, gst, p->gate_dtype, ne, nffx, g_kind, xin, count, gt);
+        int e2 = expert_gemm(up + e * ust, ust, p->up_dtype, ne, nffx, u_kind, xin, count, ut);
+        /* Stage C (lib.rs:2824-2892): gated_act_fn(Silu, None, 1.0*g, 1.0*u) */
+        for (size_t i = 0; i < count; i++)
+            for (size_t f = 0; f < nffx; f++)
+                act[i * nffx + f] = orc_silu(gt[f * count + i]) * ut[f * count + i];
+        int e3 = expert_gemm(down + e * dst_, dst_, p->down_dtype, nffx, ne, d_kind, act, count, dt_);
+        if (e1 || e2 || e3) {
+#pragma omp atomic write
+            rc = -1;
+        }
+        for (size_t i = 0; i < count; i++)
+            for (size_t d = 0; d < ne; d++) y_pairs[(p0 + i) * ne + d] = dt_[d * count + i];
+        free(xin);
+        free(gt);
+        free(ut);
+        free(act);
+        free(dt_);
+    }
+
+    /* Stage E (lib.rs:2967-2983): rank order, `*o += w_e * yv` (separate multiply and add). */
+    for (size_t r = 0; r < rows; r++) {
+        float *orow = y + r * ne;
+        for (size_t d = 0; d < ne; d++) orow[d] = 0.0f;
+        for (size_t k = 0; k < n_used; k++) {
+            float w_e = wts[r * n_used + k];
+            const float *yp = y_pairs + slot_pair[r * n_used + k] * ne;
+            for (size_t d = 0; d < ne; d++) orow[d] += w_e * yp[d];
+        }
+    }
+    free(y_pairs);
+    free(pair_row);
+    free(slot_pair);
+    free(bucket_e);
+    free(bucket_p0);
+    free(idx);
+    free(wts);
+    return rc;
+}
+
+/* ───────────────────────────── test-input recipes ───────────────────────────── */
+
+/* crates/infr-testkit/src/lib.rs:49-56 */
+void orc_lcg_bytes(uint32_t seed, size_t n, uint8_t *out) {
+    for (size_t i = 0; i < n; i++) {
+        seed = seed * 1664525u + 1013904223u;
+        out[i] = (uint8_t)(seed >> 16);
+    }
+}
+
+/* crates/infr-testkit/src/lib.rs:60-64 */
+void orc_gen_f32(size_t n, size_t salt, float *out) {
+    for (size_t i = 0; i < n; i++) out[i] = ((float)((i * 13 + salt) % 29) - 14.0f) * 0.05f;
+}
+
+static void put_f16(uint8_t *b, float v) {
+    uint16_t h = orc_f32_to_f16_bits(v);
+    b[0] = (uint8_t)(h & 0xFF);
+    b[1] = (uint8_t)(h >> 8);
+}
+
+/* crates/infr-testkit/src/lib.rs:73-93 (synth_scales), :106-123 (synth_weight): LCG payload per
+ * block seeded `seed ^ b`, then the f16 scale slots overwritten. Slot offsets from
+ * crates/infr-core/src/decode_spec.rs:319-358: Q8_0 d@0; Q4K d@0 dmin@2; Q6K d@208; Q2_0 d@0. */
+size_t orc_synth_weight(int dtype, size_t n_elem, uint32_t seed, uint8_t *out) {
+    int qpb, bpb;
+    if (!orc_block_layout(dtype, &qpb, &bpb) || dtype == ORC_F32 || dtype == ORC_F16) return 0;
+    if (n_elem % (size_t)qpb != 0) return 0;
+    size_t nblk = n_elem / (size_t)qpb;
+    for (size_t b = 0; b < nblk; b++) {
+        uint8_t *blk = out + b * (size_t)bpb;
+        orc_lcg_bytes(seed ^ (uint32_t)b, (size_t)bpb, blk);
+        switch (dtype) {
+        case ORC_Q8_0: put_f16(blk, 0.01f); break;
+        case ORC_Q4_K:
+            put_f16(blk, 0.05f);
+            put_f16(blk + 2, 0.10f);
+            break;
+        case ORC_Q6_K: put_f16(blk + 208, 0.03f); break;
+        case ORC_Q2_0: put_f16(blk, 0.05f); break;
+        }
+    }
+    return nblk * (size_t)bpb;
+}
+
+/* crates/infr-cpu/src/kernels.rs:6611-6624 */
+static uint64_t lcg64(uint64_t *s) {
+    *s = *s * 6364136223846793005ull + 1442695040888963407ull;
+    return *s;
+}
+void orc_det_bytes(size_t n, uint64_t seed, uint8_t *out) {
+    for (size_t i = 0; i < n; i++) out[i] = (uint8_t)(lcg64(&seed) >> 33);
+}
+void orc_det_x(size_t n, uint64_t seed, float *out) {
+    for (size_t i = 0; i < n; i++)
+        out[i] = ((float)(lcg64(&seed) >> 40) / (float)(1ull << 24)) * 2.0f - 1.0f;
+}

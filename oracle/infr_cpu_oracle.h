@@ -1,0 +1,158 @@
+/*
+ * CPU oracle for the quantized-matmul path of kryptic-sh/infr's `infr-cpu` backend.
+ *
+ * THIS IS TEST INFRASTRUCTURE, NOT PRODUCT CODE. It is a plain-C restatement of the reference's
+ * scalar kernels, written from the Rust source text (the reference cannot be compiled where this
+ * is built: no Rust toolchain). Only tests, the smoke check and the benchmark's CPU-baseline leg
+ * may link or load it; the shipped GPU library never does.
+ *
+ * Every function names the reference file:line it follows (paths relative to the reference
+ * checkout). All float arithmetic must be compiled with -ffp-contract=off: Rust never fuses
+ * a*b+c unless `mul_add` is written, and the places that do use `mul_add` call fmaf() here.
+ *
+ * Pinning status (what independent evidence each function is checked against lives in
+ * tests/test_oracle_*.py):
+ *   orc_rdf16 / orc_f32_to_f16   exhaustive round trip over all 65,536 f16 values + numpy float16
+ *   orc_k4                        hand-derived split-bit vector, independent numpy restatement
+ *   orc_dequant_block             reference's q2_0_single_block known answer; hand-derived
+ *                                 all-2.0 blocks; independent byte-at-a-time numpy decoders
+ *   orc_quantize_q8 / _q8_32      hand-derived tie vector (half away from zero), zero block,
+ *                                 one-hot, bsums identities, reconstruction error <= d/2
+ *   orc_vec_dot_*                 hand-derived 65024 vectors; brute-force int64 dots;
+ *                                 dot(dequant(w), dequant(q8)) at the reference's own 1e-3
+ *   orc_linear                    batch == single bit-identical; f64 oracle at the reference's 2e-2;
+ *                                 reference mode at 1e-5
+ *   orc_moe_ffn                   textbook f32 MoE (restated from the reference's moe_ref test helper)
+ *                                 at the reference's 1e-4; routing invariants
+ *   Not pinnable without the Rust binary (parity unpinned): the exact f32 bit pattern the reference
+ *   emits on a given host ISA for Q8_0 (its AVX-512 tier pairs blocks) and libm-dependent expf
+ *   bits in the MoE router/SiLU; both are immaterial at the 1e-4 gate.
+ */
+#ifndef INFR_CPU_ORACLE_H
+#define INFR_CPU_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* GGML type ids (crates/infr-gguf/src/lib.rs:330-354). */
+enum {
+    ORC_F32 = 0,
+    ORC_F16 = 1,
+    ORC_Q8_0 = 8,
+    ORC_Q4_K = 12,
+    ORC_Q6_K = 14,
+    ORC_Q2_0 = 42
+};
+
+/* Activation kinds chosen by the MoE dispatch (crates/infr-cpu/src/moe.rs:32-53). */
+enum { ORC_ACTS_SUPER = 0, ORC_ACTS_BLK32 = 1, ORC_ACTS_RAW = 2 };
+
+/* crates/infr-core/src/decode_spec.rs:319-358 — (elements, bytes) per block; 0 on unknown dtype. */
+int orc_block_layout(int dtype, int *elems, int *bytes);
+
+/* crates/infr-gguf/src/dequant.rs:68-70 (half::f16::to_f32, exact widening). */
+float orc_rdf16(const uint8_t *b);
+float orc_f16_bits_to_f32(uint16_t h);
+/* half::f16::from_f32 — IEEE round-to-nearest-even narrowing (used by the test synthesizers,
+ * crates/infr-core/src/decode_spec.rs:187-190). */
+uint16_t orc_f32_to_f16_bits(float f);
+
+/* crates/infr-gguf/src/dequant.rs:73-83 */
+void orc_k4(int j, const uint8_t *q, uint32_t *sc, uint32_t *m);
+
+/* crates/infr-gguf/src/dequant.rs:11-51 (affine: sc*code + mn, two roundings), :998-1018 (Q2_0).
+ * `out` holds nbytes/block_bytes*block_elems floats. Returns 0, or -1 on unsupported dtype. */
+int orc_dequant_block(int dtype, const uint8_t *bytes, size_t nbytes, float *out);
+
+/* crates/infr-cpu/src/quant.rs:27-58. nb = len/256 blocks (a shorter tail is dropped).
+ * qs[nb*256], d[nb], bsums[nb*8], bsums16[nb*16] (bsums16 may be NULL). */
+void orc_quantize_q8(const float *x, size_t len, int8_t *qs, float *d, int32_t *bsums,
+                     int32_t *bsums16);
+/* crates/infr-cpu/src/quant.rs:97-117. nb = len/32. qs[nb*32], d[nb], bsum[nb]. */
+void orc_quantize_q8_32(const float *x, size_t len, int8_t *qs, float *d, int32_t *bsum);
+
+/* Scalar single-row dots. The optional int-stage outputs receive the per-block integers the f32
+ * epilogue consumes (NULL to skip).
+ * Q4_K: crates/infr-cpu/src/kernels.rs:151-184 — sd[nb], sm[nb].
+ * Q6_K: kernels.rs:487-526 — isum[nb].
+ * Q8_0: kernels.rs:1170-1187 — iprod[in_f/32].
+ * Q2_0: kernels.rs:5641-5668 — iprod[in_f/32] (codes 0..3, before the -bsum correction). */
+float orc_vec_dot_q4k(const uint8_t *row, const int8_t *qs, const float *d, const int32_t *bsums,
+                      size_t in_f, int32_t *sd_out, int32_t *sm_out);
+float orc_vec_dot_q6k(const uint8_t *row, const int8_t *qs, const float *d, size_t in_f,
+                      int32_t *isum_out);
+float orc_vec_dot_q8_0(const uint8_t *row, const int8_t *qs, const float *d, size_t in_f,
+                       int32_t *iprod_out);
+float orc_vec_dot_q2_0(const uint8_t *row, const int8_t *qs, const float *d, const int32_t *bsum,
+                       size_t in_f, int32_t *iprod_out);
+
+/* crates/infr-cpu/src/kernels.rs:6557-6573 — 8 FMA accumulators, lanes summed in order, FMA tail. */
+float orc_dot(const float *a, const float *b, size_t n);
+/* kernels.rs:6578-6597 — act 0 = SiLU; gated_act_fn with clamp None. */
+float orc_silu(float g);
+
+/* crates/infr-cpu/src/lib.rs:985-1492 — the Op::Linear arm for Q4_K/Q6_K/Q8_0/Q2_0/F32 weights.
+ *   w/wbytes: the whole bound weight buffer; w_numel: its declared element count;
+ *   w_off: element offset of the first row (must be a multiple of in_f);
+ *   x[m*in_f] f32; y[m*out_f] f32 row-major.
+ *   reference_mode != 0 takes the exact branch (lib.rs:1015-1031): decode row to f32, plain dot.
+ *   threads <= 0: all OpenMP threads.
+ * Returns 0; -1 unsupported dtype/shape (the reference would take a fallback the restatement
+ * does not carry); -2 bad arguments. */
+int orc_linear(int dtype, const uint8_t *w, size_t wbytes, size_t w_numel, size_t w_off,
+               const float *x, float *y, size_t m, size_t in_f, size_t out_f, int reference_mode,
+               int threads);
+
+/* Per-block integer stages of the production path for every (row r, output o), laid out
+ * [m][out_f][blocks]: Q4_K -> a=sd, b=sm (blocks=in_f/256); Q6_K -> a=isum; Q8_0/Q2_0 -> a=iprod
+ * (blocks=in_f/32). b may be NULL except for Q4_K. */
+int orc_linear_int_stages(int dtype, const uint8_t *w, size_t wbytes, size_t w_numel, size_t w_off,
+                          const float *x, size_t m, size_t in_f, size_t out_f, int32_t *a,
+                          int32_t *b);
+
+/* f64-accumulated reference GEMM over a decoded f32 weight (crates/infr-testkit/src/lib.rs:150-163). */
+void orc_ref_linear_f64(const float *x, const float *w, size_t m, size_t in_f, size_t out_f,
+                        float *out);
+
+/* crates/infr-cpu/src/moe.rs:42-53 */
+int orc_expert_acts_kind(int dtype, size_t in_f, int int8_ok);
+
+/* Op::MoeFfn as qwen3moe builds it (crates/infr-llama/src/seam/runner.rs:3971-3997): softmax
+ * gating, norm_w, weight on the output side, split gate/up banks, SiLU, no clamp/bias/groups. */
+typedef struct {
+    uint32_t ne, n_expert, n_used, n_ff_exp, rows;
+    float scale;
+    int router_dtype, gate_dtype, up_dtype, down_dtype;
+    int reference_mode;
+} orc_moe_params;
+
+/* crates/infr-cpu/src/lib.rs:2264-2984. x, router_x: [rows, ne] f32. Banks: expert e is the e-th
+ * equal byte slice. y[rows*ne]. sel_idx/sel_w (optional, [rows*n_used]) receive the routing
+ * (descending-probability order). Returns 0 or negative on unsupported input. */
+int orc_moe_ffn(const orc_moe_params *p, const float *x, const float *router_x,
+                const uint8_t *router, size_t router_bytes, const uint8_t *gate, size_t gate_bytes,
+                const uint8_t *up, size_t up_bytes, const uint8_t *down, size_t down_bytes,
+                float *y, int32_t *sel_idx, float *sel_w, int threads);
+
+/* Test-input recipes the reference's own tests use (inputs only; it stores no expected outputs).
+ * crates/infr-testkit/src/lib.rs:49-56 */
+void orc_lcg_bytes(uint32_t seed, size_t n, uint8_t *out);
+/* crates/infr-testkit/src/lib.rs:60-64 */
+void orc_gen_f32(size_t n, size_t salt, float *out);
+/* crates/infr-testkit/src/lib.rs:73-93,106-123 + decode_spec.rs:173-190 (write_scales, f16 slots).
+ * Returns bytes written or 0 on unsupported dtype / ragged n_elem. */
+size_t orc_synth_weight(int dtype, size_t n_elem, uint32_t seed, uint8_t *out);
+/* crates/infr-cpu/src/kernels.rs:6611-6624 (kernel_tests::det_bytes / det_x). */
+void orc_det_bytes(size_t n, uint64_t seed, uint8_t *out);
+void orc_det_x(size_t n, uint64_t seed, float *out);
+
+int orc_max_threads(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,106 @@
+"""GPU parity of Op::Linear against the CPU oracle, through the C ABI.
+
+Bars: activation quantization and per-block integer stages bit-exact; Q4_K / Q6_K decode outputs
+bit-identical to the oracle (same per-block expression, same accumulation order); Q8_0 / Q2_0 and
+every m > 1 output within rel-L2 <= 1e-4 and max-abs <= 1e-3 * max|y|.
+"""
+import numpy as np
+import pytest
+
+from infr_amd import DType, synth_normal_f32, synth_weight
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+REL_L2 = 1e-4
+MAX_ABS = 1e-3
+
+
+def gate(y, want):
+    y, want = np.asarray(y, np.float64).ravel(), np.asarray(want, np.float64).ravel()
+    assert np.abs(want).max() > 1e-3, "vacuous case: oracle output is all zero"
+    rel = np.linalg.norm(y - want) / np.linalg.norm(want)
+    mx = np.abs(y - want).max() / np.abs(want).max()
+    assert rel <= REL_L2 and mx <= MAX_ABS, f"rel-L2 {rel:.3e} max-abs/|y|inf {mx:.3e}"
+    return rel, mx
+
+
+def run_linear(be, dtype, w, x, m, in_f, out_f, w_off=0, w_numel=None):
+    wb, xb = be.upload_new(w), be.upload_new(x)
+    yb = be.alloc(m * out_f * 4)
+    be.linear(dtype, wb, xb, yb, m, in_f, out_f, w_numel=w_numel, w_off=w_off)
+    return be.download(yb, np.empty((m, out_f), np.float32))
+
+
+@pytest.mark.parametrize("m,k", [(1, 256), (1, 4096), (3, 768), (8, 12288)])
+def test_quantize_q8_bit_exact(be, m, k):
+    x = synth_normal_f32(11 + k, m * k)
+    x[:7] = [0.5, 1.5, 2.5, -0.5, -1.5, 127.0, 0.0]  # exact ties: half away from zero
+    if m > 1:
+        x[k:2 * k] = 0.0  # an all-zero row: d = 0, id = 0
+    qs, d, bs, bs16 = be.quantize_q8(be.upload_new(x), m, k)
+    for r in range(m):
+        o = orc.quantize_q8(x[r * k:(r + 1) * k])
+        assert np.array_equal(qs[r], o.qs)
+        assert np.array_equal(d[r].view(np.uint32), o.d.view(np.uint32))
+        assert np.array_equal(bs[r], o.bsums)
+        assert np.array_equal(bs16[r], o.bsums16)
+
+
+@pytest.mark.parametrize("m,k", [(1, 64), (1, 4096), (5, 96), (2, 12288)])
+def test_quantize_q8_32_bit_exact(be, m, k):
+    x = synth_normal_f32(5 + k, m * k)
+    x[:6] = [0.5, 1.5, 2.5, -0.5, -1.5, 127.0]
+    qs, d, bs = be.quantize_q8_32(be.upload_new(x), m, k)
+    for r in range(m):
+        o = orc.quantize_q8_32(x[r * k:(r + 1) * k])
+        assert np.array_equal(qs[r], o.qs)
+        assert np.array_equal(d[r].view(np.uint32), o.d.view(np.uint32))
+        assert np.array_equal(bs[r], o.bsum)
+
+
+DECODE_SHAPES = [(256, 8), (768, 37), (4096, 1024), (12288, 512), (2048, 100), (5120, 64)]
+
+
+@pytest.mark.parametrize("dtype", [DType.Q4K, DType.Q6K, DType.Q8_0, DType.Q2_0])
+@pytest.mark.parametrize("in_f,out_f", DECODE_SHAPES)
+def test_decode_gemv_vs_oracle(be, dtype, in_f, out_f):
+    w = synth_weight(dtype, 100 + in_f, out_f, in_f)
+    x = synth_normal_f32(200 + out_f, in_f)
+    y = run_linear(be, dtype, w, x, 1, in_f, out_f)
+    want = orc.linear(dtype, w, x, 1, in_f, out_f)
+    gate(y, want)
+    if dtype in (DType.Q4K, DType.Q6K):
+        assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), "not bit-identical"
+
+
+@pytest.mark.parametrize("dtype", [DType.Q4K, DType.Q6K, DType.Q8_0, DType.Q2_0])
+def test_decode_int_stages_bit_exact(be, dtype):
+    in_f, out_f = 1024, 24
+    # full-range payload bytes (the reference's synth_weight recipe) stress every code value
+    w = orc.synth_weight(dtype, in_f * out_f, 0x201)
+    x = orc.gen_f32(in_f, 0x201 ^ 0x9E37)
+    a, b = be.linear_int_stages(dtype, be.upload_new(w), be.upload_new(x), 1, in_f, out_f)
+    oa, ob = orc.linear_int_stages(dtype, w, x, 1, in_f, out_f)
+    assert np.array_equal(a, oa)
+    if dtype == DType.Q4K:
+        assert np.array_equal(b, ob)
+
+
+@pytest.mark.parametrize("dtype", [DType.Q4K, DType.Q6K, DType.Q8_0, DType.Q2_0])
+@pytest.mark.parametrize("m", [2, 8])
+def test_small_batch_vs_oracle(be, dtype, m):
+    in_f, out_f = 1024, 96
+    w = synth_weight(dtype, 7, out_f, in_f)
+    x = synth_normal_f32(8, m * in_f)
+    y = run_linear(be, dtype, w, x, m, in_f, out_f)
+    gate(y, orc.linear(dtype, w, x, m, in_f, out_f))
+
+
+def test_w_off_selects_rows_of_a_concatenated_weight(be):
+    in_f, rows = 512, 48
+    w = synth_weight(DType.Q4K, 3, rows, in_f)
+    x = synth_normal_f32(4, in_f)
+    y = run_linear(be, DType.Q4K, w, x, 1, in_f, 16, w_off=16 * in_f, w_numel=rows * in_f)
+    want = orc.linear(DType.Q4K, w, x, 1, in_f, 16, w_numel=rows * in_f, w_off=16 * in_f)
+    assert np.array_equal(y.view(np.uint32), want.view(np.uint32))
