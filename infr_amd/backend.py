@@ -160,6 +160,8 @@ def synth_normal_f32(seed: int, n: int, mean: float = 0.0, sigma: float = 1.0) -
 def synth_weight(dtype: int, seed: int, rows: int, in_f: int, sigma: float = 0.02) -> np.ndarray:
     """N(0, sigma^2) weights [rows, in_f] encoded as raw blocks of ``dtype``."""
     e, b = block_layout(dtype)
+    if rows <= 0 or in_f <= 0 or in_f % e != 0:
+        raise InfrError(Status.Invalid, f"synth_weight: in_f {in_f} is not a whole number of {e}-element blocks")
     out = np.empty(rows * (in_f // e) * b, np.uint8)
     n = load_library().infr_synth_weight(int(dtype), seed, sigma, rows, in_f, out.ctypes.data)
     if n != out.size:

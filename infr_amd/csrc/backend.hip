@@ -6,6 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <atomic>
 #include <cstdio>
 #include <cstring>
@@ -27,6 +28,23 @@ struct infr_hip_plan {
     // decode replay: launch sequence recorded for one set of bound device addresses
     hipGraphExec_t exec = nullptr;
     std::vector<void*> bound;
+    // Launch schedule for the bound addresses: ops ordered by dependency level; the m == 1 ops
+    // of a level that share (dtype, in_f) form one grouped decode launch.
+    struct Step {
+        int level = 0;
+        int op = -1;              // m >= 2: index into ops
+        int dtype = 0;            // decode group
+        size_t in_f = 0;
+        int first = 0, n = 0;     // slice of descs
+        size_t tile_first = 0;    // slice of tiles
+        infr::GemvGroupPlan gp;
+    };
+    std::vector<Step> steps;
+    std::vector<infr::GemvOpDesc> descs;
+    // per-workgroup tile tables of the grouped launches, back to back (tile_first per step)
+    std::vector<infr::GemvTile> tiles;
+    infr::GemvTile* tiles_dev = nullptr;
+    size_t tiles_cap = 0;
 };
 
 struct infr_hip {
@@ -145,6 +163,18 @@ int enqueue_linear(infr_hip_t* be, int dtype, const LinearArgs& la, const float*
         return fail(be, INFR_HIP_ERR_UNSUPPORTED,
                     "linear: no kernel for dtype " + std::to_string(dtype) + " at in_f " +
                         std::to_string(in_f) + ", m " + std::to_string(m));
+    HIP_TRY(be, hipGetLastError());
+    return INFR_HIP_OK;
+}
+
+// One fused decode launch (quantize x in LDS + GEMV) for a single m == 1 Linear.
+int enqueue_gemv_single(infr_hip_t* be, int dtype, size_t in_f, const infr::GemvOpDesc& op) {
+    infr::GemvGroupPlan gp;
+    if (!infr::plan_gemv_group(dtype, in_f, &op, 1, &gp) ||
+        !infr::launch_gemv_fused(dtype, in_f, &op, 1, nullptr, gp, be->stream))
+        return fail(be, INFR_HIP_ERR_UNSUPPORTED,
+                    "linear: no decode kernel for dtype " + std::to_string(dtype) + " at in_f " +
+                        std::to_string(in_f));
     HIP_TRY(be, hipGetLastError());
     return INFR_HIP_OK;
 }
@@ -356,6 +386,12 @@ int infr_hip_linear(infr_hip_t* be, int dtype, const infr_hip_buffer_t* w, size_
     if (int rc = check_linear(be, dtype, w, w_numel, w_off, x, m, in_f, out_f, &la)) return rc;
     if (!dst || dst->len < m * out_f * sizeof(float))
         return fail(be, INFR_HIP_ERR_INVALID, "linear: dst buffer missing or too small");
+    if (m == 1) {
+        // decode: one fused launch (quantize x in LDS + GEMV)
+        const infr::GemvOpDesc op{la.wrows, static_cast<const float*>(x->ptr),
+                                  static_cast<float*>(dst->ptr), la.bpr, (int32_t)out_f};
+        return enqueue_gemv_single(be, dtype, in_f, op);
+    }
     if (int rc = ensure_act(be, m * in_f)) return rc;
     return enqueue_linear(be, dtype, la, static_cast<const float*>(x->ptr),
                           static_cast<float*>(dst->ptr), m, in_f, out_f, infr::IntStages{});
@@ -463,27 +499,119 @@ int infr_hip_compile(infr_hip_t* be, const infr_hip_op_t* ops, size_t n_ops, inf
 
 void infr_hip_plan_free(infr_hip_t* be, infr_hip_plan_t* plan) {
     if (!plan) return;
-    if (plan->exec) {
-        if (be && be->stream) (void)hipStreamSynchronize(be->stream);
-        (void)hipGraphExecDestroy(plan->exec);
-    }
+    if (be && be->stream) (void)hipStreamSynchronize(be->stream);
+    if (plan->exec) (void)hipGraphExecDestroy(plan->exec);
+    if (plan->tiles_dev) (void)hipFree(plan->tiles_dev);
     delete plan;
 }
 
-static int enqueue_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t* const* bindings) {
-    for (const auto& op : plan->ops) {
-        const infr_hip_buffer_t* w = bindings[op.weight];
-        const infr_hip_buffer_t* x = bindings[op.x];
-        infr_hip_buffer_t* dst = bindings[op.dst];
-        LinearArgs la;
-        if (int rc = check_linear(be, op.w_dtype, w, op.w_numel, op.w_off, x, op.m, op.in_f, op.out_f, &la))
+// Orders the plan's ops for the currently bound device addresses. Two ops conflict when one
+// writes memory the other reads or writes (the read/write sets of Op::io, graph.rs:1128); an op's
+// level is one more than the highest level among earlier conflicting ops, so ops of one level are
+// mutually independent and running levels in ascending order preserves every dependency.
+static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t* const* bindings) {
+    const size_t n = plan->ops.size();
+    struct Span { const uint8_t* lo; const uint8_t* hi; };
+    auto span = [](const infr_hip_buffer_t* b, size_t bytes) {
+        const uint8_t* p = static_cast<const uint8_t*>(b->ptr);
+        return Span{p, p + bytes};
+    };
+    auto overlap = [](const Span& a, const Span& b) { return a.lo < b.hi && b.lo < a.hi; };
+    std::vector<Span> rd(n), wr(n), wt(n);
+    std::vector<int> level(n, 0);
+    std::vector<LinearArgs> la(n);
+    int max_level = 0;
+    for (size_t i = 0; i < n; ++i) {
+        const auto& op = plan->ops[i];
+        if (int rc = check_linear(be, op.w_dtype, bindings[op.weight], op.w_numel, op.w_off,
+                                  bindings[op.x], op.m, op.in_f, op.out_f, &la[i]))
             return rc;
-        if (!dst || dst->len < (size_t)op.m * op.out_f * sizeof(float))
+        const size_t ybytes = (size_t)op.m * op.out_f * sizeof(float);
+        if (!bindings[op.dst] || bindings[op.dst]->len < ybytes)
             return fail(be, INFR_HIP_ERR_INVALID, "execute: dst buffer missing or too small");
-        if (int rc = enqueue_linear(be, op.w_dtype, la, static_cast<const float*>(x->ptr),
-                                    static_cast<float*>(dst->ptr), op.m, op.in_f, op.out_f,
-                                    infr::IntStages{}))
-            return rc;
+        rd[i] = span(bindings[op.x], (size_t)op.m * op.in_f * sizeof(float));
+        wr[i] = span(bindings[op.dst], ybytes);
+        wt[i] = Span{la[i].wrows, la[i].wrows + (size_t)op.out_f * la[i].bpr};
+        for (size_t j = 0; j < i; ++j)
+            if (overlap(wr[j], rd[i]) || overlap(wr[j], wr[i]) || overlap(rd[j], wr[i]) ||
+                overlap(wr[j], wt[i]) || overlap(wt[j], wr[i]))
+                level[i] = std::max(level[i], level[j] + 1);
+        max_level = std::max(max_level, level[i]);
+    }
+    plan->steps.clear();
+    plan->descs.clear();
+    plan->tiles.clear();
+    for (int lv = 0; lv <= max_level; ++lv) {
+        std::vector<char> taken(n, 0);
+        for (size_t i = 0; i < n; ++i) {
+            if (level[i] != lv || taken[i]) continue;
+            const auto& op = plan->ops[i];
+            infr_hip_plan::Step st;
+            st.level = lv;
+            if (op.m != 1) {
+                st.op = (int)i;
+                taken[i] = 1;
+                plan->steps.push_back(st);
+                continue;
+            }
+            st.dtype = op.w_dtype;
+            st.in_f = op.in_f;
+            st.first = (int)plan->descs.size();
+            for (size_t k = i; k < n; ++k) {
+                const auto& o2 = plan->ops[k];
+                if (level[k] != lv || taken[k] || o2.m != 1 || o2.w_dtype != op.w_dtype || o2.in_f != op.in_f)
+                    continue;
+                taken[k] = 1;
+                plan->descs.push_back(infr::GemvOpDesc{
+                    la[k].wrows, static_cast<const float*>(bindings[o2.x]->ptr),
+                    static_cast<float*>(bindings[o2.dst]->ptr), la[k].bpr, (int32_t)o2.out_f});
+            }
+            st.n = (int)plan->descs.size() - st.first;
+            if (!infr::plan_gemv_group(st.dtype, st.in_f, &plan->descs[st.first], st.n, &st.gp))
+                return fail(be, INFR_HIP_ERR_UNSUPPORTED,
+                            "execute: no decode kernel for dtype " + std::to_string(st.dtype) +
+                                " at in_f " + std::to_string(st.in_f));
+            st.tile_first = plan->tiles.size();
+            plan->tiles.resize(st.tile_first + (size_t)st.gp.total_wgs);
+            infr::fill_gemv_tiles(&plan->descs[st.first], st.n, st.gp, &plan->tiles[st.tile_first]);
+            plan->steps.push_back(st);
+        }
+    }
+    if (!plan->tiles.empty()) {
+        if (plan->tiles.size() > plan->tiles_cap) {
+            if (plan->tiles_dev) (void)hipFree(plan->tiles_dev);
+            plan->tiles_dev = nullptr;
+            plan->tiles_cap = 0;
+            HIP_TRY(be, hipMalloc((void**)&plan->tiles_dev, sizeof(infr::GemvTile) * plan->tiles.size()));
+            plan->tiles_cap = plan->tiles.size();
+        }
+        HIP_TRY(be, hipMemcpyAsync(plan->tiles_dev, plan->tiles.data(),
+                                   sizeof(infr::GemvTile) * plan->tiles.size(),
+                                   hipMemcpyHostToDevice, be->stream));
+        HIP_TRY(be, hipStreamSynchronize(be->stream));
+    }
+    return INFR_HIP_OK;
+}
+
+// Enqueues the scheduled launches (this is what gets recorded for replay: kernels only).
+static int enqueue_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t* const* bindings) {
+    for (const auto& st : plan->steps) {
+        if (st.op >= 0) {
+            const auto& op = plan->ops[st.op];
+            LinearArgs la;
+            if (int rc = check_linear(be, op.w_dtype, bindings[op.weight], op.w_numel, op.w_off,
+                                      bindings[op.x], op.m, op.in_f, op.out_f, &la))
+                return rc;
+            if (int rc = enqueue_linear(be, op.w_dtype, la, static_cast<const float*>(bindings[op.x]->ptr),
+                                        static_cast<float*>(bindings[op.dst]->ptr), op.m, op.in_f,
+                                        op.out_f, infr::IntStages{}))
+                return rc;
+        } else {
+            if (!infr::launch_gemv_fused(st.dtype, st.in_f, &plan->descs[st.first], st.n,
+                                         plan->tiles_dev + st.tile_first, st.gp, be->stream))
+                return fail(be, INFR_HIP_ERR_UNSUPPORTED, "execute: decode launch rejected");
+            HIP_TRY(be, hipGetLastError());
+        }
     }
     return INFR_HIP_OK;
 }
@@ -492,7 +620,8 @@ int infr_hip_execute(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t* c
                      size_t n_bindings) {
     if (!be || !plan || (!bindings && n_bindings)) return fail(be, INFR_HIP_ERR_INVALID, "execute: null argument");
     if (int rc = check_latch(be)) return rc;
-    if (!plan->ops.empty() && plan->max_tensor >= n_bindings)
+    if (plan->ops.empty()) return INFR_HIP_OK;
+    if (plan->max_tensor >= n_bindings)
         return fail(be, INFR_HIP_ERR_INVALID, "execute: a tensor id has no binding slot");
     // Replay when every bound device address is what the recording saw.
     std::vector<void*> now(n_bindings);
@@ -506,15 +635,11 @@ int infr_hip_execute(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t* c
         (void)hipGraphExecDestroy(plan->exec);
         plan->exec = nullptr;
     }
-    // Validate everything before recording so a bad binding cannot leave a capture open.
-    for (const auto& op : plan->ops) {
-        LinearArgs la;
-        if (int rc = check_linear(be, op.w_dtype, bindings[op.weight], op.w_numel, op.w_off,
-                                  bindings[op.x], op.m, op.in_f, op.out_f, &la))
-            return rc;
-        if (!bindings[op.dst] || bindings[op.dst]->len < (size_t)op.m * op.out_f * sizeof(float))
-            return fail(be, INFR_HIP_ERR_INVALID, "execute: dst buffer missing or too small");
-    }
+    // Validate and schedule before recording so a bad binding cannot leave a capture open.
+    for (const auto& op : plan->ops)
+        if (!bindings[op.weight] || !bindings[op.x] || !bindings[op.dst])
+            return fail(be, INFR_HIP_ERR_INVALID, "execute: unbound tensor");
+    if (int rc = schedule_plan(be, plan, bindings)) return rc;
     hipGraph_t graph = nullptr;
     HIP_TRY(be, hipStreamBeginCapture(be->stream, hipStreamCaptureModeThreadLocal));
     int rc = enqueue_plan(be, plan, bindings);

@@ -1,0 +1,368 @@
+// Per-format lane mappings of the decode GEMV: what a lane loads of a weight row, which
+// activation bytes it keeps in registers, and the per-block integer stage + f32 term.
+// Each format follows infr-cpu's scalar kernel for one block:
+//   Q4_K  crates/infr-cpu/src/kernels.rs:151-184     Q6_K  kernels.rs:487-526
+//   Q8_0  kernels.rs:1170-1187                       Q2_0  kernels.rs:5641-5668
+//
+// Interface of a format policy F (all members static, `t` = wave step, `lane` = 0..63):
+//   kElemsPerStep         K elements one wave step covers
+//   kPer32                activation quantizer: per-32 (true) or per-256 (false)
+//   kOrdered              per-block terms are added in ascending block order (bit-exact with the
+//                         CPU's `sumf +=` chain) instead of a butterfly
+//   units(in_f)           number of lane work units in a row (blocks for Q4_K/Q6_K ...)
+//   Row / Acts            registers for one step of a weight row / of the activation
+//   valid(t, lane, n)     does this lane have work in step t
+//   load_row, load_acts   fill them (acts from any address space: global or LDS pointers)
+//   term(...)             exact integer stage + f32 term of the lane's unit; writes stage outputs
+#pragma once
+
+#include "device_common.hpp"
+
+namespace infr {
+
+// Pointers to a quantized activation row (global memory or LDS).
+struct ActPtrs {
+    const int8_t* qs;
+    const float* d;
+    const int32_t* bsums;    // per 32
+    const int32_t* bsums16;  // per 16 (per-256 quantizer only)
+};
+
+struct StagePtrs {
+    int32_t* a;
+    int32_t* b;
+};
+
+// ───────────────────────────────────── Q4_K ─────────────────────────────────────
+// Lane l: block-in-step q = l/4, nibble pair p = l%4. Pair p's 32 bytes hold sub-block 2p in the
+// low nibbles and 2p+1 in the high nibbles, so `w & 0x0F0F0F0F` / `(w >> 4) & 0x0F0F0F0F` are
+// ready v_dot4 operands against 64 consecutive activation bytes. 16 blocks (4096 weights,
+// 2304 B) per wave step; the quad's partial integers are combined with two DPP adds.
+struct FmtQ4K {
+    static constexpr int kElemsPerStep = 4096;
+    static constexpr bool kPer32 = false;
+    static constexpr bool kOrdered = true;
+    static constexpr int kBlockBytes = 144, kBlockElems = 256;
+    struct Row {
+        v4i hdr, qa, qb;
+    };
+    struct Acts {
+        int xa[16];
+        int bs0, bs1;
+        float dact;
+    };
+    __device__ static int units(int in_f) { return in_f / 256; }
+    __device__ static bool valid(int t, int lane, int n) { return t * 16 + (lane >> 2) < n; }
+    __device__ static void load_row(Row& r, const uint8_t* rowp, int t, int lane, bool ok) {
+        if (ok) {
+            const uint8_t* blk = rowp + (size_t)(t * 16 + (lane >> 2)) * 144;
+            const int p = lane & 3;
+            r.hdr = load16(blk);
+            r.qa = load16(blk + 16 + p * 32);
+            r.qb = load16(blk + 32 + p * 32);
+        } else {
+            r.hdr = r.qa = r.qb = v4i{0, 0, 0, 0};
+        }
+    }
+    __device__ static void load_acts(Acts& a, const ActPtrs& s, int t, int lane, bool ok) {
+        if (ok) {
+            const int b = t * 16 + (lane >> 2), p = lane & 3;
+            const v4i* xp = reinterpret_cast<const v4i*>(s.qs + (size_t)b * 256 + p * 64);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const v4i v = xp[k];
+                a.xa[4 * k + 0] = v.x;
+                a.xa[4 * k + 1] = v.y;
+                a.xa[4 * k + 2] = v.z;
+                a.xa[4 * k + 3] = v.w;
+            }
+            const v2i bs = *reinterpret_cast<const v2i*>(s.bsums + (size_t)b * 8 + 2 * p);
+            a.bs0 = bs.x;
+            a.bs1 = bs.y;
+            a.dact = s.d[b];
+        } else {
+#pragma unroll
+            for (int k = 0; k < 16; ++k) a.xa[k] = 0;
+            a.bs0 = a.bs1 = 0;
+            a.dact = 0.0f;
+        }
+    }
+    // sd/sm are exact per-block integers, identical in the four lanes of a quad.
+    template <bool STAGES>
+    __device__ static float term(const Row& r, const Acts& a, int t, int lane, bool ok,
+                                 const StagePtrs& st, size_t row_units) {
+        const int p = lane & 3;
+        const uint32_t m4 = 0x0F0F0F0Fu;
+        int ip_e = 0, ip_o = 0;
+        const int wq[8] = {r.qa.x, r.qa.y, r.qa.z, r.qa.w, r.qb.x, r.qb.y, r.qb.z, r.qb.w};
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const uint32_t w = (uint32_t)wq[k];
+            ip_e = dot4((int)(w & m4), a.xa[k], ip_e);
+            ip_o = dot4((int)((w >> 4) & m4), a.xa[8 + k], ip_o);
+        }
+        uint32_t sc8[2], mn8[2];
+        k4_all((uint32_t)r.hdr.y, (uint32_t)r.hdr.z, (uint32_t)r.hdr.w, sc8, mn8);
+        const uint32_t scw = (p & 2) ? sc8[1] : sc8[0];
+        const uint32_t mnw = (p & 2) ? mn8[1] : mn8[0];
+        const int sh = (p & 1) * 16;
+        const int sc_e = (scw >> sh) & 0xFF, sc_o = (scw >> (sh + 8)) & 0xFF;
+        const int m_e = (mnw >> sh) & 0xFF, m_o = (mnw >> (sh + 8)) & 0xFF;
+        const int sd = quad_sum(__mul24(sc_e, ip_e) + __mul24(sc_o, ip_o));
+        const int sm = quad_sum(__mul24(m_e, a.bs0) + __mul24(m_o, a.bs1));
+        if (STAGES && ok && p == 0) {
+            st.a[row_units + t * 16 + (lane >> 2)] = sd;
+            st.b[row_units + t * 16 + (lane >> 2)] = sm;
+        }
+        const float d = f16_bits_to_f32((uint32_t)r.hdr.x & 0xFFFFu);
+        const float dmin = f16_bits_to_f32((uint32_t)r.hdr.x >> 16);
+        // sumf += q8.d[b] * (d * sd as f32 - dmin * sm as f32)
+        return a.dact * (d * (float)sd - dmin * (float)sm);
+    }
+};
+
+// ───────────────────────────────────── Q6_K ─────────────────────────────────────
+// Lane l: block-in-step q = l/4, half h = (l%4)/2, c = l%2 selects l in [16c, 16c+16). The lane
+// decodes the four 16-element groups {l, l+32, l+64, l+96} of its half: 64 weights, scale indices
+// h*8 + c + {0,2,4,6}. Codes stay biased (0..63) and the -32 offset is applied through the
+// activation's per-16 sums, exactly the CPU's `sc * (sumi - 32*bsum)`. 16 blocks (3360 B) per
+// wave step. Block stride 210 B is 2 mod 4: loads are 2-byte aligned.
+struct FmtQ6K {
+    static constexpr int kElemsPerStep = 4096;
+    static constexpr bool kPer32 = false;
+    static constexpr bool kOrdered = true;
+    static constexpr int kBlockBytes = 210, kBlockElems = 256;
+    struct Row {
+        v4i qla, qlb, qh;
+        v2i sc;
+        uint32_t d;
+    };
+    struct Acts {
+        int xa[16];
+        int bs16[4];
+        float dact;
+    };
+    __device__ static int units(int in_f) { return in_f / 256; }
+    __device__ static bool valid(int t, int lane, int n) { return t * 16 + (lane >> 2) < n; }
+    __device__ static void load_row(Row& r, const uint8_t* rowp, int t, int lane, bool ok) {
+        if (ok) {
+            const int h = (lane >> 1) & 1, c = lane & 1;
+            const uint8_t* blk = rowp + (size_t)(t * 16 + (lane >> 2)) * 210;
+            r.qla = load16_a2(blk + h * 64 + c * 16);
+            r.qlb = load16_a2(blk + h * 64 + 32 + c * 16);
+            r.qh = load16_a2(blk + 128 + h * 32 + c * 16);
+            __builtin_memcpy(&r.sc, __builtin_assume_aligned(blk + 192 + h * 8, 2), 8);
+            r.d = load_u16(blk + 208);
+        } else {
+            r.qla = r.qlb = r.qh = v4i{0, 0, 0, 0};
+            r.sc = v2i{0, 0};
+            r.d = 0;
+        }
+    }
+    __device__ static void load_acts(Acts& a, const ActPtrs& s, int t, int lane, bool ok) {
+        if (ok) {
+            const int b = t * 16 + (lane >> 2), h = (lane >> 1) & 1, c = lane & 1;
+            const int8_t* xb = s.qs + (size_t)b * 256 + h * 128 + c * 16;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const v4i v = *reinterpret_cast<const v4i*>(xb + 32 * k);
+                a.xa[4 * k + 0] = v.x;
+                a.xa[4 * k + 1] = v.y;
+                a.xa[4 * k + 2] = v.z;
+                a.xa[4 * k + 3] = v.w;
+                a.bs16[k] = s.bsums16[(size_t)b * 16 + h * 8 + c + 2 * k];
+            }
+            a.dact = s.d[b];
+        } else {
+#pragma unroll
+            for (int k = 0; k < 16; ++k) a.xa[k] = 0;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) a.bs16[k] = 0;
+            a.dact = 0.0f;
+        }
+    }
+    template <bool STAGES>
+    __device__ static float term(const Row& r, const Acts& a, int t, int lane, bool ok,
+                                 const StagePtrs& st, size_t row_units) {
+        const int c = lane & 1;
+        const uint32_t m4 = 0x0F0F0F0Fu, m2 = 0x30303030u;
+        const int la[4] = {r.qla.x, r.qla.y, r.qla.z, r.qla.w};
+        const int lb[4] = {r.qlb.x, r.qlb.y, r.qlb.z, r.qlb.w};
+        const int hh[4] = {r.qh.x, r.qh.y, r.qh.z, r.qh.w};
+        int sumi[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t lo = (uint32_t)la[j], hi = (uint32_t)lb[j], h = (uint32_t)hh[j];
+            sumi[0] = dot4((int)((lo & m4) | ((h << 4) & m2)), a.xa[0 + j], sumi[0]);
+            sumi[1] = dot4((int)((hi & m4) | ((h << 2) & m2)), a.xa[4 + j], sumi[1]);
+            sumi[2] = dot4((int)(((lo >> 4) & m4) | (h & m2)), a.xa[8 + j], sumi[2]);
+            sumi[3] = dot4((int)(((hi >> 4) & m4) | ((h >> 2) & m2)), a.xa[12 + j], sumi[3]);
+        }
+        // scales[h*8 + c + 2k]: byte (c + 2k) of the 8 bytes loaded at scales + h*8
+        const uint32_t lo = (uint32_t)r.sc.x >> (8 * c), hi = (uint32_t)r.sc.y >> (8 * c);
+        const int sc0 = (int)(int8_t)(lo & 0xFF), sc1 = (int)(int8_t)((lo >> 16) & 0xFF);
+        const int sc2 = (int)(int8_t)(hi & 0xFF), sc3 = (int)(int8_t)((hi >> 16) & 0xFF);
+        int part = __mul24(sc0, sumi[0] - 32 * a.bs16[0]);
+        part += __mul24(sc1, sumi[1] - 32 * a.bs16[1]);
+        part += __mul24(sc2, sumi[2] - 32 * a.bs16[2]);
+        part += __mul24(sc3, sumi[3] - 32 * a.bs16[3]);
+        const int isum = quad_sum(part);
+        if (STAGES && ok && (lane & 3) == 0) st.a[row_units + t * 16 + (lane >> 2)] = isum;
+        // sumf += d * q8.d[b] * isum as f32
+        return f16_bits_to_f32(r.d) * a.dact * (float)isum;
+    }
+};
+
+// ───────────────────────────────────── Q8_0 ─────────────────────────────────────
+// Lane l owns 32-weight block t*64 + l of the row: 34 B = f16 scale + 32 int8, 2-byte aligned.
+// 64 blocks (2048 weights, 2176 B) per wave step; the activation scale is per 256 (8 lanes).
+struct FmtQ8_0 {
+    static constexpr int kElemsPerStep = 2048;
+    static constexpr bool kPer32 = false;
+    static constexpr bool kOrdered = false;
+    static constexpr int kBlockBytes = 34, kBlockElems = 32;
+    struct Row {
+        v4i qa, qb;
+        uint32_t d;
+    };
+    struct Acts {
+        int xa[8];
+        float dact;
+    };
+    __device__ static int units(int in_f) { return in_f / 32; }
+    __device__ static bool valid(int t, int lane, int n) { return t * 64 + lane < n; }
+    __device__ static void load_row(Row& r, const uint8_t* rowp, int t, int lane, bool ok) {
+        if (ok) {
+            const uint8_t* blk = rowp + (size_t)(t * 64 + lane) * 34;
+            r.d = load_u16(blk);
+            r.qa = load16_a2(blk + 2);
+            r.qb = load16_a2(blk + 18);
+        } else {
+            r.qa = r.qb = v4i{0, 0, 0, 0};
+            r.d = 0;
+        }
+    }
+    __device__ static void load_acts(Acts& a, const ActPtrs& s, int t, int lane, bool ok) {
+        if (ok) {
+            const int wb = t * 64 + lane;
+            const v4i v0 = *reinterpret_cast<const v4i*>(s.qs + (size_t)wb * 32);
+            const v4i v1 = *reinterpret_cast<const v4i*>(s.qs + (size_t)wb * 32 + 16);
+            a.xa[0] = v0.x; a.xa[1] = v0.y; a.xa[2] = v0.z; a.xa[3] = v0.w;
+            a.xa[4] = v1.x; a.xa[5] = v1.y; a.xa[6] = v1.z; a.xa[7] = v1.w;
+            a.dact = s.d[wb >> 3];
+        } else {
+#pragma unroll
+            for (int k = 0; k < 8; ++k) a.xa[k] = 0;
+            a.dact = 0.0f;
+        }
+    }
+    template <bool STAGES>
+    __device__ static float term(const Row& r, const Acts& a, int t, int lane, bool ok,
+                                 const StagePtrs& st, size_t row_units) {
+        int ip = 0;
+        ip = dot4(r.qa.x, a.xa[0], ip);
+        ip = dot4(r.qa.y, a.xa[1], ip);
+        ip = dot4(r.qa.z, a.xa[2], ip);
+        ip = dot4(r.qa.w, a.xa[3], ip);
+        ip = dot4(r.qb.x, a.xa[4], ip);
+        ip = dot4(r.qb.y, a.xa[5], ip);
+        ip = dot4(r.qb.z, a.xa[6], ip);
+        ip = dot4(r.qb.w, a.xa[7], ip);
+        if (STAGES && ok) st.a[row_units + t * 64 + lane] = ip;
+        // sumf += d8 * d_w * iprod as f32
+        return a.dact * f16_bits_to_f32(r.d) * (float)ip;
+    }
+};
+
+// ───────────────────────────────────── Q2_0 ─────────────────────────────────────
+// Lane l owns 64-weight block t*64 + l: 18 B = f16 scale + 16 bytes of 2-bit codes, 2-byte
+// aligned. `(w >> 2s) & 0x03030303` pulls the codes of elements {4i+s} of a 16-element group into
+// the four bytes of a word; the activation bytes are transposed once per wave (v_perm_b32) into
+// that order, so each extracted word is a ready v_dot4 operand. 64 blocks (4096 weights,
+// 1152 B) per wave step. Codes stay 0..3; the -1 offset is applied as `iprod - bsum` like the CPU.
+
+// 4x4 byte transpose: out[s] byte i = in[i] byte s.
+__device__ __forceinline__ void transpose4x4(const int in[4], int out[4]) {
+    // v_perm_b32(hi, lo, sel): result byte k = byte sel[k] of the 8-byte value {hi:lo} (lo = 0..3).
+    const uint32_t a = (uint32_t)in[0], b = (uint32_t)in[1], c = (uint32_t)in[2], d = (uint32_t)in[3];
+    const uint32_t ab_lo = __builtin_amdgcn_perm(b, a, 0x05010400u);  // a0 b0 a1 b1
+    const uint32_t ab_hi = __builtin_amdgcn_perm(b, a, 0x07030602u);  // a2 b2 a3 b3
+    const uint32_t cd_lo = __builtin_amdgcn_perm(d, c, 0x05010400u);  // c0 d0 c1 d1
+    const uint32_t cd_hi = __builtin_amdgcn_perm(d, c, 0x07030602u);  // c2 d2 c3 d3
+    out[0] = (int)__builtin_amdgcn_perm(cd_lo, ab_lo, 0x05040100u);   // a0 b0 c0 d0
+    out[1] = (int)__builtin_amdgcn_perm(cd_lo, ab_lo, 0x07060302u);   // a1 b1 c1 d1
+    out[2] = (int)__builtin_amdgcn_perm(cd_hi, ab_hi, 0x05040100u);   // a2 b2 c2 d2
+    out[3] = (int)__builtin_amdgcn_perm(cd_hi, ab_hi, 0x07060302u);   // a3 b3 c3 d3
+}
+
+struct FmtQ2_0 {
+    static constexpr int kElemsPerStep = 4096;
+    static constexpr bool kPer32 = true;
+    static constexpr bool kOrdered = false;
+    static constexpr int kBlockBytes = 18, kBlockElems = 64;
+    struct Row {
+        v4i codes;
+        uint32_t d;
+    };
+    struct Acts {
+        int xt[16];  // xt[4j + s] = bytes {x[16j + 4i + s]}, i = 0..3
+        float da0, da1, fb0, fb1;
+    };
+    __device__ static int units(int in_f) { return in_f / 64; }
+    __device__ static bool valid(int t, int lane, int n) { return t * 64 + lane < n; }
+    __device__ static void load_row(Row& r, const uint8_t* rowp, int t, int lane, bool ok) {
+        if (ok) {
+            const uint8_t* blk = rowp + (size_t)(t * 64 + lane) * 18;
+            r.d = load_u16(blk);
+            r.codes = load16_a2(blk + 2);
+        } else {
+            r.codes = v4i{0, 0, 0, 0};
+            r.d = 0;
+        }
+    }
+    __device__ static void load_acts(Acts& a, const ActPtrs& s, int t, int lane, bool ok) {
+        if (ok) {
+            const int b = t * 64 + lane;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const v4i v = *reinterpret_cast<const v4i*>(s.qs + (size_t)b * 64 + 16 * j);
+                const int in[4] = {v.x, v.y, v.z, v.w};
+                transpose4x4(in, &a.xt[4 * j]);
+            }
+            a.da0 = s.d[2 * b];
+            a.da1 = s.d[2 * b + 1];
+            a.fb0 = (float)s.bsums[2 * b];
+            a.fb1 = (float)s.bsums[2 * b + 1];
+        } else {
+#pragma unroll
+            for (int k = 0; k < 16; ++k) a.xt[k] = 0;
+            a.da0 = a.da1 = a.fb0 = a.fb1 = 0.0f;
+        }
+    }
+    template <bool STAGES>
+    __device__ static float term(const Row& r, const Acts& a, int t, int lane, bool ok,
+                                 const StagePtrs& st, size_t row_units) {
+        const uint32_t cw[4] = {(uint32_t)r.codes.x, (uint32_t)r.codes.y, (uint32_t)r.codes.z,
+                                (uint32_t)r.codes.w};
+        int ip0 = 0, ip1 = 0;
+#pragma unroll
+        for (int sft = 0; sft < 4; ++sft) {
+            ip0 = dot4((int)((cw[0] >> (2 * sft)) & 0x03030303u), a.xt[0 + sft], ip0);
+            ip0 = dot4((int)((cw[1] >> (2 * sft)) & 0x03030303u), a.xt[4 + sft], ip0);
+            ip1 = dot4((int)((cw[2] >> (2 * sft)) & 0x03030303u), a.xt[8 + sft], ip1);
+            ip1 = dot4((int)((cw[3] >> (2 * sft)) & 0x03030303u), a.xt[12 + sft], ip1);
+        }
+        if (STAGES && ok) {
+            // stage layout is per 32-element sub-block: two per unit
+            st.a[2 * row_units + 2 * (t * 64 + lane)] = ip0;
+            st.a[2 * row_units + 2 * (t * 64 + lane) + 1] = ip1;
+        }
+        const float d = f16_bits_to_f32(r.d);
+        // sumf += d * q8.d[s] * (iprod as f32 - bsum[s] as f32), sub-block 2b then 2b+1
+        float s = d * a.da0 * ((float)ip0 - a.fb0);
+        s += d * a.da1 * ((float)ip1 - a.fb1);
+        return s;
+    }
+};
+
+}  // namespace infr

@@ -1,5 +1,5 @@
-// Host-side launch interface of the device kernels. Every launcher validates nothing: the C-ABI
-// layer (backend.hip) checks shapes, alignment and buffer sizes before calling in here.
+// Host-side launch interface of the device kernels. Launchers validate nothing: the C-ABI layer
+// (backend.hip) checks shapes, alignment and buffer sizes before calling in here.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -9,9 +9,8 @@
 namespace infr {
 
 // Device-resident quantized activation of m rows of k elements, laid out row-major per field.
-// super == true : per-256 `Q8`   (crates/infr-cpu/src/quant.rs:8-25):  d[m][k/256], bsums[m][k/32],
-//                 bsums16[m][k/16]
-// super == false: per-32 `Q8x32` (quant.rs:90-95): d[m][k/32], bsums[m][k/32]; bsums16 unused.
+// per-256 `Q8`   (crates/infr-cpu/src/quant.rs:8-25):  d[m][k/256], bsums[m][k/32], bsums16[m][k/16]
+// per-32 `Q8x32` (quant.rs:90-95): d[m][k/32], bsums[m][k/32]; bsums16 unused.
 struct ActQ8 {
     int8_t* qs = nullptr;
     float* d = nullptr;
@@ -29,12 +28,50 @@ struct IntStages {
     int32_t* b = nullptr;
 };
 
-// Decode GEMV, m == 1: y[o] = vec_dot(row o, act) for out_f rows of `bpr` bytes each.
-// Returns false when (dtype, in_f) has no kernel.
+// Decode GEMV over an activation that is already quantized in device memory:
+// y[o] = vec_dot(row o, act) for out_f rows of `bpr` bytes. false = no kernel for (dtype, in_f).
 bool launch_gemv(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t in_f,
                  size_t out_f, const IntStages& st, hipStream_t stream);
 
-// m >= 2: int8 MFMA GEMM over on-device quantized activations. y is [m][out_f] row-major.
+// One m == 1 Op::Linear of a fused, grouped decode launch: the kernel quantizes x itself (into
+// LDS) and produces y. All ops of a group share (dtype, in_f).
+struct GemvOpDesc {
+    const uint8_t* w;  // first selected weight row
+    const float* x;    // f32 [in_f]
+    float* y;          // f32 [out_f]
+    uint64_t bpr;      // bytes per weight row
+    int32_t out_f;
+};
+
+// What one workgroup of a grouped launch works on: `rows` consecutive weight rows of one op.
+// The launcher keeps a table of these in device memory, indexed by blockIdx.x, so a workgroup
+// finds its work with a single 32-byte scalar load.
+struct GemvTile {
+    const uint8_t* w;  // first row of the tile
+    const float* x;
+    float* y;          // output of the tile's first row
+    uint32_t bpr;
+    int32_t rows;
+};
+
+struct GemvGroupPlan {
+    int total_wgs = 0;
+    int waves_per_wg = 0;
+    int rows_per_wg = 0;
+    size_t lds_bytes = 0;
+};
+
+// Chooses workgroup shape and rows per wave for a group. false = no kernel for (dtype, in_f).
+bool plan_gemv_group(int dtype, size_t in_f, const GemvOpDesc* ops, int n, GemvGroupPlan* plan);
+// Writes the plan's total_wgs tiles for ops[0..n).
+void fill_gemv_tiles(const GemvOpDesc* ops, int n, const GemvGroupPlan& plan, GemvTile* tiles);
+
+// Launches a planned group. `tiles_dev` is the device copy of the tile table; it may be null when
+// n == 1 (the single op's descriptor then travels as a kernel argument).
+bool launch_gemv_fused(int dtype, size_t in_f, const GemvOpDesc* ops, int n, const GemvTile* tiles_dev,
+                       const GemvGroupPlan& plan, hipStream_t stream);
+
+// m >= 2: GEMM over on-device quantized activations. y is [m][out_f] row-major.
 bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
                 size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream);
 

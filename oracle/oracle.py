@@ -252,9 +252,11 @@ def moe_ffn(x, router, gate, up, down, *, ne: int, n_expert: int, n_used: int, n
     x = _c(x, np.float32).ravel()
     rows = x.size // ne
     rx = x if router_x is None else _c(router_x, np.float32).ravel()
-    router, gate, up, down = (_c(a, np.uint8).ravel() if a.dtype != np.uint8 else _c(a, np.uint8).ravel()
-                              for a in (np.asarray(router).view(np.uint8), np.asarray(gate),
-                                        np.asarray(up), np.asarray(down)))
+    def raw(a):  # banks arrive as raw bytes (quantized) or as f32 arrays (router)
+        a = np.ascontiguousarray(a)
+        return a.view(np.uint8).ravel()
+
+    router, gate, up, down = raw(router), raw(gate), raw(up), raw(down)
     p = _MoeParams(ne, n_expert, n_used, n_ff_exp, rows, scale, router_dtype, gate_dtype, up_dtype,
                    down_dtype, int(reference_mode))
     y = np.empty(rows * ne, np.float32)
