@@ -1,13 +1,210 @@
-// m >= 2: GEMM of block-quantized weights against on-device int8-quantized activations.
+// Prefill GEMM (m >= 2) of block-quantized weights against on-device int8-quantized activations.
+//
+// Q4_K runs on the int8 matrix cores. Per 256-element block infr-cpu computes, per output,
+//     sd = sum_s sc_s * (sum_l q4 * q8)     sm = sum_s m_s * bsums_s
+//     y += q8.d[b] * (d * (f32)sd - dmin * (f32)sm)            (crates/infr-cpu/src/kernels.rs:151-184)
+// with 6-bit sc_s, m_s per 32-element sub-block. The MFMA accumulates over K inside the
+// instruction, so a per-sub-block scale has to be inside the operand. q4 * sc_s needs 10 bits, so
+// the scale is split sc = 8 * sc_hi + sc_lo (3 bits each): q4 * sc_lo and q4 * sc_hi both fit int8,
+// two v_mfma_i32_32x32x32_i8 chains run over the whole block, and sd = lo + 8 * hi exactly.
+// (The alternative, one K=32 MFMA per sub-block followed by a VALU multiply, runs the legacy
+// half-rate instruction and needs eight integer multiply-adds per output per block.)
+// sm is a K = 16 product of the mins with the activation's per-32 sums split as bsum = lo + 64*hi
+// (both exact in f16): one v_mfma_f32_32x32x16_f16 whose f32 result is the exact integer.
+// The f32 epilogue then evaluates the CPU expression with separate multiplies and adds, and each
+// output accumulates its blocks in ascending order, so y is bit-identical to infr-cpu's batch
+// kernel (and to this library's m == 1 GEMV).
+//
+// Tiling. Tokens are the MFMA's M (rows of C), weight rows its N (columns): a lane's 16
+// accumulators then share one weight row, so d, dmin and the pre-scaled operand are per lane.
+// A workgroup (4 waves) covers BM tokens x 128 weight rows; each wave owns 32 weight rows for all
+// BM tokens, loads and unpacks its rows' blocks straight from global memory into MFMA B operands
+// (no LDS for weights, no redundant unpacking), and reads the activation tile, shared by the four
+// waves, from LDS. Per 256-block and 32x32 output tile: 16 int8 MFMAs + 1 f16 MFMA against
+// 7 VALU instructions per output for the epilogue.
+//
+// Other formats at m >= 2 go row by row through the decode GEMV (correct, not fast).
 #include "device_common.hpp"
 #include "kernels.hpp"
 
 namespace infr {
 
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+
+constexpr int kActRowBytes = 256 + 16;  // padded LDS row: conflict-free 16-byte reads and writes
+
+// LDS per workgroup: activation bytes | per-token scale | per-token split bsums (f16 x 16)
+template <int BM>
+struct MmqLds {
+    static constexpr int qs_off = 0;
+    static constexpr int d_off = BM * kActRowBytes;
+    static constexpr int bs_off = d_off + BM * 4;
+    static constexpr int bytes = bs_off + BM * 32;
+};
+
+struct Q4kRaw {
+    v4i hdr, q[4];
+};
+
+__device__ __forceinline__ void q4k_load_raw(Q4kRaw& r, const uint8_t* blk, int h, bool ok) {
+    if (ok) {
+        r.hdr = load16(blk);
+#pragma unroll
+        for (int p = 0; p < 4; ++p) r.q[p] = load16(blk + 16 + p * 32 + h * 16);
+    } else {
+        r.hdr = v4i{0, 0, 0, 0};
+#pragma unroll
+        for (int p = 0; p < 4; ++p) r.q[p] = v4i{0, 0, 0, 0};
+    }
+}
+
+// Packed byte-wise multiply of four codes (<= 15) by a scale digit (<= 7): no byte overflows, so
+// two 16-bit lane multiplies do it.
+__device__ __forceinline__ int scale_codes(uint32_t codes, uint32_t digit) {
+    typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+    const us2 c = __builtin_bit_cast(us2, codes);
+    const us2 s = {(unsigned short)digit, (unsigned short)digit};
+    return __builtin_bit_cast(int, (us2)(c * s));
+}
+
+template <int BM, bool STAGES>
+__global__ __launch_bounds__(256) void mmq_q4k_kernel(const uint8_t* __restrict__ w, size_t bpr,
+                                                      const int8_t* __restrict__ qs,
+                                                      const float* __restrict__ d8,
+                                                      const int32_t* __restrict__ bsums,
+                                                      float* __restrict__ y, int m, int out_f, int nb,
+                                                      int32_t* __restrict__ st_sd,
+                                                      int32_t* __restrict__ st_sm) {
+    constexpr int TB = BM / 32;  // token blocks of 32
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, h = lane >> 5;
+    const int tok0 = blockIdx.y * BM;
+    const int wrow = blockIdx.x * 128 + wave * 32 + col;
+    const bool row_ok = wrow < out_f;
+    const size_t in_f = (size_t)nb * 256;
+    const uint8_t* wrowp = w + (size_t)(row_ok ? wrow : 0) * bpr;
+
+    v16f acc[TB];
+#pragma unroll
+    for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[tb][i] = 0.0f;
+
+    Q4kRaw raw;
+    q4k_load_raw(raw, wrowp, h, row_ok);
+
+    for (int b = 0; b < nb; ++b) {
+        // ---- stage the activation tile of block b into LDS (all 256 threads) ----
+        __syncthreads();  // previous block's readers are done
+        for (int c = tid; c < BM * 16; c += 256) {
+            const int t = c >> 4, kc = c & 15;
+            const int tok = tok0 + t;
+            v4i v = {0, 0, 0, 0};
+            if (tok < m) v = *reinterpret_cast<const v4i*>(qs + (size_t)tok * in_f + (size_t)b * 256 + kc * 16);
+            *reinterpret_cast<v4i*>(lds + MmqLds<BM>::qs_off + t * kActRowBytes + kc * 16) = v;
+        }
+        for (int c = tid; c < BM * 8; c += 256) {
+            const int t = c >> 3, s = c & 7;
+            const int tok = tok0 + t;
+            const int bs = tok < m ? bsums[(size_t)tok * (nb * 8) + b * 8 + s] : 0;
+            const int lo = bs & 63;  // bsum = 64 * hi + lo, 0 <= lo < 64; both parts exact in f16
+            _Float16* p = reinterpret_cast<_Float16*>(lds + MmqLds<BM>::bs_off + t * 32);
+            p[s] = (_Float16)lo;
+            p[8 + s] = (_Float16)(bs - lo);
+        }
+        for (int t = tid; t < BM; t += 256) {
+            const int tok = tok0 + t;
+            reinterpret_cast<float*>(lds + MmqLds<BM>::d_off)[t] = tok < m ? d8[(size_t)tok * nb + b] : 0.0f;
+        }
+
+        // ---- this wave's 32 weight rows of block b -> MFMA B operands (registers) ----
+        const Q4kRaw cur = raw;
+        if (b + 1 < nb) q4k_load_raw(raw, wrowp + (size_t)(b + 1) * 144, h, row_ok);
+        uint32_t sc8[2], mn8[2];
+        k4_all((uint32_t)cur.hdr.y, (uint32_t)cur.hdr.z, (uint32_t)cur.hdr.w, sc8, mn8);
+        const float d = f16_bits_to_f32((uint32_t)cur.hdr.x & 0xFFFFu);
+        const float dmin = f16_bits_to_f32((uint32_t)cur.hdr.x >> 16);
+        v4i blo[8], bhi[8];
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const int qw[4] = {cur.q[p].x, cur.q[p].y, cur.q[p].z, cur.q[p].w};
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {  // e = 0: sub-block 2p (low nibbles), 1: 2p+1 (high)
+                const int s = 2 * p + e;
+                const uint32_t sc = (sc8[s >> 2] >> (8 * (s & 3))) & 0xFFu;
+                const uint32_t lo3 = sc & 7u, hi3 = sc >> 3;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t codes = ((uint32_t)qw[k] >> (4 * e)) & 0x0F0F0F0Fu;
+                    blo[s][k] = scale_codes(codes, lo3);
+                    bhi[s][k] = scale_codes(codes, hi3);
+                }
+            }
+        }
+        // mins as f16 for the K=16 product: k-slots 0..7 pair with bsum lo, 8..15 with 64*hi
+        v8h bm;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) bm[s] = (_Float16)(int)((mn8[s >> 2] >> (8 * (s & 3))) & 0xFFu);
+
+        __syncthreads();  // tile is in LDS
+
+#pragma unroll
+        for (int tb = 0; tb < TB; ++tb) {
+            v16i alo, ahi;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) alo[i] = ahi[i] = 0;
+            const uint8_t* arow = lds + MmqLds<BM>::qs_off + (tb * 32 + col) * kActRowBytes + h * 16;
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+                const v4i a = *reinterpret_cast<const v4i*>(arow + s * 32);
+                alo = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, blo[s], alo, 0, 0, 0);
+                ahi = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bhi[s], ahi, 0, 0, 0);
+            }
+            const v8h abs_ = *reinterpret_cast<const v8h*>(lds + MmqLds<BM>::bs_off + (tb * 32 + col) * 32 + h * 16);
+            v16f smf;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) smf[i] = 0.0f;
+            smf = __builtin_amdgcn_mfma_f32_32x32x16_f16(abs_, bm, smf, 0, 0, 0);
+            // epilogue: accumulator i of this lane is token 8*(i/4) + 4*h + i%4 of the block
+            const float* dtile = reinterpret_cast<const float*>(lds + MmqLds<BM>::d_off) + tb * 32 + 4 * h;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const v4f dq = *reinterpret_cast<const v4f*>(dtile + 8 * j);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int r = 4 * j + i;
+                    const int sd = alo[r] + (ahi[r] << 3);
+                    if (STAGES) {
+                        const int tok = tok0 + tb * 32 + 8 * j + 4 * h + i;
+                        if (row_ok && tok < m) {
+                            st_sd[((size_t)tok * out_f + wrow) * nb + b] = sd;
+                            st_sm[((size_t)tok * out_f + wrow) * nb + b] = (int)smf[r];
+                        }
+                    }
+                    // sumf += q8.d[b] * (d * sd as f32 - dmin * sm as f32)
+                    acc[tb][r] += dq[i] * (d * (float)sd - dmin * smf[r]);
+                }
+            }
+        }
+    }
+
+    if (!row_ok) return;
+#pragma unroll
+    for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int tok = tok0 + tb * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+            if (tok < m) y[(size_t)tok * out_f + wrow] = acc[tb][r];
+        }
+}
+
 // Row-at-a-time form: every activation row goes through the decode GEMV, so each output element
 // is produced by exactly the code path of m == 1 (the CPU's batch kernels are likewise
 // bit-identical to its single-row kernels, crates/infr-cpu/src/kernels.rs:9297-9405). Weights are
-// re-streamed once per row, which is only acceptable for very small m.
+// re-streamed once per row, which is only acceptable for small m.
 static bool mmq_by_rows(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y,
                         size_t m, size_t in_f, size_t out_f, const IntStages& st,
                         hipStream_t stream) {
@@ -28,8 +225,27 @@ static bool mmq_by_rows(int dtype, const uint8_t* w, size_t bpr, const ActQ8& ac
     return true;
 }
 
+template <int BM>
+static void launch_mmq_q4k(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
+                           size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream) {
+    const dim3 grid((unsigned)((out_f + 127) / 128), (unsigned)((m + BM - 1) / BM)), block(256);
+    const int nb = (int)(in_f / 256);
+    if (st.a)
+        hipLaunchKernelGGL((mmq_q4k_kernel<BM, true>), grid, block, MmqLds<BM>::bytes, stream, w, bpr,
+                           act.qs, act.d, act.bsums, y, (int)m, (int)out_f, nb, st.a, st.b);
+    else
+        hipLaunchKernelGGL((mmq_q4k_kernel<BM, false>), grid, block, MmqLds<BM>::bytes, stream, w, bpr,
+                           act.qs, act.d, act.bsums, y, (int)m, (int)out_f, nb, (int32_t*)nullptr,
+                           (int32_t*)nullptr);
+}
+
 bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
                 size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream) {
+    if (dtype == 12) {
+        if (m <= 32) launch_mmq_q4k<32>(w, bpr, act, y, m, in_f, out_f, st, stream);
+        else launch_mmq_q4k<64>(w, bpr, act, y, m, in_f, out_f, st, stream);
+        return true;
+    }
     return mmq_by_rows(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
 }
 

@@ -104,3 +104,44 @@ def test_w_off_selects_rows_of_a_concatenated_weight(be):
     y = run_linear(be, DType.Q4K, w, x, 1, in_f, 16, w_off=16 * in_f, w_numel=rows * in_f)
     want = orc.linear(DType.Q4K, w, x, 1, in_f, 16, w_numel=rows * in_f, w_off=16 * in_f)
     assert np.array_equal(y.view(np.uint32), want.view(np.uint32))
+
+
+# ───────────── prefill (m >= 2): int8 MFMA path for Q4_K ─────────────
+
+PREFILL_SHAPES = [(2, 256, 8), (8, 1024, 96), (33, 512, 200), (64, 1024, 256), (130, 768, 130), (257, 2048, 384)]
+
+
+@pytest.mark.parametrize("m,in_f,out_f", PREFILL_SHAPES)
+def test_prefill_q4k_is_bit_identical_to_oracle(be, m, in_f, out_f):
+    w = synth_weight(DType.Q4K, 300 + m, out_f, in_f)
+    x = synth_normal_f32(400 + m, m * in_f)
+    x[:in_f] *= 37.0            # rows with very different scales
+    if m > 2:
+        x[2 * in_f:3 * in_f] = 0.0   # an all-zero row
+    y = run_linear(be, DType.Q4K, w, x, m, in_f, out_f)
+    want = orc.linear(DType.Q4K, w, x, m, in_f, out_f)
+    gate(y, want)
+    assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), "not bit-identical"
+
+
+@pytest.mark.parametrize("m,in_f,out_f", [(5, 512, 40), (70, 768, 150)])
+def test_prefill_q4k_int_stages_bit_exact(be, m, in_f, out_f):
+    # full-range payload bytes: every scale, min and code value occurs (sc up to 63 exercises the
+    # split-scale operands, large |bsums| the split sums)
+    w = orc.synth_weight(DType.Q4K, in_f * out_f, 0x208)
+    x = synth_normal_f32(77, m * in_f) * np.float32(3.0)
+    x[in_f:2 * in_f] = 1e4      # saturates every code to +127: bsums reach +4064
+    x[2 * in_f:3 * in_f] = -1e4
+    a, b = be.linear_int_stages(DType.Q4K, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
+    oa, ob = orc.linear_int_stages(DType.Q4K, w, x, m, in_f, out_f)
+    assert np.array_equal(a, oa)
+    assert np.array_equal(b, ob)
+
+
+@pytest.mark.parametrize("dtype", [DType.Q6K, DType.Q8_0, DType.Q2_0])
+def test_prefill_other_formats_vs_oracle(be, dtype):
+    m, in_f, out_f = 5, 1024, 72
+    w = synth_weight(dtype, 9, out_f, in_f)
+    x = synth_normal_f32(10, m * in_f)
+    y = run_linear(be, dtype, w, x, m, in_f, out_f)
+    gate(y, orc.linear(dtype, w, x, m, in_f, out_f))
