@@ -195,6 +195,8 @@ def main():
     ap.add_argument("--layers", type=int, default=N_LAYERS)
     ap.add_argument("--no-extra", action="store_true", help="headline sweep only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--sections", default="shapes,mmq,ternary",
+                    help="comma list of secondary sections: shapes, mmq, ternary")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
@@ -229,16 +231,19 @@ def main():
     sw.free()
 
     extra = {}
-    if not args.no_extra:
+    sections = set() if args.no_extra else set(args.sections.split(","))
+    if "shapes" in sections:
         for name, dt in (("Q4_K", DType.Q4K), ("Q6_K", DType.Q6K), ("Q8_0", DType.Q8_0)):
             for m in (1, 8):
                 for (out_f, in_f) in ((4096, 4096), (1024, 4096), (12288, 4096), (4096, 12288)):
                     t, nb = single_shape(be, dt, m, in_f, out_f)
                     extra[f"gemv_{name}_m{m}_{out_f}x{in_f}_GBs"] = round(nb / (t * 1e-3) / 1e9, 1)
+    if "mmq" in sections:
         for M in (64, 512, 2048):
             t, nb = single_shape(be, DType.Q4K, M, 4096, 12288, reps=10)
             extra[f"mmq_Q4_K_M{M}_TOPS"] = round(2.0 * M * 12288 * 4096 / (t * 1e-3) / 1e12, 2)
             extra[f"mmq_Q4_K_M{M}_pct_int8_peak"] = round(100 * extra[f"mmq_Q4_K_M{M}_TOPS"] / INT8_PEAK_TOPS, 2)
+    if "ternary" in sections:
         tern = Sweep(be, DType.Q2_0, 1, N_LAYERS, head=True)
         d, w = tern.time(5, 2)
         tms = max(d, w)

@@ -24,6 +24,9 @@ SOURCES = ["backend.hip", "quant_act.hip", "gemv.hip", "mmq.hip", "synth.cpp"]
 DEVICE_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fno-fast-math",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function",
+    # keep MFMA accumulators in VGPRs: the epilogues read every accumulator with VALU
+    # instructions, and AGPR-resident results would each cost a v_accvgpr_read first
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
 ]
 
 

@@ -24,6 +24,8 @@
 // 7 VALU instructions per output for the epilogue.
 //
 // Other formats at m >= 2 go row by row through the decode GEMV (correct, not fast).
+#include <cstdlib>
+
 #include "device_common.hpp"
 #include "kernels.hpp"
 
@@ -69,6 +71,54 @@ __device__ __forceinline__ int scale_codes(uint32_t codes, uint32_t digit) {
     return __builtin_bit_cast(int, (us2)(c * s));
 }
 
+// Activation-tile staging, split in two halves so the global loads of block b+1 are in flight
+// while block b is multiplied: fetch() issues the loads into registers, store() writes them to the
+// LDS buffer once the previous readers of that buffer are past their barrier.
+template <int BM>
+struct ActStage {
+    static constexpr int kChunks = BM * 16 / 256;       // 16-byte chunks per thread
+    static constexpr int kSums = (BM * 8 + 255) / 256;  // per-32 sums per thread
+    v4i q[kChunks];
+    int bs[kSums];
+    float d;
+
+    __device__ __forceinline__ void fetch(const int8_t* qs, const float* d8, const int32_t* bsums,
+                                          int tok0, int m, int nb, int b, int tid) {
+        const size_t in_f = (size_t)nb * 256;
+#pragma unroll
+        for (int i = 0; i < kChunks; ++i) {
+            // Tokens past m are clamped to the last row: their outputs are computed and never stored.
+            const int c = tid + i * 256, t = c >> 4, kc = c & 15, tok = min(tok0 + t, m - 1);
+            q[i] = *reinterpret_cast<const v4i*>(qs + (size_t)tok * in_f + (size_t)b * 256 + kc * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < kSums; ++i) {
+            const int c = min(tid + i * 256, BM * 8 - 1), t = c >> 3, s = c & 7, tok = min(tok0 + t, m - 1);
+            bs[i] = bsums[(size_t)tok * (nb * 8) + b * 8 + s];
+        }
+        d = d8[(size_t)min(tok0 + min(tid, BM - 1), m - 1) * nb + b];
+    }
+
+    __device__ __forceinline__ void store(uint8_t* buf, int tid) const {
+#pragma unroll
+        for (int i = 0; i < kChunks; ++i) {
+            const int c = tid + i * 256, t = c >> 4, kc = c & 15;
+            *reinterpret_cast<v4i*>(buf + MmqLds<BM>::qs_off + t * kActRowBytes + kc * 16) = q[i];
+        }
+#pragma unroll
+        for (int i = 0; i < kSums; ++i) {
+            const int c = tid + i * 256, t = c >> 3, s = c & 7;
+            if (c < BM * 8) {
+                const int lo = bs[i] & 63;  // bsum = 64 * hi + lo, 0 <= lo < 64; both exact in f16
+                _Float16* p = reinterpret_cast<_Float16*>(buf + MmqLds<BM>::bs_off + t * 32);
+                p[s] = (_Float16)lo;
+                p[8 + s] = (_Float16)(bs[i] - lo);
+            }
+        }
+        if (tid < BM) reinterpret_cast<float*>(buf + MmqLds<BM>::d_off)[tid] = d;
+    }
+};
+
 template <int BM, bool STAGES>
 __global__ __launch_bounds__(256) void mmq_q4k_kernel(const uint8_t* __restrict__ w, size_t bpr,
                                                       const int8_t* __restrict__ qs,
@@ -78,13 +128,12 @@ __global__ __launch_bounds__(256) void mmq_q4k_kernel(const uint8_t* __restrict_
                                                       int32_t* __restrict__ st_sd,
                                                       int32_t* __restrict__ st_sm) {
     constexpr int TB = BM / 32;  // token blocks of 32
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // two MmqLds<BM> buffers
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, h = lane >> 5;
     const int tok0 = blockIdx.y * BM;
     const int wrow = blockIdx.x * 128 + wave * 32 + col;
     const bool row_ok = wrow < out_f;
-    const size_t in_f = (size_t)nb * 256;
     const uint8_t* wrowp = w + (size_t)(row_ok ? wrow : 0) * bpr;
 
     v16f acc[TB];
@@ -93,36 +142,23 @@ __global__ __launch_bounds__(256) void mmq_q4k_kernel(const uint8_t* __restrict_
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[tb][i] = 0.0f;
 
+    ActStage<BM> stage;
+    stage.fetch(qs, d8, bsums, tok0, m, nb, 0, tid);
     Q4kRaw raw;
     q4k_load_raw(raw, wrowp, h, row_ok);
+    stage.store(lds, tid);
+    __syncthreads();
 
     for (int b = 0; b < nb; ++b) {
-        // ---- stage the activation tile of block b into LDS (all 256 threads) ----
-        __syncthreads();  // previous block's readers are done
-        for (int c = tid; c < BM * 16; c += 256) {
-            const int t = c >> 4, kc = c & 15;
-            const int tok = tok0 + t;
-            v4i v = {0, 0, 0, 0};
-            if (tok < m) v = *reinterpret_cast<const v4i*>(qs + (size_t)tok * in_f + (size_t)b * 256 + kc * 16);
-            *reinterpret_cast<v4i*>(lds + MmqLds<BM>::qs_off + t * kActRowBytes + kc * 16) = v;
-        }
-        for (int c = tid; c < BM * 8; c += 256) {
-            const int t = c >> 3, s = c & 7;
-            const int tok = tok0 + t;
-            const int bs = tok < m ? bsums[(size_t)tok * (nb * 8) + b * 8 + s] : 0;
-            const int lo = bs & 63;  // bsum = 64 * hi + lo, 0 <= lo < 64; both parts exact in f16
-            _Float16* p = reinterpret_cast<_Float16*>(lds + MmqLds<BM>::bs_off + t * 32);
-            p[s] = (_Float16)lo;
-            p[8 + s] = (_Float16)(bs - lo);
-        }
-        for (int t = tid; t < BM; t += 256) {
-            const int tok = tok0 + t;
-            reinterpret_cast<float*>(lds + MmqLds<BM>::d_off)[t] = tok < m ? d8[(size_t)tok * nb + b] : 0.0f;
+        const uint8_t* tile = lds + (b & 1) * MmqLds<BM>::bytes;
+        // ---- request block b+1: activation tile into registers, this wave's weight rows ----
+        const Q4kRaw cur = raw;
+        if (b + 1 < nb) {
+            stage.fetch(qs, d8, bsums, tok0, m, nb, b + 1, tid);
+            q4k_load_raw(raw, wrowp + (size_t)(b + 1) * 144, h, row_ok);
         }
 
         // ---- this wave's 32 weight rows of block b -> MFMA B operands (registers) ----
-        const Q4kRaw cur = raw;
-        if (b + 1 < nb) q4k_load_raw(raw, wrowp + (size_t)(b + 1) * 144, h, row_ok);
         uint32_t sc8[2], mn8[2];
         k4_all((uint32_t)cur.hdr.y, (uint32_t)cur.hdr.z, (uint32_t)cur.hdr.w, sc8, mn8);
         const float d = f16_bits_to_f32((uint32_t)cur.hdr.x & 0xFFFFu);
@@ -149,27 +185,24 @@ __global__ __launch_bounds__(256) void mmq_q4k_kernel(const uint8_t* __restrict_
 #pragma unroll
         for (int s = 0; s < 8; ++s) bm[s] = (_Float16)(int)((mn8[s >> 2] >> (8 * (s & 3))) & 0xFFu);
 
-        __syncthreads();  // tile is in LDS
-
 #pragma unroll
         for (int tb = 0; tb < TB; ++tb) {
-            v16i alo, ahi;
+            const v16i zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            const v16f zf = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            const uint8_t* arow = tile + MmqLds<BM>::qs_off + (tb * 32 + col) * kActRowBytes + h * 16;
+            v4i a = *reinterpret_cast<const v4i*>(arow);
+            v16i alo = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, blo[0], zi, 0, 0, 0);
+            v16i ahi = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bhi[0], zi, 0, 0, 0);
 #pragma unroll
-            for (int i = 0; i < 16; ++i) alo[i] = ahi[i] = 0;
-            const uint8_t* arow = lds + MmqLds<BM>::qs_off + (tb * 32 + col) * kActRowBytes + h * 16;
-#pragma unroll
-            for (int s = 0; s < 8; ++s) {
-                const v4i a = *reinterpret_cast<const v4i*>(arow + s * 32);
+            for (int s = 1; s < 8; ++s) {
+                a = *reinterpret_cast<const v4i*>(arow + s * 32);
                 alo = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, blo[s], alo, 0, 0, 0);
                 ahi = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bhi[s], ahi, 0, 0, 0);
             }
-            const v8h abs_ = *reinterpret_cast<const v8h*>(lds + MmqLds<BM>::bs_off + (tb * 32 + col) * 32 + h * 16);
-            v16f smf;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) smf[i] = 0.0f;
-            smf = __builtin_amdgcn_mfma_f32_32x32x16_f16(abs_, bm, smf, 0, 0, 0);
+            const v8h abs_ = *reinterpret_cast<const v8h*>(tile + MmqLds<BM>::bs_off + (tb * 32 + col) * 32 + h * 16);
+            const v16f smf = __builtin_amdgcn_mfma_f32_32x32x16_f16(abs_, bm, zf, 0, 0, 0);
             // epilogue: accumulator i of this lane is token 8*(i/4) + 4*h + i%4 of the block
-            const float* dtile = reinterpret_cast<const float*>(lds + MmqLds<BM>::d_off) + tb * 32 + 4 * h;
+            const float* dtile = reinterpret_cast<const float*>(tile + MmqLds<BM>::d_off) + tb * 32 + 4 * h;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const v4f dq = *reinterpret_cast<const v4f*>(dtile + 8 * j);
@@ -189,6 +222,10 @@ __global__ __launch_bounds__(256) void mmq_q4k_kernel(const uint8_t* __restrict_
                 }
             }
         }
+
+        // ---- publish block b+1 in the other buffer (its last readers passed the previous barrier)
+        if (b + 1 < nb) stage.store(lds + ((b + 1) & 1) * MmqLds<BM>::bytes, tid);
+        __syncthreads();
     }
 
     if (!row_ok) return;
@@ -231,10 +268,10 @@ static void launch_mmq_q4k(const uint8_t* w, size_t bpr, const ActQ8& act, float
     const dim3 grid((unsigned)((out_f + 127) / 128), (unsigned)((m + BM - 1) / BM)), block(256);
     const int nb = (int)(in_f / 256);
     if (st.a)
-        hipLaunchKernelGGL((mmq_q4k_kernel<BM, true>), grid, block, MmqLds<BM>::bytes, stream, w, bpr,
+        hipLaunchKernelGGL((mmq_q4k_kernel<BM, true>), grid, block, 2 * MmqLds<BM>::bytes, stream, w, bpr,
                            act.qs, act.d, act.bsums, y, (int)m, (int)out_f, nb, st.a, st.b);
     else
-        hipLaunchKernelGGL((mmq_q4k_kernel<BM, false>), grid, block, MmqLds<BM>::bytes, stream, w, bpr,
+        hipLaunchKernelGGL((mmq_q4k_kernel<BM, false>), grid, block, 2 * MmqLds<BM>::bytes, stream, w, bpr,
                            act.qs, act.d, act.bsums, y, (int)m, (int)out_f, nb, (int32_t*)nullptr,
                            (int32_t*)nullptr);
 }
@@ -242,8 +279,13 @@ static void launch_mmq_q4k(const uint8_t* w, size_t bpr, const ActQ8& act, float
 bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
                 size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream) {
     if (dtype == 12) {
-        if (m <= 32) launch_mmq_q4k<32>(w, bpr, act, y, m, in_f, out_f, st, stream);
-        else launch_mmq_q4k<64>(w, bpr, act, y, m, in_f, out_f, st, stream);
+        static const int env_bm = getenv("INFR_HIP_MMQ_BM") ? atoi(getenv("INFR_HIP_MMQ_BM")) : 0;
+        // 32-token tiles hold three waves per SIMD; the wider tiles amortise the weight unpack better
+        // but run one wave per SIMD, which measured slower at every M tried (64..2048).
+        const size_t bm = env_bm ? (size_t)env_bm : 32;
+        if (bm <= 32) launch_mmq_q4k<32>(w, bpr, act, y, m, in_f, out_f, st, stream);
+        else if (bm <= 64) launch_mmq_q4k<64>(w, bpr, act, y, m, in_f, out_f, st, stream);
+        else launch_mmq_q4k<128>(w, bpr, act, y, m, in_f, out_f, st, stream);
         return true;
     }
     return mmq_by_rows(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
