@@ -457,11 +457,86 @@ int infr_hip_quantize_q8_32(infr_hip_t* be, const infr_hip_buffer_t* x, size_t m
     return quantize_impl(be, true, x, m, k, qs, d, bsum, nullptr);
 }
 
-int infr_hip_moe_ffn(infr_hip_t* be, const infr_hip_moe_params_t*, const infr_hip_buffer_t*,
-                     const infr_hip_buffer_t*, const infr_hip_buffer_t*, const infr_hip_buffer_t*,
-                     const infr_hip_buffer_t*, const infr_hip_buffer_t*, infr_hip_buffer_t*,
-                     infr_hip_buffer_t*, infr_hip_buffer_t*) {
-    return fail(be, INFR_HIP_ERR_UNSUPPORTED, "moe_ffn: not built yet");
+static int ensure_moe_ws(infr_hip_t* be, size_t bytes) {
+    if (bytes <= be->moe_ws_bytes) return INFR_HIP_OK;
+    HIP_TRY(be, hipStreamSynchronize(be->stream));
+    if (be->moe_ws) (void)hipFree(be->moe_ws);
+    be->moe_ws = nullptr;
+    be->moe_ws_bytes = 0;
+    HIP_TRY(be, hipMalloc(&be->moe_ws, bytes));
+    be->moe_ws_bytes = bytes;
+    return INFR_HIP_OK;
+}
+
+static size_t expert_bank_bytes(int dtype, size_t rows, size_t in_f) {
+    int qpb = 0, bpb = 0;
+    if (!infr_block_layout(dtype, &qpb, &bpb) || in_f % (size_t)qpb != 0) return 0;
+    return rows * (in_f / (size_t)qpb) * (size_t)bpb;
+}
+
+// Validates an Op::MoeFfn and fills the launch structures.
+static int check_moe(infr_hip_t* be, const infr_hip_moe_params_t* p, const infr_hip_buffer_t* x,
+                     const infr_hip_buffer_t* router_x, const infr_hip_buffer_t* router,
+                     const infr_hip_buffer_t* gate, const infr_hip_buffer_t* up,
+                     const infr_hip_buffer_t* down, infr_hip_buffer_t* dst,
+                     infr_hip_buffer_t* sel_idx, infr_hip_buffer_t* sel_w, infr::MoeShape* s,
+                     infr::MoeBuffers* b) {
+    if (!p || !x || !router_x || !router || !gate || !up || !down || !dst)
+        return fail(be, INFR_HIP_ERR_INVALID, "moe_ffn: unbound buffer");
+    if (!p->ne || !p->n_expert || !p->n_used || !p->n_ff_exp || !p->rows || p->n_used > p->n_expert)
+        return fail(be, INFR_HIP_ERR_INVALID, "moe_ffn: empty or inconsistent shape");
+    const size_t gb = expert_bank_bytes(p->gate_dtype, (size_t)p->n_expert * p->n_ff_exp, p->ne);
+    const size_t ub = expert_bank_bytes(p->up_dtype, (size_t)p->n_expert * p->n_ff_exp, p->ne);
+    const size_t db = expert_bank_bytes(p->down_dtype, (size_t)p->n_expert * p->ne, p->n_ff_exp);
+    if (!gb || !ub || !db || p->gate_dtype == INFR_DTYPE_F32 || p->up_dtype == INFR_DTYPE_F32 ||
+        p->down_dtype == INFR_DTYPE_F32)
+        return fail(be, INFR_HIP_ERR_UNSUPPORTED, "moe_ffn: expert bank dtype/shape has no kernel");
+    const size_t act_bytes = (size_t)p->rows * p->ne * sizeof(float);
+    if (gate->len < gb || up->len < ub || down->len < db ||
+        router->len < (size_t)p->n_expert * p->ne * sizeof(float) || x->len < act_bytes ||
+        router_x->len < act_bytes || dst->len < act_bytes)
+        return fail(be, INFR_HIP_ERR_INVALID, "moe_ffn: a buffer is smaller than its declared shape");
+    const size_t sel_bytes = (size_t)p->rows * p->n_used * 4;
+    if ((sel_idx && sel_idx->len < sel_bytes) || (sel_w && sel_w->len < sel_bytes))
+        return fail(be, INFR_HIP_ERR_INVALID, "moe_ffn: selection output buffer too small");
+    *s = infr::MoeShape{(int)p->ne, (int)p->n_expert, (int)p->n_used, (int)p->n_ff_exp, (int)p->rows,
+                        p->scale, p->router_dtype, p->gate_dtype, p->up_dtype, p->down_dtype};
+    b->x = static_cast<const float*>(x->ptr);
+    b->router_x = static_cast<const float*>(router_x->ptr);
+    b->router = static_cast<const float*>(router->ptr);
+    b->gate = static_cast<const uint8_t*>(gate->ptr);
+    b->up = static_cast<const uint8_t*>(up->ptr);
+    b->down = static_cast<const uint8_t*>(down->ptr);
+    // expert e = the e-th equal byte slice of the bound bank (lib.rs:2345-2347)
+    b->gate_stride = gate->len / p->n_expert;
+    b->up_stride = up->len / p->n_expert;
+    b->down_stride = down->len / p->n_expert;
+    b->dst = static_cast<float*>(dst->ptr);
+    b->sel_idx = sel_idx ? static_cast<int32_t*>(sel_idx->ptr) : nullptr;
+    b->sel_w = sel_w ? static_cast<float*>(sel_w->ptr) : nullptr;
+    return INFR_HIP_OK;
+}
+
+static int enqueue_moe(infr_hip_t* be, const infr::MoeShape& s, const infr::MoeBuffers& b) {
+    const char* msg = infr::launch_moe_ffn(s, b, be->moe_ws, be->stream);
+    if (msg) return fail(be, INFR_HIP_ERR_UNSUPPORTED, std::string("moe_ffn: ") + msg);
+    HIP_TRY(be, hipGetLastError());
+    return INFR_HIP_OK;
+}
+
+int infr_hip_moe_ffn(infr_hip_t* be, const infr_hip_moe_params_t* p, const infr_hip_buffer_t* x,
+                     const infr_hip_buffer_t* router_x, const infr_hip_buffer_t* router,
+                     const infr_hip_buffer_t* gate_exps, const infr_hip_buffer_t* up_exps,
+                     const infr_hip_buffer_t* down_exps, infr_hip_buffer_t* dst,
+                     infr_hip_buffer_t* sel_idx, infr_hip_buffer_t* sel_w) {
+    if (!be) return INFR_HIP_ERR_INVALID;
+    if (int rc = check_latch(be)) return rc;
+    infr::MoeShape s;
+    infr::MoeBuffers b;
+    if (int rc = check_moe(be, p, x, router_x, router, gate_exps, up_exps, down_exps, dst, sel_idx, sel_w, &s, &b))
+        return rc;
+    if (int rc = ensure_moe_ws(be, infr::moe_workspace_bytes(s))) return rc;
+    return enqueue_moe(be, s, b);
 }
 
 // ---- plan / execute ----
@@ -472,7 +547,7 @@ int infr_hip_compile(infr_hip_t* be, const infr_hip_op_t* ops, size_t n_ops, inf
     infr_hip_plan_t* p = new (std::nothrow) infr_hip_plan();
     if (!p) return fail(be, INFR_HIP_ERR_OTHER, "compile: out of host memory");
     p->ops.assign(ops, ops + n_ops);
-    size_t act_need = 0;
+    size_t act_need = 0, moe_need = 0;
     for (const auto& op : p->ops) {
         if (op.kind == INFR_OP_LINEAR) {
             if (!is_quant(op.w_dtype) || op.m == 0 || op.in_f == 0 || op.out_f == 0 ||
@@ -483,6 +558,18 @@ int infr_hip_compile(infr_hip_t* be, const infr_hip_op_t* ops, size_t n_ops, inf
             }
             p->max_tensor = std::max({p->max_tensor, op.x, op.weight, op.dst});
             act_need = std::max(act_need, (size_t)op.m * op.in_f);
+        } else if (op.kind == INFR_OP_MOE_FFN) {
+            const auto& mp = op.moe;
+            if (!mp.ne || !mp.n_expert || !mp.n_used || !mp.n_ff_exp || !mp.rows) {
+                delete p;
+                return fail(be, INFR_HIP_ERR_UNSUPPORTED, "compile: MoeFfn op with empty shape");
+            }
+            p->max_tensor = std::max({p->max_tensor, op.x, op.dst, op.router_x, op.router,
+                                      op.gate_exps, op.up_exps, op.down_exps});
+            const infr::MoeShape ms{(int)mp.ne, (int)mp.n_expert, (int)mp.n_used, (int)mp.n_ff_exp,
+                                    (int)mp.rows, mp.scale, mp.router_dtype, mp.gate_dtype,
+                                    mp.up_dtype, mp.down_dtype};
+            moe_need = std::max(moe_need, infr::moe_workspace_bytes(ms));
         } else {
             delete p;
             return fail(be, INFR_HIP_ERR_UNSUPPORTED, "compile: op kind " + std::to_string(op.kind));
@@ -490,6 +577,10 @@ int infr_hip_compile(infr_hip_t* be, const infr_hip_op_t* ops, size_t n_ops, inf
     }
     // Scratch is sized here so that execute never allocates (it records launches for replay).
     if (int rc = ensure_act(be, act_need)) {
+        delete p;
+        return rc;
+    }
+    if (int rc = ensure_moe_ws(be, moe_need)) {
         delete p;
         return rc;
     }
@@ -521,20 +612,36 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
     std::vector<int> level(n, 0);
     std::vector<LinearArgs> la(n);
     int max_level = 0;
+    std::vector<Span> rd2(n, Span{nullptr, nullptr});
     for (size_t i = 0; i < n; ++i) {
         const auto& op = plan->ops[i];
-        if (int rc = check_linear(be, op.w_dtype, bindings[op.weight], op.w_numel, op.w_off,
-                                  bindings[op.x], op.m, op.in_f, op.out_f, &la[i]))
-            return rc;
-        const size_t ybytes = (size_t)op.m * op.out_f * sizeof(float);
-        if (!bindings[op.dst] || bindings[op.dst]->len < ybytes)
-            return fail(be, INFR_HIP_ERR_INVALID, "execute: dst buffer missing or too small");
-        rd[i] = span(bindings[op.x], (size_t)op.m * op.in_f * sizeof(float));
-        wr[i] = span(bindings[op.dst], ybytes);
-        wt[i] = Span{la[i].wrows, la[i].wrows + (size_t)op.out_f * la[i].bpr};
+        if (op.kind == INFR_OP_MOE_FFN) {
+            infr::MoeShape ms;
+            infr::MoeBuffers mb;
+            if (int rc = check_moe(be, &op.moe, bindings[op.x], bindings[op.router_x], bindings[op.router],
+                                   bindings[op.gate_exps], bindings[op.up_exps], bindings[op.down_exps],
+                                   bindings[op.dst], nullptr, nullptr, &ms, &mb))
+                return rc;
+            const size_t abytes = (size_t)ms.rows * ms.ne * sizeof(float);
+            rd[i] = span(bindings[op.x], abytes);
+            rd2[i] = span(bindings[op.router_x], abytes);
+            wr[i] = span(bindings[op.dst], abytes);
+            wt[i] = Span{nullptr, nullptr};
+        } else {
+            if (int rc = check_linear(be, op.w_dtype, bindings[op.weight], op.w_numel, op.w_off,
+                                      bindings[op.x], op.m, op.in_f, op.out_f, &la[i]))
+                return rc;
+            const size_t ybytes = (size_t)op.m * op.out_f * sizeof(float);
+            if (!bindings[op.dst] || bindings[op.dst]->len < ybytes)
+                return fail(be, INFR_HIP_ERR_INVALID, "execute: dst buffer missing or too small");
+            rd[i] = span(bindings[op.x], (size_t)op.m * op.in_f * sizeof(float));
+            wr[i] = span(bindings[op.dst], ybytes);
+            wt[i] = Span{la[i].wrows, la[i].wrows + (size_t)op.out_f * la[i].bpr};
+        }
         for (size_t j = 0; j < i; ++j)
-            if (overlap(wr[j], rd[i]) || overlap(wr[j], wr[i]) || overlap(rd[j], wr[i]) ||
-                overlap(wr[j], wt[i]) || overlap(wt[j], wr[i]))
+            if (overlap(wr[j], rd[i]) || overlap(wr[j], rd2[i]) || overlap(wr[j], wr[i]) ||
+                overlap(rd[j], wr[i]) || overlap(rd2[j], wr[i]) || overlap(wr[j], wt[i]) ||
+                overlap(wt[j], wr[i]))
                 level[i] = std::max(level[i], level[j] + 1);
         max_level = std::max(max_level, level[i]);
     }
@@ -548,7 +655,7 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
             const auto& op = plan->ops[i];
             infr_hip_plan::Step st;
             st.level = lv;
-            if (op.m != 1) {
+            if (op.kind == INFR_OP_MOE_FFN || op.m != 1) {
                 st.op = (int)i;
                 taken[i] = 1;
                 plan->steps.push_back(st);
@@ -559,7 +666,8 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
             st.first = (int)plan->descs.size();
             for (size_t k = i; k < n; ++k) {
                 const auto& o2 = plan->ops[k];
-                if (level[k] != lv || taken[k] || o2.m != 1 || o2.w_dtype != op.w_dtype || o2.in_f != op.in_f)
+                if (level[k] != lv || taken[k] || o2.kind != INFR_OP_LINEAR || o2.m != 1 ||
+                    o2.w_dtype != op.w_dtype || o2.in_f != op.in_f)
                     continue;
                 taken[k] = 1;
                 plan->descs.push_back(infr::GemvOpDesc{
@@ -596,7 +704,16 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
 // Enqueues the scheduled launches (this is what gets recorded for replay: kernels only).
 static int enqueue_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t* const* bindings) {
     for (const auto& st : plan->steps) {
-        if (st.op >= 0) {
+        if (st.op >= 0 && plan->ops[st.op].kind == INFR_OP_MOE_FFN) {
+            const auto& op = plan->ops[st.op];
+            infr::MoeShape ms;
+            infr::MoeBuffers mb;
+            if (int rc = check_moe(be, &op.moe, bindings[op.x], bindings[op.router_x], bindings[op.router],
+                                   bindings[op.gate_exps], bindings[op.up_exps], bindings[op.down_exps],
+                                   bindings[op.dst], nullptr, nullptr, &ms, &mb))
+                return rc;
+            if (int rc = enqueue_moe(be, ms, mb)) return rc;
+        } else if (st.op >= 0) {
             const auto& op = plan->ops[st.op];
             LinearArgs la;
             if (int rc = check_linear(be, op.w_dtype, bindings[op.weight], op.w_numel, op.w_off,
@@ -636,9 +753,13 @@ int infr_hip_execute(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t* c
         plan->exec = nullptr;
     }
     // Validate and schedule before recording so a bad binding cannot leave a capture open.
-    for (const auto& op : plan->ops)
-        if (!bindings[op.weight] || !bindings[op.x] || !bindings[op.dst])
+    for (const auto& op : plan->ops) {
+        const bool moe = op.kind == INFR_OP_MOE_FFN;
+        if (!bindings[op.x] || !bindings[op.dst] || (!moe && !bindings[op.weight]) ||
+            (moe && (!bindings[op.router_x] || !bindings[op.router] || !bindings[op.gate_exps] ||
+                     !bindings[op.up_exps] || !bindings[op.down_exps])))
             return fail(be, INFR_HIP_ERR_INVALID, "execute: unbound tensor");
+    }
     if (int rc = schedule_plan(be, plan, bindings)) return rc;
     hipGraph_t graph = nullptr;
     HIP_TRY(be, hipStreamBeginCapture(be->stream, hipStreamCaptureModeThreadLocal));

@@ -75,4 +75,26 @@ bool launch_gemv_fused(int dtype, size_t in_f, const GemvOpDesc* ops, int n, con
 bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
                 size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream);
 
+// Op::MoeFfn (qwen3moe form). Expert e of a bank starts at bank + e * stride.
+struct MoeShape {
+    int ne, n_expert, n_used, n_ff, rows;
+    float scale;
+    int router_dtype, gate_dtype, up_dtype, down_dtype;
+};
+struct MoeBuffers {
+    const float* x;         // [rows, ne]
+    const float* router_x;  // [rows, ne]
+    const float* router;    // f32 [n_expert, ne]
+    const uint8_t* gate;
+    const uint8_t* up;
+    const uint8_t* down;
+    size_t gate_stride, up_stride, down_stride;
+    float* dst;             // [rows, ne]
+    int32_t* sel_idx;       // optional [rows, n_used]
+    float* sel_w;           // optional [rows, n_used]
+};
+size_t moe_workspace_bytes(const MoeShape& s);
+// Enqueues the whole op; returns nullptr or a message naming what is unsupported.
+const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* workspace, hipStream_t stream);
+
 }  // namespace infr

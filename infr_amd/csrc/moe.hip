@@ -1,0 +1,460 @@
+// Op::MoeFfn on the device, as qwen3moe emits it (softmax gating, renormalised top-k, split
+// gate/up banks, SiLU, weights applied to the expert outputs). Mirrors infr-cpu's staged
+// pipeline (crates/infr-cpu/src/lib.rs:2264-2984, crates/infr-cpu/src/moe.rs):
+//
+//   router   f32 router rows . router_x with infr-cpu's `dot` (8 FMA accumulators by index mod 8,
+//            summed in order, kernels.rs:6557-6573), evaluated in that exact order so the logits -
+//            and with them the expert selection - match the CPU bit for bit
+//   select   softmax with max-subtraction, probabilities summed in index order, stable top-n_used
+//            (ties to the lower expert index), w = p / max(sum_sel p, 1e-20) * scale  (lib.rs:2421-2543)
+//   rows == 1   the CPU multiplies DECODED f32 weights with the UNQUANTIZED activation
+//            (ActsKind::Raw, moe.rs:42-53,142-173): gate/up rows are decoded in registers with
+//            dequant_block's two roundings (sc*code + mn), FMA-accumulated against f32 x, SiLU
+//            fused; the down kernel decodes likewise and adds the experts in rank order
+//   rows >= 2   int8 path: x rows quantized per 256 once, id-gathered Q4_K/Q6_K/Q8_0 GEMVs per
+//            (row, expert) pair (the decode GEMV body, bit-identical to the CPU's batch kernels),
+//            SiLU + re-quantization, id-gathered down GEMV, rank-ordered accumulate
+// Only the selected experts' blocks are addressed: every weight pointer is
+// bank + ids[slot] * expert_stride, read on the device.
+#include <algorithm>
+
+#include "gemv_formats.hpp"
+#include "kernels.hpp"
+#include "quant_chunk.hpp"
+
+namespace infr {
+
+// ───────────────────────────── router + selection ─────────────────────────────
+
+// One 8-lane group per (row, expert): lane j owns accumulator j of infr-cpu's `dot`.
+__global__ __launch_bounds__(256) void moe_router_kernel(const float* __restrict__ router,
+                                                         const float* __restrict__ rx,
+                                                         float* __restrict__ logits, int ne,
+                                                         int n_expert, int rows) {
+    const int gid = (blockIdx.x * 256 + threadIdx.x) >> 3, j = threadIdx.x & 7;
+    const bool live = gid < rows * n_expert;
+    const int r = live ? gid / n_expert : 0, e = live ? gid % n_expert : 0;
+    const float* a = router + (size_t)e * ne;
+    const float* b = rx + (size_t)r * ne;
+    const int chunks = ne / 8;
+    float acc = 0.0f;
+    for (int c = 0; c < chunks; ++c) acc = __builtin_fmaf(a[c * 8 + j], b[c * 8 + j], acc);
+    // s = acc[0] + acc[1] + ... + acc[7] in order, then the FMA tail
+    float s = 0.0f;
+    const int base = threadIdx.x & 56;  // first lane of this group within the wave
+#pragma unroll
+    for (int k = 0; k < 8; ++k) s += __shfl(acc, base + k, kWave);
+    for (int i = chunks * 8; i < ne; ++i) s = __builtin_fmaf(a[i], b[i], s);
+    if (live && j == 0) logits[(size_t)r * n_expert + e] = s;
+}
+
+// One wavefront per row. n_expert <= 1024 (16 per lane).
+__global__ __launch_bounds__(64) void moe_select_kernel(const float* __restrict__ logits,
+                                                        int32_t* __restrict__ sel_idx,
+                                                        float* __restrict__ sel_w, int n_expert,
+                                                        int n_used, float scale) {
+    __shared__ float p[1024];
+    __shared__ float red[2];
+    const int r = blockIdx.x, lane = threadIdx.x;
+    const float* l = logits + (size_t)r * n_expert;
+    float mx = -INFINITY;
+    for (int e = lane; e < n_expert; e += 64) mx = __builtin_fmaxf(mx, l[e]);
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) mx = __builtin_fmaxf(mx, __shfl_xor(mx, off, kWave));
+    for (int e = lane; e < n_expert; e += 64) p[e] = expf(l[e] - mx);
+    __syncthreads();
+    if (lane == 0) {  // `p.iter().sum()`: index order
+        float s = 0.0f;
+        for (int e = 0; e < n_expert; ++e) s += p[e];
+        red[0] = s;
+    }
+    __syncthreads();
+    const float psum = red[0];
+    for (int e = lane; e < n_expert; e += 64) p[e] = p[e] / psum;
+    __syncthreads();
+    // stable descending top-n_used: largest p, lowest index among equals, n_used times
+    float wsum = 0.0f;
+    float my_w = 0.0f;
+    int my_e = 0;
+    for (int k = 0; k < n_used; ++k) {
+        float bv = -INFINITY;
+        int bi = 0x7FFFFFFF;
+        for (int e = lane; e < n_expert; e += 64) {
+            const float v = p[e];
+            if (v > bv || (v == bv && e < bi)) {
+                bv = v;
+                bi = e;
+            }
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            const float ov = __shfl_xor(bv, off, kWave);
+            const int oi = __shfl_xor(bi, off, kWave);
+            if (ov > bv || (ov == bv && oi < bi)) {
+                bv = ov;
+                bi = oi;
+            }
+        }
+        wsum += bv;  // selection order = the CPU's summation order
+        if (lane == k % 64) {
+            my_w = bv;
+            my_e = bi;
+        }
+        if (lane == 0) p[bi] = -1.0f;  // taken (probabilities are >= 0)
+        __syncthreads();
+        // n_used > 64 would need several values per lane; the launcher rejects it
+    }
+    wsum = __builtin_fmaxf(wsum, 1e-20f);
+    if (lane < n_used) {
+        sel_idx[(size_t)r * n_used + lane] = my_e;
+        sel_w[(size_t)r * n_used + lane] = my_w / wsum * scale;
+    }
+}
+
+// ───────────────────────────── rows == 1: f32 (ActsKind::Raw) path, Q4_K banks ─────────────────────────────
+// Lane mapping: 4 lanes per 256-block (nibble pair p = lane % 4, 64 weights), S = 4 * nb lanes per
+// weight row, 64 / S rows per wave step. A lane keeps its 64 activation floats in registers.
+
+struct Q4kF32Row {
+    v4i hdr, qa, qb;
+};
+
+__device__ __forceinline__ float q4k_f32_partial(const Q4kF32Row& r, const float* x, int p) {
+    uint32_t sc8[2], mn8[2];
+    k4_all((uint32_t)r.hdr.y, (uint32_t)r.hdr.z, (uint32_t)r.hdr.w, sc8, mn8);
+    const uint32_t scw = (p & 2) ? sc8[1] : sc8[0];
+    const uint32_t mnw = (p & 2) ? mn8[1] : mn8[0];
+    const int sh = (p & 1) * 16;
+    const float d = f16_bits_to_f32((uint32_t)r.hdr.x & 0xFFFFu);
+    const float dmin = f16_bits_to_f32((uint32_t)r.hdr.x >> 16);
+    // dequant_block: sc = f32(d) * (f32)scm_sc; mn = f32(dmin) * (f32)(-m); w = sc * code + mn
+    const float fs_e = d * (float)(int)((scw >> sh) & 0xFF), fs_o = d * (float)(int)((scw >> (sh + 8)) & 0xFF);
+    const float fm_e = dmin * (float)(-(int)((mnw >> sh) & 0xFF)), fm_o = dmin * (float)(-(int)((mnw >> (sh + 8)) & 0xFF));
+    const int wq[8] = {r.qa.x, r.qa.y, r.qa.z, r.qa.w, r.qb.x, r.qb.y, r.qb.z, r.qb.w};
+    float acc = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const uint32_t w = (uint32_t)wq[k];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float qe = (float)((w >> (8 * i)) & 0xF), qo = (float)((w >> (8 * i + 4)) & 0xF);
+            const float we = fs_e * qe + fm_e, wo = fs_o * qo + fm_o;
+            acc = __builtin_fmaf(we, x[4 * k + i], acc);
+            acc = __builtin_fmaf(wo, x[32 + 4 * k + i], acc);
+        }
+    }
+    return acc;
+}
+
+__device__ __forceinline__ void q4k_f32_load(Q4kF32Row& r, const uint8_t* rowp, int b, int p, bool ok) {
+    if (ok) {
+        const uint8_t* blk = rowp + (size_t)b * 144;
+        r.hdr = load16(blk);
+        r.qa = load16(blk + 16 + p * 32);
+        r.qb = load16(blk + 32 + p * 32);
+    } else {
+        r.hdr = r.qa = r.qb = v4i{0, 0, 0, 0};
+    }
+}
+
+// Sum over the S = 4*nb lanes of a row segment; every lane of the segment gets the total.
+__device__ __forceinline__ float seg_sum(float v, int seg_base, int nb) {
+    v += __builtin_bit_cast(float, quad_xor1(__builtin_bit_cast(int, v)));
+    v += __builtin_bit_cast(float, quad_xor2(__builtin_bit_cast(int, v)));
+    float s = 0.0f;
+    for (int i = 0; i < nb; ++i) s += __shfl(v, seg_base + 4 * i, kWave);
+    return s;
+}
+
+// gate/up: act[slot][o] = silu(gate_e[o] . x) * (up_e[o] . x), e = ids[slot]
+__global__ __launch_bounds__(256) void moe_gate_up_f32_q4k_kernel(
+    const uint8_t* __restrict__ gate, const uint8_t* __restrict__ up, size_t gate_stride,
+    size_t up_stride, const int32_t* __restrict__ ids, const float* __restrict__ x,
+    float* __restrict__ act, int ne, int nff) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nb = ne / 256, S = 4 * nb, rps = 64 / S;  // rows per wave step
+    const int seg = lane / S, within = lane % S, b = within >> 2, p = within & 3;
+    const bool lane_ok = seg < rps;
+    const int slot = blockIdx.y;
+    const int e = ids[slot];
+    const size_t bpr = (size_t)nb * 144;
+    const uint8_t* gw = gate + (size_t)e * gate_stride;
+    const uint8_t* uw = up + (size_t)e * up_stride;
+
+    float xr[64];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+        v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (lane_ok) v = *reinterpret_cast<const v4f*>(x + (size_t)b * 256 + p * 64 + 4 * k);
+        xr[4 * k + 0] = v.x; xr[4 * k + 1] = v.y; xr[4 * k + 2] = v.z; xr[4 * k + 3] = v.w;
+    }
+    // each wave takes row steps wave, wave+4*gridDim.x... within this block's range
+    const int steps_total = (nff + rps - 1) / rps;
+    for (int st = blockIdx.x * 4 + wave; st < steps_total; st += gridDim.x * 4) {
+        const int o = st * rps + seg;
+        const bool ok = lane_ok && o < nff;
+        Q4kF32Row g, u;
+        q4k_f32_load(g, gw + (size_t)(ok ? o : 0) * bpr, b, p, ok);
+        q4k_f32_load(u, uw + (size_t)(ok ? o : 0) * bpr, b, p, ok);
+        const float gs = seg_sum(q4k_f32_partial(g, xr, p), seg * S, nb);
+        const float us = seg_sum(q4k_f32_partial(u, xr, p), seg * S, nb);
+        if (ok && within == 0) act[(size_t)slot * nff + o] = gs / (1.0f + expf(-gs)) * us;
+    }
+}
+
+// down + accumulate: out[o] = sum_k w_k * (down_{ids[k]}[o] . act[k]), k in rank order
+__global__ __launch_bounds__(256) void moe_down_f32_q4k_kernel(
+    const uint8_t* __restrict__ down, size_t down_stride, const int32_t* __restrict__ ids,
+    const float* __restrict__ wts, const float* __restrict__ act, float* __restrict__ out, int nff,
+    int ne, int n_used) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nb = nff / 256, S = 4 * nb, rps = 64 / S;
+    const int seg = lane / S, within = lane % S, b = within >> 2, p = within & 3;
+    const bool lane_ok = seg < rps;
+    const size_t bpr = (size_t)nb * 144;
+    const int st = blockIdx.x * 4 + wave;  // one row step per wave
+    const int o = st * rps + seg;
+    const bool ok = lane_ok && o < ne;
+    float acc = 0.0f;
+    for (int k = 0; k < n_used; ++k) {
+        const uint8_t* dw = down + (size_t)ids[k] * down_stride;
+        Q4kF32Row r;
+        q4k_f32_load(r, dw + (size_t)(ok ? o : 0) * bpr, b, p, ok);
+        float xr[64];
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {
+            v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (lane_ok) v = *reinterpret_cast<const v4f*>(act + (size_t)k * nff + (size_t)b * 256 + p * 64 + 4 * q);
+            xr[4 * q + 0] = v.x; xr[4 * q + 1] = v.y; xr[4 * q + 2] = v.z; xr[4 * q + 3] = v.w;
+        }
+        const float yk = seg_sum(q4k_f32_partial(r, xr, p), seg * S, nb);
+        acc += wts[k] * yk;  // `*o += w_e * yv`: separate multiply and add, rank order
+    }
+    if (ok && within == 0) out[o] = acc;
+}
+
+// ───────────────────────────── rows >= 2: int8 path ─────────────────────────────
+
+// id-gathered decode GEMV over pre-quantized activation rows: pair = blockIdx.y,
+// weights = bank + ids[pair] * expert_stride, activation row = pair / n_used.
+template <typename F, int STEPS>
+__global__ __launch_bounds__(256) void gemv_id_kernel(const uint8_t* __restrict__ bank,
+                                                      size_t expert_stride, size_t bpr,
+                                                      const int32_t* __restrict__ ids, ActPtrs act,
+                                                      int in_f, int n_used, float* __restrict__ y,
+                                                      int out_f, int rows_per_wave) {
+    const int lane = threadIdx.x & 63;
+    const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int row0 = wave * rows_per_wave;
+    if (row0 >= out_f) return;
+    const int row_end = min(row0 + rows_per_wave, out_f);
+    const int pair = blockIdx.y, r = pair / n_used;
+    const uint8_t* w = bank + (size_t)ids[pair] * expert_stride;
+    const int n_units = F::units(in_f);
+    ActPtrs a;
+    a.qs = act.qs + (size_t)r * in_f;
+    a.d = act.d + (size_t)r * (in_f / 256);
+    a.bsums = act.bsums + (size_t)r * (in_f / 32);
+    a.bsums16 = act.bsums16 + (size_t)r * (in_f / 16);
+    typename F::Acts acts[STEPS];
+    typename F::Row cur[STEPS];
+    bool ok[STEPS];
+#pragma unroll
+    for (int t = 0; t < STEPS; ++t) {
+        ok[t] = F::valid(t, lane, n_units);
+        F::load_row(cur[t], w + (size_t)row0 * bpr, t, lane, ok[t]);
+        F::load_acts(acts[t], a, t, lane, ok[t]);
+    }
+    // same body as the decode GEMV (gemv.hip): per-block exact integers, CPU-ordered f32 sum
+    typename F::Row nxt[STEPS];
+    float* yo = y + (size_t)pair * out_f;
+    for (int row = row0; row < row_end; ++row) {
+        if (row + 1 < row_end) {
+#pragma unroll
+            for (int t = 0; t < STEPS; ++t) F::load_row(nxt[t], w + (size_t)(row + 1) * bpr, t, lane, ok[t]);
+        }
+        float s = 0.0f;
+#pragma unroll
+        for (int t = 0; t < STEPS; ++t) {
+            const float term = F::template term<false>(cur[t], acts[t], t, lane, ok[t],
+                                                       StagePtrs{nullptr, nullptr}, 0);
+            if (F::kOrdered) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) s += readlane_f(term, 4 * i);
+            } else {
+                s += term;
+            }
+        }
+        if (!F::kOrdered) s = wave_sum_f(s);
+        if (lane == 0) yo[row] = s;
+#pragma unroll
+        for (int t = 0; t < STEPS; ++t) cur[t] = nxt[t];
+    }
+}
+
+// act = silu(g) * u per pair row, quantized per 256 for the down bank (lib.rs:2824-2892).
+// One wavefront per 256-float chunk.
+__global__ __launch_bounds__(256) void moe_act_quant_kernel(const float* __restrict__ g,
+                                                            const float* __restrict__ u,
+                                                            int8_t* __restrict__ qs,
+                                                            float* __restrict__ d,
+                                                            int32_t* __restrict__ bsums,
+                                                            int32_t* __restrict__ bsums16,
+                                                            size_t n_elems) {
+    const int lane = threadIdx.x & 63;
+    const size_t chunk = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (chunk * 256 >= n_elems) return;
+    const v4f gv = *reinterpret_cast<const v4f*>(g + chunk * 256 + (size_t)lane * 4);
+    const v4f uv = *reinterpret_cast<const v4f*>(u + chunk * 256 + (size_t)lane * 4);
+    v4f a;
+    a.x = gv.x / (1.0f + expf(-gv.x)) * uv.x;
+    a.y = gv.y / (1.0f + expf(-gv.y)) * uv.y;
+    a.z = gv.z / (1.0f + expf(-gv.z)) * uv.z;
+    a.w = gv.w / (1.0f + expf(-gv.w)) * uv.w;
+    quantize_chunk<false>(a, true, lane, chunk, qs, d, bsums, bsums16);
+}
+
+// out[r][o] = sum_k w[r][k] * yp[r*n_used + k][o], k in rank order (lib.rs:2967-2983)
+__global__ __launch_bounds__(256) void moe_accumulate_kernel(const float* __restrict__ yp,
+                                                             const float* __restrict__ wts,
+                                                             float* __restrict__ out, int ne,
+                                                             int n_used, int rows) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (size_t)rows * ne) return;
+    const size_t r = i / ne, o = i % ne;
+    float acc = 0.0f;
+    for (int k = 0; k < n_used; ++k)
+        acc += wts[r * n_used + k] * yp[(r * n_used + k) * ne + o];
+    out[i] = acc;
+}
+
+// ───────────────────────────── launch ─────────────────────────────
+
+template <typename F>
+static bool launch_gemv_id_fmt(const uint8_t* bank, size_t expert_stride, size_t bpr,
+                               const int32_t* ids, const ActQ8& act, size_t in_f, int n_used,
+                               int pairs, float* y, size_t out_f, hipStream_t stream) {
+    const int steps = (int)((in_f + F::kElemsPerStep - 1) / F::kElemsPerStep);
+    const int rpw = 2;
+    const size_t waves = (out_f + rpw - 1) / rpw;
+    const dim3 grid((unsigned)((waves + 3) / 4), (unsigned)pairs), block(256);
+    const ActPtrs a{act.qs, act.d, act.bsums, act.bsums16};
+#define INFR_CASE(N)                                                                               \
+    case N:                                                                                        \
+        hipLaunchKernelGGL((gemv_id_kernel<F, N>), grid, block, 0, stream, bank, expert_stride, bpr, \
+                           ids, a, (int)in_f, n_used, y, (int)out_f, rpw);                         \
+        return true;
+    switch (steps) {
+        INFR_CASE(1) INFR_CASE(2) INFR_CASE(3) INFR_CASE(4)
+    default: return false;
+    }
+#undef INFR_CASE
+}
+
+static bool launch_gemv_id(int dtype, const uint8_t* bank, size_t expert_stride, size_t bpr,
+                           const int32_t* ids, const ActQ8& act, size_t in_f, int n_used, int pairs,
+                           float* y, size_t out_f, hipStream_t stream) {
+    switch (dtype) {
+    case 12: return launch_gemv_id_fmt<FmtQ4K>(bank, expert_stride, bpr, ids, act, in_f, n_used, pairs, y, out_f, stream);
+    case 14: return launch_gemv_id_fmt<FmtQ6K>(bank, expert_stride, bpr, ids, act, in_f, n_used, pairs, y, out_f, stream);
+    case 8: return launch_gemv_id_fmt<FmtQ8_0>(bank, expert_stride, bpr, ids, act, in_f, n_used, pairs, y, out_f, stream);
+    default: return false;
+    }
+}
+
+size_t moe_workspace_bytes(const MoeShape& s) {
+    const size_t pairs = (size_t)s.rows * s.n_used;
+    size_t n = 0;
+    auto add = [&n](size_t bytes) { n += (bytes + 255) / 256 * 256; };
+    add((size_t)s.rows * s.n_expert * 4);        // logits
+    add(pairs * 4);                               // sel_idx
+    add(pairs * 4);                               // sel_w
+    add(pairs * s.n_ff * 4);                      // gate out / act (rows == 1: act)
+    add(pairs * s.n_ff * 4);                      // up out
+    add(pairs * s.ne * 4);                        // per-pair down outputs
+    const size_t qmax = std::max((size_t)s.rows * s.ne, pairs * s.n_ff);
+    add(qmax);                                    // int8 activations
+    add(qmax / 32 * 4);                           // d (sized for either quantizer)
+    add(qmax / 32 * 4);                           // bsums
+    add(qmax / 16 * 4);                           // bsums16
+    return n;
+}
+
+const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hipStream_t stream) {
+    if (s.router_dtype != 0) return "router dtype must be F32";
+    if (s.n_used > 64 || s.n_expert > 1024 || s.n_used > s.n_expert) return "n_used <= 64 and n_expert <= 1024 required";
+    if (s.ne % 256 != 0 || s.n_ff % 256 != 0) return "ne and n_ff_exp must be multiples of 256";
+    const size_t pairs = (size_t)s.rows * s.n_used;
+    uint8_t* p = static_cast<uint8_t*>(ws);
+    auto take = [&p](size_t bytes) {
+        uint8_t* r = p;
+        p += (bytes + 255) / 256 * 256;
+        return r;
+    };
+    float* logits = (float*)take((size_t)s.rows * s.n_expert * 4);
+    int32_t* sel_idx = (int32_t*)take(pairs * 4);
+    float* sel_w = (float*)take(pairs * 4);
+    float* gbuf = (float*)take(pairs * s.n_ff * 4);
+    float* ubuf = (float*)take(pairs * s.n_ff * 4);
+    float* yp = (float*)take(pairs * s.ne * 4);
+    const size_t qmax = std::max((size_t)s.rows * s.ne, pairs * s.n_ff);
+    ActQ8 aq;
+    aq.qs = (int8_t*)take(qmax);
+    aq.d = (float*)take(qmax / 32 * 4);
+    aq.bsums = (int32_t*)take(qmax / 32 * 4);
+    aq.bsums16 = (int32_t*)take(qmax / 16 * 4);
+
+    const int groups = s.rows * s.n_expert;
+    hipLaunchKernelGGL(moe_router_kernel, dim3((unsigned)((groups * 8 + 255) / 256)), dim3(256), 0, stream,
+                       b.router, b.router_x, logits, s.ne, s.n_expert, s.rows);
+    hipLaunchKernelGGL(moe_select_kernel, dim3((unsigned)s.rows), dim3(64), 0, stream, logits, sel_idx,
+                       sel_w, s.n_expert, s.n_used, s.scale);
+    if (b.sel_idx) (void)hipMemcpyAsync(b.sel_idx, sel_idx, pairs * 4, hipMemcpyDeviceToDevice, stream);
+    if (b.sel_w) (void)hipMemcpyAsync(b.sel_w, sel_w, pairs * 4, hipMemcpyDeviceToDevice, stream);
+
+    if (s.rows == 1) {
+        // ActsKind::Raw for every bank (lib.rs:2359: int8_ok = rows >= 2)
+        if (s.gate_dtype != 12 || s.up_dtype != 12 || s.down_dtype != 12)
+            return "rows == 1 carries Q4_K expert banks only";
+        if (s.ne > 4096 || s.n_ff > 4096) return "rows == 1 needs ne, n_ff_exp <= 4096";
+        const int nb_g = s.ne / 256, rps_g = 64 / (4 * nb_g);
+        const int steps_g = (s.n_ff + rps_g - 1) / rps_g;
+        hipLaunchKernelGGL(moe_gate_up_f32_q4k_kernel, dim3((unsigned)((steps_g + 3) / 4), (unsigned)s.n_used),
+                           dim3(256), 0, stream, b.gate, b.up, b.gate_stride, b.up_stride, sel_idx, b.x,
+                           gbuf, s.ne, s.n_ff);
+        const int nb_d = s.n_ff / 256, rps_d = 64 / (4 * nb_d);
+        const int steps_d = (s.ne + rps_d - 1) / rps_d;
+        hipLaunchKernelGGL(moe_down_f32_q4k_kernel, dim3((unsigned)((steps_d + 3) / 4)), dim3(256), 0, stream,
+                           b.down, b.down_stride, sel_idx, sel_w, gbuf, b.dst, s.n_ff, s.ne, s.n_used);
+        return hipGetLastError() == hipSuccess ? nullptr : "kernel launch failed";
+    }
+
+    // rows >= 2: ActsKind::Super for Q4K/Q6K/Q8_0 banks with in_f % 256 == 0 (moe.rs:42-53)
+    auto bytes_per_row = [](int dtype, size_t in_f) -> size_t {
+        switch (dtype) {
+        case 12: return in_f / 256 * 144;
+        case 14: return in_f / 256 * 210;
+        case 8: return in_f / 32 * 34;
+        default: return 0;
+        }
+    };
+    const size_t gbpr = bytes_per_row(s.gate_dtype, s.ne), ubpr = bytes_per_row(s.up_dtype, s.ne);
+    const size_t dbpr = bytes_per_row(s.down_dtype, s.n_ff);
+    if (!gbpr || !ubpr || !dbpr) return "rows >= 2 carries Q4_K / Q6_K / Q8_0 expert banks";
+    launch_quantize_q8(b.x, s.rows, s.ne, false, aq, stream);
+    if (!launch_gemv_id(s.gate_dtype, b.gate, b.gate_stride, gbpr, sel_idx, aq, s.ne, s.n_used, (int)pairs, gbuf, s.n_ff, stream) ||
+        !launch_gemv_id(s.up_dtype, b.up, b.up_stride, ubpr, sel_idx, aq, s.ne, s.n_used, (int)pairs, ubuf, s.n_ff, stream))
+        return "no id-gathered kernel for this gate/up shape";
+    const size_t n_act = pairs * s.n_ff;
+    hipLaunchKernelGGL(moe_act_quant_kernel, dim3((unsigned)((n_act / 256 + 3) / 4)), dim3(256), 0, stream,
+                       gbuf, ubuf, aq.qs, aq.d, aq.bsums, aq.bsums16, n_act);
+    // the down GEMV's activation row is the pair itself: n_used = 1
+    if (!launch_gemv_id(s.down_dtype, b.down, b.down_stride, dbpr, sel_idx, aq, s.n_ff, 1, (int)pairs, yp, s.ne, stream))
+        return "no id-gathered kernel for this down shape";
+    const size_t n_out = (size_t)s.rows * s.ne;
+    hipLaunchKernelGGL(moe_accumulate_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, stream,
+                       yp, sel_w, b.dst, s.ne, s.n_used, s.rows);
+    return hipGetLastError() == hipSuccess ? nullptr : "kernel launch failed";
+}
+
+}  // namespace infr

@@ -1,0 +1,88 @@
+"""GPU parity of Op::MoeFfn against the CPU oracle, through the C ABI.
+
+rows == 1 takes the f32 (decoded weights x unquantized activation) path like infr-cpu; rows >= 2
+the int8 path. Router logits are evaluated in the CPU's FMA order, so the selected experts must
+be identical; outputs are gated at rel-L2 <= 1e-4 and max-abs <= 1e-3 * max|y| (SiLU/softmax use
+the platform's expf on either side, so the last bits may differ).
+"""
+import numpy as np
+import pytest
+
+from infr_amd import DType, synth_normal_f32, synth_weight
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def banks(seed, ne, n_expert, nff, dtype=DType.Q4K, sigma=0.02):
+    gate = synth_weight(dtype, seed, n_expert * nff, ne, sigma)
+    up = synth_weight(dtype, seed + 1, n_expert * nff, ne, sigma)
+    down = synth_weight(dtype, seed + 2, n_expert * ne, nff, sigma)
+    return gate, up, down
+
+
+def run_moe(be, x, router, gate, up, down, rows, ne, n_expert, n_used, nff, scale, dtype=DType.Q4K):
+    xb, rb = be.upload_new(x), be.upload_new(router)
+    gb, ub, db = be.upload_new(gate), be.upload_new(up), be.upload_new(down)
+    yb = be.alloc(rows * ne * 4)
+    ib, wb = be.alloc(rows * n_used * 4), be.alloc(rows * n_used * 4)
+    be.moe_ffn(xb, rb, gb, ub, db, yb, rows=rows, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
+               scale=scale, gate_dtype=dtype, up_dtype=dtype, down_dtype=dtype, sel_idx=ib, sel_w=wb)
+    return (be.download(yb, np.empty((rows, ne), np.float32)),
+            be.download(ib, np.empty((rows, n_used), np.int32)),
+            be.download(wb, np.empty((rows, n_used), np.float32)))
+
+
+def check(y, idx, w, oy, oidx, ow):
+    assert np.array_equal(idx, oidx), "expert selection differs"
+    assert np.allclose(w, ow, rtol=1e-5, atol=0)
+    a, b = y.astype(np.float64).ravel(), oy.astype(np.float64).ravel()
+    assert np.abs(b).max() > 1e-4
+    rel = np.linalg.norm(a - b) / np.linalg.norm(b)
+    mx = np.abs(a - b).max() / np.abs(b).max()
+    assert rel <= 1e-4 and mx <= 1e-3, f"rel-L2 {rel:.3e} max-abs {mx:.3e}"
+
+
+@pytest.mark.parametrize("rows", [1, 2, 5])
+@pytest.mark.parametrize("ne,n_expert,n_used,nff", [(512, 16, 4, 256), (1024, 8, 2, 768)])
+def test_moe_small_shapes(be, rows, ne, n_expert, n_used, nff):
+    gate, up, down = banks(50 + rows, ne, n_expert, nff, sigma=0.05)
+    x = synth_normal_f32(60 + rows, rows * ne)
+    router = synth_normal_f32(61, n_expert * ne, sigma=0.05)
+    got = run_moe(be, x, router, gate, up, down, rows, ne, n_expert, n_used, nff, 1.25)
+    want = orc.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff, scale=1.25)
+    check(*got, *want)
+
+
+@pytest.mark.parametrize("rows", [1, 16])
+def test_moe_qwen3_30b_a3b_shape(be, rows):
+    # 128 experts, top-8, hidden 2048, expert FFN 768, Q4_K banks
+    ne, n_expert, n_used, nff = 2048, 128, 8, 768
+    gate, up, down = banks(7, ne, n_expert, nff)
+    x = synth_normal_f32(8 + rows, rows * ne)
+    router = synth_normal_f32(9, n_expert * ne, sigma=0.03)   # logits ~ N(0, ~1.4^2)
+    got = run_moe(be, x, router, gate, up, down, rows, ne, n_expert, n_used, nff, 1.0)
+    want = orc.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff)
+    check(*got, *want)
+
+
+def test_moe_router_ties_go_to_the_lower_index(be):
+    ne, n_expert, n_used, nff = 256, 6, 3, 256
+    gate, up, down = banks(90, ne, n_expert, nff, sigma=0.05)
+    x = np.ones(ne, np.float32)
+    router = np.zeros((n_expert, ne), np.float32)
+    router[4] = 0.01
+    _, idx, _ = run_moe(be, x, router, gate, up, down, 1, ne, n_expert, n_used, nff, 1.0)
+    assert list(idx[0]) == [4, 0, 1]
+
+
+@pytest.mark.parametrize("dtype", [DType.Q6K, DType.Q8_0])
+def test_moe_int8_path_other_bank_formats(be, dtype):
+    rows, ne, n_expert, n_used, nff = 3, 512, 8, 2, 256
+    gate, up, down = banks(120, ne, n_expert, nff, dtype, sigma=0.05)
+    x = synth_normal_f32(121, rows * ne)
+    router = synth_normal_f32(122, n_expert * ne, sigma=0.05)
+    got = run_moe(be, x, router, gate, up, down, rows, ne, n_expert, n_used, nff, 1.0, dtype)
+    want = orc.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
+                       gate_dtype=int(dtype), up_dtype=int(dtype), down_dtype=int(dtype))
+    check(*got, *want)
