@@ -162,6 +162,58 @@ def single_shape(be, dtype, m, in_f, out_f, reps=40, rotate_bytes=768 << 20):
     return best / reps, nb
 
 
+def moe_bench(be, n_layers=6):
+    """Routed-expert MoE at the Qwen3-30B-A3B shape (128 experts, top-8, hidden 2048, expert FFN
+    768, Q4_K banks), 1 and 16 tokens: `n_layers` Op::MoeFfn with distinct banks in one plan, so
+    the experts stream from HBM. Bytes = 2,654,208 per selected expert (gate+up+down)."""
+    from infr_amd import Bindings, BufferUsage, DType, Graph, MoeFfn, TensorDesc, synth_normal_f32, synth_weight
+    ne, n_expert, n_used, nff = 2048, 128, 8, 768
+    per_expert = 3 * nff * ne * 144 // 256
+    protos = [be.upload_new(synth_weight(DType.Q4K, 70 + i, n_expert * (nff if i < 2 else ne),
+                                         ne if i < 2 else nff), BufferUsage.Weights) for i in range(3)]
+    router = be.upload_new(synth_normal_f32(80, n_expert * ne, sigma=0.03))
+    out, keep = {}, list(protos) + [router]
+    for rows in (1, 16):
+        g, binds = Graph(), Bindings()
+        x = synth_normal_f32(81 + rows, rows * ne)
+        xid = g.input(TensorDesc((rows, ne), DType.F32))
+        rid = g.weight(TensorDesc((n_expert, ne), DType.F32))
+        binds.bind(xid, be.upload_new(x)).bind(rid, router)
+        for layer in range(n_layers):
+            ids = []
+            for i, proto in enumerate(protos):
+                nb = proto.len_bytes()
+                wb = proto if layer == 0 else be.alloc_uninit(nb, BufferUsage.Weights)
+                if layer:
+                    be.copy_buffer(proto, wb, nb)
+                    keep.append(wb)
+                shape = (n_expert, nff, ne) if i < 2 else (n_expert, ne, nff)
+                wid = g.weight(TensorDesc(shape, DType.Q4K))
+                binds.bind(wid, wb)
+                ids.append(wid)
+            yid = g.output(TensorDesc((rows, ne), DType.F32))
+            yb = be.alloc(rows * ne * 4)
+            keep.append(yb)
+            binds.bind(yid, yb)
+            g.push(MoeFfn(xid, xid, rid, ids[0], ids[1], ids[2], yid, ne, n_expert, n_used, nff, 1.0))
+        plan = be.compile(g)
+        be.execute(plan, binds)
+        be.sync()
+        best = 1e30
+        for _ in range(3):
+            be.timer_begin()
+            be.execute(plan, binds)
+            best = min(best, be.timer_end())
+        us = best * 1e3 / n_layers
+        # every layer routes the same x through the same router: unique experts per layer
+        out[f"moe_q4k_t{rows}_us_per_layer"] = round(us, 2)
+        out[f"moe_q4k_t{rows}_pair_GBs"] = round(rows * n_used * per_expert / (us * 1e-6) / 1e9, 1)
+        plan = None
+    for b in keep:
+        b.free()
+    return out
+
+
 def cpu_baseline(dtype_name="Q4_K"):
     """The CPU oracle (C restatement of infr-cpu's scalar kernels, OpenMP over output rows with the
     reference's 16-row grain) on a bounded sample of the headline workload: one layer's seven
@@ -195,8 +247,8 @@ def main():
     ap.add_argument("--layers", type=int, default=N_LAYERS)
     ap.add_argument("--no-extra", action="store_true", help="headline sweep only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--sections", default="shapes,mmq,ternary",
-                    help="comma list of secondary sections: shapes, mmq, ternary")
+    ap.add_argument("--sections", default="shapes,mmq,ternary,moe",
+                    help="comma list of secondary sections: shapes, mmq, ternary, moe")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
@@ -211,22 +263,24 @@ def main():
     dev_ms, wall_ms = sw.time(args.steps, args.warmup)
     ms = max(dev_ms, wall_ms)
     value = sw.bytes / (ms * 1e-3) / 1e9
-    avg_launch_us = dev_ms * 1e3 / sw.launches
-    achieved = (sw.bytes / sw.launches) / (avg_launch_us * 1e-6) / 1e9
+    n_launch = max(1, sw.plan.launches())          # grouped: independent ops share a launch
+    avg_launch_us = dev_ms * 1e3 / n_launch
+    achieved = (sw.bytes / n_launch) / (avg_launch_us * 1e-6) / 1e9
     out = {
         "metric": "Q4_K GEMV HBM GB/s (% of peak) + prefill mmq int8 TOPS at M=512",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "i8", "data": "synthetic",
         "config": {"workload": f"Q4_K decode GEMV sweep, Qwen3-8B layer shapes x {args.layers} layers "
-                               f"({sw.launches} distinct matrices, {sw.bytes / 1e9:.2f} GB), batch 1",
+                               f"({sw.launches} independent Op::Linear over distinct matrices, "
+                               f"{sw.bytes / 1e9:.2f} GB, one plan), batch 1",
                    "weights": "N(0,0.02^2) seed 0 -> Q4_K", "activations": "N(0,1) f32, quantized on GPU",
                    "device": caps["device_name"], "compute_units": caps["compute_units"]},
         "pct_of_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "roofline": {"bound": "hbm", "kernel": "gemv_q4k", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": None, "avg_launch_us": round(avg_launch_us, 3),
-                     "bytes_per_launch": sw.bytes // sw.launches},
+                     "launches_per_step": n_launch, "bytes_per_launch": sw.bytes // n_launch},
     }
     sw.free()
 
@@ -250,6 +304,8 @@ def main():
         extra["ternary_Q2_0_sweep_GBs"] = round(tern.bytes / (tms * 1e-3) / 1e9, 1)
         extra["ternary_Q2_0_tok_s_equiv"] = round(1e3 / tms, 1)
         tern.free()
+    if "moe" in sections:
+        extra.update(moe_bench(be))
     out["extra"] = extra
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline()

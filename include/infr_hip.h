@@ -194,6 +194,9 @@ void infr_hip_plan_free(infr_hip_t *be, infr_hip_plan_t *plan);
  * Asynchronous: results are visible after infr_hip_sync or a download. */
 int infr_hip_execute(infr_hip_t *be, infr_hip_plan_t *plan, infr_hip_buffer_t *const *bindings,
                      size_t n_bindings);
+/* Number of kernel launches one execute of this plan issues for the bindings it last ran with
+ * (0 before the first execute). Independent decode ops of one dependency level share a launch. */
+size_t infr_hip_plan_launches(const infr_hip_plan_t *plan);
 
 /* ---- shutdown latch (crates/infr-core/src/shutdown.rs:30-60): once requested, compute entry
  * points enqueue nothing further and return INFR_HIP_ERR_ABORTED; work already enqueued drains.

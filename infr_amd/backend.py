@@ -115,6 +115,7 @@ SYMBOLS = {
     "infr_hip_compile": (C.c_int, [_vp, C.POINTER(_Op), C.c_size_t, C.POINTER(_vp)]),
     "infr_hip_plan_free": (None, [_vp, _vp]),
     "infr_hip_execute": (C.c_int, [_vp, _vp, C.POINTER(_vp), C.c_size_t]),
+    "infr_hip_plan_launches": (C.c_size_t, [_vp]),
     "infr_hip_request_shutdown": (C.c_int, [C.c_int]),
     "infr_hip_shutdown_requested": (C.c_int, []),
     "infr_hip_shutdown_signal": (C.c_int, []),
@@ -290,6 +291,10 @@ class Bindings:
 class Plan:
     def __init__(self, be: "HipBackend", handle: int, graph: Graph):
         self._be, self._h, self.graph = be, handle, graph
+
+    def launches(self) -> int:
+        """Kernel launches per execute for the bindings last run with."""
+        return load_library().infr_hip_plan_launches(self._h)
 
     def __del__(self):
         try:

@@ -588,6 +588,17 @@ int infr_hip_compile(infr_hip_t* be, const infr_hip_op_t* ops, size_t n_ops, inf
     return INFR_HIP_OK;
 }
 
+size_t infr_hip_plan_launches(const infr_hip_plan_t* plan) {
+    if (!plan) return 0;
+    size_t n = 0;
+    for (const auto& st : plan->steps) {
+        if (st.op < 0) n += 1;                                             // grouped decode launch
+        else if (plan->ops[st.op].kind == INFR_OP_MOE_FFN) n += plan->ops[st.op].moe.rows == 1 ? 4 : 8;
+        else n += 2;                                                       // quantize + GEMM
+    }
+    return n;
+}
+
 void infr_hip_plan_free(infr_hip_t* be, infr_hip_plan_t* plan) {
     if (!plan) return;
     if (be && be->stream) (void)hipStreamSynchronize(be->stream);

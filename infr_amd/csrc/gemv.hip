@@ -25,46 +25,11 @@
 #include <cstdlib>
 
 #include "gemv_formats.hpp"
+#include "gemv_rows.hpp"
 #include "kernels.hpp"
 #include "quant_chunk.hpp"
 
 namespace infr {
-
-// Rows [row0, row_end) of one weight matrix against activation registers `acts`. `cur` already
-// holds row0 (the caller issues those loads as early as it can).
-template <typename F, int STEPS, bool STAGES>
-__device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t bpr,
-                                          typename F::Row (&cur)[STEPS],
-                                          const typename F::Acts (&acts)[STEPS],
-                                          const bool (&ok)[STEPS], float* __restrict__ y, int n_units,
-                                          int row0, int row_end, int lane, const StagePtrs& st) {
-    typename F::Row nxt[STEPS];
-    for (int row = row0; row < row_end; ++row) {
-        if (row + 1 < row_end) {
-            const uint8_t* rowp = w + (size_t)(row + 1) * bpr;
-#pragma unroll
-            for (int t = 0; t < STEPS; ++t) F::load_row(nxt[t], rowp, t, lane, ok[t]);
-        }
-        float s = 0.0f;
-#pragma unroll
-        for (int t = 0; t < STEPS; ++t) {
-            const float term = F::template term<STAGES>(cur[t], acts[t], t, lane, ok[t], st,
-                                                        (size_t)row * n_units);
-            if (F::kOrdered) {
-                // Ascending block order, one add per block: the CPU's `sumf +=` chain. Lanes
-                // past the row's last block hold +0.0, which leaves the sum unchanged.
-#pragma unroll
-                for (int i = 0; i < 16; ++i) s += readlane_f(term, 4 * i);
-            } else {
-                s += term;
-            }
-        }
-        if (!F::kOrdered) s = wave_sum_f(s);
-        if (lane == 0) y[row] = s;
-#pragma unroll
-        for (int t = 0; t < STEPS; ++t) cur[t] = nxt[t];
-    }
-}
 
 template <typename F, int STEPS, bool STAGES>
 __global__ __launch_bounds__(256) void gemv_kernel(const uint8_t* __restrict__ w, size_t bpr,
@@ -76,18 +41,20 @@ __global__ __launch_bounds__(256) void gemv_kernel(const uint8_t* __restrict__ w
     if (row0 >= out_f) return;
     const int row_end = min(row0 + rows_per_wave, out_f);
     typename F::Acts acts[STEPS];
-    typename F::Row cur[STEPS];
+    typename F::Row first;
     bool ok[STEPS];
 #pragma unroll
-    for (int t = 0; t < STEPS; ++t) {
-        ok[t] = F::valid(t, lane, n_units);
-        F::load_row(cur[t], w + (size_t)row0 * bpr, t, lane, ok[t]);
-        F::load_acts(acts[t], act, t, lane, ok[t]);
-    }
-    gemv_rows<F, STEPS, STAGES>(w, bpr, cur, acts, ok, y, n_units, row0, row_end, lane, st);
+    for (int t = 0; t < STEPS; ++t) ok[t] = F::valid(t, lane, n_units);
+    F::load_row(first, w + (size_t)row0 * bpr, 0, lane, ok[0]);
+#pragma unroll
+    for (int t = 0; t < STEPS; ++t) F::load_acts(acts[t], act, t, lane, ok[t]);
+    __shared__ __attribute__((aligned(16))) float osum[F::kOrdered ? 4 * OrderedSum<STEPS>::kFloatsPerWave : 4];
+    gemv_rows<F, STEPS, STAGES>(w, bpr, first, acts, ok, y, n_units, row0, row_end, lane, st,
+                                osum + (threadIdx.x >> 6) * (F::kOrdered ? OrderedSum<STEPS>::kFloatsPerWave : 0));
 }
 
-// Fused + grouped form. LDS: qs[in_f] | d[in_f/32] | bsums[in_f/32] | bsums16[in_f/16].
+// Fused + grouped form. LDS: qs[in_f] | d[in_f/32] | bsums[in_f/32] | bsums16[in_f/16] | per-wave
+// ordered-sum scratch.
 template <typename F, int STEPS, int NW>
 __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, int single_rows,
                                                              const GemvTile* __restrict__ tiles,
@@ -131,13 +98,11 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, 
             xv[i] = *reinterpret_cast<const v4f*>(tile.x + (size_t)c * 256 + lane * 4);
     }
     const bool has_rows = row0 < tile.rows;
-    typename F::Row cur[STEPS];
+    typename F::Row first;
     bool ok[STEPS];
 #pragma unroll
-    for (int t = 0; t < STEPS; ++t) {
-        ok[t] = has_rows && F::valid(t, lane, n_units);
-        F::load_row(cur[t], tile.w + (size_t)row0 * tile.bpr, t, lane, ok[t]);
-    }
+    for (int t = 0; t < STEPS; ++t) ok[t] = has_rows && F::valid(t, lane, n_units);
+    F::load_row(first, tile.w + (size_t)row0 * tile.bpr, 0, lane, ok[0]);
 #pragma unroll
     for (int i = 0; i < kMaxChunks; ++i) {
         const int c = wave + i * NW;
@@ -152,8 +117,9 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, 
     typename F::Acts acts[STEPS];
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) F::load_acts(acts[t], act, t, lane, ok[t]);
-    gemv_rows<F, STEPS, false>(tile.w, tile.bpr, cur, acts, ok, tile.y, n_units, row0, row_end, lane,
-                               StagePtrs{nullptr, nullptr});
+    float* osum = reinterpret_cast<float*>(lds + in_f + in_f / 2) + wave * OrderedSum<STEPS>::kFloatsPerWave;
+    gemv_rows<F, STEPS, false>(tile.w, tile.bpr, first, acts, ok, tile.y, n_units, row0, row_end, lane,
+                               StagePtrs{nullptr, nullptr}, osum);
 }
 
 // ───────────────────────────────────── launch ─────────────────────────────────────
@@ -206,8 +172,8 @@ bool launch_gemv(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, floa
 // Largest workgroup (in waves) whose register budget the kernel fits without spilling: 16 waves
 // per workgroup leave 128 VGPRs per lane, 8 waves 256 (from the compiler's resource report).
 template <typename F> static int max_waves_per_wg(int steps);
-template <> int max_waves_per_wg<FmtQ4K>(int steps) { return steps <= 2 ? 16 : (steps <= 5 ? 8 : 4); }
-template <> int max_waves_per_wg<FmtQ6K>(int steps) { return steps <= 1 ? 16 : (steps <= 4 ? 8 : 4); }
+template <> int max_waves_per_wg<FmtQ4K>(int steps) { return steps <= 3 ? 16 : 8; }
+template <> int max_waves_per_wg<FmtQ6K>(int steps) { return steps <= 1 ? 16 : 8; }
 template <> int max_waves_per_wg<FmtQ8_0>(int steps) { return steps <= 4 ? 16 : 8; }
 template <> int max_waves_per_wg<FmtQ2_0>(int steps) { return steps <= 3 ? 16 : 8; }
 
@@ -218,12 +184,13 @@ static bool plan_group_fmt(size_t in_f, const GemvOpDesc* ops, int n, GemvGroupP
     size_t total_rows = 0;
     for (int i = 0; i < n; ++i) total_rows += (size_t)ops[i].out_f;
     // Every workgroup re-quantizes x (about the arithmetic of eleven weight rows at in_f 4096), so
-    // big groups take up to 256 rows per workgroup; small ones keep at least ~512 workgroups in
-    // flight. The workgroup is always as wide as the register budget allows, so that the
+    // big groups take up to 128 rows per workgroup (more than that loses to the uneven tail);
+    // small ones keep at least ~512 workgroups in flight. The workgroup is always as wide as the register budget allows, so that the
     // quantization is spread over the most waves; waves beyond the tile's rows retire after it.
     int nw = max_waves_per_wg<F>(steps);
+    if (steps >= 3 && nw > 8) nw = 8;  // long rows: 8-wave workgroups measured faster
     size_t rows_per_wg = (total_rows + 511) / 512;
-    rows_per_wg = rows_per_wg < 4 ? 4 : (rows_per_wg > 256 ? 256 : rows_per_wg);
+    rows_per_wg = rows_per_wg < 4 ? 4 : (rows_per_wg > 128 ? 128 : rows_per_wg);
     // Tuning knobs (the reference exposes its kernel-shape choices the same way,
     // kernels.vulkan.* in crates/infr-core/src/config/mod.rs:210-358).
     static const int env_nw = getenv("INFR_HIP_GEMV_WAVES") ? atoi(getenv("INFR_HIP_GEMV_WAVES")) : 0;
@@ -235,7 +202,8 @@ static bool plan_group_fmt(size_t in_f, const GemvOpDesc* ops, int n, GemvGroupP
     plan->total_wgs = wg;
     plan->waves_per_wg = nw;
     plan->rows_per_wg = (int)rows_per_wg;
-    plan->lds_bytes = in_f + in_f / 2;  // qs + d + bsums + bsums16
+    // qs + d + bsums + bsums16, then the ordered-sum scratch of every wave
+    plan->lds_bytes = in_f + in_f / 2 + (F::kOrdered ? (size_t)nw * (16 * (16 * steps + 4)) * sizeof(float) : 0);
     return true;
 }
 

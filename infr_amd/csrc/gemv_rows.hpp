@@ -1,0 +1,78 @@
+// The row loop shared by every decode-GEMV entry kernel (plain, fused/grouped, id-gathered).
+#pragma once
+
+#include "gemv_formats.hpp"
+
+namespace infr {
+
+// Per-wave LDS scratch for the ordered sum: 16 rows x (16*STEPS block terms + 4 pad) floats. The
+// row stride 4*(4*STEPS+1) dwords makes the 16 lanes' 16-byte reads hit distinct banks.
+template <int STEPS>
+struct OrderedSum {
+    static constexpr int kRowStride = 16 * STEPS + 4;
+    static constexpr int kFloatsPerWave = 16 * kRowStride;
+};
+
+// Rows [row0, row_end) of one weight matrix against activation registers `acts`. `first` already
+// holds step 0 of row0 (the caller issues those loads as early as it can). The loads run one wave
+// step (16 or 64 blocks) ahead of the arithmetic, across row boundaries, so a wave always has
+// one step's bytes in flight while it holds only two steps' worth of registers.
+//
+// Ordered formats (Q4_K, Q6_K): the CPU adds a row's per-block terms in ascending block order
+// (`sumf +=`). The quad leaders park each row's terms in LDS (`osum`, this wave's private
+// scratch) and, every 16 rows, lane i adds row i's terms in that order: the same rounding
+// sequence as the CPU at about two instructions per row instead of a 16-deep v_readlane chain
+// per step. Lanes past a row's last block contribute +0.0, which leaves the sum unchanged.
+template <typename F, int STEPS, bool STAGES>
+__device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t bpr,
+                                          const typename F::Row& first,
+                                          const typename F::Acts (&acts)[STEPS],
+                                          const bool (&ok)[STEPS], float* __restrict__ y, int n_units,
+                                          int row0, int row_end, int lane, const StagePtrs& st,
+                                          float* osum) {
+    constexpr int LS = OrderedSum<STEPS>::kRowStride;
+    typename F::Row cur = first;
+    int in_batch = 0, batch_row0 = row0;
+    for (int row = row0; row < row_end; ++row) {
+        const uint8_t* rowp = w + (size_t)row * bpr;
+        float s = 0.0f;
+#pragma unroll
+        for (int t = 0; t < STEPS; ++t) {
+            typename F::Row nxt;
+            if (t + 1 < STEPS) F::load_row(nxt, rowp, t + 1, lane, ok[t + 1 < STEPS ? t + 1 : 0]);
+            else F::load_row(nxt, rowp + bpr, 0, lane, ok[0] && row + 1 < row_end);
+            const float term = F::template term<STAGES>(cur, acts[t], t, lane, ok[t], st,
+                                                        (size_t)row * n_units);
+            if (F::kOrdered) {
+                if ((lane & 3) == 0) osum[in_batch * LS + t * 16 + (lane >> 2)] = term;
+            } else {
+                s += term;
+            }
+            cur = nxt;
+        }
+        if (F::kOrdered) {
+            if (++in_batch == 16 || row + 1 == row_end) {
+                if (lane < in_batch) {
+                    const v4f* tr = reinterpret_cast<const v4f*>(osum + lane * LS);
+                    float acc = 0.0f;
+#pragma unroll
+                    for (int k = 0; k < 4 * STEPS; ++k) {
+                        const v4f v = tr[k];
+                        acc += v.x;
+                        acc += v.y;
+                        acc += v.z;
+                        acc += v.w;
+                    }
+                    y[batch_row0 + lane] = acc;
+                }
+                batch_row0 = row + 1;
+                in_batch = 0;
+            }
+        } else {
+            s = wave_sum_f(s);
+            if (lane == 0) y[row] = s;
+        }
+    }
+}
+
+}  // namespace infr

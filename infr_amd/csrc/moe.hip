@@ -19,6 +19,7 @@
 #include <algorithm>
 
 #include "gemv_formats.hpp"
+#include "gemv_rows.hpp"
 #include "kernels.hpp"
 #include "quant_chunk.hpp"
 
@@ -257,39 +258,18 @@ __global__ __launch_bounds__(256) void gemv_id_kernel(const uint8_t* __restrict_
     a.bsums = act.bsums + (size_t)r * (in_f / 32);
     a.bsums16 = act.bsums16 + (size_t)r * (in_f / 16);
     typename F::Acts acts[STEPS];
-    typename F::Row cur[STEPS];
+    typename F::Row first;
     bool ok[STEPS];
 #pragma unroll
-    for (int t = 0; t < STEPS; ++t) {
-        ok[t] = F::valid(t, lane, n_units);
-        F::load_row(cur[t], w + (size_t)row0 * bpr, t, lane, ok[t]);
-        F::load_acts(acts[t], a, t, lane, ok[t]);
-    }
-    // same body as the decode GEMV (gemv.hip): per-block exact integers, CPU-ordered f32 sum
-    typename F::Row nxt[STEPS];
-    float* yo = y + (size_t)pair * out_f;
-    for (int row = row0; row < row_end; ++row) {
-        if (row + 1 < row_end) {
+    for (int t = 0; t < STEPS; ++t) ok[t] = F::valid(t, lane, n_units);
+    F::load_row(first, w + (size_t)row0 * bpr, 0, lane, ok[0]);
 #pragma unroll
-            for (int t = 0; t < STEPS; ++t) F::load_row(nxt[t], w + (size_t)(row + 1) * bpr, t, lane, ok[t]);
-        }
-        float s = 0.0f;
-#pragma unroll
-        for (int t = 0; t < STEPS; ++t) {
-            const float term = F::template term<false>(cur[t], acts[t], t, lane, ok[t],
-                                                       StagePtrs{nullptr, nullptr}, 0);
-            if (F::kOrdered) {
-#pragma unroll
-                for (int i = 0; i < 16; ++i) s += readlane_f(term, 4 * i);
-            } else {
-                s += term;
-            }
-        }
-        if (!F::kOrdered) s = wave_sum_f(s);
-        if (lane == 0) yo[row] = s;
-#pragma unroll
-        for (int t = 0; t < STEPS; ++t) cur[t] = nxt[t];
-    }
+    for (int t = 0; t < STEPS; ++t) F::load_acts(acts[t], a, t, lane, ok[t]);
+    // same body as the decode GEMV: per-block exact integers, CPU-ordered f32 sum
+    __shared__ __attribute__((aligned(16))) float osum[F::kOrdered ? 4 * OrderedSum<STEPS>::kFloatsPerWave : 4];
+    gemv_rows<F, STEPS, false>(w, bpr, first, acts, ok, y + (size_t)pair * out_f, n_units, row0, row_end,
+                               lane, StagePtrs{nullptr, nullptr},
+                               osum + (threadIdx.x >> 6) * (F::kOrdered ? OrderedSum<STEPS>::kFloatsPerWave : 0));
 }
 
 // act = silu(g) * u per pair row, quantized per 256 for the down bank (lib.rs:2824-2892).
