@@ -28,6 +28,8 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
+# algorithmic bytes per launch -> measured HBM bytes per launch (profiles/gemv_q4k_decode_sweep.md)
+MEASURED_TRAFFIC = {2887778304: 2892493776}
 INT8_PEAK_TOPS = 5000.0    # MI355X dense int8 MFMA, published
 
 # (name, out_f, in_f) of one Qwen3-8B decoder layer
@@ -45,14 +47,20 @@ def weight_bytes(dtype, out_f, in_f):
 
 class Sweep:
     """A decode-step matvec sweep: every projection of `n_layers` layers (+ optional lm_head) as
-    one plan of independent Op::Linear ops over distinct weight buffers."""
+    one plan of Op::Linear ops over distinct weight buffers.
 
-    def __init__(self, be, dtype, m, n_layers, seed=0, head=False, sigma=0.02):
+    chain=False: every op reads the shared input and owns its output, so all ops are independent
+    (the GEMV-bandwidth measurement; the backend groups them into one launch per in_f).
+    chain=True: a decoder layer's dependency structure, {q,k,v}(x) -> o(q) -> {gate,up}(o) ->
+    down(gate) -> next layer, i.e. four dependent launches per layer."""
+
+    def __init__(self, be, dtype, m, n_layers, seed=0, head=False, sigma=0.02, chain=False):
         from infr_amd import (Bindings, BufferUsage, DType, Graph, Linear, TensorDesc,
                               synth_normal_f32, synth_weight)
         self.be, self.dtype, self.m = be, dtype, m
         g, binds = Graph(), Bindings()
-        self.bytes = 0
+        g4096 = Graph()            # the in_f = 4096 ops alone (same tensor ids, same buffers)
+        self.bytes = self.bytes_4096 = 0
         self.launches = 0
         self.keep = []
         xs = {}
@@ -62,8 +70,9 @@ class Sweep:
             binds.bind(xid, xb)
             xs[in_f] = xid
             self.keep.append(xb)
+
         def new_out(out_f):
-            # every projection has its own output, as in a real graph: the ops are independent
+            # every projection has its own output, as in a real graph
             yid = g.output(TensorDesc((m, out_f), DType.F32))
             yb = be.alloc(m * out_f * 4)
             binds.bind(yid, yb)
@@ -75,7 +84,9 @@ class Sweep:
         for i, (name, out_f, in_f) in enumerate(LAYER):
             protos[name] = be.upload_new(synth_weight(dtype, seed + i, out_f, in_f, sigma),
                                          BufferUsage.Weights)
+        x_cur = xs[4096]
         for layer in range(n_layers):
+            outs = {}
             for name, out_f, in_f in LAYER:
                 nb = weight_bytes(dtype, out_f, in_f)
                 if layer == 0:
@@ -86,38 +97,51 @@ class Sweep:
                 wid = g.weight(TensorDesc((out_f, in_f), dtype))
                 binds.bind(wid, wb)
                 self.keep.append(wb)
-                g.push(Linear(xs[in_f], wid, new_out(out_f), m, in_f, out_f))
+                if chain:
+                    src = {"q": x_cur, "k": x_cur, "v": x_cur, "o": outs.get("q"), "gate": outs.get("o"),
+                           "up": outs.get("o"), "down": outs.get("gate")}[name]
+                else:
+                    src = xs[in_f]
+                outs[name] = new_out(out_f)
+                op = Linear(src, wid, outs[name], m, in_f, out_f)
+                g.push(op)
+                if in_f == 4096:
+                    g4096.ops.append(op)
+                    self.bytes_4096 += nb
                 self.bytes += nb
                 self.launches += 1
+            x_cur = outs["down"]
         if head:
             nb = weight_bytes(dtype, VOCAB, 4096)
             wb = be.upload_new(synth_weight(dtype, seed + 99, VOCAB, 4096, sigma), BufferUsage.Weights)
             wid = g.weight(TensorDesc((VOCAB, 4096), dtype))
             binds.bind(wid, wb)
             self.keep.append(wb)
-            g.push(Linear(xs[4096], wid, new_out(VOCAB), m, 4096, VOCAB))
+            g.push(Linear(x_cur if chain else xs[4096], wid, new_out(VOCAB), m, 4096, VOCAB))
             self.bytes += nb
             self.launches += 1
         be.sync()
+        g4096.tensors, g4096.kinds = g.tensors, g.kinds
         self.plan, self.binds = be.compile(g), binds
+        self.plan_4096 = be.compile(g4096) if not chain else None
 
-    def step(self):
-        self.be.execute(self.plan, self.binds)
+    def step(self, plan=None):
+        self.be.execute(plan or self.plan, self.binds)
 
-    def time(self, steps, warmup):
+    def time(self, steps, warmup, plan=None):
         for _ in range(warmup):
-            self.step()
+            self.step(plan)
         self.be.sync()
         t0 = time.perf_counter()
         self.be.timer_begin()
         for _ in range(steps):
-            self.step()
+            self.step(plan)
         dev_ms = self.be.timer_end()
         wall_ms = (time.perf_counter() - t0) * 1e3
         return dev_ms / steps, wall_ms / steps
 
     def free(self):
-        self.plan = None
+        self.plan = self.plan_4096 = None
         for b in self.keep:
             b.free()
         self.keep = []
@@ -247,8 +271,8 @@ def main():
     ap.add_argument("--layers", type=int, default=N_LAYERS)
     ap.add_argument("--no-extra", action="store_true", help="headline sweep only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--sections", default="shapes,mmq,ternary,moe",
-                    help="comma list of secondary sections: shapes, mmq, ternary, moe")
+    ap.add_argument("--sections", default="shapes,mmq,chain,ternary,moe",
+                    help="comma list of secondary sections: shapes, mmq, chain, ternary, moe")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
@@ -264,8 +288,17 @@ def main():
     ms = max(dev_ms, wall_ms)
     value = sw.bytes / (ms * 1e-3) / 1e9
     n_launch = max(1, sw.plan.launches())          # grouped: independent ops share a launch
-    avg_launch_us = dev_ms * 1e3 / n_launch
-    achieved = (sw.bytes / n_launch) / (avg_launch_us * 1e-6) / 1e9
+    # Dominant kernel: the in_f = 4096 Q4_K GEMV (gemv_fused_kernel<FmtQ4K, 1, 16>), 216 of the 252
+    # ops, timed alone with HIP events on the backend's stream: one launch per execute.
+    k_ms, _ = sw.time(args.steps, 2, sw.plan_4096)
+    k_launches = max(1, sw.plan_4096.launches())
+    avg_launch_us = k_ms * 1e3 / k_launches
+    bytes_per_launch = sw.bytes_4096 // k_launches
+    achieved = bytes_per_launch / (avg_launch_us * 1e-6) / 1e9
+    # HBM bytes per launch of that kernel at the default 36-layer sweep, from two rocprofv3 --pmc
+    # runs of this command (FETCH_SIZE x 1.99786 and WRITE_SIZE x 1.0, the factors a plain
+    # 28,311,552-byte device copy in the same runs gives); null for any other launch shape.
+    traffic = MEASURED_TRAFFIC.get(bytes_per_launch)
     out = {
         "metric": "Q4_K GEMV HBM GB/s (% of peak) + prefill mmq int8 TOPS at M=512",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
@@ -277,10 +310,11 @@ def main():
                    "weights": "N(0,0.02^2) seed 0 -> Q4_K", "activations": "N(0,1) f32, quantized on GPU",
                    "device": caps["device_name"], "compute_units": caps["compute_units"]},
         "pct_of_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
-        "roofline": {"bound": "hbm", "kernel": "gemv_q4k", "achieved": round(achieved, 1),
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": None, "avg_launch_us": round(avg_launch_us, 3),
-                     "launches_per_step": n_launch, "bytes_per_launch": sw.bytes // n_launch},
+        "launches_per_step": n_launch,
+        "roofline": {"bound": "hbm", "kernel": "gemv_fused_kernel<FmtQ4K, 1, 16> (in_f 4096 group)",
+                     "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "avg_launch_us": round(avg_launch_us, 3), "bytes_per_launch": bytes_per_launch},
     }
     sw.free()
 
@@ -297,6 +331,12 @@ def main():
             t, nb = single_shape(be, DType.Q4K, M, 4096, 12288, reps=10)
             extra[f"mmq_Q4_K_M{M}_TOPS"] = round(2.0 * M * 12288 * 4096 / (t * 1e-3) / 1e12, 2)
             extra[f"mmq_Q4_K_M{M}_pct_int8_peak"] = round(100 * extra[f"mmq_Q4_K_M{M}_TOPS"] / INT8_PEAK_TOPS, 2)
+    if "chain" in sections:
+        ch = Sweep(be, DType.Q4K, 1, args.layers, chain=True)
+        d, w = ch.time(10, 2)
+        extra["decode_chain_Q4_K_GBs"] = round(ch.bytes / (max(d, w) * 1e-3) / 1e9, 1)
+        extra["decode_chain_launches_per_step"] = ch.plan.launches()
+        ch.free()
     if "ternary" in sections:
         tern = Sweep(be, DType.Q2_0, 1, N_LAYERS, head=True)
         d, w = tern.time(5, 2)
