@@ -156,11 +156,9 @@ def single_shape(be, dtype, m, in_f, out_f, reps=40, rotate_bytes=768 << 20):
     g, binds, keep = Graph(), Bindings(), []
     xid = g.input(TensorDesc((m, in_f), DType.F32))
     xb = be.upload_new(synth_normal_f32(1, m * in_f))
-    yid = g.output(TensorDesc((m, out_f), DType.F32))
-    yb = be.alloc(m * out_f * 4)
-    binds.bind(xid, xb).bind(yid, yb)
+    binds.bind(xid, xb)
     proto = be.upload_new(synth_weight(dtype, 0, out_f, in_f), BufferUsage.Weights)
-    keep += [xb, yb, proto]
+    keep += [xb, proto]
     wids = []
     for c in range(copies):
         wb = proto if c == 0 else be.alloc_uninit(nb, BufferUsage.Weights)
@@ -171,6 +169,12 @@ def single_shape(be, dtype, m, in_f, out_f, reps=40, rotate_bytes=768 << 20):
         binds.bind(wid, wb)
         wids.append(wid)
     for i in range(reps):
+        # each launch owns its output: the launches are independent, as in the reference's
+        # bandwidth probe (one recorder, `reps` dispatches, crates/infr-vulkan/tests/decode_gemv_bw.rs:186-210)
+        yid = g.output(TensorDesc((m, out_f), DType.F32))
+        yb = be.alloc(m * out_f * 4)
+        keep.append(yb)
+        binds.bind(yid, yb)
         g.push(Linear(xid, wids[i % copies], yid, m, in_f, out_f))
     plan = be.compile(g)
     be.execute(plan, binds)

@@ -22,6 +22,7 @@
 // the CPU's accumulation order, so y matches infr-cpu's scalar kernel bit for bit. For Q8_0 and
 // Q2_0 (128 terms per 4096 columns) the lanes' terms are added with a fixed butterfly instead:
 // deterministic, but rounded in a different order than the CPU's sequential sum.
+#include <algorithm>
 #include <cstdlib>
 
 #include "gemv_formats.hpp"
@@ -51,6 +52,40 @@ __global__ __launch_bounds__(256) void gemv_kernel(const uint8_t* __restrict__ w
     __shared__ __attribute__((aligned(16))) float osum[F::kOrdered ? 4 * OrderedSum<STEPS>::kFloatsPerWave : 4];
     gemv_rows<F, STEPS, STAGES>(w, bpr, first, acts, ok, y, n_units, row0, row_end, lane, st,
                                 osum + (threadIdx.x >> 6) * (F::kOrdered ? OrderedSum<STEPS>::kFloatsPerWave : 0));
+}
+
+// Small batch (2..8 activation rows already quantized in device memory): weights stream once.
+template <typename F, int STEPS, int MB, bool STAGES>
+__global__ __launch_bounds__(256) void gemv_batch_kernel(const uint8_t* __restrict__ w, size_t bpr,
+                                                         ActPtrs act, int m_valid, int in_f,
+                                                         float* __restrict__ y, int out_f,
+                                                         int rows_per_wave, StagePtrs st) {
+    const int lane = threadIdx.x & 63;
+    const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int row0 = wave * rows_per_wave;
+    if (row0 >= out_f) return;
+    const int row_end = min(row0 + rows_per_wave, out_f);
+    const int n_units = F::units(in_f);
+    typename F::Acts acts[MB][STEPS];
+    typename F::Row first;
+    bool ok[STEPS];
+#pragma unroll
+    for (int t = 0; t < STEPS; ++t) ok[t] = F::valid(t, lane, n_units);
+    F::load_row(first, w + (size_t)row0 * bpr, 0, lane, ok[0]);
+    const int dper = F::kPer32 ? in_f / 32 : in_f / 256;
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi) {
+        const int r = mi < m_valid ? mi : 0;  // padding rows reuse row 0; their outputs are dropped
+        const ActPtrs a{act.qs + (size_t)r * in_f, act.d + (size_t)r * dper,
+                        act.bsums + (size_t)r * (in_f / 32), act.bsums16 + (size_t)r * (in_f / 16)};
+#pragma unroll
+        for (int t = 0; t < STEPS; ++t) F::load_acts(acts[mi][t], a, t, lane, ok[t]);
+    }
+    __shared__ __attribute__((aligned(16))) float osum[F::kOrdered ? 4 * OrderedSum<STEPS>::kFloatsPerWave : 4];
+    const size_t st_stride = (size_t)out_f * (F::kBlockElems == 64 ? 2 * n_units : n_units);
+    gemv_rows_batch<F, STEPS, MB, STAGES>(
+        w, bpr, first, acts, ok, y, (size_t)out_f, m_valid, n_units, row0, row_end, lane, st, st_stride,
+        osum + (threadIdx.x >> 6) * (F::kOrdered ? OrderedSum<STEPS>::kFloatsPerWave : 0));
 }
 
 // Fused + grouped form. LDS: qs[in_f] | d[in_f/32] | bsums[in_f/32] | bsums16[in_f/16] | per-wave
@@ -165,6 +200,65 @@ bool launch_gemv(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, floa
     case 14: return launch_plain_fmt<FmtQ6K>(w, bpr, act, y, in_f, out_f, st, stream);
     case 8: return launch_plain_fmt<FmtQ8_0>(w, bpr, act, y, in_f, out_f, st, stream);
     case 42: return launch_plain_fmt<FmtQ2_0>(w, bpr, act, y, in_f, out_f, st, stream);
+    default: return false;
+    }
+}
+
+template <typename F, int STEPS, int MB>
+static void launch_batch_one(const uint8_t* w, size_t bpr, const ActPtrs& act, int m_valid, size_t in_f,
+                             float* y, size_t out_f, const StagePtrs& st, hipStream_t stream) {
+    size_t rpw = (out_f + 4095) / 4096;
+    rpw = rpw < 2 ? 2 : (rpw > 16 ? 16 : rpw);
+    const size_t waves = (out_f + rpw - 1) / rpw;
+    const dim3 grid((unsigned)((waves + 3) / 4)), block(256);
+    if (st.a)
+        hipLaunchKernelGGL((gemv_batch_kernel<F, STEPS, MB, true>), grid, block, 0, stream, w, bpr, act,
+                           m_valid, (int)in_f, y, (int)out_f, (int)rpw, st);
+    else
+        hipLaunchKernelGGL((gemv_batch_kernel<F, STEPS, MB, false>), grid, block, 0, stream, w, bpr, act,
+                           m_valid, (int)in_f, y, (int)out_f, (int)rpw, st);
+}
+
+// m activation rows in chunks of MB <= 8 / STEPS (the activations live in registers).
+template <typename F>
+static bool launch_batch_fmt(const uint8_t* w, size_t bpr, const ActQ8& a, float* y, size_t m,
+                             size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream) {
+    const int steps = (int)((in_f + F::kElemsPerStep - 1) / F::kElemsPerStep);
+    if (steps < 1 || steps > 8) return false;
+    const size_t dper = F::kPer32 ? in_f / 32 : in_f / 256;
+    const size_t blocks = (F::kBlockElems == 64 ? 2 : 1) * (in_f / F::kBlockElems);
+    const size_t mb_max = steps == 1 ? 8 : (steps == 2 ? 4 : (steps <= 4 ? 2 : 1));
+    for (size_t r0 = 0; r0 < m; r0 += mb_max) {
+        const int mv = (int)std::min(mb_max, m - r0);
+        const ActPtrs act{a.qs + r0 * in_f, a.d + r0 * dper, a.bsums + r0 * (in_f / 32),
+                          a.bsums16 ? a.bsums16 + r0 * (in_f / 16) : nullptr};
+        const StagePtrs sp{st.a ? st.a + r0 * out_f * blocks : nullptr,
+                           st.b ? st.b + r0 * out_f * blocks : nullptr};
+        float* yo = y + r0 * out_f;
+#define INFR_B(S, MB) launch_batch_one<F, S, MB>(w, bpr, act, mv, in_f, yo, out_f, sp, stream)
+        switch (steps) {
+        case 1: if (mv > 4) INFR_B(1, 8); else if (mv > 2) INFR_B(1, 4); else if (mv > 1) INFR_B(1, 2); else INFR_B(1, 1); break;
+        case 2: if (mv > 2) INFR_B(2, 4); else if (mv > 1) INFR_B(2, 2); else INFR_B(2, 1); break;
+        case 3: if (mv > 1) INFR_B(3, 2); else INFR_B(3, 1); break;
+        case 4: if (mv > 1) INFR_B(4, 2); else INFR_B(4, 1); break;
+        case 5: INFR_B(5, 1); break;
+        case 6: INFR_B(6, 1); break;
+        case 7: INFR_B(7, 1); break;
+        default: INFR_B(8, 1); break;
+        }
+#undef INFR_B
+    }
+    return true;
+}
+
+bool launch_gemv_batch(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
+                       size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream) {
+    if (out_f == 0 || m == 0) return true;
+    switch (dtype) {
+    case 12: return launch_batch_fmt<FmtQ4K>(w, bpr, act, y, m, in_f, out_f, st, stream);
+    case 14: return launch_batch_fmt<FmtQ6K>(w, bpr, act, y, m, in_f, out_f, st, stream);
+    case 8: return launch_batch_fmt<FmtQ8_0>(w, bpr, act, y, m, in_f, out_f, st, stream);
+    case 42: return launch_batch_fmt<FmtQ2_0>(w, bpr, act, y, m, in_f, out_f, st, stream);
     default: return false;
     }
 }

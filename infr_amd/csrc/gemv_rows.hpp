@@ -75,4 +75,74 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
     }
 }
 
+// Small-batch form: MB activation rows against each weight row, so the weights stream once for
+// up to eight tokens. Every (weight row, activation) pair runs the same per-block code and the
+// same ordered sum as the single-activation loop, so each output equals the m == 1 result bit
+// for bit (the CPU's batch kernels have the same property, kernels.rs:9297-9405).
+template <typename F, int STEPS, int MB, bool STAGES>
+__device__ __forceinline__ void gemv_rows_batch(const uint8_t* __restrict__ w, size_t bpr,
+                                                const typename F::Row& first,
+                                                const typename F::Acts (&acts)[MB][STEPS],
+                                                const bool (&ok)[STEPS], float* __restrict__ y,
+                                                size_t y_stride, int m_valid, int n_units, int row0,
+                                                int row_end, int lane, const StagePtrs& st,
+                                                size_t st_stride, float* osum) {
+    constexpr int LS = OrderedSum<STEPS>::kRowStride;
+    constexpr int RB = 16 / MB;  // weight rows per ordered-sum flush
+    typename F::Row cur = first;
+    int in_batch = 0, batch_row0 = row0;
+    for (int row = row0; row < row_end; ++row) {
+        const uint8_t* rowp = w + (size_t)row * bpr;
+        float s[MB];
+#pragma unroll
+        for (int mi = 0; mi < MB; ++mi) s[mi] = 0.0f;
+#pragma unroll
+        for (int t = 0; t < STEPS; ++t) {
+            typename F::Row nxt;
+            if (t + 1 < STEPS) F::load_row(nxt, rowp, t + 1, lane, ok[t + 1 < STEPS ? t + 1 : 0]);
+            else F::load_row(nxt, rowp + bpr, 0, lane, ok[0] && row + 1 < row_end);
+#pragma unroll
+            for (int mi = 0; mi < MB; ++mi) {
+                const StagePtrs sm{STAGES ? st.a + mi * st_stride : nullptr,
+                                   STAGES && st.b ? st.b + mi * st_stride : nullptr};
+                const float term = F::template term<STAGES>(cur, acts[mi][t], t, lane,
+                                                            ok[t] && mi < m_valid, sm,
+                                                            (size_t)row * n_units);
+                if (F::kOrdered) {
+                    if ((lane & 3) == 0) osum[(in_batch * MB + mi) * LS + t * 16 + (lane >> 2)] = term;
+                } else {
+                    s[mi] += term;
+                }
+            }
+            cur = nxt;
+        }
+        if (F::kOrdered) {
+            if (++in_batch == RB || row + 1 == row_end) {
+                if (lane < in_batch * MB) {
+                    const v4f* tr = reinterpret_cast<const v4f*>(osum + lane * LS);
+                    float acc = 0.0f;
+#pragma unroll
+                    for (int k = 0; k < 4 * STEPS; ++k) {
+                        const v4f v = tr[k];
+                        acc += v.x;
+                        acc += v.y;
+                        acc += v.z;
+                        acc += v.w;
+                    }
+                    const int mi = lane % MB;
+                    if (mi < m_valid) y[(size_t)mi * y_stride + batch_row0 + lane / MB] = acc;
+                }
+                batch_row0 = row + 1;
+                in_batch = 0;
+            }
+        } else {
+#pragma unroll
+            for (int mi = 0; mi < MB; ++mi) {
+                const float tot = wave_sum_f(s[mi]);
+                if (lane == 0 && mi < m_valid) y[(size_t)mi * y_stride + row] = tot;
+            }
+        }
+    }
+}
+
 }  // namespace infr

@@ -33,6 +33,11 @@ struct IntStages {
 bool launch_gemv(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t in_f,
                  size_t out_f, const IntStages& st, hipStream_t stream);
 
+// Small-batch GEMV: m activation rows (already quantized) against every weight row, the weights
+// streamed once per chunk of up to 8 rows. y is [m][out_f]; stages [m][out_f][blocks].
+bool launch_gemv_batch(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
+                       size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream);
+
 // One m == 1 Op::Linear of a fused, grouped decode launch: the kernel quantizes x itself (into
 // LDS) and produces y. All ops of a group share (dtype, in_f).
 struct GemvOpDesc {

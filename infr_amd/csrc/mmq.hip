@@ -23,7 +23,7 @@
 // waves, from LDS. Per 256-block and 32x32 output tile: 16 int8 MFMAs + 1 f16 MFMA against
 // 7 VALU instructions per output for the epilogue.
 //
-// Other formats at m >= 2 go row by row through the decode GEMV (correct, not fast).
+// Small batches (m <= 8) and the other formats take the multi-activation dot4 GEMV (gemv.hip).
 #include <cstdlib>
 
 #include "device_common.hpp"
@@ -238,30 +238,6 @@ __global__ __launch_bounds__(256) void mmq_q4k_kernel(const uint8_t* __restrict_
         }
 }
 
-// Row-at-a-time form: every activation row goes through the decode GEMV, so each output element
-// is produced by exactly the code path of m == 1 (the CPU's batch kernels are likewise
-// bit-identical to its single-row kernels, crates/infr-cpu/src/kernels.rs:9297-9405). Weights are
-// re-streamed once per row, which is only acceptable for small m.
-static bool mmq_by_rows(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y,
-                        size_t m, size_t in_f, size_t out_f, const IntStages& st,
-                        hipStream_t stream) {
-    const bool per32 = dtype == 42;
-    const size_t dper = per32 ? in_f / 32 : in_f / 256;
-    const size_t blocks = (dtype == 12 || dtype == 14) ? in_f / 256 : in_f / 32;
-    for (size_t r = 0; r < m; ++r) {
-        ActQ8 a;
-        a.qs = act.qs + r * in_f;
-        a.d = act.d + r * dper;
-        a.bsums = act.bsums + r * (in_f / 32);
-        a.bsums16 = act.bsums16 ? act.bsums16 + r * (in_f / 16) : nullptr;
-        IntStages s;
-        if (st.a) s.a = st.a + r * out_f * blocks;
-        if (st.b) s.b = st.b + r * out_f * blocks;
-        if (!launch_gemv(dtype, w, bpr, a, y + r * out_f, in_f, out_f, s, stream)) return false;
-    }
-    return true;
-}
-
 template <int BM>
 static void launch_mmq_q4k(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
                            size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream) {
@@ -278,6 +254,11 @@ static void launch_mmq_q4k(const uint8_t* w, size_t bpr, const ActQ8& act, float
 
 bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
                 size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream) {
+    // Small batches and the formats without an MFMA kernel: dot4 GEMV with the activations of up to
+    // eight rows in registers (weights re-streamed once per eight rows beyond that).
+    static const int env_mfma_min = getenv("INFR_HIP_MMQ_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_MIN_M")) : 9;
+    if (dtype != 12 || (int)m < env_mfma_min)
+        return launch_gemv_batch(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
     if (dtype == 12) {
         static const int env_bm = getenv("INFR_HIP_MMQ_BM") ? atoi(getenv("INFR_HIP_MMQ_BM")) : 0;
         // 32-token tiles hold three waves per SIMD; the wider tiles amortise the weight unpack better
@@ -288,7 +269,7 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float
         else launch_mmq_q4k<128>(w, bpr, act, y, m, in_f, out_f, st, stream);
         return true;
     }
-    return mmq_by_rows(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
+    return false;
 }
 
 }  // namespace infr

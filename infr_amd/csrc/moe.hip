@@ -17,6 +17,7 @@
 // Only the selected experts' blocks are addressed: every weight pointer is
 // bank + ids[slot] * expert_stride, read on the device.
 #include <algorithm>
+#include <mutex>
 
 #include "gemv_formats.hpp"
 #include "gemv_rows.hpp"
@@ -27,56 +28,95 @@ namespace infr {
 
 // ───────────────────────────── router + selection ─────────────────────────────
 
-// One 8-lane group per (row, expert): lane j owns accumulator j of infr-cpu's `dot`.
+// infr-cpu's `dot` keeps 8 FMA accumulators (element i goes to accumulator i mod 8) and adds them
+// in order; each accumulator is a strictly sequential chain, so the order cannot be parallelised
+// across lanes without changing the rounding. A workgroup takes kRouterExperts expert rows for
+// one activation row: all 256 threads stage the rows and x into LDS with coalesced 16-byte loads,
+// then two lanes per expert run the chains from LDS (one float4 of four accumulators each).
+constexpr int kRouterExperts = 4;
+
 __global__ __launch_bounds__(256) void moe_router_kernel(const float* __restrict__ router,
                                                          const float* __restrict__ rx,
                                                          float* __restrict__ logits, int ne,
                                                          int n_expert, int rows) {
-    const int gid = (blockIdx.x * 256 + threadIdx.x) >> 3, j = threadIdx.x & 7;
-    const bool live = gid < rows * n_expert;
-    const int r = live ? gid / n_expert : 0, e = live ? gid % n_expert : 0;
-    const float* a = router + (size_t)e * ne;
-    const float* b = rx + (size_t)r * ne;
+    extern __shared__ __attribute__((aligned(16))) float rl[];  // [kRouterExperts][ne] | x[ne]
+    const int tid = threadIdx.x;
+    const int e0 = blockIdx.x * kRouterExperts, r = blockIdx.y;
+    const int n_e = min(kRouterExperts, n_expert - e0);
+    const int ne4 = ne / 4;
+    float* lx = rl + kRouterExperts * ne;
+    for (int i = tid; i < n_e * ne4; i += 256) {
+        const int e = i / ne4, q = i % ne4;
+        reinterpret_cast<v4f*>(rl + e * ne)[q] = reinterpret_cast<const v4f*>(router + (size_t)(e0 + e) * ne)[q];
+    }
+    for (int q = tid; q < ne4; q += 256)
+        reinterpret_cast<v4f*>(lx)[q] = reinterpret_cast<const v4f*>(rx + (size_t)r * ne)[q];
+    for (int i = ne4 * 4 + tid; i < ne; i += 256) {  // ne % 4 tail (scalar)
+        lx[i] = rx[(size_t)r * ne + i];
+        for (int e = 0; e < n_e; ++e) rl[e * ne + i] = router[(size_t)(e0 + e) * ne + i];
+    }
+    __syncthreads();
+    if (tid >= 2 * kRouterExperts) return;
+    const int e = tid >> 1, half = tid & 1;
+    const float* a = rl + e * ne;
     const int chunks = ne / 8;
-    float acc = 0.0f;
-    for (int c = 0; c < chunks; ++c) acc = __builtin_fmaf(a[c * 8 + j], b[c * 8 + j], acc);
+    v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};  // accumulators 4*half .. 4*half+3
+    if (e < n_e) {
+        for (int c = 0; c < chunks; ++c) {
+            const v4f av = *reinterpret_cast<const v4f*>(a + c * 8 + 4 * half);
+            const v4f xv = *reinterpret_cast<const v4f*>(lx + c * 8 + 4 * half);
+            acc.x = __builtin_fmaf(av.x, xv.x, acc.x);
+            acc.y = __builtin_fmaf(av.y, xv.y, acc.y);
+            acc.z = __builtin_fmaf(av.z, xv.z, acc.z);
+            acc.w = __builtin_fmaf(av.w, xv.w, acc.w);
+        }
+    }
     // s = acc[0] + acc[1] + ... + acc[7] in order, then the FMA tail
-    float s = 0.0f;
-    const int base = threadIdx.x & 56;  // first lane of this group within the wave
-#pragma unroll
-    for (int k = 0; k < 8; ++k) s += __shfl(acc, base + k, kWave);
-    for (int i = chunks * 8; i < ne; ++i) s = __builtin_fmaf(a[i], b[i], s);
-    if (live && j == 0) logits[(size_t)r * n_expert + e] = s;
+    const float h0 = __shfl(acc.x, tid | 1, kWave), h1 = __shfl(acc.y, tid | 1, kWave);
+    const float h2 = __shfl(acc.z, tid | 1, kWave), h3 = __shfl(acc.w, tid | 1, kWave);
+    if (half == 0 && e < n_e) {
+        float sum = 0.0f;
+        sum += acc.x; sum += acc.y; sum += acc.z; sum += acc.w;
+        sum += h0; sum += h1; sum += h2; sum += h3;
+        for (int i = chunks * 8; i < ne; ++i) sum = __builtin_fmaf(a[i], lx[i], sum);
+        logits[(size_t)r * n_expert + e0 + e] = sum;
+    }
 }
 
-// One wavefront per row. n_expert <= 1024 (16 per lane).
-__global__ __launch_bounds__(64) void moe_select_kernel(const float* __restrict__ logits,
-                                                        int32_t* __restrict__ sel_idx,
-                                                        float* __restrict__ sel_w, int n_expert,
-                                                        int n_used, float scale) {
-    __shared__ float p[1024];
-    __shared__ float red[2];
-    const int r = blockIdx.x, lane = threadIdx.x;
-    const float* l = logits + (size_t)r * n_expert;
+// Softmax + stable top-n_used + renormalised weights for one row, run by ONE wavefront (the
+// first 64 threads of the calling workgroup); `p` is n_expert floats of LDS, `red` two floats.
+// On return lanes 0..n_used-1 hold (expert, weight) of rank = lane. n_expert <= 1024, n_used <= 64.
+__device__ __forceinline__ void moe_select_wave(const float* __restrict__ l, float* p, float* red,
+                                                int n_expert, int n_used, float scale, int lane,
+                                                int& my_e, float& my_w) {
     float mx = -INFINITY;
     for (int e = lane; e < n_expert; e += 64) mx = __builtin_fmaxf(mx, l[e]);
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) mx = __builtin_fmaxf(mx, __shfl_xor(mx, off, kWave));
     for (int e = lane; e < n_expert; e += 64) p[e] = expf(l[e] - mx);
-    __syncthreads();
-    if (lane == 0) {  // `p.iter().sum()`: index order
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    if (lane == 0) {  // `p.iter().sum()`: index order; 16 LDS values per wait
         float s = 0.0f;
-        for (int e = 0; e < n_expert; ++e) s += p[e];
+        int e = 0;
+        for (; e + 16 <= n_expert; e += 16) {
+            const v4f a = *reinterpret_cast<const v4f*>(p + e), b = *reinterpret_cast<const v4f*>(p + e + 4);
+            const v4f c = *reinterpret_cast<const v4f*>(p + e + 8), d = *reinterpret_cast<const v4f*>(p + e + 12);
+            s += a.x; s += a.y; s += a.z; s += a.w;
+            s += b.x; s += b.y; s += b.z; s += b.w;
+            s += c.x; s += c.y; s += c.z; s += c.w;
+            s += d.x; s += d.y; s += d.z; s += d.w;
+        }
+        for (; e < n_expert; ++e) s += p[e];
         red[0] = s;
     }
-    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     const float psum = red[0];
     for (int e = lane; e < n_expert; e += 64) p[e] = p[e] / psum;
-    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     // stable descending top-n_used: largest p, lowest index among equals, n_used times
     float wsum = 0.0f;
-    float my_w = 0.0f;
-    int my_e = 0;
+    my_w = 0.0f;
+    my_e = 0;
     for (int k = 0; k < n_used; ++k) {
         float bv = -INFINITY;
         int bi = 0x7FFFFFFF;
@@ -97,18 +137,31 @@ __global__ __launch_bounds__(64) void moe_select_kernel(const float* __restrict_
             }
         }
         wsum += bv;  // selection order = the CPU's summation order
-        if (lane == k % 64) {
+        if (lane == k) {
             my_w = bv;
             my_e = bi;
         }
         if (lane == 0) p[bi] = -1.0f;  // taken (probabilities are >= 0)
-        __syncthreads();
-        // n_used > 64 would need several values per lane; the launcher rejects it
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     }
     wsum = __builtin_fmaxf(wsum, 1e-20f);
+    my_w = my_w / wsum * scale;
+}
+
+// One wavefront per row.
+__global__ __launch_bounds__(64) void moe_select_kernel(const float* __restrict__ logits,
+                                                        int32_t* __restrict__ sel_idx,
+                                                        float* __restrict__ sel_w, int n_expert,
+                                                        int n_used, float scale) {
+    __shared__ __attribute__((aligned(16))) float p[1024];
+    __shared__ float red[2];
+    const int r = blockIdx.x, lane = threadIdx.x;
+    int my_e;
+    float my_w;
+    moe_select_wave(logits + (size_t)r * n_expert, p, red, n_expert, n_used, scale, lane, my_e, my_w);
     if (lane < n_used) {
         sel_idx[(size_t)r * n_used + lane] = my_e;
-        sel_w[(size_t)r * n_used + lane] = my_w / wsum * scale;
+        sel_w[(size_t)r * n_used + lane] = my_w;
     }
 }
 
@@ -167,20 +220,22 @@ __device__ __forceinline__ float seg_sum(float v, int seg_base, int nb) {
     return s;
 }
 
-// gate/up: act[slot][o] = silu(gate_e[o] . x) * (up_e[o] . x), e = ids[slot]
+// gate/up at one token: act[slot][o] = silu(gate_e[o] . x) * (up_e[o] . x). Every workgroup
+// derives the routing from the logits itself (one wavefront, a few microseconds, cheaper than a
+// launch of its own); workgroup (0, 0) also publishes it for the down kernel and the caller.
 __global__ __launch_bounds__(256) void moe_gate_up_f32_q4k_kernel(
     const uint8_t* __restrict__ gate, const uint8_t* __restrict__ up, size_t gate_stride,
-    size_t up_stride, const int32_t* __restrict__ ids, const float* __restrict__ x,
-    float* __restrict__ act, int ne, int nff) {
+    size_t up_stride, const float* __restrict__ logits, int n_expert, int n_used, float scale,
+    int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, const float* __restrict__ x,
+    float* __restrict__ act, int ne, int nff, int steps_per_wave) {
+    __shared__ __attribute__((aligned(16))) float sp[1024];
+    __shared__ float red[2];
+    __shared__ int s_expert;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int nb = ne / 256, S = 4 * nb, rps = 64 / S;  // rows per wave step
     const int seg = lane / S, within = lane % S, b = within >> 2, p = within & 3;
     const bool lane_ok = seg < rps;
     const int slot = blockIdx.y;
-    const int e = ids[slot];
-    const size_t bpr = (size_t)nb * 144;
-    const uint8_t* gw = gate + (size_t)e * gate_stride;
-    const uint8_t* uw = up + (size_t)e * up_stride;
 
     float xr[64];
 #pragma unroll
@@ -189,9 +244,24 @@ __global__ __launch_bounds__(256) void moe_gate_up_f32_q4k_kernel(
         if (lane_ok) v = *reinterpret_cast<const v4f*>(x + (size_t)b * 256 + p * 64 + 4 * k);
         xr[4 * k + 0] = v.x; xr[4 * k + 1] = v.y; xr[4 * k + 2] = v.z; xr[4 * k + 3] = v.w;
     }
-    // each wave takes row steps wave, wave+4*gridDim.x... within this block's range
+    if (wave == 0) {
+        int my_e;
+        float my_w;
+        moe_select_wave(logits, sp, red, n_expert, n_used, scale, lane, my_e, my_w);
+        if (lane == slot) s_expert = my_e;
+        if (blockIdx.x == 0 && blockIdx.y == 0 && lane < n_used) {
+            sel_idx[lane] = my_e;
+            sel_w[lane] = my_w;
+        }
+    }
+    __syncthreads();
+    const int e = s_expert;
+    const size_t bpr = (size_t)nb * 144;
+    const uint8_t* gw = gate + (size_t)e * gate_stride;
+    const uint8_t* uw = up + (size_t)e * up_stride;
     const int steps_total = (nff + rps - 1) / rps;
-    for (int st = blockIdx.x * 4 + wave; st < steps_total; st += gridDim.x * 4) {
+    const int st0 = (blockIdx.x * 4 + wave) * steps_per_wave;
+    for (int st = st0; st < min(st0 + steps_per_wave, steps_total); ++st) {
         const int o = st * rps + seg;
         const bool ok = lane_ok && o < nff;
         Q4kF32Row g, u;
@@ -203,11 +273,16 @@ __global__ __launch_bounds__(256) void moe_gate_up_f32_q4k_kernel(
     }
 }
 
-// down + accumulate: out[o] = sum_k w_k * (down_{ids[k]}[o] . act[k]), k in rank order
+// down + accumulate at one token: out[o] = sum_k w_k * (down_{ids[k]}[o] . act[k]), k in rank
+// order. The n_used activation vectors are staged in LDS once per workgroup and all n_used weight
+// rows of a step are requested before the first is used (one memory latency, not n_used).
+constexpr int kMoeMaxUsedF32 = 8;
+
 __global__ __launch_bounds__(256) void moe_down_f32_q4k_kernel(
     const uint8_t* __restrict__ down, size_t down_stride, const int32_t* __restrict__ ids,
     const float* __restrict__ wts, const float* __restrict__ act, float* __restrict__ out, int nff,
     int ne, int n_used) {
+    extern __shared__ __attribute__((aligned(16))) float la[];  // [n_used][nff]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int nb = nff / 256, S = 4 * nb, rps = 64 / S;
     const int seg = lane / S, within = lane % S, b = within >> 2, p = within & 3;
@@ -217,19 +292,33 @@ __global__ __launch_bounds__(256) void moe_down_f32_q4k_kernel(
     const int o = st * rps + seg;
     const bool ok = lane_ok && o < ne;
     float acc = 0.0f;
-    for (int k = 0; k < n_used; ++k) {
-        const uint8_t* dw = down + (size_t)ids[k] * down_stride;
-        Q4kF32Row r;
-        q4k_f32_load(r, dw + (size_t)(ok ? o : 0) * bpr, b, p, ok);
-        float xr[64];
+    for (int k0 = 0; k0 < n_used; k0 += kMoeMaxUsedF32) {
+        const int kn = min(kMoeMaxUsedF32, n_used - k0);
+        Q4kF32Row rows[kMoeMaxUsedF32];
 #pragma unroll
-        for (int q = 0; q < 16; ++q) {
-            v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
-            if (lane_ok) v = *reinterpret_cast<const v4f*>(act + (size_t)k * nff + (size_t)b * 256 + p * 64 + 4 * q);
-            xr[4 * q + 0] = v.x; xr[4 * q + 1] = v.y; xr[4 * q + 2] = v.z; xr[4 * q + 3] = v.w;
+        for (int k = 0; k < kMoeMaxUsedF32; ++k) {
+            const bool okk = ok && k < kn;
+            const uint8_t* dw = down + (size_t)ids[okk ? k0 + k : 0] * down_stride;
+            q4k_f32_load(rows[k], dw + (size_t)(okk ? o : 0) * bpr, b, p, okk);
         }
-        const float yk = seg_sum(q4k_f32_partial(r, xr, p), seg * S, nb);
-        acc += wts[k] * yk;  // `*o += w_e * yv`: separate multiply and add, rank order
+        __syncthreads();
+        for (int i = threadIdx.x; i < kn * nff / 4; i += 256)
+            reinterpret_cast<v4f*>(la)[i] = reinterpret_cast<const v4f*>(act + (size_t)k0 * nff)[i];
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < kMoeMaxUsedF32; ++k) {
+            if (k < kn) {
+                float xr[64];
+#pragma unroll
+                for (int q = 0; q < 16; ++q) {
+                    v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
+                    if (lane_ok) v = *reinterpret_cast<const v4f*>(la + (size_t)k * nff + (size_t)b * 256 + p * 64 + 4 * q);
+                    xr[4 * q + 0] = v.x; xr[4 * q + 1] = v.y; xr[4 * q + 2] = v.z; xr[4 * q + 3] = v.w;
+                }
+                const float yk = seg_sum(q4k_f32_partial(rows[k], xr, p), seg * S, nb);
+                acc += wts[k0 + k] * yk;  // `*o += w_e * yv`: separate multiply and add, rank order
+            }
+        }
     }
     if (ok && within == 0) out[o] = acc;
 }
@@ -315,7 +404,10 @@ static bool launch_gemv_id_fmt(const uint8_t* bank, size_t expert_stride, size_t
                                const int32_t* ids, const ActQ8& act, size_t in_f, int n_used,
                                int pairs, float* y, size_t out_f, hipStream_t stream) {
     const int steps = (int)((in_f + F::kElemsPerStep - 1) / F::kElemsPerStep);
-    const int rpw = 2;
+    // enough rows per wave to amortise loading the activation registers, while keeping the grid
+    // (row tiles x pairs) well above the CU count
+    int rpw = 8;
+    while (rpw > 2 && ((out_f + rpw - 1) / rpw + 3) / 4 * (size_t)pairs < 1024) rpw /= 2;
     const size_t waves = (out_f + rpw - 1) / rpw;
     const dim3 grid((unsigned)((waves + 3) / 4), (unsigned)pairs), block(256);
     const ActPtrs a{act.qs, act.d, act.bsums, act.bsums16};
@@ -342,7 +434,19 @@ static bool launch_gemv_id(int dtype, const uint8_t* bank, size_t expert_stride,
     }
 }
 
+// The router and the one-token down kernel may stage more than the default 64 KiB of LDS.
+static void moe_raise_lds_limits() {
+    static std::once_flag once;
+    std::call_once(once, [] {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(moe_router_kernel),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(moe_down_f32_q4k_kernel),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    });
+}
+
 size_t moe_workspace_bytes(const MoeShape& s) {
+    moe_raise_lds_limits();
     const size_t pairs = (size_t)s.rows * s.n_used;
     size_t n = 0;
     auto add = [&n](size_t bytes) { n += (bytes + 255) / 256 * 256; };
@@ -384,13 +488,16 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     aq.bsums = (int32_t*)take(qmax / 32 * 4);
     aq.bsums16 = (int32_t*)take(qmax / 16 * 4);
 
-    const int groups = s.rows * s.n_expert;
-    hipLaunchKernelGGL(moe_router_kernel, dim3((unsigned)((groups * 8 + 255) / 256)), dim3(256), 0, stream,
-                       b.router, b.router_x, logits, s.ne, s.n_expert, s.rows);
-    hipLaunchKernelGGL(moe_select_kernel, dim3((unsigned)s.rows), dim3(64), 0, stream, logits, sel_idx,
-                       sel_w, s.n_expert, s.n_used, s.scale);
-    if (b.sel_idx) (void)hipMemcpyAsync(b.sel_idx, sel_idx, pairs * 4, hipMemcpyDeviceToDevice, stream);
-    if (b.sel_w) (void)hipMemcpyAsync(b.sel_w, sel_w, pairs * 4, hipMemcpyDeviceToDevice, stream);
+    moe_raise_lds_limits();
+    const size_t router_lds = (size_t)(kRouterExperts + 1) * s.ne * sizeof(float);
+    if (router_lds > 160 * 1024) return "ne too large for the router kernel's LDS staging";
+    hipLaunchKernelGGL(moe_router_kernel,
+                       dim3((unsigned)((s.n_expert + kRouterExperts - 1) / kRouterExperts), (unsigned)s.rows),
+                       dim3(256), router_lds, stream, b.router, b.router_x, logits, s.ne, s.n_expert, s.rows);
+    auto publish_selection = [&]() {
+        if (b.sel_idx) (void)hipMemcpyAsync(b.sel_idx, sel_idx, pairs * 4, hipMemcpyDeviceToDevice, stream);
+        if (b.sel_w) (void)hipMemcpyAsync(b.sel_w, sel_w, pairs * 4, hipMemcpyDeviceToDevice, stream);
+    };
 
     if (s.rows == 1) {
         // ActsKind::Raw for every bank (lib.rs:2359: int8_ok = rows >= 2)
@@ -399,16 +506,24 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
         if (s.ne > 4096 || s.n_ff > 4096) return "rows == 1 needs ne, n_ff_exp <= 4096";
         const int nb_g = s.ne / 256, rps_g = 64 / (4 * nb_g);
         const int steps_g = (s.n_ff + rps_g - 1) / rps_g;
-        hipLaunchKernelGGL(moe_gate_up_f32_q4k_kernel, dim3((unsigned)((steps_g + 3) / 4), (unsigned)s.n_used),
-                           dim3(256), 0, stream, b.gate, b.up, b.gate_stride, b.up_stride, sel_idx, b.x,
-                           gbuf, s.ne, s.n_ff);
+        // two row steps per wave once that still leaves >= ~512 workgroups
+        const int spw = steps_g * s.n_used >= 4096 ? 2 : 1;
+        hipLaunchKernelGGL(moe_gate_up_f32_q4k_kernel,
+                           dim3((unsigned)((steps_g + 4 * spw - 1) / (4 * spw)), (unsigned)s.n_used), dim3(256), 0,
+                           stream, b.gate, b.up, b.gate_stride, b.up_stride, logits, s.n_expert, s.n_used,
+                           s.scale, sel_idx, sel_w, b.x, gbuf, s.ne, s.n_ff, spw);
         const int nb_d = s.n_ff / 256, rps_d = 64 / (4 * nb_d);
         const int steps_d = (s.ne + rps_d - 1) / rps_d;
-        hipLaunchKernelGGL(moe_down_f32_q4k_kernel, dim3((unsigned)((steps_d + 3) / 4)), dim3(256), 0, stream,
-                           b.down, b.down_stride, sel_idx, sel_w, gbuf, b.dst, s.n_ff, s.ne, s.n_used);
+        const size_t down_lds = (size_t)std::min(s.n_used, kMoeMaxUsedF32) * s.n_ff * sizeof(float);
+        hipLaunchKernelGGL(moe_down_f32_q4k_kernel, dim3((unsigned)((steps_d + 3) / 4)), dim3(256), down_lds,
+                           stream, b.down, b.down_stride, sel_idx, sel_w, gbuf, b.dst, s.n_ff, s.ne, s.n_used);
+        publish_selection();
         return hipGetLastError() == hipSuccess ? nullptr : "kernel launch failed";
     }
 
+    hipLaunchKernelGGL(moe_select_kernel, dim3((unsigned)s.rows), dim3(64), 0, stream, logits, sel_idx,
+                       sel_w, s.n_expert, s.n_used, s.scale);
+    publish_selection();
     // rows >= 2: ActsKind::Super for Q4K/Q6K/Q8_0 banks with in_f % 256 == 0 (moe.rs:42-53)
     auto bytes_per_row = [](int dtype, size_t in_f) -> size_t {
         switch (dtype) {
