@@ -464,6 +464,9 @@ static int ensure_moe_ws(infr_hip_t* be, size_t bytes) {
     be->moe_ws = nullptr;
     be->moe_ws_bytes = 0;
     HIP_TRY(be, hipMalloc(&be->moe_ws, bytes));
+    // the router's ticket counters live at the start and must read zero before the first op;
+    // every op leaves them at zero again
+    HIP_TRY(be, hipMemset(be->moe_ws, 0, bytes));
     be->moe_ws_bytes = bytes;
     return INFR_HIP_OK;
 }

@@ -8,16 +8,15 @@
 //   select   softmax with max-subtraction, probabilities summed in index order, stable top-n_used
 //            (ties to the lower expert index), w = p / max(sum_sel p, 1e-20) * scale  (lib.rs:2421-2543)
 //   rows == 1   the CPU multiplies DECODED f32 weights with the UNQUANTIZED activation
-//            (ActsKind::Raw, moe.rs:42-53,142-173): gate/up rows are decoded in registers with
-//            dequant_block's two roundings (sc*code + mn), FMA-accumulated against f32 x, SiLU
-//            fused; the down kernel decodes likewise and adds the experts in rank order
+//            (ActsKind::Raw, moe.rs:42-53,142-173): gate/up rows are applied to f32 x in registers
+//            (sc * sum(code*x) + mn * sum(x) per 32 weights, all f32), SiLU fused; the down kernel
+//            does likewise and adds the experts in rank order
 //   rows >= 2   int8 path: x rows quantized per 256 once, id-gathered Q4_K/Q6_K/Q8_0 GEMVs per
 //            (row, expert) pair (the decode GEMV body, bit-identical to the CPU's batch kernels),
 //            SiLU + re-quantization, id-gathered down GEMV, rank-ordered accumulate
 // Only the selected experts' blocks are addressed: every weight pointer is
 // bank + ids[slot] * expert_stride, read on the device.
 #include <algorithm>
-#include <mutex>
 
 #include "gemv_formats.hpp"
 #include "gemv_rows.hpp"
@@ -28,152 +27,210 @@ namespace infr {
 
 // ───────────────────────────── router + selection ─────────────────────────────
 
-// infr-cpu's `dot` keeps 8 FMA accumulators (element i goes to accumulator i mod 8) and adds them
-// in order; each accumulator is a strictly sequential chain, so the order cannot be parallelised
-// across lanes without changing the rounding. A workgroup takes kRouterExperts expert rows for
-// one activation row: all 256 threads stage the rows and x into LDS with coalesced 16-byte loads,
-// then two lanes per expert run the chains from LDS (one float4 of four accumulators each).
-constexpr int kRouterExperts = 4;
+// Per-wave LDS of the selection: probabilities, the ranked winners, one reduction slot.
+struct SelectLds {
+    float p[1024];
+    float top_p[64];
+    int top_e[64];
+    float red[4];
+};
 
-__global__ __launch_bounds__(256) void moe_router_kernel(const float* __restrict__ router,
-                                                         const float* __restrict__ rx,
-                                                         float* __restrict__ logits, int ne,
-                                                         int n_expert, int rows) {
-    extern __shared__ __attribute__((aligned(16))) float rl[];  // [kRouterExperts][ne] | x[ne]
-    const int tid = threadIdx.x;
-    const int e0 = blockIdx.x * kRouterExperts, r = blockIdx.y;
-    const int n_e = min(kRouterExperts, n_expert - e0);
-    const int ne4 = ne / 4;
-    float* lx = rl + kRouterExperts * ne;
-    for (int i = tid; i < n_e * ne4; i += 256) {
-        const int e = i / ne4, q = i % ne4;
-        reinterpret_cast<v4f*>(rl + e * ne)[q] = reinterpret_cast<const v4f*>(router + (size_t)(e0 + e) * ne)[q];
-    }
-    for (int q = tid; q < ne4; q += 256)
-        reinterpret_cast<v4f*>(lx)[q] = reinterpret_cast<const v4f*>(rx + (size_t)r * ne)[q];
-    for (int i = ne4 * 4 + tid; i < ne; i += 256) {  // ne % 4 tail (scalar)
-        lx[i] = rx[(size_t)r * ne + i];
-        for (int e = 0; e < n_e; ++e) rl[e * ne + i] = router[(size_t)(e0 + e) * ne + i];
-    }
-    __syncthreads();
-    if (tid >= 2 * kRouterExperts) return;
-    const int e = tid >> 1, half = tid & 1;
-    const float* a = rl + e * ne;
-    const int chunks = ne / 8;
-    v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};  // accumulators 4*half .. 4*half+3
-    if (e < n_e) {
-        for (int c = 0; c < chunks; ++c) {
-            const v4f av = *reinterpret_cast<const v4f*>(a + c * 8 + 4 * half);
-            const v4f xv = *reinterpret_cast<const v4f*>(lx + c * 8 + 4 * half);
-            acc.x = __builtin_fmaf(av.x, xv.x, acc.x);
-            acc.y = __builtin_fmaf(av.y, xv.y, acc.y);
-            acc.z = __builtin_fmaf(av.z, xv.z, acc.z);
-            acc.w = __builtin_fmaf(av.w, xv.w, acc.w);
-        }
-    }
-    // s = acc[0] + acc[1] + ... + acc[7] in order, then the FMA tail
-    const float h0 = __shfl(acc.x, tid | 1, kWave), h1 = __shfl(acc.y, tid | 1, kWave);
-    const float h2 = __shfl(acc.z, tid | 1, kWave), h3 = __shfl(acc.w, tid | 1, kWave);
-    if (half == 0 && e < n_e) {
-        float sum = 0.0f;
-        sum += acc.x; sum += acc.y; sum += acc.z; sum += acc.w;
-        sum += h0; sum += h1; sum += h2; sum += h3;
-        for (int i = chunks * 8; i < ne; ++i) sum = __builtin_fmaf(a[i], lx[i], sum);
-        logits[(size_t)r * n_expert + e0 + e] = sum;
-    }
-}
-
-// Softmax + stable top-n_used + renormalised weights for one row, run by ONE wavefront (the
-// first 64 threads of the calling workgroup); `p` is n_expert floats of LDS, `red` two floats.
+// Softmax + stable top-n_used + renormalised weights for one row, run by ONE wavefront.
 // On return lanes 0..n_used-1 hold (expert, weight) of rank = lane. n_expert <= 1024, n_used <= 64.
-__device__ __forceinline__ void moe_select_wave(const float* __restrict__ l, float* p, float* red,
+__device__ __forceinline__ void moe_select_wave(const float* __restrict__ l, SelectLds& s,
                                                 int n_expert, int n_used, float scale, int lane,
                                                 int& my_e, float& my_w) {
+    float* p = s.p;
     float mx = -INFINITY;
     for (int e = lane; e < n_expert; e += 64) mx = __builtin_fmaxf(mx, l[e]);
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) mx = __builtin_fmaxf(mx, __shfl_xor(mx, off, kWave));
     for (int e = lane; e < n_expert; e += 64) p[e] = expf(l[e] - mx);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     if (lane == 0) {  // `p.iter().sum()`: index order; 16 LDS values per wait
-        float s = 0.0f;
+        float sum = 0.0f;
         int e = 0;
         for (; e + 16 <= n_expert; e += 16) {
             const v4f a = *reinterpret_cast<const v4f*>(p + e), b = *reinterpret_cast<const v4f*>(p + e + 4);
             const v4f c = *reinterpret_cast<const v4f*>(p + e + 8), d = *reinterpret_cast<const v4f*>(p + e + 12);
-            s += a.x; s += a.y; s += a.z; s += a.w;
-            s += b.x; s += b.y; s += b.z; s += b.w;
-            s += c.x; s += c.y; s += c.z; s += c.w;
-            s += d.x; s += d.y; s += d.z; s += d.w;
+            sum += a.x; sum += a.y; sum += a.z; sum += a.w;
+            sum += b.x; sum += b.y; sum += b.z; sum += b.w;
+            sum += c.x; sum += c.y; sum += c.z; sum += c.w;
+            sum += d.x; sum += d.y; sum += d.z; sum += d.w;
         }
-        for (; e < n_expert; ++e) s += p[e];
-        red[0] = s;
+        for (; e < n_expert; ++e) sum += p[e];
+        s.red[0] = sum;
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    const float psum = red[0];
+    const float psum = s.red[0];
     for (int e = lane; e < n_expert; e += 64) p[e] = p[e] / psum;
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    // stable descending top-n_used: largest p, lowest index among equals, n_used times
-    float wsum = 0.0f;
-    my_w = 0.0f;
-    my_e = 0;
-    for (int k = 0; k < n_used; ++k) {
-        float bv = -INFINITY;
-        int bi = 0x7FFFFFFF;
+
+    if (n_expert <= 256) {
+        // stable descending order by counting: rank(e) = #{j : p[j] > p[e] or (p[j] == p[e] and j < e)}
         for (int e = lane; e < n_expert; e += 64) {
             const float v = p[e];
-            if (v > bv || (v == bv && e < bi)) {
-                bv = v;
-                bi = e;
+            int rank = 0, j = 0;
+            for (; j + 4 <= n_expert; j += 4) {
+                const v4f q = *reinterpret_cast<const v4f*>(p + j);
+                rank += (q.x > v || (q.x == v && j + 0 < e)) ? 1 : 0;
+                rank += (q.y > v || (q.y == v && j + 1 < e)) ? 1 : 0;
+                rank += (q.z > v || (q.z == v && j + 2 < e)) ? 1 : 0;
+                rank += (q.w > v || (q.w == v && j + 3 < e)) ? 1 : 0;
+            }
+            for (; j < n_expert; ++j) rank += (p[j] > v || (p[j] == v && j < e)) ? 1 : 0;
+            if (rank < n_used) {
+                s.top_e[rank] = e;
+                s.top_p[rank] = v;
             }
         }
+    } else {
+        // largest p, lowest index among equals, n_used times
+        for (int k = 0; k < n_used; ++k) {
+            float bv = -INFINITY;
+            int bi = 0x7FFFFFFF;
+            for (int e = lane; e < n_expert; e += 64) {
+                const float v = p[e];
+                if (v > bv || (v == bv && e < bi)) {
+                    bv = v;
+                    bi = e;
+                }
+            }
 #pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) {
-            const float ov = __shfl_xor(bv, off, kWave);
-            const int oi = __shfl_xor(bi, off, kWave);
-            if (ov > bv || (ov == bv && oi < bi)) {
-                bv = ov;
-                bi = oi;
+            for (int off = 32; off >= 1; off >>= 1) {
+                const float ov = __shfl_xor(bv, off, kWave);
+                const int oi = __shfl_xor(bi, off, kWave);
+                if (ov > bv || (ov == bv && oi < bi)) {
+                    bv = ov;
+                    bi = oi;
+                }
             }
+            if (lane == 0) {
+                s.top_e[k] = bi;
+                s.top_p[k] = bv;
+                p[bi] = -1.0f;  // taken (probabilities are >= 0)
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         }
-        wsum += bv;  // selection order = the CPU's summation order
-        if (lane == k) {
-            my_w = bv;
-            my_e = bi;
-        }
-        if (lane == 0) p[bi] = -1.0f;  // taken (probabilities are >= 0)
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    float wsum = 0.0f;  // summed in rank order, as the CPU sums its selection
+    for (int k = 0; k < n_used; ++k) wsum += s.top_p[k];
     wsum = __builtin_fmaxf(wsum, 1e-20f);
-    my_w = my_w / wsum * scale;
+    my_e = lane < n_used ? s.top_e[lane] : 0;
+    my_w = lane < n_used ? s.top_p[lane] / wsum * scale : 0.0f;
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");  // the LDS may be reused for the next row
 }
 
-// One wavefront per row.
-__global__ __launch_bounds__(64) void moe_select_kernel(const float* __restrict__ logits,
-                                                        int32_t* __restrict__ sel_idx,
-                                                        float* __restrict__ sel_w, int n_expert,
-                                                        int n_used, float scale) {
-    __shared__ __attribute__((aligned(16))) float p[1024];
-    __shared__ float red[2];
-    const int r = blockIdx.x, lane = threadIdx.x;
-    int my_e;
-    float my_w;
-    moe_select_wave(logits + (size_t)r * n_expert, p, red, n_expert, n_used, scale, lane, my_e, my_w);
-    if (lane < n_used) {
-        sel_idx[(size_t)r * n_used + lane] = my_e;
-        sel_w[(size_t)r * n_used + lane] = my_w;
+// infr-cpu's `dot` keeps 8 FMA accumulators (element i goes to accumulator i mod 8) and adds them
+// in order; each accumulator is a strictly sequential chain, so the order cannot be parallelised
+// across lanes without changing the rounding. A workgroup takes kRouterExperts expert rows and
+// kRouterTokens activation rows: all 256 threads stage K-chunks of them into LDS with coalesced
+// 16-byte loads, and two lanes per (expert, token) pair run the chains from LDS (one float4 of
+// four accumulators each), carrying them across chunks.
+// The last workgroup to finish a token tile (a ticket counter per tile, left at zero again)
+// runs the selection for the tile's rows, which saves a launch. ne % 8 == 0 is required.
+constexpr int kRouterExperts = 4, kRouterTokens = 8, kRouterChunk = 512;
+
+__global__ __launch_bounds__(256) void moe_router_kernel(
+    const float* __restrict__ router, const float* __restrict__ rx, float* __restrict__ logits,
+    int* __restrict__ tickets, int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, int ne,
+    int n_expert, int rows, int n_used, float scale, int kc) {
+    extern __shared__ __attribute__((aligned(16))) float rl[];  // [kRouterExperts][kc] | [kRouterTokens][kc]
+    __shared__ __attribute__((aligned(16))) SelectLds sel[4];
+    __shared__ int s_last;
+    const int tid = threadIdx.x;
+    const int e0 = blockIdx.x * kRouterExperts, t0 = blockIdx.y * kRouterTokens;
+    const int n_e = min(kRouterExperts, n_expert - e0), n_t = min(kRouterTokens, rows - t0);
+    float* lw = rl;
+    float* lx = rl + kRouterExperts * kc;
+    const int pair = tid >> 1, half = tid & 1;
+    const int e = pair % kRouterExperts, t = pair / kRouterExperts;
+    const bool active = t < kRouterTokens && e < n_e && t < n_t;
+    v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};  // accumulators 4*half .. 4*half+3
+    for (int k0 = 0; k0 < ne; k0 += kc) {
+        const int n = min(kc, ne - k0), n4 = n / 4;
+        if (k0) __syncthreads();
+        for (int i = tid; i < (n_e + n_t) * n4; i += 256) {
+            const int row = i / n4, q = i % n4;
+            const float* src = row < n_e ? router + (size_t)(e0 + row) * ne : rx + (size_t)(t0 + row - n_e) * ne;
+            float* dst = row < n_e ? lw + row * kc : lx + (row - n_e) * kc;
+            reinterpret_cast<v4f*>(dst)[q] = reinterpret_cast<const v4f*>(src + k0)[q];
+        }
+        __syncthreads();
+        if (active) {
+            const float* a = lw + e * kc + 4 * half;
+            const float* xx = lx + t * kc + 4 * half;
+            for (int c = 0; c < n / 8; ++c) {
+                const v4f av = *reinterpret_cast<const v4f*>(a + c * 8);
+                const v4f xv = *reinterpret_cast<const v4f*>(xx + c * 8);
+                acc.x = __builtin_fmaf(av.x, xv.x, acc.x);
+                acc.y = __builtin_fmaf(av.y, xv.y, acc.y);
+                acc.z = __builtin_fmaf(av.z, xv.z, acc.z);
+                acc.w = __builtin_fmaf(av.w, xv.w, acc.w);
+            }
+        }
     }
+    // s = acc[0] + acc[1] + ... + acc[7] in order
+    const float h0 = __shfl(acc.x, tid | 1, kWave), h1 = __shfl(acc.y, tid | 1, kWave);
+    const float h2 = __shfl(acc.z, tid | 1, kWave), h3 = __shfl(acc.w, tid | 1, kWave);
+    if (active && half == 0) {
+        float sum = 0.0f;
+        sum += acc.x; sum += acc.y; sum += acc.z; sum += acc.w;
+        sum += h0; sum += h1; sum += h2; sum += h3;
+        logits[(size_t)(t0 + t) * n_expert + e0 + e] = sum;
+    }
+    // ticket: the workgroup that sees every other one of its tile done selects for the tile
+    __threadfence();
+    __syncthreads();
+    if (tid == 0) s_last = atomicAdd(&tickets[blockIdx.y], 1) == (int)gridDim.x - 1;
+    __syncthreads();
+    if (!s_last) return;
+    __threadfence();
+    const int wave = tid >> 6, lane = tid & 63;
+    for (int r = t0 + wave; r < t0 + n_t; r += 4) {
+        int my_e;
+        float my_w;
+        moe_select_wave(logits + (size_t)r * n_expert, sel[wave], n_expert, n_used, scale, lane, my_e, my_w);
+        if (lane < n_used) {
+            sel_idx[(size_t)r * n_used + lane] = my_e;
+            sel_w[(size_t)r * n_used + lane] = my_w;
+        }
+    }
+    if (tid == 0) tickets[blockIdx.y] = 0;
 }
 
 // ───────────────────────────── rows == 1: f32 (ActsKind::Raw) path, Q4_K banks ─────────────────────────────
 // Lane mapping: 4 lanes per 256-block (nibble pair p = lane % 4, 64 weights), S = 4 * nb lanes per
 // weight row, 64 / S rows per wave step. A lane keeps its 64 activation floats in registers.
+// The CPU decodes w = sc*code + mn to f32 and runs an f32 dot; here the same sum is factored per
+// 32 weights as sc * sum(code * x) + mn * sum(x) (one conversion and one FMA per weight), which
+// moves the result by f32 rounding only - orders of magnitude inside the 1e-4 relative bound
+// this path is held to.
 
 struct Q4kF32Row {
     v4i hdr, qa, qb;
 };
 
-__device__ __forceinline__ float q4k_f32_partial(const Q4kF32Row& r, const float* x, int p) {
+struct Q4kF32X {
+    float x[64];
+    float sum_lo, sum_hi;  // sum of x[0..32), x[32..64)
+};
+
+__device__ __forceinline__ void q4k_f32_load_x(Q4kF32X& a, const float* src, bool ok) {
+    float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+        v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (ok) v = *reinterpret_cast<const v4f*>(src + 4 * k);
+        a.x[4 * k + 0] = v.x; a.x[4 * k + 1] = v.y; a.x[4 * k + 2] = v.z; a.x[4 * k + 3] = v.w;
+        if (k < 8) { s0 += v.x + v.y; s1 += v.z + v.w; } else { s2 += v.x + v.y; s3 += v.z + v.w; }
+    }
+    a.sum_lo = s0 + s1;
+    a.sum_hi = s2 + s3;
+}
+
+__device__ __forceinline__ float q4k_f32_partial(const Q4kF32Row& r, const Q4kF32X& a, int p) {
     uint32_t sc8[2], mn8[2];
     k4_all((uint32_t)r.hdr.y, (uint32_t)r.hdr.z, (uint32_t)r.hdr.w, sc8, mn8);
     const uint32_t scw = (p & 2) ? sc8[1] : sc8[0];
@@ -181,23 +238,24 @@ __device__ __forceinline__ float q4k_f32_partial(const Q4kF32Row& r, const float
     const int sh = (p & 1) * 16;
     const float d = f16_bits_to_f32((uint32_t)r.hdr.x & 0xFFFFu);
     const float dmin = f16_bits_to_f32((uint32_t)r.hdr.x >> 16);
-    // dequant_block: sc = f32(d) * (f32)scm_sc; mn = f32(dmin) * (f32)(-m); w = sc * code + mn
-    const float fs_e = d * (float)(int)((scw >> sh) & 0xFF), fs_o = d * (float)(int)((scw >> (sh + 8)) & 0xFF);
-    const float fm_e = dmin * (float)(-(int)((mnw >> sh) & 0xFF)), fm_o = dmin * (float)(-(int)((mnw >> (sh + 8)) & 0xFF));
+    const float fs_lo = d * (float)(int)((scw >> sh) & 0xFF), fs_hi = d * (float)(int)((scw >> (sh + 8)) & 0xFF);
+    const float fm_lo = dmin * (float)(int)((mnw >> sh) & 0xFF), fm_hi = dmin * (float)(int)((mnw >> (sh + 8)) & 0xFF);
     const int wq[8] = {r.qa.x, r.qa.y, r.qa.z, r.qa.w, r.qb.x, r.qb.y, r.qb.z, r.qb.w};
-    float acc = 0.0f;
+    float lo0 = 0.0f, lo1 = 0.0f, hi0 = 0.0f, hi1 = 0.0f;
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
         const uint32_t w = (uint32_t)wq[k];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float qe = (float)((w >> (8 * i)) & 0xF), qo = (float)((w >> (8 * i + 4)) & 0xF);
-            const float we = fs_e * qe + fm_e, wo = fs_o * qo + fm_o;
-            acc = __builtin_fmaf(we, x[4 * k + i], acc);
-            acc = __builtin_fmaf(wo, x[32 + 4 * k + i], acc);
-        }
+        const uint32_t l = w & 0x0F0F0F0Fu, h = (w >> 4) & 0x0F0F0F0Fu;
+        lo0 = __builtin_fmaf((float)(l & 0xFF), a.x[4 * k + 0], lo0);
+        lo1 = __builtin_fmaf((float)((l >> 8) & 0xFF), a.x[4 * k + 1], lo1);
+        lo0 = __builtin_fmaf((float)((l >> 16) & 0xFF), a.x[4 * k + 2], lo0);
+        lo1 = __builtin_fmaf((float)(l >> 24), a.x[4 * k + 3], lo1);
+        hi0 = __builtin_fmaf((float)(h & 0xFF), a.x[32 + 4 * k + 0], hi0);
+        hi1 = __builtin_fmaf((float)((h >> 8) & 0xFF), a.x[32 + 4 * k + 1], hi1);
+        hi0 = __builtin_fmaf((float)((h >> 16) & 0xFF), a.x[32 + 4 * k + 2], hi0);
+        hi1 = __builtin_fmaf((float)(h >> 24), a.x[32 + 4 * k + 3], hi1);
     }
-    return acc;
+    return (fs_lo * (lo0 + lo1) - fm_lo * a.sum_lo) + (fs_hi * (hi0 + hi1) - fm_hi * a.sum_hi);
 }
 
 __device__ __forceinline__ void q4k_f32_load(Q4kF32Row& r, const uint8_t* rowp, int b, int p, bool ok) {
@@ -220,107 +278,105 @@ __device__ __forceinline__ float seg_sum(float v, int seg_base, int nb) {
     return s;
 }
 
-// gate/up at one token: act[slot][o] = silu(gate_e[o] . x) * (up_e[o] . x). Every workgroup
-// derives the routing from the logits itself (one wavefront, a few microseconds, cheaper than a
-// launch of its own); workgroup (0, 0) also publishes it for the down kernel and the caller.
+// gate/up at one token: act[slot][o] = silu(gate_e[o] . x) * (up_e[o] . x), e = ids[slot].
+// A wave takes steps_per_wave consecutive row steps and keeps the next step's rows in flight.
 __global__ __launch_bounds__(256) void moe_gate_up_f32_q4k_kernel(
     const uint8_t* __restrict__ gate, const uint8_t* __restrict__ up, size_t gate_stride,
-    size_t up_stride, const float* __restrict__ logits, int n_expert, int n_used, float scale,
-    int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, const float* __restrict__ x,
+    size_t up_stride, const int32_t* __restrict__ ids, const float* __restrict__ x,
     float* __restrict__ act, int ne, int nff, int steps_per_wave) {
-    __shared__ __attribute__((aligned(16))) float sp[1024];
-    __shared__ float red[2];
-    __shared__ int s_expert;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int nb = ne / 256, S = 4 * nb, rps = 64 / S;  // rows per wave step
     const int seg = lane / S, within = lane % S, b = within >> 2, p = within & 3;
     const bool lane_ok = seg < rps;
     const int slot = blockIdx.y;
-
-    float xr[64];
-#pragma unroll
-    for (int k = 0; k < 16; ++k) {
-        v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (lane_ok) v = *reinterpret_cast<const v4f*>(x + (size_t)b * 256 + p * 64 + 4 * k);
-        xr[4 * k + 0] = v.x; xr[4 * k + 1] = v.y; xr[4 * k + 2] = v.z; xr[4 * k + 3] = v.w;
-    }
-    if (wave == 0) {
-        int my_e;
-        float my_w;
-        moe_select_wave(logits, sp, red, n_expert, n_used, scale, lane, my_e, my_w);
-        if (lane == slot) s_expert = my_e;
-        if (blockIdx.x == 0 && blockIdx.y == 0 && lane < n_used) {
-            sel_idx[lane] = my_e;
-            sel_w[lane] = my_w;
-        }
-    }
-    __syncthreads();
-    const int e = s_expert;
+    const int steps_total = (nff + rps - 1) / rps;
+    const int st0 = (blockIdx.x * 4 + wave) * steps_per_wave;
+    if (st0 >= steps_total) return;
+    const int st_end = min(st0 + steps_per_wave, steps_total);
+    const int e = ids[slot];
     const size_t bpr = (size_t)nb * 144;
     const uint8_t* gw = gate + (size_t)e * gate_stride;
     const uint8_t* uw = up + (size_t)e * up_stride;
-    const int steps_total = (nff + rps - 1) / rps;
-    const int st0 = (blockIdx.x * 4 + wave) * steps_per_wave;
-    for (int st = st0; st < min(st0 + steps_per_wave, steps_total); ++st) {
-        const int o = st * rps + seg;
+    Q4kF32Row g, u;
+    {
+        const int o = st0 * rps + seg;
         const bool ok = lane_ok && o < nff;
-        Q4kF32Row g, u;
         q4k_f32_load(g, gw + (size_t)(ok ? o : 0) * bpr, b, p, ok);
         q4k_f32_load(u, uw + (size_t)(ok ? o : 0) * bpr, b, p, ok);
-        const float gs = seg_sum(q4k_f32_partial(g, xr, p), seg * S, nb);
-        const float us = seg_sum(q4k_f32_partial(u, xr, p), seg * S, nb);
+    }
+    Q4kF32X xa;
+    q4k_f32_load_x(xa, x + (size_t)b * 256 + p * 64, lane_ok);
+    for (int st = st0; st < st_end; ++st) {
+        const int o = st * rps + seg;
+        const bool ok = lane_ok && o < nff;
+        const Q4kF32Row gc = g, uc = u;
+        if (st + 1 < st_end) {
+            const int o2 = o + rps;
+            const bool ok2 = lane_ok && o2 < nff;
+            q4k_f32_load(g, gw + (size_t)(ok2 ? o2 : 0) * bpr, b, p, ok2);
+            q4k_f32_load(u, uw + (size_t)(ok2 ? o2 : 0) * bpr, b, p, ok2);
+        }
+        const float gs = seg_sum(q4k_f32_partial(gc, xa, p), seg * S, nb);
+        const float us = seg_sum(q4k_f32_partial(uc, xa, p), seg * S, nb);
         if (ok && within == 0) act[(size_t)slot * nff + o] = gs / (1.0f + expf(-gs)) * us;
     }
 }
 
 // down + accumulate at one token: out[o] = sum_k w_k * (down_{ids[k]}[o] . act[k]), k in rank
-// order. The n_used activation vectors are staged in LDS once per workgroup and all n_used weight
-// rows of a step are requested before the first is used (one memory latency, not n_used).
-constexpr int kMoeMaxUsedF32 = 8;
+// order. One wave per selected expert (up to 16 at a time), every wave of a workgroup on the same
+// `steps` row steps; the per-expert results meet in LDS and are added in rank order with a
+// separate multiply and add, as the CPU's `*o += w_e * yv`.
+constexpr int kDownMaxSteps = 4, kDownMaxWaves = 16;
 
-__global__ __launch_bounds__(256) void moe_down_f32_q4k_kernel(
+__global__ __launch_bounds__(1024) void moe_down_f32_q4k_kernel(
     const uint8_t* __restrict__ down, size_t down_stride, const int32_t* __restrict__ ids,
     const float* __restrict__ wts, const float* __restrict__ act, float* __restrict__ out, int nff,
-    int ne, int n_used) {
-    extern __shared__ __attribute__((aligned(16))) float la[];  // [n_used][nff]
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int ne, int n_used, int steps) {
+    __shared__ float ys[kDownMaxSteps][kDownMaxWaves][16];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     const int nb = nff / 256, S = 4 * nb, rps = 64 / S;
     const int seg = lane / S, within = lane % S, b = within >> 2, p = within & 3;
     const bool lane_ok = seg < rps;
     const size_t bpr = (size_t)nb * 144;
-    const int st = blockIdx.x * 4 + wave;  // one row step per wave
-    const int o = st * rps + seg;
-    const bool ok = lane_ok && o < ne;
+    const int st0 = blockIdx.x * steps;
+    const int own_s = threadIdx.x / rps, own_seg = threadIdx.x % rps;  // output this thread adds up
+    const bool owner = (int)threadIdx.x < steps * rps;
     float acc = 0.0f;
-    for (int k0 = 0; k0 < n_used; k0 += kMoeMaxUsedF32) {
-        const int kn = min(kMoeMaxUsedF32, n_used - k0);
-        Q4kF32Row rows[kMoeMaxUsedF32];
-#pragma unroll
-        for (int k = 0; k < kMoeMaxUsedF32; ++k) {
-            const bool okk = ok && k < kn;
-            const uint8_t* dw = down + (size_t)ids[okk ? k0 + k : 0] * down_stride;
-            q4k_f32_load(rows[k], dw + (size_t)(okk ? o : 0) * bpr, b, p, okk);
-        }
-        __syncthreads();
-        for (int i = threadIdx.x; i < kn * nff / 4; i += 256)
-            reinterpret_cast<v4f*>(la)[i] = reinterpret_cast<const v4f*>(act + (size_t)k0 * nff)[i];
-        __syncthreads();
-#pragma unroll
-        for (int k = 0; k < kMoeMaxUsedF32; ++k) {
-            if (k < kn) {
-                float xr[64];
-#pragma unroll
-                for (int q = 0; q < 16; ++q) {
-                    v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
-                    if (lane_ok) v = *reinterpret_cast<const v4f*>(la + (size_t)k * nff + (size_t)b * 256 + p * 64 + 4 * q);
-                    xr[4 * q + 0] = v.x; xr[4 * q + 1] = v.y; xr[4 * q + 2] = v.z; xr[4 * q + 3] = v.w;
+    for (int k0 = 0; k0 < n_used; k0 += nw) {
+        const int k = k0 + wave;
+        if (k0) __syncthreads();
+        if (k < n_used) {
+            const uint8_t* dw = down + (size_t)ids[k] * down_stride;
+            Q4kF32Row row;
+            {
+                const int o = st0 * rps + seg;
+                const bool ok = lane_ok && o < ne;
+                q4k_f32_load(row, dw + (size_t)(ok ? o : 0) * bpr, b, p, ok);
+            }
+            Q4kF32X xa;
+            q4k_f32_load_x(xa, act + (size_t)k * nff + (size_t)b * 256 + p * 64, lane_ok);
+            for (int s = 0; s < steps; ++s) {
+                const int o = (st0 + s) * rps + seg;
+                const Q4kF32Row cur = row;
+                if (s + 1 < steps) {
+                    const int o2 = o + rps;
+                    const bool ok2 = lane_ok && o2 < ne;
+                    q4k_f32_load(row, dw + (size_t)(ok2 ? o2 : 0) * bpr, b, p, ok2);
                 }
-                const float yk = seg_sum(q4k_f32_partial(rows[k], xr, p), seg * S, nb);
-                acc += wts[k0 + k] * yk;  // `*o += w_e * yv`: separate multiply and add, rank order
+                const float yk = seg_sum(q4k_f32_partial(cur, xa, p), seg * S, nb);
+                if (lane_ok && within == 0) ys[s][wave][seg] = yk;
             }
         }
+        __syncthreads();
+        if (owner) {
+            const int kn = min(nw, n_used - k0);
+            for (int j = 0; j < kn; ++j) acc += wts[k0 + j] * ys[own_s][j][own_seg];
+        }
     }
-    if (ok && within == 0) out[o] = acc;
+    if (owner) {
+        const int o = (st0 + own_s) * rps + own_seg;
+        if (o < ne) out[o] = acc;
+    }
 }
 
 // ───────────────────────────── rows >= 2: int8 path ─────────────────────────────
@@ -434,22 +490,11 @@ static bool launch_gemv_id(int dtype, const uint8_t* bank, size_t expert_stride,
     }
 }
 
-// The router and the one-token down kernel may stage more than the default 64 KiB of LDS.
-static void moe_raise_lds_limits() {
-    static std::once_flag once;
-    std::call_once(once, [] {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(moe_router_kernel),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(moe_down_f32_q4k_kernel),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    });
-}
-
 size_t moe_workspace_bytes(const MoeShape& s) {
-    moe_raise_lds_limits();
     const size_t pairs = (size_t)s.rows * s.n_used;
     size_t n = 0;
     auto add = [&n](size_t bytes) { n += (bytes + 255) / 256 * 256; };
+    add(((size_t)s.rows + kRouterTokens - 1) / kRouterTokens * 4);  // router tickets (first: zero between ops)
     add((size_t)s.rows * s.n_expert * 4);        // logits
     add(pairs * 4);                               // sel_idx
     add(pairs * 4);                               // sel_w
@@ -475,6 +520,8 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
         p += (bytes + 255) / 256 * 256;
         return r;
     };
+    const size_t tiles = ((size_t)s.rows + kRouterTokens - 1) / kRouterTokens;
+    int* tickets = (int*)take(tiles * 4);
     float* logits = (float*)take((size_t)s.rows * s.n_expert * 4);
     int32_t* sel_idx = (int32_t*)take(pairs * 4);
     float* sel_w = (float*)take(pairs * 4);
@@ -488,42 +535,40 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     aq.bsums = (int32_t*)take(qmax / 32 * 4);
     aq.bsums16 = (int32_t*)take(qmax / 16 * 4);
 
-    moe_raise_lds_limits();
-    const size_t router_lds = (size_t)(kRouterExperts + 1) * s.ne * sizeof(float);
-    if (router_lds > 160 * 1024) return "ne too large for the router kernel's LDS staging";
+    // whole rows in one chunk when they fit 64 KiB of LDS, else kRouterChunk columns at a time
+    const int n_t = std::min(s.rows, kRouterTokens);
+    const int kc = (size_t)(kRouterExperts + n_t) * s.ne * 4 <= 64 * 1024 ? s.ne : kRouterChunk;
+    const size_t router_lds = (size_t)(kRouterExperts + n_t) * kc * sizeof(float);
     hipLaunchKernelGGL(moe_router_kernel,
-                       dim3((unsigned)((s.n_expert + kRouterExperts - 1) / kRouterExperts), (unsigned)s.rows),
-                       dim3(256), router_lds, stream, b.router, b.router_x, logits, s.ne, s.n_expert, s.rows);
-    auto publish_selection = [&]() {
-        if (b.sel_idx) (void)hipMemcpyAsync(b.sel_idx, sel_idx, pairs * 4, hipMemcpyDeviceToDevice, stream);
-        if (b.sel_w) (void)hipMemcpyAsync(b.sel_w, sel_w, pairs * 4, hipMemcpyDeviceToDevice, stream);
-    };
+                       dim3((unsigned)((s.n_expert + kRouterExperts - 1) / kRouterExperts), (unsigned)tiles),
+                       dim3(256), router_lds, stream, b.router, b.router_x, logits, tickets, sel_idx, sel_w,
+                       s.ne, s.n_expert, s.rows, s.n_used, s.scale, kc);
+    if (b.sel_idx) (void)hipMemcpyAsync(b.sel_idx, sel_idx, pairs * 4, hipMemcpyDeviceToDevice, stream);
+    if (b.sel_w) (void)hipMemcpyAsync(b.sel_w, sel_w, pairs * 4, hipMemcpyDeviceToDevice, stream);
 
     if (s.rows == 1) {
         // ActsKind::Raw for every bank (lib.rs:2359: int8_ok = rows >= 2)
         if (s.gate_dtype != 12 || s.up_dtype != 12 || s.down_dtype != 12)
             return "rows == 1 carries Q4_K expert banks only";
         if (s.ne > 4096 || s.n_ff > 4096) return "rows == 1 needs ne, n_ff_exp <= 4096";
+        // row steps per wave: amortise the 64 activation registers while keeping >= ~1024 waves
+        auto steps_per_wave = [](int wave_steps) { return std::max(1, std::min(4, wave_steps / 1024)); };
         const int nb_g = s.ne / 256, rps_g = 64 / (4 * nb_g);
         const int steps_g = (s.n_ff + rps_g - 1) / rps_g;
-        // two row steps per wave once that still leaves >= ~512 workgroups
-        const int spw = steps_g * s.n_used >= 4096 ? 2 : 1;
+        const int spw = steps_per_wave(steps_g * s.n_used);
         hipLaunchKernelGGL(moe_gate_up_f32_q4k_kernel,
                            dim3((unsigned)((steps_g + 4 * spw - 1) / (4 * spw)), (unsigned)s.n_used), dim3(256), 0,
-                           stream, b.gate, b.up, b.gate_stride, b.up_stride, logits, s.n_expert, s.n_used,
-                           s.scale, sel_idx, sel_w, b.x, gbuf, s.ne, s.n_ff, spw);
+                           stream, b.gate, b.up, b.gate_stride, b.up_stride, sel_idx, b.x, gbuf, s.ne, s.n_ff, spw);
         const int nb_d = s.n_ff / 256, rps_d = 64 / (4 * nb_d);
         const int steps_d = (s.ne + rps_d - 1) / rps_d;
-        const size_t down_lds = (size_t)std::min(s.n_used, kMoeMaxUsedF32) * s.n_ff * sizeof(float);
-        hipLaunchKernelGGL(moe_down_f32_q4k_kernel, dim3((unsigned)((steps_d + 3) / 4)), dim3(256), down_lds,
-                           stream, b.down, b.down_stride, sel_idx, sel_w, gbuf, b.dst, s.n_ff, s.ne, s.n_used);
-        publish_selection();
+        const int spw_d = std::min(kDownMaxSteps, steps_per_wave(steps_d * s.n_used));
+        const int nw_d = std::min(s.n_used, kDownMaxWaves);
+        hipLaunchKernelGGL(moe_down_f32_q4k_kernel, dim3((unsigned)((steps_d + spw_d - 1) / spw_d)),
+                           dim3((unsigned)(64 * nw_d)), 0, stream, b.down, b.down_stride, sel_idx, sel_w, gbuf,
+                           b.dst, s.n_ff, s.ne, s.n_used, spw_d);
         return hipGetLastError() == hipSuccess ? nullptr : "kernel launch failed";
     }
 
-    hipLaunchKernelGGL(moe_select_kernel, dim3((unsigned)s.rows), dim3(64), 0, stream, logits, sel_idx,
-                       sel_w, s.n_expert, s.n_used, s.scale);
-    publish_selection();
     // rows >= 2: ActsKind::Super for Q4K/Q6K/Q8_0 banks with in_f % 256 == 0 (moe.rs:42-53)
     auto bytes_per_row = [](int dtype, size_t in_f) -> size_t {
         switch (dtype) {
