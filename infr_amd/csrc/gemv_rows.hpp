@@ -75,6 +75,57 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
     }
 }
 
+// Folded form for short rows of the 16-blocks-per-step formats (Q4_K, Q6_K) with nb <= 8 blocks
+// per row: consecutive weight rows are contiguous in memory, so one wave step takes
+// rps = 16 / nb whole rows at once (block slot q = lane / 4 -> row q / nb, block q % nb) instead of
+// leaving the lanes past the row's end idle. `acts` must hold activation block q % nb for this
+// lane. Per-(row, block) terms are the same code as the unfolded loop and are added per row in
+// ascending block order, so every output equals the unfolded result bit for bit.
+// `osum` is this wave's OrderedSum<1> scratch.
+template <typename F>
+__device__ __forceinline__ void gemv_rows_folded(const uint8_t* __restrict__ w, size_t bpr, int nb,
+                                                 const typename F::Acts& acts,
+                                                 float* __restrict__ y, int row0, int row_end,
+                                                 int lane, float* osum) {
+    static_assert(F::kOrdered, "folded rows exist for the ordered 16-block formats");
+    constexpr int LS = OrderedSum<1>::kRowStride;
+    const int q = lane >> 2, rps = 16 / nb;
+    const int rq = q / nb, bq = q - rq * nb;
+    const bool lane_ok = rq < rps;
+    // columns nb..15 of a scratch row are never written: zero them once so the flush can add all 16
+    for (int i = lane; i < OrderedSum<1>::kFloatsPerWave; i += 64) osum[i] = 0.0f;
+    typename F::Row cur;
+    F::load_row(cur, w + (size_t)row0 * bpr, 0, lane, lane_ok && row0 + rq < row_end);
+    int in_batch = 0, batch_row0 = row0;
+    for (int row = row0; row < row_end; row += rps) {
+        const int nr = row + rps;
+        typename F::Row nxt;
+        F::load_row(nxt, w + (size_t)nr * bpr, 0, lane, lane_ok && nr + rq < row_end);
+        const bool ok = lane_ok && row + rq < row_end;
+        const float term = F::template term<false>(cur, acts, 0, lane, ok, StagePtrs{nullptr, nullptr}, 0);
+        if ((lane & 3) == 0 && lane_ok) osum[(in_batch + rq) * LS + bq] = ok ? term : 0.0f;
+        in_batch += rps;
+        cur = nxt;
+        if (in_batch + rps > 16 || nr >= row_end) {
+            if (lane < in_batch && batch_row0 + lane < row_end) {
+                const v4f* tr = reinterpret_cast<const v4f*>(osum + lane * LS);
+                float acc = 0.0f;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const v4f v = tr[k];
+                    acc += v.x;
+                    acc += v.y;
+                    acc += v.z;
+                    acc += v.w;
+                }
+                y[batch_row0 + lane] = acc;
+            }
+            batch_row0 = nr;
+            in_batch = 0;
+        }
+    }
+}
+
 // Small-batch form: MB activation rows against each weight row, so the weights stream once for
 // up to eight tokens. Every (weight row, activation) pair runs the same per-block code and the
 // same ordered sum as the single-activation loop, so each output equals the m == 1 result bit

@@ -27,177 +27,195 @@ namespace infr {
 
 // ───────────────────────────── router + selection ─────────────────────────────
 
-// Per-wave LDS of the selection: probabilities, the ranked winners, one reduction slot.
+// LDS of one selection: probabilities, their ranks, the ranked winners, reduction slots.
 struct SelectLds {
     float p[1024];
+    int rank[1024];
     float top_p[64];
     int top_e[64];
-    float red[4];
+    float red[8];
 };
 
-// Softmax + stable top-n_used + renormalised weights for one row, run by ONE wavefront.
-// On return lanes 0..n_used-1 hold (expert, weight) of rank = lane. n_expert <= 1024, n_used <= 64.
-__device__ __forceinline__ void moe_select_wave(const float* __restrict__ l, SelectLds& s,
-                                                int n_expert, int n_used, float scale, int lane,
-                                                int& my_e, float& my_w) {
-    float* p = s.p;
+// Softmax + stable top-n_used + renormalised weights for one row, run by a whole 256-thread
+// workgroup. n_expert <= 1024, n_used <= 64. Order-sensitive parts follow the CPU: probabilities
+// are summed in index order by one thread, the stable descending sort is realised by counting
+// rank(e) = #{j : p[j] > p[e] or (p[j] == p[e] and j < e)} on the NORMALISED probabilities
+// (normalising can create ties that the raw exponentials do not have), and the selected
+// probabilities are summed in rank order.
+__device__ __forceinline__ void moe_select_block(const float* __restrict__ l, SelectLds& s,
+                                                 int n_expert, int n_used, float scale, int tid,
+                                                 int32_t* __restrict__ out_idx,
+                                                 float* __restrict__ out_w) {
+    const int lane = tid & 63, wave = tid >> 6;
+    float lv[4];
     float mx = -INFINITY;
-    for (int e = lane; e < n_expert; e += 64) mx = __builtin_fmaxf(mx, l[e]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int e = tid + 256 * i;
+        lv[i] = e < n_expert ? l[e] : -INFINITY;
+        mx = __builtin_fmaxf(mx, lv[i]);
+    }
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) mx = __builtin_fmaxf(mx, __shfl_xor(mx, off, kWave));
-    for (int e = lane; e < n_expert; e += 64) p[e] = expf(l[e] - mx);
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    if (lane == 0) {  // `p.iter().sum()`: index order; 16 LDS values per wait
+    if (lane == 0) s.red[wave] = mx;
+    __syncthreads();
+    mx = __builtin_fmaxf(__builtin_fmaxf(s.red[0], s.red[1]), __builtin_fmaxf(s.red[2], s.red[3]));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int e = tid + 256 * i;
+        if (e < n_expert) {
+            lv[i] = expf(lv[i] - mx);
+            s.p[e] = lv[i];
+            s.rank[e] = 0;
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {  // `p.iter().sum()`: index order; 32 LDS values per wait
         float sum = 0.0f;
         int e = 0;
-        for (; e + 16 <= n_expert; e += 16) {
-            const v4f a = *reinterpret_cast<const v4f*>(p + e), b = *reinterpret_cast<const v4f*>(p + e + 4);
-            const v4f c = *reinterpret_cast<const v4f*>(p + e + 8), d = *reinterpret_cast<const v4f*>(p + e + 12);
-            sum += a.x; sum += a.y; sum += a.z; sum += a.w;
-            sum += b.x; sum += b.y; sum += b.z; sum += b.w;
-            sum += c.x; sum += c.y; sum += c.z; sum += c.w;
-            sum += d.x; sum += d.y; sum += d.z; sum += d.w;
-        }
-        for (; e < n_expert; ++e) sum += p[e];
-        s.red[0] = sum;
-    }
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    const float psum = s.red[0];
-    for (int e = lane; e < n_expert; e += 64) p[e] = p[e] / psum;
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-
-    if (n_expert <= 256) {
-        // stable descending order by counting: rank(e) = #{j : p[j] > p[e] or (p[j] == p[e] and j < e)}
-        for (int e = lane; e < n_expert; e += 64) {
-            const float v = p[e];
-            int rank = 0, j = 0;
-            for (; j + 4 <= n_expert; j += 4) {
-                const v4f q = *reinterpret_cast<const v4f*>(p + j);
-                rank += (q.x > v || (q.x == v && j + 0 < e)) ? 1 : 0;
-                rank += (q.y > v || (q.y == v && j + 1 < e)) ? 1 : 0;
-                rank += (q.z > v || (q.z == v && j + 2 < e)) ? 1 : 0;
-                rank += (q.w > v || (q.w == v && j + 3 < e)) ? 1 : 0;
-            }
-            for (; j < n_expert; ++j) rank += (p[j] > v || (p[j] == v && j < e)) ? 1 : 0;
-            if (rank < n_used) {
-                s.top_e[rank] = e;
-                s.top_p[rank] = v;
-            }
-        }
-    } else {
-        // largest p, lowest index among equals, n_used times
-        for (int k = 0; k < n_used; ++k) {
-            float bv = -INFINITY;
-            int bi = 0x7FFFFFFF;
-            for (int e = lane; e < n_expert; e += 64) {
-                const float v = p[e];
-                if (v > bv || (v == bv && e < bi)) {
-                    bv = v;
-                    bi = e;
-                }
-            }
+        for (; e + 32 <= n_expert; e += 32) {
+            v4f q[8];
 #pragma unroll
-            for (int off = 32; off >= 1; off >>= 1) {
-                const float ov = __shfl_xor(bv, off, kWave);
-                const int oi = __shfl_xor(bi, off, kWave);
-                if (ov > bv || (ov == bv && oi < bi)) {
-                    bv = ov;
-                    bi = oi;
-                }
+            for (int k = 0; k < 8; ++k) q[k] = *reinterpret_cast<const v4f*>(s.p + e + 4 * k);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                sum += q[k].x; sum += q[k].y; sum += q[k].z; sum += q[k].w;
             }
-            if (lane == 0) {
-                s.top_e[k] = bi;
-                s.top_p[k] = bv;
-                p[bi] = -1.0f;  // taken (probabilities are >= 0)
-            }
-            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        }
+        for (; e < n_expert; ++e) sum += s.p[e];
+        s.red[4] = sum;
+    }
+    __syncthreads();
+    const float psum = s.red[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int e = tid + 256 * i;
+        if (e < n_expert) s.p[e] = lv[i] / psum;
+    }
+    __syncthreads();
+    // rank by counting: `parts` threads share an expert when n_expert < 256
+    const int parts = n_expert <= 128 ? 256 / n_expert : 1;
+    const int span = ((n_expert + parts - 1) / parts + 3) & ~3;
+    for (int item = tid; item < n_expert * parts; item += 256) {
+        const int e = item % n_expert, part = item / n_expert;
+        const float v = s.p[e];
+        const int j0 = part * span, j1 = min(n_expert, j0 + span);
+        int cnt = 0, j = j0;
+        for (; j + 4 <= j1; j += 4) {
+            const v4f q = *reinterpret_cast<const v4f*>(s.p + j);
+            cnt += (q.x > v ? 1 : 0) + ((q.x == v && j + 0 < e) ? 1 : 0);
+            cnt += (q.y > v ? 1 : 0) + ((q.y == v && j + 1 < e) ? 1 : 0);
+            cnt += (q.z > v ? 1 : 0) + ((q.z == v && j + 2 < e) ? 1 : 0);
+            cnt += (q.w > v ? 1 : 0) + ((q.w == v && j + 3 < e) ? 1 : 0);
+        }
+        for (; j < j1; ++j) {
+            const float q = s.p[j];
+            cnt += (q > v ? 1 : 0) + ((q == v && j < e) ? 1 : 0);
+        }
+        if (parts > 1) atomicAdd(&s.rank[e], cnt);
+        else s.rank[e] = cnt;
+    }
+    __syncthreads();
+    for (int e = tid; e < n_expert; e += 256) {
+        const int r = s.rank[e];
+        if (r < n_used) {
+            s.top_e[r] = e;
+            s.top_p[r] = s.p[e];
         }
     }
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    float wsum = 0.0f;  // summed in rank order, as the CPU sums its selection
-    for (int k = 0; k < n_used; ++k) wsum += s.top_p[k];
-    wsum = __builtin_fmaxf(wsum, 1e-20f);
-    my_e = lane < n_used ? s.top_e[lane] : 0;
-    my_w = lane < n_used ? s.top_p[lane] / wsum * scale : 0.0f;
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");  // the LDS may be reused for the next row
+    __syncthreads();
+    if (tid < n_used) {
+        float wsum = 0.0f;  // summed in rank order, as the CPU sums its selection
+        for (int k = 0; k < n_used; ++k) wsum += s.top_p[k];
+        wsum = __builtin_fmaxf(wsum, 1e-20f);
+        out_idx[tid] = s.top_e[tid];
+        out_w[tid] = s.top_p[tid] / wsum * scale;
+    }
+}
+
+// One workgroup per row (used when there are several rows; a single row is selected by the
+// router kernel itself).
+__global__ __launch_bounds__(256) void moe_select_kernel(const float* __restrict__ logits,
+                                                         int32_t* __restrict__ sel_idx,
+                                                         float* __restrict__ sel_w, int n_expert,
+                                                         int n_used, float scale) {
+    __shared__ __attribute__((aligned(16))) SelectLds s;
+    const size_t r = blockIdx.x;
+    moe_select_block(logits + r * n_expert, s, n_expert, n_used, scale, threadIdx.x, sel_idx + r * n_used,
+                     sel_w + r * n_used);
 }
 
 // infr-cpu's `dot` keeps 8 FMA accumulators (element i goes to accumulator i mod 8) and adds them
 // in order; each accumulator is a strictly sequential chain, so the order cannot be parallelised
-// across lanes without changing the rounding. A workgroup takes kRouterExperts expert rows and
-// kRouterTokens activation rows: all 256 threads stage K-chunks of them into LDS with coalesced
-// 16-byte loads, and two lanes per (expert, token) pair run the chains from LDS (one float4 of
-// four accumulators each), carrying them across chunks.
-// The last workgroup to finish a token tile (a ticket counter per tile, left at zero again)
-// runs the selection for the tile's rows, which saves a launch. ne % 8 == 0 is required.
-constexpr int kRouterExperts = 4, kRouterTokens = 8, kRouterChunk = 512;
+// beyond the 8 accumulators without changing the rounding. A workgroup takes `epw` expert rows
+// (1 or 4) and 32 / epw activation rows: all 256 threads stage K-chunks of them into LDS with
+// coalesced 16-byte loads, and eight lanes per (expert, token) pair - one accumulator each - run
+// the chains from LDS, carrying them across chunks.
+// With a single row (tickets != nullptr) the last workgroup to finish - a ticket counter, left
+// at zero again - runs the selection too, which saves a launch. ne % 8 == 0 is required.
+constexpr int kRouterPairs = 32, kRouterChunk = 512;
 
 __global__ __launch_bounds__(256) void moe_router_kernel(
     const float* __restrict__ router, const float* __restrict__ rx, float* __restrict__ logits,
     int* __restrict__ tickets, int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, int ne,
-    int n_expert, int rows, int n_used, float scale, int kc) {
-    extern __shared__ __attribute__((aligned(16))) float rl[];  // [kRouterExperts][kc] | [kRouterTokens][kc]
-    __shared__ __attribute__((aligned(16))) SelectLds sel[4];
+    int n_expert, int rows, int n_used, float scale, int kc, int epw) {
+    extern __shared__ __attribute__((aligned(16))) float rl[];  // [epw][kc + 8] | [32 / epw][kc + 8]
+    __shared__ __attribute__((aligned(16))) SelectLds sel;
     __shared__ int s_last;
     const int tid = threadIdx.x;
-    const int e0 = blockIdx.x * kRouterExperts, t0 = blockIdx.y * kRouterTokens;
-    const int n_e = min(kRouterExperts, n_expert - e0), n_t = min(kRouterTokens, rows - t0);
+    const int tpw = kRouterPairs / epw;
+    const int e0 = blockIdx.x * epw, t0 = blockIdx.y * tpw;
+    const int n_e = min(epw, n_expert - e0), n_t = min(tpw, rows - t0);
+    // rows are kc + 8 floats apart in LDS: the lanes of different pairs then read different banks
+    const int ld = kc + 8;
     float* lw = rl;
-    float* lx = rl + kRouterExperts * kc;
-    const int pair = tid >> 1, half = tid & 1;
-    const int e = pair % kRouterExperts, t = pair / kRouterExperts;
-    const bool active = t < kRouterTokens && e < n_e && t < n_t;
-    v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};  // accumulators 4*half .. 4*half+3
+    float* lx = rl + epw * ld;
+    const int pair = tid >> 3, j = tid & 7;
+    const int e = pair % epw, t = pair / epw;
+    const bool active = e < n_e && t < n_t;
+    float acc = 0.0f;  // accumulator j
     for (int k0 = 0; k0 < ne; k0 += kc) {
         const int n = min(kc, ne - k0), n4 = n / 4;
+        const int total = (n_e + n_t) * n4;
         if (k0) __syncthreads();
-        for (int i = tid; i < (n_e + n_t) * n4; i += 256) {
-            const int row = i / n4, q = i % n4;
-            const float* src = row < n_e ? router + (size_t)(e0 + row) * ne : rx + (size_t)(t0 + row - n_e) * ne;
-            float* dst = row < n_e ? lw + row * kc : lx + (row - n_e) * kc;
-            reinterpret_cast<v4f*>(dst)[q] = reinterpret_cast<const v4f*>(src + k0)[q];
+        for (int base = 0; base < total; base += 256 * 8) {  // eight loads in flight per thread
+            v4f tmp[8];
+            float* dst[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int i = base + u * 256 + tid;
+                const int row = i / n4, q = i % n4;
+                const float* src = row < n_e ? router + (size_t)(e0 + row) * ne : rx + (size_t)(t0 + row - n_e) * ne;
+                dst[u] = (row < n_e ? lw + row * ld : lx + (row - n_e) * ld) + 4 * q;
+                if (i < total) tmp[u] = reinterpret_cast<const v4f*>(src + k0)[q];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (base + u * 256 + tid < total) *reinterpret_cast<v4f*>(dst[u]) = tmp[u];
         }
         __syncthreads();
         if (active) {
-            const float* a = lw + e * kc + 4 * half;
-            const float* xx = lx + t * kc + 4 * half;
-            for (int c = 0; c < n / 8; ++c) {
-                const v4f av = *reinterpret_cast<const v4f*>(a + c * 8);
-                const v4f xv = *reinterpret_cast<const v4f*>(xx + c * 8);
-                acc.x = __builtin_fmaf(av.x, xv.x, acc.x);
-                acc.y = __builtin_fmaf(av.y, xv.y, acc.y);
-                acc.z = __builtin_fmaf(av.z, xv.z, acc.z);
-                acc.w = __builtin_fmaf(av.w, xv.w, acc.w);
-            }
+            const float* a = lw + e * ld + j;
+            const float* xx = lx + t * ld + j;
+#pragma unroll 16
+            for (int c = 0; c < n / 8; ++c) acc = __builtin_fmaf(a[c * 8], xx[c * 8], acc);
         }
     }
     // s = acc[0] + acc[1] + ... + acc[7] in order
-    const float h0 = __shfl(acc.x, tid | 1, kWave), h1 = __shfl(acc.y, tid | 1, kWave);
-    const float h2 = __shfl(acc.z, tid | 1, kWave), h3 = __shfl(acc.w, tid | 1, kWave);
-    if (active && half == 0) {
-        float sum = 0.0f;
-        sum += acc.x; sum += acc.y; sum += acc.z; sum += acc.w;
-        sum += h0; sum += h1; sum += h2; sum += h3;
-        logits[(size_t)(t0 + t) * n_expert + e0 + e] = sum;
-    }
-    // ticket: the workgroup that sees every other one of its tile done selects for the tile
+    float sum = 0.0f;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) sum += __shfl(acc, (tid & ~7) + q, kWave);
+    if (active && j == 0) logits[(size_t)(t0 + t) * n_expert + e0 + e] = sum;
+    if (!tickets) return;
+    // ticket: the workgroup that sees every other one done selects
     __threadfence();
     __syncthreads();
-    if (tid == 0) s_last = atomicAdd(&tickets[blockIdx.y], 1) == (int)gridDim.x - 1;
+    if (tid == 0) s_last = atomicAdd(tickets, 1) == (int)gridDim.x - 1;
     __syncthreads();
     if (!s_last) return;
     __threadfence();
-    const int wave = tid >> 6, lane = tid & 63;
-    for (int r = t0 + wave; r < t0 + n_t; r += 4) {
-        int my_e;
-        float my_w;
-        moe_select_wave(logits + (size_t)r * n_expert, sel[wave], n_expert, n_used, scale, lane, my_e, my_w);
-        if (lane < n_used) {
-            sel_idx[(size_t)r * n_used + lane] = my_e;
-            sel_w[(size_t)r * n_used + lane] = my_w;
-        }
-    }
-    if (tid == 0) tickets[blockIdx.y] = 0;
+    moe_select_block(logits, sel, n_expert, n_used, scale, tid, sel_idx, sel_w);
+    if (tid == 0) *tickets = 0;
 }
 
 // ───────────────────────────── rows == 1: f32 (ActsKind::Raw) path, Q4_K banks ─────────────────────────────
@@ -417,6 +435,35 @@ __global__ __launch_bounds__(256) void gemv_id_kernel(const uint8_t* __restrict_
                                osum + (threadIdx.x >> 6) * (F::kOrdered ? OrderedSum<STEPS>::kFloatsPerWave : 0));
 }
 
+// The same for short rows (in_f <= 2048) of Q4_K / Q6_K banks: 16 / nb rows per wave step.
+template <typename F>
+__global__ __launch_bounds__(256) void gemv_id_folded_kernel(const uint8_t* __restrict__ bank,
+                                                             size_t expert_stride, size_t bpr,
+                                                             const int32_t* __restrict__ ids,
+                                                             ActPtrs act, int in_f, int n_used,
+                                                             float* __restrict__ y, int out_f,
+                                                             int rows_per_wave) {
+    const int lane = threadIdx.x & 63;
+    const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int row0 = wave * rows_per_wave;
+    if (row0 >= out_f) return;
+    const int row_end = min(row0 + rows_per_wave, out_f);
+    const int pair = blockIdx.y, r = pair / n_used;
+    const uint8_t* w = bank + (size_t)ids[pair] * expert_stride;
+    const int nb = in_f / 256, q = lane >> 2;
+    const int shift = q - q % nb;  // load_acts addresses block q; this lane wants block q % nb
+    ActPtrs a;
+    a.qs = act.qs + (size_t)r * in_f - (size_t)shift * 256;
+    a.d = act.d + (size_t)r * nb - shift;
+    a.bsums = act.bsums + (size_t)r * (in_f / 32) - shift * 8;
+    a.bsums16 = act.bsums16 + (size_t)r * (in_f / 16) - shift * 16;
+    typename F::Acts acts;
+    F::load_acts(acts, a, 0, lane, q / nb < 16 / nb);
+    __shared__ __attribute__((aligned(16))) float osum[4 * OrderedSum<1>::kFloatsPerWave];
+    gemv_rows_folded<F>(w, bpr, nb, acts, y + (size_t)pair * out_f, row0, row_end, lane,
+                        osum + (threadIdx.x >> 6) * OrderedSum<1>::kFloatsPerWave);
+}
+
 // act = silu(g) * u per pair row, quantized per 256 for the down bank (lib.rs:2824-2892).
 // One wavefront per 256-float chunk.
 __global__ __launch_bounds__(256) void moe_act_quant_kernel(const float* __restrict__ g,
@@ -460,13 +507,27 @@ static bool launch_gemv_id_fmt(const uint8_t* bank, size_t expert_stride, size_t
                                const int32_t* ids, const ActQ8& act, size_t in_f, int n_used,
                                int pairs, float* y, size_t out_f, hipStream_t stream) {
     const int steps = (int)((in_f + F::kElemsPerStep - 1) / F::kElemsPerStep);
+    const ActPtrs a{act.qs, act.d, act.bsums, act.bsums16};
+    if constexpr (F::kOrdered) {
+        if (in_f <= 2048) {  // short rows: fold 16 / nb rows into each wave step
+            const int rps = 16 / (int)(in_f / 256);
+            int wave_steps = 8;
+            while (wave_steps > 1 && ((out_f + rps * wave_steps - 1) / (rps * wave_steps) + 3) / 4 * (size_t)pairs < 1024)
+                wave_steps /= 2;
+            const int rpw = rps * wave_steps;
+            const size_t waves = (out_f + rpw - 1) / rpw;
+            hipLaunchKernelGGL((gemv_id_folded_kernel<F>), dim3((unsigned)((waves + 3) / 4), (unsigned)pairs),
+                               dim3(256), 0, stream, bank, expert_stride, bpr, ids, a, (int)in_f, n_used, y,
+                               (int)out_f, rpw);
+            return true;
+        }
+    }
     // enough rows per wave to amortise loading the activation registers, while keeping the grid
     // (row tiles x pairs) well above the CU count
     int rpw = 8;
     while (rpw > 2 && ((out_f + rpw - 1) / rpw + 3) / 4 * (size_t)pairs < 1024) rpw /= 2;
     const size_t waves = (out_f + rpw - 1) / rpw;
     const dim3 grid((unsigned)((waves + 3) / 4), (unsigned)pairs), block(256);
-    const ActPtrs a{act.qs, act.d, act.bsums, act.bsums16};
 #define INFR_CASE(N)                                                                               \
     case N:                                                                                        \
         hipLaunchKernelGGL((gemv_id_kernel<F, N>), grid, block, 0, stream, bank, expert_stride, bpr, \
@@ -494,7 +555,7 @@ size_t moe_workspace_bytes(const MoeShape& s) {
     const size_t pairs = (size_t)s.rows * s.n_used;
     size_t n = 0;
     auto add = [&n](size_t bytes) { n += (bytes + 255) / 256 * 256; };
-    add(((size_t)s.rows + kRouterTokens - 1) / kRouterTokens * 4);  // router tickets (first: zero between ops)
+    add(4);                                       // router ticket (first: zero between ops)
     add((size_t)s.rows * s.n_expert * 4);        // logits
     add(pairs * 4);                               // sel_idx
     add(pairs * 4);                               // sel_w
@@ -520,8 +581,7 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
         p += (bytes + 255) / 256 * 256;
         return r;
     };
-    const size_t tiles = ((size_t)s.rows + kRouterTokens - 1) / kRouterTokens;
-    int* tickets = (int*)take(tiles * 4);
+    int* tickets = (int*)take(4);
     float* logits = (float*)take((size_t)s.rows * s.n_expert * 4);
     int32_t* sel_idx = (int32_t*)take(pairs * 4);
     float* sel_w = (float*)take(pairs * 4);
@@ -535,14 +595,19 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     aq.bsums = (int32_t*)take(qmax / 32 * 4);
     aq.bsums16 = (int32_t*)take(qmax / 16 * 4);
 
+    // one expert per workgroup at a single row (more workgroups), four once rows fill the pairs;
     // whole rows in one chunk when they fit 64 KiB of LDS, else kRouterChunk columns at a time
-    const int n_t = std::min(s.rows, kRouterTokens);
-    const int kc = (size_t)(kRouterExperts + n_t) * s.ne * 4 <= 64 * 1024 ? s.ne : kRouterChunk;
-    const size_t router_lds = (size_t)(kRouterExperts + n_t) * kc * sizeof(float);
+    const int epw = s.rows == 1 ? 1 : 4, tpw = kRouterPairs / epw;
+    const int n_t = std::min(s.rows, tpw);
+    const int kc = (size_t)(epw + n_t) * (s.ne + 8) * 4 <= 64 * 1024 ? s.ne : kRouterChunk;
+    const size_t router_lds = (size_t)(epw + n_t) * (kc + 8) * sizeof(float);
     hipLaunchKernelGGL(moe_router_kernel,
-                       dim3((unsigned)((s.n_expert + kRouterExperts - 1) / kRouterExperts), (unsigned)tiles),
-                       dim3(256), router_lds, stream, b.router, b.router_x, logits, tickets, sel_idx, sel_w,
-                       s.ne, s.n_expert, s.rows, s.n_used, s.scale, kc);
+                       dim3((unsigned)((s.n_expert + epw - 1) / epw), (unsigned)((s.rows + tpw - 1) / tpw)),
+                       dim3(256), router_lds, stream, b.router, b.router_x, logits, s.rows == 1 ? tickets : nullptr,
+                       sel_idx, sel_w, s.ne, s.n_expert, s.rows, s.n_used, s.scale, kc, epw);
+    if (s.rows > 1)
+        hipLaunchKernelGGL(moe_select_kernel, dim3((unsigned)s.rows), dim3(256), 0, stream, logits, sel_idx,
+                           sel_w, s.n_expert, s.n_used, s.scale);
     if (b.sel_idx) (void)hipMemcpyAsync(b.sel_idx, sel_idx, pairs * 4, hipMemcpyDeviceToDevice, stream);
     if (b.sel_w) (void)hipMemcpyAsync(b.sel_w, sel_w, pairs * 4, hipMemcpyDeviceToDevice, stream);
 
