@@ -436,12 +436,16 @@ __global__ __launch_bounds__(256) void gemv_id_kernel(const uint8_t* __restrict_
 }
 
 // The same for short rows (in_f <= 2048) of Q4_K / Q6_K banks: 16 / nb rows per wave step.
+// blockIdx.z selects one of two same-shaped banks (gate and up share a launch).
 template <typename F>
-__global__ __launch_bounds__(256) void gemv_id_folded_kernel(const uint8_t* __restrict__ bank,
-                                                             size_t expert_stride, size_t bpr,
+__global__ __launch_bounds__(256) void gemv_id_folded_kernel(const uint8_t* __restrict__ bank0,
+                                                             const uint8_t* __restrict__ bank1,
+                                                             size_t expert_stride0,
+                                                             size_t expert_stride1, size_t bpr,
                                                              const int32_t* __restrict__ ids,
                                                              ActPtrs act, int in_f, int n_used,
-                                                             float* __restrict__ y, int out_f,
+                                                             float* __restrict__ y0,
+                                                             float* __restrict__ y1, int out_f,
                                                              int rows_per_wave) {
     const int lane = threadIdx.x & 63;
     const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -449,7 +453,9 @@ __global__ __launch_bounds__(256) void gemv_id_folded_kernel(const uint8_t* __re
     if (row0 >= out_f) return;
     const int row_end = min(row0 + rows_per_wave, out_f);
     const int pair = blockIdx.y, r = pair / n_used;
-    const uint8_t* w = bank + (size_t)ids[pair] * expert_stride;
+    const bool second = blockIdx.z != 0;
+    const uint8_t* w = (second ? bank1 : bank0) + (size_t)ids[pair] * (second ? expert_stride1 : expert_stride0);
+    float* y = second ? y1 : y0;
     const int nb = in_f / 256, q = lane >> 2;
     const int shift = q - q % nb;  // load_acts addresses block q; this lane wants block q % nb
     ActPtrs a;
@@ -502,10 +508,13 @@ __global__ __launch_bounds__(256) void moe_accumulate_kernel(const float* __rest
 
 // ───────────────────────────── launch ─────────────────────────────
 
+// `bank1`/`y1` (optional): a second bank of the same dtype and shape against the same activations.
 template <typename F>
 static bool launch_gemv_id_fmt(const uint8_t* bank, size_t expert_stride, size_t bpr,
                                const int32_t* ids, const ActQ8& act, size_t in_f, int n_used,
-                               int pairs, float* y, size_t out_f, hipStream_t stream) {
+                               int pairs, float* y, size_t out_f, hipStream_t stream,
+                               const uint8_t* bank1 = nullptr, size_t expert_stride1 = 0,
+                               float* y1 = nullptr) {
     const int steps = (int)((in_f + F::kElemsPerStep - 1) / F::kElemsPerStep);
     const ActPtrs a{act.qs, act.d, act.bsums, act.bsums16};
     if constexpr (F::kOrdered) {
@@ -516,12 +525,16 @@ static bool launch_gemv_id_fmt(const uint8_t* bank, size_t expert_stride, size_t
                 wave_steps /= 2;
             const int rpw = rps * wave_steps;
             const size_t waves = (out_f + rpw - 1) / rpw;
-            hipLaunchKernelGGL((gemv_id_folded_kernel<F>), dim3((unsigned)((waves + 3) / 4), (unsigned)pairs),
-                               dim3(256), 0, stream, bank, expert_stride, bpr, ids, a, (int)in_f, n_used, y,
-                               (int)out_f, rpw);
+            hipLaunchKernelGGL((gemv_id_folded_kernel<F>),
+                               dim3((unsigned)((waves + 3) / 4), (unsigned)pairs, bank1 ? 2u : 1u), dim3(256), 0,
+                               stream, bank, bank1, expert_stride, expert_stride1, bpr, ids, a, (int)in_f,
+                               n_used, y, y1, (int)out_f, rpw);
             return true;
         }
     }
+    if (bank1)  // long rows: one launch per bank
+        return launch_gemv_id_fmt<F>(bank, expert_stride, bpr, ids, act, in_f, n_used, pairs, y, out_f, stream) &&
+               launch_gemv_id_fmt<F>(bank1, expert_stride1, bpr, ids, act, in_f, n_used, pairs, y1, out_f, stream);
     // enough rows per wave to amortise loading the activation registers, while keeping the grid
     // (row tiles x pairs) well above the CU count
     int rpw = 8;
@@ -542,11 +555,12 @@ static bool launch_gemv_id_fmt(const uint8_t* bank, size_t expert_stride, size_t
 
 static bool launch_gemv_id(int dtype, const uint8_t* bank, size_t expert_stride, size_t bpr,
                            const int32_t* ids, const ActQ8& act, size_t in_f, int n_used, int pairs,
-                           float* y, size_t out_f, hipStream_t stream) {
+                           float* y, size_t out_f, hipStream_t stream, const uint8_t* bank1 = nullptr,
+                           size_t expert_stride1 = 0, float* y1 = nullptr) {
     switch (dtype) {
-    case 12: return launch_gemv_id_fmt<FmtQ4K>(bank, expert_stride, bpr, ids, act, in_f, n_used, pairs, y, out_f, stream);
-    case 14: return launch_gemv_id_fmt<FmtQ6K>(bank, expert_stride, bpr, ids, act, in_f, n_used, pairs, y, out_f, stream);
-    case 8: return launch_gemv_id_fmt<FmtQ8_0>(bank, expert_stride, bpr, ids, act, in_f, n_used, pairs, y, out_f, stream);
+    case 12: return launch_gemv_id_fmt<FmtQ4K>(bank, expert_stride, bpr, ids, act, in_f, n_used, pairs, y, out_f, stream, bank1, expert_stride1, y1);
+    case 14: return launch_gemv_id_fmt<FmtQ6K>(bank, expert_stride, bpr, ids, act, in_f, n_used, pairs, y, out_f, stream, bank1, expert_stride1, y1);
+    case 8: return launch_gemv_id_fmt<FmtQ8_0>(bank, expert_stride, bpr, ids, act, in_f, n_used, pairs, y, out_f, stream, bank1, expert_stride1, y1);
     default: return false;
     }
 }
@@ -647,9 +661,15 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     const size_t dbpr = bytes_per_row(s.down_dtype, s.n_ff);
     if (!gbpr || !ubpr || !dbpr) return "rows >= 2 carries Q4_K / Q6_K / Q8_0 expert banks";
     launch_quantize_q8(b.x, s.rows, s.ne, false, aq, stream);
-    if (!launch_gemv_id(s.gate_dtype, b.gate, b.gate_stride, gbpr, sel_idx, aq, s.ne, s.n_used, (int)pairs, gbuf, s.n_ff, stream) ||
-        !launch_gemv_id(s.up_dtype, b.up, b.up_stride, ubpr, sel_idx, aq, s.ne, s.n_used, (int)pairs, ubuf, s.n_ff, stream))
-        return "no id-gathered kernel for this gate/up shape";
+    const bool gate_up_ok =
+        s.gate_dtype == s.up_dtype
+            ? launch_gemv_id(s.gate_dtype, b.gate, b.gate_stride, gbpr, sel_idx, aq, s.ne, s.n_used, (int)pairs, gbuf,
+                             s.n_ff, stream, b.up, b.up_stride, ubuf)
+            : launch_gemv_id(s.gate_dtype, b.gate, b.gate_stride, gbpr, sel_idx, aq, s.ne, s.n_used, (int)pairs, gbuf,
+                             s.n_ff, stream) &&
+                  launch_gemv_id(s.up_dtype, b.up, b.up_stride, ubpr, sel_idx, aq, s.ne, s.n_used, (int)pairs, ubuf,
+                                 s.n_ff, stream);
+    if (!gate_up_ok) return "no id-gathered kernel for this gate/up shape";
     const size_t n_act = pairs * s.n_ff;
     hipLaunchKernelGGL(moe_act_quant_kernel, dim3((unsigned)((n_act / 256 + 3) / 4)), dim3(256), 0, stream,
                        gbuf, ubuf, aq.qs, aq.d, aq.bsums, aq.bsums16, n_act);
