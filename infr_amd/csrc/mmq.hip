@@ -120,7 +120,8 @@ struct ActStage {
 };
 
 template <int BM, bool STAGES>
-__global__ __launch_bounds__(256) void mmq_q4k_kernel(const uint8_t* __restrict__ w, size_t bpr,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 32 ? 3 : 2, BM == 32 ? 3 : 2)))
+void mmq_q4k_kernel(const uint8_t* __restrict__ w, size_t bpr,
                                                       const int8_t* __restrict__ qs,
                                                       const float* __restrict__ d8,
                                                       const int32_t* __restrict__ bsums,
@@ -261,9 +262,10 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float
         return launch_gemv_batch(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
     if (dtype == 12) {
         static const int env_bm = getenv("INFR_HIP_MMQ_BM") ? atoi(getenv("INFR_HIP_MMQ_BM")) : 0;
-        // 32-token tiles hold three waves per SIMD; the wider tiles amortise the weight unpack better
-        // but run one wave per SIMD, which measured slower at every M tried (64..2048).
-        const size_t bm = env_bm ? (size_t)env_bm : 32;
+        // 64-token tiles amortise the weight unpack over two token blocks at two waves per SIMD and
+        // measured ~10-14 % faster than 32-token tiles (three waves per SIMD) from M = 512 up; below
+        // that the 32-token grid fills the chip better. 128-token tiles spill.
+        const size_t bm = env_bm ? (size_t)env_bm : (m >= 256 ? 64 : 32);
         if (bm <= 32) launch_mmq_q4k<32>(w, bpr, act, y, m, in_f, out_f, st, stream);
         else if (bm <= 64) launch_mmq_q4k<64>(w, bpr, act, y, m, in_f, out_f, st, stream);
         else launch_mmq_q4k<128>(w, bpr, act, y, m, in_f, out_f, st, stream);
