@@ -182,8 +182,10 @@ static bool launch_plain_fmt(const uint8_t* w, size_t bpr, const ActQ8& a, float
     const int steps = (int)((in_f + F::kElemsPerStep - 1) / F::kElemsPerStep);
     const int n_units = (int)(in_f / F::kBlockElems);
     // Rows per wavefront: enough waves to cover the machine several times over.
+    static const int env_rpw = getenv("INFR_HIP_BATCH_ROWS") ? atoi(getenv("INFR_HIP_BATCH_ROWS")) : 0;
     size_t rpw = (out_f + 4095) / 4096;
     rpw = rpw < 2 ? 2 : (rpw > 16 ? 16 : rpw);
+    if (env_rpw > 0) rpw = (size_t)env_rpw;
     const size_t waves = (out_f + rpw - 1) / rpw;
     const dim3 grid((unsigned)((waves + 3) / 4));
     const ActPtrs act{a.qs, a.d, a.bsums, a.bsums16};
@@ -207,8 +209,10 @@ bool launch_gemv(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, floa
 template <typename F, int STEPS, int MB>
 static void launch_batch_one(const uint8_t* w, size_t bpr, const ActPtrs& act, int m_valid, size_t in_f,
                              float* y, size_t out_f, const StagePtrs& st, hipStream_t stream) {
+    static const int env_rpw = getenv("INFR_HIP_BATCH_ROWS") ? atoi(getenv("INFR_HIP_BATCH_ROWS")) : 0;
     size_t rpw = (out_f + 4095) / 4096;
     rpw = rpw < 2 ? 2 : (rpw > 16 ? 16 : rpw);
+    if (env_rpw > 0) rpw = (size_t)env_rpw;
     const size_t waves = (out_f + rpw - 1) / rpw;
     const dim3 grid((unsigned)((waves + 3) / 4)), block(256);
     if (st.a)

@@ -239,6 +239,182 @@ void mmq_q4k_kernel(const uint8_t* __restrict__ w, size_t bpr,
         }
 }
 
+// ───────────────────────────── skinny form: up to 32 tokens per workgroup ─────────────────────────────
+// With few tokens there are too few 32 x 128 output tiles to fill the chip, and a wave that walks
+// all of K alone is serial for nb blocks. Here a workgroup owns 32 weight rows x 32 tokens and
+// splits K over its NW waves: in every round wave w takes block round*NW + w - loads its weight
+// rows and the activation fragments straight from global memory (L2), unpacks, runs the same 17
+// MFMAs - and parks the exact per-block integers (sd, sm) in LDS. After a barrier all NW*64
+// threads run the f32 epilogue, each for 16/NW of a lane position's outputs, walking the round's
+// blocks in ascending order: the same operations in the same order as the CPU, so the result is
+// bit-identical to the tiled kernel and the GEMV, at NW-fold K parallelism.
+template <int NW, bool STAGES>
+__global__ __launch_bounds__(NW * 64) void mmq_skinny_q4k_kernel(
+    const uint8_t* __restrict__ w, size_t bpr, const int8_t* __restrict__ qs,
+    const float* __restrict__ d8, const int32_t* __restrict__ bsums, float* __restrict__ y, int m,
+    int out_f, int nb, int32_t* __restrict__ st_sd, int32_t* __restrict__ st_sm) {
+    constexpr int RG = 16 / NW;  // accumulators per epilogue thread
+    typedef int vrgi __attribute__((ext_vector_type(RG)));
+    typedef float vrgf __attribute__((ext_vector_type(RG)));
+    __shared__ __attribute__((aligned(16))) int sd_l[NW][NW][64][RG];    // [writer][reader group][lane]
+    __shared__ __attribute__((aligned(16))) float sm_l[NW][NW][64][RG];
+    __shared__ float dd_l[NW][32][2];                                    // d, dmin per writer and row
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, h = lane >> 5;
+    const int tok0 = blockIdx.y * 32;
+    const int wrow = blockIdx.x * 32 + col;
+    const bool row_ok = wrow < out_f;
+    const uint8_t* wrowp = w + (size_t)(row_ok ? wrow : 0) * bpr;
+    const size_t in_f = (size_t)nb * 256;
+    const int atok = min(tok0 + col, m - 1);  // this lane's activation row as MFMA A operand
+    // tokens of this thread's epilogue outputs: accumulator r = RG*wave + i of lane position `lane`
+    int etok[RG];
+#pragma unroll
+    for (int i = 0; i < RG; ++i) {
+        const int r = RG * wave + i;
+        etok[i] = tok0 + 8 * (r >> 2) + 4 * h + (r & 3);
+    }
+    float acc[RG];
+#pragma unroll
+    for (int i = 0; i < RG; ++i) acc[i] = 0.0f;
+
+    // Everything a round reads from global memory is requested one round ahead: the weight rows
+    // (HBM), the activation fragments, per-32 sums and scales (L2).
+    struct RoundIn {
+        Q4kRaw raw;
+        v4i a[8], bs0, bs1;
+        float dq[NW][RG];
+    };
+    auto request = [&](RoundIn& in, int round) {
+        const int b = round * NW + wave;
+        const bool has = b < nb;
+        const int bc = has ? b : 0;
+        const int8_t* ap = qs + (size_t)atok * in_f + (size_t)bc * 256 + h * 16;
+#pragma unroll
+        for (int sb = 0; sb < 8; ++sb) in.a[sb] = *reinterpret_cast<const v4i*>(ap + sb * 32);
+        in.bs0 = *reinterpret_cast<const v4i*>(bsums + (size_t)atok * (nb * 8) + bc * 8);
+        in.bs1 = *reinterpret_cast<const v4i*>(bsums + (size_t)atok * (nb * 8) + bc * 8 + 4);
+#pragma unroll
+        for (int j = 0; j < NW; ++j)
+#pragma unroll
+            for (int i = 0; i < RG; ++i) {
+                const int bj = min(round * NW + j, nb - 1);
+                in.dq[j][i] = d8[(size_t)min(etok[i], m - 1) * nb + bj];
+            }
+        q4k_load_raw(in.raw, wrowp + (size_t)bc * 144, h, row_ok && has);
+    };
+    RoundIn nxt;
+    request(nxt, 0);
+    const int rounds = (nb + NW - 1) / NW;
+    for (int round = 0; round < rounds; ++round) {
+        const int b = round * NW + wave;
+        const bool has = b < nb;
+        const RoundIn in = nxt;
+        if (round + 1 < rounds) request(nxt, round + 1);
+        const Q4kRaw& cur = in.raw;
+        const v4i (&a)[8] = in.a;
+        const float (&dq)[NW][RG] = in.dq;
+        if (has) {
+            const v4i bs0 = in.bs0, bs1 = in.bs1;
+
+            uint32_t sc8[2], mn8[2];
+            k4_all((uint32_t)cur.hdr.y, (uint32_t)cur.hdr.z, (uint32_t)cur.hdr.w, sc8, mn8);
+            v4i blo[8], bhi[8];
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const int qw[4] = {cur.q[p].x, cur.q[p].y, cur.q[p].z, cur.q[p].w};
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const int sb = 2 * p + e;
+                    const uint32_t sc = (sc8[sb >> 2] >> (8 * (sb & 3))) & 0xFFu;
+                    const uint32_t lo3 = sc & 7u, hi3 = sc >> 3;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const uint32_t codes = ((uint32_t)qw[k] >> (4 * e)) & 0x0F0F0F0Fu;
+                        blo[sb][k] = scale_codes(codes, lo3);
+                        bhi[sb][k] = scale_codes(codes, hi3);
+                    }
+                }
+            }
+            v8h bm;
+#pragma unroll
+            for (int sb = 0; sb < 8; ++sb) bm[sb] = (_Float16)(int)((mn8[sb >> 2] >> (8 * (sb & 3))) & 0xFFu);
+            // per-32 sums split bsum = lo + 64*hi': the h = 0 lanes carry lo, the h = 1 lanes bsum - lo
+            const int bsv[8] = {bs0.x, bs0.y, bs0.z, bs0.w, bs1.x, bs1.y, bs1.z, bs1.w};
+            v8h abs_;
+#pragma unroll
+            for (int sb = 0; sb < 8; ++sb) {
+                const int lo = bsv[sb] & 63;
+                abs_[sb] = (_Float16)(h ? bsv[sb] - lo : lo);
+            }
+            const v16i zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            const v16f zf = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            v16i alo = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[0], blo[0], zi, 0, 0, 0);
+            v16i ahi = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[0], bhi[0], zi, 0, 0, 0);
+#pragma unroll
+            for (int sb = 1; sb < 8; ++sb) {
+                alo = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[sb], blo[sb], alo, 0, 0, 0);
+                ahi = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[sb], bhi[sb], ahi, 0, 0, 0);
+            }
+            const v16f smf = __builtin_amdgcn_mfma_f32_32x32x16_f16(abs_, bm, zf, 0, 0, 0);
+#pragma unroll
+            for (int g = 0; g < NW; ++g) {
+                vrgi sdv;
+                vrgf smv;
+#pragma unroll
+                for (int i = 0; i < RG; ++i) {
+                    const int r = RG * g + i;
+                    sdv[i] = alo[r] + (ahi[r] << 3);
+                    smv[i] = smf[r];
+                    if (STAGES) {
+                        const int tok = tok0 + 8 * (r >> 2) + 4 * h + (r & 3);
+                        if (row_ok && tok < m) {
+                            st_sd[((size_t)tok * out_f + wrow) * nb + b] = sdv[i];
+                            st_sm[((size_t)tok * out_f + wrow) * nb + b] = (int)smv[i];
+                        }
+                    }
+                }
+                *reinterpret_cast<vrgi*>(&sd_l[wave][g][lane][0]) = sdv;
+                *reinterpret_cast<vrgf*>(&sm_l[wave][g][lane][0]) = smv;
+            }
+            if (h == 0) {
+                dd_l[wave][col][0] = f16_bits_to_f32((uint32_t)cur.hdr.x & 0xFFFFu);
+                dd_l[wave][col][1] = f16_bits_to_f32((uint32_t)cur.hdr.x >> 16);
+            }
+        }
+        __syncthreads();
+        // f32 epilogue, blocks in ascending order: sumf += q8.d[b] * (d * sd as f32 - dmin * sm as f32)
+#pragma unroll
+        for (int j = 0; j < NW; ++j) {
+            if (round * NW + j < nb) {
+                const vrgi sdv = *reinterpret_cast<const vrgi*>(&sd_l[j][wave][lane][0]);
+                const vrgf smv = *reinterpret_cast<const vrgf*>(&sm_l[j][wave][lane][0]);
+                const float d = dd_l[j][col][0], dmin = dd_l[j][col][1];
+#pragma unroll
+                for (int i = 0; i < RG; ++i) acc[i] += dq[j][i] * (d * (float)sdv[i] - dmin * smv[i]);
+            }
+        }
+        __syncthreads();
+    }
+    if (!row_ok) return;
+#pragma unroll
+    for (int i = 0; i < RG; ++i)
+        if (etok[i] < m) y[(size_t)etok[i] * out_f + wrow] = acc[i];
+}
+
+template <int NW>
+static void launch_mmq_skinny_q4k(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
+                                  size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream) {
+    const dim3 grid((unsigned)((out_f + 31) / 32), (unsigned)((m + 31) / 32)), block(NW * 64);
+    const int nb = (int)(in_f / 256);
+    if (st.a)
+        hipLaunchKernelGGL((mmq_skinny_q4k_kernel<NW, true>), grid, block, 0, stream, w, bpr, act.qs, act.d,
+                           act.bsums, y, (int)m, (int)out_f, nb, st.a, st.b);
+    else
+        hipLaunchKernelGGL((mmq_skinny_q4k_kernel<NW, false>), grid, block, 0, stream, w, bpr, act.qs, act.d,
+                           act.bsums, y, (int)m, (int)out_f, nb, (int32_t*)nullptr, (int32_t*)nullptr);
+}
+
 template <int BM>
 static void launch_mmq_q4k(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
                            size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream) {
@@ -257,9 +433,20 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float
                 size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream) {
     // Small batches and the formats without an MFMA kernel: dot4 GEMV with the activations of up to
     // eight rows in registers (weights re-streamed once per eight rows beyond that).
-    static const int env_mfma_min = getenv("INFR_HIP_MMQ_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_MIN_M")) : 9;
+    static const int env_mfma_min = getenv("INFR_HIP_MMQ_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_MIN_M")) : 2;
+    static const int env_skinny_max = getenv("INFR_HIP_MMQ_SKINNY_MAX_M") ? atoi(getenv("INFR_HIP_MMQ_SKINNY_MAX_M")) : 32;
     if (dtype != 12 || (int)m < env_mfma_min)
         return launch_gemv_batch(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
+    if ((int)m <= env_skinny_max) {
+        // K split over the waves of a workgroup: four blocks per round; eight for long rows or when
+        // four would leave most SIMDs without a wave
+        static const int env_nw = getenv("INFR_HIP_MMQ_SKINNY_WAVES") ? atoi(getenv("INFR_HIP_MMQ_SKINNY_WAVES")) : 0;
+        const size_t wgs = (out_f + 31) / 32 * ((m + 31) / 32);
+        const bool eight = env_nw ? env_nw == 8 : (in_f >= 8192 || (wgs * 4 < 1024 && in_f >= 2048));
+        if (eight) launch_mmq_skinny_q4k<8>(w, bpr, act, y, m, in_f, out_f, st, stream);
+        else launch_mmq_skinny_q4k<4>(w, bpr, act, y, m, in_f, out_f, st, stream);
+        return true;
+    }
     if (dtype == 12) {
         static const int env_bm = getenv("INFR_HIP_MMQ_BM") ? atoi(getenv("INFR_HIP_MMQ_BM")) : 0;
         // 64-token tiles amortise the weight unpack over two token blocks at two waves per SIMD and
