@@ -90,6 +90,9 @@ bool is_quant(int dt) {
 // (crates/infr-cpu/src/lib.rs:1043-1076): per-32 only for Q2_0 among the formats carried here.
 bool act_per32(int dt) { return dt == INFR_DTYPE_Q2_0; }
 
+// Activation scratch for m rows: the prefill kernels read tokens in groups of 32.
+static size_t act_scratch_elems(size_t m, size_t in_f) { return (m == 1 ? 1 : (m + 31) / 32 * 32) * in_f; }
+
 int ensure_act(infr_hip_t* be, size_t elems) {
     if (elems <= be->act_cap_elems) return INFR_HIP_OK;
     HIP_TRY(be, hipStreamSynchronize(be->stream));
@@ -153,12 +156,14 @@ int check_linear(infr_hip_t* be, int dtype, const infr_hip_buffer_t* w, size_t w
 
 int enqueue_linear(infr_hip_t* be, int dtype, const LinearArgs& la, const float* x, float* y,
                    size_t m, size_t in_f, size_t out_f, const infr::IntStages& st) {
-    infr::launch_quantize_q8(x, m, in_f, act_per32(dtype), be->act, be->stream);
     bool ok;
-    if (m == 1)
+    if (m == 1) {
+        infr::launch_quantize_q8(x, m, in_f, act_per32(dtype), be->act, be->stream);
         ok = infr::launch_gemv(dtype, la.wrows, la.bpr, be->act, y, in_f, out_f, st, be->stream);
-    else
-        ok = infr::launch_mmq(dtype, la.wrows, la.bpr, be->act, y, m, in_f, out_f, st, be->stream);
+    } else {
+        // quantizes x into the scratch in the layout its kernel reads, then multiplies
+        ok = infr::launch_mmq(dtype, la.wrows, la.bpr, x, be->act, y, m, in_f, out_f, st, be->stream);
+    }
     if (!ok)
         return fail(be, INFR_HIP_ERR_UNSUPPORTED,
                     "linear: no kernel for dtype " + std::to_string(dtype) + " at in_f " +
@@ -392,7 +397,7 @@ int infr_hip_linear(infr_hip_t* be, int dtype, const infr_hip_buffer_t* w, size_
                                   static_cast<float*>(dst->ptr), la.bpr, (int32_t)out_f};
         return enqueue_gemv_single(be, dtype, in_f, op);
     }
-    if (int rc = ensure_act(be, m * in_f)) return rc;
+    if (int rc = ensure_act(be, act_scratch_elems(m, in_f))) return rc;
     return enqueue_linear(be, dtype, la, static_cast<const float*>(x->ptr),
                           static_cast<float*>(dst->ptr), m, in_f, out_f, infr::IntStages{});
 }
@@ -410,7 +415,7 @@ int infr_hip_linear_int_stages(infr_hip_t* be, int dtype, const infr_hip_buffer_
     if (!a || a->len < need) return fail(be, INFR_HIP_ERR_INVALID, "int_stages: buffer a too small");
     if (dtype == INFR_DTYPE_Q4_K && (!b || b->len < need))
         return fail(be, INFR_HIP_ERR_INVALID, "int_stages: Q4_K needs buffer b");
-    if (int rc = ensure_act(be, m * in_f)) return rc;
+    if (int rc = ensure_act(be, act_scratch_elems(m, in_f))) return rc;
     // y is not wanted here; use a transient output
     float* y = nullptr;
     HIP_TRY(be, hipMalloc((void**)&y, m * out_f * sizeof(float)));
@@ -560,7 +565,7 @@ int infr_hip_compile(infr_hip_t* be, const infr_hip_op_t* ops, size_t n_ops, inf
                 return fail(be, INFR_HIP_ERR_UNSUPPORTED, "compile: Linear op with unsupported dtype/shape");
             }
             p->max_tensor = std::max({p->max_tensor, op.x, op.weight, op.dst});
-            act_need = std::max(act_need, (size_t)op.m * op.in_f);
+            act_need = std::max(act_need, act_scratch_elems(op.m, op.in_f));
         } else if (op.kind == INFR_OP_MOE_FFN) {
             const auto& mp = op.moe;
             if (!mp.ne || !mp.n_expert || !mp.n_used || !mp.n_ff_exp || !mp.rows) {

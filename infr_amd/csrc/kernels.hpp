@@ -21,6 +21,8 @@ struct ActQ8 {
 // quantize_q8 / quantize_q8_32 over m*k contiguous floats.
 void launch_quantize_q8(const float* x, size_t m, size_t k, bool per32, const ActQ8& out,
                         hipStream_t stream);
+// Per-256 quantizer writing MFMA A-operand order (token groups of 32) into the same buffers.
+void launch_quantize_q8_tiled(const float* x, size_t m, size_t k, const ActQ8& out, hipStream_t stream);
 
 // Optional per-block integer-stage outputs, i32 [m][out_f][blocks] (nullptr = not wanted).
 struct IntStages {
@@ -77,8 +79,10 @@ bool launch_gemv_fused(int dtype, size_t in_f, const GemvOpDesc* ops, int n, con
                        const GemvGroupPlan& plan, hipStream_t stream);
 
 // m >= 2: GEMM over on-device quantized activations. y is [m][out_f] row-major.
-bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
-                size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream);
+// m >= 2: quantizes x [m, in_f] into `act` (sized for m rounded up to 32 rows) in the layout the
+// chosen kernel reads, then multiplies.
+bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const ActQ8& act, float* y,
+                size_t m, size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream);
 
 // Op::MoeFfn (qwen3moe form). Expert e of a bank starts at bank + e * stride.
 struct MoeShape {

@@ -23,7 +23,8 @@
 // waves, from LDS. Per 256-block and 32x32 output tile: 16 int8 MFMAs + 1 f16 MFMA against
 // 7 VALU instructions per output for the epilogue.
 //
-// Small batches (m <= 8) and the other formats take the multi-activation dot4 GEMV (gemv.hip).
+// This tiled kernel serves 33..127 tokens; fewer take the skinny kernel and more the shared-operand
+// kernel, both further down. The other formats take the multi-activation dot4 GEMV (gemv.hip).
 #include <cstdlib>
 
 #include "device_common.hpp"
@@ -120,8 +121,7 @@ struct ActStage {
 };
 
 template <int BM, bool STAGES>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 32 ? 3 : 2, BM == 32 ? 3 : 2)))
-void mmq_q4k_kernel(const uint8_t* __restrict__ w, size_t bpr,
+__global__ __launch_bounds__(256) void mmq_q4k_kernel(const uint8_t* __restrict__ w, size_t bpr,
                                                       const int8_t* __restrict__ qs,
                                                       const float* __restrict__ d8,
                                                       const int32_t* __restrict__ bsums,
@@ -237,6 +237,231 @@ void mmq_q4k_kernel(const uint8_t* __restrict__ w, size_t bpr,
             const int tok = tok0 + tb * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
             if (tok < m) y[(size_t)tok * out_f + wrow] = acc[tb][r];
         }
+}
+
+// ───────────────────────────── shared-operand form: 128 tokens x 32*T rows per workgroup ─────────────────────────────
+// The tiled kernel above unpacks a weight block once per 32*TB tokens and is bound by that VALU
+// work. Here the four waves of a workgroup own 32 tokens each and share the unpacked rows through
+// LDS: wave w unpacks nibble pair w (sub-blocks 2w, 2w+1) of every row of the block - a quarter of
+// the work - into MFMA B-operand order, double-buffered so that block b+1 is unpacked while block
+// b is multiplied, one barrier per block. The unpack cost per 32x32 output tile falls from ~250
+// (or ~125 at 64-token tiles) to ~60 VALU instructions, each wave carries one or two accumulator
+// tiles only, and the activation fragments go from global memory (L2) straight to registers.
+// Integers, epilogue expression and block order are those of the tiled kernel: same bits.
+template <int T>
+struct SharedLds {
+    static constexpr int b_bytes = 8 * 2 * T * 1024;   // [sub-block][plane][row tile][lane] x 16 B
+    static constexpr int mn_off = b_bytes;             // [row tile][row][8] f16 mins
+    static constexpr int dd_off = mn_off + T * 32 * 16;  // [row tile][row] (d, dmin)
+    static constexpr int bytes = dd_off + T * 32 * 8;
+};
+
+template <int T, bool STAGES>
+__global__ __launch_bounds__(256) void mmq_shared_q4k_kernel(
+    const uint8_t* __restrict__ w, size_t bpr, const int8_t* __restrict__ qs,
+    const float* __restrict__ d8, const _Float16* __restrict__ bsh, float* __restrict__ y, int m,
+    int out_f, int nb, int32_t* __restrict__ st_sd, int32_t* __restrict__ st_sm) {
+    typedef SharedLds<T> L;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * L::bytes];
+    __shared__ __attribute__((aligned(16))) float dql[4][32];  // per wave: its tokens' activation scales
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, h = lane >> 5;
+    const int tok0 = blockIdx.y * 128 + wave * 32;
+    const int row0 = blockIdx.x * (32 * T);
+    const int p = wave;  // the nibble pair this wave unpacks
+
+    const uint8_t* wrowp[T];
+    bool row_ok[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        row_ok[t] = row0 + 32 * t + col < out_f;
+        wrowp[t] = w + (size_t)(row_ok[t] ? row0 + 32 * t + col : 0) * bpr;
+    }
+    v16f acc[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[t][i] = 0.0f;
+
+    v4i hdr[T], qv[T];  // raw bytes of the block to unpack next
+    auto request_rows = [&](int b) {
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            const uint8_t* blk = wrowp[t] + (size_t)b * 144;
+            hdr[t] = load16(blk);
+            qv[t] = load16(blk + 16 + p * 32 + h * 16);
+        }
+    };
+    auto unpack_to = [&](uint8_t* buf) {
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            uint32_t sc8[2], mn8[2];
+            k4_all((uint32_t)hdr[t].y, (uint32_t)hdr[t].z, (uint32_t)hdr[t].w, sc8, mn8);
+            const uint32_t scw = (p & 2) ? sc8[1] : sc8[0], mnw = (p & 2) ? mn8[1] : mn8[0];
+            const int sh = (p & 1) * 16;
+            const int qw[4] = {qv[t].x, qv[t].y, qv[t].z, qv[t].w};
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {  // e = 0: sub-block 2p (low nibbles), 1: 2p+1 (high)
+                const uint32_t sc = (scw >> (sh + 8 * e)) & 0xFFu;
+                const uint32_t lo3 = sc & 7u, hi3 = sc >> 3;
+                v4i blo, bhi;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t codes = ((uint32_t)qw[k] >> (4 * e)) & 0x0F0F0F0Fu;
+                    blo[k] = scale_codes(codes, lo3);
+                    bhi[k] = scale_codes(codes, hi3);
+                }
+                uint8_t* dst = buf + (size_t)(((2 * p + e) * 2) * T + t) * 1024 + lane * 16;
+                *reinterpret_cast<v4i*>(dst) = blo;
+                *reinterpret_cast<v4i*>(dst + T * 1024) = bhi;
+            }
+            if (h == 0) {
+                // the two mins of this pair as f16, k-slots 2p and 2p+1 of the row's eight
+                typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+                const h2 mn = {(_Float16)(int)((mnw >> sh) & 0xFFu), (_Float16)(int)((mnw >> (sh + 8)) & 0xFFu)};
+                *reinterpret_cast<h2*>(buf + L::mn_off + (t * 32 + col) * 16 + p * 4) = mn;
+                if (p == 0) {
+                    float* dd = reinterpret_cast<float*>(buf + L::dd_off) + (t * 32 + col) * 2;
+                    dd[0] = f16_bits_to_f32((uint32_t)hdr[t].x & 0xFFFFu);
+                    dd[1] = f16_bits_to_f32((uint32_t)hdr[t].x >> 16);
+                }
+            }
+        }
+    };
+    // activation fragments in the tiled quantizer's order: every load is a contiguous kilobyte
+    v4i a[8];
+    v8h abs_;  // split per-32 sums: the h = 0 lanes carry bsum & 63, the h = 1 lanes the rest
+    float dtok;
+    // this wave's group of 32 tokens; a wave wholly past m recomputes the last group (nothing is stored)
+    const size_t g = min((size_t)blockIdx.y * 4 + wave, (size_t)(m - 1) / 32);
+    auto request_acts = [&](int b) {
+        const size_t gb = g * nb + b;
+        const int8_t* ap = qs + gb * (8 * 1024) + lane * 16;
+#pragma unroll
+        for (int sb = 0; sb < 8; ++sb) a[sb] = *reinterpret_cast<const v4i*>(ap + sb * 1024);
+        abs_ = *reinterpret_cast<const v8h*>(bsh + (gb * 64 + lane) * 8);
+        dtok = d8[gb * 32 + col];
+    };
+
+    // Requests past the last block are clamped to it (redundant loads, never consumed) so that the
+    // loop body is straight-line code and every wait covers exactly the loads it needs.
+    // The prologue leaves the same loads pending, in the same order (weight rows older than the
+    // activation fragments), as the loop's back edge does.
+    request_rows(0);
+    unpack_to(lds);
+    request_rows(min(1, nb - 1));
+    request_acts(0);
+    __syncthreads();
+
+    for (int b = 0; b < nb; ++b) {
+        const uint8_t* cur = lds + (b & 1) * L::bytes;
+        // ---- unpack block b+1 into the other buffer, then ask for block b+2's bytes ----
+        unpack_to(lds + ((b + 1) & 1) * L::bytes);
+        request_rows(min(b + 2, nb - 1));
+        // ---- this wave's 32 tokens of block b ----
+        const v8h abs_b = abs_;
+        if (h == 0) dql[wave][col] = dtok;
+        v16i alo[T], ahi[T];
+        const v16i zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        const v16f zf = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        __builtin_amdgcn_s_setprio(1);  // matrix work first: the other waves' VALU fills the gaps
+        // B fragments run one sub-block ahead of the MFMAs that consume them
+        v4i flo[T], fhi[T];
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            const uint8_t* src = cur + (size_t)t * 1024 + lane * 16;
+            flo[t] = *reinterpret_cast<const v4i*>(src);
+            fhi[t] = *reinterpret_cast<const v4i*>(src + T * 1024);
+        }
+#pragma unroll
+        for (int sb = 0; sb < 8; ++sb) {
+            v4i nlo[T], nhi[T];
+            if (sb < 7) {
+#pragma unroll
+                for (int t = 0; t < T; ++t) {
+                    const uint8_t* src = cur + (size_t)(((sb + 1) * 2) * T + t) * 1024 + lane * 16;
+                    nlo[t] = *reinterpret_cast<const v4i*>(src);
+                    nhi[t] = *reinterpret_cast<const v4i*>(src + T * 1024);
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                alo[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[sb], flo[t], sb ? alo[t] : zi, 0, 0, 0);
+                ahi[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[sb], fhi[t], sb ? ahi[t] : zi, 0, 0, 0);
+            }
+            if (sb < 7) {
+#pragma unroll
+                for (int t = 0; t < T; ++t) {
+                    flo[t] = nlo[t];
+                    fhi[t] = nhi[t];
+                }
+            }
+        }
+        // issue order: the LDS reads of sub-block s+1 go out before the MFMAs of sub-block s
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * T, 0);
+#pragma unroll
+        for (int sb = 0; sb < 7; ++sb) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 2 * T, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 2 * T, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 2 * T, 0);
+        __builtin_amdgcn_s_setprio(0);
+        // the activation registers are free: fetch block b+1 while the epilogue runs
+        const int b_this = b;
+        request_acts(min(b + 1, nb - 1));
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            const v8h bm = *reinterpret_cast<const v8h*>(cur + L::mn_off + (t * 32 + col) * 16);
+            const v16f smf = __builtin_amdgcn_mfma_f32_32x32x16_f16(abs_b, bm, zf, 0, 0, 0);
+            const float* dd = reinterpret_cast<const float*>(cur + L::dd_off) + (t * 32 + col) * 2;
+            const float d = dd[0], dmin = dd[1];
+            const int wrow = row0 + 32 * t + col;
+            // accumulator i of this lane is token 8*(i/4) + 4*h + i%4 of the wave's 32
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const v4f dq = *reinterpret_cast<const v4f*>(&dql[wave][8 * j + 4 * h]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int r = 4 * j + i;
+                    const int sd = alo[t][r] + (ahi[t][r] << 3);
+                    if (STAGES) {
+                        const int tok = tok0 + 8 * j + 4 * h + i;
+                        if (row_ok[t] && tok < m) {
+                            st_sd[((size_t)tok * out_f + wrow) * nb + b_this] = sd;
+                            st_sm[((size_t)tok * out_f + wrow) * nb + b_this] = (int)smf[r];
+                        }
+                    }
+                    // sumf += q8.d[b] * (d * sd as f32 - dmin * sm as f32)
+                    acc[t][r] += dq[i] * (d * (float)sd - dmin * smf[r]);
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        if (!row_ok[t]) continue;
+        const int wrow = row0 + 32 * t + col;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int tok = tok0 + 8 * (r >> 2) + 4 * h + (r & 3);
+            if (tok < m) y[(size_t)tok * out_f + wrow] = acc[t][r];
+        }
+    }
+}
+
+template <int T>
+static void launch_mmq_shared_q4k(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
+                                  size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream) {
+    const dim3 grid((unsigned)((out_f + 32 * T - 1) / (32 * T)), (unsigned)((m + 127) / 128)), block(256);
+    const int nb = (int)(in_f / 256);
+    if (st.a)
+        hipLaunchKernelGGL((mmq_shared_q4k_kernel<T, true>), grid, block, 0, stream, w, bpr, act.qs, act.d,
+                           reinterpret_cast<const _Float16*>(act.bsums), y, (int)m, (int)out_f, nb, st.a, st.b);
+    else
+        hipLaunchKernelGGL((mmq_shared_q4k_kernel<T, false>), grid, block, 0, stream, w, bpr, act.qs, act.d,
+                           reinterpret_cast<const _Float16*>(act.bsums), y, (int)m, (int)out_f, nb, (int32_t*)nullptr, (int32_t*)nullptr);
 }
 
 // ───────────────────────────── skinny form: up to 32 tokens per workgroup ─────────────────────────────
@@ -429,36 +654,38 @@ static void launch_mmq_q4k(const uint8_t* w, size_t bpr, const ActQ8& act, float
                            (int32_t*)nullptr);
 }
 
-bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
-                size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream) {
-    // Small batches and the formats without an MFMA kernel: dot4 GEMV with the activations of up to
-    // eight rows in registers (weights re-streamed once per eight rows beyond that).
-    static const int env_mfma_min = getenv("INFR_HIP_MMQ_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_MIN_M")) : 2;
+bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const ActQ8& act, float* y,
+                size_t m, size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream) {
+    // Q4_K routes by token count (thresholds from sweeps at K = 4096, N = 12288; the env knobs exist
+    // for such sweeps):
+    //   2..32      skinny kernel, K split over the waves of a workgroup
+    //   33..127    tiled kernel, 32 tokens x 128 rows per workgroup (most workgroups for few tokens)
+    //   128..      shared-operand kernel, 128 tokens x 32 rows (x 64 rows from 1024 tokens up)
+    // The other formats take the dot4 GEMV with the activations of up to eight rows in registers
+    // (weights re-streamed once per eight rows beyond that).
     static const int env_skinny_max = getenv("INFR_HIP_MMQ_SKINNY_MAX_M") ? atoi(getenv("INFR_HIP_MMQ_SKINNY_MAX_M")) : 32;
-    if (dtype != 12 || (int)m < env_mfma_min)
-        return launch_gemv_batch(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
+    static const int env_shared_min = getenv("INFR_HIP_MMQ_SHARED_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_SHARED_MIN_M")) : 128;
+    static const int env_shared_rows = getenv("INFR_HIP_MMQ_SHARED_ROWS") ? atoi(getenv("INFR_HIP_MMQ_SHARED_ROWS")) : 0;
+    if (dtype == 12 && (int)m >= env_shared_min) {
+        launch_quantize_q8_tiled(x, m, in_f, act, stream);
+        const bool wide = env_shared_rows ? env_shared_rows == 64 : m >= 1024;
+        if (wide) launch_mmq_shared_q4k<2>(w, bpr, act, y, m, in_f, out_f, st, stream);
+        else launch_mmq_shared_q4k<1>(w, bpr, act, y, m, in_f, out_f, st, stream);
+        return true;
+    }
+    launch_quantize_q8(x, m, in_f, dtype == 42, act, stream);
+    if (dtype != 12) return launch_gemv_batch(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
     if ((int)m <= env_skinny_max) {
-        // K split over the waves of a workgroup: four blocks per round; eight for long rows or when
-        // four would leave most SIMDs without a wave
-        static const int env_nw = getenv("INFR_HIP_MMQ_SKINNY_WAVES") ? atoi(getenv("INFR_HIP_MMQ_SKINNY_WAVES")) : 0;
+        // four blocks per round; eight for long rows or when four would leave most SIMDs without a wave
         const size_t wgs = (out_f + 31) / 32 * ((m + 31) / 32);
-        const bool eight = env_nw ? env_nw == 8 : (in_f >= 8192 || (wgs * 4 < 1024 && in_f >= 2048));
-        if (eight) launch_mmq_skinny_q4k<8>(w, bpr, act, y, m, in_f, out_f, st, stream);
-        else launch_mmq_skinny_q4k<4>(w, bpr, act, y, m, in_f, out_f, st, stream);
+        if (in_f >= 8192 || (wgs * 4 < 1024 && in_f >= 2048))
+            launch_mmq_skinny_q4k<8>(w, bpr, act, y, m, in_f, out_f, st, stream);
+        else
+            launch_mmq_skinny_q4k<4>(w, bpr, act, y, m, in_f, out_f, st, stream);
         return true;
     }
-    if (dtype == 12) {
-        static const int env_bm = getenv("INFR_HIP_MMQ_BM") ? atoi(getenv("INFR_HIP_MMQ_BM")) : 0;
-        // 64-token tiles amortise the weight unpack over two token blocks at two waves per SIMD and
-        // measured ~10-14 % faster than 32-token tiles (three waves per SIMD) from M = 512 up; below
-        // that the 32-token grid fills the chip better. 128-token tiles spill.
-        const size_t bm = env_bm ? (size_t)env_bm : (m >= 256 ? 64 : 32);
-        if (bm <= 32) launch_mmq_q4k<32>(w, bpr, act, y, m, in_f, out_f, st, stream);
-        else if (bm <= 64) launch_mmq_q4k<64>(w, bpr, act, y, m, in_f, out_f, st, stream);
-        else launch_mmq_q4k<128>(w, bpr, act, y, m, in_f, out_f, st, stream);
-        return true;
-    }
-    return false;
+    launch_mmq_q4k<32>(w, bpr, act, y, m, in_f, out_f, st, stream);
+    return true;
 }
 
 }  // namespace infr

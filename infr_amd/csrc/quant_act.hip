@@ -27,6 +27,47 @@ __global__ __launch_bounds__(256) void quantize_q8_kernel(const float* __restric
     quantize_chunk<PER32>(v, live, lane, chunk, qs, d, bsums, bsums16);
 }
 
+// The per-256 quantizer writing MFMA A-operand order for the shared-operand prefill kernel
+// (same codes, scales and sums; only their place in memory differs). Tokens go in groups of 32;
+// for group g and block b:
+//   qs    [(g*nb + b)*8 + sub-block][lane = h*32 + token%32][16 B]: k = 16h .. 16h+15 of the sub-block
+//   d     [(g*nb + b)*32 + token%32]
+//   bsums (read as f16) [(g*nb + b)*64 + h*32 + token%32][8]: per-32 sums split bsum = lo + rest,
+//         lo = bsum & 63 in the h = 0 half, bsum - lo in the h = 1 half (both exact in f16)
+// so that a wave's fragment load is one contiguous kilobyte. Slots of tokens past m are not written.
+__global__ __launch_bounds__(256) void quantize_q8_tiled_kernel(const float* __restrict__ x,
+                                                                int8_t* __restrict__ qs,
+                                                                float* __restrict__ d,
+                                                                _Float16* __restrict__ bsh,
+                                                                size_t n_chunks, int nb) {
+    const int lane = threadIdx.x & 63;
+    const size_t chunk = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (chunk >= n_chunks) return;  // wave-uniform
+    const v4f v = *reinterpret_cast<const v4f*>(x + chunk * 256 + (size_t)lane * 4);
+    uint32_t packed;
+    float dd;
+    int s, s16;
+    quantize_chunk_values<false>(v, packed, dd, s, s16);
+    const size_t tok = chunk / nb, b = chunk % nb;
+    const size_t gb = (tok >> 5) * nb + b;
+    const int col = (int)(tok & 31);
+    const int sb = lane >> 3, h = (lane >> 2) & 1, j4 = lane & 3;
+    reinterpret_cast<uint32_t*>(qs)[((gb * 8 + sb) * 64 + h * 32 + col) * 4 + j4] = packed;
+    if (lane == 0) d[gb * 32 + col] = dd;
+    if ((lane & 7) == 0) {
+        const int lo = s & 63;
+        bsh[(gb * 64 + col) * 8 + sb] = (_Float16)lo;
+        bsh[(gb * 64 + 32 + col) * 8 + sb] = (_Float16)(s - lo);
+    }
+}
+
+void launch_quantize_q8_tiled(const float* x, size_t m, size_t k, const ActQ8& out, hipStream_t stream) {
+    const size_t n_chunks = m * k / 256;
+    if (n_chunks == 0) return;
+    hipLaunchKernelGGL(quantize_q8_tiled_kernel, dim3((unsigned)((n_chunks + 3) / 4)), dim3(256), 0, stream, x,
+                       out.qs, out.d, reinterpret_cast<_Float16*>(out.bsums), n_chunks, (int)(k / 256));
+}
+
 void launch_quantize_q8(const float* x, size_t m, size_t k, bool per32, const ActQ8& out,
                         hipStream_t stream) {
     const size_t n_elems = m * k;
