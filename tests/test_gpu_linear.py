@@ -145,3 +145,39 @@ def test_prefill_other_formats_vs_oracle(be, dtype):
     x = synth_normal_f32(10, m * in_f)
     y = run_linear(be, dtype, w, x, m, in_f, out_f)
     gate(y, orc.linear(dtype, w, x, m, in_f, out_f))
+
+
+# ───────────── hand-derived known answers (tests/golden/known_answers.json), no oracle involved ─────────────
+
+def _golden():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "known_answers.json")) as f:
+        return json.load(f)
+
+
+@pytest.mark.parametrize("case", _golden()["dots"], ids=lambda c: c["name"])
+@pytest.mark.parametrize("m", [1, 3, 40, 130])
+def test_known_answer_dots_on_the_device(be, case, m):
+    """Every kernel route (decode GEMV, batch GEMV, skinny / tiled / shared MFMA) against values
+    derived on paper: out_f copies of the row, m copies of the all-127 activation."""
+    row = b"".join(bytes.fromhex(h) * n for h, n in case["parts"])
+    out_f, in_f, dtype = 37, case["in_f"], case["dtype"]
+    w = np.frombuffer(row * out_f, np.uint8)
+    x = np.full(m * in_f, 127.0, np.float32)
+    y = run_linear(be, dtype, w, x, m, in_f, out_f)
+    assert np.all(y == np.float32(case["y"]))
+    a, b = be.linear_int_stages(dtype, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
+    assert np.array_equal(a.reshape(m * out_f, -1), np.tile(np.array(case["int_a"], np.int32), (m * out_f, 1)))
+    if "int_b" in case:
+        assert np.array_equal(b.reshape(m * out_f, -1), np.tile(np.array(case["int_b"], np.int32), (m * out_f, 1)))
+
+
+def test_known_answer_quantizer_ties_on_the_device(be):
+    g = _golden()["quantize_q8"]
+    x = np.zeros(g["k"], np.float32)
+    x[:len(g["x_head"])] = g["x_head"]
+    qs, d, bs, bs16 = be.quantize_q8(be.upload_new(x), 1, g["k"])
+    assert d[0, 0] == g["d"] and list(qs[0, :len(g["q_head"])]) == g["q_head"]
+    assert not qs[0, len(g["q_head"]):].any()
+    assert bs[0, 0] == g["bsums0"] and bs16[0, 0] == g["bsums16_0"] and not bs[0, 1:].any() and not bs16[0, 1:].any()

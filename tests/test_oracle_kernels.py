@@ -295,3 +295,24 @@ def test_linear_rejects_ragged_in_f():
     w = orc.synth_weight(orc.Q8_0, 96 * 4, 1)
     with pytest.raises(ValueError):
         orc.linear(orc.Q8_0, w, np.zeros(96, np.float32), 1, 96, 4)   # per-32 Q8_0 arm is not restated
+
+
+# ───────────── the committed known-answer fixture, through Op::Linear ─────────────
+
+def _golden():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "known_answers.json")) as f:
+        return json.load(f)
+
+
+@pytest.mark.parametrize("case", _golden()["dots"], ids=lambda c: c["name"])
+def test_golden_known_answers_through_linear(case):
+    row = np.frombuffer(b"".join(bytes.fromhex(h) * n for h, n in case["parts"]), np.uint8)
+    w = np.tile(row, 3)
+    y = orc.linear(case["dtype"], w, np.tile(X127, 2), 2, case["in_f"], 3)
+    assert np.all(y == np.float32(case["y"]))
+    a, b = orc.linear_int_stages(case["dtype"], w, np.tile(X127, 2), 2, case["in_f"], 3)
+    assert np.array_equal(np.asarray(a).reshape(6, -1), np.tile(np.array(case["int_a"], np.int32), (6, 1)))
+    if "int_b" in case:
+        assert np.array_equal(np.asarray(b).reshape(6, -1), np.tile(np.array(case["int_b"], np.int32), (6, 1)))
