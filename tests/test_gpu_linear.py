@@ -181,3 +181,57 @@ def test_known_answer_quantizer_ties_on_the_device(be):
     assert d[0, 0] == g["d"] and list(qs[0, :len(g["q_head"])]) == g["q_head"]
     assert not qs[0, len(g["q_head"]):].any()
     assert bs[0, 0] == g["bsums0"] and bs16[0, 0] == g["bsums16_0"] and not bs[0, 1:].any() and not bs16[0, 1:].any()
+
+
+# ───────────── full benchmark sizes: sampled rows against the oracle + batch == single ─────────────
+
+def _oracle_rows(dtype, w, x, m, in_f, out_f, row0, n):
+    """Oracle output for weight rows [row0, row0 + n) only (Op::Linear's w_off slicing)."""
+    return orc.linear(dtype, w, x, m, in_f, n, w_numel=out_f * in_f, w_off=row0 * in_f)
+
+
+@pytest.mark.parametrize("dtype", [DType.Q4K, DType.Q6K, DType.Q8_0, DType.Q2_0])
+@pytest.mark.parametrize("in_f,out_f", [(4096, 12288), (12288, 4096)])
+def test_full_size_decode_rows_vs_oracle(be, dtype, in_f, out_f):
+    w = synth_weight(dtype, 900 + in_f, out_f, in_f)
+    x = synth_normal_f32(901, in_f)
+    y = run_linear(be, dtype, w, x, 1, in_f, out_f)
+    for row0 in (0, out_f // 2 - 7, out_f - 48):
+        want = _oracle_rows(dtype, w, x, 1, in_f, out_f, row0, 48)
+        got = y[:, row0:row0 + 48]
+        gate(got, want)
+        if dtype in (DType.Q4K, DType.Q6K):
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), "not bit-identical"
+
+
+@pytest.mark.parametrize("m", [8, 64, 512, 1100])
+def test_full_size_prefill_q4k(be, m):
+    """K = 4096 -> N = 12288 at the benchmark's token counts (every Q4_K kernel route): sampled
+    rows bit-identical to the oracle, and every token's row equal to its own m = 1 result."""
+    in_f, out_f = 4096, 12288
+    w = synth_weight(DType.Q4K, 910, out_f, in_f)
+    x = synth_normal_f32(911 + m, m * in_f)
+    wb = be.upload_new(w)
+    yb = be.alloc(m * out_f * 4)
+    be.linear(DType.Q4K, wb, be.upload_new(x), yb, m, in_f, out_f)
+    y = be.download(yb, np.empty((m, out_f), np.float32))
+    toks = sorted({0, 1, m // 2, m - 1})
+    for row0 in (0, 6000, out_f - 32):
+        want = _oracle_rows(DType.Q4K, w, x[np.concatenate([np.arange(t * in_f, (t + 1) * in_f) for t in toks])],
+                            len(toks), in_f, out_f, row0, 32)
+        got = y[toks, row0:row0 + 32]
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), "not bit-identical"
+    y1 = be.alloc(out_f * 4)
+    for t in toks:
+        be.linear(DType.Q4K, wb, be.upload_new(x[t * in_f:(t + 1) * in_f]), y1, 1, in_f, out_f)
+        single = be.download(y1, np.empty((1, out_f), np.float32))
+        assert np.array_equal(single[0].view(np.uint32), y[t].view(np.uint32)), "batch != single"
+
+
+def test_ternary_output_head_rows_vs_oracle(be):
+    in_f, out_f = 4096, 151936
+    w = synth_weight(DType.Q2_0, 920, out_f, in_f)
+    x = synth_normal_f32(921, in_f)
+    y = run_linear(be, DType.Q2_0, w, x, 1, in_f, out_f)
+    for row0 in (0, 77777, out_f - 64):
+        gate(y[:, row0:row0 + 64], _oracle_rows(DType.Q2_0, w, x, 1, in_f, out_f, row0, 64))
