@@ -86,3 +86,58 @@ def test_moe_int8_path_other_bank_formats(be, dtype):
     want = orc.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
                        gate_dtype=int(dtype), up_dtype=int(dtype), down_dtype=int(dtype))
     check(*got, *want)
+
+
+@pytest.mark.parametrize("rows", [1, 6])
+def test_moe_in_a_plan_replays(be, rows):
+    """Two Op::MoeFfn separated by a Linear in one compiled plan (the second routes the first's
+    output), executed three times with fresh inputs: every replay must match the oracle chain."""
+    from infr_amd import Bindings, Graph, Linear, MoeFfn, TensorDesc
+    ne, n_expert, n_used, nff = 512, 16, 4, 256
+    router = synth_normal_f32(31, n_expert * ne, sigma=0.05)
+    b1, b2 = banks(32, ne, n_expert, nff, sigma=0.05), banks(36, ne, n_expert, nff, sigma=0.05)
+    wmid = synth_weight(DType.Q4K, 40, ne, ne, 0.05)
+    g, binds = Graph(), Bindings()
+    xid = g.input(TensorDesc((rows, ne), DType.F32))
+    xb = be.alloc(rows * ne * 4)
+    rid = g.weight(TensorDesc((n_expert, ne), DType.F32))
+    binds.bind(xid, xb).bind(rid, be.upload_new(router))
+
+    def bank_ids(bk):
+        ids = []
+        for i, w in enumerate(bk):
+            shape = (n_expert, nff, ne) if i < 2 else (n_expert, ne, nff)
+            wid = g.weight(TensorDesc(shape, DType.Q4K))
+            binds.bind(wid, be.upload_new(w))
+            ids.append(wid)
+        return ids
+
+    outs = []
+    for _ in range(3):
+        t = g.output(TensorDesc((rows, ne), DType.F32))
+        outs.append((t, be.alloc(rows * ne * 4)))
+        binds.bind(t, outs[-1][1])
+    i1, i2 = bank_ids(b1), bank_ids(b2)
+    mid = g.weight(TensorDesc((ne, ne), DType.Q4K))
+    binds.bind(mid, be.upload_new(wmid))
+    g.push(MoeFfn(xid, xid, rid, i1[0], i1[1], i1[2], outs[0][0], ne, n_expert, n_used, nff, 1.5))
+    g.push(Linear(outs[0][0], mid, outs[1][0], rows, ne, ne))
+    g.push(MoeFfn(outs[1][0], outs[1][0], rid, i2[0], i2[1], i2[2], outs[2][0], ne, n_expert, n_used, nff, 1.0))
+    plan = be.compile(g)
+    def gate_out(got, want):
+        a, b = got.astype(np.float64).ravel(), np.asarray(want, np.float64).ravel()
+        assert np.abs(b).max() > 1e-4
+        rel = np.linalg.norm(a - b) / np.linalg.norm(b)
+        mx = np.abs(a - b).max() / np.abs(b).max()
+        assert rel <= 1e-4 and mx <= 1e-3, f"rel-L2 {rel:.3e} max-abs {mx:.3e}"
+
+    kw = dict(ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff)
+    for rep in range(3):
+        x = synth_normal_f32(500 + rep, rows * ne)
+        be.upload(xb, x)
+        be.execute(plan, binds)
+        got = [be.download(b, np.empty((rows, ne), np.float32)) for _, b in outs]
+        # each stage is gated on its own: downstream oracles are fed the device's upstream output
+        gate_out(got[0], orc.moe_ffn(x, router, *b1, scale=1.5, **kw)[0])
+        gate_out(got[1], orc.linear(DType.Q4K, wmid, got[0].ravel(), rows, ne, ne))
+        gate_out(got[2], orc.moe_ffn(got[1].ravel(), router, *b2, scale=1.0, **kw)[0])
