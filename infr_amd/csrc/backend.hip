@@ -32,12 +32,15 @@ struct infr_hip_plan {
     // of a level that share (dtype, in_f) form one grouped decode launch.
     struct Step {
         int level = 0;
-        int op = -1;              // m >= 2: index into ops
-        int dtype = 0;            // decode group
+        int op = -1;              // ungrouped op (MoeFfn, larger m): index into ops
+        int dtype = 0;            // group
         size_t in_f = 0;
+        size_t m = 1;             // 1: decode group; 2..32: small-batch group
         int first = 0, n = 0;     // slice of descs
-        size_t tile_first = 0;    // slice of tiles
+        size_t tile_first = 0;    // slice of tiles (decode) / btiles (small batch)
         infr::GemvGroupPlan gp;
+        infr::BatchGroupPlan bp;
+        size_t qtile_first = 0, qtile_n = 0;  // small batch: slice of qtiles
     };
     std::vector<Step> steps;
     std::vector<infr::GemvOpDesc> descs;
@@ -45,6 +48,12 @@ struct infr_hip_plan {
     std::vector<infr::GemvTile> tiles;
     infr::GemvTile* tiles_dev = nullptr;
     size_t tiles_cap = 0;
+    // small-batch groups: quantizer and GEMM tile tables
+    std::vector<infr::QuantTile> qtiles;
+    std::vector<infr::BatchTile> btiles;
+    infr::QuantTile* qtiles_dev = nullptr;
+    infr::BatchTile* btiles_dev = nullptr;
+    size_t qtiles_cap = 0, btiles_cap = 0;
 };
 
 struct infr_hip {
@@ -92,6 +101,27 @@ bool act_per32(int dt) { return dt == INFR_DTYPE_Q2_0; }
 
 // Activation scratch for m rows: the prefill kernels read tokens in groups of 32.
 static size_t act_scratch_elems(size_t m, size_t in_f) { return (m == 1 ? 1 : (m + 31) / 32 * 32) * in_f; }
+
+// Ops that run in small-batch groups inside plans: the K-split MFMA kernel takes Q4_K up to 32
+// rows, the dot4 batch kernel the other formats up to 8.
+static bool small_batch(const infr_hip_op_t& op) {
+    return op.m >= 2 && op.m <= (op.w_dtype == INFR_DTYPE_Q4_K ? 32u : 8u);
+}
+
+// (Re)allocates a device table when it grew and enqueues the copy on the backend stream.
+template <typename T>
+static int upload_table(infr_hip_t* be, const std::vector<T>& host, T** dev, size_t* cap) {
+    if (host.empty()) return INFR_HIP_OK;
+    if (host.size() > *cap) {
+        if (*dev) (void)hipFree(*dev);
+        *dev = nullptr;
+        *cap = 0;
+        HIP_TRY(be, hipMalloc((void**)dev, sizeof(T) * host.size()));
+        *cap = host.size();
+    }
+    HIP_TRY(be, hipMemcpyAsync(*dev, host.data(), sizeof(T) * host.size(), hipMemcpyHostToDevice, be->stream));
+    return INFR_HIP_OK;
+}
 
 int ensure_act(infr_hip_t* be, size_t elems) {
     if (elems <= be->act_cap_elems) return INFR_HIP_OK;
@@ -555,7 +585,7 @@ int infr_hip_compile(infr_hip_t* be, const infr_hip_op_t* ops, size_t n_ops, inf
     infr_hip_plan_t* p = new (std::nothrow) infr_hip_plan();
     if (!p) return fail(be, INFR_HIP_ERR_OTHER, "compile: out of host memory");
     p->ops.assign(ops, ops + n_ops);
-    size_t act_need = 0, moe_need = 0;
+    size_t act_need = 0, moe_need = 0, batch_need = 0;  // batch_need: every small-batch op in one level
     for (const auto& op : p->ops) {
         if (op.kind == INFR_OP_LINEAR) {
             if (!is_quant(op.w_dtype) || op.m == 0 || op.in_f == 0 || op.out_f == 0 ||
@@ -566,6 +596,7 @@ int infr_hip_compile(infr_hip_t* be, const infr_hip_op_t* ops, size_t n_ops, inf
             }
             p->max_tensor = std::max({p->max_tensor, op.x, op.weight, op.dst});
             act_need = std::max(act_need, act_scratch_elems(op.m, op.in_f));
+            if (small_batch(op)) batch_need += ((size_t)op.m * op.in_f + 255) / 256 * 256;
         } else if (op.kind == INFR_OP_MOE_FFN) {
             const auto& mp = op.moe;
             if (!mp.ne || !mp.n_expert || !mp.n_used || !mp.n_ff_exp || !mp.rows) {
@@ -584,7 +615,7 @@ int infr_hip_compile(infr_hip_t* be, const infr_hip_op_t* ops, size_t n_ops, inf
         }
     }
     // Scratch is sized here so that execute never allocates (it records launches for replay).
-    if (int rc = ensure_act(be, act_need)) {
+    if (int rc = ensure_act(be, std::max(act_need, batch_need))) {
         delete p;
         return rc;
     }
@@ -600,7 +631,7 @@ size_t infr_hip_plan_launches(const infr_hip_plan_t* plan) {
     if (!plan) return 0;
     size_t n = 0;
     for (const auto& st : plan->steps) {
-        if (st.op < 0) n += 1;                                             // grouped decode launch
+        if (st.op < 0) n += st.m > 1 ? 2 : 1;                              // grouped launch (+ grouped quantize)
         else if (plan->ops[st.op].kind == INFR_OP_MOE_FFN) n += plan->ops[st.op].moe.rows == 1 ? 4 : 8;
         else n += 2;                                                       // quantize + GEMM
     }
@@ -612,6 +643,8 @@ void infr_hip_plan_free(infr_hip_t* be, infr_hip_plan_t* plan) {
     if (be && be->stream) (void)hipStreamSynchronize(be->stream);
     if (plan->exec) (void)hipGraphExecDestroy(plan->exec);
     if (plan->tiles_dev) (void)hipFree(plan->tiles_dev);
+    if (plan->qtiles_dev) (void)hipFree(plan->qtiles_dev);
+    if (plan->btiles_dev) (void)hipFree(plan->btiles_dev);
     delete plan;
 }
 
@@ -667,6 +700,8 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
     plan->steps.clear();
     plan->descs.clear();
     plan->tiles.clear();
+    plan->qtiles.clear();
+    plan->btiles.clear();
     for (int lv = 0; lv <= max_level; ++lv) {
         std::vector<char> taken(n, 0);
         for (size_t i = 0; i < n; ++i) {
@@ -674,6 +709,50 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
             const auto& op = plan->ops[i];
             infr_hip_plan::Step st;
             st.level = lv;
+            if (op.kind == INFR_OP_LINEAR && small_batch(op)) {
+                // small-batch group: same (dtype, in_f, m) in this level -> one quantize launch over
+                // the distinct activation tensors + one GEMM launch over a tile table
+                st.dtype = op.w_dtype;
+                st.in_f = op.in_f;
+                st.m = op.m;
+                st.first = (int)plan->descs.size();
+                std::vector<const float*> xs;
+                std::vector<uint32_t> elem0;
+                const size_t x_elems = ((size_t)op.m * op.in_f + 255) / 256 * 256;
+                for (size_t k = i; k < n; ++k) {
+                    const auto& o2 = plan->ops[k];
+                    if (level[k] != lv || taken[k] || o2.kind != INFR_OP_LINEAR || o2.m != op.m ||
+                        o2.w_dtype != op.w_dtype || o2.in_f != op.in_f)
+                        continue;
+                    taken[k] = 1;
+                    const float* x = static_cast<const float*>(bindings[o2.x]->ptr);
+                    size_t xi = 0;
+                    while (xi < xs.size() && xs[xi] != x) ++xi;
+                    if (xi == xs.size()) xs.push_back(x);
+                    elem0.push_back((uint32_t)(xi * x_elems));
+                    plan->descs.push_back(infr::GemvOpDesc{la[k].wrows, x, static_cast<float*>(bindings[o2.dst]->ptr),
+                                                           la[k].bpr, (int32_t)o2.out_f});
+                }
+                st.n = (int)plan->descs.size() - st.first;
+                if (xs.size() * x_elems > be->act_cap_elems)
+                    return fail(be, INFR_HIP_ERR_OTHER, "execute: activation scratch smaller than the plan needs");
+                if (!infr::plan_batch_group(st.dtype, st.m, st.in_f, &plan->descs[st.first], st.n, &st.bp))
+                    return fail(be, INFR_HIP_ERR_UNSUPPORTED,
+                                "execute: no small-batch kernel for dtype " + std::to_string(st.dtype) +
+                                    " at in_f " + std::to_string(st.in_f));
+                st.tile_first = plan->btiles.size();
+                plan->btiles.resize(st.tile_first + st.bp.total_wgs);
+                infr::fill_batch_tiles(&plan->descs[st.first], elem0.data(), st.n, st.bp, &plan->btiles[st.tile_first]);
+                st.qtile_first = plan->qtiles.size();
+                const size_t n_elems = (size_t)op.m * op.in_f;
+                for (size_t xi = 0; xi < xs.size(); ++xi)
+                    for (size_t e = 0; e < n_elems; e += 1024)
+                        plan->qtiles.push_back(infr::QuantTile{xs[xi] + e, (uint32_t)((xi * x_elems + e) / 256),
+                                                               (uint32_t)std::min<size_t>(1024, n_elems - e)});
+                st.qtile_n = plan->qtiles.size() - st.qtile_first;
+                plan->steps.push_back(st);
+                continue;
+            }
             if (op.kind == INFR_OP_MOE_FFN || op.m != 1) {
                 st.op = (int)i;
                 taken[i] = 1;
@@ -704,19 +783,10 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
             plan->steps.push_back(st);
         }
     }
-    if (!plan->tiles.empty()) {
-        if (plan->tiles.size() > plan->tiles_cap) {
-            if (plan->tiles_dev) (void)hipFree(plan->tiles_dev);
-            plan->tiles_dev = nullptr;
-            plan->tiles_cap = 0;
-            HIP_TRY(be, hipMalloc((void**)&plan->tiles_dev, sizeof(infr::GemvTile) * plan->tiles.size()));
-            plan->tiles_cap = plan->tiles.size();
-        }
-        HIP_TRY(be, hipMemcpyAsync(plan->tiles_dev, plan->tiles.data(),
-                                   sizeof(infr::GemvTile) * plan->tiles.size(),
-                                   hipMemcpyHostToDevice, be->stream));
-        HIP_TRY(be, hipStreamSynchronize(be->stream));
-    }
+    if (int rc = upload_table(be, plan->tiles, &plan->tiles_dev, &plan->tiles_cap)) return rc;
+    if (int rc = upload_table(be, plan->qtiles, &plan->qtiles_dev, &plan->qtiles_cap)) return rc;
+    if (int rc = upload_table(be, plan->btiles, &plan->btiles_dev, &plan->btiles_cap)) return rc;
+    HIP_TRY(be, hipStreamSynchronize(be->stream));
     return INFR_HIP_OK;
 }
 
@@ -742,6 +812,16 @@ static int enqueue_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t
                                         static_cast<float*>(bindings[op.dst]->ptr), op.m, op.in_f,
                                         op.out_f, infr::IntStages{}))
                 return rc;
+        } else if (st.m > 1) {
+            infr::launch_quantize_q8_group(plan->qtiles_dev + st.qtile_first, st.qtile_n, act_per32(st.dtype),
+                                           be->act, be->stream);
+            if (st.bp.kind == 1)
+                infr::launch_mmq_skinny_group(st.m, st.in_f, plan->btiles_dev + st.tile_first, st.bp, be->act,
+                                              be->stream);
+            else if (!infr::launch_gemv_batch_group(st.dtype, st.m, st.in_f, plan->btiles_dev + st.tile_first,
+                                                    st.bp, be->act, be->stream))
+                return fail(be, INFR_HIP_ERR_UNSUPPORTED, "execute: small-batch launch rejected");
+            HIP_TRY(be, hipGetLastError());
         } else {
             if (!infr::launch_gemv_fused(st.dtype, st.in_f, &plan->descs[st.first], st.n,
                                          plan->tiles_dev + st.tile_first, st.gp, be->stream))

@@ -55,16 +55,33 @@ __global__ __launch_bounds__(256) void gemv_kernel(const uint8_t* __restrict__ w
 }
 
 // Small batch (2..8 activation rows already quantized in device memory): weights stream once.
+// With `tiles` (plans) a workgroup takes one table entry - some rows of one of several ops - and
+// blockIdx.y selects the pass of MB activation rows; `m_valid` is then the op's total row count.
 template <typename F, int STEPS, int MB, bool STAGES>
 __global__ __launch_bounds__(256) void gemv_batch_kernel(const uint8_t* __restrict__ w, size_t bpr,
                                                          ActPtrs act, int m_valid, int in_f,
                                                          float* __restrict__ y, int out_f,
-                                                         int rows_per_wave, StagePtrs st) {
+                                                         int rows_per_wave, StagePtrs st,
+                                                         const BatchTile* __restrict__ tiles) {
     const int lane = threadIdx.x & 63;
-    const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    int n_rows = out_f;
+    size_t act_elem0 = 0;
+    if (tiles) {
+        const BatchTile t = tiles[blockIdx.x];
+        const int pass = blockIdx.y;
+        w = t.w;
+        bpr = t.bpr;
+        out_f = (int)t.out_f;
+        n_rows = (int)t.rows;
+        y = t.y + (size_t)pass * MB * out_f;
+        act_elem0 = (size_t)t.act_elem0 + (size_t)pass * MB * in_f;
+        m_valid = min(MB, m_valid - pass * MB);
+        wave = threadIdx.x >> 6;
+    }
     const int row0 = wave * rows_per_wave;
-    if (row0 >= out_f) return;
-    const int row_end = min(row0 + rows_per_wave, out_f);
+    if (row0 >= n_rows) return;
+    const int row_end = min(row0 + rows_per_wave, n_rows);
     const int n_units = F::units(in_f);
     typename F::Acts acts[MB][STEPS];
     typename F::Row first;
@@ -72,12 +89,12 @@ __global__ __launch_bounds__(256) void gemv_batch_kernel(const uint8_t* __restri
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) ok[t] = F::valid(t, lane, n_units);
     F::load_row(first, w + (size_t)row0 * bpr, 0, lane, ok[0]);
-    const int dper = F::kPer32 ? in_f / 32 : in_f / 256;
 #pragma unroll
     for (int mi = 0; mi < MB; ++mi) {
         const int r = mi < m_valid ? mi : 0;  // padding rows reuse row 0; their outputs are dropped
-        const ActPtrs a{act.qs + (size_t)r * in_f, act.d + (size_t)r * dper,
-                        act.bsums + (size_t)r * (in_f / 32), act.bsums16 + (size_t)r * (in_f / 16)};
+        const size_t e = act_elem0 + (size_t)r * in_f;
+        const ActPtrs a{act.qs + e, act.d + e / (F::kPer32 ? 32 : 256), act.bsums + e / 32,
+                        act.bsums16 + e / 16};
 #pragma unroll
         for (int t = 0; t < STEPS; ++t) F::load_acts(acts[mi][t], a, t, lane, ok[t]);
     }
@@ -217,10 +234,92 @@ static void launch_batch_one(const uint8_t* w, size_t bpr, const ActPtrs& act, i
     const dim3 grid((unsigned)((waves + 3) / 4)), block(256);
     if (st.a)
         hipLaunchKernelGGL((gemv_batch_kernel<F, STEPS, MB, true>), grid, block, 0, stream, w, bpr, act,
-                           m_valid, (int)in_f, y, (int)out_f, (int)rpw, st);
+                           m_valid, (int)in_f, y, (int)out_f, (int)rpw, st, (const BatchTile*)nullptr);
     else
         hipLaunchKernelGGL((gemv_batch_kernel<F, STEPS, MB, false>), grid, block, 0, stream, w, bpr, act,
-                           m_valid, (int)in_f, y, (int)out_f, (int)rpw, st);
+                           m_valid, (int)in_f, y, (int)out_f, (int)rpw, st, (const BatchTile*)nullptr);
+}
+
+// Activation rows per pass of the batch kernel (they live in registers).
+static int batch_rows_per_pass(int steps) { return steps == 1 ? 8 : (steps == 2 ? 4 : (steps <= 4 ? 2 : 1)); }
+
+template <typename F, int STEPS, int MB>
+static void launch_batch_group_one(const BatchTile* tiles, const BatchGroupPlan& gp, const ActPtrs& act,
+                                   int m, size_t in_f, hipStream_t stream) {
+    const dim3 grid((unsigned)gp.total_wgs, (unsigned)((m + MB - 1) / MB)), block(256);
+    hipLaunchKernelGGL((gemv_batch_kernel<F, STEPS, MB, false>), grid, block, 0, stream,
+                       (const uint8_t*)nullptr, (size_t)0, act, m, (int)in_f, (float*)nullptr, 0,
+                       gp.rows_per_wave, StagePtrs{nullptr, nullptr}, tiles);
+}
+
+template <typename F>
+static bool launch_batch_group_fmt(const BatchTile* tiles, const BatchGroupPlan& gp, const ActQ8& a,
+                                   size_t m, size_t in_f, hipStream_t stream) {
+    const int steps = (int)((in_f + F::kElemsPerStep - 1) / F::kElemsPerStep);
+    const ActPtrs act{a.qs, a.d, a.bsums, a.bsums16};
+    const int mb = std::min((int)m, batch_rows_per_pass(steps));
+#define INFR_G(S, MB) launch_batch_group_one<F, S, MB>(tiles, gp, act, (int)m, in_f, stream)
+    switch (steps) {
+    case 1: if (mb > 4) INFR_G(1, 8); else if (mb > 2) INFR_G(1, 4); else INFR_G(1, 2); break;
+    case 2: if (mb > 2) INFR_G(2, 4); else INFR_G(2, 2); break;
+    case 3: INFR_G(3, 2); break;
+    case 4: INFR_G(4, 2); break;
+    case 5: INFR_G(5, 1); break;
+    case 6: INFR_G(6, 1); break;
+    case 7: INFR_G(7, 1); break;
+    case 8: INFR_G(8, 1); break;
+    default: return false;
+    }
+#undef INFR_G
+    return true;
+}
+
+bool launch_gemv_batch_group(int dtype, size_t m, size_t in_f, const BatchTile* tiles_dev,
+                             const BatchGroupPlan& plan, const ActQ8& act, hipStream_t stream) {
+    switch (dtype) {
+    case 12: return launch_batch_group_fmt<FmtQ4K>(tiles_dev, plan, act, m, in_f, stream);
+    case 14: return launch_batch_group_fmt<FmtQ6K>(tiles_dev, plan, act, m, in_f, stream);
+    case 8: return launch_batch_group_fmt<FmtQ8_0>(tiles_dev, plan, act, m, in_f, stream);
+    case 42: return launch_batch_group_fmt<FmtQ2_0>(tiles_dev, plan, act, m, in_f, stream);
+    default: return false;
+    }
+}
+
+bool plan_batch_group(int dtype, size_t m, size_t in_f, const GemvOpDesc* ops, int n, BatchGroupPlan* plan) {
+    size_t total_rows = 0;
+    for (int i = 0; i < n; ++i) total_rows += (size_t)ops[i].out_f;
+    BatchGroupPlan gp;
+    if (dtype == 12) {  // Q4_K: the K-split MFMA kernel, 32 rows per workgroup
+        if (in_f % 256 != 0 || m > 32) return false;
+        gp.kind = 1;
+        gp.rows_per_wg = 32;
+        const size_t wgs = (total_rows + 31) / 32;
+        gp.waves = (in_f >= 8192 || (wgs * 4 < 1024 && in_f >= 2048)) ? 8 : 4;
+    } else {
+        if (dtype != 14 && dtype != 8 && dtype != 42) return false;
+        const size_t per_step = dtype == 8 ? 2048 : 4096;
+        const size_t steps = (in_f + per_step - 1) / per_step;
+        if (steps < 1 || steps > 8 || m > 8) return false;
+        size_t rpw = (total_rows + 4095) / 4096;
+        rpw = rpw < 2 ? 2 : (rpw > 16 ? 16 : rpw);
+        gp.kind = 0;
+        gp.rows_per_wave = (int)rpw;
+        gp.rows_per_wg = (int)rpw * 4;
+    }
+    gp.total_wgs = 0;
+    for (int i = 0; i < n; ++i) gp.total_wgs += ((size_t)ops[i].out_f + gp.rows_per_wg - 1) / gp.rows_per_wg;
+    *plan = gp;
+    return true;
+}
+
+void fill_batch_tiles(const GemvOpDesc* ops, const uint32_t* act_elem0, int n, const BatchGroupPlan& plan,
+                      BatchTile* out) {
+    size_t k = 0;
+    for (int i = 0; i < n; ++i)
+        for (int r0 = 0; r0 < ops[i].out_f; r0 += plan.rows_per_wg)
+            out[k++] = BatchTile{ops[i].w + (size_t)r0 * ops[i].bpr, ops[i].y + r0, act_elem0[i],
+                                 (uint32_t)ops[i].out_f, (uint32_t)std::min(plan.rows_per_wg, ops[i].out_f - r0),
+                                 (uint32_t)ops[i].bpr};
 }
 
 // m activation rows in chunks of MB <= 8 / STEPS (the activations live in registers).
@@ -231,7 +330,7 @@ static bool launch_batch_fmt(const uint8_t* w, size_t bpr, const ActQ8& a, float
     if (steps < 1 || steps > 8) return false;
     const size_t dper = F::kPer32 ? in_f / 32 : in_f / 256;
     const size_t blocks = (F::kBlockElems == 64 ? 2 : 1) * (in_f / F::kBlockElems);
-    const size_t mb_max = steps == 1 ? 8 : (steps == 2 ? 4 : (steps <= 4 ? 2 : 1));
+    const size_t mb_max = (size_t)batch_rows_per_pass(steps);
     for (size_t r0 = 0; r0 < m; r0 += mb_max) {
         const int mv = (int)std::min(mb_max, m - r0);
         const ActPtrs act{a.qs + r0 * in_f, a.d + r0 * dper, a.bsums + r0 * (in_f / 32),

@@ -21,6 +21,15 @@ struct ActQ8 {
 // quantize_q8 / quantize_q8_32 over m*k contiguous floats.
 void launch_quantize_q8(const float* x, size_t m, size_t k, bool per32, const ActQ8& out,
                         hipStream_t stream);
+// Several activation tensors in one launch (plans): workgroup i quantizes `n_chunks` <= 4
+// consecutive 256-float chunks of `x` into chunk slots chunk0.. of the shared scratch.
+struct QuantTile {
+    const float* x;      // first float of the workgroup's chunks
+    uint32_t chunk0;     // destination chunk index
+    uint32_t n_elems;    // floats to quantize (<= 1024; a per-32 input may end inside a chunk)
+};
+void launch_quantize_q8_group(const QuantTile* tiles_dev, size_t n_tiles, bool per32, const ActQ8& out,
+                              hipStream_t stream);
 // Per-256 quantizer writing MFMA A-operand order (token groups of 32) into the same buffers.
 void launch_quantize_q8_tiled(const float* x, size_t m, size_t k, const ActQ8& out, hipStream_t stream);
 
@@ -83,6 +92,32 @@ bool launch_gemv_fused(int dtype, size_t in_f, const GemvOpDesc* ops, int n, con
 // chosen kernel reads, then multiplies.
 bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const ActQ8& act, float* y,
                 size_t m, size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream);
+
+// Small-batch ops of one dependency level that share (dtype, in_f, m), as ONE launch: the
+// workgroups index a tile table. `act_elem0` is where the op's quantized activation rows start
+// in the scratch (elements; a multiple of 256).
+struct BatchTile {
+    const uint8_t* w;    // first weight row of the tile
+    float* y;            // y + first row
+    uint32_t act_elem0;
+    uint32_t out_f;      // row stride of y
+    uint32_t rows;       // weight rows in this tile
+    uint32_t bpr;
+};
+struct BatchGroupPlan {
+    int kind = 0;          // 0: dot4 batch GEMV, 1: K-split MFMA kernel (Q4_K)
+    int rows_per_wg = 0;
+    int rows_per_wave = 0; // kind 0
+    int waves = 4;         // kind 1: waves per workgroup (4 or 8)
+    size_t total_wgs = 0;
+};
+bool plan_batch_group(int dtype, size_t m, size_t in_f, const GemvOpDesc* ops, int n, BatchGroupPlan* plan);
+void fill_batch_tiles(const GemvOpDesc* ops, const uint32_t* act_elem0, int n, const BatchGroupPlan& plan,
+                      BatchTile* out);
+bool launch_gemv_batch_group(int dtype, size_t m, size_t in_f, const BatchTile* tiles_dev,
+                             const BatchGroupPlan& plan, const ActQ8& act, hipStream_t stream);
+void launch_mmq_skinny_group(size_t m, size_t in_f, const BatchTile* tiles_dev, const BatchGroupPlan& plan,
+                             const ActQ8& act, hipStream_t stream);
 
 // Op::MoeFfn (qwen3moe form). Expert e of a bank starts at bank + e * stride.
 struct MoeShape {

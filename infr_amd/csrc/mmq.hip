@@ -477,7 +477,8 @@ template <int NW, bool STAGES>
 __global__ __launch_bounds__(NW * 64) void mmq_skinny_q4k_kernel(
     const uint8_t* __restrict__ w, size_t bpr, const int8_t* __restrict__ qs,
     const float* __restrict__ d8, const int32_t* __restrict__ bsums, float* __restrict__ y, int m,
-    int out_f, int nb, int32_t* __restrict__ st_sd, int32_t* __restrict__ st_sm) {
+    int out_f, int nb, int32_t* __restrict__ st_sd, int32_t* __restrict__ st_sm,
+    const BatchTile* __restrict__ tiles) {
     constexpr int RG = 16 / NW;  // accumulators per epilogue thread
     typedef int vrgi __attribute__((ext_vector_type(RG)));
     typedef float vrgf __attribute__((ext_vector_type(RG)));
@@ -487,10 +488,24 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny_q4k_kernel(
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, h = lane >> 5;
     const int tok0 = blockIdx.y * 32;
-    const int wrow = blockIdx.x * 32 + col;
-    const bool row_ok = wrow < out_f;
-    const uint8_t* wrowp = w + (size_t)(row_ok ? wrow : 0) * bpr;
     const size_t in_f = (size_t)nb * 256;
+    // This workgroup's 32 weight rows: a table entry (plans: rows of one of several ops, whose
+    // activation rows start at act_elem0 of the scratch) or computed from the single op.
+    int wrow = blockIdx.x * 32 + col;  // output column relative to y
+    bool row_ok = wrow < out_f;
+    if (tiles) {
+        const BatchTile t = tiles[blockIdx.x];
+        w = t.w;
+        bpr = t.bpr;
+        y = t.y;
+        out_f = (int)t.out_f;
+        wrow = col;
+        row_ok = col < (int)t.rows;
+        qs += t.act_elem0;
+        d8 += t.act_elem0 / 256;
+        bsums += t.act_elem0 / 32;
+    }
+    const uint8_t* wrowp = w + (size_t)(row_ok ? wrow : 0) * bpr;
     const int atok = min(tok0 + col, m - 1);  // this lane's activation row as MFMA A operand
     // tokens of this thread's epilogue outputs: accumulator r = RG*wave + i of lane position `lane`
     int etok[RG];
@@ -634,10 +649,25 @@ static void launch_mmq_skinny_q4k(const uint8_t* w, size_t bpr, const ActQ8& act
     const int nb = (int)(in_f / 256);
     if (st.a)
         hipLaunchKernelGGL((mmq_skinny_q4k_kernel<NW, true>), grid, block, 0, stream, w, bpr, act.qs, act.d,
-                           act.bsums, y, (int)m, (int)out_f, nb, st.a, st.b);
+                           act.bsums, y, (int)m, (int)out_f, nb, st.a, st.b, (const BatchTile*)nullptr);
     else
         hipLaunchKernelGGL((mmq_skinny_q4k_kernel<NW, false>), grid, block, 0, stream, w, bpr, act.qs, act.d,
-                           act.bsums, y, (int)m, (int)out_f, nb, (int32_t*)nullptr, (int32_t*)nullptr);
+                           act.bsums, y, (int)m, (int)out_f, nb, (int32_t*)nullptr, (int32_t*)nullptr,
+                           (const BatchTile*)nullptr);
+}
+
+void launch_mmq_skinny_group(size_t m, size_t in_f, const BatchTile* tiles_dev, const BatchGroupPlan& plan,
+                             const ActQ8& act, hipStream_t stream) {
+    const dim3 grid((unsigned)plan.total_wgs, (unsigned)((m + 31) / 32));
+    const int nb = (int)(in_f / 256);
+    if (plan.waves == 8)
+        hipLaunchKernelGGL((mmq_skinny_q4k_kernel<8, false>), grid, dim3(512), 0, stream, (const uint8_t*)nullptr,
+                           (size_t)0, act.qs, act.d, act.bsums, (float*)nullptr, (int)m, 0, nb,
+                           (int32_t*)nullptr, (int32_t*)nullptr, tiles_dev);
+    else
+        hipLaunchKernelGGL((mmq_skinny_q4k_kernel<4, false>), grid, dim3(256), 0, stream, (const uint8_t*)nullptr,
+                           (size_t)0, act.qs, act.d, act.bsums, (float*)nullptr, (int)m, 0, nb,
+                           (int32_t*)nullptr, (int32_t*)nullptr, tiles_dev);
 }
 
 template <int BM>

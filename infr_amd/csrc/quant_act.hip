@@ -68,6 +68,32 @@ void launch_quantize_q8_tiled(const float* x, size_t m, size_t k, const ActQ8& o
                        out.qs, out.d, reinterpret_cast<_Float16*>(out.bsums), n_chunks, (int)(k / 256));
 }
 
+template <bool PER32>
+__global__ __launch_bounds__(256) void quantize_q8_group_kernel(const QuantTile* __restrict__ tiles,
+                                                                int8_t* __restrict__ qs,
+                                                                float* __restrict__ d,
+                                                                int32_t* __restrict__ bsums,
+                                                                int32_t* __restrict__ bsums16) {
+    const QuantTile t = tiles[blockIdx.x];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if ((uint32_t)wave * 256 >= t.n_elems) return;  // wave-uniform
+    const bool live = (uint32_t)wave * 256 + (uint32_t)lane * 4 < t.n_elems;
+    v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (live) v = *reinterpret_cast<const v4f*>(t.x + wave * 256 + lane * 4);
+    quantize_chunk<PER32>(v, live, lane, (size_t)t.chunk0 + wave, qs, d, bsums, bsums16);
+}
+
+void launch_quantize_q8_group(const QuantTile* tiles_dev, size_t n_tiles, bool per32, const ActQ8& out,
+                              hipStream_t stream) {
+    if (n_tiles == 0) return;
+    if (per32)
+        hipLaunchKernelGGL(quantize_q8_group_kernel<true>, dim3((unsigned)n_tiles), dim3(256), 0, stream,
+                           tiles_dev, out.qs, out.d, out.bsums, (int32_t*)nullptr);
+    else
+        hipLaunchKernelGGL(quantize_q8_group_kernel<false>, dim3((unsigned)n_tiles), dim3(256), 0, stream,
+                           tiles_dev, out.qs, out.d, out.bsums, out.bsums16);
+}
+
 void launch_quantize_q8(const float* x, size_t m, size_t k, bool per32, const ActQ8& out,
                         hipStream_t stream) {
     const size_t n_elems = m * k;

@@ -98,3 +98,47 @@ def test_in_place_chain_is_ordered(be):
     y2 = orc.linear(DType.Q4K, wc, x, 1, in_f, in_f).ravel()
     assert np.array_equal(bits(be.download(zb, np.empty(in_f, np.float32))), bits(z))
     assert np.array_equal(bits(be.download(yb, np.empty(in_f, np.float32))), bits(y2))
+
+
+@pytest.mark.parametrize("m", [2, 5, 8, 19])
+def test_small_batch_ops_run_as_groups(be, m):
+    """m = 2..32 inside a plan: ops of a level that share (dtype, in_f, m) become one quantize
+    launch over the distinct activation tensors plus one GEMM launch over a tile table. q/k/v
+    share x, a second level consumes the first, and every replay is checked against the oracle."""
+    H, KV, FF = 512, 256, 1024
+    fmts = [DType.Q4K] if m > 8 else [DType.Q4K, DType.Q6K, DType.Q8_0, DType.Q2_0]
+    for dt in fmts:
+        spec = [("q", dt, H, H, "x"), ("k", dt, KV, H, "x"), ("v", dt, KV + 40, H, "x2"),
+                ("o", dt, H, H, "q"), ("up", dt, FF, H, "q"), ("down", dt, 200, FF, "up")]
+        g, binds = Graph(), Bindings()
+        tid, bufs = {}, {}
+        for name in ("x", "x2"):
+            tid[name] = g.input(TensorDesc((m, H), DType.F32))
+            bufs[name] = be.alloc(m * H * 4)
+            binds.bind(tid[name], bufs[name])
+        weights = {}
+        for i, (name, d, out_f, in_f, src) in enumerate(spec):
+            weights[name] = synth_weight(d, 60 + i, out_f, in_f, 0.05)
+            wid = g.weight(TensorDesc((out_f, in_f), d))
+            binds.bind(wid, be.upload_new(weights[name]))
+            tid[name] = g.output(TensorDesc((m, out_f), DType.F32))
+            bufs[name] = be.alloc(m * out_f * 4)
+            binds.bind(tid[name], bufs[name])
+            g.push(Linear(tid[src], wid, tid[name], m, in_f, out_f))
+        plan = be.compile(g)
+        for rep in range(2):
+            want = {"x": synth_normal_f32(700 + rep, m * H), "x2": synth_normal_f32(710 + rep, m * H)}
+            be.upload(bufs["x"], want["x"])
+            be.upload(bufs["x2"], want["x2"])
+            be.execute(plan, binds)
+            assert plan.launches() == 6, plan.launches()  # three levels x (quantize + GEMM)
+            for name, d, out_f, in_f, src in spec:
+                got = be.download(bufs[name], np.empty((m, out_f), np.float32))
+                # each op is checked on the device's own input, so one op's rounding does not leak
+                src_dev = want[src] if src in want else be.download(bufs[src], np.empty(m * in_f, np.float32))
+                ref = orc.linear(d, weights[name], src_dev, m, in_f, out_f)
+                if d in (DType.Q4K, DType.Q6K):
+                    assert np.array_equal(bits(got), bits(ref)), f"{name} {d} differs on execute {rep}"
+                else:
+                    a, b = got.astype(np.float64).ravel(), ref.astype(np.float64).ravel()
+                    assert np.linalg.norm(a - b) <= 1e-4 * np.linalg.norm(b), f"{name} {d}"
