@@ -59,11 +59,31 @@ __device__ __forceinline__ float readlane_f(float v, int lane) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
 }
 
-// Butterfly sum over the 64 lanes (order fixed by the lane pairing, so runs are reproducible).
+// Sum over the 64 lanes without touching LDS: DPP adds inside each row of 16 lanes (quad swaps,
+// then the two mirrors leave the row total in every lane), then the four row totals are read out
+// as scalars and added in row order. The pairing is fixed, so runs are reproducible. The total is
+// valid in every lane.
 __device__ __forceinline__ float wave_sum_f(float v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
+    auto dpp_add = [](float x, int ctrl_tag) {
+        const int xi = __builtin_bit_cast(int, x);
+        int o;
+        switch (ctrl_tag) {
+        case 0: o = __builtin_amdgcn_mov_dpp(xi, 0xB1, 0xF, 0xF, true); break;   // quad_perm [1,0,3,2]
+        case 1: o = __builtin_amdgcn_mov_dpp(xi, 0x4E, 0xF, 0xF, true); break;   // quad_perm [2,3,0,1]
+        case 2: o = __builtin_amdgcn_mov_dpp(xi, 0x141, 0xF, 0xF, true); break;  // row_half_mirror
+        default: o = __builtin_amdgcn_mov_dpp(xi, 0x140, 0xF, 0xF, true); break; // row_mirror
+        }
+        return x + __builtin_bit_cast(float, o);
+    };
+    v = dpp_add(v, 0);
+    v = dpp_add(v, 1);
+    v = dpp_add(v, 2);
+    v = dpp_add(v, 3);
+    float s = readlane_f(v, 0);
+    s += readlane_f(v, 16);
+    s += readlane_f(v, 32);
+    s += readlane_f(v, 48);
+    return s;
 }
 __device__ __forceinline__ int wave_sum_i(int v) {
 #pragma unroll
