@@ -374,6 +374,45 @@ template <> int max_waves_per_wg<FmtQ6K>(int steps) { return steps <= 1 ? 16 : 8
 template <> int max_waves_per_wg<FmtQ8_0>(int steps) { return steps <= 4 ? 16 : 8; }
 template <> int max_waves_per_wg<FmtQ2_0>(int steps) { return steps <= 3 ? 16 : 8; }
 
+// Workgroups of the fused kernel that one compute unit holds at once (registers, LDS, wave slots),
+// as the runtime computes it for the exact instantiation; 0 if the query fails.
+template <typename F, int NW>
+static int fused_wgs_per_cu_nw(int steps, size_t lds_bytes) {
+    int nblk = 0;
+#define INFR_CASE(N)                                                                                  \
+    case N:                                                                                           \
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(                                             \
+                &nblk, reinterpret_cast<const void*>(&gemv_fused_kernel<F, N, NW>), NW * 64, lds_bytes) != hipSuccess) \
+            nblk = 0;                                                                                 \
+        break;
+    switch (steps) {
+        INFR_CASE(1) INFR_CASE(2) INFR_CASE(3) INFR_CASE(4)
+        INFR_CASE(5) INFR_CASE(6) INFR_CASE(7) INFR_CASE(8)
+    default: break;
+    }
+#undef INFR_CASE
+    return nblk;
+}
+template <typename F>
+static int fused_wgs_per_cu(int steps, int nw, size_t lds_bytes) {
+    switch (nw) {
+    case 4: return fused_wgs_per_cu_nw<F, 4>(steps, lds_bytes);
+    case 8: return fused_wgs_per_cu_nw<F, 8>(steps, lds_bytes);
+    case 16: return fused_wgs_per_cu_nw<F, 16>(steps, lds_bytes);
+    default: return 0;
+    }
+}
+static int device_cu_count() {
+    static const int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+            n = 0;
+        return n;
+    }();
+    return cus;
+}
+
 template <typename F>
 static bool plan_group_fmt(size_t in_f, const GemvOpDesc* ops, int n, GemvGroupPlan* plan) {
     const int steps = (int)((in_f + F::kElemsPerStep - 1) / F::kElemsPerStep);
@@ -386,13 +425,41 @@ static bool plan_group_fmt(size_t in_f, const GemvOpDesc* ops, int n, GemvGroupP
     // quantization is spread over the most waves; waves beyond the tile's rows retire after it.
     int nw = max_waves_per_wg<F>(steps);
     if (steps >= 3 && nw > 8) nw = 8;  // long rows: 8-wave workgroups measured faster
-    size_t rows_per_wg = (total_rows + 511) / 512;
-    rows_per_wg = rows_per_wg < 4 ? 4 : (rows_per_wg > 128 ? 128 : rows_per_wg);
     // Tuning knobs (the reference exposes its kernel-shape choices the same way,
     // kernels.vulkan.* in crates/infr-core/src/config/mod.rs:210-358).
     static const int env_nw = getenv("INFR_HIP_GEMV_WAVES") ? atoi(getenv("INFR_HIP_GEMV_WAVES")) : 0;
     static const int env_rows = getenv("INFR_HIP_GEMV_ROWS") ? atoi(getenv("INFR_HIP_GEMV_ROWS")) : 0;
     if ((env_nw == 4 || env_nw == 8 || env_nw == 16) && env_nw <= nw) nw = env_nw;
+    size_t rows_per_wg = (total_rows + 511) / 512;
+    rows_per_wg = rows_per_wg < 4 ? 4 : (rows_per_wg > 128 ? 128 : rows_per_wg);
+    const size_t lds_bytes = in_f + in_f / 2 + (F::kOrdered ? (size_t)nw * (16 * (16 * steps + 4)) * sizeof(float) : 0);
+    // Wave quantisation: the chip holds `resident` workgroups at once, and a grid of only a few
+    // such rounds that needs a little more than a whole number of them idles most of the machine
+    // during the last one. For those grids take, among tile heights near the one above, the one
+    // with the least modelled time rounds x (rows + fixed cost), the fixed cost being the
+    // per-workgroup quantization of x (about eleven rows' worth). Grids of many rounds keep the
+    // 128-row tiles: their tail is small and taller tiles measured slower.
+    static const int env_model = getenv("INFR_HIP_GEMV_ROUNDS") ? atoi(getenv("INFR_HIP_GEMV_ROUNDS")) : 1;
+    const int resident = device_cu_count() * fused_wgs_per_cu<F>(steps, nw, lds_bytes);
+    auto wgs_at = [&](size_t r) {
+        size_t w = 0;
+        for (int i = 0; i < n; ++i) w += ((size_t)ops[i].out_f + r - 1) / r;
+        return w;
+    };
+    if (env_model && resident > 0 && wgs_at(rows_per_wg) < (size_t)resident * 4) {
+        const size_t lo = std::max<size_t>(4, rows_per_wg / 2), hi = std::max<size_t>(rows_per_wg * 2, 160);
+        double best = 1e300;
+        size_t best_r = rows_per_wg;
+        for (size_t r = lo; r <= hi; ++r) {
+            const size_t rounds = (wgs_at(r) + resident - 1) / resident;
+            const double cost = (double)rounds * ((double)r + 11.0);
+            if (cost < best * 0.999) {  // ties go to the smaller tile
+                best = cost;
+                best_r = r;
+            }
+        }
+        rows_per_wg = best_r;
+    }
     if (env_rows >= 1 && env_rows <= 4096) rows_per_wg = (size_t)env_rows;
     int wg = 0;
     for (int i = 0; i < n; ++i) wg += (int)(((size_t)ops[i].out_f + rows_per_wg - 1) / rows_per_wg);
@@ -400,7 +467,7 @@ static bool plan_group_fmt(size_t in_f, const GemvOpDesc* ops, int n, GemvGroupP
     plan->waves_per_wg = nw;
     plan->rows_per_wg = (int)rows_per_wg;
     // qs + d + bsums + bsums16, then the ordered-sum scratch of every wave
-    plan->lds_bytes = in_f + in_f / 2 + (F::kOrdered ? (size_t)nw * (16 * (16 * steps + 4)) * sizeof(float) : 0);
+    plan->lds_bytes = lds_bytes;
     return true;
 }
 
