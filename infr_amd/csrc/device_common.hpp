@@ -36,6 +36,25 @@ __device__ __forceinline__ uint32_t load_u16(const uint8_t* p) {
     return v;
 }
 
+// 16-byte load from a 4-byte-aligned address (a dword-aligned multi-dword load runs at full rate;
+// one at 2-byte alignment does not).
+__device__ __forceinline__ v4i load16_a4(const uint8_t* p) {
+    v4i v;
+    __builtin_memcpy(&v, __builtin_assume_aligned(p, 4), 16);
+    return v;
+}
+
+// Q8_0 blocks (34 B stride) start at a 4-byte boundary or 2 bytes past one, and a 16-byte load at
+// 2-byte alignment runs far below full rate (measured: +20 % GEMV bandwidth without them; Q6_K and
+// Q2_0, with fewer bytes per misaligned load, measured no gain and keep the plain loads). The
+// Q8_0 loader fetches dwords from the boundary at or below the block and realigns in registers:
+// realign2(lo, hi, odd) = the four bytes that follow byte 2 (block at the boundary) or byte 4
+// (block 2 past it, `odd`) of the eight bytes {lo, hi}.
+__device__ __forceinline__ int realign2(int lo, int hi, uint32_t sel) {
+    return (int)__builtin_amdgcn_perm((uint32_t)hi, (uint32_t)lo, sel);
+}
+__device__ __forceinline__ uint32_t realign2_selector(bool odd) { return odd ? 0x07060504u : 0x05040302u; }
+
 // signed int8x4 . int8x4 + acc  (v_dot4_i32_i8)
 __device__ __forceinline__ int dot4(int a, int b, int acc) {
     return __builtin_amdgcn_sdot4(a, b, acc, false);

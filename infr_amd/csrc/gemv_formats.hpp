@@ -231,12 +231,28 @@ struct FmtQ8_0 {
     };
     __device__ static int units(int in_f) { return in_f / 32; }
     __device__ static bool valid(int t, int lane, int n) { return t * 64 + lane < n; }
+    // Dword-aligned loads + register realignment (see realign2): a block 2 bytes past a 4-byte
+    // boundary reads the 2 bytes before it (the previous block of the row or buffer) and never
+    // past its own end.
     __device__ static void load_row(Row& r, const uint8_t* rowp, int t, int lane, bool ok) {
         if (ok) {
             const uint8_t* blk = rowp + (size_t)(t * 64 + lane) * 34;
-            r.d = load_u16(blk);
-            r.qa = load16_a2(blk + 2);
-            r.qb = load16_a2(blk + 18);
+            const bool odd = (reinterpret_cast<uintptr_t>(blk) & 2) != 0;
+            const uint8_t* a = blk - (odd ? 2 : 0);
+            const v4i lo = load16_a4(a), hi = load16_a4(a + 16);
+            // last dword: bytes 32..33 always belong to the block, 34..35 only to an odd one
+            uint32_t tail = load_u16(a + 32);
+            if (odd) tail |= load_u16(a + 34) << 16;
+            const uint32_t sel = realign2_selector(odd);
+            r.d = odd ? (uint32_t)lo.x >> 16 : (uint32_t)lo.x & 0xFFFFu;
+            r.qa.x = realign2(lo.x, lo.y, sel);
+            r.qa.y = realign2(lo.y, lo.z, sel);
+            r.qa.z = realign2(lo.z, lo.w, sel);
+            r.qa.w = realign2(lo.w, hi.x, sel);
+            r.qb.x = realign2(hi.x, hi.y, sel);
+            r.qb.y = realign2(hi.y, hi.z, sel);
+            r.qb.z = realign2(hi.z, hi.w, sel);
+            r.qb.w = realign2(hi.w, (int)tail, sel);
         } else {
             r.qa = r.qb = v4i{0, 0, 0, 0};
             r.d = 0;
