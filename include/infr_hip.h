@@ -169,7 +169,19 @@ int infr_hip_moe_ffn(infr_hip_t *be, const infr_hip_moe_params_t *p, const infr_
 
 /* ---- graph level: Backend::compile / execute (backend.rs:560-577) over a flat C mirror of
  * infr_core::graph::Graph restricted to the ops of this path ---- */
-typedef enum { INFR_OP_LINEAR = 1, INFR_OP_MOE_FFN = 2 } infr_hip_op_kind;
+typedef enum {
+    INFR_OP_LINEAR = 1,
+    INFR_OP_MOE_FFN = 2,
+    /* the ops either side of every Linear in a decoder layer */
+    INFR_OP_RMS_NORM = 3,        /* Op::RmsNorm, graph.rs:139-148; CPU arm lib.rs:802-825 */
+    INFR_OP_RMS_NORM_ADD = 4,    /* Op::RmsNormAdd, graph.rs:149-158; lib.rs:826-850 */
+    INFR_OP_GATED_ACT = 5,       /* Op::GatedAct, graph.rs:697-735; lib.rs:1890-1944 */
+    INFR_OP_GATED_ACT_FUSED = 6, /* Op::GatedActFused, graph.rs:736-748; lib.rs:1945-1971 */
+    INFR_OP_ADD = 7              /* Op::Add, graph.rs:749-755; lib.rs:1972-1988 */
+} infr_hip_op_kind;
+
+/* Activation (crates/infr-core/src/graph.rs, act_fn in crates/infr-cpu/src/kernels.rs:6578-6585) */
+typedef enum { INFR_ACT_SILU = 0, INFR_ACT_GELU = 1, INFR_ACT_SIGMOID = 2 } infr_activation;
 
 typedef struct {
     int kind;      /* infr_hip_op_kind */
@@ -182,6 +194,18 @@ typedef struct {
     /* Op::MoeFfn */
     uint32_t router_x, router, gate_exps, up_exps, down_exps;
     infr_hip_moe_params_t moe;
+    /* Elementwise ops, all f32. They reuse the fields above:
+     *   RmsNorm / RmsNormAdd   x, weight (f32 [dim]), dst, m = rows, in_f = dim, eps
+     *   GatedAct               x = gate, aux = up, dst, m = rows, in_f = nff, act, up_off, up_stride,
+     *                          gate_stride, gate_block_width, has_clamp / clamp (swiglu_clamp)
+     *   GatedActFused          x = gu [rows, 2*nff], dst, m = rows, in_f = nff, act, has_clamp / clamp
+     *   Add                    x = a, aux = b, dst, in_f = n (m = 1); in place when dst == x */
+    uint32_t aux;
+    float eps;
+    int act; /* infr_activation */
+    uint32_t up_off, up_stride, gate_stride, gate_block_width;
+    int has_clamp;
+    float clamp;
 } infr_hip_op_t;
 
 /* Backend::compile: validates and stores the op list (the reference's GraphPlan clones the

@@ -4,6 +4,7 @@
 ``include/infr_hip.h``; ``infr_amd.build`` compiles the HIP sources into ``libinfr_hip.so``.
 """
 from .backend import (  # noqa: F401
-    Bindings, Buffer, BufferUsage, DType, Graph, HipBackend, InfrError, Linear, MoeFfn, Plan,
-    Status, TensorDesc, TensorId, block_layout, load_library, synth_normal_f32, synth_weight,
+    Activation, Add, Bindings, Buffer, BufferUsage, DType, GatedAct, GatedActFused, Graph, HipBackend,
+    InfrError, Linear, MoeFfn, Plan, RmsNorm, RmsNormAdd, Status, TensorDesc, TensorId, block_layout,
+    load_library, synth_normal_f32, synth_weight,
 )

@@ -71,7 +71,10 @@ class _Op(C.Structure):
                 ("m", C.c_uint32), ("in_f", C.c_uint32), ("out_f", C.c_uint32),
                 ("w_off", C.c_uint64), ("w_numel", C.c_uint64), ("w_dtype", C.c_int),
                 ("router_x", C.c_uint32), ("router", C.c_uint32), ("gate_exps", C.c_uint32),
-                ("up_exps", C.c_uint32), ("down_exps", C.c_uint32), ("moe", _MoeParams)]
+                ("up_exps", C.c_uint32), ("down_exps", C.c_uint32), ("moe", _MoeParams),
+                ("aux", C.c_uint32), ("eps", C.c_float), ("act", C.c_int), ("up_off", C.c_uint32),
+                ("up_stride", C.c_uint32), ("gate_stride", C.c_uint32), ("gate_block_width", C.c_uint32),
+                ("has_clamp", C.c_int), ("clamp", C.c_float)]
 
 
 class _Caps(C.Structure):
@@ -217,6 +220,71 @@ class MoeFfn:
     n_used: int
     n_ff_exp: int
     scale: float = 1.0
+
+
+class Activation(IntEnum):
+    """crates/infr-core/src/graph.rs Activation; act_fn, crates/infr-cpu/src/kernels.rs:6578-6585."""
+    Silu = 0
+    Gelu = 1
+    Sigmoid = 2
+
+
+@dataclass
+class RmsNorm:
+    """Op::RmsNorm (graph.rs:139-148): dst = rmsnorm(x) * weight over the last `dim` of each row."""
+    x: TensorId
+    weight: TensorId
+    dst: TensorId
+    rows: int
+    dim: int
+    eps: float
+
+
+@dataclass
+class RmsNormAdd:
+    """Op::RmsNormAdd (graph.rs:149-158): dst += rmsnorm(x) * weight."""
+    x: TensorId
+    weight: TensorId
+    dst: TensorId
+    rows: int
+    dim: int
+    eps: float
+
+
+@dataclass
+class GatedAct:
+    """Op::GatedAct (graph.rs:697-735): dst[r, i] = act(gate[r, i]) * up[r, i + up_off]."""
+    gate: TensorId
+    up: TensorId
+    dst: TensorId
+    rows: int
+    nff: int
+    act: int = 0
+    up_off: int = 0
+    up_stride: int = 0
+    gate_stride: int = 0
+    gate_block_width: int = 0
+    swiglu_clamp: float | None = None
+
+
+@dataclass
+class GatedActFused:
+    """Op::GatedActFused (graph.rs:736-748): gu is [rows, 2*nff], gate half first."""
+    gu: TensorId
+    dst: TensorId
+    rows: int
+    nff: int
+    act: int = 0
+    swiglu_clamp: float | None = None
+
+
+@dataclass
+class Add:
+    """Op::Add (graph.rs:749-755): dst[i] = a[i] + b[i]; in place when dst == a."""
+    a: TensorId
+    b: TensorId
+    dst: TensorId
+    n: int
 
 
 @dataclass
@@ -393,6 +461,26 @@ class HipBackend:
                 o.moe = _MoeParams(op.ne, op.n_expert, op.n_used, op.n_ff_exp, rows, op.scale,
                                    int(g.desc(op.router).dtype), int(g.desc(op.gate_exps).dtype),
                                    int(g.desc(op.up_exps).dtype), int(g.desc(op.down_exps).dtype))
+            elif isinstance(op, (RmsNorm, RmsNormAdd)):
+                o.kind = 3 if isinstance(op, RmsNorm) else 4
+                o.x, o.weight, o.dst = op.x.id, op.weight.id, op.dst.id
+                o.m, o.in_f, o.eps = op.rows, op.dim, op.eps
+            elif isinstance(op, GatedAct):
+                o.kind = 5
+                o.x, o.aux, o.dst = op.gate.id, op.up.id, op.dst.id
+                o.m, o.in_f, o.act = op.rows, op.nff, int(op.act)
+                o.up_off, o.up_stride = op.up_off, op.up_stride
+                o.gate_stride, o.gate_block_width = op.gate_stride, op.gate_block_width
+                o.has_clamp, o.clamp = op.swiglu_clamp is not None, op.swiglu_clamp or 0.0
+            elif isinstance(op, GatedActFused):
+                o.kind = 6
+                o.x, o.dst = op.gu.id, op.dst.id
+                o.m, o.in_f, o.act = op.rows, op.nff, int(op.act)
+                o.has_clamp, o.clamp = op.swiglu_clamp is not None, op.swiglu_clamp or 0.0
+            elif isinstance(op, Add):
+                o.kind = 7
+                o.x, o.aux, o.dst = op.a.id, op.b.id, op.dst.id
+                o.m, o.in_f = 1, op.n
             else:
                 raise InfrError(Status.Unsupported, f"op {type(op).__name__} is not on this path")
         h = _vp()

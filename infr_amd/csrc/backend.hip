@@ -102,6 +102,85 @@ bool act_per32(int dt) { return dt == INFR_DTYPE_Q2_0; }
 // Activation scratch for m rows: the prefill kernels read tokens in groups of 32.
 static size_t act_scratch_elems(size_t m, size_t in_f) { return (m == 1 ? 1 : (m + 31) / 32 * 32) * in_f; }
 
+static bool is_elementwise(int kind) { return kind >= INFR_OP_RMS_NORM && kind <= INFR_OP_ADD; }
+
+// Bound f32 operands of an elementwise op, validated against the sizes the op addresses.
+struct ElementwiseArgs {
+    const float* x = nullptr;    // RmsNorm x / GatedAct gate / GatedActFused gu / Add a
+    const float* aux = nullptr;  // RmsNorm weight / GatedAct up / Add b
+    float* dst = nullptr;
+    size_t x_elems = 0, aux_elems = 0, dst_elems = 0;
+};
+
+static int check_elementwise(infr_hip_t* be, const infr_hip_op_t& op, infr_hip_buffer_t* const* bindings,
+                             ElementwiseArgs* a) {
+    const size_t rows = op.m, n = op.in_f;
+    const infr_hip_buffer_t* xb = bindings[op.x];
+    const infr_hip_buffer_t* db = bindings[op.dst];
+    const infr_hip_buffer_t* ab = nullptr;
+    a->dst_elems = rows * n;
+    switch (op.kind) {
+    case INFR_OP_RMS_NORM:
+    case INFR_OP_RMS_NORM_ADD:
+        ab = bindings[op.weight];
+        a->x_elems = rows * n;
+        a->aux_elems = n;
+        break;
+    case INFR_OP_GATED_ACT: {
+        ab = bindings[op.aux];
+        const size_t grow = (op.gate_block_width > 0 || op.gate_stride > 0) ? op.gate_stride : n;
+        // last gate element addressed: the interleaved layout reaches 2x the row's width
+        const size_t glast = op.gate_block_width > 0 ? (n / (op.gate_block_width / 2)) * op.gate_block_width : n;
+        a->x_elems = (rows - 1) * grow + glast;
+        a->aux_elems = (rows - 1) * (op.up_stride ? op.up_stride : n) + op.up_off + n;
+        if (op.gate_block_width > 0 && n % (op.gate_block_width / 2) != 0)
+            return fail(be, INFR_HIP_ERR_UNSUPPORTED, "gated_act: nff is not a whole number of gate blocks");
+        break;
+    }
+    case INFR_OP_GATED_ACT_FUSED:
+        a->x_elems = rows * 2 * n;
+        break;
+    default:  // Add
+        ab = bindings[op.aux];
+        a->x_elems = a->aux_elems = rows * n;
+        break;
+    }
+    if (!xb || !db || (a->aux_elems && !ab)) return fail(be, INFR_HIP_ERR_INVALID, "elementwise op: unbound buffer");
+    if (xb->len < a->x_elems * 4 || db->len < a->dst_elems * 4 || (ab && ab->len < a->aux_elems * 4))
+        return fail(be, INFR_HIP_ERR_INVALID, "elementwise op: buffer too small for the shape");
+    a->x = static_cast<const float*>(xb->ptr);
+    a->aux = ab ? static_cast<const float*>(ab->ptr) : nullptr;
+    a->dst = static_cast<float*>(db->ptr);
+    return INFR_HIP_OK;
+}
+
+static int enqueue_elementwise(infr_hip_t* be, const infr_hip_op_t& op, const ElementwiseArgs& a) {
+    switch (op.kind) {
+    case INFR_OP_RMS_NORM:
+    case INFR_OP_RMS_NORM_ADD:
+        infr::launch_rms_norm(a.x, a.aux, a.dst, op.m, op.in_f, op.eps, op.kind == INFR_OP_RMS_NORM_ADD, be->stream);
+        break;
+    case INFR_OP_GATED_ACT:
+        infr::launch_gated_act(a.x, a.aux, a.dst,
+                               infr::GatedActShape{op.m, op.in_f, op.act, op.up_off, op.up_stride, op.gate_stride,
+                                                   op.gate_block_width, op.has_clamp, op.clamp},
+                               be->stream);
+        break;
+    case INFR_OP_GATED_ACT_FUSED:
+        // the combined buffer is the strided form of the same kernel: gate rows 2*nff apart, up at +nff
+        infr::launch_gated_act(a.x, a.x, a.dst,
+                               infr::GatedActShape{op.m, op.in_f, op.act, op.in_f, 2 * op.in_f, 2 * op.in_f, 0,
+                                                   op.has_clamp, op.clamp},
+                               be->stream);
+        break;
+    default:
+        infr::launch_add(a.x, a.aux, a.dst, (size_t)op.m * op.in_f, be->stream);
+        break;
+    }
+    HIP_TRY(be, hipGetLastError());
+    return INFR_HIP_OK;
+}
+
 // Ops that run in small-batch groups inside plans: the K-split MFMA kernel takes Q4_K up to 32
 // rows, the dot4 batch kernel the other formats up to 8.
 static bool small_batch(const infr_hip_op_t& op) {
@@ -609,6 +688,19 @@ int infr_hip_compile(infr_hip_t* be, const infr_hip_op_t* ops, size_t n_ops, inf
                                     (int)mp.rows, mp.scale, mp.router_dtype, mp.gate_dtype,
                                     mp.up_dtype, mp.down_dtype};
             moe_need = std::max(moe_need, infr::moe_workspace_bytes(ms));
+        } else if (is_elementwise(op.kind)) {
+            const bool clamp_ok = !op.has_clamp || op.act != INFR_ACT_SIGMOID;  // lib.rs:1903-1907
+            const bool act_ok = op.act >= INFR_ACT_SILU && op.act <= INFR_ACT_SIGMOID;
+            if (op.m == 0 || op.in_f == 0 || !clamp_ok || !act_ok ||
+                (op.kind == INFR_OP_GATED_ACT && op.gate_block_width % 2 != 0)) {
+                delete p;
+                return fail(be, INFR_HIP_ERR_UNSUPPORTED, "compile: elementwise op with unsupported shape or mode");
+            }
+            p->max_tensor = std::max({p->max_tensor, op.x, op.dst});
+            if (op.kind == INFR_OP_RMS_NORM || op.kind == INFR_OP_RMS_NORM_ADD)
+                p->max_tensor = std::max(p->max_tensor, op.weight);
+            if (op.kind == INFR_OP_GATED_ACT || op.kind == INFR_OP_ADD)
+                p->max_tensor = std::max(p->max_tensor, op.aux);
         } else {
             delete p;
             return fail(be, INFR_HIP_ERR_UNSUPPORTED, "compile: op kind " + std::to_string(op.kind));
@@ -632,7 +724,8 @@ size_t infr_hip_plan_launches(const infr_hip_plan_t* plan) {
     size_t n = 0;
     for (const auto& st : plan->steps) {
         if (st.op < 0) n += st.m > 1 ? 2 : 1;                              // grouped launch (+ grouped quantize)
-        else if (plan->ops[st.op].kind == INFR_OP_MOE_FFN) n += plan->ops[st.op].moe.rows == 1 ? 4 : 8;
+        else if (plan->ops[st.op].kind == INFR_OP_MOE_FFN) n += plan->ops[st.op].moe.rows == 1 ? 3 : 7;
+        else if (is_elementwise(plan->ops[st.op].kind)) n += 1;
         else n += 2;                                                       // quantize + GEMM
     }
     return n;
@@ -678,6 +771,15 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
             rd[i] = span(bindings[op.x], abytes);
             rd2[i] = span(bindings[op.router_x], abytes);
             wr[i] = span(bindings[op.dst], abytes);
+            wt[i] = Span{nullptr, nullptr};
+        } else if (is_elementwise(op.kind)) {
+            ElementwiseArgs ea;
+            if (int rc = check_elementwise(be, op, bindings, &ea)) return rc;
+            rd[i] = Span{reinterpret_cast<const uint8_t*>(ea.x), reinterpret_cast<const uint8_t*>(ea.x + ea.x_elems)};
+            if (ea.aux)
+                rd2[i] = Span{reinterpret_cast<const uint8_t*>(ea.aux),
+                              reinterpret_cast<const uint8_t*>(ea.aux + ea.aux_elems)};
+            wr[i] = Span{reinterpret_cast<const uint8_t*>(ea.dst), reinterpret_cast<const uint8_t*>(ea.dst + ea.dst_elems)};
             wt[i] = Span{nullptr, nullptr};
         } else {
             if (int rc = check_linear(be, op.w_dtype, bindings[op.weight], op.w_numel, op.w_off,
@@ -753,7 +855,7 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
                 plan->steps.push_back(st);
                 continue;
             }
-            if (op.kind == INFR_OP_MOE_FFN || op.m != 1) {
+            if (op.kind != INFR_OP_LINEAR || op.m != 1) {
                 st.op = (int)i;
                 taken[i] = 1;
                 plan->steps.push_back(st);
@@ -802,6 +904,10 @@ static int enqueue_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t
                                    bindings[op.dst], nullptr, nullptr, &ms, &mb))
                 return rc;
             if (int rc = enqueue_moe(be, ms, mb)) return rc;
+        } else if (st.op >= 0 && is_elementwise(plan->ops[st.op].kind)) {
+            ElementwiseArgs ea;
+            if (int rc = check_elementwise(be, plan->ops[st.op], bindings, &ea)) return rc;
+            if (int rc = enqueue_elementwise(be, plan->ops[st.op], ea)) return rc;
         } else if (st.op >= 0) {
             const auto& op = plan->ops[st.op];
             LinearArgs la;

@@ -1,0 +1,92 @@
+// The ops either side of every Linear in a decoder layer: RmsNorm / RmsNormAdd
+// (crates/infr-cpu/src/lib.rs:802-850), GatedAct / GatedActFused (lib.rs:1890-1971, act_fn and
+// gated_act_fn kernels.rs:6578-6597) and Add (lib.rs:1972-1988). All are HBM-bound streams of a
+// few bytes per element; in plans the decode GEMV absorbs them (see gemv.hip), these stand-alone
+// kernels serve every other case.
+//
+// Numerics. Add and the gated activation are elementwise f32 with the CPU's operation order
+// (`act(g) * u`, `x * s * w` left to right, no FMA); expf / tanhf are the device's, so the last
+// bit can differ from the host libm. RmsNorm's sum of squares is a tree over the row, not the
+// CPU's index-order chain (4096 dependent adds would cost ~15 us): s agrees to ~1e-7 relative.
+#include "device_common.hpp"
+#include "kernels.hpp"
+
+namespace infr {
+
+__device__ __forceinline__ float act_fn(int act, float g) {
+    switch (act) {
+    case 1: return 0.5f * g * (1.0f + tanhf(0.7978846f * (g + 0.044715f * g * g * g)));
+    case 2: return 1.0f / (1.0f + expf(-g));
+    default: return g / (1.0f + expf(-g));
+    }
+}
+
+__device__ __forceinline__ float gated_act_fn(int act, bool has_clamp, float l, float gate, float up) {
+    if (has_clamp) {
+        gate = gate < l ? gate : l;
+        up = up < -l ? -l : (up > l ? l : up);
+    }
+    return act_fn(act, gate) * up;
+}
+
+// One workgroup per row.
+__global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__ x,
+                                                       const float* __restrict__ w, float* out,
+                                                       int dim, float eps, int accumulate) {
+    __shared__ float part[4];
+    const float* xr = x + (size_t)blockIdx.x * dim;
+    float* orow = out + (size_t)blockIdx.x * dim;
+    float s = 0.0f;
+    for (int i = threadIdx.x; i < dim; i += 256) s += xr[i] * xr[i];
+    s = wave_sum_f(s);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
+    __syncthreads();
+    const float ss = ((part[0] + part[1]) + (part[2] + part[3])) / (float)dim;
+    const float scale = 1.0f / sqrtf(ss + eps);
+    for (int i = threadIdx.x; i < dim; i += 256) {
+        const float v = xr[i] * scale * w[i];
+        orow[i] = accumulate ? orow[i] + v : v;
+    }
+}
+
+__global__ __launch_bounds__(256) void gated_act_kernel(const float* __restrict__ gate,
+                                                        const float* __restrict__ up,
+                                                        float* __restrict__ out, GatedActShape s) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)s.rows * s.nff) return;
+    const size_t r = idx / s.nff, i = idx % s.nff;
+    const size_t gb = (s.gate_block_width > 0 || s.gate_stride > 0) ? r * s.gate_stride : r * s.nff;
+    const size_t ub = (s.up_stride == 0 ? r * s.nff : r * s.up_stride) + s.up_off;
+    size_t gi = gb + i;
+    if (s.gate_block_width > 0) {
+        const size_t headw = s.gate_block_width / 2;
+        gi = gb + (i / headw) * s.gate_block_width + headw + i % headw;
+    }
+    out[idx] = gated_act_fn(s.act, s.has_clamp != 0, s.clamp, gate[gi], up[ub + i]);
+}
+
+__global__ __launch_bounds__(256) void add_kernel(const float* a, const float* b, float* out, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] = a[i] + b[i];
+}
+
+void launch_rms_norm(const float* x, const float* w, float* out, size_t rows, size_t dim, float eps,
+                     bool accumulate, hipStream_t stream) {
+    if (rows == 0 || dim == 0) return;
+    hipLaunchKernelGGL(rms_norm_kernel, dim3((unsigned)rows), dim3(256), 0, stream, x, w, out, (int)dim, eps,
+                       accumulate ? 1 : 0);
+}
+
+void launch_gated_act(const float* gate, const float* up, float* out, const GatedActShape& s,
+                      hipStream_t stream) {
+    const size_t n = (size_t)s.rows * s.nff;
+    if (n == 0) return;
+    hipLaunchKernelGGL(gated_act_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, gate, up, out, s);
+}
+
+void launch_add(const float* a, const float* b, float* out, size_t n, hipStream_t stream) {
+    if (n == 0) return;
+    hipLaunchKernelGGL(add_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, a, b, out, n);
+}
+
+}  // namespace infr

@@ -119,6 +119,20 @@ bool launch_gemv_batch_group(int dtype, size_t m, size_t in_f, const BatchTile* 
 void launch_mmq_skinny_group(size_t m, size_t in_f, const BatchTile* tiles_dev, const BatchGroupPlan& plan,
                              const ActQ8& act, hipStream_t stream);
 
+// Elementwise ops either side of a Linear (elementwise.hip).
+struct GatedActShape {
+    uint32_t rows, nff;
+    int act;  // 0 SiLU, 1 GELU (tanh form), 2 sigmoid
+    uint32_t up_off, up_stride, gate_stride, gate_block_width;
+    int has_clamp;
+    float clamp;
+};
+void launch_rms_norm(const float* x, const float* w, float* out, size_t rows, size_t dim, float eps,
+                     bool accumulate, hipStream_t stream);
+void launch_gated_act(const float* gate, const float* up, float* out, const GatedActShape& s,
+                      hipStream_t stream);
+void launch_add(const float* a, const float* b, float* out, size_t n, hipStream_t stream);
+
 // Op::MoeFfn (qwen3moe form). Expert e of a bank starts at bank + e * stride.
 struct MoeShape {
     int ne, n_expert, n_used, n_ff, rows;

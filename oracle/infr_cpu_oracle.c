@@ -403,6 +403,71 @@ float orc_dot(const float *a, const float *b, size_t n) {
 /* crates/infr-cpu/src/kernels.rs:6578-6585 (Activation::Silu) */
 float orc_silu(float g) { return g / (1.0f + expf(-g)); }
 
+/* crates/infr-cpu/src/kernels.rs:6578-6585 */
+float orc_act(int act, float g) {
+    switch (act) {
+    case ORC_ACT_GELU: return 0.5f * g * (1.0f + tanhf(0.7978846f * (g + 0.044715f * g * g * g)));
+    case ORC_ACT_SIGMOID: return 1.0f / (1.0f + expf(-g));
+    default: return g / (1.0f + expf(-g));
+    }
+}
+
+/* crates/infr-cpu/src/kernels.rs:6591-6597 (f32::min / f32::clamp on non-NaN inputs) */
+float orc_gated_act(int act, int has_clamp, float l, float gate, float up) {
+    if (!has_clamp) return orc_act(act, gate) * up;
+    const float g = gate < l ? gate : l;
+    const float u = up < -l ? -l : (up > l ? l : up);
+    return orc_act(act, g) * u;
+}
+
+/* crates/infr-cpu/src/lib.rs:802-850 */
+void orc_rms_norm(const float *x, const float *w, float *out, size_t rows, size_t dim, float eps,
+                  int accumulate) {
+    for (size_t r = 0; r < rows; r++) {
+        const float *xr = x + r * dim;
+        float sum = 0.0f;
+        for (size_t i = 0; i < dim; i++) sum += xr[i] * xr[i];
+        const float ss = sum / (float)dim;
+        const float s = 1.0f / sqrtf(ss + eps);
+        for (size_t i = 0; i < dim; i++) {
+            const float v = xr[i] * s * w[i];
+            if (accumulate) out[r * dim + i] += v;
+            else out[r * dim + i] = v;
+        }
+    }
+}
+
+/* crates/infr-cpu/src/lib.rs:1890-1944 */
+void orc_gated_act_op(const float *gate, const float *up, float *out, size_t rows, size_t nff,
+                      int act, size_t up_off, size_t up_stride, size_t gate_stride,
+                      size_t gate_block_width, int has_clamp, float clamp) {
+    for (size_t r = 0; r < rows; r++) {
+        const size_t gb = (gate_block_width > 0 || gate_stride > 0) ? r * gate_stride : r * nff;
+        const size_t ub = up_stride == 0 ? r * nff + up_off : r * up_stride + up_off;
+        for (size_t i = 0; i < nff; i++) {
+            size_t gi = gb + i;
+            if (gate_block_width > 0) {
+                const size_t headw = gate_block_width / 2;
+                gi = gb + (i / headw) * gate_block_width + headw + i % headw;
+            }
+            out[r * nff + i] = orc_gated_act(act, has_clamp, clamp, gate[gi], up[ub + i]);
+        }
+    }
+}
+
+/* crates/infr-cpu/src/lib.rs:1945-1971 */
+void orc_gated_act_fused(const float *gu, float *out, size_t rows, size_t nff, int act,
+                         int has_clamp, float clamp) {
+    for (size_t r = 0; r < rows; r++)
+        for (size_t i = 0; i < nff; i++)
+            out[r * nff + i] = orc_gated_act(act, has_clamp, clamp, gu[r * 2 * nff + i], gu[r * 2 * nff + nff + i]);
+}
+
+/* crates/infr-cpu/src/lib.rs:1972-1988 */
+void orc_add(const float *a, const float *b, float *out, size_t n) {
+    for (size_t i = 0; i < n; i++) out[i] = a[i] + b[i];
+}
+
 /* ───────────────────────────── Op::Linear ───────────────────────────── */
 
 typedef struct {

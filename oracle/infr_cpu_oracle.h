@@ -95,6 +95,28 @@ float orc_dot(const float *a, const float *b, size_t n);
 /* kernels.rs:6578-6597 — act 0 = SiLU; gated_act_fn with clamp None. */
 float orc_silu(float g);
 
+/* ---- the ops either side of a Linear ---- */
+enum { ORC_ACT_SILU = 0, ORC_ACT_GELU = 1, ORC_ACT_SIGMOID = 2 };
+/* act_fn, kernels.rs:6578-6585 (Silu, gelu_pytorch_tanh, Sigmoid). */
+float orc_act(int act, float g);
+/* gated_act_fn, kernels.rs:6591-6597: act(gate) * up, or with a clamp
+ * act(min(gate, l)) * clamp(up, -l, l). */
+float orc_gated_act(int act, int has_clamp, float clamp, float gate, float up);
+/* Op::RmsNorm / Op::RmsNormAdd arms, crates/infr-cpu/src/lib.rs:802-850: per row
+ * ss = (sum_i x_i*x_i, in index order) / dim; s = 1 / sqrt(ss + eps); out_i = x_i * s * w_i
+ * (accumulate != 0: out_i += ...). */
+void orc_rms_norm(const float *x, const float *w, float *out, size_t rows, size_t dim, float eps,
+                  int accumulate);
+/* Op::GatedAct arm, lib.rs:1890-1944, with its strides, offset and interleaved-gate layout. */
+void orc_gated_act_op(const float *gate, const float *up, float *out, size_t rows, size_t nff,
+                      int act, size_t up_off, size_t up_stride, size_t gate_stride,
+                      size_t gate_block_width, int has_clamp, float clamp);
+/* Op::GatedActFused arm, lib.rs:1945-1971: gu is [rows, 2*nff], gate half first. */
+void orc_gated_act_fused(const float *gu, float *out, size_t rows, size_t nff, int act,
+                         int has_clamp, float clamp);
+/* Op::Add arm, lib.rs:1972-1988. */
+void orc_add(const float *a, const float *b, float *out, size_t n);
+
 /* crates/infr-cpu/src/lib.rs:985-1492 — the Op::Linear arm for Q4_K/Q6_K/Q8_0/Q2_0/F32 weights.
  *   w/wbytes: the whole bound weight buffer; w_numel: its declared element count;
  *   w_off: element offset of the first row (must be a multiple of in_f);

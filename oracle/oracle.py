@@ -201,6 +201,60 @@ def silu(g: float) -> np.float32:
     return np.float32(_silu(np.float32(g)))
 
 
+SILU, GELU, SIGMOID = 0, 1, 2
+_act = _sig("orc_act", C.c_float, C.c_int, C.c_float)
+_gated = _sig("orc_gated_act", C.c_float, C.c_int, C.c_int, C.c_float, C.c_float, C.c_float)
+_rms = _sig("orc_rms_norm", None, _f32p, _f32p, _f32p, C.c_size_t, C.c_size_t, C.c_float, C.c_int)
+_gact = _sig("orc_gated_act_op", None, _f32p, _f32p, _f32p, C.c_size_t, C.c_size_t, C.c_int, C.c_size_t,
+             C.c_size_t, C.c_size_t, C.c_size_t, C.c_int, C.c_float)
+_gactf = _sig("orc_gated_act_fused", None, _f32p, _f32p, C.c_size_t, C.c_size_t, C.c_int, C.c_int, C.c_float)
+_addop = _sig("orc_add", None, _f32p, _f32p, _f32p, C.c_size_t)
+
+
+def act(kind: int, g: float) -> np.float32:
+    """act_fn (kernels.rs:6578-6585)."""
+    return np.float32(_act(kind, np.float32(g)))
+
+
+def gated_act_fn(kind: int, clamp, gate: float, up: float) -> np.float32:
+    """gated_act_fn (kernels.rs:6591-6597); ``clamp`` is None or the limit."""
+    return np.float32(_gated(kind, clamp is not None, np.float32(clamp or 0.0), np.float32(gate), np.float32(up)))
+
+
+def rms_norm(x, w, rows: int, dim: int, eps: float, into=None) -> np.ndarray:
+    """Op::RmsNorm; with ``into`` (a [rows, dim] array) Op::RmsNormAdd: into += rmsnorm(x) * w."""
+    x, w = _c(x, np.float32).ravel(), _c(w, np.float32).ravel()
+    out = np.zeros(rows * dim, np.float32) if into is None else _c(into, np.float32).ravel().copy()
+    _rms(_p(x, _f32p), _p(w, _f32p), _p(out, _f32p), rows, dim, np.float32(eps), into is not None)
+    return out.reshape(rows, dim)
+
+
+def gated_act(gate, up, rows: int, nff: int, kind: int = SILU, *, up_off: int = 0, up_stride: int = 0,
+              gate_stride: int = 0, gate_block_width: int = 0, clamp=None) -> np.ndarray:
+    """Op::GatedAct (lib.rs:1890-1944)."""
+    gate, up = _c(gate, np.float32).ravel(), _c(up, np.float32).ravel()
+    out = np.empty(rows * nff, np.float32)
+    _gact(_p(gate, _f32p), _p(up, _f32p), _p(out, _f32p), rows, nff, kind, up_off, up_stride, gate_stride,
+          gate_block_width, clamp is not None, np.float32(clamp or 0.0))
+    return out.reshape(rows, nff)
+
+
+def gated_act_fused(gu, rows: int, nff: int, kind: int = SILU, *, clamp=None) -> np.ndarray:
+    """Op::GatedActFused (lib.rs:1945-1971)."""
+    gu = _c(gu, np.float32).ravel()
+    out = np.empty(rows * nff, np.float32)
+    _gactf(_p(gu, _f32p), _p(out, _f32p), rows, nff, kind, clamp is not None, np.float32(clamp or 0.0))
+    return out.reshape(rows, nff)
+
+
+def add(a, b) -> np.ndarray:
+    """Op::Add (lib.rs:1972-1988)."""
+    a, b = _c(a, np.float32).ravel(), _c(b, np.float32).ravel()
+    out = np.empty(a.size, np.float32)
+    _addop(_p(a, _f32p), _p(b, _f32p), _p(out, _f32p), a.size)
+    return out
+
+
 def linear(dtype: int, w, x, m: int, in_f: int, out_f: int, *, w_numel: int | None = None,
            w_off: int = 0, reference_mode: bool = False, threads: int = 0) -> np.ndarray:
     """Op::Linear on the CPU oracle. ``w`` is the whole bound weight buffer (raw GGUF blocks)."""
