@@ -147,6 +147,77 @@ class Sweep:
         self.keep = []
 
 
+def layer_bench(be, n_layers, dtype=None):
+    """A decode step through `n_layers` Qwen3-8B-shaped decoder layers without attention:
+    RmsNorm -> {q, k, v} -> o(q) -> Add -> RmsNorm -> {gate, up} -> GatedAct -> down -> Add, every op
+    reading what the previous one wrote. The plan absorbs the norms, the gated activation and the
+    residual adds into the decode GEMVs (4 launches per layer instead of 9). Returns
+    (ms per step, weight bytes, launches per step)."""
+    from infr_amd import (Add, Bindings, BufferUsage, DType, GatedAct, Graph, Linear, RmsNorm, TensorDesc,
+                          synth_normal_f32, synth_weight)
+    dtype = dtype or DType.Q4K
+    H, KV, FF = 4096, 1024, 12288
+    g, binds, keep = Graph(), Bindings(), []
+
+    def f32(shape, data=None, out=False):
+        t = (g.output if out else g.input)(TensorDesc(shape, DType.F32))
+        n = 1
+        for d in shape:
+            n *= d
+        b = be.upload_new(data) if data is not None else be.alloc(n * 4)
+        keep.append(b)
+        binds.bind(t, b)
+        return t
+    x = f32((1, H), synth_normal_f32(1, H))
+    protos = {name: be.upload_new(synth_weight(dtype, i, out_f, in_f), BufferUsage.Weights)
+              for i, (name, out_f, in_f) in enumerate(LAYER)}
+    keep += list(protos.values())
+    total = 0
+    for layer in range(n_layers):
+        w = {}
+        for name, out_f, in_f in LAYER:
+            nb = weight_bytes(dtype, out_f, in_f)
+            wb = protos[name]
+            if layer:
+                wb = be.alloc_uninit(nb, BufferUsage.Weights)
+                be.copy_buffer(protos[name], wb, nb)
+                keep.append(wb)
+            w[name] = g.weight(TensorDesc((out_f, in_f), dtype))
+            binds.bind(w[name], wb)
+            total += nb
+        n1, n2 = (f32((H,), synth_normal_f32(2 + i, H, mean=1.0, sigma=0.1)) for i in range(2))
+        h1, q, k, v, o = (f32((1, d), out=True) for d in (H, H, KV, KV, H))
+        h2, gt, up, act, dn = (f32((1, d), out=True) for d in (H, FF, FF, FF, H))
+        g.push(RmsNorm(x, n1, h1, 1, H, 1e-6))
+        g.push(Linear(h1, w["q"], q, 1, H, H))
+        g.push(Linear(h1, w["k"], k, 1, H, KV))
+        g.push(Linear(h1, w["v"], v, 1, H, KV))
+        g.push(Linear(q, w["o"], o, 1, H, H))
+        g.push(Add(o, x, x, H))
+        g.push(RmsNorm(x, n2, h2, 1, H, 1e-6))
+        g.push(Linear(h2, w["gate"], gt, 1, H, FF))
+        g.push(Linear(h2, w["up"], up, 1, H, FF))
+        g.push(GatedAct(gt, up, act, 1, FF))
+        g.push(Linear(act, w["down"], dn, 1, FF, H))
+        g.push(Add(dn, x, x, H))
+    be.sync()
+    plan = be.compile(g)
+    for _ in range(2):
+        be.execute(plan, binds)
+    be.sync()
+    steps, t0 = 10, time.perf_counter()
+    be.timer_begin()
+    for _ in range(steps):
+        be.execute(plan, binds)
+    dev = be.timer_end() / steps
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    launches = plan.launches()
+    plan = None
+    for b in keep:
+        b.free()
+    return max(dev, wall), total, launches
+
+
 def single_shape(be, dtype, m, in_f, out_f, reps=40, rotate_bytes=768 << 20):
     """One shape, cold: rotate through enough distinct copies of the weight to exceed the last
     level cache, `reps` back-to-back launches. Returns (ms per launch, weight bytes)."""
@@ -275,8 +346,8 @@ def main():
     ap.add_argument("--layers", type=int, default=N_LAYERS)
     ap.add_argument("--no-extra", action="store_true", help="headline sweep only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--sections", default="shapes,mmq,chain,ternary,moe",
-                    help="comma list of secondary sections: shapes, mmq, chain, ternary, moe")
+    ap.add_argument("--sections", default="shapes,mmq,chain,layer,ternary,moe",
+                    help="comma list of secondary sections: shapes, mmq, chain, layer, ternary, moe")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
@@ -341,6 +412,24 @@ def main():
         extra["decode_chain_Q4_K_GBs"] = round(ch.bytes / (max(d, w) * 1e-3) / 1e9, 1)
         extra["decode_chain_launches_per_step"] = ch.plan.launches()
         ch.free()
+    if "layer" in sections:
+        ms, nb, launches = layer_bench(be, args.layers)
+        extra["decode_layer_Q4_K_GBs"] = round(nb / (ms * 1e-3) / 1e9, 1)
+        extra["decode_layer_us_per_layer"] = round(ms * 1e3 / args.layers, 2)
+        extra["decode_layer_launches_per_step"] = launches
+        if os.environ.get("INFR_HIP_FUSE", "1") != "0":
+            # the same plan with the absorption switched off (a fresh process: the switch is read once)
+            import subprocess
+            env = dict(os.environ, INFR_HIP_FUSE="0")
+            r = subprocess.run([sys.executable, os.path.abspath(__file__), "--no-cpu", "--sections", "layer",
+                                "--layers", str(args.layers), "--steps", "1", "--warmup", "1"],
+                               env=env, capture_output=True, text=True)
+            for line in r.stdout.splitlines():
+                if line.startswith("{"):
+                    ex = json.loads(line)["extra"]
+                    extra["decode_layer_unfused_Q4_K_GBs"] = ex["decode_layer_Q4_K_GBs"]
+                    extra["decode_layer_unfused_us_per_layer"] = ex["decode_layer_us_per_layer"]
+                    extra["decode_layer_unfused_launches_per_step"] = ex["decode_layer_launches_per_step"]
     if "ternary" in sections:
         tern = Sweep(be, DType.Q2_0, 1, N_LAYERS, head=True)
         d, w = tern.time(5, 2)

@@ -752,12 +752,21 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
         const uint8_t* p = static_cast<const uint8_t*>(b->ptr);
         return Span{p, p + bytes};
     };
+    auto fspan = [](const float* p, size_t elems) {
+        return Span{reinterpret_cast<const uint8_t*>(p), reinterpret_cast<const uint8_t*>(p + elems)};
+    };
     auto overlap = [](const Span& a, const Span& b) { return a.lo < b.hi && b.lo < a.hi; };
-    std::vector<Span> rd(n), wr(n), wt(n);
+    auto any_overlap = [&](const std::vector<Span>& a, const std::vector<Span>& b) {
+        for (const auto& x : a)
+            for (const auto& y : b)
+                if (overlap(x, y)) return true;
+        return false;
+    };
+    // reads / writes: device ranges an op reads (activations and weights) and writes
+    std::vector<std::vector<Span>> rd(n), wr(n);
     std::vector<int> level(n, 0);
     std::vector<LinearArgs> la(n);
-    int max_level = 0;
-    std::vector<Span> rd2(n, Span{nullptr, nullptr});
+    std::vector<ElementwiseArgs> ea(n);
     for (size_t i = 0; i < n; ++i) {
         const auto& op = plan->ops[i];
         if (op.kind == INFR_OP_MOE_FFN) {
@@ -768,19 +777,13 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
                                    bindings[op.dst], nullptr, nullptr, &ms, &mb))
                 return rc;
             const size_t abytes = (size_t)ms.rows * ms.ne * sizeof(float);
-            rd[i] = span(bindings[op.x], abytes);
-            rd2[i] = span(bindings[op.router_x], abytes);
-            wr[i] = span(bindings[op.dst], abytes);
-            wt[i] = Span{nullptr, nullptr};
+            rd[i] = {span(bindings[op.x], abytes), span(bindings[op.router_x], abytes)};
+            wr[i] = {span(bindings[op.dst], abytes)};
         } else if (is_elementwise(op.kind)) {
-            ElementwiseArgs ea;
-            if (int rc = check_elementwise(be, op, bindings, &ea)) return rc;
-            rd[i] = Span{reinterpret_cast<const uint8_t*>(ea.x), reinterpret_cast<const uint8_t*>(ea.x + ea.x_elems)};
-            if (ea.aux)
-                rd2[i] = Span{reinterpret_cast<const uint8_t*>(ea.aux),
-                              reinterpret_cast<const uint8_t*>(ea.aux + ea.aux_elems)};
-            wr[i] = Span{reinterpret_cast<const uint8_t*>(ea.dst), reinterpret_cast<const uint8_t*>(ea.dst + ea.dst_elems)};
-            wt[i] = Span{nullptr, nullptr};
+            if (int rc = check_elementwise(be, op, bindings, &ea[i])) return rc;
+            rd[i] = {fspan(ea[i].x, ea[i].x_elems)};
+            if (ea[i].aux) rd[i].push_back(fspan(ea[i].aux, ea[i].aux_elems));
+            wr[i] = {fspan(ea[i].dst, ea[i].dst_elems)};
         } else {
             if (int rc = check_linear(be, op.w_dtype, bindings[op.weight], op.w_numel, op.w_off,
                                       bindings[op.x], op.m, op.in_f, op.out_f, &la[i]))
@@ -788,17 +791,109 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
             const size_t ybytes = (size_t)op.m * op.out_f * sizeof(float);
             if (!bindings[op.dst] || bindings[op.dst]->len < ybytes)
                 return fail(be, INFR_HIP_ERR_INVALID, "execute: dst buffer missing or too small");
-            rd[i] = span(bindings[op.x], (size_t)op.m * op.in_f * sizeof(float));
-            wr[i] = span(bindings[op.dst], ybytes);
-            wt[i] = Span{la[i].wrows, la[i].wrows + (size_t)op.out_f * la[i].bpr};
+            rd[i] = {span(bindings[op.x], (size_t)op.m * op.in_f * sizeof(float)),
+                     Span{la[i].wrows, la[i].wrows + (size_t)op.out_f * la[i].bpr}};
+            wr[i] = {span(bindings[op.dst], ybytes)};
         }
-        for (size_t j = 0; j < i; ++j)
-            if (overlap(wr[j], rd[i]) || overlap(wr[j], rd2[i]) || overlap(wr[j], wr[i]) ||
-                overlap(rd[j], wr[i]) || overlap(rd2[j], wr[i]) || overlap(wr[j], wt[i]) ||
-                overlap(wt[j], wr[i]))
+    }
+
+    // ---- absorb the ops around m == 1 Linears into the decode GEMV (see infr::GemvFusion) ----
+    // pre[i]  >= 0: Linear i computes its x from op pre[i]'s inputs (GatedAct / GatedActFused / RmsNorm)
+    // post[i] >= 0: Linear i also writes Op::Add post[i]
+    // absorbed[k]: op k runs inside some Linear and is not scheduled on its own
+    std::vector<int> pre(n, -1), post(n, -1);
+    std::vector<char> absorbed(n, 0), publishes(n, 0);
+    static const int env_fuse = getenv("INFR_HIP_FUSE") ? atoi(getenv("INFR_HIP_FUSE")) : 1;
+    auto decode_linear = [&](size_t i) { return plan->ops[i].kind == INFR_OP_LINEAR && plan->ops[i].m == 1; };
+    for (size_t k = 0; env_fuse && k < n; ++k) {
+        const auto& p = plan->ops[k];
+        const bool gated = (p.kind == INFR_OP_GATED_ACT && p.gate_block_width == 0) || p.kind == INFR_OP_GATED_ACT_FUSED;
+        if (!(gated || p.kind == INFR_OP_RMS_NORM) || p.m != 1 || p.in_f % 4 != 0) continue;
+        // every reader of the producer's dst must be a later decode Linear taking exactly that
+        // vector as x, with the producer's inputs and dst untouched in between
+        std::vector<size_t> users;
+        bool ok = true;
+        for (size_t i = 0; ok && i < n; ++i) {
+            if (i == k || !any_overlap(rd[i], wr[k])) continue;
+            ok = i > k && decode_linear(i) && plan->ops[i].in_f == p.in_f &&
+                 static_cast<const float*>(bindings[plan->ops[i].x]->ptr) == ea[k].dst;
+            if (ok) users.push_back(i);
+        }
+        if (!ok || users.empty()) continue;
+        for (size_t j = k + 1; ok && j <= users.back(); ++j)
+            ok = !any_overlap(wr[j], rd[k]) && (!any_overlap(wr[j], wr[k]));
+        if (!ok) continue;
+        for (size_t u : users) ok = ok && pre[u] < 0;
+        if (!ok) continue;
+        absorbed[k] = 1;
+        for (size_t u : users) {
+            pre[u] = (int)k;
+            // the consumer reads the producer's inputs instead of its dst; the first one stores dst
+            rd[u][0] = rd[k][0];
+            for (size_t q = 1; q < rd[k].size(); ++q) rd[u].push_back(rd[k][q]);
+        }
+        publishes[users.front()] = 1;
+        wr[users.front()].push_back(wr[k][0]);
+    }
+    for (size_t k = 0; env_fuse && k < n; ++k) {
+        const auto& a = plan->ops[k];
+        if (a.kind != INFR_OP_ADD) continue;
+        // a = the output of an earlier decode Linear of the same length; nothing in between may
+        // touch dst or write b (the sum is produced at the Linear's place in the order)
+        for (size_t i = 0; i < k; ++i) {
+            if (!decode_linear(i) || post[i] >= 0 || plan->ops[i].out_f != a.in_f ||
+                static_cast<const float*>(bindings[plan->ops[i].dst]->ptr) != ea[k].x)
+                continue;
+            bool ok = true;
+            const std::vector<Span> b_span{fspan(ea[k].aux, ea[k].aux_elems)};
+            for (size_t j = i + 1; ok && j < k; ++j)
+                ok = !any_overlap(wr[j], wr[k]) && !any_overlap(rd[j], wr[k]) && !any_overlap(wr[j], b_span) &&
+                     !any_overlap(wr[j], wr[i]);
+            // the Linear's own inputs must not alias the Add's destination
+            ok = ok && !any_overlap(rd[i], wr[k]);
+            if (!ok) continue;
+            post[i] = (int)k;
+            absorbed[k] = 1;
+            rd[i].push_back(b_span[0]);
+            wr[i].push_back(wr[k][0]);
+            break;
+        }
+    }
+
+    int max_level = 0;
+    for (size_t i = 0; i < n; ++i) {
+        if (absorbed[i]) continue;
+        for (size_t j = 0; j < i; ++j) {
+            if (absorbed[j]) continue;
+            if (any_overlap(wr[j], rd[i]) || any_overlap(wr[j], wr[i]) || any_overlap(rd[j], wr[i]))
                 level[i] = std::max(level[i], level[j] + 1);
+        }
         max_level = std::max(max_level, level[i]);
     }
+    auto fusion_of = [&](size_t k) {
+        infr::GemvFusion f;
+        if (pre[k] >= 0) {
+            const auto& p = plan->ops[pre[k]];
+            const ElementwiseArgs& e = ea[pre[k]];
+            if (p.kind == INFR_OP_RMS_NORM) {
+                f.pre = 2;
+                f.x2 = e.aux;
+                f.eps = p.eps;
+            } else {
+                f.pre = 1;
+                f.x2 = p.kind == INFR_OP_GATED_ACT_FUSED ? e.x + p.in_f : e.aux + p.up_off;
+                f.act = p.act;
+                f.has_clamp = p.has_clamp;
+                f.clamp = p.clamp;
+            }
+            f.pre_dst = publishes[k] ? e.dst : nullptr;
+        }
+        if (post[k] >= 0) {
+            f.add_b = ea[post[k]].aux;
+            f.add_dst = ea[post[k]].dst;
+        }
+        return f;
+    };
     plan->steps.clear();
     plan->descs.clear();
     plan->tiles.clear();
@@ -807,7 +902,7 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
     for (int lv = 0; lv <= max_level; ++lv) {
         std::vector<char> taken(n, 0);
         for (size_t i = 0; i < n; ++i) {
-            if (level[i] != lv || taken[i]) continue;
+            if (level[i] != lv || taken[i] || absorbed[i]) continue;
             const auto& op = plan->ops[i];
             infr_hip_plan::Step st;
             st.level = lv;
@@ -866,13 +961,14 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
             st.first = (int)plan->descs.size();
             for (size_t k = i; k < n; ++k) {
                 const auto& o2 = plan->ops[k];
-                if (level[k] != lv || taken[k] || o2.kind != INFR_OP_LINEAR || o2.m != 1 ||
+                if (level[k] != lv || taken[k] || absorbed[k] || o2.kind != INFR_OP_LINEAR || o2.m != 1 ||
                     o2.w_dtype != op.w_dtype || o2.in_f != op.in_f)
                     continue;
                 taken[k] = 1;
-                plan->descs.push_back(infr::GemvOpDesc{
-                    la[k].wrows, static_cast<const float*>(bindings[o2.x]->ptr),
-                    static_cast<float*>(bindings[o2.dst]->ptr), la[k].bpr, (int32_t)o2.out_f});
+                // with an absorbed producer the GEMV starts from the producer's first input
+                const float* xsrc = pre[k] >= 0 ? ea[pre[k]].x : static_cast<const float*>(bindings[o2.x]->ptr);
+                plan->descs.push_back(infr::GemvOpDesc{la[k].wrows, xsrc, static_cast<float*>(bindings[o2.dst]->ptr),
+                                                       la[k].bpr, (int32_t)o2.out_f, fusion_of(k)});
             }
             st.n = (int)plan->descs.size() - st.first;
             if (!infr::plan_gemv_group(st.dtype, st.in_f, &plan->descs[st.first], st.n, &st.gp))

@@ -105,6 +105,22 @@ __global__ __launch_bounds__(256) void gemv_batch_kernel(const uint8_t* __restri
         osum + (threadIdx.x >> 6) * (F::kOrdered ? OrderedSum<STEPS>::kFloatsPerWave : 0));
 }
 
+// act(gate) * up with the optional clamp, as Op::GatedAct evaluates one element
+// (gated_act_fn, crates/infr-cpu/src/kernels.rs:6591-6597).
+__device__ __forceinline__ float fused_gated_act(int act, bool has_clamp, float l, float gate, float up) {
+    if (has_clamp) {
+        gate = gate < l ? gate : l;
+        up = up < -l ? -l : (up > l ? l : up);
+    }
+    float a;
+    switch (act) {
+    case 1: a = 0.5f * gate * (1.0f + tanhf(0.7978846f * (gate + 0.044715f * gate * gate * gate))); break;
+    case 2: a = 1.0f / (1.0f + expf(-gate)); break;
+    default: a = gate / (1.0f + expf(-gate)); break;
+    }
+    return a * up;
+}
+
 // Fused + grouped form. LDS: qs[in_f] | d[in_f/32] | bsums[in_f/32] | bsums16[in_f/16] | per-wave
 // ordered-sum scratch.
 template <typename F, int STEPS, int NW>
@@ -126,6 +142,12 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, 
         tile.y = single.y + first;
         tile.bpr = (uint32_t)single.bpr;
         tile.rows = min(single_rows, single.out_f - first);
+        tile.fus = single.fus;
+        if (tile.fus.add_dst) {
+            tile.fus.add_b += first;
+            tile.fus.add_dst += first;
+        }
+        if (blockIdx.x != 0) tile.fus.pre_dst = nullptr;
     }
     const int rpw = (tile.rows + NW - 1) / NW;
     const int n_units = F::units(in_f);
@@ -155,6 +177,47 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, 
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) ok[t] = has_rows && F::valid(t, lane, n_units);
     F::load_row(first, tile.w + (size_t)row0 * tile.bpr, 0, lane, ok[0]);
+    // An absorbed producer of x (workgroup-uniform branch): every workgroup recomputes the vector
+    // from the producer's inputs - cheaper than a launch of its own - and the op's first
+    // workgroup stores it where the producer would have.
+    if (tile.fus.pre != 0) {
+        float scale = 1.0f;
+        if (tile.fus.pre == 2) {  // RmsNorm: mean square over the row, tree order fixed by NW
+            float* part = reinterpret_cast<float*>(lds);  // qs area, not yet written
+            float sq = 0.0f;
+#pragma unroll
+            for (int i = 0; i < kMaxChunks; ++i)
+                sq += (xv[i].x * xv[i].x + xv[i].y * xv[i].y) + (xv[i].z * xv[i].z + xv[i].w * xv[i].w);
+            sq = wave_sum_f(sq);
+            if (lane == 0) part[wave] = sq;
+            __syncthreads();
+            float tot = 0.0f;
+#pragma unroll
+            for (int wv = 0; wv < NW; ++wv) tot += part[wv];
+            __syncthreads();  // `part` is about to be overwritten by the quantized codes
+            scale = 1.0f / sqrtf(tot / (float)in_f + tile.fus.eps);
+        }
+#pragma unroll
+        for (int i = 0; i < kMaxChunks; ++i) {
+            const int c = wave + i * NW;
+            if (c < n_chunks && c * 256 + lane * 4 < in_f) {
+                const v4f o = *reinterpret_cast<const v4f*>(tile.fus.x2 + (size_t)c * 256 + lane * 4);
+                v4f r;
+                if (tile.fus.pre == 2) {
+                    r = v4f{xv[i].x * scale * o.x, xv[i].y * scale * o.y, xv[i].z * scale * o.z, xv[i].w * scale * o.w};
+                } else {
+                    const bool hc = tile.fus.has_clamp != 0;
+                    r.x = fused_gated_act(tile.fus.act, hc, tile.fus.clamp, xv[i].x, o.x);
+                    r.y = fused_gated_act(tile.fus.act, hc, tile.fus.clamp, xv[i].y, o.y);
+                    r.z = fused_gated_act(tile.fus.act, hc, tile.fus.clamp, xv[i].z, o.z);
+                    r.w = fused_gated_act(tile.fus.act, hc, tile.fus.clamp, xv[i].w, o.w);
+                }
+                xv[i] = r;
+                if (tile.fus.pre_dst)
+                    *reinterpret_cast<v4f*>(tile.fus.pre_dst + (size_t)c * 256 + lane * 4) = r;
+            }
+        }
+    }
 #pragma unroll
     for (int i = 0; i < kMaxChunks; ++i) {
         const int c = wave + i * NW;
@@ -171,7 +234,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, 
     for (int t = 0; t < STEPS; ++t) F::load_acts(acts[t], act, t, lane, ok[t]);
     float* osum = reinterpret_cast<float*>(lds + in_f + in_f / 2) + wave * OrderedSum<STEPS>::kFloatsPerWave;
     gemv_rows<F, STEPS, false>(tile.w, tile.bpr, first, acts, ok, tile.y, n_units, row0, row_end, lane,
-                               StagePtrs{nullptr, nullptr}, osum);
+                               StagePtrs{nullptr, nullptr}, osum, tile.fus.add_b, tile.fus.add_dst);
 }
 
 // ───────────────────────────────────── launch ─────────────────────────────────────
@@ -433,14 +496,20 @@ static bool plan_group_fmt(size_t in_f, const GemvOpDesc* ops, int n, GemvGroupP
     size_t rows_per_wg = (total_rows + 511) / 512;
     rows_per_wg = rows_per_wg < 4 ? 4 : (rows_per_wg > 128 ? 128 : rows_per_wg);
     const size_t lds_bytes = in_f + in_f / 2 + (F::kOrdered ? (size_t)nw * (16 * (16 * steps + 4)) * sizeof(float) : 0);
-    // Wave quantisation: the chip holds `resident` workgroups at once, and a grid of only a few
-    // such rounds that needs a little more than a whole number of them idles most of the machine
-    // during the last one. For those grids take, among tile heights near the one above, the one
-    // with the least modelled time rounds x (rows + fixed cost), the fixed cost being the
-    // per-workgroup quantization of x (about eleven rows' worth). Grids of many rounds keep the
-    // 128-row tiles: their tail is small and taller tiles measured slower.
+    // Grids of only a few rounds: a grid that needs a little more than a whole number of rounds
+    // idles most of the machine during the last one, and workgroups that share a compute unit
+    // share its pipes, so what counts is workgroups per compute unit. For those grids take, among
+    // tile heights near the one above, the one with the least modelled time
+    // ceil(workgroups / CUs) x (rows + fixed cost); the fixed cost is the per-workgroup prologue
+    // in units of a weight row: about eleven for quantizing x, more when the prologue also
+    // evaluates an absorbed gated activation (expf per element) or RmsNorm. Grids of many rounds
+    // keep the 128-row tiles: their tail is small and taller tiles measured slower.
     static const int env_model = getenv("INFR_HIP_GEMV_ROUNDS") ? atoi(getenv("INFR_HIP_GEMV_ROUNDS")) : 1;
     const int resident = device_cu_count() * fused_wgs_per_cu<F>(steps, nw, lds_bytes);
+    const int cus = device_cu_count();
+    double fixed = 11.0;
+    for (int i = 0; i < n; ++i)
+        fixed = std::max(fixed, ops[i].fus.pre == 1 ? 32.0 : (ops[i].fus.pre == 2 ? 15.0 : 11.0));
     auto wgs_at = [&](size_t r) {
         size_t w = 0;
         for (int i = 0; i < n; ++i) w += ((size_t)ops[i].out_f + r - 1) / r;
@@ -451,8 +520,8 @@ static bool plan_group_fmt(size_t in_f, const GemvOpDesc* ops, int n, GemvGroupP
         double best = 1e300;
         size_t best_r = rows_per_wg;
         for (size_t r = lo; r <= hi; ++r) {
-            const size_t rounds = (wgs_at(r) + resident - 1) / resident;
-            const double cost = (double)rounds * ((double)r + 11.0);
+            const size_t rounds = (wgs_at(r) + cus - 1) / cus;
+            const double cost = (double)rounds * ((double)r + fixed);
             if (cost < best * 0.999) {  // ties go to the smaller tile
                 best = cost;
                 best_r = r;
@@ -493,6 +562,12 @@ void fill_gemv_tiles(const GemvOpDesc* ops, int n, const GemvGroupPlan& plan, Ge
             tl.y = ops[i].y + r;
             tl.bpr = (uint32_t)ops[i].bpr;
             tl.rows = ops[i].out_f - r < per_wg ? ops[i].out_f - r : per_wg;
+            tl.fus = ops[i].fus;
+            if (tl.fus.add_dst) {
+                tl.fus.add_b += r;
+                tl.fus.add_dst += r;
+            }
+            if (r != 0) tl.fus.pre_dst = nullptr;
         }
 }
 

@@ -29,7 +29,8 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
                                           const typename F::Acts (&acts)[STEPS],
                                           const bool (&ok)[STEPS], float* __restrict__ y, int n_units,
                                           int row0, int row_end, int lane, const StagePtrs& st,
-                                          float* osum) {
+                                          float* osum, const float* add_b = nullptr,
+                                          float* add_dst = nullptr) {
     constexpr int LS = OrderedSum<STEPS>::kRowStride;
     typename F::Row cur = first;
     int in_batch = 0, batch_row0 = row0;
@@ -64,13 +65,18 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
                         acc += v.w;
                     }
                     y[batch_row0 + lane] = acc;
+                    // an absorbed Op::Add: dst = a + b with a = this output
+                    if (add_dst) add_dst[batch_row0 + lane] = acc + add_b[batch_row0 + lane];
                 }
                 batch_row0 = row + 1;
                 in_batch = 0;
             }
         } else {
             s = wave_sum_f(s);
-            if (lane == 0) y[row] = s;
+            if (lane == 0) {
+                y[row] = s;
+                if (add_dst) add_dst[row] = s + add_b[row];
+            }
         }
     }
 }

@@ -51,23 +51,43 @@ bool launch_gemv_batch(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act
 
 // One m == 1 Op::Linear of a fused, grouped decode launch: the kernel quantizes x itself (into
 // LDS) and produces y. All ops of a group share (dtype, in_f).
+// What the decode GEMV can absorb from the ops around an m == 1 Linear (plans fuse them):
+//   before: x = gated_act(gate, up) (Op::GatedAct / GatedActFused) or x = rmsnorm(x_in) * w
+//           (Op::RmsNorm), computed by every workgroup in its quantization prologue; the first
+//           workgroup of the op also stores that f32 vector to `pre_dst` (the absorbed op's dst)
+//   after:  add_dst[row] = y[row] + add_b[row] (Op::Add), next to the plain y store
+struct GemvFusion {
+    const float* x2 = nullptr;   // GatedAct: up; RmsNorm: weight
+    float* pre_dst = nullptr;    // nullptr: computed but not stored
+    const float* add_b = nullptr;
+    float* add_dst = nullptr;    // nullptr: no Add
+    int32_t pre = 0;             // 0 none, 1 gated activation, 2 RmsNorm
+    int32_t act = 0;             // gated activation kind (0 SiLU, 1 GELU, 2 sigmoid)
+    int32_t has_clamp = 0;
+    float clamp = 0.0f;
+    float eps = 0.0f;
+};
+
 struct GemvOpDesc {
     const uint8_t* w;  // first selected weight row
-    const float* x;    // f32 [in_f]
+    const float* x;    // f32 [in_f] (gate / un-normalised input when fus.pre != 0)
     float* y;          // f32 [out_f]
     uint64_t bpr;      // bytes per weight row
     int32_t out_f;
+    GemvFusion fus;
 };
 
 // What one workgroup of a grouped launch works on: `rows` consecutive weight rows of one op.
 // The launcher keeps a table of these in device memory, indexed by blockIdx.x, so a workgroup
-// finds its work with a single 32-byte scalar load.
+// finds its work with one run of scalar loads.
 struct GemvTile {
     const uint8_t* w;  // first row of the tile
     const float* x;
     float* y;          // output of the tile's first row
     uint32_t bpr;
     int32_t rows;
+    GemvFusion fus;    // add_b / add_dst already offset to the tile's first row; pre_dst only in
+                       // the op's first tile
 };
 
 struct GemvGroupPlan {

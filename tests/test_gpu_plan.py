@@ -142,3 +142,126 @@ def test_small_batch_ops_run_as_groups(be, m):
                 else:
                     a, b = got.astype(np.float64).ravel(), ref.astype(np.float64).ravel()
                     assert np.linalg.norm(a - b) <= 1e-4 * np.linalg.norm(b), f"{name} {d}"
+
+
+def _rel(a, b):
+    a, b = np.asarray(a, np.float64).ravel(), np.asarray(b, np.float64).ravel()
+    return np.linalg.norm(a - b) / np.linalg.norm(b)
+
+
+@pytest.mark.parametrize("combined_gu", [False, True])
+def test_decoder_layer_without_attention_fuses_into_four_launches(be, combined_gu):
+    """RmsNorm -> {q, k, v}; o(q) -> Add; RmsNorm -> gate/up -> GatedAct -> down -> Add at m = 1.
+    The norms, the gated activation and the residual adds are absorbed by the decode GEMVs: four
+    launches instead of nine, every intermediate tensor still written, each stage within the
+    path's 1e-4 of the oracle fed with the device's own upstream tensors."""
+    from infr_amd import Add, GatedAct, GatedActFused, RmsNorm
+    H, KV, FF = 1024, 256, 2816
+    rng_w = lambda seed, n: synth_normal_f32(seed, n) * np.float32(0.1) + np.float32(1.0)
+    g, binds, bufs, host = Graph(), Bindings(), {}, {}
+
+    def tensor(name, shape, data=None, kind="input"):
+        t = (g.input if kind == "input" else g.output)(TensorDesc(shape, DType.F32))
+        n = int(np.prod(shape))
+        bufs[name] = be.upload_new(data) if data is not None else be.alloc(n * 4)
+        host[name] = data
+        binds.bind(t, bufs[name])
+        return t
+
+    def weight(name, dt, out_f, in_f, seed):
+        host[name] = synth_weight(dt, seed, out_f, in_f, 0.05)
+        t = g.weight(TensorDesc((out_f, in_f), dt))
+        binds.bind(t, be.upload_new(host[name]))
+        return t
+
+    x = tensor("x", (1, H))
+    n1w, n2w = tensor("n1w", (H,), rng_w(1, H)), tensor("n2w", (H,), rng_w(2, H))
+    h1, q, k, v, o = (tensor(nm, (1, d), kind="output") for nm, d in
+                      [("h1", H), ("q", H), ("k", KV), ("v", KV), ("o", H)])
+    h2, act, down = tensor("h2", (1, H), kind="output"), tensor("act", (1, FF), kind="output"), tensor("down", (1, H), kind="output")
+    wq, wk, wv = weight("wq", DType.Q4K, H, H, 11), weight("wk", DType.Q4K, KV, H, 12), weight("wv", DType.Q6K, KV, H, 13)
+    wo, wd = weight("wo", DType.Q4K, H, H, 14), weight("wd", DType.Q6K, H, FF, 15)
+    g.push(RmsNorm(x, n1w, h1, 1, H, 1e-6))
+    g.push(Linear(h1, wq, q, 1, H, H))
+    g.push(Linear(h1, wk, k, 1, H, KV))
+    g.push(Linear(h1, wv, v, 1, H, KV))
+    g.push(Linear(q, wo, o, 1, H, H))
+    g.push(Add(o, x, x, H))                      # residual in place: x = o + x
+    g.push(RmsNorm(x, n2w, h2, 1, H, 1e-6))
+    if combined_gu:
+        wgu = weight("wgu", DType.Q4K, 2 * FF, H, 16)
+        gu = tensor("gu", (1, 2 * FF), kind="output")
+        g.push(Linear(h2, wgu, gu, 1, H, 2 * FF))
+        g.push(GatedActFused(gu, act, 1, FF))
+    else:
+        wg, wu = weight("wg", DType.Q4K, FF, H, 16), weight("wu", DType.Q4K, FF, H, 17)
+        gt, up = tensor("gate", (1, FF), kind="output"), tensor("up", (1, FF), kind="output")
+        g.push(Linear(h2, wg, gt, 1, H, FF))
+        g.push(Linear(h2, wu, up, 1, H, FF))
+        g.push(GatedAct(gt, up, act, 1, FF))
+    g.push(Linear(act, wd, down, 1, FF, H))
+    g.push(Add(down, x, x, H))
+    plan = be.compile(g)
+    get = lambda nm, n: be.download(bufs[nm], np.empty(n, np.float32))
+    for rep in range(3):
+        x0 = synth_normal_f32(800 + rep, H)
+        be.upload(bufs["x"], x0)
+        be.execute(plan, binds)
+        # q/k (Q4_K) and v (Q6_K) are separate launches; o; gate/up; down -> 5 groups here
+        assert plan.launches() == 5, plan.launches()
+        d = {nm: get(nm, n) for nm, n in [("h1", H), ("q", H), ("k", KV), ("v", KV), ("o", H), ("h2", H),
+                                          ("act", FF), ("down", H), ("x", H)]}
+        assert _rel(d["h1"], orc.rms_norm(x0, host["n1w"], 1, H, 1e-6)) < 1e-6
+        assert _rel(d["q"], orc.linear(DType.Q4K, host["wq"], d["h1"], 1, H, H)) < 1e-4
+        assert _rel(d["k"], orc.linear(DType.Q4K, host["wk"], d["h1"], 1, H, KV)) < 1e-4
+        assert _rel(d["v"], orc.linear(DType.Q6K, host["wv"], d["h1"], 1, H, KV)) < 1e-4
+        o_want = orc.linear(DType.Q4K, host["wo"], d["q"], 1, H, H).ravel()
+        assert np.array_equal(bits(d["o"]), bits(o_want))      # no absorbed producer: bit-identical
+        x1 = orc.add(d["o"], x0)
+        assert _rel(d["h2"], orc.rms_norm(x1, host["n2w"], 1, H, 1e-6)) < 1e-6
+        if combined_gu:
+            gu_d = get("gu", 2 * FF)
+            assert _rel(gu_d, orc.linear(DType.Q4K, host["wgu"], d["h2"], 1, H, 2 * FF)) < 1e-4
+            act_want = orc.gated_act_fused(gu_d, 1, FF)
+        else:
+            g_d, u_d = get("gate", FF), get("up", FF)
+            assert _rel(g_d, orc.linear(DType.Q4K, host["wg"], d["h2"], 1, H, FF)) < 1e-4
+            assert _rel(u_d, orc.linear(DType.Q4K, host["wu"], d["h2"], 1, H, FF)) < 1e-4
+            act_want = orc.gated_act(g_d, u_d, 1, FF)
+        assert _rel(d["act"], act_want) < 1e-6
+        assert _rel(d["down"], orc.linear(DType.Q6K, host["wd"], d["act"], 1, FF, H)) < 1e-4
+        assert np.array_equal(bits(d["x"]), bits(orc.add(d["down"], x1)))   # both adds are exact
+
+
+def test_fusion_is_refused_when_it_would_reorder_a_dependency(be):
+    """A reader of the norm's output that is not a decode Linear, and a writer of the residual
+    between a Linear and its Add, both keep the ops separate; results follow program order."""
+    from infr_amd import Add, RmsNorm
+    H = 512
+    g, binds = Graph(), Bindings()
+    ids = {}
+    for nm in ("x", "w", "h", "h_copy", "y", "r", "zero"):
+        ids[nm] = g.input(TensorDesc((H,), DType.F32))
+    wq = g.weight(TensorDesc((H, H), DType.Q4K))
+    w_host = synth_weight(DType.Q4K, 5, H, H, 0.05)
+    x0, nw = synth_normal_f32(1, H), synth_normal_f32(2, H) + np.float32(1.0)
+    r0 = synth_normal_f32(3, H)
+    b = {"x": be.upload_new(x0), "w": be.upload_new(nw), "h": be.alloc(H * 4), "h_copy": be.alloc(H * 4),
+         "y": be.alloc(H * 4), "r": be.upload_new(r0), "zero": be.alloc(H * 4)}
+    for nm, buf in b.items():
+        binds.bind(ids[nm], buf)
+    binds.bind(wq, be.upload_new(w_host))
+    g.push(RmsNorm(ids["x"], ids["w"], ids["h"], 1, H, 1e-6))
+    g.push(Add(ids["h"], ids["zero"], ids["h_copy"], H))       # a non-Linear reader of h: no absorption
+    g.push(Linear(ids["h"], wq, ids["y"], 1, H, H))
+    g.push(Add(ids["r"], ids["r"], ids["r"], H))               # r *= 2 between the Linear and its Add
+    g.push(Add(ids["y"], ids["r"], ids["r"], H))               # must see the doubled r
+    plan = be.compile(g)
+    be.execute(plan, binds)
+    assert plan.launches() == 5
+    h = be.download(b["h"], np.empty(H, np.float32))
+    assert np.array_equal(bits(be.download(b["h_copy"], np.empty(H, np.float32))), bits(h))
+    y = be.download(b["y"], np.empty(H, np.float32))
+    assert np.array_equal(bits(y), bits(orc.linear(DType.Q4K, w_host, h, 1, H, H).ravel()))
+    want_r = orc.add(y, orc.add(r0, r0))
+    assert np.array_equal(bits(be.download(b["r"], np.empty(H, np.float32))), bits(want_r))
