@@ -1056,12 +1056,17 @@ int infr_hip_execute(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t* c
     // Validate and schedule before recording so a bad binding cannot leave a capture open.
     for (const auto& op : plan->ops) {
         const bool moe = op.kind == INFR_OP_MOE_FFN;
-        if (!bindings[op.x] || !bindings[op.dst] || (!moe && !bindings[op.weight]) ||
+        // elementwise ops name their second operand per kind; check_elementwise validates it
+        if (!bindings[op.x] || !bindings[op.dst] || (op.kind == INFR_OP_LINEAR && !bindings[op.weight]) ||
             (moe && (!bindings[op.router_x] || !bindings[op.router] || !bindings[op.gate_exps] ||
                      !bindings[op.up_exps] || !bindings[op.down_exps])))
             return fail(be, INFR_HIP_ERR_INVALID, "execute: unbound tensor");
     }
     if (int rc = schedule_plan(be, plan, bindings)) return rc;
+    // INFR_HIP_GRAPH=0: enqueue the launches directly on every execute instead of replaying a
+    // recorded graph (for comparing the two submission paths).
+    static const int env_graph = getenv("INFR_HIP_GRAPH") ? atoi(getenv("INFR_HIP_GRAPH")) : 1;
+    if (!env_graph) return enqueue_plan(be, plan, bindings);
     hipGraph_t graph = nullptr;
     HIP_TRY(be, hipStreamBeginCapture(be->stream, hipStreamCaptureModeThreadLocal));
     int rc = enqueue_plan(be, plan, bindings);
