@@ -97,7 +97,10 @@ bool is_quant(int dt) {
 }
 // Which activation quantizer infr-cpu's dispatch pairs with the weight dtype
 // (crates/infr-cpu/src/lib.rs:1043-1076): per-32 only for Q2_0 among the formats carried here.
-bool act_per32(int dt) { return dt == INFR_DTYPE_Q2_0; }
+// Per-32 activation quantizer: Q2_0 always, Q8_0 for rows that are not whole 256s (lib.rs:1037-1076).
+bool act_per32(int dt, size_t in_f) { return dt == INFR_DTYPE_Q2_0 || (dt == INFR_DTYPE_Q8_0 && in_f % 256 != 0); }
+// Row lengths a format accepts: whole weight blocks.
+size_t in_f_multiple(int dt) { return dt == INFR_DTYPE_Q2_0 ? 64 : (dt == INFR_DTYPE_Q8_0 ? 32 : 256); }
 
 // Activation scratch for m rows: the prefill kernels read tokens in groups of 32.
 static size_t act_scratch_elems(size_t m, size_t in_f) { return (m == 1 ? 1 : (m + 31) / 32 * 32) * in_f; }
@@ -240,7 +243,7 @@ int check_linear(infr_hip_t* be, int dtype, const infr_hip_buffer_t* w, size_t w
     int qpb = 0, bpb = 0;
     infr_block_layout(dtype, &qpb, &bpb);
     // The per-256 activation quantizer drops a sub-256 tail (quant.rs:28); reject, never truncate.
-    const size_t need = act_per32(dtype) ? 64 : 256;
+    const size_t need = in_f_multiple(dtype);
     if (in_f % need != 0)
         return fail(be, INFR_HIP_ERR_UNSUPPORTED,
                     "linear: in_f " + std::to_string(in_f) + " is not a multiple of " +
@@ -267,7 +270,7 @@ int enqueue_linear(infr_hip_t* be, int dtype, const LinearArgs& la, const float*
                    size_t m, size_t in_f, size_t out_f, const infr::IntStages& st) {
     bool ok;
     if (m == 1) {
-        infr::launch_quantize_q8(x, m, in_f, act_per32(dtype), be->act, be->stream);
+        infr::launch_quantize_q8(x, m, in_f, act_per32(dtype, in_f), be->act, be->stream);
         ok = infr::launch_gemv(dtype, la.wrows, la.bpr, be->act, y, in_f, out_f, st, be->stream);
     } else {
         // quantizes x into the scratch in the layout its kernel reads, then multiplies
@@ -668,7 +671,7 @@ int infr_hip_compile(infr_hip_t* be, const infr_hip_op_t* ops, size_t n_ops, inf
     for (const auto& op : p->ops) {
         if (op.kind == INFR_OP_LINEAR) {
             if (!is_quant(op.w_dtype) || op.m == 0 || op.in_f == 0 || op.out_f == 0 ||
-                op.in_f % (act_per32(op.w_dtype) ? 64 : 256) != 0 || op.w_numel % op.in_f != 0 ||
+                op.in_f % in_f_multiple(op.w_dtype) != 0 || op.w_numel % op.in_f != 0 ||
                 op.w_off % op.in_f != 0) {
                 delete p;
                 return fail(be, INFR_HIP_ERR_UNSUPPORTED, "compile: Linear op with unsupported dtype/shape");
@@ -1015,7 +1018,7 @@ static int enqueue_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t
                                         op.out_f, infr::IntStages{}))
                 return rc;
         } else if (st.m > 1) {
-            infr::launch_quantize_q8_group(plan->qtiles_dev + st.qtile_first, st.qtile_n, act_per32(st.dtype),
+            infr::launch_quantize_q8_group(plan->qtiles_dev + st.qtile_first, st.qtile_n, act_per32(st.dtype, st.in_f),
                                            be->act, be->stream);
             if (st.bp.kind == 1)
                 infr::launch_mmq_skinny_group(st.m, st.in_f, plan->btiles_dev + st.tile_first, st.bp, be->act,

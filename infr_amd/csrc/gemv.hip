@@ -280,7 +280,8 @@ bool launch_gemv(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, floa
     switch (dtype) {
     case 12: return launch_plain_fmt<FmtQ4K>(w, bpr, act, y, in_f, out_f, st, stream);
     case 14: return launch_plain_fmt<FmtQ6K>(w, bpr, act, y, in_f, out_f, st, stream);
-    case 8: return launch_plain_fmt<FmtQ8_0>(w, bpr, act, y, in_f, out_f, st, stream);
+    case 8:
+        return in_f % 256 == 0 ? launch_plain_fmt<FmtQ8_0>(w, bpr, act, y, in_f, out_f, st, stream) : launch_plain_fmt<FmtQ8_0_32>(w, bpr, act, y, in_f, out_f, st, stream);
     case 42: return launch_plain_fmt<FmtQ2_0>(w, bpr, act, y, in_f, out_f, st, stream);
     default: return false;
     }
@@ -342,7 +343,8 @@ bool launch_gemv_batch_group(int dtype, size_t m, size_t in_f, const BatchTile* 
     switch (dtype) {
     case 12: return launch_batch_group_fmt<FmtQ4K>(tiles_dev, plan, act, m, in_f, stream);
     case 14: return launch_batch_group_fmt<FmtQ6K>(tiles_dev, plan, act, m, in_f, stream);
-    case 8: return launch_batch_group_fmt<FmtQ8_0>(tiles_dev, plan, act, m, in_f, stream);
+    case 8:
+        return in_f % 256 == 0 ? launch_batch_group_fmt<FmtQ8_0>(tiles_dev, plan, act, m, in_f, stream) : launch_batch_group_fmt<FmtQ8_0_32>(tiles_dev, plan, act, m, in_f, stream);
     case 42: return launch_batch_group_fmt<FmtQ2_0>(tiles_dev, plan, act, m, in_f, stream);
     default: return false;
     }
@@ -423,7 +425,8 @@ bool launch_gemv_batch(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act
     switch (dtype) {
     case 12: return launch_batch_fmt<FmtQ4K>(w, bpr, act, y, m, in_f, out_f, st, stream);
     case 14: return launch_batch_fmt<FmtQ6K>(w, bpr, act, y, m, in_f, out_f, st, stream);
-    case 8: return launch_batch_fmt<FmtQ8_0>(w, bpr, act, y, m, in_f, out_f, st, stream);
+    case 8:
+        return in_f % 256 == 0 ? launch_batch_fmt<FmtQ8_0>(w, bpr, act, y, m, in_f, out_f, st, stream) : launch_batch_fmt<FmtQ8_0_32>(w, bpr, act, y, m, in_f, out_f, st, stream);
     case 42: return launch_batch_fmt<FmtQ2_0>(w, bpr, act, y, m, in_f, out_f, st, stream);
     default: return false;
     }
@@ -435,6 +438,7 @@ template <typename F> static int max_waves_per_wg(int steps);
 template <> int max_waves_per_wg<FmtQ4K>(int steps) { return steps <= 3 ? 16 : 8; }
 template <> int max_waves_per_wg<FmtQ6K>(int steps) { return steps <= 1 ? 16 : 8; }
 template <> int max_waves_per_wg<FmtQ8_0>(int steps) { return steps <= 4 ? 16 : 8; }
+template <> int max_waves_per_wg<FmtQ8_0_32>(int steps) { return steps <= 4 ? 16 : 8; }
 template <> int max_waves_per_wg<FmtQ2_0>(int steps) { return steps <= 3 ? 16 : 8; }
 
 // Workgroups of the fused kernel that one compute unit holds at once (registers, LDS, wave slots),
@@ -545,7 +549,8 @@ bool plan_gemv_group(int dtype, size_t in_f, const GemvOpDesc* ops, int n, GemvG
     switch (dtype) {
     case 12: return plan_group_fmt<FmtQ4K>(in_f, ops, n, plan);
     case 14: return plan_group_fmt<FmtQ6K>(in_f, ops, n, plan);
-    case 8: return plan_group_fmt<FmtQ8_0>(in_f, ops, n, plan);
+    case 8:
+        return in_f % 256 == 0 ? plan_group_fmt<FmtQ8_0>(in_f, ops, n, plan) : plan_group_fmt<FmtQ8_0_32>(in_f, ops, n, plan);
     case 42: return plan_group_fmt<FmtQ2_0>(in_f, ops, n, plan);
     default: return false;
     }
@@ -614,7 +619,8 @@ bool launch_gemv_fused(int dtype, size_t in_f, const GemvOpDesc* ops, int n, con
     switch (dtype) {
     case 12: return launch_fused_fmt<FmtQ4K>(in_f, ops[0], tiles_dev, plan, stream);
     case 14: return launch_fused_fmt<FmtQ6K>(in_f, ops[0], tiles_dev, plan, stream);
-    case 8: return launch_fused_fmt<FmtQ8_0>(in_f, ops[0], tiles_dev, plan, stream);
+    case 8:
+        return in_f % 256 == 0 ? launch_fused_fmt<FmtQ8_0>(in_f, ops[0], tiles_dev, plan, stream) : launch_fused_fmt<FmtQ8_0_32>(in_f, ops[0], tiles_dev, plan, stream);
     case 42: return launch_fused_fmt<FmtQ2_0>(in_f, ops[0], tiles_dev, plan, stream);
     default: return false;
     }

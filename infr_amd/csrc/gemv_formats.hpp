@@ -215,10 +215,13 @@ struct FmtQ6K {
 
 // ───────────────────────────────────── Q8_0 ─────────────────────────────────────
 // Lane l owns 32-weight block t*64 + l of the row: 34 B = f16 scale + 32 int8, 2-byte aligned.
-// 64 blocks (2048 weights, 2176 B) per wave step; the activation scale is per 256 (8 lanes).
-struct FmtQ8_0 {
+// 64 blocks (2048 weights, 2176 B) per wave step. Rows of whole 256s take the per-256 activation
+// (scale shared by 8 lanes, kernels.rs:1170-1187); rows that are a multiple of 32 only take the
+// per-32 activation, one scale per block (P32; kernels.rs:4972-4991, lib.rs:1037-1042).
+template <bool P32>
+struct FmtQ8_0T {
     static constexpr int kElemsPerStep = 2048;
-    static constexpr bool kPer32 = false;
+    static constexpr bool kPer32 = P32;
     static constexpr bool kOrdered = false;
     static constexpr int kBlockBytes = 34, kBlockElems = 32;
     struct Row {
@@ -265,7 +268,7 @@ struct FmtQ8_0 {
             const v4i v1 = *reinterpret_cast<const v4i*>(s.qs + (size_t)wb * 32 + 16);
             a.xa[0] = v0.x; a.xa[1] = v0.y; a.xa[2] = v0.z; a.xa[3] = v0.w;
             a.xa[4] = v1.x; a.xa[5] = v1.y; a.xa[6] = v1.z; a.xa[7] = v1.w;
-            a.dact = s.d[wb >> 3];
+            a.dact = s.d[P32 ? wb : wb >> 3];
         } else {
 #pragma unroll
             for (int k = 0; k < 8; ++k) a.xa[k] = 0;
@@ -285,10 +288,12 @@ struct FmtQ8_0 {
         ip = dot4(r.qb.z, a.xa[6], ip);
         ip = dot4(r.qb.w, a.xa[7], ip);
         if (STAGES && ok) st.a[row_units + t * 64 + lane] = ip;
-        // sumf += d8 * d_w * iprod as f32
+        // sumf += d8 * d_w * iprod as f32   (per-32: d_w * d_x[b] * iprod - the same product)
         return a.dact * f16_bits_to_f32(r.d) * (float)ip;
     }
 };
+using FmtQ8_0 = FmtQ8_0T<false>;
+using FmtQ8_0_32 = FmtQ8_0T<true>;
 
 // ───────────────────────────────────── Q2_0 ─────────────────────────────────────
 // Lane l owns 64-weight block t*64 + l: 18 B = f16 scale + 16 bytes of 2-bit codes, 2-byte

@@ -338,6 +338,24 @@ float orc_vec_dot_q6k(const uint8_t *row, const int8_t *qs8, const float *d8, si
     return sumf;
 }
 
+/* crates/infr-cpu/src/kernels.rs:4972-4991 (vec_dot_q8_0_32_batch_scalar, one activation row):
+ * Q8_0 rows whose length is a multiple of 32 but not of 256, against the per-32 activation. */
+float orc_vec_dot_q8_0_32(const uint8_t *row, const int8_t *qs, const float *d32, size_t in_f,
+                          int32_t *iprod_out) {
+    size_t nb = in_f / 32;
+    float sumf = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * 34;
+        float d_w = orc_rdf16(blk);
+        const int8_t *qw = (const int8_t *)(blk + 2);
+        int32_t iprod = 0;
+        for (int i = 0; i < 32; i++) iprod += (int32_t)qw[i] * (int32_t)qs[b * 32 + i];
+        if (iprod_out) iprod_out[b] = iprod;
+        sumf += d_w * d32[b] * (float)iprod; /* (d_arr[b] * q8.d[b]) * (iprod as f32) */
+    }
+    return sumf;
+}
+
 /* crates/infr-cpu/src/kernels.rs:1170-1187 (vec_dot_q8_0_scalar): weight blocks of 32 against the
  * per-256 activation scale. */
 float orc_vec_dot_q8_0(const uint8_t *row, const int8_t *qs8, const float *d8, size_t in_f,
@@ -477,8 +495,10 @@ typedef struct {
     int32_t *bsums16; /* per 16 (Q8 only) */
 } acts_t;
 
-static int is_q8_super(int dtype) {
-    return dtype == ORC_Q4_K || dtype == ORC_Q6_K || dtype == ORC_Q8_0;
+/* lib.rs:1037-1062: per-256 `Q8` for the 256-block formats and for Q8_0 rows of whole 256s;
+ * a Q8_0 row that is a multiple of 32 only takes the per-32 `Q8x32` (q8_0_blk32). */
+static int is_q8_super(int dtype, size_t in_f) {
+    return dtype == ORC_Q4_K || dtype == ORC_Q6_K || (dtype == ORC_Q8_0 && in_f % 256 == 0);
 }
 
 static void acts_free(acts_t *a) {
@@ -493,7 +513,7 @@ static void acts_free(acts_t *a) {
 static int acts_build(int dtype, const float *x, size_t m, size_t in_f, acts_t *a) {
     memset(a, 0, sizeof *a);
     a->qs = (int8_t *)malloc(m * in_f);
-    if (is_q8_super(dtype)) {
+    if (is_q8_super(dtype, in_f)) {
         size_t nb = in_f / 256;
         a->d = (float *)malloc(sizeof(float) * m * nb);
         a->bsums = (int32_t *)malloc(sizeof(int32_t) * m * nb * 8);
@@ -527,6 +547,8 @@ static float row_dot(int dtype, const uint8_t *row, const acts_t *a, size_t r, s
         return orc_vec_dot_q6k(row, a->qs + r * in_f, a->d + r * nb, in_f, ia);
     }
     case ORC_Q8_0: {
+        if (in_f % 256 != 0)
+            return orc_vec_dot_q8_0_32(row, a->qs + r * in_f, a->d + r * (in_f / 32), in_f, ia);
         size_t nb = in_f / 256;
         return orc_vec_dot_q8_0(row, a->qs + r * in_f, a->d + r * nb, in_f, ia);
     }
@@ -541,12 +563,13 @@ static float row_dot(int dtype, const uint8_t *row, const acts_t *a, size_t r, s
 
 static int linear_shape_ok(int dtype, size_t in_f) {
     /* The restatement carries the arms the four formats take when in_f is block-aligned:
-     * Q4K/Q6K: 256-element weight blocks; Q8_0 with in_f % 256 != 0 would go to the per-32 kernel
-     * (lib.rs:1037-1042) which is not restated; Q2_0 needs in_f % 64 == 0 (lib.rs:1406). */
+     * Q4K/Q6K: 256-element weight blocks; Q8_0: whole 32-blocks, per-256 activations when in_f is
+     * a multiple of 256 and the per-32 kernel otherwise (lib.rs:1037-1042); Q2_0 needs
+     * in_f % 64 == 0 (lib.rs:1406). */
     switch (dtype) {
     case ORC_Q4_K:
-    case ORC_Q6_K:
-    case ORC_Q8_0: return in_f % 256 == 0;
+    case ORC_Q6_K: return in_f % 256 == 0;
+    case ORC_Q8_0: return in_f % 32 == 0;
     case ORC_Q2_0: return in_f % 64 == 0;
     case ORC_F32: return 1;
     default: return 0;

@@ -87,6 +87,9 @@ float orc_vec_dot_q6k(const uint8_t *row, const int8_t *qs, const float *d, size
                       int32_t *isum_out);
 float orc_vec_dot_q8_0(const uint8_t *row, const int8_t *qs, const float *d, size_t in_f,
                        int32_t *iprod_out);
+/* kernels.rs:4972-4991 — Q8_0 against the per-32 activation (in_f % 256 != 0). */
+float orc_vec_dot_q8_0_32(const uint8_t *row, const int8_t *qs, const float *d32, size_t in_f,
+                          int32_t *iprod_out);
 float orc_vec_dot_q2_0(const uint8_t *row, const int8_t *qs, const float *d, const int32_t *bsum,
                        size_t in_f, int32_t *iprod_out);
 

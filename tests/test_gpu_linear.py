@@ -235,3 +235,17 @@ def test_ternary_output_head_rows_vs_oracle(be):
     y = run_linear(be, DType.Q2_0, w, x, 1, in_f, out_f)
     for row0 in (0, 77777, out_f - 64):
         gate(y[:, row0:row0 + 64], _oracle_rows(DType.Q2_0, w, x, 1, in_f, out_f, row0, 64))
+
+
+# ───────────── Q8_0 rows that are whole 32s but not whole 256s: the per-32 arm ─────────────
+
+@pytest.mark.parametrize("m", [1, 3, 8, 20])
+@pytest.mark.parametrize("in_f,out_f", [(96, 40), (1152, 300), (2080, 64), (4128, 33)])
+def test_q8_0_per32_rows_vs_oracle(be, m, in_f, out_f):
+    w = synth_weight(DType.Q8_0, 70 + in_f, out_f, in_f)
+    x = synth_normal_f32(71 + m, m * in_f)
+    y = run_linear(be, DType.Q8_0, w, x, m, in_f, out_f)
+    gate(y, orc.linear(DType.Q8_0, w, x, m, in_f, out_f))
+    a, _ = be.linear_int_stages(DType.Q8_0, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
+    oa, _ = orc.linear_int_stages(DType.Q8_0, w, x, m, in_f, out_f)
+    assert np.array_equal(a, oa)

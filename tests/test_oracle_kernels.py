@@ -292,9 +292,14 @@ def test_linear_int_stages_agree_with_row_kernels():
 
 
 def test_linear_rejects_ragged_in_f():
-    w = orc.synth_weight(orc.Q8_0, 96 * 4, 1)
+    # a row must be a whole number of weight blocks: Q4_K needs 256s (a per-256 quantizer would
+    # silently drop the tail, quant.rs:28), Q2_0 whole 64s
+    w = orc.synth_weight(orc.Q4_K, 256 * 4, 1)
     with pytest.raises(ValueError):
-        orc.linear(orc.Q8_0, w, np.zeros(96, np.float32), 1, 96, 4)   # per-32 Q8_0 arm is not restated
+        orc.linear(orc.Q4_K, w, np.zeros(128, np.float32), 1, 128, 8)
+    w = orc.synth_weight(orc.Q2_0, 64 * 4, 1)
+    with pytest.raises(ValueError):
+        orc.linear(orc.Q2_0, w, np.zeros(32, np.float32), 1, 32, 8)
 
 
 # ───────────── the committed known-answer fixture, through Op::Linear ─────────────
@@ -310,9 +315,36 @@ def _golden():
 def test_golden_known_answers_through_linear(case):
     row = np.frombuffer(b"".join(bytes.fromhex(h) * n for h, n in case["parts"]), np.uint8)
     w = np.tile(row, 3)
-    y = orc.linear(case["dtype"], w, np.tile(X127, 2), 2, case["in_f"], 3)
+    x = np.full(2 * case["in_f"], 127.0, np.float32)
+    y = orc.linear(case["dtype"], w, x, 2, case["in_f"], 3)
     assert np.all(y == np.float32(case["y"]))
-    a, b = orc.linear_int_stages(case["dtype"], w, np.tile(X127, 2), 2, case["in_f"], 3)
+    a, b = orc.linear_int_stages(case["dtype"], w, x, 2, case["in_f"], 3)
     assert np.array_equal(np.asarray(a).reshape(6, -1), np.tile(np.array(case["int_a"], np.int32), (6, 1)))
     if "int_b" in case:
         assert np.array_equal(np.asarray(b).reshape(6, -1), np.tile(np.array(case["int_b"], np.int32), (6, 1)))
+
+
+# ───────────── Q8_0 rows that are a multiple of 32 only: the per-32 arm ─────────────
+
+@pytest.mark.parametrize("in_f", [32, 96, 1152])
+def test_q8_0_per32_arm_against_brute_force_and_dequant(in_f):
+    out_f = 5
+    w = orc.synth_weight(orc.Q8_0, in_f * out_f, 0x231)
+    x = orc.gen_f32(in_f, 7)
+    y = orc.linear(orc.Q8_0, w, x, 1, in_f, out_f).ravel()
+    ia, _ = orc.linear_int_stages(orc.Q8_0, w, x, 1, in_f, out_f)
+    q = orc.quantize_q8_32(x)
+    blocks = w.reshape(out_f, in_f // 32, 34)
+    for o in range(out_f):
+        acc = np.float32(0.0)
+        for b in range(in_f // 32):
+            qw = blocks[o, b, 2:].view(np.int8).astype(np.int64)
+            ip = int(qw @ q.qs[b * 32:(b + 1) * 32].astype(np.int64))
+            assert ia.reshape(out_f, -1)[o, b] == ip
+            d_w = np.float32(orc.f16_bits_to_f32(int(blocks[o, b, 0]) | int(blocks[o, b, 1]) << 8))
+            acc = np.float32(acc + np.float32(np.float32(d_w * q.d[b]) * np.float32(ip)))
+        assert y[o] == acc
+    # and against the decoded weights in f64, at the reference's production bound
+    wf = np.concatenate([orc.dequant_block(orc.Q8_0, blocks[o].ravel()) for o in range(out_f)]).reshape(out_f, in_f)
+    ref = wf.astype(np.float64) @ x.astype(np.float64)
+    assert np.abs(y - ref).max() <= 2e-2 * np.abs(ref).max()
