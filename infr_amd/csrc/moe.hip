@@ -8,9 +8,9 @@
 //   select   softmax with max-subtraction, probabilities summed in index order, stable top-n_used
 //            (ties to the lower expert index), w = p / max(sum_sel p, 1e-20) * scale  (lib.rs:2421-2543)
 //   rows == 1   the CPU multiplies DECODED f32 weights with the UNQUANTIZED activation
-//            (ActsKind::Raw, moe.rs:42-53,142-173): gate/up rows are applied to f32 x in registers
-//            (sc * sum(code*x) + mn * sum(x) per 32 weights, all f32), SiLU fused; the down kernel
-//            does likewise and adds the experts in rank order
+//            (ActsKind::Raw, moe.rs:42-53,142-173): gate/up rows of Q4_K / Q6_K / Q8_0 banks are
+//            applied to f32 x in registers (sc * sum(code*x) + mn * sum(x) per scale group, all
+//            f32), SiLU fused; the down kernel does likewise and adds the experts in rank order
 //   rows >= 2   int8 path: x rows quantized per 256 once, id-gathered Q4_K/Q6_K/Q8_0 GEMVs per
 //            (row, expert) pair (the decode GEMV body, bit-identical to the CPU's batch kernels),
 //            SiLU + re-quantization, id-gathered down GEMV, rank-ordered accumulate
@@ -218,93 +218,202 @@ __global__ __launch_bounds__(256) void moe_router_kernel(
     if (tid == 0) *tickets = 0;
 }
 
-// ───────────────────────────── rows == 1: f32 (ActsKind::Raw) path, Q4_K banks ─────────────────────────────
-// Lane mapping: 4 lanes per 256-block (nibble pair p = lane % 4, 64 weights), S = 4 * nb lanes per
-// weight row, 64 / S rows per wave step. A lane keeps its 64 activation floats in registers.
-// The CPU decodes w = sc*code + mn to f32 and runs an f32 dot; here the same sum is factored per
-// 32 weights as sc * sum(code * x) + mn * sum(x) (one conversion and one FMA per weight), which
-// moves the result by f32 rounding only - orders of magnitude inside the 1e-4 relative bound
-// this path is held to.
+// ───────────────────────────── rows == 1: f32 (ActsKind::Raw) path ─────────────────────────────
+// A lane owns 64 consecutive-or-strided weights of a row ("unit" u of the row's in_f / 64) and
+// keeps the matching 64 activation floats in registers; S = in_f / 64 lanes cover a weight row and
+// 64 / S rows run per wave step. The CPU decodes each weight to f32 (dequant_block) and runs an
+// f32 dot; here the same sum is factored per scale group as sc * sum(code * x) + mn * sum(x)
+// (one conversion and one FMA per weight), which moves the result by f32 rounding only - orders
+// of magnitude inside the 1e-4 relative bound this path is held to. One policy per bank format:
+//   Row / load_row(r, row pointer, u, ok)      the lane's bytes of a weight row
+//   X   / load_x(x, activation row, u, ok)     its activation floats and the group sums it needs
+//   partial(r, x, u)                           sum over the lane's 64 weights of w * x
 
-struct Q4kF32Row {
-    v4i hdr, qa, qb;
+// Q4_K: unit u = (block u/4, nibble pair u%4): sub-block 2p in the low nibbles of the pair's
+// 32 bytes, 2p+1 in the high ones. w = (d*sc)*code - dmin*m.
+struct RawQ4K {
+    static constexpr int kBlockBytes = 144;
+    struct Row {
+        v4i hdr, qa, qb;
+    };
+    struct X {
+        float x[64];
+        float sum_lo, sum_hi;  // sum of x[0..32), x[32..64)
+    };
+    __device__ static void load_row(Row& r, const uint8_t* rowp, int u, bool ok) {
+        if (ok) {
+            const uint8_t* blk = rowp + (size_t)(u >> 2) * 144;
+            const int p = u & 3;
+            r.hdr = load16(blk);
+            r.qa = load16(blk + 16 + p * 32);
+            r.qb = load16(blk + 32 + p * 32);
+        } else {
+            r.hdr = r.qa = r.qb = v4i{0, 0, 0, 0};
+        }
+    }
+    __device__ static void load_x(X& a, const float* xrow, int u, bool ok) {
+        const float* src = xrow + (size_t)u * 64;
+        float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (ok) v = *reinterpret_cast<const v4f*>(src + 4 * k);
+            a.x[4 * k + 0] = v.x; a.x[4 * k + 1] = v.y; a.x[4 * k + 2] = v.z; a.x[4 * k + 3] = v.w;
+            if (k < 8) { s0 += v.x + v.y; s1 += v.z + v.w; } else { s2 += v.x + v.y; s3 += v.z + v.w; }
+        }
+        a.sum_lo = s0 + s1;
+        a.sum_hi = s2 + s3;
+    }
+    __device__ static float partial(const Row& r, const X& a, int u) {
+        const int p = u & 3;
+        uint32_t sc8[2], mn8[2];
+        k4_all((uint32_t)r.hdr.y, (uint32_t)r.hdr.z, (uint32_t)r.hdr.w, sc8, mn8);
+        const uint32_t scw = (p & 2) ? sc8[1] : sc8[0];
+        const uint32_t mnw = (p & 2) ? mn8[1] : mn8[0];
+        const int sh = (p & 1) * 16;
+        const float d = f16_bits_to_f32((uint32_t)r.hdr.x & 0xFFFFu);
+        const float dmin = f16_bits_to_f32((uint32_t)r.hdr.x >> 16);
+        const float fs_lo = d * (float)(int)((scw >> sh) & 0xFF), fs_hi = d * (float)(int)((scw >> (sh + 8)) & 0xFF);
+        const float fm_lo = dmin * (float)(int)((mnw >> sh) & 0xFF), fm_hi = dmin * (float)(int)((mnw >> (sh + 8)) & 0xFF);
+        const int wq[8] = {r.qa.x, r.qa.y, r.qa.z, r.qa.w, r.qb.x, r.qb.y, r.qb.z, r.qb.w};
+        float lo0 = 0.0f, lo1 = 0.0f, hi0 = 0.0f, hi1 = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const uint32_t w = (uint32_t)wq[k];
+            const uint32_t l = w & 0x0F0F0F0Fu, h = (w >> 4) & 0x0F0F0F0Fu;
+            lo0 = __builtin_fmaf((float)(l & 0xFF), a.x[4 * k + 0], lo0);
+            lo1 = __builtin_fmaf((float)((l >> 8) & 0xFF), a.x[4 * k + 1], lo1);
+            lo0 = __builtin_fmaf((float)((l >> 16) & 0xFF), a.x[4 * k + 2], lo0);
+            lo1 = __builtin_fmaf((float)(l >> 24), a.x[4 * k + 3], lo1);
+            hi0 = __builtin_fmaf((float)(h & 0xFF), a.x[32 + 4 * k + 0], hi0);
+            hi1 = __builtin_fmaf((float)((h >> 8) & 0xFF), a.x[32 + 4 * k + 1], hi1);
+            hi0 = __builtin_fmaf((float)((h >> 16) & 0xFF), a.x[32 + 4 * k + 2], hi0);
+            hi1 = __builtin_fmaf((float)(h >> 24), a.x[32 + 4 * k + 3], hi1);
+        }
+        return (fs_lo * (lo0 + lo1) - fm_lo * a.sum_lo) + (fs_hi * (hi0 + hi1) - fm_hi * a.sum_hi);
+    }
 };
 
-struct Q4kF32X {
-    float x[64];
-    float sum_lo, sum_hi;  // sum of x[0..32), x[32..64)
+// Q6_K: unit u = (block u/4, half h = (u%4)/2, c = u%2) as in the decode GEMV: the lane decodes
+// the four 16-element groups {l, l+32, l+64, l+96}, l in [16c, 16c+16), of its 128-element half;
+// group k has scale index h*8 + c + 2k. w = d * sc * (q - 32).
+struct RawQ6K {
+    static constexpr int kBlockBytes = 210;
+    typedef FmtQ6K::Row Row;
+    struct X {
+        float x[64];    // x[16k + j] = element 128h + 32k + 16c + j of the block
+        float gsum[4];  // sum over each group's 16 activations
+    };
+    __device__ static void load_row(Row& r, const uint8_t* rowp, int u, bool ok) {
+        FmtQ6K::load_row(r, rowp, 0, u, ok);
+    }
+    __device__ static void load_x(X& a, const float* xrow, int u, bool ok) {
+        const int h = (u >> 1) & 1, c = u & 1;
+        const float* src = xrow + (size_t)(u >> 2) * 256 + h * 128 + c * 16;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
+                if (ok) v = *reinterpret_cast<const v4f*>(src + 32 * k + 4 * q);
+                a.x[16 * k + 4 * q + 0] = v.x; a.x[16 * k + 4 * q + 1] = v.y;
+                a.x[16 * k + 4 * q + 2] = v.z; a.x[16 * k + 4 * q + 3] = v.w;
+                s0 += v.x + v.y;
+                s1 += v.z + v.w;
+            }
+            a.gsum[k] = s0 + s1;
+        }
+    }
+    __device__ static float partial(const Row& r, const X& a, int u) {
+        const int c = u & 1;
+        const uint32_t m4 = 0x0F0F0F0Fu, m2 = 0x30303030u;
+        const int la[4] = {r.qla.x, r.qla.y, r.qla.z, r.qla.w};
+        const int lb[4] = {r.qlb.x, r.qlb.y, r.qlb.z, r.qlb.w};
+        const int hh[4] = {r.qh.x, r.qh.y, r.qh.z, r.qh.w};
+        float dotq[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t lo = (uint32_t)la[j], hi = (uint32_t)lb[j], hb = (uint32_t)hh[j];
+            const uint32_t w[4] = {(lo & m4) | ((hb << 4) & m2), (hi & m4) | ((hb << 2) & m2),
+                                   ((lo >> 4) & m4) | (hb & m2), ((hi >> 4) & m4) | ((hb >> 2) & m2)};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                dotq[k] = __builtin_fmaf((float)(w[k] & 0xFF), a.x[16 * k + 4 * j + 0], dotq[k]);
+                dotq[k] = __builtin_fmaf((float)((w[k] >> 8) & 0xFF), a.x[16 * k + 4 * j + 1], dotq[k]);
+                dotq[k] = __builtin_fmaf((float)((w[k] >> 16) & 0xFF), a.x[16 * k + 4 * j + 2], dotq[k]);
+                dotq[k] = __builtin_fmaf((float)(w[k] >> 24), a.x[16 * k + 4 * j + 3], dotq[k]);
+            }
+        }
+        const uint32_t lo = (uint32_t)r.sc.x >> (8 * c), hi = (uint32_t)r.sc.y >> (8 * c);
+        const float sc[4] = {(float)(int)(int8_t)(lo & 0xFF), (float)(int)(int8_t)((lo >> 16) & 0xFF),
+                             (float)(int)(int8_t)(hi & 0xFF), (float)(int)(int8_t)((hi >> 16) & 0xFF)};
+        const float d = f16_bits_to_f32(r.d);
+        float acc = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) acc += (d * sc[k]) * (dotq[k] - 32.0f * a.gsum[k]);
+        return acc;
+    }
 };
 
-__device__ __forceinline__ void q4k_f32_load_x(Q4kF32X& a, const float* src, bool ok) {
-    float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+// Q8_0: unit u = the two 32-blocks 2u, 2u+1. w = d * q.
+struct RawQ8_0 {
+    static constexpr int kBlockBytes = 8 * 34;  // per 256 elements
+    struct Row {
+        FmtQ8_0::Row b0, b1;
+    };
+    struct X {
+        float x[64];
+    };
+    __device__ static void load_row(Row& r, const uint8_t* rowp, int u, bool ok) {
+        FmtQ8_0::load_row(r.b0, rowp, 0, 2 * u, ok);
+        FmtQ8_0::load_row(r.b1, rowp, 0, 2 * u + 1, ok);
+    }
+    __device__ static void load_x(X& a, const float* xrow, int u, bool ok) {
+        const float* src = xrow + (size_t)u * 64;
 #pragma unroll
-    for (int k = 0; k < 16; ++k) {
-        v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (ok) v = *reinterpret_cast<const v4f*>(src + 4 * k);
-        a.x[4 * k + 0] = v.x; a.x[4 * k + 1] = v.y; a.x[4 * k + 2] = v.z; a.x[4 * k + 3] = v.w;
-        if (k < 8) { s0 += v.x + v.y; s1 += v.z + v.w; } else { s2 += v.x + v.y; s3 += v.z + v.w; }
+        for (int k = 0; k < 16; ++k) {
+            v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (ok) v = *reinterpret_cast<const v4f*>(src + 4 * k);
+            a.x[4 * k + 0] = v.x; a.x[4 * k + 1] = v.y; a.x[4 * k + 2] = v.z; a.x[4 * k + 3] = v.w;
+        }
     }
-    a.sum_lo = s0 + s1;
-    a.sum_hi = s2 + s3;
-}
-
-__device__ __forceinline__ float q4k_f32_partial(const Q4kF32Row& r, const Q4kF32X& a, int p) {
-    uint32_t sc8[2], mn8[2];
-    k4_all((uint32_t)r.hdr.y, (uint32_t)r.hdr.z, (uint32_t)r.hdr.w, sc8, mn8);
-    const uint32_t scw = (p & 2) ? sc8[1] : sc8[0];
-    const uint32_t mnw = (p & 2) ? mn8[1] : mn8[0];
-    const int sh = (p & 1) * 16;
-    const float d = f16_bits_to_f32((uint32_t)r.hdr.x & 0xFFFFu);
-    const float dmin = f16_bits_to_f32((uint32_t)r.hdr.x >> 16);
-    const float fs_lo = d * (float)(int)((scw >> sh) & 0xFF), fs_hi = d * (float)(int)((scw >> (sh + 8)) & 0xFF);
-    const float fm_lo = dmin * (float)(int)((mnw >> sh) & 0xFF), fm_hi = dmin * (float)(int)((mnw >> (sh + 8)) & 0xFF);
-    const int wq[8] = {r.qa.x, r.qa.y, r.qa.z, r.qa.w, r.qb.x, r.qb.y, r.qb.z, r.qb.w};
-    float lo0 = 0.0f, lo1 = 0.0f, hi0 = 0.0f, hi1 = 0.0f;
+    __device__ static float block_dot(const FmtQ8_0::Row& b, const float* x) {
+        const int q[8] = {b.qa.x, b.qa.y, b.qa.z, b.qa.w, b.qb.x, b.qb.y, b.qb.z, b.qb.w};
+        float s0 = 0.0f, s1 = 0.0f;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
-        const uint32_t w = (uint32_t)wq[k];
-        const uint32_t l = w & 0x0F0F0F0Fu, h = (w >> 4) & 0x0F0F0F0Fu;
-        lo0 = __builtin_fmaf((float)(l & 0xFF), a.x[4 * k + 0], lo0);
-        lo1 = __builtin_fmaf((float)((l >> 8) & 0xFF), a.x[4 * k + 1], lo1);
-        lo0 = __builtin_fmaf((float)((l >> 16) & 0xFF), a.x[4 * k + 2], lo0);
-        lo1 = __builtin_fmaf((float)(l >> 24), a.x[4 * k + 3], lo1);
-        hi0 = __builtin_fmaf((float)(h & 0xFF), a.x[32 + 4 * k + 0], hi0);
-        hi1 = __builtin_fmaf((float)((h >> 8) & 0xFF), a.x[32 + 4 * k + 1], hi1);
-        hi0 = __builtin_fmaf((float)((h >> 16) & 0xFF), a.x[32 + 4 * k + 2], hi0);
-        hi1 = __builtin_fmaf((float)(h >> 24), a.x[32 + 4 * k + 3], hi1);
+        for (int k = 0; k < 8; ++k) {
+            s0 = __builtin_fmaf((float)(int)(int8_t)(q[k] & 0xFF), x[4 * k + 0], s0);
+            s1 = __builtin_fmaf((float)(int)(int8_t)((q[k] >> 8) & 0xFF), x[4 * k + 1], s1);
+            s0 = __builtin_fmaf((float)(int)(int8_t)((q[k] >> 16) & 0xFF), x[4 * k + 2], s0);
+            s1 = __builtin_fmaf((float)(q[k] >> 24), x[4 * k + 3], s1);
+        }
+        return f16_bits_to_f32(b.d) * (s0 + s1);
     }
-    return (fs_lo * (lo0 + lo1) - fm_lo * a.sum_lo) + (fs_hi * (hi0 + hi1) - fm_hi * a.sum_hi);
-}
-
-__device__ __forceinline__ void q4k_f32_load(Q4kF32Row& r, const uint8_t* rowp, int b, int p, bool ok) {
-    if (ok) {
-        const uint8_t* blk = rowp + (size_t)b * 144;
-        r.hdr = load16(blk);
-        r.qa = load16(blk + 16 + p * 32);
-        r.qb = load16(blk + 32 + p * 32);
-    } else {
-        r.hdr = r.qa = r.qb = v4i{0, 0, 0, 0};
+    __device__ static float partial(const Row& r, const X& a, int) {
+        return block_dot(r.b0, a.x) + block_dot(r.b1, a.x + 32);
     }
-}
+};
 
-// Sum over the S = 4*nb lanes of a row segment; every lane of the segment gets the total.
-__device__ __forceinline__ float seg_sum(float v, int seg_base, int nb) {
+// Sum over the S lanes (a multiple of 4) of a row segment; every lane of the segment gets the total.
+__device__ __forceinline__ float seg_sum(float v, int seg_base, int quads) {
     v += __builtin_bit_cast(float, quad_xor1(__builtin_bit_cast(int, v)));
     v += __builtin_bit_cast(float, quad_xor2(__builtin_bit_cast(int, v)));
     float s = 0.0f;
-    for (int i = 0; i < nb; ++i) s += __shfl(v, seg_base + 4 * i, kWave);
+    for (int i = 0; i < quads; ++i) s += __shfl(v, seg_base + 4 * i, kWave);
     return s;
 }
 
 // gate/up at one token: act[slot][o] = silu(gate_e[o] . x) * (up_e[o] . x), e = ids[slot].
 // A wave takes steps_per_wave consecutive row steps and keeps the next step's rows in flight.
-__global__ __launch_bounds__(256) void moe_gate_up_f32_q4k_kernel(
+template <typename P>
+__global__ __launch_bounds__(256) void moe_gate_up_f32_kernel(
     const uint8_t* __restrict__ gate, const uint8_t* __restrict__ up, size_t gate_stride,
     size_t up_stride, const int32_t* __restrict__ ids, const float* __restrict__ x,
     float* __restrict__ act, int ne, int nff, int steps_per_wave) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int nb = ne / 256, S = 4 * nb, rps = 64 / S;  // rows per wave step
-    const int seg = lane / S, within = lane % S, b = within >> 2, p = within & 3;
+    const int S = ne / 64, rps = 64 / S;  // lanes per weight row, rows per wave step
+    const int seg = lane / S, u = lane % S;
     const bool lane_ok = seg < rps;
     const int slot = blockIdx.y;
     const int steps_total = (nff + rps - 1) / rps;
@@ -312,31 +421,31 @@ __global__ __launch_bounds__(256) void moe_gate_up_f32_q4k_kernel(
     if (st0 >= steps_total) return;
     const int st_end = min(st0 + steps_per_wave, steps_total);
     const int e = ids[slot];
-    const size_t bpr = (size_t)nb * 144;
+    const size_t bpr = (size_t)(ne / 256) * P::kBlockBytes;
     const uint8_t* gw = gate + (size_t)e * gate_stride;
     const uint8_t* uw = up + (size_t)e * up_stride;
-    Q4kF32Row g, u;
+    typename P::Row g, up_r;
     {
         const int o = st0 * rps + seg;
         const bool ok = lane_ok && o < nff;
-        q4k_f32_load(g, gw + (size_t)(ok ? o : 0) * bpr, b, p, ok);
-        q4k_f32_load(u, uw + (size_t)(ok ? o : 0) * bpr, b, p, ok);
+        P::load_row(g, gw + (size_t)(ok ? o : 0) * bpr, u, ok);
+        P::load_row(up_r, uw + (size_t)(ok ? o : 0) * bpr, u, ok);
     }
-    Q4kF32X xa;
-    q4k_f32_load_x(xa, x + (size_t)b * 256 + p * 64, lane_ok);
+    typename P::X xa;
+    P::load_x(xa, x, u, lane_ok);
     for (int st = st0; st < st_end; ++st) {
         const int o = st * rps + seg;
         const bool ok = lane_ok && o < nff;
-        const Q4kF32Row gc = g, uc = u;
+        const typename P::Row gc = g, uc = up_r;
         if (st + 1 < st_end) {
             const int o2 = o + rps;
             const bool ok2 = lane_ok && o2 < nff;
-            q4k_f32_load(g, gw + (size_t)(ok2 ? o2 : 0) * bpr, b, p, ok2);
-            q4k_f32_load(u, uw + (size_t)(ok2 ? o2 : 0) * bpr, b, p, ok2);
+            P::load_row(g, gw + (size_t)(ok2 ? o2 : 0) * bpr, u, ok2);
+            P::load_row(up_r, uw + (size_t)(ok2 ? o2 : 0) * bpr, u, ok2);
         }
-        const float gs = seg_sum(q4k_f32_partial(gc, xa, p), seg * S, nb);
-        const float us = seg_sum(q4k_f32_partial(uc, xa, p), seg * S, nb);
-        if (ok && within == 0) act[(size_t)slot * nff + o] = gs / (1.0f + expf(-gs)) * us;
+        const float gs = seg_sum(P::partial(gc, xa, u), seg * S, S / 4);
+        const float us = seg_sum(P::partial(uc, xa, u), seg * S, S / 4);
+        if (ok && u == 0) act[(size_t)slot * nff + o] = gs / (1.0f + expf(-gs)) * us;
     }
 }
 
@@ -346,16 +455,17 @@ __global__ __launch_bounds__(256) void moe_gate_up_f32_q4k_kernel(
 // separate multiply and add, as the CPU's `*o += w_e * yv`.
 constexpr int kDownMaxSteps = 4, kDownMaxWaves = 16;
 
-__global__ __launch_bounds__(1024) void moe_down_f32_q4k_kernel(
+template <typename P>
+__global__ __launch_bounds__(1024) void moe_down_f32_kernel(
     const uint8_t* __restrict__ down, size_t down_stride, const int32_t* __restrict__ ids,
     const float* __restrict__ wts, const float* __restrict__ act, float* __restrict__ out, int nff,
     int ne, int n_used, int steps) {
     __shared__ float ys[kDownMaxSteps][kDownMaxWaves][16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
-    const int nb = nff / 256, S = 4 * nb, rps = 64 / S;
-    const int seg = lane / S, within = lane % S, b = within >> 2, p = within & 3;
+    const int S = nff / 64, rps = 64 / S;
+    const int seg = lane / S, u = lane % S;
     const bool lane_ok = seg < rps;
-    const size_t bpr = (size_t)nb * 144;
+    const size_t bpr = (size_t)(nff / 256) * P::kBlockBytes;
     const int st0 = blockIdx.x * steps;
     const int own_s = threadIdx.x / rps, own_seg = threadIdx.x % rps;  // output this thread adds up
     const bool owner = (int)threadIdx.x < steps * rps;
@@ -365,24 +475,24 @@ __global__ __launch_bounds__(1024) void moe_down_f32_q4k_kernel(
         if (k0) __syncthreads();
         if (k < n_used) {
             const uint8_t* dw = down + (size_t)ids[k] * down_stride;
-            Q4kF32Row row;
+            typename P::Row row;
             {
                 const int o = st0 * rps + seg;
                 const bool ok = lane_ok && o < ne;
-                q4k_f32_load(row, dw + (size_t)(ok ? o : 0) * bpr, b, p, ok);
+                P::load_row(row, dw + (size_t)(ok ? o : 0) * bpr, u, ok);
             }
-            Q4kF32X xa;
-            q4k_f32_load_x(xa, act + (size_t)k * nff + (size_t)b * 256 + p * 64, lane_ok);
+            typename P::X xa;
+            P::load_x(xa, act + (size_t)k * nff, u, lane_ok);
             for (int s = 0; s < steps; ++s) {
                 const int o = (st0 + s) * rps + seg;
-                const Q4kF32Row cur = row;
+                const typename P::Row cur = row;
                 if (s + 1 < steps) {
                     const int o2 = o + rps;
                     const bool ok2 = lane_ok && o2 < ne;
-                    q4k_f32_load(row, dw + (size_t)(ok2 ? o2 : 0) * bpr, b, p, ok2);
+                    P::load_row(row, dw + (size_t)(ok2 ? o2 : 0) * bpr, u, ok2);
                 }
-                const float yk = seg_sum(q4k_f32_partial(cur, xa, p), seg * S, nb);
-                if (lane_ok && within == 0) ys[s][wave][seg] = yk;
+                const float yk = seg_sum(P::partial(cur, xa, u), seg * S, S / 4);
+                if (lane_ok && u == 0) ys[s][wave][seg] = yk;
             }
         }
         __syncthreads();
@@ -627,24 +737,35 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
 
     if (s.rows == 1) {
         // ActsKind::Raw for every bank (lib.rs:2359: int8_ok = rows >= 2)
-        if (s.gate_dtype != 12 || s.up_dtype != 12 || s.down_dtype != 12)
-            return "rows == 1 carries Q4_K expert banks only";
+        auto raw_ok = [](int dt) { return dt == 12 || dt == 14 || dt == 8; };
+        if (!raw_ok(s.gate_dtype) || s.up_dtype != s.gate_dtype || !raw_ok(s.down_dtype))
+            return "rows == 1 carries Q4_K / Q6_K / Q8_0 expert banks (gate and up of one format)";
         if (s.ne > 4096 || s.n_ff > 4096) return "rows == 1 needs ne, n_ff_exp <= 4096";
         // row steps per wave: amortise the 64 activation registers while keeping >= ~1024 waves
         auto steps_per_wave = [](int wave_steps) { return std::max(1, std::min(4, wave_steps / 1024)); };
-        const int nb_g = s.ne / 256, rps_g = 64 / (4 * nb_g);
+        const int rps_g = 64 / (s.ne / 64);
         const int steps_g = (s.n_ff + rps_g - 1) / rps_g;
         const int spw = steps_per_wave(steps_g * s.n_used);
-        hipLaunchKernelGGL(moe_gate_up_f32_q4k_kernel,
-                           dim3((unsigned)((steps_g + 4 * spw - 1) / (4 * spw)), (unsigned)s.n_used), dim3(256), 0,
-                           stream, b.gate, b.up, b.gate_stride, b.up_stride, sel_idx, b.x, gbuf, s.ne, s.n_ff, spw);
-        const int nb_d = s.n_ff / 256, rps_d = 64 / (4 * nb_d);
+        const dim3 grid_g((unsigned)((steps_g + 4 * spw - 1) / (4 * spw)), (unsigned)s.n_used);
+#define INFR_GATE_UP(P)                                                                                    \
+    hipLaunchKernelGGL((moe_gate_up_f32_kernel<P>), grid_g, dim3(256), 0, stream, b.gate, b.up, b.gate_stride, \
+                       b.up_stride, sel_idx, b.x, gbuf, s.ne, s.n_ff, spw)
+        if (s.gate_dtype == 12) INFR_GATE_UP(RawQ4K);
+        else if (s.gate_dtype == 14) INFR_GATE_UP(RawQ6K);
+        else INFR_GATE_UP(RawQ8_0);
+#undef INFR_GATE_UP
+        const int rps_d = 64 / (s.n_ff / 64);
         const int steps_d = (s.ne + rps_d - 1) / rps_d;
         const int spw_d = std::min(kDownMaxSteps, steps_per_wave(steps_d * s.n_used));
         const int nw_d = std::min(s.n_used, kDownMaxWaves);
-        hipLaunchKernelGGL(moe_down_f32_q4k_kernel, dim3((unsigned)((steps_d + spw_d - 1) / spw_d)),
-                           dim3((unsigned)(64 * nw_d)), 0, stream, b.down, b.down_stride, sel_idx, sel_w, gbuf,
-                           b.dst, s.n_ff, s.ne, s.n_used, spw_d);
+        const dim3 grid_d((unsigned)((steps_d + spw_d - 1) / spw_d));
+#define INFR_DOWN(P)                                                                                     \
+    hipLaunchKernelGGL((moe_down_f32_kernel<P>), grid_d, dim3((unsigned)(64 * nw_d)), 0, stream, b.down,   \
+                       b.down_stride, sel_idx, sel_w, gbuf, b.dst, s.n_ff, s.ne, s.n_used, spw_d)
+        if (s.down_dtype == 12) INFR_DOWN(RawQ4K);
+        else if (s.down_dtype == 14) INFR_DOWN(RawQ6K);
+        else INFR_DOWN(RawQ8_0);
+#undef INFR_DOWN
         return hipGetLastError() == hipSuccess ? nullptr : "kernel launch failed";
     }
 

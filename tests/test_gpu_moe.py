@@ -141,3 +141,27 @@ def test_moe_in_a_plan_replays(be, rows):
         gate_out(got[0], orc.moe_ffn(x, router, *b1, scale=1.5, **kw)[0])
         gate_out(got[1], orc.linear(DType.Q4K, wmid, got[0].ravel(), rows, ne, ne))
         gate_out(got[2], orc.moe_ffn(got[1].ravel(), router, *b2, scale=1.0, **kw)[0])
+
+
+@pytest.mark.parametrize("gu_dtype,down_dtype", [(DType.Q6K, DType.Q6K), (DType.Q8_0, DType.Q8_0),
+                                                 (DType.Q4K, DType.Q6K), (DType.Q8_0, DType.Q4K)])
+@pytest.mark.parametrize("ne,nff", [(512, 256), (2048, 768)])
+def test_moe_one_token_other_bank_formats(be, gu_dtype, down_dtype, ne, nff):
+    """rows == 1 (decoded-f32-weights path) for Q6_K / Q8_0 banks and the mixed layouts real files
+    use (Q4_K gate/up with a Q6_K down)."""
+    n_expert, n_used = 16, 4
+    gate = synth_weight(gu_dtype, 130, n_expert * nff, ne, 0.05)
+    up = synth_weight(gu_dtype, 131, n_expert * nff, ne, 0.05)
+    down = synth_weight(down_dtype, 132, n_expert * ne, nff, 0.05)
+    x = synth_normal_f32(133, ne)
+    router = synth_normal_f32(134, n_expert * ne, sigma=0.05)
+    xb, rb = be.upload_new(x), be.upload_new(router)
+    gb, ub, db = be.upload_new(gate), be.upload_new(up), be.upload_new(down)
+    yb, ib, wb = be.alloc(ne * 4), be.alloc(n_used * 4), be.alloc(n_used * 4)
+    be.moe_ffn(xb, rb, gb, ub, db, yb, rows=1, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff, scale=1.0,
+               gate_dtype=gu_dtype, up_dtype=gu_dtype, down_dtype=down_dtype, sel_idx=ib, sel_w=wb)
+    got = (be.download(yb, np.empty((1, ne), np.float32)), be.download(ib, np.empty((1, n_used), np.int32)),
+           be.download(wb, np.empty((1, n_used), np.float32)))
+    want = orc.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
+                       gate_dtype=int(gu_dtype), up_dtype=int(gu_dtype), down_dtype=int(down_dtype))
+    check(*got, *want)
