@@ -313,6 +313,36 @@ def moe_bench(be, n_layers=6):
     return out
 
 
+def load_bench(be, n_layers=8):
+    """A synthetic checkpoint of `n_layers` Qwen3-8B layers (Q4_K projections, Q6_K down) written
+    as a GGUF file, then opened and uploaded tensor by tensor through the reader: page cache ->
+    HBM over PCIe. Returns (open ms, upload ms, bytes)."""
+    import tempfile
+    from infr_amd import DType, synth_weight
+    from infr_amd.gguf import Gguf, write_gguf
+    tensors = []
+    for l in range(n_layers):
+        for name, out_f, in_f in LAYER:
+            dt = DType.Q6K if name == "down" else DType.Q4K
+            tensors.append((f"blk.{l}.{name}.weight", (in_f, out_f), int(dt), synth_weight(dt, 900 + l, out_f, in_f)))
+    with tempfile.TemporaryDirectory() as d:
+        path = os.path.join(d, "synthetic.gguf")
+        write_gguf(path, {"general.architecture": "qwen3", "qwen3.block_count": n_layers}, tensors)
+        del tensors
+        t0 = time.perf_counter()
+        g = Gguf.open(path)
+        t1 = time.perf_counter()
+        infos = g.tensors()
+        bufs = [g.upload(be, t.name) for t in infos]
+        be.sync()
+        t2 = time.perf_counter()
+        nbytes = sum(t.nbytes for t in infos)
+        for b in bufs:
+            b.free()
+        g.close()
+    return (t1 - t0) * 1e3, (t2 - t1) * 1e3, nbytes
+
+
 def cpu_baseline(dtype_name="Q4_K"):
     """The CPU oracle (C restatement of infr-cpu's scalar kernels, OpenMP over output rows with the
     reference's 16-row grain) on a bounded sample of the headline workload: one layer's seven
@@ -346,8 +376,8 @@ def main():
     ap.add_argument("--layers", type=int, default=N_LAYERS)
     ap.add_argument("--no-extra", action="store_true", help="headline sweep only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--sections", default="shapes,mmq,chain,layer,ternary,moe",
-                    help="comma list of secondary sections: shapes, mmq, chain, layer, ternary, moe")
+    ap.add_argument("--sections", default="shapes,mmq,chain,layer,ternary,moe,load",
+                    help="comma list of secondary sections: shapes, mmq, chain, layer, ternary, moe, load")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
@@ -439,6 +469,11 @@ def main():
         tern.free()
     if "moe" in sections:
         extra.update(moe_bench(be))
+    if "load" in sections:
+        open_ms, up_ms, nb = load_bench(be)
+        extra["gguf_open_ms"] = round(open_ms, 2)
+        extra["gguf_upload_GBs_pcie_inclusive"] = round(nb / (up_ms * 1e-3) / 1e9, 2)
+        extra["gguf_upload_bytes"] = nb
     out["extra"] = extra
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline()

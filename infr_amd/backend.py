@@ -87,8 +87,8 @@ class _Caps(C.Structure):
                 ("device_name", C.c_char * 64)]
 
 
-# Every symbol include/infr_hip.h declares: (restype, argtypes).
 _vp = C.c_void_p
+# Every symbol include/infr_hip.h declares: (restype, argtypes).
 SYMBOLS = {
     "infr_hip_create": (C.c_int, [C.c_int, C.POINTER(_vp)]),
     "infr_hip_destroy": (None, [_vp]),
@@ -129,6 +129,47 @@ SYMBOLS = {
     "infr_synth_weight": (C.c_size_t, [C.c_int, C.c_uint64, C.c_float, C.c_size_t, C.c_size_t, _vp]),
     "infr_block_layout": (C.c_int, [C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
 }
+
+
+class _GgufTensor(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("ggml_type", C.c_int), ("n_dims", C.c_int),
+                ("shape", C.c_uint64 * 4), ("numel", C.c_uint64), ("offset", C.c_uint64),
+                ("nbytes", C.c_size_t)]
+
+
+# Every symbol include/infr_gguf.h declares.
+SYMBOLS.update({
+    "infr_gguf_open": (C.c_int, [C.c_char_p, C.POINTER(_vp)]),
+    "infr_gguf_close": (None, [_vp]),
+    "infr_gguf_last_error": (C.c_char_p, []),
+    "infr_gguf_n_tensors": (C.c_size_t, [_vp]),
+    "infr_gguf_tensor": (C.c_int, [_vp, C.c_size_t, C.POINTER(_GgufTensor)]),
+    "infr_gguf_find": (C.c_int64, [_vp, C.c_char_p]),
+    "infr_gguf_tensor_bytes": (C.c_int, [_vp, C.c_char_p, C.POINTER(_vp), C.POINTER(C.c_size_t)]),
+    "infr_gguf_tensor_file_range": (C.c_int, [_vp, C.c_char_p, C.POINTER(C.c_uint64), C.POINTER(C.c_size_t)]),
+    "infr_gguf_n_shards": (C.c_size_t, [_vp]),
+    "infr_gguf_shard": (C.c_int, [_vp, C.c_size_t, C.POINTER(C.c_char_p), C.POINTER(C.c_uint64)]),
+    "infr_gguf_n_meta": (C.c_size_t, [_vp]),
+    "infr_gguf_meta_key": (C.c_char_p, [_vp, C.c_size_t]),
+    "infr_gguf_meta_get": (_vp, [_vp, C.c_char_p]),
+    "infr_gguf_value_kind": (C.c_int, [_vp]),
+    "infr_gguf_value_u64": (C.c_int, [_vp, C.POINTER(C.c_uint64)]),
+    "infr_gguf_value_i64": (C.c_int, [_vp, C.POINTER(C.c_int64)]),
+    "infr_gguf_value_f64": (C.c_int, [_vp, C.POINTER(C.c_double)]),
+    "infr_gguf_value_bool": (C.c_int, [_vp, C.POINTER(C.c_int)]),
+    "infr_gguf_value_str": (C.c_int, [_vp, C.POINTER(_vp), C.POINTER(C.c_size_t)]),
+    "infr_gguf_value_arr_len": (C.c_int, [_vp, C.POINTER(C.c_size_t)]),
+    "infr_gguf_value_arr_at": (_vp, [_vp, C.c_size_t]),
+    "infr_gguf_chat_template": (C.c_char_p, [_vp]),
+    "infr_gguf_block_layout": (C.c_int, [C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "infr_gguf_nbytes": (C.c_size_t, [C.c_int, C.c_uint64, C.POINTER(C.c_int)]),
+    "infr_gguf_parse_shard": (C.c_int, [C.c_char_p, C.c_char_p, C.c_size_t, C.POINTER(C.c_size_t),
+                                        C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.POINTER(C.c_size_t)]),
+    "infr_gguf_shard_set": (C.c_size_t, [C.c_char_p, C.c_size_t, C.c_char_p, C.c_size_t]),
+    "infr_gguf_upload": (C.c_int, [_vp, C.c_char_p, _vp, C.POINTER(_vp)]),
+    "infr_gguf_upload_concat": (C.c_int, [_vp, C.POINTER(C.c_char_p), C.c_size_t, _vp, C.POINTER(_vp),
+                                          C.POINTER(C.c_size_t)]),
+})
 
 _lib = None
 
