@@ -40,9 +40,15 @@ typedef enum {
  * (crates/infr-gguf/src/lib.rs:330-354; crates/infr-core/src/tensor.rs:7-57). */
 typedef enum {
     INFR_DTYPE_F32 = 0,
+    INFR_DTYPE_Q4_0 = 2,  /* 32 / 18 B:  [f16 d][u8 qs[16]]             w = d*(q-8)        :311-312 */
+    INFR_DTYPE_Q4_1 = 3,  /* 32 / 20 B:  [f16 d][f16 m][u8 qs[16]]      w = d*q+m          :313-314 */
+    INFR_DTYPE_Q5_0 = 6,  /* 32 / 22 B:  [f16 d][u32 qh][u8 qs[16]]     w = d*(q-16)       :315-316 */
+    INFR_DTYPE_Q5_1 = 7,  /* 32 / 24 B:  [f16 d][f16 m][u32 qh][u8 qs[16]]  w = d*q+m      :317-318 */
     INFR_DTYPE_Q8_0 = 8,  /* 32 elems / 34 B:  [f16 d][i8 qs[32]]            decode_spec.rs:319-320 */
     INFR_DTYPE_Q4_K = 12, /* 256 / 144 B: [f16 d][f16 dmin][u8 sc[12]][u8 qs[128]]        :326-327 */
+    INFR_DTYPE_Q5_K = 13, /* 256 / 176 B: [f16 d][f16 dmin][u8 sc[12]][u8 qh[32]][u8 qs[128]] :328-329 */
     INFR_DTYPE_Q6_K = 14, /* 256 / 210 B: [u8 ql[128]][u8 qh[64]][i8 sc[16]][f16 d]       :330-331 */
+    INFR_DTYPE_IQ4_NL = 20, /* 32 / 18 B: [f16 d][u8 qs[16]]  w = d*codebook[q]           :349-350 */
     INFR_DTYPE_Q2_0 = 42  /* 64 / 18 B:   [f16 d][u8 qs[16]] ternary-style 2-bit codes    :357-358 */
 } infr_dtype;
 

@@ -22,9 +22,15 @@ LIB_PATH = os.path.join(_HERE, "libinfr_hip.so")
 class DType(IntEnum):
     """GGML type ids (crates/infr-gguf/src/lib.rs:330-354)."""
     F32 = 0
+    Q4_0 = 2
+    Q4_1 = 3
+    Q5_0 = 6
+    Q5_1 = 7
     Q8_0 = 8
     Q4K = 12
+    Q5K = 13
     Q6K = 14
+    IQ4NL = 20
     Q2_0 = 42
 
 
@@ -549,9 +555,9 @@ class HipBackend:
         if w_numel is None:
             e, b = block_layout(dtype)
             w_numel = w.len_bytes() // b * e
-        blocks = in_f // 256 if dtype in (DType.Q4K, DType.Q6K) else in_f // 32
+        blocks = in_f // 256 if dtype in (DType.Q4K, DType.Q5K, DType.Q6K) else in_f // 32
         a = self.alloc(m * out_f * blocks * 4)
-        b_ = self.alloc(m * out_f * blocks * 4) if dtype == DType.Q4K else None
+        b_ = self.alloc(m * out_f * blocks * 4) if dtype in (DType.Q4K, DType.Q5K) else None
         self._check(self._lib.infr_hip_linear_int_stages(
             self._h, int(dtype), w._h, w_numel, w_off, x._h, m, in_f, out_f, a._h,
             b_._h if b_ else None))

@@ -91,16 +91,30 @@ int fail(infr_hip_t* be, int code, const std::string& msg) {
                         std::string(#expr) + ": " + hipGetErrorString(e__));                 \
     } while (0)
 
+// Weight formats Op::Linear has kernels for.
 bool is_quant(int dt) {
-    return dt == INFR_DTYPE_Q4_K || dt == INFR_DTYPE_Q6_K || dt == INFR_DTYPE_Q8_0 ||
-           dt == INFR_DTYPE_Q2_0;
+    switch (dt) {
+    case INFR_DTYPE_Q4_0: case INFR_DTYPE_Q4_1: case INFR_DTYPE_Q5_0: case INFR_DTYPE_Q5_1:
+    case INFR_DTYPE_Q8_0: case INFR_DTYPE_Q4_K: case INFR_DTYPE_Q5_K: case INFR_DTYPE_Q6_K:
+    case INFR_DTYPE_IQ4_NL: case INFR_DTYPE_Q2_0: return true;
+    default: return false;
+    }
 }
-// Which activation quantizer infr-cpu's dispatch pairs with the weight dtype
-// (crates/infr-cpu/src/lib.rs:1043-1076): per-32 only for Q2_0 among the formats carried here.
-// Per-32 activation quantizer: Q2_0 always, Q8_0 for rows that are not whole 256s (lib.rs:1037-1076).
-bool act_per32(int dt, size_t in_f) { return dt == INFR_DTYPE_Q2_0 || (dt == INFR_DTYPE_Q8_0 && in_f % 256 != 0); }
+// Formats Op::MoeFfn's expert banks may hold.
+bool is_moe_quant(int dt) {
+    return dt == INFR_DTYPE_Q4_K || dt == INFR_DTYPE_Q6_K || dt == INFR_DTYPE_Q8_0;
+}
+bool act_per32(int dt, size_t in_f) { return infr::act_is_per32(dt, in_f); }
 // Row lengths a format accepts: whole weight blocks.
-size_t in_f_multiple(int dt) { return dt == INFR_DTYPE_Q2_0 ? 64 : (dt == INFR_DTYPE_Q8_0 ? 32 : 256); }
+size_t in_f_multiple(int dt) {
+    int e = 0, b = 0;
+    return infr_block_layout(dt, &e, &b) ? (size_t)e : 256;
+}
+// Blocks per row of the per-block integer stage outputs: per 256 for the K-quants, per 32 otherwise.
+size_t stage_blocks(int dt, size_t in_f) {
+    return (dt == INFR_DTYPE_Q4_K || dt == INFR_DTYPE_Q5_K || dt == INFR_DTYPE_Q6_K) ? in_f / 256 : in_f / 32;
+}
+bool has_two_stages(int dt) { return dt == INFR_DTYPE_Q4_K || dt == INFR_DTYPE_Q5_K; }
 
 // Activation scratch for m rows: the prefill kernels read tokens in groups of 32.
 static size_t act_scratch_elems(size_t m, size_t in_f) { return (m == 1 ? 1 : (m + 31) / 32 * 32) * in_f; }
@@ -269,7 +283,12 @@ int check_linear(infr_hip_t* be, int dtype, const infr_hip_buffer_t* w, size_t w
 int enqueue_linear(infr_hip_t* be, int dtype, const LinearArgs& la, const float* x, float* y,
                    size_t m, size_t in_f, size_t out_f, const infr::IntStages& st) {
     bool ok;
-    if (m == 1) {
+    if (infr::gemv_takes_f32_activations(dtype, m)) {
+        if (st.a)
+            return fail(be, INFR_HIP_ERR_UNSUPPORTED,
+                        "int_stages: one token of dtype " + std::to_string(dtype) + " has no integer stage");
+        ok = infr::launch_gemv_f32act(dtype, la.wrows, la.bpr, x, y, in_f, out_f, be->stream);
+    } else if (m == 1) {
         infr::launch_quantize_q8(x, m, in_f, act_per32(dtype, in_f), be->act, be->stream);
         ok = infr::launch_gemv(dtype, la.wrows, la.bpr, be->act, y, in_f, out_f, st, be->stream);
     } else {
@@ -503,7 +522,7 @@ int infr_hip_linear(infr_hip_t* be, int dtype, const infr_hip_buffer_t* w, size_
     if (int rc = check_linear(be, dtype, w, w_numel, w_off, x, m, in_f, out_f, &la)) return rc;
     if (!dst || dst->len < m * out_f * sizeof(float))
         return fail(be, INFR_HIP_ERR_INVALID, "linear: dst buffer missing or too small");
-    if (m == 1) {
+    if (m == 1 && !infr::gemv_takes_f32_activations(dtype, m)) {
         // decode: one fused launch (quantize x in LDS + GEMV)
         const infr::GemvOpDesc op{la.wrows, static_cast<const float*>(x->ptr),
                                   static_cast<float*>(dst->ptr), la.bpr, (int32_t)out_f};
@@ -522,11 +541,11 @@ int infr_hip_linear_int_stages(infr_hip_t* be, int dtype, const infr_hip_buffer_
     if (int rc = check_latch(be)) return rc;
     LinearArgs la;
     if (int rc = check_linear(be, dtype, w, w_numel, w_off, x, m, in_f, out_f, &la)) return rc;
-    const size_t blocks = (dtype == INFR_DTYPE_Q4_K || dtype == INFR_DTYPE_Q6_K) ? in_f / 256 : in_f / 32;
+    const size_t blocks = stage_blocks(dtype, in_f);
     const size_t need = m * out_f * blocks * sizeof(int32_t);
     if (!a || a->len < need) return fail(be, INFR_HIP_ERR_INVALID, "int_stages: buffer a too small");
-    if (dtype == INFR_DTYPE_Q4_K && (!b || b->len < need))
-        return fail(be, INFR_HIP_ERR_INVALID, "int_stages: Q4_K needs buffer b");
+    if (has_two_stages(dtype) && (!b || b->len < need))
+        return fail(be, INFR_HIP_ERR_INVALID, "int_stages: Q4_K / Q5_K need buffer b");
     if (int rc = ensure_act(be, act_scratch_elems(m, in_f))) return rc;
     // y is not wanted here; use a transient output
     float* y = nullptr;
@@ -608,8 +627,8 @@ static int check_moe(infr_hip_t* be, const infr_hip_moe_params_t* p, const infr_
     const size_t gb = expert_bank_bytes(p->gate_dtype, (size_t)p->n_expert * p->n_ff_exp, p->ne);
     const size_t ub = expert_bank_bytes(p->up_dtype, (size_t)p->n_expert * p->n_ff_exp, p->ne);
     const size_t db = expert_bank_bytes(p->down_dtype, (size_t)p->n_expert * p->ne, p->n_ff_exp);
-    if (!gb || !ub || !db || p->gate_dtype == INFR_DTYPE_F32 || p->up_dtype == INFR_DTYPE_F32 ||
-        p->down_dtype == INFR_DTYPE_F32)
+    if (!gb || !ub || !db || !is_moe_quant(p->gate_dtype) || !is_moe_quant(p->up_dtype) ||
+        !is_moe_quant(p->down_dtype))
         return fail(be, INFR_HIP_ERR_UNSUPPORTED, "moe_ffn: expert bank dtype/shape has no kernel");
     const size_t act_bytes = (size_t)p->rows * p->ne * sizeof(float);
     if (gate->len < gb || up->len < ub || down->len < db ||
@@ -807,7 +826,10 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
     std::vector<int> pre(n, -1), post(n, -1);
     std::vector<char> absorbed(n, 0), publishes(n, 0);
     static const int env_fuse = getenv("INFR_HIP_FUSE") ? atoi(getenv("INFR_HIP_FUSE")) : 1;
-    auto decode_linear = [&](size_t i) { return plan->ops[i].kind == INFR_OP_LINEAR && plan->ops[i].m == 1; };
+    auto decode_linear = [&](size_t i) {
+        return plan->ops[i].kind == INFR_OP_LINEAR && plan->ops[i].m == 1 &&
+               !infr::gemv_takes_f32_activations(plan->ops[i].w_dtype, 1);
+    };
     for (size_t k = 0; env_fuse && k < n; ++k) {
         const auto& p = plan->ops[k];
         const bool gated = (p.kind == INFR_OP_GATED_ACT && p.gate_block_width == 0) || p.kind == INFR_OP_GATED_ACT_FUSED;
@@ -953,7 +975,7 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
                 plan->steps.push_back(st);
                 continue;
             }
-            if (op.kind != INFR_OP_LINEAR || op.m != 1) {
+            if (op.kind != INFR_OP_LINEAR || op.m != 1 || infr::gemv_takes_f32_activations(op.w_dtype, op.m)) {
                 st.op = (int)i;
                 taken[i] = 1;
                 plan->steps.push_back(st);
@@ -965,7 +987,8 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
             for (size_t k = i; k < n; ++k) {
                 const auto& o2 = plan->ops[k];
                 if (level[k] != lv || taken[k] || absorbed[k] || o2.kind != INFR_OP_LINEAR || o2.m != 1 ||
-                    o2.w_dtype != op.w_dtype || o2.in_f != op.in_f)
+                    o2.w_dtype != op.w_dtype || o2.in_f != op.in_f ||
+                    (op.w_dtype == INFR_DTYPE_Q8_0 && (o2.in_f % 256 == 0) != (op.in_f % 256 == 0)))
                     continue;
                 taken[k] = 1;
                 // with an absorbed producer the GEMV starts from the producer's first input

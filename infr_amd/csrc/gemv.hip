@@ -22,332 +22,38 @@
 // the CPU's accumulation order, so y matches infr-cpu's scalar kernel bit for bit. For Q8_0 and
 // Q2_0 (128 terms per 4096 columns) the lanes' terms are added with a fixed butterfly instead:
 // deterministic, but rounded in a different order than the CPU's sequential sum.
-#include <algorithm>
-#include <cstdlib>
-
-#include "gemv_formats.hpp"
-#include "gemv_rows.hpp"
-#include "kernels.hpp"
-#include "quant_chunk.hpp"
+#include "gemv_impl.hpp"
 
 namespace infr {
 
-template <typename F, int STEPS, bool STAGES>
-__global__ __launch_bounds__(256) void gemv_kernel(const uint8_t* __restrict__ w, size_t bpr,
-                                                   ActPtrs act, float* __restrict__ y, int n_units,
-                                                   int out_f, int rows_per_wave, StagePtrs st) {
-    const int lane = threadIdx.x & 63;
-    const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int row0 = wave * rows_per_wave;
-    if (row0 >= out_f) return;
-    const int row_end = min(row0 + rows_per_wave, out_f);
-    typename F::Acts acts[STEPS];
-    typename F::Row first;
-    bool ok[STEPS];
-#pragma unroll
-    for (int t = 0; t < STEPS; ++t) ok[t] = F::valid(t, lane, n_units);
-    F::load_row(first, w + (size_t)row0 * bpr, 0, lane, ok[0]);
-#pragma unroll
-    for (int t = 0; t < STEPS; ++t) F::load_acts(acts[t], act, t, lane, ok[t]);
-    __shared__ __attribute__((aligned(16))) float osum[F::kOrdered ? 4 * OrderedSum<STEPS>::kFloatsPerWave : 4];
-    gemv_rows<F, STEPS, STAGES>(w, bpr, first, acts, ok, y, n_units, row0, row_end, lane, st,
-                                osum + (threadIdx.x >> 6) * (F::kOrdered ? OrderedSum<STEPS>::kFloatsPerWave : 0));
-}
-
-// Small batch (2..8 activation rows already quantized in device memory): weights stream once.
-// With `tiles` (plans) a workgroup takes one table entry - some rows of one of several ops - and
-// blockIdx.y selects the pass of MB activation rows; `m_valid` is then the op's total row count.
-template <typename F, int STEPS, int MB, bool STAGES>
-__global__ __launch_bounds__(256) void gemv_batch_kernel(const uint8_t* __restrict__ w, size_t bpr,
-                                                         ActPtrs act, int m_valid, int in_f,
-                                                         float* __restrict__ y, int out_f,
-                                                         int rows_per_wave, StagePtrs st,
-                                                         const BatchTile* __restrict__ tiles) {
-    const int lane = threadIdx.x & 63;
-    int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
-    int n_rows = out_f;
-    size_t act_elem0 = 0;
-    if (tiles) {
-        const BatchTile t = tiles[blockIdx.x];
-        const int pass = blockIdx.y;
-        w = t.w;
-        bpr = t.bpr;
-        out_f = (int)t.out_f;
-        n_rows = (int)t.rows;
-        y = t.y + (size_t)pass * MB * out_f;
-        act_elem0 = (size_t)t.act_elem0 + (size_t)pass * MB * in_f;
-        m_valid = min(MB, m_valid - pass * MB);
-        wave = threadIdx.x >> 6;
+// One table per format; each is defined in the gemv_fmt_*.hip that instantiates the format.
+static const GemvFormatOps* format_ops(int dtype, size_t in_f) {
+    switch (dtype) {
+    case 12: return &gemv_ops_q4k();
+    case 14: return &gemv_ops_q6k();
+    case 8: return in_f % 256 == 0 ? &gemv_ops_q8_0() : &gemv_ops_q8_0_32();
+    case 42: return &gemv_ops_q2_0();
+    case 13: return &gemv_ops_q5k();
+    case 2: return &gemv_ops_q4_0();
+    case 3: return &gemv_ops_q4_1();
+    case 6: return &gemv_ops_q5_0();
+    case 7: return &gemv_ops_q5_1();
+    case 20: return &gemv_ops_iq4nl();
+    default: return nullptr;
     }
-    const int row0 = wave * rows_per_wave;
-    if (row0 >= n_rows) return;
-    const int row_end = min(row0 + rows_per_wave, n_rows);
-    const int n_units = F::units(in_f);
-    typename F::Acts acts[MB][STEPS];
-    typename F::Row first;
-    bool ok[STEPS];
-#pragma unroll
-    for (int t = 0; t < STEPS; ++t) ok[t] = F::valid(t, lane, n_units);
-    F::load_row(first, w + (size_t)row0 * bpr, 0, lane, ok[0]);
-#pragma unroll
-    for (int mi = 0; mi < MB; ++mi) {
-        const int r = mi < m_valid ? mi : 0;  // padding rows reuse row 0; their outputs are dropped
-        const size_t e = act_elem0 + (size_t)r * in_f;
-        const ActPtrs a{act.qs + e, act.d + e / (F::kPer32 ? 32 : 256), act.bsums + e / 32,
-                        act.bsums16 + e / 16};
-#pragma unroll
-        for (int t = 0; t < STEPS; ++t) F::load_acts(acts[mi][t], a, t, lane, ok[t]);
-    }
-    __shared__ __attribute__((aligned(16))) float osum[F::kOrdered ? 4 * OrderedSum<STEPS>::kFloatsPerWave : 4];
-    const size_t st_stride = (size_t)out_f * (F::kBlockElems == 64 ? 2 * n_units : n_units);
-    gemv_rows_batch<F, STEPS, MB, STAGES>(
-        w, bpr, first, acts, ok, y, (size_t)out_f, m_valid, n_units, row0, row_end, lane, st, st_stride,
-        osum + (threadIdx.x >> 6) * (F::kOrdered ? OrderedSum<STEPS>::kFloatsPerWave : 0));
-}
-
-// act(gate) * up with the optional clamp, as Op::GatedAct evaluates one element
-// (gated_act_fn, crates/infr-cpu/src/kernels.rs:6591-6597).
-__device__ __forceinline__ float fused_gated_act(int act, bool has_clamp, float l, float gate, float up) {
-    if (has_clamp) {
-        gate = gate < l ? gate : l;
-        up = up < -l ? -l : (up > l ? l : up);
-    }
-    float a;
-    switch (act) {
-    case 1: a = 0.5f * gate * (1.0f + tanhf(0.7978846f * (gate + 0.044715f * gate * gate * gate))); break;
-    case 2: a = 1.0f / (1.0f + expf(-gate)); break;
-    default: a = gate / (1.0f + expf(-gate)); break;
-    }
-    return a * up;
-}
-
-// Fused + grouped form. LDS: qs[in_f] | d[in_f/32] | bsums[in_f/32] | bsums16[in_f/16] | per-wave
-// ordered-sum scratch.
-template <typename F, int STEPS, int NW>
-__global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, int single_rows,
-                                                             const GemvTile* __restrict__ tiles,
-                                                             int in_f) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-
-    // This workgroup's rows: one table entry, or computed from the single op's descriptor.
-    GemvTile tile;
-    if (tiles != nullptr) {
-        tile = tiles[blockIdx.x];
-    } else {
-        const int first = (int)blockIdx.x * single_rows;
-        tile.w = single.w + (size_t)first * single.bpr;
-        tile.x = single.x;
-        tile.y = single.y + first;
-        tile.bpr = (uint32_t)single.bpr;
-        tile.rows = min(single_rows, single.out_f - first);
-        tile.fus = single.fus;
-        if (tile.fus.add_dst) {
-            tile.fus.add_b += first;
-            tile.fus.add_dst += first;
-        }
-        if (blockIdx.x != 0) tile.fus.pre_dst = nullptr;
-    }
-    const int rpw = (tile.rows + NW - 1) / NW;
-    const int n_units = F::units(in_f);
-    const int row0 = wave * rpw;
-    const int row_end = min(row0 + rpw, tile.rows);
-
-    int8_t* l_qs = reinterpret_cast<int8_t*>(lds);
-    float* l_d = reinterpret_cast<float*>(lds + in_f);
-    int32_t* l_bs = reinterpret_cast<int32_t*>(lds + in_f + in_f / 8);
-    int32_t* l_bs16 = reinterpret_cast<int32_t*>(lds + in_f + in_f / 4);
-
-    // The wave's share of x (256-float chunks w, w+NW, ...) is requested first, then the first
-    // weight row: the row streams in from HBM while x is quantized.
-    const int n_chunks = (in_f + 255) / 256;
-    constexpr int kMaxChunks = (STEPS * F::kElemsPerStep / 256 + NW - 1) / NW;
-    v4f xv[kMaxChunks];
-#pragma unroll
-    for (int i = 0; i < kMaxChunks; ++i) {
-        const int c = wave + i * NW;
-        xv[i] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-        if (c < n_chunks && c * 256 + lane * 4 < in_f)
-            xv[i] = *reinterpret_cast<const v4f*>(tile.x + (size_t)c * 256 + lane * 4);
-    }
-    const bool has_rows = row0 < tile.rows;
-    typename F::Row first;
-    bool ok[STEPS];
-#pragma unroll
-    for (int t = 0; t < STEPS; ++t) ok[t] = has_rows && F::valid(t, lane, n_units);
-    F::load_row(first, tile.w + (size_t)row0 * tile.bpr, 0, lane, ok[0]);
-    // An absorbed producer of x (workgroup-uniform branch): every workgroup recomputes the vector
-    // from the producer's inputs - cheaper than a launch of its own - and the op's first
-    // workgroup stores it where the producer would have.
-    if (tile.fus.pre != 0) {
-        float scale = 1.0f;
-        if (tile.fus.pre == 2) {  // RmsNorm: mean square over the row, tree order fixed by NW
-            float* part = reinterpret_cast<float*>(lds);  // qs area, not yet written
-            float sq = 0.0f;
-#pragma unroll
-            for (int i = 0; i < kMaxChunks; ++i)
-                sq += (xv[i].x * xv[i].x + xv[i].y * xv[i].y) + (xv[i].z * xv[i].z + xv[i].w * xv[i].w);
-            sq = wave_sum_f(sq);
-            if (lane == 0) part[wave] = sq;
-            __syncthreads();
-            float tot = 0.0f;
-#pragma unroll
-            for (int wv = 0; wv < NW; ++wv) tot += part[wv];
-            __syncthreads();  // `part` is about to be overwritten by the quantized codes
-            scale = 1.0f / sqrtf(tot / (float)in_f + tile.fus.eps);
-        }
-#pragma unroll
-        for (int i = 0; i < kMaxChunks; ++i) {
-            const int c = wave + i * NW;
-            if (c < n_chunks && c * 256 + lane * 4 < in_f) {
-                const v4f o = *reinterpret_cast<const v4f*>(tile.fus.x2 + (size_t)c * 256 + lane * 4);
-                v4f r;
-                if (tile.fus.pre == 2) {
-                    r = v4f{xv[i].x * scale * o.x, xv[i].y * scale * o.y, xv[i].z * scale * o.z, xv[i].w * scale * o.w};
-                } else {
-                    const bool hc = tile.fus.has_clamp != 0;
-                    r.x = fused_gated_act(tile.fus.act, hc, tile.fus.clamp, xv[i].x, o.x);
-                    r.y = fused_gated_act(tile.fus.act, hc, tile.fus.clamp, xv[i].y, o.y);
-                    r.z = fused_gated_act(tile.fus.act, hc, tile.fus.clamp, xv[i].z, o.z);
-                    r.w = fused_gated_act(tile.fus.act, hc, tile.fus.clamp, xv[i].w, o.w);
-                }
-                xv[i] = r;
-                if (tile.fus.pre_dst)
-                    *reinterpret_cast<v4f*>(tile.fus.pre_dst + (size_t)c * 256 + lane * 4) = r;
-            }
-        }
-    }
-#pragma unroll
-    for (int i = 0; i < kMaxChunks; ++i) {
-        const int c = wave + i * NW;
-        if (c < n_chunks)
-            quantize_chunk<F::kPer32>(xv[i], c * 256 + lane * 4 < in_f, lane, (size_t)c, l_qs, l_d,
-                                      l_bs, F::kPer32 ? nullptr : l_bs16);
-    }
-    __syncthreads();
-    if (!has_rows) return;
-
-    ActPtrs act{l_qs, l_d, l_bs, l_bs16};
-    typename F::Acts acts[STEPS];
-#pragma unroll
-    for (int t = 0; t < STEPS; ++t) F::load_acts(acts[t], act, t, lane, ok[t]);
-    float* osum = reinterpret_cast<float*>(lds + in_f + in_f / 2) + wave * OrderedSum<STEPS>::kFloatsPerWave;
-    gemv_rows<F, STEPS, false>(tile.w, tile.bpr, first, acts, ok, tile.y, n_units, row0, row_end, lane,
-                               StagePtrs{nullptr, nullptr}, osum, tile.fus.add_b, tile.fus.add_dst);
-}
-
-// ───────────────────────────────────── launch ─────────────────────────────────────
-
-template <typename F, bool STAGES>
-static bool launch_plain(int steps, dim3 grid, hipStream_t stream, const uint8_t* w, size_t bpr,
-                         const ActPtrs& act, float* y, int n_units, int out_f, int rpw,
-                         const StagePtrs& st) {
-#define INFR_CASE(N)                                                                             \
-    case N:                                                                                      \
-        hipLaunchKernelGGL((gemv_kernel<F, N, STAGES>), grid, dim3(256), 0, stream, w, bpr, act, y, \
-                           n_units, out_f, rpw, st);                                             \
-        return true;
-    switch (steps) {
-        INFR_CASE(1) INFR_CASE(2) INFR_CASE(3) INFR_CASE(4)
-        INFR_CASE(5) INFR_CASE(6) INFR_CASE(7) INFR_CASE(8)
-    default: return false;
-    }
-#undef INFR_CASE
-}
-
-template <typename F>
-static bool launch_plain_fmt(const uint8_t* w, size_t bpr, const ActQ8& a, float* y, size_t in_f,
-                             size_t out_f, const IntStages& st, hipStream_t stream) {
-    const int steps = (int)((in_f + F::kElemsPerStep - 1) / F::kElemsPerStep);
-    const int n_units = (int)(in_f / F::kBlockElems);
-    // Rows per wavefront: enough waves to cover the machine several times over.
-    static const int env_rpw = getenv("INFR_HIP_BATCH_ROWS") ? atoi(getenv("INFR_HIP_BATCH_ROWS")) : 0;
-    size_t rpw = (out_f + 4095) / 4096;
-    rpw = rpw < 2 ? 2 : (rpw > 16 ? 16 : rpw);
-    if (env_rpw > 0) rpw = (size_t)env_rpw;
-    const size_t waves = (out_f + rpw - 1) / rpw;
-    const dim3 grid((unsigned)((waves + 3) / 4));
-    const ActPtrs act{a.qs, a.d, a.bsums, a.bsums16};
-    const StagePtrs sp{st.a, st.b};
-    return st.a ? launch_plain<F, true>(steps, grid, stream, w, bpr, act, y, n_units, (int)out_f, (int)rpw, sp)
-                : launch_plain<F, false>(steps, grid, stream, w, bpr, act, y, n_units, (int)out_f, (int)rpw, sp);
 }
 
 bool launch_gemv(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t in_f,
                  size_t out_f, const IntStages& st, hipStream_t stream) {
     if (out_f == 0) return true;
-    switch (dtype) {
-    case 12: return launch_plain_fmt<FmtQ4K>(w, bpr, act, y, in_f, out_f, st, stream);
-    case 14: return launch_plain_fmt<FmtQ6K>(w, bpr, act, y, in_f, out_f, st, stream);
-    case 8:
-        return in_f % 256 == 0 ? launch_plain_fmt<FmtQ8_0>(w, bpr, act, y, in_f, out_f, st, stream) : launch_plain_fmt<FmtQ8_0_32>(w, bpr, act, y, in_f, out_f, st, stream);
-    case 42: return launch_plain_fmt<FmtQ2_0>(w, bpr, act, y, in_f, out_f, st, stream);
-    default: return false;
-    }
-}
-
-template <typename F, int STEPS, int MB>
-static void launch_batch_one(const uint8_t* w, size_t bpr, const ActPtrs& act, int m_valid, size_t in_f,
-                             float* y, size_t out_f, const StagePtrs& st, hipStream_t stream) {
-    static const int env_rpw = getenv("INFR_HIP_BATCH_ROWS") ? atoi(getenv("INFR_HIP_BATCH_ROWS")) : 0;
-    size_t rpw = (out_f + 4095) / 4096;
-    rpw = rpw < 2 ? 2 : (rpw > 16 ? 16 : rpw);
-    if (env_rpw > 0) rpw = (size_t)env_rpw;
-    const size_t waves = (out_f + rpw - 1) / rpw;
-    const dim3 grid((unsigned)((waves + 3) / 4)), block(256);
-    if (st.a)
-        hipLaunchKernelGGL((gemv_batch_kernel<F, STEPS, MB, true>), grid, block, 0, stream, w, bpr, act,
-                           m_valid, (int)in_f, y, (int)out_f, (int)rpw, st, (const BatchTile*)nullptr);
-    else
-        hipLaunchKernelGGL((gemv_batch_kernel<F, STEPS, MB, false>), grid, block, 0, stream, w, bpr, act,
-                           m_valid, (int)in_f, y, (int)out_f, (int)rpw, st, (const BatchTile*)nullptr);
-}
-
-// Activation rows per pass of the batch kernel (they live in registers).
-static int batch_rows_per_pass(int steps) { return steps == 1 ? 8 : (steps == 2 ? 4 : (steps <= 4 ? 2 : 1)); }
-
-template <typename F, int STEPS, int MB>
-static void launch_batch_group_one(const BatchTile* tiles, const BatchGroupPlan& gp, const ActPtrs& act,
-                                   int m, size_t in_f, hipStream_t stream) {
-    const dim3 grid((unsigned)gp.total_wgs, (unsigned)((m + MB - 1) / MB)), block(256);
-    hipLaunchKernelGGL((gemv_batch_kernel<F, STEPS, MB, false>), grid, block, 0, stream,
-                       (const uint8_t*)nullptr, (size_t)0, act, m, (int)in_f, (float*)nullptr, 0,
-                       gp.rows_per_wave, StagePtrs{nullptr, nullptr}, tiles);
-}
-
-template <typename F>
-static bool launch_batch_group_fmt(const BatchTile* tiles, const BatchGroupPlan& gp, const ActQ8& a,
-                                   size_t m, size_t in_f, hipStream_t stream) {
-    const int steps = (int)((in_f + F::kElemsPerStep - 1) / F::kElemsPerStep);
-    const ActPtrs act{a.qs, a.d, a.bsums, a.bsums16};
-    const int mb = std::min((int)m, batch_rows_per_pass(steps));
-#define INFR_G(S, MB) launch_batch_group_one<F, S, MB>(tiles, gp, act, (int)m, in_f, stream)
-    switch (steps) {
-    case 1: if (mb > 4) INFR_G(1, 8); else if (mb > 2) INFR_G(1, 4); else INFR_G(1, 2); break;
-    case 2: if (mb > 2) INFR_G(2, 4); else INFR_G(2, 2); break;
-    case 3: INFR_G(3, 2); break;
-    case 4: INFR_G(4, 2); break;
-    case 5: INFR_G(5, 1); break;
-    case 6: INFR_G(6, 1); break;
-    case 7: INFR_G(7, 1); break;
-    case 8: INFR_G(8, 1); break;
-    default: return false;
-    }
-#undef INFR_G
-    return true;
+    const GemvFormatOps* f = format_ops(dtype, in_f);
+    return f && f->plain && f->plain(w, bpr, act, y, in_f, out_f, st, stream);
 }
 
 bool launch_gemv_batch_group(int dtype, size_t m, size_t in_f, const BatchTile* tiles_dev,
                              const BatchGroupPlan& plan, const ActQ8& act, hipStream_t stream) {
-    switch (dtype) {
-    case 12: return launch_batch_group_fmt<FmtQ4K>(tiles_dev, plan, act, m, in_f, stream);
-    case 14: return launch_batch_group_fmt<FmtQ6K>(tiles_dev, plan, act, m, in_f, stream);
-    case 8:
-        return in_f % 256 == 0 ? launch_batch_group_fmt<FmtQ8_0>(tiles_dev, plan, act, m, in_f, stream) : launch_batch_group_fmt<FmtQ8_0_32>(tiles_dev, plan, act, m, in_f, stream);
-    case 42: return launch_batch_group_fmt<FmtQ2_0>(tiles_dev, plan, act, m, in_f, stream);
-    default: return false;
-    }
+    const GemvFormatOps* f = format_ops(dtype, in_f);
+    return f && f->batch_group(tiles_dev, plan, act, m, in_f, stream);
 }
 
 bool plan_batch_group(int dtype, size_t m, size_t in_f, const GemvOpDesc* ops, int n, BatchGroupPlan* plan) {
@@ -361,8 +67,9 @@ bool plan_batch_group(int dtype, size_t m, size_t in_f, const GemvOpDesc* ops, i
         const size_t wgs = (total_rows + 31) / 32;
         gp.waves = (in_f >= 8192 || (wgs * 4 < 1024 && in_f >= 2048)) ? 8 : 4;
     } else {
-        if (dtype != 14 && dtype != 8 && dtype != 42) return false;
-        const size_t per_step = dtype == 8 ? 2048 : 4096;
+        const GemvFormatOps* f = format_ops(dtype, in_f);
+        if (!f) return false;
+        const size_t per_step = (size_t)f->elems_per_step;
         const size_t steps = (in_f + per_step - 1) / per_step;
         if (steps < 1 || steps > 8 || m > 8) return false;
         size_t rpw = (total_rows + 4095) / 4096;
@@ -387,173 +94,17 @@ void fill_batch_tiles(const GemvOpDesc* ops, const uint32_t* act_elem0, int n, c
                                  (uint32_t)ops[i].bpr};
 }
 
-// m activation rows in chunks of MB <= 8 / STEPS (the activations live in registers).
-template <typename F>
-static bool launch_batch_fmt(const uint8_t* w, size_t bpr, const ActQ8& a, float* y, size_t m,
-                             size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream) {
-    const int steps = (int)((in_f + F::kElemsPerStep - 1) / F::kElemsPerStep);
-    if (steps < 1 || steps > 8) return false;
-    const size_t dper = F::kPer32 ? in_f / 32 : in_f / 256;
-    const size_t blocks = (F::kBlockElems == 64 ? 2 : 1) * (in_f / F::kBlockElems);
-    const size_t mb_max = (size_t)batch_rows_per_pass(steps);
-    for (size_t r0 = 0; r0 < m; r0 += mb_max) {
-        const int mv = (int)std::min(mb_max, m - r0);
-        const ActPtrs act{a.qs + r0 * in_f, a.d + r0 * dper, a.bsums + r0 * (in_f / 32),
-                          a.bsums16 ? a.bsums16 + r0 * (in_f / 16) : nullptr};
-        const StagePtrs sp{st.a ? st.a + r0 * out_f * blocks : nullptr,
-                           st.b ? st.b + r0 * out_f * blocks : nullptr};
-        float* yo = y + r0 * out_f;
-#define INFR_B(S, MB) launch_batch_one<F, S, MB>(w, bpr, act, mv, in_f, yo, out_f, sp, stream)
-        switch (steps) {
-        case 1: if (mv > 4) INFR_B(1, 8); else if (mv > 2) INFR_B(1, 4); else if (mv > 1) INFR_B(1, 2); else INFR_B(1, 1); break;
-        case 2: if (mv > 2) INFR_B(2, 4); else if (mv > 1) INFR_B(2, 2); else INFR_B(2, 1); break;
-        case 3: if (mv > 1) INFR_B(3, 2); else INFR_B(3, 1); break;
-        case 4: if (mv > 1) INFR_B(4, 2); else INFR_B(4, 1); break;
-        case 5: INFR_B(5, 1); break;
-        case 6: INFR_B(6, 1); break;
-        case 7: INFR_B(7, 1); break;
-        default: INFR_B(8, 1); break;
-        }
-#undef INFR_B
-    }
-    return true;
-}
-
 bool launch_gemv_batch(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
                        size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream) {
     if (out_f == 0 || m == 0) return true;
-    switch (dtype) {
-    case 12: return launch_batch_fmt<FmtQ4K>(w, bpr, act, y, m, in_f, out_f, st, stream);
-    case 14: return launch_batch_fmt<FmtQ6K>(w, bpr, act, y, m, in_f, out_f, st, stream);
-    case 8:
-        return in_f % 256 == 0 ? launch_batch_fmt<FmtQ8_0>(w, bpr, act, y, m, in_f, out_f, st, stream) : launch_batch_fmt<FmtQ8_0_32>(w, bpr, act, y, m, in_f, out_f, st, stream);
-    case 42: return launch_batch_fmt<FmtQ2_0>(w, bpr, act, y, m, in_f, out_f, st, stream);
-    default: return false;
-    }
-}
-
-// Largest workgroup (in waves) whose register budget the kernel fits without spilling: 16 waves
-// per workgroup leave 128 VGPRs per lane, 8 waves 256 (from the compiler's resource report).
-template <typename F> static int max_waves_per_wg(int steps);
-template <> int max_waves_per_wg<FmtQ4K>(int steps) { return steps <= 3 ? 16 : 8; }
-template <> int max_waves_per_wg<FmtQ6K>(int steps) { return steps <= 1 ? 16 : 8; }
-template <> int max_waves_per_wg<FmtQ8_0>(int steps) { return steps <= 4 ? 16 : 8; }
-template <> int max_waves_per_wg<FmtQ8_0_32>(int steps) { return steps <= 4 ? 16 : 8; }
-template <> int max_waves_per_wg<FmtQ2_0>(int steps) { return steps <= 3 ? 16 : 8; }
-
-// Workgroups of the fused kernel that one compute unit holds at once (registers, LDS, wave slots),
-// as the runtime computes it for the exact instantiation; 0 if the query fails.
-template <typename F, int NW>
-static int fused_wgs_per_cu_nw(int steps, size_t lds_bytes) {
-    int nblk = 0;
-#define INFR_CASE(N)                                                                                  \
-    case N:                                                                                           \
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(                                             \
-                &nblk, reinterpret_cast<const void*>(&gemv_fused_kernel<F, N, NW>), NW * 64, lds_bytes) != hipSuccess) \
-            nblk = 0;                                                                                 \
-        break;
-    switch (steps) {
-        INFR_CASE(1) INFR_CASE(2) INFR_CASE(3) INFR_CASE(4)
-        INFR_CASE(5) INFR_CASE(6) INFR_CASE(7) INFR_CASE(8)
-    default: break;
-    }
-#undef INFR_CASE
-    return nblk;
-}
-template <typename F>
-static int fused_wgs_per_cu(int steps, int nw, size_t lds_bytes) {
-    switch (nw) {
-    case 4: return fused_wgs_per_cu_nw<F, 4>(steps, lds_bytes);
-    case 8: return fused_wgs_per_cu_nw<F, 8>(steps, lds_bytes);
-    case 16: return fused_wgs_per_cu_nw<F, 16>(steps, lds_bytes);
-    default: return 0;
-    }
-}
-static int device_cu_count() {
-    static const int cus = [] {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess ||
-            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
-            n = 0;
-        return n;
-    }();
-    return cus;
-}
-
-template <typename F>
-static bool plan_group_fmt(size_t in_f, const GemvOpDesc* ops, int n, GemvGroupPlan* plan) {
-    const int steps = (int)((in_f + F::kElemsPerStep - 1) / F::kElemsPerStep);
-    if (steps < 1 || steps > 8) return false;
-    size_t total_rows = 0;
-    for (int i = 0; i < n; ++i) total_rows += (size_t)ops[i].out_f;
-    // Every workgroup re-quantizes x (about the arithmetic of eleven weight rows at in_f 4096), so
-    // big groups take up to 128 rows per workgroup (more than that loses to the uneven tail);
-    // small ones keep at least ~512 workgroups in flight. The workgroup is always as wide as the register budget allows, so that the
-    // quantization is spread over the most waves; waves beyond the tile's rows retire after it.
-    int nw = max_waves_per_wg<F>(steps);
-    if (steps >= 3 && nw > 8) nw = 8;  // long rows: 8-wave workgroups measured faster
-    // Tuning knobs (the reference exposes its kernel-shape choices the same way,
-    // kernels.vulkan.* in crates/infr-core/src/config/mod.rs:210-358).
-    static const int env_nw = getenv("INFR_HIP_GEMV_WAVES") ? atoi(getenv("INFR_HIP_GEMV_WAVES")) : 0;
-    static const int env_rows = getenv("INFR_HIP_GEMV_ROWS") ? atoi(getenv("INFR_HIP_GEMV_ROWS")) : 0;
-    if ((env_nw == 4 || env_nw == 8 || env_nw == 16) && env_nw <= nw) nw = env_nw;
-    size_t rows_per_wg = (total_rows + 511) / 512;
-    rows_per_wg = rows_per_wg < 4 ? 4 : (rows_per_wg > 128 ? 128 : rows_per_wg);
-    const size_t lds_bytes = in_f + in_f / 2 + (F::kOrdered ? (size_t)nw * (16 * (16 * steps + 4)) * sizeof(float) : 0);
-    // Grids of only a few rounds: a grid that needs a little more than a whole number of rounds
-    // idles most of the machine during the last one, and workgroups that share a compute unit
-    // share its pipes, so what counts is workgroups per compute unit. For those grids take, among
-    // tile heights near the one above, the one with the least modelled time
-    // ceil(workgroups / CUs) x (rows + fixed cost); the fixed cost is the per-workgroup prologue
-    // in units of a weight row: about eleven for quantizing x, more when the prologue also
-    // evaluates an absorbed gated activation (expf per element) or RmsNorm. Grids of many rounds
-    // keep the 128-row tiles: their tail is small and taller tiles measured slower.
-    static const int env_model = getenv("INFR_HIP_GEMV_ROUNDS") ? atoi(getenv("INFR_HIP_GEMV_ROUNDS")) : 1;
-    const int resident = device_cu_count() * fused_wgs_per_cu<F>(steps, nw, lds_bytes);
-    const int cus = device_cu_count();
-    double fixed = 11.0;
-    for (int i = 0; i < n; ++i)
-        fixed = std::max(fixed, ops[i].fus.pre == 1 ? 32.0 : (ops[i].fus.pre == 2 ? 15.0 : 11.0));
-    auto wgs_at = [&](size_t r) {
-        size_t w = 0;
-        for (int i = 0; i < n; ++i) w += ((size_t)ops[i].out_f + r - 1) / r;
-        return w;
-    };
-    if (env_model && resident > 0 && wgs_at(rows_per_wg) < (size_t)resident * 4) {
-        const size_t lo = std::max<size_t>(4, rows_per_wg / 2), hi = std::max<size_t>(rows_per_wg * 2, 160);
-        double best = 1e300;
-        size_t best_r = rows_per_wg;
-        for (size_t r = lo; r <= hi; ++r) {
-            const size_t rounds = (wgs_at(r) + cus - 1) / cus;
-            const double cost = (double)rounds * ((double)r + fixed);
-            if (cost < best * 0.999) {  // ties go to the smaller tile
-                best = cost;
-                best_r = r;
-            }
-        }
-        rows_per_wg = best_r;
-    }
-    if (env_rows >= 1 && env_rows <= 4096) rows_per_wg = (size_t)env_rows;
-    int wg = 0;
-    for (int i = 0; i < n; ++i) wg += (int)(((size_t)ops[i].out_f + rows_per_wg - 1) / rows_per_wg);
-    plan->total_wgs = wg;
-    plan->waves_per_wg = nw;
-    plan->rows_per_wg = (int)rows_per_wg;
-    // qs + d + bsums + bsums16, then the ordered-sum scratch of every wave
-    plan->lds_bytes = lds_bytes;
-    return true;
+    const GemvFormatOps* f = format_ops(dtype, in_f);
+    return f && f->batch(w, bpr, act, y, m, in_f, out_f, st, stream);
 }
 
 bool plan_gemv_group(int dtype, size_t in_f, const GemvOpDesc* ops, int n, GemvGroupPlan* plan) {
     if (n <= 0) return false;
-    switch (dtype) {
-    case 12: return plan_group_fmt<FmtQ4K>(in_f, ops, n, plan);
-    case 14: return plan_group_fmt<FmtQ6K>(in_f, ops, n, plan);
-    case 8:
-        return in_f % 256 == 0 ? plan_group_fmt<FmtQ8_0>(in_f, ops, n, plan) : plan_group_fmt<FmtQ8_0_32>(in_f, ops, n, plan);
-    case 42: return plan_group_fmt<FmtQ2_0>(in_f, ops, n, plan);
-    default: return false;
-    }
+    const GemvFormatOps* f = format_ops(dtype, in_f);
+    return f && f->plan_group && f->plan_group(in_f, ops, n, plan);
 }
 
 void fill_gemv_tiles(const GemvOpDesc* ops, int n, const GemvGroupPlan& plan, GemvTile* tiles) {
@@ -576,54 +127,13 @@ void fill_gemv_tiles(const GemvOpDesc* ops, int n, const GemvGroupPlan& plan, Ge
         }
 }
 
-static bool bpr_too_big(const GemvOpDesc* ops, int n) {
-    for (int i = 0; i < n; ++i)
-        if (ops[i].bpr > 0xFFFFFFFFull) return true;
-    return false;
-}
-
-template <typename F, int NW>
-static bool launch_fused_nw(int steps, size_t in_f, const GemvOpDesc& op, const GemvTile* tiles_dev,
-                            const GemvGroupPlan& plan, hipStream_t stream) {
-    const dim3 grid((unsigned)plan.total_wgs), block(NW * 64);
-#define INFR_CASE(N)                                                                          \
-    case N:                                                                                   \
-        hipLaunchKernelGGL((gemv_fused_kernel<F, N, NW>), grid, block, plan.lds_bytes, stream, \
-                           op, plan.rows_per_wg, tiles_dev, (int)in_f);                     \
-        return true;
-    switch (steps) {
-        INFR_CASE(1) INFR_CASE(2) INFR_CASE(3) INFR_CASE(4)
-        INFR_CASE(5) INFR_CASE(6) INFR_CASE(7) INFR_CASE(8)
-    default: return false;
-    }
-#undef INFR_CASE
-}
-
-template <typename F>
-static bool launch_fused_fmt(size_t in_f, const GemvOpDesc& op, const GemvTile* tiles_dev,
-                             const GemvGroupPlan& plan, hipStream_t stream) {
-    const int steps = (int)((in_f + F::kElemsPerStep - 1) / F::kElemsPerStep);
-    switch (plan.waves_per_wg) {
-    case 4: return launch_fused_nw<F, 4>(steps, in_f, op, tiles_dev, plan, stream);
-    case 8: return launch_fused_nw<F, 8>(steps, in_f, op, tiles_dev, plan, stream);
-    case 16: return launch_fused_nw<F, 16>(steps, in_f, op, tiles_dev, plan, stream);
-    default: return false;
-    }
-}
-
 bool launch_gemv_fused(int dtype, size_t in_f, const GemvOpDesc* ops, int n, const GemvTile* tiles_dev,
                        const GemvGroupPlan& plan, hipStream_t stream) {
     if (n <= 0 || plan.total_wgs <= 0) return n == 0;
     if (n > 1 && tiles_dev == nullptr) return false;
     if (bpr_too_big(ops, n)) return false;
-    switch (dtype) {
-    case 12: return launch_fused_fmt<FmtQ4K>(in_f, ops[0], tiles_dev, plan, stream);
-    case 14: return launch_fused_fmt<FmtQ6K>(in_f, ops[0], tiles_dev, plan, stream);
-    case 8:
-        return in_f % 256 == 0 ? launch_fused_fmt<FmtQ8_0>(in_f, ops[0], tiles_dev, plan, stream) : launch_fused_fmt<FmtQ8_0_32>(in_f, ops[0], tiles_dev, plan, stream);
-    case 42: return launch_fused_fmt<FmtQ2_0>(in_f, ops[0], tiles_dev, plan, stream);
-    default: return false;
-    }
+    const GemvFormatOps* f = format_ops(dtype, in_f);
+    return f && f->fused && f->fused(in_f, ops[0], tiles_dev, plan, stream);
 }
 
 }  // namespace infr

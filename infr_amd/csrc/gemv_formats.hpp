@@ -3,12 +3,17 @@
 // Each format follows infr-cpu's scalar kernel for one block:
 //   Q4_K  crates/infr-cpu/src/kernels.rs:151-184     Q6_K  kernels.rs:487-526
 //   Q8_0  kernels.rs:1170-1187                       Q2_0  kernels.rs:5641-5668
+//   Q5_K  kernels.rs:1286-1327
+//   Q4_0  kernels.rs:5496-5520   Q4_1  :5793-5822    Q5_0  :5350-5377   Q5_1  :5948-5980
+//   IQ4_NL  kernels.rs:6128-6152
 //
 // Interface of a format policy F (all members static, `t` = wave step, `lane` = 0..63):
 //   kElemsPerStep         K elements one wave step covers
 //   kPer32                activation quantizer: per-32 (true) or per-256 (false)
 //   kOrdered              per-block terms are added in ascending block order (bit-exact with the
 //                         CPU's `sumf +=` chain) instead of a butterfly
+//   kWide16Steps          up to this many wave steps per row the fused kernel fits 16 waves per
+//                         workgroup (128 VGPRs per lane) without spilling; beyond it, 8 waves
 //   units(in_f)           number of lane work units in a row (blocks for Q4_K/Q6_K ...)
 //   Row / Acts            registers for one step of a weight row / of the activation
 //   valid(t, lane, n)     does this lane have work in step t
@@ -43,6 +48,7 @@ struct FmtQ4K {
     static constexpr bool kPer32 = false;
     static constexpr bool kOrdered = true;
     static constexpr int kBlockBytes = 144, kBlockElems = 256;
+    static constexpr int kWide16Steps = 3;
     struct Row {
         v4i hdr, qa, qb;
     };
@@ -132,6 +138,7 @@ struct FmtQ6K {
     static constexpr bool kPer32 = false;
     static constexpr bool kOrdered = true;
     static constexpr int kBlockBytes = 210, kBlockElems = 256;
+    static constexpr int kWide16Steps = 1;
     struct Row {
         v4i qla, qlb, qh;
         v2i sc;
@@ -224,6 +231,7 @@ struct FmtQ8_0T {
     static constexpr bool kPer32 = P32;
     static constexpr bool kOrdered = false;
     static constexpr int kBlockBytes = 34, kBlockElems = 32;
+    static constexpr int kWide16Steps = 4;
     struct Row {
         v4i qa, qb;
         uint32_t d;
@@ -321,6 +329,7 @@ struct FmtQ2_0 {
     static constexpr bool kPer32 = true;
     static constexpr bool kOrdered = false;
     static constexpr int kBlockBytes = 18, kBlockElems = 64;
+    static constexpr int kWide16Steps = 3;
     struct Row {
         v4i codes;
         uint32_t d;
@@ -357,7 +366,10 @@ struct FmtQ2_0 {
         } else {
 #pragma unroll
             for (int k = 0; k < 16; ++k) a.xt[k] = 0;
-            a.da0 = a.da1 = a.fb0 = a.fb1 = 0.0f;
+            a.da0 = 0.0f;
+            a.da1 = 0.0f;
+            a.fb0 = 0.0f;
+            a.fb1 = 0.0f;
         }
     }
     template <bool STAGES>
@@ -385,5 +397,214 @@ struct FmtQ2_0 {
         return s;
     }
 };
+
+// ───────────────────────────────────── Q5_K ─────────────────────────────────────
+// Q4_K's lane mapping (block-in-step q = l/4, nibble pair p = l%4) on the 176-byte block
+// [f16 d][f16 dmin][u8 scales[12]][u8 qh[32]][u8 ql[128]]: the 5th code bit of sub-block s,
+// element l, is bit s of qh[l], so pair p takes bits 2p (even sub-block) and 2p+1 (odd) of the 32
+// qh bytes, which all four lanes of the quad load (same cache lines). Block stride 176 B is a
+// multiple of 16: every load is 16-byte aligned.
+struct FmtQ5K {
+    static constexpr int kElemsPerStep = 4096;
+    static constexpr bool kPer32 = false;
+    static constexpr bool kOrdered = true;
+    static constexpr int kBlockBytes = 176, kBlockElems = 256;
+    static constexpr int kWide16Steps = 2;
+    struct Row {
+        v4i hdr, ha, hb, qa, qb;
+    };
+    typedef FmtQ4K::Acts Acts;
+    __device__ static int units(int in_f) { return in_f / 256; }
+    __device__ static bool valid(int t, int lane, int n) { return t * 16 + (lane >> 2) < n; }
+    __device__ static void load_row(Row& r, const uint8_t* rowp, int t, int lane, bool ok) {
+        if (ok) {
+            const uint8_t* blk = rowp + (size_t)(t * 16 + (lane >> 2)) * 176;
+            const int p = lane & 3;
+            r.hdr = load16(blk);
+            r.ha = load16(blk + 16);
+            r.hb = load16(blk + 32);
+            r.qa = load16(blk + 48 + p * 32);
+            r.qb = load16(blk + 64 + p * 32);
+        } else {
+            r.hdr = r.ha = r.hb = r.qa = r.qb = v4i{0, 0, 0, 0};
+        }
+    }
+    __device__ static void load_acts(Acts& a, const ActPtrs& s, int t, int lane, bool ok) {
+        FmtQ4K::load_acts(a, s, t, lane, ok);
+    }
+    template <bool STAGES>
+    __device__ static float term(const Row& r, const Acts& a, int t, int lane, bool ok,
+                                 const StagePtrs& st, size_t row_units) {
+        const int p = lane & 3;
+        const uint32_t m4 = 0x0F0F0F0Fu, b1 = 0x01010101u;
+        int ip_e = 0, ip_o = 0;
+        const int wq[8] = {r.qa.x, r.qa.y, r.qa.z, r.qa.w, r.qb.x, r.qb.y, r.qb.z, r.qb.w};
+        const int hq[8] = {r.ha.x, r.ha.y, r.ha.z, r.ha.w, r.hb.x, r.hb.y, r.hb.z, r.hb.w};
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const uint32_t w = (uint32_t)wq[k], h = (uint32_t)hq[k] >> (2 * p);
+            ip_e = dot4((int)((w & m4) | ((h & b1) << 4)), a.xa[k], ip_e);
+            ip_o = dot4((int)(((w >> 4) & m4) | (((h >> 1) & b1) << 4)), a.xa[8 + k], ip_o);
+        }
+        uint32_t sc8[2], mn8[2];
+        k4_all((uint32_t)r.hdr.y, (uint32_t)r.hdr.z, (uint32_t)r.hdr.w, sc8, mn8);
+        const uint32_t scw = (p & 2) ? sc8[1] : sc8[0];
+        const uint32_t mnw = (p & 2) ? mn8[1] : mn8[0];
+        const int sh = (p & 1) * 16;
+        const int sc_e = (scw >> sh) & 0xFF, sc_o = (scw >> (sh + 8)) & 0xFF;
+        const int m_e = (mnw >> sh) & 0xFF, m_o = (mnw >> (sh + 8)) & 0xFF;
+        // |ip| <= 32 * 31 * 127 < 2^17 and sc < 2^6: the 24-bit multiply is exact
+        const int sd = quad_sum(__mul24(sc_e, ip_e) + __mul24(sc_o, ip_o));
+        const int sm = quad_sum(__mul24(m_e, a.bs0) + __mul24(m_o, a.bs1));
+        if (STAGES && ok && p == 0) {
+            st.a[row_units + t * 16 + (lane >> 2)] = sd;
+            st.b[row_units + t * 16 + (lane >> 2)] = sm;
+        }
+        const float d = f16_bits_to_f32((uint32_t)r.hdr.x & 0xFFFFu);
+        const float dmin = f16_bits_to_f32((uint32_t)r.hdr.x >> 16);
+        // sumf += q8.d[b] * (d * sd as f32 - dmin * sm as f32)
+        return a.dact * (d * (float)sd - dmin * (float)sm);
+    }
+};
+
+// ───────────────── Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL: 32 weights per block ─────────────────
+// Lane l owns block t*64 + l of the row: an f16 scale (plus an f16 min for the _1 formats, plus a
+// 32-bit mask of 5th code bits for the Q5 formats) and 16 bytes of nibbles. Byte j holds element j
+// in its low nibble and element j+16 in its high nibble, so `w & 0x0F0F0F0F` and `(w >> 4) & ...`
+// of the four nibble words are ready v_dot4 operands against activation words 0..3 and 4..7. The
+// 5th bits of four consecutive elements are spread from the mask to bit 4 of four bytes with one
+// multiply; IQ4_NL's nibbles index a 16-entry signed table through two v_perm_b32 and a select.
+// Against the per-32 activation (scale and code sum per block). 64 blocks (2048 weights) per wave
+// step. Strides 18 and 22 are 2 mod 4: those blocks are fetched as dwords from the 4-byte boundary
+// at or below the block and realigned in registers (realign2); strides 20 and 24 are dword-aligned.
+enum class Nib32 { Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL };
+
+__device__ __forceinline__ uint32_t spread4_to_bit4(uint32_t bits) {
+    // bits 0..3 -> bit 4 of bytes 0..3 (the four partial products land on distinct bits)
+    return (__umul24(bits & 0xFu, 0x00204081u) & 0x01010101u) << 4;
+}
+
+// KVALUES_IQ4NL (crates/infr-gguf/src/dequant.rs:439-441) as four little-endian words of int8.
+__device__ __forceinline__ int iq4nl_lookup(uint32_t nib) {
+    const uint32_t sel = nib & 0x07070707u;
+    const uint32_t lo = __builtin_amdgcn_perm(0xF6EADDCFu, 0xBFAD9881u, sel);  // entries 0..7
+    const uint32_t hi = __builtin_amdgcn_perm(0x71594535u, 0x26190D01u, sel);  // entries 8..15
+    const uint32_t pick = ((nib >> 3) & 0x01010101u) * 0xFFu;                  // 0xFF where nibble >= 8
+    return (int)((hi & pick) | (lo & ~pick));
+}
+
+template <Nib32 K>
+struct FmtNib32 {
+    static constexpr bool kAffine = K == Nib32::Q4_1 || K == Nib32::Q5_1;
+    static constexpr bool kFive = K == Nib32::Q5_0 || K == Nib32::Q5_1;
+    static constexpr int kElemsPerStep = 2048;
+    static constexpr bool kPer32 = true;
+    static constexpr bool kOrdered = false;
+    static constexpr int kBlockBytes = 18 + (kAffine ? 2 : 0) + (kFive ? 4 : 0), kBlockElems = 32;
+    static constexpr int kWide16Steps = 4;
+    struct Row {
+        v4i qs;
+        uint32_t dm;  // f16 d in the low half, f16 m (affine formats) in the high half
+        uint32_t qh;
+    };
+    struct Acts {
+        int xa[8];
+        float dact, fbs;
+    };
+    __device__ static int units(int in_f) { return in_f / 32; }
+    __device__ static bool valid(int t, int lane, int n) { return t * 64 + lane < n; }
+    __device__ static void load_row(Row& r, const uint8_t* rowp, int t, int lane, bool ok) {
+        if (!ok) {
+            r.qs = v4i{0, 0, 0, 0};
+            r.dm = 0;
+            r.qh = 0;
+            return;
+        }
+        const uint8_t* blk = rowp + (size_t)(t * 64 + lane) * kBlockBytes;
+        if (kAffine) {
+            // [d m][qh][qs x4]: every field on a dword
+            uint32_t hdr;
+            __builtin_memcpy(&hdr, __builtin_assume_aligned(blk, 4), 4);
+            r.dm = hdr;
+            if (kFive) __builtin_memcpy(&r.qh, __builtin_assume_aligned(blk + 4, 4), 4);
+            else r.qh = 0;
+            r.qs = load16_a4(blk + (kFive ? 8 : 4));
+        } else {
+            // [d][qh?][qs x4] with the payload 2 bytes past the block start: dwords from the
+            // boundary at or below the block; an odd block (2 past a boundary) reads the 2 bytes
+            // before it, an even one stops at its own last 2 bytes.
+            const bool odd = (reinterpret_cast<uintptr_t>(blk) & 2) != 0;
+            const uint8_t* a = blk - (odd ? 2 : 0);
+            const uint32_t sel = realign2_selector(odd);
+            constexpr int kWords = kFive ? 5 : 4;  // payload dwords after the scale
+            int w[kWords + 1];
+            const v4i lo = load16_a4(a);
+            w[0] = lo.x; w[1] = lo.y; w[2] = lo.z; w[3] = lo.w;
+            if (kFive) __builtin_memcpy(&w[4], __builtin_assume_aligned(a + 16, 4), 4);
+            uint32_t tail = load_u16(a + 4 * kWords);
+            if (odd) tail |= load_u16(a + 4 * kWords + 2) << 16;
+            w[kWords] = (int)tail;
+            r.dm = odd ? (uint32_t)w[0] >> 16 : (uint32_t)w[0] & 0xFFFFu;
+            int pay[kWords];
+#pragma unroll
+            for (int k = 0; k < kWords; ++k) pay[k] = realign2(w[k], w[k + 1], sel);
+            r.qh = kFive ? (uint32_t)pay[0] : 0u;
+            r.qs = v4i{pay[kWords - 4], pay[kWords - 3], pay[kWords - 2], pay[kWords - 1]};
+        }
+    }
+    __device__ static void load_acts(Acts& a, const ActPtrs& s, int t, int lane, bool ok) {
+        if (ok) {
+            const int b = t * 64 + lane;
+            const v4i v0 = *reinterpret_cast<const v4i*>(s.qs + (size_t)b * 32);
+            const v4i v1 = *reinterpret_cast<const v4i*>(s.qs + (size_t)b * 32 + 16);
+            a.xa[0] = v0.x; a.xa[1] = v0.y; a.xa[2] = v0.z; a.xa[3] = v0.w;
+            a.xa[4] = v1.x; a.xa[5] = v1.y; a.xa[6] = v1.z; a.xa[7] = v1.w;
+            a.dact = s.d[b];
+            a.fbs = (float)s.bsums[b];
+        } else {
+#pragma unroll
+            for (int k = 0; k < 8; ++k) a.xa[k] = 0;
+            a.dact = 0.0f;
+            a.fbs = 0.0f;
+        }
+    }
+    template <bool STAGES>
+    __device__ static float term(const Row& r, const Acts& a, int t, int lane, bool ok,
+                                 const StagePtrs& st, size_t row_units) {
+        const uint32_t m4 = 0x0F0F0F0Fu;
+        const int qw[4] = {r.qs.x, r.qs.y, r.qs.z, r.qs.w};
+        int ip = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t w = (uint32_t)qw[k];
+            uint32_t lo = w & m4, hi = (w >> 4) & m4;
+            if (K == Nib32::IQ4_NL) {
+                lo = (uint32_t)iq4nl_lookup(lo);
+                hi = (uint32_t)iq4nl_lookup(hi);
+            }
+            if (kFive) {
+                lo |= spread4_to_bit4(r.qh >> (4 * k));
+                hi |= spread4_to_bit4(r.qh >> (16 + 4 * k));
+            }
+            ip = dot4((int)lo, a.xa[k], ip);
+            ip = dot4((int)hi, a.xa[4 + k], ip);
+        }
+        if (STAGES && ok) st.a[row_units + t * 64 + lane] = ip;
+        const float d = f16_bits_to_f32(r.dm & 0xFFFFu);
+        if (kAffine) {
+            // sumf += q8.d[b] * (d * iprod as f32 + m * q8.bsum[b] as f32)
+            const float mw = f16_bits_to_f32(r.dm >> 16);
+            return a.dact * (d * (float)ip + mw * a.fbs);
+        }
+        if (K == Nib32::IQ4_NL) return d * a.dact * (float)ip;  // d * q8.d[b] * iprod as f32
+        // sumf += d * q8.d[b] * (iprod as f32 - OFFSET * q8.bsum[b] as f32), OFFSET = 8 or 16
+        return d * a.dact * ((float)ip - (kFive ? 16.0f : 8.0f) * a.fbs);
+    }
+};
+using FmtQ4_0 = FmtNib32<Nib32::Q4_0>;
+using FmtQ4_1 = FmtNib32<Nib32::Q4_1>;
+using FmtQ5_0 = FmtNib32<Nib32::Q5_0>;
+using FmtQ5_1 = FmtNib32<Nib32::Q5_1>;
+using FmtIQ4NL = FmtNib32<Nib32::IQ4_NL>;
 
 }  // namespace infr

@@ -139,6 +139,48 @@ bool launch_gemv_batch_group(int dtype, size_t m, size_t in_f, const BatchTile* 
 void launch_mmq_skinny_group(size_t m, size_t in_f, const BatchTile* tiles_dev, const BatchGroupPlan& plan,
                              const ActQ8& act, hipStream_t stream);
 
+// Which activation quantizer infr-cpu's dispatch pairs with a weight format
+// (crates/infr-cpu/src/lib.rs:1037-1076, 1322-1412): per-32 `Q8x32` for the 32-weight-block
+// formats and Q2_0, and for Q8_0 rows that are not whole 256s; per-256 `Q8` otherwise.
+inline bool act_is_per32(int dtype, size_t in_f) {
+    switch (dtype) {
+    case 2: case 3: case 6: case 7: case 20: case 42: return true;
+    case 8: return in_f % 256 != 0;
+    default: return false;
+    }
+}
+
+// One token of a format without an int8 decode arm multiplies f32 activations (gemv_f32act.hip).
+bool gemv_takes_f32_activations(int dtype, size_t m);
+bool launch_gemv_f32act(int dtype, const uint8_t* w, size_t bpr, const float* x, float* y, size_t in_f,
+                        size_t out_f, hipStream_t stream);
+
+// The decode-GEMV launchers of one weight format. Each format's kernels are instantiated in one
+// translation unit, which also defines its accessor below.
+struct GemvFormatOps {
+    int elems_per_step = 0;  // K elements one wave step covers
+    bool (*plain)(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t in_f, size_t out_f,
+                  const IntStages& st, hipStream_t stream) = nullptr;
+    bool (*batch)(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
+                  size_t out_f, const IntStages& st, hipStream_t stream) = nullptr;
+    bool (*batch_group)(const BatchTile* tiles, const BatchGroupPlan& plan, const ActQ8& act, size_t m,
+                        size_t in_f, hipStream_t stream) = nullptr;
+    bool (*plan_group)(size_t in_f, const GemvOpDesc* ops, int n, GemvGroupPlan* plan) = nullptr;
+    bool (*fused)(size_t in_f, const GemvOpDesc& op, const GemvTile* tiles_dev, const GemvGroupPlan& plan,
+                  hipStream_t stream) = nullptr;
+};
+const GemvFormatOps& gemv_ops_q4k();
+const GemvFormatOps& gemv_ops_q6k();
+const GemvFormatOps& gemv_ops_q8_0();
+const GemvFormatOps& gemv_ops_q8_0_32();
+const GemvFormatOps& gemv_ops_q2_0();
+const GemvFormatOps& gemv_ops_q5k();
+const GemvFormatOps& gemv_ops_q4_0();
+const GemvFormatOps& gemv_ops_q4_1();
+const GemvFormatOps& gemv_ops_q5_0();  // batch launchers only: one token takes the f32 kernel
+const GemvFormatOps& gemv_ops_q5_1();
+const GemvFormatOps& gemv_ops_iq4nl();
+
 // Elementwise ops either side of a Linear (elementwise.hip).
 struct GatedActShape {
     uint32_t rows, nff;

@@ -703,7 +703,7 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
         else launch_mmq_shared_q4k<1>(w, bpr, act, y, m, in_f, out_f, st, stream);
         return true;
     }
-    launch_quantize_q8(x, m, in_f, dtype == 42 || (dtype == 8 && in_f % 256 != 0), act, stream);
+    launch_quantize_q8(x, m, in_f, act_is_per32(dtype, in_f), act, stream);
     if (dtype != 12) return launch_gemv_batch(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
     if ((int)m <= env_skinny_max) {
         // four blocks per round; eight for long rows or when four would leave most SIMDs without a wave

@@ -1,6 +1,6 @@
 // Deterministic synthetic inputs (host only). The reference ships no weight quantizer: it only
 // reads GGUF, and its tests synthesize valid blocks (crates/infr-testkit/src/lib.rs:106-123).
-// These encoders turn N(0, sigma^2) draws into valid Q4_K / Q6_K / Q8_0 / Q2_0 blocks so that
+// These encoders turn N(0, sigma^2) draws into valid blocks of every format the kernels take, so that
 // benchmarks and parity tests on any machine see byte-identical weights. Any valid encoder works
 // for parity: CPU oracle and GPU consume the same bytes.
 //
@@ -205,6 +205,109 @@ void encode_q8_0(const float* x, uint8_t* blk) {
         blk[2 + i] = (uint8_t)(int8_t)(d > 0.0f ? clampi((int)std::lround(x[i] / d), -127, 127) : 0);
 }
 
+// 256 floats -> one 176-byte Q5_K block: Q4_K's construction on a 5-bit grid; the 5th code bit
+// of sub-block s goes to bit s of qh[l].
+void encode_q5k(const float* x, uint8_t* blk) {
+    float scale[8], minv[8];
+    float max_scale = 0.0f, max_min = 0.0f;
+    for (int s = 0; s < 8; ++s) {
+        float lo = 0.0f, hi = 0.0f;
+        for (int l = 0; l < 32; ++l) {
+            lo = std::min(lo, x[s * 32 + l]);
+            hi = std::max(hi, x[s * 32 + l]);
+        }
+        scale[s] = (hi - lo) / 31.0f;
+        minv[s] = -lo;
+        max_scale = std::max(max_scale, scale[s]);
+        max_min = std::max(max_min, minv[s]);
+    }
+    put_f16(blk, max_scale / 63.0f);
+    put_f16(blk + 2, max_min / 63.0f);
+    const float d = f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+    const float dmin = f16_to_f32((uint16_t)(blk[2] | (blk[3] << 8)));
+    int sc[8], mn[8];
+    for (int s = 0; s < 8; ++s) {
+        sc[s] = d > 0.0f ? clampi((int)std::lround(scale[s] / d), 0, 63) : 0;
+        mn[s] = dmin > 0.0f ? clampi((int)std::lround(minv[s] / dmin), 0, 63) : 0;
+    }
+    uint8_t* scales = blk + 4;
+    std::memset(scales, 0, 12);
+    for (int j = 0; j < 8; ++j) {
+        if (j < 4) {
+            scales[j] |= (uint8_t)sc[j];
+            scales[j + 4] |= (uint8_t)mn[j];
+        } else {
+            scales[j + 4] = (uint8_t)((sc[j] & 0xF) | ((mn[j] & 0xF) << 4));
+            scales[j - 4] |= (uint8_t)((sc[j] >> 4) << 6);
+            scales[j] |= (uint8_t)((mn[j] >> 4) << 6);
+        }
+    }
+    uint8_t* qh = blk + 16;
+    uint8_t* qs = blk + 48;
+    std::memset(qh, 0, 32 + 128);
+    for (int s = 0; s < 8; ++s) {
+        const float ws = d * (float)sc[s], wm = dmin * (float)mn[s];
+        for (int l = 0; l < 32; ++l) {
+            const int q = ws > 0.0f ? clampi((int)std::lround((x[s * 32 + l] + wm) / ws), 0, 31) : 0;
+            qs[(s / 2) * 32 + l] |= (uint8_t)((q & 0xF) << ((s & 1) * 4));
+            qh[l] |= (uint8_t)((q >> 4) << s);
+        }
+    }
+}
+
+// The 16-entry codebook of IQ4_NL (crates/infr-gguf/src/dequant.rs:439-441).
+const int kIq4nl[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+
+// 32 floats -> one block of a 32-weight format. Element j's code goes to the low nibble of qs[j],
+// element j+16's to the high nibble; the 5-bit formats put the 5th bit of element e in bit e of qh.
+//   Q4_0 [d][qs]: symmetric, code = round(x/d) + 8        Q5_0 [d][qh][qs]: ... + 16
+//   Q4_1 [d][m][qs]: affine on [min x, max x]             Q5_1 [d][m][qh][qs]
+//   IQ4_NL [d][qs]: nearest codebook value of x/d
+void encode_blk32(int dtype, const float* x, uint8_t* blk) {
+    const bool affine = dtype == INFR_DTYPE_Q4_1 || dtype == INFR_DTYPE_Q5_1;
+    const bool five = dtype == INFR_DTYPE_Q5_0 || dtype == INFR_DTYPE_Q5_1;
+    const int levels = five ? 32 : 16;
+    float lo = x[0], hi = x[0], amax = 0.0f;
+    for (int i = 0; i < 32; ++i) {
+        lo = std::min(lo, x[i]);
+        hi = std::max(hi, x[i]);
+        amax = std::max(amax, std::fabs(x[i]));
+    }
+    int code[32];
+    uint8_t* p = blk + 2;
+    if (affine) {
+        put_f16(blk, (hi - lo) / (float)(levels - 1));
+        put_f16(blk + 2, lo);
+        const float d = f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+        const float m = f16_to_f32((uint16_t)(blk[2] | (blk[3] << 8)));
+        for (int i = 0; i < 32; ++i)
+            code[i] = d > 0.0f ? clampi((int)std::lround((x[i] - m) / d), 0, levels - 1) : 0;
+        p = blk + 4;
+    } else if (dtype == INFR_DTYPE_IQ4_NL) {
+        put_f16(blk, amax / 127.0f);
+        const float d = f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+        for (int i = 0; i < 32; ++i) {
+            const float v = d > 0.0f ? x[i] / d : 0.0f;
+            int best = 0;
+            for (int c = 1; c < 16; ++c)
+                if (std::fabs(v - (float)kIq4nl[c]) < std::fabs(v - (float)kIq4nl[best])) best = c;
+            code[i] = best;
+        }
+    } else {
+        put_f16(blk, amax / (float)(levels / 2 - 1));
+        const float d = f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+        for (int i = 0; i < 32; ++i)
+            code[i] = (d > 0.0f ? clampi((int)std::lround(x[i] / d), -(levels / 2), levels / 2 - 1) : 0) + levels / 2;
+    }
+    if (five) {
+        uint32_t qh = 0;
+        for (int i = 0; i < 32; ++i) qh |= (uint32_t)(code[i] >> 4) << i;
+        std::memcpy(p, &qh, 4);
+        p += 4;
+    }
+    for (int j = 0; j < 16; ++j) p[j] = (uint8_t)((code[j] & 0xF) | ((code[j + 16] & 0xF) << 4));
+}
+
 template <typename F>
 void parallel_rows(size_t rows, F&& fn) {
     unsigned nt = std::thread::hardware_concurrency();
@@ -235,6 +338,12 @@ int infr_block_layout(int dtype, int* elems, int* bytes) {
     case INFR_DTYPE_Q4_K: e = 256; b = 144; break;
     case INFR_DTYPE_Q6_K: e = 256; b = 210; break;
     case INFR_DTYPE_Q2_0: e = 64; b = 18; break;
+    case INFR_DTYPE_Q4_0: e = 32; b = 18; break;
+    case INFR_DTYPE_Q4_1: e = 32; b = 20; break;
+    case INFR_DTYPE_Q5_0: e = 32; b = 22; break;
+    case INFR_DTYPE_Q5_1: e = 32; b = 24; break;
+    case INFR_DTYPE_Q5_K: e = 256; b = 176; break;
+    case INFR_DTYPE_IQ4_NL: e = 32; b = 18; break;
     default: return 0;
     }
     if (elems) *elems = e;
@@ -279,8 +388,10 @@ size_t infr_synth_weight(int dtype, uint64_t seed, float sigma, size_t rows, siz
             for (int i = 0; i < qpb; ++i) x[(size_t)i] = sigma * (float)g.next();
             uint8_t* blk = row + b * (size_t)bpb;
             if (dtype == INFR_DTYPE_Q4_K) encode_q4k(x.data(), blk);
+            else if (dtype == INFR_DTYPE_Q5_K) encode_q5k(x.data(), blk);
             else if (dtype == INFR_DTYPE_Q6_K) encode_q6k(x.data(), blk);
-            else encode_q8_0(x.data(), blk);
+            else if (dtype == INFR_DTYPE_Q8_0) encode_q8_0(x.data(), blk);
+            else encode_blk32(dtype, x.data(), blk);
         }
     });
     return rows * bpr;

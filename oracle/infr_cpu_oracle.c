@@ -14,14 +14,21 @@
 
 /* ───────────────────────────── block geometry ───────────────────────────── */
 
-/* crates/infr-core/src/decode_spec.rs:319-358: Q8_0 (32,34), Q4K (256,144), Q6K (256,210),
+/* crates/infr-core/src/decode_spec.rs:305-358: Q4_0 (32,18), Q4_1 (32,20), Q5_0 (32,22),
+ * Q5_1 (32,24), Q8_0 (32,34), Q4K (256,144), Q5K (256,176), Q6K (256,210), IQ4_NL (32,18),
  * Q2_0 (64,18). */
 int orc_block_layout(int dtype, int *elems, int *bytes) {
     int e = 0, b = 0;
     switch (dtype) {
     case ORC_F32: e = 1; b = 4; break;
     case ORC_F16: e = 1; b = 2; break;
+    case ORC_Q4_0: e = 32; b = 18; break;
+    case ORC_Q4_1: e = 32; b = 20; break;
+    case ORC_Q5_0: e = 32; b = 22; break;
+    case ORC_Q5_1: e = 32; b = 24; break;
+    case ORC_IQ4_NL: e = 32; b = 18; break;
     case ORC_Q8_0: e = 32; b = 34; break;
+    case ORC_Q5_K: e = 256; b = 176; break;
     case ORC_Q4_K: e = 256; b = 144; break;
     case ORC_Q6_K: e = 256; b = 210; break;
     case ORC_Q2_0: e = 64; b = 18; break;
@@ -111,6 +118,9 @@ void orc_k4(int j, const uint8_t *q, uint32_t *sc, uint32_t *m) {
 
 /* ───────────────────────────── host decode ───────────────────────────── */
 
+/* crates/infr-gguf/src/dequant.rs:439-441 */
+const int8_t orc_kvalues_iq4nl[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+
 /* crates/infr-gguf/src/dequant.rs:11-51: for affine quants the factored form is expanded as
  *   sc = f32(d) * (f32)scm_sc;  mn = f32(dmin) * (f32)scm_m;  out = sc * (f32)code + mn
  * (separate multiply and add). Factored arms: Q8_0 :209-219, Q4K :311-331, Q6K :361-385.
@@ -183,6 +193,73 @@ int orc_dequant_block(int dtype, const uint8_t *bytes, size_t nbytes, float *out
                         o[base + l + 32 * k] = sc * (float)c[k] + mn;
                     }
                 }
+            }
+        }
+        return 0;
+    case ORC_Q4_0:
+    case ORC_Q4_1:
+    case ORC_Q5_0:
+    case ORC_Q5_1:
+        /* dequant.rs:141-207: (scale, min) multipliers (1,-8) on (d,d) for Q4_0, (1,1) on (d,m) for
+         * Q4_1, (1,-16) on (d,d) for Q5_0, (1,1) on (d,m) for Q5_1; the 5th code bit of element j
+         * is qh bit j, of element j+16 qh bit j+16. */
+        for (size_t b = 0; b < nblk; b++) {
+            const uint8_t *blk = bytes + b * (size_t)bpb;
+            int affine = dtype == ORC_Q4_1 || dtype == ORC_Q5_1;
+            int five = dtype == ORC_Q5_0 || dtype == ORC_Q5_1;
+            float d = orc_rdf16(blk);
+            float dm = affine ? orc_rdf16(blk + 2) : d;
+            const uint8_t *p = blk + (affine ? 4 : 2);
+            uint32_t qh = 0;
+            if (five) {
+                qh = (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
+                p += 4;
+            }
+            float sc = d * (float)1;
+            float mn = dm * (float)(affine ? 1 : (five ? -16 : -8));
+            for (int j = 0; j < 16; j++) {
+                uint32_t xh0 = five ? ((qh >> j) << 4) & 0x10 : 0;
+                uint32_t xh1 = five ? (qh >> (j + 12)) & 0x10 : 0;
+                uint8_t c0 = (uint8_t)(((uint32_t)p[j] & 0x0F) | xh0);
+                uint8_t c1 = (uint8_t)(((uint32_t)p[j] >> 4) | xh1);
+                out[b * 32 + j] = sc * (float)c0 + mn;
+                out[b * 32 + j + 16] = sc * (float)c1 + mn;
+            }
+        }
+        return 0;
+    case ORC_Q5_K:
+        /* dequant.rs:332-358: Q4_K's layout with a 5th code bit from qh[32] (bit 2j for the even
+         * sub-block of pair j, bit 2j+1 for the odd one). */
+        for (size_t b = 0; b < nblk; b++) {
+            const uint8_t *blk = bytes + b * 176;
+            float d = orc_rdf16(blk);
+            float dmin = orc_rdf16(blk + 2);
+            const uint8_t *scales = blk + 4, *qh = blk + 16, *qs = blk + 48;
+            float *o = out + b * 256;
+            for (int j = 0; j < 4; j++) {
+                uint32_t sc1, m1, sc2, m2;
+                orc_k4(2 * j, scales, &sc1, &m1);
+                orc_k4(2 * j + 1, scales, &sc2, &m2);
+                float fs1 = d * (float)(int16_t)sc1, fm1 = dmin * (float)(int16_t)(-(int16_t)m1);
+                float fs2 = d * (float)(int16_t)sc2, fm2 = dmin * (float)(int16_t)(-(int16_t)m2);
+                for (int l = 0; l < 32; l++) {
+                    uint8_t v = qs[j * 32 + l];
+                    uint8_t c1 = (uint8_t)((v & 0xF) + ((qh[l] >> (2 * j)) & 1 ? 16 : 0));
+                    uint8_t c2 = (uint8_t)((v >> 4) + ((qh[l] >> (2 * j + 1)) & 1 ? 16 : 0));
+                    o[j * 64 + l] = fs1 * (float)c1 + fm1;
+                    o[j * 64 + 32 + l] = fs2 * (float)c2 + fm2;
+                }
+            }
+        }
+        return 0;
+    case ORC_IQ4_NL:
+        /* dequant.rs:495-512: pure codebook, d * KVALUES_IQ4NL[nibble]. */
+        for (size_t b = 0; b < nblk; b++) {
+            const uint8_t *blk = bytes + b * 18;
+            float d = orc_rdf16(blk);
+            for (int j = 0; j < 16; j++) {
+                out[b * 32 + j] = d * (float)orc_kvalues_iq4nl[blk[2 + j] & 0xF];
+                out[b * 32 + j + 16] = d * (float)orc_kvalues_iq4nl[blk[2 + j] >> 4];
             }
         }
         return 0;
@@ -404,6 +481,95 @@ float orc_vec_dot_q2_0(const uint8_t *row, const int8_t *qs8, const float *d8, c
     return sumf;
 }
 
+/* crates/infr-cpu/src/kernels.rs:1286-1327 (vec_dot_q5k_scalar). */
+float orc_vec_dot_q5k(const uint8_t *row, const int8_t *qs8, const float *d8, const int32_t *bsums,
+                      size_t in_f, int32_t *sd_out, int32_t *sm_out) {
+    size_t nb = in_f / 256;
+    float sumf = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * 176;
+        float d = orc_rdf16(blk);
+        float dmin = orc_rdf16(blk + 2);
+        const uint8_t *scales = blk + 4, *qh = blk + 16, *ql = blk + 48;
+        const int8_t *q8b = qs8 + b * 256;
+        int32_t sd = 0, sm = 0;
+        uint8_t u1 = 1, u2 = 2;
+        for (int j = 0; j < 4; j++) {
+            uint32_t sc_e, m_e, sc_o, m_o;
+            orc_k4(2 * j, scales, &sc_e, &m_e);
+            orc_k4(2 * j + 1, scales, &sc_o, &m_o);
+            const int8_t *q8_e = q8b + 2 * j * 32, *q8_o = q8b + (2 * j + 1) * 32;
+            int32_t iprod_e = 0, iprod_o = 0;
+            for (int l = 0; l < 32; l++) {
+                uint8_t v = ql[j * 32 + l];
+                int32_t q5_e = (int32_t)(v & 0xF) + ((qh[l] & u1) ? 16 : 0);
+                int32_t q5_o = (int32_t)(v >> 4) + ((qh[l] & u2) ? 16 : 0);
+                iprod_e += q5_e * (int32_t)q8_e[l];
+                iprod_o += q5_o * (int32_t)q8_o[l];
+            }
+            sd += (int32_t)sc_e * iprod_e + (int32_t)sc_o * iprod_o;
+            sm += (int32_t)m_e * bsums[b * 8 + 2 * j] + (int32_t)m_o * bsums[b * 8 + 2 * j + 1];
+            u1 = (uint8_t)(u1 << 2);
+            u2 = (uint8_t)(u2 << 2);
+        }
+        if (sd_out) sd_out[b] = sd;
+        if (sm_out) sm_out[b] = sm;
+        sumf += d8[b] * (d * (float)sd - dmin * (float)sm);
+    }
+    return sumf;
+}
+
+/* The 32-weight-block formats against the per-32 activation, one activation row of the batch
+ * scalars: Q4_0 kernels.rs:5496-5520, Q4_1 :5793-5822, Q5_0 :5350-5377, Q5_1 :5948-5980,
+ * IQ4_NL :6128-6152. Element j of a block takes the low nibble of qs[j], element j+16 the high
+ * nibble; Q5_x add qh bit j / j+16 as the 5th code bit. Per-block f32 terms, as written there:
+ *   Q4_0   d*d8 * (iprod - 8*bsum)        Q5_0   d*d8 * (iprod - 16*bsum)
+ *   Q4_1   d8 * (d*iprod + m*bsum)        Q5_1   d8 * (d*iprod + m*bsum)
+ *   IQ4_NL d*d8 * iprod   (iprod over the signed codebook values) */
+float orc_vec_dot_blk32(int dtype, const uint8_t *row, const int8_t *qs8, const float *d8,
+                        const int32_t *bsum, size_t in_f, int32_t *iprod_out) {
+    int qpb, bpb;
+    if (!orc_block_layout(dtype, &qpb, &bpb) || qpb != 32) return 0.0f;
+    int affine = dtype == ORC_Q4_1 || dtype == ORC_Q5_1;
+    int five = dtype == ORC_Q5_0 || dtype == ORC_Q5_1;
+    size_t nb = in_f / 32;
+    float sumf = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * (size_t)bpb;
+        float d = orc_rdf16(blk);
+        float mw = affine ? orc_rdf16(blk + 2) : 0.0f;
+        const uint8_t *p = blk + (affine ? 4 : 2);
+        uint32_t qh = 0;
+        if (five) {
+            qh = (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
+            p += 4;
+        }
+        const int8_t *q8b = qs8 + b * 32;
+        int32_t iprod = 0;
+        for (int j = 0; j < 16; j++) {
+            int32_t c0, c1;
+            if (dtype == ORC_IQ4_NL) {
+                c0 = orc_kvalues_iq4nl[p[j] & 0x0F];
+                c1 = orc_kvalues_iq4nl[p[j] >> 4];
+            } else {
+                uint32_t xh0 = five ? ((qh >> j) << 4) & 0x10 : 0;
+                uint32_t xh1 = five ? (qh >> (j + 12)) & 0x10 : 0;
+                c0 = (int32_t)(((uint32_t)p[j] & 0x0F) | xh0);
+                c1 = (int32_t)(((uint32_t)p[j] >> 4) | xh1);
+            }
+            iprod += c0 * (int32_t)q8b[j] + c1 * (int32_t)q8b[j + 16];
+        }
+        if (iprod_out) iprod_out[b] = iprod;
+        if (affine)
+            sumf += d8[b] * (d * (float)iprod + mw * (float)bsum[b]);
+        else if (dtype == ORC_IQ4_NL)
+            sumf += d * d8[b] * (float)iprod;
+        else
+            sumf += d * d8[b] * ((float)iprod - (five ? 16.0f : 8.0f) * (float)bsum[b]);
+    }
+    return sumf;
+}
+
 /* crates/infr-cpu/src/kernels.rs:6557-6573 */
 float orc_dot(const float *a, const float *b, size_t n) {
     size_t chunks = n / 8;
@@ -498,7 +664,8 @@ typedef struct {
 /* lib.rs:1037-1062: per-256 `Q8` for the 256-block formats and for Q8_0 rows of whole 256s;
  * a Q8_0 row that is a multiple of 32 only takes the per-32 `Q8x32` (q8_0_blk32). */
 static int is_q8_super(int dtype, size_t in_f) {
-    return dtype == ORC_Q4_K || dtype == ORC_Q6_K || (dtype == ORC_Q8_0 && in_f % 256 == 0);
+    return dtype == ORC_Q4_K || dtype == ORC_Q5_K || dtype == ORC_Q6_K ||
+           (dtype == ORC_Q8_0 && in_f % 256 == 0);
 }
 
 static void acts_free(acts_t *a) {
@@ -556,6 +723,19 @@ static float row_dot(int dtype, const uint8_t *row, const acts_t *a, size_t r, s
         size_t nb = in_f / 32;
         return orc_vec_dot_q2_0(row, a->qs + r * in_f, a->d + r * nb, a->bsums + r * nb, in_f, ia);
     }
+    case ORC_Q5_K: {
+        size_t nb = in_f / 256;
+        return orc_vec_dot_q5k(row, a->qs + r * in_f, a->d + r * nb, a->bsums + r * nb * 8, in_f,
+                               ia, ib);
+    }
+    case ORC_Q4_0:
+    case ORC_Q4_1:
+    case ORC_Q5_0:
+    case ORC_Q5_1:
+    case ORC_IQ4_NL: {
+        size_t nb = in_f / 32;
+        return orc_vec_dot_blk32(dtype, row, a->qs + r * in_f, a->d + r * nb, a->bsums + r * nb, in_f, ia);
+    }
     default:
         return 0.0f;
     }
@@ -568,7 +748,13 @@ static int linear_shape_ok(int dtype, size_t in_f) {
      * in_f % 64 == 0 (lib.rs:1406). */
     switch (dtype) {
     case ORC_Q4_K:
+    case ORC_Q5_K:
     case ORC_Q6_K: return in_f % 256 == 0;
+    case ORC_Q4_0:
+    case ORC_Q4_1:
+    case ORC_Q5_0:
+    case ORC_Q5_1:
+    case ORC_IQ4_NL:
     case ORC_Q8_0: return in_f % 32 == 0;
     case ORC_Q2_0: return in_f % 64 == 0;
     case ORC_F32: return 1;
@@ -603,8 +789,11 @@ int orc_linear(int dtype, const uint8_t *w, size_t wbytes, size_t w_numel, size_
 #endif
     (void)nt;
 
-    if (dtype == ORC_F32 || reference_mode) {
-        /* lib.rs:1015-1031 (reference mode) / :1162,1443-1448 (F32 weights): decode row, dot(). */
+    if (dtype == ORC_F32 || reference_mode || (dtype == ORC_Q5_0 && m == 1)) {
+        /* lib.rs:1015-1031 (reference mode) / :1162,1443-1448 (F32 weights): decode row, dot().
+         * Q5_0 has no arm in the one-token match (lib.rs:1081-1165), so decode takes its last arm,
+         * `dot(&bytes_to_f32(row, dt), xrow)` (:1165): f32 activations, no int8 rounding. With
+         * m >= 2 it takes the per-32 int8 kernel (:1322-1329). */
 #pragma omp parallel num_threads(nt)
         {
             float *wf = (float *)malloc(sizeof(float) * in_f);
@@ -652,7 +841,7 @@ int orc_linear_int_stages(int dtype, const uint8_t *w, size_t wbytes, size_t w_n
     size_t row0 = w_off / in_f;
     if (row0 + out_f > total_rows) return -2;
     const uint8_t *wb = w + row0 * bpr;
-    size_t blocks = (dtype == ORC_Q4_K || dtype == ORC_Q6_K) ? in_f / 256 : in_f / 32;
+    size_t blocks = (dtype == ORC_Q4_K || dtype == ORC_Q5_K || dtype == ORC_Q6_K) ? in_f / 256 : in_f / 32;
     acts_t a;
     acts_build(dtype, x, m, in_f, &a);
 #pragma omp parallel for schedule(dynamic, 8)
@@ -891,7 +1080,8 @@ static void put_f16(uint8_t *b, float v) {
 
 /* crates/infr-testkit/src/lib.rs:73-93 (synth_scales), :106-123 (synth_weight): LCG payload per
  * block seeded `seed ^ b`, then the f16 scale slots overwritten. Slot offsets from
- * crates/infr-core/src/decode_spec.rs:319-358: Q8_0 d@0; Q4K d@0 dmin@2; Q6K d@208; Q2_0 d@0. */
+ * crates/infr-core/src/decode_spec.rs:305-358: Q8_0 d@0; Q4K/Q5K d@0 dmin@2; Q6K d@208; Q2_0 d@0;
+ * Q4_0/Q5_0/IQ4_NL d@0; Q4_1/Q5_1 d@0 m@2. Magnitudes from synth_scales (testkit lib.rs:73-93). */
 size_t orc_synth_weight(int dtype, size_t n_elem, uint32_t seed, uint8_t *out) {
     int qpb, bpb;
     if (!orc_block_layout(dtype, &qpb, &bpb) || dtype == ORC_F32 || dtype == ORC_F16) return 0;
@@ -908,6 +1098,18 @@ size_t orc_synth_weight(int dtype, size_t n_elem, uint32_t seed, uint8_t *out) {
             break;
         case ORC_Q6_K: put_f16(blk + 208, 0.03f); break;
         case ORC_Q2_0: put_f16(blk, 0.05f); break;
+        case ORC_Q5_K:
+            put_f16(blk, 0.05f);
+            put_f16(blk + 2, 0.10f);
+            break;
+        case ORC_Q4_0:
+        case ORC_Q5_0: put_f16(blk, 0.04f); break;
+        case ORC_Q4_1:
+        case ORC_Q5_1:
+            put_f16(blk, 0.04f);
+            put_f16(blk + 2, -0.30f);
+            break;
+        case ORC_IQ4_NL: put_f16(blk, 0.004f); break;
         }
     }
     return nblk * (size_t)bpb;

@@ -42,9 +42,15 @@ extern "C" {
 enum {
     ORC_F32 = 0,
     ORC_F16 = 1,
+    ORC_Q4_0 = 2,
+    ORC_Q4_1 = 3,
+    ORC_Q5_0 = 6,
+    ORC_Q5_1 = 7,
     ORC_Q8_0 = 8,
     ORC_Q4_K = 12,
+    ORC_Q5_K = 13,
     ORC_Q6_K = 14,
+    ORC_IQ4_NL = 20,
     ORC_Q2_0 = 42
 };
 
@@ -92,6 +98,15 @@ float orc_vec_dot_q8_0_32(const uint8_t *row, const int8_t *qs, const float *d32
                           int32_t *iprod_out);
 float orc_vec_dot_q2_0(const uint8_t *row, const int8_t *qs, const float *d, const int32_t *bsum,
                        size_t in_f, int32_t *iprod_out);
+/* Q5_K: kernels.rs:1286-1327 — sd[nb], sm[nb] like Q4_K. */
+float orc_vec_dot_q5k(const uint8_t *row, const int8_t *qs, const float *d, const int32_t *bsums,
+                      size_t in_f, int32_t *sd_out, int32_t *sm_out);
+/* Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL against the per-32 activation: kernels.rs:5496-5520,
+ * 5793-5822, 5350-5377, 5948-5980, 6128-6152 — iprod[in_f/32] (raw codes; IQ4_NL: codebook values). */
+float orc_vec_dot_blk32(int dtype, const uint8_t *row, const int8_t *qs, const float *d,
+                        const int32_t *bsum, size_t in_f, int32_t *iprod_out);
+/* crates/infr-gguf/src/dequant.rs:439-441 */
+extern const int8_t orc_kvalues_iq4nl[16];
 
 /* crates/infr-cpu/src/kernels.rs:6557-6573 — 8 FMA accumulators, lanes summed in order, FMA tail. */
 float orc_dot(const float *a, const float *b, size_t n);

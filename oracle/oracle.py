@@ -18,6 +18,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libinfr_cpu_oracle.so")
 
 F32, F16, Q8_0, Q4_K, Q6_K, Q2_0 = 0, 1, 8, 12, 14, 42
+Q4_0, Q4_1, Q5_0, Q5_1, Q5_K, IQ4_NL = 2, 3, 6, 7, 13, 20
+KVALUES_IQ4NL = (-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113)
 ACTS_SUPER, ACTS_BLK32, ACTS_RAW = 0, 1, 2
 
 
@@ -63,6 +65,8 @@ _vd_q4k = _sig("orc_vec_dot_q4k", C.c_float, _u8p, _i8p, _f32p, _i32p, C.c_size_
 _vd_q6k = _sig("orc_vec_dot_q6k", C.c_float, _u8p, _i8p, _f32p, C.c_size_t, _i32p)
 _vd_q80 = _sig("orc_vec_dot_q8_0", C.c_float, _u8p, _i8p, _f32p, C.c_size_t, _i32p)
 _vd_q20 = _sig("orc_vec_dot_q2_0", C.c_float, _u8p, _i8p, _f32p, _i32p, C.c_size_t, _i32p)
+_vd_q5k = _sig("orc_vec_dot_q5k", C.c_float, _u8p, _i8p, _f32p, _i32p, C.c_size_t, _i32p, _i32p)
+_vd_b32 = _sig("orc_vec_dot_blk32", C.c_float, C.c_int, _u8p, _i8p, _f32p, _i32p, C.c_size_t, _i32p)
 _dot = _sig("orc_dot", C.c_float, _f32p, _f32p, C.c_size_t)
 _silu = _sig("orc_silu", C.c_float, C.c_float)
 _linear = _sig("orc_linear", C.c_int, C.c_int, _u8p, C.c_size_t, C.c_size_t, C.c_size_t, _f32p,
@@ -192,6 +196,25 @@ def vec_dot_q2_0(row, q8: Q8x32, in_f: int, stages: bool = False):
     return (np.float32(y), ip) if stages else np.float32(y)
 
 
+def vec_dot_q5k(row, q8: Q8, in_f: int, stages: bool = False):
+    row = _c(row, np.uint8)
+    nb = in_f // 256
+    sd = np.empty(nb, np.int32) if stages else None
+    sm = np.empty(nb, np.int32) if stages else None
+    y = _vd_q5k(_p(row, _u8p), _p(q8.qs, _i8p), _p(q8.d, _f32p), _p(q8.bsums, _i32p), in_f,
+                _p(sd, _i32p), _p(sm, _i32p))
+    return (np.float32(y), sd, sm) if stages else np.float32(y)
+
+
+def vec_dot_blk32(dtype: int, row, q8: Q8x32, in_f: int, stages: bool = False):
+    """Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL against the per-32 activation."""
+    row = _c(row, np.uint8)
+    ip = np.empty(in_f // 32, np.int32) if stages else None
+    y = _vd_b32(dtype, _p(row, _u8p), _p(q8.qs, _i8p), _p(q8.d, _f32p), _p(q8.bsum, _i32p), in_f,
+                _p(ip, _i32p))
+    return (np.float32(y), ip) if stages else np.float32(y)
+
+
 def dot(a, b) -> np.float32:
     a, b = _c(a, np.float32), _c(b, np.float32)
     return np.float32(_dot(_p(a, _f32p), _p(b, _f32p), min(a.size, b.size)))
@@ -278,9 +301,9 @@ def linear_int_stages(dtype: int, w, x, m: int, in_f: int, out_f: int, *,
     if w_numel is None:
         e, b = block_layout(dtype)
         w_numel = w.size // b * e
-    blocks = in_f // 256 if dtype in (Q4_K, Q6_K) else in_f // 32
+    blocks = in_f // 256 if dtype in (Q4_K, Q5_K, Q6_K) else in_f // 32
     a = np.empty((m, out_f, blocks), np.int32)
-    b_ = np.empty((m, out_f, blocks), np.int32) if dtype == Q4_K else None
+    b_ = np.empty((m, out_f, blocks), np.int32) if dtype in (Q4_K, Q5_K) else None
     rc = _linear_int(dtype, _p(w, _u8p), w.size, w_numel, w_off, _p(x, _f32p), m, in_f, out_f,
                      _p(a, _i32p), _p(b_, _i32p))
     if rc != 0:

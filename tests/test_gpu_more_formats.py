@@ -1,0 +1,167 @@
+"""GPU parity of Op::Linear for Q5_K, Q4_0, Q4_1, Q5_0, Q5_1 and IQ4_NL against the CPU oracle,
+through the C ABI. Integer stages bit-exact; Q5_K outputs bit-identical (same per-block expression
+and the CPU's accumulation order); the 32-weight-block formats within rel-L2 <= 1e-4 and
+max-abs <= 1e-3 * max|y| (their per-block terms are added in a different order than the CPU's).
+One token of Q5_0 multiplies f32 activations, as infr-cpu does."""
+import numpy as np
+import pytest
+
+from infr_amd import (Bindings, DType, Graph, InfrError, Linear, Status, TensorDesc, synth_normal_f32,
+                      synth_weight)
+from oracle import oracle as orc
+from tests.test_gpu_linear import _oracle_rows, gate, run_linear
+
+pytestmark = pytest.mark.gpu
+
+BLK32 = [DType.Q4_0, DType.Q4_1, DType.Q5_0, DType.Q5_1, DType.IQ4NL]
+ALL = BLK32 + [DType.Q5K]
+ids = lambda d: DType(d).name
+
+
+def shapes(dtype):
+    if dtype == DType.Q5K:
+        return [(256, 8), (768, 37), (4096, 256), (12288, 96), (5120, 64)]
+    return [(32, 8), (96, 37), (2048, 100), (4096, 256), (4128, 33), (12288, 96), (1152, 300)]
+
+
+@pytest.mark.parametrize("dtype", ALL, ids=ids)
+def test_decode_vs_oracle(be, dtype):
+    for in_f, out_f in shapes(dtype):
+        w = synth_weight(dtype, 100 + in_f, out_f, in_f)
+        x = synth_normal_f32(200 + out_f, in_f)
+        y = run_linear(be, dtype, w, x, 1, in_f, out_f)
+        want = orc.linear(dtype, w, x, 1, in_f, out_f)
+        gate(y, want)
+        if dtype == DType.Q5K:
+            assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), f"not bit-identical at {in_f}x{out_f}"
+
+
+@pytest.mark.parametrize("dtype", ALL, ids=ids)
+@pytest.mark.parametrize("m", [1, 3])
+def test_int_stages_bit_exact(be, dtype, m):
+    in_f, out_f = 1024, 24
+    # full-range payload bytes (the reference's synth_weight recipe): every code and 5th-bit pattern
+    w = orc.synth_weight(dtype, in_f * out_f, 0x301 + dtype)
+    x = orc.gen_f32(m * in_f, 0x9E37 + dtype)
+    if dtype == DType.Q5_0 and m == 1:
+        with pytest.raises(InfrError) as e:
+            be.linear_int_stages(dtype, be.upload_new(w), be.upload_new(x), 1, in_f, out_f)
+        assert e.value.status == Status.Unsupported       # one token of Q5_0 has no integer stage
+        return
+    a, b = be.linear_int_stages(dtype, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
+    oa, ob = orc.linear_int_stages(dtype, w, x, m, in_f, out_f)
+    assert np.array_equal(a, oa)
+    if dtype == DType.Q5K:
+        assert np.array_equal(b, ob)
+
+
+@pytest.mark.parametrize("dtype", ALL, ids=ids)
+def test_full_range_payload_decode(be, dtype):
+    """LCG payload bytes with the reference's scale magnitudes: all 16 / 32 code values, both nibble
+    halves, odd and even block alignment."""
+    in_f, out_f = 2048 if dtype != DType.Q5K else 2304, 50
+    w = orc.synth_weight(dtype, in_f * out_f, 0x77)
+    x = synth_normal_f32(5, in_f)
+    gate(run_linear(be, dtype, w, x, 1, in_f, out_f), orc.linear(dtype, w, x, 1, in_f, out_f))
+
+
+@pytest.mark.parametrize("dtype", ALL, ids=ids)
+@pytest.mark.parametrize("m", [2, 8, 40, 130])
+def test_batches_vs_oracle(be, dtype, m):
+    in_f, out_f = 1024, 96
+    w = synth_weight(dtype, 7, out_f, in_f)
+    x = synth_normal_f32(8 + m, m * in_f)
+    x[:in_f] *= 29.0
+    x[in_f:2 * in_f] = 0.0           # an all-zero row
+    y = run_linear(be, dtype, w, x, m, in_f, out_f)
+    want = orc.linear(dtype, w, x, m, in_f, out_f)
+    assert np.all(y[1] == 0.0)
+    gate(y, want)
+    if dtype == DType.Q5K and m <= 8:
+        assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), "not bit-identical"
+
+
+def test_q5_0_one_token_is_the_f32_path_not_the_int8_one(be):
+    in_f, out_f = 2048, 64
+    w = synth_weight(DType.Q5_0, 31, out_f, in_f)
+    x = synth_normal_f32(32, 2 * in_f)
+    y1 = run_linear(be, DType.Q5_0, w, x[:in_f], 1, in_f, out_f)
+    y2 = run_linear(be, DType.Q5_0, w, x, 2, in_f, out_f)
+    exact = orc.linear(DType.Q5_0, w, x[:in_f], 1, in_f, out_f, reference_mode=True)
+    gate(y1, exact)                                   # f32 activations: 1e-4 against decode + dot
+    gate(y2, orc.linear(DType.Q5_0, w, x, 2, in_f, out_f))
+    # and the int8 result really is a different number, so the gate above tells the arms apart
+    rel = np.linalg.norm(y2[0] - exact[0]) / np.linalg.norm(exact[0])
+    assert rel > 3e-4, rel
+
+
+@pytest.mark.parametrize("dtype", ALL, ids=ids)
+def test_full_size_rows_vs_oracle(be, dtype):
+    in_f, out_f = 4096, 12288
+    w = synth_weight(dtype, 900 + int(dtype), out_f, in_f)
+    x = synth_normal_f32(901, in_f)
+    y = run_linear(be, dtype, w, x, 1, in_f, out_f)
+    for row0 in (0, out_f // 2 - 7, out_f - 48):
+        want = _oracle_rows(dtype, w, x, 1, in_f, out_f, row0, 48)
+        got = y[:, row0:row0 + 48]
+        gate(got, want)
+        if dtype == DType.Q5K:
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), "not bit-identical"
+
+
+def test_w_off_on_2_mod_4_strides(be):
+    """Row slices of a concatenated Q4_0 weight whose row stride (in_f/32*18) is 2 mod 4: rows start
+    on both alignments."""
+    in_f, rows = 32 * 9, 40                             # bpr = 162
+    w = synth_weight(DType.Q4_0, 3, rows, in_f)
+    x = synth_normal_f32(4, in_f)
+    for row0, n in ((0, 40), (7, 16), (33, 7)):
+        y = run_linear(be, DType.Q4_0, w, x, 1, in_f, n, w_off=row0 * in_f, w_numel=rows * in_f)
+        gate(y, orc.linear(DType.Q4_0, w, x, 1, in_f, n, w_numel=rows * in_f, w_off=row0 * in_f))
+
+
+def test_plan_with_mixed_formats_replays(be):
+    """One plan holding a decode Linear of every format (Q5_0 as a launch of its own beside the
+    grouped ones) and a small-batch pair, executed twice with fresh inputs."""
+    in_f, out_f, m = 1024, 64, 4
+    g = Graph()
+    x1 = g.input(TensorDesc((1, in_f), DType.F32))
+    xm = g.input(TensorDesc((m, in_f), DType.F32))
+    binds = Bindings()
+    ws, outs = {}, []
+    for dt in ALL + [DType.Q4K]:
+        wt = g.weight(TensorDesc((out_f, in_f), dt))
+        ws[dt] = synth_weight(dt, 50 + int(dt), out_f, in_f)
+        binds.bind(wt, be.upload_new(ws[dt]))
+        y = g.output(TensorDesc((1, out_f), DType.F32))
+        g.push(Linear(x1, wt, y, 1, in_f, out_f))
+        yb = be.alloc(out_f * 4)
+        binds.bind(y, yb)
+        outs.append((dt, 1, yb))
+        if dt in (DType.Q5_0, DType.Q5K):
+            ym = g.output(TensorDesc((m, out_f), DType.F32))
+            g.push(Linear(xm, wt, ym, m, in_f, out_f))
+            ymb = be.alloc(m * out_f * 4)
+            binds.bind(ym, ymb)
+            outs.append((dt, m, ymb))
+    plan = be.compile(g)
+    x1b, xmb = be.alloc(in_f * 4), be.alloc(m * in_f * 4)
+    binds.bind(x1, x1b).bind(xm, xmb)
+    for rep in range(2):
+        a, b = synth_normal_f32(70 + rep, in_f), synth_normal_f32(80 + rep, m * in_f)
+        be.upload(x1b, a)
+        be.upload(xmb, b)
+        be.execute(plan, binds)
+        for dt, rows, yb in outs:
+            got = be.download(yb, np.empty((rows, out_f), np.float32))
+            gate(got, orc.linear(dt, ws[dt], a if rows == 1 else b, rows, in_f, out_f))
+
+
+def test_ragged_rows_are_refused(be):
+    w = be.upload_new(np.zeros(4096, np.uint8))
+    x = be.upload_new(np.zeros(4096, np.float32))
+    y = be.alloc(4096)
+    for dt, in_f in ((DType.Q4_0, 48), (DType.Q5_1, 16), (DType.Q5K, 128), (DType.IQ4NL, 40)):
+        with pytest.raises(InfrError) as e:
+            be.linear(dt, w, x, y, 1, in_f, 2, w_numel=2 * in_f)
+        assert e.value.status == Status.Unsupported
