@@ -376,8 +376,8 @@ def main():
     ap.add_argument("--layers", type=int, default=N_LAYERS)
     ap.add_argument("--no-extra", action="store_true", help="headline sweep only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--sections", default="shapes,mmq,chain,layer,ternary,moe,load",
-                    help="comma list of secondary sections: shapes, mmq, chain, layer, ternary, moe, load")
+    ap.add_argument("--sections", default="shapes,formats,mmq,chain,layer,ternary,moe,load",
+                    help="comma list of secondary sections: shapes, formats, mmq, chain, layer, ternary, moe, load")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
@@ -429,6 +429,13 @@ def main():
         for name, dt in (("Q4_K", DType.Q4K), ("Q6_K", DType.Q6K), ("Q8_0", DType.Q8_0)):
             for m in (1, 8):
                 for (out_f, in_f) in ((4096, 4096), (1024, 4096), (12288, 4096), (4096, 12288)):
+                    t, nb = single_shape(be, dt, m, in_f, out_f)
+                    extra[f"gemv_{name}_m{m}_{out_f}x{in_f}_GBs"] = round(nb / (t * 1e-3) / 1e9, 1)
+    if "formats" in sections:
+        for name, dt in (("Q5_K", DType.Q5K), ("Q4_0", DType.Q4_0), ("Q4_1", DType.Q4_1), ("Q5_0", DType.Q5_0),
+                         ("Q5_1", DType.Q5_1), ("IQ4_NL", DType.IQ4NL), ("Q2_0", DType.Q2_0)):
+            for m in (1, 8):
+                for (out_f, in_f) in ((4096, 4096), (12288, 4096), (4096, 12288)):
                     t, nb = single_shape(be, dt, m, in_f, out_f)
                     extra[f"gemv_{name}_m{m}_{out_f}x{in_f}_GBs"] = round(nb / (t * 1e-3) / 1e9, 1)
     if "mmq" in sections:

@@ -17,7 +17,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libinfr_hip.so")
 OBJ = os.path.join(HERE, "build")
 
-SOURCES = ["backend.hip", "quant_act.hip", "gemv.hip", "gemv_fmt_kquant.hip", "gemv_fmt_blk32.hip", "gemv_fmt_q5k.hip", "gemv_fmt_nib4.hip", "gemv_fmt_nib5.hip", "gemv_f32act.hip", "mmq.hip", "moe.hip", "elementwise.hip", "synth.cpp", "gguf.cpp"]
+SOURCES = ["backend.hip", "quant_act.hip", "gemv.hip", "gemv_fmt_kquant.hip", "gemv_fmt_blk32.hip", "gemv_fmt_q5k.hip", "gemv_fmt_nib4.hip", "gemv_fmt_nib5.hip", "gemv_fmt_pair.hip", "gemv_f32act.hip", "mmq.hip", "moe.hip", "elementwise.hip", "synth.cpp", "gguf.cpp"]
 
 # -ffp-contract=off: the f32 epilogues restate infr-cpu's expressions, which never fuse a multiply
 # into an add; -packed-fp32-ops off: packed FP32 forms are not used on this hardware pool.
@@ -39,7 +39,9 @@ def hipcc() -> str:
 
 def _compile(src: str) -> str:
     obj = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
-    cmd = [hipcc(), *DEVICE_FLAGS, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
+    # INFR_HIP_BUILD_FLAGS: extra compiler flags (e.g. -DINFR_PF_Q8_0=2) for measurement builds
+    extra = os.environ.get("INFR_HIP_BUILD_FLAGS", "").split()
+    cmd = [hipcc(), *DEVICE_FLAGS, *extra, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src}:\n{r.stderr[-4000:]}")
@@ -50,13 +52,14 @@ def build(verbose: bool = False) -> str:
     os.makedirs(OBJ, exist_ok=True)
     with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
         objs = list(ex.map(_compile, SOURCES))
-    cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
+    lib = os.environ.get("INFR_HIP_BUILD_OUT", LIB)  # measurement builds go elsewhere
+    cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib, *objs]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stderr[-4000:]}")
     if verbose:
-        print(f"built {LIB}")
-    return LIB
+        print(f"built {lib}")
+    return lib
 
 
 if __name__ == "__main__":

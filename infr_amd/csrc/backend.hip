@@ -277,6 +277,12 @@ int check_linear(infr_hip_t* be, int dtype, const infr_hip_buffer_t* w, size_t w
         return fail(be, INFR_HIP_ERR_UNSUPPORTED, "linear: dimension exceeds 2^31");
     out->wrows = static_cast<const uint8_t*>(w->ptr) + row0 * bpr;
     out->bpr = bpr;
+    // The kernels fetch blocks with 2-, 4- or 16-byte loads according to the block stride and
+    // assume the first row starts where a row stride of that alignment would put it.
+    const uintptr_t align = bpr % 16 == 0 ? 16 : (bpr % 4 == 0 ? 4 : 2);
+    if (reinterpret_cast<uintptr_t>(out->wrows) % align != 0)
+        return fail(be, INFR_HIP_ERR_INVALID,
+                    "linear: weight rows start at an address that is not " + std::to_string(align) + "-byte aligned");
     return INFR_HIP_OK;
 }
 

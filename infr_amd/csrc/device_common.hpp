@@ -20,29 +20,40 @@ __device__ __forceinline__ float f16_bits_to_f32(uint32_t bits16) {
     return (float)__builtin_bit_cast(_Float16, (uint16_t)bits16);
 }
 
+// Weights, activations and outputs handed to the kernels always live in device memory, but a
+// pointer that reaches a kernel through a table in memory (the per-workgroup tile tables) is a
+// generic one to the compiler, and loads through it become FLAT loads. Those count against the
+// LDS counter as well as the memory counter, so every wait for an LDS access would also wait for
+// the weight loads issued just before it - the prefetch of the next row would never overlap the
+// arithmetic of the current one. gload / gstore access a pointer as the global-memory pointer it is.
+#ifndef INFR_GLOBAL
+#define INFR_GLOBAL __attribute__((address_space(1)))
+#endif
+template <typename T>
+__device__ __forceinline__ T gload(const void* p) {
+    return *(const INFR_GLOBAL T*)p;
+}
+template <typename T>
+__device__ __forceinline__ void gstore(void* p, T v) {
+    *(INFR_GLOBAL T*)p = v;
+}
+
+typedef v4i v4i_a4 __attribute__((aligned(4)));
+typedef v4i v4i_a2 __attribute__((aligned(2)));
+typedef v2i v2i_a2 __attribute__((aligned(2)));
+typedef int v3i __attribute__((ext_vector_type(3)));
+typedef v3i v3i_a4 __attribute__((aligned(4)));
+
 // 16-byte load from an address that is only 2-byte aligned (Q6_K / Q8_0 / Q2_0 block strides
 // are 2 mod 4). gfx950 global loads take any alignment in the HSA unaligned-access mode.
-__device__ __forceinline__ v4i load16_a2(const uint8_t* p) {
-    v4i v;
-    __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 16);
-    return v;
-}
-__device__ __forceinline__ v4i load16(const uint8_t* p) {
-    return *reinterpret_cast<const v4i*>(__builtin_assume_aligned(p, 16));
-}
-__device__ __forceinline__ uint32_t load_u16(const uint8_t* p) {
-    uint16_t v;
-    __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 2);
-    return v;
-}
+__device__ __forceinline__ v4i load16_a2(const uint8_t* p) { return gload<v4i_a2>(p); }
+__device__ __forceinline__ v4i load16(const uint8_t* p) { return gload<v4i>(p); }
+__device__ __forceinline__ uint32_t load_u16(const uint8_t* p) { return gload<uint16_t>(p); }
 
 // 16-byte load from a 4-byte-aligned address (a dword-aligned multi-dword load runs at full rate;
 // one at 2-byte alignment does not).
-__device__ __forceinline__ v4i load16_a4(const uint8_t* p) {
-    v4i v;
-    __builtin_memcpy(&v, __builtin_assume_aligned(p, 4), 16);
-    return v;
-}
+__device__ __forceinline__ v4i load16_a4(const uint8_t* p) { return gload<v4i_a4>(p); }
+__device__ __forceinline__ int load_u32(const uint8_t* p) { return gload<int>(p); }
 
 // Q8_0 blocks (34 B stride) start at a 4-byte boundary or 2 bytes past one, and a 16-byte load at
 // 2-byte alignment runs far below full rate (measured: +20 % GEMV bandwidth without them; Q6_K and

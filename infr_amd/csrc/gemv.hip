@@ -31,14 +31,14 @@ static const GemvFormatOps* format_ops(int dtype, size_t in_f) {
     switch (dtype) {
     case 12: return &gemv_ops_q4k();
     case 14: return &gemv_ops_q6k();
-    case 8: return in_f % 256 == 0 ? &gemv_ops_q8_0() : &gemv_ops_q8_0_32();
-    case 42: return &gemv_ops_q2_0();
+    case 8: return in_f % 256 == 0 ? &gemv_ops_q8_0() : (in_f % 64 == 0 ? &gemv_ops_q8_0_32_aligned() : &gemv_ops_q8_0_32());
+    case 42: return in_f % 128 == 0 ? &gemv_ops_q2_0_aligned() : &gemv_ops_q2_0();
     case 13: return &gemv_ops_q5k();
-    case 2: return &gemv_ops_q4_0();
+    case 2: return in_f % 64 == 0 ? &gemv_ops_q4_0_pair() : &gemv_ops_q4_0();
     case 3: return &gemv_ops_q4_1();
-    case 6: return &gemv_ops_q5_0();
+    case 6: return in_f % 64 == 0 ? &gemv_ops_q5_0_pair() : &gemv_ops_q5_0();
     case 7: return &gemv_ops_q5_1();
-    case 20: return &gemv_ops_iq4nl();
+    case 20: return in_f % 64 == 0 ? &gemv_ops_iq4nl_pair() : &gemv_ops_iq4nl();
     default: return nullptr;
     }
 }

@@ -12,6 +12,9 @@
 //   kPer32                activation quantizer: per-32 (true) or per-256 (false)
 //   kOrdered              per-block terms are added in ascending block order (bit-exact with the
 //                         CPU's `sumf +=` chain) instead of a butterfly
+//   kPrefetch             wave steps whose loads are in flight ahead of the arithmetic (1 for every
+//                         format: depths of 2 and 3 measured 3-10 % slower on the small-block
+//                         formats, whose occupancy already covers the latency)
 //   kWide16Steps          up to this many wave steps per row the fused kernel fits 16 waves per
 //                         workgroup (128 VGPRs per lane) without spilling; beyond it, 8 waves
 //   units(in_f)           number of lane work units in a row (blocks for Q4_K/Q6_K ...)
@@ -49,6 +52,7 @@ struct FmtQ4K {
     static constexpr bool kOrdered = true;
     static constexpr int kBlockBytes = 144, kBlockElems = 256;
     static constexpr int kWide16Steps = 3;
+    static constexpr int kPrefetch = 1;
     struct Row {
         v4i hdr, qa, qb;
     };
@@ -139,6 +143,7 @@ struct FmtQ6K {
     static constexpr bool kOrdered = true;
     static constexpr int kBlockBytes = 210, kBlockElems = 256;
     static constexpr int kWide16Steps = 1;
+    static constexpr int kPrefetch = 1;
     struct Row {
         v4i qla, qlb, qh;
         v2i sc;
@@ -158,7 +163,7 @@ struct FmtQ6K {
             r.qla = load16_a2(blk + h * 64 + c * 16);
             r.qlb = load16_a2(blk + h * 64 + 32 + c * 16);
             r.qh = load16_a2(blk + 128 + h * 32 + c * 16);
-            __builtin_memcpy(&r.sc, __builtin_assume_aligned(blk + 192 + h * 8, 2), 8);
+            r.sc = gload<v2i_a2>(blk + 192 + h * 8);
             r.d = load_u16(blk + 208);
         } else {
             r.qla = r.qlb = r.qh = v4i{0, 0, 0, 0};
@@ -225,13 +230,17 @@ struct FmtQ6K {
 // 64 blocks (2048 weights, 2176 B) per wave step. Rows of whole 256s take the per-256 activation
 // (scale shared by 8 lanes, kernels.rs:1170-1187); rows that are a multiple of 32 only take the
 // per-32 activation, one scale per block (P32; kernels.rs:4972-4991, lib.rs:1037-1042).
-template <bool P32>
+// ALIGNED (rows of whole 64s: an even number of blocks, so rows start on a dword and the block
+// parity gives the alignment): the last dword is fetched whole - an even block's runs 2 bytes into
+// its odd neighbour, inside the row - which saves the second, conditional 2-byte load.
+template <bool P32, bool ALIGNED = false>
 struct FmtQ8_0T {
     static constexpr int kElemsPerStep = 2048;
     static constexpr bool kPer32 = P32;
     static constexpr bool kOrdered = false;
     static constexpr int kBlockBytes = 34, kBlockElems = 32;
     static constexpr int kWide16Steps = 4;
+    static constexpr int kPrefetch = 1;
     struct Row {
         v4i qa, qb;
         uint32_t d;
@@ -248,12 +257,17 @@ struct FmtQ8_0T {
     __device__ static void load_row(Row& r, const uint8_t* rowp, int t, int lane, bool ok) {
         if (ok) {
             const uint8_t* blk = rowp + (size_t)(t * 64 + lane) * 34;
-            const bool odd = (reinterpret_cast<uintptr_t>(blk) & 2) != 0;
+            const bool odd = ALIGNED ? (lane & 1) != 0 : (reinterpret_cast<uintptr_t>(blk) & 2) != 0;
             const uint8_t* a = blk - (odd ? 2 : 0);
             const v4i lo = load16_a4(a), hi = load16_a4(a + 16);
             // last dword: bytes 32..33 always belong to the block, 34..35 only to an odd one
-            uint32_t tail = load_u16(a + 32);
-            if (odd) tail |= load_u16(a + 34) << 16;
+            uint32_t tail;
+            if (ALIGNED) {
+                tail = (uint32_t)load_u32(a + 32);
+            } else {
+                tail = load_u16(a + 32);
+                if (odd) tail |= load_u16(a + 34) << 16;
+            }
             const uint32_t sel = realign2_selector(odd);
             r.d = odd ? (uint32_t)lo.x >> 16 : (uint32_t)lo.x & 0xFFFFu;
             r.qa.x = realign2(lo.x, lo.y, sel);
@@ -300,8 +314,10 @@ struct FmtQ8_0T {
         return a.dact * f16_bits_to_f32(r.d) * (float)ip;
     }
 };
-using FmtQ8_0 = FmtQ8_0T<false>;
+using FmtQ8_0 = FmtQ8_0T<false>;        // any row alignment (expert banks)
+using FmtQ8_0A = FmtQ8_0T<false, true>;  // per-256 activation: rows are whole 256s, always aligned
 using FmtQ8_0_32 = FmtQ8_0T<true>;
+using FmtQ8_0_32A = FmtQ8_0T<true, true>;
 
 // ───────────────────────────────────── Q2_0 ─────────────────────────────────────
 // Lane l owns 64-weight block t*64 + l: 18 B = f16 scale + 16 bytes of 2-bit codes, 2-byte
@@ -324,12 +340,19 @@ __device__ __forceinline__ void transpose4x4(const int in[4], int out[4]) {
     out[3] = (int)__builtin_amdgcn_perm(cd_hi, ab_hi, 0x07060302u);   // a3 b3 c3 d3
 }
 
-struct FmtQ2_0 {
+// ALIGNED: rows of whole 128s have an even number of blocks, so every row starts on a dword and
+// blocks alternate between a dword boundary and 2 bytes past one. Each lane then fetches its block
+// with two dword-aligned loads (5 dwords from the boundary at or below the block; an even block's
+// last dword runs 2 bytes into its odd neighbour, which is always inside the row) and realigns in
+// registers, instead of one 16-byte load at 2-byte alignment, which runs well below full rate.
+template <bool ALIGNED>
+struct FmtQ2_0T {
     static constexpr int kElemsPerStep = 4096;
     static constexpr bool kPer32 = true;
     static constexpr bool kOrdered = false;
     static constexpr int kBlockBytes = 18, kBlockElems = 64;
     static constexpr int kWide16Steps = 3;
+    static constexpr int kPrefetch = 1;
     struct Row {
         v4i codes;
         uint32_t d;
@@ -343,8 +366,19 @@ struct FmtQ2_0 {
     __device__ static void load_row(Row& r, const uint8_t* rowp, int t, int lane, bool ok) {
         if (ok) {
             const uint8_t* blk = rowp + (size_t)(t * 64 + lane) * 18;
-            r.d = load_u16(blk);
-            r.codes = load16_a2(blk + 2);
+            if (ALIGNED) {
+                const bool odd = (lane & 1) != 0;  // t * 64 is even
+                const uint8_t* a = blk - (odd ? 2 : 0);
+                const v4i lo = load16_a4(a);
+                const int w4 = load_u32(a + 16);
+                const uint32_t sel = realign2_selector(odd);
+                r.d = odd ? (uint32_t)lo.x >> 16 : (uint32_t)lo.x & 0xFFFFu;
+                r.codes = v4i{realign2(lo.x, lo.y, sel), realign2(lo.y, lo.z, sel), realign2(lo.z, lo.w, sel),
+                              realign2(lo.w, w4, sel)};
+            } else {
+                r.d = load_u16(blk);
+                r.codes = load16_a2(blk + 2);
+            }
         } else {
             r.codes = v4i{0, 0, 0, 0};
             r.d = 0;
@@ -397,6 +431,8 @@ struct FmtQ2_0 {
         return s;
     }
 };
+using FmtQ2_0 = FmtQ2_0T<false>;
+using FmtQ2_0A = FmtQ2_0T<true>;
 
 // ───────────────────────────────────── Q5_K ─────────────────────────────────────
 // Q4_K's lane mapping (block-in-step q = l/4, nibble pair p = l%4) on the 176-byte block
@@ -410,6 +446,7 @@ struct FmtQ5K {
     static constexpr bool kOrdered = true;
     static constexpr int kBlockBytes = 176, kBlockElems = 256;
     static constexpr int kWide16Steps = 2;
+    static constexpr int kPrefetch = 1;
     struct Row {
         v4i hdr, ha, hb, qa, qb;
     };
@@ -502,6 +539,7 @@ struct FmtNib32 {
     static constexpr bool kOrdered = false;
     static constexpr int kBlockBytes = 18 + (kAffine ? 2 : 0) + (kFive ? 4 : 0), kBlockElems = 32;
     static constexpr int kWide16Steps = 4;
+    static constexpr int kPrefetch = 1;
     struct Row {
         v4i qs;
         uint32_t dm;  // f16 d in the low half, f16 m (affine formats) in the high half
@@ -523,11 +561,8 @@ struct FmtNib32 {
         const uint8_t* blk = rowp + (size_t)(t * 64 + lane) * kBlockBytes;
         if (kAffine) {
             // [d m][qh][qs x4]: every field on a dword
-            uint32_t hdr;
-            __builtin_memcpy(&hdr, __builtin_assume_aligned(blk, 4), 4);
-            r.dm = hdr;
-            if (kFive) __builtin_memcpy(&r.qh, __builtin_assume_aligned(blk + 4, 4), 4);
-            else r.qh = 0;
+            r.dm = (uint32_t)load_u32(blk);
+            r.qh = kFive ? (uint32_t)load_u32(blk + 4) : 0u;
             r.qs = load16_a4(blk + (kFive ? 8 : 4));
         } else {
             // [d][qh?][qs x4] with the payload 2 bytes past the block start: dwords from the
@@ -540,7 +575,7 @@ struct FmtNib32 {
             int w[kWords + 1];
             const v4i lo = load16_a4(a);
             w[0] = lo.x; w[1] = lo.y; w[2] = lo.z; w[3] = lo.w;
-            if (kFive) __builtin_memcpy(&w[4], __builtin_assume_aligned(a + 16, 4), 4);
+            if (kFive) w[4] = load_u32(a + 16);
             uint32_t tail = load_u16(a + 4 * kWords);
             if (odd) tail |= load_u16(a + 4 * kWords + 2) << 16;
             w[kWords] = (int)tail;
@@ -606,5 +641,139 @@ using FmtQ4_1 = FmtNib32<Nib32::Q4_1>;
 using FmtQ5_0 = FmtNib32<Nib32::Q5_0>;
 using FmtQ5_1 = FmtNib32<Nib32::Q5_1>;
 using FmtIQ4NL = FmtNib32<Nib32::IQ4_NL>;
+
+// Pair form of the formats whose block stride is 2 mod 4 (Q4_0 / IQ4_NL 18 B, Q5_0 22 B), for rows
+// of whole 64s: two consecutive blocks are 36 / 44 bytes, a whole number of dwords, and every row
+// starts on a dword. Lane l owns the pair t*64 + l (64 weights): three dword-aligned loads fetch it
+// and only the first block's payload needs realigning (it starts 2 bytes into a dword; the second
+// block's starts on one). Fewer, fuller load instructions per byte than the one-block form, whose
+// blocks alternate between the two alignments. 64 pairs (4096 weights) per wave step. The two
+// blocks' terms are added in block order.
+template <Nib32 K>
+struct FmtNib32Pair {
+    static_assert(K == Nib32::Q4_0 || K == Nib32::IQ4_NL || K == Nib32::Q5_0, "2-mod-4 strides only");
+    static constexpr bool kFive = K == Nib32::Q5_0;
+    static constexpr int kElemsPerStep = 4096;
+    static constexpr bool kPer32 = true;
+    static constexpr bool kOrdered = false;
+    static constexpr int kOneBlock = kFive ? 22 : 18;
+    static constexpr int kBlockBytes = 2 * kOneBlock, kBlockElems = 64;
+    static constexpr int kWide16Steps = 3;
+    static constexpr int kPrefetch = 1;
+    struct Row {
+        v4i q0, q1;
+        uint32_t d01;  // f16 d of block 0 in the low half, of block 1 in the high half
+        uint32_t qh0, qh1;
+    };
+    struct Acts {
+        int xa[16];
+        float da0, da1, fb0, fb1;
+    };
+    __device__ static int units(int in_f) { return in_f / 64; }
+    __device__ static bool valid(int t, int lane, int n) { return t * 64 + lane < n; }
+    __device__ static void load_row(Row& r, const uint8_t* rowp, int t, int lane, bool ok) {
+        if (!ok) {
+            r.q0 = v4i{0, 0, 0, 0};
+            r.q1 = v4i{0, 0, 0, 0};
+            r.d01 = 0;
+            r.qh0 = 0;
+            r.qh1 = 0;
+            return;
+        }
+        const uint8_t* p = rowp + (size_t)(t * 64 + lane) * kBlockBytes;
+        const uint32_t sel = 0x05040302u;  // bytes 2..5 of a dword pair
+        if (!kFive) {
+            // dwords 0..8: [d0 | qs0 (16 B, from byte 2)] [.. | d1 (bytes 18,19)] [qs1 (dwords 5..8)]
+            const v4i a = load16_a4(p);
+            const int w4 = load_u32(p + 16);
+            r.q1 = load16_a4(p + 20);
+            r.q0 = v4i{realign2(a.x, a.y, sel), realign2(a.y, a.z, sel), realign2(a.z, a.w, sel),
+                       realign2(a.w, w4, sel)};
+            r.d01 = ((uint32_t)a.x & 0xFFFFu) | ((uint32_t)w4 & 0xFFFF0000u);
+            r.qh0 = 0;
+            r.qh1 = 0;
+        } else {
+            // dwords 0..10: d0 | qh0 (bytes 2..5) | qs0 (bytes 6..21) | d1 (22,23) | qh1 (dword 6) |
+            // qs1 (dwords 7..10)
+            const v4i a = load16_a4(p), b = load16_a4(p + 16);
+            const v3i c3 = gload<v3i_a4>(p + 32);
+            const int c[3] = {c3.x, c3.y, c3.z};
+            r.qh0 = (uint32_t)realign2(a.x, a.y, sel);
+            r.q0 = v4i{realign2(a.y, a.z, sel), realign2(a.z, a.w, sel), realign2(a.w, b.x, sel),
+                       realign2(b.x, b.y, sel)};
+            r.d01 = ((uint32_t)a.x & 0xFFFFu) | ((uint32_t)b.y & 0xFFFF0000u);
+            r.qh1 = (uint32_t)b.z;
+            r.q1 = v4i{b.w, c[0], c[1], c[2]};
+        }
+    }
+    __device__ static void load_acts(Acts& a, const ActPtrs& s, int t, int lane, bool ok) {
+        if (ok) {
+            const int u = t * 64 + lane;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const v4i v = *reinterpret_cast<const v4i*>(s.qs + (size_t)u * 64 + 16 * k);
+                a.xa[4 * k + 0] = v.x;
+                a.xa[4 * k + 1] = v.y;
+                a.xa[4 * k + 2] = v.z;
+                a.xa[4 * k + 3] = v.w;
+            }
+            a.da0 = s.d[2 * u];
+            a.da1 = s.d[2 * u + 1];
+            a.fb0 = (float)s.bsums[2 * u];
+            a.fb1 = (float)s.bsums[2 * u + 1];
+        } else {
+#pragma unroll
+            for (int k = 0; k < 16; ++k) a.xa[k] = 0;
+            a.da0 = 0.0f;
+            a.da1 = 0.0f;
+            a.fb0 = 0.0f;
+            a.fb1 = 0.0f;
+        }
+    }
+    __device__ static int block_iprod(const v4i& q, uint32_t qh, const int* xa) {
+        const uint32_t m4 = 0x0F0F0F0Fu;
+        const int qw[4] = {q.x, q.y, q.z, q.w};
+        int ip = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t w = (uint32_t)qw[k];
+            uint32_t lo = w & m4, hi = (w >> 4) & m4;
+            if (K == Nib32::IQ4_NL) {
+                lo = (uint32_t)iq4nl_lookup(lo);
+                hi = (uint32_t)iq4nl_lookup(hi);
+            }
+            if (kFive) {
+                lo |= spread4_to_bit4(qh >> (4 * k));
+                hi |= spread4_to_bit4(qh >> (16 + 4 * k));
+            }
+            ip = dot4((int)lo, xa[k], ip);
+            ip = dot4((int)hi, xa[4 + k], ip);
+        }
+        return ip;
+    }
+    template <bool STAGES>
+    __device__ static float term(const Row& r, const Acts& a, int t, int lane, bool ok,
+                                 const StagePtrs& st, size_t row_units) {
+        const int ip0 = block_iprod(r.q0, r.qh0, &a.xa[0]);
+        const int ip1 = block_iprod(r.q1, r.qh1, &a.xa[8]);
+        if (STAGES && ok) {
+            st.a[2 * row_units + 2 * (t * 64 + lane)] = ip0;
+            st.a[2 * row_units + 2 * (t * 64 + lane) + 1] = ip1;
+        }
+        const float d0 = f16_bits_to_f32(r.d01 & 0xFFFFu), d1 = f16_bits_to_f32(r.d01 >> 16);
+        if (K == Nib32::IQ4_NL) {
+            float s = d0 * a.da0 * (float)ip0;
+            s += d1 * a.da1 * (float)ip1;
+            return s;
+        }
+        const float off = kFive ? 16.0f : 8.0f;
+        float s = d0 * a.da0 * ((float)ip0 - off * a.fb0);
+        s += d1 * a.da1 * ((float)ip1 - off * a.fb1);
+        return s;
+    }
+};
+using FmtQ4_0Pair = FmtNib32Pair<Nib32::Q4_0>;
+using FmtIQ4NLPair = FmtNib32Pair<Nib32::IQ4_NL>;
+using FmtQ5_0Pair = FmtNib32Pair<Nib32::Q5_0>;
 
 }  // namespace infr

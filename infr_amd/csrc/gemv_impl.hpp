@@ -150,7 +150,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, 
         const int c = wave + i * NW;
         xv[i] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
         if (c < n_chunks && c * 256 + lane * 4 < in_f)
-            xv[i] = *reinterpret_cast<const v4f*>(tile.x + (size_t)c * 256 + lane * 4);
+            xv[i] = gload<v4f>(tile.x + (size_t)c * 256 + lane * 4);
     }
     const bool has_rows = row0 < tile.rows;
     typename F::Row first;
@@ -182,7 +182,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, 
         for (int i = 0; i < kMaxChunks; ++i) {
             const int c = wave + i * NW;
             if (c < n_chunks && c * 256 + lane * 4 < in_f) {
-                const v4f o = *reinterpret_cast<const v4f*>(tile.fus.x2 + (size_t)c * 256 + lane * 4);
+                const v4f o = gload<v4f>(tile.fus.x2 + (size_t)c * 256 + lane * 4);
                 v4f r;
                 if (tile.fus.pre == 2) {
                     r = v4f{xv[i].x * scale * o.x, xv[i].y * scale * o.y, xv[i].z * scale * o.z, xv[i].w * scale * o.w};
@@ -195,7 +195,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, 
                 }
                 xv[i] = r;
                 if (tile.fus.pre_dst)
-                    *reinterpret_cast<v4f*>(tile.fus.pre_dst + (size_t)c * 256 + lane * 4) = r;
+                    gstore<v4f>(tile.fus.pre_dst + (size_t)c * 256 + lane * 4, r);
             }
         }
     }

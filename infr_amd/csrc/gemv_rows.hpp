@@ -14,9 +14,9 @@ struct OrderedSum {
 };
 
 // Rows [row0, row_end) of one weight matrix against activation registers `acts`. `first` already
-// holds step 0 of row0 (the caller issues those loads as early as it can). The loads run one wave
-// step (16 or 64 blocks) ahead of the arithmetic, across row boundaries, so a wave always has
-// one step's bytes in flight while it holds only two steps' worth of registers.
+// holds step 0 of row0 (the caller issues those loads as early as it can). The loads run
+// F::kPrefetch wave steps (16 or 64 blocks each) ahead of the arithmetic, across row boundaries,
+// so a wave always has that many steps' bytes in flight.
 //
 // Ordered formats (Q4_K, Q6_K): the CPU adds a row's per-block terms in ascending block order
 // (`sumf +=`). The quad leaders park each row's terms in LDS (`osum`, this wave's private
@@ -32,7 +32,13 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
                                           float* osum, const float* add_b = nullptr,
                                           float* add_dst = nullptr) {
     constexpr int LS = OrderedSum<STEPS>::kRowStride;
-    typename F::Row cur = first;
+    constexpr int D = F::kPrefetch;  // wave steps in flight ahead of the arithmetic
+    typename F::Row q[D];            // q[i]: the step i ahead of the one being computed
+    q[0] = first;
+#pragma unroll
+    for (int i = 1; i < D; ++i)
+        F::load_row(q[i], w + (size_t)(row0 + i / STEPS) * bpr, i % STEPS, lane,
+                    ok[i % STEPS] && row0 + i / STEPS < row_end);
     int in_batch = 0, batch_row0 = row0;
     for (int row = row0; row < row_end; ++row) {
         const uint8_t* rowp = w + (size_t)row * bpr;
@@ -40,16 +46,18 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
 #pragma unroll
         for (int t = 0; t < STEPS; ++t) {
             typename F::Row nxt;
-            if (t + 1 < STEPS) F::load_row(nxt, rowp, t + 1, lane, ok[t + 1 < STEPS ? t + 1 : 0]);
-            else F::load_row(nxt, rowp + bpr, 0, lane, ok[0] && row + 1 < row_end);
-            const float term = F::template term<STAGES>(cur, acts[t], t, lane, ok[t], st,
+            F::load_row(nxt, rowp + (size_t)((t + D) / STEPS) * bpr, (t + D) % STEPS, lane,
+                        ok[(t + D) % STEPS] && row + (t + D) / STEPS < row_end);
+            const float term = F::template term<STAGES>(q[0], acts[t], t, lane, ok[t], st,
                                                         (size_t)row * n_units);
             if (F::kOrdered) {
                 if ((lane & 3) == 0) osum[in_batch * LS + t * 16 + (lane >> 2)] = term;
             } else {
                 s += term;
             }
-            cur = nxt;
+#pragma unroll
+            for (int i = 0; i + 1 < D; ++i) q[i] = q[i + 1];
+            q[D - 1] = nxt;
         }
         if (F::kOrdered) {
             if (++in_batch == 16 || row + 1 == row_end) {
@@ -64,9 +72,9 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
                         acc += v.z;
                         acc += v.w;
                     }
-                    y[batch_row0 + lane] = acc;
+                    gstore<float>(y + batch_row0 + lane, acc);
                     // an absorbed Op::Add: dst = a + b with a = this output
-                    if (add_dst) add_dst[batch_row0 + lane] = acc + add_b[batch_row0 + lane];
+                    if (add_dst) gstore<float>(add_dst + batch_row0 + lane, acc + gload<float>(add_b + batch_row0 + lane));
                 }
                 batch_row0 = row + 1;
                 in_batch = 0;
@@ -74,8 +82,8 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
         } else {
             s = wave_sum_f(s);
             if (lane == 0) {
-                y[row] = s;
-                if (add_dst) add_dst[row] = s + add_b[row];
+                gstore<float>(y + row, s);
+                if (add_dst) gstore<float>(add_dst + row, s + gload<float>(add_b + row));
             }
         }
     }
@@ -124,7 +132,7 @@ __device__ __forceinline__ void gemv_rows_folded(const uint8_t* __restrict__ w, 
                     acc += v.z;
                     acc += v.w;
                 }
-                y[batch_row0 + lane] = acc;
+                gstore<float>(y + batch_row0 + lane, acc);
             }
             batch_row0 = nr;
             in_batch = 0;
@@ -146,7 +154,13 @@ __device__ __forceinline__ void gemv_rows_batch(const uint8_t* __restrict__ w, s
                                                 size_t st_stride, float* osum) {
     constexpr int LS = OrderedSum<STEPS>::kRowStride;
     constexpr int RB = 16 / MB;  // weight rows per ordered-sum flush
-    typename F::Row cur = first;
+    constexpr int D = F::kPrefetch;
+    typename F::Row q[D];
+    q[0] = first;
+#pragma unroll
+    for (int i = 1; i < D; ++i)
+        F::load_row(q[i], w + (size_t)(row0 + i / STEPS) * bpr, i % STEPS, lane,
+                    ok[i % STEPS] && row0 + i / STEPS < row_end);
     int in_batch = 0, batch_row0 = row0;
     for (int row = row0; row < row_end; ++row) {
         const uint8_t* rowp = w + (size_t)row * bpr;
@@ -156,13 +170,13 @@ __device__ __forceinline__ void gemv_rows_batch(const uint8_t* __restrict__ w, s
 #pragma unroll
         for (int t = 0; t < STEPS; ++t) {
             typename F::Row nxt;
-            if (t + 1 < STEPS) F::load_row(nxt, rowp, t + 1, lane, ok[t + 1 < STEPS ? t + 1 : 0]);
-            else F::load_row(nxt, rowp + bpr, 0, lane, ok[0] && row + 1 < row_end);
+            F::load_row(nxt, rowp + (size_t)((t + D) / STEPS) * bpr, (t + D) % STEPS, lane,
+                        ok[(t + D) % STEPS] && row + (t + D) / STEPS < row_end);
 #pragma unroll
             for (int mi = 0; mi < MB; ++mi) {
                 const StagePtrs sm{STAGES ? st.a + mi * st_stride : nullptr,
                                    STAGES && st.b ? st.b + mi * st_stride : nullptr};
-                const float term = F::template term<STAGES>(cur, acts[mi][t], t, lane,
+                const float term = F::template term<STAGES>(q[0], acts[mi][t], t, lane,
                                                             ok[t] && mi < m_valid, sm,
                                                             (size_t)row * n_units);
                 if (F::kOrdered) {
@@ -171,7 +185,9 @@ __device__ __forceinline__ void gemv_rows_batch(const uint8_t* __restrict__ w, s
                     s[mi] += term;
                 }
             }
-            cur = nxt;
+#pragma unroll
+            for (int i = 0; i + 1 < D; ++i) q[i] = q[i + 1];
+            q[D - 1] = nxt;
         }
         if (F::kOrdered) {
             if (++in_batch == RB || row + 1 == row_end) {
@@ -187,7 +203,7 @@ __device__ __forceinline__ void gemv_rows_batch(const uint8_t* __restrict__ w, s
                         acc += v.w;
                     }
                     const int mi = lane % MB;
-                    if (mi < m_valid) y[(size_t)mi * y_stride + batch_row0 + lane / MB] = acc;
+                    if (mi < m_valid) gstore<float>(y + (size_t)mi * y_stride + batch_row0 + lane / MB, acc);
                 }
                 batch_row0 = row + 1;
                 in_batch = 0;
@@ -196,7 +212,7 @@ __device__ __forceinline__ void gemv_rows_batch(const uint8_t* __restrict__ w, s
 #pragma unroll
             for (int mi = 0; mi < MB; ++mi) {
                 const float tot = wave_sum_f(s[mi]);
-                if (lane == 0 && mi < m_valid) y[(size_t)mi * y_stride + row] = tot;
+                if (lane == 0 && mi < m_valid) gstore<float>(y + (size_t)mi * y_stride + row, tot);
             }
         }
     }

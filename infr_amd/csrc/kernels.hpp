@@ -173,13 +173,19 @@ const GemvFormatOps& gemv_ops_q4k();
 const GemvFormatOps& gemv_ops_q6k();
 const GemvFormatOps& gemv_ops_q8_0();
 const GemvFormatOps& gemv_ops_q8_0_32();
+const GemvFormatOps& gemv_ops_q8_0_32_aligned();  // rows of whole 64s
 const GemvFormatOps& gemv_ops_q2_0();
+const GemvFormatOps& gemv_ops_q2_0_aligned();  // rows of whole 128s
 const GemvFormatOps& gemv_ops_q5k();
 const GemvFormatOps& gemv_ops_q4_0();
 const GemvFormatOps& gemv_ops_q4_1();
 const GemvFormatOps& gemv_ops_q5_0();  // batch launchers only: one token takes the f32 kernel
 const GemvFormatOps& gemv_ops_q5_1();
 const GemvFormatOps& gemv_ops_iq4nl();
+// rows of whole 64s: two 2-mod-4-stride blocks per lane
+const GemvFormatOps& gemv_ops_q4_0_pair();
+const GemvFormatOps& gemv_ops_iq4nl_pair();
+const GemvFormatOps& gemv_ops_q5_0_pair();
 
 // Elementwise ops either side of a Linear (elementwise.hip).
 struct GatedActShape {

@@ -639,7 +639,7 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny_q4k_kernel(
     if (!row_ok) return;
 #pragma unroll
     for (int i = 0; i < RG; ++i)
-        if (etok[i] < m) y[(size_t)etok[i] * out_f + wrow] = acc[i];
+        if (etok[i] < m) gstore<float>(y + (size_t)etok[i] * out_f + wrow, acc[i]);
 }
 
 template <int NW>
