@@ -404,6 +404,10 @@ def main():
     # runs of this command (FETCH_SIZE x 1.99786 and WRITE_SIZE x 1.0, the factors a plain
     # 28,311,552-byte device copy in the same runs gives); null for any other launch shape.
     traffic = MEASURED_TRAFFIC.get(bytes_per_launch)
+    # what a kernel that only fetches reaches here: a read-only streaming pass over 2 GiB, same run
+    probe = be.alloc_uninit(2 << 30)
+    stream_read = be.stream_read_gbs(probe, reps=10)
+    probe.free()
     out = {
         "metric": "Q4_K GEMV HBM GB/s (% of peak) + prefill mmq int8 TOPS at M=512",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
@@ -419,7 +423,9 @@ def main():
         "roofline": {"bound": "hbm", "kernel": "gemv_fused_kernel<FmtQ4K, 1, 16> (in_f 4096 group)",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
-                     "avg_launch_us": round(avg_launch_us, 3), "bytes_per_launch": bytes_per_launch},
+                     "avg_launch_us": round(avg_launch_us, 3), "bytes_per_launch": bytes_per_launch,
+                     "stream_read_GBs": round(stream_read, 1),
+                     "frac_of_stream_read": round(achieved / stream_read, 4)},
     }
     sw.free()
 

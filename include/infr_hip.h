@@ -241,6 +241,11 @@ void infr_hip_reset_shutdown(void); /* tests only: the reference's latch is mono
  * stream (the reference's per-op timing seam, crates/infr-core/src/prof.rs:1-80) ---- */
 int infr_hip_timer_begin(infr_hip_t *be);
 int infr_hip_timer_end(infr_hip_t *be, float *elapsed_ms); /* synchronises */
+/* Measurement aid with no counterpart in the reference: reads the first `bytes` of `src` `reps`
+ * times with a plain streaming kernel (16-byte loads, no arithmetic) and reports the device time of
+ * those passes - the read bandwidth this device gives a kernel that only fetches, which the
+ * HBM-bound GEMVs are compared with. Synchronises. */
+int infr_hip_stream_read(infr_hip_t *be, const infr_hip_buffer_t *src, size_t bytes, int reps, float *elapsed_ms);
 
 /* ---- deterministic synthetic inputs (host side, no device work). The reference has no weight
  * quantizer (it only reads GGUF) and its tests synthesize valid blocks

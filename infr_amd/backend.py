@@ -131,6 +131,7 @@ SYMBOLS = {
     "infr_hip_reset_shutdown": (None, []),
     "infr_hip_timer_begin": (C.c_int, [_vp]),
     "infr_hip_timer_end": (C.c_int, [_vp, C.POINTER(C.c_float)]),
+    "infr_hip_stream_read": (C.c_int, [_vp, _vp, C.c_size_t, C.c_int, C.POINTER(C.c_float)]),
     "infr_synth_normal_f32": (None, [C.c_uint64, C.c_float, C.c_float, C.c_size_t, _vp]),
     "infr_synth_weight": (C.c_size_t, [C.c_int, C.c_uint64, C.c_float, C.c_size_t, C.c_size_t, _vp]),
     "infr_block_layout": (C.c_int, [C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
@@ -596,6 +597,13 @@ class HipBackend:
             sel_idx._h if sel_idx else None, sel_w._h if sel_w else None))
 
     # -- measurement --
+    def stream_read_gbs(self, buf: Buffer, nbytes: int | None = None, reps: int = 10) -> float:
+        """GB/s of a plain read-only streaming kernel over ``buf`` (what fetching alone reaches)."""
+        n = buf.len_bytes() if nbytes is None else nbytes
+        ms = C.c_float()
+        self._check(self._lib.infr_hip_stream_read(self._h, buf._h, n, reps, C.byref(ms)))
+        return n * reps / (ms.value * 1e-3) / 1e9
+
     def timer_begin(self) -> None:
         self._check(self._lib.infr_hip_timer_begin(self._h))
 

@@ -1142,4 +1142,24 @@ int infr_hip_timer_end(infr_hip_t* be, float* elapsed_ms) {
     return INFR_HIP_OK;
 }
 
+int infr_hip_stream_read(infr_hip_t* be, const infr_hip_buffer_t* src, size_t bytes, int reps, float* elapsed_ms) {
+    if (!be || !src || !elapsed_ms || reps <= 0) return fail(be, INFR_HIP_ERR_INVALID, "stream_read: bad argument");
+    if (bytes > src->len || bytes < 16) return fail(be, INFR_HIP_ERR_INVALID, "stream_read: size outside the buffer");
+    if (int rc = check_latch(be)) return rc;
+    static const int env_wgs = getenv("INFR_HIP_PROBE_WGS") ? atoi(getenv("INFR_HIP_PROBE_WGS")) : 64;
+    const int wgs = std::max(1, be->props.multiProcessorCount) * std::max(1, env_wgs);
+    int* out = nullptr;
+    HIP_TRY(be, hipMalloc((void**)&out, sizeof(int) * (size_t)wgs));
+    infr::launch_stream_read(src->ptr, bytes, out, wgs, be->stream);  // untimed first pass
+    hipError_t e = hipEventRecord(be->ev0, be->stream);
+    for (int r = 0; r < reps && e == hipSuccess; ++r) infr::launch_stream_read(src->ptr, bytes, out, wgs, be->stream);
+    if (e == hipSuccess) e = hipEventRecord(be->ev1, be->stream);
+    if (e == hipSuccess) e = hipEventSynchronize(be->ev1);
+    if (e == hipSuccess) e = hipEventElapsedTime(elapsed_ms, be->ev0, be->ev1);
+    if (e == hipSuccess) e = hipGetLastError();
+    (void)hipFree(out);
+    if (e != hipSuccess) return fail(be, INFR_HIP_ERR_BACKEND, std::string("stream_read: ") + hipGetErrorString(e));
+    return INFR_HIP_OK;
+}
+
 }  // extern "C"

@@ -89,4 +89,32 @@ void launch_add(const float* a, const float* b, float* out, size_t n, hipStream_
     hipLaunchKernelGGL(add_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, a, b, out, n);
 }
 
+// Measurement aid: a read-only streaming pass over `bytes` of device memory with nothing but
+// 16-byte loads and a xor, i.e. what a kernel that only had to fetch the weights could reach on
+// this device. Each workgroup walks 16 KB chunks grid-stride; one word per workgroup is written so
+// the loads cannot be dropped.
+__global__ __launch_bounds__(256) void stream_read_kernel(const v4i* __restrict__ src, size_t n_vec,
+                                                          int* __restrict__ out) {
+    const size_t chunk = 1024;  // v4i per workgroup per iteration: 4 per thread
+    v4i acc = v4i{0, 0, 0, 0};
+    for (size_t base = (size_t)blockIdx.x * chunk; base < n_vec; base += (size_t)gridDim.x * chunk) {
+        v4i v[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const size_t i = base + k * 256 + threadIdx.x;
+            v[k] = i < n_vec ? gload<v4i>(src + i) : v4i{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) acc ^= v[k];
+    }
+    const int r = acc.x ^ acc.y ^ acc.z ^ acc.w;
+    if (threadIdx.x == 0 || r == 0x5EEDF00D) out[blockIdx.x] = r;
+}
+
+void launch_stream_read(const void* src, size_t bytes, int* out, int workgroups, hipStream_t stream) {
+    if (bytes < 16 || workgroups <= 0) return;
+    hipLaunchKernelGGL(stream_read_kernel, dim3((unsigned)workgroups), dim3(256), 0, stream,
+                       static_cast<const v4i*>(src), bytes / 16, out);
+}
+
 }  // namespace infr

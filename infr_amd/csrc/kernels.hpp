@@ -155,6 +155,9 @@ bool gemv_takes_f32_activations(int dtype, size_t m);
 bool launch_gemv_f32act(int dtype, const uint8_t* w, size_t bpr, const float* x, float* y, size_t in_f,
                         size_t out_f, hipStream_t stream);
 
+// Read-only streaming pass (measurement aid): `out` holds one int per workgroup.
+void launch_stream_read(const void* src, size_t bytes, int* out, int workgroups, hipStream_t stream);
+
 // The decode-GEMV launchers of one weight format. Each format's kernels are instantiated in one
 // translation unit, which also defines its accessor below.
 struct GemvFormatOps {

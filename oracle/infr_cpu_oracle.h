@@ -20,6 +20,14 @@
  *                                 one-hot, bsums identities, reconstruction error <= d/2
  *   orc_vec_dot_*                 hand-derived 65024 vectors; brute-force int64 dots;
  *                                 dot(dequant(w), dequant(q8)) at the reference's own 1e-3
+ *   Q5_K / Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL (dequant, orc_vec_dot_q5k, orc_vec_dot_blk32)
+ *                                 the reference's five single-block known answers; hand blocks for
+ *                                 the 5th code bit; independent numpy decoders bit for bit; int64
+ *                                 brute-force stages; per-block f32 terms re-evaluated in numpy f32
+ *   orc_vec_dot_q8_0_32           brute-force int64 dots; hand-derived known answer
+ *   orc_rms_norm / orc_gated_act* / orc_add / orc_act
+ *                                 closed forms at hand-picked points; layouts against written-out
+ *                                 index arithmetic
  *   orc_linear                    batch == single bit-identical; f64 oracle at the reference's 2e-2;
  *                                 reference mode at 1e-5
  *   orc_moe_ffn                   textbook f32 MoE (restated from the reference's moe_ref test helper)
