@@ -72,11 +72,20 @@ bool plan_batch_group(int dtype, size_t m, size_t in_f, const GemvOpDesc* ops, i
         const size_t per_step = (size_t)f->elems_per_step;
         const size_t steps = (in_f + per_step - 1) / per_step;
         if (steps < 1 || steps > 8 || m > 8) return false;
-        size_t rpw = (total_rows + 4095) / 4096;
-        rpw = rpw < 2 ? 2 : (rpw > 16 ? 16 : rpw);
         gp.kind = 0;
-        gp.rows_per_wave = (int)rpw;
-        gp.rows_per_wg = (int)rpw * 4;
+        if (steps == 1) {
+            size_t rpw = (total_rows + 4095) / 4096;
+            rpw = rpw < 2 ? 2 : (rpw > 16 ? 16 : rpw);
+            gp.rows_per_wave = (int)rpw;
+            gp.rows_per_wg = (int)rpw * 4;
+        } else {
+            // K-split form: a tile is one workgroup's rows, whole flush groups of 64 / MB rows
+            const size_t rb = 64 / (m > 4 ? 8 : (m > 2 ? 4 : 2));
+            static const int env_rows = getenv("INFR_HIP_BATCH_KS_ROWS") ? atoi(getenv("INFR_HIP_BATCH_KS_ROWS")) : 0;
+            size_t r = ((env_rows > 0 ? (size_t)env_rows : (total_rows + 4095) / 4096) + rb - 1) / rb * rb;
+            gp.rows_per_wave = 0;
+            gp.rows_per_wg = (int)(r < rb ? rb : (r > 32 && rb <= 32 ? 32 : r));
+        }
     }
     gp.total_wgs = 0;
     for (int i = 0; i < n; ++i) gp.total_wgs += ((size_t)ops[i].out_f + gp.rows_per_wg - 1) / gp.rows_per_wg;

@@ -86,6 +86,111 @@ __global__ __launch_bounds__(256) void gemv_batch_kernel(const uint8_t* __restri
         osum + (threadIdx.x >> 6) * (F::kOrdered ? OrderedSum<STEPS>::kFloatsPerWave : 0));
 }
 
+// Small batch over rows longer than one wave step: K split over the waves of a workgroup. Wave w
+// owns wave step w of every row of the workgroup's tile, so the activations of all MB tokens for
+// that step fit its registers and the weights stream ONCE for the whole batch (the one-wave form
+// above has to re-stream them once per 8 / STEPS tokens). Per row every wave leaves its share in
+// LDS - for the ordered formats the per-block terms themselves, otherwise its lanes' sum - and after
+// each group of rows the workgroup's threads finish one (row, token) output each: the terms in
+// ascending block order, i.e. the CPU's `sumf +=` chain (bit-identical for Q4_K / Q5_K / Q6_K), or
+// the waves' sums in wave order. Two LDS buffers alternate, so one barrier per group suffices.
+// blockDim.x = 64 * (wave steps of a row), at most 512. Loads run two rows ahead.
+template <int MB>
+struct BatchKs {
+    static constexpr int kRowsPerFlush = 64 / MB;  // 64 (row, token) outputs per flush
+    __host__ __device__ static constexpr int row_stride(bool ordered, int nw) { return ordered ? nw * 16 + 4 : nw; }
+    __host__ __device__ static constexpr size_t lds_bytes(bool ordered, int nw) {
+        return (size_t)2 * 64 * row_stride(ordered, nw) * sizeof(float);
+    }
+};
+
+template <typename F, int MB, bool STAGES>
+__global__ __launch_bounds__(512) void gemv_batch_ks_kernel(const uint8_t* __restrict__ w, size_t bpr,
+                                                            ActPtrs act, int m_valid, int in_f,
+                                                            float* __restrict__ y, int out_f,
+                                                            int rows_per_wg, StagePtrs st,
+                                                            const BatchTile* __restrict__ tiles) {
+    extern __shared__ __attribute__((aligned(16))) float ks_lds[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    int row0 = blockIdx.x * rows_per_wg, n_rows = out_f;
+    size_t act_elem0 = 0;
+    if (tiles) {
+        const BatchTile t = tiles[blockIdx.x];
+        const int pass = blockIdx.y;
+        w = t.w;
+        bpr = t.bpr;
+        out_f = (int)t.out_f;
+        n_rows = (int)t.rows;
+        y = t.y + (size_t)pass * MB * out_f;
+        act_elem0 = (size_t)t.act_elem0 + (size_t)pass * MB * in_f;
+        m_valid = min(MB, m_valid - pass * MB);
+        row0 = 0;
+        rows_per_wg = n_rows;
+    }
+    if (row0 >= n_rows) return;
+    const int row_end = min(row0 + rows_per_wg, n_rows);
+    const int n_units = F::units(in_f);
+    const bool ok = F::valid(wave, lane, n_units);
+    typename F::Row q0, q1;  // this wave's step of the current row and of the next
+    F::load_row(q0, w + (size_t)row0 * bpr, wave, lane, ok);
+    F::load_row(q1, w + (size_t)(row0 + 1) * bpr, wave, lane, ok && row0 + 1 < row_end);
+    typename F::Acts acts[MB];
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi) {
+        const int r = mi < m_valid ? mi : 0;  // padding rows reuse row 0; their outputs are dropped
+        const size_t e = act_elem0 + (size_t)r * in_f;
+        const ActPtrs a{act.qs + e, act.d + e / (F::kPer32 ? 32 : 256), act.bsums + e / 32,
+                        act.bsums16 + e / 16};
+        F::load_acts(acts[mi], a, wave, lane, ok);
+    }
+    constexpr int RB = BatchKs<MB>::kRowsPerFlush;
+    const int ls = BatchKs<MB>::row_stride(F::kOrdered, nw);
+    const size_t st_stride = (size_t)out_f * (F::kBlockElems == 64 ? 2 * n_units : n_units);
+    int buf = 0;
+    for (int batch0 = row0; batch0 < row_end; batch0 += RB, buf ^= 1) {
+        float* B = ks_lds + (size_t)buf * 64 * ls;
+        const int nr = min(RB, row_end - batch0);
+        for (int r = 0; r < nr; ++r) {
+            const int row = batch0 + r;
+            typename F::Row q2;
+            F::load_row(q2, w + (size_t)(row + 2) * bpr, wave, lane, ok && row + 2 < row_end);
+#pragma unroll
+            for (int mi = 0; mi < MB; ++mi) {
+                const StagePtrs sm{STAGES ? st.a + mi * st_stride : nullptr,
+                                   STAGES && st.b ? st.b + mi * st_stride : nullptr};
+                const float term = F::template term<STAGES>(q0, acts[mi], wave, lane, ok && mi < m_valid, sm,
+                                                            (size_t)row * n_units);
+                if (F::kOrdered) {
+                    if ((lane & 3) == 0) B[(r * MB + mi) * ls + wave * 16 + (lane >> 2)] = term;
+                } else {
+                    const float tot = wave_sum_f(term);
+                    if (lane == 0) B[(r * MB + mi) * ls + wave] = tot;
+                }
+            }
+            q0 = q1;
+            q1 = q2;
+        }
+        __syncthreads();
+        for (int task = threadIdx.x; task < nr * MB; task += blockDim.x) {
+            const float* tr = B + (size_t)task * ls;
+            float acc = 0.0f;
+            if (F::kOrdered) {
+                for (int k = 0; k < 4 * nw; ++k) {
+                    const v4f v = reinterpret_cast<const v4f*>(tr)[k];
+                    acc += v.x;
+                    acc += v.y;
+                    acc += v.z;
+                    acc += v.w;
+                }
+            } else {
+                for (int k = 0; k < nw; ++k) acc += tr[k];
+            }
+            const int mi = task % MB;
+            if (mi < m_valid) gstore<float>(y + (size_t)mi * out_f + batch0 + task / MB, acc);
+        }
+    }
+}
+
 // act(gate) * up with the optional clamp, as Op::GatedAct evaluates one element
 // (gated_act_fn, crates/infr-cpu/src/kernels.rs:6591-6597).
 __device__ __forceinline__ float fused_gated_act(int act, bool has_clamp, float l, float gate, float up) {
@@ -272,8 +377,34 @@ static void launch_batch_one(const uint8_t* w, size_t bpr, const ActPtrs& act, i
                            m_valid, (int)in_f, y, (int)out_f, (int)rpw, st, (const BatchTile*)nullptr);
 }
 
-// Activation rows per pass of the batch kernel (they live in registers).
-static int batch_rows_per_pass(int steps) { return steps == 1 ? 8 : (steps == 2 ? 4 : (steps <= 4 ? 2 : 1)); }
+// Activation rows per pass of the batch kernels (they live in registers): the K-split form keeps
+// one wave step per wave, so it takes eight whatever the row length.
+static int batch_rows_per_pass(int steps) {
+    (void)steps;
+    return 8;
+}
+
+// Rows per workgroup of the K-split form: whole flush groups; 8 to 16 rows measured best for eight
+// tokens (larger tiles leave too few workgroups, and the one-wave form with several passes was no
+// faster on any shape tried).
+template <int MB>
+static int batch_ks_rows_per_wg(size_t total_rows) {
+    static const int env = getenv("INFR_HIP_BATCH_KS_ROWS") ? atoi(getenv("INFR_HIP_BATCH_KS_ROWS")) : 0;
+    constexpr int RB = BatchKs<MB>::kRowsPerFlush;
+    if (env > 0) return (env + RB - 1) / RB * RB;
+    size_t r = (total_rows + 4095) / 4096;  // about 4096 workgroups for a large group of rows
+    r = (r + RB - 1) / RB * RB;
+    return (int)(r < (size_t)RB ? RB : (r > 32 && RB <= 32 ? 32 : r));
+}
+
+template <typename F, int MB, bool STAGES>
+static void launch_batch_ks(const uint8_t* w, size_t bpr, const ActPtrs& act, int m_valid, size_t in_f,
+                            float* y, size_t out_f, const StagePtrs& st, int steps, const BatchTile* tiles,
+                            dim3 grid, int rows_per_wg, hipStream_t stream) {
+    hipLaunchKernelGGL((gemv_batch_ks_kernel<F, MB, STAGES>), grid, dim3((unsigned)steps * 64),
+                       BatchKs<MB>::lds_bytes(F::kOrdered, steps), stream, w, bpr, act, m_valid, (int)in_f, y,
+                       (int)out_f, rows_per_wg, st, tiles);
+}
 
 template <typename F, int STEPS, int MB>
 static void launch_batch_group_one(const BatchTile* tiles, const BatchGroupPlan& gp, const ActPtrs& act,
@@ -289,19 +420,20 @@ static bool launch_batch_group_fmt(const BatchTile* tiles, const BatchGroupPlan&
                                    size_t m, size_t in_f, hipStream_t stream) {
     const int steps = (int)((in_f + F::kElemsPerStep - 1) / F::kElemsPerStep);
     const ActPtrs act{a.qs, a.d, a.bsums, a.bsums16};
+    if (steps < 1 || steps > 8) return false;
     const int mb = std::min((int)m, batch_rows_per_pass(steps));
-#define INFR_G(S, MB) launch_batch_group_one<F, S, MB>(tiles, gp, act, (int)m, in_f, stream)
-    switch (steps) {
-    case 1: if (mb > 4) INFR_G(1, 8); else if (mb > 2) INFR_G(1, 4); else INFR_G(1, 2); break;
-    case 2: if (mb > 2) INFR_G(2, 4); else INFR_G(2, 2); break;
-    case 3: INFR_G(3, 2); break;
-    case 4: INFR_G(4, 2); break;
-    case 5: INFR_G(5, 1); break;
-    case 6: INFR_G(6, 1); break;
-    case 7: INFR_G(7, 1); break;
-    case 8: INFR_G(8, 1); break;
-    default: return false;
+    if (steps == 1) {
+        if (mb > 4) launch_batch_group_one<F, 1, 8>(tiles, gp, act, (int)m, in_f, stream);
+        else if (mb > 2) launch_batch_group_one<F, 1, 4>(tiles, gp, act, (int)m, in_f, stream);
+        else launch_batch_group_one<F, 1, 2>(tiles, gp, act, (int)m, in_f, stream);
+        return true;
     }
+    // rows longer than a wave step: K split over the workgroup's waves, one tile per workgroup
+    const StagePtrs none{nullptr, nullptr};
+#define INFR_G(MB)                                                                                         \
+    launch_batch_ks<F, MB, false>(nullptr, 0, act, (int)m, in_f, nullptr, 0, none, steps, tiles,           \
+                                  dim3((unsigned)gp.total_wgs, (unsigned)((m + MB - 1) / MB)), 0, stream)
+    if (mb > 4) INFR_G(8); else if (mb > 2) INFR_G(4); else INFR_G(2);
 #undef INFR_G
     return true;
 }
@@ -322,17 +454,21 @@ static bool launch_batch_fmt(const uint8_t* w, size_t bpr, const ActQ8& a, float
         const StagePtrs sp{st.a ? st.a + r0 * out_f * blocks : nullptr,
                            st.b ? st.b + r0 * out_f * blocks : nullptr};
         float* yo = y + r0 * out_f;
-#define INFR_B(S, MB) launch_batch_one<F, S, MB>(w, bpr, act, mv, in_f, yo, out_f, sp, stream)
-        switch (steps) {
-        case 1: if (mv > 4) INFR_B(1, 8); else if (mv > 2) INFR_B(1, 4); else if (mv > 1) INFR_B(1, 2); else INFR_B(1, 1); break;
-        case 2: if (mv > 2) INFR_B(2, 4); else if (mv > 1) INFR_B(2, 2); else INFR_B(2, 1); break;
-        case 3: if (mv > 1) INFR_B(3, 2); else INFR_B(3, 1); break;
-        case 4: if (mv > 1) INFR_B(4, 2); else INFR_B(4, 1); break;
-        case 5: INFR_B(5, 1); break;
-        case 6: INFR_B(6, 1); break;
-        case 7: INFR_B(7, 1); break;
-        default: INFR_B(8, 1); break;
+        if (steps == 1) {
+            if (mv > 4) launch_batch_one<F, 1, 8>(w, bpr, act, mv, in_f, yo, out_f, sp, stream);
+            else if (mv > 2) launch_batch_one<F, 1, 4>(w, bpr, act, mv, in_f, yo, out_f, sp, stream);
+            else if (mv > 1) launch_batch_one<F, 1, 2>(w, bpr, act, mv, in_f, yo, out_f, sp, stream);
+            else launch_batch_one<F, 1, 1>(w, bpr, act, mv, in_f, yo, out_f, sp, stream);
+            continue;
         }
+#define INFR_B(MB)                                                                                          \
+    do {                                                                                                    \
+        const int rpw = batch_ks_rows_per_wg<MB>(out_f);                                                    \
+        const dim3 grid((unsigned)((out_f + rpw - 1) / rpw));                                               \
+        if (st.a) launch_batch_ks<F, MB, true>(w, bpr, act, mv, in_f, yo, out_f, sp, steps, nullptr, grid, rpw, stream); \
+        else launch_batch_ks<F, MB, false>(w, bpr, act, mv, in_f, yo, out_f, sp, steps, nullptr, grid, rpw, stream);     \
+    } while (0)
+        if (mv > 4) INFR_B(8); else if (mv > 2) INFR_B(4); else if (mv > 1) INFR_B(2); else INFR_B(1);
 #undef INFR_B
     }
     return true;
