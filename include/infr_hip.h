@@ -40,6 +40,7 @@ typedef enum {
  * (crates/infr-gguf/src/lib.rs:330-354; crates/infr-core/src/tensor.rs:7-57). */
 typedef enum {
     INFR_DTYPE_F32 = 0,
+    INFR_DTYPE_F16 = 1,   /* embedding tables only */
     INFR_DTYPE_Q4_0 = 2,  /* 32 / 18 B:  [f16 d][u8 qs[16]]             w = d*(q-8)        :311-312 */
     INFR_DTYPE_Q4_1 = 3,  /* 32 / 20 B:  [f16 d][f16 m][u8 qs[16]]      w = d*q+m          :313-314 */
     INFR_DTYPE_Q5_0 = 6,  /* 32 / 22 B:  [f16 d][u32 qh][u8 qs[16]]     w = d*(q-16)       :315-316 */
@@ -49,6 +50,7 @@ typedef enum {
     INFR_DTYPE_Q5_K = 13, /* 256 / 176 B: [f16 d][f16 dmin][u8 sc[12]][u8 qh[32]][u8 qs[128]] :328-329 */
     INFR_DTYPE_Q6_K = 14, /* 256 / 210 B: [u8 ql[128]][u8 qh[64]][i8 sc[16]][f16 d]       :330-331 */
     INFR_DTYPE_IQ4_NL = 20, /* 32 / 18 B: [f16 d][u8 qs[16]]  w = d*codebook[q]           :349-350 */
+    INFR_DTYPE_BF16 = 30, /* embedding tables only */
     INFR_DTYPE_Q2_0 = 42  /* 64 / 18 B:   [f16 d][u8 qs[16]] ternary-style 2-bit codes    :357-358 */
 } infr_dtype;
 
@@ -173,6 +175,15 @@ int infr_hip_moe_ffn(infr_hip_t *be, const infr_hip_moe_params_t *p, const infr_
                      const infr_hip_buffer_t *down_exps, infr_hip_buffer_t *dst,
                      infr_hip_buffer_t *sel_idx, infr_hip_buffer_t *sel_w);
 
+/* Op::EmbedGather (crates/infr-core/src/graph.rs:853-865; CPU arm crates/infr-cpu/src/lib.rs:2084-2111):
+ * dst[r, :] = decode(table[ids[r], :]) * scale for `rows` rows of `ne` elements. `table` holds
+ * `table_numel / ne` rows of raw `dtype` blocks (every Linear weight format, F32, F16, BF16); `ids`
+ * holds `rows` int32 token ids. Outputs equal infr-cpu's host decode times `scale` bit for bit. An id
+ * outside the table gives a row of NaN (infr-cpu panics there); nothing is read out of bounds. */
+int infr_hip_embed_gather(infr_hip_t *be, int dtype, const infr_hip_buffer_t *table, size_t table_numel,
+                          const infr_hip_buffer_t *ids, size_t rows, size_t ne, float scale,
+                          infr_hip_buffer_t *dst);
+
 /* ---- graph level: Backend::compile / execute (backend.rs:560-577) over a flat C mirror of
  * infr_core::graph::Graph restricted to the ops of this path ---- */
 typedef enum {
@@ -183,7 +194,8 @@ typedef enum {
     INFR_OP_RMS_NORM_ADD = 4,    /* Op::RmsNormAdd, graph.rs:149-158; lib.rs:826-850 */
     INFR_OP_GATED_ACT = 5,       /* Op::GatedAct, graph.rs:697-735; lib.rs:1890-1944 */
     INFR_OP_GATED_ACT_FUSED = 6, /* Op::GatedActFused, graph.rs:736-748; lib.rs:1945-1971 */
-    INFR_OP_ADD = 7              /* Op::Add, graph.rs:749-755; lib.rs:1972-1988 */
+    INFR_OP_ADD = 7,             /* Op::Add, graph.rs:749-755; lib.rs:1972-1988 */
+    INFR_OP_EMBED_GATHER = 8     /* Op::EmbedGather, graph.rs:853-865; lib.rs:2084-2111 */
 } infr_hip_op_kind;
 
 /* Activation (crates/infr-core/src/graph.rs, act_fn in crates/infr-cpu/src/kernels.rs:6578-6585) */
@@ -205,13 +217,16 @@ typedef struct {
      *   GatedAct               x = gate, aux = up, dst, m = rows, in_f = nff, act, up_off, up_stride,
      *                          gate_stride, gate_block_width, has_clamp / clamp (swiglu_clamp)
      *   GatedActFused          x = gu [rows, 2*nff], dst, m = rows, in_f = nff, act, has_clamp / clamp
-     *   Add                    x = a, aux = b, dst, in_f = n (m = 1); in place when dst == x */
+     *   Add                    x = a, aux = b, dst, in_f = n (m = 1); in place when dst == x
+     * EmbedGather: x = ids (int32 [rows]), weight = table, dst (f32 [rows, ne]), m = rows, in_f = ne,
+     *   w_numel = the table's element count, w_dtype, scale */
     uint32_t aux;
     float eps;
     int act; /* infr_activation */
     uint32_t up_off, up_stride, gate_stride, gate_block_width;
     int has_clamp;
     float clamp;
+    float scale; /* EmbedGather */
 } infr_hip_op_t;
 
 /* Backend::compile: validates and stores the op list (the reference's GraphPlan clones the

@@ -4,7 +4,7 @@
 ``include/infr_hip.h``; ``infr_amd.build`` compiles the HIP sources into ``libinfr_hip.so``.
 """
 from .backend import (  # noqa: F401
-    Activation, Add, Bindings, Buffer, BufferUsage, DType, GatedAct, GatedActFused, Graph, HipBackend,
+    Activation, Add, Bindings, Buffer, BufferUsage, DType, EmbedGather, GatedAct, GatedActFused, Graph, HipBackend,
     InfrError, Linear, MoeFfn, Plan, RmsNorm, RmsNormAdd, Status, TensorDesc, TensorId, block_layout,
     load_library, synth_normal_f32, synth_weight,
 )

@@ -22,6 +22,7 @@ LIB_PATH = os.path.join(_HERE, "libinfr_hip.so")
 class DType(IntEnum):
     """GGML type ids (crates/infr-gguf/src/lib.rs:330-354)."""
     F32 = 0
+    F16 = 1      # embedding tables only
     Q4_0 = 2
     Q4_1 = 3
     Q5_0 = 6
@@ -31,6 +32,8 @@ class DType(IntEnum):
     Q5K = 13
     Q6K = 14
     IQ4NL = 20
+    BF16 = 30    # embedding tables only
+    I32 = 26     # token ids (never a weight here)
     Q2_0 = 42
 
 
@@ -80,7 +83,7 @@ class _Op(C.Structure):
                 ("up_exps", C.c_uint32), ("down_exps", C.c_uint32), ("moe", _MoeParams),
                 ("aux", C.c_uint32), ("eps", C.c_float), ("act", C.c_int), ("up_off", C.c_uint32),
                 ("up_stride", C.c_uint32), ("gate_stride", C.c_uint32), ("gate_block_width", C.c_uint32),
-                ("has_clamp", C.c_int), ("clamp", C.c_float)]
+                ("has_clamp", C.c_int), ("clamp", C.c_float), ("scale", C.c_float)]
 
 
 class _Caps(C.Structure):
@@ -121,6 +124,7 @@ SYMBOLS = {
                                              C.c_size_t, C.c_size_t, C.c_size_t, _vp, _vp]),
     "infr_hip_moe_ffn": (C.c_int, [_vp, C.POINTER(_MoeParams), _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                    _vp, _vp]),
+    "infr_hip_embed_gather": (C.c_int, [_vp, C.c_int, _vp, C.c_size_t, _vp, C.c_size_t, C.c_size_t, C.c_float, _vp]),
     "infr_hip_compile": (C.c_int, [_vp, C.POINTER(_Op), C.c_size_t, C.POINTER(_vp)]),
     "infr_hip_plan_free": (None, [_vp, _vp]),
     "infr_hip_execute": (C.c_int, [_vp, _vp, C.POINTER(_vp), C.c_size_t]),
@@ -336,6 +340,17 @@ class Add:
 
 
 @dataclass
+class EmbedGather:
+    """Op::EmbedGather (graph.rs:853-865): dst[r, :] = decode(table[ids[r], :]) * scale."""
+    ids: TensorId
+    table: TensorId
+    dst: TensorId
+    rows: int
+    ne: int
+    scale: float = 1.0
+
+
+@dataclass
 class Graph:
     """Ordered op list over declared tensors (crates/infr-core/src/graph.rs:1317-1460)."""
     tensors: list = field(default_factory=list)
@@ -529,6 +544,12 @@ class HipBackend:
                 o.kind = 7
                 o.x, o.aux, o.dst = op.a.id, op.b.id, op.dst.id
                 o.m, o.in_f = 1, op.n
+            elif isinstance(op, EmbedGather):
+                o.kind = 8
+                o.x, o.weight, o.dst = op.ids.id, op.table.id, op.dst.id
+                o.m, o.in_f, o.scale = op.rows, op.ne, op.scale
+                o.w_numel = g.desc(op.table).numel()
+                o.w_dtype = int(g.desc(op.table).dtype)
             else:
                 raise InfrError(Status.Unsupported, f"op {type(op).__name__} is not on this path")
         h = _vp()
@@ -583,6 +604,11 @@ class HipBackend:
         return (self.download(qs, np.empty((m, k), np.int8)),
                 self.download(d, np.empty((m, k // 32), np.float32)),
                 self.download(bs, np.empty((m, k // 32), np.int32)))
+
+    def embed_gather(self, dtype: int, table: Buffer, table_numel: int, ids: Buffer, rows: int, ne: int,
+                     dst: Buffer, scale: float = 1.0) -> None:
+        self._check(self._lib.infr_hip_embed_gather(self._h, int(dtype), table._h, table_numel, ids._h, rows,
+                                                    ne, scale, dst._h))
 
     def moe_ffn(self, x: Buffer, router: Buffer, gate: Buffer, up: Buffer, down: Buffer,
                 dst: Buffer, *, rows: int, ne: int, n_expert: int, n_used: int, n_ff_exp: int,

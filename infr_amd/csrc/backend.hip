@@ -321,6 +321,35 @@ int enqueue_gemv_single(infr_hip_t* be, int dtype, size_t in_f, const infr::Gemv
     return INFR_HIP_OK;
 }
 
+struct EmbedArgs {
+    const uint8_t* table;
+    size_t bpr, total_rows;
+};
+
+// Shape/size validation of an Op::EmbedGather (table rows as lib.rs:2099-2100 derives them).
+int check_embed(infr_hip_t* be, int dtype, const infr_hip_buffer_t* table, size_t table_numel,
+                const infr_hip_buffer_t* ids, size_t rows, size_t ne, const infr_hip_buffer_t* dst,
+                EmbedArgs* out) {
+    if (!table || !ids || !dst) return fail(be, INFR_HIP_ERR_INVALID, "embed_gather: unbound buffer");
+    int qpb = 0, bpb = 0;
+    if (!infr::embed_gather_supported(dtype) || !infr_block_layout(dtype, &qpb, &bpb))
+        return fail(be, INFR_HIP_ERR_UNSUPPORTED, "embed_gather: table dtype " + std::to_string(dtype) + " has no decoder");
+    if (rows == 0 || ne == 0 || ne % (size_t)qpb != 0 || table_numel == 0 || table_numel % ne != 0)
+        return fail(be, INFR_HIP_ERR_UNSUPPORTED, "embed_gather: rows must be whole blocks and the table whole rows");
+    if (ne > 0x7FFFFFFFull || rows > 65535 || table_numel / ne > 0x7FFFFFFFull)
+        return fail(be, INFR_HIP_ERR_UNSUPPORTED, "embed_gather: dimension out of range");
+    out->total_rows = table_numel / ne;
+    out->bpr = ne / (size_t)qpb * (size_t)bpb;
+    out->table = static_cast<const uint8_t*>(table->ptr);
+    if (table->len < out->total_rows * out->bpr)
+        return fail(be, INFR_HIP_ERR_INVALID, "embed_gather: table buffer smaller than its declared shape");
+    if (ids->len < rows * sizeof(int32_t) || dst->len < rows * ne * sizeof(float))
+        return fail(be, INFR_HIP_ERR_INVALID, "embed_gather: ids or dst buffer too small");
+    if (reinterpret_cast<uintptr_t>(out->table) % 2 != 0)
+        return fail(be, INFR_HIP_ERR_INVALID, "embed_gather: table is not 2-byte aligned");
+    return INFR_HIP_OK;
+}
+
 int check_latch(infr_hip_t* be) {
     if (g_shutdown_signo.load(std::memory_order_relaxed) != 0)
         return fail(be, INFR_HIP_ERR_ABORTED, "shutdown requested");
@@ -539,6 +568,19 @@ int infr_hip_linear(infr_hip_t* be, int dtype, const infr_hip_buffer_t* w, size_
                           static_cast<float*>(dst->ptr), m, in_f, out_f, infr::IntStages{});
 }
 
+int infr_hip_embed_gather(infr_hip_t* be, int dtype, const infr_hip_buffer_t* table, size_t table_numel,
+                          const infr_hip_buffer_t* ids, size_t rows, size_t ne, float scale,
+                          infr_hip_buffer_t* dst) {
+    if (!be) return INFR_HIP_ERR_INVALID;
+    if (int rc = check_latch(be)) return rc;
+    EmbedArgs ea;
+    if (int rc = check_embed(be, dtype, table, table_numel, ids, rows, ne, dst, &ea)) return rc;
+    infr::launch_embed_gather(dtype, ea.table, ea.bpr, ea.total_rows, static_cast<const int32_t*>(ids->ptr), rows,
+                              ne, scale, static_cast<float*>(dst->ptr), be->stream);
+    HIP_TRY(be, hipGetLastError());
+    return INFR_HIP_OK;
+}
+
 int infr_hip_linear_int_stages(infr_hip_t* be, int dtype, const infr_hip_buffer_t* w,
                                size_t w_numel, size_t w_off, const infr_hip_buffer_t* x, size_t m,
                                size_t in_f, size_t out_f, infr_hip_buffer_t* a,
@@ -729,6 +771,15 @@ int infr_hip_compile(infr_hip_t* be, const infr_hip_op_t* ops, size_t n_ops, inf
                 p->max_tensor = std::max(p->max_tensor, op.weight);
             if (op.kind == INFR_OP_GATED_ACT || op.kind == INFR_OP_ADD)
                 p->max_tensor = std::max(p->max_tensor, op.aux);
+        } else if (op.kind == INFR_OP_EMBED_GATHER) {
+            int qpb = 0, bpb = 0;
+            if (!infr::embed_gather_supported(op.w_dtype) || !infr_block_layout(op.w_dtype, &qpb, &bpb) ||
+                op.m == 0 || op.in_f == 0 || op.in_f % (uint32_t)qpb != 0 || op.w_numel == 0 ||
+                op.w_numel % op.in_f != 0) {
+                delete p;
+                return fail(be, INFR_HIP_ERR_UNSUPPORTED, "compile: EmbedGather op with unsupported dtype/shape");
+            }
+            p->max_tensor = std::max({p->max_tensor, op.x, op.weight, op.dst});
         } else {
             delete p;
             return fail(be, INFR_HIP_ERR_UNSUPPORTED, "compile: op kind " + std::to_string(op.kind));
@@ -753,7 +804,7 @@ size_t infr_hip_plan_launches(const infr_hip_plan_t* plan) {
     for (const auto& st : plan->steps) {
         if (st.op < 0) n += st.m > 1 ? 2 : 1;                              // grouped launch (+ grouped quantize)
         else if (plan->ops[st.op].kind == INFR_OP_MOE_FFN) n += plan->ops[st.op].moe.rows == 1 ? 3 : 7;
-        else if (is_elementwise(plan->ops[st.op].kind)) n += 1;
+        else if (is_elementwise(plan->ops[st.op].kind) || plan->ops[st.op].kind == INFR_OP_EMBED_GATHER) n += 1;
         else n += 2;                                                       // quantize + GEMM
     }
     return n;
@@ -807,6 +858,14 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
             const size_t abytes = (size_t)ms.rows * ms.ne * sizeof(float);
             rd[i] = {span(bindings[op.x], abytes), span(bindings[op.router_x], abytes)};
             wr[i] = {span(bindings[op.dst], abytes)};
+        } else if (op.kind == INFR_OP_EMBED_GATHER) {
+            EmbedArgs eg;
+            if (int rc = check_embed(be, op.w_dtype, bindings[op.weight], op.w_numel, bindings[op.x], op.m, op.in_f,
+                                     bindings[op.dst], &eg))
+                return rc;
+            rd[i] = {span(bindings[op.x], (size_t)op.m * sizeof(int32_t)),
+                     Span{eg.table, eg.table + eg.total_rows * eg.bpr}};
+            wr[i] = {span(bindings[op.dst], (size_t)op.m * op.in_f * sizeof(float))};
         } else if (is_elementwise(op.kind)) {
             if (int rc = check_elementwise(be, op, bindings, &ea[i])) return rc;
             rd[i] = {fspan(ea[i].x, ea[i].x_elems)};
@@ -1032,6 +1091,16 @@ static int enqueue_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t
                                    bindings[op.dst], nullptr, nullptr, &ms, &mb))
                 return rc;
             if (int rc = enqueue_moe(be, ms, mb)) return rc;
+        } else if (st.op >= 0 && plan->ops[st.op].kind == INFR_OP_EMBED_GATHER) {
+            const auto& op = plan->ops[st.op];
+            EmbedArgs eg;
+            if (int rc = check_embed(be, op.w_dtype, bindings[op.weight], op.w_numel, bindings[op.x], op.m, op.in_f,
+                                     bindings[op.dst], &eg))
+                return rc;
+            infr::launch_embed_gather(op.w_dtype, eg.table, eg.bpr, eg.total_rows,
+                                      static_cast<const int32_t*>(bindings[op.x]->ptr), op.m, op.in_f, op.scale,
+                                      static_cast<float*>(bindings[op.dst]->ptr), be->stream);
+            HIP_TRY(be, hipGetLastError());
         } else if (st.op >= 0 && is_elementwise(plan->ops[st.op].kind)) {
             ElementwiseArgs ea;
             if (int rc = check_elementwise(be, plan->ops[st.op], bindings, &ea)) return rc;
@@ -1089,7 +1158,7 @@ int infr_hip_execute(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t* c
     for (const auto& op : plan->ops) {
         const bool moe = op.kind == INFR_OP_MOE_FFN;
         // elementwise ops name their second operand per kind; check_elementwise validates it
-        if (!bindings[op.x] || !bindings[op.dst] || (op.kind == INFR_OP_LINEAR && !bindings[op.weight]) ||
+        if (!bindings[op.x] || !bindings[op.dst] || ((op.kind == INFR_OP_LINEAR || op.kind == INFR_OP_EMBED_GATHER) && !bindings[op.weight]) ||
             (moe && (!bindings[op.router_x] || !bindings[op.router] || !bindings[op.gate_exps] ||
                      !bindings[op.up_exps] || !bindings[op.down_exps])))
             return fail(be, INFR_HIP_ERR_INVALID, "execute: unbound tensor");

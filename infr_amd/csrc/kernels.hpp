@@ -155,6 +155,11 @@ bool gemv_takes_f32_activations(int dtype, size_t m);
 bool launch_gemv_f32act(int dtype, const uint8_t* w, size_t bpr, const float* x, float* y, size_t in_f,
                         size_t out_f, hipStream_t stream);
 
+// Op::EmbedGather: dst[r, :] = decode(table[ids[r], :]) * scale, rows decoded from the raw blocks.
+bool embed_gather_supported(int dtype);
+void launch_embed_gather(int dtype, const uint8_t* table, size_t bpr, size_t total_rows, const int32_t* ids,
+                         size_t rows, size_t ne, float scale, float* dst, hipStream_t stream);
+
 // Read-only streaming pass (measurement aid): `out` holds one int per workgroup.
 void launch_stream_read(const void* src, size_t bytes, int* out, int workgroups, hipStream_t stream);
 

@@ -334,6 +334,8 @@ int infr_block_layout(int dtype, int* elems, int* bytes) {
     int e, b;
     switch (dtype) {
     case INFR_DTYPE_F32: e = 1; b = 4; break;
+    case INFR_DTYPE_F16: e = 1; b = 2; break;
+    case INFR_DTYPE_BF16: e = 1; b = 2; break;
     case INFR_DTYPE_Q8_0: e = 32; b = 34; break;
     case INFR_DTYPE_Q4_K: e = 256; b = 144; break;
     case INFR_DTYPE_Q6_K: e = 256; b = 210; break;
@@ -364,7 +366,7 @@ void infr_synth_normal_f32(uint64_t seed, float mean, float sigma, size_t n, flo
 size_t infr_synth_weight(int dtype, uint64_t seed, float sigma, size_t rows, size_t in_f,
                          uint8_t* out) {
     int qpb, bpb;
-    if (!out || !infr_block_layout(dtype, &qpb, &bpb) || dtype == INFR_DTYPE_F32) return 0;
+    if (!out || !infr_block_layout(dtype, &qpb, &bpb) || qpb == 1) return 0;
     if (in_f == 0 || in_f % (size_t)qpb != 0) return 0;
     const size_t bpr = in_f / (size_t)qpb * (size_t)bpb;
     parallel_rows(rows, [&](size_t r) {

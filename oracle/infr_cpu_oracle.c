@@ -22,6 +22,7 @@ int orc_block_layout(int dtype, int *elems, int *bytes) {
     switch (dtype) {
     case ORC_F32: e = 1; b = 4; break;
     case ORC_F16: e = 1; b = 2; break;
+    case ORC_BF16: e = 1; b = 2; break;
     case ORC_Q4_0: e = 32; b = 18; break;
     case ORC_Q4_1: e = 32; b = 20; break;
     case ORC_Q5_0: e = 32; b = 22; break;
@@ -135,6 +136,12 @@ int orc_dequant_block(int dtype, const uint8_t *bytes, size_t nbytes, float *out
         return 0;
     case ORC_F16:
         for (size_t i = 0; i < nblk; i++) out[i] = orc_rdf16(bytes + 2 * i);
+        return 0;
+    case ORC_BF16: /* dequant.rs:19-22: the 16 bits are the top half of the f32 */
+        for (size_t i = 0; i < nblk; i++) {
+            uint32_t u = ((uint32_t)bytes[2 * i] | ((uint32_t)bytes[2 * i + 1] << 8)) << 16;
+            memcpy(&out[i], &u, 4);
+        }
         return 0;
     case ORC_Q8_0:
         for (size_t b = 0; b < nblk; b++) {
@@ -650,6 +657,32 @@ void orc_gated_act_fused(const float *gu, float *out, size_t rows, size_t nff, i
 /* crates/infr-cpu/src/lib.rs:1972-1988 */
 void orc_add(const float *a, const float *b, float *out, size_t n) {
     for (size_t i = 0; i < n; i++) out[i] = a[i] + b[i];
+}
+
+/* ───────────────────────────── Op::EmbedGather ───────────────────────────── */
+
+/* crates/infr-cpu/src/lib.rs:2084-2111: total_rows = numel / ne, bpr = bytes / total_rows; per row
+ * decode the token's row with the host decode and multiply by `scale`. Returns -2 where the
+ * reference would panic (an id past the table), -1 on a dtype the decode does not carry. */
+int orc_embed_gather(int dtype, const uint8_t *table, size_t table_bytes, size_t table_numel,
+                     const int32_t *ids, size_t rows, size_t ne, float scale, float *out) {
+    if (!table || !ids || !out || ne == 0 || table_numel % ne != 0) return -2;
+    size_t total_rows = table_numel / ne;
+    size_t bpr = table_bytes / total_rows;
+    float *row = (float *)malloc(sizeof(float) * ne);
+    for (size_t r = 0; r < rows; r++) {
+        if (ids[r] < 0 || (size_t)ids[r] >= total_rows) {
+            free(row);
+            return -2;
+        }
+        if (orc_dequant_block(dtype, table + (size_t)ids[r] * bpr, bpr, row) != 0) {
+            free(row);
+            return -1;
+        }
+        for (size_t e = 0; e < ne; e++) out[r * ne + e] = row[e] * scale;
+    }
+    free(row);
+    return 0;
 }
 
 /* ───────────────────────────── Op::Linear ───────────────────────────── */

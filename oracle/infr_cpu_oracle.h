@@ -59,6 +59,7 @@ enum {
     ORC_Q5_K = 13,
     ORC_Q6_K = 14,
     ORC_IQ4_NL = 20,
+    ORC_BF16 = 30,
     ORC_Q2_0 = 42
 };
 
@@ -142,6 +143,11 @@ void orc_gated_act_fused(const float *gu, float *out, size_t rows, size_t nff, i
                          int has_clamp, float clamp);
 /* Op::Add arm, lib.rs:1972-1988. */
 void orc_add(const float *a, const float *b, float *out, size_t n);
+
+/* Op::EmbedGather arm, crates/infr-cpu/src/lib.rs:2084-2111: out[r, :] = dequant(table row ids[r]) * scale.
+ * Returns 0; -1 unsupported dtype; -2 bad arguments or an id outside the table (the reference panics). */
+int orc_embed_gather(int dtype, const uint8_t *table, size_t table_bytes, size_t table_numel,
+                     const int32_t *ids, size_t rows, size_t ne, float scale, float *out);
 
 /* crates/infr-cpu/src/lib.rs:985-1492 — the Op::Linear arm for Q4_K/Q6_K/Q8_0/Q2_0/F32 weights.
  *   w/wbytes: the whole bound weight buffer; w_numel: its declared element count;

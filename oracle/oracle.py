@@ -19,6 +19,7 @@ _LIB_PATH = os.path.join(_HERE, "libinfr_cpu_oracle.so")
 
 F32, F16, Q8_0, Q4_K, Q6_K, Q2_0 = 0, 1, 8, 12, 14, 42
 Q4_0, Q4_1, Q5_0, Q5_1, Q5_K, IQ4_NL = 2, 3, 6, 7, 13, 20
+BF16 = 30
 KVALUES_IQ4NL = (-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113)
 ACTS_SUPER, ACTS_BLK32, ACTS_RAW = 0, 1, 2
 
@@ -67,6 +68,8 @@ _vd_q80 = _sig("orc_vec_dot_q8_0", C.c_float, _u8p, _i8p, _f32p, C.c_size_t, _i3
 _vd_q20 = _sig("orc_vec_dot_q2_0", C.c_float, _u8p, _i8p, _f32p, _i32p, C.c_size_t, _i32p)
 _vd_q5k = _sig("orc_vec_dot_q5k", C.c_float, _u8p, _i8p, _f32p, _i32p, C.c_size_t, _i32p, _i32p)
 _vd_b32 = _sig("orc_vec_dot_blk32", C.c_float, C.c_int, _u8p, _i8p, _f32p, _i32p, C.c_size_t, _i32p)
+_embed = _sig("orc_embed_gather", C.c_int, C.c_int, _u8p, C.c_size_t, C.c_size_t, _i32p, C.c_size_t, C.c_size_t,
+              C.c_float, _f32p)
 _dot = _sig("orc_dot", C.c_float, _f32p, _f32p, C.c_size_t)
 _silu = _sig("orc_silu", C.c_float, C.c_float)
 _linear = _sig("orc_linear", C.c_int, C.c_int, _u8p, C.c_size_t, C.c_size_t, C.c_size_t, _f32p,
@@ -213,6 +216,17 @@ def vec_dot_blk32(dtype: int, row, q8: Q8x32, in_f: int, stages: bool = False):
     y = _vd_b32(dtype, _p(row, _u8p), _p(q8.qs, _i8p), _p(q8.d, _f32p), _p(q8.bsum, _i32p), in_f,
                 _p(ip, _i32p))
     return (np.float32(y), ip) if stages else np.float32(y)
+
+
+def embed_gather(dtype: int, table, table_numel: int, ids, ne: int, scale: float = 1.0) -> np.ndarray:
+    """Op::EmbedGather on the CPU oracle: rows of ``table`` (raw blocks) decoded and scaled."""
+    table = _c(table, np.uint8).ravel() if np.asarray(table).dtype == np.uint8 else np.ascontiguousarray(table).view(np.uint8).ravel()
+    ids = _c(ids, np.int32).ravel()
+    out = np.empty((ids.size, ne), np.float32)
+    rc = _embed(dtype, _p(table, _u8p), table.size, table_numel, _p(ids, _i32p), ids.size, ne, scale, _p(out, _f32p))
+    if rc != 0:
+        raise ValueError(f"oracle embed_gather failed rc={rc}")
+    return out
 
 
 def dot(a, b) -> np.float32:
