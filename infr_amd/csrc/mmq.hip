@@ -704,7 +704,8 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
         return true;
     }
     launch_quantize_q8(x, m, in_f, act_is_per32(dtype, in_f), act, stream);
-    if (dtype != 12) return launch_gemv_batch(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
+    static const int env_dot4_max = getenv("INFR_HIP_Q4K_DOT4_MAX_M") ? atoi(getenv("INFR_HIP_Q4K_DOT4_MAX_M")) : 0;
+    if (dtype != 12 || (int)m <= env_dot4_max) return launch_gemv_batch(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
     if ((int)m <= env_skinny_max) {
         // four blocks per round; eight for long rows or when four would leave most SIMDs without a wave
         const size_t wgs = (out_f + 31) / 32 * ((m + 31) / 32);
