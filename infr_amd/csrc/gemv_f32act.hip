@@ -6,11 +6,12 @@
 //
 // One workgroup stages x in LDS once (padded by 4 floats per 32 so that the lanes' 16-byte reads
 // spread over all banks) and its four waves walk the tile's rows; lane l owns 32-weight block
-// t*64 + l of the row, fetched with the same loader as the int8 kernel. Weights are decoded with
-// the host decode's expression, sc * code + mn with sc = d * 1 and mn = d * (-16)
-// (crates/infr-gguf/src/dequant.rs:38-44, 173-189), and accumulated with fused multiply-adds as
-// `dot` does (kernels.rs:6557-6573); the order of the additions differs from the CPU's eight
-// accumulators, within f32 rounding. HBM-bound on the weight bytes (22 B per 32 weights).
+// t*64 + l of the row, fetched with the same loader as the int8 kernel. The host decode gives
+// w = d * code + d * (-16) (crates/infr-gguf/src/dequant.rs:38-44, 173-189); the kernel takes d out
+// of a block's 32 products: d * (sum code * x - 16 * sum x), the code sum as byte-to-float conversions (v_cvt_f32_ubyte) and FMAs
+// and the block sums of x computed once per workgroup. Same value in exact arithmetic, f32 rounding
+// in a different order than the CPU's `dot` (kernels.rs:6557-6573): about 1e-6 relative. The loop
+// is instruction-bound (two VALU operations per weight), not HBM-bound.
 #include "gemv_formats.hpp"
 #include "kernels.hpp"
 
@@ -22,40 +23,68 @@ __global__ __launch_bounds__(256) void gemv_f32act_kernel(const uint8_t* __restr
                                                           float* __restrict__ y, int in_f, int out_f,
                                                           int rows_per_wg) {
     extern __shared__ __attribute__((aligned(16))) float lx[];
+    const int nb = in_f / 32;
+    float* lsx = lx + (size_t)nb * 36;  // per-block sums of x
     for (int i = threadIdx.x * 4; i < in_f; i += 1024)
-        *reinterpret_cast<v4f*>(lx + i + (i >> 5) * 4) = *reinterpret_cast<const v4f*>(x + i);
+        *reinterpret_cast<v4f*>(lx + i + (i >> 5) * 4) = gload<v4f>(x + i);
+    __syncthreads();
+    for (int b = threadIdx.x; b < nb; b += 256) {
+        const v4f* xb = reinterpret_cast<const v4f*>(lx + (size_t)b * 36);
+        float sx = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const v4f v = xb[k];
+            sx += (v.x + v.y) + (v.z + v.w);
+        }
+        lsx[b] = sx;
+    }
     __syncthreads();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int nb = in_f / 32, steps = (nb + 63) / 64;
+    const int steps = (nb + 63) / 64;
     const int row_end = min(out_f, ((int)blockIdx.x + 1) * rows_per_wg);
-    for (int row = (int)blockIdx.x * rows_per_wg + wave; row < row_end; row += 4) {
-        const uint8_t* rowp = w + (size_t)row * bpr;
-        float acc = 0.0f;
-        for (int t = 0; t < steps; ++t) {
-            const bool ok = F::valid(t, lane, nb);
-            typename F::Row r;
-            F::load_row(r, rowp, t, lane, ok);
-            if (!ok) continue;
-            const float d = f16_bits_to_f32(r.dm & 0xFFFFu);
-            const float sc = d * 1.0f, mn = d * -16.0f;
-            const v4f* xb = reinterpret_cast<const v4f*>(lx + (size_t)(t * 64 + lane) * 36);
-            const int qw[4] = {r.qs.x, r.qs.y, r.qs.z, r.qs.w};
+    // The wave's (row, step) sequence is walked with the next step's block already requested.
+    int row = (int)blockIdx.x * rows_per_wg + wave, t = 0;
+    typename F::Row cur;
+    F::load_row(cur, w + (size_t)(row < row_end ? row : 0) * bpr, 0, lane, row < row_end && F::valid(0, lane, nb));
+    float acc = 0.0f;
+    while (row < row_end) {
+        const bool last = t + 1 == steps;
+        const int nrow = last ? row + 4 : row, nt = last ? 0 : t + 1;
+        typename F::Row nxt;
+        F::load_row(nxt, w + (size_t)(nrow < row_end ? nrow : 0) * bpr, nt, lane, nrow < row_end && F::valid(nt, lane, nb));
+        if (F::valid(t, lane, nb)) {
+            const int b = t * 64 + lane;
+            const v4f* xb = reinterpret_cast<const v4f*>(lx + (size_t)b * 36);
+            const int qw[4] = {cur.qs.x, cur.qs.y, cur.qs.z, cur.qs.w};
+            // sum over the block of code * x, then d * (that - 16 * sum x): the host decode's
+            // d * code + d * (-16) with the common factor taken out of the 32 products
+            float s1 = 0.0f;
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 const uint32_t wq = (uint32_t)qw[k];
-                const uint32_t lo = (wq & 0x0F0F0F0Fu) | spread4_to_bit4(r.qh >> (4 * k));
-                const uint32_t hi = ((wq >> 4) & 0x0F0F0F0Fu) | spread4_to_bit4(r.qh >> (16 + 4 * k));
+                const uint32_t lo = (wq & 0x0F0F0F0Fu) | spread4_to_bit4(cur.qh >> (4 * k));
+                const uint32_t hi = ((wq >> 4) & 0x0F0F0F0Fu) | spread4_to_bit4(cur.qh >> (16 + 4 * k));
                 const v4f x0 = xb[k], x1 = xb[4 + k];
-                const float xl[4] = {x0.x, x0.y, x0.z, x0.w}, xh[4] = {x1.x, x1.y, x1.z, x1.w};
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    acc = __builtin_fmaf(sc * (float)((lo >> (8 * j)) & 0xFFu) + mn, xl[j], acc);
-                    acc = __builtin_fmaf(sc * (float)((hi >> (8 * j)) & 0xFFu) + mn, xh[j], acc);
-                }
+                s1 = __builtin_fmaf((float)(lo & 0xFFu), x0.x, s1);
+                s1 = __builtin_fmaf((float)((lo >> 8) & 0xFFu), x0.y, s1);
+                s1 = __builtin_fmaf((float)((lo >> 16) & 0xFFu), x0.z, s1);
+                s1 = __builtin_fmaf((float)(lo >> 24), x0.w, s1);
+                s1 = __builtin_fmaf((float)(hi & 0xFFu), x1.x, s1);
+                s1 = __builtin_fmaf((float)((hi >> 8) & 0xFFu), x1.y, s1);
+                s1 = __builtin_fmaf((float)((hi >> 16) & 0xFFu), x1.z, s1);
+                s1 = __builtin_fmaf((float)(hi >> 24), x1.w, s1);
             }
+            const float d = f16_bits_to_f32(cur.dm & 0xFFFFu);
+            acc = __builtin_fmaf(d, s1 - 16.0f * lsx[b], acc);
         }
-        acc = wave_sum_f(acc);
-        if (lane == 0) y[row] = acc;
+        if (last) {
+            const float tot = wave_sum_f(acc);
+            if (lane == 0) gstore<float>(y + row, tot);
+            acc = 0.0f;
+        }
+        cur = nxt;
+        row = nrow;
+        t = nt;
     }
 }
 
@@ -64,7 +93,7 @@ bool gemv_takes_f32_activations(int dtype, size_t m) { return dtype == 6 && m ==
 bool launch_gemv_f32act(int dtype, const uint8_t* w, size_t bpr, const float* x, float* y, size_t in_f,
                         size_t out_f, hipStream_t stream) {
     if (dtype != 6 || in_f % 32 != 0) return false;
-    const size_t lds = (in_f + in_f / 8) * sizeof(float);
+    const size_t lds = (in_f + in_f / 8 + in_f / 32) * sizeof(float);
     if (lds > 64 * 1024) return false;  // rows longer than 14,563 elements: no kernel
     if (out_f == 0) return true;
     // enough workgroups to cover the machine a few times, at least 4 rows each (one per wave)

@@ -12,9 +12,6 @@
 //   kPer32                activation quantizer: per-32 (true) or per-256 (false)
 //   kOrdered              per-block terms are added in ascending block order (bit-exact with the
 //                         CPU's `sumf +=` chain) instead of a butterfly
-//   kPrefetch             wave steps whose loads are in flight ahead of the arithmetic (1 for every
-//                         format: depths of 2 and 3 measured 3-10 % slower on the small-block
-//                         formats, whose occupancy already covers the latency)
 //   kWide16Steps          up to this many wave steps per row the fused kernel fits 16 waves per
 //                         workgroup (128 VGPRs per lane) without spilling; beyond it, 8 waves
 //   units(in_f)           number of lane work units in a row (blocks for Q4_K/Q6_K ...)
@@ -52,7 +49,6 @@ struct FmtQ4K {
     static constexpr bool kOrdered = true;
     static constexpr int kBlockBytes = 144, kBlockElems = 256;
     static constexpr int kWide16Steps = 3;
-    static constexpr int kPrefetch = 1;
     struct Row {
         v4i hdr, qa, qb;
     };
@@ -143,7 +139,6 @@ struct FmtQ6K {
     static constexpr bool kOrdered = true;
     static constexpr int kBlockBytes = 210, kBlockElems = 256;
     static constexpr int kWide16Steps = 1;
-    static constexpr int kPrefetch = 1;
     struct Row {
         v4i qla, qlb, qh;
         v2i sc;
@@ -240,7 +235,6 @@ struct FmtQ8_0T {
     static constexpr bool kOrdered = false;
     static constexpr int kBlockBytes = 34, kBlockElems = 32;
     static constexpr int kWide16Steps = 4;
-    static constexpr int kPrefetch = 1;
     struct Row {
         v4i qa, qb;
         uint32_t d;
@@ -352,7 +346,6 @@ struct FmtQ2_0T {
     static constexpr bool kOrdered = false;
     static constexpr int kBlockBytes = 18, kBlockElems = 64;
     static constexpr int kWide16Steps = 3;
-    static constexpr int kPrefetch = 1;
     struct Row {
         v4i codes;
         uint32_t d;
@@ -446,7 +439,6 @@ struct FmtQ5K {
     static constexpr bool kOrdered = true;
     static constexpr int kBlockBytes = 176, kBlockElems = 256;
     static constexpr int kWide16Steps = 2;
-    static constexpr int kPrefetch = 1;
     struct Row {
         v4i hdr, ha, hb, qa, qb;
     };
@@ -539,7 +531,6 @@ struct FmtNib32 {
     static constexpr bool kOrdered = false;
     static constexpr int kBlockBytes = 18 + (kAffine ? 2 : 0) + (kFive ? 4 : 0), kBlockElems = 32;
     static constexpr int kWide16Steps = 4;
-    static constexpr int kPrefetch = 1;
     struct Row {
         v4i qs;
         uint32_t dm;  // f16 d in the low half, f16 m (affine formats) in the high half
@@ -659,7 +650,6 @@ struct FmtNib32Pair {
     static constexpr int kOneBlock = kFive ? 22 : 18;
     static constexpr int kBlockBytes = 2 * kOneBlock, kBlockElems = 64;
     static constexpr int kWide16Steps = 3;
-    static constexpr int kPrefetch = 1;
     struct Row {
         v4i q0, q1;
         uint32_t d01;  // f16 d of block 0 in the low half, of block 1 in the high half

@@ -14,9 +14,10 @@ struct OrderedSum {
 };
 
 // Rows [row0, row_end) of one weight matrix against activation registers `acts`. `first` already
-// holds step 0 of row0 (the caller issues those loads as early as it can). The loads run
-// F::kPrefetch wave steps (16 or 64 blocks each) ahead of the arithmetic, across row boundaries,
-// so a wave always has that many steps' bytes in flight.
+// holds step 0 of row0 (the caller issues those loads as early as it can). The loads run one wave
+// step (16 or 64 blocks) ahead of the arithmetic, across row boundaries, so a wave always has one
+// step's bytes in flight (two and three steps ahead measured 3-10 % slower on the small-block
+// formats, whose occupancy already covers the latency).
 //
 // Ordered formats (Q4_K, Q6_K): the CPU adds a row's per-block terms in ascending block order
 // (`sumf +=`). The quad leaders park each row's terms in LDS (`osum`, this wave's private
@@ -32,32 +33,26 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
                                           float* osum, const float* add_b = nullptr,
                                           float* add_dst = nullptr) {
     constexpr int LS = OrderedSum<STEPS>::kRowStride;
-    constexpr int D = F::kPrefetch;  // wave steps in flight ahead of the arithmetic
-    typename F::Row q[D];            // q[i]: the step i ahead of the one being computed
-    q[0] = first;
-#pragma unroll
-    for (int i = 1; i < D; ++i)
-        F::load_row(q[i], w + (size_t)(row0 + i / STEPS) * bpr, i % STEPS, lane,
-                    ok[i % STEPS] && row0 + i / STEPS < row_end);
     int in_batch = 0, batch_row0 = row0;
-    for (int row = row0; row < row_end; ++row) {
+    // One row: `cur0` holds its step 0; the loads of step t + 1 are issued before step t is
+    // computed, and the last step's prefetch - step 0 of the next row - lands in `next0`.
+    auto do_row = [&](int row, const typename F::Row& cur0, typename F::Row& next0) {
         const uint8_t* rowp = w + (size_t)row * bpr;
         float s = 0.0f;
+        typename F::Row cur = cur0;
 #pragma unroll
         for (int t = 0; t < STEPS; ++t) {
             typename F::Row nxt;
-            F::load_row(nxt, rowp + (size_t)((t + D) / STEPS) * bpr, (t + D) % STEPS, lane,
-                        ok[(t + D) % STEPS] && row + (t + D) / STEPS < row_end);
-            const float term = F::template term<STAGES>(q[0], acts[t], t, lane, ok[t], st,
+            if (t + 1 < STEPS) F::load_row(nxt, rowp, t + 1, lane, ok[t + 1 < STEPS ? t + 1 : 0]);
+            else F::load_row(next0, rowp + bpr, 0, lane, ok[0] && row + 1 < row_end);
+            const float term = F::template term<STAGES>(cur, acts[t], t, lane, ok[t], st,
                                                         (size_t)row * n_units);
             if (F::kOrdered) {
                 if ((lane & 3) == 0) osum[in_batch * LS + t * 16 + (lane >> 2)] = term;
             } else {
                 s += term;
             }
-#pragma unroll
-            for (int i = 0; i + 1 < D; ++i) q[i] = q[i + 1];
-            q[D - 1] = nxt;
+            if (t + 1 < STEPS) cur = nxt;
         }
         if (F::kOrdered) {
             if (++in_batch == 16 || row + 1 == row_end) {
@@ -86,6 +81,12 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
                 if (add_dst) gstore<float>(add_dst + row, s + gload<float>(add_b + row));
             }
         }
+    };
+    typename F::Row cur = first;
+    for (int row = row0; row < row_end; ++row) {
+        typename F::Row nxt;
+        do_row(row, cur, nxt);
+        cur = nxt;
     }
 }
 
@@ -154,13 +155,7 @@ __device__ __forceinline__ void gemv_rows_batch(const uint8_t* __restrict__ w, s
                                                 size_t st_stride, float* osum) {
     constexpr int LS = OrderedSum<STEPS>::kRowStride;
     constexpr int RB = 16 / MB;  // weight rows per ordered-sum flush
-    constexpr int D = F::kPrefetch;
-    typename F::Row q[D];
-    q[0] = first;
-#pragma unroll
-    for (int i = 1; i < D; ++i)
-        F::load_row(q[i], w + (size_t)(row0 + i / STEPS) * bpr, i % STEPS, lane,
-                    ok[i % STEPS] && row0 + i / STEPS < row_end);
+    typename F::Row cur = first;
     int in_batch = 0, batch_row0 = row0;
     for (int row = row0; row < row_end; ++row) {
         const uint8_t* rowp = w + (size_t)row * bpr;
@@ -170,13 +165,13 @@ __device__ __forceinline__ void gemv_rows_batch(const uint8_t* __restrict__ w, s
 #pragma unroll
         for (int t = 0; t < STEPS; ++t) {
             typename F::Row nxt;
-            F::load_row(nxt, rowp + (size_t)((t + D) / STEPS) * bpr, (t + D) % STEPS, lane,
-                        ok[(t + D) % STEPS] && row + (t + D) / STEPS < row_end);
+            if (t + 1 < STEPS) F::load_row(nxt, rowp, t + 1, lane, ok[t + 1 < STEPS ? t + 1 : 0]);
+            else F::load_row(nxt, rowp + bpr, 0, lane, ok[0] && row + 1 < row_end);
 #pragma unroll
             for (int mi = 0; mi < MB; ++mi) {
                 const StagePtrs sm{STAGES ? st.a + mi * st_stride : nullptr,
                                    STAGES && st.b ? st.b + mi * st_stride : nullptr};
-                const float term = F::template term<STAGES>(q[0], acts[mi][t], t, lane,
+                const float term = F::template term<STAGES>(cur, acts[mi][t], t, lane,
                                                             ok[t] && mi < m_valid, sm,
                                                             (size_t)row * n_units);
                 if (F::kOrdered) {
@@ -185,9 +180,7 @@ __device__ __forceinline__ void gemv_rows_batch(const uint8_t* __restrict__ w, s
                     s[mi] += term;
                 }
             }
-#pragma unroll
-            for (int i = 0; i + 1 < D; ++i) q[i] = q[i + 1];
-            q[D - 1] = nxt;
+            cur = nxt;
         }
         if (F::kOrdered) {
             if (++in_batch == RB || row + 1 == row_end) {
