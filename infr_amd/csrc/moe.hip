@@ -294,6 +294,64 @@ struct RawQ4K {
     }
 };
 
+// Q5_K: RawQ4K's mapping on the 176-byte block; the 5th code bit of sub-block s, element l, is
+// bit s of qh[l], so pair p adds bits 2p / 2p+1 of the block's 32 qh bytes to its two nibbles.
+struct RawQ5K {
+    static constexpr int kBlockBytes = 176;
+    struct Row {
+        v4i hdr, ha, hb, qa, qb;
+    };
+    typedef RawQ4K::X X;
+    __device__ static void load_row(Row& r, const uint8_t* rowp, int u, bool ok) {
+        if (ok) {
+            const uint8_t* blk = rowp + (size_t)(u >> 2) * 176;
+            const int p = u & 3;
+            r.hdr = load16(blk);
+            r.ha = load16(blk + 16);
+            r.hb = load16(blk + 32);
+            r.qa = load16(blk + 48 + p * 32);
+            r.qb = load16(blk + 64 + p * 32);
+        } else {
+            r.hdr = v4i{0, 0, 0, 0};
+            r.ha = v4i{0, 0, 0, 0};
+            r.hb = v4i{0, 0, 0, 0};
+            r.qa = v4i{0, 0, 0, 0};
+            r.qb = v4i{0, 0, 0, 0};
+        }
+    }
+    __device__ static void load_x(X& a, const float* xrow, int u, bool ok) { RawQ4K::load_x(a, xrow, u, ok); }
+    __device__ static float partial(const Row& r, const X& a, int u) {
+        const int p = u & 3;
+        uint32_t sc8[2], mn8[2];
+        k4_all((uint32_t)r.hdr.y, (uint32_t)r.hdr.z, (uint32_t)r.hdr.w, sc8, mn8);
+        const uint32_t scw = (p & 2) ? sc8[1] : sc8[0];
+        const uint32_t mnw = (p & 2) ? mn8[1] : mn8[0];
+        const int sh = (p & 1) * 16;
+        const float d = f16_bits_to_f32((uint32_t)r.hdr.x & 0xFFFFu);
+        const float dmin = f16_bits_to_f32((uint32_t)r.hdr.x >> 16);
+        const float fs_lo = d * (float)(int)((scw >> sh) & 0xFF), fs_hi = d * (float)(int)((scw >> (sh + 8)) & 0xFF);
+        const float fm_lo = dmin * (float)(int)((mnw >> sh) & 0xFF), fm_hi = dmin * (float)(int)((mnw >> (sh + 8)) & 0xFF);
+        const int wq[8] = {r.qa.x, r.qa.y, r.qa.z, r.qa.w, r.qb.x, r.qb.y, r.qb.z, r.qb.w};
+        const int hq[8] = {r.ha.x, r.ha.y, r.ha.z, r.ha.w, r.hb.x, r.hb.y, r.hb.z, r.hb.w};
+        float lo0 = 0.0f, lo1 = 0.0f, hi0 = 0.0f, hi1 = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const uint32_t w = (uint32_t)wq[k], hb = (uint32_t)hq[k] >> (2 * p);
+            const uint32_t l = (w & 0x0F0F0F0Fu) | ((hb & 0x01010101u) << 4);
+            const uint32_t h = ((w >> 4) & 0x0F0F0F0Fu) | (((hb >> 1) & 0x01010101u) << 4);
+            lo0 = __builtin_fmaf((float)(l & 0xFF), a.x[4 * k + 0], lo0);
+            lo1 = __builtin_fmaf((float)((l >> 8) & 0xFF), a.x[4 * k + 1], lo1);
+            lo0 = __builtin_fmaf((float)((l >> 16) & 0xFF), a.x[4 * k + 2], lo0);
+            lo1 = __builtin_fmaf((float)(l >> 24), a.x[4 * k + 3], lo1);
+            hi0 = __builtin_fmaf((float)(h & 0xFF), a.x[32 + 4 * k + 0], hi0);
+            hi1 = __builtin_fmaf((float)((h >> 8) & 0xFF), a.x[32 + 4 * k + 1], hi1);
+            hi0 = __builtin_fmaf((float)((h >> 16) & 0xFF), a.x[32 + 4 * k + 2], hi0);
+            hi1 = __builtin_fmaf((float)(h >> 24), a.x[32 + 4 * k + 3], hi1);
+        }
+        return (fs_lo * (lo0 + lo1) - fm_lo * a.sum_lo) + (fs_hi * (hi0 + hi1) - fm_hi * a.sum_hi);
+    }
+};
+
 // Q6_K: unit u = (block u/4, half h = (u%4)/2, c = u%2) as in the decode GEMV: the lane decodes
 // the four 16-element groups {l, l+32, l+64, l+96}, l in [16c, 16c+16), of its 128-element half;
 // group k has scale index h*8 + c + 2k. w = d * sc * (q - 32).
@@ -669,6 +727,7 @@ static bool launch_gemv_id(int dtype, const uint8_t* bank, size_t expert_stride,
                            size_t expert_stride1 = 0, float* y1 = nullptr) {
     switch (dtype) {
     case 12: return launch_gemv_id_fmt<FmtQ4K>(bank, expert_stride, bpr, ids, act, in_f, n_used, pairs, y, out_f, stream, bank1, expert_stride1, y1);
+    case 13: return launch_gemv_id_fmt<FmtQ5K>(bank, expert_stride, bpr, ids, act, in_f, n_used, pairs, y, out_f, stream, bank1, expert_stride1, y1);
     case 14: return launch_gemv_id_fmt<FmtQ6K>(bank, expert_stride, bpr, ids, act, in_f, n_used, pairs, y, out_f, stream, bank1, expert_stride1, y1);
     case 8: return launch_gemv_id_fmt<FmtQ8_0>(bank, expert_stride, bpr, ids, act, in_f, n_used, pairs, y, out_f, stream, bank1, expert_stride1, y1);
     default: return false;
@@ -737,9 +796,9 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
 
     if (s.rows == 1) {
         // ActsKind::Raw for every bank (lib.rs:2359: int8_ok = rows >= 2)
-        auto raw_ok = [](int dt) { return dt == 12 || dt == 14 || dt == 8; };
+        auto raw_ok = [](int dt) { return dt == 12 || dt == 13 || dt == 14 || dt == 8; };
         if (!raw_ok(s.gate_dtype) || s.up_dtype != s.gate_dtype || !raw_ok(s.down_dtype))
-            return "rows == 1 carries Q4_K / Q6_K / Q8_0 expert banks (gate and up of one format)";
+            return "rows == 1 carries Q4_K / Q5_K / Q6_K / Q8_0 expert banks (gate and up of one format)";
         if (s.ne > 4096 || s.n_ff > 4096) return "rows == 1 needs ne, n_ff_exp <= 4096";
         // row steps per wave: amortise the 64 activation registers while keeping >= ~1024 waves
         auto steps_per_wave = [](int wave_steps) { return std::max(1, std::min(4, wave_steps / 1024)); };
@@ -751,6 +810,7 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     hipLaunchKernelGGL((moe_gate_up_f32_kernel<P>), grid_g, dim3(256), 0, stream, b.gate, b.up, b.gate_stride, \
                        b.up_stride, sel_idx, b.x, gbuf, s.ne, s.n_ff, spw)
         if (s.gate_dtype == 12) INFR_GATE_UP(RawQ4K);
+        else if (s.gate_dtype == 13) INFR_GATE_UP(RawQ5K);
         else if (s.gate_dtype == 14) INFR_GATE_UP(RawQ6K);
         else INFR_GATE_UP(RawQ8_0);
 #undef INFR_GATE_UP
@@ -763,6 +823,7 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     hipLaunchKernelGGL((moe_down_f32_kernel<P>), grid_d, dim3((unsigned)(64 * nw_d)), 0, stream, b.down,   \
                        b.down_stride, sel_idx, sel_w, gbuf, b.dst, s.n_ff, s.ne, s.n_used, spw_d)
         if (s.down_dtype == 12) INFR_DOWN(RawQ4K);
+        else if (s.down_dtype == 13) INFR_DOWN(RawQ5K);
         else if (s.down_dtype == 14) INFR_DOWN(RawQ6K);
         else INFR_DOWN(RawQ8_0);
 #undef INFR_DOWN
@@ -773,6 +834,7 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     auto bytes_per_row = [](int dtype, size_t in_f) -> size_t {
         switch (dtype) {
         case 12: return in_f / 256 * 144;
+        case 13: return in_f / 256 * 176;
         case 14: return in_f / 256 * 210;
         case 8: return in_f / 32 * 34;
         default: return 0;
@@ -780,7 +842,7 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     };
     const size_t gbpr = bytes_per_row(s.gate_dtype, s.ne), ubpr = bytes_per_row(s.up_dtype, s.ne);
     const size_t dbpr = bytes_per_row(s.down_dtype, s.n_ff);
-    if (!gbpr || !ubpr || !dbpr) return "rows >= 2 carries Q4_K / Q6_K / Q8_0 expert banks";
+    if (!gbpr || !ubpr || !dbpr) return "rows >= 2 carries Q4_K / Q5_K / Q6_K / Q8_0 expert banks";
     launch_quantize_q8(b.x, s.rows, s.ne, false, aq, stream);
     const bool gate_up_ok =
         s.gate_dtype == s.up_dtype

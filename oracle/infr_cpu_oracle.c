@@ -904,9 +904,9 @@ void orc_ref_linear_f64(const float *x, const float *w, size_t m, size_t in_f, s
 
 /* crates/infr-cpu/src/moe.rs:42-53 (restricted to the dtypes this restatement decodes). */
 int orc_expert_acts_kind(int dtype, size_t in_f, int int8_ok) {
-    if (int8_ok && (dtype == ORC_Q4_K || dtype == ORC_Q6_K || dtype == ORC_Q8_0) && in_f % 256 == 0)
+    if (int8_ok && (dtype == ORC_Q4_K || dtype == ORC_Q6_K || dtype == ORC_Q8_0 || dtype == ORC_Q5_K) && in_f % 256 == 0)
         return ORC_ACTS_SUPER;
-    if (int8_ok && dtype == ORC_Q8_0 && in_f % 32 == 0) return ORC_ACTS_BLK32;
+    if (int8_ok && (dtype == ORC_Q8_0 || dtype == ORC_Q5_0) && in_f % 32 == 0) return ORC_ACTS_BLK32;
     return ORC_ACTS_RAW;
 }
 

@@ -76,7 +76,7 @@ def test_moe_router_ties_go_to_the_lower_index(be):
     assert list(idx[0]) == [4, 0, 1]
 
 
-@pytest.mark.parametrize("dtype", [DType.Q6K, DType.Q8_0])
+@pytest.mark.parametrize("dtype", [DType.Q6K, DType.Q8_0, DType.Q5K])
 def test_moe_int8_path_other_bank_formats(be, dtype):
     rows, ne, n_expert, n_used, nff = 3, 512, 8, 2, 256
     gate, up, down = banks(120, ne, n_expert, nff, dtype, sigma=0.05)
@@ -144,6 +144,7 @@ def test_moe_in_a_plan_replays(be, rows):
 
 
 @pytest.mark.parametrize("gu_dtype,down_dtype", [(DType.Q6K, DType.Q6K), (DType.Q8_0, DType.Q8_0),
+                                                 (DType.Q5K, DType.Q5K), (DType.Q5K, DType.Q6K),
                                                  (DType.Q4K, DType.Q6K), (DType.Q8_0, DType.Q4K)])
 @pytest.mark.parametrize("ne,nff", [(512, 256), (2048, 768)])
 def test_moe_one_token_other_bank_formats(be, gu_dtype, down_dtype, ne, nff):

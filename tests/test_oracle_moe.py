@@ -32,7 +32,7 @@ def make_banks(seed, ne, n_expert, n_ff, dtype):
     return gate, up, down
 
 
-@pytest.mark.parametrize("dtype", [orc.Q4_K, orc.Q6_K, orc.Q8_0])
+@pytest.mark.parametrize("dtype", [orc.Q4_K, orc.Q6_K, orc.Q8_0, orc.Q5_K])
 def test_rows1_matches_textbook_moe(dtype):
     ne, n_expert, n_used, n_ff = 256, 8, 2, 256
     rng = np.random.default_rng(4)
@@ -98,5 +98,9 @@ def test_expert_acts_kind_dispatch():
     assert orc.expert_acts_kind(orc.Q4_K, 2048, True) == orc.ACTS_SUPER
     assert orc.expert_acts_kind(orc.Q4_K, 2048, False) == orc.ACTS_RAW
     assert orc.expert_acts_kind(orc.Q8_0, 704, True) == orc.ACTS_BLK32
+    assert orc.expert_acts_kind(orc.Q5_K, 2048, True) == orc.ACTS_SUPER
+    assert orc.expert_acts_kind(orc.Q5_0, 704, True) == orc.ACTS_BLK32
+    assert orc.expert_acts_kind(orc.Q5_0, 704, False) == orc.ACTS_RAW
+    assert orc.expert_acts_kind(orc.Q4_0, 2048, True) == orc.ACTS_RAW
     assert orc.expert_acts_kind(orc.Q2_0, 2048, True) == orc.ACTS_RAW
     assert orc.expert_acts_kind(orc.F32, 2048, True) == orc.ACTS_RAW
