@@ -263,8 +263,10 @@ def single_shape(be, dtype, m, in_f, out_f, reps=40, rotate_bytes=768 << 20):
 
 def moe_bench(be, n_layers=6):
     """Routed-expert MoE at the Qwen3-30B-A3B shape (128 experts, top-8, hidden 2048, expert FFN
-    768, Q4_K banks), 1 and 16 tokens: `n_layers` Op::MoeFfn with distinct banks in one plan, so
-    the experts stream from HBM. Bytes = 2,654,208 per selected expert (gate+up+down)."""
+    768, Q4_K banks), 1 and 16 tokens, and prefill batches of 64 / 512 / 2048 tokens (pairs bucketed
+    by expert, int8 MFMA): `n_layers` Op::MoeFfn with distinct banks in one plan, so the experts
+    stream from HBM. Bytes = 2,654,208 per selected expert (gate+up+down); ops = 2 per weight and
+    pair."""
     from infr_amd import Bindings, BufferUsage, DType, Graph, MoeFfn, TensorDesc, synth_normal_f32, synth_weight
     ne, n_expert, n_used, nff = 2048, 128, 8, 768
     per_expert = 3 * nff * ne * 144 // 256
@@ -272,7 +274,7 @@ def moe_bench(be, n_layers=6):
                                          ne if i < 2 else nff), BufferUsage.Weights) for i in range(3)]
     router = be.upload_new(synth_normal_f32(80, n_expert * ne, sigma=0.03))
     out, keep = {}, list(protos) + [router]
-    for rows in (1, 16):
+    for rows in (1, 16, 64, 512, 2048):
         g, binds = Graph(), Bindings()
         x = synth_normal_f32(81 + rows, rows * ne)
         xid = g.input(TensorDesc((rows, ne), DType.F32))
@@ -307,6 +309,8 @@ def moe_bench(be, n_layers=6):
         # every layer routes the same x through the same router: unique experts per layer
         out[f"moe_q4k_t{rows}_us_per_layer"] = round(us, 2)
         out[f"moe_q4k_t{rows}_pair_GBs"] = round(rows * n_used * per_expert / (us * 1e-6) / 1e9, 1)
+        if rows >= 64:
+            out[f"moe_q4k_t{rows}_TOPS"] = round(rows * n_used * 3 * nff * ne * 2 / (us * 1e-6) / 1e12, 1)
         plan = None
     for b in keep:
         b.free()

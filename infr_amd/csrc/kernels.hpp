@@ -227,6 +227,21 @@ struct MoeBuffers {
     int32_t* sel_idx;       // optional [rows, n_used]
     float* sel_w;           // optional [rows, n_used]
 };
+// Routed pairs bucketed by expert, in tiles of at most 32 pairs of one expert each (device arrays;
+// `*n_tiles` of the `max_tiles` entries exist). `perm` lists the pairs expert by expert.
+struct MoeTileTable {
+    const int32_t* n_tiles;
+    const int32_t* expert;
+    const int32_t* slot0;
+    const int32_t* count;
+    const int32_t* perm;
+    int max_tiles;
+};
+// Q4_K int8-MFMA GEMM over such tiles: tile i multiplies rows perm[slot0[i]..] / act_div of the
+// quantized activations with expert[i]'s slice of `bank` and writes y[perm[..], :]. Same integers
+// and f32 epilogue as the dense kernel, so every output equals the per-pair GEMV's bit for bit.
+void launch_mmq_q4k_gathered(const uint8_t* bank, size_t expert_stride, size_t bpr, const ActQ8& act, int act_div,
+                             const MoeTileTable& t, float* y, size_t in_f, size_t out_f, hipStream_t stream);
 size_t moe_workspace_bytes(const MoeShape& s);
 // Enqueues the whole op; returns nullptr or a message naming what is unsupported.
 const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* workspace, hipStream_t stream);

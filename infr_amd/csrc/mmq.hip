@@ -83,21 +83,33 @@ struct ActStage {
     int bs[kSums];
     float d;
 
+    // Activation rows of this thread's pieces, resolved once per tile: `row_of(t)` maps tile slot
+    // t to a row of the quantized activations. Slots past the tile's last row repeat a valid row:
+    // their outputs are computed and never stored.
+    int q_row[kChunks], bs_row[kSums], d_row;
+    template <typename RowOf>
+    __device__ __forceinline__ void resolve(int tid, RowOf row_of) {
+#pragma unroll
+        for (int i = 0; i < kChunks; ++i) q_row[i] = row_of((tid + i * 256) >> 4);
+#pragma unroll
+        for (int i = 0; i < kSums; ++i) bs_row[i] = row_of(min(tid + i * 256, BM * 8 - 1) >> 3);
+        d_row = row_of(min(tid, BM - 1));
+    }
+
     __device__ __forceinline__ void fetch(const int8_t* qs, const float* d8, const int32_t* bsums,
-                                          int tok0, int m, int nb, int b, int tid) {
+                                          int nb, int b, int tid) {
         const size_t in_f = (size_t)nb * 256;
 #pragma unroll
         for (int i = 0; i < kChunks; ++i) {
-            // Tokens past m are clamped to the last row: their outputs are computed and never stored.
-            const int c = tid + i * 256, t = c >> 4, kc = c & 15, tok = min(tok0 + t, m - 1);
-            q[i] = *reinterpret_cast<const v4i*>(qs + (size_t)tok * in_f + (size_t)b * 256 + kc * 16);
+            const int kc = (tid + i * 256) & 15;
+            q[i] = *reinterpret_cast<const v4i*>(qs + (size_t)q_row[i] * in_f + (size_t)b * 256 + kc * 16);
         }
 #pragma unroll
         for (int i = 0; i < kSums; ++i) {
-            const int c = min(tid + i * 256, BM * 8 - 1), t = c >> 3, s = c & 7, tok = min(tok0 + t, m - 1);
-            bs[i] = bsums[(size_t)tok * (nb * 8) + b * 8 + s];
+            const int s = min(tid + i * 256, BM * 8 - 1) & 7;
+            bs[i] = bsums[(size_t)bs_row[i] * (nb * 8) + b * 8 + s];
         }
-        d = d8[(size_t)min(tok0 + min(tid, BM - 1), m - 1) * nb + b];
+        d = d8[(size_t)d_row * nb + b];
     }
 
     __device__ __forceinline__ void store(uint8_t* buf, int tid) const {
@@ -120,22 +132,62 @@ struct ActStage {
     }
 };
 
-template <int BM, bool STAGES>
+// Which rows a workgroup's tile of BM slots stands for.
+// Dense: tile blockIdx.y is tokens [BM * y, BM * y + BM) of an [m, in_f] activation and writes the
+// same rows of y.
+struct DenseTiles {
+    int m;
+    __device__ __forceinline__ bool select(int /*tile*/, size_t& /*w_off*/) const { return true; }
+    __device__ __forceinline__ int count(int tile, int bm) const { return min(bm, m - tile * bm); }
+    __device__ __forceinline__ int act_row(int tile, int bm, int t) const { return min(tile * bm + t, m - 1); }
+    __device__ __forceinline__ int out_row(int tile, int bm, int t) const { return tile * bm + t; }
+};
+// Gathered (routed experts): tile i covers `count[i]` entries of `perm` starting at `slot0[i]`, all
+// routed to expert `expert[i]`, whose weights start `expert_stride` bytes apart. An entry p is a
+// (token, rank) pair: it reads activation row p / act_div and writes output row p. Tiles at or
+// past `*n_tiles` do not exist (the grid is sized for the worst case).
+struct GatheredTiles {
+    const int32_t* n_tiles;
+    const int32_t* expert;
+    const int32_t* slot0;
+    const int32_t* count_;
+    const int32_t* perm;
+    size_t expert_stride;
+    int act_div;
+    __device__ __forceinline__ bool select(int tile, size_t& w_off) const {
+        if (tile >= *n_tiles) return false;
+        w_off = (size_t)expert[tile] * expert_stride;
+        return true;
+    }
+    __device__ __forceinline__ int count(int tile, int /*bm*/) const { return count_[tile]; }
+    __device__ __forceinline__ int act_row(int tile, int /*bm*/, int t) const {
+        return perm[slot0[tile] + min(t, count_[tile] - 1)] / act_div;
+    }
+    __device__ __forceinline__ int out_row(int tile, int /*bm*/, int t) const {
+        return perm[slot0[tile] + min(t, count_[tile] - 1)];
+    }
+};
+
+template <int BM, bool STAGES, typename TILES>
 __global__ __launch_bounds__(256) void mmq_q4k_kernel(const uint8_t* __restrict__ w, size_t bpr,
                                                       const int8_t* __restrict__ qs,
                                                       const float* __restrict__ d8,
                                                       const int32_t* __restrict__ bsums,
-                                                      float* __restrict__ y, int m, int out_f, int nb,
+                                                      float* __restrict__ y, TILES tiles, int out_f, int nb,
                                                       int32_t* __restrict__ st_sd,
                                                       int32_t* __restrict__ st_sm) {
     constexpr int TB = BM / 32;  // token blocks of 32
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // two MmqLds<BM> buffers
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, h = lane >> 5;
-    const int tok0 = blockIdx.y * BM;
+    const int tile_y = blockIdx.y;
+    size_t w_off = 0;
+    if (!tiles.select(tile_y, w_off)) return;  // uniform over the workgroup, before any barrier
+    const int n_slots = tiles.count(tile_y, BM);
+    const int tok0 = tile_y * BM;  // dense tiles only (the integer stages)
     const int wrow = blockIdx.x * 128 + wave * 32 + col;
     const bool row_ok = wrow < out_f;
-    const uint8_t* wrowp = w + (size_t)(row_ok ? wrow : 0) * bpr;
+    const uint8_t* wrowp = w + w_off + (size_t)(row_ok ? wrow : 0) * bpr;
 
     v16f acc[TB];
 #pragma unroll
@@ -144,7 +196,8 @@ __global__ __launch_bounds__(256) void mmq_q4k_kernel(const uint8_t* __restrict_
         for (int i = 0; i < 16; ++i) acc[tb][i] = 0.0f;
 
     ActStage<BM> stage;
-    stage.fetch(qs, d8, bsums, tok0, m, nb, 0, tid);
+    stage.resolve(tid, [&](int t) { return tiles.act_row(tile_y, BM, t); });
+    stage.fetch(qs, d8, bsums, nb, 0, tid);
     Q4kRaw raw;
     q4k_load_raw(raw, wrowp, h, row_ok);
     stage.store(lds, tid);
@@ -155,7 +208,7 @@ __global__ __launch_bounds__(256) void mmq_q4k_kernel(const uint8_t* __restrict_
         // ---- request block b+1: activation tile into registers, this wave's weight rows ----
         const Q4kRaw cur = raw;
         if (b + 1 < nb) {
-            stage.fetch(qs, d8, bsums, tok0, m, nb, b + 1, tid);
+            stage.fetch(qs, d8, bsums, nb, b + 1, tid);
             q4k_load_raw(raw, wrowp + (size_t)(b + 1) * 144, h, row_ok);
         }
 
@@ -212,8 +265,8 @@ __global__ __launch_bounds__(256) void mmq_q4k_kernel(const uint8_t* __restrict_
                     const int r = 4 * j + i;
                     const int sd = alo[r] + (ahi[r] << 3);
                     if (STAGES) {
-                        const int tok = tok0 + tb * 32 + 8 * j + 4 * h + i;
-                        if (row_ok && tok < m) {
+                        const int slot = tb * 32 + 8 * j + 4 * h + i, tok = tok0 + slot;
+                        if (row_ok && slot < n_slots) {
                             st_sd[((size_t)tok * out_f + wrow) * nb + b] = sd;
                             st_sm[((size_t)tok * out_f + wrow) * nb + b] = (int)smf[r];
                         }
@@ -234,8 +287,8 @@ __global__ __launch_bounds__(256) void mmq_q4k_kernel(const uint8_t* __restrict_
     for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const int tok = tok0 + tb * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-            if (tok < m) y[(size_t)tok * out_f + wrow] = acc[tb][r];
+            const int slot = tb * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+            if (slot < n_slots) y[(size_t)tiles.out_row(tile_y, BM, slot) * out_f + wrow] = acc[tb][r];
         }
 }
 
@@ -676,12 +729,21 @@ static void launch_mmq_q4k(const uint8_t* w, size_t bpr, const ActQ8& act, float
     const dim3 grid((unsigned)((out_f + 127) / 128), (unsigned)((m + BM - 1) / BM)), block(256);
     const int nb = (int)(in_f / 256);
     if (st.a)
-        hipLaunchKernelGGL((mmq_q4k_kernel<BM, true>), grid, block, 2 * MmqLds<BM>::bytes, stream, w, bpr,
-                           act.qs, act.d, act.bsums, y, (int)m, (int)out_f, nb, st.a, st.b);
+        hipLaunchKernelGGL((mmq_q4k_kernel<BM, true, DenseTiles>), grid, block, 2 * MmqLds<BM>::bytes, stream, w,
+                           bpr, act.qs, act.d, act.bsums, y, DenseTiles{(int)m}, (int)out_f, nb, st.a, st.b);
     else
-        hipLaunchKernelGGL((mmq_q4k_kernel<BM, false>), grid, block, 2 * MmqLds<BM>::bytes, stream, w, bpr,
-                           act.qs, act.d, act.bsums, y, (int)m, (int)out_f, nb, (int32_t*)nullptr,
+        hipLaunchKernelGGL((mmq_q4k_kernel<BM, false, DenseTiles>), grid, block, 2 * MmqLds<BM>::bytes, stream, w,
+                           bpr, act.qs, act.d, act.bsums, y, DenseTiles{(int)m}, (int)out_f, nb, (int32_t*)nullptr,
                            (int32_t*)nullptr);
+}
+
+void launch_mmq_q4k_gathered(const uint8_t* bank, size_t expert_stride, size_t bpr, const ActQ8& act, int act_div,
+                             const MoeTileTable& t, float* y, size_t in_f, size_t out_f, hipStream_t stream) {
+    const dim3 grid((unsigned)((out_f + 127) / 128), (unsigned)t.max_tiles), block(256);
+    const GatheredTiles g{t.n_tiles, t.expert, t.slot0, t.count, t.perm, expert_stride, act_div};
+    hipLaunchKernelGGL((mmq_q4k_kernel<32, false, GatheredTiles>), grid, block, 2 * MmqLds<32>::bytes, stream, bank,
+                       bpr, act.qs, act.d, act.bsums, y, g, (int)out_f, (int)(in_f / 256), (int32_t*)nullptr,
+                       (int32_t*)nullptr);
 }
 
 bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const ActQ8& act, float* y,

@@ -218,6 +218,82 @@ __global__ __launch_bounds__(256) void moe_router_kernel(
     if (tid == 0) *tickets = 0;
 }
 
+// Prefill form of the router (rows >= kRtMinRows): the same eight accumulator chains per
+// (expert, token) dot, register-tiled so that LDS is read half a word per FMA instead of two. A
+// workgroup of two wavefronts takes 16 experts x 16 tokens; its 16 groups of eight lanes each own
+// a 4 x 4 tile of pairs - experts eg + 4i, tokens tg + 4i, so that the lanes of a wavefront read 32
+// distinct banks - and lane j of a group carries accumulator j of all 16 pairs. The next K-chunk
+// is fetched into registers while the current one is multiplied.
+constexpr int kRtE = 16, kRtT = 16, kRtK = 256, kRtThreads = 128, kRtMinRows = 256;
+constexpr int kRtLoads = (kRtE + kRtT) * (kRtK / 4) / kRtThreads;  // 16-byte loads per thread and chunk
+
+__global__ __launch_bounds__(kRtThreads) void moe_router_tile_kernel(const float* __restrict__ router,
+                                                                     const float* __restrict__ rx,
+                                                                     float* __restrict__ logits, int ne,
+                                                                     int n_expert, int rows) {
+    __shared__ __attribute__((aligned(16))) float lrow[kRtE + kRtT][kRtK + 8];  // experts, then tokens
+    const int tid = threadIdx.x, j = tid & 7, tile = tid >> 3;
+    const int eg = tile & 3, tg = tile >> 2;
+    const int e0 = blockIdx.x * kRtE, t0 = blockIdx.y * kRtT;
+    // this thread's pieces of a chunk: row (i * kRtThreads + tid) / 64, float4 column % 64;
+    // rows past the last expert / token repeat it (computed, never stored)
+    const float* src[kRtLoads];
+#pragma unroll
+    for (int i = 0; i < kRtLoads; ++i) {
+        const int idx = i * kRtThreads + tid, row = idx / (kRtK / 4), q = idx % (kRtK / 4);
+        src[i] = (row < kRtE ? router + (size_t)min(e0 + row, n_expert - 1) * ne
+                             : rx + (size_t)min(t0 + row - kRtE, rows - 1) * ne) + 4 * q;
+    }
+    v4f stage[kRtLoads];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < kRtLoads; ++i) {
+            const int q = (i * kRtThreads + tid) % (kRtK / 4);
+            stage[i] = k0 + 4 * q < ne ? *reinterpret_cast<const v4f*>(src[i] + k0) : v4f{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    };
+    float acc[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) acc[a][b] = 0.0f;
+    fetch(0);
+    for (int k0 = 0; k0 < ne; k0 += kRtK) {
+        const int n = min(kRtK, ne - k0);
+        if (k0) __syncthreads();  // the previous chunk's readers are done
+#pragma unroll
+        for (int i = 0; i < kRtLoads; ++i) {
+            const int idx = i * kRtThreads + tid;
+            reinterpret_cast<v4f*>(&lrow[idx / (kRtK / 4)][0])[idx % (kRtK / 4)] = stage[i];
+        }
+        __syncthreads();
+        if (k0 + kRtK < ne) fetch(k0 + kRtK);
+#pragma unroll 4
+        for (int c = 0; c < n / 8; ++c) {
+            float a[4], x[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                a[i] = lrow[eg + 4 * i][c * 8 + j];
+                x[i] = lrow[kRtE + tg + 4 * i][c * 8 + j];
+            }
+#pragma unroll
+            for (int ie = 0; ie < 4; ++ie)
+#pragma unroll
+                for (int it = 0; it < 4; ++it) acc[ie][it] = __builtin_fmaf(a[ie], x[it], acc[ie][it]);
+        }
+    }
+#pragma unroll
+    for (int ie = 0; ie < 4; ++ie)
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            float sum = 0.0f;  // acc[0] + acc[1] + ... + acc[7] in order
+#pragma unroll
+            for (int q = 0; q < 8; ++q) sum += __shfl(acc[ie][it], (tid & 63 & ~7) + q, kWave);
+            const int e = e0 + eg + 4 * ie, t = t0 + tg + 4 * it;
+            if (j == 0 && e < n_expert && t < rows) logits[(size_t)t * n_expert + e] = sum;
+        }
+}
+
 // ───────────────────────────── rows == 1: f32 (ActsKind::Raw) path ─────────────────────────────
 // A lane owns 64 consecutive-or-strided weights of a row ("unit" u of the row's in_f / 64) and
 // keeps the matching 64 activation floats in registers; S = in_f / 64 lanes cover a weight row and
@@ -674,6 +750,49 @@ __global__ __launch_bounds__(256) void moe_accumulate_kernel(const float* __rest
     out[i] = acc;
 }
 
+// Buckets the routed pairs by expert for the prefill path: perm = pair ids grouped by expert,
+// plus one tile entry per 32 pairs of an expert. One workgroup; the order of pairs inside a bucket
+// depends on the order the atomics land in and does not matter (each pair's outputs are its own).
+constexpr int kBucketThreads = 1024;
+__global__ __launch_bounds__(kBucketThreads) void moe_bucket_kernel(
+    const int32_t* __restrict__ sel_idx, int pairs, int n_expert, int32_t* __restrict__ perm,
+    int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_slot0, int32_t* __restrict__ tile_count,
+    int32_t* __restrict__ n_tiles) {
+    constexpr int tile_rows = 32;  // 64-pair tiles measured slower (704 us against 554 at 2048 tokens)
+    __shared__ int cnt[kBucketThreads], off[kBucketThreads], toff[kBucketThreads], cursor[kBucketThreads];
+    const int tid = threadIdx.x;
+    cnt[tid] = 0;
+    cursor[tid] = 0;
+    __syncthreads();
+    for (int p = tid; p < pairs; p += kBucketThreads) atomicAdd(&cnt[sel_idx[p]], 1);
+    __syncthreads();
+    const int mine = tid < n_expert ? cnt[tid] : 0, my_tiles = (mine + tile_rows - 1) / tile_rows;
+    off[tid] = mine;
+    toff[tid] = my_tiles;
+    __syncthreads();
+    for (int d = 1; d < kBucketThreads; d <<= 1) {  // inclusive scans of both arrays
+        const int a = tid >= d ? off[tid - d] : 0, b = tid >= d ? toff[tid - d] : 0;
+        __syncthreads();
+        off[tid] += a;
+        toff[tid] += b;
+        __syncthreads();
+    }
+    const int first_slot = off[tid] - mine, first_tile = toff[tid] - my_tiles;
+    if (tid == kBucketThreads - 1) *n_tiles = toff[tid];
+    for (int k = 0; k < my_tiles; ++k) {
+        tile_expert[first_tile + k] = tid;
+        tile_slot0[first_tile + k] = first_slot + tile_rows * k;
+        tile_count[first_tile + k] = min(tile_rows, mine - tile_rows * k);
+    }
+    __syncthreads();
+    off[tid] = first_slot;
+    __syncthreads();
+    for (int p = tid; p < pairs; p += kBucketThreads) {
+        const int e = sel_idx[p];
+        perm[off[e] + atomicAdd(&cursor[e], 1)] = p;
+    }
+}
+
 // ───────────────────────────── launch ─────────────────────────────
 
 // `bank1`/`y1` (optional): a second bank of the same dtype and shape against the same activations.
@@ -750,6 +869,12 @@ size_t moe_workspace_bytes(const MoeShape& s) {
     add(qmax / 32 * 4);                           // d (sized for either quantizer)
     add(qmax / 32 * 4);                           // bsums
     add(qmax / 16 * 4);                           // bsums16
+    const size_t max_tiles = pairs / 32 + std::min((size_t)s.n_expert, pairs);
+    add(4);                                       // n_tiles
+    add(pairs * 4);                               // perm
+    add(max_tiles * 4);                           // tile expert
+    add(max_tiles * 4);                           // tile slot0
+    add(max_tiles * 4);                           // tile count
     return n;
 }
 
@@ -777,6 +902,12 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     aq.d = (float*)take(qmax / 32 * 4);
     aq.bsums = (int32_t*)take(qmax / 32 * 4);
     aq.bsums16 = (int32_t*)take(qmax / 16 * 4);
+    const size_t max_tiles = pairs / 32 + std::min((size_t)s.n_expert, pairs);
+    int32_t* n_tiles = (int32_t*)take(4);
+    int32_t* perm = (int32_t*)take(pairs * 4);
+    int32_t* tile_expert = (int32_t*)take(max_tiles * 4);
+    int32_t* tile_slot0 = (int32_t*)take(max_tiles * 4);
+    int32_t* tile_count = (int32_t*)take(max_tiles * 4);
 
     // one expert per workgroup at a single row (more workgroups), four once rows fill the pairs;
     // whole rows in one chunk when they fit 64 KiB of LDS, else kRouterChunk columns at a time
@@ -784,10 +915,16 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     const int n_t = std::min(s.rows, tpw);
     const int kc = (size_t)(epw + n_t) * (s.ne + 8) * 4 <= 64 * 1024 ? s.ne : kRouterChunk;
     const size_t router_lds = (size_t)(epw + n_t) * (kc + 8) * sizeof(float);
-    hipLaunchKernelGGL(moe_router_kernel,
-                       dim3((unsigned)((s.n_expert + epw - 1) / epw), (unsigned)((s.rows + tpw - 1) / tpw)),
-                       dim3(256), router_lds, stream, b.router, b.router_x, logits, s.rows == 1 ? tickets : nullptr,
-                       sel_idx, sel_w, s.ne, s.n_expert, s.rows, s.n_used, s.scale, kc, epw);
+    if (s.rows >= kRtMinRows)
+        hipLaunchKernelGGL(moe_router_tile_kernel,
+                           dim3((unsigned)((s.n_expert + kRtE - 1) / kRtE), (unsigned)((s.rows + kRtT - 1) / kRtT)),
+                           dim3(kRtThreads), 0, stream, b.router, b.router_x, logits, s.ne, s.n_expert, s.rows);
+    else
+        hipLaunchKernelGGL(moe_router_kernel,
+                           dim3((unsigned)((s.n_expert + epw - 1) / epw), (unsigned)((s.rows + tpw - 1) / tpw)),
+                           dim3(256), router_lds, stream, b.router, b.router_x, logits,
+                           s.rows == 1 ? tickets : nullptr, sel_idx, sel_w, s.ne, s.n_expert, s.rows, s.n_used,
+                           s.scale, kc, epw);
     if (s.rows > 1)
         hipLaunchKernelGGL(moe_select_kernel, dim3((unsigned)s.rows), dim3(256), 0, stream, logits, sel_idx,
                            sel_w, s.n_expert, s.n_used, s.scale);
@@ -844,6 +981,26 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     const size_t dbpr = bytes_per_row(s.down_dtype, s.n_ff);
     if (!gbpr || !ubpr || !dbpr) return "rows >= 2 carries Q4_K / Q5_K / Q6_K / Q8_0 expert banks";
     launch_quantize_q8(b.x, s.rows, s.ne, false, aq, stream);
+    const size_t n_act = pairs * s.n_ff, n_out = (size_t)s.rows * s.ne;
+    // Prefill-sized batches of all-Q4_K banks: bucket the pairs by expert and run the int8-MFMA
+    // GEMM per (expert, 32 pairs) tile, so an expert's weights are read once per 32 of its pairs
+    // instead of once per pair. From an average of `bucket_min` pairs per expert up (the
+    // per-pair GEMVs win below: most tiles would hold one or two pairs).
+    static const int bucket_min = getenv("INFR_HIP_MOE_BUCKET_MIN") ? atoi(getenv("INFR_HIP_MOE_BUCKET_MIN")) : 4;
+    if (s.gate_dtype == 12 && s.up_dtype == 12 && s.down_dtype == 12 && bucket_min > 0 &&
+        pairs >= (size_t)bucket_min * s.n_expert && pairs <= (size_t)1 << 24) {
+        hipLaunchKernelGGL(moe_bucket_kernel, dim3(1), dim3(kBucketThreads), 0, stream, sel_idx, (int)pairs,
+                           s.n_expert, perm, tile_expert, tile_slot0, tile_count, n_tiles);
+        const MoeTileTable tt{n_tiles, tile_expert, tile_slot0, tile_count, perm, (int)max_tiles};
+        launch_mmq_q4k_gathered(b.gate, b.gate_stride, gbpr, aq, s.n_used, tt, gbuf, s.ne, s.n_ff, stream);
+        launch_mmq_q4k_gathered(b.up, b.up_stride, ubpr, aq, s.n_used, tt, ubuf, s.ne, s.n_ff, stream);
+        hipLaunchKernelGGL(moe_act_quant_kernel, dim3((unsigned)((n_act / 256 + 3) / 4)), dim3(256), 0, stream,
+                           gbuf, ubuf, aq.qs, aq.d, aq.bsums, aq.bsums16, n_act);
+        launch_mmq_q4k_gathered(b.down, b.down_stride, dbpr, aq, 1, tt, yp, s.n_ff, s.ne, stream);
+        hipLaunchKernelGGL(moe_accumulate_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, stream,
+                           yp, sel_w, b.dst, s.ne, s.n_used, s.rows);
+        return hipGetLastError() == hipSuccess ? nullptr : "kernel launch failed";
+    }
     const bool gate_up_ok =
         s.gate_dtype == s.up_dtype
             ? launch_gemv_id(s.gate_dtype, b.gate, b.gate_stride, gbpr, sel_idx, aq, s.ne, s.n_used, (int)pairs, gbuf,
@@ -853,13 +1010,11 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
                   launch_gemv_id(s.up_dtype, b.up, b.up_stride, ubpr, sel_idx, aq, s.ne, s.n_used, (int)pairs, ubuf,
                                  s.n_ff, stream);
     if (!gate_up_ok) return "no id-gathered kernel for this gate/up shape";
-    const size_t n_act = pairs * s.n_ff;
     hipLaunchKernelGGL(moe_act_quant_kernel, dim3((unsigned)((n_act / 256 + 3) / 4)), dim3(256), 0, stream,
                        gbuf, ubuf, aq.qs, aq.d, aq.bsums, aq.bsums16, n_act);
     // the down GEMV's activation row is the pair itself: n_used = 1
     if (!launch_gemv_id(s.down_dtype, b.down, b.down_stride, dbpr, sel_idx, aq, s.n_ff, 1, (int)pairs, yp, s.ne, stream))
         return "no id-gathered kernel for this down shape";
-    const size_t n_out = (size_t)s.rows * s.ne;
     hipLaunchKernelGGL(moe_accumulate_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, stream,
                        yp, sel_w, b.dst, s.ne, s.n_used, s.rows);
     return hipGetLastError() == hipSuccess ? nullptr : "kernel launch failed";

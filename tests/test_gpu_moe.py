@@ -166,3 +166,55 @@ def test_moe_one_token_other_bank_formats(be, gu_dtype, down_dtype, ne, nff):
     want = orc.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
                        gate_dtype=int(gu_dtype), up_dtype=int(gu_dtype), down_dtype=int(down_dtype))
     check(*got, *want)
+
+
+@pytest.mark.parametrize("rows,ne,n_expert,n_used,nff", [(64, 512, 16, 4, 256), (40, 1024, 8, 2, 768),
+                                                         (200, 512, 16, 4, 512),
+                                                         (400, 512, 8, 2, 256)])     # the tiled router (rows >= 256), ~100 pairs per expert
+def test_moe_prefill_buckets_vs_oracle(be, rows, ne, n_expert, n_used, nff):
+    """Prefill-sized batches of all-Q4_K banks: pairs bucketed by expert, int8-MFMA GEMM per (expert,
+    32 pairs) tile. Same integers and epilogue as the per-pair GEMVs: the first two tokens of the
+    batch, run again as a batch of two (per-pair path), give the same bits."""
+    gate, up, down = banks(70 + rows, ne, n_expert, nff, sigma=0.05)
+    x = synth_normal_f32(71 + rows, rows * ne)
+    router = synth_normal_f32(72, n_expert * ne, sigma=0.05)
+    got = run_moe(be, x, router, gate, up, down, rows, ne, n_expert, n_used, nff, 1.0)
+    want = orc.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff, scale=1.0)
+    check(*got, *want)
+    two = run_moe(be, x[:2 * ne], router, gate, up, down, 2, ne, n_expert, n_used, nff, 1.0)
+    assert np.array_equal(two[1], got[1][:2])
+    assert np.array_equal(two[0].view(np.uint32), got[0][:2].view(np.uint32)), "bucketed != per-pair"
+
+
+def test_moe_prefill_buckets_with_idle_and_crowded_experts(be):
+    """A router that sends every token to the same two experts plus one of two others: buckets of
+    0, a few and > 32 pairs (several tiles per expert, a ragged last tile)."""
+    rows, ne, n_expert, n_used, nff = 75, 512, 16, 3, 256
+    gate, up, down = banks(90, ne, n_expert, nff, sigma=0.05)
+    x = np.abs(synth_normal_f32(91, rows * ne)) + np.float32(0.1)     # all-positive activations
+    router = np.zeros((n_expert, ne), np.float32)
+    router[3], router[11] = 0.05, 0.04                                 # always the top two
+    router[5, :ne // 2], router[6, ne // 2:] = 0.06, 0.06              # third place depends on the token
+    x = x.reshape(rows, ne)
+    x[::7, :ne // 2] *= 3.0
+    x = x.ravel()
+    got = run_moe(be, x, router.ravel(), gate, up, down, rows, ne, n_expert, n_used, nff, 1.0)
+    want = orc.moe_ffn(x, router.ravel(), gate, up, down, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
+                       scale=1.0)
+    assert set(np.unique(got[1])) <= {3, 5, 6, 11} and np.bincount(got[1].ravel(), minlength=16)[3] == rows
+    check(*got, *want)
+
+
+def test_moe_qwen3_30b_a3b_prefill(be):
+    """512 tokens at the Qwen3-30B-A3B shape (4096 pairs over 128 experts), sampled rows against the
+    oracle run on those rows alone (each token's output is independent of the rest of the batch)."""
+    ne, n_expert, n_used, nff, rows = 2048, 128, 8, 768, 512
+    gate, up, down = banks(7, ne, n_expert, nff)
+    x = synth_normal_f32(8, rows * ne)
+    router = synth_normal_f32(9, n_expert * ne, sigma=0.05)
+    y, idx, w = run_moe(be, x, router, gate, up, down, rows, ne, n_expert, n_used, nff, 1.0)
+    pick = [0, 1, 255, 256, 510, 511]
+    xs = np.concatenate([x[r * ne:(r + 1) * ne] for r in pick])
+    want = orc.moe_ffn(xs, router, gate, up, down, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff, scale=1.0)
+    check(y[pick], idx[pick], w[pick], *want)
+    assert np.isfinite(y).all() and len(np.unique(idx)) > 100        # most experts are touched
