@@ -14,11 +14,16 @@
 //                         CPU's `sumf +=` chain) instead of a butterfly
 //   kWide16Steps          up to this many wave steps per row the fused kernel fits 16 waves per
 //                         workgroup (128 VGPRs per lane) without spilling; beyond it, 8 waves
+//   kRowAhead             rows of several wave steps request step t of the next row before step t
+//                         of this one is computed (a whole row in flight) instead of one step ahead
+//   kClampedLoads         has load_row_clamped: for a row known to be readable, lanes without
+//                         work read block 0 instead of being masked off
 //   units(in_f)           number of lane work units in a row (blocks for Q4_K/Q6_K ...)
 //   Row / Acts            registers for one step of a weight row / of the activation
 //   valid(t, lane, n)     does this lane have work in step t
 //   load_row, load_acts   fill them (acts from any address space: global or LDS pointers)
 //   term(...)             exact integer stage + f32 term of the lane's unit; writes stage outputs
+//   term_shared(...)      optional: the same when one weight row meets several activation rows
 #pragma once
 
 #include "device_common.hpp"
@@ -49,6 +54,8 @@ struct FmtQ4K {
     static constexpr bool kOrdered = true;
     static constexpr int kBlockBytes = 144, kBlockElems = 256;
     static constexpr int kWide16Steps = 3;
+    static constexpr bool kClampedLoads = false;
+    static constexpr bool kRowAhead = false;
     struct Row {
         v4i hdr, qa, qb;
     };
@@ -139,6 +146,8 @@ struct FmtQ6K {
     static constexpr bool kOrdered = true;
     static constexpr int kBlockBytes = 210, kBlockElems = 256;
     static constexpr int kWide16Steps = 1;
+    static constexpr bool kClampedLoads = false;
+    static constexpr bool kRowAhead = false;
     struct Row {
         v4i qla, qlb, qh;
         v2i sc;
@@ -235,6 +244,8 @@ struct FmtQ8_0T {
     static constexpr bool kOrdered = false;
     static constexpr int kBlockBytes = 34, kBlockElems = 32;
     static constexpr int kWide16Steps = 4;
+    static constexpr bool kClampedLoads = false;
+    static constexpr bool kRowAhead = false;
     struct Row {
         v4i qa, qb;
         uint32_t d;
@@ -346,6 +357,8 @@ struct FmtQ2_0T {
     static constexpr bool kOrdered = false;
     static constexpr int kBlockBytes = 18, kBlockElems = 64;
     static constexpr int kWide16Steps = 3;
+    static constexpr bool kClampedLoads = true;
+    static constexpr bool kRowAhead = true;
     struct Row {
         v4i codes;
         uint32_t d;
@@ -358,23 +371,30 @@ struct FmtQ2_0T {
     __device__ static bool valid(int t, int lane, int n) { return t * 64 + lane < n; }
     __device__ static void load_row(Row& r, const uint8_t* rowp, int t, int lane, bool ok) {
         if (ok) {
-            const uint8_t* blk = rowp + (size_t)(t * 64 + lane) * 18;
-            if (ALIGNED) {
-                const bool odd = (lane & 1) != 0;  // t * 64 is even
-                const uint8_t* a = blk - (odd ? 2 : 0);
-                const v4i lo = load16_a4(a);
-                const int w4 = load_u32(a + 16);
-                const uint32_t sel = realign2_selector(odd);
-                r.d = odd ? (uint32_t)lo.x >> 16 : (uint32_t)lo.x & 0xFFFFu;
-                r.codes = v4i{realign2(lo.x, lo.y, sel), realign2(lo.y, lo.z, sel), realign2(lo.z, lo.w, sel),
-                              realign2(lo.w, w4, sel)};
-            } else {
-                r.d = load_u16(blk);
-                r.codes = load16_a2(blk + 2);
-            }
+            load_row_clamped(r, rowp, t, lane, true);
         } else {
             r.codes = v4i{0, 0, 0, 0};
             r.d = 0;
+        }
+    }
+    // For a `rowp` that is a readable row whatever `ok` says: lanes past the row's last block read
+    // block 0 instead of being masked off (their activations are zero, so what they load
+    // contributes +0.0), and the loads carry no predicate.
+    __device__ static void load_row_clamped(Row& r, const uint8_t* rowp, int t, int lane, bool ok) {
+        const int idx = ok ? t * 64 + lane : 0;
+        const uint8_t* blk = rowp + (size_t)idx * 18;
+        if (ALIGNED) {
+            const bool odd = (idx & 1) != 0;
+            const uint8_t* a = blk - (odd ? 2 : 0);
+            const v4i lo = load16_a4(a);
+            const int w4 = load_u32(a + 16);
+            const uint32_t sel = realign2_selector(odd);
+            r.d = odd ? (uint32_t)lo.x >> 16 : (uint32_t)lo.x & 0xFFFFu;
+            r.codes = v4i{realign2(lo.x, lo.y, sel), realign2(lo.y, lo.z, sel), realign2(lo.z, lo.w, sel),
+                          realign2(lo.w, w4, sel)};
+        } else {
+            r.d = load_u16(blk);
+            r.codes = load16_a2(blk + 2);
         }
     }
     __device__ static void load_acts(Acts& a, const ActPtrs& s, int t, int lane, bool ok) {
@@ -402,15 +422,46 @@ struct FmtQ2_0T {
     template <bool STAGES>
     __device__ static float term(const Row& r, const Acts& a, int t, int lane, bool ok,
                                  const StagePtrs& st, size_t row_units) {
+        return term_impl<STAGES, false>(r, a, t, lane, ok, st, row_units);
+    }
+    // One weight row against several activation rows: the unpacked code words are shared by all
+    // of them, so the plain four-shift unpack with one accumulator per sub-block is cheaper there
+    // than the two-accumulator form below.
+    template <bool STAGES>
+    __device__ static float term_shared(const Row& r, const Acts& a, int t, int lane, bool ok,
+                                        const StagePtrs& st, size_t row_units) {
+        return term_impl<STAGES, true>(r, a, t, lane, ok, st, row_units);
+    }
+    template <bool STAGES, bool SHARED>
+    __device__ static float term_impl(const Row& r, const Acts& a, int t, int lane, bool ok,
+                                      const StagePtrs& st, size_t row_units) {
         const uint32_t cw[4] = {(uint32_t)r.codes.x, (uint32_t)r.codes.y, (uint32_t)r.codes.z,
                                 (uint32_t)r.codes.w};
         int ip0 = 0, ip1 = 0;
+        if (SHARED) {
 #pragma unroll
-        for (int sft = 0; sft < 4; ++sft) {
-            ip0 = dot4((int)((cw[0] >> (2 * sft)) & 0x03030303u), a.xt[0 + sft], ip0);
-            ip0 = dot4((int)((cw[1] >> (2 * sft)) & 0x03030303u), a.xt[4 + sft], ip0);
-            ip1 = dot4((int)((cw[2] >> (2 * sft)) & 0x03030303u), a.xt[8 + sft], ip1);
-            ip1 = dot4((int)((cw[3] >> (2 * sft)) & 0x03030303u), a.xt[12 + sft], ip1);
+            for (int sft = 0; sft < 4; ++sft) {
+                ip0 = dot4((int)((cw[0] >> (2 * sft)) & 0x03030303u), a.xt[0 + sft], ip0);
+                ip0 = dot4((int)((cw[1] >> (2 * sft)) & 0x03030303u), a.xt[4 + sft], ip0);
+                ip1 = dot4((int)((cw[2] >> (2 * sft)) & 0x03030303u), a.xt[8 + sft], ip1);
+                ip1 = dot4((int)((cw[3] >> (2 * sft)) & 0x03030303u), a.xt[12 + sft], ip1);
+            }
+        } else {
+            // Code k of every byte (bits 2k, 2k+1): k = 0 and 1 are masked out of w and w >> 2 as
+            // they are; k = 2 and 3 are masked in place at bits 4-5 of the same two words, i.e.
+            // 16 x code (<= 48, still a positive int8), and their dot is divided by 16 afterwards
+            // (exact). One shift per word instead of three.
+            int lo[2] = {0, 0}, hi[2] = {0, 0};
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const uint32_t c = cw[w], c2 = c >> 2;
+                lo[w >> 1] = dot4((int)(c & 0x03030303u), a.xt[4 * w + 0], lo[w >> 1]);
+                lo[w >> 1] = dot4((int)(c2 & 0x03030303u), a.xt[4 * w + 1], lo[w >> 1]);
+                hi[w >> 1] = dot4((int)(c & 0x30303030u), a.xt[4 * w + 2], hi[w >> 1]);
+                hi[w >> 1] = dot4((int)(c2 & 0x30303030u), a.xt[4 * w + 3], hi[w >> 1]);
+            }
+            ip0 = lo[0] + (hi[0] >> 4);
+            ip1 = lo[1] + (hi[1] >> 4);
         }
         if (STAGES && ok) {
             // stage layout is per 32-element sub-block: two per unit
@@ -439,6 +490,8 @@ struct FmtQ5K {
     static constexpr bool kOrdered = true;
     static constexpr int kBlockBytes = 176, kBlockElems = 256;
     static constexpr int kWide16Steps = 2;
+    static constexpr bool kClampedLoads = false;
+    static constexpr bool kRowAhead = false;
     struct Row {
         v4i hdr, ha, hb, qa, qb;
     };
@@ -531,6 +584,10 @@ struct FmtNib32 {
     static constexpr bool kOrdered = false;
     static constexpr int kBlockBytes = 18 + (kAffine ? 2 : 0) + (kFive ? 4 : 0), kBlockElems = 32;
     static constexpr int kWide16Steps = 4;
+    static constexpr bool kClampedLoads = false;
+    // long rows load a whole row ahead where that measured faster (Q4_1 +5 %, Q5_1 +1 %; the
+    // 18-byte-block kinds and every other format are as fast or faster one step ahead)
+    static constexpr bool kRowAhead = K == Nib32::Q4_1 || K == Nib32::Q5_1;
     struct Row {
         v4i qs;
         uint32_t dm;  // f16 d in the low half, f16 m (affine formats) in the high half
@@ -650,6 +707,8 @@ struct FmtNib32Pair {
     static constexpr int kOneBlock = kFive ? 22 : 18;
     static constexpr int kBlockBytes = 2 * kOneBlock, kBlockElems = 64;
     static constexpr int kWide16Steps = 3;
+    static constexpr bool kClampedLoads = false;
+    static constexpr bool kRowAhead = false;
     struct Row {
         v4i q0, q1;
         uint32_t d01;  // f16 d of block 0 in the low half, of block 1 in the high half

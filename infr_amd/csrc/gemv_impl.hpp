@@ -158,7 +158,7 @@ __global__ __launch_bounds__(512) void gemv_batch_ks_kernel(const uint8_t* __res
             for (int mi = 0; mi < MB; ++mi) {
                 const StagePtrs sm{STAGES ? st.a + mi * st_stride : nullptr,
                                    STAGES && st.b ? st.b + mi * st_stride : nullptr};
-                const float term = F::template term<STAGES>(q0, acts[mi], wave, lane, ok && mi < m_valid, sm,
+                const float term = term_shared<F, STAGES>(q0, acts[mi], wave, lane, ok && mi < m_valid, sm,
                                                             (size_t)row * n_units);
                 if (F::kOrdered) {
                     if ((lane & 3) == 0) B[(r * MB + mi) * ls + wave * 16 + (lane >> 2)] = term;

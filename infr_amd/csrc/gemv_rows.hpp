@@ -1,6 +1,8 @@
 // The row loop shared by every decode-GEMV entry kernel (plain, fused/grouped, id-gathered).
 #pragma once
 
+#include <type_traits>
+
 #include "gemv_formats.hpp"
 
 namespace infr {
@@ -12,6 +14,26 @@ struct OrderedSum {
     static constexpr int kRowStride = 16 * STEPS + 4;
     static constexpr int kFloatsPerWave = 16 * kRowStride;
 };
+
+// The per-block term of one weight row when the same row meets several activation rows in
+// registers: the format's shared-unpack form where it has one.
+template <typename F, typename = void>
+struct HasSharedTerm : std::false_type {};
+template <typename F>
+struct HasSharedTerm<F, std::void_t<decltype(&F::template term_shared<false>)>> : std::true_type {};
+template <typename F, bool STAGES>
+__device__ __forceinline__ float term_shared(const typename F::Row& r, const typename F::Acts& a, int t, int lane,
+                                             bool ok, const StagePtrs& st, size_t row_units) {
+    if constexpr (HasSharedTerm<F>::value) return F::template term_shared<STAGES>(r, a, t, lane, ok, st, row_units);
+    else return F::template term<STAGES>(r, a, t, lane, ok, st, row_units);
+}
+
+// Step 0 of a row known to be readable, through the format's unpredicated loader where it has one.
+template <typename F>
+__device__ __forceinline__ void load_row_clamped(typename F::Row& r, const uint8_t* rowp, int lane, bool ok) {
+    if constexpr (F::kClampedLoads) F::load_row_clamped(r, rowp, 0, lane, ok);
+    else F::load_row(r, rowp, 0, lane, ok);
+}
 
 // Rows [row0, row_end) of one weight matrix against activation registers `acts`. `first` already
 // holds step 0 of row0 (the caller issues those loads as early as it can). The loads run one wave
@@ -34,26 +56,15 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
                                           float* add_dst = nullptr) {
     constexpr int LS = OrderedSum<STEPS>::kRowStride;
     int in_batch = 0, batch_row0 = row0;
-    // One row: `cur0` holds its step 0; the loads of step t + 1 are issued before step t is
-    // computed, and the last step's prefetch - step 0 of the next row - lands in `next0`.
-    auto do_row = [&](int row, const typename F::Row& cur0, typename F::Row& next0) {
-        const uint8_t* rowp = w + (size_t)row * bpr;
-        float s = 0.0f;
-        typename F::Row cur = cur0;
-#pragma unroll
-        for (int t = 0; t < STEPS; ++t) {
-            typename F::Row nxt;
-            if (t + 1 < STEPS) F::load_row(nxt, rowp, t + 1, lane, ok[t + 1 < STEPS ? t + 1 : 0]);
-            else F::load_row(next0, rowp + bpr, 0, lane, ok[0] && row + 1 < row_end);
-            const float term = F::template term<STAGES>(cur, acts[t], t, lane, ok[t], st,
-                                                        (size_t)row * n_units);
-            if (F::kOrdered) {
-                if ((lane & 3) == 0) osum[in_batch * LS + t * 16 + (lane >> 2)] = term;
-            } else {
-                s += term;
-            }
-            if (t + 1 < STEPS) cur = nxt;
+    // A row's step-t term: parked for the ordered sum, or added to the lane's partial sum.
+    auto take_term = [&](int t, float term, float& s) {
+        if (F::kOrdered) {
+            if ((lane & 3) == 0) osum[in_batch * LS + t * 16 + (lane >> 2)] = term;
+        } else {
+            s += term;
         }
+    };
+    auto finish_row = [&](int row, float s) {
         if (F::kOrdered) {
             if (++in_batch == 16 || row + 1 == row_end) {
                 if (lane < in_batch) {
@@ -81,6 +92,51 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
                 if (add_dst) gstore<float>(add_dst + row, s + gload<float>(add_b + row));
             }
         }
+    };
+    if constexpr (STEPS > 1 && F::kRowAhead) {
+        // Long rows run in eight-wave workgroups, where one step ahead is too few bytes in flight:
+        // the loads run a whole row ahead - step t of the next row is requested before step t of
+        // this one is computed.
+        if (row0 >= row_end) return;
+        typename F::Row cur[STEPS];
+        cur[0] = first;
+#pragma unroll
+        for (int t = 1; t < STEPS; ++t) F::load_row(cur[t], w + (size_t)row0 * bpr, t, lane, ok[t]);
+        for (int row = row0; row < row_end; ++row) {
+            const uint8_t* rowp = w + (size_t)row * bpr;
+            const bool more = row + 1 < row_end;
+            typename F::Row nxt[STEPS];
+            float s = 0.0f;
+#pragma unroll
+            for (int t = 0; t < STEPS; ++t) {
+                // unpredicated where the format can: the wave's last row requests itself again
+                if constexpr (F::kClampedLoads) F::load_row_clamped(nxt[t], more ? rowp + bpr : rowp, t, lane, ok[t]);
+                else F::load_row(nxt[t], rowp + bpr, t, lane, ok[t] && more);
+                take_term(t, F::template term<STAGES>(cur[t], acts[t], t, lane, ok[t], st, (size_t)row * n_units), s);
+            }
+            finish_row(row, s);
+#pragma unroll
+            for (int t = 0; t < STEPS; ++t) cur[t] = nxt[t];
+        }
+        return;
+    }
+    // One row: `cur0` holds its step 0; the loads of step t + 1 are issued before step t is
+    // computed, and the last step's prefetch - step 0 of the next row - lands in `next0`.
+    auto do_row = [&](int row, const typename F::Row& cur0, typename F::Row& next0) {
+        const uint8_t* rowp = w + (size_t)row * bpr;
+        float s = 0.0f;
+        typename F::Row cur = cur0;
+#pragma unroll
+        for (int t = 0; t < STEPS; ++t) {
+            typename F::Row nxt;
+            if (t + 1 < STEPS) F::load_row(nxt, rowp, t + 1, lane, ok[t + 1 < STEPS ? t + 1 : 0]);
+            else if (F::kClampedLoads)  // the wave's last row prefetches itself again: no predicate
+                load_row_clamped<F>(next0, row + 1 < row_end ? rowp + bpr : rowp, lane, ok[0]);
+            else F::load_row(next0, rowp + bpr, 0, lane, ok[0] && row + 1 < row_end);
+            take_term(t, F::template term<STAGES>(cur, acts[t], t, lane, ok[t], st, (size_t)row * n_units), s);
+            if (t + 1 < STEPS) cur = nxt;
+        }
+        finish_row(row, s);
     };
     typename F::Row cur = first;
     for (int row = row0; row < row_end; ++row) {
@@ -171,7 +227,7 @@ __device__ __forceinline__ void gemv_rows_batch(const uint8_t* __restrict__ w, s
             for (int mi = 0; mi < MB; ++mi) {
                 const StagePtrs sm{STAGES ? st.a + mi * st_stride : nullptr,
                                    STAGES && st.b ? st.b + mi * st_stride : nullptr};
-                const float term = F::template term<STAGES>(cur, acts[mi][t], t, lane,
+                const float term = term_shared<F, STAGES>(cur, acts[mi][t], t, lane,
                                                             ok[t] && mi < m_valid, sm,
                                                             (size_t)row * n_units);
                 if (F::kOrdered) {
