@@ -381,7 +381,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="headline sweep only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--sections", default="shapes,formats,mmq,chain,layer,ternary,moe,load",
-                    help="comma list of secondary sections: shapes, formats, mmq, chain, layer, ternary, moe, load")
+                    help="comma list of secondary sections: shapes, formats, mmq, chain, layer, ternary, moe, load; mmq_scaling (off by default)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
@@ -453,6 +453,13 @@ def main():
             t, nb = single_shape(be, DType.Q4K, M, 4096, 12288, reps=10)
             extra[f"mmq_Q4_K_M{M}_TOPS"] = round(2.0 * M * 12288 * 4096 / (t * 1e-3) / 1e12, 2)
             extra[f"mmq_Q4_K_M{M}_pct_int8_peak"] = round(100 * extra[f"mmq_Q4_K_M{M}_TOPS"] / INT8_PEAK_TOPS, 2)
+    if "mmq_scaling" in sections:
+        # the same prefill kernel on grids of 64 .. 4096 workgroups (32 rows x 128 tokens each,
+        # M = 512, K = 16384): TOPS per resident workgroup falls as the device fills, which with
+        # the clock counters of a profiler run separates per-workgroup latency from the power limit
+        for out_f in (512, 2048, 8192, 32768):
+            t, nb = single_shape(be, DType.Q4K, 512, 16384, out_f, reps=6, rotate_bytes=1)
+            extra[f"mmq_Q4_K_M512_K16384_N{out_f}_TOPS"] = round(2.0 * 512 * out_f * 16384 / (t * 1e-3) / 1e12, 2)
     if "chain" in sections:
         ch = Sweep(be, DType.Q4K, 1, args.layers, chain=True)
         d, w = ch.time(10, 2)
