@@ -4,6 +4,8 @@
 // CPU code calls mul_add (then __builtin_fmaf is written out here).
 #pragma once
 
+#include <type_traits>
+
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -115,6 +117,51 @@ __device__ __forceinline__ float wave_sum_f(float v) {
     s += readlane_f(v, 48);
     return s;
 }
+// MB per-lane values -> one: lane L returns the sum over its row of 16 lanes of value number
+// L % MB. Each transposing stage halves the values a lane carries (it keeps the half its own lane
+// bit selects and hands the other half to the partner lane), so reducing MB values costs about
+// 3 * (MB - 1) instructions plus the rotations, instead of MB whole-wave reductions. MB in {2, 4, 8}.
+template <int MB>
+__device__ __forceinline__ float row16_transpose_sum(const float (&v)[MB], int lane) {
+    static_assert(MB == 2 || MB == 4 || MB == 8, "2, 4 or 8 values");
+    auto dpp = [](float x, auto ctrl) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), decltype(ctrl)::value,
+                                                                  0xF, 0xF, true));
+    };
+    using QuadXor1 = std::integral_constant<int, 0xB1>;    // quad_perm [1,0,3,2]
+    using QuadXor2 = std::integral_constant<int, 0x4E>;    // quad_perm [2,3,0,1]
+    using HalfMirror = std::integral_constant<int, 0x141>; // lane i <-> 7 - i of each 8
+    using Ror4 = std::integral_constant<int, 0x124>;       // rotate right by 4 within the row of 16
+    using Ror8 = std::integral_constant<int, 0x128>;
+    float a[4];
+    if constexpr (MB == 8) {
+        // partner L ^ 7 sits in the other half of the 8: lanes with bit 2 keep values 4..7
+        const bool up = (lane & 4) != 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) a[j] = (up ? v[4 + j] : v[j]) + dpp(up ? v[j] : v[4 + j], HalfMirror{});
+    } else {
+#pragma unroll
+        for (int j = 0; j < MB; ++j) a[j] = v[j];
+    }
+    float b[2];
+    if constexpr (MB >= 4) {
+        const bool odd = (lane & 1) != 0;  // partner L ^ 1: odd lanes keep the odd values
+#pragma unroll
+        for (int j = 0; j < 2; ++j) b[j] = (odd ? a[2 * j + 1] : a[2 * j]) + dpp(odd ? a[2 * j] : a[2 * j + 1], QuadXor1{});
+        const bool hi = (lane & 2) != 0;   // partner L ^ 2: lanes with bit 1 keep value pair 1
+        float r = (hi ? b[1] : b[0]) + dpp(hi ? b[0] : b[1], QuadXor2{});
+        // lane L: value (L % MB) summed over its 8 (MB == 8) or 4 (MB == 4) lanes
+        if constexpr (MB == 4) r += dpp(r, Ror4{});
+        return r + dpp(r, Ror8{});
+    } else {
+        const bool odd = (lane & 1) != 0;
+        float r = (odd ? a[1] : a[0]) + dpp(odd ? a[0] : a[1], QuadXor1{});
+        r += dpp(r, QuadXor2{});
+        r += dpp(r, Ror4{});
+        return r + dpp(r, Ror8{});
+    }
+}
+
 __device__ __forceinline__ int wave_sum_i(int v) {
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);

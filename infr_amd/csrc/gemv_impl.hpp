@@ -90,7 +90,7 @@ __global__ __launch_bounds__(256) void gemv_batch_kernel(const uint8_t* __restri
 // owns wave step w of every row of the workgroup's tile, so the activations of all MB tokens for
 // that step fit its registers and the weights stream ONCE for the whole batch (the one-wave form
 // above has to re-stream them once per 8 / STEPS tokens). Per row every wave leaves its share in
-// LDS - for the ordered formats the per-block terms themselves, otherwise its lanes' sum - and after
+// LDS - for the ordered formats the per-block terms themselves, otherwise four partial sums - and after
 // each group of rows the workgroup's threads finish one (row, token) output each: the terms in
 // ascending block order, i.e. the CPU's `sumf +=` chain (bit-identical for Q4_K / Q5_K / Q6_K), or
 // the waves' sums in wave order. Two LDS buffers alternate, so one barrier per group suffices.
@@ -98,7 +98,8 @@ __global__ __launch_bounds__(256) void gemv_batch_kernel(const uint8_t* __restri
 template <int MB>
 struct BatchKs {
     static constexpr int kRowsPerFlush = 64 / MB;  // 64 (row, token) outputs per flush
-    __host__ __device__ static constexpr int row_stride(bool ordered, int nw) { return ordered ? nw * 16 + 4 : nw; }
+    // floats per (row, token): the waves' per-block terms (ordered) or their four row-of-16 sums
+    __host__ __device__ static constexpr int row_stride(bool ordered, int nw) { return ordered ? nw * 16 + 4 : nw * 4; }
     __host__ __device__ static constexpr size_t lds_bytes(bool ordered, int nw) {
         return (size_t)2 * 64 * row_stride(ordered, nw) * sizeof(float);
     }
@@ -154,17 +155,29 @@ __global__ __launch_bounds__(512) void gemv_batch_ks_kernel(const uint8_t* __res
             const int row = batch0 + r;
             typename F::Row q2;
             F::load_row(q2, w + (size_t)(row + 2) * bpr, wave, lane, ok && row + 2 < row_end);
+            float terms[MB];
 #pragma unroll
             for (int mi = 0; mi < MB; ++mi) {
                 const StagePtrs sm{STAGES ? st.a + mi * st_stride : nullptr,
                                    STAGES && st.b ? st.b + mi * st_stride : nullptr};
-                const float term = term_shared<F, STAGES>(q0, acts[mi], wave, lane, ok && mi < m_valid, sm,
-                                                            (size_t)row * n_units);
+                terms[mi] = term_shared<F, STAGES>(q0, acts[mi], wave, lane, ok && mi < m_valid, sm,
+                                                   (size_t)row * n_units);
                 if (F::kOrdered) {
-                    if ((lane & 3) == 0) B[(r * MB + mi) * ls + wave * 16 + (lane >> 2)] = term;
+                    if ((lane & 3) == 0) B[(r * MB + mi) * ls + wave * 16 + (lane >> 2)] = terms[mi];
+                }
+            }
+            if (!F::kOrdered) {
+                // all MB tokens' lane terms reduced together: lane L ends with token L % MB summed
+                // over its row of 16 lanes, and the first MB lanes of each row park that
+                if constexpr (MB == 2 || MB == 4 || MB == 8) {
+                    const float part = row16_transpose_sum<MB>(terms, lane);
+                    if ((lane & 15) < MB) B[(r * MB + (lane & (MB - 1))) * ls + wave * 4 + (lane >> 4)] = part;
                 } else {
-                    const float tot = wave_sum_f(term);
-                    if (lane == 0) B[(r * MB + mi) * ls + wave] = tot;
+#pragma unroll
+                    for (int mi = 0; mi < MB; ++mi) {
+                        const float tot = wave_sum_f(terms[mi]);
+                        if (lane < 4) B[(r * MB + mi) * ls + wave * 4 + lane] = lane == 0 ? tot : 0.0f;
+                    }
                 }
             }
             q0 = q1;
@@ -183,7 +196,7 @@ __global__ __launch_bounds__(512) void gemv_batch_ks_kernel(const uint8_t* __res
                     acc += v.w;
                 }
             } else {
-                for (int k = 0; k < nw; ++k) acc += tr[k];
+                for (int k = 0; k < 4 * nw; ++k) acc += tr[k];
             }
             const int mi = task % MB;
             if (mi < m_valid) gstore<float>(y + (size_t)mi * out_f + batch0 + task / MB, acc);

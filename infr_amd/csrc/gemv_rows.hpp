@@ -259,9 +259,19 @@ __device__ __forceinline__ void gemv_rows_batch(const uint8_t* __restrict__ w, s
             }
         } else {
 #pragma unroll
-            for (int mi = 0; mi < MB; ++mi) {
-                const float tot = wave_sum_f(s[mi]);
-                if (lane == 0 && mi < m_valid) gstore<float>(y + (size_t)mi * y_stride + row, tot);
+            if constexpr (MB == 2 || MB == 4 || MB == 8) {
+                // the MB tokens' lane sums reduced together: lane L carries token L % MB summed over
+                // its row of 16 lanes; two cross-row exchanges finish it
+                float part = row16_transpose_sum<MB>(s, lane);
+                part += __shfl_xor(part, 16, kWave);
+                part += __shfl_xor(part, 32, kWave);
+                if (lane < MB && lane < m_valid) gstore<float>(y + (size_t)lane * y_stride + row, part);
+            } else {
+#pragma unroll
+                for (int mi = 0; mi < MB; ++mi) {
+                    const float tot = wave_sum_f(s[mi]);
+                    if (lane == 0 && mi < m_valid) gstore<float>(y + (size_t)mi * y_stride + row, tot);
+                }
             }
         }
     }
