@@ -18,6 +18,10 @@
 //                         of this one is computed (a whole row in flight) instead of one step ahead
 //   kClampedLoads         has load_row_clamped: for a row known to be readable, lanes without
 //                         work read block 0 instead of being masked off
+//   kLaneSums             butterfly formats: the lanes' row sums of eight rows are parked in LDS and
+//                         reduced together instead of one whole-wave reduction per row (Q4_0
+//                         +14 % at 4096 x 4096, IQ4_NL +6 % at 4096 x 12288, Q8_0 +1-2 %; Q2_0
+//                         measured 12-17 % slower that way and keeps the per-row reduction)
 //   units(in_f)           number of lane work units in a row (blocks for Q4_K/Q6_K ...)
 //   Row / Acts            registers for one step of a weight row / of the activation
 //   valid(t, lane, n)     does this lane have work in step t
@@ -55,6 +59,7 @@ struct FmtQ4K {
     static constexpr int kBlockBytes = 144, kBlockElems = 256;
     static constexpr int kWide16Steps = 3;
     static constexpr bool kClampedLoads = false;
+    static constexpr bool kLaneSums = true;
     static constexpr bool kRowAhead = false;
     struct Row {
         v4i hdr, qa, qb;
@@ -147,6 +152,7 @@ struct FmtQ6K {
     static constexpr int kBlockBytes = 210, kBlockElems = 256;
     static constexpr int kWide16Steps = 1;
     static constexpr bool kClampedLoads = false;
+    static constexpr bool kLaneSums = true;
     static constexpr bool kRowAhead = false;
     struct Row {
         v4i qla, qlb, qh;
@@ -245,6 +251,7 @@ struct FmtQ8_0T {
     static constexpr int kBlockBytes = 34, kBlockElems = 32;
     static constexpr int kWide16Steps = 4;
     static constexpr bool kClampedLoads = false;
+    static constexpr bool kLaneSums = true;
     static constexpr bool kRowAhead = false;
     struct Row {
         v4i qa, qb;
@@ -358,6 +365,7 @@ struct FmtQ2_0T {
     static constexpr int kBlockBytes = 18, kBlockElems = 64;
     static constexpr int kWide16Steps = 3;
     static constexpr bool kClampedLoads = true;
+    static constexpr bool kLaneSums = false;
     static constexpr bool kRowAhead = true;
     struct Row {
         v4i codes;
@@ -491,6 +499,7 @@ struct FmtQ5K {
     static constexpr int kBlockBytes = 176, kBlockElems = 256;
     static constexpr int kWide16Steps = 2;
     static constexpr bool kClampedLoads = false;
+    static constexpr bool kLaneSums = true;
     static constexpr bool kRowAhead = false;
     struct Row {
         v4i hdr, ha, hb, qa, qb;
@@ -585,6 +594,7 @@ struct FmtNib32 {
     static constexpr int kBlockBytes = 18 + (kAffine ? 2 : 0) + (kFive ? 4 : 0), kBlockElems = 32;
     static constexpr int kWide16Steps = 4;
     static constexpr bool kClampedLoads = false;
+    static constexpr bool kLaneSums = true;
     // long rows load a whole row ahead where that measured faster (Q4_1 +5 %, Q5_1 +1 %; the
     // 18-byte-block kinds and every other format are as fast or faster one step ahead)
     static constexpr bool kRowAhead = K == Nib32::Q4_1 || K == Nib32::Q5_1;
@@ -708,6 +718,7 @@ struct FmtNib32Pair {
     static constexpr int kBlockBytes = 2 * kOneBlock, kBlockElems = 64;
     static constexpr int kWide16Steps = 3;
     static constexpr bool kClampedLoads = false;
+    static constexpr bool kLaneSums = true;
     static constexpr bool kRowAhead = false;
     struct Row {
         v4i q0, q1;

@@ -30,9 +30,9 @@ __global__ __launch_bounds__(256) void gemv_kernel(const uint8_t* __restrict__ w
     F::load_row(first, w + (size_t)row0 * bpr, 0, lane, ok[0]);
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) F::load_acts(acts[t], act, t, lane, ok[t]);
-    __shared__ __attribute__((aligned(16))) float osum[F::kOrdered ? 4 * OrderedSum<STEPS>::kFloatsPerWave : 4];
+    __shared__ __attribute__((aligned(16))) float osum[4 * RowSumScratch<F, STEPS>::kFloatsPerWave];
     gemv_rows<F, STEPS, STAGES>(w, bpr, first, acts, ok, y, n_units, row0, row_end, lane, st,
-                                osum + (threadIdx.x >> 6) * (F::kOrdered ? OrderedSum<STEPS>::kFloatsPerWave : 0));
+                                osum + (threadIdx.x >> 6) * RowSumScratch<F, STEPS>::kFloatsPerWave);
 }
 
 // Small batch (2..8 activation rows already quantized in device memory): weights stream once.
@@ -340,7 +340,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, 
     typename F::Acts acts[STEPS];
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) F::load_acts(acts[t], act, t, lane, ok[t]);
-    float* osum = reinterpret_cast<float*>(lds + in_f + in_f / 2) + wave * OrderedSum<STEPS>::kFloatsPerWave;
+    float* osum = reinterpret_cast<float*>(lds + in_f + in_f / 2) + wave * RowSumScratch<F, STEPS>::kFloatsPerWave;
     gemv_rows<F, STEPS, false>(tile.w, tile.bpr, first, acts, ok, tile.y, n_units, row0, row_end, lane,
                                StagePtrs{nullptr, nullptr}, osum, tile.fus.add_b, tile.fus.add_dst);
 }
@@ -555,7 +555,9 @@ static bool plan_group_fmt(size_t in_f, const GemvOpDesc* ops, int n, GemvGroupP
     if ((env_nw == 4 || env_nw == 8 || env_nw == 16) && env_nw <= nw) nw = env_nw;
     size_t rows_per_wg = (total_rows + 511) / 512;
     rows_per_wg = rows_per_wg < 4 ? 4 : (rows_per_wg > 128 ? 128 : rows_per_wg);
-    const size_t lds_bytes = in_f + in_f / 2 + (F::kOrdered ? (size_t)nw * (16 * (16 * steps + 4)) * sizeof(float) : 0);
+    // activations, then every wave's row-sum scratch (OrderedSum<steps> or LaneSums)
+    const size_t lds_bytes = in_f + in_f / 2 +
+                             (size_t)nw * (F::kOrdered ? 16 * (16 * steps + 4) : (F::kLaneSums ? LaneSums::kFloatsPerWave : 0)) * sizeof(float);
     // Grids of only a few rounds: a grid that needs a little more than a whole number of rounds
     // idles most of the machine during the last one, and workgroups that share a compute unit
     // share its pipes, so what counts is workgroups per compute unit. For those grids take, among

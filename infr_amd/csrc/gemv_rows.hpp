@@ -28,6 +28,19 @@ __device__ __forceinline__ float term_shared(const typename F::Row& r, const typ
     else return F::template term<STAGES>(r, a, t, lane, ok, st, row_units);
 }
 
+// Per-wave LDS scratch of the butterfly formats: the lanes' sums of 8 rows, 64 + 4 pad floats per row
+// (the pad spreads the flush's 16-byte reads over the banks).
+struct LaneSums {
+    static constexpr int kRows = 8, kRowStride = 68;
+    static constexpr int kFloatsPerWave = kRows * kRowStride;
+};
+// What gemv_rows needs per wave, by format.
+template <typename F, int STEPS>
+struct RowSumScratch {
+    static constexpr int kFloatsPerWave =
+        F::kOrdered ? OrderedSum<STEPS>::kFloatsPerWave : (F::kLaneSums ? LaneSums::kFloatsPerWave : 1);
+};
+
 // Step 0 of a row known to be readable, through the format's unpredicated loader where it has one.
 template <typename F>
 __device__ __forceinline__ void load_row_clamped(typename F::Row& r, const uint8_t* rowp, int lane, bool ok) {
@@ -85,11 +98,30 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
                 batch_row0 = row + 1;
                 in_batch = 0;
             }
-        } else {
+        } else if (!F::kLaneSums) {
             s = wave_sum_f(s);
             if (lane == 0) {
                 gstore<float>(y + row, s);
                 if (add_dst) gstore<float>(add_dst + row, s + gload<float>(add_b + row));
+            }
+        } else {
+            // The lanes' sums of up to eight rows are parked in LDS and reduced together: lane L
+            // adds eighth L / 8 of row L % 8, then the eighths meet over lanes L ^ 8, ^ 16, ^ 32 -
+            // about two instructions per row where a whole-wave reduction per row costs twelve.
+            osum[in_batch * LaneSums::kRowStride + lane] = s;
+            if (++in_batch == LaneSums::kRows || row + 1 == row_end) {
+                const v4f* tr = reinterpret_cast<const v4f*>(osum + (lane & 7) * LaneSums::kRowStride + (lane >> 3) * 8);
+                const v4f a = tr[0], b = tr[1];
+                float acc = ((a.x + a.y) + (a.z + a.w)) + ((b.x + b.y) + (b.z + b.w));
+                acc += __shfl_xor(acc, 8, kWave);
+                acc += __shfl_xor(acc, 16, kWave);
+                acc += __shfl_xor(acc, 32, kWave);
+                if (lane < in_batch) {
+                    gstore<float>(y + batch_row0 + lane, acc);
+                    if (add_dst) gstore<float>(add_dst + batch_row0 + lane, acc + gload<float>(add_b + batch_row0 + lane));
+                }
+                batch_row0 = row + 1;
+                in_batch = 0;
             }
         }
     };
@@ -258,7 +290,6 @@ __device__ __forceinline__ void gemv_rows_batch(const uint8_t* __restrict__ w, s
                 in_batch = 0;
             }
         } else {
-#pragma unroll
             if constexpr (MB == 2 || MB == 4 || MB == 8) {
                 // the MB tokens' lane sums reduced together: lane L carries token L % MB summed over
                 // its row of 16 lanes; two cross-row exchanges finish it

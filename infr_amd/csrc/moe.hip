@@ -673,10 +673,10 @@ __global__ __launch_bounds__(256) void gemv_id_kernel(const uint8_t* __restrict_
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) F::load_acts(acts[t], a, t, lane, ok[t]);
     // same body as the decode GEMV: per-block exact integers, CPU-ordered f32 sum
-    __shared__ __attribute__((aligned(16))) float osum[F::kOrdered ? 4 * OrderedSum<STEPS>::kFloatsPerWave : 4];
+    __shared__ __attribute__((aligned(16))) float osum[4 * RowSumScratch<F, STEPS>::kFloatsPerWave];
     gemv_rows<F, STEPS, false>(w, bpr, first, acts, ok, y + (size_t)pair * out_f, n_units, row0, row_end,
                                lane, StagePtrs{nullptr, nullptr},
-                               osum + (threadIdx.x >> 6) * (F::kOrdered ? OrderedSum<STEPS>::kFloatsPerWave : 0));
+                               osum + (threadIdx.x >> 6) * RowSumScratch<F, STEPS>::kFloatsPerWave);
 }
 
 // The same for short rows (in_f <= 2048) of Q4_K / Q6_K banks: 16 / nb rows per wave step.
