@@ -165,3 +165,25 @@ def test_ragged_rows_are_refused(be):
         with pytest.raises(InfrError) as e:
             be.linear(dt, w, x, y, 1, in_f, 2, w_numel=2 * in_f)
         assert e.value.status == Status.Unsupported
+
+
+def test_rows_beyond_eight_wave_steps_are_refused_not_truncated(be):
+    """in_f above the formats' bound (32768; 16384 for Q8_0 / Q4_1 / Q5_1) is Unsupported, and the
+    bound itself still computes."""
+    for dt, in_f in ((DType.Q8_0, 16384 + 32), (DType.Q4_1, 16384 + 32), (DType.Q5K, 32768 + 256)):
+        w = be.alloc(block_bytes(dt, in_f) * 2)
+        x = be.alloc(in_f * 4)
+        y = be.alloc(8)
+        with pytest.raises(InfrError) as e:
+            be.linear(dt, w, x, y, 1, in_f, 2)
+        assert e.value.status == Status.Unsupported
+    in_f, out_f = 16384, 24
+    w = synth_weight(DType.Q8_0, 77, out_f, in_f)
+    x = synth_normal_f32(78, in_f)
+    gate(run_linear(be, DType.Q8_0, w, x, 1, in_f, out_f), orc.linear(DType.Q8_0, w, x, 1, in_f, out_f))
+
+
+def block_bytes(dt, in_f):
+    from infr_amd import block_layout
+    e, b = block_layout(dt)
+    return in_f // e * b
