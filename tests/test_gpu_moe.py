@@ -88,7 +88,7 @@ def test_moe_int8_path_other_bank_formats(be, dtype):
     check(*got, *want)
 
 
-@pytest.mark.parametrize("rows", [1, 6])
+@pytest.mark.parametrize("rows", [1, 6, 72])     # 72: the expert-bucketed prefill path, captured and replayed
 def test_moe_in_a_plan_replays(be, rows):
     """Two Op::MoeFfn separated by a Linear in one compiled plan (the second routes the first's
     output), executed three times with fresh inputs: every replay must match the oracle chain."""
