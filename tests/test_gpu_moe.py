@@ -218,3 +218,24 @@ def test_moe_qwen3_30b_a3b_prefill(be):
     want = orc.moe_ffn(xs, router, gate, up, down, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff, scale=1.0)
     check(y[pick], idx[pick], w[pick], *want)
     assert np.isfinite(y).all() and len(np.unique(idx)) > 100        # most experts are touched
+
+
+@pytest.mark.parametrize("gu,down", [(DType.Q4K, DType.Q6K), (DType.Q6K, DType.Q4K)])
+def test_moe_prefill_buckets_with_mixed_bank_formats(be, gu, down):
+    """A Q4_K_M file's mix (Q4_K gate / up beside a Q6_K down bank) and its mirror: the Q4_K banks
+    take the bucketed MFMA GEMM, the others the per-pair GEMVs, in one op."""
+    rows, ne, n_expert, n_used, nff = 96, 512, 16, 4, 256
+    gate_w = synth_weight(gu, 201, n_expert * nff, ne, 0.05)
+    up_w = synth_weight(gu, 202, n_expert * nff, ne, 0.05)
+    down_w = synth_weight(down, 203, n_expert * ne, nff, 0.05)
+    x = synth_normal_f32(204, rows * ne)
+    router = synth_normal_f32(205, n_expert * ne, sigma=0.05)
+    yb, ib, wb = be.alloc(rows * ne * 4), be.alloc(rows * n_used * 4), be.alloc(rows * n_used * 4)
+    be.moe_ffn(be.upload_new(x), be.upload_new(router), be.upload_new(gate_w), be.upload_new(up_w),
+               be.upload_new(down_w), yb, rows=rows, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
+               scale=1.0, gate_dtype=gu, up_dtype=gu, down_dtype=down, sel_idx=ib, sel_w=wb)
+    got = (be.download(yb, np.empty((rows, ne), np.float32)), be.download(ib, np.empty((rows, n_used), np.int32)),
+           be.download(wb, np.empty((rows, n_used), np.float32)))
+    want = orc.moe_ffn(x, router, gate_w, up_w, down_w, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
+                       scale=1.0, gate_dtype=int(gu), up_dtype=int(gu), down_dtype=int(down))
+    check(*got, *want)
