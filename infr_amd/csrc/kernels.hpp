@@ -227,6 +227,10 @@ struct MoeBuffers {
     int32_t* sel_idx;       // optional [rows, n_used]
     float* sel_w;           // optional [rows, n_used]
 };
+// Q6_K prefill GEMM on the int8 matrix cores (any m; used from 33 tokens): activations in the tiled quantizer's layout
+// (launch_quantize_q8_tiled); st.a, when set, receives isum per (token, row, 256-block).
+void launch_mmq_shared_q6k(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
+                           size_t out_f, const IntStages& st, hipStream_t stream);
 // Routed pairs bucketed by expert, in tiles of at most 32 pairs of one expert each (device arrays;
 // `*n_tiles` of the `max_tiles` entries exist). `perm` lists the pairs expert by expert.
 struct MoeTileTable {

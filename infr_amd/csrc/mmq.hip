@@ -753,8 +753,9 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
     //   2..32      skinny kernel, K split over the waves of a workgroup
     //   33..127    tiled kernel, 32 tokens x 128 rows per workgroup (most workgroups for few tokens)
     //   128..      shared-operand kernel, 128 tokens x 32 rows (x 64 rows from 1024 tokens up)
-    // The other formats take the dot4 GEMV with the activations of up to eight rows in registers
-    // (weights re-streamed once per eight rows beyond that).
+    // Q6_K from 33 tokens: its own shared-operand MFMA kernel (mmq_q6k.hip). Otherwise the other
+    // formats take the dot4 GEMV with the activations of up to eight rows in registers (weights
+    // re-streamed once per eight rows beyond that).
     static const int env_skinny_max = getenv("INFR_HIP_MMQ_SKINNY_MAX_M") ? atoi(getenv("INFR_HIP_MMQ_SKINNY_MAX_M")) : 32;
     static const int env_shared_min = getenv("INFR_HIP_MMQ_SHARED_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_SHARED_MIN_M")) : 128;
     static const int env_shared_rows = getenv("INFR_HIP_MMQ_SHARED_ROWS") ? atoi(getenv("INFR_HIP_MMQ_SHARED_ROWS")) : 0;
@@ -763,6 +764,15 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
         const bool wide = env_shared_rows ? env_shared_rows == 64 : m >= 1024;
         if (wide) launch_mmq_shared_q4k<2>(w, bpr, act, y, m, in_f, out_f, st, stream);
         else launch_mmq_shared_q4k<1>(w, bpr, act, y, m, in_f, out_f, st, stream);
+        return true;
+    }
+    // Q6_K: the MFMA kernel's time is flat up to 128 tokens (63 / 103 / 39 us at 12288 x 4096,
+    // 4096 x 12288, 1024 x 4096) and the dot4 batches cost ~3.5 / 3.2 / 1.1 us per token there, so
+    // it takes over from 33 tokens
+    static const int env_q6k_min = getenv("INFR_HIP_MMQ_Q6K_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_Q6K_MIN_M")) : 33;
+    if (dtype == 14 && (int)m >= env_q6k_min) {
+        launch_quantize_q8_tiled(x, m, in_f, act, stream);
+        launch_mmq_shared_q6k(w, bpr, act, y, m, in_f, out_f, st, stream);
         return true;
     }
     launch_quantize_q8(x, m, in_f, act_is_per32(dtype, in_f), act, stream);

@@ -147,6 +147,55 @@ def test_prefill_other_formats_vs_oracle(be, dtype):
     gate(y, orc.linear(dtype, w, x, m, in_f, out_f))
 
 
+# ───────────── prefill of Q6_K from 33 tokens: its own int8 MFMA kernel ─────────────
+
+@pytest.mark.parametrize("m,in_f,out_f", [(33, 512, 40), (128, 256, 32), (130, 768, 130), (257, 2048, 384),
+                                         (600, 1024, 100)])
+def test_prefill_q6k_mfma_is_bit_identical_to_oracle(be, m, in_f, out_f):
+    w = synth_weight(DType.Q6K, 310 + m, out_f, in_f)
+    x = synth_normal_f32(410 + m, m * in_f)
+    x[:in_f] *= 37.0
+    x[2 * in_f:3 * in_f] = 0.0
+    y = run_linear(be, DType.Q6K, w, x, m, in_f, out_f)
+    want = orc.linear(DType.Q6K, w, x, m, in_f, out_f)
+    gate(y, want)
+    assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), "not bit-identical"
+
+
+def test_prefill_q6k_mfma_int_stage_bit_exact(be):
+    # full-range payload: every 6-bit code, every int8 group scale (-128 included), saturated rows
+    m, in_f, out_f = 140, 768, 70
+    w = orc.synth_weight(DType.Q6K, in_f * out_f, 0x20A)
+    x = synth_normal_f32(78, m * in_f) * np.float32(3.0)
+    x[in_f:2 * in_f] = 1e4
+    x[2 * in_f:3 * in_f] = -1e4
+    a, _ = be.linear_int_stages(DType.Q6K, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
+    oa, _ = orc.linear_int_stages(DType.Q6K, w, x, m, in_f, out_f)
+    assert np.array_equal(a, oa)
+
+
+def test_full_size_prefill_q6k(be):
+    """4096 x 12288 (a Q4_K_M file's ffn_down) at 512 tokens: sampled rows bit-identical to the oracle
+    and to each token's own one-token result."""
+    m, in_f, out_f = 512, 12288, 4096
+    w = synth_weight(DType.Q6K, 930, out_f, in_f)
+    x = synth_normal_f32(931, m * in_f)
+    wb = be.upload_new(w)
+    yb = be.alloc(m * out_f * 4)
+    be.linear(DType.Q6K, wb, be.upload_new(x), yb, m, in_f, out_f)
+    y = be.download(yb, np.empty((m, out_f), np.float32))
+    toks = [0, 1, 255, 511]
+    xs = x[np.concatenate([np.arange(t * in_f, (t + 1) * in_f) for t in toks])]
+    for row0 in (0, 2000, out_f - 32):
+        want = _oracle_rows(DType.Q6K, w, xs, len(toks), in_f, out_f, row0, 32)
+        assert np.array_equal(y[toks, row0:row0 + 32].view(np.uint32), want.view(np.uint32)), "not bit-identical"
+    y1 = be.alloc(out_f * 4)
+    for t in toks[:2]:
+        be.linear(DType.Q6K, wb, be.upload_new(x[t * in_f:(t + 1) * in_f]), y1, 1, in_f, out_f)
+        single = be.download(y1, np.empty((1, out_f), np.float32))
+        assert np.array_equal(single[0].view(np.uint32), y[t].view(np.uint32)), "batch != single"
+
+
 # ───────────── hand-derived known answers (tests/golden/known_answers.json), no oracle involved ─────────────
 
 def _golden():
