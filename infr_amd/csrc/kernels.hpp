@@ -231,6 +231,12 @@ struct MoeBuffers {
 // (launch_quantize_q8_tiled); st.a, when set, receives isum per (token, row, 256-block).
 void launch_mmq_shared_q6k(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
                            size_t out_f, const IntStages& st, hipStream_t stream);
+// The same for Q8_0 rows that are whole 256s; st.a receives iprod per (token, row, 32-block).
+void launch_mmq_shared_q8_0(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
+                            size_t out_f, const IntStages& st, hipStream_t stream);
+// The same for Q5_K; st.a / st.b receive sd / sm per (token, row, 256-block).
+void launch_mmq_shared_q5k(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
+                           size_t out_f, const IntStages& st, hipStream_t stream);
 // Routed pairs bucketed by expert, in tiles of at most 32 pairs of one expert each (device arrays;
 // `*n_tiles` of the `max_tiles` entries exist). `perm` lists the pairs expert by expert.
 struct MoeTileTable {

@@ -753,7 +753,8 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
     //   2..32      skinny kernel, K split over the waves of a workgroup
     //   33..127    tiled kernel, 32 tokens x 128 rows per workgroup (most workgroups for few tokens)
     //   128..      shared-operand kernel, 128 tokens x 32 rows (x 64 rows from 1024 tokens up)
-    // Q6_K from 33 tokens: its own shared-operand MFMA kernel (mmq_q6k.hip). Otherwise the other
+    // Q5_K, Q6_K and Q8_0 (rows of whole 256s) from 33 tokens: their own shared-operand MFMA kernels
+    // (mmq_q5k.hip, mmq_q6k.hip, mmq_q8_0.hip). Otherwise the other
     // formats take the dot4 GEMV with the activations of up to eight rows in registers (weights
     // re-streamed once per eight rows beyond that).
     static const int env_skinny_max = getenv("INFR_HIP_MMQ_SKINNY_MAX_M") ? atoi(getenv("INFR_HIP_MMQ_SKINNY_MAX_M")) : 32;
@@ -773,6 +774,18 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
     if (dtype == 14 && (int)m >= env_q6k_min) {
         launch_quantize_q8_tiled(x, m, in_f, act, stream);
         launch_mmq_shared_q6k(w, bpr, act, y, m, in_f, out_f, st, stream);
+        return true;
+    }
+    static const int env_q5k_min = getenv("INFR_HIP_MMQ_Q5K_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_Q5K_MIN_M")) : 33;
+    if (dtype == 13 && (int)m >= env_q5k_min) {
+        launch_quantize_q8_tiled(x, m, in_f, act, stream);
+        launch_mmq_shared_q5k(w, bpr, act, y, m, in_f, out_f, st, stream);
+        return true;
+    }
+    static const int env_q8_0_min = getenv("INFR_HIP_MMQ_Q8_0_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_Q8_0_MIN_M")) : 33;
+    if (dtype == 8 && in_f % 256 == 0 && (int)m >= env_q8_0_min) {
+        launch_quantize_q8_tiled(x, m, in_f, act, stream);
+        launch_mmq_shared_q8_0(w, bpr, act, y, m, in_f, out_f, st, stream);
         return true;
     }
     launch_quantize_q8(x, m, in_f, act_is_per32(dtype, in_f), act, stream);

@@ -196,6 +196,62 @@ def test_full_size_prefill_q6k(be):
         assert np.array_equal(single[0].view(np.uint32), y[t].view(np.uint32)), "batch != single"
 
 
+# ───────────── prefill of Q5_K from 33 tokens: its own int8 MFMA kernel ─────────────
+
+@pytest.mark.parametrize("m,in_f,out_f", [(33, 512, 40), (128, 256, 32), (130, 768, 130), (257, 2048, 384),
+                                         (600, 1024, 100)])
+def test_prefill_q5k_mfma_is_bit_identical_to_oracle(be, m, in_f, out_f):
+    w = synth_weight(DType.Q5K, 330 + m, out_f, in_f)
+    x = synth_normal_f32(430 + m, m * in_f)
+    x[:in_f] *= 37.0
+    x[2 * in_f:3 * in_f] = 0.0
+    y = run_linear(be, DType.Q5K, w, x, m, in_f, out_f)
+    want = orc.linear(DType.Q5K, w, x, m, in_f, out_f)
+    gate(y, want)
+    assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), "not bit-identical"
+
+
+def test_prefill_q5k_mfma_int_stages_bit_exact(be):
+    # full-range payload: every 5-bit code, every 6-bit scale and min, saturated rows (|bsums| up to 4064)
+    m, in_f, out_f = 140, 768, 70
+    w = orc.synth_weight(DType.Q5K, in_f * out_f, 0x209)
+    x = synth_normal_f32(80, m * in_f) * np.float32(3.0)
+    x[in_f:2 * in_f] = 1e4
+    x[2 * in_f:3 * in_f] = -1e4
+    a, b = be.linear_int_stages(DType.Q5K, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
+    oa, ob = orc.linear_int_stages(DType.Q5K, w, x, m, in_f, out_f)
+    assert np.array_equal(a, oa)
+    assert np.array_equal(b, ob)
+
+
+# ───────────── prefill of Q8_0 (rows of whole 256s) from 33 tokens: its own int8 MFMA kernel ─────────────
+
+@pytest.mark.parametrize("m,in_f,out_f", [(33, 512, 40), (128, 256, 32), (130, 768, 130), (257, 2048, 384),
+                                         (600, 1024, 100), (70, 1056, 64)])      # 1056: the per-32 arm, dot4
+def test_prefill_q8_0_mfma_vs_oracle(be, m, in_f, out_f):
+    w = synth_weight(DType.Q8_0, 320 + m, out_f, in_f)
+    x = synth_normal_f32(420 + m, m * in_f)
+    x[:in_f] *= 37.0
+    x[2 * in_f:3 * in_f] = 0.0
+    y = run_linear(be, DType.Q8_0, w, x, m, in_f, out_f)
+    want = orc.linear(DType.Q8_0, w, x, m, in_f, out_f)
+    assert np.all(y[2] == 0.0)
+    gate(y, want)
+    rel = np.linalg.norm(y.astype(np.float64) - want) / np.linalg.norm(want)
+    assert rel < 2e-6, rel            # the same terms in another association: rounding level
+
+
+def test_prefill_q8_0_mfma_int_stage_bit_exact(be):
+    m, in_f, out_f = 140, 768, 70
+    w = orc.synth_weight(DType.Q8_0, in_f * out_f, 0x205)          # full-range int8 codes
+    x = synth_normal_f32(79, m * in_f) * np.float32(3.0)
+    x[in_f:2 * in_f] = 1e4
+    x[2 * in_f:3 * in_f] = -1e4
+    a, _ = be.linear_int_stages(DType.Q8_0, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
+    oa, _ = orc.linear_int_stages(DType.Q8_0, w, x, m, in_f, out_f)
+    assert np.array_equal(a, oa)
+
+
 # ───────────── hand-derived known answers (tests/golden/known_answers.json), no oracle involved ─────────────
 
 def _golden():
