@@ -753,8 +753,9 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
     //   2..32      skinny kernel, K split over the waves of a workgroup
     //   33..127    tiled kernel, 32 tokens x 128 rows per workgroup (most workgroups for few tokens)
     //   128..      shared-operand kernel, 128 tokens x 32 rows (x 64 rows from 1024 tokens up)
-    // Q5_K, Q6_K and Q8_0 (rows of whole 256s) from 33 tokens: their own shared-operand MFMA kernels
-    // (mmq_q5k.hip, mmq_q6k.hip, mmq_q8_0.hip). Otherwise the other
+    // Q5_K, Q6_K from 33 tokens, Q8_0 (33) and the 32-weight-block formats (65) on rows of whole 256s:
+    // their own shared-operand MFMA kernels (mmq_q5k.hip, mmq_q6k.hip, mmq_q8_0.hip,
+    // mmq_nib32.hip). Otherwise the other
     // formats take the dot4 GEMV with the activations of up to eight rows in registers (weights
     // re-streamed once per eight rows beyond that).
     static const int env_skinny_max = getenv("INFR_HIP_MMQ_SKINNY_MAX_M") ? atoi(getenv("INFR_HIP_MMQ_SKINNY_MAX_M")) : 32;
@@ -781,6 +782,14 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
         launch_quantize_q8_tiled(x, m, in_f, act, stream);
         launch_mmq_shared_q5k(w, bpr, act, y, m, in_f, out_f, st, stream);
         return true;
+    }
+    // (their kernel's flat time up to 128 tokens, ~145 us at 4096 x 12288, meets the dot4 batches'
+    // ~2.1 us per token at 64 tokens)
+    static const int env_nib_min = getenv("INFR_HIP_MMQ_NIB32_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_NIB32_MIN_M")) : 65;
+    if ((dtype == 2 || dtype == 3 || dtype == 6 || dtype == 7 || dtype == 20) && in_f % 256 == 0 &&
+        (int)m >= env_nib_min) {
+        launch_quantize_q8_32_tiled(x, m, in_f, act, stream);
+        return launch_mmq_shared_nib32(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
     }
     static const int env_q8_0_min = getenv("INFR_HIP_MMQ_Q8_0_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_Q8_0_MIN_M")) : 33;
     if (dtype == 8 && in_f % 256 == 0 && (int)m >= env_q8_0_min) {

@@ -1,0 +1,199 @@
+// Prefill GEMM (65 tokens and up) of the 32-weight-block formats Q4_0, Q4_1, Q5_0, Q5_1 and IQ4_NL on
+// the int8 matrix cores, for rows that are whole 256s.
+//
+// infr-cpu multiplies these against the per-32 activation (scale d8 and code sum bsum per 32
+// elements) and adds per block (crates/infr-cpu/src/kernels.rs:5496-5520, :5793-5822, :5350-5377,
+// :5948-5980, :6128-6152)
+//     Q4_0   d*d8 * (iprod - 8*bsum)        Q5_0   d*d8 * (iprod - 16*bsum)
+//     Q4_1   d8 * (d*iprod + m*bsum)        Q5_1   d8 * (d*iprod + m*bsum)
+//     IQ4_NL d*d8 * iprod                   (iprod over the signed codebook values)
+// The codes (0..15, 0..31, or the codebook's int8) are int8 operands, so iprod is one
+// v_mfma_i32_32x32x32_i8 per block, exact. Every format's term is d8 * (A * iprod + B * bsum) with
+// two per-block constants (A = d; B = -8d, -16d, m or 0), evaluated with one conversion, one
+// multiply and two FMAs per output and block: the CPU's terms in another association (these formats'
+// one-token kernels already differ from the CPU by their butterfly sums), ~1e-7 relative.
+//
+// Tiling as the other shared-operand kernels: 128 tokens x 32 weight rows per workgroup, wave w owns
+// tokens 32w..32w+31 and unpacks blocks 2w, 2w+1 of every row of a 256-element step into LDS in
+// MFMA B order (double-buffered, one barrier per step). Element j of a block is the low nibble of
+// qs[j], element j + 16 the high nibble (plus bit j / j + 16 of qh as the fifth code bit), so the
+// h = 0 lanes of the B operand take the low nibbles of the block's 16 bytes and the h = 1 lanes the
+// high ones.
+#include "gemv_formats.hpp"
+#include "kernels.hpp"
+
+namespace infr {
+
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+// LDS of one 256-element step: B operands [block][lane] x 16 B | A [row][8] | B [row][8] (f32)
+struct Nib32Lds {
+    static constexpr int a_off = 8 * 1024;
+    static constexpr int b_off = a_off + 32 * 8 * 4;
+    static constexpr int bytes = b_off + 32 * 8 * 4;
+};
+
+template <Nib32 K, bool STAGES>
+__global__ __launch_bounds__(256) void mmq_shared_nib32_kernel(
+    const uint8_t* __restrict__ w, size_t bpr, const int8_t* __restrict__ qs, const float* __restrict__ d8,
+    const float* __restrict__ bsf, float* __restrict__ y, int m, int out_f, int nb, int32_t* __restrict__ st_iprod) {
+    constexpr bool kAffine = K == Nib32::Q4_1 || K == Nib32::Q5_1;
+    constexpr bool kFive = K == Nib32::Q5_0 || K == Nib32::Q5_1;
+    constexpr int kBlockBytes = 18 + (kAffine ? 2 : 0) + (kFive ? 4 : 0);
+    constexpr int kQhOff = kAffine ? 4 : 2, kQsOff = kBlockBytes - 16;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * Nib32Lds::bytes];
+    __shared__ __attribute__((aligned(16))) float dql[4][8][32], bql[4][8][32];  // per wave: [block][token]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, h = lane >> 5;
+    const int tok0 = blockIdx.y * 128 + wave * 32;
+    const int wrow = blockIdx.x * 32 + col;
+    const bool row_ok = wrow < out_f;
+    const uint8_t* wrowp = w + (size_t)(row_ok ? wrow : 0) * bpr;
+    const int p = wave;  // this wave unpacks blocks 2p and 2p+1 of the step
+
+    float acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+
+    struct Raw {
+        v4i q[2];
+        uint32_t d[2], mw[2], qh[2];
+    };
+    auto request_rows = [&](Raw& r, int b) {
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const uint8_t* blk = wrowp + ((size_t)b * 8 + 2 * p + e) * kBlockBytes;  // 2-byte aligned
+            r.q[e] = load16_a2(blk + kQsOff);
+            r.d[e] = load_u16(blk);
+            r.mw[e] = kAffine ? load_u16(blk + 2) : 0u;
+            r.qh[e] = kFive ? (load_u16(blk + kQhOff) | (load_u16(blk + kQhOff + 2) << 16)) : 0u;
+        }
+    };
+    auto unpack_to = [&](uint8_t* buf, const Raw& r) {
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            v4i out;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                uint32_t c = ((uint32_t)r.q[e][k] >> (4 * h)) & 0x0F0F0F0Fu;
+                if (K == Nib32::IQ4_NL) c = (uint32_t)iq4nl_lookup(c);
+                if (kFive) c |= spread4_to_bit4(r.qh[e] >> (16 * h + 4 * k));
+                out[k] = (int)c;
+            }
+            *reinterpret_cast<v4i*>(buf + (size_t)(2 * p + e) * 1024 + lane * 16) = out;
+            if (h == 0) {
+                const float d = f16_bits_to_f32(r.d[e]);
+                const float bb = kAffine ? f16_bits_to_f32(r.mw[e])
+                                         : (K == Nib32::IQ4_NL ? 0.0f : (kFive ? -16.0f : -8.0f) * d);
+                reinterpret_cast<float*>(buf + Nib32Lds::a_off)[col * 8 + 2 * p + e] = d;
+                reinterpret_cast<float*>(buf + Nib32Lds::b_off)[col * 8 + 2 * p + e] = bb;
+            }
+        }
+    };
+    // activation fragments in the tiled quantizer's order: every load is a contiguous kilobyte
+    v4i a[8];
+    v4f dt[2], bt[2];  // this lane's token: the step's eight block scales and code sums
+    // this wave's group of 32 tokens; a wave wholly past m recomputes the last group (nothing is stored)
+    const size_t g = min((size_t)blockIdx.y * 4 + wave, (size_t)(m - 1) / 32);
+    auto request_acts = [&](int b) {
+        const size_t gb = g * nb + b;
+        const int8_t* ap = qs + gb * (8 * 1024) + lane * 16;
+#pragma unroll
+        for (int sb = 0; sb < 8; ++sb) a[sb] = *reinterpret_cast<const v4i*>(ap + sb * 1024);
+        const v4f* dp = reinterpret_cast<const v4f*>(d8 + (gb * 32 + col) * 8);
+        const v4f* bp = reinterpret_cast<const v4f*>(bsf + (gb * 32 + col) * 8);
+        dt[0] = dp[0];
+        dt[1] = dp[1];
+        bt[0] = bp[0];
+        bt[1] = bp[1];
+    };
+
+    Raw raw;
+    request_rows(raw, 0);
+    unpack_to(lds, raw);
+    request_rows(raw, min(1, nb - 1));
+    request_acts(0);
+    __syncthreads();
+
+    for (int b = 0; b < nb; ++b) {
+        const uint8_t* cur = lds + (b & 1) * Nib32Lds::bytes;
+        // ---- unpack step b+1 into the other buffer, then ask for step b+2's bytes ----
+        unpack_to(lds + ((b + 1) & 1) * Nib32Lds::bytes, raw);
+        request_rows(raw, min(b + 2, nb - 1));
+        if (h == 0) {
+            const float dv[8] = {dt[0].x, dt[0].y, dt[0].z, dt[0].w, dt[1].x, dt[1].y, dt[1].z, dt[1].w};
+            const float bv[8] = {bt[0].x, bt[0].y, bt[0].z, bt[0].w, bt[1].x, bt[1].y, bt[1].z, bt[1].w};
+#pragma unroll
+            for (int sb = 0; sb < 8; ++sb) {
+                dql[wave][sb][col] = dv[sb];
+                bql[wave][sb][col] = bv[sb];
+            }
+        }
+        const v4f* ap = reinterpret_cast<const v4f*>(cur + Nib32Lds::a_off + col * 32);
+        const v4f* bp = reinterpret_cast<const v4f*>(cur + Nib32Lds::b_off + col * 32);
+        const v4f a0 = ap[0], a1 = ap[1], b0 = bp[0], b1 = bp[1];
+        const float ca[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+        const float cb[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+        const v16i zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int sb = 0; sb < 8; ++sb) {
+            const v4i bf = *reinterpret_cast<const v4i*>(cur + (size_t)sb * 1024 + lane * 16);
+            const v16i r = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[sb], bf, zi, 0, 0, 0);
+            // accumulator i of this lane is token 8*(i/4) + 4*h + i%4 of the wave's 32
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const v4f dq = *reinterpret_cast<const v4f*>(&dql[wave][sb][8 * j + 4 * h]);
+                const v4f bq = *reinterpret_cast<const v4f*>(&bql[wave][sb][8 * j + 4 * h]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int ri = 4 * j + i;
+                    if (STAGES) {
+                        const int tok = tok0 + 8 * j + 4 * h + i;
+                        if (row_ok && tok < m) st_iprod[((size_t)tok * out_f + wrow) * (nb * 8) + b * 8 + sb] = r[ri];
+                    }
+                    // d8 * (A * iprod + B * bsum)
+                    const float t = __builtin_fmaf(cb[sb], bq[i], ca[sb] * (float)r[ri]);
+                    acc[ri] = __builtin_fmaf(dq[i], t, acc[ri]);
+                }
+            }
+        }
+        // the activation registers are free: fetch step b+1
+        request_acts(min(b + 1, nb - 1));
+        __syncthreads();
+    }
+
+    if (!row_ok) return;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int tok = tok0 + 8 * (r >> 2) + 4 * h + (r & 3);
+        if (tok < m) y[(size_t)tok * out_f + wrow] = acc[r];
+    }
+}
+
+template <Nib32 K>
+static void launch_nib32(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
+                         size_t out_f, const IntStages& st, hipStream_t stream) {
+    const dim3 grid((unsigned)((out_f + 31) / 32), (unsigned)((m + 127) / 128)), block(256);
+    const int nb = (int)(in_f / 256);
+    const float* bsf = reinterpret_cast<const float*>(act.bsums);
+    if (st.a)
+        hipLaunchKernelGGL((mmq_shared_nib32_kernel<K, true>), grid, block, 0, stream, w, bpr, act.qs, act.d, bsf, y,
+                           (int)m, (int)out_f, nb, st.a);
+    else
+        hipLaunchKernelGGL((mmq_shared_nib32_kernel<K, false>), grid, block, 0, stream, w, bpr, act.qs, act.d, bsf, y,
+                           (int)m, (int)out_f, nb, (int32_t*)nullptr);
+}
+
+bool launch_mmq_shared_nib32(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
+                             size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream) {
+    switch (dtype) {
+    case 2: launch_nib32<Nib32::Q4_0>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
+    case 3: launch_nib32<Nib32::Q4_1>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
+    case 6: launch_nib32<Nib32::Q5_0>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
+    case 7: launch_nib32<Nib32::Q5_1>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
+    case 20: launch_nib32<Nib32::IQ4_NL>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
+    default: return false;
+    }
+}
+
+}  // namespace infr

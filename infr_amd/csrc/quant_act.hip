@@ -68,6 +68,40 @@ void launch_quantize_q8_tiled(const float* x, size_t m, size_t k, const ActQ8& o
                        out.qs, out.d, reinterpret_cast<_Float16*>(out.bsums), n_chunks, (int)(k / 256));
 }
 
+// The per-32 quantizer (quantize_q8_32, crates/infr-cpu/src/quant.rs:97-117) in the same tiled code
+// order, for the MFMA prefill kernels of the 32-weight-block formats (k % 256 == 0): scales and code
+// sums as f32 [(g*nb + b)*32 + token%32][8 blocks of the 256-element step] (|sum| <= 4064: exact).
+__global__ __launch_bounds__(256) void quantize_q8_32_tiled_kernel(const float* __restrict__ x,
+                                                                   int8_t* __restrict__ qs,
+                                                                   float* __restrict__ d,
+                                                                   float* __restrict__ bsf,
+                                                                   size_t n_chunks, int nb) {
+    const int lane = threadIdx.x & 63;
+    const size_t chunk = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (chunk >= n_chunks) return;  // wave-uniform
+    const v4f v = *reinterpret_cast<const v4f*>(x + chunk * 256 + (size_t)lane * 4);
+    uint32_t packed;
+    float dd;
+    int s, s16;
+    quantize_chunk_values<true>(v, packed, dd, s, s16);
+    const size_t tok = chunk / nb, b = chunk % nb;
+    const size_t gb = (tok >> 5) * nb + b;
+    const int col = (int)(tok & 31);
+    const int sb = lane >> 3, h = (lane >> 2) & 1, j4 = lane & 3;
+    reinterpret_cast<uint32_t*>(qs)[((gb * 8 + sb) * 64 + h * 32 + col) * 4 + j4] = packed;
+    if ((lane & 7) == 0) {
+        d[(gb * 32 + col) * 8 + sb] = dd;
+        bsf[(gb * 32 + col) * 8 + sb] = (float)s;
+    }
+}
+
+void launch_quantize_q8_32_tiled(const float* x, size_t m, size_t k, const ActQ8& out, hipStream_t stream) {
+    const size_t n_chunks = m * k / 256;
+    if (n_chunks == 0) return;
+    hipLaunchKernelGGL(quantize_q8_32_tiled_kernel, dim3((unsigned)((n_chunks + 3) / 4)), dim3(256), 0, stream, x,
+                       out.qs, out.d, reinterpret_cast<float*>(out.bsums), n_chunks, (int)(k / 256));
+}
+
 template <bool PER32>
 __global__ __launch_bounds__(256) void quantize_q8_group_kernel(const QuantTile* __restrict__ tiles,
                                                                 int8_t* __restrict__ qs,

@@ -187,3 +187,30 @@ def block_bytes(dt, in_f):
     from infr_amd import block_layout
     e, b = block_layout(dt)
     return in_f // e * b
+
+
+@pytest.mark.parametrize("dtype", BLK32, ids=ids)
+def test_prefill_mfma_blk32_formats(be, dtype):
+    """From 65 tokens, rows of whole 256s: the int8-MFMA kernel of the 32-weight-block formats. iprod
+    per block bit-exact on full-range payloads; outputs at rounding level of the oracle (the same
+    terms in another association)."""
+    for m, in_f, out_f in ((65, 512, 40), (130, 768, 130), (257, 2048, 96), (70, 1056, 64)):   # 1056: dot4 arm
+        w = synth_weight(dtype, 500 + m, out_f, in_f)
+        x = synth_normal_f32(600 + m, m * in_f)
+        x[:in_f] *= 37.0
+        x[2 * in_f:3 * in_f] = 0.0
+        y = run_linear(be, dtype, w, x, m, in_f, out_f)
+        want = orc.linear(dtype, w, x, m, in_f, out_f)
+        assert np.all(y[2] == 0.0)
+        gate(y, want)
+        rel = np.linalg.norm(y.astype(np.float64) - want) / np.linalg.norm(want)
+        assert rel < 3e-6, (m, in_f, rel)
+    m, in_f, out_f = 140, 768, 70
+    w = orc.synth_weight(dtype, in_f * out_f, 0x310 + dtype)
+    x = synth_normal_f32(81, m * in_f) * np.float32(3.0)
+    x[in_f:2 * in_f] = 1e4
+    x[2 * in_f:3 * in_f] = -1e4
+    a, _ = be.linear_int_stages(dtype, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
+    oa, _ = orc.linear_int_stages(dtype, w, x, m, in_f, out_f)
+    assert np.array_equal(a, oa)
+    gate(run_linear(be, dtype, w, x, m, in_f, out_f), orc.linear(dtype, w, x, m, in_f, out_f))
