@@ -33,8 +33,10 @@ void launch_quantize_q8_group(const QuantTile* tiles_dev, size_t n_tiles, bool p
 // Per-256 quantizer writing MFMA A-operand order (token groups of 32) into the same buffers.
 void launch_quantize_q8_tiled(const float* x, size_t m, size_t k, const ActQ8& out, hipStream_t stream);
 // Per-32 quantizer in the tiled code order (k % 256 == 0): out.d f32 [(g*nb + b)*32 + token%32][8],
-// out.bsums the code sums in the same order, as f32.
-void launch_quantize_q8_32_tiled(const float* x, size_t m, size_t k, const ActQ8& out, hipStream_t stream);
+// out.bsums the code sums in the same order, as f32. transposed16: every 16-element group's codes 4 x 4
+// transposed (dword i = elements i, 4 + i, 8 + i, 12 + i), the order Q2_0's prefill kernel multiplies in.
+void launch_quantize_q8_32_tiled(const float* x, size_t m, size_t k, bool transposed16, const ActQ8& out,
+                                 hipStream_t stream);
 
 // Optional per-block integer-stage outputs, i32 [m][out_f][blocks] (nullptr = not wanted).
 struct IntStages {
@@ -240,8 +242,9 @@ void launch_mmq_shared_q8_0(const uint8_t* w, size_t bpr, const ActQ8& act, floa
 // The same for Q5_K; st.a / st.b receive sd / sm per (token, row, 256-block).
 void launch_mmq_shared_q5k(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
                            size_t out_f, const IntStages& st, hipStream_t stream);
-// The same for Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL rows that are whole 256s, against the per-32 activation in
-// the tiled order (launch_quantize_q8_32_tiled); st.a receives iprod per (token, row, 32-block).
+// The same for Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL (and Q2_0: transposed16 activations) rows that are whole
+// 256s, against the per-32 activation in the tiled order (launch_quantize_q8_32_tiled); st.a receives
+// iprod per (token, row, 32-element block).
 bool launch_mmq_shared_nib32(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
                              size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream);
 // Routed pairs bucketed by expert, in tiles of at most 32 pairs of one expert each (device arrays;

@@ -788,7 +788,12 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
     static const int env_nib_min = getenv("INFR_HIP_MMQ_NIB32_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_NIB32_MIN_M")) : 65;
     if ((dtype == 2 || dtype == 3 || dtype == 6 || dtype == 7 || dtype == 20) && in_f % 256 == 0 &&
         (int)m >= env_nib_min) {
-        launch_quantize_q8_32_tiled(x, m, in_f, act, stream);
+        launch_quantize_q8_32_tiled(x, m, in_f, false, act, stream);
+        return launch_mmq_shared_nib32(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
+    }
+    static const int env_q2_min = getenv("INFR_HIP_MMQ_Q2_0_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_Q2_0_MIN_M")) : 65;
+    if (dtype == 42 && in_f % 256 == 0 && (int)m >= env_q2_min) {
+        launch_quantize_q8_32_tiled(x, m, in_f, true, act, stream);
         return launch_mmq_shared_nib32(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
     }
     static const int env_q8_0_min = getenv("INFR_HIP_MMQ_Q8_0_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_Q8_0_MIN_M")) : 33;

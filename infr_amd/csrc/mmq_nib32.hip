@@ -170,6 +170,130 @@ __global__ __launch_bounds__(256) void mmq_shared_nib32_kernel(
     }
 }
 
+// Q2_0 (64 weights per 18-byte block [f16 d][16 bytes of 2-bit codes], weight = (code - 1) * d, two
+// per-32 activation sub-blocks per block; crates/infr-cpu/src/kernels.rs:5641-5668): the same kernel
+// with A = d, B = -d for both sub-blocks of a block. Code j of a block sits in bits 2(j % 4) of byte
+// j / 4, so one dword of codes is 16 elements and (dword >> 2i) & 0x03030303 is elements i, 4 + i,
+// 8 + i, 12 + i: the activations arrive in that order inside every 16 (the transposed16 quantizer).
+// Wave w unpacks block w of the step (sub-blocks 2w, 2w+1); lane (row, h) takes dword 2e + h.
+template <bool STAGES>
+__global__ __launch_bounds__(256) void mmq_shared_q2_0_kernel(
+    const uint8_t* __restrict__ w, size_t bpr, const int8_t* __restrict__ qs, const float* __restrict__ d8,
+    const float* __restrict__ bsf, float* __restrict__ y, int m, int out_f, int nb, int32_t* __restrict__ st_iprod) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * Nib32Lds::bytes];
+    __shared__ __attribute__((aligned(16))) float dql[4][8][32], bql[4][8][32];  // per wave: [sub-block][token]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, h = lane >> 5;
+    const int tok0 = blockIdx.y * 128 + wave * 32;
+    const int wrow = blockIdx.x * 32 + col;
+    const bool row_ok = wrow < out_f;
+    const uint8_t* wrowp = w + (size_t)(row_ok ? wrow : 0) * bpr;
+    const int p = wave;
+
+    float acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+
+    struct Raw {
+        uint32_t c[2], d;
+    };
+    auto request_rows = [&](Raw& r, int b) {
+        const uint8_t* blk = wrowp + ((size_t)b * 4 + p) * 18;  // 2-byte aligned
+        r.d = load_u16(blk);
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const uint8_t* cp = blk + 2 + 8 * e + 4 * h;
+            r.c[e] = load_u16(cp) | (load_u16(cp + 2) << 16);
+        }
+    };
+    auto unpack_to = [&](uint8_t* buf, const Raw& r) {
+        const float d = f16_bits_to_f32(r.d);
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            v4i out;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) out[i] = (int)((r.c[e] >> (2 * i)) & 0x03030303u);
+            *reinterpret_cast<v4i*>(buf + (size_t)(2 * p + e) * 1024 + lane * 16) = out;
+            if (h == 0) {
+                reinterpret_cast<float*>(buf + Nib32Lds::a_off)[col * 8 + 2 * p + e] = d;
+                reinterpret_cast<float*>(buf + Nib32Lds::b_off)[col * 8 + 2 * p + e] = -d;
+            }
+        }
+    };
+    v4i a[8];
+    v4f dt[2], bt[2];
+    const size_t g = min((size_t)blockIdx.y * 4 + wave, (size_t)(m - 1) / 32);
+    auto request_acts = [&](int b) {
+        const size_t gb = g * nb + b;
+        const int8_t* ap = qs + gb * (8 * 1024) + lane * 16;
+#pragma unroll
+        for (int sb = 0; sb < 8; ++sb) a[sb] = *reinterpret_cast<const v4i*>(ap + sb * 1024);
+        const v4f* dp = reinterpret_cast<const v4f*>(d8 + (gb * 32 + col) * 8);
+        const v4f* bp = reinterpret_cast<const v4f*>(bsf + (gb * 32 + col) * 8);
+        dt[0] = dp[0];
+        dt[1] = dp[1];
+        bt[0] = bp[0];
+        bt[1] = bp[1];
+    };
+
+    Raw raw;
+    request_rows(raw, 0);
+    unpack_to(lds, raw);
+    request_rows(raw, min(1, nb - 1));
+    request_acts(0);
+    __syncthreads();
+
+    for (int b = 0; b < nb; ++b) {
+        const uint8_t* cur = lds + (b & 1) * Nib32Lds::bytes;
+        unpack_to(lds + ((b + 1) & 1) * Nib32Lds::bytes, raw);
+        request_rows(raw, min(b + 2, nb - 1));
+        if (h == 0) {
+            const float dv[8] = {dt[0].x, dt[0].y, dt[0].z, dt[0].w, dt[1].x, dt[1].y, dt[1].z, dt[1].w};
+            const float bv[8] = {bt[0].x, bt[0].y, bt[0].z, bt[0].w, bt[1].x, bt[1].y, bt[1].z, bt[1].w};
+#pragma unroll
+            for (int sb = 0; sb < 8; ++sb) {
+                dql[wave][sb][col] = dv[sb];
+                bql[wave][sb][col] = bv[sb];
+            }
+        }
+        const v4f* ap = reinterpret_cast<const v4f*>(cur + Nib32Lds::a_off + col * 32);
+        const v4f* bp = reinterpret_cast<const v4f*>(cur + Nib32Lds::b_off + col * 32);
+        const v4f a0 = ap[0], a1 = ap[1], b0 = bp[0], b1 = bp[1];
+        const float ca[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+        const float cb[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+        const v16i zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int sb = 0; sb < 8; ++sb) {
+            const v4i bf = *reinterpret_cast<const v4i*>(cur + (size_t)sb * 1024 + lane * 16);
+            const v16i r = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[sb], bf, zi, 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const v4f dq = *reinterpret_cast<const v4f*>(&dql[wave][sb][8 * j + 4 * h]);
+                const v4f bq = *reinterpret_cast<const v4f*>(&bql[wave][sb][8 * j + 4 * h]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int ri = 4 * j + i;
+                    if (STAGES) {
+                        const int tok = tok0 + 8 * j + 4 * h + i;
+                        if (row_ok && tok < m) st_iprod[((size_t)tok * out_f + wrow) * (nb * 8) + b * 8 + sb] = r[ri];
+                    }
+                    const float t = __builtin_fmaf(cb[sb], bq[i], ca[sb] * (float)r[ri]);
+                    acc[ri] = __builtin_fmaf(dq[i], t, acc[ri]);
+                }
+            }
+        }
+        request_acts(min(b + 1, nb - 1));
+        __syncthreads();
+    }
+
+    if (!row_ok) return;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int tok = tok0 + 8 * (r >> 2) + 4 * h + (r & 3);
+        if (tok < m) y[(size_t)tok * out_f + wrow] = acc[r];
+    }
+}
+
 template <Nib32 K>
 static void launch_nib32(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
                          size_t out_f, const IntStages& st, hipStream_t stream) {
@@ -192,6 +316,17 @@ bool launch_mmq_shared_nib32(int dtype, const uint8_t* w, size_t bpr, const ActQ
     case 6: launch_nib32<Nib32::Q5_0>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
     case 7: launch_nib32<Nib32::Q5_1>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
     case 20: launch_nib32<Nib32::IQ4_NL>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
+    case 42: {
+        const dim3 grid((unsigned)((out_f + 31) / 32), (unsigned)((m + 127) / 128)), block(256);
+        const float* bsf = reinterpret_cast<const float*>(act.bsums);
+        if (st.a)
+            hipLaunchKernelGGL((mmq_shared_q2_0_kernel<true>), grid, block, 0, stream, w, bpr, act.qs, act.d, bsf, y,
+                               (int)m, (int)out_f, (int)(in_f / 256), st.a);
+        else
+            hipLaunchKernelGGL((mmq_shared_q2_0_kernel<false>), grid, block, 0, stream, w, bpr, act.qs, act.d, bsf, y,
+                               (int)m, (int)out_f, (int)(in_f / 256), (int32_t*)nullptr);
+        return true;
+    }
     default: return false;
     }
 }

@@ -71,6 +71,11 @@ void launch_quantize_q8_tiled(const float* x, size_t m, size_t k, const ActQ8& o
 // The per-32 quantizer (quantize_q8_32, crates/infr-cpu/src/quant.rs:97-117) in the same tiled code
 // order, for the MFMA prefill kernels of the 32-weight-block formats (k % 256 == 0): scales and code
 // sums as f32 [(g*nb + b)*32 + token%32][8 blocks of the 256-element step] (|sum| <= 4064: exact).
+// T16: the codes of every 16-element group are stored 4 x 4 transposed (dword i of the group holds
+// elements i, 4 + i, 8 + i, 12 + i), the K order in which Q2_0's 2-bit codes unpack with one shift and
+// one mask per dword; the matrix product does not care about the order inside a group as long as
+// both operands share it.
+template <bool T16>
 __global__ __launch_bounds__(256) void quantize_q8_32_tiled_kernel(const float* __restrict__ x,
                                                                    int8_t* __restrict__ qs,
                                                                    float* __restrict__ d,
@@ -88,6 +93,17 @@ __global__ __launch_bounds__(256) void quantize_q8_32_tiled_kernel(const float* 
     const size_t gb = (tok >> 5) * nb + b;
     const int col = (int)(tok & 31);
     const int sb = lane >> 3, h = (lane >> 2) & 1, j4 = lane & 3;
+    if (T16) {
+        // lanes 4g..4g+3 hold the group's dwords P0..P3 (elements 4j..4j+3); lane i leaves with byte i
+        // of each
+        const int base = lane & ~3;
+        const uint32_t p0 = (uint32_t)__shfl((int)packed, base, kWave), p1 = (uint32_t)__shfl((int)packed, base + 1, kWave);
+        const uint32_t p2 = (uint32_t)__shfl((int)packed, base + 2, kWave), p3 = (uint32_t)__shfl((int)packed, base + 3, kWave);
+        const uint32_t sel = (uint32_t)j4 | ((uint32_t)(4 + j4) << 8);       // byte i of src1, byte i of src0
+        const uint32_t t01 = __builtin_amdgcn_perm(p1, p0, sel) & 0xFFFFu;   // (P0.b_i, P1.b_i)
+        const uint32_t t23 = __builtin_amdgcn_perm(p3, p2, sel) & 0xFFFFu;   // (P2.b_i, P3.b_i)
+        packed = t01 | (t23 << 16);
+    }
     reinterpret_cast<uint32_t*>(qs)[((gb * 8 + sb) * 64 + h * 32 + col) * 4 + j4] = packed;
     if ((lane & 7) == 0) {
         d[(gb * 32 + col) * 8 + sb] = dd;
@@ -95,11 +111,17 @@ __global__ __launch_bounds__(256) void quantize_q8_32_tiled_kernel(const float* 
     }
 }
 
-void launch_quantize_q8_32_tiled(const float* x, size_t m, size_t k, const ActQ8& out, hipStream_t stream) {
+void launch_quantize_q8_32_tiled(const float* x, size_t m, size_t k, bool transposed16, const ActQ8& out,
+                                 hipStream_t stream) {
     const size_t n_chunks = m * k / 256;
     if (n_chunks == 0) return;
-    hipLaunchKernelGGL(quantize_q8_32_tiled_kernel, dim3((unsigned)((n_chunks + 3) / 4)), dim3(256), 0, stream, x,
-                       out.qs, out.d, reinterpret_cast<float*>(out.bsums), n_chunks, (int)(k / 256));
+    const dim3 grid((unsigned)((n_chunks + 3) / 4));
+    if (transposed16)
+        hipLaunchKernelGGL(quantize_q8_32_tiled_kernel<true>, grid, dim3(256), 0, stream, x, out.qs, out.d,
+                           reinterpret_cast<float*>(out.bsums), n_chunks, (int)(k / 256));
+    else
+        hipLaunchKernelGGL(quantize_q8_32_tiled_kernel<false>, grid, dim3(256), 0, stream, x, out.qs, out.d,
+                           reinterpret_cast<float*>(out.bsums), n_chunks, (int)(k / 256));
 }
 
 template <bool PER32>

@@ -252,6 +252,34 @@ def test_prefill_q8_0_mfma_int_stage_bit_exact(be):
     assert np.array_equal(a, oa)
 
 
+# ───────────── prefill of Q2_0 (rows of whole 256s) from 65 tokens: its own int8 MFMA kernel ─────────────
+
+@pytest.mark.parametrize("m,in_f,out_f", [(65, 512, 40), (130, 768, 130), (257, 2048, 384), (600, 1024, 100),
+                                         (70, 320, 64)])                        # 320: not whole 256s, dot4
+def test_prefill_q2_0_mfma_vs_oracle(be, m, in_f, out_f):
+    w = synth_weight(DType.Q2_0, 340 + m, out_f, in_f)
+    x = synth_normal_f32(440 + m, m * in_f)
+    x[:in_f] *= 37.0
+    x[2 * in_f:3 * in_f] = 0.0
+    y = run_linear(be, DType.Q2_0, w, x, m, in_f, out_f)
+    want = orc.linear(DType.Q2_0, w, x, m, in_f, out_f)
+    assert np.all(y[2] == 0.0)
+    gate(y, want)
+    rel = np.linalg.norm(y.astype(np.float64) - want) / np.linalg.norm(want)
+    assert rel < 3e-6, rel
+
+
+def test_prefill_q2_0_mfma_int_stage_bit_exact(be):
+    m, in_f, out_f = 140, 768, 70
+    w = orc.synth_weight(DType.Q2_0, in_f * out_f, 0x216)          # all four code values
+    x = synth_normal_f32(82, m * in_f) * np.float32(3.0)
+    x[in_f:2 * in_f] = 1e4
+    x[2 * in_f:3 * in_f] = -1e4
+    a, _ = be.linear_int_stages(DType.Q2_0, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
+    oa, _ = orc.linear_int_stages(DType.Q2_0, w, x, m, in_f, out_f)
+    assert np.array_equal(a, oa)
+
+
 # ───────────── hand-derived known answers (tests/golden/known_answers.json), no oracle involved ─────────────
 
 def _golden():
