@@ -982,21 +982,31 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     if (!gbpr || !ubpr || !dbpr) return "rows >= 2 carries Q4_K / Q5_K / Q6_K / Q8_0 expert banks";
     launch_quantize_q8(b.x, s.rows, s.ne, false, aq, stream);
     const size_t n_act = pairs * s.n_ff, n_out = (size_t)s.rows * s.ne;
-    // Prefill-sized batches: the pairs are bucketed by expert and every Q4_K bank runs the
+    // Prefill-sized batches: the pairs are bucketed by expert and every Q4_K or Q6_K bank runs its
     // int8-MFMA GEMM per (expert, 32 pairs) tile, so an expert's weights are read once per 32 of
     // its pairs instead of once per pair. From an average of `bucket_min` pairs per expert up (the
     // per-pair GEMVs win below: most tiles would hold one or two pairs). Banks of other formats keep
-    // the per-pair GEMVs (a Q4_K_M file's Q6_K `ffn_down_exps` beside Q4_K gate / up).
+    // the per-pair GEMVs.
     static const int bucket_min = getenv("INFR_HIP_MOE_BUCKET_MIN") ? atoi(getenv("INFR_HIP_MOE_BUCKET_MIN")) : 4;
+    // (a Q6_K tile costs more than a Q4_K one: at four pairs per expert its per-pair GEMVs are still
+    // ahead, 199 us against 214 per layer; from eight it is bucketed)
+    auto has_mfma = [&](int dt) {
+        return (dt == 12 && pairs >= (size_t)bucket_min * s.n_expert) || (dt == 14 && pairs >= (size_t)2 * bucket_min * s.n_expert);
+    };
+    auto launch_gathered = [&](int dt, const uint8_t* bank, size_t stride, size_t bpr_, int act_div, const MoeTileTable& t,
+                               float* out, size_t in_f, size_t out_f) {
+        if (dt == 12) launch_mmq_q4k_gathered(bank, stride, bpr_, aq, act_div, t, out, in_f, out_f, stream);
+        else launch_mmq_q6k_gathered(bank, stride, bpr_, aq, act_div, t, out, in_f, out_f, stream);
+    };
     const bool bucketed = bucket_min > 0 && pairs >= (size_t)bucket_min * s.n_expert && pairs <= (size_t)1 << 24 &&
-                          (s.gate_dtype == 12 || s.up_dtype == 12 || s.down_dtype == 12);
+                          (has_mfma(s.gate_dtype) || has_mfma(s.up_dtype) || has_mfma(s.down_dtype));
     const MoeTileTable tt{n_tiles, tile_expert, tile_slot0, tile_count, perm, (int)max_tiles};
     if (bucketed)
         hipLaunchKernelGGL(moe_bucket_kernel, dim3(1), dim3(kBucketThreads), 0, stream, sel_idx, (int)pairs,
                            s.n_expert, perm, tile_expert, tile_slot0, tile_count, n_tiles);
-    const bool gate_mfma = bucketed && s.gate_dtype == 12, up_mfma = bucketed && s.up_dtype == 12;
-    if (gate_mfma) launch_mmq_q4k_gathered(b.gate, b.gate_stride, gbpr, aq, s.n_used, tt, gbuf, s.ne, s.n_ff, stream);
-    if (up_mfma) launch_mmq_q4k_gathered(b.up, b.up_stride, ubpr, aq, s.n_used, tt, ubuf, s.ne, s.n_ff, stream);
+    const bool gate_mfma = bucketed && has_mfma(s.gate_dtype), up_mfma = bucketed && has_mfma(s.up_dtype);
+    if (gate_mfma) launch_gathered(s.gate_dtype, b.gate, b.gate_stride, gbpr, s.n_used, tt, gbuf, s.ne, s.n_ff);
+    if (up_mfma) launch_gathered(s.up_dtype, b.up, b.up_stride, ubpr, s.n_used, tt, ubuf, s.ne, s.n_ff);
     bool gate_up_ok = true;
     if (!gate_mfma && !up_mfma && s.gate_dtype == s.up_dtype) {
         gate_up_ok = launch_gemv_id(s.gate_dtype, b.gate, b.gate_stride, gbpr, sel_idx, aq, s.ne, s.n_used, (int)pairs,
@@ -1013,8 +1023,8 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     hipLaunchKernelGGL(moe_act_quant_kernel, dim3((unsigned)((n_act / 256 + 3) / 4)), dim3(256), 0, stream,
                        gbuf, ubuf, aq.qs, aq.d, aq.bsums, aq.bsums16, n_act);
     // the down projection's activation row is the pair itself: n_used = 1
-    if (bucketed && s.down_dtype == 12)
-        launch_mmq_q4k_gathered(b.down, b.down_stride, dbpr, aq, 1, tt, yp, s.n_ff, s.ne, stream);
+    if (bucketed && has_mfma(s.down_dtype))
+        launch_gathered(s.down_dtype, b.down, b.down_stride, dbpr, 1, tt, yp, s.n_ff, s.ne);
     else if (!launch_gemv_id(s.down_dtype, b.down, b.down_stride, dbpr, sel_idx, aq, s.n_ff, 1, (int)pairs, yp, s.ne, stream))
         return "no id-gathered kernel for this down shape";
     hipLaunchKernelGGL(moe_accumulate_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, stream,

@@ -220,11 +220,14 @@ def test_moe_qwen3_30b_a3b_prefill(be):
     assert np.isfinite(y).all() and len(np.unique(idx)) > 100        # most experts are touched
 
 
-@pytest.mark.parametrize("gu,down", [(DType.Q4K, DType.Q6K), (DType.Q6K, DType.Q4K)])
+@pytest.mark.parametrize("gu,down", [(DType.Q4K, DType.Q6K), (DType.Q6K, DType.Q4K), (DType.Q6K, DType.Q6K),
+                                     (DType.Q4K, DType.Q8_0)])
 def test_moe_prefill_buckets_with_mixed_bank_formats(be, gu, down):
-    """A Q4_K_M file's mix (Q4_K gate / up beside a Q6_K down bank) and its mirror: the Q4_K banks
-    take the bucketed MFMA GEMM, the others the per-pair GEMVs, in one op."""
-    rows, ne, n_expert, n_used, nff = 96, 512, 16, 4, 256
+    """A Q4_K_M file's mix (Q4_K gate / up beside a Q6_K down bank), its mirror, all-Q6_K, and a bank
+    without a bucketed kernel: Q4_K and Q6_K banks take their bucketed MFMA GEMM, the others the
+    per-pair GEMVs, in one op - and the first two tokens, run again as a batch of two (per-pair
+    GEMVs throughout), give the same bits."""
+    rows, ne, n_expert, n_used, nff = 96, 512, 16, 4, 256          # 24 pairs per expert
     gate_w = synth_weight(gu, 201, n_expert * nff, ne, 0.05)
     up_w = synth_weight(gu, 202, n_expert * nff, ne, 0.05)
     down_w = synth_weight(down, 203, n_expert * ne, nff, 0.05)
@@ -239,3 +242,10 @@ def test_moe_prefill_buckets_with_mixed_bank_formats(be, gu, down):
     want = orc.moe_ffn(x, router, gate_w, up_w, down_w, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
                        scale=1.0, gate_dtype=int(gu), up_dtype=int(gu), down_dtype=int(down))
     check(*got, *want)
+    y2 = be.alloc(2 * ne * 4)
+    be.moe_ffn(be.upload_new(x[:2 * ne]), be.upload_new(router), be.upload_new(gate_w), be.upload_new(up_w),
+               be.upload_new(down_w), y2, rows=2, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
+               scale=1.0, gate_dtype=gu, up_dtype=gu, down_dtype=down)
+    two = be.download(y2, np.empty((2, ne), np.float32))
+    if DType.Q8_0 not in (gu, down):       # the ordered formats: bit-identical whichever kernel ran
+        assert np.array_equal(two.view(np.uint32), got[0][:2].view(np.uint32)), "bucketed != per-pair"
