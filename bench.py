@@ -11,7 +11,7 @@ bytes / wall time of the timed steps (inputs resident in HBM), the reference's G
 The same JSON line carries `roofline` for the dominant kernel (the Q4_K GEMV; achieved = weight
 bytes per launch / average launch duration from HIP events on the backend's stream), the
 `cpu_baseline` (the C restatement of infr-cpu's scalar kernels on the host cores, bounded sample)
-and `extra` with the secondary figures BASELINE.json names: Q6_K / Q8_0 GEMV, batch 8, prefill
+and `extra` with the secondary figures of the benchmark's other configurations: Q6_K / Q8_0 GEMV, batch 8, prefill
 mmq int8 TOPS at M in {64, 512, 2048}, the ternary Q2_0 sweep and the MoE routed-expert GEMV.
 """
 from __future__ import annotations
