@@ -131,8 +131,8 @@ int infr_hip_sync(infr_hip_t *be);
  * Q4_K/Q6_K/Q8_0, crates/infr-cpu/src/quant.rs:27-58; per-32 for Q2_0, quant.rs:97-117), the
  * integer dot is exact, and the f32 epilogue follows the CPU kernels' expression per block.
  * in_f must be a whole number of weight blocks (256 for the K-quants, 64 for Q2_0, 32 otherwise): a
- * shorter tail is rejected, never truncated. in_f above 32768 (Q8_0, Q4_1, Q5_1: 16384) returns
- * INFR_HIP_ERR_UNSUPPORTED, except Q4_K at m >= 2. */
+ * shorter tail is rejected, never truncated. in_f above 32768 (Q8_0, Q4_1, Q5_1: 16384) must be a
+ * multiple of 256 (it then runs the prefill kernels at any m), else INFR_HIP_ERR_UNSUPPORTED. */
 int infr_hip_linear(infr_hip_t *be, int dtype, const infr_hip_buffer_t *w, size_t w_numel,
                     size_t w_off, const infr_hip_buffer_t *x, infr_hip_buffer_t *dst, size_t m,
                     size_t in_f, size_t out_f);

@@ -117,7 +117,7 @@ size_t stage_blocks(int dt, size_t in_f) {
 bool has_two_stages(int dt) { return dt == INFR_DTYPE_Q4_K || dt == INFR_DTYPE_Q5_K; }
 
 // Activation scratch for m rows: the prefill kernels read tokens in groups of 32.
-static size_t act_scratch_elems(size_t m, size_t in_f) { return (m == 1 ? 1 : (m + 31) / 32 * 32) * in_f; }
+static size_t act_scratch_elems(size_t m, size_t in_f) { return (m + 31) / 32 * 32 * in_f; }
 
 static bool is_elementwise(int kind) { return kind >= INFR_OP_RMS_NORM && kind <= INFR_OP_ADD; }
 
@@ -198,10 +198,18 @@ static int enqueue_elementwise(infr_hip_t* be, const infr_hip_op_t& op, const El
     return INFR_HIP_OK;
 }
 
+// Linears that are launched on their own, outside the fused / grouped decode and small-batch
+// launches: one token of a format whose CPU arm multiplies f32 activations, and rows too long for
+// the decode mapping (those go to the prefill kernels at any m).
+static bool runs_alone(int dtype, size_t m, size_t in_f) {
+    return infr::gemv_takes_f32_activations(dtype, m) || infr::gemv_row_too_long(dtype, in_f);
+}
+
 // Ops that run in small-batch groups inside plans: the K-split MFMA kernel takes Q4_K up to 32
 // rows, the dot4 batch kernel the other formats up to 8.
 static bool small_batch(const infr_hip_op_t& op) {
-    return op.m >= 2 && op.m <= (op.w_dtype == INFR_DTYPE_Q4_K ? 32u : 8u);
+    return op.m >= 2 && op.m <= (op.w_dtype == INFR_DTYPE_Q4_K ? 32u : 8u) &&
+           !infr::gemv_row_too_long(op.w_dtype, op.in_f);
 }
 
 // (Re)allocates a device table when it grew and enqueues the copy on the backend stream.
@@ -294,7 +302,7 @@ int enqueue_linear(infr_hip_t* be, int dtype, const LinearArgs& la, const float*
             return fail(be, INFR_HIP_ERR_UNSUPPORTED,
                         "int_stages: one token of dtype " + std::to_string(dtype) + " has no integer stage");
         ok = infr::launch_gemv_f32act(dtype, la.wrows, la.bpr, x, y, in_f, out_f, be->stream);
-    } else if (m == 1) {
+    } else if (m == 1 && !infr::gemv_row_too_long(dtype, in_f)) {
         infr::launch_quantize_q8(x, m, in_f, act_per32(dtype, in_f), be->act, be->stream);
         ok = infr::launch_gemv(dtype, la.wrows, la.bpr, be->act, y, in_f, out_f, st, be->stream);
     } else {
@@ -557,7 +565,7 @@ int infr_hip_linear(infr_hip_t* be, int dtype, const infr_hip_buffer_t* w, size_
     if (int rc = check_linear(be, dtype, w, w_numel, w_off, x, m, in_f, out_f, &la)) return rc;
     if (!dst || dst->len < m * out_f * sizeof(float))
         return fail(be, INFR_HIP_ERR_INVALID, "linear: dst buffer missing or too small");
-    if (m == 1 && !infr::gemv_takes_f32_activations(dtype, m)) {
+    if (m == 1 && !runs_alone(dtype, m, in_f)) {
         // decode: one fused launch (quantize x in LDS + GEMV)
         const infr::GemvOpDesc op{la.wrows, static_cast<const float*>(x->ptr),
                                   static_cast<float*>(dst->ptr), la.bpr, (int32_t)out_f};
@@ -893,7 +901,7 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
     static const int env_fuse = getenv("INFR_HIP_FUSE") ? atoi(getenv("INFR_HIP_FUSE")) : 1;
     auto decode_linear = [&](size_t i) {
         return plan->ops[i].kind == INFR_OP_LINEAR && plan->ops[i].m == 1 &&
-               !infr::gemv_takes_f32_activations(plan->ops[i].w_dtype, 1);
+               !runs_alone(plan->ops[i].w_dtype, 1, plan->ops[i].in_f);
     };
     for (size_t k = 0; env_fuse && k < n; ++k) {
         const auto& p = plan->ops[k];
@@ -1040,7 +1048,7 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
                 plan->steps.push_back(st);
                 continue;
             }
-            if (op.kind != INFR_OP_LINEAR || op.m != 1 || infr::gemv_takes_f32_activations(op.w_dtype, op.m)) {
+            if (op.kind != INFR_OP_LINEAR || op.m != 1 || runs_alone(op.w_dtype, op.m, op.in_f)) {
                 st.op = (int)i;
                 taken[i] = 1;
                 plan->steps.push_back(st);

@@ -43,6 +43,11 @@ static const GemvFormatOps* format_ops(int dtype, size_t in_f) {
     }
 }
 
+bool gemv_row_too_long(int dtype, size_t in_f) {
+    const GemvFormatOps* o = format_ops(dtype, in_f);
+    return o != nullptr && in_f > (size_t)8 * (size_t)o->elems_per_step;
+}
+
 bool launch_gemv(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t in_f,
                  size_t out_f, const IntStages& st, hipStream_t stream) {
     if (out_f == 0) return true;

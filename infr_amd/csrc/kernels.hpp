@@ -182,6 +182,9 @@ struct GemvFormatOps {
     bool (*fused)(size_t in_f, const GemvOpDesc& op, const GemvTile* tiles_dev, const GemvGroupPlan& plan,
                   hipStream_t stream) = nullptr;
 };
+// Rows longer than eight wave steps of the format's decode mapping have no decode or small-batch
+// kernel; when they are whole 256s the prefill kernels (which walk the blocks) take them at any m.
+bool gemv_row_too_long(int dtype, size_t in_f);
 const GemvFormatOps& gemv_ops_q4k();
 const GemvFormatOps& gemv_ops_q6k();
 const GemvFormatOps& gemv_ops_q8_0();

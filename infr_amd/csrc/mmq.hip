@@ -651,10 +651,13 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
     // mmq_nib32.hip). Otherwise the other
     // formats take the dot4 GEMV with the activations of up to eight rows in registers (weights
     // re-streamed once per eight rows beyond that).
+    // rows beyond the decode / small-batch kernels' length, when whole 256s, take the MFMA kernel of
+    // their format at any token count (a 128-token tile for one token: slow, but exact and bounded)
+    const bool long_row = gemv_row_too_long(dtype, in_f) && in_f % 256 == 0;
     static const int env_skinny_max = getenv("INFR_HIP_MMQ_SKINNY_MAX_M") ? atoi(getenv("INFR_HIP_MMQ_SKINNY_MAX_M")) : 32;
     static const int env_shared_min = getenv("INFR_HIP_MMQ_SHARED_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_SHARED_MIN_M")) : 128;
     static const int env_shared_rows = getenv("INFR_HIP_MMQ_SHARED_ROWS") ? atoi(getenv("INFR_HIP_MMQ_SHARED_ROWS")) : 0;
-    if (dtype == 12 && (int)m >= env_shared_min) {
+    if (dtype == 12 && ((int)m >= env_shared_min || long_row)) {
         launch_quantize_q8_tiled(x, m, in_f, act, stream);
         const bool wide = env_shared_rows ? env_shared_rows == 64 : m >= 1024;
         if (wide) launch_mmq_shared_q4k<2>(w, bpr, act, y, m, in_f, out_f, st, stream);
@@ -665,13 +668,13 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
     // 4096 x 12288, 1024 x 4096) and the dot4 batches cost ~3.5 / 3.2 / 1.1 us per token there, so
     // it takes over from 33 tokens
     static const int env_q6k_min = getenv("INFR_HIP_MMQ_Q6K_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_Q6K_MIN_M")) : 33;
-    if (dtype == 14 && (int)m >= env_q6k_min) {
+    if (dtype == 14 && ((int)m >= env_q6k_min || long_row)) {
         launch_quantize_q8_tiled(x, m, in_f, act, stream);
         launch_mmq_shared_q6k(w, bpr, act, y, m, in_f, out_f, st, stream);
         return true;
     }
     static const int env_q5k_min = getenv("INFR_HIP_MMQ_Q5K_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_Q5K_MIN_M")) : 33;
-    if (dtype == 13 && (int)m >= env_q5k_min) {
+    if (dtype == 13 && ((int)m >= env_q5k_min || long_row)) {
         launch_quantize_q8_tiled(x, m, in_f, act, stream);
         launch_mmq_shared_q5k(w, bpr, act, y, m, in_f, out_f, st, stream);
         return true;
@@ -680,17 +683,17 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
     // ~2.1 us per token at 64 tokens)
     static const int env_nib_min = getenv("INFR_HIP_MMQ_NIB32_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_NIB32_MIN_M")) : 65;
     if ((dtype == 2 || dtype == 3 || dtype == 6 || dtype == 7 || dtype == 20) && in_f % 256 == 0 &&
-        (int)m >= env_nib_min) {
+        ((int)m >= env_nib_min || long_row)) {
         launch_quantize_q8_32_tiled(x, m, in_f, false, act, stream);
         return launch_mmq_shared_nib32(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
     }
     static const int env_q2_min = getenv("INFR_HIP_MMQ_Q2_0_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_Q2_0_MIN_M")) : 65;
-    if (dtype == 42 && in_f % 256 == 0 && (int)m >= env_q2_min) {
+    if (dtype == 42 && in_f % 256 == 0 && ((int)m >= env_q2_min || long_row)) {
         launch_quantize_q8_32_tiled(x, m, in_f, true, act, stream);
         return launch_mmq_shared_nib32(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
     }
     static const int env_q8_0_min = getenv("INFR_HIP_MMQ_Q8_0_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_Q8_0_MIN_M")) : 33;
-    if (dtype == 8 && in_f % 256 == 0 && (int)m >= env_q8_0_min) {
+    if (dtype == 8 && in_f % 256 == 0 && ((int)m >= env_q8_0_min || long_row)) {
         launch_quantize_q8_tiled(x, m, in_f, act, stream);
         launch_mmq_shared_q8_0(w, bpr, act, y, m, in_f, out_f, st, stream);
         return true;

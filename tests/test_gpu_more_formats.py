@@ -167,20 +167,57 @@ def test_ragged_rows_are_refused(be):
         assert e.value.status == Status.Unsupported
 
 
-def test_rows_beyond_eight_wave_steps_are_refused_not_truncated(be):
-    """in_f above the formats' bound (32768; 16384 for Q8_0 / Q4_1 / Q5_1) is Unsupported, and the
-    bound itself still computes."""
-    for dt, in_f in ((DType.Q8_0, 16384 + 32), (DType.Q4_1, 16384 + 32), (DType.Q5K, 32768 + 256)):
+def test_rows_beyond_eight_wave_steps(be):
+    """in_f above the decode kernels' bound (32768; 16384 for Q8_0 / Q4_1 / Q5_1): rows of whole 256s
+    run the prefill kernels at any token count - same integers, same results - and other lengths are
+    Unsupported, never truncated. The bound itself still takes the decode kernel."""
+    for dt, in_f in ((DType.Q8_0, 16384 + 32), (DType.Q4_1, 16384 + 32), (DType.Q5_0, 32768 + 256)):
         w = be.alloc(block_bytes(dt, in_f) * 2)
         x = be.alloc(in_f * 4)
         y = be.alloc(8)
         with pytest.raises(InfrError) as e:
-            be.linear(dt, w, x, y, 1, in_f, 2)
+            be.linear(dt, w, x, y, 1, in_f, 2)      # (one token of Q5_0 multiplies f32 activations: no int8 arm)
         assert e.value.status == Status.Unsupported
     in_f, out_f = 16384, 24
     w = synth_weight(DType.Q8_0, 77, out_f, in_f)
     x = synth_normal_f32(78, in_f)
     gate(run_linear(be, DType.Q8_0, w, x, 1, in_f, out_f), orc.linear(DType.Q8_0, w, x, 1, in_f, out_f))
+    for dt, in_f in ((DType.Q4K, 33024), (DType.Q5K, 33024), (DType.Q6K, 33024), (DType.Q8_0, 16640),
+                     (DType.Q4_0, 33024), (DType.Q4_1, 16640), (DType.Q2_0, 33024)):
+        out_f = 40
+        w = synth_weight(dt, 90 + int(dt), out_f, in_f)
+        for m in (1, 5, 40):
+            x = synth_normal_f32(91 + m, m * in_f)
+            y = run_linear(be, dt, w, x, m, in_f, out_f)
+            want = orc.linear(dt, w, x, m, in_f, out_f)
+            gate(y, want)
+            if dt in (DType.Q4K, DType.Q5K, DType.Q6K):
+                assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), (dt, m)
+
+
+def test_long_rows_inside_a_plan(be):
+    in_f, out_f = 33024, 32
+    g, binds = Graph(), Bindings()
+    x1 = g.input(TensorDesc((1, in_f), DType.F32))
+    xs = synth_normal_f32(5, in_f)
+    binds.bind(x1, be.upload_new(xs))
+    outs = []
+    for dt in (DType.Q4K, DType.Q6K):
+        w = synth_weight(dt, 60 + int(dt), out_f, in_f)
+        wt = g.weight(TensorDesc((out_f, in_f), dt))
+        binds.bind(wt, be.upload_new(w))
+        yt = g.output(TensorDesc((1, out_f), DType.F32))
+        yb = be.alloc(out_f * 4)
+        binds.bind(yt, yb)
+        g.push(Linear(x1, wt, yt, 1, in_f, out_f))
+        outs.append((dt, w, yb))
+    plan = be.compile(g)
+    for _ in range(2):
+        be.execute(plan, binds)
+        for dt, w, yb in outs:
+            got = be.download(yb, np.empty((1, out_f), np.float32))
+            want = orc.linear(dt, w, xs, 1, in_f, out_f)
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), dt
 
 
 def block_bytes(dt, in_f):
