@@ -265,9 +265,11 @@ struct MoeTileTable {
 // and f32 epilogue as the dense kernel, so every output equals the per-pair GEMV's bit for bit.
 void launch_mmq_q4k_gathered(const uint8_t* bank, size_t expert_stride, size_t bpr, const ActQ8& act, int act_div,
                              const MoeTileTable& t, float* y, size_t in_f, size_t out_f, hipStream_t stream);
-// The same over a Q6_K bank (mmq_q6k.hip).
-void launch_mmq_q6k_gathered(const uint8_t* bank, size_t expert_stride, size_t bpr, const ActQ8& act, int act_div,
-                             const MoeTileTable& t, float* y, size_t in_f, size_t out_f, hipStream_t stream);
+// The same by bank format: Q4_K through the call above, Q5_K / Q6_K / Q8_0 through their tile kernels
+// (mmq_gathered.hip). false: the format has no bucketed kernel.
+bool launch_mmq_gathered(int dtype, const uint8_t* bank, size_t expert_stride, size_t bpr, const ActQ8& act,
+                         int act_div, const MoeTileTable& t, float* y, size_t in_f, size_t out_f,
+                         hipStream_t stream);
 size_t moe_workspace_bytes(const MoeShape& s);
 // Enqueues the whole op; returns nullptr or a message naming what is unsupported.
 const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* workspace, hipStream_t stream);

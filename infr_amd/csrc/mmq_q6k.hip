@@ -19,7 +19,6 @@
 // contiguous kilobyte per load.
 #include "device_common.hpp"
 #include "kernels.hpp"
-#include "mmq_tiles.hpp"
 
 namespace infr {
 
@@ -164,127 +163,6 @@ __global__ __launch_bounds__(256) void mmq_shared_q6k_kernel(
         const int tok = tok0 + 8 * (r >> 2) + 4 * h + (r & 3);
         if (tok < m) y[(size_t)tok * out_f + wrow] = acc[r];
     }
-}
-
-// Routed-expert form (MoE prefill with a Q6_K bank): tiles of up to 32 pairs of one expert, as the
-// Q4_K tiled kernel takes them (mmq_tiles.hpp). A workgroup covers the tile's pairs x 128 rows of the
-// expert; every wave unpacks its own 32 rows - lane (row, h) the 16-element halves 16h..16h+15 of all
-// eight sub-blocks - into B operands held in registers, and the activation tile (row-major per-256
-// quantized rows, gathered through `perm`) sits in double-buffered LDS. A group's MFMA reads the
-// activations of the other half from zero bytes. Integers, epilogue and block order are the dense
-// kernel's: every pair's outputs equal the per-pair GEMV's bit for bit.
-__global__ __launch_bounds__(256) void mmq_q6k_gathered_kernel(const uint8_t* __restrict__ w, size_t bpr,
-                                                               const int8_t* __restrict__ qs,
-                                                               const float* __restrict__ d8,
-                                                               const int32_t* __restrict__ bsums,
-                                                               float* __restrict__ y, GatheredTiles tiles,
-                                                               int out_f, int nb) {
-    constexpr int BM = 32;
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * MmqLds<BM>::bytes];
-    __shared__ __attribute__((aligned(16))) int zero16[4];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int col = lane & 31, h = lane >> 5;
-    const int tile_y = blockIdx.y;
-    size_t w_off = 0;
-    if (!tiles.select(tile_y, w_off)) return;  // uniform over the workgroup, before any barrier
-    const int n_slots = tiles.count(tile_y, BM);
-    const int wrow = blockIdx.x * 128 + wave * 32 + col;
-    const bool row_ok = wrow < out_f;
-    const uint8_t* wrowp = w + w_off + (size_t)(row_ok ? wrow : 0) * bpr;
-    if (tid < 4) zero16[tid] = 0;
-
-    float acc[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
-
-    struct Raw {
-        v4i ql[4], qh[2], sc;  // ql[2 * half + (qd & 1)], qh[half]: this lane's 16 bytes of each
-        uint32_t d;
-    };
-    auto load_raw = [&](Raw& r, int b) {
-        const uint8_t* blk = wrowp + (size_t)b * 210;  // 2-byte aligned
-#pragma unroll
-        for (int k = 0; k < 4; ++k) r.ql[k] = load16_a2(blk + 32 * k + 16 * h);
-        r.qh[0] = load16_a2(blk + 128 + 16 * h);
-        r.qh[1] = load16_a2(blk + 160 + 16 * h);
-        r.sc = load16_a2(blk + 192);
-        r.d = load_u16(blk + 208);
-    };
-
-    ActStage<BM> stage;
-    stage.resolve(tid, [&](int t) { return tiles.act_row(tile_y, BM, t); });
-    stage.fetch(qs, d8, bsums, nb, 0, tid);
-    Raw raw;
-    load_raw(raw, 0);
-    stage.store(lds, tid);
-    __syncthreads();
-
-    for (int b = 0; b < nb; ++b) {
-        const uint8_t* tile = lds + (b & 1) * MmqLds<BM>::bytes;
-        const Raw cur = raw;
-        if (b + 1 < nb) {
-            stage.fetch(qs, d8, bsums, nb, b + 1, tid);
-            load_raw(raw, b + 1);
-        }
-        // ---- this lane's row of block b -> eight B operands (q - 32 as int8) ----
-        v4i bf[8];
-#pragma unroll
-        for (int sb = 0; sb < 8; ++sb) {
-            const int half = sb >> 2, qd = sb & 3;
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const uint32_t nib = ((uint32_t)cur.ql[2 * half + (qd & 1)][k] >> (4 * (qd >> 1))) & 0x0F0F0F0Fu;
-                const uint32_t hb = ((uint32_t)cur.qh[half][k] >> (2 * qd)) & 0x03030303u;
-                bf[sb][k] = (int)((((hb << 4) | nib) + 0x60606060u) ^ 0x80808080u);
-            }
-        }
-        const int scw[4] = {cur.sc.x, cur.sc.y, cur.sc.z, cur.sc.w};
-        const float d = f16_bits_to_f32(cur.d);
-        const v16i zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        v16i isum;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) isum[i] = 0;
-        // the tile's token `col` as MFMA A operand: group 2s multiplies the k < 16 half, 2s+1 the other
-        const uint8_t* arow = tile + MmqLds<BM>::qs_off + col * kActRowBytes + h * 16;
-        const uint8_t* zero = reinterpret_cast<const uint8_t*>(zero16);
-#pragma unroll
-        for (int sb = 0; sb < 8; ++sb) {
-            const v4i a0 = *reinterpret_cast<const v4i*>(h == 0 ? arow + sb * 32 : zero);
-            const v4i a1 = *reinterpret_cast<const v4i*>(h == 1 ? arow + sb * 32 : zero);
-            const v16i r0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, bf[sb], zi, 0, 0, 0);
-            const v16i r1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, bf[sb], zi, 0, 0, 0);
-            const int g0 = 2 * sb, g1 = 2 * sb + 1;
-            const int sc0 = __builtin_amdgcn_sbfe(scw[g0 >> 2], 8 * (g0 & 3), 8);
-            const int sc1 = __builtin_amdgcn_sbfe(scw[g1 >> 2], 8 * (g1 & 3), 8);
-#pragma unroll
-            for (int i = 0; i < 16; ++i) isum[i] += __mul24(r0[i], sc0) + __mul24(r1[i], sc1);
-        }
-        // epilogue: accumulator i of this lane is slot 8*(i/4) + 4*h + i%4 of the tile
-        const float* dtile = reinterpret_cast<const float*>(tile + MmqLds<BM>::d_off) + 4 * h;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const v4f dq = *reinterpret_cast<const v4f*>(dtile + 8 * j);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) acc[4 * j + i] += (d * dq[i]) * (float)isum[4 * j + i];
-        }
-        if (b + 1 < nb) stage.store(lds + ((b + 1) & 1) * MmqLds<BM>::bytes, tid);
-        __syncthreads();
-    }
-
-    if (!row_ok) return;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const int slot = 8 * (r >> 2) + 4 * h + (r & 3);
-        if (slot < n_slots) y[(size_t)tiles.out_row(tile_y, BM, slot) * out_f + wrow] = acc[r];
-    }
-}
-
-void launch_mmq_q6k_gathered(const uint8_t* bank, size_t expert_stride, size_t bpr, const ActQ8& act, int act_div,
-                             const MoeTileTable& t, float* y, size_t in_f, size_t out_f, hipStream_t stream) {
-    const dim3 grid((unsigned)((out_f + 127) / 128), (unsigned)t.max_tiles), block(256);
-    const GatheredTiles g{t.n_tiles, t.expert, t.slot0, t.count, t.perm, expert_stride, act_div};
-    hipLaunchKernelGGL(mmq_q6k_gathered_kernel, grid, block, 0, stream, bank, bpr, act.qs, act.d, act.bsums, y, g,
-                       (int)out_f, (int)(in_f / 256));
 }
 
 void launch_mmq_shared_q6k(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,

@@ -982,21 +982,21 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     if (!gbpr || !ubpr || !dbpr) return "rows >= 2 carries Q4_K / Q5_K / Q6_K / Q8_0 expert banks";
     launch_quantize_q8(b.x, s.rows, s.ne, false, aq, stream);
     const size_t n_act = pairs * s.n_ff, n_out = (size_t)s.rows * s.ne;
-    // Prefill-sized batches: the pairs are bucketed by expert and every Q4_K or Q6_K bank runs its
+    // Prefill-sized batches: the pairs are bucketed by expert and every bank runs its format's
     // int8-MFMA GEMM per (expert, 32 pairs) tile, so an expert's weights are read once per 32 of
     // its pairs instead of once per pair. From an average of `bucket_min` pairs per expert up (the
-    // per-pair GEMVs win below: most tiles would hold one or two pairs). Banks of other formats keep
-    // the per-pair GEMVs.
+    // per-pair GEMVs win below: most tiles would hold one or two pairs).
     static const int bucket_min = getenv("INFR_HIP_MOE_BUCKET_MIN") ? atoi(getenv("INFR_HIP_MOE_BUCKET_MIN")) : 4;
-    // (a Q6_K tile costs more than a Q4_K one: at four pairs per expert its per-pair GEMVs are still
-    // ahead, 199 us against 214 per layer; from eight it is bucketed)
+    // (a Q6_K tile costs more than the others': at four pairs per expert its per-pair GEMVs tie with
+    // the tiles, 313 us per layer either way, and it is bucketed from eight; Q5_K and Q8_0 banks
+    // gain from four on, 179 against 254 and 299 against 399 us)
     auto has_mfma = [&](int dt) {
-        return (dt == 12 && pairs >= (size_t)bucket_min * s.n_expert) || (dt == 14 && pairs >= (size_t)2 * bucket_min * s.n_expert);
+        return ((dt == 12 || dt == 13 || dt == 8) && pairs >= (size_t)bucket_min * s.n_expert) ||
+               (dt == 14 && pairs >= (size_t)2 * bucket_min * s.n_expert);
     };
     auto launch_gathered = [&](int dt, const uint8_t* bank, size_t stride, size_t bpr_, int act_div, const MoeTileTable& t,
                                float* out, size_t in_f, size_t out_f) {
-        if (dt == 12) launch_mmq_q4k_gathered(bank, stride, bpr_, aq, act_div, t, out, in_f, out_f, stream);
-        else launch_mmq_q6k_gathered(bank, stride, bpr_, aq, act_div, t, out, in_f, out_f, stream);
+        (void)launch_mmq_gathered(dt, bank, stride, bpr_, aq, act_div, t, out, in_f, out_f, stream);
     };
     const bool bucketed = bucket_min > 0 && pairs >= (size_t)bucket_min * s.n_expert && pairs <= (size_t)1 << 24 &&
                           (has_mfma(s.gate_dtype) || has_mfma(s.up_dtype) || has_mfma(s.down_dtype));

@@ -221,12 +221,13 @@ def test_moe_qwen3_30b_a3b_prefill(be):
 
 
 @pytest.mark.parametrize("gu,down", [(DType.Q4K, DType.Q6K), (DType.Q6K, DType.Q4K), (DType.Q6K, DType.Q6K),
-                                     (DType.Q4K, DType.Q8_0)])
+                                     (DType.Q4K, DType.Q8_0), (DType.Q5K, DType.Q5K), (DType.Q5K, DType.Q6K),
+                                     (DType.Q8_0, DType.Q8_0)])
 def test_moe_prefill_buckets_with_mixed_bank_formats(be, gu, down):
-    """A Q4_K_M file's mix (Q4_K gate / up beside a Q6_K down bank), its mirror, all-Q6_K, and a bank
-    without a bucketed kernel: Q4_K and Q6_K banks take their bucketed MFMA GEMM, the others the
-    per-pair GEMVs, in one op - and the first two tokens, run again as a batch of two (per-pair
-    GEMVs throughout), give the same bits."""
+    """A Q4_K_M file's mix (Q4_K gate / up beside a Q6_K down bank), its mirror, a Q5_K_M file's mix,
+    and all-Q6_K / Q5_K / Q8_0: every bank takes its format's bucketed MFMA GEMM in one op - and the
+    first two tokens, run again as a batch of two (per-pair GEMVs throughout), give the same bits in
+    the formats whose sums are ordered."""
     rows, ne, n_expert, n_used, nff = 96, 512, 16, 4, 256          # 24 pairs per expert
     gate_w = synth_weight(gu, 201, n_expert * nff, ne, 0.05)
     up_w = synth_weight(gu, 202, n_expert * nff, ne, 0.05)
