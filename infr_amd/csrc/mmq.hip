@@ -602,8 +602,294 @@ static void launch_mmq_skinny_q4k(const uint8_t* w, size_t bpr, const ActQ8& act
                            (const BatchTile*)nullptr);
 }
 
+// ───────────────────────────── up to 16 tokens: 16 x 16 tiles, K split over waves, no exchange of integers ─────────────────────────────
+// Decode batches (2..16 tokens) are bound by memory instructions and by VALU work per weight byte,
+// not by the matrix cores. v_mfma_i32_16x16x64_i8 tiles of 16 tokens x 16 weight rows waste little
+// on absent tokens, and one 64-byte run of a row feeds four lanes: lane (row r, K quarter kq)
+// fetches bytes 64c + 16kq .. + 15 of the block's codes for c = 0, 1 and both nibbles of every byte
+// are operands - the low nibbles of chunk c are one K = 64 step (sub-blocks 4c + 2(kq/2), elements
+// 16(kq%2)..), the high nibbles the next (sub-blocks 4c + 2(kq/2) + 1) - so nothing is fetched
+// twice. A workgroup covers 16 rows (half of a 32-row tile, blockIdx.y) and splits K over its NW
+// waves in contiguous ranges of BPW blocks: a wave asks for all its weight bytes at once, keeps the
+// exact integers (sd, sm) of its blocks in registers, and the f32 epilogue - the CPU's expression,
+// blocks in ascending order - is handed from wave to wave through LDS (four floats per lane,
+// NW - 1 barriers). A block's activations (MT tokens x 256 codes, their per-32 sums) come in with
+// whole-line loads, one block ahead, and pass through a wave-private LDS tile into operand order:
+// fetching the operands lane by lane took twice the memory instructions and kept the address
+// units 80 % busy. The weights take the same route, two blocks (288 contiguous bytes of each of
+// the 16 rows) at a time: neighbouring lanes then fetch neighbouring 16-byte pieces of one row and
+// the loads leave the first-level cache as 64-byte requests, where a lane per row made every
+// request 32 bytes - half of a DRAM burst. Same integers and the same f32 operations in the same
+// order as the kernels above: bit-identical results.
+template <int NW, int BPW, int MT, bool STAGES>
+__global__ __launch_bounds__(NW * 64) void mmq_skinny16_q4k_kernel(
+    const uint8_t* __restrict__ w, size_t bpr, const int8_t* __restrict__ qs,
+    const float* __restrict__ d8, const int32_t* __restrict__ bsums, float* __restrict__ y, int m,
+    int out_f, int nb, int32_t* __restrict__ st_sd, int32_t* __restrict__ st_sm,
+    const BatchTile* __restrict__ tiles) {
+    typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+    constexpr int kTokStride = 256 + 16;            // one token's codes of a block, padded against bank conflicts
+    constexpr int kBsOff = MT * kTokStride;         // [token][8] per-32 sums
+    constexpr int kTileBytes = kBsOff + MT * 32;
+    constexpr int kPh = 2;                          // blocks of weights staged at a time
+    constexpr int kRowStride = kPh * 144 + 16;      // padded: eight rows' 16-byte reads cover all banks
+    constexpr int kChunks = 16 * kPh * 9, kIt = (kChunks + 63) / 64;
+    static_assert(BPW % kPh == 0, "a wave's blocks are whole stages");
+    __shared__ __attribute__((aligned(16))) uint8_t w_l[NW][16 * kRowStride];
+    __shared__ __attribute__((aligned(16))) uint8_t act_l[NW][kTileBytes];
+    __shared__ __attribute__((aligned(16))) float dq_l[NW][MT][BPW];
+    __shared__ __attribute__((aligned(16))) float chain_l[64][4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r16 = lane & 15, kq = lane >> 4, g = kq >> 1, hh = kq & 1;
+    const int rt = blockIdx.y * 16 + r16;  // row inside the 32-row tile
+    const size_t in_f = (size_t)nb * 256;
+    int wrow = blockIdx.x * 32 + rt;
+    bool row_ok = wrow < out_f;
+    bool any_row = (int)blockIdx.x * 32 + (int)blockIdx.y * 16 < out_f;
+    if (tiles) {
+        const BatchTile t = tiles[blockIdx.x];
+        w = t.w;
+        bpr = t.bpr;
+        y = t.y;
+        out_f = (int)t.out_f;
+        wrow = rt;
+        row_ok = rt < (int)t.rows;
+        any_row = (int)blockIdx.y * 16 < (int)t.rows;
+        qs += t.act_elem0;
+        d8 += t.act_elem0 / 256;
+        bsums += t.act_elem0 / 32;
+    }
+    if (!any_row) return;  // uniform over the workgroup, before any barrier
+    const int b0 = wave * BPW;
+    // Weight stage: 16-byte piece q % 18 of row q / 18 of the half tile, q = lane + 64 it; rows past the
+    // matrix repeat the half's first row (their outputs are never stored).
+    const int rows_here = (tiles ? (int)tiles[blockIdx.x].rows : out_f - (int)blockIdx.x * 32) - (int)blockIdx.y * 16;
+    const uint8_t* wbase = w + (size_t)(wrow - r16) * bpr;  // first row of this half
+    uint32_t goff[kIt], loff[kIt];
+#pragma unroll
+    for (int it = 0; it < kIt; ++it) {
+        const int q = min(lane + 64 * it, kChunks - 1);
+        const int row = q / (kPh * 9), piece = q % (kPh * 9);
+        goff[it] = (uint32_t)((row < rows_here ? row : 0) * bpr) + piece * 16;
+        loff[it] = row * kRowStride + piece * 16;
+    }
+    v4i wreg[kIt];
+    auto request_rows = [&](int ph) {
+        const int bs = min(b0 + kPh * ph, nb - kPh);  // past the end: a redundant stage, never used
+#pragma unroll
+        for (int it = 0; it < kIt; ++it)
+            if (lane + 64 * it < kChunks) wreg[it] = load16(wbase + goff[it] + (size_t)bs * 144);
+    };
+    uint8_t* wl = w_l[wave];
+    auto publish_rows = [&]() {
+#pragma unroll
+        for (int it = 0; it < kIt; ++it)
+            if (lane + 64 * it < kChunks) *reinterpret_cast<v4i*>(wl + loff[it]) = wreg[it];
+    };
+    request_rows(0);
+    struct Raw {
+        v4i hdr, q[2];
+    };
+    const uint8_t* wfrag = wl + r16 * kRowStride;
+    // the activation scales of the wave's blocks: dq_l[token][j]
+    for (int i = lane; i < MT * BPW; i += 64) {
+        const int tok = min(i / BPW, m - 1), b = min(b0 + i % BPW, nb - 1);
+        (&dq_l[wave][0][0])[i] = d8[(size_t)tok * nb + b];
+    }
+    // a block's activations: 16-byte piece `chunk & 15` of token `chunk >> 4` (absent tokens repeat the
+    // last one: their products land in accumulators that are never stored)
+    v4i areg[MT / 4], bsreg = {0, 0, 0, 0};
+    auto request_acts = [&](int j) {
+        const int b = min(b0 + j, nb - 1);
+#pragma unroll
+        for (int it = 0; it < MT / 4; ++it) {
+            const int chunk = lane + 64 * it;
+            areg[it] = *reinterpret_cast<const v4i*>(qs + (size_t)min(chunk >> 4, m - 1) * in_f + (size_t)b * 256 + (chunk & 15) * 16);
+        }
+        if (lane < MT * 2)
+            bsreg = *reinterpret_cast<const v4i*>(bsums + (size_t)min(lane >> 1, m - 1) * (nb * 8) + b * 8 + (lane & 1) * 4);
+    };
+    uint8_t* tile = act_l[wave];
+    auto publish_acts = [&]() {
+#pragma unroll
+        for (int it = 0; it < MT / 4; ++it) {
+            const int chunk = lane + 64 * it;
+            *reinterpret_cast<v4i*>(tile + (chunk >> 4) * kTokStride + (chunk & 15) * 16) = areg[it];
+        }
+        if (lane < MT * 2) *reinterpret_cast<v4i*>(tile + kBsOff + lane * 16) = bsreg;
+    };
+    // the wave's lanes exchange data through its own LDS tile: order the tile's writes and reads
+    auto wave_sync = [&]() {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+    request_acts(0);
+    // this lane as A operand: token r16 (rows of absent tokens hold another token's codes)
+    const uint8_t* afrag = tile + (r16 & (MT - 1)) * kTokStride + 16 * hh;
+    const uint8_t* bsfrag = tile + kBsOff + (r16 & (MT - 1)) * 32 + 16 * hh;
+
+    int sd[BPW][4];
+    float sm[BPW][4];
+    uint32_t ddm[BPW];  // (d, dmin) of this lane's row
+#pragma unroll
+    for (int j = 0; j < BPW; ++j) {
+        wave_sync();  // the previous block's operand reads are done
+        publish_acts();
+        if (j + 1 < BPW) request_acts(j + 1);
+        if (j % kPh == 0) {
+            publish_rows();
+            if (j + kPh < BPW) request_rows(j / kPh + 1);
+        }
+        wave_sync();
+        Raw r;
+        r.hdr = *reinterpret_cast<const v4i*>(wfrag + (j % kPh) * 144);
+        r.q[0] = *reinterpret_cast<const v4i*>(wfrag + (j % kPh) * 144 + 16 + 16 * kq);
+        r.q[1] = *reinterpret_cast<const v4i*>(wfrag + (j % kPh) * 144 + 16 + 64 + 16 * kq);
+        ddm[j] = (uint32_t)r.hdr.x;
+        uint32_t sc8[2], mn8[2];
+        k4_all((uint32_t)r.hdr.y, (uint32_t)r.hdr.z, (uint32_t)r.hdr.w, sc8, mn8);
+        v4i alo = {0, 0, 0, 0}, ahi = {0, 0, 0, 0};
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {  // step s: chunk c = s / 2, nibble e = s % 2
+            const int c = s >> 1, e = s & 1;
+            const uint32_t sc = (sc8[c] >> (8 * (2 * g + e))) & 0xFFu;
+            const uint32_t lo3 = sc & 7u, hi3 = sc >> 3;
+            const int qw[4] = {r.q[c].x, r.q[c].y, r.q[c].z, r.q[c].w};
+            v4i blo, bhi;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t codes = ((uint32_t)qw[k] >> (4 * e)) & 0x0F0F0F0Fu;
+                blo[k] = scale_codes(codes, lo3);
+                bhi[k] = scale_codes(codes, hi3);
+            }
+            const v4i a = *reinterpret_cast<const v4i*>(afrag + (4 * c + 2 * g + e) * 32);
+            alo = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, blo, alo, 0, 0, 0);
+            ahi = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bhi, ahi, 0, 0, 0);
+        }
+        // sm: K = 16 slots = (bsum & 63 | the rest) x sub-blocks 0..7; this lane carries slots 4kq..4kq+3,
+        // sub-blocks 4hh..4hh+3 of part g
+        const uint32_t mnw = mn8[hh];
+        const v4h bm = {(_Float16)(int)(mnw & 0xFFu), (_Float16)(int)((mnw >> 8) & 0xFFu),
+                        (_Float16)(int)((mnw >> 16) & 0xFFu), (_Float16)(int)(mnw >> 24)};
+        const v4i bs = *reinterpret_cast<const v4i*>(bsfrag);
+        const int bsv[4] = {bs.x, bs.y, bs.z, bs.w};
+        v4h abs_;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int lo = bsv[k] & 63;
+            abs_[k] = (_Float16)(g ? bsv[k] - lo : lo);
+        }
+        const v4f smf = __builtin_amdgcn_mfma_f32_16x16x16f16(abs_, bm, v4f{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            sd[j][i] = alo[i] + (ahi[i] << 3);
+            sm[j][i] = smf[i];
+            if (STAGES) {
+                const int tok = 4 * kq + i;
+                if (row_ok && tok < m && b0 + j < nb) {
+                    st_sd[((size_t)tok * out_f + wrow) * nb + b0 + j] = sd[j][i];
+                    st_sm[((size_t)tok * out_f + wrow) * nb + b0 + j] = (int)smf[i];
+                }
+            }
+        }
+    }
+    wave_sync();  // dq_l was written by this wave's lanes
+
+    // f32 epilogue handed down the waves: sumf += q8.d[b] * (d * sd as f32 - dmin * sm as f32), b ascending;
+    // this lane's accumulators are tokens 4kq .. 4kq + 3 of row r16
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int k = 0; k < NW; ++k) {
+        if (wave == k) {
+            if (k > 0) {
+                const v4f prev = *reinterpret_cast<const v4f*>(&chain_l[lane][0]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[i] = prev[i];
+            }
+#pragma unroll
+            for (int j = 0; j < BPW; ++j) {
+                if (b0 + j < nb) {
+                    const float d = f16_bits_to_f32(ddm[j] & 0xFFFFu);
+                    const float dmin = f16_bits_to_f32(ddm[j] >> 16);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float dq = dq_l[wave][(4 * kq + i) & (MT - 1)][j];
+                        acc[i] += dq * (d * (float)sd[j][i] - dmin * sm[j][i]);
+                    }
+                }
+            }
+            if (k + 1 < NW) *reinterpret_cast<v4f*>(&chain_l[lane][0]) = v4f{acc[0], acc[1], acc[2], acc[3]};
+        }
+        if (k + 1 < NW) __syncthreads();
+    }
+    if (wave != NW - 1 || !row_ok) return;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int tok = 4 * kq + i;
+        if (tok < m) gstore<float>(y + (size_t)tok * out_f + wrow, acc[i]);
+    }
+}
+
+// Waves per workgroup and blocks per wave for rows of nb blocks; false: the older kernel takes them.
+static bool skinny16_shape(int nb, int* nw, int* bpw) {
+    static const int env_nw = getenv("INFR_HIP_SKINNY16_WAVES") ? atoi(getenv("INFR_HIP_SKINNY16_WAVES")) : 0;
+    int n = env_nw ? env_nw : (nb <= 16 ? 4 : 8);
+    if (n != 4 && n != 8) n = 8;
+    if (nb < 2 || nb % 2 != 0) return false;  // weights are staged two blocks at a time
+    int per = (nb + n - 1) / n;
+    per = per <= 2 ? 2 : (per + 1) / 2 * 2;
+    if (per > 8) return false;
+    *nw = n;
+    *bpw = per;
+    return true;
+}
+
+template <bool STAGES>
+static bool launch_mmq_skinny16(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
+                                size_t out_f, size_t wgs, const IntStages& st, const BatchTile* tiles,
+                                hipStream_t stream) {
+    const int nb = (int)(in_f / 256);
+    int nw = 0, bpw = 0;
+    if (m > 16 || !skinny16_shape(nb, &nw, &bpw)) return false;
+    const dim3 grid((unsigned)wgs, 2);
+#define INFR_S16(NW_, BPW_, MT_)                                                                              \
+    hipLaunchKernelGGL((mmq_skinny16_q4k_kernel<NW_, BPW_, MT_, STAGES>), grid, dim3(NW_ * 64), 0, stream, w, bpr, \
+                       act.qs, act.d, act.bsums, y, (int)m, (int)out_f, nb, st.a, st.b, tiles)
+    if (nw == 4 && m <= 8) {
+        switch (bpw) {
+        case 2: INFR_S16(4, 2, 8); break;
+        case 4: INFR_S16(4, 4, 8); break;
+        case 6: INFR_S16(4, 6, 8); break;
+        default: INFR_S16(4, 8, 8); break;
+        }
+    } else if (nw == 4) {
+        switch (bpw) {
+        case 2: INFR_S16(4, 2, 16); break;
+        case 4: INFR_S16(4, 4, 16); break;
+        case 6: INFR_S16(4, 6, 16); break;
+        default: INFR_S16(4, 8, 16); break;
+        }
+    } else if (m <= 8) {
+        switch (bpw) {
+        case 2: INFR_S16(8, 2, 8); break;
+        case 4: INFR_S16(8, 4, 8); break;
+        case 6: INFR_S16(8, 6, 8); break;
+        default: INFR_S16(8, 8, 8); break;
+        }
+    } else {
+        return false;  // eight waves with 16-token tiles would need more than 64 KB of LDS
+    }
+#undef INFR_S16
+    return true;
+}
+
 void launch_mmq_skinny_group(size_t m, size_t in_f, const BatchTile* tiles_dev, const BatchGroupPlan& plan,
                              const ActQ8& act, hipStream_t stream) {
+    static const int env_s16_max = getenv("INFR_HIP_SKINNY16_MAX_M") ? atoi(getenv("INFR_HIP_SKINNY16_MAX_M")) : 16;
+    if ((int)m <= env_s16_max &&
+        launch_mmq_skinny16<false>(nullptr, 0, act, nullptr, m, in_f, 0, plan.total_wgs, IntStages{}, tiles_dev, stream))
+        return;
     const dim3 grid((unsigned)plan.total_wgs, (unsigned)((m + 31) / 32));
     const int nb = (int)(in_f / 256);
     if (plan.waves == 8)
@@ -701,6 +987,13 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
     launch_quantize_q8(x, m, in_f, act_is_per32(dtype, in_f), act, stream);
     static const int env_dot4_max = getenv("INFR_HIP_Q4K_DOT4_MAX_M") ? atoi(getenv("INFR_HIP_Q4K_DOT4_MAX_M")) : 0;
     if (dtype != 12 || (int)m <= env_dot4_max) return launch_gemv_batch(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
+    static const int env_s16_max = getenv("INFR_HIP_SKINNY16_MAX_M") ? atoi(getenv("INFR_HIP_SKINNY16_MAX_M")) : 16;
+    if ((int)m <= env_s16_max) {
+        const size_t wgs = (out_f + 31) / 32;
+        if (st.a ? launch_mmq_skinny16<true>(w, bpr, act, y, m, in_f, out_f, wgs, st, nullptr, stream)
+                 : launch_mmq_skinny16<false>(w, bpr, act, y, m, in_f, out_f, wgs, st, nullptr, stream))
+            return true;
+    }
     if ((int)m <= env_skinny_max) {
         // four blocks per round; eight for long rows or when four would leave most SIMDs without a wave
         const size_t wgs = (out_f + 31) / 32 * ((m + 31) / 32);
