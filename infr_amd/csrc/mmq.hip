@@ -631,10 +631,9 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_q4k_kernel(
     constexpr int kTokStride = 256 + 16;            // one token's codes of a block, padded against bank conflicts
     constexpr int kBsOff = MT * kTokStride;         // [token][8] per-32 sums
     constexpr int kTileBytes = kBsOff + MT * 32;
-    constexpr int kPh = 2;                          // blocks of weights staged at a time
+    constexpr int kPh = BPW;                        // blocks of weights staged at a time: the wave's share of a pass
     constexpr int kRowStride = kPh * 144 + 16;      // padded: eight rows' 16-byte reads cover all banks
-    constexpr int kChunks = 16 * kPh * 9, kIt = (kChunks + 63) / 64;
-    static_assert(BPW % kPh == 0, "a wave's blocks are whole stages");
+    constexpr int kPieces = kPh * 9, kIt = (kPieces + 3) / 4;  // 16-byte pieces of a row's stage
     __shared__ __attribute__((aligned(16))) uint8_t w_l[NW][16 * kRowStride];
     __shared__ __attribute__((aligned(16))) uint8_t act_l[NW][kTileBytes];
     __shared__ __attribute__((aligned(16))) float dq_l[NW][MT][BPW];
@@ -660,54 +659,48 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_q4k_kernel(
         bsums += t.act_elem0 / 32;
     }
     if (!any_row) return;  // uniform over the workgroup, before any barrier
-    const int b0 = wave * BPW;
-    // Weight stage: 16-byte piece q % 18 of row q / 18 of the half tile, q = lane + 64 it; rows past the
-    // matrix repeat the half's first row (their outputs are never stored).
+    // K in passes of NW * BPW blocks; in a pass wave w owns blocks (pass * NW + w) * BPW .. + BPW - 1
+    const int n_pass = (nb + NW * BPW - 1) / (NW * BPW);
+    // Weight stage: lane (row = lane / 4, pq = lane % 4) takes the 16-byte pieces pq, pq + 4, .. of its
+    // row's BPW blocks - a quad of lanes fetches 64 contiguous bytes - so every address is one
+    // per-lane offset plus a constant; rows past the matrix repeat the half's first row (their
+    // outputs are never stored).
     const int rows_here = (tiles ? (int)tiles[blockIdx.x].rows : out_f - (int)blockIdx.x * 32) - (int)blockIdx.y * 16;
     const uint8_t* wbase = w + (size_t)(wrow - r16) * bpr;  // first row of this half
-    uint32_t goff[kIt], loff[kIt];
-#pragma unroll
-    for (int it = 0; it < kIt; ++it) {
-        const int q = min(lane + 64 * it, kChunks - 1);
-        const int row = q / (kPh * 9), piece = q % (kPh * 9);
-        goff[it] = (uint32_t)((row < rows_here ? row : 0) * bpr) + piece * 16;
-        loff[it] = row * kRowStride + piece * 16;
-    }
+    const int srow = lane >> 2, pq = lane & 3;
+    const uint32_t goff = (uint32_t)((srow < rows_here ? srow : 0) * bpr) + pq * 16;
+    const uint32_t loff = srow * kRowStride + pq * 16;
     v4i wreg[kIt];
-    auto request_rows = [&](int ph) {
-        const int bs = min(b0 + kPh * ph, nb - kPh);  // past the end: a redundant stage, never used
+    auto request_rows = [&](int b) {  // blocks b .. b + BPW - 1; past the end: a redundant stage, never used
+        const uint8_t* src = wbase + (size_t)min(b, nb - kPh) * 144;
 #pragma unroll
         for (int it = 0; it < kIt; ++it)
-            if (lane + 64 * it < kChunks) wreg[it] = load16(wbase + goff[it] + (size_t)bs * 144);
+            if (pq + 4 * it < kPieces) wreg[it] = load16(src + goff + 64 * it);
     };
     uint8_t* wl = w_l[wave];
     auto publish_rows = [&]() {
 #pragma unroll
         for (int it = 0; it < kIt; ++it)
-            if (lane + 64 * it < kChunks) *reinterpret_cast<v4i*>(wl + loff[it]) = wreg[it];
+            if (pq + 4 * it < kPieces) *reinterpret_cast<v4i*>(wl + loff + 64 * it) = wreg[it];
     };
-    request_rows(0);
     struct Raw {
         v4i hdr, q[2];
     };
     const uint8_t* wfrag = wl + r16 * kRowStride;
-    // the activation scales of the wave's blocks: dq_l[token][j]
-    for (int i = lane; i < MT * BPW; i += 64) {
-        const int tok = min(i / BPW, m - 1), b = min(b0 + i % BPW, nb - 1);
-        (&dq_l[wave][0][0])[i] = d8[(size_t)tok * nb + b];
-    }
     // a block's activations: 16-byte piece `chunk & 15` of token `chunk >> 4` (absent tokens repeat the
     // last one: their products land in accumulators that are never stored)
     v4i areg[MT / 4], bsreg = {0, 0, 0, 0};
-    auto request_acts = [&](int j) {
-        const int b = min(b0 + j, nb - 1);
+    uint32_t aoff[MT / 4];
 #pragma unroll
-        for (int it = 0; it < MT / 4; ++it) {
-            const int chunk = lane + 64 * it;
-            areg[it] = *reinterpret_cast<const v4i*>(qs + (size_t)min(chunk >> 4, m - 1) * in_f + (size_t)b * 256 + (chunk & 15) * 16);
-        }
-        if (lane < MT * 2)
-            bsreg = *reinterpret_cast<const v4i*>(bsums + (size_t)min(lane >> 1, m - 1) * (nb * 8) + b * 8 + (lane & 1) * 4);
+    for (int it = 0; it < MT / 4; ++it) aoff[it] = (uint32_t)min((lane >> 4) + 4 * it, m - 1) * (uint32_t)in_f + (lane & 15) * 16;
+    const uint32_t boff = (uint32_t)min(lane >> 1, m - 1) * (uint32_t)(nb * 32) + (lane & 1) * 16;
+    auto request_acts = [&](int b_) {
+        const int b = min(b_, nb - 1);
+        const int8_t* src = qs + (size_t)b * 256;
+        const uint8_t* bsrc = reinterpret_cast<const uint8_t*>(bsums) + (size_t)b * 32;
+#pragma unroll
+        for (int it = 0; it < MT / 4; ++it) areg[it] = *reinterpret_cast<const v4i*>(src + aoff[it]);
+        if (lane < MT * 2) bsreg = *reinterpret_cast<const v4i*>(bsrc + boff);
     };
     uint8_t* tile = act_l[wave];
     auto publish_acts = [&]() {
@@ -718,110 +711,129 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_q4k_kernel(
         }
         if (lane < MT * 2) *reinterpret_cast<v4i*>(tile + kBsOff + lane * 16) = bsreg;
     };
-    // the wave's lanes exchange data through its own LDS tile: order the tile's writes and reads
+    // the wave's lanes exchange data through its own LDS tiles: order the tiles' writes and reads
     auto wave_sync = [&]() {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     };
-    request_acts(0);
     // this lane as A operand: token r16 (rows of absent tokens hold another token's codes)
     const uint8_t* afrag = tile + (r16 & (MT - 1)) * kTokStride + 16 * hh;
     const uint8_t* bsfrag = tile + kBsOff + (r16 & (MT - 1)) * 32 + 16 * hh;
 
-    int sd[BPW][4];
-    float sm[BPW][4];
-    uint32_t ddm[BPW];  // (d, dmin) of this lane's row
+    uint32_t dqoff[(MT * BPW + 63) / 64];
 #pragma unroll
-    for (int j = 0; j < BPW; ++j) {
-        wave_sync();  // the previous block's operand reads are done
-        publish_acts();
-        if (j + 1 < BPW) request_acts(j + 1);
-        if (j % kPh == 0) {
-            publish_rows();
-            if (j + kPh < BPW) request_rows(j / kPh + 1);
+    for (int it = 0; it < (MT * BPW + 63) / 64; ++it) {
+        const int i = lane + 64 * it;
+        dqoff[it] = (uint32_t)min(i / BPW, m - 1) * (uint32_t)nb + i % BPW;
+    }
+    request_rows(wave * BPW);
+    request_acts(wave * BPW);
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // this lane's outputs: tokens 4kq .. 4kq + 3 of row r16
+    for (int pass = 0; pass < n_pass; ++pass) {
+        const int b0 = (pass * NW + wave) * BPW;
+        const int b0_next = b0 + NW * BPW;  // next pass (past the end: clamped, never used)
+        // the activation scales of the wave's blocks: dq_l[token][j]
+        {
+            const float* dsrc = d8 + min(b0, nb - BPW);
+#pragma unroll
+            for (int it = 0; it < (MT * BPW + 63) / 64; ++it)
+                if (lane + 64 * it < MT * BPW) (&dq_l[wave][0][0])[lane + 64 * it] = dsrc[dqoff[it]];
         }
-        wave_sync();
-        Raw r;
-        r.hdr = *reinterpret_cast<const v4i*>(wfrag + (j % kPh) * 144);
-        r.q[0] = *reinterpret_cast<const v4i*>(wfrag + (j % kPh) * 144 + 16 + 16 * kq);
-        r.q[1] = *reinterpret_cast<const v4i*>(wfrag + (j % kPh) * 144 + 16 + 64 + 16 * kq);
-        ddm[j] = (uint32_t)r.hdr.x;
-        uint32_t sc8[2], mn8[2];
-        k4_all((uint32_t)r.hdr.y, (uint32_t)r.hdr.z, (uint32_t)r.hdr.w, sc8, mn8);
-        v4i alo = {0, 0, 0, 0}, ahi = {0, 0, 0, 0};
+        int sd[BPW][4];
+        float sm[BPW][4];
+        uint32_t ddm[BPW];  // (d, dmin) of this lane's row
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {  // step s: chunk c = s / 2, nibble e = s % 2
-            const int c = s >> 1, e = s & 1;
-            const uint32_t sc = (sc8[c] >> (8 * (2 * g + e))) & 0xFFu;
-            const uint32_t lo3 = sc & 7u, hi3 = sc >> 3;
-            const int qw[4] = {r.q[c].x, r.q[c].y, r.q[c].z, r.q[c].w};
-            v4i blo, bhi;
+        for (int j = 0; j < BPW; ++j) {
+            wave_sync();  // the previous block's operand reads are done
+            publish_acts();
+            if (j + 1 < BPW) request_acts(b0 + j + 1);
+            else if (pass + 1 < n_pass) request_acts(b0_next);
+            if (j == 0) {
+                publish_rows();
+                if (pass + 1 < n_pass) request_rows(b0_next);
+            }
+            wave_sync();
+            Raw r;
+            r.hdr = *reinterpret_cast<const v4i*>(wfrag + (j % kPh) * 144);
+            r.q[0] = *reinterpret_cast<const v4i*>(wfrag + (j % kPh) * 144 + 16 + 16 * kq);
+            r.q[1] = *reinterpret_cast<const v4i*>(wfrag + (j % kPh) * 144 + 16 + 64 + 16 * kq);
+            ddm[j] = (uint32_t)r.hdr.x;
+            uint32_t sc8[2], mn8[2];
+            k4_all((uint32_t)r.hdr.y, (uint32_t)r.hdr.z, (uint32_t)r.hdr.w, sc8, mn8);
+            v4i alo = {0, 0, 0, 0}, ahi = {0, 0, 0, 0};
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {  // step s: chunk c = s / 2, nibble e = s % 2
+                const int c = s >> 1, e = s & 1;
+                const uint32_t sc = (sc8[c] >> (8 * (2 * g + e))) & 0xFFu;
+                const uint32_t lo3 = sc & 7u, hi3 = sc >> 3;
+                const int qw[4] = {r.q[c].x, r.q[c].y, r.q[c].z, r.q[c].w};
+                v4i blo, bhi;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t codes = ((uint32_t)qw[k] >> (4 * e)) & 0x0F0F0F0Fu;
+                    blo[k] = scale_codes(codes, lo3);
+                    bhi[k] = scale_codes(codes, hi3);
+                }
+                const v4i a = *reinterpret_cast<const v4i*>(afrag + (4 * c + 2 * g + e) * 32);
+                alo = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, blo, alo, 0, 0, 0);
+                ahi = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bhi, ahi, 0, 0, 0);
+            }
+            // sm: K = 16 slots = (bsum & 63 | the rest) x sub-blocks 0..7; this lane carries slots
+            // 4kq..4kq+3, sub-blocks 4hh..4hh+3 of part g
+            const uint32_t mnw = mn8[hh];
+            const v4h bm = {(_Float16)(int)(mnw & 0xFFu), (_Float16)(int)((mnw >> 8) & 0xFFu),
+                            (_Float16)(int)((mnw >> 16) & 0xFFu), (_Float16)(int)(mnw >> 24)};
+            const v4i bs = *reinterpret_cast<const v4i*>(bsfrag);
+            const int bsv[4] = {bs.x, bs.y, bs.z, bs.w};
+            v4h abs_;
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
-                const uint32_t codes = ((uint32_t)qw[k] >> (4 * e)) & 0x0F0F0F0Fu;
-                blo[k] = scale_codes(codes, lo3);
-                bhi[k] = scale_codes(codes, hi3);
+                const int lo = bsv[k] & 63;
+                abs_[k] = (_Float16)(g ? bsv[k] - lo : lo);
             }
-            const v4i a = *reinterpret_cast<const v4i*>(afrag + (4 * c + 2 * g + e) * 32);
-            alo = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, blo, alo, 0, 0, 0);
-            ahi = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bhi, ahi, 0, 0, 0);
-        }
-        // sm: K = 16 slots = (bsum & 63 | the rest) x sub-blocks 0..7; this lane carries slots 4kq..4kq+3,
-        // sub-blocks 4hh..4hh+3 of part g
-        const uint32_t mnw = mn8[hh];
-        const v4h bm = {(_Float16)(int)(mnw & 0xFFu), (_Float16)(int)((mnw >> 8) & 0xFFu),
-                        (_Float16)(int)((mnw >> 16) & 0xFFu), (_Float16)(int)(mnw >> 24)};
-        const v4i bs = *reinterpret_cast<const v4i*>(bsfrag);
-        const int bsv[4] = {bs.x, bs.y, bs.z, bs.w};
-        v4h abs_;
+            const v4f smf = __builtin_amdgcn_mfma_f32_16x16x16f16(abs_, bm, v4f{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const int lo = bsv[k] & 63;
-            abs_[k] = (_Float16)(g ? bsv[k] - lo : lo);
-        }
-        const v4f smf = __builtin_amdgcn_mfma_f32_16x16x16f16(abs_, bm, v4f{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            sd[j][i] = alo[i] + (ahi[i] << 3);
-            sm[j][i] = smf[i];
-            if (STAGES) {
-                const int tok = 4 * kq + i;
-                if (row_ok && tok < m && b0 + j < nb) {
-                    st_sd[((size_t)tok * out_f + wrow) * nb + b0 + j] = sd[j][i];
-                    st_sm[((size_t)tok * out_f + wrow) * nb + b0 + j] = (int)smf[i];
-                }
-            }
-        }
-    }
-    wave_sync();  // dq_l was written by this wave's lanes
-
-    // f32 epilogue handed down the waves: sumf += q8.d[b] * (d * sd as f32 - dmin * sm as f32), b ascending;
-    // this lane's accumulators are tokens 4kq .. 4kq + 3 of row r16
-    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-    for (int k = 0; k < NW; ++k) {
-        if (wave == k) {
-            if (k > 0) {
-                const v4f prev = *reinterpret_cast<const v4f*>(&chain_l[lane][0]);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[i] = prev[i];
-            }
-#pragma unroll
-            for (int j = 0; j < BPW; ++j) {
-                if (b0 + j < nb) {
-                    const float d = f16_bits_to_f32(ddm[j] & 0xFFFFu);
-                    const float dmin = f16_bits_to_f32(ddm[j] >> 16);
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const float dq = dq_l[wave][(4 * kq + i) & (MT - 1)][j];
-                        acc[i] += dq * (d * (float)sd[j][i] - dmin * sm[j][i]);
+            for (int i = 0; i < 4; ++i) {
+                sd[j][i] = alo[i] + (ahi[i] << 3);
+                sm[j][i] = smf[i];
+                if (STAGES) {
+                    const int tok = 4 * kq + i;
+                    if (row_ok && tok < m && b0 + j < nb) {
+                        st_sd[((size_t)tok * out_f + wrow) * nb + b0 + j] = sd[j][i];
+                        st_sm[((size_t)tok * out_f + wrow) * nb + b0 + j] = (int)smf[i];
                     }
                 }
             }
-            if (k + 1 < NW) *reinterpret_cast<v4f*>(&chain_l[lane][0]) = v4f{acc[0], acc[1], acc[2], acc[3]};
         }
-        if (k + 1 < NW) __syncthreads();
+        wave_sync();  // dq_l was written by this wave's lanes
+
+        // f32 epilogue handed down the waves: sumf += q8.d[b] * (d * sd as f32 - dmin * sm as f32), b ascending
+#pragma unroll
+        for (int k = 0; k < NW; ++k) {
+            if (wave == k) {
+                if (k > 0 || pass > 0) {
+                    const v4f prev = *reinterpret_cast<const v4f*>(&chain_l[lane][0]);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[i] = prev[i];
+                }
+#pragma unroll
+                for (int j = 0; j < BPW; ++j) {
+                    if (b0 + j < nb) {
+                        const float d = f16_bits_to_f32(ddm[j] & 0xFFFFu);
+                        const float dmin = f16_bits_to_f32(ddm[j] >> 16);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const float dq = dq_l[wave][(4 * kq + i) & (MT - 1)][j];
+                            acc[i] += dq * (d * (float)sd[j][i] - dmin * sm[j][i]);
+                        }
+                    }
+                }
+                if (k + 1 < NW || pass + 1 < n_pass)
+                    *reinterpret_cast<v4f*>(&chain_l[lane][0]) = v4f{acc[0], acc[1], acc[2], acc[3]};
+            }
+            if (k + 1 < NW || pass + 1 < n_pass) __syncthreads();
+        }
     }
     if (wave != NW - 1 || !row_ok) return;
 #pragma unroll
@@ -831,17 +843,19 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_q4k_kernel(
     }
 }
 
-// Waves per workgroup and blocks per wave for rows of nb blocks; false: the older kernel takes them.
-static bool skinny16_shape(int nb, int* nw, int* bpw) {
+// Waves per workgroup and blocks per wave and pass for rows of nb blocks; false: the older kernel takes them.
+static bool skinny16_shape(int nb, size_t m, int* nw, int* bpw) {
     static const int env_nw = getenv("INFR_HIP_SKINNY16_WAVES") ? atoi(getenv("INFR_HIP_SKINNY16_WAVES")) : 0;
-    int n = env_nw ? env_nw : (nb <= 16 ? 4 : 8);
-    if (n != 4 && n != 8) n = 8;
-    if (nb < 2 || nb % 2 != 0) return false;  // weights are staged two blocks at a time
-    int per = (nb + n - 1) / n;
-    per = per <= 2 ? 2 : (per + 1) / 2 * 2;
-    if (per > 8) return false;
+    static const int env_bpw = getenv("INFR_HIP_SKINNY16_BLOCKS") ? atoi(getenv("INFR_HIP_SKINNY16_BLOCKS")) : 0;
+    if (m > 16) return false;
+    int n = env_nw == 8 ? 8 : 4;
+    if (m > 8) n = 4;  // eight waves with 16-token tiles would need more than 64 KB of LDS
     *nw = n;
-    *bpw = per;
+    // (four blocks per wave and pass - 576-byte, 64-byte-aligned runs per row - measured 20-25 % slower:
+    // a wave then computes for longer before it asks for more)
+    *bpw = env_bpw == 2 || env_bpw == 4 ? env_bpw : 2;
+    if (nb % 4 != 0) *bpw = 2;
+    if (nb < *bpw || nb % *bpw != 0) return false;  // weights are staged BPW blocks at a time
     return true;
 }
 
@@ -851,34 +865,20 @@ static bool launch_mmq_skinny16(const uint8_t* w, size_t bpr, const ActQ8& act, 
                                 hipStream_t stream) {
     const int nb = (int)(in_f / 256);
     int nw = 0, bpw = 0;
-    if (m > 16 || !skinny16_shape(nb, &nw, &bpw)) return false;
+    if (!skinny16_shape(nb, m, &nw, &bpw)) return false;
     const dim3 grid((unsigned)wgs, 2);
 #define INFR_S16(NW_, BPW_, MT_)                                                                              \
     hipLaunchKernelGGL((mmq_skinny16_q4k_kernel<NW_, BPW_, MT_, STAGES>), grid, dim3(NW_ * 64), 0, stream, w, bpr, \
                        act.qs, act.d, act.bsums, y, (int)m, (int)out_f, nb, st.a, st.b, tiles)
     if (nw == 4 && m <= 8) {
-        switch (bpw) {
-        case 2: INFR_S16(4, 2, 8); break;
-        case 4: INFR_S16(4, 4, 8); break;
-        case 6: INFR_S16(4, 6, 8); break;
-        default: INFR_S16(4, 8, 8); break;
-        }
+        if (bpw == 2) INFR_S16(4, 2, 8);
+        else INFR_S16(4, 4, 8);
     } else if (nw == 4) {
-        switch (bpw) {
-        case 2: INFR_S16(4, 2, 16); break;
-        case 4: INFR_S16(4, 4, 16); break;
-        case 6: INFR_S16(4, 6, 16); break;
-        default: INFR_S16(4, 8, 16); break;
-        }
-    } else if (m <= 8) {
-        switch (bpw) {
-        case 2: INFR_S16(8, 2, 8); break;
-        case 4: INFR_S16(8, 4, 8); break;
-        case 6: INFR_S16(8, 6, 8); break;
-        default: INFR_S16(8, 8, 8); break;
-        }
+        if (bpw == 2) INFR_S16(4, 2, 16);
+        else INFR_S16(4, 4, 16);
     } else {
-        return false;  // eight waves with 16-token tiles would need more than 64 KB of LDS
+        if (bpw == 2) INFR_S16(8, 2, 8);
+        else INFR_S16(8, 4, 8);
     }
 #undef INFR_S16
     return true;
