@@ -205,11 +205,13 @@ static bool runs_alone(int dtype, size_t m, size_t in_f) {
     return infr::gemv_takes_f32_activations(dtype, m) || infr::gemv_row_too_long(dtype, in_f);
 }
 
-// Ops that run in small-batch groups inside plans: the K-split MFMA kernel takes Q4_K up to 32
-// rows, the dot4 batch kernel the other formats up to 8.
+// Ops that run in small-batch groups inside plans: the K-split MFMA kernels take Q4_K up to 32
+// rows and Q5_K up to 16 (rows of an even number of blocks), the dot4 batch kernel the other
+// formats up to 8.
 static bool small_batch(const infr_hip_op_t& op) {
-    return op.m >= 2 && op.m <= (op.w_dtype == INFR_DTYPE_Q4_K ? 32u : 8u) &&
-           !infr::gemv_row_too_long(op.w_dtype, op.in_f);
+    if (op.m < 2 || infr::gemv_row_too_long(op.w_dtype, op.in_f)) return false;
+    if (op.w_dtype == INFR_DTYPE_Q4_K) return op.m <= 32;
+    return op.m <= 8 || infr::mmq_skinny16_takes(op.w_dtype, op.m, op.in_f);
 }
 
 // (Re)allocates a device table when it grew and enqueues the copy on the backend stream.
@@ -1127,7 +1129,7 @@ static int enqueue_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t
             infr::launch_quantize_q8_group(plan->qtiles_dev + st.qtile_first, st.qtile_n, act_per32(st.dtype, st.in_f),
                                            be->act, be->stream);
             if (st.bp.kind == 1)
-                infr::launch_mmq_skinny_group(st.m, st.in_f, plan->btiles_dev + st.tile_first, st.bp, be->act,
+                infr::launch_mmq_skinny_group(st.dtype, st.m, st.in_f, plan->btiles_dev + st.tile_first, st.bp, be->act,
                                               be->stream);
             else if (!infr::launch_gemv_batch_group(st.dtype, st.m, st.in_f, plan->btiles_dev + st.tile_first,
                                                     st.bp, be->act, be->stream))

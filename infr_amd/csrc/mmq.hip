@@ -621,25 +621,129 @@ static void launch_mmq_skinny_q4k(const uint8_t* w, size_t bpr, const ActQ8& act
 // the loads leave the first-level cache as 64-byte requests, where a lane per row made every
 // request 32 bytes - half of a DRAM burst. Same integers and the same f32 operations in the same
 // order as the kernels above: bit-identical results.
-template <int NW, int BPW, int MT, bool STAGES>
-__global__ __launch_bounds__(NW * 64) void mmq_skinny16_q4k_kernel(
+//
+// The format supplies one block's integers: block() reads this lane's row (weight row r16 of the
+// half tile, staged in LDS), token r16's codes and per-32 sums as A operands, and returns
+// sd = sum_s sc_s * (q . q8) and sm = sum_s m_s * bsum_s for tokens 4kq .. 4kq + 3 of row r16.
+struct Skinny16Q4K {
+    static constexpr int kBlockBytes = 144;
+    // Q4_K: the scale split sc = 8 hi + lo folded into two operand sets, two chains of four K = 64 steps
+    __device__ static void block(const uint8_t* wblk, const uint8_t* arow, const uint8_t* bsrow, int kq,
+                                 int (&sd)[4], float (&sm)[4], uint32_t& ddm) {
+        typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+        const int g = kq >> 1, hh = kq & 1;
+        const v4i hdr = *reinterpret_cast<const v4i*>(wblk);
+        v4i q[2];
+        q[0] = *reinterpret_cast<const v4i*>(wblk + 16 + 16 * kq);
+        q[1] = *reinterpret_cast<const v4i*>(wblk + 16 + 64 + 16 * kq);
+        ddm = (uint32_t)hdr.x;
+        uint32_t sc8[2], mn8[2];
+        k4_all((uint32_t)hdr.y, (uint32_t)hdr.z, (uint32_t)hdr.w, sc8, mn8);
+        v4i alo = {0, 0, 0, 0}, ahi = {0, 0, 0, 0};
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {  // step s: chunk c = s / 2, nibble e = s % 2
+            const int c = s >> 1, e = s & 1;
+            const uint32_t sc = (sc8[c] >> (8 * (2 * g + e))) & 0xFFu;
+            const uint32_t lo3 = sc & 7u, hi3 = sc >> 3;
+            const int qw[4] = {q[c].x, q[c].y, q[c].z, q[c].w};
+            v4i blo, bhi;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t codes = ((uint32_t)qw[k] >> (4 * e)) & 0x0F0F0F0Fu;
+                blo[k] = scale_codes(codes, lo3);
+                bhi[k] = scale_codes(codes, hi3);
+            }
+            const v4i a = *reinterpret_cast<const v4i*>(arow + (4 * c + 2 * g + e) * 32 + 16 * hh);
+            alo = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, blo, alo, 0, 0, 0);
+            ahi = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bhi, ahi, 0, 0, 0);
+        }
+        const v4f smf = mins_dot_sums(mn8[hh], bsrow, g, hh);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            sd[i] = alo[i] + (ahi[i] << 3);
+            sm[i] = smf[i];
+        }
+    }
+    // sm as a K = 16 f16 product: slots = (bsum & 63 | the rest) x sub-blocks 0..7; lane (., kq) carries
+    // slots 4kq..4kq+3: sub-blocks 4hh..4hh+3 (their mins are the bytes of `mnw`) of part g
+    __device__ static v4f mins_dot_sums(uint32_t mnw, const uint8_t* bsrow, int g, int hh) {
+        typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+        const v4h bm = {(_Float16)(int)(mnw & 0xFFu), (_Float16)(int)((mnw >> 8) & 0xFFu),
+                        (_Float16)(int)((mnw >> 16) & 0xFFu), (_Float16)(int)(mnw >> 24)};
+        const v4i bs = *reinterpret_cast<const v4i*>(bsrow + 16 * hh);
+        const int bsv[4] = {bs.x, bs.y, bs.z, bs.w};
+        v4h abs_;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int lo = bsv[k] & 63;
+            abs_[k] = (_Float16)(g ? bsv[k] - lo : lo);
+        }
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(abs_, bm, v4f{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+    }
+};
+
+// Q5_K (176-byte block: d, dmin, scales[12], qh[32], qs[128]; crates/infr-cpu/src/kernels.rs q5_k dot):
+// a 5-bit code times a 6-bit scale has no int8 split of two digits, so a sub-block is one
+// v_mfma_i32_16x16x32_i8 (lane (., kq): elements 8kq .. 8kq + 7) scaled into sd by a 24-bit
+// multiply-add; sm and the epilogue are Q4_K's.
+struct Skinny16Q5K {
+    static constexpr int kBlockBytes = 176;
+    __device__ static void block(const uint8_t* wblk, const uint8_t* arow, const uint8_t* bsrow, int kq,
+                                 int (&sd)[4], float (&sm)[4], uint32_t& ddm) {
+        typedef int v2i __attribute__((ext_vector_type(2)));
+        const int g = kq >> 1, hh = kq & 1;
+        const v4i hdr = *reinterpret_cast<const v4i*>(wblk);
+        const v2i qh = *reinterpret_cast<const v2i*>(wblk + 16 + 8 * kq);
+        v2i qs[4];
+#pragma unroll
+        for (int p = 0; p < 4; ++p) qs[p] = *reinterpret_cast<const v2i*>(wblk + 48 + 32 * p + 8 * kq);
+        ddm = (uint32_t)hdr.x;
+        uint32_t sc8[2], mn8[2];
+        k4_all((uint32_t)hdr.y, (uint32_t)hdr.z, (uint32_t)hdr.w, sc8, mn8);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sd[i] = 0;
+#pragma unroll
+        for (int sb = 0; sb < 8; ++sb) {
+            const int p = sb >> 1, e = sb & 1;
+            v2i b;
+#pragma unroll
+            for (int k = 0; k < 2; ++k) {
+                const uint32_t nib = ((uint32_t)qs[p][k] >> (4 * e)) & 0x0F0F0F0Fu;
+                const uint32_t hb = ((uint32_t)qh[k] >> sb) & 0x01010101u;
+                b[k] = (int)((hb << 4) | nib);
+            }
+            const v2i a = *reinterpret_cast<const v2i*>(arow + sb * 32 + 8 * kq);
+            const v4i r = __builtin_amdgcn_mfma_i32_16x16x32_i8(__builtin_bit_cast(long, a), __builtin_bit_cast(long, b),
+                                                                v4i{0, 0, 0, 0}, 0, 0, 0);
+            const int sc = (int)((sc8[sb >> 2] >> (8 * (sb & 3))) & 0xFFu);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sd[i] += __mul24(r[i], sc);
+        }
+        const v4f smf = Skinny16Q4K::mins_dot_sums(mn8[hh], bsrow, g, hh);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sm[i] = smf[i];
+    }
+};
+
+template <typename F, int NW, int BPW, int MT, bool STAGES>
+__global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
     const uint8_t* __restrict__ w, size_t bpr, const int8_t* __restrict__ qs,
     const float* __restrict__ d8, const int32_t* __restrict__ bsums, float* __restrict__ y, int m,
     int out_f, int nb, int32_t* __restrict__ st_sd, int32_t* __restrict__ st_sm,
     const BatchTile* __restrict__ tiles) {
-    typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+    constexpr int kBlk = F::kBlockBytes;
     constexpr int kTokStride = 256 + 16;            // one token's codes of a block, padded against bank conflicts
     constexpr int kBsOff = MT * kTokStride;         // [token][8] per-32 sums
     constexpr int kTileBytes = kBsOff + MT * 32;
     constexpr int kPh = BPW;                        // blocks of weights staged at a time: the wave's share of a pass
-    constexpr int kRowStride = kPh * 144 + 16;      // padded: eight rows' 16-byte reads cover all banks
-    constexpr int kPieces = kPh * 9, kIt = (kPieces + 3) / 4;  // 16-byte pieces of a row's stage
+    constexpr int kRowStride = kPh * kBlk + 16;     // padded: eight rows' 16-byte reads cover all banks
+    constexpr int kPieces = kPh * kBlk / 16, kIt = (kPieces + 3) / 4;  // 16-byte pieces of a row's stage
     __shared__ __attribute__((aligned(16))) uint8_t w_l[NW][16 * kRowStride];
     __shared__ __attribute__((aligned(16))) uint8_t act_l[NW][kTileBytes];
     __shared__ __attribute__((aligned(16))) float dq_l[NW][MT][BPW];
     __shared__ __attribute__((aligned(16))) float chain_l[64][4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int r16 = lane & 15, kq = lane >> 4, g = kq >> 1, hh = kq & 1;
+    const int r16 = lane & 15, kq = lane >> 4;
     const int rt = blockIdx.y * 16 + r16;  // row inside the 32-row tile
     const size_t in_f = (size_t)nb * 256;
     int wrow = blockIdx.x * 32 + rt;
@@ -672,7 +776,7 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_q4k_kernel(
     const uint32_t loff = srow * kRowStride + pq * 16;
     v4i wreg[kIt];
     auto request_rows = [&](int b) {  // blocks b .. b + BPW - 1; past the end: a redundant stage, never used
-        const uint8_t* src = wbase + (size_t)min(b, nb - kPh) * 144;
+        const uint8_t* src = wbase + (size_t)min(b, nb - kPh) * kBlk;
 #pragma unroll
         for (int it = 0; it < kIt; ++it)
             if (pq + 4 * it < kPieces) wreg[it] = load16(src + goff + 64 * it);
@@ -682,9 +786,6 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_q4k_kernel(
 #pragma unroll
         for (int it = 0; it < kIt; ++it)
             if (pq + 4 * it < kPieces) *reinterpret_cast<v4i*>(wl + loff + 64 * it) = wreg[it];
-    };
-    struct Raw {
-        v4i hdr, q[2];
     };
     const uint8_t* wfrag = wl + r16 * kRowStride;
     // a block's activations: 16-byte piece `chunk & 15` of token `chunk >> 4` (absent tokens repeat the
@@ -718,8 +819,8 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_q4k_kernel(
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     };
     // this lane as A operand: token r16 (rows of absent tokens hold another token's codes)
-    const uint8_t* afrag = tile + (r16 & (MT - 1)) * kTokStride + 16 * hh;
-    const uint8_t* bsfrag = tile + kBsOff + (r16 & (MT - 1)) * 32 + 16 * hh;
+    const uint8_t* afrag = tile + (r16 & (MT - 1)) * kTokStride;
+    const uint8_t* bsfrag = tile + kBsOff + (r16 & (MT - 1)) * 32;
 
     uint32_t dqoff[(MT * BPW + 63) / 64];
 #pragma unroll
@@ -754,54 +855,14 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_q4k_kernel(
                 if (pass + 1 < n_pass) request_rows(b0_next);
             }
             wave_sync();
-            Raw r;
-            r.hdr = *reinterpret_cast<const v4i*>(wfrag + (j % kPh) * 144);
-            r.q[0] = *reinterpret_cast<const v4i*>(wfrag + (j % kPh) * 144 + 16 + 16 * kq);
-            r.q[1] = *reinterpret_cast<const v4i*>(wfrag + (j % kPh) * 144 + 16 + 64 + 16 * kq);
-            ddm[j] = (uint32_t)r.hdr.x;
-            uint32_t sc8[2], mn8[2];
-            k4_all((uint32_t)r.hdr.y, (uint32_t)r.hdr.z, (uint32_t)r.hdr.w, sc8, mn8);
-            v4i alo = {0, 0, 0, 0}, ahi = {0, 0, 0, 0};
+            F::block(wfrag + (j % kPh) * kBlk, afrag, bsfrag, kq, sd[j], sm[j], ddm[j]);
+            if (STAGES) {
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {  // step s: chunk c = s / 2, nibble e = s % 2
-                const int c = s >> 1, e = s & 1;
-                const uint32_t sc = (sc8[c] >> (8 * (2 * g + e))) & 0xFFu;
-                const uint32_t lo3 = sc & 7u, hi3 = sc >> 3;
-                const int qw[4] = {r.q[c].x, r.q[c].y, r.q[c].z, r.q[c].w};
-                v4i blo, bhi;
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const uint32_t codes = ((uint32_t)qw[k] >> (4 * e)) & 0x0F0F0F0Fu;
-                    blo[k] = scale_codes(codes, lo3);
-                    bhi[k] = scale_codes(codes, hi3);
-                }
-                const v4i a = *reinterpret_cast<const v4i*>(afrag + (4 * c + 2 * g + e) * 32);
-                alo = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, blo, alo, 0, 0, 0);
-                ahi = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bhi, ahi, 0, 0, 0);
-            }
-            // sm: K = 16 slots = (bsum & 63 | the rest) x sub-blocks 0..7; this lane carries slots
-            // 4kq..4kq+3, sub-blocks 4hh..4hh+3 of part g
-            const uint32_t mnw = mn8[hh];
-            const v4h bm = {(_Float16)(int)(mnw & 0xFFu), (_Float16)(int)((mnw >> 8) & 0xFFu),
-                            (_Float16)(int)((mnw >> 16) & 0xFFu), (_Float16)(int)(mnw >> 24)};
-            const v4i bs = *reinterpret_cast<const v4i*>(bsfrag);
-            const int bsv[4] = {bs.x, bs.y, bs.z, bs.w};
-            v4h abs_;
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const int lo = bsv[k] & 63;
-                abs_[k] = (_Float16)(g ? bsv[k] - lo : lo);
-            }
-            const v4f smf = __builtin_amdgcn_mfma_f32_16x16x16f16(abs_, bm, v4f{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                sd[j][i] = alo[i] + (ahi[i] << 3);
-                sm[j][i] = smf[i];
-                if (STAGES) {
+                for (int i = 0; i < 4; ++i) {
                     const int tok = 4 * kq + i;
                     if (row_ok && tok < m && b0 + j < nb) {
                         st_sd[((size_t)tok * out_f + wrow) * nb + b0 + j] = sd[j][i];
-                        st_sm[((size_t)tok * out_f + wrow) * nb + b0 + j] = (int)smf[i];
+                        st_sm[((size_t)tok * out_f + wrow) * nb + b0 + j] = (int)sm[j][i];
                     }
                 }
             }
@@ -843,11 +904,12 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_q4k_kernel(
     }
 }
 
-// Waves per workgroup and blocks per wave and pass for rows of nb blocks; false: the older kernel takes them.
-static bool skinny16_shape(int nb, size_t m, int* nw, int* bpw) {
+// Waves per workgroup and blocks per wave and pass for rows of nb blocks; false: another kernel takes them.
+static bool skinny16_shape(int dtype, int nb, size_t m, int* nw, int* bpw) {
     static const int env_nw = getenv("INFR_HIP_SKINNY16_WAVES") ? atoi(getenv("INFR_HIP_SKINNY16_WAVES")) : 0;
     static const int env_bpw = getenv("INFR_HIP_SKINNY16_BLOCKS") ? atoi(getenv("INFR_HIP_SKINNY16_BLOCKS")) : 0;
-    if (m > 16) return false;
+    static const int env_max = getenv("INFR_HIP_SKINNY16_MAX_M") ? atoi(getenv("INFR_HIP_SKINNY16_MAX_M")) : 16;
+    if ((dtype != 12 && dtype != 13) || m > 16 || (int)m > env_max) return false;
     int n = env_nw == 8 ? 8 : 4;
     if (m > 8) n = 4;  // eight waves with 16-token tiles would need more than 64 KB of LDS
     *nw = n;
@@ -859,16 +921,18 @@ static bool skinny16_shape(int nb, size_t m, int* nw, int* bpw) {
     return true;
 }
 
-template <bool STAGES>
-static bool launch_mmq_skinny16(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
-                                size_t out_f, size_t wgs, const IntStages& st, const BatchTile* tiles,
-                                hipStream_t stream) {
-    const int nb = (int)(in_f / 256);
+bool mmq_skinny16_takes(int dtype, size_t m, size_t in_f) {
     int nw = 0, bpw = 0;
-    if (!skinny16_shape(nb, m, &nw, &bpw)) return false;
+    return in_f % 256 == 0 && skinny16_shape(dtype, (int)(in_f / 256), m, &nw, &bpw);
+}
+
+template <typename F, bool STAGES>
+static void launch_mmq_skinny16_fmt(int nw, int bpw, const uint8_t* w, size_t bpr, const ActQ8& act, float* y,
+                                    size_t m, int nb, size_t out_f, size_t wgs, const IntStages& st,
+                                    const BatchTile* tiles, hipStream_t stream) {
     const dim3 grid((unsigned)wgs, 2);
 #define INFR_S16(NW_, BPW_, MT_)                                                                              \
-    hipLaunchKernelGGL((mmq_skinny16_q4k_kernel<NW_, BPW_, MT_, STAGES>), grid, dim3(NW_ * 64), 0, stream, w, bpr, \
+    hipLaunchKernelGGL((mmq_skinny16_kernel<F, NW_, BPW_, MT_, STAGES>), grid, dim3(NW_ * 64), 0, stream, w, bpr, \
                        act.qs, act.d, act.bsums, y, (int)m, (int)out_f, nb, st.a, st.b, tiles)
     if (nw == 4 && m <= 8) {
         if (bpw == 2) INFR_S16(4, 2, 8);
@@ -881,14 +945,26 @@ static bool launch_mmq_skinny16(const uint8_t* w, size_t bpr, const ActQ8& act, 
         else INFR_S16(8, 4, 8);
     }
 #undef INFR_S16
+}
+
+template <bool STAGES>
+static bool launch_mmq_skinny16(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
+                                size_t in_f, size_t out_f, size_t wgs, const IntStages& st, const BatchTile* tiles,
+                                hipStream_t stream) {
+    const int nb = (int)(in_f / 256);
+    int nw = 0, bpw = 0;
+    if (in_f % 256 != 0 || !skinny16_shape(dtype, nb, m, &nw, &bpw)) return false;
+    if (dtype == 12)
+        launch_mmq_skinny16_fmt<Skinny16Q4K, STAGES>(nw, bpw, w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
+    else
+        launch_mmq_skinny16_fmt<Skinny16Q5K, STAGES>(nw, bpw, w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     return true;
 }
 
-void launch_mmq_skinny_group(size_t m, size_t in_f, const BatchTile* tiles_dev, const BatchGroupPlan& plan,
-                             const ActQ8& act, hipStream_t stream) {
-    static const int env_s16_max = getenv("INFR_HIP_SKINNY16_MAX_M") ? atoi(getenv("INFR_HIP_SKINNY16_MAX_M")) : 16;
-    if ((int)m <= env_s16_max &&
-        launch_mmq_skinny16<false>(nullptr, 0, act, nullptr, m, in_f, 0, plan.total_wgs, IntStages{}, tiles_dev, stream))
+void launch_mmq_skinny_group(int dtype, size_t m, size_t in_f, const BatchTile* tiles_dev,
+                             const BatchGroupPlan& plan, const ActQ8& act, hipStream_t stream) {
+    if (launch_mmq_skinny16<false>(dtype, nullptr, 0, act, nullptr, m, in_f, 0, plan.total_wgs, IntStages{}, tiles_dev,
+                                   stream))
         return;
     const dim3 grid((unsigned)plan.total_wgs, (unsigned)((m + 31) / 32));
     const int nb = (int)(in_f / 256);
@@ -986,14 +1062,12 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
     }
     launch_quantize_q8(x, m, in_f, act_is_per32(dtype, in_f), act, stream);
     static const int env_dot4_max = getenv("INFR_HIP_Q4K_DOT4_MAX_M") ? atoi(getenv("INFR_HIP_Q4K_DOT4_MAX_M")) : 0;
-    if (dtype != 12 || (int)m <= env_dot4_max) return launch_gemv_batch(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
-    static const int env_s16_max = getenv("INFR_HIP_SKINNY16_MAX_M") ? atoi(getenv("INFR_HIP_SKINNY16_MAX_M")) : 16;
-    if ((int)m <= env_s16_max) {
+    if ((dtype != 12 || (int)m > env_dot4_max) && mmq_skinny16_takes(dtype, m, in_f)) {
         const size_t wgs = (out_f + 31) / 32;
-        if (st.a ? launch_mmq_skinny16<true>(w, bpr, act, y, m, in_f, out_f, wgs, st, nullptr, stream)
-                 : launch_mmq_skinny16<false>(w, bpr, act, y, m, in_f, out_f, wgs, st, nullptr, stream))
-            return true;
+        return st.a ? launch_mmq_skinny16<true>(dtype, w, bpr, act, y, m, in_f, out_f, wgs, st, nullptr, stream)
+                    : launch_mmq_skinny16<false>(dtype, w, bpr, act, y, m, in_f, out_f, wgs, st, nullptr, stream);
     }
+    if (dtype != 12 || (int)m <= env_dot4_max) return launch_gemv_batch(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
     if ((int)m <= env_skinny_max) {
         // four blocks per round; eight for long rows or when four would leave most SIMDs without a wave
         const size_t wgs = (out_f + 31) / 32 * ((m + 31) / 32);

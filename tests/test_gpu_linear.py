@@ -124,6 +124,36 @@ def test_prefill_q4k_is_bit_identical_to_oracle(be, m, in_f, out_f):
     assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), "not bit-identical"
 
 
+# 2..16 tokens on rows of an even number of blocks: 16 x 16 MFMA tiles, K split over the waves of a
+# workgroup in passes of eight blocks (one pass, several, a ragged last one, waves past the end),
+# 8- and 16-token tiles, a ragged last row tile
+@pytest.mark.parametrize("m,in_f,out_f", [(3, 4096, 48), (8, 5632, 40), (7, 8192, 24), (9, 512, 16),
+                                          (12, 2048, 100), (16, 4096, 33), (16, 6144, 64)])
+@pytest.mark.parametrize("dtype", [DType.Q4K, DType.Q5K])
+def test_small_batch_kquant_mfma_is_bit_identical_to_oracle(be, dtype, m, in_f, out_f):
+    w = synth_weight(dtype, 500 + m, out_f, in_f)
+    x = synth_normal_f32(600 + m, m * in_f)
+    x[:in_f] *= 37.0
+    x[(m - 1) * in_f:] *= 0.01
+    y = run_linear(be, dtype, w, x, m, in_f, out_f)
+    want = orc.linear(dtype, w, x, m, in_f, out_f)
+    assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), "not bit-identical"
+
+
+@pytest.mark.parametrize("m,in_f,out_f", [(6, 4608, 40), (13, 1024, 50)])
+@pytest.mark.parametrize("dtype,seed", [(DType.Q4K, 0x209), (DType.Q5K, 0x20A)])
+def test_small_batch_kquant_mfma_int_stages_bit_exact(be, dtype, seed, m, in_f, out_f):
+    # full-range payload bytes and saturated activation rows: every scale, min and code value,
+    # block sums up to +-4064
+    w = orc.synth_weight(dtype, in_f * out_f, seed)
+    x = synth_normal_f32(78, m * in_f) * np.float32(3.0)
+    x[in_f:2 * in_f] = 1e4
+    x[2 * in_f:3 * in_f] = -1e4
+    a, b = be.linear_int_stages(dtype, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
+    oa, ob = orc.linear_int_stages(dtype, w, x, m, in_f, out_f)
+    assert np.array_equal(a, oa) and np.array_equal(b, ob)
+
+
 @pytest.mark.parametrize("m,in_f,out_f", [(5, 512, 40), (70, 768, 150)])
 def test_prefill_q4k_int_stages_bit_exact(be, m, in_f, out_f):
     # full-range payload bytes: every scale, min and code value occurs (sc up to 63 exercises the

@@ -100,13 +100,13 @@ def test_in_place_chain_is_ordered(be):
     assert np.array_equal(bits(be.download(yb, np.empty(in_f, np.float32))), bits(y2))
 
 
-@pytest.mark.parametrize("m", [2, 5, 8, 19])
+@pytest.mark.parametrize("m", [2, 5, 8, 12, 16, 19])
 def test_small_batch_ops_run_as_groups(be, m):
     """m = 2..32 inside a plan: ops of a level that share (dtype, in_f, m) become one quantize
     launch over the distinct activation tensors plus one GEMM launch over a tile table. q/k/v
     share x, a second level consumes the first, and every replay is checked against the oracle."""
     H, KV, FF = 512, 256, 1024
-    fmts = [DType.Q4K] if m > 8 else [DType.Q4K, DType.Q6K, DType.Q8_0, DType.Q2_0]
+    fmts = ([DType.Q4K] if m > 16 else [DType.Q4K, DType.Q5K]) if m > 8 else [DType.Q4K, DType.Q5K, DType.Q6K, DType.Q8_0, DType.Q2_0]
     for dt in fmts:
         spec = [("q", dt, H, H, "x"), ("k", dt, KV, H, "x"), ("v", dt, KV + 40, H, "x2"),
                 ("o", dt, H, H, "q"), ("up", dt, FF, H, "q"), ("down", dt, 200, FF, "up")]
@@ -137,7 +137,7 @@ def test_small_batch_ops_run_as_groups(be, m):
                 # each op is checked on the device's own input, so one op's rounding does not leak
                 src_dev = want[src] if src in want else be.download(bufs[src], np.empty(m * in_f, np.float32))
                 ref = orc.linear(d, weights[name], src_dev, m, in_f, out_f)
-                if d in (DType.Q4K, DType.Q6K):
+                if d in (DType.Q4K, DType.Q5K, DType.Q6K):
                     assert np.array_equal(bits(got), bits(ref)), f"{name} {d} differs on execute {rep}"
                 else:
                     a, b = got.astype(np.float64).ravel(), ref.astype(np.float64).ravel()
