@@ -628,9 +628,15 @@ static void launch_mmq_skinny_q4k(const uint8_t* w, size_t bpr, const ActQ8& act
 struct Skinny16Q4K {
     static constexpr int kBlockBytes = 144;
     // Q4_K: the scale split sc = 8 hi + lo folded into two operand sets, two chains of four K = 64 steps
-    __device__ static void block(const uint8_t* wblk, const uint8_t* arow, const uint8_t* bsrow, int kq,
-                                 int (&sd)[4], float (&sm)[4], uint32_t& ddm) {
-        typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+    static constexpr int kRowStride = 2 * kBlockBytes + 16;  // two blocks, padded: eight rows' 16-byte reads cover all banks
+    // sumf += q8.d[b] * (d * sd as f32 - dmin * sm as f32)
+    __device__ static float accumulate(float acc, float dq, uint32_t ddm, int sd, float sm) {
+        const float d = f16_bits_to_f32(ddm & 0xFFFFu), dmin = f16_bits_to_f32(ddm >> 16);
+        return acc + dq * (d * (float)sd - dmin * sm);
+    }
+    __device__ static void block(const uint8_t* wrow, int jj, const uint8_t* arow, const uint8_t* zrow,
+                                 const uint8_t* bsrow, int kq, int (&sd)[4], float (&sm)[4], uint32_t& ddm) {
+        const uint8_t* wblk = wrow + jj * kBlockBytes;
         const int g = kq >> 1, hh = kq & 1;
         const v4i hdr = *reinterpret_cast<const v4i*>(wblk);
         v4i q[2];
@@ -688,9 +694,14 @@ struct Skinny16Q4K {
 // multiply-add; sm and the epilogue are Q4_K's.
 struct Skinny16Q5K {
     static constexpr int kBlockBytes = 176;
-    __device__ static void block(const uint8_t* wblk, const uint8_t* arow, const uint8_t* bsrow, int kq,
-                                 int (&sd)[4], float (&sm)[4], uint32_t& ddm) {
+    static constexpr int kRowStride = 2 * kBlockBytes + 16;
+    __device__ static float accumulate(float acc, float dq, uint32_t ddm, int sd, float sm) {
+        return Skinny16Q4K::accumulate(acc, dq, ddm, sd, sm);
+    }
+    __device__ static void block(const uint8_t* wrow, int jj, const uint8_t* arow, const uint8_t* zrow,
+                                 const uint8_t* bsrow, int kq, int (&sd)[4], float (&sm)[4], uint32_t& ddm) {
         typedef int v2i __attribute__((ext_vector_type(2)));
+        const uint8_t* wblk = wrow + jj * kBlockBytes;
         const int g = kq >> 1, hh = kq & 1;
         const v4i hdr = *reinterpret_cast<const v4i*>(wblk);
         const v2i qh = *reinterpret_cast<const v2i*>(wblk + 16 + 8 * kq);
@@ -725,6 +736,78 @@ struct Skinny16Q5K {
     }
 };
 
+// Q6_K (210-byte block: ql[128], qh[64], int8 scales[16], d; crates/infr-cpu/src/kernels.rs:487-526):
+// isum = sum_g sc_g * (sum over the group's 16 of (q - 32) * q8), y += (d * q8.d[b]) * isum. A K = 32
+// step holds two groups of 16 (lanes kq 0, 1 and kq 2, 3); each is multiplied alone - the other
+// group's activation lanes read a row of zero bytes - and scaled into isum by a 24-bit
+// multiply-add. A stage of two blocks is 420 bytes from a 4-byte boundary, so its second block sits
+// 2 bytes off a boundary in LDS: it is read as aligned words and shifted in registers.
+struct Skinny16Q6K {
+    typedef int v2i __attribute__((ext_vector_type(2)));
+    static constexpr int kBlockBytes = 210;
+    static constexpr int kRowStride = 432;  // 420 rounded up to 16: 108 words, eight rows' reads cover all banks
+    // sumf += d * q8.d[b] * (isum as f32), evaluated (d * q8.d[b]) * isum
+    __device__ static float accumulate(float acc, float dq, uint32_t ddm, int sd, float) {
+        return acc + (f16_bits_to_f32(ddm) * dq) * (float)sd;
+    }
+    template <bool ODD>
+    __device__ static v2i read8(const uint8_t* blk, int o) {
+        if (!ODD) return *reinterpret_cast<const v2i*>(blk + o);
+        const uint8_t* p = blk - 2 + o;
+        const v2i lo = *reinterpret_cast<const v2i*>(p);
+        const int hi = *reinterpret_cast<const int*>(p + 8);
+        return v2i{(int)__builtin_amdgcn_alignbyte((uint32_t)lo.y, (uint32_t)lo.x, 2),
+                   (int)__builtin_amdgcn_alignbyte((uint32_t)hi, (uint32_t)lo.y, 2)};
+    }
+    template <bool ODD>
+    __device__ static void block_at(const uint8_t* blk, const uint8_t* arow, const uint8_t* zrow, int kq, int (&sd)[4],
+                                    uint32_t& ddm) {
+        v2i ql[2][2], qh[2];
+#pragma unroll
+        for (int n = 0; n < 2; ++n) {
+            ql[n][0] = read8<ODD>(blk, 64 * n + 8 * kq);
+            ql[n][1] = read8<ODD>(blk, 64 * n + 32 + 8 * kq);
+            qh[n] = read8<ODD>(blk, 128 + 32 * n + 8 * kq);
+        }
+        const v2i s01 = read8<ODD>(blk, 192), s23 = read8<ODD>(blk, 200);
+        const int scw[4] = {s01.x, s01.y, s23.x, s23.y};
+        ddm = *reinterpret_cast<const uint16_t*>(blk + 208);
+        // group 2s in the K-slots of lanes kq 0, 1, group 2s+1 in those of kq 2, 3
+        const uint8_t* a0p = (kq < 2 ? arow : zrow) + 8 * kq;
+        const uint8_t* a1p = (kq < 2 ? zrow : arow) + 8 * kq;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sd[i] = 0;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {  // elements 32s .. 32s + 31: half n, quarter t of the half
+            const int n = s >> 2, t = s & 3;
+            v2i b;
+#pragma unroll
+            for (int k = 0; k < 2; ++k) {
+                const uint32_t nib = ((uint32_t)ql[n][t & 1][k] >> (4 * (t >> 1))) & 0x0F0F0F0Fu;
+                const uint32_t hb = ((uint32_t)qh[n][k] >> (2 * t)) & 0x03030303u;
+                b[k] = (int)((((hb << 4) | nib) + 0x60606060u) ^ 0x80808080u);  // q - 32 as int8
+            }
+            const long bl = __builtin_bit_cast(long, b);
+            const v2i a0 = *reinterpret_cast<const v2i*>(a0p + 32 * s);
+            const v2i a1 = *reinterpret_cast<const v2i*>(a1p + 32 * s);
+            const v4i r0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(__builtin_bit_cast(long, a0), bl, v4i{0, 0, 0, 0}, 0, 0, 0);
+            const v4i r1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(__builtin_bit_cast(long, a1), bl, v4i{0, 0, 0, 0}, 0, 0, 0);
+            const int g0 = 2 * s, g1 = 2 * s + 1;
+            const int sc0 = __builtin_amdgcn_sbfe(scw[g0 >> 2], 8 * (g0 & 3), 8);
+            const int sc1 = __builtin_amdgcn_sbfe(scw[g1 >> 2], 8 * (g1 & 3), 8);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sd[i] += __mul24(r0[i], sc0) + __mul24(r1[i], sc1);
+        }
+    }
+    __device__ static void block(const uint8_t* wrow, int jj, const uint8_t* arow, const uint8_t* zrow,
+                                 const uint8_t*, int kq, int (&sd)[4], float (&sm)[4], uint32_t& ddm) {
+        if (jj & 1) block_at<true>(wrow + jj * kBlockBytes, arow, zrow, kq, sd, ddm);
+        else block_at<false>(wrow + jj * kBlockBytes, arow, zrow, kq, sd, ddm);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sm[i] = 0.0f;
+    }
+};
+
 template <typename F, int NW, int BPW, int MT, bool STAGES>
 __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
     const uint8_t* __restrict__ w, size_t bpr, const int8_t* __restrict__ qs,
@@ -734,10 +817,14 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
     constexpr int kBlk = F::kBlockBytes;
     constexpr int kTokStride = 256 + 16;            // one token's codes of a block, padded against bank conflicts
     constexpr int kBsOff = MT * kTokStride;         // [token][8] per-32 sums
-    constexpr int kTileBytes = kBsOff + MT * 32;
+    constexpr int kZeroOff = kBsOff + MT * 32;      // 256 zero bytes: the codes of a token that is not there
+    constexpr int kTileBytes = kZeroOff + 256;
     constexpr int kPh = BPW;                        // blocks of weights staged at a time: the wave's share of a pass
-    constexpr int kRowStride = kPh * kBlk + 16;     // padded: eight rows' 16-byte reads cover all banks
-    constexpr int kPieces = kPh * kBlk / 16, kIt = (kPieces + 3) / 4;  // 16-byte pieces of a row's stage
+    constexpr int kRowStride = BPW == 2 ? F::kRowStride : kPh * kBlk + 16;
+    // a row's stage in 16-byte pieces, and a last piece of one word (Q6_K: 420 = 26 x 16 + 4)
+    constexpr int kFull = kPh * kBlk / 16, kTail = kPh * kBlk % 16;
+    static_assert(kTail == 0 || kTail == 4, "a stage is whole 16-byte pieces plus at most one word");
+    constexpr int kPieces = kFull + (kTail ? 1 : 0), kIt = (kPieces + 3) / 4;
     __shared__ __attribute__((aligned(16))) uint8_t w_l[NW][16 * kRowStride];
     __shared__ __attribute__((aligned(16))) uint8_t act_l[NW][kTileBytes];
     __shared__ __attribute__((aligned(16))) float dq_l[NW][MT][BPW];
@@ -778,14 +865,18 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
     auto request_rows = [&](int b) {  // blocks b .. b + BPW - 1; past the end: a redundant stage, never used
         const uint8_t* src = wbase + (size_t)min(b, nb - kPh) * kBlk;
 #pragma unroll
-        for (int it = 0; it < kIt; ++it)
-            if (pq + 4 * it < kPieces) wreg[it] = load16(src + goff + 64 * it);
+        for (int it = 0; it < kIt; ++it) {
+            if (pq + 4 * it < kFull) wreg[it] = kBlk % 16 == 0 ? load16(src + goff + 64 * it) : load16_a4(src + goff + 64 * it);
+            else if (kTail && pq + 4 * it == kFull) wreg[it].x = load_u32(src + goff + 64 * it);
+        }
     };
     uint8_t* wl = w_l[wave];
     auto publish_rows = [&]() {
 #pragma unroll
-        for (int it = 0; it < kIt; ++it)
-            if (pq + 4 * it < kPieces) *reinterpret_cast<v4i*>(wl + loff + 64 * it) = wreg[it];
+        for (int it = 0; it < kIt; ++it) {
+            if (pq + 4 * it < kFull) *reinterpret_cast<v4i*>(wl + loff + 64 * it) = wreg[it];
+            else if (kTail && pq + 4 * it == kFull) *reinterpret_cast<int*>(wl + loff + 64 * it) = wreg[it].x;
+        }
     };
     const uint8_t* wfrag = wl + r16 * kRowStride;
     // a block's activations: 16-byte piece `chunk & 15` of token `chunk >> 4` (absent tokens repeat the
@@ -821,6 +912,8 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
     // this lane as A operand: token r16 (rows of absent tokens hold another token's codes)
     const uint8_t* afrag = tile + (r16 & (MT - 1)) * kTokStride;
     const uint8_t* bsfrag = tile + kBsOff + (r16 & (MT - 1)) * 32;
+    const uint8_t* zrow = tile + kZeroOff;
+    *reinterpret_cast<int*>(tile + kZeroOff + lane * 4) = 0;  // ordered before the first read by the loop's wave_sync
 
     uint32_t dqoff[(MT * BPW + 63) / 64];
 #pragma unroll
@@ -855,21 +948,21 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
                 if (pass + 1 < n_pass) request_rows(b0_next);
             }
             wave_sync();
-            F::block(wfrag + (j % kPh) * kBlk, afrag, bsfrag, kq, sd[j], sm[j], ddm[j]);
+            F::block(wfrag, j % kPh, afrag, zrow, bsfrag, kq, sd[j], sm[j], ddm[j]);
             if (STAGES) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int tok = 4 * kq + i;
                     if (row_ok && tok < m && b0 + j < nb) {
                         st_sd[((size_t)tok * out_f + wrow) * nb + b0 + j] = sd[j][i];
-                        st_sm[((size_t)tok * out_f + wrow) * nb + b0 + j] = (int)sm[j][i];
+                        if (st_sm) st_sm[((size_t)tok * out_f + wrow) * nb + b0 + j] = (int)sm[j][i];
                     }
                 }
             }
         }
         wave_sync();  // dq_l was written by this wave's lanes
 
-        // f32 epilogue handed down the waves: sumf += q8.d[b] * (d * sd as f32 - dmin * sm as f32), b ascending
+        // f32 epilogue handed down the waves: the format's CPU expression per block, b ascending
 #pragma unroll
         for (int k = 0; k < NW; ++k) {
             if (wave == k) {
@@ -881,13 +974,9 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
 #pragma unroll
                 for (int j = 0; j < BPW; ++j) {
                     if (b0 + j < nb) {
-                        const float d = f16_bits_to_f32(ddm[j] & 0xFFFFu);
-                        const float dmin = f16_bits_to_f32(ddm[j] >> 16);
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            const float dq = dq_l[wave][(4 * kq + i) & (MT - 1)][j];
-                            acc[i] += dq * (d * (float)sd[j][i] - dmin * sm[j][i]);
-                        }
+                        for (int i = 0; i < 4; ++i)
+                            acc[i] = F::accumulate(acc[i], dq_l[wave][(4 * kq + i) & (MT - 1)][j], ddm[j], sd[j][i], sm[j][i]);
                     }
                 }
                 if (k + 1 < NW || pass + 1 < n_pass)
@@ -909,14 +998,14 @@ static bool skinny16_shape(int dtype, int nb, size_t m, int* nw, int* bpw) {
     static const int env_nw = getenv("INFR_HIP_SKINNY16_WAVES") ? atoi(getenv("INFR_HIP_SKINNY16_WAVES")) : 0;
     static const int env_bpw = getenv("INFR_HIP_SKINNY16_BLOCKS") ? atoi(getenv("INFR_HIP_SKINNY16_BLOCKS")) : 0;
     static const int env_max = getenv("INFR_HIP_SKINNY16_MAX_M") ? atoi(getenv("INFR_HIP_SKINNY16_MAX_M")) : 16;
-    if ((dtype != 12 && dtype != 13) || m > 16 || (int)m > env_max) return false;
+    if ((dtype != 12 && dtype != 13 && dtype != 14) || m > 16 || (int)m > env_max) return false;
     int n = env_nw == 8 ? 8 : 4;
     if (m > 8) n = 4;  // eight waves with 16-token tiles would need more than 64 KB of LDS
     *nw = n;
     // (four blocks per wave and pass - 576-byte, 64-byte-aligned runs per row - measured 20-25 % slower:
     // a wave then computes for longer before it asks for more)
     *bpw = env_bpw == 2 || env_bpw == 4 ? env_bpw : 2;
-    if (nb % 4 != 0) *bpw = 2;
+    if (nb % 4 != 0 || dtype == 14) *bpw = 2;  // (a Q6_K stage of four blocks would end in an 8-byte piece)
     if (nb < *bpw || nb % *bpw != 0) return false;  // weights are staged BPW blocks at a time
     return true;
 }
@@ -947,6 +1036,21 @@ static void launch_mmq_skinny16_fmt(int nw, int bpw, const uint8_t* w, size_t bp
 #undef INFR_S16
 }
 
+// Q6_K: two blocks per wave and pass only
+template <bool STAGES>
+static void launch_mmq_skinny16_q6k(int nw, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, int nb,
+                                    size_t out_f, size_t wgs, const IntStages& st, const BatchTile* tiles,
+                                    hipStream_t stream) {
+    const dim3 grid((unsigned)wgs, 2);
+#define INFR_S16(NW_, MT_)                                                                                        \
+    hipLaunchKernelGGL((mmq_skinny16_kernel<Skinny16Q6K, NW_, 2, MT_, STAGES>), grid, dim3(NW_ * 64), 0, stream, w, \
+                       bpr, act.qs, act.d, act.bsums, y, (int)m, (int)out_f, nb, st.a, st.b, tiles)
+    if (nw == 4 && m <= 8) INFR_S16(4, 8);
+    else if (nw == 4) INFR_S16(4, 16);
+    else INFR_S16(8, 8);
+#undef INFR_S16
+}
+
 template <bool STAGES>
 static bool launch_mmq_skinny16(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
                                 size_t in_f, size_t out_f, size_t wgs, const IntStages& st, const BatchTile* tiles,
@@ -956,8 +1060,10 @@ static bool launch_mmq_skinny16(int dtype, const uint8_t* w, size_t bpr, const A
     if (in_f % 256 != 0 || !skinny16_shape(dtype, nb, m, &nw, &bpw)) return false;
     if (dtype == 12)
         launch_mmq_skinny16_fmt<Skinny16Q4K, STAGES>(nw, bpw, w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
-    else
+    else if (dtype == 13)
         launch_mmq_skinny16_fmt<Skinny16Q5K, STAGES>(nw, bpw, w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
+    else
+        launch_mmq_skinny16_q6k<STAGES>(nw, w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     return true;
 }
 

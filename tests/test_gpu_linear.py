@@ -129,7 +129,7 @@ def test_prefill_q4k_is_bit_identical_to_oracle(be, m, in_f, out_f):
 # 8- and 16-token tiles, a ragged last row tile
 @pytest.mark.parametrize("m,in_f,out_f", [(3, 4096, 48), (8, 5632, 40), (7, 8192, 24), (9, 512, 16),
                                           (12, 2048, 100), (16, 4096, 33), (16, 6144, 64)])
-@pytest.mark.parametrize("dtype", [DType.Q4K, DType.Q5K])
+@pytest.mark.parametrize("dtype", [DType.Q4K, DType.Q5K, DType.Q6K])
 def test_small_batch_kquant_mfma_is_bit_identical_to_oracle(be, dtype, m, in_f, out_f):
     w = synth_weight(dtype, 500 + m, out_f, in_f)
     x = synth_normal_f32(600 + m, m * in_f)
@@ -141,7 +141,7 @@ def test_small_batch_kquant_mfma_is_bit_identical_to_oracle(be, dtype, m, in_f, 
 
 
 @pytest.mark.parametrize("m,in_f,out_f", [(6, 4608, 40), (13, 1024, 50)])
-@pytest.mark.parametrize("dtype,seed", [(DType.Q4K, 0x209), (DType.Q5K, 0x20A)])
+@pytest.mark.parametrize("dtype,seed", [(DType.Q4K, 0x209), (DType.Q5K, 0x20A), (DType.Q6K, 0x20B)])
 def test_small_batch_kquant_mfma_int_stages_bit_exact(be, dtype, seed, m, in_f, out_f):
     # full-range payload bytes and saturated activation rows: every scale, min and code value,
     # block sums up to +-4064
@@ -151,7 +151,9 @@ def test_small_batch_kquant_mfma_int_stages_bit_exact(be, dtype, seed, m, in_f, 
     x[2 * in_f:3 * in_f] = -1e4
     a, b = be.linear_int_stages(dtype, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
     oa, ob = orc.linear_int_stages(dtype, w, x, m, in_f, out_f)
-    assert np.array_equal(a, oa) and np.array_equal(b, ob)
+    assert np.array_equal(a, oa)
+    if dtype != DType.Q6K:      # Q6_K has one integer stage (isum)
+        assert np.array_equal(b, ob)
 
 
 @pytest.mark.parametrize("m,in_f,out_f", [(5, 512, 40), (70, 768, 150)])

@@ -106,7 +106,7 @@ def test_small_batch_ops_run_as_groups(be, m):
     launch over the distinct activation tensors plus one GEMM launch over a tile table. q/k/v
     share x, a second level consumes the first, and every replay is checked against the oracle."""
     H, KV, FF = 512, 256, 1024
-    fmts = ([DType.Q4K] if m > 16 else [DType.Q4K, DType.Q5K]) if m > 8 else [DType.Q4K, DType.Q5K, DType.Q6K, DType.Q8_0, DType.Q2_0]
+    fmts = ([DType.Q4K] if m > 16 else [DType.Q4K, DType.Q5K, DType.Q6K]) if m > 8 else [DType.Q4K, DType.Q5K, DType.Q6K, DType.Q8_0, DType.Q2_0]
     for dt in fmts:
         spec = [("q", dt, H, H, "x"), ("k", dt, KV, H, "x"), ("v", dt, KV + 40, H, "x2"),
                 ("o", dt, H, H, "q"), ("up", dt, FF, H, "q"), ("down", dt, 200, FF, "up")]
