@@ -999,6 +999,9 @@ static bool skinny16_shape(int dtype, int nb, size_t m, int* nw, int* bpw) {
     static const int env_bpw = getenv("INFR_HIP_SKINNY16_BLOCKS") ? atoi(getenv("INFR_HIP_SKINNY16_BLOCKS")) : 0;
     static const int env_max = getenv("INFR_HIP_SKINNY16_MAX_M") ? atoi(getenv("INFR_HIP_SKINNY16_MAX_M")) : 16;
     if ((dtype != 12 && dtype != 13 && dtype != 14) || m > 16 || (int)m > env_max) return false;
+    // the dot4 batch kernels, which unpack a weight once per two or four tokens, stay ahead at the
+    // bottom: Q5_K at two tokens (4.3-5.3 against 3.8-4.4 TB/s), Q6_K up to four (3.6-4.5 against 3.3-3.9)
+    if ((dtype == 13 && m < 3) || (dtype == 14 && m < 5)) return false;
     int n = env_nw == 8 ? 8 : 4;
     if (m > 8) n = 4;  // eight waves with 16-token tiles would need more than 64 KB of LDS
     *nw = n;
