@@ -36,6 +36,7 @@ INT8_PEAK_TOPS = 5000.0    # MI355X dense int8 MFMA, published
 LAYER = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
          ("gate", 12288, 4096), ("up", 12288, 4096), ("down", 4096, 12288)]
 N_LAYERS = 36
+RAMP_STEPS = 60            # untimed executes before the warmup steps: the clocks take ~30 ms of load to settle
 VOCAB = 151936
 
 
@@ -248,10 +249,15 @@ def single_shape(be, dtype, m, in_f, out_f, reps=40, rotate_bytes=768 << 20):
         binds.bind(yid, yb)
         g.push(Linear(xid, wids[i % copies], yid, m, in_f, out_f))
     plan = be.compile(g)
-    be.execute(plan, binds)
-    be.sync()
+    # untimed: keep the device loaded for ~30 ms so that its clocks have settled (see RAMP_STEPS)
+    t0 = time.perf_counter()
+    while True:
+        be.execute(plan, binds)
+        be.sync()
+        if time.perf_counter() - t0 > 0.03:
+            break
     best = 1e30
-    for _ in range(3):
+    for _ in range(5):
         be.timer_begin()
         be.execute(plan, binds)
         best = min(best, be.timer_end())
@@ -376,7 +382,7 @@ def cpu_baseline(dtype_name="Q4_K"):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--layers", type=int, default=N_LAYERS)
     ap.add_argument("--no-extra", action="store_true", help="headline sweep only")
@@ -394,6 +400,11 @@ def main():
     caps = be.capabilities()
 
     sw = Sweep(be, DType.Q4K, 1, args.layers)
+    # The device raises its clocks over the first ~30 ms of continuous load (the same plan runs at
+    # 5.2 TB/s in its first five executes after an idle period and at 5.7 TB/s from the fortieth on),
+    # and an idle half second resets that. A sustained figure is what the metric asks for, so an
+    # untimed ramp of RAMP_STEPS executes precedes the W warmup steps; it is reported in `config`.
+    sw.time(RAMP_STEPS, 0)
     dev_ms, wall_ms = sw.time(args.steps, args.warmup)
     ms = max(dev_ms, wall_ms)
     value = sw.bytes / (ms * 1e-3) / 1e9
@@ -422,6 +433,7 @@ def main():
                                f"({sw.launches} independent Op::Linear over distinct matrices, "
                                f"{sw.bytes / 1e9:.2f} GB, one plan), batch 1",
                    "weights": "N(0,0.02^2) seed 0 -> Q4_K", "activations": "N(0,1) f32, quantized on GPU",
+                   "clock_ramp_steps_untimed": RAMP_STEPS,
                    "device": caps["device_name"], "compute_units": caps["compute_units"]},
         "pct_of_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "launches_per_step": n_launch,
