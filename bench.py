@@ -466,6 +466,12 @@ def main():
             t, nb = single_shape(be, DType.Q4K, M, 4096, 12288, reps=10)
             extra[f"mmq_Q4_K_M{M}_TOPS"] = round(2.0 * M * 12288 * 4096 / (t * 1e-3) / 1e12, 2)
             extra[f"mmq_Q4_K_M{M}_pct_int8_peak"] = round(100 * extra[f"mmq_Q4_K_M{M}_TOPS"] / INT8_PEAK_TOPS, 2)
+        # the matrix rate the device sustains on a register-only loop of the same MFMA (no memory
+        # traffic): constant operands, and pseudo-random operands as the kernels feed it
+        extra["mfma_i8_peak_const_operands_TOPS"] = round(be.mfma_i8_peak_tops(4, 4096, False), 1)
+        extra["mfma_i8_peak_random_operands_TOPS"] = round(be.mfma_i8_peak_tops(4, 4096, True), 1)
+        extra["mmq_Q4_K_M512_pct_of_measured_mfma_peak"] = round(
+            100 * extra["mmq_Q4_K_M512_TOPS"] / extra["mfma_i8_peak_random_operands_TOPS"], 2)
         # the other formats with an MFMA prefill kernel, at the ffn_down shape 4096 x 12288 (Q6_K there
         # in a Q4_K_M file)
         for name, dt in (("Q6_K", DType.Q6K), ("Q5_K", DType.Q5K), ("Q8_0", DType.Q8_0), ("Q4_0", DType.Q4_0),

@@ -263,6 +263,12 @@ int infr_hip_timer_end(infr_hip_t *be, float *elapsed_ms); /* synchronises */
  * those passes - the read bandwidth this device gives a kernel that only fetches, which the
  * HBM-bound GEMVs are compared with. Synchronises. */
 int infr_hip_stream_read(infr_hip_t *be, const infr_hip_buffer_t *src, size_t bytes, int reps, float *elapsed_ms);
+/* Measurement aid with no counterpart in the reference: `iters` rounds of four independent
+ * v_mfma_i32_32x32x32_i8 per wave, `waves_per_simd` (1..8) waves on every SIMD, operands in registers
+ * (small constants, or pseudo-random bytes when random_data != 0). Reports the device time of one
+ * launch and the integer operations it performed: the int8 matrix rate this device sustains with no
+ * memory traffic, which the prefill kernels are compared with. Synchronises. */
+int infr_hip_mfma_i8_peak(infr_hip_t *be, int waves_per_simd, int iters, int random_data, float *elapsed_ms, double *ops);
 
 /* ---- deterministic synthetic inputs (host side, no device work). The reference has no weight
  * quantizer (it only reads GGUF) and its tests synthesize valid blocks

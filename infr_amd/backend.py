@@ -16,7 +16,8 @@ from enum import IntEnum
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libinfr_hip.so")
+# INFR_HIP_LIB: a measurement build of the library (infr_amd.build with INFR_HIP_BUILD_OUT) instead
+LIB_PATH = os.environ.get("INFR_HIP_LIB") or os.path.join(_HERE, "libinfr_hip.so")
 
 
 class DType(IntEnum):
@@ -136,6 +137,7 @@ SYMBOLS = {
     "infr_hip_timer_begin": (C.c_int, [_vp]),
     "infr_hip_timer_end": (C.c_int, [_vp, C.POINTER(C.c_float)]),
     "infr_hip_stream_read": (C.c_int, [_vp, _vp, C.c_size_t, C.c_int, C.POINTER(C.c_float)]),
+    "infr_hip_mfma_i8_peak": (C.c_int, [_vp, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_double)]),
     "infr_synth_normal_f32": (None, [C.c_uint64, C.c_float, C.c_float, C.c_size_t, _vp]),
     "infr_synth_weight": (C.c_size_t, [C.c_int, C.c_uint64, C.c_float, C.c_size_t, C.c_size_t, _vp]),
     "infr_block_layout": (C.c_int, [C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
@@ -629,6 +631,13 @@ class HipBackend:
         ms = C.c_float()
         self._check(self._lib.infr_hip_stream_read(self._h, buf._h, n, reps, C.byref(ms)))
         return n * reps / (ms.value * 1e-3) / 1e9
+
+    def mfma_i8_peak_tops(self, waves_per_simd: int = 4, iters: int = 4096, random_data: bool = True) -> float:
+        """TOP/s of a register-only int8 MFMA loop (the matrix rate the device sustains by itself)."""
+        ms, ops = C.c_float(), C.c_double()
+        self._check(self._lib.infr_hip_mfma_i8_peak(self._h, waves_per_simd, iters, int(random_data),
+                                                    C.byref(ms), C.byref(ops)))
+        return ops.value / (ms.value * 1e-3) / 1e12
 
     def timer_begin(self) -> None:
         self._check(self._lib.infr_hip_timer_begin(self._h))

@@ -1241,4 +1241,24 @@ int infr_hip_stream_read(infr_hip_t* be, const infr_hip_buffer_t* src, size_t by
     return INFR_HIP_OK;
 }
 
+int infr_hip_mfma_i8_peak(infr_hip_t* be, int waves_per_simd, int iters, int random_data, float* elapsed_ms, double* ops) {
+    if (!be || !elapsed_ms || !ops || waves_per_simd <= 0 || waves_per_simd > 8 || iters <= 0 || iters > (1 << 20))
+        return fail(be, INFR_HIP_ERR_INVALID, "mfma_i8_peak: bad argument");
+    if (int rc = check_latch(be)) return rc;
+    const int wgs = std::max(1, be->props.multiProcessorCount) * waves_per_simd;  // four waves each: one per SIMD
+    int* out = nullptr;
+    HIP_TRY(be, hipMalloc((void**)&out, sizeof(int) * (size_t)wgs));
+    infr::launch_mfma_i8_peak(out, wgs, iters, random_data, be->stream);  // untimed first pass
+    hipError_t e = hipEventRecord(be->ev0, be->stream);
+    if (e == hipSuccess) infr::launch_mfma_i8_peak(out, wgs, iters, random_data, be->stream);
+    if (e == hipSuccess) e = hipEventRecord(be->ev1, be->stream);
+    if (e == hipSuccess) e = hipEventSynchronize(be->ev1);
+    if (e == hipSuccess) e = hipEventElapsedTime(elapsed_ms, be->ev0, be->ev1);
+    if (e == hipSuccess) e = hipGetLastError();
+    (void)hipFree(out);
+    if (e != hipSuccess) return fail(be, INFR_HIP_ERR_BACKEND, std::string("mfma_i8_peak: ") + hipGetErrorString(e));
+    *ops = 2.0 * 32 * 32 * 32 * 4.0 * (double)iters * 4.0 * (double)wgs;
+    return INFR_HIP_OK;
+}
+
 }  // extern "C"

@@ -117,4 +117,40 @@ void launch_stream_read(const void* src, size_t bytes, int* out, int workgroups,
                        static_cast<const v4i*>(src), bytes / 16, out);
 }
 
+// Measurement aid: nothing but v_mfma_i32_32x32x32_i8 on four independent accumulator tiles per
+// wave, `iters` rounds, operands held in registers - the int8 matrix rate this device sustains with
+// no memory traffic at all. random_data = 0 multiplies small constants; 1 fills the operands with
+// pseudo-random bytes (weights-times-digit range on one side, full int8 on the other), which is what
+// the prefill kernels feed the matrix cores and draws more power per instruction.
+__global__ __launch_bounds__(256) void mfma_i8_peak_kernel(int* __restrict__ out, int iters, int random_data) {
+    typedef int v16i __attribute__((ext_vector_type(16)));
+    v4i a = {1, 2, 3, 4}, b = {5, 6, 7, 8};
+    if (random_data) {
+        uint32_t hsh = (threadIdx.x + 1) * 2654435761u + blockIdx.x * 40503u;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            hsh = hsh * 1664525u + 1013904223u;
+            a[i] = (int)(hsh ^ (hsh >> 13));
+            hsh = hsh * 1664525u + 1013904223u;
+            b[i] = (int)((hsh ^ (hsh >> 11)) & 0x3F3F3F3Fu);
+        }
+    }
+    v16i c0 = {}, c1 = {}, c2 = {}, c3 = {};
+    for (int i = 0; i < iters; ++i) {
+        c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c0, 0, 0, 0);
+        c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c1, 0, 0, 0);
+        c2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c2, 0, 0, 0);
+        c3 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c3, 0, 0, 0);
+    }
+    int r = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) r ^= c0[i] ^ c1[i] ^ c2[i] ^ c3[i];
+    if (r == 0x5EEDF00D) out[blockIdx.x] = r;  // keeps the chain alive; practically never taken
+}
+
+void launch_mfma_i8_peak(int* out, int workgroups, int iters, int random_data, hipStream_t stream) {
+    if (workgroups <= 0 || iters <= 0) return;
+    hipLaunchKernelGGL(mfma_i8_peak_kernel, dim3((unsigned)workgroups), dim3(256), 0, stream, out, iters, random_data);
+}
+
 }  // namespace infr

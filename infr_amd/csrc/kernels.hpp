@@ -170,6 +170,7 @@ void launch_embed_gather(int dtype, const uint8_t* table, size_t bpr, size_t tot
 
 // Read-only streaming pass (measurement aid): `out` holds one int per workgroup.
 void launch_stream_read(const void* src, size_t bytes, int* out, int workgroups, hipStream_t stream);
+void launch_mfma_i8_peak(int* out, int workgroups, int iters, int random_data, hipStream_t stream);
 
 // The decode-GEMV launchers of one weight format. Each format's kernels are instantiated in one
 // translation unit, which also defines its accessor below.

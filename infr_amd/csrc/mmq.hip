@@ -202,6 +202,17 @@ struct SharedLds {
     static constexpr int bytes = dd_off + T * 32 * 8;
 };
 
+// Measurement builds only (-DINFR_MMQ_ABLATE=<bits>, results are wrong): take one component out of
+// the shared-operand kernel's loop to see what it costs. 1: the activation fragment loads, 2: the
+// unpack with its row loads and LDS writes, 4: the LDS operand reads after sub-block 0, 8: the f32
+// epilogue (one integer instruction per output instead), 16: the weight row loads alone.
+#ifndef INFR_MMQ_ABLATE
+#define INFR_MMQ_ABLATE 0
+#endif
+#if INFR_MMQ_ABLATE
+#warning "INFR_MMQ_ABLATE is set: mmq_shared_q4k_kernel computes wrong results (measurement build)"
+#endif
+
 template <int T, bool STAGES>
 __global__ __launch_bounds__(256) void mmq_shared_q4k_kernel(
     const uint8_t* __restrict__ w, size_t bpr, const int8_t* __restrict__ qs,
@@ -302,8 +313,11 @@ __global__ __launch_bounds__(256) void mmq_shared_q4k_kernel(
     for (int b = 0; b < nb; ++b) {
         const uint8_t* cur = lds + (b & 1) * L::bytes;
         // ---- unpack block b+1 into the other buffer, then ask for block b+2's bytes ----
-        unpack_to(lds + ((b + 1) & 1) * L::bytes);
-        request_rows(min(b + 2, nb - 1));
+        if (!(INFR_MMQ_ABLATE & 2)) {
+            unpack_to(lds + ((b + 1) & 1) * L::bytes);
+            if (!(INFR_MMQ_ABLATE & 16)) request_rows(min(b + 2, nb - 1));
+            else asm volatile("" : "+v"(hdr[0]), "+v"(qv[0]));
+        }
         // ---- this wave's 32 tokens of block b ----
         const v8h abs_b = abs_;
         if (h == 0) dql[wave][col] = dtok;
@@ -322,7 +336,7 @@ __global__ __launch_bounds__(256) void mmq_shared_q4k_kernel(
 #pragma unroll
         for (int sb = 0; sb < 8; ++sb) {
             v4i nlo[T], nhi[T];
-            if (sb < 7) {
+            if (sb < 7 && !(INFR_MMQ_ABLATE & 4)) {
 #pragma unroll
                 for (int t = 0; t < T; ++t) {
                     const uint8_t* src = cur + (size_t)(((sb + 1) * 2) * T + t) * 1024 + lane * 16;
@@ -335,7 +349,7 @@ __global__ __launch_bounds__(256) void mmq_shared_q4k_kernel(
                 alo[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[sb], flo[t], sb ? alo[t] : zi, 0, 0, 0);
                 ahi[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[sb], fhi[t], sb ? ahi[t] : zi, 0, 0, 0);
             }
-            if (sb < 7) {
+            if (sb < 7 && !(INFR_MMQ_ABLATE & 4)) {
 #pragma unroll
                 for (int t = 0; t < T; ++t) {
                     flo[t] = nlo[t];
@@ -354,7 +368,7 @@ __global__ __launch_bounds__(256) void mmq_shared_q4k_kernel(
         __builtin_amdgcn_s_setprio(0);
         // the activation registers are free: fetch block b+1 while the epilogue runs
         const int b_this = b;
-        request_acts(min(b + 1, nb - 1));
+        if (!(INFR_MMQ_ABLATE & 1)) request_acts(min(b + 1, nb - 1));
 #pragma unroll
         for (int t = 0; t < T; ++t) {
             const v8h bm = *reinterpret_cast<const v8h*>(cur + L::mn_off + (t * 32 + col) * 16);
@@ -378,7 +392,10 @@ __global__ __launch_bounds__(256) void mmq_shared_q4k_kernel(
                         }
                     }
                     // sumf += q8.d[b] * (d * sd as f32 - dmin * sm as f32)
-                    acc[t][r] += dq[i] * (d * (float)sd - dmin * smf[r]);
+                    if (INFR_MMQ_ABLATE & 8)
+                        acc[t][r] = __builtin_bit_cast(float, __builtin_bit_cast(int, acc[t][r]) ^ sd);
+                    else
+                        acc[t][r] += dq[i] * (d * (float)sd - dmin * smf[r]);
                 }
             }
         }

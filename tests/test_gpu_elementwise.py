@@ -123,3 +123,21 @@ def test_shape_and_binding_errors(be):
     g2.push(GatedActFused(a, a, 1, 4, Activation.Sigmoid, swiglu_clamp=1.0))
     with pytest.raises(InfrError):
         be.compile(g2)
+
+
+def test_measurement_probes_report_sane_rates(be):
+    """The two measurement aids (no counterpart in the reference): a register-only int8 MFMA loop and
+    a read-only streaming pass. Both must finish and report a positive rate below the published peaks
+    (5 POP/s int8, 8 TB/s); bad arguments are refused."""
+    from infr_amd import InfrError
+    for random_data in (False, True):
+        tops = be.mfma_i8_peak_tops(2, 256, random_data)
+        assert 10.0 < tops < 5200.0, tops
+    with pytest.raises(InfrError):
+        be.mfma_i8_peak_tops(0, 256, True)
+    with pytest.raises(InfrError):
+        be.mfma_i8_peak_tops(2, 0, True)
+    buf = be.alloc(64 << 20)
+    gbs = be.stream_read_gbs(buf, reps=3)
+    buf.free()
+    assert 100.0 < gbs < 8200.0, gbs
