@@ -148,6 +148,17 @@ class Sweep:
         self.keep = []
 
 
+def settle_clocks(be, plan, binds, seconds=0.03):
+    """Untimed: keep the device loaded with `plan` for ~30 ms so that its clocks have settled
+    (see RAMP_STEPS); every section's timing starts from the same state."""
+    t0 = time.perf_counter()
+    while True:
+        be.execute(plan, binds)
+        be.sync()
+        if time.perf_counter() - t0 > seconds:
+            break
+
+
 def layer_bench(be, n_layers, dtype=None):
     """A decode step through `n_layers` Qwen3-8B-shaped decoder layers without attention:
     RmsNorm -> {q, k, v} -> o(q) -> Add -> RmsNorm -> {gate, up} -> GatedAct -> down -> Add, every op
@@ -203,9 +214,7 @@ def layer_bench(be, n_layers, dtype=None):
         g.push(Add(dn, x, x, H))
     be.sync()
     plan = be.compile(g)
-    for _ in range(2):
-        be.execute(plan, binds)
-    be.sync()
+    settle_clocks(be, plan, binds)
     steps, t0 = 10, time.perf_counter()
     be.timer_begin()
     for _ in range(steps):
@@ -249,13 +258,7 @@ def single_shape(be, dtype, m, in_f, out_f, reps=40, rotate_bytes=768 << 20):
         binds.bind(yid, yb)
         g.push(Linear(xid, wids[i % copies], yid, m, in_f, out_f))
     plan = be.compile(g)
-    # untimed: keep the device loaded for ~30 ms so that its clocks have settled (see RAMP_STEPS)
-    t0 = time.perf_counter()
-    while True:
-        be.execute(plan, binds)
-        be.sync()
-        if time.perf_counter() - t0 > 0.03:
-            break
+    settle_clocks(be, plan, binds)
     best = 1e30
     for _ in range(5):
         be.timer_begin()
@@ -304,8 +307,7 @@ def moe_bench(be, n_layers=6):
             binds.bind(yid, yb)
             g.push(MoeFfn(xid, xid, rid, ids[0], ids[1], ids[2], yid, ne, n_expert, n_used, nff, 1.0))
         plan = be.compile(g)
-        be.execute(plan, binds)
-        be.sync()
+        settle_clocks(be, plan, binds)
         best = 1e30
         for _ in range(3):
             be.timer_begin()
@@ -488,6 +490,7 @@ def main():
             extra[f"mmq_Q4_K_M512_K16384_N{out_f}_TOPS"] = round(2.0 * 512 * out_f * 16384 / (t * 1e-3) / 1e12, 2)
     if "chain" in sections:
         ch = Sweep(be, DType.Q4K, 1, args.layers, chain=True)
+        settle_clocks(be, ch.plan, ch.binds)
         d, w = ch.time(10, 2)
         extra["decode_chain_Q4_K_GBs"] = round(ch.bytes / (max(d, w) * 1e-3) / 1e9, 1)
         extra["decode_chain_launches_per_step"] = ch.plan.launches()
@@ -512,6 +515,7 @@ def main():
                     extra["decode_layer_unfused_launches_per_step"] = ex["decode_layer_launches_per_step"]
     if "ternary" in sections:
         tern = Sweep(be, DType.Q2_0, 1, N_LAYERS, head=True)
+        settle_clocks(be, tern.plan, tern.binds)
         d, w = tern.time(5, 2)
         tms = max(d, w)
         extra["ternary_Q2_0_sweep_GBs"] = round(tern.bytes / (tms * 1e-3) / 1e9, 1)
