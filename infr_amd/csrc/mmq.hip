@@ -213,19 +213,24 @@ struct SharedLds {
 #warning "INFR_MMQ_ABLATE is set: mmq_shared_q4k_kernel computes wrong results (measurement build)"
 #endif
 
-template <int T, bool STAGES>
-__global__ __launch_bounds__(256) void mmq_shared_q4k_kernel(
+template <int T, bool STAGES, int NW = 4>
+__global__ __launch_bounds__(NW * 64) void mmq_shared_q4k_kernel(
     const uint8_t* __restrict__ w, size_t bpr, const int8_t* __restrict__ qs,
     const float* __restrict__ d8, const _Float16* __restrict__ bsh, float* __restrict__ y, int m,
     int out_f, int nb, int32_t* __restrict__ st_sd, int32_t* __restrict__ st_sm) {
     typedef SharedLds<T> L;
     __shared__ __attribute__((aligned(16))) uint8_t lds[2 * L::bytes];
-    __shared__ __attribute__((aligned(16))) float dql[4][32];  // per wave: its tokens' activation scales
+    __shared__ __attribute__((aligned(16))) float dql[NW][32];  // per wave: its tokens' activation scales
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, h = lane >> 5;
-    const int tok0 = blockIdx.y * 128 + wave * 32;
+    const int tok0 = blockIdx.y * (32 * NW) + wave * 32;
     const int row0 = blockIdx.x * (32 * T);
-    const int p = wave;  // the nibble pair this wave unpacks
+    // the nibble pair this wave unpacks; with eight waves (T = 2) the upper four take the second
+    // row tile, so a wave unpacks one tile's pair instead of both
+    static_assert(NW == 4 || (NW == 8 && T == 2), "eight waves split the unpack of two row tiles");
+    const int p = wave & 3;
+    constexpr int TU = NW == 8 ? 1 : T;      // row tiles a wave unpacks
+    const int tu0 = NW == 8 ? wave >> 2 : 0;  // the first of them
 
     const uint8_t* wrowp[T];
     bool row_ok[T];
@@ -240,23 +245,27 @@ __global__ __launch_bounds__(256) void mmq_shared_q4k_kernel(
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[t][i] = 0.0f;
 
-    v4i hdr[T], qv[T];  // raw bytes of the block to unpack next
+    v4i hdr[TU], qv[TU];  // raw bytes of the block to unpack next
+    const uint8_t* urowp[TU];
+#pragma unroll
+    for (int u = 0; u < TU; ++u) urowp[u] = NW == 8 ? (tu0 ? wrowp[T - 1] : wrowp[0]) : wrowp[u];
     auto request_rows = [&](int b) {
 #pragma unroll
-        for (int t = 0; t < T; ++t) {
-            const uint8_t* blk = wrowp[t] + (size_t)b * 144;
-            hdr[t] = load16(blk);
-            qv[t] = load16(blk + 16 + p * 32 + h * 16);
+        for (int u = 0; u < TU; ++u) {
+            const uint8_t* blk = urowp[u] + (size_t)b * 144;
+            hdr[u] = load16(blk);
+            qv[u] = load16(blk + 16 + p * 32 + h * 16);
         }
     };
     auto unpack_to = [&](uint8_t* buf) {
 #pragma unroll
-        for (int t = 0; t < T; ++t) {
+        for (int u = 0; u < TU; ++u) {
+            const int t = tu0 + u;
             uint32_t sc8[2], mn8[2];
-            k4_all((uint32_t)hdr[t].y, (uint32_t)hdr[t].z, (uint32_t)hdr[t].w, sc8, mn8);
+            k4_all((uint32_t)hdr[u].y, (uint32_t)hdr[u].z, (uint32_t)hdr[u].w, sc8, mn8);
             const uint32_t scw = (p & 2) ? sc8[1] : sc8[0], mnw = (p & 2) ? mn8[1] : mn8[0];
             const int sh = (p & 1) * 16;
-            const int qw[4] = {qv[t].x, qv[t].y, qv[t].z, qv[t].w};
+            const int qw[4] = {qv[u].x, qv[u].y, qv[u].z, qv[u].w};
 #pragma unroll
             for (int e = 0; e < 2; ++e) {  // e = 0: sub-block 2p (low nibbles), 1: 2p+1 (high)
                 const uint32_t sc = (scw >> (sh + 8 * e)) & 0xFFu;
@@ -279,8 +288,8 @@ __global__ __launch_bounds__(256) void mmq_shared_q4k_kernel(
                 *reinterpret_cast<h2*>(buf + L::mn_off + (t * 32 + col) * 16 + p * 4) = mn;
                 if (p == 0) {
                     float* dd = reinterpret_cast<float*>(buf + L::dd_off) + (t * 32 + col) * 2;
-                    dd[0] = f16_bits_to_f32((uint32_t)hdr[t].x & 0xFFFFu);
-                    dd[1] = f16_bits_to_f32((uint32_t)hdr[t].x >> 16);
+                    dd[0] = f16_bits_to_f32((uint32_t)hdr[u].x & 0xFFFFu);
+                    dd[1] = f16_bits_to_f32((uint32_t)hdr[u].x >> 16);
                 }
             }
         }
@@ -290,7 +299,7 @@ __global__ __launch_bounds__(256) void mmq_shared_q4k_kernel(
     v8h abs_;  // split per-32 sums: the h = 0 lanes carry bsum & 63, the h = 1 lanes the rest
     float dtok;
     // this wave's group of 32 tokens; a wave wholly past m recomputes the last group (nothing is stored)
-    const size_t g = min((size_t)blockIdx.y * 4 + wave, (size_t)(m - 1) / 32);
+    const size_t g = min((size_t)blockIdx.y * NW + wave, (size_t)(m - 1) / 32);
     auto request_acts = [&](int b) {
         const size_t gb = g * nb + b;
         const int8_t* ap = qs + gb * (8 * 1024) + lane * 16;
@@ -414,16 +423,16 @@ __global__ __launch_bounds__(256) void mmq_shared_q4k_kernel(
     }
 }
 
-template <int T>
+template <int T, int NW = 4>
 static void launch_mmq_shared_q4k(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
                                   size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream) {
-    const dim3 grid((unsigned)((out_f + 32 * T - 1) / (32 * T)), (unsigned)((m + 127) / 128)), block(256);
+    const dim3 grid((unsigned)((out_f + 32 * T - 1) / (32 * T)), (unsigned)((m + 32 * NW - 1) / (32 * NW))), block(NW * 64);
     const int nb = (int)(in_f / 256);
     if (st.a)
-        hipLaunchKernelGGL((mmq_shared_q4k_kernel<T, true>), grid, block, 0, stream, w, bpr, act.qs, act.d,
+        hipLaunchKernelGGL((mmq_shared_q4k_kernel<T, true, NW>), grid, block, 0, stream, w, bpr, act.qs, act.d,
                            reinterpret_cast<const _Float16*>(act.bsums), y, (int)m, (int)out_f, nb, st.a, st.b);
     else
-        hipLaunchKernelGGL((mmq_shared_q4k_kernel<T, false>), grid, block, 0, stream, w, bpr, act.qs, act.d,
+        hipLaunchKernelGGL((mmq_shared_q4k_kernel<T, false, NW>), grid, block, 0, stream, w, bpr, act.qs, act.d,
                            reinterpret_cast<const _Float16*>(act.bsums), y, (int)m, (int)out_f, nb, (int32_t*)nullptr, (int32_t*)nullptr);
 }
 
@@ -1148,7 +1157,12 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
     if (dtype == 12 && ((int)m >= env_shared_min || long_row)) {
         launch_quantize_q8_tiled(x, m, in_f, act, stream);
         const bool wide = env_shared_rows ? env_shared_rows == 64 : m >= 1024;
-        if (wide) launch_mmq_shared_q4k<2>(w, bpr, act, y, m, in_f, out_f, st, stream);
+        // two row tiles: eight waves (256 tokens) per workgroup, each unpacking one tile's nibble pair -
+        // half the unpack work and row loads per output tile; 729 / 763 / 766 against 669 / 719 / 731
+        // TOPS at 1024 / 2048 / 4096 tokens (12288 x 4096)
+        static const int env_w8 = getenv("INFR_HIP_MMQ_SHARED_WAVES") ? atoi(getenv("INFR_HIP_MMQ_SHARED_WAVES")) : 8;
+        if (wide && env_w8 == 8) launch_mmq_shared_q4k<2, 8>(w, bpr, act, y, m, in_f, out_f, st, stream);
+        else if (wide) launch_mmq_shared_q4k<2>(w, bpr, act, y, m, in_f, out_f, st, stream);
         else launch_mmq_shared_q4k<1>(w, bpr, act, y, m, in_f, out_f, st, stream);
         return true;
     }

@@ -108,7 +108,9 @@ def test_w_off_selects_rows_of_a_concatenated_weight(be):
 
 # ───────────── prefill (m >= 2): int8 MFMA path for Q4_K ─────────────
 
-PREFILL_SHAPES = [(2, 256, 8), (8, 1024, 96), (33, 512, 200), (64, 1024, 256), (130, 768, 130), (257, 2048, 384)]
+# 1024 and above: 64 rows x 256 tokens on eight waves (a ragged last tile in both directions)
+PREFILL_SHAPES = [(2, 256, 8), (8, 1024, 96), (33, 512, 200), (64, 1024, 256), (130, 768, 130), (257, 2048, 384),
+                  (1024, 256, 64), (1059, 512, 72)]
 
 
 @pytest.mark.parametrize("m,in_f,out_f", PREFILL_SHAPES)
@@ -156,7 +158,7 @@ def test_small_batch_kquant_mfma_int_stages_bit_exact(be, dtype, seed, m, in_f, 
         assert np.array_equal(b, ob)
 
 
-@pytest.mark.parametrize("m,in_f,out_f", [(5, 512, 40), (70, 768, 150)])
+@pytest.mark.parametrize("m,in_f,out_f", [(5, 512, 40), (70, 768, 150), (200, 512, 40), (1030, 256, 70)])
 def test_prefill_q4k_int_stages_bit_exact(be, m, in_f, out_f):
     # full-range payload bytes: every scale, min and code value occurs (sc up to 63 exercises the
     # split-scale operands, large |bsums| the split sums)
