@@ -62,6 +62,41 @@ def test_quantize_q8_32_bit_exact(be, m, k):
 DECODE_SHAPES = [(256, 8), (768, 37), (4096, 1024), (12288, 512), (2048, 100), (5120, 64)]
 
 
+def test_headline_configuration_q4k_4096x4096(be):
+    """The benchmark's own CPU-runnable case: W[4096, 4096] ~ N(0, 0.02^2) from seed 0 as Q4_K, x[1, 4096]
+    ~ N(0, 1) from seed 1; activation codes and block integers bit-exact, y bit-identical."""
+    n = k = 4096
+    w = synth_weight(DType.Q4K, 0, n, k, 0.02)
+    x = synth_normal_f32(1, k)
+    qs, d, bs, _ = be.quantize_q8(be.upload_new(x), 1, k)
+    o = orc.quantize_q8(x)
+    assert np.array_equal(qs[0], o.qs) and np.array_equal(d[0].view(np.uint32), o.d.view(np.uint32))
+    assert np.array_equal(bs[0], o.bsums)
+    a, b = be.linear_int_stages(DType.Q4K, be.upload_new(w), be.upload_new(x), 1, k, n)
+    oa, ob = orc.linear_int_stages(DType.Q4K, w, x, 1, k, n)
+    assert np.array_equal(a, oa) and np.array_equal(b, ob)
+    y = run_linear(be, DType.Q4K, w, x, 1, k, n)
+    want = orc.linear(DType.Q4K, w, x, 1, k, n)
+    gate(y, want)
+    assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), "not bit-identical"
+
+
+# the decode set at Qwen3-8B layer shapes, batch 1 and 8 (rows cut to 256: a row's arithmetic does not
+# depend on how many rows there are, and the oracle stays within seconds)
+@pytest.mark.parametrize("dtype", [DType.Q4K, DType.Q6K, DType.Q8_0])
+@pytest.mark.parametrize("m", [1, 8])
+@pytest.mark.parametrize("in_f", [4096, 12288])
+def test_decode_set_shapes_batch_1_and_8(be, dtype, m, in_f):
+    out_f = 256
+    w = synth_weight(dtype, 0, out_f, in_f, 0.02)
+    x = synth_normal_f32(1, m * in_f)
+    y = run_linear(be, dtype, w, x, m, in_f, out_f)
+    want = orc.linear(dtype, w, x, m, in_f, out_f)
+    gate(y, want)
+    if dtype in (DType.Q4K, DType.Q6K):
+        assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), "not bit-identical"
+
+
 @pytest.mark.parametrize("dtype", [DType.Q4K, DType.Q6K, DType.Q8_0, DType.Q2_0])
 @pytest.mark.parametrize("in_f,out_f", DECODE_SHAPES)
 def test_decode_gemv_vs_oracle(be, dtype, in_f, out_f):
