@@ -135,12 +135,26 @@ __device__ __forceinline__ void moe_select_block(const float* __restrict__ l, Se
 
 // One workgroup per row (used when there are several rows; a single row is selected by the
 // router kernel itself).
+// When x is given, the workgroup first quantizes its row of the expert input (per-256 `Q8`, the
+// layout of quantize_q8_kernel; ne a multiple of 256): one launch less in front of the expert GEMVs.
 __global__ __launch_bounds__(256) void moe_select_kernel(const float* __restrict__ logits,
                                                          int32_t* __restrict__ sel_idx,
                                                          float* __restrict__ sel_w, int n_expert,
-                                                         int n_used, float scale) {
+                                                         int n_used, float scale,
+                                                         const float* __restrict__ x, int ne,
+                                                         int8_t* __restrict__ qs, float* __restrict__ qd,
+                                                         int32_t* __restrict__ bsums,
+                                                         int32_t* __restrict__ bsums16) {
     __shared__ __attribute__((aligned(16))) SelectLds s;
     const size_t r = blockIdx.x;
+    if (x) {
+        const int lane = threadIdx.x & 63, nchunk = ne / 256;
+        for (int c = threadIdx.x >> 6; c < nchunk; c += 4) {  // wave-uniform
+            const size_t chunk = r * nchunk + c;
+            const v4f v = *reinterpret_cast<const v4f*>(x + chunk * 256 + (size_t)lane * 4);
+            quantize_chunk<false>(v, true, lane, chunk, qs, qd, bsums, bsums16);
+        }
+    }
     moe_select_block(logits + r * n_expert, s, n_expert, n_used, scale, threadIdx.x, sel_idx + r * n_used,
                      sel_w + r * n_used);
 }
@@ -925,9 +939,13 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
                            dim3(256), router_lds, stream, b.router, b.router_x, logits,
                            s.rows == 1 ? tickets : nullptr, sel_idx, sel_w, s.ne, s.n_expert, s.rows, s.n_used,
                            s.scale, kc, epw);
+    // the expert input is quantized by the selection kernel's workgroups (one per row) when its rows
+    // are whole 256s
+    const bool quant_in_select = s.rows > 1 && s.ne % 256 == 0;
     if (s.rows > 1)
         hipLaunchKernelGGL(moe_select_kernel, dim3((unsigned)s.rows), dim3(256), 0, stream, logits, sel_idx,
-                           sel_w, s.n_expert, s.n_used, s.scale);
+                           sel_w, s.n_expert, s.n_used, s.scale, quant_in_select ? b.x : (const float*)nullptr,
+                           s.ne, aq.qs, aq.d, aq.bsums, aq.bsums16);
     if (b.sel_idx) (void)hipMemcpyAsync(b.sel_idx, sel_idx, pairs * 4, hipMemcpyDeviceToDevice, stream);
     if (b.sel_w) (void)hipMemcpyAsync(b.sel_w, sel_w, pairs * 4, hipMemcpyDeviceToDevice, stream);
 
@@ -980,7 +998,7 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     const size_t gbpr = bytes_per_row(s.gate_dtype, s.ne), ubpr = bytes_per_row(s.up_dtype, s.ne);
     const size_t dbpr = bytes_per_row(s.down_dtype, s.n_ff);
     if (!gbpr || !ubpr || !dbpr) return "rows >= 2 carries Q4_K / Q5_K / Q6_K / Q8_0 expert banks";
-    launch_quantize_q8(b.x, s.rows, s.ne, false, aq, stream);
+    if (!quant_in_select) launch_quantize_q8(b.x, s.rows, s.ne, false, aq, stream);
     const size_t n_act = pairs * s.n_ff, n_out = (size_t)s.rows * s.ne;
     // Prefill-sized batches: the pairs are bucketed by expert and every bank runs its format's
     // int8-MFMA GEMM per (expert, 32 pairs) tile, so an expert's weights are read once per 32 of
