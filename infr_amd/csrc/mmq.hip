@@ -1156,7 +1156,12 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
     static const int env_shared_rows = getenv("INFR_HIP_MMQ_SHARED_ROWS") ? atoi(getenv("INFR_HIP_MMQ_SHARED_ROWS")) : 0;
     if (dtype == 12 && ((int)m >= env_shared_min || long_row)) {
         launch_quantize_q8_tiled(x, m, in_f, act, stream);
-        const bool wide = env_shared_rows ? env_shared_rows == 64 : m >= 1024;
+        // (896 / 1000 tokens at 12288 x 4096: 658 / 730 against 622 / 627 TOPS; at 768 and below the
+        // 32-row form is ahead)
+        // 256-token tiles pad up to 128 tokens more than 128-token tiles do: taken when both pad alike,
+        // or when that padding is small against the batch
+        const size_t pad_w = (m + 255) / 256 * 256, pad_n = (m + 127) / 128 * 128;
+        const bool wide = env_shared_rows ? env_shared_rows == 64 : (m > 768 && (pad_w == pad_n || pad_w >= 2048));
         // two row tiles: eight waves (256 tokens) per workgroup, each unpacking one tile's nibble pair -
         // half the unpack work and row loads per output tile; 729 / 763 / 766 against 669 / 719 / 731
         // TOPS at 1024 / 2048 / 4096 tokens (12288 x 4096)

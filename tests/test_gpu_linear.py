@@ -143,9 +143,10 @@ def test_w_off_selects_rows_of_a_concatenated_weight(be):
 
 # ───────────── prefill (m >= 2): int8 MFMA path for Q4_K ─────────────
 
-# 1024 and above: 64 rows x 256 tokens on eight waves (a ragged last tile in both directions)
+# above 768 tokens: 64 rows x 256 tokens on eight waves where the padding allows (ragged last tiles in both
+# directions), else the 32-row form
 PREFILL_SHAPES = [(2, 256, 8), (8, 1024, 96), (33, 512, 200), (64, 1024, 256), (130, 768, 130), (257, 2048, 384),
-                  (1024, 256, 64), (1059, 512, 72)]
+                  (800, 256, 64), (900, 256, 64), (1024, 256, 64), (1200, 512, 72), (2100, 256, 40)]
 
 
 @pytest.mark.parametrize("m,in_f,out_f", PREFILL_SHAPES)
