@@ -75,7 +75,9 @@ typedef struct {
     int i8_dot;               /* packed 4x int8 dot (v_dot4) */
     int coopmat_i8_m, coopmat_i8_n, coopmat_i8_k; /* int8 MFMA tile */
     int decode_replay;        /* execute() replays a recorded launch sequence */
-    int combined_gu, embed_gather, gpu_sample, argmax_rows, gated_rmsnorm; /* all 0: plain ops */
+    int combined_gu;          /* 1: Linear onto [gate | up] + Op::GatedActFused (backend.rs:160-164) */
+    int embed_gather;         /* 1: Op::EmbedGather decodes table rows on the device */
+    int gpu_sample, argmax_rows, gated_rmsnorm; /* 0: the runner keeps these on the host */
     int graph_input_inplace;
     int unified_memory;
     uint64_t device_memory_bytes;

@@ -28,6 +28,7 @@ struct infr_hip_plan {
     // decode replay: launch sequence recorded for one set of bound device addresses
     hipGraphExec_t exec = nullptr;
     std::vector<void*> bound;
+    uint64_t scratch_epoch = 0;  // the backend's scratch epoch the recording was made under
     // Launch schedule for the bound addresses: ops ordered by dependency level; the m == 1 ops
     // of a level that share (dtype, in_f) form one grouped decode launch.
     struct Step {
@@ -70,6 +71,10 @@ struct infr_hip {
     // MoE scratch
     void* moe_ws = nullptr;
     size_t moe_ws_bytes = 0;
+    // Counts reallocations of the scratch above. A recorded launch sequence carries the scratch
+    // addresses in its kernel arguments, so a plan replays only while the epoch it was recorded
+    // under is still current (Internal scratch is the backend's to keep valid, backend.rs:8-13).
+    uint64_t scratch_epoch = 0;
 };
 
 namespace {
@@ -232,6 +237,7 @@ static int upload_table(infr_hip_t* be, const std::vector<T>& host, T** dev, siz
 int ensure_act(infr_hip_t* be, size_t elems) {
     if (elems <= be->act_cap_elems) return INFR_HIP_OK;
     HIP_TRY(be, hipStreamSynchronize(be->stream));
+    ++be->scratch_epoch;
     if (be->act.qs) {
         (void)hipFree(be->act.qs);
         (void)hipFree(be->act.d);
@@ -434,6 +440,8 @@ int infr_hip_capabilities(const infr_hip_t* be, infr_hip_caps_t* out) {
     out->coopmat_i8_n = 32;
     out->coopmat_i8_k = 32;
     out->decode_replay = 1;
+    out->combined_gu = 1;   // a Linear onto [gate | up] followed by Op::GatedActFused is a plan op here
+    out->embed_gather = 1;  // Op::EmbedGather decodes table rows on the device
     out->graph_input_inplace = 1;
     out->unified_memory = 0;
     out->device_memory_bytes = be->props.totalGlobalMem;
@@ -654,6 +662,7 @@ int infr_hip_quantize_q8_32(infr_hip_t* be, const infr_hip_buffer_t* x, size_t m
 static int ensure_moe_ws(infr_hip_t* be, size_t bytes) {
     if (bytes <= be->moe_ws_bytes) return INFR_HIP_OK;
     HIP_TRY(be, hipStreamSynchronize(be->stream));
+    ++be->scratch_epoch;
     if (be->moe_ws) (void)hipFree(be->moe_ws);
     be->moe_ws = nullptr;
     be->moe_ws_bytes = 0;
@@ -909,13 +918,28 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
         const auto& p = plan->ops[k];
         const bool gated = (p.kind == INFR_OP_GATED_ACT && p.gate_block_width == 0) || p.kind == INFR_OP_GATED_ACT_FUSED;
         if (!(gated || p.kind == INFR_OP_RMS_NORM) || p.m != 1 || p.in_f % 4 != 0) continue;
-        // every reader of the producer's dst must be a later decode Linear taking exactly that
-        // vector as x, with the producer's inputs and dst untouched in between
+        // A producer that runs in place (dst overlapping one of its inputs) cannot be absorbed:
+        // every workgroup of the consumer re-reads the producer's inputs while the first one
+        // stores dst, so later workgroups would apply the op to its own result.
+        if (any_overlap(wr[k], rd[k])) continue;
+        // The definition's live range ends at the next op that overwrites dst (scratch tensors
+        // are reused from layer to layer, graph.rs:10-14): readers beyond it see that op's value.
+        // An op that overwrites only part of dst keeps the whole plan as the range.
+        size_t end = n - 1;
+        for (size_t j = k + 1; j < n; ++j) {
+            if (!any_overlap(wr[j], wr[k])) continue;
+            bool covers = false;
+            for (const auto& w : wr[j]) covers = covers || (w.lo <= wr[k][0].lo && w.hi >= wr[k][0].hi);
+            if (covers) end = j;
+            break;
+        }
+        // every reader of this definition must be a decode Linear taking exactly that vector as
+        // x, with the producer's inputs and dst untouched up to the last of them
         std::vector<size_t> users;
         bool ok = true;
-        for (size_t i = 0; ok && i < n; ++i) {
-            if (i == k || !any_overlap(rd[i], wr[k])) continue;
-            ok = i > k && decode_linear(i) && plan->ops[i].in_f == p.in_f &&
+        for (size_t i = k + 1; ok && i <= end; ++i) {
+            if (!any_overlap(rd[i], wr[k])) continue;
+            ok = decode_linear(i) && plan->ops[i].in_f == p.in_f &&
                  static_cast<const float*>(bindings[plan->ops[i].x]->ptr) == ea[k].dst;
             if (ok) users.push_back(i);
         }
@@ -1155,7 +1179,7 @@ int infr_hip_execute(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t* c
     // Replay when every bound device address is what the recording saw.
     std::vector<void*> now(n_bindings);
     for (size_t i = 0; i < n_bindings; ++i) now[i] = bindings[i] ? bindings[i]->ptr : nullptr;
-    if (plan->exec && now == plan->bound) {
+    if (plan->exec && now == plan->bound && plan->scratch_epoch == be->scratch_epoch) {
         HIP_TRY(be, hipGraphLaunch(plan->exec, be->stream));
         return INFR_HIP_OK;
     }
@@ -1194,6 +1218,7 @@ int infr_hip_execute(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t* c
         return fail(be, INFR_HIP_ERR_BACKEND, std::string("hipGraphInstantiate: ") + hipGetErrorString(e));
     }
     plan->bound = now;
+    plan->scratch_epoch = be->scratch_epoch;
     HIP_TRY(be, hipGraphLaunch(plan->exec, be->stream));
     return INFR_HIP_OK;
 }

@@ -298,6 +298,9 @@ static void hip_backend_honours_the_seam_contract(HipBackend& be) {
     EXPECT(!be.name().empty(), "name");
     const Capabilities caps = be.capabilities();
     EXPECT(caps.i8 && caps.i8_dot && caps.decode_replay, "capabilities");
+    // both ops are built here, so the runner may emit them (backend.rs:160-164)
+    EXPECT(caps.combined_gu == 1 && caps.embed_gather == 1, "combined_gu / embed_gather are advertised");
+    EXPECT(caps.gpu_sample == 0 && caps.argmax_rows == 0 && caps.gated_rmsnorm == 0, "host-side ops stay off");
     // alloc is zero-initialised (calloc semantics, backend.rs:491-496)
     Buffer z = be.alloc(4096, BufferUsage::Activations);
     std::vector<uint8_t> host(4096, 0xAB);

@@ -265,3 +265,185 @@ def test_fusion_is_refused_when_it_would_reorder_a_dependency(be):
     assert np.array_equal(bits(y), bits(orc.linear(DType.Q4K, w_host, h, 1, H, H).ravel()))
     want_r = orc.add(y, orc.add(r0, r0))
     assert np.array_equal(bits(be.download(b["r"], np.empty(H, np.float32))), bits(want_r))
+
+
+def test_in_place_producers_are_not_absorbed(be):
+    """The runner emits in-place producers at decode (GatedAct{gate: g, dst: g} followed by
+    Linear{x: g}, crates/infr-llama/src/seam/runner.rs:4305-4326). Every workgroup of an
+    absorbing GEMV would re-read the producer's input while the first one overwrites it, so such
+    producers run as their own launch: outputs equal the oracle's on the first execute and on replays."""
+    from infr_amd import Activation, GatedAct, RmsNorm
+    H, KV, FF = 1024, 256, 4096
+    g, binds = Graph(), Bindings()
+    x, nw = g.input(TensorDesc((1, H), DType.F32)), g.input(TensorDesc((H,), DType.F32))
+    gate, up = g.input(TensorDesc((1, FF), DType.F32)), g.input(TensorDesc((1, FF), DType.F32))
+    xb, gb = be.alloc(H * 4), be.alloc(FF * 4)
+    nw_h = synth_normal_f32(2, H) * np.float32(0.1) + np.float32(1.0)
+    up_h = synth_normal_f32(3, FF)
+    binds.bind(x, xb).bind(nw, be.upload_new(nw_h)).bind(gate, gb).bind(up, be.upload_new(up_h))
+    ws, outs = {}, {}
+    for nm, dt, out_f, in_f in [("q", DType.Q4K, H, H), ("k", DType.Q4K, KV, H), ("v", DType.Q6K, KV, H),
+                                ("down", DType.Q4K, 3072, FF)]:
+        ws[nm] = synth_weight(dt, 20 + len(ws), out_f, in_f, 0.05)
+        wid = g.weight(TensorDesc((out_f, in_f), dt))
+        oid = g.output(TensorDesc((1, out_f), DType.F32))
+        outs[nm] = (dt, out_f, in_f, be.alloc(out_f * 4))
+        binds.bind(wid, be.upload_new(ws[nm])).bind(oid, outs[nm][3])
+        outs[nm] += (wid, oid)
+    g.push(RmsNorm(x, nw, x, 1, H, 1e-6))                       # in place: x = rmsnorm(x) * w
+    for nm in ("q", "k", "v"):
+        g.push(Linear(x, outs[nm][4], outs[nm][5], 1, H, outs[nm][1]))
+    g.push(GatedAct(gate, up, gate, 1, FF, act=int(Activation.Gelu)))   # in place: gate = gelu(gate) * up
+    g.push(Linear(gate, outs["down"][4], outs["down"][5], 1, FF, 3072))  # 3072 rows: many workgroups
+    plan = be.compile(g)
+    for rep in range(3):
+        x0, g0 = synth_normal_f32(40 + rep, H), synth_normal_f32(50 + rep, FF)
+        be.upload(xb, x0)
+        be.upload(gb, g0)
+        be.execute(plan, binds)
+        assert plan.launches() == 5, plan.launches()             # norm, {q, k}, v, act, down
+        h = be.download(xb, np.empty(H, np.float32))
+        a = be.download(gb, np.empty(FF, np.float32))
+        assert _rel(h, orc.rms_norm(x0, nw_h, 1, H, 1e-6)) < 2e-6
+        assert _rel(a, orc.gated_act(g0, up_h, 1, FF, int(Activation.Gelu))) < 2e-6
+        for nm, src in (("q", h), ("k", h), ("v", h), ("down", a)):
+            dt, out_f, in_f, buf = outs[nm][:4]
+            got = be.download(buf, np.empty(out_f, np.float32))
+            want = orc.linear(dt, ws[nm], src, 1, in_f, out_f).ravel()
+            assert np.array_equal(bits(got), bits(want)), f"{nm} differs on execute {rep}"
+
+
+def test_two_layers_sharing_scratch_tensors_still_fuse(be):
+    """The runner reuses the norm / gate / act scratch tensors from layer to layer
+    (crates/infr-core/src/graph.rs:10-14). A producer's readers are those up to the next op that
+    overwrites its dst, so each layer's norm and gated activation are absorbed: two layers of
+    norm -> {gate, up} -> act -> down -> add run in four launches, not ten."""
+    from infr_amd import Add, GatedAct, RmsNorm
+    H, FF, L = 512, 1536, 2
+    g, binds, host = Graph(), Bindings(), {}
+    x = g.input(TensorDesc((1, H), DType.F32))
+    xb = be.alloc(H * 4)
+    binds.bind(x, xb)
+    scratch = {}
+    for nm, n in (("xn", H), ("gate", FF), ("up", FF), ("act", FF), ("down", H)):
+        scratch[nm] = (g.output(TensorDesc((1, n), DType.F32)), be.alloc(n * 4))
+        binds.bind(*scratch[nm])
+    for l in range(L):
+        host[l] = {"nw": synth_normal_f32(100 + l, H) * np.float32(0.1) + np.float32(1.0)}
+        nw = g.input(TensorDesc((H,), DType.F32))
+        binds.bind(nw, be.upload_new(host[l]["nw"]))
+        wid = {}
+        for nm, out_f, in_f in (("wg", FF, H), ("wu", FF, H), ("wd", H, FF)):
+            host[l][nm] = synth_weight(DType.Q4K, 110 + 10 * l + len(wid), out_f, in_f, 0.05)
+            wid[nm] = g.weight(TensorDesc((out_f, in_f), DType.Q4K))
+            binds.bind(wid[nm], be.upload_new(host[l][nm]))
+        g.push(RmsNorm(x, nw, scratch["xn"][0], 1, H, 1e-6))
+        g.push(Linear(scratch["xn"][0], wid["wg"], scratch["gate"][0], 1, H, FF))
+        g.push(Linear(scratch["xn"][0], wid["wu"], scratch["up"][0], 1, H, FF))
+        g.push(GatedAct(scratch["gate"][0], scratch["up"][0], scratch["act"][0], 1, FF))
+        g.push(Linear(scratch["act"][0], wid["wd"], scratch["down"][0], 1, FF, H))
+        g.push(Add(scratch["down"][0], x, x, H))
+    plan = be.compile(g)
+    for rep in range(3):
+        x0 = synth_normal_f32(300 + rep, H)
+        be.upload(xb, x0)
+        be.execute(plan, binds)
+        assert plan.launches() == 2 * L, plan.launches()
+        # the oracle chain, each stage fed the previous stage's oracle value: the absorbed norm and
+        # activation differ from the stand-alone ops by ~1e-7 relative, the gate is 1e-4 end to end
+        xr = x0
+        for l in range(L):
+            xn = orc.rms_norm(xr, host[l]["nw"], 1, H, 1e-6)
+            gt = orc.linear(DType.Q4K, host[l]["wg"], xn, 1, H, FF)
+            up = orc.linear(DType.Q4K, host[l]["wu"], xn, 1, H, FF)
+            act = orc.gated_act(gt, up, 1, FF)
+            dn = orc.linear(DType.Q4K, host[l]["wd"], act, 1, FF, H)
+            xr = orc.add(dn, xr)
+        got = be.download(xb, np.empty(H, np.float32))
+        assert _rel(got, xr) < 1e-4, _rel(got, xr)
+        # the scratch tensors hold the LAST layer's values, as in program order
+        assert _rel(be.download(scratch["act"][1], np.empty(FF, np.float32)), act) < 1e-4
+        assert _rel(be.download(scratch["xn"][1], np.empty(H, np.float32)), xn) < 1e-4
+
+
+def test_plans_survive_backend_scratch_regrowth(be):
+    """A recorded plan carries the backend's scratch addresses. Compiling a plan that needs far more
+    scratch reallocates it, so the first plan must be recorded again instead of replaying launches
+    that point at freed memory (Internal scratch is the backend's to keep valid,
+    crates/infr-core/src/backend.rs:8-13)."""
+    from infr_amd import HipBackend, MoeFfn
+    own = HipBackend(0)          # a backend of its own, so the scratch starts small
+    try:
+        ne, n_expert, n_used, nff, rows = 512, 16, 4, 256, 2
+        in_f, out_f, m = 512, 384, 8
+        w = synth_weight(DType.Q6K, 1, out_f, in_f, 0.05)
+        router = synth_normal_f32(2, n_expert * ne, sigma=0.05)
+        gate = synth_weight(DType.Q4K, 3, n_expert * nff, ne, 0.05)
+        up = synth_weight(DType.Q4K, 4, n_expert * nff, ne, 0.05)
+        down = synth_weight(DType.Q4K, 5, n_expert * ne, nff, 0.05)
+        g, binds = Graph(), Bindings()
+        x = g.input(TensorDesc((m, in_f), DType.F32))
+        mx = g.input(TensorDesc((rows, ne), DType.F32))
+        xb, mxb = own.alloc(m * in_f * 4), own.alloc(rows * ne * 4)
+        y, my = g.output(TensorDesc((m, out_f), DType.F32)), g.output(TensorDesc((rows, ne), DType.F32))
+        yb, myb = own.alloc(m * out_f * 4), own.alloc(rows * ne * 4)
+        wid, rid = g.weight(TensorDesc((out_f, in_f), DType.Q6K)), g.weight(TensorDesc((n_expert, ne), DType.F32))
+        gid, uid = (g.weight(TensorDesc((n_expert, nff, ne), DType.Q4K)) for _ in range(2))
+        did = g.weight(TensorDesc((n_expert, ne, nff), DType.Q4K))
+        binds.bind(x, xb).bind(mx, mxb).bind(y, yb).bind(my, myb).bind(wid, own.upload_new(w))
+        binds.bind(rid, own.upload_new(router)).bind(gid, own.upload_new(gate)).bind(uid, own.upload_new(up))
+        binds.bind(did, own.upload_new(down))
+        g.push(Linear(x, wid, y, m, in_f, out_f))
+        g.push(MoeFfn(mx, mx, rid, gid, uid, did, my, ne, n_expert, n_used, nff))
+        plan_a = own.compile(g)
+
+        def run_a(seed):
+            x0, mx0 = synth_normal_f32(seed, m * in_f), synth_normal_f32(seed + 1, rows * ne)
+            own.upload(xb, x0)
+            own.upload(mxb, mx0)
+            own.execute(plan_a, binds)
+            got = own.download(yb, np.empty((m, out_f), np.float32))
+            assert np.array_equal(bits(got), bits(orc.linear(DType.Q6K, w, x0, m, in_f, out_f)))
+            want, _, _ = orc.moe_ffn(mx0, router, gate, up, down, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff)
+            assert _rel(own.download(myb, np.empty((rows, ne), np.float32)), want) < 1e-4
+
+        run_a(10)
+        run_a(20)                                            # a replay
+        # plan B: 600 tokens of a longer row and a 300-row MoE need far larger scratch
+        gB, bB = Graph(), Bindings()
+        mB, kB, nB, rB = 600, 2048, 256, 300
+        wB = synth_weight(DType.Q4K, 7, nB, kB, 0.05)
+        xB, yB = gB.input(TensorDesc((mB, kB), DType.F32)), gB.output(TensorDesc((mB, nB), DType.F32))
+        xBh = synth_normal_f32(8, mB * kB)
+        yBb = own.alloc(mB * nB * 4)
+        wBid = gB.weight(TensorDesc((nB, kB), DType.Q4K))
+        mxB, myB = gB.input(TensorDesc((rB, ne), DType.F32)), gB.output(TensorDesc((rB, ne), DType.F32))
+        mxBh = synth_normal_f32(9, rB * ne)
+        myBb = own.alloc(rB * ne * 4)
+        bB.bind(xB, own.upload_new(xBh)).bind(yB, yBb).bind(wBid, own.upload_new(wB))
+        bB.bind(mxB, own.upload_new(mxBh)).bind(myB, myBb)
+        ids = []
+        for arr, shape, dt in ((router, (n_expert, ne), DType.F32), (gate, (n_expert, nff, ne), DType.Q4K),
+                               (up, (n_expert, nff, ne), DType.Q4K), (down, (n_expert, ne, nff), DType.Q4K)):
+            ids.append(gB.weight(TensorDesc(shape, dt)))
+            bB.bind(ids[-1], own.upload_new(arr))
+        gB.push(Linear(xB, wBid, yB, mB, kB, nB))
+        gB.push(MoeFfn(mxB, mxB, ids[0], ids[1], ids[2], ids[3], myB, ne, n_expert, n_used, nff))
+        plan_b = own.compile(gB)
+        own.execute(plan_b, bB)
+        gotB = own.download(yBb, np.empty((mB, nB), np.float32))
+        rows_chk = [0, 1, 31, 32, 299, 599]
+        wantB = orc.linear(DType.Q4K, wB, xBh.reshape(mB, kB)[rows_chk].ravel(), len(rows_chk), kB, nB)
+        assert np.array_equal(bits(gotB[rows_chk]), bits(wantB))
+        run_a(30)                                            # plan A after the scratch moved
+        run_a(40)
+        own.execute(plan_b, bB)                              # and B again, replayed
+        assert np.array_equal(bits(own.download(yBb, np.empty((mB, nB), np.float32))[rows_chk]), bits(wantB))
+    finally:
+        own.close()
+
+
+def test_capabilities_advertise_the_ops_that_are_built(be):
+    caps = be.capabilities()
+    assert caps["combined_gu"] == 1 and caps["embed_gather"] == 1 and caps["decode_replay"] == 1
+    assert caps["gpu_sample"] == 0 and caps["argmax_rows"] == 0 and caps["gated_rmsnorm"] == 0
