@@ -139,6 +139,21 @@ int infr_hip_linear(infr_hip_t *be, int dtype, const infr_hip_buffer_t *w, size_
                     size_t w_off, const infr_hip_buffer_t *x, infr_hip_buffer_t *dst, size_t m,
                     size_t in_f, size_t out_f);
 
+/* Op::Linear without any device allocation. No counterpart in the reference: it is for callers
+ * that cannot allocate device memory around the call - code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc. Arguments, kernels and results are those of
+ * infr_hip_linear; the quantized activation of m >= 2 goes into a static device array of the
+ * library instead of the backend's grow-on-demand scratch, so ceil32(m) * in_f must not exceed
+ * 4,194,304 elements (e.g. 1024 tokens of 4096), else INFR_HIP_ERR_UNSUPPORTED. Each GPU holds one
+ * such array (6 MiB) until the process ends and every backend on that GPU shares it: calls that
+ * overlap on one GPU, from different backends or streams, race. The array keeps the last call's
+ * contents and nothing needs clearing: the quantizer writes every slot of the m tokens, and what
+ * the kernels compute from the stale slots of the padding tokens (m rounded up to 32) is never
+ * stored. */
+int infr_hip_linear_noalloc(infr_hip_t *be, int dtype, const infr_hip_buffer_t *w, size_t w_numel,
+                            size_t w_off, const infr_hip_buffer_t *x, infr_hip_buffer_t *dst, size_t m,
+                            size_t in_f, size_t out_f);
+
 /* quantize_q8 (crates/infr-cpu/src/quant.rs:27-58) for m rows of k floats (k % 256 == 0):
  *   qs i8 [m,k]; d f32 [m,k/256]; bsums i32 [m,k/32]; bsums16 i32 [m,k/16] (may be NULL).
  * Exposes the integer stage so callers can check it bit-for-bit. */

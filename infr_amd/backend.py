@@ -119,6 +119,8 @@ SYMBOLS = {
     "infr_hip_sync": (C.c_int, [_vp]),
     "infr_hip_linear": (C.c_int, [_vp, C.c_int, _vp, C.c_size_t, C.c_size_t, _vp, _vp, C.c_size_t,
                                   C.c_size_t, C.c_size_t]),
+    "infr_hip_linear_noalloc": (C.c_int, [_vp, C.c_int, _vp, C.c_size_t, C.c_size_t, _vp, _vp, C.c_size_t,
+                                          C.c_size_t, C.c_size_t]),
     "infr_hip_quantize_q8": (C.c_int, [_vp, _vp, C.c_size_t, C.c_size_t, _vp, _vp, _vp, _vp]),
     "infr_hip_quantize_q8_32": (C.c_int, [_vp, _vp, C.c_size_t, C.c_size_t, _vp, _vp, _vp]),
     "infr_hip_linear_int_stages": (C.c_int, [_vp, C.c_int, _vp, C.c_size_t, C.c_size_t, _vp,
@@ -573,6 +575,15 @@ class HipBackend:
             w_numel = w.len_bytes() // b * e
         self._check(self._lib.infr_hip_linear(self._h, int(dtype), w._h, w_numel, w_off, x._h,
                                               dst._h, m, in_f, out_f))
+
+    def linear_noalloc(self, dtype: int, w: Buffer, x: Buffer, dst: Buffer, m: int, in_f: int, out_f: int,
+                       w_numel: int | None = None, w_off: int = 0) -> None:
+        """infr_hip_linear over the library's static device scratch: allocates nothing."""
+        if w_numel is None:
+            e, b = block_layout(dtype)
+            w_numel = w.len_bytes() // b * e
+        self._check(self._lib.infr_hip_linear_noalloc(self._h, int(dtype), w._h, w_numel, w_off, x._h,
+                                                      dst._h, m, in_f, out_f))
 
     def linear_int_stages(self, dtype: int, w: Buffer, x: Buffer, m: int, in_f: int, out_f: int,
                           w_numel: int | None = None, w_off: int = 0):

@@ -10,6 +10,7 @@
 #include <atomic>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <string>
 #include <vector>
@@ -68,6 +69,8 @@ struct infr_hip {
     // terms: backend-allocated, graph.rs:109-122). Grow-only.
     infr::ActQ8 act;
     size_t act_cap_elems = 0;
+    // The same four arrays inside this device's static scratch (infr_hip_linear_noalloc).
+    infr::ActQ8 static_act;
     // MoE scratch
     void* moe_ws = nullptr;
     size_t moe_ws_bytes = 0;
@@ -77,7 +80,33 @@ struct infr_hip {
     uint64_t scratch_epoch = 0;
 };
 
+// ---- static device scratch of the allocation-free Op::Linear entry point ----
+// Quantized activation of up to kStaticActElems elements (tokens rounded up to 32, times in_f):
+// codes, then per-32 scales, per-32 sums and per-16 sums, the four arrays of infr::ActQ8 back to
+// back. Every device the library runs on holds its own copy of this array at its own address
+// until the process ends; the name below is only a host-side handle for hipGetSymbolAddress.
+constexpr size_t kStaticActElems = (size_t)4 << 20;
+constexpr size_t kStaticActBytes = kStaticActElems + kStaticActElems / 32 * 4 * 2 + kStaticActElems / 16 * 4;
+static __device__ __align__(256) unsigned char scratch[kStaticActBytes];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+unsigned char* g_scratch_ptr[kMaxDevices] = {};  // device address of `scratch` per device, 0 = not asked yet
+
+// The device address of this device's copy of `scratch`; `device` must be current.
+hipError_t static_scratch_ptr(int device, unsigned char** out) {
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[device]) {
+        void* p = nullptr;
+        hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        g_scratch_ptr[device] = static_cast<unsigned char*>(p);
+    }
+    *out = g_scratch_ptr[device];
+    return hipSuccess;
+}
 
 thread_local std::string g_create_err;
 std::atomic<int> g_shutdown_signo{0};
@@ -303,7 +332,7 @@ int check_linear(infr_hip_t* be, int dtype, const infr_hip_buffer_t* w, size_t w
 }
 
 int enqueue_linear(infr_hip_t* be, int dtype, const LinearArgs& la, const float* x, float* y,
-                   size_t m, size_t in_f, size_t out_f, const infr::IntStages& st) {
+                   size_t m, size_t in_f, size_t out_f, const infr::IntStages& st, const infr::ActQ8& act) {
     bool ok;
     if (infr::gemv_takes_f32_activations(dtype, m)) {
         if (st.a)
@@ -311,11 +340,11 @@ int enqueue_linear(infr_hip_t* be, int dtype, const LinearArgs& la, const float*
                         "int_stages: one token of dtype " + std::to_string(dtype) + " has no integer stage");
         ok = infr::launch_gemv_f32act(dtype, la.wrows, la.bpr, x, y, in_f, out_f, be->stream);
     } else if (m == 1 && !infr::gemv_row_too_long(dtype, in_f)) {
-        infr::launch_quantize_q8(x, m, in_f, act_per32(dtype, in_f), be->act, be->stream);
-        ok = infr::launch_gemv(dtype, la.wrows, la.bpr, be->act, y, in_f, out_f, st, be->stream);
+        infr::launch_quantize_q8(x, m, in_f, act_per32(dtype, in_f), act, be->stream);
+        ok = infr::launch_gemv(dtype, la.wrows, la.bpr, act, y, in_f, out_f, st, be->stream);
     } else {
         // quantizes x into the scratch in the layout its kernel reads, then multiplies
-        ok = infr::launch_mmq(dtype, la.wrows, la.bpr, x, be->act, y, m, in_f, out_f, st, be->stream);
+        ok = infr::launch_mmq(dtype, la.wrows, la.bpr, x, act, y, m, in_f, out_f, st, be->stream);
     }
     if (!ok)
         return fail(be, INFR_HIP_ERR_UNSUPPORTED,
@@ -384,7 +413,7 @@ int infr_hip_create(int device, infr_hip_t** out) {
     if (e != hipSuccess || n <= 0)
         return fail(nullptr, INFR_HIP_ERR_BACKEND,
                     std::string("no HIP device: ") + (e != hipSuccess ? hipGetErrorString(e) : "count is 0"));
-    if (device < 0 || device >= n)
+    if (device < 0 || device >= n || device >= kMaxDevices)
         return fail(nullptr, INFR_HIP_ERR_INVALID, "create: device index out of range");
     infr_hip_t* be = new (std::nothrow) infr_hip();
     if (!be) return fail(nullptr, INFR_HIP_ERR_OTHER, "create: out of host memory");
@@ -403,6 +432,13 @@ int infr_hip_create(int device, infr_hip_t** out) {
         infr_hip_destroy(be);
         return fail(nullptr, INFR_HIP_ERR_UNSUPPORTED, msg);
     }
+    // this device's copy of the static scratch (the device is current here)
+    unsigned char* sp = nullptr;
+    if ((e = static_scratch_ptr(device, &sp)) != hipSuccess) return bail("hipGetSymbolAddress(scratch)", e);
+    be->static_act.qs = reinterpret_cast<int8_t*>(sp);
+    be->static_act.d = reinterpret_cast<float*>(sp + kStaticActElems);
+    be->static_act.bsums = reinterpret_cast<int32_t*>(sp + kStaticActElems + kStaticActElems / 32 * 4);
+    be->static_act.bsums16 = reinterpret_cast<int32_t*>(sp + kStaticActElems + kStaticActElems / 32 * 4 * 2);
     if ((e = hipStreamCreateWithFlags(&be->stream, hipStreamNonBlocking)) != hipSuccess)
         return bail("hipStreamCreate", e);
     if ((e = hipEventCreate(&be->ev0)) != hipSuccess) return bail("hipEventCreate", e);
@@ -583,7 +619,31 @@ int infr_hip_linear(infr_hip_t* be, int dtype, const infr_hip_buffer_t* w, size_
     }
     if (int rc = ensure_act(be, act_scratch_elems(m, in_f))) return rc;
     return enqueue_linear(be, dtype, la, static_cast<const float*>(x->ptr),
-                          static_cast<float*>(dst->ptr), m, in_f, out_f, infr::IntStages{});
+                          static_cast<float*>(dst->ptr), m, in_f, out_f, infr::IntStages{}, be->act);
+}
+
+int infr_hip_linear_noalloc(infr_hip_t* be, int dtype, const infr_hip_buffer_t* w, size_t w_numel,
+                            size_t w_off, const infr_hip_buffer_t* x, infr_hip_buffer_t* dst, size_t m,
+                            size_t in_f, size_t out_f) {
+    if (!be) return INFR_HIP_ERR_INVALID;
+    if (int rc = check_latch(be)) return rc;
+    LinearArgs la;
+    if (int rc = check_linear(be, dtype, w, w_numel, w_off, x, m, in_f, out_f, &la)) return rc;
+    if (!dst || dst->len < m * out_f * sizeof(float))
+        return fail(be, INFR_HIP_ERR_INVALID, "linear_noalloc: dst buffer missing or too small");
+    if (m == 1 && !runs_alone(dtype, m, in_f)) {
+        // decode: the fused launch keeps the quantized activation in LDS and needs no scratch
+        const infr::GemvOpDesc op{la.wrows, static_cast<const float*>(x->ptr),
+                                  static_cast<float*>(dst->ptr), la.bpr, (int32_t)out_f};
+        return enqueue_gemv_single(be, dtype, in_f, op);
+    }
+    if (act_scratch_elems(m, in_f) > kStaticActElems)
+        return fail(be, INFR_HIP_ERR_UNSUPPORTED,
+                    "linear_noalloc: " + std::to_string(act_scratch_elems(m, in_f)) +
+                        " activation elements (tokens rounded up to 32, times in_f) exceed the static scratch of " +
+                        std::to_string(kStaticActElems));
+    return enqueue_linear(be, dtype, la, static_cast<const float*>(x->ptr), static_cast<float*>(dst->ptr), m,
+                          in_f, out_f, infr::IntStages{}, be->static_act);
 }
 
 int infr_hip_embed_gather(infr_hip_t* be, int dtype, const infr_hip_buffer_t* table, size_t table_numel,
@@ -619,7 +679,7 @@ int infr_hip_linear_int_stages(infr_hip_t* be, int dtype, const infr_hip_buffer_
     infr::IntStages st;
     st.a = static_cast<int32_t*>(a->ptr);
     st.b = b ? static_cast<int32_t*>(b->ptr) : nullptr;
-    int rc = enqueue_linear(be, dtype, la, static_cast<const float*>(x->ptr), y, m, in_f, out_f, st);
+    int rc = enqueue_linear(be, dtype, la, static_cast<const float*>(x->ptr), y, m, in_f, out_f, st, be->act);
     (void)hipStreamSynchronize(be->stream);
     (void)hipFree(y);
     return rc;
@@ -1147,7 +1207,7 @@ static int enqueue_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t
                 return rc;
             if (int rc = enqueue_linear(be, op.w_dtype, la, static_cast<const float*>(bindings[op.x]->ptr),
                                         static_cast<float*>(bindings[op.dst]->ptr), op.m, op.in_f,
-                                        op.out_f, infr::IntStages{}))
+                                        op.out_f, infr::IntStages{}, be->act))
                 return rc;
         } else if (st.m > 1) {
             infr::launch_quantize_q8_group(plan->qtiles_dev + st.qtile_first, st.qtile_n, act_per32(st.dtype, st.in_f),
