@@ -254,6 +254,11 @@ void launch_mmq_shared_q5k(const uint8_t* w, size_t bpr, const ActQ8& act, float
 // iprod per (token, row, 32-element block).
 bool launch_mmq_shared_nib32(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
                              size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream);
+// Q4_K strip form (mmq_q4k_strip.hip): 256 tokens x 96 rows per workgroup, activations in the tiled
+// quantizer's layout. `takes` says whether the grid fills the device well enough to prefer it.
+bool mmq_strip_q4k_takes(size_t m, size_t out_f);
+void launch_mmq_strip_q4k(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
+                          size_t out_f, const IntStages& st, hipStream_t stream);
 // Routed pairs bucketed by expert, in tiles of at most 32 pairs of one expert each (device arrays;
 // `*n_tiles` of the `max_tiles` entries exist). `perm` lists the pairs expert by expert.
 struct MoeTileTable {

@@ -1156,6 +1156,10 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
     static const int env_shared_rows = getenv("INFR_HIP_MMQ_SHARED_ROWS") ? atoi(getenv("INFR_HIP_MMQ_SHARED_ROWS")) : 0;
     if (dtype == 12 && ((int)m >= env_shared_min || long_row)) {
         launch_quantize_q8_tiled(x, m, in_f, act, stream);
+        if (mmq_strip_q4k_takes(m, out_f)) {
+            launch_mmq_strip_q4k(w, bpr, act, y, m, in_f, out_f, st, stream);
+            return true;
+        }
         // (896 / 1000 tokens at 12288 x 4096: 658 / 730 against 622 / 627 TOPS; at 768 and below the
         // 32-row form is ahead)
         // 256-token tiles pad up to 128 tokens more than 128-token tiles do: taken when both pad alike,

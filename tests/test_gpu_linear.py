@@ -407,10 +407,12 @@ def test_full_size_decode_rows_vs_oracle(be, dtype, in_f, out_f):
             assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), "not bit-identical"
 
 
-@pytest.mark.parametrize("m", [8, 64, 512, 1100])
+@pytest.mark.parametrize("m", [8, 64, 512, 1024, 1100, 2048])
 def test_full_size_prefill_q4k(be, m):
-    """K = 4096 -> N = 12288 at the benchmark's token counts (every Q4_K kernel route): sampled
-    rows bit-identical to the oracle, and every token's row equal to its own m = 1 result."""
+    """K = 4096 -> N = 12288 at the benchmark's token counts (every Q4_K kernel route; 512, 1024 and
+    2048 tokens fill whole rounds of the 96-row strip kernel, 1100 takes the 32-row shared-operand
+    form): sampled rows bit-identical to the oracle, and every token's row equal to its own m = 1
+    result."""
     in_f, out_f = 4096, 12288
     w = synth_weight(DType.Q4K, 910, out_f, in_f)
     x = synth_normal_f32(911 + m, m * in_f)
@@ -429,6 +431,59 @@ def test_full_size_prefill_q4k(be, m):
         be.linear(DType.Q4K, wb, be.upload_new(x[t * in_f:(t + 1) * in_f]), y1, 1, in_f, out_f)
         single = be.download(y1, np.empty((1, out_f), np.float32))
         assert np.array_equal(single[0].view(np.uint32), y[t].view(np.uint32)), "batch != single"
+
+
+@pytest.mark.parametrize("m,in_f,out_f", [(2560, 256, 2304), (2400, 768, 2300), (512, 512, 12288)])
+def test_q4k_strip_route_is_exact(be, m, in_f, out_f):
+    """Grids of (nearly) whole rounds of 256 workgroups take the strip kernel (256 tokens x 96 rows
+    per workgroup): ragged last strip and token group, one and several blocks per row. Per-block
+    sd / sm exact and y bit-identical on sampled tokens, full-range payloads."""
+    w = orc.synth_weight(DType.Q4K, in_f * out_f, 0x300 + in_f)      # full-range payload bytes
+    x = synth_normal_f32(778 + m, m * in_f) * np.float32(3.0)
+    x[in_f:2 * in_f] = 1e4      # saturates every code to +127: bsums reach +4064
+    x[2 * in_f:3 * in_f] = -1e4
+    wb, xb = be.upload_new(w), be.upload_new(x)
+    yb = be.alloc(m * out_f * 4)
+    be.linear(DType.Q4K, wb, xb, yb, m, in_f, out_f)
+    y = be.download(yb, np.empty((m, out_f), np.float32))
+    toks = sorted({0, 1, 2, 31, 32, 255, 256, m // 2 + 3, m - 33, m - 1})
+    xs = x.reshape(m, in_f)[toks].ravel()
+    want = orc.linear(DType.Q4K, w, xs, len(toks), in_f, out_f)
+    assert np.array_equal(y[toks].view(np.uint32), want.view(np.uint32)), "not bit-identical"
+    sd, sm = be.linear_int_stages(DType.Q4K, wb, xb, m, in_f, out_f)
+    osd, osm = orc.linear_int_stages(DType.Q4K, w, xs, len(toks), in_f, out_f)
+    assert np.array_equal(sd[toks], osd) and np.array_equal(sm[toks], osm)
+
+
+def test_q4k_eight_wave_form_at_sixteen_blocks(be):
+    """1280 tokens x 4096 rows pads alike in 128- and 256-token tiles and does not fill the strip
+    kernel's rounds: the eight-wave 64-row x 256-token form, here with 16 blocks per row (its
+    double-buffered block loop at the benchmark's K)."""
+    m, in_f, out_f = 1280, 4096, 4096
+    w = synth_weight(DType.Q4K, 930, out_f, in_f)
+    x = synth_normal_f32(931, m * in_f)
+    y = run_linear(be, DType.Q4K, w, x, m, in_f, out_f)
+    toks = [0, 255, 256, 640, 1279]
+    for row0 in (0, 2040, out_f - 32):
+        want = _oracle_rows(DType.Q4K, w, x.reshape(m, in_f)[toks].ravel(), len(toks), in_f, out_f, row0, 32)
+        assert np.array_equal(y[toks, row0:row0 + 32].view(np.uint32), want.view(np.uint32)), "not bit-identical"
+
+
+@pytest.mark.parametrize("dtype", [DType.Q6K, DType.Q8_0])
+@pytest.mark.parametrize("in_f,out_f", [(4096, 12288), (12288, 4096)])
+def test_full_size_batch8_rows_vs_oracle(be, dtype, in_f, out_f):
+    """Eight tokens at the full Qwen3-8B grids (the tile heights a grid of 12288 or 4096 rows gets
+    differ from a 256-row one's): sampled rows against the oracle."""
+    m = 8
+    w = synth_weight(dtype, 940 + in_f, out_f, in_f)
+    x = synth_normal_f32(941, m * in_f)
+    y = run_linear(be, dtype, w, x, m, in_f, out_f)
+    for row0 in (0, out_f // 2 - 5, out_f - 40):
+        want = _oracle_rows(dtype, w, x, m, in_f, out_f, row0, 40)
+        got = y[:, row0:row0 + 40]
+        gate(got, want)
+        if dtype == DType.Q6K:
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), "not bit-identical"
 
 
 def test_ternary_output_head_rows_vs_oracle(be):
