@@ -64,6 +64,7 @@ class Sweep:
         self.bytes = self.bytes_4096 = 0
         self.launches = 0
         self.keep = []
+        self.out_bufs = {}          # layer 0's outputs by projection name (for the parity gate)
         xs = {}
         for in_f in (4096, 12288):
             xid = g.input(TensorDesc((m, in_f), DType.F32))
@@ -104,6 +105,8 @@ class Sweep:
                 else:
                     src = xs[in_f]
                 outs[name] = new_out(out_f)
+                if layer == 0:
+                    self.out_bufs[name] = self.keep[-1]
                 op = Linear(src, wid, outs[name], m, in_f, out_f)
                 g.push(op)
                 if in_f == 4096:
@@ -146,6 +149,60 @@ class Sweep:
         for b in self.keep:
             b.free()
         self.keep = []
+
+
+def parity_gate_sweep(be, sw, dtype):
+    """Untimed check of what the timed plan computed: sampled rows of three of its outputs (a q, a
+    gate and a down projection of layer 0) against the CPU oracle on the same bytes. Q4_K decode
+    outputs must be bit-identical. Returns "ok" or raises."""
+    from infr_amd import DType, synth_normal_f32, synth_weight
+    from oracle import oracle as orc
+    for i, (name, out_f, in_f) in enumerate(LAYER):
+        if name not in ("q", "gate", "down"):
+            continue
+        yb = sw.out_bufs[name]
+        rows = 64
+        w = synth_weight(dtype, i, out_f, in_f)
+        x = synth_normal_f32(1 + in_f, sw.m * in_f)
+        e, bpb = __import__("infr_amd").block_layout(dtype)
+        bpr = in_f // e * bpb
+        for row0 in (0, out_f - rows):
+            got = be.download(yb, np.empty((sw.m, out_f), np.float32))[:, row0:row0 + rows]
+            want = orc.linear(dtype, w[row0 * bpr:(row0 + rows) * bpr], x, sw.m, in_f, rows)
+            if dtype in (DType.Q4K, DType.Q6K):
+                if not np.array_equal(got.view(np.uint32), want.view(np.uint32)):
+                    raise SystemExit(f"parity gate: {name} rows {row0}.. differ from the oracle")
+            else:
+                rel = np.linalg.norm(got.astype(np.float64) - want) / np.linalg.norm(want)
+                if rel > 1e-4:
+                    raise SystemExit(f"parity gate: {name} rel-L2 {rel:.2e}")
+    return "ok"
+
+
+def parity_gate_linear(be, dtype, m, in_f, out_f, tokens, rows=32):
+    """Untimed: one Op::Linear at the timed shape, sampled tokens x rows against the oracle
+    (bit-identical for the K-quants, rel-L2 <= 1e-4 otherwise)."""
+    from infr_amd import DType, synth_normal_f32, synth_weight
+    from oracle import oracle as orc
+    w = synth_weight(dtype, 0, out_f, in_f)
+    x = synth_normal_f32(1, m * in_f)
+    wb, xb, yb = be.upload_new(w), be.upload_new(x), be.alloc(m * out_f * 4)
+    be.linear(dtype, wb, xb, yb, m, in_f, out_f)
+    y = be.download(yb, np.empty((m, out_f), np.float32))
+    for b in (wb, xb, yb):
+        b.free()
+    e, bpb = __import__("infr_amd").block_layout(dtype)
+    bpr = in_f // e * bpb
+    xs = x.reshape(m, in_f)[tokens].ravel()
+    for row0 in (0, out_f // 2, out_f - rows):
+        want = orc.linear(dtype, w[row0 * bpr:(row0 + rows) * bpr], xs, len(tokens), in_f, rows)
+        got = y[tokens, row0:row0 + rows]
+        if dtype in (DType.Q4K, DType.Q5K, DType.Q6K):
+            if not np.array_equal(got.view(np.uint32), want.view(np.uint32)):
+                raise SystemExit(f"parity gate: Linear m={m} {in_f}->{out_f} rows {row0}.. differ from the oracle")
+        elif np.linalg.norm(got.astype(np.float64) - want) > 1e-4 * np.linalg.norm(want):
+            raise SystemExit(f"parity gate: Linear m={m} {in_f}->{out_f} outside rel-L2 1e-4")
+    return "ok"
 
 
 def settle_clocks(be, plan, binds, seconds=0.03):
@@ -314,9 +371,22 @@ def moe_bench(be, n_layers=6):
             be.execute(plan, binds)
             best = min(best, be.timer_end())
         us = best * 1e3 / n_layers
-        # every layer routes the same x through the same router: unique experts per layer
+        # every layer routes the same x through the same router: the distinct experts a layer
+        # touches come from the routing itself (one untimed direct call)
+        idx_b, y_b = be.alloc(rows * n_used * 4), be.alloc(rows * ne * 4)
+        be.moe_ffn(binds.get(xid), router, protos[0], protos[1], protos[2], y_b, rows=rows, ne=ne, n_expert=n_expert,
+                   n_used=n_used, n_ff_exp=nff, scale=1.0, sel_idx=idx_b)
+        unique = int(np.unique(be.download(idx_b, np.empty(rows * n_used, np.int32))).size)
+        idx_b.free()
+        y_b.free()
         out[f"moe_q4k_t{rows}_us_per_layer"] = round(us, 2)
-        out[f"moe_q4k_t{rows}_pair_GBs"] = round(rows * n_used * per_expert / (us * 1e-6) / 1e9, 1)
+        out[f"moe_q4k_t{rows}_unique_experts"] = unique
+        # HBM figure: the bytes of the distinct experts touched, each counted once
+        out[f"moe_q4k_t{rows}_unique_expert_GBs"] = round(unique * per_expert / (us * 1e-6) / 1e9, 1)
+        if rows <= 16:
+            # no-reuse figure (every (token, expert) pair's bytes, as the reference's dense-equivalent
+            # convention, crates/infr-metal/tests/moe_bw.rs:150-157): not a bandwidth once pairs share experts
+            out[f"moe_q4k_t{rows}_per_pair_no_reuse_GBs"] = round(rows * n_used * per_expert / (us * 1e-6) / 1e9, 1)
         if rows >= 64:
             out[f"moe_q4k_t{rows}_TOPS"] = round(rows * n_used * 3 * nff * ne * 2 / (us * 1e-6) / 1e12, 1)
         plan = None
@@ -389,6 +459,7 @@ def main():
     ap.add_argument("--layers", type=int, default=N_LAYERS)
     ap.add_argument("--no-extra", action="store_true", help="headline sweep only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-parity", action="store_true", help="skip the untimed oracle checks of the timed outputs")
     ap.add_argument("--sections", default="shapes,formats,mmq,chain,layer,ternary,moe,load",
                     help="comma list of secondary sections: shapes, formats, mmq, chain, layer, ternary, moe, load; mmq_scaling (off by default)")
     args = ap.parse_args()
@@ -426,6 +497,7 @@ def main():
     probe = be.alloc_uninit(2 << 30)
     stream_read = be.stream_read_gbs(probe, reps=10)
     probe.free()
+    parity = "skipped (--no-parity)" if args.no_parity else parity_gate_sweep(be, sw, DType.Q4K)
     out = {
         "metric": "Q4_K GEMV HBM GB/s (% of peak) + prefill mmq int8 TOPS at M=512",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
@@ -436,6 +508,7 @@ def main():
                                f"{sw.bytes / 1e9:.2f} GB, one plan), batch 1",
                    "weights": "N(0,0.02^2) seed 0 -> Q4_K", "activations": "N(0,1) f32, quantized on GPU",
                    "clock_ramp_steps_untimed": RAMP_STEPS,
+                   "parity": parity,
                    "device": caps["device_name"], "compute_units": caps["compute_units"]},
         "pct_of_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "launches_per_step": n_launch,
@@ -456,6 +529,11 @@ def main():
                 for (out_f, in_f) in ((4096, 4096), (1024, 4096), (12288, 4096), (4096, 12288)):
                     t, nb = single_shape(be, dt, m, in_f, out_f)
                     extra[f"gemv_{name}_m{m}_{out_f}x{in_f}_GBs"] = round(nb / (t * 1e-3) / 1e9, 1)
+        # the same shapes warm: two copies of one matrix (19-57 MB), resident in the 256 MB Infinity
+        # Cache, so these are cache figures and not HBM bandwidth
+        for (out_f, in_f) in ((4096, 4096), (1024, 4096), (12288, 4096), (4096, 12288)):
+            t, nb = single_shape(be, DType.Q4K, 1, in_f, out_f, rotate_bytes=1)
+            extra[f"gemv_Q4_K_m1_{out_f}x{in_f}_warm_cache_resident_GBs"] = round(nb / (t * 1e-3) / 1e9, 1)
     if "formats" in sections:
         for name, dt in (("Q5_K", DType.Q5K), ("Q4_0", DType.Q4_0), ("Q4_1", DType.Q4_1), ("Q5_0", DType.Q5_0),
                          ("Q5_1", DType.Q5_1), ("IQ4_NL", DType.IQ4NL), ("Q2_0", DType.Q2_0)):
@@ -468,6 +546,18 @@ def main():
             t, nb = single_shape(be, DType.Q4K, M, 4096, 12288, reps=10)
             extra[f"mmq_Q4_K_M{M}_TOPS"] = round(2.0 * M * 12288 * 4096 / (t * 1e-3) / 1e12, 2)
             extra[f"mmq_Q4_K_M{M}_pct_int8_peak"] = round(100 * extra[f"mmq_Q4_K_M{M}_TOPS"] / INT8_PEAK_TOPS, 2)
+            if M == 512:
+                # the prefill half of the metric: one Op::Linear = the activation quantizer's launch and
+                # the int8-MFMA kernel's (ten back-to-back ops over rotated weight copies, HIP events
+                # on the backend's stream); ops = 2 M N K
+                ops = 2.0 * M * 12288 * 4096
+                out["roofline_mmq"] = {
+                    "bound": "mfma", "kernel": "quantize_q8_tiled_kernel + mmq_strip_q4k_kernel (M=512, K=4096, N=12288)",
+                    "achieved": round(ops / (t * 1e-3) / 1e12, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                    "frac": round(ops / (t * 1e-3) / 1e12 / INT8_PEAK_TOPS, 4), "traffic": None,
+                    "avg_launch_us": round(t * 1e3, 2), "ops_per_launch": ops,
+                    "parity": "skipped (--no-parity)" if args.no_parity else
+                              parity_gate_linear(be, DType.Q4K, M, 4096, 12288, [0, 255, 256, 511])}
         # the matrix rate the device sustains on a register-only loop of the same MFMA (no memory
         # traffic): constant operands, and pseudo-random operands as the kernels feed it
         extra["mfma_i8_peak_const_operands_TOPS"] = round(be.mfma_i8_peak_tops(4, 4096, False), 1)

@@ -339,9 +339,6 @@ int enqueue_linear(infr_hip_t* be, int dtype, const LinearArgs& la, const float*
             return fail(be, INFR_HIP_ERR_UNSUPPORTED,
                         "int_stages: one token of dtype " + std::to_string(dtype) + " has no integer stage");
         ok = infr::launch_gemv_f32act(dtype, la.wrows, la.bpr, x, y, in_f, out_f, be->stream);
-    } else if (m == 1 && !infr::gemv_row_too_long(dtype, in_f)) {
-        infr::launch_quantize_q8(x, m, in_f, act_per32(dtype, in_f), act, be->stream);
-        ok = infr::launch_gemv(dtype, la.wrows, la.bpr, act, y, in_f, out_f, st, be->stream);
     } else {
         // quantizes x into the scratch in the layout its kernel reads, then multiplies
         ok = infr::launch_mmq(dtype, la.wrows, la.bpr, x, act, y, m, in_f, out_f, st, be->stream);
@@ -679,7 +676,16 @@ int infr_hip_linear_int_stages(infr_hip_t* be, int dtype, const infr_hip_buffer_
     infr::IntStages st;
     st.a = static_cast<int32_t*>(a->ptr);
     st.b = b ? static_cast<int32_t*>(b->ptr) : nullptr;
-    int rc = enqueue_linear(be, dtype, la, static_cast<const float*>(x->ptr), y, m, in_f, out_f, st, be->act);
+    int rc;
+    if (m == 1 && !runs_alone(dtype, m, in_f)) {
+        // one token: the decode kernel infr_hip_linear launches, writing its integers as well
+        infr::GemvOpDesc op{la.wrows, static_cast<const float*>(x->ptr), y, la.bpr, (int32_t)out_f};
+        op.st_a = st.a;
+        op.st_b = st.b;
+        rc = enqueue_gemv_single(be, dtype, in_f, op);
+    } else {
+        rc = enqueue_linear(be, dtype, la, static_cast<const float*>(x->ptr), y, m, in_f, out_f, st, be->act);
+    }
     (void)hipStreamSynchronize(be->stream);
     (void)hipFree(y);
     return rc;
@@ -969,6 +975,7 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
     // absorbed[k]: op k runs inside some Linear and is not scheduled on its own
     std::vector<int> pre(n, -1), post(n, -1);
     std::vector<char> absorbed(n, 0), publishes(n, 0);
+    // INFR_HIP_FUSE=0: every op a launch of its own (for comparing against the absorbed form)
     static const int env_fuse = getenv("INFR_HIP_FUSE") ? atoi(getenv("INFR_HIP_FUSE")) : 1;
     auto decode_linear = [&](size_t i) {
         return plan->ops[i].kind == INFR_OP_LINEAR && plan->ops[i].m == 1 &&
@@ -1310,8 +1317,7 @@ int infr_hip_stream_read(infr_hip_t* be, const infr_hip_buffer_t* src, size_t by
     if (!be || !src || !elapsed_ms || reps <= 0) return fail(be, INFR_HIP_ERR_INVALID, "stream_read: bad argument");
     if (bytes > src->len || bytes < 16) return fail(be, INFR_HIP_ERR_INVALID, "stream_read: size outside the buffer");
     if (int rc = check_latch(be)) return rc;
-    static const int env_wgs = getenv("INFR_HIP_PROBE_WGS") ? atoi(getenv("INFR_HIP_PROBE_WGS")) : 64;
-    const int wgs = std::max(1, be->props.multiProcessorCount) * std::max(1, env_wgs);
+    const int wgs = std::max(1, be->props.multiProcessorCount) * 64;
     int* out = nullptr;
     HIP_TRY(be, hipMalloc((void**)&out, sizeof(int) * (size_t)wgs));
     infr::launch_stream_read(src->ptr, bytes, out, wgs, be->stream);  // untimed first pass

@@ -48,13 +48,6 @@ bool gemv_row_too_long(int dtype, size_t in_f) {
     return o != nullptr && in_f > (size_t)8 * (size_t)o->elems_per_step;
 }
 
-bool launch_gemv(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t in_f,
-                 size_t out_f, const IntStages& st, hipStream_t stream) {
-    if (out_f == 0) return true;
-    const GemvFormatOps* f = format_ops(dtype, in_f);
-    return f && f->plain && f->plain(w, bpr, act, y, in_f, out_f, st, stream);
-}
-
 bool launch_gemv_batch_group(int dtype, size_t m, size_t in_f, const BatchTile* tiles_dev,
                              const BatchGroupPlan& plan, const ActQ8& act, hipStream_t stream) {
     const GemvFormatOps* f = format_ops(dtype, in_f);
@@ -65,11 +58,10 @@ bool plan_batch_group(int dtype, size_t m, size_t in_f, const GemvOpDesc* ops, i
     size_t total_rows = 0;
     for (int i = 0; i < n; ++i) total_rows += (size_t)ops[i].out_f;
     BatchGroupPlan gp;
-    static const int env_dot4_max = getenv("INFR_HIP_Q4K_DOT4_MAX_M") ? atoi(getenv("INFR_HIP_Q4K_DOT4_MAX_M")) : 0;
     if ((dtype == 13 || dtype == 14) && mmq_skinny16_takes(dtype, m, in_f)) {  // Q5_K, Q6_K, 2..16 tokens: the K-split MFMA kernel
         gp.kind = 1;
         gp.rows_per_wg = 32;
-    } else if (dtype == 12 && (int)m > env_dot4_max) {  // Q4_K: the K-split MFMA kernels, 32 rows per workgroup
+    } else if (dtype == 12) {  // Q4_K: the K-split MFMA kernels, 32 rows per workgroup
         if (in_f % 256 != 0 || m > 32) return false;
         gp.kind = 1;
         gp.rows_per_wg = 32;
@@ -90,8 +82,7 @@ bool plan_batch_group(int dtype, size_t m, size_t in_f, const GemvOpDesc* ops, i
         } else {
             // K-split form: a tile is one workgroup's rows, whole flush groups of 64 / MB rows
             const size_t rb = 64 / (m > 4 ? 8 : (m > 2 ? 4 : 2));
-            static const int env_rows = getenv("INFR_HIP_BATCH_KS_ROWS") ? atoi(getenv("INFR_HIP_BATCH_KS_ROWS")) : 0;
-            size_t r = ((env_rows > 0 ? (size_t)env_rows : (total_rows + 4095) / 4096) + rb - 1) / rb * rb;
+            size_t r = ((total_rows + 4095) / 4096 + rb - 1) / rb * rb;
             gp.rows_per_wave = 0;
             gp.rows_per_wg = (int)(r < rb ? rb : (r > 32 && rb <= 32 ? 32 : r));
         }

@@ -13,28 +13,6 @@
 
 namespace infr {
 
-template <typename F, int STEPS, bool STAGES>
-__global__ __launch_bounds__(256) void gemv_kernel(const uint8_t* __restrict__ w, size_t bpr,
-                                                   ActPtrs act, float* __restrict__ y, int n_units,
-                                                   int out_f, int rows_per_wave, StagePtrs st) {
-    const int lane = threadIdx.x & 63;
-    const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int row0 = wave * rows_per_wave;
-    if (row0 >= out_f) return;
-    const int row_end = min(row0 + rows_per_wave, out_f);
-    typename F::Acts acts[STEPS];
-    typename F::Row first;
-    bool ok[STEPS];
-#pragma unroll
-    for (int t = 0; t < STEPS; ++t) ok[t] = F::valid(t, lane, n_units);
-    F::load_row(first, w + (size_t)row0 * bpr, 0, lane, ok[0]);
-#pragma unroll
-    for (int t = 0; t < STEPS; ++t) F::load_acts(acts[t], act, t, lane, ok[t]);
-    __shared__ __attribute__((aligned(16))) float osum[4 * RowSumScratch<F, STEPS>::kFloatsPerWave];
-    gemv_rows<F, STEPS, STAGES>(w, bpr, first, acts, ok, y, n_units, row0, row_end, lane, st,
-                                osum + (threadIdx.x >> 6) * RowSumScratch<F, STEPS>::kFloatsPerWave);
-}
-
 // Small batch (2..8 activation rows already quantized in device memory): weights stream once.
 // With `tiles` (plans) a workgroup takes one table entry - some rows of one of several ops - and
 // blockIdx.y selects the pass of MB activation rows; `m_valid` is then the op's total row count.
@@ -231,7 +209,8 @@ __device__ __forceinline__ float fused_gated_act(int act, bool has_clamp, float 
 
 // Fused + grouped form. LDS: qs[in_f] | d[in_f/32] | bsums[in_f/32] | bsums16[in_f/16] | per-wave
 // ordered-sum scratch.
-template <typename F, int STEPS, int NW>
+// STAGES: the per-block integers of every row also go to single.st_a / st_b (single-op launches only).
+template <typename F, int STEPS, int NW, bool STAGES>
 __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, int single_rows,
                                                              const GemvTile* __restrict__ tiles,
                                                              int in_f) {
@@ -241,10 +220,12 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, 
 
     // This workgroup's rows: one table entry, or computed from the single op's descriptor.
     GemvTile tile;
+    int first_row = 0;
     if (tiles != nullptr) {
         tile = tiles[blockIdx.x];
     } else {
         const int first = (int)blockIdx.x * single_rows;
+        first_row = first;
         tile.w = single.w + (size_t)first * single.bpr;
         tile.x = single.x;
         tile.y = single.y + first;
@@ -341,54 +322,20 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, 
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) F::load_acts(acts[t], act, t, lane, ok[t]);
     float* osum = reinterpret_cast<float*>(lds + in_f + in_f / 2) + wave * RowSumScratch<F, STEPS>::kFloatsPerWave;
-    gemv_rows<F, STEPS, false>(tile.w, tile.bpr, first, acts, ok, tile.y, n_units, row0, row_end, lane,
-                               StagePtrs{nullptr, nullptr}, osum, tile.fus.add_b, tile.fus.add_dst);
+    // stage outputs are indexed by the op's row: offset them to the tile's first
+    const size_t st_off = (size_t)first_row * (F::kBlockElems == 64 ? 2 * n_units : n_units);
+    const StagePtrs st{STAGES ? single.st_a + st_off : nullptr, STAGES && single.st_b ? single.st_b + st_off : nullptr};
+    gemv_rows<F, STEPS, STAGES>(tile.w, tile.bpr, first, acts, ok, tile.y, n_units, row0, row_end, lane, st, osum,
+                                tile.fus.add_b, tile.fus.add_dst);
 }
 
 // ───────────────────────────────────── launch ─────────────────────────────────────
 
-template <typename F, bool STAGES>
-static bool launch_plain(int steps, dim3 grid, hipStream_t stream, const uint8_t* w, size_t bpr,
-                         const ActPtrs& act, float* y, int n_units, int out_f, int rpw,
-                         const StagePtrs& st) {
-#define INFR_CASE(N)                                                                             \
-    case N:                                                                                      \
-        hipLaunchKernelGGL((gemv_kernel<F, N, STAGES>), grid, dim3(256), 0, stream, w, bpr, act, y, \
-                           n_units, out_f, rpw, st);                                             \
-        return true;
-    switch (steps) {
-        INFR_CASE(1) INFR_CASE(2) INFR_CASE(3) INFR_CASE(4)
-        INFR_CASE(5) INFR_CASE(6) INFR_CASE(7) INFR_CASE(8)
-    default: return false;
-    }
-#undef INFR_CASE
-}
-
-template <typename F>
-static bool launch_plain_fmt(const uint8_t* w, size_t bpr, const ActQ8& a, float* y, size_t in_f,
-                             size_t out_f, const IntStages& st, hipStream_t stream) {
-    const int steps = (int)((in_f + F::kElemsPerStep - 1) / F::kElemsPerStep);
-    const int n_units = (int)(in_f / F::kBlockElems);
-    // Rows per wavefront: enough waves to cover the machine several times over.
-    static const int env_rpw = getenv("INFR_HIP_BATCH_ROWS") ? atoi(getenv("INFR_HIP_BATCH_ROWS")) : 0;
-    size_t rpw = (out_f + 4095) / 4096;
-    rpw = rpw < 2 ? 2 : (rpw > 16 ? 16 : rpw);
-    if (env_rpw > 0) rpw = (size_t)env_rpw;
-    const size_t waves = (out_f + rpw - 1) / rpw;
-    const dim3 grid((unsigned)((waves + 3) / 4));
-    const ActPtrs act{a.qs, a.d, a.bsums, a.bsums16};
-    const StagePtrs sp{st.a, st.b};
-    return st.a ? launch_plain<F, true>(steps, grid, stream, w, bpr, act, y, n_units, (int)out_f, (int)rpw, sp)
-                : launch_plain<F, false>(steps, grid, stream, w, bpr, act, y, n_units, (int)out_f, (int)rpw, sp);
-}
-
 template <typename F, int STEPS, int MB>
 static void launch_batch_one(const uint8_t* w, size_t bpr, const ActPtrs& act, int m_valid, size_t in_f,
                              float* y, size_t out_f, const StagePtrs& st, hipStream_t stream) {
-    static const int env_rpw = getenv("INFR_HIP_BATCH_ROWS") ? atoi(getenv("INFR_HIP_BATCH_ROWS")) : 0;
     size_t rpw = (out_f + 4095) / 4096;
     rpw = rpw < 2 ? 2 : (rpw > 16 ? 16 : rpw);
-    if (env_rpw > 0) rpw = (size_t)env_rpw;
     const size_t waves = (out_f + rpw - 1) / rpw;
     const dim3 grid((unsigned)((waves + 3) / 4)), block(256);
     if (st.a)
@@ -411,9 +358,7 @@ static int batch_rows_per_pass(int steps) {
 // faster on any shape tried).
 template <int MB>
 static int batch_ks_rows_per_wg(size_t total_rows) {
-    static const int env = getenv("INFR_HIP_BATCH_KS_ROWS") ? atoi(getenv("INFR_HIP_BATCH_KS_ROWS")) : 0;
     constexpr int RB = BatchKs<MB>::kRowsPerFlush;
-    if (env > 0) return (env + RB - 1) / RB * RB;
     size_t r = (total_rows + 4095) / 4096;  // about 4096 workgroups for a large group of rows
     r = (r + RB - 1) / RB * RB;
     return (int)(r < (size_t)RB ? RB : (r > 32 && RB <= 32 ? 32 : r));
@@ -505,7 +450,7 @@ static int fused_wgs_per_cu_nw(int steps, size_t lds_bytes) {
 #define INFR_CASE(N)                                                                                  \
     case N:                                                                                           \
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(                                             \
-                &nblk, reinterpret_cast<const void*>(&gemv_fused_kernel<F, N, NW>), NW * 64, lds_bytes) != hipSuccess) \
+                &nblk, reinterpret_cast<const void*>(&gemv_fused_kernel<F, N, NW, false>), NW * 64, lds_bytes) != hipSuccess) \
             nblk = 0;                                                                                 \
         break;
     switch (steps) {
@@ -548,11 +493,6 @@ static bool plan_group_fmt(size_t in_f, const GemvOpDesc* ops, int n, GemvGroupP
     // quantization is spread over the most waves; waves beyond the tile's rows retire after it.
     int nw = steps <= F::kWide16Steps ? 16 : 8;
     if (steps >= 3 && nw > 8) nw = 8;  // long rows: 8-wave workgroups measured faster
-    // Tuning knobs (the reference exposes its kernel-shape choices the same way,
-    // kernels.vulkan.* in crates/infr-core/src/config/mod.rs:210-358).
-    static const int env_nw = getenv("INFR_HIP_GEMV_WAVES") ? atoi(getenv("INFR_HIP_GEMV_WAVES")) : 0;
-    static const int env_rows = getenv("INFR_HIP_GEMV_ROWS") ? atoi(getenv("INFR_HIP_GEMV_ROWS")) : 0;
-    if ((env_nw == 4 || env_nw == 8 || env_nw == 16) && env_nw <= nw) nw = env_nw;
     size_t rows_per_wg = (total_rows + 511) / 512;
     rows_per_wg = rows_per_wg < 4 ? 4 : (rows_per_wg > 128 ? 128 : rows_per_wg);
     // activations, then every wave's row-sum scratch (OrderedSum<steps> or LaneSums)
@@ -566,7 +506,6 @@ static bool plan_group_fmt(size_t in_f, const GemvOpDesc* ops, int n, GemvGroupP
     // in units of a weight row: about eleven for quantizing x, more when the prologue also
     // evaluates an absorbed gated activation (expf per element) or RmsNorm. Grids of many rounds
     // keep the 128-row tiles: their tail is small and taller tiles measured slower.
-    static const int env_model = getenv("INFR_HIP_GEMV_ROUNDS") ? atoi(getenv("INFR_HIP_GEMV_ROUNDS")) : 1;
     const int resident = device_cu_count() * fused_wgs_per_cu<F>(steps, nw, lds_bytes);
     const int cus = device_cu_count();
     double fixed = 11.0;
@@ -577,7 +516,7 @@ static bool plan_group_fmt(size_t in_f, const GemvOpDesc* ops, int n, GemvGroupP
         for (int i = 0; i < n; ++i) w += ((size_t)ops[i].out_f + r - 1) / r;
         return w;
     };
-    if (env_model && resident > 0 && wgs_at(rows_per_wg) < (size_t)resident * 4) {
+    if (resident > 0 && wgs_at(rows_per_wg) < (size_t)resident * 4) {
         const size_t lo = std::max<size_t>(4, rows_per_wg / 2), hi = std::max<size_t>(rows_per_wg * 2, 160);
         double best = 1e300;
         size_t best_r = rows_per_wg;
@@ -591,7 +530,6 @@ static bool plan_group_fmt(size_t in_f, const GemvOpDesc* ops, int n, GemvGroupP
         }
         rows_per_wg = best_r;
     }
-    if (env_rows >= 1 && env_rows <= 4096) rows_per_wg = (size_t)env_rows;
     int wg = 0;
     for (int i = 0; i < n; ++i) wg += (int)(((size_t)ops[i].out_f + rows_per_wg - 1) / rows_per_wg);
     plan->total_wgs = wg;
@@ -608,14 +546,14 @@ static bool bpr_too_big(const GemvOpDesc* ops, int n) {
     return false;
 }
 
-template <typename F, int NW>
+template <typename F, int NW, bool STAGES>
 static bool launch_fused_nw(int steps, size_t in_f, const GemvOpDesc& op, const GemvTile* tiles_dev,
                             const GemvGroupPlan& plan, hipStream_t stream) {
     const dim3 grid((unsigned)plan.total_wgs), block(NW * 64);
-#define INFR_CASE(N)                                                                          \
-    case N:                                                                                   \
-        hipLaunchKernelGGL((gemv_fused_kernel<F, N, NW>), grid, block, plan.lds_bytes, stream, \
-                           op, plan.rows_per_wg, tiles_dev, (int)in_f);                     \
+#define INFR_CASE(N)                                                                                  \
+    case N:                                                                                           \
+        hipLaunchKernelGGL((gemv_fused_kernel<F, N, NW, STAGES>), grid, block, plan.lds_bytes, stream, \
+                           op, plan.rows_per_wg, tiles_dev, (int)in_f);                             \
         return true;
     switch (steps) {
         INFR_CASE(1) INFR_CASE(2) INFR_CASE(3) INFR_CASE(4)
@@ -629,10 +567,20 @@ template <typename F>
 static bool launch_fused_fmt(size_t in_f, const GemvOpDesc& op, const GemvTile* tiles_dev,
                              const GemvGroupPlan& plan, hipStream_t stream) {
     const int steps = (int)((in_f + F::kElemsPerStep - 1) / F::kElemsPerStep);
+    if (op.st_a != nullptr) {
+        // the integer-stage outputs: the same kernel, single-op launches only
+        if (tiles_dev != nullptr) return false;
+        switch (plan.waves_per_wg) {
+        case 4: return launch_fused_nw<F, 4, true>(steps, in_f, op, tiles_dev, plan, stream);
+        case 8: return launch_fused_nw<F, 8, true>(steps, in_f, op, tiles_dev, plan, stream);
+        case 16: return launch_fused_nw<F, 16, true>(steps, in_f, op, tiles_dev, plan, stream);
+        default: return false;
+        }
+    }
     switch (plan.waves_per_wg) {
-    case 4: return launch_fused_nw<F, 4>(steps, in_f, op, tiles_dev, plan, stream);
-    case 8: return launch_fused_nw<F, 8>(steps, in_f, op, tiles_dev, plan, stream);
-    case 16: return launch_fused_nw<F, 16>(steps, in_f, op, tiles_dev, plan, stream);
+    case 4: return launch_fused_nw<F, 4, false>(steps, in_f, op, tiles_dev, plan, stream);
+    case 8: return launch_fused_nw<F, 8, false>(steps, in_f, op, tiles_dev, plan, stream);
+    case 16: return launch_fused_nw<F, 16, false>(steps, in_f, op, tiles_dev, plan, stream);
     default: return false;
     }
 }
@@ -646,7 +594,6 @@ GemvFormatOps make_gemv_format_ops() {
     o.batch = &launch_batch_fmt<F>;
     o.batch_group = &launch_batch_group_fmt<F>;
     if constexpr (DECODE) {
-        o.plain = &launch_plain_fmt<F>;
         o.plan_group = &plan_group_fmt<F>;
         o.fused = &launch_fused_fmt<F>;
     }

@@ -44,11 +44,6 @@ struct IntStages {
     int32_t* b = nullptr;
 };
 
-// Decode GEMV over an activation that is already quantized in device memory:
-// y[o] = vec_dot(row o, act) for out_f rows of `bpr` bytes. false = no kernel for (dtype, in_f).
-bool launch_gemv(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t in_f,
-                 size_t out_f, const IntStages& st, hipStream_t stream);
-
 // Small-batch GEMV: m activation rows (already quantized) against every weight row, the weights
 // streamed once per chunk of up to 8 rows. y is [m][out_f]; stages [m][out_f][blocks].
 bool launch_gemv_batch(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
@@ -80,6 +75,9 @@ struct GemvOpDesc {
     uint64_t bpr;      // bytes per weight row
     int32_t out_f;
     GemvFusion fus;
+    // optional per-block integer stages, i32 [out_f][blocks] (single-op launches only)
+    int32_t* st_a = nullptr;
+    int32_t* st_b = nullptr;
 };
 
 // What one workgroup of a grouped launch works on: `rows` consecutive weight rows of one op.
@@ -176,8 +174,6 @@ void launch_mfma_i8_peak(int* out, int workgroups, int iters, int random_data, h
 // translation unit, which also defines its accessor below.
 struct GemvFormatOps {
     int elems_per_step = 0;  // K elements one wave step covers
-    bool (*plain)(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t in_f, size_t out_f,
-                  const IntStages& st, hipStream_t stream) = nullptr;
     bool (*batch)(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
                   size_t out_f, const IntStages& st, hipStream_t stream) = nullptr;
     bool (*batch_group)(const BatchTile* tiles, const BatchGroupPlan& plan, const ActQ8& act, size_t m,

@@ -202,17 +202,6 @@ struct SharedLds {
     static constexpr int bytes = dd_off + T * 32 * 8;
 };
 
-// Measurement builds only (-DINFR_MMQ_ABLATE=<bits>, results are wrong): take one component out of
-// the shared-operand kernel's loop to see what it costs. 1: the activation fragment loads, 2: the
-// unpack with its row loads and LDS writes, 4: the LDS operand reads after sub-block 0, 8: the f32
-// epilogue (one integer instruction per output instead), 16: the weight row loads alone.
-#ifndef INFR_MMQ_ABLATE
-#define INFR_MMQ_ABLATE 0
-#endif
-#if INFR_MMQ_ABLATE
-#warning "INFR_MMQ_ABLATE is set: mmq_shared_q4k_kernel computes wrong results (measurement build)"
-#endif
-
 template <int T, bool STAGES, int NW = 4>
 __global__ __launch_bounds__(NW * 64) void mmq_shared_q4k_kernel(
     const uint8_t* __restrict__ w, size_t bpr, const int8_t* __restrict__ qs,
@@ -322,11 +311,8 @@ __global__ __launch_bounds__(NW * 64) void mmq_shared_q4k_kernel(
     for (int b = 0; b < nb; ++b) {
         const uint8_t* cur = lds + (b & 1) * L::bytes;
         // ---- unpack block b+1 into the other buffer, then ask for block b+2's bytes ----
-        if (!(INFR_MMQ_ABLATE & 2)) {
-            unpack_to(lds + ((b + 1) & 1) * L::bytes);
-            if (!(INFR_MMQ_ABLATE & 16)) request_rows(min(b + 2, nb - 1));
-            else asm volatile("" : "+v"(hdr[0]), "+v"(qv[0]));
-        }
+        unpack_to(lds + ((b + 1) & 1) * L::bytes);
+        request_rows(min(b + 2, nb - 1));
         // ---- this wave's 32 tokens of block b ----
         const v8h abs_b = abs_;
         if (h == 0) dql[wave][col] = dtok;
@@ -345,7 +331,7 @@ __global__ __launch_bounds__(NW * 64) void mmq_shared_q4k_kernel(
 #pragma unroll
         for (int sb = 0; sb < 8; ++sb) {
             v4i nlo[T], nhi[T];
-            if (sb < 7 && !(INFR_MMQ_ABLATE & 4)) {
+            if (sb < 7) {
 #pragma unroll
                 for (int t = 0; t < T; ++t) {
                     const uint8_t* src = cur + (size_t)(((sb + 1) * 2) * T + t) * 1024 + lane * 16;
@@ -358,7 +344,7 @@ __global__ __launch_bounds__(NW * 64) void mmq_shared_q4k_kernel(
                 alo[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[sb], flo[t], sb ? alo[t] : zi, 0, 0, 0);
                 ahi[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[sb], fhi[t], sb ? ahi[t] : zi, 0, 0, 0);
             }
-            if (sb < 7 && !(INFR_MMQ_ABLATE & 4)) {
+            if (sb < 7) {
 #pragma unroll
                 for (int t = 0; t < T; ++t) {
                     flo[t] = nlo[t];
@@ -377,7 +363,7 @@ __global__ __launch_bounds__(NW * 64) void mmq_shared_q4k_kernel(
         __builtin_amdgcn_s_setprio(0);
         // the activation registers are free: fetch block b+1 while the epilogue runs
         const int b_this = b;
-        if (!(INFR_MMQ_ABLATE & 1)) request_acts(min(b + 1, nb - 1));
+        request_acts(min(b + 1, nb - 1));
 #pragma unroll
         for (int t = 0; t < T; ++t) {
             const v8h bm = *reinterpret_cast<const v8h*>(cur + L::mn_off + (t * 32 + col) * 16);
@@ -401,10 +387,7 @@ __global__ __launch_bounds__(NW * 64) void mmq_shared_q4k_kernel(
                         }
                     }
                     // sumf += q8.d[b] * (d * sd as f32 - dmin * sm as f32)
-                    if (INFR_MMQ_ABLATE & 8)
-                        acc[t][r] = __builtin_bit_cast(float, __builtin_bit_cast(int, acc[t][r]) ^ sd);
-                    else
-                        acc[t][r] += dq[i] * (d * (float)sd - dmin * smf[r]);
+                    acc[t][r] += dq[i] * (d * (float)sd - dmin * smf[r]);
                 }
             }
         }
@@ -1019,65 +1002,34 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
     }
 }
 
-// Waves per workgroup and blocks per wave and pass for rows of nb blocks; false: another kernel takes them.
-static bool skinny16_shape(int dtype, int nb, size_t m, int* nw, int* bpw) {
-    static const int env_nw = getenv("INFR_HIP_SKINNY16_WAVES") ? atoi(getenv("INFR_HIP_SKINNY16_WAVES")) : 0;
-    static const int env_bpw = getenv("INFR_HIP_SKINNY16_BLOCKS") ? atoi(getenv("INFR_HIP_SKINNY16_BLOCKS")) : 0;
-    static const int env_max = getenv("INFR_HIP_SKINNY16_MAX_M") ? atoi(getenv("INFR_HIP_SKINNY16_MAX_M")) : 16;
-    if ((dtype != 12 && dtype != 13 && dtype != 14) || m > 16 || (int)m > env_max) return false;
+// Which batches the 16-token K-split kernel takes: Q4_K, Q5_K and Q6_K rows of an even number of
+// 256-blocks (weights are staged two blocks at a time), up to 16 tokens. Four waves per workgroup;
+// (eight measured no faster, and four blocks per wave and pass - 576-byte, 64-byte-aligned runs per
+// row - measured 20-25 % slower: a wave then computes for longer before it asks for more).
+constexpr int kSkinny16Waves = 4, kSkinny16Blocks = 2;
+static bool skinny16_shape(int dtype, int nb, size_t m) {
+    if ((dtype != 12 && dtype != 13 && dtype != 14) || m > 16) return false;
     // the dot4 batch kernels, which unpack a weight once per two or four tokens, stay ahead at the
     // bottom: Q5_K at two tokens (4.3-5.3 against 3.8-4.4 TB/s), Q6_K up to four (3.6-4.5 against 3.3-3.9)
     if ((dtype == 13 && m < 3) || (dtype == 14 && m < 5)) return false;
-    int n = env_nw == 8 ? 8 : 4;
-    if (m > 8) n = 4;  // eight waves with 16-token tiles would need more than 64 KB of LDS
-    *nw = n;
-    // (four blocks per wave and pass - 576-byte, 64-byte-aligned runs per row - measured 20-25 % slower:
-    // a wave then computes for longer before it asks for more)
-    *bpw = env_bpw == 2 || env_bpw == 4 ? env_bpw : 2;
-    if (nb % 4 != 0 || dtype == 14) *bpw = 2;  // (a Q6_K stage of four blocks would end in an 8-byte piece)
-    if (nb < *bpw || nb % *bpw != 0) return false;  // weights are staged BPW blocks at a time
-    return true;
+    return nb >= kSkinny16Blocks && nb % kSkinny16Blocks == 0;
 }
 
 bool mmq_skinny16_takes(int dtype, size_t m, size_t in_f) {
-    int nw = 0, bpw = 0;
-    return in_f % 256 == 0 && skinny16_shape(dtype, (int)(in_f / 256), m, &nw, &bpw);
+    return in_f % 256 == 0 && skinny16_shape(dtype, (int)(in_f / 256), m);
 }
 
 template <typename F, bool STAGES>
-static void launch_mmq_skinny16_fmt(int nw, int bpw, const uint8_t* w, size_t bpr, const ActQ8& act, float* y,
-                                    size_t m, int nb, size_t out_f, size_t wgs, const IntStages& st,
-                                    const BatchTile* tiles, hipStream_t stream) {
-    const dim3 grid((unsigned)wgs, 2);
-#define INFR_S16(NW_, BPW_, MT_)                                                                              \
-    hipLaunchKernelGGL((mmq_skinny16_kernel<F, NW_, BPW_, MT_, STAGES>), grid, dim3(NW_ * 64), 0, stream, w, bpr, \
-                       act.qs, act.d, act.bsums, y, (int)m, (int)out_f, nb, st.a, st.b, tiles)
-    if (nw == 4 && m <= 8) {
-        if (bpw == 2) INFR_S16(4, 2, 8);
-        else INFR_S16(4, 4, 8);
-    } else if (nw == 4) {
-        if (bpw == 2) INFR_S16(4, 2, 16);
-        else INFR_S16(4, 4, 16);
-    } else {
-        if (bpw == 2) INFR_S16(8, 2, 8);
-        else INFR_S16(8, 4, 8);
-    }
-#undef INFR_S16
-}
-
-// Q6_K: two blocks per wave and pass only
-template <bool STAGES>
-static void launch_mmq_skinny16_q6k(int nw, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, int nb,
+static void launch_mmq_skinny16_fmt(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, int nb,
                                     size_t out_f, size_t wgs, const IntStages& st, const BatchTile* tiles,
                                     hipStream_t stream) {
-    const dim3 grid((unsigned)wgs, 2);
-#define INFR_S16(NW_, MT_)                                                                                        \
-    hipLaunchKernelGGL((mmq_skinny16_kernel<Skinny16Q6K, NW_, 2, MT_, STAGES>), grid, dim3(NW_ * 64), 0, stream, w, \
-                       bpr, act.qs, act.d, act.bsums, y, (int)m, (int)out_f, nb, st.a, st.b, tiles)
-    if (nw == 4 && m <= 8) INFR_S16(4, 8);
-    else if (nw == 4) INFR_S16(4, 16);
-    else INFR_S16(8, 8);
-#undef INFR_S16
+    const dim3 grid((unsigned)wgs, 2), block(kSkinny16Waves * 64);
+    if (m <= 8)
+        hipLaunchKernelGGL((mmq_skinny16_kernel<F, kSkinny16Waves, kSkinny16Blocks, 8, STAGES>), grid, block, 0, stream,
+                           w, bpr, act.qs, act.d, act.bsums, y, (int)m, (int)out_f, nb, st.a, st.b, tiles);
+    else
+        hipLaunchKernelGGL((mmq_skinny16_kernel<F, kSkinny16Waves, kSkinny16Blocks, 16, STAGES>), grid, block, 0, stream,
+                           w, bpr, act.qs, act.d, act.bsums, y, (int)m, (int)out_f, nb, st.a, st.b, tiles);
 }
 
 template <bool STAGES>
@@ -1085,14 +1037,13 @@ static bool launch_mmq_skinny16(int dtype, const uint8_t* w, size_t bpr, const A
                                 size_t in_f, size_t out_f, size_t wgs, const IntStages& st, const BatchTile* tiles,
                                 hipStream_t stream) {
     const int nb = (int)(in_f / 256);
-    int nw = 0, bpw = 0;
-    if (in_f % 256 != 0 || !skinny16_shape(dtype, nb, m, &nw, &bpw)) return false;
+    if (in_f % 256 != 0 || !skinny16_shape(dtype, nb, m)) return false;
     if (dtype == 12)
-        launch_mmq_skinny16_fmt<Skinny16Q4K, STAGES>(nw, bpw, w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
+        launch_mmq_skinny16_fmt<Skinny16Q4K, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     else if (dtype == 13)
-        launch_mmq_skinny16_fmt<Skinny16Q5K, STAGES>(nw, bpw, w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
+        launch_mmq_skinny16_fmt<Skinny16Q5K, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     else
-        launch_mmq_skinny16_q6k<STAGES>(nw, w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
+        launch_mmq_skinny16_fmt<Skinny16Q6K, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     return true;
 }
 
@@ -1138,8 +1089,7 @@ void launch_mmq_q4k_gathered(const uint8_t* bank, size_t expert_stride, size_t b
 
 bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const ActQ8& act, float* y,
                 size_t m, size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream) {
-    // Q4_K routes by token count (thresholds from sweeps at K = 4096, N = 12288; the env knobs exist
-    // for such sweeps):
+    // Q4_K routes by token count (thresholds from sweeps at K = 4096, N = 12288):
     //   2..32      skinny kernel, K split over the waves of a workgroup
     //   33..127    tiled kernel, 32 tokens x 128 rows per workgroup (most workgroups for few tokens)
     //   128..      shared-operand kernel, 128 tokens x 32 rows (x 64 rows from 1024 tokens up)
@@ -1151,10 +1101,7 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
     // rows beyond the decode / small-batch kernels' length, when whole 256s, take the MFMA kernel of
     // their format at any token count (a 128-token tile for one token: slow, but exact and bounded)
     const bool long_row = gemv_row_too_long(dtype, in_f) && in_f % 256 == 0;
-    static const int env_skinny_max = getenv("INFR_HIP_MMQ_SKINNY_MAX_M") ? atoi(getenv("INFR_HIP_MMQ_SKINNY_MAX_M")) : 32;
-    static const int env_shared_min = getenv("INFR_HIP_MMQ_SHARED_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_SHARED_MIN_M")) : 128;
-    static const int env_shared_rows = getenv("INFR_HIP_MMQ_SHARED_ROWS") ? atoi(getenv("INFR_HIP_MMQ_SHARED_ROWS")) : 0;
-    if (dtype == 12 && ((int)m >= env_shared_min || long_row)) {
+    if (dtype == 12 && (m >= 128 || long_row)) {
         launch_quantize_q8_tiled(x, m, in_f, act, stream);
         if (mmq_strip_q4k_takes(m, out_f)) {
             launch_mmq_strip_q4k(w, bpr, act, y, m, in_f, out_f, st, stream);
@@ -1165,59 +1112,51 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
         // 256-token tiles pad up to 128 tokens more than 128-token tiles do: taken when both pad alike,
         // or when that padding is small against the batch
         const size_t pad_w = (m + 255) / 256 * 256, pad_n = (m + 127) / 128 * 128;
-        const bool wide = env_shared_rows ? env_shared_rows == 64 : (m > 768 && (pad_w == pad_n || pad_w >= 2048));
+        const bool wide = m > 768 && (pad_w == pad_n || pad_w >= 2048);
         // two row tiles: eight waves (256 tokens) per workgroup, each unpacking one tile's nibble pair -
         // half the unpack work and row loads per output tile; 729 / 763 / 766 against 669 / 719 / 731
         // TOPS at 1024 / 2048 / 4096 tokens (12288 x 4096)
-        static const int env_w8 = getenv("INFR_HIP_MMQ_SHARED_WAVES") ? atoi(getenv("INFR_HIP_MMQ_SHARED_WAVES")) : 8;
-        if (wide && env_w8 == 8) launch_mmq_shared_q4k<2, 8>(w, bpr, act, y, m, in_f, out_f, st, stream);
-        else if (wide) launch_mmq_shared_q4k<2>(w, bpr, act, y, m, in_f, out_f, st, stream);
+        if (wide) launch_mmq_shared_q4k<2, 8>(w, bpr, act, y, m, in_f, out_f, st, stream);
         else launch_mmq_shared_q4k<1>(w, bpr, act, y, m, in_f, out_f, st, stream);
         return true;
     }
     // Q6_K: the MFMA kernel's time is flat up to 128 tokens (63 / 103 / 39 us at 12288 x 4096,
     // 4096 x 12288, 1024 x 4096) and the dot4 batches cost ~3.5 / 3.2 / 1.1 us per token there, so
     // it takes over from 33 tokens
-    static const int env_q6k_min = getenv("INFR_HIP_MMQ_Q6K_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_Q6K_MIN_M")) : 33;
-    if (dtype == 14 && ((int)m >= env_q6k_min || long_row)) {
+    if (dtype == 14 && (m >= 33 || long_row)) {
         launch_quantize_q8_tiled(x, m, in_f, act, stream);
         launch_mmq_shared_q6k(w, bpr, act, y, m, in_f, out_f, st, stream);
         return true;
     }
-    static const int env_q5k_min = getenv("INFR_HIP_MMQ_Q5K_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_Q5K_MIN_M")) : 33;
-    if (dtype == 13 && ((int)m >= env_q5k_min || long_row)) {
+    if (dtype == 13 && (m >= 33 || long_row)) {
         launch_quantize_q8_tiled(x, m, in_f, act, stream);
         launch_mmq_shared_q5k(w, bpr, act, y, m, in_f, out_f, st, stream);
         return true;
     }
     // (their kernel's flat time up to 128 tokens, ~145 us at 4096 x 12288, meets the dot4 batches'
     // ~2.1 us per token at 64 tokens)
-    static const int env_nib_min = getenv("INFR_HIP_MMQ_NIB32_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_NIB32_MIN_M")) : 65;
     if ((dtype == 2 || dtype == 3 || dtype == 6 || dtype == 7 || dtype == 20) && in_f % 256 == 0 &&
-        ((int)m >= env_nib_min || long_row)) {
+        (m >= 65 || long_row)) {
         launch_quantize_q8_32_tiled(x, m, in_f, false, act, stream);
         return launch_mmq_shared_nib32(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
     }
-    static const int env_q2_min = getenv("INFR_HIP_MMQ_Q2_0_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_Q2_0_MIN_M")) : 65;
-    if (dtype == 42 && in_f % 256 == 0 && ((int)m >= env_q2_min || long_row)) {
+    if (dtype == 42 && in_f % 256 == 0 && (m >= 65 || long_row)) {
         launch_quantize_q8_32_tiled(x, m, in_f, true, act, stream);
         return launch_mmq_shared_nib32(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
     }
-    static const int env_q8_0_min = getenv("INFR_HIP_MMQ_Q8_0_MIN_M") ? atoi(getenv("INFR_HIP_MMQ_Q8_0_MIN_M")) : 33;
-    if (dtype == 8 && in_f % 256 == 0 && ((int)m >= env_q8_0_min || long_row)) {
+    if (dtype == 8 && in_f % 256 == 0 && (m >= 33 || long_row)) {
         launch_quantize_q8_tiled(x, m, in_f, act, stream);
         launch_mmq_shared_q8_0(w, bpr, act, y, m, in_f, out_f, st, stream);
         return true;
     }
     launch_quantize_q8(x, m, in_f, act_is_per32(dtype, in_f), act, stream);
-    static const int env_dot4_max = getenv("INFR_HIP_Q4K_DOT4_MAX_M") ? atoi(getenv("INFR_HIP_Q4K_DOT4_MAX_M")) : 0;
-    if ((dtype != 12 || (int)m > env_dot4_max) && mmq_skinny16_takes(dtype, m, in_f)) {
+    if (mmq_skinny16_takes(dtype, m, in_f)) {
         const size_t wgs = (out_f + 31) / 32;
         return st.a ? launch_mmq_skinny16<true>(dtype, w, bpr, act, y, m, in_f, out_f, wgs, st, nullptr, stream)
                     : launch_mmq_skinny16<false>(dtype, w, bpr, act, y, m, in_f, out_f, wgs, st, nullptr, stream);
     }
-    if (dtype != 12 || (int)m <= env_dot4_max) return launch_gemv_batch(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
-    if ((int)m <= env_skinny_max) {
+    if (dtype != 12) return launch_gemv_batch(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
+    if (m <= 32) {
         // four blocks per round; eight for long rows or when four would leave most SIMDs without a wave
         const size_t wgs = (out_f + 31) / 32 * ((m + 31) / 32);
         if (in_f >= 8192 || (wgs * 4 < 1024 && in_f >= 2048))

@@ -1004,7 +1004,7 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     // int8-MFMA GEMM per (expert, 32 pairs) tile, so an expert's weights are read once per 32 of
     // its pairs instead of once per pair. From an average of `bucket_min` pairs per expert up (the
     // per-pair GEMVs win below: most tiles would hold one or two pairs).
-    static const int bucket_min = getenv("INFR_HIP_MOE_BUCKET_MIN") ? atoi(getenv("INFR_HIP_MOE_BUCKET_MIN")) : 4;
+    constexpr int bucket_min = 4;
     // (a Q6_K tile costs more than the others': at four pairs per expert its per-pair GEMVs tie with
     // the tiles, 313 us per layer either way, and it is bucketed from eight; Q5_K and Q8_0 banks
     // gain from four on, 179 against 254 and 299 against 399 us)

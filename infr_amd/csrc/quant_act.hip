@@ -34,38 +34,67 @@ __global__ __launch_bounds__(256) void quantize_q8_kernel(const float* __restric
 //   d     [(g*nb + b)*32 + token%32]
 //   bsums (read as f16) [(g*nb + b)*64 + h*32 + token%32][8]: per-32 sums split bsum = lo + rest,
 //         lo = bsum & 63 in the h = 0 half, bsum - lo in the h = 1 half (both exact in f16)
-// so that a wave's fragment load is one contiguous kilobyte. Slots of tokens past m are not written.
-__global__ __launch_bounds__(256) void quantize_q8_tiled_kernel(const float* __restrict__ x,
+// so that a wave's fragment load is one contiguous kilobyte.
+// One workgroup makes the whole 8 KiB code tile of (token group g, block b): each of its sixteen
+// waves quantizes two tokens' chunks, the codes cross through LDS, and the tile leaves as 512
+// contiguous 16-byte stores - a wave that
+// wrote its own token's codes in place would scatter every store over sixteen 128-byte lines.
+// Tokens past m quantize zeros (their slots hold d = 0 and zero codes).
+constexpr int kTiledQuantWaves = 16, kTiledQuantPerWave = 32 / kTiledQuantWaves;
+__global__ __launch_bounds__(kTiledQuantWaves * 64) void quantize_q8_tiled_kernel(const float* __restrict__ x,
                                                                 int8_t* __restrict__ qs,
                                                                 float* __restrict__ d,
                                                                 _Float16* __restrict__ bsh,
-                                                                size_t n_chunks, int nb) {
-    const int lane = threadIdx.x & 63;
-    const size_t chunk = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (chunk >= n_chunks) return;  // wave-uniform
-    const v4f v = *reinterpret_cast<const v4f*>(x + chunk * 256 + (size_t)lane * 4);
-    uint32_t packed;
-    float dd;
-    int s, s16;
-    quantize_chunk_values<false>(v, packed, dd, s, s16);
-    const size_t tok = chunk / nb, b = chunk % nb;
-    const size_t gb = (tok >> 5) * nb + b;
-    const int col = (int)(tok & 31);
-    const int sb = lane >> 3, h = (lane >> 2) & 1, j4 = lane & 3;
-    reinterpret_cast<uint32_t*>(qs)[((gb * 8 + sb) * 64 + h * 32 + col) * 4 + j4] = packed;
-    if (lane == 0) d[gb * 32 + col] = dd;
-    if ((lane & 7) == 0) {
-        const int lo = s & 63;
-        bsh[(gb * 64 + col) * 8 + sb] = (_Float16)lo;
-        bsh[(gb * 64 + 32 + col) * 8 + sb] = (_Float16)(s - lo);
+                                                                int m, int nb) {
+    // [sub-block][lane = h*32 + token][16 B], each sub-block's KiB followed by 16 B of padding so
+    // that the lanes of a wave (eight sub-blocks x two halves x four dwords of one token) spread
+    // over the banks
+    constexpr int kSbStride = 1024 + 16;
+    __shared__ __attribute__((aligned(16))) uint8_t tile[8 * kSbStride];
+    __shared__ __attribute__((aligned(16))) _Float16 sums[64 * 8];
+    __shared__ float scales[32];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int b = blockIdx.x, g = blockIdx.y;
+    const size_t in_f = (size_t)nb * 256;
+    constexpr int PW = kTiledQuantPerWave;
+    v4f v[PW];
+#pragma unroll
+    for (int i = 0; i < PW; ++i) {
+        const int tok = g * 32 + wave * PW + i;
+        v[i] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+        if (tok < m) v[i] = gload<v4f>(x + (size_t)tok * in_f + (size_t)b * 256 + lane * 4);
     }
+    const int sb = lane >> 3, h = (lane >> 2) & 1, j4 = lane & 3;
+#pragma unroll
+    for (int i = 0; i < PW; ++i) {
+        const int col = wave * PW + i;
+        uint32_t packed;
+        float dd;
+        int s, s16;
+        quantize_chunk_values<false>(v[i], packed, dd, s, s16);
+        *reinterpret_cast<uint32_t*>(tile + sb * kSbStride + (h * 32 + col) * 16 + j4 * 4) = packed;
+        if (lane == 0) scales[col] = dd;
+        if ((lane & 7) == 0) {
+            const int lo = s & 63;
+            sums[col * 8 + sb] = (_Float16)lo;
+            sums[(32 + col) * 8 + sb] = (_Float16)(s - lo);
+        }
+    }
+    __syncthreads();
+    const size_t gb = (size_t)g * nb + b;
+    if (tid < 512) {
+        const int piece = tid;  // 16-byte piece of the tile: [sub-block][lane]
+        const v4i c = *reinterpret_cast<const v4i*>(tile + (piece >> 6) * kSbStride + (piece & 63) * 16);
+        gstore<v4i>(qs + gb * (8 * 1024) + (size_t)piece * 16, c);
+    }
+    if (tid < 64) gstore<v4i>(bsh + (gb * 64 + tid) * 8, *reinterpret_cast<const v4i*>(&sums[tid * 8]));
+    if (tid < 32) gstore<float>(d + gb * 32 + tid, scales[tid]);
 }
 
 void launch_quantize_q8_tiled(const float* x, size_t m, size_t k, const ActQ8& out, hipStream_t stream) {
-    const size_t n_chunks = m * k / 256;
-    if (n_chunks == 0) return;
-    hipLaunchKernelGGL(quantize_q8_tiled_kernel, dim3((unsigned)((n_chunks + 3) / 4)), dim3(256), 0, stream, x,
-                       out.qs, out.d, reinterpret_cast<_Float16*>(out.bsums), n_chunks, (int)(k / 256));
+    if (m == 0 || k < 256) return;
+    hipLaunchKernelGGL(quantize_q8_tiled_kernel, dim3((unsigned)(k / 256), (unsigned)((m + 31) / 32)),
+                       dim3(kTiledQuantWaves * 64), 0, stream, x, out.qs, out.d, reinterpret_cast<_Float16*>(out.bsums), (int)m, (int)(k / 256));
 }
 
 // The per-32 quantizer (quantize_q8_32, crates/infr-cpu/src/quant.rs:97-117) in the same tiled code

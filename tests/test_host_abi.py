@@ -95,3 +95,73 @@ def test_synth_q2_0_codes_are_ternary():
     assert codes.max() == 2 and set(np.unique(codes)) == {0, 1, 2}
     frac = [(codes == v).mean() for v in (0, 1, 2)]
     assert all(abs(f - 1 / 3) < 0.02 for f in frac)
+
+
+# ---- the Rust mirror in INTEGRATION.md against the C header's layout ----
+
+_RUST_TYPES = {"i32": (4, 4), "u32": (4, 4), "f32": (4, 4), "u64": (8, 8), "i64": (8, 8), "usize": (8, 8)}
+
+
+def _rust_repr_c_structs():
+    """name -> [(field, size, align)] for every `#[repr(C)] ... pub struct` in INTEGRATION.md."""
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    out = {}
+    for name, body in re.findall(r"#\[repr\(C\)\][^{;]*?pub struct (\w+)\s*\{(.*?)\}", text, flags=re.S):
+        body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+        body = re.sub(r"//[^\n]*", "", body)
+        fields = []
+        for decl in [d.strip() for d in body.split(",") if d.strip()]:
+            fname, ftype = [t.strip() for t in decl.split(":", 1)]
+            arr = re.fullmatch(r"\[(\w+);\s*(\d+)\]", ftype)
+            if arr:
+                size, align = (1, 1) if arr.group(1) in ("c_char", "u8", "i8") else _RUST_TYPES[arr.group(1)]
+                fields.append((fname, size * int(arr.group(2)), align))
+            elif ftype in _RUST_TYPES:
+                fields.append((fname, *_RUST_TYPES[ftype]))
+            else:
+                fields.append((fname, ftype, None))        # a nested struct, resolved below
+        out[name] = fields
+    return out
+
+
+def _repr_c_layout(structs, name):
+    """offsets, size and alignment of a #[repr(C)] struct: C's rules, which repr(C) promises."""
+    off, max_align, offsets = 0, 1, {}
+    for fname, size, align in structs[name]:
+        if align is None:
+            _, size, align = _repr_c_layout(structs, size)
+        off = (off + align - 1) // align * align
+        offsets[fname] = off
+        off += size
+        max_align = max(max_align, align)
+    return offsets, (off + max_align - 1) // max_align * max_align, max_align
+
+
+def _c_layout(tmp_path, ctype, fields):
+    """offsetof of every field and sizeof, as gcc lays out the public header's struct."""
+    import subprocess
+    src = tmp_path / f"layout_{ctype}.c"
+    lines = "\n".join(f'    printf("{f} %zu\\n", offsetof({ctype}, {f}));' for f in fields)
+    src.write_text(f'#include <stddef.h>\n#include <stdio.h>\n#include "infr_hip.h"\nint main(void) {{\n{lines}\n'
+                   f'    printf("sizeof %zu\\n", sizeof({ctype}));\n    return 0;\n}}\n')
+    exe = tmp_path / f"layout_{ctype}"
+    subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
+    return dict(zip(out[0::2], map(int, out[1::2])))
+
+
+@pytest.mark.parametrize("rust,ctype", [("HipOp", "infr_hip_op_t"), ("HipMoe", "infr_hip_moe_params_t"),
+                                        ("HipCaps", "infr_hip_caps_t")])
+def test_rust_mirror_structs_match_the_c_header(tmp_path, rust, ctype):
+    """The `impl Backend for HipBackend` shim cannot be compiled here (no Rust toolchain); what can be
+    checked is that its #[repr(C)] structs still describe the header's structs field by field."""
+    structs = _rust_repr_c_structs()
+    assert rust in structs, f"INTEGRATION.md no longer declares {rust}"
+    offsets, size, _ = _repr_c_layout(structs, rust)
+    c = _c_layout(tmp_path, ctype, list(offsets))          # a field the header lacks fails to compile
+    assert c.pop("sizeof") == size, f"{rust} and {ctype} differ in size"
+    assert c == offsets
+    # and the header has no field the mirror lacks: the ctypes mirror lists them all
+    ct = {"HipOp": B._Op, "HipMoe": B._MoeParams, "HipCaps": B._Caps}[rust]
+    assert [f[0] for f in ct._fields_] == list(offsets)
+    assert ctypes.sizeof(ct) == size
