@@ -162,26 +162,33 @@ __global__ __launch_bounds__(256) void moe_select_kernel(const float* __restrict
 // infr-cpu's `dot` keeps 8 FMA accumulators (element i goes to accumulator i mod 8) and adds them
 // in order; each accumulator is a strictly sequential chain, so the order cannot be parallelised
 // beyond the 8 accumulators without changing the rounding. A workgroup takes `epw` expert rows
-// (1 or 4) and 32 / epw activation rows: all 256 threads stage K-chunks of them into LDS with
+// (1, 4 or 8) and 32 / epw activation rows: all 256 threads stage K-chunks of them into LDS with
 // coalesced 16-byte loads, and eight lanes per (expert, token) pair - one accumulator each - run
-// the chains from LDS, carrying them across chunks.
+// the chains from LDS, carrying them across chunks. A row sits in LDS accumulator-major (element i
+// at [i % 8][i / 8]), so a lane reads four steps of its chain with one 16-byte access.
 // With a single row (tickets != nullptr) the last workgroup to finish - a ticket counter, left
-// at zero again - runs the selection too, which saves a launch. ne % 8 == 0 is required.
+// at zero again - runs the selection too, which saves a launch; eight experts per workgroup keep
+// that to a handful of tickets (atomics on one address complete one after another, ~65 ns each).
+// ne % 32 == 0 is required.
 constexpr int kRouterPairs = 32, kRouterChunk = 512;
+// floats between two staged rows of kc elements: eight accumulator rows of kc / 8 + 4
+__host__ __device__ constexpr int router_row_floats(int kc) { return 8 * (kc / 8 + 4); }
 
+// NL: 16-byte loads a thread has in flight while staging (24 at a single row: the nine rows of a
+// workgroup arrive in one round trip)
+template <int NL>
 __global__ __launch_bounds__(256) void moe_router_kernel(
     const float* __restrict__ router, const float* __restrict__ rx, float* __restrict__ logits,
     int* __restrict__ tickets, int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, int ne,
     int n_expert, int rows, int n_used, float scale, int kc, int epw) {
-    extern __shared__ __attribute__((aligned(16))) float rl[];  // [epw][kc + 8] | [32 / epw][kc + 8]
+    extern __shared__ __attribute__((aligned(16))) float rl[];  // [epw] rows | [32 / epw] rows
     __shared__ __attribute__((aligned(16))) SelectLds sel;
     __shared__ int s_last;
     const int tid = threadIdx.x;
     const int tpw = kRouterPairs / epw;
     const int e0 = blockIdx.x * epw, t0 = blockIdx.y * tpw;
     const int n_e = min(epw, n_expert - e0), n_t = min(tpw, rows - t0);
-    // rows are kc + 8 floats apart in LDS: the lanes of different pairs then read different banks
-    const int ld = kc + 8;
+    const int ld = router_row_floats(kc), la = kc / 8 + 4;  // row and accumulator-row strides
     float* lw = rl;
     float* lx = rl + epw * ld;
     const int pair = tid >> 3, j = tid & 7;
@@ -192,27 +199,39 @@ __global__ __launch_bounds__(256) void moe_router_kernel(
         const int n = min(kc, ne - k0), n4 = n / 4;
         const int total = (n_e + n_t) * n4;
         if (k0) __syncthreads();
-        for (int base = 0; base < total; base += 256 * 8) {  // eight loads in flight per thread
-            v4f tmp[8];
-            float* dst[8];
+        for (int base = 0; base < total; base += 256 * NL) {  // NL loads in flight per thread
+            v4f tmp[NL];
+            float* dst[NL];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
+            for (int u = 0; u < NL; ++u) {
                 const int i = base + u * 256 + tid;
                 const int row = i / n4, q = i % n4;
                 const float* src = row < n_e ? router + (size_t)(e0 + row) * ne : rx + (size_t)(t0 + row - n_e) * ne;
-                dst[u] = (row < n_e ? lw + row * ld : lx + (row - n_e) * ld) + 4 * q;
+                // elements 4q .. 4q+3 are accumulators 4(q & 1) .. +3 at step q / 2
+                dst[u] = (row < n_e ? lw + row * ld : lx + (row - n_e) * ld) + 4 * (q & 1) * la + (q >> 1);
                 if (i < total) tmp[u] = reinterpret_cast<const v4f*>(src + k0)[q];
             }
 #pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (base + u * 256 + tid < total) *reinterpret_cast<v4f*>(dst[u]) = tmp[u];
+            for (int u = 0; u < NL; ++u)
+                if (base + u * 256 + tid < total) {
+                    dst[u][0] = tmp[u].x;
+                    dst[u][la] = tmp[u].y;
+                    dst[u][2 * la] = tmp[u].z;
+                    dst[u][3 * la] = tmp[u].w;
+                }
         }
         __syncthreads();
         if (active) {
-            const float* a = lw + e * ld + j;
-            const float* xx = lx + t * ld + j;
-#pragma unroll 16
-            for (int c = 0; c < n / 8; ++c) acc = __builtin_fmaf(a[c * 8], xx[c * 8], acc);
+            const v4f* a = reinterpret_cast<const v4f*>(lw + e * ld + j * la);
+            const v4f* xx = reinterpret_cast<const v4f*>(lx + t * ld + j * la);
+#pragma unroll 8
+            for (int c = 0; c < n / 32; ++c) {
+                const v4f av = a[c], xv = xx[c];
+                acc = __builtin_fmaf(av.x, xv.x, acc);
+                acc = __builtin_fmaf(av.y, xv.y, acc);
+                acc = __builtin_fmaf(av.z, xv.z, acc);
+                acc = __builtin_fmaf(av.w, xv.w, acc);
+            }
         }
     }
     // s = acc[0] + acc[1] + ... + acc[7] in order
@@ -553,93 +572,88 @@ __device__ __forceinline__ float seg_sum(float v, int seg_base, int quads) {
 }
 
 // gate/up at one token: act[slot][o] = silu(gate_e[o] . x) * (up_e[o] . x), e = ids[slot].
-// A wave takes steps_per_wave consecutive row steps and keeps the next step's rows in flight.
-template <typename P>
+// A wave takes SPW consecutive row steps and requests all their rows before it computes the
+// first: at one token the kernel is a few memory round trips deep, so every request it can make
+// up front is a round trip less.
+template <typename P, int SPW>
 __global__ __launch_bounds__(256) void moe_gate_up_f32_kernel(
     const uint8_t* __restrict__ gate, const uint8_t* __restrict__ up, size_t gate_stride,
     size_t up_stride, const int32_t* __restrict__ ids, const float* __restrict__ x,
-    float* __restrict__ act, int ne, int nff, int steps_per_wave) {
+    float* __restrict__ act, int ne, int nff) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int S = ne / 64, rps = 64 / S;  // lanes per weight row, rows per wave step
     const int seg = lane / S, u = lane % S;
     const bool lane_ok = seg < rps;
     const int slot = blockIdx.y;
     const int steps_total = (nff + rps - 1) / rps;
-    const int st0 = (blockIdx.x * 4 + wave) * steps_per_wave;
+    const int st0 = (blockIdx.x * 4 + wave) * SPW;
     if (st0 >= steps_total) return;
-    const int st_end = min(st0 + steps_per_wave, steps_total);
     const int e = ids[slot];
     const size_t bpr = (size_t)(ne / 256) * P::kBlockBytes;
     const uint8_t* gw = gate + (size_t)e * gate_stride;
     const uint8_t* uw = up + (size_t)e * up_stride;
-    typename P::Row g, up_r;
-    {
-        const int o = st0 * rps + seg;
+    typename P::Row g[SPW], up_r[SPW];
+#pragma unroll
+    for (int i = 0; i < SPW; ++i) {
+        const int o = (st0 + i) * rps + seg;
         const bool ok = lane_ok && o < nff;
-        P::load_row(g, gw + (size_t)(ok ? o : 0) * bpr, u, ok);
-        P::load_row(up_r, uw + (size_t)(ok ? o : 0) * bpr, u, ok);
+        P::load_row(g[i], gw + (size_t)(ok ? o : 0) * bpr, u, ok);
+        P::load_row(up_r[i], uw + (size_t)(ok ? o : 0) * bpr, u, ok);
     }
     typename P::X xa;
     P::load_x(xa, x, u, lane_ok);
-    for (int st = st0; st < st_end; ++st) {
-        const int o = st * rps + seg;
+#pragma unroll
+    for (int i = 0; i < SPW; ++i) {
+        const int o = (st0 + i) * rps + seg;
         const bool ok = lane_ok && o < nff;
-        const typename P::Row gc = g, uc = up_r;
-        if (st + 1 < st_end) {
-            const int o2 = o + rps;
-            const bool ok2 = lane_ok && o2 < nff;
-            P::load_row(g, gw + (size_t)(ok2 ? o2 : 0) * bpr, u, ok2);
-            P::load_row(up_r, uw + (size_t)(ok2 ? o2 : 0) * bpr, u, ok2);
-        }
-        const float gs = seg_sum(P::partial(gc, xa, u), seg * S, S / 4);
-        const float us = seg_sum(P::partial(uc, xa, u), seg * S, S / 4);
+        const float gs = seg_sum(P::partial(g[i], xa, u), seg * S, S / 4);
+        const float us = seg_sum(P::partial(up_r[i], xa, u), seg * S, S / 4);
         if (ok && u == 0) act[(size_t)slot * nff + o] = gs / (1.0f + expf(-gs)) * us;
     }
 }
 
 // down + accumulate at one token: out[o] = sum_k w_k * (down_{ids[k]}[o] . act[k]), k in rank
 // order. One wave per selected expert (up to 16 at a time), every wave of a workgroup on the same
-// `steps` row steps; the per-expert results meet in LDS and are added in rank order with a
-// separate multiply and add, as the CPU's `*o += w_e * yv`.
+// STEPS row steps, all requested up front; the per-expert results meet in LDS and are added in rank
+// order with a separate multiply and add, as the CPU's `*o += w_e * yv`.
 constexpr int kDownMaxSteps = 4, kDownMaxWaves = 16;
+#ifndef MOE_WAVES_WANTED
+#define MOE_WAVES_WANTED 1024
+#endif
+constexpr int kMoeWavesWanted = MOE_WAVES_WANTED;
 
-template <typename P>
+template <typename P, int STEPS>
 __global__ __launch_bounds__(1024) void moe_down_f32_kernel(
     const uint8_t* __restrict__ down, size_t down_stride, const int32_t* __restrict__ ids,
     const float* __restrict__ wts, const float* __restrict__ act, float* __restrict__ out, int nff,
-    int ne, int n_used, int steps) {
+    int ne, int n_used) {
     __shared__ float ys[kDownMaxSteps][kDownMaxWaves][16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     const int S = nff / 64, rps = 64 / S;
     const int seg = lane / S, u = lane % S;
     const bool lane_ok = seg < rps;
     const size_t bpr = (size_t)(nff / 256) * P::kBlockBytes;
-    const int st0 = blockIdx.x * steps;
+    const int st0 = blockIdx.x * STEPS;
     const int own_s = threadIdx.x / rps, own_seg = threadIdx.x % rps;  // output this thread adds up
-    const bool owner = (int)threadIdx.x < steps * rps;
+    const bool owner = (int)threadIdx.x < STEPS * rps;
     float acc = 0.0f;
     for (int k0 = 0; k0 < n_used; k0 += nw) {
         const int k = k0 + wave;
         if (k0) __syncthreads();
         if (k < n_used) {
             const uint8_t* dw = down + (size_t)ids[k] * down_stride;
-            typename P::Row row;
-            {
-                const int o = st0 * rps + seg;
+            typename P::Row row[STEPS];
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s) {
+                const int o = (st0 + s) * rps + seg;
                 const bool ok = lane_ok && o < ne;
-                P::load_row(row, dw + (size_t)(ok ? o : 0) * bpr, u, ok);
+                P::load_row(row[s], dw + (size_t)(ok ? o : 0) * bpr, u, ok);
             }
             typename P::X xa;
             P::load_x(xa, act + (size_t)k * nff, u, lane_ok);
-            for (int s = 0; s < steps; ++s) {
-                const int o = (st0 + s) * rps + seg;
-                const typename P::Row cur = row;
-                if (s + 1 < steps) {
-                    const int o2 = o + rps;
-                    const bool ok2 = lane_ok && o2 < ne;
-                    P::load_row(row, dw + (size_t)(ok2 ? o2 : 0) * bpr, u, ok2);
-                }
-                const float yk = seg_sum(P::partial(cur, xa, u), seg * S, S / 4);
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s) {
+                const float yk = seg_sum(P::partial(row[s], xa, u), seg * S, S / 4);
                 if (lane_ok && u == 0) ys[s][wave][seg] = yk;
             }
         }
@@ -923,22 +937,32 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     int32_t* tile_slot0 = (int32_t*)take(max_tiles * 4);
     int32_t* tile_count = (int32_t*)take(max_tiles * 4);
 
-    // one expert per workgroup at a single row (more workgroups), four once rows fill the pairs;
-    // whole rows in one chunk when they fit 64 KiB of LDS, else kRouterChunk columns at a time
-    const int epw = s.rows == 1 ? 1 : 4, tpw = kRouterPairs / epw;
+    // eight experts per workgroup at a single row (few tickets), four once rows fill the pairs; whole
+    // rows in one chunk when they fit the LDS a workgroup may have, else kRouterChunk columns at a time
+    constexpr size_t kRouterLdsMax = 144 * 1024;
+    int epw = s.rows == 1 ? 8 : 4;
+    while (epw > 1 && (size_t)(epw + 1) * router_row_floats(s.ne) * sizeof(float) > kRouterLdsMax) epw /= 2;
+    const int tpw = kRouterPairs / epw;
     const int n_t = std::min(s.rows, tpw);
-    const int kc = (size_t)(epw + n_t) * (s.ne + 8) * 4 <= 64 * 1024 ? s.ne : kRouterChunk;
-    const size_t router_lds = (size_t)(epw + n_t) * (kc + 8) * sizeof(float);
+    const int kc = (size_t)(epw + n_t) * router_row_floats(s.ne) * sizeof(float) <= (s.rows == 1 ? kRouterLdsMax : 64 * 1024)
+                       ? s.ne : kRouterChunk;
+    const size_t router_lds = (size_t)(epw + n_t) * router_row_floats(kc) * sizeof(float);
+    if (router_lds > 64 * 1024)
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_router_kernel<24>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)router_lds);
     if (s.rows >= kRtMinRows)
         hipLaunchKernelGGL(moe_router_tile_kernel,
                            dim3((unsigned)((s.n_expert + kRtE - 1) / kRtE), (unsigned)((s.rows + kRtT - 1) / kRtT)),
                            dim3(kRtThreads), 0, stream, b.router, b.router_x, logits, s.ne, s.n_expert, s.rows);
+    else if (s.rows == 1)
+        hipLaunchKernelGGL(moe_router_kernel<24>, dim3((unsigned)((s.n_expert + epw - 1) / epw), 1), dim3(256), router_lds,
+                           stream, b.router, b.router_x, logits, tickets, sel_idx, sel_w, s.ne, s.n_expert, s.rows,
+                           s.n_used, s.scale, kc, epw);
     else
-        hipLaunchKernelGGL(moe_router_kernel,
+        hipLaunchKernelGGL(moe_router_kernel<8>,
                            dim3((unsigned)((s.n_expert + epw - 1) / epw), (unsigned)((s.rows + tpw - 1) / tpw)),
-                           dim3(256), router_lds, stream, b.router, b.router_x, logits,
-                           s.rows == 1 ? tickets : nullptr, sel_idx, sel_w, s.ne, s.n_expert, s.rows, s.n_used,
-                           s.scale, kc, epw);
+                           dim3(256), router_lds, stream, b.router, b.router_x, logits, (int*)nullptr, sel_idx, sel_w,
+                           s.ne, s.n_expert, s.rows, s.n_used, s.scale, kc, epw);
     // the expert input is quantized by the selection kernel's workgroups (one per row) when its rows
     // are whole 256s
     const bool quant_in_select = s.rows > 1 && s.ne % 256 == 0;
@@ -956,32 +980,48 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
             return "rows == 1 carries Q4_K / Q5_K / Q6_K / Q8_0 expert banks (gate and up of one format)";
         if (s.ne > 4096 || s.n_ff > 4096) return "rows == 1 needs ne, n_ff_exp <= 4096";
         // row steps per wave: amortise the 64 activation registers while keeping >= ~1024 waves
-        auto steps_per_wave = [](int wave_steps) { return std::max(1, std::min(4, wave_steps / 1024)); };
+        auto steps_per_wave = [](int wave_steps) { return std::max(1, std::min(4, wave_steps / kMoeWavesWanted)); };
         const int rps_g = 64 / (s.ne / 64);
         const int steps_g = (s.n_ff + rps_g - 1) / rps_g;
         const int spw = steps_per_wave(steps_g * s.n_used);
         const dim3 grid_g((unsigned)((steps_g + 4 * spw - 1) / (4 * spw)), (unsigned)s.n_used);
-#define INFR_GATE_UP(P)                                                                                    \
-    hipLaunchKernelGGL((moe_gate_up_f32_kernel<P>), grid_g, dim3(256), 0, stream, b.gate, b.up, b.gate_stride, \
-                       b.up_stride, sel_idx, b.x, gbuf, s.ne, s.n_ff, spw)
-        if (s.gate_dtype == 12) INFR_GATE_UP(RawQ4K);
-        else if (s.gate_dtype == 13) INFR_GATE_UP(RawQ5K);
-        else if (s.gate_dtype == 14) INFR_GATE_UP(RawQ6K);
-        else INFR_GATE_UP(RawQ8_0);
+#define INFR_GATE_UP_N(P, N)                                                                                  \
+    hipLaunchKernelGGL((moe_gate_up_f32_kernel<P, N>), grid_g, dim3(256), 0, stream, b.gate, b.up, b.gate_stride, \
+                       b.up_stride, sel_idx, b.x, gbuf, s.ne, s.n_ff)
+#define INFR_GATE_UP(P)                 \
+    switch (spw) {                      \
+    case 1: INFR_GATE_UP_N(P, 1); break; \
+    case 2: INFR_GATE_UP_N(P, 2); break; \
+    case 3: INFR_GATE_UP_N(P, 3); break; \
+    default: INFR_GATE_UP_N(P, 4); break; \
+    }
+        if (s.gate_dtype == 12) INFR_GATE_UP(RawQ4K)
+        else if (s.gate_dtype == 13) INFR_GATE_UP(RawQ5K)
+        else if (s.gate_dtype == 14) INFR_GATE_UP(RawQ6K)
+        else INFR_GATE_UP(RawQ8_0)
 #undef INFR_GATE_UP
+#undef INFR_GATE_UP_N
         const int rps_d = 64 / (s.n_ff / 64);
         const int steps_d = (s.ne + rps_d - 1) / rps_d;
         const int spw_d = std::min(kDownMaxSteps, steps_per_wave(steps_d * s.n_used));
         const int nw_d = std::min(s.n_used, kDownMaxWaves);
         const dim3 grid_d((unsigned)((steps_d + spw_d - 1) / spw_d));
-#define INFR_DOWN(P)                                                                                     \
-    hipLaunchKernelGGL((moe_down_f32_kernel<P>), grid_d, dim3((unsigned)(64 * nw_d)), 0, stream, b.down,   \
-                       b.down_stride, sel_idx, sel_w, gbuf, b.dst, s.n_ff, s.ne, s.n_used, spw_d)
-        if (s.down_dtype == 12) INFR_DOWN(RawQ4K);
-        else if (s.down_dtype == 13) INFR_DOWN(RawQ5K);
-        else if (s.down_dtype == 14) INFR_DOWN(RawQ6K);
-        else INFR_DOWN(RawQ8_0);
+#define INFR_DOWN_N(P, N)                                                                                   \
+    hipLaunchKernelGGL((moe_down_f32_kernel<P, N>), grid_d, dim3((unsigned)(64 * nw_d)), 0, stream, b.down,   \
+                       b.down_stride, sel_idx, sel_w, gbuf, b.dst, s.n_ff, s.ne, s.n_used)
+#define INFR_DOWN(P)                 \
+    switch (spw_d) {                 \
+    case 1: INFR_DOWN_N(P, 1); break; \
+    case 2: INFR_DOWN_N(P, 2); break; \
+    case 3: INFR_DOWN_N(P, 3); break; \
+    default: INFR_DOWN_N(P, 4); break; \
+    }
+        if (s.down_dtype == 12) INFR_DOWN(RawQ4K)
+        else if (s.down_dtype == 13) INFR_DOWN(RawQ5K)
+        else if (s.down_dtype == 14) INFR_DOWN(RawQ6K)
+        else INFR_DOWN(RawQ8_0)
 #undef INFR_DOWN
+#undef INFR_DOWN_N
         return hipGetLastError() == hipSuccess ? nullptr : "kernel launch failed";
     }
 
