@@ -45,6 +45,10 @@ struct infr_hip_plan {
         size_t qtile_first = 0, qtile_n = 0;  // small batch: slice of qtiles
     };
     std::vector<Step> steps;
+    // per op: the Op::Add a MoeFfn's last kernel also produces (-1: none), and whether that
+    // Add's residual is its first operand
+    std::vector<int> moe_add;
+    std::vector<char> moe_add_resid_is_a;
     std::vector<infr::GemvOpDesc> descs;
     // per-workgroup tile tables of the grouped launches, back to back (tile_first per step)
     std::vector<infr::GemvTile> tiles;
@@ -1026,24 +1030,40 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
         publishes[users.front()] = 1;
         wr[users.front()].push_back(wr[k][0]);
     }
+    // Op::Add after its producer (fusion.rs:155-260): one operand is the output of an earlier decode
+    // Linear or MoeFfn of the same length, the other is the residual; the producer's last kernel
+    // then also writes the sum (f32 addition commutes, so either operand order gives the CPU's bits).
+    std::vector<const float*> resid(n, nullptr);
+    plan->moe_add.assign(n, -1);
+    plan->moe_add_resid_is_a.assign(n, 0);
     for (size_t k = 0; env_fuse && k < n; ++k) {
         const auto& a = plan->ops[k];
-        if (a.kind != INFR_OP_ADD) continue;
-        // a = the output of an earlier decode Linear of the same length; nothing in between may
-        // touch dst or write b (the sum is produced at the Linear's place in the order)
+        if (a.kind != INFR_OP_ADD || ea[k].x == ea[k].aux) continue;
+        const size_t n_add = (size_t)a.m * a.in_f;
+        // nothing between the producer and the Add may touch the Add's dst or write the residual
+        // or the producer's dst (the sum is produced at the producer's place in the order)
         for (size_t i = 0; i < k; ++i) {
-            if (!decode_linear(i) || post[i] >= 0 || plan->ops[i].out_f != a.in_f ||
-                static_cast<const float*>(bindings[plan->ops[i].dst]->ptr) != ea[k].x)
-                continue;
+            const auto& pr = plan->ops[i];
+            const bool lin = decode_linear(i) && pr.out_f == n_add;
+            const bool moe = pr.kind == INFR_OP_MOE_FFN && (size_t)pr.moe.rows * pr.moe.ne == n_add;
+            if ((!lin && !moe) || post[i] >= 0) continue;
+            const float* pdst = static_cast<const float*>(bindings[pr.dst]->ptr);
+            if (pdst != ea[k].x && pdst != ea[k].aux) continue;
+            const bool resid_is_a = pdst == ea[k].aux;
             bool ok = true;
-            const std::vector<Span> b_span{fspan(ea[k].aux, ea[k].aux_elems)};
+            const std::vector<Span> b_span{fspan(resid_is_a ? ea[k].x : ea[k].aux, n_add)};
             for (size_t j = i + 1; ok && j < k; ++j)
                 ok = !any_overlap(wr[j], wr[k]) && !any_overlap(rd[j], wr[k]) && !any_overlap(wr[j], b_span) &&
                      !any_overlap(wr[j], wr[i]);
-            // the Linear's own inputs must not alias the Add's destination
+            // the producer's own inputs must not alias the Add's destination
             ok = ok && !any_overlap(rd[i], wr[k]);
             if (!ok) continue;
             post[i] = (int)k;
+            resid[i] = resid_is_a ? ea[k].x : ea[k].aux;
+            if (moe) {
+                plan->moe_add[i] = (int)k;
+                plan->moe_add_resid_is_a[i] = resid_is_a;
+            }
             absorbed[k] = 1;
             rd[i].push_back(b_span[0]);
             wr[i].push_back(wr[k][0]);
@@ -1080,7 +1100,7 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
             f.pre_dst = publishes[k] ? e.dst : nullptr;
         }
         if (post[k] >= 0) {
-            f.add_b = ea[post[k]].aux;
+            f.add_b = resid[k];
             f.add_dst = ea[post[k]].dst;
         }
         return f;
@@ -1191,6 +1211,12 @@ static int enqueue_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t
                                    bindings[op.gate_exps], bindings[op.up_exps], bindings[op.down_exps],
                                    bindings[op.dst], nullptr, nullptr, &ms, &mb))
                 return rc;
+            if (plan->moe_add[st.op] >= 0) {
+                ElementwiseArgs add;
+                if (int rc = check_elementwise(be, plan->ops[plan->moe_add[st.op]], bindings, &add)) return rc;
+                mb.add_b = plan->moe_add_resid_is_a[st.op] ? add.x : add.aux;
+                mb.add_dst = add.dst;
+            }
             if (int rc = enqueue_moe(be, ms, mb)) return rc;
         } else if (st.op >= 0 && plan->ops[st.op].kind == INFR_OP_EMBED_GATHER) {
             const auto& op = plan->ops[st.op];

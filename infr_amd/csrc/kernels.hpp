@@ -234,6 +234,10 @@ struct MoeBuffers {
     float* dst;             // [rows, ne]
     int32_t* sel_idx;       // optional [rows, n_used]
     float* sel_w;           // optional [rows, n_used]
+    // absorbed Op::Add (fusion.rs:155-200): add_dst[i] = dst[i] + add_b[i] from the kernel that
+    // produces dst; add_dst may be add_b (each element is read and written by one thread)
+    const float* add_b = nullptr;
+    float* add_dst = nullptr;
 };
 // Q6_K prefill GEMM on the int8 matrix cores (any m; used from 33 tokens): activations in the tiled quantizer's layout
 // (launch_quantize_q8_tiled); st.a, when set, receives isum per (token, row, 256-block).

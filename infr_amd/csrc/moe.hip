@@ -617,16 +617,13 @@ __global__ __launch_bounds__(256) void moe_gate_up_f32_kernel(
 // STEPS row steps, all requested up front; the per-expert results meet in LDS and are added in rank
 // order with a separate multiply and add, as the CPU's `*o += w_e * yv`.
 constexpr int kDownMaxSteps = 4, kDownMaxWaves = 16;
-#ifndef MOE_WAVES_WANTED
-#define MOE_WAVES_WANTED 1024
-#endif
-constexpr int kMoeWavesWanted = MOE_WAVES_WANTED;
+constexpr int kMoeWavesWanted = 1024;
 
 template <typename P, int STEPS>
 __global__ __launch_bounds__(1024) void moe_down_f32_kernel(
     const uint8_t* __restrict__ down, size_t down_stride, const int32_t* __restrict__ ids,
-    const float* __restrict__ wts, const float* __restrict__ act, float* __restrict__ out, int nff,
-    int ne, int n_used) {
+    const float* __restrict__ wts, const float* __restrict__ act, float* __restrict__ out,
+    const float* add_b, float* add_dst, int nff, int ne, int n_used) {
     __shared__ float ys[kDownMaxSteps][kDownMaxWaves][16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     const int S = nff / 64, rps = 64 / S;
@@ -665,7 +662,10 @@ __global__ __launch_bounds__(1024) void moe_down_f32_kernel(
     }
     if (owner) {
         const int o = (st0 + own_s) * rps + own_seg;
-        if (o < ne) out[o] = acc;
+        if (o < ne) {
+            out[o] = acc;
+            if (add_dst) add_dst[o] = acc + add_b[o];
+        }
     }
 }
 
@@ -767,8 +767,9 @@ __global__ __launch_bounds__(256) void moe_act_quant_kernel(const float* __restr
 // out[r][o] = sum_k w[r][k] * yp[r*n_used + k][o], k in rank order (lib.rs:2967-2983)
 __global__ __launch_bounds__(256) void moe_accumulate_kernel(const float* __restrict__ yp,
                                                              const float* __restrict__ wts,
-                                                             float* __restrict__ out, int ne,
-                                                             int n_used, int rows) {
+                                                             float* __restrict__ out,
+                                                             const float* add_b, float* add_dst,
+                                                             int ne, int n_used, int rows) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= (size_t)rows * ne) return;
     const size_t r = i / ne, o = i % ne;
@@ -776,6 +777,7 @@ __global__ __launch_bounds__(256) void moe_accumulate_kernel(const float* __rest
     for (int k = 0; k < n_used; ++k)
         acc += wts[r * n_used + k] * yp[(r * n_used + k) * ne + o];
     out[i] = acc;
+    if (add_dst) add_dst[i] = acc + add_b[i];
 }
 
 // Buckets the routed pairs by expert for the prefill path: perm = pair ids grouped by expert,
@@ -1008,7 +1010,7 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
         const dim3 grid_d((unsigned)((steps_d + spw_d - 1) / spw_d));
 #define INFR_DOWN_N(P, N)                                                                                   \
     hipLaunchKernelGGL((moe_down_f32_kernel<P, N>), grid_d, dim3((unsigned)(64 * nw_d)), 0, stream, b.down,   \
-                       b.down_stride, sel_idx, sel_w, gbuf, b.dst, s.n_ff, s.ne, s.n_used)
+                       b.down_stride, sel_idx, sel_w, gbuf, b.dst, b.add_b, b.add_dst, s.n_ff, s.ne, s.n_used)
 #define INFR_DOWN(P)                 \
     switch (spw_d) {                 \
     case 1: INFR_DOWN_N(P, 1); break; \
@@ -1086,7 +1088,7 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     else if (!launch_gemv_id(s.down_dtype, b.down, b.down_stride, dbpr, sel_idx, aq, s.n_ff, 1, (int)pairs, yp, s.ne, stream))
         return "no id-gathered kernel for this down shape";
     hipLaunchKernelGGL(moe_accumulate_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, stream,
-                       yp, sel_w, b.dst, s.ne, s.n_used, s.rows);
+                       yp, sel_w, b.dst, b.add_b, b.add_dst, s.ne, s.n_used, s.rows);
     return hipGetLastError() == hipSuccess ? nullptr : "kernel launch failed";
 }
 

@@ -447,3 +447,42 @@ def test_capabilities_advertise_the_ops_that_are_built(be):
     caps = be.capabilities()
     assert caps["combined_gu"] == 1 and caps["embed_gather"] == 1 and caps["decode_replay"] == 1
     assert caps["gpu_sample"] == 0 and caps["argmax_rows"] == 0 and caps["gated_rmsnorm"] == 0
+
+
+@pytest.mark.parametrize("rows", [1, 3])
+@pytest.mark.parametrize("resid_first", [True, False])
+def test_moe_residual_add_rides_in_the_last_moe_kernel(be, rows, resid_first):
+    """MoeFfn -> Add(residual) (crates/infr-core/src/fusion.rs:155-200): the Add is produced by the
+    kernel that accumulates the experts, in place on the residual stream, with the un-added MoE
+    output still stored; the sum is the CPU's `a + b` bit for bit."""
+    from infr_amd import Add, MoeFfn
+    ne, n_expert, n_used, nff = 512, 16, 4, 256
+    router = synth_normal_f32(2, n_expert * ne, sigma=0.05)
+    gate = synth_weight(DType.Q4K, 3, n_expert * nff, ne, 0.05)
+    up = synth_weight(DType.Q4K, 4, n_expert * nff, ne, 0.05)
+    down = synth_weight(DType.Q6K, 5, n_expert * ne, nff, 0.05)
+    g, binds = Graph(), Bindings()
+    xn = g.input(TensorDesc((rows, ne), DType.F32))
+    h = g.input(TensorDesc((rows, ne), DType.F32))
+    y = g.output(TensorDesc((rows, ne), DType.F32))
+    xnb, hb, yb = (be.alloc(rows * ne * 4) for _ in range(3))
+    rid = g.weight(TensorDesc((n_expert, ne), DType.F32))
+    gid, uid = (g.weight(TensorDesc((n_expert, nff, ne), DType.Q4K)) for _ in range(2))
+    did = g.weight(TensorDesc((n_expert, ne, nff), DType.Q6K))
+    binds.bind(xn, xnb).bind(h, hb).bind(y, yb).bind(rid, be.upload_new(router))
+    binds.bind(gid, be.upload_new(gate)).bind(uid, be.upload_new(up)).bind(did, be.upload_new(down))
+    g.push(MoeFfn(xn, xn, rid, gid, uid, did, y, ne, n_expert, n_used, nff))
+    g.push(Add(h, y, h, rows * ne) if resid_first else Add(y, h, h, rows * ne))
+    plan = be.compile(g)
+    for seed in (10, 20, 30):                               # the second and third are replays
+        xn0, h0 = synth_normal_f32(seed, rows * ne), synth_normal_f32(seed + 1, rows * ne)
+        be.upload(xnb, xn0)
+        be.upload(hb, h0)
+        be.execute(plan, binds)
+        got_y = be.download(yb, np.empty(rows * ne, np.float32))
+        got_h = be.download(hb, np.empty(rows * ne, np.float32))
+        want, _, _ = orc.moe_ffn(xn0, router, gate, up, down, ne=ne, n_expert=n_expert, n_used=n_used,
+                                 n_ff_exp=nff, down_dtype=DType.Q6K)
+        assert _rel(got_y, want.ravel()) < 1e-4
+        assert np.array_equal(bits(got_h), bits(h0 + got_y))
+    assert plan.launches() == (3 if rows == 1 else 7)       # no launch of its own for the Add
