@@ -49,7 +49,8 @@ __device__ __forceinline__ void load_row_clamped(typename F::Row& r, const uint8
 }
 
 // Rows [row0, row_end) of one weight matrix against activation registers `acts`. `first` already
-// holds step 0 of row0 (the caller issues those loads as early as it can). The loads run one wave
+// holds step 0 of row0 - every step of it when FIRST_WHOLE - (the caller issues those loads as
+// early as it can). The loads run one wave
 // step (16 or 64 blocks) ahead of the arithmetic, across row boundaries, so a wave always has one
 // step's bytes in flight (two and three steps ahead measured 3-10 % slower on the small-block
 // formats, whose occupancy already covers the latency).
@@ -59,14 +60,24 @@ __device__ __forceinline__ void load_row_clamped(typename F::Row& r, const uint8
 // scratch) and, every 16 rows, lane i adds row i's terms in that order: the same rounding
 // sequence as the CPU at about two instructions per row instead of a 16-deep v_readlane chain
 // per step. Lanes past a row's last block contribute +0.0, which leaves the sum unchanged.
-template <typename F, int STEPS, bool STAGES>
+//
+// `add_first` is add_b[row0 + lane], requested by the caller ahead of its prologue (an absorbed
+// Op::Add); rows 64 and up of a wave read add_b when they are stored.
+template <typename F, int STEPS, bool STAGES, bool FIRST_WHOLE = false>
 __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t bpr,
-                                          const typename F::Row& first,
+                                          const typename F::Row (&first)[FIRST_WHOLE ? STEPS : 1],
                                           const typename F::Acts (&acts)[STEPS],
                                           const bool (&ok)[STEPS], float* __restrict__ y, int n_units,
                                           int row0, int row_end, int lane, const StagePtrs& st,
                                           float* osum, const float* add_b = nullptr,
-                                          float* add_dst = nullptr) {
+                                          float* add_dst = nullptr, float add_first = 0.0f) {
+    // The residual of row r for an absorbed Add, from the lanes' prefetched values while
+    // r - row0 < 64 (every lane of the wave must call this; `wanted` guards the late read).
+    auto residual = [&](int r, bool wanted) {
+        const float pf = __shfl(add_first, (r - row0) & 63, kWave);
+        if (r - row0 < 64) return pf;
+        return wanted ? gload<float>(add_b + r) : 0.0f;
+    };
     constexpr int LS = OrderedSum<STEPS>::kRowStride;
     int in_batch = 0, batch_row0 = row0;
     // A row's step-t term: parked for the ordered sum, or added to the lane's partial sum.
@@ -80,6 +91,7 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
     auto finish_row = [&](int row, float s) {
         if (F::kOrdered) {
             if (++in_batch == 16 || row + 1 == row_end) {
+                const float resid = add_dst ? residual(batch_row0 + lane, lane < in_batch) : 0.0f;
                 if (lane < in_batch) {
                     const v4f* tr = reinterpret_cast<const v4f*>(osum + lane * LS);
                     float acc = 0.0f;
@@ -93,16 +105,17 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
                     }
                     gstore<float>(y + batch_row0 + lane, acc);
                     // an absorbed Op::Add: dst = a + b with a = this output
-                    if (add_dst) gstore<float>(add_dst + batch_row0 + lane, acc + gload<float>(add_b + batch_row0 + lane));
+                    if (add_dst) gstore<float>(add_dst + batch_row0 + lane, acc + resid);
                 }
                 batch_row0 = row + 1;
                 in_batch = 0;
             }
         } else if (!F::kLaneSums) {
             s = wave_sum_f(s);
+            const float resid = add_dst ? residual(row, lane == 0) : 0.0f;
             if (lane == 0) {
                 gstore<float>(y + row, s);
-                if (add_dst) gstore<float>(add_dst + row, s + gload<float>(add_b + row));
+                if (add_dst) gstore<float>(add_dst + row, s + resid);
             }
         } else {
             // The lanes' sums of up to eight rows are parked in LDS and reduced together: lane L
@@ -116,9 +129,10 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
                 acc += __shfl_xor(acc, 8, kWave);
                 acc += __shfl_xor(acc, 16, kWave);
                 acc += __shfl_xor(acc, 32, kWave);
+                const float resid = add_dst ? residual(batch_row0 + lane, lane < in_batch) : 0.0f;
                 if (lane < in_batch) {
                     gstore<float>(y + batch_row0 + lane, acc);
-                    if (add_dst) gstore<float>(add_dst + batch_row0 + lane, acc + gload<float>(add_b + batch_row0 + lane));
+                    if (add_dst) gstore<float>(add_dst + batch_row0 + lane, acc + resid);
                 }
                 batch_row0 = row + 1;
                 in_batch = 0;
@@ -131,9 +145,12 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
         // this one is computed.
         if (row0 >= row_end) return;
         typename F::Row cur[STEPS];
-        cur[0] = first;
+        cur[0] = first[0];
 #pragma unroll
-        for (int t = 1; t < STEPS; ++t) F::load_row(cur[t], w + (size_t)row0 * bpr, t, lane, ok[t]);
+        for (int t = 1; t < STEPS; ++t) {
+            if constexpr (FIRST_WHOLE) cur[t] = first[t];
+            else F::load_row(cur[t], w + (size_t)row0 * bpr, t, lane, ok[t]);
+        }
         for (int row = row0; row < row_end; ++row) {
             const uint8_t* rowp = w + (size_t)row * bpr;
             const bool more = row + 1 < row_end;
@@ -170,8 +187,22 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
         }
         finish_row(row, s);
     };
-    typename F::Row cur = first;
-    for (int row = row0; row < row_end; ++row) {
+    typename F::Row cur = first[0];
+    int row = row0;
+    if constexpr (FIRST_WHOLE && STEPS > 1) {
+        if (row < row_end) {  // every step of the first row is here already
+            const uint8_t* rowp = w + (size_t)row * bpr;
+            if (F::kClampedLoads) load_row_clamped<F>(cur, row + 1 < row_end ? rowp + bpr : rowp, lane, ok[0]);
+            else F::load_row(cur, rowp + bpr, 0, lane, ok[0] && row + 1 < row_end);
+            float s = 0.0f;
+#pragma unroll
+            for (int t = 0; t < STEPS; ++t)
+                take_term(t, F::template term<STAGES>(first[t], acts[t], t, lane, ok[t], st, (size_t)row * n_units), s);
+            finish_row(row, s);
+            ++row;
+        }
+    }
+    for (; row < row_end; ++row) {
         typename F::Row nxt;
         do_row(row, cur, nxt);
         cur = nxt;

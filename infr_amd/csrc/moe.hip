@@ -42,6 +42,9 @@ struct SelectLds {
 // rank(e) = #{j : p[j] > p[e] or (p[j] == p[e] and j < e)} on the NORMALISED probabilities
 // (normalising can create ties that the raw exponentials do not have), and the selected
 // probabilities are summed in rank order.
+// COHERENT: the logits were written by other workgroups of the same launch (with device-scope
+// stores) and are read past this compute unit's and this die's caches.
+template <bool COHERENT = false>
 __device__ __forceinline__ void moe_select_block(const float* __restrict__ l, SelectLds& s,
                                                  int n_expert, int n_used, float scale, int tid,
                                                  int32_t* __restrict__ out_idx,
@@ -52,7 +55,9 @@ __device__ __forceinline__ void moe_select_block(const float* __restrict__ l, Se
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int e = tid + 256 * i;
-        lv[i] = e < n_expert ? l[e] : -INFINITY;
+        lv[i] = e >= n_expert ? -INFINITY
+                : COHERENT   ? __hip_atomic_load(l + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                             : l[e];
         mx = __builtin_fmaxf(mx, lv[i]);
     }
 #pragma unroll
@@ -238,16 +243,22 @@ __global__ __launch_bounds__(256) void moe_router_kernel(
     float sum = 0.0f;
 #pragma unroll
     for (int q = 0; q < 8; ++q) sum += __shfl(acc, (tid & ~7) + q, kWave);
-    if (active && j == 0) logits[(size_t)(t0 + t) * n_expert + e0 + e] = sum;
-    if (!tickets) return;
-    // ticket: the workgroup that sees every other one done selects
-    __threadfence();
+    if (!tickets) {
+        if (active && j == 0) logits[(size_t)(t0 + t) * n_expert + e0 + e] = sum;
+        return;
+    }
+    // ticket: the workgroup that sees every other one done selects. The logits go to memory with
+    // device-scope stores and come back with device-scope loads, and each thread waits for its
+    // store before the barrier in front of the ticket: a device-wide fence pair instead (write
+    // back and invalidate the whole L2 of the die) costs several microseconds per workgroup.
+    if (active && j == 0)
+        __hip_atomic_store(logits + (size_t)(t0 + t) * n_expert + e0 + e, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (tid == 0) s_last = atomicAdd(tickets, 1) == (int)gridDim.x - 1;
     __syncthreads();
     if (!s_last) return;
-    __threadfence();
-    moe_select_block(logits, sel, n_expert, n_used, scale, tid, sel_idx, sel_w);
+    moe_select_block<true>(logits, sel, n_expert, n_used, scale, tid, sel_idx, sel_w);
     if (tid == 0) *tickets = 0;
 }
 
@@ -693,11 +704,11 @@ __global__ __launch_bounds__(256) void gemv_id_kernel(const uint8_t* __restrict_
     a.bsums = act.bsums + (size_t)r * (in_f / 32);
     a.bsums16 = act.bsums16 + (size_t)r * (in_f / 16);
     typename F::Acts acts[STEPS];
-    typename F::Row first;
+    typename F::Row first[1];
     bool ok[STEPS];
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) ok[t] = F::valid(t, lane, n_units);
-    F::load_row(first, w + (size_t)row0 * bpr, 0, lane, ok[0]);
+    F::load_row(first[0], w + (size_t)row0 * bpr, 0, lane, ok[0]);
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) F::load_acts(acts[t], a, t, lane, ok[t]);
     // same body as the decode GEMV: per-block exact integers, CPU-ordered f32 sum

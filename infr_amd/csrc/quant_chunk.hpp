@@ -6,39 +6,64 @@
 // global memory or in LDS.
 #pragma once
 
+#include <type_traits>
+
 #include "device_common.hpp"
 
 namespace infr {
+
+// Maximum over the lanes of a block without touching LDS: DPP exchanges inside the row of 16 lanes
+// (quad swaps, then the mirrors: after the quad steps the four lanes of a quad agree, so mirroring
+// the 8 and the 16 brings in exactly the other half), and for 64 lanes the four row maxima are read
+// out as scalars. A maximum does not depend on the order, so any pairing gives the CPU's amax.
+template <int LANES>
+__device__ __forceinline__ float lanes_max(float v) {
+    static_assert(LANES == 8 || LANES == 64, "a 32-element or a 256-element block");
+    auto step = [](float x, auto ctrl) {
+        const int o = __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), decltype(ctrl)::value, 0xF, 0xF, true);
+        return __builtin_fmaxf(x, __builtin_bit_cast(float, o));
+    };
+    v = step(v, std::integral_constant<int, 0xB1>{});   // quad_perm [1,0,3,2]
+    v = step(v, std::integral_constant<int, 0x4E>{});   // quad_perm [2,3,0,1]
+    v = step(v, std::integral_constant<int, 0x141>{});  // row_half_mirror
+    if constexpr (LANES == 64) {
+        v = step(v, std::integral_constant<int, 0x140>{});  // row_mirror
+        v = __builtin_fmaxf(__builtin_fmaxf(readlane_f(v, 0), readlane_f(v, 16)),
+                            __builtin_fmaxf(readlane_f(v, 32), readlane_f(v, 48)));
+    }
+    return v;
+}
 
 // The arithmetic alone: this lane's four codes (packed little-endian), the block scale, and the
 // code sums over the lane's 16- and 32-element groups (valid in every lane of the group).
 template <bool PER32>
 __device__ __forceinline__ void quantize_chunk_values(v4f v, uint32_t& packed, float& dd, int& s32,
                                                       int& s16) {
-    float amax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v.x), __builtin_fabsf(v.y)),
-                                 __builtin_fmaxf(__builtin_fabsf(v.z), __builtin_fabsf(v.w)));
-    // Maximum over the block's lanes: 8 lanes (32 floats) or all 64 (256 floats).
-#pragma unroll
-    for (int off = 1; off < (PER32 ? 8 : 64); off <<= 1)
-        amax = __builtin_fmaxf(amax, __shfl_xor(amax, off, kWave));
-
+    const float amax = lanes_max<PER32 ? 8 : 64>(
+        __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v.x), __builtin_fabsf(v.y)),
+                        __builtin_fmaxf(__builtin_fabsf(v.z), __builtin_fabsf(v.w))));
     dd = amax / 127.0f;
     const float id = dd > 0.0f ? 1.0f / dd : 0.0f;
 
+    // `(f * id).round().clamp(-127, 127) as i8`. round() is half away from zero: for |x| < 2^23 that
+    // is trunc(x + copysign(0.5 - 2^-25, x)) - adding 0.5 itself would carry 0.49999997 up to 1 -
+    // and the conversion to integer truncates by itself. |f * id| <= 127 (1 + 2^-22) < 127.5, so the
+    // clamp never changes a finite value; NaN converts to 0 here as it does in the CPU's `as i8`.
     auto q1 = [id](float f) -> int {
-        float r = roundf(f * id);
-        r = r < -127.0f ? -127.0f : r;
-        r = r > 127.0f ? 127.0f : r;
-        return (int)r;
+        const float x = f * id;
+        const float half = __builtin_bit_cast(
+            float, (__builtin_bit_cast(uint32_t, x) & 0x80000000u) | 0x3EFFFFFFu);  // copysign(0.49999997, x)
+        return (int)(x + half);
     };
     const int q0 = q1(v.x), q1_ = q1(v.y), q2 = q1(v.z), q3 = q1(v.w);
-    packed = (uint32_t)(q0 & 0xFF) | ((uint32_t)(q1_ & 0xFF) << 8) | ((uint32_t)(q2 & 0xFF) << 16) |
-             ((uint32_t)(q3 & 0xFF) << 24);
-    int s = q0 + q1_ + q2 + q3;  // 4 elements
-    s += __shfl_xor(s, 1, kWave);
-    s += __shfl_xor(s, 2, kWave);  // 16 elements: lanes 4g..4g+3
+    // low bytes of the four codes: two byte permutes and a shift-or
+    const uint32_t lo = __builtin_amdgcn_perm((uint32_t)q1_, (uint32_t)q0, 0x0C0C0400u);
+    const uint32_t hi = __builtin_amdgcn_perm((uint32_t)q3, (uint32_t)q2, 0x0C0C0400u);
+    packed = lo | (hi << 16);
+    int s = dot4((int)packed, 0x01010101, 0);  // the lane's 4 codes
+    s = quad_sum(s);                           // 16 elements: lanes 4g..4g+3
     s16 = s;
-    s += __shfl_xor(s, 4, kWave);  // 32 elements: lanes 8g..8g+7
+    s += __builtin_amdgcn_mov_dpp(s, 0x141, 0xF, 0xF, true);  // row_half_mirror: the 8's other quad
     s32 = s;
 }
 

@@ -59,6 +59,31 @@ def test_quantize_q8_32_bit_exact(be, m, k):
         assert np.array_equal(bs[r], o.bsum)
 
 
+def test_quantizers_round_every_code_boundary_like_the_cpu(be):
+    """round() is half away from zero (crates/infr-cpu/src/quant.rs:27-58, 97-117). With amax = 127 the
+    scale is exactly 1, so the codes are round(x) itself: every boundary k + 0.5 for k = 0 .. 126, the
+    floats just below and just above it, and their negatives, in both quantizers. (The device rounds
+    by adding copysign(0.5 - 2^-25, x) and truncating, which must agree at all of them.)"""
+    ks = np.arange(0, 127, dtype=np.float32) + np.float32(0.5)
+    vals = np.concatenate([ks, np.nextafter(ks, np.float32(0)), np.nextafter(ks, np.float32(200)),
+                           np.float32([0.0, 1e-30, 0.25, 126.99999, 127.0])]).astype(np.float32)
+    vals = np.concatenate([vals, -vals])
+    n = -(-vals.size // 256) * 256
+    x = np.zeros(n, np.float32)
+    x[:vals.size] = vals
+    x[255::256] = 127.0                       # every 256-block (and below: every 32-block) has amax = 127
+    qs, d, bs, bs16 = be.quantize_q8(be.upload_new(x), 1, n)
+    o = orc.quantize_q8(x)
+    assert np.all(o.d == 1.0)
+    assert np.array_equal(qs[0], o.qs) and np.array_equal(bs[0], o.bsums) and np.array_equal(bs16[0], o.bsums16)
+    x32 = x.copy()
+    x32[31::32] = 127.0
+    qs, d, bs = be.quantize_q8_32(be.upload_new(x32), 1, n)
+    o = orc.quantize_q8_32(x32)
+    assert np.all(o.d == 1.0)
+    assert np.array_equal(qs[0], o.qs) and np.array_equal(bs[0], o.bsum)
+
+
 DECODE_SHAPES = [(256, 8), (768, 37), (4096, 1024), (12288, 512), (2048, 100), (5120, 64)]
 
 
