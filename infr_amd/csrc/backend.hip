@@ -140,7 +140,13 @@ bool is_quant(int dt) {
 }
 // Formats Op::MoeFfn's expert banks may hold.
 bool is_moe_quant(int dt) {
-    return dt == INFR_DTYPE_Q4_K || dt == INFR_DTYPE_Q5_K || dt == INFR_DTYPE_Q6_K || dt == INFR_DTYPE_Q8_0;
+    switch (dt) {
+    case INFR_DTYPE_Q4_K: case INFR_DTYPE_Q5_K: case INFR_DTYPE_Q6_K: case INFR_DTYPE_Q8_0:
+    case INFR_DTYPE_Q4_0: case INFR_DTYPE_Q4_1: case INFR_DTYPE_Q5_0: case INFR_DTYPE_Q5_1:
+    case INFR_DTYPE_IQ4_NL: case INFR_DTYPE_Q2_0:
+        return true;
+    default: return false;
+    }
 }
 bool act_per32(int dt, size_t in_f) { return infr::act_is_per32(dt, in_f); }
 // Row lengths a format accepts: whole weight blocks.

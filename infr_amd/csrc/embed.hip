@@ -5,96 +5,12 @@
 // codebook formats d * value), so every output equals `bytes_to_f32(row)[e] * scale` bit for bit.
 // A token id outside the table yields a row of NaN (the CPU backend panics on the slice); nothing
 // is read out of bounds. HBM-bound on rows * (row bytes + 4 * ne), a few MB per prefill.
-#include "device_common.hpp"
+#include "decode_element.hpp"
 #include "kernels.hpp"
 
 namespace infr {
 
 namespace {
-
-__device__ __forceinline__ uint32_t ld8(const uint8_t* p) { return gload<uint8_t>(p); }
-__device__ __forceinline__ float ldf16(const uint8_t* p) { return f16_bits_to_f32(gload<uint16_t>(p)); }
-
-// get_scale_min_k4 for one sub-block (crates/infr-gguf/src/dequant.rs:73-83)
-__device__ __forceinline__ void k4_one(int j, const uint8_t* q, int* sc, int* m) {
-    if (j < 4) {
-        *sc = (int)(ld8(q + j) & 63);
-        *m = (int)(ld8(q + j + 4) & 63);
-    } else {
-        *sc = (int)((ld8(q + j + 4) & 0xF) | ((ld8(q + j - 4) >> 6) << 4));
-        *m = (int)((ld8(q + j + 4) >> 4) | ((ld8(q + j) >> 6) << 4));
-    }
-}
-
-// Element e of a row stored in `dtype` (ggml type id); rowp is the row's first byte.
-__device__ float decode_element(int dtype, const uint8_t* rowp, int e) {
-    switch (dtype) {
-    case 0: return gload<float>(rowp + (size_t)e * 4);
-    case 1: return ldf16(rowp + (size_t)e * 2);
-    case 30: return __builtin_bit_cast(float, (uint32_t)gload<uint16_t>(rowp + (size_t)e * 2) << 16);
-    case 8: {  // Q8_0: (d*1) * (q+128) + d*(-128)
-        const uint8_t* blk = rowp + (size_t)(e >> 5) * 34;
-        const float d = ldf16(blk);
-        const int q = (int)(int8_t)ld8(blk + 2 + (e & 31));
-        return (d * 1.0f) * (float)(q + 128) + d * -128.0f;
-    }
-    case 2: case 3: case 6: case 7: {  // Q4_0, Q4_1, Q5_0, Q5_1
-        const bool affine = dtype == 3 || dtype == 7, five = dtype == 6 || dtype == 7;
-        const int bytes = 18 + (affine ? 2 : 0) + (five ? 4 : 0);
-        const uint8_t* blk = rowp + (size_t)(e >> 5) * bytes;
-        const int i = e & 31, j = i & 15;
-        const float d = ldf16(blk);
-        const uint8_t* p = blk + (affine ? 4 : 2);
-        uint32_t code_hi = 0;
-        if (five) {
-            const uint32_t qh = ld8(p) | (ld8(p + 1) << 8) | (ld8(p + 2) << 16) | (ld8(p + 3) << 24);
-            code_hi = ((qh >> i) & 1u) << 4;
-            p += 4;
-        }
-        const uint32_t b = ld8(p + j);
-        const uint32_t code = (i < 16 ? (b & 0xF) : (b >> 4)) | code_hi;
-        const float mn = affine ? ldf16(blk + 2) * 1.0f : d * (five ? -16.0f : -8.0f);
-        return (d * 1.0f) * (float)code + mn;
-    }
-    case 12: case 13: {  // Q4_K, Q5_K
-        const int bytes = dtype == 12 ? 144 : 176;
-        const uint8_t* blk = rowp + (size_t)(e >> 8) * bytes;
-        const int i = e & 255, s = i >> 5, l = i & 31;
-        int sc, m;
-        k4_one(s, blk + 4, &sc, &m);
-        const uint8_t* qs = blk + (dtype == 12 ? 16 : 48);
-        const uint32_t b = ld8(qs + (s >> 1) * 32 + l);
-        uint32_t code = (s & 1) ? (b >> 4) : (b & 0xF);
-        if (dtype == 13) code += ((ld8(blk + 16 + l) >> s) & 1u) ? 16u : 0u;
-        const float fs = ldf16(blk) * (float)sc, fm = ldf16(blk + 2) * (float)(-m);
-        return fs * (float)code + fm;
-    }
-    case 14: {  // Q6_K
-        const uint8_t* blk = rowp + (size_t)(e >> 8) * 210;
-        const int i = e & 255, half = i >> 7, r = i & 127, col = r >> 5, l = r & 31;
-        const uint32_t lb = ld8(blk + half * 64 + (col & 1) * 32 + l);
-        const uint32_t lo = col >= 2 ? (lb >> 4) : (lb & 0xF);
-        const uint32_t hi = (ld8(blk + 128 + half * 32 + l) >> (2 * col)) & 3u;
-        const int s = (int)(int8_t)ld8(blk + 192 + half * 8 + 2 * col + (l >> 4));
-        const float d = ldf16(blk + 208);
-        return (d * (float)s) * (float)(lo | (hi << 4)) + d * (float)(-32 * s);
-    }
-    case 20: {  // IQ4_NL
-        const int kv[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
-        const uint8_t* blk = rowp + (size_t)(e >> 5) * 18;
-        const int i = e & 31;
-        const uint32_t b = ld8(blk + 2 + (i & 15));
-        return ldf16(blk) * (float)kv[i < 16 ? (b & 0xF) : (b >> 4)];
-    }
-    case 42: {  // Q2_0
-        const uint8_t* blk = rowp + (size_t)(e >> 6) * 18;
-        const int j = e & 63;
-        const int q = (int)((ld8(blk + 2 + (j >> 2)) >> ((j & 3) * 2)) & 3u);
-        return (float)(q - 1) * ldf16(blk);
-    }
-    default: return 0.0f;
-    }
-}
 
 __global__ __launch_bounds__(256) void embed_gather_kernel(int dtype, const uint8_t* __restrict__ table,
                                                            size_t bpr, int total_rows,

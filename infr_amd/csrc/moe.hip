@@ -21,6 +21,7 @@
 #include "gemv_formats.hpp"
 #include "gemv_rows.hpp"
 #include "kernels.hpp"
+#include "decode_element.hpp"
 #include "quant_chunk.hpp"
 
 namespace infr {
@@ -700,9 +701,9 @@ __global__ __launch_bounds__(256) void gemv_id_kernel(const uint8_t* __restrict_
     const int n_units = F::units(in_f);
     ActPtrs a;
     a.qs = act.qs + (size_t)r * in_f;
-    a.d = act.d + (size_t)r * (in_f / 256);
+    a.d = act.d + (size_t)r * (in_f / (F::kPer32 ? 32 : 256));
     a.bsums = act.bsums + (size_t)r * (in_f / 32);
-    a.bsums16 = act.bsums16 + (size_t)r * (in_f / 16);
+    a.bsums16 = F::kPer32 ? nullptr : act.bsums16 + (size_t)r * (in_f / 16);
     typename F::Acts acts[STEPS];
     typename F::Row first[1];
     bool ok[STEPS];
@@ -755,6 +756,7 @@ __global__ __launch_bounds__(256) void gemv_id_folded_kernel(const uint8_t* __re
 
 // act = silu(g) * u per pair row, quantized per 256 for the down bank (lib.rs:2824-2892).
 // One wavefront per 256-float chunk.
+template <bool PER32>
 __global__ __launch_bounds__(256) void moe_act_quant_kernel(const float* __restrict__ g,
                                                             const float* __restrict__ u,
                                                             int8_t* __restrict__ qs,
@@ -772,7 +774,46 @@ __global__ __launch_bounds__(256) void moe_act_quant_kernel(const float* __restr
     a.y = gv.y / (1.0f + expf(-gv.y)) * uv.y;
     a.z = gv.z / (1.0f + expf(-gv.z)) * uv.z;
     a.w = gv.w / (1.0f + expf(-gv.w)) * uv.w;
-    quantize_chunk<false>(a, true, lane, chunk, qs, d, bsums, bsums16);
+    quantize_chunk<PER32>(a, true, lane, chunk, qs, d, bsums, PER32 ? nullptr : bsums16);
+}
+
+// The same activation kept in f32 (in place over g) for a down bank that multiplies raw rows.
+__global__ __launch_bounds__(256) void moe_act_f32_kernel(float* __restrict__ g, const float* __restrict__ u,
+                                                          size_t n_elems) {
+    const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= n_elems) return;
+    const v4f gv = *reinterpret_cast<const v4f*>(g + i), uv = *reinterpret_cast<const v4f*>(u + i);
+    v4f a;
+    a.x = gv.x / (1.0f + expf(-gv.x)) * uv.x;
+    a.y = gv.y / (1.0f + expf(-gv.y)) * uv.y;
+    a.z = gv.z / (1.0f + expf(-gv.z)) * uv.z;
+    a.w = gv.w / (1.0f + expf(-gv.w)) * uv.w;
+    *reinterpret_cast<v4f*>(g + i) = a;
+}
+
+// `ActsKind::Raw` for any bank format (crates/infr-cpu/src/moe.rs:143-172): the weight row is decoded
+// to f32 as the host decode does and multiplied with `dot` (kernels.rs:6557-6573) - eight FMA chains
+// by element index mod 8, added in order - against the f32 activation row, so every output equals
+// the CPU's bit for bit. Eight lanes per output row, one chain each; pair = blockIdx.y,
+// activation row = pair / act_div. This is the arm of the formats infr-cpu has no int8 expert
+// kernel for, and of single rows of shapes the factored one-token kernels do not take: a fallback
+// there as here (one byte load and a dozen instructions per weight).
+__global__ __launch_bounds__(256) void moe_raw_dot_kernel(int dtype, const uint8_t* __restrict__ bank,
+                                                          size_t expert_stride, size_t bpr,
+                                                          const int32_t* __restrict__ ids,
+                                                          const float* __restrict__ acts, int act_div,
+                                                          int in_f, float* __restrict__ y, int out_f) {
+    const int pair = blockIdx.y, j = threadIdx.x & 7;
+    const int o = (int)blockIdx.x * 32 + ((int)threadIdx.x >> 3);
+    const bool live = o < out_f;
+    const uint8_t* rowp = bank + (size_t)ids[pair] * expert_stride + (size_t)(live ? o : 0) * bpr;
+    const float* x = acts + (size_t)(pair / act_div) * in_f;
+    float acc = 0.0f;
+    for (int i = j; i < in_f; i += 8) acc = __builtin_fmaf(decode_element(dtype, rowp, i), x[i], acc);
+    float sum = 0.0f;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) sum += __shfl(acc, ((int)threadIdx.x & ~7) + q, kWave);
+    if (live && j == 0) y[(size_t)pair * out_f + o] = sum;
 }
 
 // out[r][o] = sum_k w[r][k] * yp[r*n_used + k][o], k in rank order (lib.rs:2967-2983)
@@ -890,6 +931,7 @@ static bool launch_gemv_id(int dtype, const uint8_t* bank, size_t expert_stride,
     case 13: return launch_gemv_id_fmt<FmtQ5K>(bank, expert_stride, bpr, ids, act, in_f, n_used, pairs, y, out_f, stream, bank1, expert_stride1, y1);
     case 14: return launch_gemv_id_fmt<FmtQ6K>(bank, expert_stride, bpr, ids, act, in_f, n_used, pairs, y, out_f, stream, bank1, expert_stride1, y1);
     case 8: return launch_gemv_id_fmt<FmtQ8_0>(bank, expert_stride, bpr, ids, act, in_f, n_used, pairs, y, out_f, stream, bank1, expert_stride1, y1);
+    case 6: return launch_gemv_id_fmt<FmtNib32<Nib32::Q5_0>>(bank, expert_stride, bpr, ids, act, in_f, n_used, pairs, y, out_f, stream, bank1, expert_stride1, y1);
     default: return false;
     }
 }
@@ -910,6 +952,9 @@ size_t moe_workspace_bytes(const MoeShape& s) {
     add(qmax / 32 * 4);                           // d (sized for either quantizer)
     add(qmax / 32 * 4);                           // bsums
     add(qmax / 16 * 4);                           // bsums16
+    add(qmax);                                    // per-32 int8 activations (Q5_0 banks)
+    add(qmax / 32 * 4);                           // their d
+    add(qmax / 32 * 4);                           // their bsums
     const size_t max_tiles = pairs / 32 + std::min((size_t)s.n_expert, pairs);
     add(4);                                       // n_tiles
     add(pairs * 4);                               // perm
@@ -943,6 +988,11 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     aq.d = (float*)take(qmax / 32 * 4);
     aq.bsums = (int32_t*)take(qmax / 32 * 4);
     aq.bsums16 = (int32_t*)take(qmax / 16 * 4);
+    ActQ8 aq32;
+    aq32.qs = (int8_t*)take(qmax);
+    aq32.d = (float*)take(qmax / 32 * 4);
+    aq32.bsums = (int32_t*)take(qmax / 32 * 4);
+    aq32.bsums16 = nullptr;
     const size_t max_tiles = pairs / 32 + std::min((size_t)s.n_expert, pairs);
     int32_t* n_tiles = (int32_t*)take(4);
     int32_t* perm = (int32_t*)take(pairs * 4);
@@ -976,9 +1026,39 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
                            dim3((unsigned)((s.n_expert + epw - 1) / epw), (unsigned)((s.rows + tpw - 1) / tpw)),
                            dim3(256), router_lds, stream, b.router, b.router_x, logits, (int*)nullptr, sel_idx, sel_w,
                            s.ne, s.n_expert, s.rows, s.n_used, s.scale, kc, epw);
-    // the expert input is quantized by the selection kernel's workgroups (one per row) when its rows
-    // are whole 256s
-    const bool quant_in_select = s.rows > 1 && s.ne % 256 == 0;
+    auto bytes_per_row = [](int dtype, size_t in_f) -> size_t {
+        switch (dtype) {
+        case 12: return in_f / 256 * 144;
+        case 13: return in_f / 256 * 176;
+        case 14: return in_f / 256 * 210;
+        case 8: return in_f / 32 * 34;
+        case 2: case 20: return in_f / 32 * 18;
+        case 3: return in_f / 32 * 20;
+        case 6: return in_f / 32 * 22;
+        case 7: return in_f / 32 * 24;
+        case 42: return in_f / 64 * 18;
+        default: return 0;
+        }
+    };
+    const size_t gbpr = bytes_per_row(s.gate_dtype, s.ne), ubpr = bytes_per_row(s.up_dtype, s.ne);
+    const size_t dbpr = bytes_per_row(s.down_dtype, s.n_ff);
+    if (!gbpr || !ubpr || !dbpr) return "expert bank format has no kernel";
+    // expert_acts_kind (moe.rs:42-53) with whole-256 rows: per-256 int8 activations (Super) for the
+    // K-quants and Q8_0, per-32 (Blk32) for Q5_0, f32 rows (Raw) for everything else - and for
+    // every bank when there is a single row (int8_ok = rows >= 2, lib.rs:2359).
+    enum { kSuper = 0, kBlk32 = 1, kRaw = 2 };
+    auto acts_kind = [&](int dt) {
+        if (s.rows < 2) return (int)kRaw;
+        return dt == 12 || dt == 13 || dt == 14 || dt == 8 ? (int)kSuper : (dt == 6 ? (int)kBlk32 : (int)kRaw);
+    };
+    const int kg = acts_kind(s.gate_dtype), ku = acts_kind(s.up_dtype), kd = acts_kind(s.down_dtype);
+    auto launch_raw = [&](int dt, const uint8_t* bank, size_t stride, size_t bpr_, const float* acts, int act_div,
+                          size_t in_f, float* out, size_t out_f) {
+        hipLaunchKernelGGL(moe_raw_dot_kernel, dim3((unsigned)((out_f + 31) / 32), (unsigned)pairs), dim3(256), 0,
+                           stream, dt, bank, stride, bpr_, sel_idx, acts, act_div, (int)in_f, out, (int)out_f);
+    };
+    // the expert input is quantized per 256 by the selection kernel's workgroups (one per row)
+    const bool quant_in_select = s.rows > 1 && (kg == kSuper || ku == kSuper);
     if (s.rows > 1)
         hipLaunchKernelGGL(moe_select_kernel, dim3((unsigned)s.rows), dim3(256), 0, stream, logits, sel_idx,
                            sel_w, s.n_expert, s.n_used, s.scale, quant_in_select ? b.x : (const float*)nullptr,
@@ -989,9 +1069,20 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     if (s.rows == 1) {
         // ActsKind::Raw for every bank (lib.rs:2359: int8_ok = rows >= 2)
         auto raw_ok = [](int dt) { return dt == 12 || dt == 13 || dt == 14 || dt == 8; };
-        if (!raw_ok(s.gate_dtype) || s.up_dtype != s.gate_dtype || !raw_ok(s.down_dtype))
-            return "rows == 1 carries Q4_K / Q5_K / Q6_K / Q8_0 expert banks (gate and up of one format)";
-        if (s.ne > 4096 || s.n_ff > 4096) return "rows == 1 needs ne, n_ff_exp <= 4096";
+        if (!raw_ok(s.gate_dtype) || s.up_dtype != s.gate_dtype || !raw_ok(s.down_dtype) || s.ne > 4096 ||
+            s.n_ff > 4096) {
+            // other formats, mixed gate / up formats, rows too long for the factored kernels'
+            // registers: the decode-and-dot form of every stage
+            launch_raw(s.gate_dtype, b.gate, b.gate_stride, gbpr, b.x, s.n_used, s.ne, gbuf, s.n_ff);
+            launch_raw(s.up_dtype, b.up, b.up_stride, ubpr, b.x, s.n_used, s.ne, ubuf, s.n_ff);
+            const size_t n_act1 = pairs * s.n_ff;
+            hipLaunchKernelGGL(moe_act_f32_kernel, dim3((unsigned)((n_act1 / 4 + 255) / 256)), dim3(256), 0, stream,
+                               gbuf, ubuf, n_act1);
+            launch_raw(s.down_dtype, b.down, b.down_stride, dbpr, gbuf, 1, s.n_ff, yp, s.ne);
+            hipLaunchKernelGGL(moe_accumulate_kernel, dim3((unsigned)((s.ne + 255) / 256)), dim3(256), 0, stream, yp,
+                               sel_w, b.dst, b.add_b, b.add_dst, s.ne, s.n_used, s.rows);
+            return hipGetLastError() == hipSuccess ? nullptr : "kernel launch failed";
+        }
         // row steps per wave: amortise the 64 activation registers while keeping >= ~1024 waves
         auto steps_per_wave = [](int wave_steps) { return std::max(1, std::min(4, wave_steps / kMoeWavesWanted)); };
         const int rps_g = 64 / (s.ne / 64);
@@ -1038,20 +1129,9 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
         return hipGetLastError() == hipSuccess ? nullptr : "kernel launch failed";
     }
 
-    // rows >= 2: ActsKind::Super for Q4K/Q6K/Q8_0 banks with in_f % 256 == 0 (moe.rs:42-53)
-    auto bytes_per_row = [](int dtype, size_t in_f) -> size_t {
-        switch (dtype) {
-        case 12: return in_f / 256 * 144;
-        case 13: return in_f / 256 * 176;
-        case 14: return in_f / 256 * 210;
-        case 8: return in_f / 32 * 34;
-        default: return 0;
-        }
-    };
-    const size_t gbpr = bytes_per_row(s.gate_dtype, s.ne), ubpr = bytes_per_row(s.up_dtype, s.ne);
-    const size_t dbpr = bytes_per_row(s.down_dtype, s.n_ff);
-    if (!gbpr || !ubpr || !dbpr) return "rows >= 2 carries Q4_K / Q5_K / Q6_K / Q8_0 expert banks";
-    if (!quant_in_select) launch_quantize_q8(b.x, s.rows, s.ne, false, aq, stream);
+    // rows >= 2
+    if ((kg == kSuper || ku == kSuper) && !quant_in_select) launch_quantize_q8(b.x, s.rows, s.ne, false, aq, stream);
+    if (kg == kBlk32 || ku == kBlk32) launch_quantize_q8(b.x, s.rows, s.ne, true, aq32, stream);
     const size_t n_act = pairs * s.n_ff, n_out = (size_t)s.rows * s.ne;
     // Prefill-sized batches: the pairs are bucketed by expert and every bank runs its format's
     // int8-MFMA GEMM per (expert, 32 pairs) tile, so an expert's weights are read once per 32 of
@@ -1079,24 +1159,40 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     if (gate_mfma) launch_gathered(s.gate_dtype, b.gate, b.gate_stride, gbpr, s.n_used, tt, gbuf, s.ne, s.n_ff);
     if (up_mfma) launch_gathered(s.up_dtype, b.up, b.up_stride, ubpr, s.n_used, tt, ubuf, s.ne, s.n_ff);
     bool gate_up_ok = true;
-    if (!gate_mfma && !up_mfma && s.gate_dtype == s.up_dtype) {
-        gate_up_ok = launch_gemv_id(s.gate_dtype, b.gate, b.gate_stride, gbpr, sel_idx, aq, s.ne, s.n_used, (int)pairs,
-                                    gbuf, s.n_ff, stream, b.up, b.up_stride, ubuf);
+    if (!gate_mfma && !up_mfma && s.gate_dtype == s.up_dtype && kg != kRaw) {
+        gate_up_ok = launch_gemv_id(s.gate_dtype, b.gate, b.gate_stride, gbpr, sel_idx, kg == kBlk32 ? aq32 : aq, s.ne,
+                                    s.n_used, (int)pairs, gbuf, s.n_ff, stream, b.up, b.up_stride, ubuf);
     } else {
-        if (!gate_mfma)
-            gate_up_ok = launch_gemv_id(s.gate_dtype, b.gate, b.gate_stride, gbpr, sel_idx, aq, s.ne, s.n_used,
-                                        (int)pairs, gbuf, s.n_ff, stream);
-        if (!up_mfma)
-            gate_up_ok = gate_up_ok && launch_gemv_id(s.up_dtype, b.up, b.up_stride, ubpr, sel_idx, aq, s.ne, s.n_used,
-                                                      (int)pairs, ubuf, s.n_ff, stream);
+        if (kg == kRaw)
+            launch_raw(s.gate_dtype, b.gate, b.gate_stride, gbpr, b.x, s.n_used, s.ne, gbuf, s.n_ff);
+        else if (!gate_mfma)
+            gate_up_ok = launch_gemv_id(s.gate_dtype, b.gate, b.gate_stride, gbpr, sel_idx, kg == kBlk32 ? aq32 : aq,
+                                        s.ne, s.n_used, (int)pairs, gbuf, s.n_ff, stream);
+        if (ku == kRaw)
+            launch_raw(s.up_dtype, b.up, b.up_stride, ubpr, b.x, s.n_used, s.ne, ubuf, s.n_ff);
+        else if (!up_mfma)
+            gate_up_ok = gate_up_ok && launch_gemv_id(s.up_dtype, b.up, b.up_stride, ubpr, sel_idx,
+                                                      ku == kBlk32 ? aq32 : aq, s.ne, s.n_used, (int)pairs, ubuf,
+                                                      s.n_ff, stream);
     }
     if (!gate_up_ok) return "no id-gathered kernel for this gate/up shape";
-    hipLaunchKernelGGL(moe_act_quant_kernel, dim3((unsigned)((n_act / 256 + 3) / 4)), dim3(256), 0, stream,
-                       gbuf, ubuf, aq.qs, aq.d, aq.bsums, aq.bsums16, n_act);
+    // act = silu(g) * u in the form the down bank multiplies: per-256 codes, per-32 codes, or f32
+    if (kd == kSuper)
+        hipLaunchKernelGGL(moe_act_quant_kernel<false>, dim3((unsigned)((n_act / 256 + 3) / 4)), dim3(256), 0, stream,
+                           gbuf, ubuf, aq.qs, aq.d, aq.bsums, aq.bsums16, n_act);
+    else if (kd == kBlk32)
+        hipLaunchKernelGGL(moe_act_quant_kernel<true>, dim3((unsigned)((n_act / 256 + 3) / 4)), dim3(256), 0, stream,
+                           gbuf, ubuf, aq32.qs, aq32.d, aq32.bsums, (int32_t*)nullptr, n_act);
+    else
+        hipLaunchKernelGGL(moe_act_f32_kernel, dim3((unsigned)((n_act / 4 + 255) / 256)), dim3(256), 0, stream, gbuf,
+                           ubuf, n_act);
     // the down projection's activation row is the pair itself: n_used = 1
-    if (bucketed && has_mfma(s.down_dtype))
+    if (kd == kRaw)
+        launch_raw(s.down_dtype, b.down, b.down_stride, dbpr, gbuf, 1, s.n_ff, yp, s.ne);
+    else if (bucketed && has_mfma(s.down_dtype))
         launch_gathered(s.down_dtype, b.down, b.down_stride, dbpr, 1, tt, yp, s.n_ff, s.ne);
-    else if (!launch_gemv_id(s.down_dtype, b.down, b.down_stride, dbpr, sel_idx, aq, s.n_ff, 1, (int)pairs, yp, s.ne, stream))
+    else if (!launch_gemv_id(s.down_dtype, b.down, b.down_stride, dbpr, sel_idx, kd == kBlk32 ? aq32 : aq, s.n_ff, 1,
+                             (int)pairs, yp, s.ne, stream))
         return "no id-gathered kernel for this down shape";
     hipLaunchKernelGGL(moe_accumulate_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, stream,
                        yp, sel_w, b.dst, b.add_b, b.add_dst, s.ne, s.n_used, s.rows);

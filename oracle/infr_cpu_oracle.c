@@ -912,13 +912,15 @@ int orc_expert_acts_kind(int dtype, size_t in_f, int int8_ok) {
 
 /* One expert bank applied to `count` activation rows: out_t[o*count + i], o-major
  * (crates/infr-cpu/src/moe.rs:66-175). Super: per-256 int8 activations through the batch kernels
- * (bit-identical to the single-row kernels); Raw: weight row decoded once, f32 dot(). */
+ * (bit-identical to the single-row kernels); Blk32: per-32 int8 activations through
+ * vec_dot_q8_0_32_batch / vec_dot_q5_0_32_batch (moe.rs:115-141; the 8-row tile computes the same
+ * per-row values); Raw: weight row decoded once, f32 dot(). */
 static int expert_gemm(const uint8_t *wbytes, size_t wlen, int dt, size_t in_f, size_t out_f,
                        int kind, const float *xin, size_t count, float *out_t) {
     size_t bpr = wlen / out_f;
-    if (kind == ORC_ACTS_SUPER) {
+    if (kind == ORC_ACTS_SUPER || kind == ORC_ACTS_BLK32) {
         acts_t a;
-        acts_build(dt, xin, count, in_f, &a);
+        acts_build(dt, xin, count, in_f, &a); /* per 256 or per 32 by (dt, in_f), as the kind */
         for (size_t o = 0; o < out_f; o++)
             for (size_t i = 0; i < count; i++)
                 out_t[o * count + i] = row_dot(dt, wbytes + o * bpr, &a, i, in_f, NULL, NULL);
@@ -938,7 +940,7 @@ static int expert_gemm(const uint8_t *wbytes, size_t wlen, int dt, size_t in_f, 
         free(wf);
         return 0;
     }
-    return -1; /* Blk32 (Q8_0 with in_f % 256 != 0) is not restated */
+    return -1;
 }
 
 int orc_moe_ffn(const orc_moe_params *p, const float *x, const float *router_x,

@@ -250,3 +250,62 @@ def test_moe_prefill_buckets_with_mixed_bank_formats(be, gu, down):
     two = be.download(y2, np.empty((2, ne), np.float32))
     if DType.Q8_0 not in (gu, down):       # the ordered formats: bit-identical whichever kernel ran
         assert np.array_equal(two.view(np.uint32), got[0][:2].view(np.uint32)), "bucketed != per-pair"
+
+
+def run_moe_mixed(be, x, router, gate, up, down, rows, ne, n_expert, n_used, nff, dts):
+    xb, rb = be.upload_new(x), be.upload_new(router)
+    gb, ub, db = be.upload_new(gate), be.upload_new(up), be.upload_new(down)
+    yb = be.alloc(rows * ne * 4)
+    ib, wb = be.alloc(rows * n_used * 4), be.alloc(rows * n_used * 4)
+    be.moe_ffn(xb, rb, gb, ub, db, yb, rows=rows, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
+               gate_dtype=dts[0], up_dtype=dts[1], down_dtype=dts[2], sel_idx=ib, sel_w=wb)
+    return (be.download(yb, np.empty((rows, ne), np.float32)),
+            be.download(ib, np.empty((rows, n_used), np.int32)),
+            be.download(wb, np.empty((rows, n_used), np.float32)))
+
+
+@pytest.mark.parametrize("rows", [1, 5])
+@pytest.mark.parametrize("dtype", [DType.Q4_0, DType.Q4_1, DType.Q5_0, DType.Q5_1, DType.IQ4NL, DType.Q2_0])
+def test_moe_banks_in_the_32_block_formats(be, dtype, rows):
+    """expert_acts_kind (crates/infr-cpu/src/moe.rs:42-53): Q5_0 banks take per-32 int8 activations
+    from two rows up (Blk32), the other 32-block formats and every single-row call multiply decoded
+    f32 weights with the raw activation row (Raw)."""
+    ne, n_expert, n_used, nff = 512, 8, 2, 256
+    gate, up, down = banks(200 + int(dtype), ne, n_expert, nff, dtype, sigma=0.05)
+    x = synth_normal_f32(230 + rows, rows * ne)
+    router = synth_normal_f32(231, n_expert * ne, sigma=0.05)
+    got = run_moe(be, x, router, gate, up, down, rows, ne, n_expert, n_used, nff, 1.0, dtype)
+    want = orc.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
+                       gate_dtype=int(dtype), up_dtype=int(dtype), down_dtype=int(dtype))
+    check(*got, *want)
+
+
+@pytest.mark.parametrize("rows", [1, 4, 40])     # 40 rows of 8 experts: the bucketed Q4_K gate beside the rest
+def test_moe_banks_of_three_different_kinds(be, rows):
+    """gate Q4_K (per-256 activations), up Q5_0 (per-32), down Q4_0 (raw f32 rows) in one op: every
+    bank takes the activation form its own format asks for."""
+    ne, n_expert, n_used, nff = 512, 8, 2, 256
+    dts = (DType.Q4K, DType.Q5_0, DType.Q4_0)
+    gate = synth_weight(dts[0], 301, n_expert * nff, ne, 0.05)
+    up = synth_weight(dts[1], 302, n_expert * nff, ne, 0.05)
+    down = synth_weight(dts[2], 303, n_expert * ne, nff, 0.05)
+    x = synth_normal_f32(304 + rows, rows * ne)
+    router = synth_normal_f32(305, n_expert * ne, sigma=0.05)
+    got = run_moe_mixed(be, x, router, gate, up, down, rows, ne, n_expert, n_used, nff, dts)
+    want = orc.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
+                       gate_dtype=int(dts[0]), up_dtype=int(dts[1]), down_dtype=int(dts[2]))
+    check(*got, *want)
+
+
+@pytest.mark.parametrize("dtype", [DType.Q4K, DType.Q6K])
+def test_moe_single_row_of_a_hidden_size_above_4096(be, dtype):
+    """The factored one-token kernels keep a row's activations in registers (up to 4096 of them);
+    longer rows take the decode-and-dot form of the same Raw arithmetic."""
+    rows, ne, n_expert, n_used, nff = 1, 8192, 4, 2, 512
+    gate, up, down = banks(400, ne, n_expert, nff, dtype, sigma=0.03)
+    x = synth_normal_f32(401, rows * ne)
+    router = synth_normal_f32(402, n_expert * ne, sigma=0.02)
+    got = run_moe(be, x, router, gate, up, down, rows, ne, n_expert, n_used, nff, 1.0, dtype)
+    want = orc.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
+                       gate_dtype=int(dtype), up_dtype=int(dtype), down_dtype=int(dtype))
+    check(*got, *want)
