@@ -104,3 +104,26 @@ def test_expert_acts_kind_dispatch():
     assert orc.expert_acts_kind(orc.Q4_0, 2048, True) == orc.ACTS_RAW
     assert orc.expert_acts_kind(orc.Q2_0, 2048, True) == orc.ACTS_RAW
     assert orc.expert_acts_kind(orc.F32, 2048, True) == orc.ACTS_RAW
+
+
+@pytest.mark.parametrize("dtype,int8", [(orc.Q5_0, True), (orc.Q4_0, False), (orc.Q4_1, False), (orc.Q5_1, False),
+                                        (orc.IQ4_NL, False), (orc.Q2_0, False)])
+def test_32_block_bank_formats_against_textbook(dtype, int8):
+    """moe.rs:42-53 at rows >= 2: Q5_0 banks take per-32 int8 activations (the reference's ~4e-3
+    class of error, and a result that differs from the exact mode); the other 32-block formats
+    stay on decoded f32 weights x raw activations, i.e. the exact mode bit for bit."""
+    ne, n_expert, n_used, n_ff, rows = 256, 8, 2, 256, 3
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal(rows * ne).astype(np.float32)
+    router = (rng.standard_normal(n_expert * ne) * 0.1).astype(np.float32)
+    gate, up, down = make_banks(50, ne, n_expert, n_ff, dtype)
+    kw = dict(ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=n_ff, gate_dtype=dtype, up_dtype=dtype, down_dtype=dtype)
+    y, idx, _ = orc.moe_ffn(x, router, gate, up, down, **kw)
+    yref = orc.moe_ffn(x, router, gate, up, down, reference_mode=True, **kw)[0]
+    gf, uf, df = (orc.dequant_block(dtype, b) for b in (gate, up, down))
+    for r in range(rows):
+        want, want_idx = moe_ref(x[r * ne:(r + 1) * ne], router, gf, uf, df, ne, n_expert, n_used, n_ff, np.float32(1))
+        assert list(idx[r]) == want_idx
+        assert np.abs(yref[r] - want).max() < 1e-4
+        assert np.abs(y[r] - want).max() < (2e-2 * np.abs(want).max() if int8 else 1e-4)
+    assert np.array_equal(y, yref) != int8
