@@ -143,13 +143,12 @@ int infr_hip_linear(infr_hip_t *be, int dtype, const infr_hip_buffer_t *w, size_
  * that cannot allocate device memory around the call - code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc. Arguments, kernels and results are those of
  * infr_hip_linear; the quantized activation of m >= 2 goes into a static device array of the
- * library instead of the backend's grow-on-demand scratch, so ceil32(m) * in_f must not exceed
- * 4,194,304 elements (e.g. 1024 tokens of 4096), else INFR_HIP_ERR_UNSUPPORTED. Each GPU holds one
+ * library instead of the backend's grow-on-demand scratch, so ceil32(m) * ceil256(in_f) must not
+ * exceed 4,194,304 elements (e.g. 1024 tokens of 4096), else INFR_HIP_ERR_UNSUPPORTED. Each GPU holds one
  * such array (6 MiB) until the process ends and every backend on that GPU shares it: calls that
  * overlap on one GPU, from different backends or streams, race. The array keeps the last call's
- * contents and nothing needs clearing: the quantizer writes every slot of the m tokens, and what
- * the kernels compute from the stale slots of the padding tokens (m rounded up to 32) is never
- * stored. */
+ * contents and nothing needs clearing: the quantizer writes every slot the kernels read for the m
+ * tokens, and what they compute for the padding tokens (m rounded up to 32) is never stored. */
 int infr_hip_linear_noalloc(infr_hip_t *be, int dtype, const infr_hip_buffer_t *w, size_t w_numel,
                             size_t w_off, const infr_hip_buffer_t *x, infr_hip_buffer_t *dst, size_t m,
                             size_t in_f, size_t out_f);

@@ -85,7 +85,8 @@ struct infr_hip {
 };
 
 // ---- static device scratch of the allocation-free Op::Linear entry point ----
-// Quantized activation of up to kStaticActElems elements (tokens rounded up to 32, times in_f):
+// Quantized activation of up to kStaticActElems elements (tokens rounded up to 32, times in_f
+// rounded up to 256):
 // codes, then per-32 scales, per-32 sums and per-16 sums, the four arrays of infr::ActQ8 back to
 // back. Every device the library runs on holds its own copy of this array at its own address
 // until the process ends; the name below is only a host-side handle for hipGetSymbolAddress.
@@ -161,7 +162,9 @@ size_t stage_blocks(int dt, size_t in_f) {
 bool has_two_stages(int dt) { return dt == INFR_DTYPE_Q4_K || dt == INFR_DTYPE_Q5_K; }
 
 // Activation scratch for m rows: the prefill kernels read tokens in groups of 32.
-static size_t act_scratch_elems(size_t m, size_t in_f) { return (m + 31) / 32 * 32 * in_f; }
+// Tokens rounded up to the 32 of a tile, rows to the 256 of a step (the tiled per-32 quantizer pads
+// rows that end inside a step).
+static size_t act_scratch_elems(size_t m, size_t in_f) { return (m + 31) / 32 * 32 * ((in_f + 255) / 256 * 256); }
 
 static bool is_elementwise(int kind) { return kind >= INFR_OP_RMS_NORM && kind <= INFR_OP_ADD; }
 
@@ -647,7 +650,7 @@ int infr_hip_linear_noalloc(infr_hip_t* be, int dtype, const infr_hip_buffer_t* 
     if (act_scratch_elems(m, in_f) > kStaticActElems)
         return fail(be, INFR_HIP_ERR_UNSUPPORTED,
                     "linear_noalloc: " + std::to_string(act_scratch_elems(m, in_f)) +
-                        " activation elements (tokens rounded up to 32, times in_f) exceed the static scratch of " +
+                        " activation elements (tokens rounded up to 32, times in_f rounded up to 256) exceed the static scratch of " +
                         std::to_string(kStaticActElems));
     return enqueue_linear(be, dtype, la, static_cast<const float*>(x->ptr), static_cast<float*>(dst->ptr), m,
                           in_f, out_f, infr::IntStages{}, be->static_act);

@@ -32,7 +32,8 @@ void launch_quantize_q8_group(const QuantTile* tiles_dev, size_t n_tiles, bool p
                               hipStream_t stream);
 // Per-256 quantizer writing MFMA A-operand order (token groups of 32) into the same buffers.
 void launch_quantize_q8_tiled(const float* x, size_t m, size_t k, const ActQ8& out, hipStream_t stream);
-// Per-32 quantizer in the tiled code order (k % 256 == 0): out.d f32 [(g*nb + b)*32 + token%32][8],
+// Per-32 quantizer in the tiled code order (k % 32 == 0; a row is padded with zero blocks to whole
+// 256-element steps, nb = ceil(k / 256)): out.d f32 [(g*nb + b)*32 + token%32][8],
 // out.bsums the code sums in the same order, as f32. transposed16: every 16-element group's codes 4 x 4
 // transposed (dword i = elements i, 4 + i, 8 + i, 12 + i), the order Q2_0's prefill kernel multiplies in.
 void launch_quantize_q8_32_tiled(const float* x, size_t m, size_t k, bool transposed16, const ActQ8& out,

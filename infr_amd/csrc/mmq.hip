@@ -1135,12 +1135,14 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
     }
     // (their kernel's flat time up to 128 tokens, ~145 us at 4096 x 12288, meets the dot4 batches'
     // ~2.1 us per token at 64 tokens)
-    if ((dtype == 2 || dtype == 3 || dtype == 6 || dtype == 7 || dtype == 20) && in_f % 256 == 0 &&
-        (m >= 65 || long_row)) {
+    // (rows that are not whole 256s included: the kernel pads the last step; Q8_0 rows of that kind
+    // multiply the per-32 activation like these formats, crates/infr-cpu/src/lib.rs:1037-1042)
+    if ((dtype == 2 || dtype == 3 || dtype == 6 || dtype == 7 || dtype == 20 || (dtype == 8 && in_f % 256 != 0)) &&
+        in_f % 32 == 0 && (m >= 65 || long_row)) {
         launch_quantize_q8_32_tiled(x, m, in_f, false, act, stream);
         return launch_mmq_shared_nib32(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
     }
-    if (dtype == 42 && in_f % 256 == 0 && (m >= 65 || long_row)) {
+    if (dtype == 42 && in_f % 64 == 0 && (m >= 65 || long_row)) {
         launch_quantize_q8_32_tiled(x, m, in_f, true, act, stream);
         return launch_mmq_shared_nib32(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
     }

@@ -1,5 +1,9 @@
 // Prefill GEMM (65 tokens and up) of the 32-weight-block formats Q4_0, Q4_1, Q5_0, Q5_1 and IQ4_NL on
-// the int8 matrix cores, for rows that are whole 256s.
+// the int8 matrix cores, and of Q8_0 rows that are not whole 256s (which infr-cpu multiplies against
+// the per-32 activation as well: `q8_0_blk32`, crates/infr-cpu/src/lib.rs:1037-1042, d*d8 * iprod per
+// block, kernels.rs:1170-1187). A row may end inside a 256-element step: the quantizer pads the
+// activation with zero codes, scales and sums up to the step, and the blocks past the row's end
+// are not read (their A and B constants are zero), so the padded blocks add +0.0.
 //
 // infr-cpu multiplies these against the per-32 activation (scale d8 and code sum bsum per 32
 // elements) and adds per block (crates/infr-cpu/src/kernels.rs:5496-5520, :5793-5822, :5350-5377,
@@ -33,14 +37,20 @@ struct Nib32Lds {
     static constexpr int bytes = b_off + 32 * 8 * 4;
 };
 
-template <Nib32 K, bool STAGES>
+// The formats of this kernel: the five nibble formats and Q8_0 against per-32 activations.
+enum class Blk32 { Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, Q8_0 };
+
+// nb: 256-element steps (the last one may be partly past the row); nblk: 32-weight blocks of a row
+template <Blk32 K, bool STAGES>
 __global__ __launch_bounds__(256) void mmq_shared_nib32_kernel(
     const uint8_t* __restrict__ w, size_t bpr, const int8_t* __restrict__ qs, const float* __restrict__ d8,
-    const float* __restrict__ bsf, float* __restrict__ y, int m, int out_f, int nb, int32_t* __restrict__ st_iprod) {
-    constexpr bool kAffine = K == Nib32::Q4_1 || K == Nib32::Q5_1;
-    constexpr bool kFive = K == Nib32::Q5_0 || K == Nib32::Q5_1;
-    constexpr int kBlockBytes = 18 + (kAffine ? 2 : 0) + (kFive ? 4 : 0);
-    constexpr int kQhOff = kAffine ? 4 : 2, kQsOff = kBlockBytes - 16;
+    const float* __restrict__ bsf, float* __restrict__ y, int m, int out_f, int nb, int nblk,
+    int32_t* __restrict__ st_iprod) {
+    constexpr bool kAffine = K == Blk32::Q4_1 || K == Blk32::Q5_1;
+    constexpr bool kFive = K == Blk32::Q5_0 || K == Blk32::Q5_1;
+    constexpr bool kBytes = K == Blk32::Q8_0;  // codes are whole bytes: 32 of them per block
+    constexpr int kBlockBytes = kBytes ? 34 : 18 + (kAffine ? 2 : 0) + (kFive ? 4 : 0);
+    constexpr int kQhOff = kAffine ? 4 : 2, kQsOff = kBytes ? 2 : kBlockBytes - 16;
     __shared__ __attribute__((aligned(16))) uint8_t lds[2 * Nib32Lds::bytes];
     __shared__ __attribute__((aligned(16))) float dql[4][8][32], bql[4][8][32];  // per wave: [block][token]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -62,10 +72,12 @@ __global__ __launch_bounds__(256) void mmq_shared_nib32_kernel(
     auto request_rows = [&](Raw& r, int b) {
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-            const uint8_t* blk = wrowp + ((size_t)b * 8 + 2 * p + e) * kBlockBytes;  // 2-byte aligned
-            r.q[e] = load16_a2(blk + kQsOff);
-            r.d[e] = load_u16(blk);
-            r.mw[e] = kAffine ? load_u16(blk + 2) : 0u;
+            const int bi = b * 8 + 2 * p + e;
+            const bool in_row = bi < nblk;  // wave-uniform; past the row's end: block 0 again, scale 0
+            const uint8_t* blk = wrowp + (size_t)(in_row ? bi : 0) * kBlockBytes;  // 2-byte aligned
+            r.q[e] = load16_a2(blk + kQsOff + (kBytes ? 16 * h : 0));
+            r.d[e] = in_row ? load_u16(blk) : 0u;
+            r.mw[e] = kAffine && in_row ? load_u16(blk + 2) : 0u;
             r.qh[e] = kFive ? (load_u16(blk + kQhOff) | (load_u16(blk + kQhOff + 2) << 16)) : 0u;
         }
     };
@@ -75,8 +87,9 @@ __global__ __launch_bounds__(256) void mmq_shared_nib32_kernel(
             v4i out;
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
-                uint32_t c = ((uint32_t)r.q[e][k] >> (4 * h)) & 0x0F0F0F0Fu;
-                if (K == Nib32::IQ4_NL) c = (uint32_t)iq4nl_lookup(c);
+                uint32_t c = (uint32_t)r.q[e][k];
+                if (!kBytes) c = (c >> (4 * h)) & 0x0F0F0F0Fu;
+                if (K == Blk32::IQ4_NL) c = (uint32_t)iq4nl_lookup(c);
                 if (kFive) c |= spread4_to_bit4(r.qh[e] >> (16 * h + 4 * k));
                 out[k] = (int)c;
             }
@@ -84,7 +97,7 @@ __global__ __launch_bounds__(256) void mmq_shared_nib32_kernel(
             if (h == 0) {
                 const float d = f16_bits_to_f32(r.d[e]);
                 const float bb = kAffine ? f16_bits_to_f32(r.mw[e])
-                                         : (K == Nib32::IQ4_NL ? 0.0f : (kFive ? -16.0f : -8.0f) * d);
+                                         : (K == Blk32::IQ4_NL || kBytes ? 0.0f : (kFive ? -16.0f : -8.0f) * d);
                 reinterpret_cast<float*>(buf + Nib32Lds::a_off)[col * 8 + 2 * p + e] = d;
                 reinterpret_cast<float*>(buf + Nib32Lds::b_off)[col * 8 + 2 * p + e] = bb;
             }
@@ -149,7 +162,7 @@ __global__ __launch_bounds__(256) void mmq_shared_nib32_kernel(
                     const int ri = 4 * j + i;
                     if (STAGES) {
                         const int tok = tok0 + 8 * j + 4 * h + i;
-                        if (row_ok && tok < m) st_iprod[((size_t)tok * out_f + wrow) * (nb * 8) + b * 8 + sb] = r[ri];
+                        if (row_ok && tok < m && b * 8 + sb < nblk) st_iprod[((size_t)tok * out_f + wrow) * nblk + b * 8 + sb] = r[ri];
                     }
                     // d8 * (A * iprod + B * bsum)
                     const float t = __builtin_fmaf(cb[sb], bq[i], ca[sb] * (float)r[ri]);
@@ -179,7 +192,8 @@ __global__ __launch_bounds__(256) void mmq_shared_nib32_kernel(
 template <bool STAGES>
 __global__ __launch_bounds__(256) void mmq_shared_q2_0_kernel(
     const uint8_t* __restrict__ w, size_t bpr, const int8_t* __restrict__ qs, const float* __restrict__ d8,
-    const float* __restrict__ bsf, float* __restrict__ y, int m, int out_f, int nb, int32_t* __restrict__ st_iprod) {
+    const float* __restrict__ bsf, float* __restrict__ y, int m, int out_f, int nb, int nblk,
+    int32_t* __restrict__ st_iprod) {
     __shared__ __attribute__((aligned(16))) uint8_t lds[2 * Nib32Lds::bytes];
     __shared__ __attribute__((aligned(16))) float dql[4][8][32], bql[4][8][32];  // per wave: [sub-block][token]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -198,8 +212,9 @@ __global__ __launch_bounds__(256) void mmq_shared_q2_0_kernel(
         uint32_t c[2], d;
     };
     auto request_rows = [&](Raw& r, int b) {
-        const uint8_t* blk = wrowp + ((size_t)b * 4 + p) * 18;  // 2-byte aligned
-        r.d = load_u16(blk);
+        const bool in_row = (b * 4 + p) * 2 < nblk;  // nblk counts 32-element sub-blocks
+        const uint8_t* blk = wrowp + (size_t)(in_row ? b * 4 + p : 0) * 18;  // 2-byte aligned
+        r.d = in_row ? load_u16(blk) : 0u;
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const uint8_t* cp = blk + 2 + 8 * e + 4 * h;
@@ -275,7 +290,7 @@ __global__ __launch_bounds__(256) void mmq_shared_q2_0_kernel(
                     const int ri = 4 * j + i;
                     if (STAGES) {
                         const int tok = tok0 + 8 * j + 4 * h + i;
-                        if (row_ok && tok < m) st_iprod[((size_t)tok * out_f + wrow) * (nb * 8) + b * 8 + sb] = r[ri];
+                        if (row_ok && tok < m && b * 8 + sb < nblk) st_iprod[((size_t)tok * out_f + wrow) * nblk + b * 8 + sb] = r[ri];
                     }
                     const float t = __builtin_fmaf(cb[sb], bq[i], ca[sb] * (float)r[ri]);
                     acc[ri] = __builtin_fmaf(dq[i], t, acc[ri]);
@@ -294,37 +309,38 @@ __global__ __launch_bounds__(256) void mmq_shared_q2_0_kernel(
     }
 }
 
-template <Nib32 K>
+template <Blk32 K>
 static void launch_nib32(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
                          size_t out_f, const IntStages& st, hipStream_t stream) {
     const dim3 grid((unsigned)((out_f + 31) / 32), (unsigned)((m + 127) / 128)), block(256);
-    const int nb = (int)(in_f / 256);
+    const int nb = (int)((in_f + 255) / 256), nblk = (int)(in_f / 32);
     const float* bsf = reinterpret_cast<const float*>(act.bsums);
     if (st.a)
         hipLaunchKernelGGL((mmq_shared_nib32_kernel<K, true>), grid, block, 0, stream, w, bpr, act.qs, act.d, bsf, y,
-                           (int)m, (int)out_f, nb, st.a);
+                           (int)m, (int)out_f, nb, nblk, st.a);
     else
         hipLaunchKernelGGL((mmq_shared_nib32_kernel<K, false>), grid, block, 0, stream, w, bpr, act.qs, act.d, bsf, y,
-                           (int)m, (int)out_f, nb, (int32_t*)nullptr);
+                           (int)m, (int)out_f, nb, nblk, (int32_t*)nullptr);
 }
 
 bool launch_mmq_shared_nib32(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
                              size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream) {
     switch (dtype) {
-    case 2: launch_nib32<Nib32::Q4_0>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
-    case 3: launch_nib32<Nib32::Q4_1>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
-    case 6: launch_nib32<Nib32::Q5_0>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
-    case 7: launch_nib32<Nib32::Q5_1>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
-    case 20: launch_nib32<Nib32::IQ4_NL>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
+    case 2: launch_nib32<Blk32::Q4_0>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
+    case 3: launch_nib32<Blk32::Q4_1>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
+    case 6: launch_nib32<Blk32::Q5_0>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
+    case 7: launch_nib32<Blk32::Q5_1>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
+    case 20: launch_nib32<Blk32::IQ4_NL>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
+    case 8: launch_nib32<Blk32::Q8_0>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
     case 42: {
         const dim3 grid((unsigned)((out_f + 31) / 32), (unsigned)((m + 127) / 128)), block(256);
         const float* bsf = reinterpret_cast<const float*>(act.bsums);
         if (st.a)
             hipLaunchKernelGGL((mmq_shared_q2_0_kernel<true>), grid, block, 0, stream, w, bpr, act.qs, act.d, bsf, y,
-                               (int)m, (int)out_f, (int)(in_f / 256), st.a);
+                               (int)m, (int)out_f, (int)((in_f + 255) / 256), (int)(in_f / 32), st.a);
         else
             hipLaunchKernelGGL((mmq_shared_q2_0_kernel<false>), grid, block, 0, stream, w, bpr, act.qs, act.d, bsf, y,
-                               (int)m, (int)out_f, (int)(in_f / 256), (int32_t*)nullptr);
+                               (int)m, (int)out_f, (int)((in_f + 255) / 256), (int)(in_f / 32), (int32_t*)nullptr);
         return true;
     }
     default: return false;

@@ -109,16 +109,19 @@ __global__ __launch_bounds__(256) void quantize_q8_32_tiled_kernel(const float* 
                                                                    int8_t* __restrict__ qs,
                                                                    float* __restrict__ d,
                                                                    float* __restrict__ bsf,
-                                                                   size_t n_chunks, int nb) {
+                                                                   size_t n_chunks, int nb, int k) {
     const int lane = threadIdx.x & 63;
     const size_t chunk = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (chunk >= n_chunks) return;  // wave-uniform
-    const v4f v = *reinterpret_cast<const v4f*>(x + chunk * 256 + (size_t)lane * 4);
+    // chunk = 256-element step b of token tok; a row that ends inside its last step is padded with
+    // zeros there (whole 32-element groups: codes, scale and sum all zero)
+    const size_t tok = chunk / nb, b = chunk % nb;
+    v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
+    if ((int)b * 256 + lane * 4 < k) v = *reinterpret_cast<const v4f*>(x + tok * k + b * 256 + (size_t)lane * 4);
     uint32_t packed;
     float dd;
     int s, s16;
     quantize_chunk_values<true>(v, packed, dd, s, s16);
-    const size_t tok = chunk / nb, b = chunk % nb;
     const size_t gb = (tok >> 5) * nb + b;
     const int col = (int)(tok & 31);
     const int sb = lane >> 3, h = (lane >> 2) & 1, j4 = lane & 3;
@@ -142,15 +145,15 @@ __global__ __launch_bounds__(256) void quantize_q8_32_tiled_kernel(const float* 
 
 void launch_quantize_q8_32_tiled(const float* x, size_t m, size_t k, bool transposed16, const ActQ8& out,
                                  hipStream_t stream) {
-    const size_t n_chunks = m * k / 256;
+    const size_t nb = (k + 255) / 256, n_chunks = m * nb;
     if (n_chunks == 0) return;
     const dim3 grid((unsigned)((n_chunks + 3) / 4));
     if (transposed16)
         hipLaunchKernelGGL(quantize_q8_32_tiled_kernel<true>, grid, dim3(256), 0, stream, x, out.qs, out.d,
-                           reinterpret_cast<float*>(out.bsums), n_chunks, (int)(k / 256));
+                           reinterpret_cast<float*>(out.bsums), n_chunks, (int)nb, (int)k);
     else
         hipLaunchKernelGGL(quantize_q8_32_tiled_kernel<false>, grid, dim3(256), 0, stream, x, out.qs, out.d,
-                           reinterpret_cast<float*>(out.bsums), n_chunks, (int)(k / 256));
+                           reinterpret_cast<float*>(out.bsums), n_chunks, (int)nb, (int)k);
 }
 
 template <bool PER32>

@@ -231,7 +231,7 @@ def test_prefill_mfma_blk32_formats(be, dtype):
     """From 65 tokens, rows of whole 256s: the int8-MFMA kernel of the 32-weight-block formats. iprod
     per block bit-exact on full-range payloads; outputs at rounding level of the oracle (the same
     terms in another association)."""
-    for m, in_f, out_f in ((65, 512, 40), (130, 768, 130), (257, 2048, 96), (70, 1056, 64)):   # 1056: dot4 arm
+    for m, in_f, out_f in ((65, 512, 40), (130, 768, 130), (257, 2048, 96), (70, 1056, 64)):   # 1056: a ragged last step
         w = synth_weight(dtype, 500 + m, out_f, in_f)
         x = synth_normal_f32(600 + m, m * in_f)
         x[:in_f] *= 37.0
@@ -247,6 +247,36 @@ def test_prefill_mfma_blk32_formats(be, dtype):
     x = synth_normal_f32(81, m * in_f) * np.float32(3.0)
     x[in_f:2 * in_f] = 1e4
     x[2 * in_f:3 * in_f] = -1e4
+    a, _ = be.linear_int_stages(dtype, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
+    oa, _ = orc.linear_int_stages(dtype, w, x, m, in_f, out_f)
+    assert np.array_equal(a, oa)
+    gate(run_linear(be, dtype, w, x, m, in_f, out_f), orc.linear(dtype, w, x, m, in_f, out_f))
+
+
+@pytest.mark.parametrize("dtype", BLK32 + [DType.Q8_0, DType.Q2_0], ids=ids)
+def test_prefill_mfma_rows_that_are_not_whole_256s(be, dtype):
+    """Rows of whole 32-weight blocks that end inside a 256-element step (the gemma widths the
+    reference calls out, crates/infr-cpu/src/lib.rs:1037-1042; Q8_0 rows of that kind multiply the
+    per-32 activation like the nibble formats; Q2_0 needs whole 64s) take the same int8-MFMA
+    kernel, the last step padded with zero blocks: iprod of every real block bit-exact, outputs at
+    the rounding level of the oracle."""
+    q2 = dtype == DType.Q2_0
+    for m, in_f, out_f in ((100, 1152, 96), (65, 1056 if not q2 else 1088, 40), (200, 2112, 70),
+                           (129, 96 if not q2 else 64, 33), (70, 4128 if not q2 else 4160, 48)):
+        w = synth_weight(dtype, 700 + m, out_f, in_f)
+        x = synth_normal_f32(800 + m, m * in_f)
+        x[:in_f] *= 37.0
+        x[2 * in_f:3 * in_f] = 0.0
+        y = run_linear(be, dtype, w, x, m, in_f, out_f)
+        want = orc.linear(dtype, w, x, m, in_f, out_f)
+        assert np.all(y[2] == 0.0)
+        gate(y, want)
+        rel = np.linalg.norm(y.astype(np.float64) - want) / np.linalg.norm(want)
+        assert rel < 3e-6, (m, in_f, rel)
+    m, in_f, out_f = 70, 1184 if not q2 else 1216, 50
+    w = orc.synth_weight(dtype, in_f * out_f, 0x320 + dtype)     # full-range payload bytes
+    x = synth_normal_f32(82, m * in_f) * np.float32(3.0)
+    x[in_f:2 * in_f] = 1e4
     a, _ = be.linear_int_stages(dtype, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
     oa, _ = orc.linear_int_stages(dtype, w, x, m, in_f, out_f)
     assert np.array_equal(a, oa)
