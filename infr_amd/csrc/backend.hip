@@ -49,6 +49,8 @@ struct infr_hip_plan {
     // Add's residual is its first operand
     std::vector<int> moe_add;
     std::vector<char> moe_add_resid_is_a;
+    // per op: the single-row Op::RmsNorm a MoeFfn's router kernel also computes (-1: none)
+    std::vector<int> moe_norm;
     std::vector<infr::GemvOpDesc> descs;
     // per-workgroup tile tables of the grouped launches, back to back (tile_first per step)
     std::vector<infr::GemvTile> tiles;
@@ -988,6 +990,7 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
     // absorbed[k]: op k runs inside some Linear and is not scheduled on its own
     std::vector<int> pre(n, -1), post(n, -1);
     std::vector<char> absorbed(n, 0), publishes(n, 0);
+    plan->moe_norm.assign(n, -1);
     // INFR_HIP_FUSE=0: every op a launch of its own (for comparing against the absorbed form)
     static const int env_fuse = getenv("INFR_HIP_FUSE") ? atoi(getenv("INFR_HIP_FUSE")) : 1;
     auto decode_linear = [&](size_t i) {
@@ -1017,11 +1020,33 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
         // x, with the producer's inputs and dst untouched up to the last of them
         std::vector<size_t> users;
         bool ok = true;
+        int moe_user = -1;  // a single-row MoeFfn reading dst as both x and router_x (fusion.rs:58-73)
         for (size_t i = k + 1; ok && i <= end; ++i) {
             if (!any_overlap(rd[i], wr[k])) continue;
-            ok = decode_linear(i) && plan->ops[i].in_f == p.in_f &&
-                 static_cast<const float*>(bindings[plan->ops[i].x]->ptr) == ea[k].dst;
+            const auto& u = plan->ops[i];
+            if (p.kind == INFR_OP_RMS_NORM && u.kind == INFR_OP_MOE_FFN && u.moe.rows == 1 && u.moe.ne == p.in_f &&
+                static_cast<const float*>(bindings[u.x]->ptr) == ea[k].dst &&
+                static_cast<const float*>(bindings[u.router_x]->ptr) == ea[k].dst && moe_user < 0 && users.empty()) {
+                moe_user = (int)i;
+                continue;
+            }
+            ok = moe_user < 0 && decode_linear(i) && u.in_f == p.in_f &&
+                 static_cast<const float*>(bindings[u.x]->ptr) == ea[k].dst;
             if (ok) users.push_back(i);
+        }
+        if (ok && moe_user >= 0) {
+            // the MoeFfn is the definition's only reader: its router kernel normalises the row and
+            // stores dst; nothing up to it may touch the norm's inputs or dst
+            for (size_t j = k + 1; ok && j < (size_t)moe_user; ++j)
+                ok = !any_overlap(wr[j], rd[k]) && !any_overlap(wr[j], wr[k]);
+            // the op's own output must not land on the norm's inputs (its kernels re-read them)
+            ok = ok && !any_overlap(wr[moe_user], rd[k]);
+            if (!ok) continue;
+            absorbed[k] = 1;
+            plan->moe_norm[moe_user] = (int)k;
+            for (const auto& r : rd[k]) rd[moe_user].push_back(r);
+            wr[moe_user].push_back(wr[k][0]);
+            continue;
         }
         if (!ok || users.empty()) continue;
         for (size_t j = k + 1; ok && j <= users.back(); ++j)
@@ -1064,8 +1089,10 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
             for (size_t j = i + 1; ok && j < k; ++j)
                 ok = !any_overlap(wr[j], wr[k]) && !any_overlap(rd[j], wr[k]) && !any_overlap(wr[j], b_span) &&
                      !any_overlap(wr[j], wr[i]);
-            // the producer's own inputs must not alias the Add's destination
-            ok = ok && !any_overlap(rd[i], wr[k]);
+            // a Linear's own inputs must not alias the Add's destination (its workgroups read them
+            // while others already store); a MoeFfn reads its inputs in launches that finish before
+            // the one that stores
+            ok = ok && (moe || !any_overlap(rd[i], wr[k]));
             if (!ok) continue;
             post[i] = (int)k;
             resid[i] = resid_is_a ? ea[k].x : ea[k].aux;
@@ -1220,6 +1247,15 @@ static int enqueue_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t
                                    bindings[op.gate_exps], bindings[op.up_exps], bindings[op.down_exps],
                                    bindings[op.dst], nullptr, nullptr, &ms, &mb))
                 return rc;
+            if (plan->moe_norm[st.op] >= 0) {
+                const auto& nop = plan->ops[plan->moe_norm[st.op]];
+                ElementwiseArgs norm;
+                if (int rc = check_elementwise(be, nop, bindings, &norm)) return rc;
+                mb.router_x = norm.x;
+                mb.norm_w = norm.aux;
+                mb.norm_dst = norm.dst;
+                mb.norm_eps = nop.eps;
+            }
             if (plan->moe_add[st.op] >= 0) {
                 ElementwiseArgs add;
                 if (int rc = check_elementwise(be, plan->ops[plan->moe_add[st.op]], bindings, &add)) return rc;

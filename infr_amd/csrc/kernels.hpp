@@ -239,6 +239,12 @@ struct MoeBuffers {
     // produces dst; add_dst may be add_b (each element is read and written by one thread)
     const float* add_b = nullptr;
     float* add_dst = nullptr;
+    // absorbed single-row Op::RmsNorm in front (fusion.rs:58-73, `moe_ok`): router_x is then the
+    // norm's input; the router kernel normalises it (rms_norm_kernel's arithmetic and order), its
+    // first workgroup stores the result to `norm_dst`, and x must be that same `norm_dst`
+    const float* norm_w = nullptr;
+    float* norm_dst = nullptr;
+    float norm_eps = 0.0f;
 };
 // Q6_K prefill GEMM on the int8 matrix cores (any m; used from 33 tokens): activations in the tiled quantizer's layout
 // (launch_quantize_q8_tiled); st.a, when set, receives isum per (token, row, 256-block).

@@ -186,11 +186,25 @@ template <int NL>
 __global__ __launch_bounds__(256) void moe_router_kernel(
     const float* __restrict__ router, const float* __restrict__ rx, float* __restrict__ logits,
     int* __restrict__ tickets, int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, int ne,
-    int n_expert, int rows, int n_used, float scale, int kc, int epw) {
+    int n_expert, int rows, int n_used, float scale, int kc, int epw, const float* __restrict__ norm_w,
+    float* __restrict__ norm_dst, float norm_eps) {
     extern __shared__ __attribute__((aligned(16))) float rl[];  // [epw] rows | [32 / epw] rows
     __shared__ __attribute__((aligned(16))) SelectLds sel;
     __shared__ int s_last;
     const int tid = threadIdx.x;
+    // An absorbed RmsNorm of the single activation row: the scale with rms_norm_kernel's own
+    // reduction (stride-256 partial sums, wave sums, ((p0 + p1) + (p2 + p3))), applied while the
+    // row is staged; the first workgroup stores the normalised row for the expert kernels.
+    float nscale = 1.0f;
+    if (norm_w) {
+        float s = 0.0f;
+        for (int i = tid; i < ne; i += 256) s += rx[i] * rx[i];
+        s = wave_sum_f(s);
+        if ((tid & 63) == 0) sel.red[tid >> 6] = s;
+        __syncthreads();
+        const float ss = ((sel.red[0] + sel.red[1]) + (sel.red[2] + sel.red[3])) / (float)ne;
+        nscale = 1.0f / sqrtf(ss + norm_eps);
+    }
     const int tpw = kRouterPairs / epw;
     const int e0 = blockIdx.x * epw, t0 = blockIdx.y * tpw;
     const int n_e = min(epw, n_expert - e0), n_t = min(tpw, rows - t0);
@@ -215,7 +229,15 @@ __global__ __launch_bounds__(256) void moe_router_kernel(
                 const float* src = row < n_e ? router + (size_t)(e0 + row) * ne : rx + (size_t)(t0 + row - n_e) * ne;
                 // elements 4q .. 4q+3 are accumulators 4(q & 1) .. +3 at step q / 2
                 dst[u] = (row < n_e ? lw + row * ld : lx + (row - n_e) * ld) + 4 * (q & 1) * la + (q >> 1);
-                if (i < total) tmp[u] = reinterpret_cast<const v4f*>(src + k0)[q];
+                if (i < total) {
+                    tmp[u] = reinterpret_cast<const v4f*>(src + k0)[q];
+                    if (norm_w && row >= n_e) {
+                        const v4f wv = reinterpret_cast<const v4f*>(norm_w + k0)[q];
+                        tmp[u] = v4f{tmp[u].x * nscale * wv.x, tmp[u].y * nscale * wv.y, tmp[u].z * nscale * wv.z,
+                                     tmp[u].w * nscale * wv.w};
+                        if (norm_dst && blockIdx.x == 0) reinterpret_cast<v4f*>(norm_dst + k0)[q] = tmp[u];
+                    }
+                }
             }
 #pragma unroll
             for (int u = 0; u < NL; ++u)
@@ -966,6 +988,7 @@ size_t moe_workspace_bytes(const MoeShape& s) {
 
 const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hipStream_t stream) {
     if (s.router_dtype != 0) return "router dtype must be F32";
+    if (b.norm_w && (s.rows != 1 || b.x != b.norm_dst)) return "an absorbed RmsNorm needs a single row read from its dst";
     if (s.n_used > 64 || s.n_expert > 1024 || s.n_used > s.n_expert) return "n_used <= 64 and n_expert <= 1024 required";
     if (s.ne % 256 != 0 || s.n_ff % 256 != 0) return "ne and n_ff_exp must be multiples of 256";
     const size_t pairs = (size_t)s.rows * s.n_used;
@@ -1020,12 +1043,13 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     else if (s.rows == 1)
         hipLaunchKernelGGL(moe_router_kernel<24>, dim3((unsigned)((s.n_expert + epw - 1) / epw), 1), dim3(256), router_lds,
                            stream, b.router, b.router_x, logits, tickets, sel_idx, sel_w, s.ne, s.n_expert, s.rows,
-                           s.n_used, s.scale, kc, epw);
+                           s.n_used, s.scale, kc, epw, b.norm_w, b.norm_dst, b.norm_eps);
     else
         hipLaunchKernelGGL(moe_router_kernel<8>,
                            dim3((unsigned)((s.n_expert + epw - 1) / epw), (unsigned)((s.rows + tpw - 1) / tpw)),
                            dim3(256), router_lds, stream, b.router, b.router_x, logits, (int*)nullptr, sel_idx, sel_w,
-                           s.ne, s.n_expert, s.rows, s.n_used, s.scale, kc, epw);
+                           s.ne, s.n_expert, s.rows, s.n_used, s.scale, kc, epw, (const float*)nullptr, (float*)nullptr,
+                           0.0f);
     auto bytes_per_row = [](int dtype, size_t in_f) -> size_t {
         switch (dtype) {
         case 12: return in_f / 256 * 144;

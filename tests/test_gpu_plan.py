@@ -486,3 +486,57 @@ def test_moe_residual_add_rides_in_the_last_moe_kernel(be, rows, resid_first):
         assert _rel(got_y, want.ravel()) < 1e-4
         assert np.array_equal(bits(got_h), bits(h0 + got_y))
     assert plan.launches() == (3 if rows == 1 else 7)       # no launch of its own for the Add
+
+
+def test_single_row_rms_norm_rides_in_the_moe_router_kernel(be):
+    """RmsNorm -> MoeFfn(rows == 1) reading the normalised row as x and router_x
+    (crates/infr-core/src/fusion.rs:58-73, `moe_ok`) -> Add(residual): three launches for the whole
+    sublayer. The router kernel normalises with the stand-alone kernel's own arithmetic, so the MoE
+    output equals, bit for bit, that of a plan in which a second reader of the normalised row keeps
+    the RmsNorm a launch of its own."""
+    from infr_amd import Add, MoeFfn, RmsNorm
+    ne, n_expert, n_used, nff = 1024, 16, 4, 256
+    router = synth_normal_f32(2, n_expert * ne, sigma=0.05)
+    gate = synth_weight(DType.Q4K, 3, n_expert * nff, ne, 0.05)
+    up = synth_weight(DType.Q4K, 4, n_expert * nff, ne, 0.05)
+    down = synth_weight(DType.Q4K, 5, n_expert * ne, nff, 0.05)
+    nw = synth_normal_f32(6, ne, mean=1.0, sigma=0.1)
+    shared = [be.upload_new(a) for a in (router, gate, up, down, nw)]
+
+    def build(extra_reader):
+        g, binds = Graph(), Bindings()
+        h = g.input(TensorDesc((1, ne), DType.F32))
+        xn, y, junk = (g.output(TensorDesc((1, ne), DType.F32)) for _ in range(3))
+        bufs = {t: be.alloc(ne * 4) for t in (h, xn, y, junk)}
+        for t, b in bufs.items():
+            binds.bind(t, b)
+        rid = g.weight(TensorDesc((n_expert, ne), DType.F32))
+        gid, uid = (g.weight(TensorDesc((n_expert, nff, ne), DType.Q4K)) for _ in range(2))
+        did = g.weight(TensorDesc((n_expert, ne, nff), DType.Q4K))
+        wid = g.weight(TensorDesc((ne,), DType.F32))
+        for t, b in zip((rid, gid, uid, did, wid), shared):
+            binds.bind(t, b)
+        g.push(RmsNorm(h, wid, xn, 1, ne, 1e-6))
+        g.push(MoeFfn(xn, xn, rid, gid, uid, did, y, ne, n_expert, n_used, nff))
+        g.push(Add(h, y, h, ne))
+        if extra_reader:
+            g.push(Add(xn, xn, junk, ne))
+        return be.compile(g), binds, bufs[h], bufs[xn], bufs[y]
+
+    fused, plain = build(False), build(True)
+    for seed in (10, 20, 30):
+        h0 = synth_normal_f32(seed, ne)
+        outs = []
+        for plan, binds, hb, xnb, yb in (fused, plain):
+            be.upload(hb, h0)
+            be.execute(plan, binds)
+            outs.append([be.download(b, np.empty(ne, np.float32)) for b in (hb, xnb, yb)])
+        for a, b in zip(*outs):
+            assert np.array_equal(bits(a), bits(b))
+        h1, xn1, y1 = outs[0]
+        xn_ref = orc.rms_norm(h0, nw, 1, ne, 1e-6)
+        assert _rel(xn1, xn_ref) < 2e-6
+        want, _, _ = orc.moe_ffn(xn_ref, router, gate, up, down, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff)
+        assert _rel(y1, want.ravel()) < 1e-4
+        assert np.array_equal(bits(h1), bits(h0 + y1))
+    assert fused[0].launches() == 3 and plain[0].launches() == 5
