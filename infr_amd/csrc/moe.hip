@@ -1159,12 +1159,13 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     const size_t n_act = pairs * s.n_ff, n_out = (size_t)s.rows * s.ne;
     // Prefill-sized batches: the pairs are bucketed by expert and every bank runs its format's
     // int8-MFMA GEMM per (expert, 32 pairs) tile, so an expert's weights are read once per 32 of
-    // its pairs instead of once per pair. From an average of `bucket_min` pairs per expert up (the
-    // per-pair GEMVs win below: most tiles would hold one or two pairs).
-    constexpr int bucket_min = 4;
+    // its pairs instead of once per pair. From an average of `bucket_min` pairs per expert up: the
+    // tiles' time is flat in the number of pairs there (Q4_K banks, 128 experts, top-8: 125-130 us per
+    // layer from 32 to 96 tokens) while the per-pair GEMVs grow by ~2.6 us per token (126 us at 32
+    // tokens, 168 at 48); with one pair per expert the tiles lose (103 against 87 us at 16 tokens).
+    constexpr int bucket_min = 2;
     // (a Q6_K tile costs more than the others': at four pairs per expert its per-pair GEMVs tie with
-    // the tiles, 313 us per layer either way, and it is bucketed from eight; Q5_K and Q8_0 banks
-    // gain from four on, 179 against 254 and 299 against 399 us)
+    // the tiles, 313 us per layer either way, so it is bucketed from four)
     auto has_mfma = [&](int dt) {
         return ((dt == 12 || dt == 13 || dt == 8) && pairs >= (size_t)bucket_min * s.n_expert) ||
                (dt == 14 && pairs >= (size_t)2 * bucket_min * s.n_expert);
