@@ -30,6 +30,7 @@ struct infr_hip_plan {
     hipGraphExec_t exec = nullptr;
     std::vector<void*> bound;
     uint64_t scratch_epoch = 0;  // the backend's scratch epoch the recording was made under
+    size_t recorded_nodes = 0;   // nodes of the recorded graph: the launches of one execute
     // Launch schedule for the bound addresses: ops ordered by dependency level; the m == 1 ops
     // of a level that share (dtype, in_f) form one grouped decode launch.
     struct Step {
@@ -900,10 +901,12 @@ int infr_hip_compile(infr_hip_t* be, const infr_hip_op_t* ops, size_t n_ops, inf
 
 size_t infr_hip_plan_launches(const infr_hip_plan_t* plan) {
     if (!plan) return 0;
+    if (plan->recorded_nodes) return plan->recorded_nodes;
+    // nothing recorded (direct submission): the common forms' counts
     size_t n = 0;
     for (const auto& st : plan->steps) {
         if (st.op < 0) n += st.m > 1 ? 2 : 1;                              // grouped launch (+ grouped quantize)
-        else if (plan->ops[st.op].kind == INFR_OP_MOE_FFN) n += plan->ops[st.op].moe.rows == 1 ? 3 : 7;
+        else if (plan->ops[st.op].kind == INFR_OP_MOE_FFN) n += plan->ops[st.op].moe.rows == 1 ? 3 : 6;
         else if (is_elementwise(plan->ops[st.op].kind) || plan->ops[st.op].kind == INFR_OP_EMBED_GATHER) n += 1;
         else n += 2;                                                       // quantize + GEMM
     }
@@ -1349,6 +1352,8 @@ int infr_hip_execute(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t* c
         return rc;
     }
     if (e != hipSuccess) return fail(be, INFR_HIP_ERR_BACKEND, std::string("hipStreamEndCapture: ") + hipGetErrorString(e));
+    size_t n_nodes = 0;
+    plan->recorded_nodes = hipGraphGetNodes(graph, nullptr, &n_nodes) == hipSuccess ? n_nodes : 0;
     e = hipGraphInstantiate(&plan->exec, graph, nullptr, nullptr, 0);
     (void)hipGraphDestroy(graph);
     if (e != hipSuccess) {
