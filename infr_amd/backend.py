@@ -16,8 +16,7 @@ from enum import IntEnum
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# INFR_HIP_LIB: a measurement build of the library (infr_amd.build with INFR_HIP_BUILD_OUT) instead
-LIB_PATH = os.environ.get("INFR_HIP_LIB") or os.path.join(_HERE, "libinfr_hip.so")
+LIB_PATH = os.path.join(_HERE, "libinfr_hip.so")
 
 
 class DType(IntEnum):

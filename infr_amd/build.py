@@ -37,22 +37,21 @@ def hipcc() -> str:
     return exe
 
 
-def _compile(src: str) -> str:
-    obj = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
-    # INFR_HIP_BUILD_FLAGS: extra compiler flags (e.g. -DINFR_PF_Q8_0=2) for measurement builds
-    extra = os.environ.get("INFR_HIP_BUILD_FLAGS", "").split()
-    cmd = [hipcc(), *DEVICE_FLAGS, *extra, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
+def _compile(src: str, extra_flags: tuple = (), obj_dir: str = OBJ) -> str:
+    obj = os.path.join(obj_dir, os.path.splitext(src)[0] + ".o")
+    cmd = [hipcc(), *DEVICE_FLAGS, *extra_flags, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src}:\n{r.stderr[-4000:]}")
     return obj
 
 
-def build(verbose: bool = False) -> str:
-    os.makedirs(OBJ, exist_ok=True)
+def build(verbose: bool = False, lib: str = LIB, extra_flags: tuple = (), obj_dir: str = OBJ) -> str:
+    """Compiles every source and links ``lib``. ``extra_flags`` / ``obj_dir`` serve builds of a
+    variant of the library beside the product's (the defaults are the product)."""
+    os.makedirs(obj_dir, exist_ok=True)
     with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
-        objs = list(ex.map(_compile, SOURCES))
-    lib = os.environ.get("INFR_HIP_BUILD_OUT", LIB)  # measurement builds go elsewhere
+        objs = list(ex.map(lambda src: _compile(src, tuple(extra_flags), obj_dir), SOURCES))
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib, *objs]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
