@@ -482,7 +482,7 @@ def main():
     ms = max(dev_ms, wall_ms)
     value = sw.bytes / (ms * 1e-3) / 1e9
     n_launch = max(1, sw.plan.launches())          # grouped: independent ops share a launch
-    # Dominant kernel: the in_f = 4096 Q4_K GEMV (gemv_fused_kernel<FmtQ4K, 1, 16>), 216 of the 252
+    # Dominant kernel: the in_f = 4096 Q4_K GEMV (gemv_fused_kernel<FmtQ4K, 1, 8>), 216 of the 252
     # ops, timed alone with HIP events on the backend's stream: one launch per execute.
     k_ms, _ = sw.time(args.steps, 2, sw.plan_4096)
     k_launches = max(1, sw.plan_4096.launches())
@@ -512,7 +512,7 @@ def main():
                    "device": caps["device_name"], "compute_units": caps["compute_units"]},
         "pct_of_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "launches_per_step": n_launch,
-        "roofline": {"bound": "hbm", "kernel": "gemv_fused_kernel<FmtQ4K, 1, 16> (in_f 4096 group)",
+        "roofline": {"bound": "hbm", "kernel": "gemv_fused_kernel<FmtQ4K, 1, 8> (in_f 4096 group)",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "avg_launch_us": round(avg_launch_us, 3), "bytes_per_launch": bytes_per_launch,
