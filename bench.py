@@ -29,7 +29,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
 # algorithmic bytes per launch -> measured HBM bytes per launch (profiles/gemv_q4k_decode_sweep.md)
-MEASURED_TRAFFIC = {2887778304: 2895427797}
+MEASURED_TRAFFIC = {2887778304: 2896067761}
 INT8_PEAK_TOPS = 5000.0    # MI355X dense int8 MFMA, published
 
 # (name, out_f, in_f) of one Qwen3-8B decoder layer
