@@ -559,14 +559,17 @@ static bool plan_group_fmt(size_t in_f, const GemvOpDesc* ops, int n, GemvGroupP
     // spread over the widest workgroup that fits the registers (18.1 -> 15.4 us for a 4096 x 12288
     // Q4_K matrix behind an absorbed gated activation).
     if (steps <= F::kWide16Steps && cus > 0 && wg <= cus) nw = 16;
-    // Many rounds of one-step rows: eight-wave workgroups of 64 rows, so that two or three of them
+    // Many rounds of one-step rows: eight-wave workgroups of 64 rows or more, so that two or three of them
     // share a compute unit and one's prologue runs under the others' streaming (16-wave workgroups
     // fill the registers alone). Measured on the 216-matrix in_f 4096 group: Q4_K 6.05 -> 6.19 TB/s,
     // Q6_K 4.84 -> 5.25 and 5.35 -> 5.80 on its two shapes, Q5_K +3 %, the 32-weight-block formats
     // and Q2_0 unchanged; 32-row tiles cost those up to 15 % (more prologues per weight byte).
     if (steps == 1 && cus > 0 && wg > 4 * cus) {
         nw = 8;
-        rows_per_wg = std::min<size_t>(rows_per_wg, 64);
+        // (at least 64 rows and ~144 KB of weights per prologue: Q2_0's 1152-byte rows take 128 -
+        // its sweep runs at 5.3 TB/s so, 4.9 with 64)
+        const size_t cap = std::max<size_t>(64, (size_t)147456 / std::max<size_t>(1, ops[0].bpr));
+        rows_per_wg = std::min<size_t>(rows_per_wg, cap);
         wg = 0;
         for (int i = 0; i < n; ++i) wg += (int)(((size_t)ops[i].out_f + rows_per_wg - 1) / rows_per_wg);
     }
