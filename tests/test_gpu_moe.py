@@ -297,11 +297,13 @@ def test_moe_banks_of_three_different_kinds(be, rows):
     check(*got, *want)
 
 
+@pytest.mark.parametrize("rows", [1, 3])
 @pytest.mark.parametrize("dtype", [DType.Q4K, DType.Q6K])
-def test_moe_single_row_of_a_hidden_size_above_4096(be, dtype):
+def test_moe_hidden_size_above_4096(be, dtype, rows):
     """The factored one-token kernels keep a row's activations in registers (up to 4096 of them);
-    longer rows take the decode-and-dot form of the same Raw arithmetic."""
-    rows, ne, n_expert, n_used, nff = 1, 8192, 4, 2, 512
+    longer single rows take the decode-and-dot form of the same Raw arithmetic. Two rows and more
+    run the id-gathered int8 GEMVs at any length their wave steps reach."""
+    ne, n_expert, n_used, nff = 8192, 4, 2, 512
     gate, up, down = banks(400, ne, n_expert, nff, dtype, sigma=0.03)
     x = synth_normal_f32(401, rows * ne)
     router = synth_normal_f32(402, n_expert * ne, sigma=0.02)
