@@ -290,6 +290,10 @@ def single_shape(be, dtype, m, in_f, out_f, reps=40, rotate_bytes=768 << 20):
     level cache, `reps` back-to-back launches. Returns (ms per launch, weight bytes)."""
     from infr_amd import Bindings, BufferUsage, DType, Graph, Linear, TensorDesc, synth_normal_f32, synth_weight
     nb = weight_bytes(dtype, out_f, in_f)
+    # small matrices: enough ops that a plan moves ~384 MB, so the fixed cost of one graph launch
+    # (~8 us against a 20 us kernel for forty 1024 x 4096 matrices) does not pass for bandwidth
+    if rotate_bytes > 1 and m <= 8:
+        reps = max(reps, -(-(384 << 20) // nb))
     copies = max(2, min(reps, -(-rotate_bytes // nb)))
     g, binds, keep = Graph(), Bindings(), []
     xid = g.input(TensorDesc((m, in_f), DType.F32))
