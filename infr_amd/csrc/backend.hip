@@ -347,6 +347,13 @@ int check_linear(infr_hip_t* be, int dtype, const infr_hip_buffer_t* w, size_t w
     return INFR_HIP_OK;
 }
 
+// A Linear whose dst overlaps its x (the CPU arm computes into a fresh vector first, lib.rs:985-1492,
+// so that is a legal graph). The one-launch decode kernels read x in every workgroup while others
+// already store y, so such an op takes a path that consumes x before anything is written.
+static bool floats_overlap(const float* a, size_t na, const float* b, size_t nb) {
+    return a < b + nb && b < a + na;
+}
+
 int enqueue_linear(infr_hip_t* be, int dtype, const LinearArgs& la, const float* x, float* y,
                    size_t m, size_t in_f, size_t out_f, const infr::IntStages& st, const infr::ActQ8& act) {
     bool ok;
@@ -354,6 +361,12 @@ int enqueue_linear(infr_hip_t* be, int dtype, const LinearArgs& la, const float*
         if (st.a)
             return fail(be, INFR_HIP_ERR_UNSUPPORTED,
                         "int_stages: one token of dtype " + std::to_string(dtype) + " has no integer stage");
+        if (floats_overlap(x, m * in_f, y, m * out_f)) {
+            // in place: the kernel reads a copy of x parked in the activation scratch
+            float* copy = reinterpret_cast<float*>(act.qs);
+            HIP_TRY(be, hipMemcpyAsync(copy, x, m * in_f * sizeof(float), hipMemcpyDeviceToDevice, be->stream));
+            x = copy;
+        }
         ok = infr::launch_gemv_f32act(dtype, la.wrows, la.bpr, x, y, in_f, out_f, be->stream);
     } else {
         // quantizes x into the scratch in the layout its kernel reads, then multiplies
@@ -624,7 +637,8 @@ int infr_hip_linear(infr_hip_t* be, int dtype, const infr_hip_buffer_t* w, size_
     if (int rc = check_linear(be, dtype, w, w_numel, w_off, x, m, in_f, out_f, &la)) return rc;
     if (!dst || dst->len < m * out_f * sizeof(float))
         return fail(be, INFR_HIP_ERR_INVALID, "linear: dst buffer missing or too small");
-    if (m == 1 && !runs_alone(dtype, m, in_f)) {
+    const bool in_place = floats_overlap(static_cast<const float*>(x->ptr), m * in_f, static_cast<float*>(dst->ptr), m * out_f);
+    if (m == 1 && !runs_alone(dtype, m, in_f) && !in_place) {
         // decode: one fused launch (quantize x in LDS + GEMV)
         const infr::GemvOpDesc op{la.wrows, static_cast<const float*>(x->ptr),
                                   static_cast<float*>(dst->ptr), la.bpr, (int32_t)out_f};
@@ -644,7 +658,8 @@ int infr_hip_linear_noalloc(infr_hip_t* be, int dtype, const infr_hip_buffer_t* 
     if (int rc = check_linear(be, dtype, w, w_numel, w_off, x, m, in_f, out_f, &la)) return rc;
     if (!dst || dst->len < m * out_f * sizeof(float))
         return fail(be, INFR_HIP_ERR_INVALID, "linear_noalloc: dst buffer missing or too small");
-    if (m == 1 && !runs_alone(dtype, m, in_f)) {
+    const bool in_place = floats_overlap(static_cast<const float*>(x->ptr), m * in_f, static_cast<float*>(dst->ptr), m * out_f);
+    if (m == 1 && !runs_alone(dtype, m, in_f) && !in_place) {
         // decode: the fused launch keeps the quantized activation in LDS and needs no scratch
         const infr::GemvOpDesc op{la.wrows, static_cast<const float*>(x->ptr),
                                   static_cast<float*>(dst->ptr), la.bpr, (int32_t)out_f};
@@ -996,9 +1011,15 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
     plan->moe_norm.assign(n, -1);
     // INFR_HIP_FUSE=0: every op a launch of its own (for comparing against the absorbed form)
     static const int env_fuse = getenv("INFR_HIP_FUSE") ? atoi(getenv("INFR_HIP_FUSE")) : 1;
+    // (a one-row Linear in place on its x runs alone, through the quantize-then-multiply path)
+    // (taken from the ops as written: absorbing an Add later puts the residual among the Linear's spans)
+    std::vector<char> in_place(n, 0);
+    for (size_t i = 0; i < n; ++i)
+        in_place[i] = plan->ops[i].kind == INFR_OP_LINEAR && any_overlap(rd[i], wr[i]);
+    auto self_alias = [&](size_t i) { return in_place[i] != 0; };
     auto decode_linear = [&](size_t i) {
         return plan->ops[i].kind == INFR_OP_LINEAR && plan->ops[i].m == 1 &&
-               !runs_alone(plan->ops[i].w_dtype, 1, plan->ops[i].in_f);
+               !runs_alone(plan->ops[i].w_dtype, 1, plan->ops[i].in_f) && !self_alias(i);
     };
     for (size_t k = 0; env_fuse && k < n; ++k) {
         const auto& p = plan->ops[k];
@@ -1200,7 +1221,7 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
                 plan->steps.push_back(st);
                 continue;
             }
-            if (op.kind != INFR_OP_LINEAR || op.m != 1 || runs_alone(op.w_dtype, op.m, op.in_f)) {
+            if (op.kind != INFR_OP_LINEAR || op.m != 1 || runs_alone(op.w_dtype, op.m, op.in_f) || self_alias(i)) {
                 st.op = (int)i;
                 taken[i] = 1;
                 plan->steps.push_back(st);
@@ -1212,7 +1233,7 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
             for (size_t k = i; k < n; ++k) {
                 const auto& o2 = plan->ops[k];
                 if (level[k] != lv || taken[k] || absorbed[k] || o2.kind != INFR_OP_LINEAR || o2.m != 1 ||
-                    o2.w_dtype != op.w_dtype || o2.in_f != op.in_f ||
+                    o2.w_dtype != op.w_dtype || o2.in_f != op.in_f || self_alias(k) ||
                     (op.w_dtype == INFR_DTYPE_Q8_0 && (o2.in_f % 256 == 0) != (op.in_f % 256 == 0)))
                     continue;
                 taken[k] = 1;

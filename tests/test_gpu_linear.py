@@ -157,6 +157,23 @@ def test_small_batch_vs_oracle(be, dtype, m):
     gate(y, orc.linear(dtype, w, x, m, in_f, out_f))
 
 
+@pytest.mark.parametrize("dtype", [DType.Q4K, DType.Q6K, DType.Q8_0, DType.Q5_0])
+@pytest.mark.parametrize("noalloc", [False, True])
+def test_one_row_linear_in_place_on_its_input(be, dtype, noalloc):
+    # dst == x is a legal graph (the CPU arm builds its result in a fresh vector, lib.rs:985-1492):
+    # every output row must see the x from before the op. 4096 rows span many workgroups.
+    n = 4096
+    w = synth_weight(dtype, 0x51, n, n, sigma=0.02)
+    x = synth_normal_f32(0x52, n)
+    wb, xb = be.upload_new(w), be.upload_new(x)
+    (be.linear_noalloc if noalloc else be.linear)(dtype, wb, xb, xb, 1, n, n)
+    y = be.download(xb, np.empty((1, n), np.float32))
+    want = orc.linear(dtype, w, x, 1, n, n)
+    gate(y, want)
+    if dtype in (DType.Q4K, DType.Q6K):
+        assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), "not bit-identical"
+
+
 def test_w_off_selects_rows_of_a_concatenated_weight(be):
     in_f, rows = 512, 48
     w = synth_weight(DType.Q4K, 3, rows, in_f)

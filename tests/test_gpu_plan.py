@@ -100,6 +100,32 @@ def test_in_place_chain_is_ordered(be):
     assert np.array_equal(bits(be.download(yb, np.empty(in_f, np.float32))), bits(y2))
 
 
+def test_one_row_linear_in_place_inside_a_plan(be):
+    # y = A y next to a sibling z = B y that reads the old y first (program order), then y = C y
+    # again: the in-place ops must neither join a group nor overtake the reader.
+    n = 2048
+    g, binds = Graph(), Bindings()
+    yid = g.output(TensorDesc((1, n), DType.F32))
+    zid = g.output(TensorDesc((1, n), DType.F32))
+    y0 = synth_normal_f32(0x61, n)
+    ws = [synth_weight(DType.Q4K, s, n, n, sigma=0.03) for s in (0x62, 0x63, 0x64)]
+    ids = [g.weight(TensorDesc((n, n), DType.Q4K)) for _ in ws]
+    yb, zb = be.upload_new(y0), be.alloc(n * 4)
+    binds.bind(yid, yb).bind(zid, zb)
+    for i, w in zip(ids, ws):
+        binds.bind(i, be.upload_new(w))
+    g.push(Linear(yid, ids[0], zid, 1, n, n))   # z = B y0
+    g.push(Linear(yid, ids[1], yid, 1, n, n))   # y = A y0   (in place)
+    g.push(Linear(yid, ids[2], yid, 1, n, n))   # y = C y    (in place again)
+    plan = be.compile(g)
+    be.execute(plan, binds)
+    z = orc.linear(DType.Q4K, ws[0], y0, 1, n, n).ravel()
+    y1 = orc.linear(DType.Q4K, ws[1], y0, 1, n, n).ravel()
+    y2 = orc.linear(DType.Q4K, ws[2], y1, 1, n, n).ravel()
+    assert np.array_equal(bits(be.download(zb, np.empty(n, np.float32))), bits(z))
+    assert np.array_equal(bits(be.download(yb, np.empty(n, np.float32))), bits(y2))
+
+
 @pytest.mark.parametrize("m", [2, 5, 8, 12, 16, 19])
 def test_small_batch_ops_run_as_groups(be, m):
     """m = 2..32 inside a plan: ops of a level that share (dtype, in_f, m) become one quantize
