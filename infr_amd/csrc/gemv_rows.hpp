@@ -78,6 +78,9 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
         if (r - row0 < 64) return pf;
         return wanted ? gload<float>(add_b + r) : 0.0f;
     };
+    // An absorbed Add may name this op's own dst as its dst (y = y + b as the graph writes it):
+    // then only the sum is stored, through add_dst alone.
+    const bool plain_y = y != add_dst;
     constexpr int LS = OrderedSum<STEPS>::kRowStride;
     int in_batch = 0, batch_row0 = row0;
     // A row's step-t term: parked for the ordered sum, or added to the lane's partial sum.
@@ -103,7 +106,7 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
                         acc += v.z;
                         acc += v.w;
                     }
-                    gstore<float>(y + batch_row0 + lane, acc);
+                    if (plain_y) gstore<float>(y + batch_row0 + lane, acc);
                     // an absorbed Op::Add: dst = a + b with a = this output
                     if (add_dst) gstore<float>(add_dst + batch_row0 + lane, acc + resid);
                 }
@@ -114,7 +117,7 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
             s = wave_sum_f(s);
             const float resid = add_dst ? residual(row, lane == 0) : 0.0f;
             if (lane == 0) {
-                gstore<float>(y + row, s);
+                if (plain_y) gstore<float>(y + row, s);
                 if (add_dst) gstore<float>(add_dst + row, s + resid);
             }
         } else {
@@ -131,7 +134,7 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
                 acc += __shfl_xor(acc, 32, kWave);
                 const float resid = add_dst ? residual(batch_row0 + lane, lane < in_batch) : 0.0f;
                 if (lane < in_batch) {
-                    gstore<float>(y + batch_row0 + lane, acc);
+                    if (plain_y) gstore<float>(y + batch_row0 + lane, acc);
                     if (add_dst) gstore<float>(add_dst + batch_row0 + lane, acc + resid);
                 }
                 batch_row0 = row + 1;

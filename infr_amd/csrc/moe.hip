@@ -697,7 +697,7 @@ __global__ __launch_bounds__(1024) void moe_down_f32_kernel(
     if (owner) {
         const int o = (st0 + own_s) * rps + own_seg;
         if (o < ne) {
-            out[o] = acc;
+            if (out != add_dst) out[o] = acc;  // an Add in place on this op's dst stores the sum only
             if (add_dst) add_dst[o] = acc + add_b[o];
         }
     }
@@ -850,7 +850,7 @@ __global__ __launch_bounds__(256) void moe_accumulate_kernel(const float* __rest
     float acc = 0.0f;
     for (int k = 0; k < n_used; ++k)
         acc += wts[r * n_used + k] * yp[(r * n_used + k) * ne + o];
-    out[i] = acc;
+    if (out != add_dst) out[i] = acc;  // an Add in place on this op's dst stores the sum only
     if (add_dst) add_dst[i] = acc + add_b[i];
 }
 

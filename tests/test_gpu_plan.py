@@ -100,6 +100,34 @@ def test_in_place_chain_is_ordered(be):
     assert np.array_equal(bits(be.download(yb, np.empty(in_f, np.float32))), bits(y2))
 
 
+@pytest.mark.parametrize("dtype", [DType.Q4K, DType.Q8_0])
+@pytest.mark.parametrize("y_first", [True, False])
+def test_add_in_place_on_the_linear_output_is_absorbed(be, dtype, y_first):
+    # y = W x; y = y + r: the absorbed Add's dst is the Linear's own dst, which then holds the sum
+    from infr_amd import Add
+    n = 1024
+    g, binds = Graph(), Bindings()
+    xid, rid = (g.input(TensorDesc((1, n), DType.F32)) for _ in range(2))
+    yid = g.output(TensorDesc((1, n), DType.F32))
+    wid = g.weight(TensorDesc((n, n), dtype))
+    x, r = synth_normal_f32(0x71, n), synth_normal_f32(0x72, n)
+    w = synth_weight(dtype, 0x73, n, n, sigma=0.03)
+    yb = be.alloc(n * 4)
+    binds.bind(xid, be.upload_new(x)).bind(rid, be.upload_new(r)).bind(yid, yb).bind(wid, be.upload_new(w))
+    g.push(Linear(xid, wid, yid, 1, n, n))
+    g.push(Add(yid, rid, yid, n) if y_first else Add(rid, yid, yid, n))
+    plan = be.compile(g)
+    for _ in range(2):
+        be.execute(plan, binds)
+        got = be.download(yb, np.empty(n, np.float32))
+        want = orc.linear(dtype, w, x, 1, n, n).ravel() + r
+        assert plan.launches() == 1
+        if dtype == DType.Q4K:
+            assert np.array_equal(bits(got), bits(want))
+        else:
+            assert _rel(got, want) < 1e-5
+
+
 def test_one_row_linear_in_place_inside_a_plan(be):
     # y = A y next to a sibling z = B y that reads the old y first (program order), then y = C y
     # again: the in-place ops must neither join a group nor overtake the reader.

@@ -1,0 +1,205 @@
+"""Random op programs over a small pool of activation tensors, scheduled as ONE plan (levels,
+grouped launches, producers and residual adds absorbed into the decode GEMVs and the MoE kernels)
+against the same ops executed one plan per op in program order.
+
+The pool is small on purpose: tensors are reused, overwritten, read after being overwritten and
+written in place, which is what the scheduler's hazard rules exist for (a runner reuses its norm /
+gate / act scratch tensors from layer to layer, crates/infr-core/src/graph.rs:10-14). Every tensor
+of the pool is compared, not only the last one written.
+
+Bar: rel-L2 <= 2e-3 per tensor. The absorbed RmsNorm sums its squares over more waves than the
+stand-alone kernel and the absorbed gated activation uses the hardware exponential, so the two
+executions differ in the last bit of some activations, and a last-bit change can move an int8 code
+of the next quantization (one code of 256 is ~5e-4 of an output). A dependency that is broken
+shows as a difference of order one: a stale or half-written operand.
+"""
+import zlib
+
+import numpy as np
+import pytest
+
+from infr_amd import (Add, Bindings, DType, GatedAct, Graph, Linear, MoeFfn, RmsNorm, RmsNormAdd, TensorDesc,
+                      synth_normal_f32, synth_weight)
+
+pytestmark = pytest.mark.gpu
+
+WIDTHS = (256, 512, 1024)
+PER_WIDTH = 3
+LINEAR_DTYPES = (DType.Q4K, DType.Q4K, DType.Q6K, DType.Q8_0, DType.Q5_0, DType.Q2_0)
+MOE = dict(ne=512, n_expert=8, n_used=2, nff=256)
+
+
+def stable_seed(key):
+    return zlib.crc32(repr(key).encode()) & 0xFFFF
+
+
+def random_program(rng, n_ops):
+    """Op specs over pool tensors named (width, index); weights are named by what they multiply.
+    Half of the draws are single ops over random tensors, half are the sequences the scheduler
+    absorbs (a norm or a gated activation in front of Linears, an Add behind a Linear or a MoeFfn,
+    a norm in front of a MoeFfn), their tensors drawn from the same small pool so that they
+    collide with each other and with the ops around them."""
+    prog = []
+    t = lambda w: (w, int(rng.integers(PER_WIDTH)))
+    width = lambda: int(rng.choice(WIDTHS))
+    dtype = lambda: LINEAR_DTYPES[rng.integers(len(LINEAR_DTYPES))]
+    linear = lambda x, dst: ("linear", x, dst, dtype(), int(rng.integers(4)))
+
+    def add_behind(y):
+        r, d = t(y[0]), (y, t(y[0]))[rng.integers(2)]
+        if rng.integers(3) == 0:
+            d = r                                   # the residual stream updated in place
+        return ("add", y, r, d) if rng.integers(2) else ("add", r, y, d)
+
+    while len(prog) < n_ops:
+        kind = rng.choice(["linear", "norm", "add", "gated", "norm_add", "moe",
+                           "norm>linears", "gated>linear", "linear>add", "moe>add", "norm>moe>add", "layer"])
+        if kind == "linear":
+            prog.append(linear(t(width()), t(width())))          # equal widths may pick dst == x
+        elif kind in ("norm", "norm_add"):
+            w = width()
+            prog.append((kind, t(w), t(w), int(rng.integers(2))))
+        elif kind == "add":
+            w = width()
+            prog.append(("add", t(w), t(w), t(w)))
+        elif kind == "gated":
+            w = width()
+            prog.append(("gated", t(w), t(w), t(w)))
+        elif kind == "moe":
+            prog.append(("moe", t(MOE["ne"]), t(MOE["ne"]), int(rng.integers(2))))
+        elif kind == "norm>linears":
+            w = width()
+            h = t(w)
+            prog.append(("norm", t(w), h, int(rng.integers(2))))
+            for _ in range(int(rng.integers(1, 4))):
+                prog.append(linear(h, t(width())))
+        elif kind == "gated>linear":
+            w = width()
+            a = t(w)
+            prog.append(("gated", t(w), t(w), a))
+            prog.append(linear(a, t(width())))
+        elif kind == "linear>add":
+            y = t(width())
+            prog.append(linear(t(width()), y))
+            prog.append(add_behind(y))
+        elif kind == "moe>add":
+            y = t(MOE["ne"])
+            prog.append(("moe", t(MOE["ne"]), y, int(rng.integers(2))))
+            prog.append(add_behind(y))
+        elif kind == "norm>moe>add":
+            h, y = t(MOE["ne"]), t(MOE["ne"])
+            prog.append(("norm", t(MOE["ne"]), h, int(rng.integers(2))))
+            prog.append(("moe", h, y, int(rng.integers(2))))
+            prog.append(add_behind(y))
+        else:  # norm -> two projections -> gated -> down -> residual add
+            w, ff = width(), width()
+            x, h, g, u, a, y = t(w), t(w), t(ff), t(ff), t(ff), t(w)
+            prog += [("norm", x, h, 0), linear(h, g), linear(h, u), ("gated", g, u, a), linear(a, y),
+                     ("add", y, x, x)]
+    return prog
+
+
+class Pool:
+    """Device buffers of the pool and of every weight a program names, shared by all its graphs."""
+
+    def __init__(self, be, m, prog, seed):
+        self.be, self.m = be, m
+        self.act = {(w, i): be.alloc(m * w * 4) for w in WIDTHS for i in range(PER_WIDTH)}
+        self.init = {k: synth_normal_f32(seed * 100 + 7 * k[0] + k[1], m * k[0]) for k in self.act}
+        self.weights = {}
+        for op in prog:
+            if op[0] == "linear":
+                _, x, dst, dt, which = op
+                key = ("lin", dst[0], x[0], int(dt), which)
+                if key not in self.weights:
+                    data = synth_weight(dt, stable_seed(key), dst[0], x[0], sigma=0.03)
+                    self.weights[key] = (TensorDesc((dst[0], x[0]), dt), be.upload_new(data))
+            elif op[0] in ("norm", "norm_add"):
+                key = ("nw", op[1][0], op[3])
+                if key not in self.weights:
+                    data = synth_normal_f32(stable_seed(key), key[1], mean=1.0, sigma=0.1)
+                    self.weights[key] = (TensorDesc((key[1],), DType.F32), be.upload_new(data))
+            elif op[0] == "moe":
+                ne, n_e, nff = MOE["ne"], MOE["n_expert"], MOE["nff"]
+                for part, desc, data in (
+                        ("router", TensorDesc((n_e, ne), DType.F32), lambda s: synth_normal_f32(s, n_e * ne, sigma=0.05)),
+                        ("gate", TensorDesc((n_e, nff, ne), DType.Q4K), lambda s: synth_weight(DType.Q4K, s, n_e * nff, ne, 0.05)),
+                        ("up", TensorDesc((n_e, nff, ne), DType.Q4K), lambda s: synth_weight(DType.Q4K, s, n_e * nff, ne, 0.05)),
+                        ("down", TensorDesc((n_e, ne, nff), DType.Q6K), lambda s: synth_weight(DType.Q6K, s, n_e * ne, nff, 0.05))):
+                    key = ("moe", part, op[3])
+                    if key not in self.weights:
+                        self.weights[key] = (desc, be.upload_new(data(stable_seed(key))))
+
+    def reset(self):
+        for k, buf in self.act.items():
+            self.be.upload(buf, self.init[k])
+
+    def snapshot(self):
+        return {k: self.be.download(buf, np.empty(self.m * k[0], np.float32)) for k, buf in self.act.items()}
+
+    def graph(self, ops):
+        """One graph holding `ops`, every pool tensor and named weight declared and bound."""
+        g, binds, m = Graph(), Bindings(), self.m
+        aid = {}
+        for k, buf in self.act.items():
+            aid[k] = g.output(TensorDesc((m, k[0]), DType.F32))
+            binds.bind(aid[k], buf)
+        wid = {}
+        for key, (desc, buf) in self.weights.items():
+            wid[key] = g.weight(desc)
+            binds.bind(wid[key], buf)
+        for op in ops:
+            if op[0] == "linear":
+                _, x, dst, dt, which = op
+                g.push(Linear(aid[x], wid[("lin", dst[0], x[0], int(dt), which)], aid[dst], m, x[0], dst[0]))
+            elif op[0] == "norm":
+                g.push(RmsNorm(aid[op[1]], wid[("nw", op[1][0], op[3])], aid[op[2]], m, op[1][0], 1e-6))
+            elif op[0] == "norm_add":
+                g.push(RmsNormAdd(aid[op[1]], wid[("nw", op[1][0], op[3])], aid[op[2]], m, op[1][0], 1e-6))
+            elif op[0] == "add":
+                g.push(Add(aid[op[1]], aid[op[2]], aid[op[3]], m * op[1][0]))
+            elif op[0] == "gated":
+                g.push(GatedAct(aid[op[1]], aid[op[2]], aid[op[3]], m, op[1][0]))
+            else:
+                _, x, dst, which = op
+                w = lambda part: wid[("moe", part, which)]
+                g.push(MoeFfn(aid[x], aid[x], w("router"), w("gate"), w("up"), w("down"), aid[dst],
+                              MOE["ne"], MOE["n_expert"], MOE["n_used"], MOE["nff"]))
+        return g, binds
+
+
+REL_L2 = 2e-3
+
+
+def rel_l2(got, want):
+    g, w = got.astype(np.float64), want.astype(np.float64)
+    return np.linalg.norm(g - w) / max(np.linalg.norm(w), 1e-30)
+
+
+def describe(prog):
+    return "\n".join(f"  {i:2d}: {op}" for i, op in enumerate(prog))
+
+
+@pytest.mark.parametrize("m,seed", [(1, s) for s in range(16)] + [(3, s) for s in range(100, 106)] +
+                         [(8, s) for s in range(200, 203)])
+def test_scheduled_plan_equals_the_ops_run_one_by_one(be, m, seed):
+    rng = np.random.default_rng(seed)
+    prog = random_program(rng, int(rng.integers(6, 15)))
+    pool = Pool(be, m, prog, seed)
+    # program order, one plan per op: nothing to group, absorb or reorder
+    pool.reset()
+    for op in prog:
+        g, binds = pool.graph([op])
+        be.execute(be.compile(g), binds)
+    want = pool.snapshot()
+    assert all(np.isfinite(v).all() for v in want.values()), "program overflowed: not a useful case"
+    g, binds = pool.graph(prog)
+    plan = be.compile(g)
+    for rep in range(2):                                    # the second execute replays the recording
+        pool.reset()
+        be.execute(plan, binds)
+        got = pool.snapshot()
+        for k in want:
+            assert rel_l2(got[k], want[k]) <= REL_L2, (
+                f"tensor {k} off by {rel_l2(got[k], want[k]):.2e} on execute {rep} (m = {m}, seed = {seed}, "
+                f"{plan.launches()} launches for {len(prog)} ops):\n{describe(prog)}")
