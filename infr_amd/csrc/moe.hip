@@ -130,7 +130,7 @@ __device__ __forceinline__ void moe_select_block(const float* __restrict__ l, Se
         }
     }
     __syncthreads();
-    if (tid < n_used) {
+    if (out_idx && tid < n_used) {  // (without outputs the caller reads s.top_e)
         float wsum = 0.0f;  // summed in rank order, as the CPU sums its selection
         for (int k = 0; k < n_used; ++k) wsum += s.top_p[k];
         wsum = __builtin_fmaxf(wsum, 1e-20f);
@@ -172,9 +172,11 @@ __global__ __launch_bounds__(256) void moe_select_kernel(const float* __restrict
 // coalesced 16-byte loads, and eight lanes per (expert, token) pair - one accumulator each - run
 // the chains from LDS, carrying them across chunks. A row sits in LDS accumulator-major (element i
 // at [i % 8][i / 8]), so a lane reads four steps of its chain with one 16-byte access.
-// With a single row (tickets != nullptr) the last workgroup to finish - a ticket counter, left
-// at zero again - runs the selection too, which saves a launch; eight experts per workgroup keep
-// that to a handful of tickets (atomics on one address complete one after another, ~65 ns each).
+// A single row of banks in the factored kernels' formats leaves only logits here (one expert per
+// workgroup; the gate / up kernel selects in its prologue). For any other single row (tickets !=
+// nullptr) the last workgroup to finish - a ticket counter, left at zero again - runs the
+// selection too, which saves a launch; eight experts per workgroup keep that to a handful of
+// tickets (atomics on one address complete one after another, ~65 ns each).
 // ne % 32 == 0 is required.
 constexpr int kRouterPairs = 32, kRouterChunk = 512;
 // floats between two staged rows of kc elements: eight accumulator rows of kc / 8 + 4
@@ -605,15 +607,17 @@ __device__ __forceinline__ float seg_sum(float v, int seg_base, int quads) {
     return s;
 }
 
-// gate/up at one token: act[slot][o] = silu(gate_e[o] . x) * (up_e[o] . x), e = ids[slot].
+// gate/up at one token: act[slot][o] = silu(gate_e[o] . x) * (up_e[o] . x), e = the expert of rank `slot`.
 // A wave takes SPW consecutive row steps and requests all their rows before it computes the
 // first: at one token the kernel is a few memory round trips deep, so every request it can make
 // up front is a round trip less.
 template <typename P, int SPW>
 __global__ __launch_bounds__(256) void moe_gate_up_f32_kernel(
     const uint8_t* __restrict__ gate, const uint8_t* __restrict__ up, size_t gate_stride,
-    size_t up_stride, const int32_t* __restrict__ ids, const float* __restrict__ x,
+    size_t up_stride, const float* __restrict__ logits, int n_expert, int n_used, float scale,
+    int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, const float* __restrict__ x,
     float* __restrict__ act, int ne, int nff) {
+    __shared__ __attribute__((aligned(16))) SelectLds sel;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int S = ne / 64, rps = 64 / S;  // lanes per weight row, rows per wave step
     const int seg = lane / S, u = lane % S;
@@ -621,8 +625,17 @@ __global__ __launch_bounds__(256) void moe_gate_up_f32_kernel(
     const int slot = blockIdx.y;
     const int steps_total = (nff + rps - 1) / rps;
     const int st0 = (blockIdx.x * 4 + wave) * SPW;
+    // the activation does not depend on the routing: requested first, it arrives under the selection
+    typename P::X xa;
+    P::load_x(xa, x, u, lane_ok);
+    // Every workgroup selects for itself from the router's logits (a few hundred bytes and a few
+    // barriers) instead of waiting for a selection kernel in between; the first one also leaves
+    // the ranked experts and weights for the down kernel.
+    const bool first = blockIdx.x == 0 && blockIdx.y == 0;
+    moe_select_block(logits, sel, n_expert, n_used, scale, threadIdx.x, first ? sel_idx : nullptr,
+                     first ? sel_w : nullptr);
     if (st0 >= steps_total) return;
-    const int e = ids[slot];
+    const int e = sel.top_e[slot];
     const size_t bpr = (size_t)(ne / 256) * P::kBlockBytes;
     const uint8_t* gw = gate + (size_t)e * gate_stride;
     const uint8_t* uw = up + (size_t)e * up_stride;
@@ -634,8 +647,6 @@ __global__ __launch_bounds__(256) void moe_gate_up_f32_kernel(
         P::load_row(g[i], gw + (size_t)(ok ? o : 0) * bpr, u, ok);
         P::load_row(up_r[i], uw + (size_t)(ok ? o : 0) * bpr, u, ok);
     }
-    typename P::X xa;
-    P::load_x(xa, x, u, lane_ok);
 #pragma unroll
     for (int i = 0; i < SPW; ++i) {
         const int o = (st0 + i) * rps + seg;
@@ -1023,15 +1034,23 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     int32_t* tile_slot0 = (int32_t*)take(max_tiles * 4);
     int32_t* tile_count = (int32_t*)take(max_tiles * 4);
 
-    // eight experts per workgroup at a single row (few tickets), four once rows fill the pairs; whole
-    // rows in one chunk when they fit the LDS a workgroup may have, else kRouterChunk columns at a time
+    // One row in the formats of the factored kernels: the gate / up kernel selects in its own
+    // prologue, so the router only leaves the logits - one expert per workgroup, nothing to wait for.
+    auto raw_ok = [](int dt) { return dt == 12 || dt == 13 || dt == 14 || dt == 8; };
+    const bool fast1 = s.rows == 1 && raw_ok(s.gate_dtype) && s.up_dtype == s.gate_dtype && raw_ok(s.down_dtype) &&
+                       s.ne <= 4096 && s.n_ff <= 4096;
+    // Otherwise eight experts per workgroup at a single row (few tickets), four once rows fill the
+    // pairs; whole rows in one chunk when they fit the LDS a workgroup may have, else kRouterChunk
+    // columns at a time
     constexpr size_t kRouterLdsMax = 144 * 1024;
-    int epw = s.rows == 1 ? 8 : 4;
+    int epw = fast1 ? 1 : (s.rows == 1 ? 8 : 4);
     while (epw > 1 && (size_t)(epw + 1) * router_row_floats(s.ne) * sizeof(float) > kRouterLdsMax) epw /= 2;
     const int tpw = kRouterPairs / epw;
     const int n_t = std::min(s.rows, tpw);
-    const int kc = (size_t)(epw + n_t) * router_row_floats(s.ne) * sizeof(float) <= (s.rows == 1 ? kRouterLdsMax : 64 * 1024)
-                       ? s.ne : kRouterChunk;
+    // (whole rows also for a few rows, while the grid is a single round of one workgroup per compute unit)
+    const bool one_round = (size_t)((s.n_expert + epw - 1) / epw) * ((s.rows + tpw - 1) / tpw) <= 256;
+    const bool whole_rows = (size_t)(epw + n_t) * router_row_floats(s.ne) * sizeof(float) <= (one_round ? kRouterLdsMax : 64 * 1024);
+    const int kc = whole_rows ? s.ne : kRouterChunk;
     const size_t router_lds = (size_t)(epw + n_t) * router_row_floats(kc) * sizeof(float);
     if (router_lds > 64 * 1024)
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_router_kernel<24>),
@@ -1042,8 +1061,14 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
                            dim3(kRtThreads), 0, stream, b.router, b.router_x, logits, s.ne, s.n_expert, s.rows);
     else if (s.rows == 1)
         hipLaunchKernelGGL(moe_router_kernel<24>, dim3((unsigned)((s.n_expert + epw - 1) / epw), 1), dim3(256), router_lds,
-                           stream, b.router, b.router_x, logits, tickets, sel_idx, sel_w, s.ne, s.n_expert, s.rows,
-                           s.n_used, s.scale, kc, epw, b.norm_w, b.norm_dst, b.norm_eps);
+                           stream, b.router, b.router_x, logits, fast1 ? (int*)nullptr : tickets, sel_idx, sel_w, s.ne,
+                           s.n_expert, s.rows, s.n_used, s.scale, kc, epw, b.norm_w, b.norm_dst, b.norm_eps);
+    else if (whole_rows && router_lds > 64 * 1024)
+        hipLaunchKernelGGL(moe_router_kernel<24>,
+                           dim3((unsigned)((s.n_expert + epw - 1) / epw), (unsigned)((s.rows + tpw - 1) / tpw)),
+                           dim3(256), router_lds, stream, b.router, b.router_x, logits, (int*)nullptr, sel_idx, sel_w,
+                           s.ne, s.n_expert, s.rows, s.n_used, s.scale, kc, epw, (const float*)nullptr, (float*)nullptr,
+                           0.0f);
     else
         hipLaunchKernelGGL(moe_router_kernel<8>,
                            dim3((unsigned)((s.n_expert + epw - 1) / epw), (unsigned)((s.rows + tpw - 1) / tpw)),
@@ -1087,14 +1112,15 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
         hipLaunchKernelGGL(moe_select_kernel, dim3((unsigned)s.rows), dim3(256), 0, stream, logits, sel_idx,
                            sel_w, s.n_expert, s.n_used, s.scale, quant_in_select ? b.x : (const float*)nullptr,
                            s.ne, aq.qs, aq.d, aq.bsums, aq.bsums16);
-    if (b.sel_idx) (void)hipMemcpyAsync(b.sel_idx, sel_idx, pairs * 4, hipMemcpyDeviceToDevice, stream);
-    if (b.sel_w) (void)hipMemcpyAsync(b.sel_w, sel_w, pairs * 4, hipMemcpyDeviceToDevice, stream);
+    auto export_selection = [&] {
+        if (b.sel_idx) (void)hipMemcpyAsync(b.sel_idx, sel_idx, pairs * 4, hipMemcpyDeviceToDevice, stream);
+        if (b.sel_w) (void)hipMemcpyAsync(b.sel_w, sel_w, pairs * 4, hipMemcpyDeviceToDevice, stream);
+    };
+    if (!fast1) export_selection();
 
     if (s.rows == 1) {
         // ActsKind::Raw for every bank (lib.rs:2359: int8_ok = rows >= 2)
-        auto raw_ok = [](int dt) { return dt == 12 || dt == 13 || dt == 14 || dt == 8; };
-        if (!raw_ok(s.gate_dtype) || s.up_dtype != s.gate_dtype || !raw_ok(s.down_dtype) || s.ne > 4096 ||
-            s.n_ff > 4096) {
+        if (!fast1) {
             // other formats, mixed gate / up formats, rows too long for the factored kernels'
             // registers: the decode-and-dot form of every stage
             launch_raw(s.gate_dtype, b.gate, b.gate_stride, gbpr, b.x, s.n_used, s.ne, gbuf, s.n_ff);
@@ -1115,7 +1141,7 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
         const dim3 grid_g((unsigned)((steps_g + 4 * spw - 1) / (4 * spw)), (unsigned)s.n_used);
 #define INFR_GATE_UP_N(P, N)                                                                                  \
     hipLaunchKernelGGL((moe_gate_up_f32_kernel<P, N>), grid_g, dim3(256), 0, stream, b.gate, b.up, b.gate_stride, \
-                       b.up_stride, sel_idx, b.x, gbuf, s.ne, s.n_ff)
+                       b.up_stride, logits, s.n_expert, s.n_used, s.scale, sel_idx, sel_w, b.x, gbuf, s.ne, s.n_ff)
 #define INFR_GATE_UP(P)                 \
     switch (spw) {                      \
     case 1: INFR_GATE_UP_N(P, 1); break; \
@@ -1129,6 +1155,7 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
         else INFR_GATE_UP(RawQ8_0)
 #undef INFR_GATE_UP
 #undef INFR_GATE_UP_N
+        export_selection();
         const int rps_d = 64 / (s.n_ff / 64);
         const int steps_d = (s.ne + rps_d - 1) / rps_d;
         const int spw_d = std::min(kDownMaxSteps, steps_per_wave(steps_d * s.n_used));
