@@ -921,7 +921,7 @@ size_t infr_hip_plan_launches(const infr_hip_plan_t* plan) {
     size_t n = 0;
     for (const auto& st : plan->steps) {
         if (st.op < 0) n += st.m > 1 ? 2 : 1;                              // grouped launch (+ grouped quantize)
-        else if (plan->ops[st.op].kind == INFR_OP_MOE_FFN) n += plan->ops[st.op].moe.rows == 1 ? 3 : 6;
+        else if (plan->ops[st.op].kind == INFR_OP_MOE_FFN) n += plan->ops[st.op].moe.rows == 1 ? 3 : 4;
         else if (is_elementwise(plan->ops[st.op].kind) || plan->ops[st.op].kind == INFR_OP_EMBED_GATHER) n += 1;
         else n += 2;                                                       // quantize + GEMM
     }

@@ -219,11 +219,13 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
 // lane. Per-(row, block) terms are the same code as the unfolded loop and are added per row in
 // ascending block order, so every output equals the unfolded result bit for bit.
 // `osum` is this wave's OrderedSum<1> scratch.
-template <typename F>
+// Y_GLOBAL = false: `y` is not device memory (a caller's LDS row); `first`, when given, is the
+// step at row0, requested by the caller ahead of its own prologue.
+template <typename F, bool Y_GLOBAL = true>
 __device__ __forceinline__ void gemv_rows_folded(const uint8_t* __restrict__ w, size_t bpr, int nb,
                                                  const typename F::Acts& acts,
                                                  float* __restrict__ y, int row0, int row_end,
-                                                 int lane, float* osum) {
+                                                 int lane, float* osum, const typename F::Row* first = nullptr) {
     static_assert(F::kOrdered, "folded rows exist for the ordered 16-block formats");
     constexpr int LS = OrderedSum<1>::kRowStride;
     const int q = lane >> 2, rps = 16 / nb;
@@ -232,7 +234,8 @@ __device__ __forceinline__ void gemv_rows_folded(const uint8_t* __restrict__ w, 
     // columns nb..15 of a scratch row are never written: zero them once so the flush can add all 16
     for (int i = lane; i < OrderedSum<1>::kFloatsPerWave; i += 64) osum[i] = 0.0f;
     typename F::Row cur;
-    F::load_row(cur, w + (size_t)row0 * bpr, 0, lane, lane_ok && row0 + rq < row_end);
+    if (first) cur = *first;
+    else F::load_row(cur, w + (size_t)row0 * bpr, 0, lane, lane_ok && row0 + rq < row_end);
     int in_batch = 0, batch_row0 = row0;
     for (int row = row0; row < row_end; row += rps) {
         const int nr = row + rps;
@@ -255,7 +258,8 @@ __device__ __forceinline__ void gemv_rows_folded(const uint8_t* __restrict__ w, 
                     acc += v.z;
                     acc += v.w;
                 }
-                gstore<float>(y + batch_row0 + lane, acc);
+                if (Y_GLOBAL) gstore<float>(y + batch_row0 + lane, acc);
+                else y[batch_row0 + lane] = acc;
             }
             batch_row0 = nr;
             in_batch = 0;

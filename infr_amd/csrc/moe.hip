@@ -188,7 +188,7 @@ template <int NL>
 __global__ __launch_bounds__(256) void moe_router_kernel(
     const float* __restrict__ router, const float* __restrict__ rx, float* __restrict__ logits,
     int* __restrict__ tickets, int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, int ne,
-    int n_expert, int rows, int n_used, float scale, int kc, int epw, const float* __restrict__ norm_w,
+    int n_expert, int rows, int n_used, float scale, int kc, int epw, int tpw, const float* __restrict__ norm_w,
     float* __restrict__ norm_dst, float norm_eps) {
     extern __shared__ __attribute__((aligned(16))) float rl[];  // [epw] rows | [32 / epw] rows
     __shared__ __attribute__((aligned(16))) SelectLds sel;
@@ -207,7 +207,6 @@ __global__ __launch_bounds__(256) void moe_router_kernel(
         const float ss = ((sel.red[0] + sel.red[1]) + (sel.red[2] + sel.red[3])) / (float)ne;
         nscale = 1.0f / sqrtf(ss + norm_eps);
     }
-    const int tpw = kRouterPairs / epw;
     const int e0 = blockIdx.x * epw, t0 = blockIdx.y * tpw;
     const int n_e = min(epw, n_expert - e0), n_t = min(tpw, rows - t0);
     const int ld = router_row_floats(kc), la = kc / 8 + 4;  // row and accumulator-row strides
@@ -810,6 +809,78 @@ __global__ __launch_bounds__(256) void moe_act_quant_kernel(const float* __restr
     quantize_chunk<PER32>(a, true, lane, chunk, qs, d, bsums, PER32 ? nullptr : bsums16);
 }
 
+// A few rows, short expert rows (n_ff <= 2048) of a 16-block format: activation, down projection
+// and the weighted sum over a token's experts in one launch. A workgroup is a token and a tile of
+// output rows; wave k takes the token's k-th expert: it requests its first weight step, builds
+// act = silu(g) * u of its pair and quantizes it per 256 into its own LDS (the stand-alone kernel's
+// arithmetic), runs the folded decode body into an LDS row, and after a barrier thread o adds
+// w_k * y_k[o] over the experts in rank order with a separate multiply and add - the values and
+// the order of moe_act_quant_kernel, the id-gathered GEMV and moe_accumulate_kernel, without the
+// two launches in between and without the per-pair outputs going through memory.
+// LDS per wave: qs[nff] | d[nff / 256, padded to 4] | bsums[nff / 32] | bsums16[nff / 16] | ordered-sum scratch | y[rows_per_wg]
+__host__ __device__ constexpr size_t moe_down_fused_y_offset(int nff) {
+    return (size_t)nff + (size_t)((nff / 256 + 3) / 4 * 4 + nff / 32 + nff / 16 + OrderedSum<1>::kFloatsPerWave) * 4;
+}
+__host__ __device__ constexpr size_t moe_down_fused_wave_bytes(int nff, int rows_per_wg) {
+    return (moe_down_fused_y_offset(nff) + (size_t)rows_per_wg * 4 + 15) / 16 * 16;
+}
+template <typename F>
+__global__ __launch_bounds__(1024) void moe_down_fused_kernel(
+    const uint8_t* __restrict__ bank, size_t expert_stride, size_t bpr, const int32_t* __restrict__ ids,
+    const float* __restrict__ wts, const float* __restrict__ g, const float* __restrict__ u,
+    float* __restrict__ out, const float* add_b, float* add_dst, int nff, int ne, int n_used, int rows_per_wg) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t dlds[];
+    const int lane = threadIdx.x & 63, k = threadIdx.x >> 6;
+    const int token = blockIdx.y, pair = token * n_used + k;
+    const int row0 = blockIdx.x * rows_per_wg, row_end = min(row0 + rows_per_wg, ne);
+    const int nb = nff / 256;
+    const size_t wave_bytes = moe_down_fused_wave_bytes(nff, rows_per_wg);
+    uint8_t* mine = dlds + (size_t)k * wave_bytes;
+    int8_t* qs = reinterpret_cast<int8_t*>(mine);
+    float* d = reinterpret_cast<float*>(mine + nff);
+    int32_t* bsums = reinterpret_cast<int32_t*>(d + (nb + 3) / 4 * 4);
+    int32_t* bsums16 = bsums + nff / 32;
+    float* osum = reinterpret_cast<float*>(bsums16 + nff / 16);
+    const size_t y_off = moe_down_fused_y_offset(nff);
+    float* yk = reinterpret_cast<float*>(mine + y_off);
+    const uint8_t* w = bank + (size_t)ids[pair] * expert_stride;
+    const int q = lane >> 2, rq = q / nb;
+    typename F::Row first;
+    F::load_row(first, w + (size_t)row0 * bpr, 0, lane, rq < 16 / nb && row0 + rq < row_end);
+    for (int c = 0; c < nb; ++c) {
+        const v4f gv = *reinterpret_cast<const v4f*>(g + (size_t)pair * nff + c * 256 + lane * 4);
+        const v4f uv = *reinterpret_cast<const v4f*>(u + (size_t)pair * nff + c * 256 + lane * 4);
+        v4f a;
+        a.x = gv.x / (1.0f + expf(-gv.x)) * uv.x;
+        a.y = gv.y / (1.0f + expf(-gv.y)) * uv.y;
+        a.z = gv.z / (1.0f + expf(-gv.z)) * uv.z;
+        a.w = gv.w / (1.0f + expf(-gv.w)) * uv.w;
+        quantize_chunk<false>(a, true, lane, (size_t)c, qs, d, bsums, bsums16);
+    }
+    __syncthreads();
+    const int shift = q - q % nb;  // load_acts addresses block q; this lane wants block q % nb
+    ActPtrs a;
+    a.qs = qs - (ptrdiff_t)shift * 256;
+    a.d = d - shift;
+    a.bsums = bsums - shift * 8;
+    a.bsums16 = bsums16 - shift * 16;
+    typename F::Acts acts;
+    F::load_acts(acts, a, 0, lane, q / nb < 16 / nb);
+    gemv_rows_folded<F, false>(w, bpr, nb, acts, yk - row0, row0, row_end, lane, osum, &first);
+    __syncthreads();
+    const int o = (int)threadIdx.x;
+    if (o < row_end - row0) {
+        float acc = 0.0f;
+        for (int j = 0; j < n_used; ++j) {
+            const float* yj = reinterpret_cast<const float*>(dlds + (size_t)j * wave_bytes + y_off);
+            acc += wts[token * n_used + j] * yj[o];
+        }
+        const size_t i = (size_t)token * ne + row0 + o;
+        if (out != add_dst) out[i] = acc;  // an Add in place on this op's dst stores the sum only
+        if (add_dst) add_dst[i] = acc + add_b[i];
+    }
+}
+
 // The same activation kept in f32 (in place over g) for a down bank that multiplies raw rows.
 __global__ __launch_bounds__(256) void moe_act_f32_kernel(float* __restrict__ g, const float* __restrict__ u,
                                                           size_t n_elems) {
@@ -969,6 +1040,37 @@ static bool launch_gemv_id(int dtype, const uint8_t* bank, size_t expert_stride,
     }
 }
 
+// Activation + down + accumulate in one launch (moe_down_fused_kernel) where that form exists:
+// a 16-block bank format, whole expert rows of at most 2048, up to 16 experts per token, 64 KB of LDS.
+template <typename F>
+static bool launch_moe_down_fused_fmt(const uint8_t* bank, size_t stride, size_t bpr, const int32_t* ids,
+                                      const float* wts, const float* g, const float* u, float* out,
+                                      const float* add_b, float* add_dst, int nff, int ne, int n_used, int rows,
+                                      hipStream_t stream) {
+    const int rps = 16 / (nff / 256);
+    int wave_steps = 8;  // rows per workgroup: enough waves in all (as the id-gathered launches size theirs)
+    while (wave_steps > 1 && (size_t)((ne + rps * wave_steps - 1) / (rps * wave_steps)) * rows * n_used < 4096)
+        wave_steps /= 2;
+    const int rows_per_wg = rps * wave_steps;
+    const size_t lds = moe_down_fused_wave_bytes(nff, rows_per_wg) * n_used;
+    if (lds > 64 * 1024) return false;
+    hipLaunchKernelGGL((moe_down_fused_kernel<F>), dim3((unsigned)((ne + rows_per_wg - 1) / rows_per_wg), (unsigned)rows),
+                       dim3((unsigned)(64 * n_used)), lds, stream, bank, stride, bpr, ids, wts, g, u, out, add_b, add_dst,
+                       nff, ne, n_used, rows_per_wg);
+    return true;
+}
+static bool launch_moe_down_fused(int dtype, const uint8_t* bank, size_t stride, size_t bpr, const int32_t* ids,
+                                  const float* wts, const float* g, const float* u, float* out, const float* add_b,
+                                  float* add_dst, int nff, int ne, int n_used, int rows, hipStream_t stream) {
+    if (nff > 2048 || nff % 256 != 0 || n_used > 16 || rows > 65535) return false;
+    switch (dtype) {
+    case 12: return launch_moe_down_fused_fmt<FmtQ4K>(bank, stride, bpr, ids, wts, g, u, out, add_b, add_dst, nff, ne, n_used, rows, stream);
+    case 13: return launch_moe_down_fused_fmt<FmtQ5K>(bank, stride, bpr, ids, wts, g, u, out, add_b, add_dst, nff, ne, n_used, rows, stream);
+    case 14: return launch_moe_down_fused_fmt<FmtQ6K>(bank, stride, bpr, ids, wts, g, u, out, add_b, add_dst, nff, ne, n_used, rows, stream);
+    default: return false;
+    }
+}
+
 size_t moe_workspace_bytes(const MoeShape& s) {
     const size_t pairs = (size_t)s.rows * s.n_used;
     size_t n = 0;
@@ -1044,8 +1146,16 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     // columns at a time
     constexpr size_t kRouterLdsMax = 144 * 1024;
     int epw = fast1 ? 1 : (s.rows == 1 ? 8 : 4);
+    int tpw = kRouterPairs / epw;
+    if (s.rows > 1) {
+        // a few rows: fewer (expert, token) pairs per workgroup, so that about 256 workgroups share
+        // the staging (16 tokens x 128 experts: 2 x 4 pairs each instead of 4 x 8 on 64 workgroups)
+        int per_wg = 1;
+        while (per_wg < kRouterPairs && (size_t)s.n_expert * s.rows > (size_t)256 * per_wg) per_wg *= 2;
+        epw = per_wg >= 16 ? 4 : (per_wg >= 4 ? 2 : 1);
+        tpw = per_wg / epw;
+    }
     while (epw > 1 && (size_t)(epw + 1) * router_row_floats(s.ne) * sizeof(float) > kRouterLdsMax) epw /= 2;
-    const int tpw = kRouterPairs / epw;
     const int n_t = std::min(s.rows, tpw);
     // (whole rows also for a few rows, while the grid is a single round of one workgroup per compute unit)
     const bool one_round = (size_t)((s.n_expert + epw - 1) / epw) * ((s.rows + tpw - 1) / tpw) <= 256;
@@ -1062,18 +1172,18 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     else if (s.rows == 1)
         hipLaunchKernelGGL(moe_router_kernel<24>, dim3((unsigned)((s.n_expert + epw - 1) / epw), 1), dim3(256), router_lds,
                            stream, b.router, b.router_x, logits, fast1 ? (int*)nullptr : tickets, sel_idx, sel_w, s.ne,
-                           s.n_expert, s.rows, s.n_used, s.scale, kc, epw, b.norm_w, b.norm_dst, b.norm_eps);
+                           s.n_expert, s.rows, s.n_used, s.scale, kc, epw, tpw, b.norm_w, b.norm_dst, b.norm_eps);
     else if (whole_rows && router_lds > 64 * 1024)
         hipLaunchKernelGGL(moe_router_kernel<24>,
                            dim3((unsigned)((s.n_expert + epw - 1) / epw), (unsigned)((s.rows + tpw - 1) / tpw)),
                            dim3(256), router_lds, stream, b.router, b.router_x, logits, (int*)nullptr, sel_idx, sel_w,
-                           s.ne, s.n_expert, s.rows, s.n_used, s.scale, kc, epw, (const float*)nullptr, (float*)nullptr,
+                           s.ne, s.n_expert, s.rows, s.n_used, s.scale, kc, epw, tpw, (const float*)nullptr, (float*)nullptr,
                            0.0f);
     else
         hipLaunchKernelGGL(moe_router_kernel<8>,
                            dim3((unsigned)((s.n_expert + epw - 1) / epw), (unsigned)((s.rows + tpw - 1) / tpw)),
                            dim3(256), router_lds, stream, b.router, b.router_x, logits, (int*)nullptr, sel_idx, sel_w,
-                           s.ne, s.n_expert, s.rows, s.n_used, s.scale, kc, epw, (const float*)nullptr, (float*)nullptr,
+                           s.ne, s.n_expert, s.rows, s.n_used, s.scale, kc, epw, tpw, (const float*)nullptr, (float*)nullptr,
                            0.0f);
     auto bytes_per_row = [](int dtype, size_t in_f) -> size_t {
         switch (dtype) {
@@ -1228,6 +1338,11 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
                                                       s.n_ff, stream);
     }
     if (!gate_up_ok) return "no id-gathered kernel for this gate/up shape";
+    // a few rows: activation, down projection and the sum over a token's experts in one launch
+    if (kd == kSuper && !(bucketed && has_mfma(s.down_dtype)) &&
+        launch_moe_down_fused(s.down_dtype, b.down, b.down_stride, dbpr, sel_idx, sel_w, gbuf, ubuf, b.dst, b.add_b,
+                              b.add_dst, s.n_ff, s.ne, s.n_used, s.rows, stream))
+        return hipGetLastError() == hipSuccess ? nullptr : "kernel launch failed";
     // act = silu(g) * u in the form the down bank multiplies: per-256 codes, per-32 codes, or f32
     if (kd == kSuper)
         hipLaunchKernelGGL(moe_act_quant_kernel<false>, dim3((unsigned)((n_act / 256 + 3) / 4)), dim3(256), 0, stream,
