@@ -1,0 +1,62 @@
+"""Op::Linear on random shapes against the CPU oracle: every format, token counts on both sides of
+every route's threshold (1, 2..16, 17..32, 33..127, 128.., the per-32 formats' 65), row lengths
+that are and are not whole 256s, weight-row windows (`w_off`) into a larger matrix.
+
+The directed tests pin each kernel at the sizes it was written for; this one is for the seams
+between them: a threshold off by one, a tile that assumes a multiple it is not given, a row window
+that starts inside a tile. Bars are the path's: K-quant outputs bit-identical to the oracle
+(same per-block expression, same order), the other formats within rel-L2 <= 1e-4 and
+max-abs <= 1e-3 * max|y|.
+"""
+import numpy as np
+import pytest
+
+from infr_amd import DType, block_layout, synth_normal_f32
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+FORMATS = (DType.Q4K, DType.Q5K, DType.Q6K, DType.Q8_0, DType.Q2_0, DType.Q4_0, DType.Q4_1, DType.Q5_0, DType.Q5_1,
+           DType.IQ4NL)
+BIT_IDENTICAL = (DType.Q4K, DType.Q5K, DType.Q6K)
+TOKENS = (1, 1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 24, 31, 32, 33, 40, 63, 64, 65, 66, 96, 127, 128, 129, 130, 200,
+          255, 256, 257, 300)
+
+
+def draw_case(rng):
+    dtype = FORMATS[rng.integers(len(FORMATS))]
+    unit, _ = block_layout(dtype)
+    # row lengths: whole 256s mostly, for the 32- and 64-element formats also rows that end inside one
+    if unit < 256 and rng.integers(3) == 0:
+        in_f = unit * int(rng.integers(1, 1 + 2304 // unit))
+    else:
+        in_f = 256 * int(rng.integers(1, 10))
+    m = int(TOKENS[rng.integers(len(TOKENS))])
+    out_f = int(rng.choice([1, 7, 16, 31, 32, 33, 64, 96, 100, 128, 130, 257, 384]))
+    extra_before, extra_after = (int(rng.integers(0, 40)) if rng.integers(2) else 0 for _ in range(2))
+    return dtype, m, in_f, out_f, extra_before, extra_after
+
+
+@pytest.mark.parametrize("seed", range(160))
+def test_linear_on_a_random_shape_matches_the_oracle(be, seed):
+    rng = np.random.default_rng(0xF00D + seed)
+    dtype, m, in_f, out_f, before, after = draw_case(rng)
+    rows = before + out_f + after
+    # full-range payload bytes (the reference's synth_weight recipe): every code value, every scale
+    w = orc.synth_weight(dtype, rows * in_f, 0x5EED + seed)
+    x = synth_normal_f32(0xACE + seed, m * in_f)
+    if m > 2:
+        x[in_f:2 * in_f] = 0.0                     # an all-zero token: scale 0, inverse 0
+    case = f"dtype {int(dtype)} m {m} in_f {in_f} out_f {out_f} rows {before}+{out_f}+{after}"
+    yb = be.alloc(m * out_f * 4)
+    be.linear(dtype, be.upload_new(w), be.upload_new(x), yb, m, in_f, out_f, w_numel=rows * in_f, w_off=before * in_f)
+    got = be.download(yb, np.empty((m, out_f), np.float32))
+    want = orc.linear(dtype, w, x, m, in_f, out_f, w_numel=rows * in_f, w_off=before * in_f).reshape(m, out_f)
+    assert np.isfinite(want).all(), case
+    if dtype in BIT_IDENTICAL:
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), f"not bit-identical: {case}"
+    else:
+        g, t = got.astype(np.float64), want.astype(np.float64)
+        rel = np.linalg.norm(g - t) / max(np.linalg.norm(t), 1e-30)
+        mx = np.abs(g - t).max() / max(np.abs(t).max(), 1e-30)
+        assert rel <= 1e-4 and mx <= 1e-3, f"rel-L2 {rel:.2e} max-abs {mx:.2e}: {case}"
