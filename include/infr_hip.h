@@ -180,13 +180,13 @@ typedef struct {
     uint32_t ne, n_expert, n_used, n_ff_exp, rows;
     float scale;
     int router_dtype; /* INFR_DTYPE_F32 */
-    int gate_dtype, up_dtype, down_dtype; /* any quantized INFR_DTYPE_*, each bank its own */
+    int gate_dtype, up_dtype, down_dtype; /* any INFR_DTYPE_* (quantized, or plain F32 / F16 / BF16 rows), each bank its own */
 } infr_hip_moe_params_t;
 
 /* CPU arm: crates/infr-cpu/src/lib.rs:2264-2984, crates/infr-cpu/src/moe.rs. As there, rows == 1
  * multiplies decoded f32 weights with the unquantized activation; rows >= 2 takes, per bank
  * (expert_acts_kind, moe.rs:42-53), per-256 int8 activations (Q4_K, Q5_K, Q6_K, Q8_0), per-32 int8
- * activations (Q5_0), or the same f32 arm (the other formats). ne and n_ff_exp are multiples of 256.
+ * activations (Q5_0), or the same f32 arm (every other format). ne and n_ff_exp are multiples of 256.
  * Only the selected experts' blocks are read. sel_idx (i32) / sel_w (f32), [rows, n_used], are
  * optional outputs of the routing in descending-probability order. */
 int infr_hip_moe_ffn(infr_hip_t *be, const infr_hip_moe_params_t *p, const infr_hip_buffer_t *x,

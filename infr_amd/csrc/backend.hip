@@ -142,12 +142,14 @@ bool is_quant(int dt) {
     default: return false;
     }
 }
-// Formats Op::MoeFfn's expert banks may hold.
+// Formats Op::MoeFfn's expert banks may hold: every Linear weight format, and plain f32 / f16 / bf16
+// rows (expert_acts_kind's Raw arm decodes any of them, crates/infr-cpu/src/moe.rs:42-53).
 bool is_moe_quant(int dt) {
     switch (dt) {
     case INFR_DTYPE_Q4_K: case INFR_DTYPE_Q5_K: case INFR_DTYPE_Q6_K: case INFR_DTYPE_Q8_0:
     case INFR_DTYPE_Q4_0: case INFR_DTYPE_Q4_1: case INFR_DTYPE_Q5_0: case INFR_DTYPE_Q5_1:
     case INFR_DTYPE_IQ4_NL: case INFR_DTYPE_Q2_0:
+    case INFR_DTYPE_F32: case INFR_DTYPE_F16: case INFR_DTYPE_BF16:
         return true;
     default: return false;
     }

@@ -1196,6 +1196,8 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
         case 6: return in_f / 32 * 22;
         case 7: return in_f / 32 * 24;
         case 42: return in_f / 64 * 18;
+        case 0: return in_f * 4;
+        case 1: case 30: return in_f * 2;
         default: return 0;
         }
     };

@@ -280,6 +280,31 @@ def test_moe_banks_in_the_32_block_formats(be, dtype, rows):
     check(*got, *want)
 
 
+@pytest.mark.parametrize("rows", [1, 6])
+@pytest.mark.parametrize("dtype", [DType.F32, DType.F16, DType.BF16])
+def test_moe_banks_of_plain_float_rows(be, dtype, rows):
+    """Unquantized expert banks take expert_acts_kind's Raw arm at every row count
+    (crates/infr-cpu/src/moe.rs:42-53: anything without an int8 arm), decoded by
+    crates/infr-gguf/src/dequant.rs:13-22 and multiplied in `dot`'s order."""
+    ne, n_expert, n_used, nff = 512, 8, 2, 256
+
+    def rows_of(seed, n):
+        w = synth_normal_f32(seed, n, sigma=0.05)
+        if dtype == DType.F16:
+            return w.astype(np.float16).view(np.uint8)
+        if dtype == DType.BF16:
+            return (w.view(np.uint32) >> 16).astype(np.uint16).view(np.uint8)
+        return w.view(np.uint8)
+
+    gate, up, down = rows_of(401, n_expert * nff * ne), rows_of(402, n_expert * nff * ne), rows_of(403, n_expert * ne * nff)
+    x = synth_normal_f32(404 + rows, rows * ne)
+    router = synth_normal_f32(405, n_expert * ne, sigma=0.05)
+    got = run_moe_mixed(be, x, router, gate, up, down, rows, ne, n_expert, n_used, nff, (dtype,) * 3)
+    want = orc.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
+                       gate_dtype=int(dtype), up_dtype=int(dtype), down_dtype=int(dtype))
+    check(*got, *want)
+
+
 @pytest.mark.parametrize("rows", [1, 4, 40])     # 40 rows of 8 experts: the bucketed Q4_K gate beside the rest
 def test_moe_banks_of_three_different_kinds(be, rows):
     """gate Q4_K (per-256 activations), up Q5_0 (per-32), down Q4_0 (raw f32 rows) in one op: every

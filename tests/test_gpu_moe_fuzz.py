@@ -25,7 +25,20 @@ from oracle import oracle as orc
 pytestmark = pytest.mark.gpu
 
 BANK_FORMATS = (DType.Q4K, DType.Q4K, DType.Q5K, DType.Q6K, DType.Q8_0, DType.Q5_0, DType.Q4_0, DType.Q4_1,
-                DType.Q5_1, DType.IQ4NL, DType.Q2_0)
+                DType.Q5_1, DType.IQ4NL, DType.Q2_0, DType.F32, DType.F16, DType.BF16)
+
+
+def bank(dtype, seed, rows, in_f):
+    """N(0, 0.05^2) rows as raw bytes of `dtype`; the float formats are plain arrays (f16 rounded to
+    nearest, bf16 the top half of the f32 pattern, crates/infr-gguf/src/dequant.rs:19-22)."""
+    if dtype in (DType.F32, DType.F16, DType.BF16):
+        w = synth_normal_f32(seed, rows * in_f, sigma=0.05)
+        if dtype == DType.F16:
+            return w.astype(np.float16).view(np.uint8)
+        if dtype == DType.BF16:
+            return (w.view(np.uint32) >> 16).astype(np.uint16).view(np.uint8)
+        return w.view(np.uint8)
+    return synth_weight(dtype, seed, rows, in_f, 0.05)
 
 
 def draw_case(rng):
@@ -47,9 +60,9 @@ def test_moe_ffn_on_a_random_shape_matches_the_oracle(be, seed):
     rng = np.random.default_rng(0xB0A + seed)
     rows, ne, n_expert, n_used, nff, dts, scale = draw_case(rng)
     case = f"rows {rows} ne {ne} experts {n_expert} top-{n_used} nff {nff} banks {[int(d) for d in dts]} scale {scale}"
-    gate = synth_weight(dts[0], 3 * seed + 1, n_expert * nff, ne, 0.05)
-    up = synth_weight(dts[1], 3 * seed + 2, n_expert * nff, ne, 0.05)
-    down = synth_weight(dts[2], 3 * seed + 3, n_expert * ne, nff, 0.05)
+    gate = bank(dts[0], 3 * seed + 1, n_expert * nff, ne)
+    up = bank(dts[1], 3 * seed + 2, n_expert * nff, ne)
+    down = bank(dts[2], 3 * seed + 3, n_expert * ne, nff)
     x = synth_normal_f32(0xC0 + seed, rows * ne)
     router = synth_normal_f32(0xD0 + seed, n_expert * ne, sigma=0.05)
     xb, rb = be.upload_new(x), be.upload_new(router)
