@@ -40,7 +40,7 @@ typedef enum {
  * (crates/infr-gguf/src/lib.rs:330-354; crates/infr-core/src/tensor.rs:7-57). */
 typedef enum {
     INFR_DTYPE_F32 = 0,
-    INFR_DTYPE_F16 = 1,   /* embedding tables only */
+    INFR_DTYPE_F16 = 1,   /* plain rows: embedding tables, Linear weights, MoE router and banks */
     INFR_DTYPE_Q4_0 = 2,  /* 32 / 18 B:  [f16 d][u8 qs[16]]             w = d*(q-8)        :311-312 */
     INFR_DTYPE_Q4_1 = 3,  /* 32 / 20 B:  [f16 d][f16 m][u8 qs[16]]      w = d*q+m          :313-314 */
     INFR_DTYPE_Q5_0 = 6,  /* 32 / 22 B:  [f16 d][u32 qh][u8 qs[16]]     w = d*(q-16)       :315-316 */
@@ -50,7 +50,7 @@ typedef enum {
     INFR_DTYPE_Q5_K = 13, /* 256 / 176 B: [f16 d][f16 dmin][u8 sc[12]][u8 qh[32]][u8 qs[128]] :328-329 */
     INFR_DTYPE_Q6_K = 14, /* 256 / 210 B: [u8 ql[128]][u8 qh[64]][i8 sc[16]][f16 d]       :330-331 */
     INFR_DTYPE_IQ4_NL = 20, /* 32 / 18 B: [f16 d][u8 qs[16]]  w = d*codebook[q]           :349-350 */
-    INFR_DTYPE_BF16 = 30, /* embedding tables only */
+    INFR_DTYPE_BF16 = 30, /* plain rows, as F16 */
     INFR_DTYPE_Q2_0 = 42  /* 64 / 18 B:   [f16 d][u8 qs[16]] ternary-style 2-bit codes    :357-358 */
 } infr_dtype;
 
@@ -134,7 +134,11 @@ int infr_hip_sync(infr_hip_t *be);
  * integer dot is exact, and the f32 epilogue follows the CPU kernels' expression per block.
  * in_f must be a whole number of weight blocks (256 for the K-quants, 64 for Q2_0, 32 otherwise): a
  * shorter tail is rejected, never truncated. in_f above 32768 (Q8_0, Q4_1, Q5_1: 16384) must be a
- * multiple of 256 (it then runs the prefill kernels at any m), else INFR_HIP_ERR_UNSUPPORTED. */
+ * multiple of 256 (it then runs the prefill kernels at any m), else INFR_HIP_ERR_UNSUPPORTED.
+ * Unquantized rows (F32, F16, BF16; in_f a multiple of 32) are multiplied as the CPU arm does
+ * (lib.rs:1162-1164, 1443-1462: dot / dot_f16 / dot_bf16 - weights widened exactly, eight FMA
+ * chains over the columns i mod 8, added in order): outputs equal infr-cpu's bit for bit. That
+ * form is for the odd small matrix a quantized file keeps in floating point, not for speed. */
 int infr_hip_linear(infr_hip_t *be, int dtype, const infr_hip_buffer_t *w, size_t w_numel,
                     size_t w_off, const infr_hip_buffer_t *x, infr_hip_buffer_t *dst, size_t m,
                     size_t in_f, size_t out_f);
@@ -179,7 +183,7 @@ int infr_hip_linear_int_stages(infr_hip_t *be, int dtype, const infr_hip_buffer_
 typedef struct {
     uint32_t ne, n_expert, n_used, n_ff_exp, rows;
     float scale;
-    int router_dtype; /* INFR_DTYPE_F32 */
+    int router_dtype; /* INFR_DTYPE_F32, _F16 or _BF16 */
     int gate_dtype, up_dtype, down_dtype; /* any INFR_DTYPE_* (quantized, or plain F32 / F16 / BF16 rows), each bank its own */
 } infr_hip_moe_params_t;
 

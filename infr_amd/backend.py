@@ -22,7 +22,7 @@ LIB_PATH = os.path.join(_HERE, "libinfr_hip.so")
 class DType(IntEnum):
     """GGML type ids (crates/infr-gguf/src/lib.rs:330-354)."""
     F32 = 0
-    F16 = 1      # embedding tables only
+    F16 = 1      # plain rows: embedding tables, Linear weights, MoE router and banks
     Q4_0 = 2
     Q4_1 = 3
     Q5_0 = 6
@@ -32,7 +32,7 @@ class DType(IntEnum):
     Q5K = 13
     Q6K = 14
     IQ4NL = 20
-    BF16 = 30    # embedding tables only
+    BF16 = 30    # plain rows, as F16
     I32 = 26     # token ids (never a weight here)
     Q2_0 = 42
 

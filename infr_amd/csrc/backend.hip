@@ -156,7 +156,11 @@ bool is_moe_quant(int dt) {
 }
 bool act_per32(int dt, size_t in_f) { return infr::act_is_per32(dt, in_f); }
 // Row lengths a format accepts: whole weight blocks.
+// Unquantized weight rows: Op::Linear multiplies them with dot / dot_f16 / dot_bf16
+// (crates/infr-cpu/src/lib.rs:1162-1165, 1443-1462).
+bool is_plain(int dt) { return dt == INFR_DTYPE_F32 || dt == INFR_DTYPE_F16 || dt == INFR_DTYPE_BF16; }
 size_t in_f_multiple(int dt) {
+    if (is_plain(dt)) return 32;  // the row-dot kernel stages whole groups of 32 columns
     int e = 0, b = 0;
     return infr_block_layout(dt, &e, &b) ? (size_t)e : 256;
 }
@@ -170,6 +174,11 @@ bool has_two_stages(int dt) { return dt == INFR_DTYPE_Q4_K || dt == INFR_DTYPE_Q
 // Tokens rounded up to the 32 of a tile, rows to the 256 of a step (the tiled per-32 quantizer pads
 // rows that end inside a step).
 static size_t act_scratch_elems(size_t m, size_t in_f) { return (m + 31) / 32 * 32 * ((in_f + 255) / 256 * 256); }
+// What an Op::Linear needs of it: unquantized weights quantize nothing, but an op in place on its x
+// parks a copy of x there (4 bytes per element).
+static size_t linear_scratch_elems(int dtype, size_t m, size_t in_f) {
+    return is_plain(dtype) ? m * in_f * sizeof(float) : act_scratch_elems(m, in_f);
+}
 
 static bool is_elementwise(int kind) { return kind >= INFR_OP_RMS_NORM && kind <= INFR_OP_ADD; }
 
@@ -254,14 +263,14 @@ static int enqueue_elementwise(infr_hip_t* be, const infr_hip_op_t& op, const El
 // launches: one token of a format whose CPU arm multiplies f32 activations, and rows too long for
 // the decode mapping (those go to the prefill kernels at any m).
 static bool runs_alone(int dtype, size_t m, size_t in_f) {
-    return infr::gemv_takes_f32_activations(dtype, m) || infr::gemv_row_too_long(dtype, in_f);
+    return is_plain(dtype) || infr::gemv_takes_f32_activations(dtype, m) || infr::gemv_row_too_long(dtype, in_f);
 }
 
 // Ops that run in small-batch groups inside plans: the K-split MFMA kernels take Q4_K up to 32
 // rows and Q5_K up to 16 (rows of an even number of blocks), the dot4 batch kernel the other
 // formats up to 8.
 static bool small_batch(const infr_hip_op_t& op) {
-    if (op.m < 2 || infr::gemv_row_too_long(op.w_dtype, op.in_f)) return false;
+    if (op.m < 2 || is_plain(op.w_dtype) || infr::gemv_row_too_long(op.w_dtype, op.in_f)) return false;
     if (op.w_dtype == INFR_DTYPE_Q4_K) return op.m <= 32;
     return op.m <= 8 || infr::mmq_skinny16_takes(op.w_dtype, op.m, op.in_f);
 }
@@ -313,7 +322,7 @@ int check_linear(infr_hip_t* be, int dtype, const infr_hip_buffer_t* w, size_t w
                  size_t w_off, const infr_hip_buffer_t* x, size_t m, size_t in_f, size_t out_f,
                  LinearArgs* out) {
     if (!w || !x) return fail(be, INFR_HIP_ERR_INVALID, "linear: unbound buffer");
-    if (!is_quant(dtype))
+    if (!is_quant(dtype) && !is_plain(dtype))
         return fail(be, INFR_HIP_ERR_UNSUPPORTED,
                     "linear: weight dtype " + std::to_string(dtype) + " has no kernel");
     if (m == 0 || in_f == 0 || out_f == 0) return fail(be, INFR_HIP_ERR_INVALID, "linear: empty shape");
@@ -359,7 +368,16 @@ static bool floats_overlap(const float* a, size_t na, const float* b, size_t nb)
 int enqueue_linear(infr_hip_t* be, int dtype, const LinearArgs& la, const float* x, float* y,
                    size_t m, size_t in_f, size_t out_f, const infr::IntStages& st, const infr::ActQ8& act) {
     bool ok;
-    if (infr::gemv_takes_f32_activations(dtype, m)) {
+    if (is_plain(dtype)) {
+        if (st.a) return fail(be, INFR_HIP_ERR_UNSUPPORTED, "int_stages: unquantized weights have no integer stage");
+        if (floats_overlap(x, m * in_f, y, m * out_f)) {
+            // in place: every workgroup reads x while others store y; multiply a copy of x
+            float* copy = reinterpret_cast<float*>(act.qs);
+            HIP_TRY(be, hipMemcpyAsync(copy, x, m * in_f * sizeof(float), hipMemcpyDeviceToDevice, be->stream));
+            x = copy;
+        }
+        ok = infr::launch_linear_plain_rows(dtype, la.wrows, x, y, m, in_f, out_f, be->stream);
+    } else if (infr::gemv_takes_f32_activations(dtype, m)) {
         if (st.a)
             return fail(be, INFR_HIP_ERR_UNSUPPORTED,
                         "int_stages: one token of dtype " + std::to_string(dtype) + " has no integer stage");
@@ -646,7 +664,7 @@ int infr_hip_linear(infr_hip_t* be, int dtype, const infr_hip_buffer_t* w, size_
                                   static_cast<float*>(dst->ptr), la.bpr, (int32_t)out_f};
         return enqueue_gemv_single(be, dtype, in_f, op);
     }
-    if (int rc = ensure_act(be, act_scratch_elems(m, in_f))) return rc;
+    if (int rc = ensure_act(be, linear_scratch_elems(dtype, m, in_f))) return rc;
     return enqueue_linear(be, dtype, la, static_cast<const float*>(x->ptr),
                           static_cast<float*>(dst->ptr), m, in_f, out_f, infr::IntStages{}, be->act);
 }
@@ -667,9 +685,9 @@ int infr_hip_linear_noalloc(infr_hip_t* be, int dtype, const infr_hip_buffer_t* 
                                   static_cast<float*>(dst->ptr), la.bpr, (int32_t)out_f};
         return enqueue_gemv_single(be, dtype, in_f, op);
     }
-    if (act_scratch_elems(m, in_f) > kStaticActElems)
+    if (linear_scratch_elems(dtype, m, in_f) > kStaticActElems)
         return fail(be, INFR_HIP_ERR_UNSUPPORTED,
-                    "linear_noalloc: " + std::to_string(act_scratch_elems(m, in_f)) +
+                    "linear_noalloc: " + std::to_string(linear_scratch_elems(dtype, m, in_f)) +
                         " activation elements (tokens rounded up to 32, times in_f rounded up to 256) exceed the static scratch of " +
                         std::to_string(kStaticActElems));
     return enqueue_linear(be, dtype, la, static_cast<const float*>(x->ptr), static_cast<float*>(dst->ptr), m,
@@ -794,11 +812,11 @@ static int check_moe(infr_hip_t* be, const infr_hip_moe_params_t* p, const infr_
     const size_t ub = expert_bank_bytes(p->up_dtype, (size_t)p->n_expert * p->n_ff_exp, p->ne);
     const size_t db = expert_bank_bytes(p->down_dtype, (size_t)p->n_expert * p->ne, p->n_ff_exp);
     if (!gb || !ub || !db || !is_moe_quant(p->gate_dtype) || !is_moe_quant(p->up_dtype) ||
-        !is_moe_quant(p->down_dtype))
+        !is_moe_quant(p->down_dtype) || !is_plain(p->router_dtype))
         return fail(be, INFR_HIP_ERR_UNSUPPORTED, "moe_ffn: expert bank dtype/shape has no kernel");
     const size_t act_bytes = (size_t)p->rows * p->ne * sizeof(float);
     if (gate->len < gb || up->len < ub || down->len < db ||
-        router->len < (size_t)p->n_expert * p->ne * sizeof(float) || x->len < act_bytes ||
+        router->len < (size_t)p->n_expert * p->ne * (p->router_dtype == INFR_DTYPE_F32 ? 4 : 2) || x->len < act_bytes ||
         router_x->len < act_bytes || dst->len < act_bytes)
         return fail(be, INFR_HIP_ERR_INVALID, "moe_ffn: a buffer is smaller than its declared shape");
     const size_t sel_bytes = (size_t)p->rows * p->n_used * 4;
@@ -855,14 +873,14 @@ int infr_hip_compile(infr_hip_t* be, const infr_hip_op_t* ops, size_t n_ops, inf
     size_t act_need = 0, moe_need = 0, batch_need = 0;  // batch_need: every small-batch op in one level
     for (const auto& op : p->ops) {
         if (op.kind == INFR_OP_LINEAR) {
-            if (!is_quant(op.w_dtype) || op.m == 0 || op.in_f == 0 || op.out_f == 0 ||
+            if ((!is_quant(op.w_dtype) && !is_plain(op.w_dtype)) || op.m == 0 || op.in_f == 0 || op.out_f == 0 ||
                 op.in_f % in_f_multiple(op.w_dtype) != 0 || op.w_numel % op.in_f != 0 ||
                 op.w_off % op.in_f != 0) {
                 delete p;
                 return fail(be, INFR_HIP_ERR_UNSUPPORTED, "compile: Linear op with unsupported dtype/shape");
             }
             p->max_tensor = std::max({p->max_tensor, op.x, op.weight, op.dst});
-            act_need = std::max(act_need, act_scratch_elems(op.m, op.in_f));
+            act_need = std::max(act_need, linear_scratch_elems(op.w_dtype, op.m, op.in_f));
             if (small_batch(op)) batch_need += ((size_t)op.m * op.in_f + 255) / 256 * 256;
         } else if (op.kind == INFR_OP_MOE_FFN) {
             const auto& mp = op.moe;

@@ -289,5 +289,9 @@ bool launch_mmq_gathered(int dtype, const uint8_t* bank, size_t expert_stride, s
 size_t moe_workspace_bytes(const MoeShape& s);
 // Enqueues the whole op; returns nullptr or a message naming what is unsupported.
 const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* workspace, hipStream_t stream);
+// Op::Linear over plain f32 (dtype 0), f16 (1) or bf16 (30) weight rows: y[t, o] = dot(w[o], x[t]) in
+// infr-cpu's `dot` order (in_f a multiple of 32). False when the shape has no launch.
+bool launch_linear_plain_rows(int dtype, const void* w, const float* x, float* y, size_t m, size_t in_f, size_t out_f,
+                              hipStream_t stream);
 
 }  // namespace infr

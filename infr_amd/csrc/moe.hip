@@ -178,15 +178,36 @@ __global__ __launch_bounds__(256) void moe_select_kernel(const float* __restrict
 // selection too, which saves a launch; eight experts per workgroup keep that to a handful of
 // tickets (atomics on one address complete one after another, ~65 ns each).
 // ne % 32 == 0 is required.
+// Four consecutive elements of a plain row of f32 (WT 0), f16 (1) or bf16 (30) as f32, widened
+// exactly (crates/infr-gguf/src/dequant.rs:13-22): what dot / dot_f16 / dot_bf16 multiply
+// (crates/infr-cpu/src/kernels.rs:6505-6573).
+template <int WT>
+__device__ __forceinline__ v4f row_load4(const void* row, size_t elem) {
+    if constexpr (WT == 0) {
+        return *reinterpret_cast<const v4f*>(static_cast<const float*>(row) + elem);
+    } else {
+        const v2i raw = *reinterpret_cast<const v2i*>(static_cast<const uint16_t*>(row) + elem);
+        const uint32_t lo = (uint32_t)raw.x, hi = (uint32_t)raw.y;
+        if constexpr (WT == 1)
+            return v4f{f16_bits_to_f32(lo & 0xFFFFu), f16_bits_to_f32(lo >> 16), f16_bits_to_f32(hi & 0xFFFFu),
+                       f16_bits_to_f32(hi >> 16)};
+        else
+            return v4f{__builtin_bit_cast(float, lo << 16), __builtin_bit_cast(float, lo & 0xFFFF0000u),
+                       __builtin_bit_cast(float, hi << 16), __builtin_bit_cast(float, hi & 0xFFFF0000u)};
+    }
+}
+template <int WT>
+__host__ __device__ constexpr size_t row_elem_bytes() { return WT == 0 ? 4 : 2; }
+
 constexpr int kRouterPairs = 32, kRouterChunk = 512;
 // floats between two staged rows of kc elements: eight accumulator rows of kc / 8 + 4
 __host__ __device__ constexpr int router_row_floats(int kc) { return 8 * (kc / 8 + 4); }
 
 // NL: 16-byte loads a thread has in flight while staging (24 at a single row: the nine rows of a
 // workgroup arrive in one round trip)
-template <int NL>
+template <int NL, int WT = 0>
 __global__ __launch_bounds__(256) void moe_router_kernel(
-    const float* __restrict__ router, const float* __restrict__ rx, float* __restrict__ logits,
+    const void* __restrict__ router, const float* __restrict__ rx, float* __restrict__ logits,
     int* __restrict__ tickets, int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, int ne,
     int n_expert, int rows, int n_used, float scale, int kc, int epw, int tpw, const float* __restrict__ norm_w,
     float* __restrict__ norm_dst, float norm_eps) {
@@ -227,11 +248,14 @@ __global__ __launch_bounds__(256) void moe_router_kernel(
             for (int u = 0; u < NL; ++u) {
                 const int i = base + u * 256 + tid;
                 const int row = i / n4, q = i % n4;
-                const float* src = row < n_e ? router + (size_t)(e0 + row) * ne : rx + (size_t)(t0 + row - n_e) * ne;
                 // elements 4q .. 4q+3 are accumulators 4(q & 1) .. +3 at step q / 2
                 dst[u] = (row < n_e ? lw + row * ld : lx + (row - n_e) * ld) + 4 * (q & 1) * la + (q >> 1);
                 if (i < total) {
-                    tmp[u] = reinterpret_cast<const v4f*>(src + k0)[q];
+                    if (row < n_e)
+                        tmp[u] = row_load4<WT>(static_cast<const uint8_t*>(router) + (size_t)(e0 + row) * ne * row_elem_bytes<WT>(),
+                                               (size_t)k0 + 4 * q);
+                    else
+                        tmp[u] = reinterpret_cast<const v4f*>(rx + (size_t)(t0 + row - n_e) * ne + k0)[q];
                     if (norm_w && row >= n_e) {
                         const v4f wv = reinterpret_cast<const v4f*>(norm_w + k0)[q];
                         tmp[u] = v4f{tmp[u].x * nscale * wv.x, tmp[u].y * nscale * wv.y, tmp[u].z * nscale * wv.z,
@@ -295,7 +319,8 @@ __global__ __launch_bounds__(256) void moe_router_kernel(
 constexpr int kRtE = 16, kRtT = 16, kRtK = 256, kRtThreads = 128, kRtMinRows = 256;
 constexpr int kRtLoads = (kRtE + kRtT) * (kRtK / 4) / kRtThreads;  // 16-byte loads per thread and chunk
 
-__global__ __launch_bounds__(kRtThreads) void moe_router_tile_kernel(const float* __restrict__ router,
+template <int WT = 0>
+__global__ __launch_bounds__(kRtThreads) void moe_router_tile_kernel(const void* __restrict__ router,
                                                                      const float* __restrict__ rx,
                                                                      float* __restrict__ logits, int ne,
                                                                      int n_expert, int rows) {
@@ -305,19 +330,22 @@ __global__ __launch_bounds__(kRtThreads) void moe_router_tile_kernel(const float
     const int e0 = blockIdx.x * kRtE, t0 = blockIdx.y * kRtT;
     // this thread's pieces of a chunk: row (i * kRtThreads + tid) / 64, float4 column % 64;
     // rows past the last expert / token repeat it (computed, never stored)
-    const float* src[kRtLoads];
+    const void* src[kRtLoads];  // the row each piece comes from: a weight row (WT) or an activation row (f32)
 #pragma unroll
     for (int i = 0; i < kRtLoads; ++i) {
-        const int idx = i * kRtThreads + tid, row = idx / (kRtK / 4), q = idx % (kRtK / 4);
-        src[i] = (row < kRtE ? router + (size_t)min(e0 + row, n_expert - 1) * ne
-                             : rx + (size_t)min(t0 + row - kRtE, rows - 1) * ne) + 4 * q;
+        const int idx = i * kRtThreads + tid, row = idx / (kRtK / 4);
+        src[i] = row < kRtE ? static_cast<const void*>(static_cast<const uint8_t*>(router) +
+                                                       (size_t)min(e0 + row, n_expert - 1) * ne * row_elem_bytes<WT>())
+                            : static_cast<const void*>(rx + (size_t)min(t0 + row - kRtE, rows - 1) * ne);
     }
     v4f stage[kRtLoads];
     auto fetch = [&](int k0) {
 #pragma unroll
         for (int i = 0; i < kRtLoads; ++i) {
-            const int q = (i * kRtThreads + tid) % (kRtK / 4);
-            stage[i] = k0 + 4 * q < ne ? *reinterpret_cast<const v4f*>(src[i] + k0) : v4f{0.0f, 0.0f, 0.0f, 0.0f};
+            const int idx = i * kRtThreads + tid, row = idx / (kRtK / 4), q = idx % (kRtK / 4);
+            if (k0 + 4 * q >= ne) stage[i] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+            else if (row < kRtE) stage[i] = row_load4<WT>(src[i], (size_t)k0 + 4 * q);
+            else stage[i] = row_load4<0>(src[i], (size_t)k0 + 4 * q);
         }
     };
     float acc[4][4];
@@ -1071,6 +1099,75 @@ static bool launch_moe_down_fused(int dtype, const uint8_t* bank, size_t stride,
     }
 }
 
+// logits[t * n_rows_w + r] = dot(w[r], x[t]) in infr-cpu's `dot` order, for `n_rows_w` plain rows of
+// `ne` f32 (WT 0), f16 (1) or bf16 (30) weights against `rows` activation rows: the MoE router, and
+// Op::Linear over unquantized weights. With a single row and `logits_only` unset the last workgroup
+// also selects (tickets, sel_idx, sel_w).
+template <int WT>
+static void launch_row_dots(const void* w, const float* x, float* logits, int ne, int n_rows_w, int rows,
+                            bool logits_only, int* tickets, int32_t* sel_idx, float* sel_w, int n_used, float scale,
+                            const float* norm_w, float* norm_dst, float norm_eps, hipStream_t stream) {
+    // One weight row per workgroup when only logits are wanted of a single row (nothing to wait
+    // for); eight at a single row that ends in the selection (few tickets), four once rows fill the
+    // pairs; whole rows in one chunk when they fit the LDS a workgroup may have, else kRouterChunk
+    // columns at a time
+    constexpr size_t kRouterLdsMax = 144 * 1024;
+    int epw = logits_only ? 1 : (rows == 1 ? 8 : 4);
+    int tpw = kRouterPairs / epw;
+    if (rows > 1) {
+        // a few rows: fewer (expert, token) pairs per workgroup, so that about 256 workgroups share
+        // the staging (16 tokens x 128 experts: 2 x 4 pairs each instead of 4 x 8 on 64 workgroups)
+        int per_wg = 1;
+        while (per_wg < kRouterPairs && (size_t)n_rows_w * rows > (size_t)256 * per_wg) per_wg *= 2;
+        epw = per_wg >= 16 ? 4 : (per_wg >= 4 ? 2 : 1);
+        tpw = per_wg / epw;
+    }
+    while (epw > 1 && (size_t)(epw + 1) * router_row_floats(ne) * sizeof(float) > kRouterLdsMax) epw /= 2;
+    const int n_t = std::min(rows, tpw);
+    // (whole rows also for a few rows, while the grid is a single round of one workgroup per compute unit)
+    const bool one_round = (size_t)((n_rows_w + epw - 1) / epw) * ((rows + tpw - 1) / tpw) <= 256;
+    const bool whole_rows = (size_t)(epw + n_t) * router_row_floats(ne) * sizeof(float) <= (one_round ? kRouterLdsMax : 64 * 1024);
+    const int kc = whole_rows ? ne : kRouterChunk;
+    const size_t router_lds = (size_t)(epw + n_t) * router_row_floats(kc) * sizeof(float);
+    if (router_lds > 64 * 1024)
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_router_kernel<24, WT>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)router_lds);
+    if (rows >= kRtMinRows)
+        hipLaunchKernelGGL(moe_router_tile_kernel<WT>,
+                           dim3((unsigned)((n_rows_w + kRtE - 1) / kRtE), (unsigned)((rows + kRtT - 1) / kRtT)),
+                           dim3(kRtThreads), 0, stream, w, x, logits, ne, n_rows_w, rows);
+    else if (rows == 1)
+        hipLaunchKernelGGL((moe_router_kernel<24, WT>), dim3((unsigned)((n_rows_w + epw - 1) / epw), 1), dim3(256), router_lds,
+                           stream, w, x, logits, logits_only ? (int*)nullptr : tickets, sel_idx, sel_w, ne,
+                           n_rows_w, rows, n_used, scale, kc, epw, tpw, norm_w, norm_dst, norm_eps);
+    else if (whole_rows && router_lds > 64 * 1024)
+        hipLaunchKernelGGL((moe_router_kernel<24, WT>),
+                           dim3((unsigned)((n_rows_w + epw - 1) / epw), (unsigned)((rows + tpw - 1) / tpw)),
+                           dim3(256), router_lds, stream, w, x, logits, (int*)nullptr, sel_idx, sel_w,
+                           ne, n_rows_w, rows, n_used, scale, kc, epw, tpw, (const float*)nullptr, (float*)nullptr,
+                           0.0f);
+    else
+        hipLaunchKernelGGL((moe_router_kernel<8, WT>),
+                           dim3((unsigned)((n_rows_w + epw - 1) / epw), (unsigned)((rows + tpw - 1) / tpw)),
+                           dim3(256), router_lds, stream, w, x, logits, (int*)nullptr, sel_idx, sel_w,
+                           ne, n_rows_w, rows, n_used, scale, kc, epw, tpw, (const float*)nullptr, (float*)nullptr,
+                           0.0f);
+}
+
+// Op::Linear over plain f32 / f16 / bf16 weight rows (crates/infr-cpu/src/lib.rs:1162-1165,
+// 1443-1462: dot / dot_f16 / dot_bf16 per output): y[t, o] = dot(w[o], x[t]), the CPU's bits.
+bool launch_linear_plain_rows(int dtype, const void* w, const float* x, float* y, size_t m, size_t in_f, size_t out_f,
+                              hipStream_t stream) {
+    if (in_f % 32 != 0 || in_f > (size_t)1 << 30 || out_f > (size_t)1 << 30 || m > (size_t)1 << 30) return false;
+    switch (dtype) {
+    case 0: launch_row_dots<0>(w, x, y, (int)in_f, (int)out_f, (int)m, true, nullptr, nullptr, nullptr, 0, 0.0f, nullptr, nullptr, 0.0f, stream); break;
+    case 1: launch_row_dots<1>(w, x, y, (int)in_f, (int)out_f, (int)m, true, nullptr, nullptr, nullptr, 0, 0.0f, nullptr, nullptr, 0.0f, stream); break;
+    case 30: launch_row_dots<30>(w, x, y, (int)in_f, (int)out_f, (int)m, true, nullptr, nullptr, nullptr, 0, 0.0f, nullptr, nullptr, 0.0f, stream); break;
+    default: return false;
+    }
+    return hipGetLastError() == hipSuccess;
+}
+
 size_t moe_workspace_bytes(const MoeShape& s) {
     const size_t pairs = (size_t)s.rows * s.n_used;
     size_t n = 0;
@@ -1100,7 +1197,7 @@ size_t moe_workspace_bytes(const MoeShape& s) {
 }
 
 const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hipStream_t stream) {
-    if (s.router_dtype != 0) return "router dtype must be F32";
+    if (s.router_dtype != 0 && s.router_dtype != 1 && s.router_dtype != 30) return "router dtype must be F32, F16 or BF16";
     if (b.norm_w && (s.rows != 1 || b.x != b.norm_dst)) return "an absorbed RmsNorm needs a single row read from its dst";
     if (s.n_used > 64 || s.n_expert > 1024 || s.n_used > s.n_expert) return "n_used <= 64 and n_expert <= 1024 required";
     if (s.ne % 256 != 0 || s.n_ff % 256 != 0) return "ne and n_ff_exp must be multiples of 256";
@@ -1141,50 +1238,11 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     auto raw_ok = [](int dt) { return dt == 12 || dt == 13 || dt == 14 || dt == 8; };
     const bool fast1 = s.rows == 1 && raw_ok(s.gate_dtype) && s.up_dtype == s.gate_dtype && raw_ok(s.down_dtype) &&
                        s.ne <= 4096 && s.n_ff <= 4096;
-    // Otherwise eight experts per workgroup at a single row (few tickets), four once rows fill the
-    // pairs; whole rows in one chunk when they fit the LDS a workgroup may have, else kRouterChunk
-    // columns at a time
-    constexpr size_t kRouterLdsMax = 144 * 1024;
-    int epw = fast1 ? 1 : (s.rows == 1 ? 8 : 4);
-    int tpw = kRouterPairs / epw;
-    if (s.rows > 1) {
-        // a few rows: fewer (expert, token) pairs per workgroup, so that about 256 workgroups share
-        // the staging (16 tokens x 128 experts: 2 x 4 pairs each instead of 4 x 8 on 64 workgroups)
-        int per_wg = 1;
-        while (per_wg < kRouterPairs && (size_t)s.n_expert * s.rows > (size_t)256 * per_wg) per_wg *= 2;
-        epw = per_wg >= 16 ? 4 : (per_wg >= 4 ? 2 : 1);
-        tpw = per_wg / epw;
+    switch (s.router_dtype) {
+    case 0: launch_row_dots<0>(b.router, b.router_x, logits, s.ne, s.n_expert, s.rows, fast1, tickets, sel_idx, sel_w, s.n_used, s.scale, b.norm_w, b.norm_dst, b.norm_eps, stream); break;
+    case 1: launch_row_dots<1>(b.router, b.router_x, logits, s.ne, s.n_expert, s.rows, fast1, tickets, sel_idx, sel_w, s.n_used, s.scale, b.norm_w, b.norm_dst, b.norm_eps, stream); break;
+    default: launch_row_dots<30>(b.router, b.router_x, logits, s.ne, s.n_expert, s.rows, fast1, tickets, sel_idx, sel_w, s.n_used, s.scale, b.norm_w, b.norm_dst, b.norm_eps, stream); break;
     }
-    while (epw > 1 && (size_t)(epw + 1) * router_row_floats(s.ne) * sizeof(float) > kRouterLdsMax) epw /= 2;
-    const int n_t = std::min(s.rows, tpw);
-    // (whole rows also for a few rows, while the grid is a single round of one workgroup per compute unit)
-    const bool one_round = (size_t)((s.n_expert + epw - 1) / epw) * ((s.rows + tpw - 1) / tpw) <= 256;
-    const bool whole_rows = (size_t)(epw + n_t) * router_row_floats(s.ne) * sizeof(float) <= (one_round ? kRouterLdsMax : 64 * 1024);
-    const int kc = whole_rows ? s.ne : kRouterChunk;
-    const size_t router_lds = (size_t)(epw + n_t) * router_row_floats(kc) * sizeof(float);
-    if (router_lds > 64 * 1024)
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_router_kernel<24>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)router_lds);
-    if (s.rows >= kRtMinRows)
-        hipLaunchKernelGGL(moe_router_tile_kernel,
-                           dim3((unsigned)((s.n_expert + kRtE - 1) / kRtE), (unsigned)((s.rows + kRtT - 1) / kRtT)),
-                           dim3(kRtThreads), 0, stream, b.router, b.router_x, logits, s.ne, s.n_expert, s.rows);
-    else if (s.rows == 1)
-        hipLaunchKernelGGL(moe_router_kernel<24>, dim3((unsigned)((s.n_expert + epw - 1) / epw), 1), dim3(256), router_lds,
-                           stream, b.router, b.router_x, logits, fast1 ? (int*)nullptr : tickets, sel_idx, sel_w, s.ne,
-                           s.n_expert, s.rows, s.n_used, s.scale, kc, epw, tpw, b.norm_w, b.norm_dst, b.norm_eps);
-    else if (whole_rows && router_lds > 64 * 1024)
-        hipLaunchKernelGGL(moe_router_kernel<24>,
-                           dim3((unsigned)((s.n_expert + epw - 1) / epw), (unsigned)((s.rows + tpw - 1) / tpw)),
-                           dim3(256), router_lds, stream, b.router, b.router_x, logits, (int*)nullptr, sel_idx, sel_w,
-                           s.ne, s.n_expert, s.rows, s.n_used, s.scale, kc, epw, tpw, (const float*)nullptr, (float*)nullptr,
-                           0.0f);
-    else
-        hipLaunchKernelGGL(moe_router_kernel<8>,
-                           dim3((unsigned)((s.n_expert + epw - 1) / epw), (unsigned)((s.rows + tpw - 1) / tpw)),
-                           dim3(256), router_lds, stream, b.router, b.router_x, logits, (int*)nullptr, sel_idx, sel_w,
-                           s.ne, s.n_expert, s.rows, s.n_used, s.scale, kc, epw, tpw, (const float*)nullptr, (float*)nullptr,
-                           0.0f);
     auto bytes_per_row = [](int dtype, size_t in_f) -> size_t {
         switch (dtype) {
         case 12: return in_f / 256 * 144;

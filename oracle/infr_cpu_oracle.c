@@ -790,7 +790,9 @@ static int linear_shape_ok(int dtype, size_t in_f) {
     case ORC_IQ4_NL:
     case ORC_Q8_0: return in_f % 32 == 0;
     case ORC_Q2_0: return in_f % 64 == 0;
-    case ORC_F32: return 1;
+    case ORC_F32:
+    case ORC_F16:
+    case ORC_BF16: return 1; /* dot / dot_f16 / dot_bf16, any length (lib.rs:1162-1164, 1443-1462) */
     default: return 0;
     }
 }
@@ -822,8 +824,10 @@ int orc_linear(int dtype, const uint8_t *w, size_t wbytes, size_t w_numel, size_
 #endif
     (void)nt;
 
-    if (dtype == ORC_F32 || reference_mode || (dtype == ORC_Q5_0 && m == 1)) {
-        /* lib.rs:1015-1031 (reference mode) / :1162,1443-1448 (F32 weights): decode row, dot().
+    if (dtype == ORC_F32 || dtype == ORC_F16 || dtype == ORC_BF16 || reference_mode || (dtype == ORC_Q5_0 && m == 1)) {
+        /* lib.rs:1015-1031 (reference mode) / :1162-1164,1443-1462 (F32 / F16 / BF16 weights): decode
+         * row, dot(). dot_f16 and dot_bf16 (kernels.rs:6505-6549) widen each weight exactly and run
+         * dot's own eight FMA chains, so decoding the row first gives their bits.
          * Q5_0 has no arm in the one-token match (lib.rs:1081-1165), so decode takes its last arm,
          * `dot(&bytes_to_f32(row, dt), xrow)` (:1165): f32 activations, no int8 rounding. With
          * m >= 2 it takes the per-32 int8 kernel (:1322-1329). */

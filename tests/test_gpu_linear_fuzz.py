@@ -17,15 +17,16 @@ from oracle import oracle as orc
 pytestmark = pytest.mark.gpu
 
 FORMATS = (DType.Q4K, DType.Q5K, DType.Q6K, DType.Q8_0, DType.Q2_0, DType.Q4_0, DType.Q4_1, DType.Q5_0, DType.Q5_1,
-           DType.IQ4NL)
-BIT_IDENTICAL = (DType.Q4K, DType.Q5K, DType.Q6K)
+           DType.IQ4NL, DType.F32, DType.F16, DType.BF16)
+PLAIN = (DType.F32, DType.F16, DType.BF16)
+BIT_IDENTICAL = (DType.Q4K, DType.Q5K, DType.Q6K) + PLAIN
 TOKENS = (1, 1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 24, 31, 32, 33, 40, 63, 64, 65, 66, 96, 127, 128, 129, 130, 200,
           255, 256, 257, 300)
 
 
 def draw_case(rng):
     dtype = FORMATS[rng.integers(len(FORMATS))]
-    unit, _ = block_layout(dtype)
+    unit = 32 if dtype in PLAIN else block_layout(dtype)[0]
     # row lengths: whole 256s mostly, for the 32- and 64-element formats also rows that end inside one
     if unit < 256 and rng.integers(3) == 0:
         in_f = unit * int(rng.integers(1, 1 + 2304 // unit))
@@ -43,7 +44,12 @@ def test_linear_on_a_random_shape_matches_the_oracle(be, seed):
     dtype, m, in_f, out_f, before, after = draw_case(rng)
     rows = before + out_f + after
     # full-range payload bytes (the reference's synth_weight recipe): every code value, every scale
-    w = orc.synth_weight(dtype, rows * in_f, 0x5EED + seed)
+    if dtype in PLAIN:
+        w32 = synth_normal_f32(0x5EED + seed, rows * in_f, sigma=0.05)
+        w = (w32 if dtype == DType.F32 else w32.astype(np.float16) if dtype == DType.F16
+             else (w32.view(np.uint32) >> 16).astype(np.uint16)).view(np.uint8)
+    else:
+        w = orc.synth_weight(dtype, rows * in_f, 0x5EED + seed)
     x = synth_normal_f32(0xACE + seed, m * in_f)
     if m > 2:
         x[in_f:2 * in_f] = 0.0                     # an all-zero token: scale 0, inverse 0

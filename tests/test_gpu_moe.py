@@ -305,6 +305,30 @@ def test_moe_banks_of_plain_float_rows(be, dtype, rows):
     check(*got, *want)
 
 
+@pytest.mark.parametrize("rows", [1, 3, 300])      # 300: the register-tiled router
+@pytest.mark.parametrize("router_dtype", [DType.F16, DType.BF16])
+def test_moe_router_weights_in_half_precision(be, router_dtype, rows):
+    """The router matrix is one more bank to the CPU arm (expert_gemm over router_dtype,
+    crates/infr-cpu/src/lib.rs:2376-2395): f16 / bf16 rows are widened exactly and multiplied in
+    `dot`'s order, so the selection still equals the oracle's."""
+    ne, n_expert, n_used, nff = 512, 16, 4, 256
+    gate, up, down = banks(410, ne, n_expert, nff, sigma=0.05)
+    r32 = synth_normal_f32(413, n_expert * ne, sigma=0.05)
+    router = (r32.astype(np.float16) if router_dtype == DType.F16
+              else (r32.view(np.uint32) >> 16).astype(np.uint16)).view(np.uint8)
+    x = synth_normal_f32(414 + rows, rows * ne)
+    xb, rb = be.upload_new(x), be.upload_new(router)
+    gb, ub, db = be.upload_new(gate), be.upload_new(up), be.upload_new(down)
+    yb, ib, wb = be.alloc(rows * ne * 4), be.alloc(rows * n_used * 4), be.alloc(rows * n_used * 4)
+    be.moe_ffn(xb, rb, gb, ub, db, yb, rows=rows, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
+               router_dtype=router_dtype, sel_idx=ib, sel_w=wb)
+    got = (be.download(yb, np.empty((rows, ne), np.float32)), be.download(ib, np.empty((rows, n_used), np.int32)),
+           be.download(wb, np.empty((rows, n_used), np.float32)))
+    want = orc.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
+                       router_dtype=int(router_dtype))
+    check(*got, *want)
+
+
 @pytest.mark.parametrize("rows", [1, 4, 40])     # 40 rows of 8 experts: the bucketed Q4_K gate beside the rest
 def test_moe_banks_of_three_different_kinds(be, rows):
     """gate Q4_K (per-256 activations), up Q5_0 (per-32), down Q4_0 (raw f32 rows) in one op: every

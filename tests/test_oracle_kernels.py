@@ -235,6 +235,28 @@ def test_dot_is_eight_lane_fma():
     assert orc.dot(a, b) == s
 
 
+@pytest.mark.parametrize("m", [1, 3])
+def test_linear_over_plain_rows_is_dot_over_the_widened_row(m):
+    # lib.rs:1162-1164, 1443-1462: F32 / F16 / BF16 weights go through dot / dot_f16 / dot_bf16, which
+    # widen each weight exactly (kernels.rs:6505-6549) and run dot's chains. Widened here by numpy
+    # (float16 -> float32) and by bit arithmetic (bf16 = the top half of the f32 pattern), then fed
+    # to the eight-chain restatement pinned above: the three dtypes must give those bits.
+    in_f, out_f = 104, 5      # 13 chunks of eight: chains and no tail; a tail is covered above
+    rng = np.random.default_rng(5)
+    w = (rng.standard_normal(out_f * in_f) * 0.05).astype(np.float32)
+    x = rng.standard_normal(m * in_f).astype(np.float32)
+    f16 = w.astype(np.float16)
+    bf16 = (w.view(np.uint32) >> 16).astype(np.uint16)
+    cases = [(orc.F32, w.view(np.uint8), w),
+             (orc.F16, f16.view(np.uint8), f16.astype(np.float32)),
+             (orc.BF16, bf16.view(np.uint8), (bf16.astype(np.uint32) << 16).view(np.float32))]
+    for dtype, raw, widened in cases:
+        got = orc.linear(dtype, raw, x, m, in_f, out_f).reshape(m, out_f)
+        for r in range(m):
+            for o in range(out_f):
+                assert got[r, o] == orc.dot(widened[o * in_f:(o + 1) * in_f], x[r * in_f:(r + 1) * in_f])
+
+
 # ───────────── Op::Linear: the reference's op-level sweep ─────────────
 
 # position of each format in WEIGHT_QUANTS (decode_spec.rs:255-280) -> testkit seed 0x201 + i
