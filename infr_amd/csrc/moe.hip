@@ -896,8 +896,7 @@ __global__ __launch_bounds__(1024) void moe_down_fused_kernel(
     F::load_acts(acts, a, 0, lane, q / nb < 16 / nb);
     gemv_rows_folded<F, false>(w, bpr, nb, acts, yk - row0, row0, row_end, lane, osum, &first);
     __syncthreads();
-    const int o = (int)threadIdx.x;
-    if (o < row_end - row0) {
+    for (int o = (int)threadIdx.x; o < row_end - row0; o += (int)blockDim.x) {  // (one expert per token: 64 threads)
         float acc = 0.0f;
         for (int j = 0; j < n_used; ++j) {
             const float* yj = reinterpret_cast<const float*>(dlds + (size_t)j * wave_bytes + y_off);

@@ -305,6 +305,19 @@ def test_moe_banks_of_plain_float_rows(be, dtype, rows):
     check(*got, *want)
 
 
+def test_moe_one_expert_per_token_with_tall_down_tiles(be):
+    """n_used == 1 gives the fused down launch one wave per workgroup; with 130 tokens of a 4096-wide
+    model its tiles are 128 output rows tall, more than that workgroup has threads: the weighted
+    sum has to walk them."""
+    rows, ne, n_expert, n_used, nff = 130, 4096, 72, 1, 256
+    gate, up, down = banks(420, ne, n_expert, nff, sigma=0.05)
+    x = synth_normal_f32(421, rows * ne)
+    router = synth_normal_f32(422, n_expert * ne, sigma=0.02)
+    got = run_moe(be, x, router, gate, up, down, rows, ne, n_expert, n_used, nff, 1.0)
+    want = orc.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff)
+    check(*got, *want)
+
+
 @pytest.mark.parametrize("rows", [1, 3, 300])      # 300: the register-tiled router
 @pytest.mark.parametrize("router_dtype", [DType.F16, DType.BF16])
 def test_moe_router_weights_in_half_precision(be, router_dtype, rows):
