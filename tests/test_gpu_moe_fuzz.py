@@ -42,11 +42,14 @@ def bank(dtype, seed, rows, in_f):
 
 
 def draw_case(rng):
-    ne = 256 * int(rng.integers(1, 5))
-    nff = 256 * int(rng.integers(1, 4))
-    n_expert = int(rng.choice([2, 4, 8, 16, 32, 48]))
-    n_used = int(rng.choice([u for u in (1, 2, 3, 4, 8, 20, 32) if u <= n_expert]))
-    rows = int(rng.choice([1, 1, 2, 3, 4, 5, 8, 9, 16, 17, 31, 33, 48, 64, 70]))
+    while True:
+        ne = int(rng.choice([256, 512, 768, 1024, 1024, 2048, 4096]))
+        nff = 256 * int(rng.integers(1, 4))
+        n_expert = int(rng.choice([2, 4, 8, 16, 32, 48, 72, 128]))
+        if n_expert * nff * ne <= 1 << 24:      # banks of at most 16 M weights each
+            break
+    n_used = int(rng.choice([u for u in (1, 1, 2, 3, 4, 8, 20, 32) if u <= n_expert]))
+    rows = int(rng.choice([1, 1, 2, 3, 4, 5, 8, 9, 16, 17, 31, 33, 48, 64, 70, 130, 200]))
     if rng.integers(2):
         dts = (BANK_FORMATS[rng.integers(len(BANK_FORMATS))],) * 3          # one format, as most files have
     else:
