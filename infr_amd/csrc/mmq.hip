@@ -635,6 +635,7 @@ static void launch_mmq_skinny_q4k(const uint8_t* w, size_t bpr, const ActQ8& act
 // half tile, staged in LDS), token r16's codes and per-32 sums as A operands, and returns
 // sd = sum_s sc_s * (q . q8) and sm = sum_s m_s * bsum_s for tokens 4kq .. 4kq + 3 of row r16.
 struct Skinny16Q4K {
+    static constexpr bool kSubScales = false;
     static constexpr int kBlockBytes = 144;
     // Q4_K: the scale split sc = 8 hi + lo folded into two operand sets, two chains of four K = 64 steps
     static constexpr int kRowStride = 2 * kBlockBytes + 16;  // two blocks, padded: eight rows' 16-byte reads cover all banks
@@ -702,6 +703,7 @@ struct Skinny16Q4K {
 // v_mfma_i32_16x16x32_i8 (lane (., kq): elements 8kq .. 8kq + 7) scaled into sd by a 24-bit
 // multiply-add; sm and the epilogue are Q4_K's.
 struct Skinny16Q5K {
+    static constexpr bool kSubScales = false;
     static constexpr int kBlockBytes = 176;
     static constexpr int kRowStride = 2 * kBlockBytes + 16;
     __device__ static float accumulate(float acc, float dq, uint32_t ddm, int sd, float sm) {
@@ -752,6 +754,7 @@ struct Skinny16Q5K {
 // multiply-add. A stage of two blocks is 420 bytes from a 4-byte boundary, so its second block sits
 // 2 bytes off a boundary in LDS: it is read as aligned words and shifted in registers.
 struct Skinny16Q6K {
+    static constexpr bool kSubScales = false;
     typedef int v2i __attribute__((ext_vector_type(2)));
     static constexpr int kBlockBytes = 210;
     static constexpr int kRowStride = 432;  // 420 rounded up to 16: 108 words, eight rows' reads cover all banks
@@ -814,6 +817,57 @@ struct Skinny16Q6K {
         else block_at<false>(wrow + jj * kBlockBytes, arow, zrow, kq, sd, ddm);
 #pragma unroll
         for (int i = 0; i < 4; ++i) sm[i] = 0.0f;
+    }
+};
+
+// Q8_0 (34-byte blocks: f16 d, 32 int8 codes; crates/infr-cpu/src/kernels.rs:1170-1187): a 256-element
+// step is eight blocks, 272 bytes, each with a scale of its own. The stored codes are the operand:
+// one v_mfma_i32_16x16x32_i8 per block gives its exact iprod, and the f32 side is the CPU's chain
+// `sumf += (q8.d[b] * d_w) * (iprod as f32)` block by block - so these outputs equal infr-cpu's
+// scalar kernel bit for bit, which the dot4 batches (a fixed tree over the lanes) do not.
+// kSubScales: a step's integers are 8 x 4 (block s, output i at [4 s + i]) and `ddm` its eight
+// scales, two to a word. Blocks start 2 bytes off a word boundary on every other block: those codes
+// are read as aligned words and shifted.
+struct Skinny16Q8_0 {
+    typedef int v2i __attribute__((ext_vector_type(2)));
+    static constexpr bool kSubScales = true;
+    static constexpr int kBlockBytes = 272;
+    static constexpr int kRowStride = 2 * kBlockBytes + 16;  // 140 words: eight rows' 16-byte reads cover all banks
+    __device__ static void block(const uint8_t* wrow, int jj, const uint8_t* arow, int kq, int (&ip)[32],
+                                 uint32_t (&dw)[4]) {
+        const uint8_t* blk = wrow + jj * kBlockBytes;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const uint8_t* sb = blk + s * 34;
+            v2i b;
+            if (s & 1) {  // codes at 34 s + 2 + 8 kq: a word boundary
+                b.x = *reinterpret_cast<const int*>(sb + 2 + 8 * kq);
+                b.y = *reinterpret_cast<const int*>(sb + 6 + 8 * kq);
+            } else {      // two bytes past one
+                const int w0 = *reinterpret_cast<const int*>(sb + 8 * kq);
+                const int w1 = *reinterpret_cast<const int*>(sb + 4 + 8 * kq);
+                const int w2 = *reinterpret_cast<const int*>(sb + 8 + 8 * kq);
+                b.x = (int)__builtin_amdgcn_alignbyte((uint32_t)w1, (uint32_t)w0, 2);
+                b.y = (int)__builtin_amdgcn_alignbyte((uint32_t)w2, (uint32_t)w1, 2);
+            }
+            const v2i a = *reinterpret_cast<const v2i*>(arow + s * 32 + 8 * kq);
+            const v4i r = __builtin_amdgcn_mfma_i32_16x16x32_i8(__builtin_bit_cast(long, a), __builtin_bit_cast(long, b),
+                                                                v4i{0, 0, 0, 0}, 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) ip[4 * s + i] = r[i];
+            const uint32_t d16 = *reinterpret_cast<const uint16_t*>(sb);
+            if (s & 1) dw[s >> 1] |= d16 << 16;
+            else dw[s >> 1] = d16;
+        }
+    }
+    // sumf += (q8.d[b] * d_w) * (iprod as f32), the step's eight blocks in order
+    __device__ static void accumulate(float (&acc)[4], const float (&dq)[4], const uint32_t (&dw)[4], const int (&ip)[32]) {
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const float d = f16_bits_to_f32((dw[s >> 1] >> (16 * (s & 1))) & 0xFFFFu);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] += (dq[i] * d) * (float)ip[4 * s + i];
+        }
     }
 };
 
@@ -943,9 +997,10 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
             for (int it = 0; it < (MT * BPW + 63) / 64; ++it)
                 if (lane + 64 * it < MT * BPW) (&dq_l[wave][0][0])[lane + 64 * it] = dsrc[dqoff[it]];
         }
-        int sd[BPW][4];
+        constexpr bool kSub = F::kSubScales;  // a step's integers: one per output, or one per 32-block and output
+        int sd[BPW][kSub ? 32 : 4];
         float sm[BPW][4];
-        uint32_t ddm[BPW];  // (d, dmin) of this lane's row
+        uint32_t ddm[BPW][kSub ? 4 : 1];  // (d, dmin) of this lane's row, or the step's eight block scales
 #pragma unroll
         for (int j = 0; j < BPW; ++j) {
             wave_sync();  // the previous block's operand reads are done
@@ -957,14 +1012,21 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
                 if (pass + 1 < n_pass) request_rows(b0_next);
             }
             wave_sync();
-            F::block(wfrag, j % kPh, afrag, zrow, bsfrag, kq, sd[j], sm[j], ddm[j]);
+            if constexpr (kSub) F::block(wfrag, j % kPh, afrag, kq, sd[j], ddm[j]);
+            else F::block(wfrag, j % kPh, afrag, zrow, bsfrag, kq, sd[j], sm[j], ddm[j][0]);
             if (STAGES) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int tok = 4 * kq + i;
                     if (row_ok && tok < m && b0 + j < nb) {
-                        st_sd[((size_t)tok * out_f + wrow) * nb + b0 + j] = sd[j][i];
-                        if (st_sm) st_sm[((size_t)tok * out_f + wrow) * nb + b0 + j] = (int)sm[j][i];
+                        if constexpr (kSub) {
+#pragma unroll
+                            for (int s8 = 0; s8 < 8; ++s8)
+                                st_sd[((size_t)tok * out_f + wrow) * ((size_t)nb * 8) + (size_t)(b0 + j) * 8 + s8] = sd[j][4 * s8 + i];
+                        } else {
+                            st_sd[((size_t)tok * out_f + wrow) * nb + b0 + j] = sd[j][i];
+                            if (st_sm) st_sm[((size_t)tok * out_f + wrow) * nb + b0 + j] = (int)sm[j][i];
+                        }
                     }
                 }
             }
@@ -983,9 +1045,16 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
 #pragma unroll
                 for (int j = 0; j < BPW; ++j) {
                     if (b0 + j < nb) {
+                        if constexpr (kSub) {
+                            float dqv[4];
 #pragma unroll
-                        for (int i = 0; i < 4; ++i)
-                            acc[i] = F::accumulate(acc[i], dq_l[wave][(4 * kq + i) & (MT - 1)][j], ddm[j], sd[j][i], sm[j][i]);
+                            for (int i = 0; i < 4; ++i) dqv[i] = dq_l[wave][(4 * kq + i) & (MT - 1)][j];
+                            F::accumulate(acc, dqv, ddm[j], sd[j]);
+                        } else {
+#pragma unroll
+                            for (int i = 0; i < 4; ++i)
+                                acc[i] = F::accumulate(acc[i], dq_l[wave][(4 * kq + i) & (MT - 1)][j], ddm[j][0], sd[j][i], sm[j][i]);
+                        }
                     }
                 }
                 if (k + 1 < NW || pass + 1 < n_pass)
@@ -1002,13 +1071,18 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
     }
 }
 
-// Which batches the 16-token K-split kernel takes: Q4_K, Q5_K and Q6_K rows of an even number of
+// Which batches the 16-token K-split kernel takes: Q4_K, Q5_K, Q6_K and Q8_0 rows of an even number of
 // 256-blocks (weights are staged two blocks at a time), up to 16 tokens. Four waves per workgroup;
 // (eight measured no faster, and four blocks per wave and pass - 576-byte, 64-byte-aligned runs per
 // row - measured 20-25 % slower: a wave then computes for longer before it asks for more).
 constexpr int kSkinny16Waves = 4, kSkinny16Blocks = 2;
 static bool skinny16_shape(int dtype, int nb, size_t m) {
-    if ((dtype != 12 && dtype != 13 && dtype != 14) || m > 16) return false;
+    if ((dtype != 12 && dtype != 13 && dtype != 14 && dtype != 8) || m > 16) return false;
+    // Q8_0: the dot4 batches stay ahead up to eight tokens on rows of one or two wave steps (4.2 / 3.8 /
+    // 4.8 against 3.8 / 3.3 / 4.2 TB/s at eight tokens on the 4096-column shapes, 5.1-5.9 at two to
+    // four); this kernel takes 9..16 tokens (one pass over the weights instead of two) and, from
+    // five tokens, rows of 8192 columns and more (4.4 against 3.95 TB/s at 4096 x 12288)
+    if (dtype == 8 && !(m > 8 || (m >= 5 && nb >= 32))) return false;
     // the dot4 batch kernels, which unpack a weight once per two or four tokens, stay ahead at the
     // bottom: Q5_K at two tokens (4.3-5.3 against 3.8-4.4 TB/s), Q6_K up to four (3.6-4.5 against 3.3-3.9)
     if ((dtype == 13 && m < 3) || (dtype == 14 && m < 5)) return false;
@@ -1042,6 +1116,8 @@ static bool launch_mmq_skinny16(int dtype, const uint8_t* w, size_t bpr, const A
         launch_mmq_skinny16_fmt<Skinny16Q4K, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     else if (dtype == 13)
         launch_mmq_skinny16_fmt<Skinny16Q5K, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
+    else if (dtype == 8)
+        launch_mmq_skinny16_fmt<Skinny16Q8_0, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     else
         launch_mmq_skinny16_fmt<Skinny16Q6K, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     return true;

@@ -220,6 +220,23 @@ def test_small_batch_kquant_mfma_is_bit_identical_to_oracle(be, dtype, m, in_f, 
     assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), "not bit-identical"
 
 
+@pytest.mark.parametrize("m,in_f,out_f", [(9, 4096, 48), (13, 512, 40), (16, 5632, 24), (12, 1024, 70), (6, 8192, 40),
+                                          (5, 12288, 33)])
+def test_q8_0_on_the_sixteen_token_mfma_kernel_is_bit_identical_to_oracle(be, m, in_f, out_f):
+    """9..16 tokens of Q8_0 (and 5..8 on rows of 8192 columns up) take the K-split MFMA kernel: one
+    exact iprod per 34-byte block and the CPU's chain `sumf += (q8.d * d_w) * iprod` block by block
+    (crates/infr-cpu/src/kernels.rs:1170-1187) handed from wave to wave, so unlike the dot4 batches
+    these outputs equal the scalar kernel's bits; the per-block integers are exact as everywhere."""
+    w = orc.synth_weight(DType.Q8_0, in_f * out_f, 0x20C)
+    x = orc.gen_f32(m * in_f, 0x20C ^ 0x9E37)
+    y = run_linear(be, DType.Q8_0, w, x, m, in_f, out_f)
+    want = orc.linear(DType.Q8_0, w, x, m, in_f, out_f)
+    assert np.array_equal(y.view(np.uint32), want.reshape(m, out_f).view(np.uint32)), "not bit-identical"
+    a, _ = be.linear_int_stages(DType.Q8_0, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
+    oa, _ = orc.linear_int_stages(DType.Q8_0, w, x, m, in_f, out_f)
+    assert np.array_equal(a, oa)
+
+
 @pytest.mark.parametrize("m,in_f,out_f", [(6, 4608, 40), (13, 1024, 50)])
 @pytest.mark.parametrize("dtype,seed", [(DType.Q4K, 0x209), (DType.Q5K, 0x20A), (DType.Q6K, 0x20B)])
 def test_small_batch_kquant_mfma_int_stages_bit_exact(be, dtype, seed, m, in_f, out_f):
