@@ -635,6 +635,7 @@ static void launch_mmq_skinny_q4k(const uint8_t* w, size_t bpr, const ActQ8& act
 // half tile, staged in LDS), token r16's codes and per-32 sums as A operands, and returns
 // sd = sum_s sc_s * (q . q8) and sm = sum_s m_s * bsum_s for tokens 4kq .. 4kq + 3 of row r16.
 struct Skinny16Q4K {
+    static constexpr bool kPer32Acts = false, kTranspose16 = false;
     static constexpr bool kSubScales = false;
     static constexpr int kBlockBytes = 144;
     // Q4_K: the scale split sc = 8 hi + lo folded into two operand sets, two chains of four K = 64 steps
@@ -703,6 +704,7 @@ struct Skinny16Q4K {
 // v_mfma_i32_16x16x32_i8 (lane (., kq): elements 8kq .. 8kq + 7) scaled into sd by a 24-bit
 // multiply-add; sm and the epilogue are Q4_K's.
 struct Skinny16Q5K {
+    static constexpr bool kPer32Acts = false, kTranspose16 = false;
     static constexpr bool kSubScales = false;
     static constexpr int kBlockBytes = 176;
     static constexpr int kRowStride = 2 * kBlockBytes + 16;
@@ -754,6 +756,7 @@ struct Skinny16Q5K {
 // multiply-add. A stage of two blocks is 420 bytes from a 4-byte boundary, so its second block sits
 // 2 bytes off a boundary in LDS: it is read as aligned words and shifted in registers.
 struct Skinny16Q6K {
+    static constexpr bool kPer32Acts = false, kTranspose16 = false;
     static constexpr bool kSubScales = false;
     typedef int v2i __attribute__((ext_vector_type(2)));
     static constexpr int kBlockBytes = 210;
@@ -829,6 +832,7 @@ struct Skinny16Q6K {
 // scales, two to a word. Blocks start 2 bytes off a word boundary on every other block: those codes
 // are read as aligned words and shifted.
 struct Skinny16Q8_0 {
+    static constexpr bool kPer32Acts = false, kTranspose16 = false;
     typedef int v2i __attribute__((ext_vector_type(2)));
     static constexpr bool kSubScales = true;
     static constexpr int kBlockBytes = 272;
@@ -871,6 +875,73 @@ struct Skinny16Q8_0 {
     }
 };
 
+// Q2_0 (18-byte blocks of 64: f16 d, 16 bytes of 2-bit codes; crates/infr-cpu/src/kernels.rs:5641-5668)
+// against the per-32 activation: a 256-element step is four blocks, 72 bytes, and eight 32-element
+// halves, each with its own activation scale and code sum. `(word >> 2 i) & 0x03030303` is codes
+// i, 4 + i, 8 + i, 12 + i of a word's sixteen, so the activation tile holds every 16 codes 4 x 4
+// transposed (kTranspose16: done in registers on the way into LDS) and a half is one
+// v_mfma_i32_16x16x32_i8 after two shifts and two masks. The lane turns each half's exact integer
+// into the CPU's f32 term `(d * q8.d[s]) * (iprod - bsum[s]) as f32` at once (both integers and their
+// difference are exact in f32) - the scales and sums of its four output tokens are in LDS then -
+// and the wave-to-wave chain adds the terms in block order: infr-cpu's bits. `ip` carries the
+// terms' bit patterns; `raw` the integers for the stage outputs.
+struct Skinny16Q2_0 {
+    typedef int v2i __attribute__((ext_vector_type(2)));
+    static constexpr bool kSubScales = true, kPer32Acts = true, kTranspose16 = true;
+    static constexpr int kBlockBytes = 72;
+    static constexpr int kRowStride = 2 * kBlockBytes;  // 36 words: eight rows' 16-byte reads cover all banks
+    template <int MT, int DQ_STRIDE>
+    __device__ static void block(const uint8_t* wrow, int jj, const uint8_t* arow, const uint8_t* bs_base,
+                                 const float* dq_base, int kq, int (&ip)[32], int (&raw)[32]) {
+        const uint8_t* blk = wrow + jj * kBlockBytes;
+        const int i0 = 2 * (kq & 1);
+        // this lane's output tokens 4 kq .. 4 kq + 3: their eight scales and eight code sums of the step
+        v4f dq[4][2];
+        v4i bs[4][2];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int tok = (4 * kq + i) & (MT - 1);
+            dq[i][0] = *reinterpret_cast<const v4f*>(dq_base + tok * DQ_STRIDE + jj * 8);
+            dq[i][1] = *reinterpret_cast<const v4f*>(dq_base + tok * DQ_STRIDE + jj * 8 + 4);
+            bs[i][0] = *reinterpret_cast<const v4i*>(bs_base + tok * 32);
+            bs[i][1] = *reinterpret_cast<const v4i*>(bs_base + tok * 32 + 16);
+        }
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const int q = s >> 1;  // the half's 64-block
+            const int off = 18 * q + 2 + 8 * (s & 1) + 4 * (kq >> 1);  // this lane's word of the half's codes
+            uint32_t cw;
+            if (q & 1) {
+                cw = *reinterpret_cast<const uint32_t*>(blk + off);
+            } else {  // 2 bytes past a word boundary
+                const uint32_t w0 = *reinterpret_cast<const uint32_t*>(blk + off - 2);
+                const uint32_t w1 = *reinterpret_cast<const uint32_t*>(blk + off + 2);
+                cw = __builtin_amdgcn_alignbyte(w1, w0, 2);
+            }
+            v2i b;
+            b.x = (int)((cw >> (2 * i0)) & 0x03030303u);
+            b.y = (int)((cw >> (2 * i0 + 2)) & 0x03030303u);
+            const v2i a = *reinterpret_cast<const v2i*>(arow + s * 32 + 8 * kq);
+            const v4i r = __builtin_amdgcn_mfma_i32_16x16x32_i8(__builtin_bit_cast(long, a), __builtin_bit_cast(long, b),
+                                                                v4i{0, 0, 0, 0}, 0, 0, 0);
+            const float d = f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(blk + 18 * q));
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                raw[4 * s + i] = r[i];
+                const float term = (d * dq[i][s >> 2][s & 3]) * (float)(r[i] - bs[i][s >> 2][s & 3]);
+                ip[4 * s + i] = __builtin_bit_cast(int, term);
+            }
+        }
+    }
+    // sumf += term, the step's eight halves in order
+    __device__ static void accumulate(float (&acc)[4], const float (&)[4], const uint32_t (&)[4], const int (&ip)[32]) {
+#pragma unroll
+        for (int s = 0; s < 8; ++s)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] += __builtin_bit_cast(float, ip[4 * s + i]);
+    }
+};
+
 template <typename F, int NW, int BPW, int MT, bool STAGES>
 __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
     const uint8_t* __restrict__ w, size_t bpr, const int8_t* __restrict__ qs,
@@ -890,7 +961,8 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
     constexpr int kPieces = kFull + (kTail ? 1 : 0), kIt = (kPieces + 3) / 4;
     __shared__ __attribute__((aligned(16))) uint8_t w_l[NW][16 * kRowStride];
     __shared__ __attribute__((aligned(16))) uint8_t act_l[NW][kTileBytes];
-    __shared__ __attribute__((aligned(16))) float dq_l[NW][MT][BPW];
+    constexpr int kDq = BPW * (F::kPer32Acts ? 8 : 1);  // activation scales per token and pass: per 256 or per 32
+    __shared__ __attribute__((aligned(16))) float dq_l[NW][MT][kDq];
     __shared__ __attribute__((aligned(16))) float chain_l[64][4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r16 = lane & 15, kq = lane >> 4;
@@ -909,7 +981,7 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
         row_ok = rt < (int)t.rows;
         any_row = (int)blockIdx.y * 16 < (int)t.rows;
         qs += t.act_elem0;
-        d8 += t.act_elem0 / 256;
+        d8 += t.act_elem0 / (F::kPer32Acts ? 32 : 256);
         bsums += t.act_elem0 / 32;
     }
     if (!any_row) return;  // uniform over the workgroup, before any barrier
@@ -962,7 +1034,16 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
 #pragma unroll
         for (int it = 0; it < MT / 4; ++it) {
             const int chunk = lane + 64 * it;
-            *reinterpret_cast<v4i*>(tile + (chunk >> 4) * kTokStride + (chunk & 15) * 16) = areg[it];
+            v4i piece = areg[it];
+            if constexpr (F::kTranspose16) {
+                // the piece's 16 codes 4 x 4 transposed: word i = codes i, 4 + i, 8 + i, 12 + i
+                const uint32_t d0 = (uint32_t)piece.x, d1 = (uint32_t)piece.y, d2 = (uint32_t)piece.z, d3 = (uint32_t)piece.w;
+                const uint32_t a = __builtin_amdgcn_perm(d1, d0, 0x05010400u), b = __builtin_amdgcn_perm(d1, d0, 0x07030602u);
+                const uint32_t c = __builtin_amdgcn_perm(d3, d2, 0x05010400u), d = __builtin_amdgcn_perm(d3, d2, 0x07030602u);
+                piece = v4i{(int)__builtin_amdgcn_perm(c, a, 0x05040100u), (int)__builtin_amdgcn_perm(c, a, 0x07060302u),
+                            (int)__builtin_amdgcn_perm(d, b, 0x05040100u), (int)__builtin_amdgcn_perm(d, b, 0x07060302u)};
+            }
+            *reinterpret_cast<v4i*>(tile + (chunk >> 4) * kTokStride + (chunk & 15) * 16) = piece;
         }
         if (lane < MT * 2) *reinterpret_cast<v4i*>(tile + kBsOff + lane * 16) = bsreg;
     };
@@ -984,6 +1065,10 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
         const int i = lane + 64 * it;
         dqoff[it] = (uint32_t)min(i / BPW, m - 1) * (uint32_t)nb + i % BPW;
     }
+    // per-32 activations: a pass's scales of a token are 8 BPW consecutive floats, four to a lane
+    constexpr int kDqQuads = BPW * 2;  // 16-byte pieces per token and pass
+    const uint32_t dq32off = (uint32_t)min(lane / kDqQuads, m - 1) * (uint32_t)(nb * 8) + (lane % kDqQuads) * 4;
+    static_assert(!F::kPer32Acts || MT * kDqQuads <= 64, "one 16-byte piece of scales per lane");
     request_rows(wave * BPW);
     request_acts(wave * BPW);
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // this lane's outputs: tokens 4kq .. 4kq + 3 of row r16
@@ -991,7 +1076,11 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
         const int b0 = (pass * NW + wave) * BPW;
         const int b0_next = b0 + NW * BPW;  // next pass (past the end: clamped, never used)
         // the activation scales of the wave's blocks: dq_l[token][j]
-        {
+        if constexpr (F::kPer32Acts) {
+            if (lane < MT * kDqQuads)
+                *reinterpret_cast<v4f*>(&dq_l[wave][0][0] + lane * 4) =
+                    *reinterpret_cast<const v4f*>(d8 + (size_t)min(b0, nb - BPW) * 8 + dq32off);
+        } else {
             const float* dsrc = d8 + min(b0, nb - BPW);
 #pragma unroll
             for (int it = 0; it < (MT * BPW + 63) / 64; ++it)
@@ -1012,7 +1101,10 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
                 if (pass + 1 < n_pass) request_rows(b0_next);
             }
             wave_sync();
-            if constexpr (kSub) F::block(wfrag, j % kPh, afrag, kq, sd[j], ddm[j]);
+            int raw[kSub && F::kPer32Acts ? 32 : 1];  // the integers behind a policy's f32 terms (stage outputs)
+            if constexpr (kSub && F::kPer32Acts)
+                F::template block<MT, kDq>(wfrag, j % kPh, afrag, tile + kBsOff, &dq_l[wave][0][0], kq, sd[j], raw);
+            else if constexpr (kSub) F::block(wfrag, j % kPh, afrag, kq, sd[j], ddm[j]);
             else F::block(wfrag, j % kPh, afrag, zrow, bsfrag, kq, sd[j], sm[j], ddm[j][0]);
             if (STAGES) {
 #pragma unroll
@@ -1022,7 +1114,8 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
                         if constexpr (kSub) {
 #pragma unroll
                             for (int s8 = 0; s8 < 8; ++s8)
-                                st_sd[((size_t)tok * out_f + wrow) * ((size_t)nb * 8) + (size_t)(b0 + j) * 8 + s8] = sd[j][4 * s8 + i];
+                                st_sd[((size_t)tok * out_f + wrow) * ((size_t)nb * 8) + (size_t)(b0 + j) * 8 + s8] =
+                                    F::kPer32Acts ? raw[F::kPer32Acts ? 4 * s8 + i : 0] : sd[j][4 * s8 + i];
                         } else {
                             st_sd[((size_t)tok * out_f + wrow) * nb + b0 + j] = sd[j][i];
                             if (st_sm) st_sm[((size_t)tok * out_f + wrow) * nb + b0 + j] = (int)sm[j][i];
@@ -1071,18 +1164,21 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
     }
 }
 
-// Which batches the 16-token K-split kernel takes: Q4_K, Q5_K, Q6_K and Q8_0 rows of an even number of
+// Which batches the 16-token K-split kernel takes: Q4_K, Q5_K, Q6_K, Q8_0 and Q2_0 rows of an even number of
 // 256-blocks (weights are staged two blocks at a time), up to 16 tokens. Four waves per workgroup;
 // (eight measured no faster, and four blocks per wave and pass - 576-byte, 64-byte-aligned runs per
 // row - measured 20-25 % slower: a wave then computes for longer before it asks for more).
 constexpr int kSkinny16Waves = 4, kSkinny16Blocks = 2;
 static bool skinny16_shape(int dtype, int nb, size_t m) {
-    if ((dtype != 12 && dtype != 13 && dtype != 14 && dtype != 8) || m > 16) return false;
+    if ((dtype != 12 && dtype != 13 && dtype != 14 && dtype != 8 && dtype != 42) || m > 16) return false;
     // Q8_0: the dot4 batches stay ahead up to eight tokens on rows of one or two wave steps (4.2 / 3.8 /
     // 4.8 against 3.8 / 3.3 / 4.2 TB/s at eight tokens on the 4096-column shapes, 5.1-5.9 at two to
     // four); this kernel takes 9..16 tokens (one pass over the weights instead of two) and, from
     // five tokens, rows of 8192 columns and more (4.4 against 3.95 TB/s at 4096 x 12288)
     if (dtype == 8 && !(m > 8 || (m >= 5 && nb >= 32))) return false;
+    // Q2_0: 72 bytes a step make this kernel compute-bound (1.0-1.3 TB/s at any token count, what the
+    // dot4 batches reach at eight tokens): it takes 9..16 tokens, where they would need two passes
+    if (dtype == 42 && m <= 8) return false;
     // the dot4 batch kernels, which unpack a weight once per two or four tokens, stay ahead at the
     // bottom: Q5_K at two tokens (4.3-5.3 against 3.8-4.4 TB/s), Q6_K up to four (3.6-4.5 against 3.3-3.9)
     if ((dtype == 13 && m < 3) || (dtype == 14 && m < 5)) return false;
@@ -1118,6 +1214,8 @@ static bool launch_mmq_skinny16(int dtype, const uint8_t* w, size_t bpr, const A
         launch_mmq_skinny16_fmt<Skinny16Q5K, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     else if (dtype == 8)
         launch_mmq_skinny16_fmt<Skinny16Q8_0, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
+    else if (dtype == 42)
+        launch_mmq_skinny16_fmt<Skinny16Q2_0, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     else
         launch_mmq_skinny16_fmt<Skinny16Q6K, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     return true;

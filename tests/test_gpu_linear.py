@@ -237,6 +237,21 @@ def test_q8_0_on_the_sixteen_token_mfma_kernel_is_bit_identical_to_oracle(be, m,
     assert np.array_equal(a, oa)
 
 
+@pytest.mark.parametrize("m,in_f,out_f", [(9, 4096, 48), (13, 512, 40), (16, 5632, 24), (12, 1024, 70), (11, 12288, 33)])
+def test_q2_0_on_the_sixteen_token_mfma_kernel_is_bit_identical_to_oracle(be, m, in_f, out_f):
+    """9..16 tokens of Q2_0 on the K-split MFMA kernel: one exact iprod per 32-element half against
+    the per-32 activation, the CPU's term `(d * q8.d[s]) * (iprod - bsum[s])` per half and its chain
+    in block order (crates/infr-cpu/src/kernels.rs:5641-5668): the scalar kernel's bits."""
+    w = orc.synth_weight(DType.Q2_0, in_f * out_f, 0x20D)
+    x = orc.gen_f32(m * in_f, 0x20D ^ 0x9E37)
+    y = run_linear(be, DType.Q2_0, w, x, m, in_f, out_f)
+    want = orc.linear(DType.Q2_0, w, x, m, in_f, out_f)
+    assert np.array_equal(y.view(np.uint32), want.reshape(m, out_f).view(np.uint32)), "not bit-identical"
+    a, _ = be.linear_int_stages(DType.Q2_0, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
+    oa, _ = orc.linear_int_stages(DType.Q2_0, w, x, m, in_f, out_f)
+    assert np.array_equal(a, oa)
+
+
 @pytest.mark.parametrize("m,in_f,out_f", [(6, 4608, 40), (13, 1024, 50)])
 @pytest.mark.parametrize("dtype,seed", [(DType.Q4K, 0x209), (DType.Q5K, 0x20A), (DType.Q6K, 0x20B)])
 def test_small_batch_kquant_mfma_int_stages_bit_exact(be, dtype, seed, m, in_f, out_f):
