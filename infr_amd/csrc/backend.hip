@@ -272,7 +272,7 @@ static bool runs_alone(int dtype, size_t m, size_t in_f) {
 static bool small_batch(const infr_hip_op_t& op) {
     if (op.m < 2 || is_plain(op.w_dtype) || infr::gemv_row_too_long(op.w_dtype, op.in_f)) return false;
     if (op.w_dtype == INFR_DTYPE_Q4_K) return op.m <= 32;
-    return op.m <= 8 || infr::mmq_skinny16_takes(op.w_dtype, op.m, op.in_f);
+    return op.m <= 8 || infr::mmq_skinny16_takes(op.w_dtype, op.m, op.in_f, op.out_f);
 }
 
 // (Re)allocates a device table when it grew and enqueues the copy on the backend stream.

@@ -144,7 +144,7 @@ void launch_mmq_skinny_group(int dtype, size_t m, size_t in_f, const BatchTile* 
                              const BatchGroupPlan& plan, const ActQ8& act, hipStream_t stream);
 // Q4_K / Q5_K batches of 2..16 tokens on rows of an even number of 256-blocks: the K-split MFMA
 // kernel with 16 x 16 tiles (mmq.hip) takes them, alone or as a plan's group of 32-row tiles.
-bool mmq_skinny16_takes(int dtype, size_t m, size_t in_f);
+bool mmq_skinny16_takes(int dtype, size_t m, size_t in_f, size_t out_f);
 
 // Which activation quantizer infr-cpu's dispatch pairs with a weight format
 // (crates/infr-cpu/src/lib.rs:1037-1076, 1322-1412): per-32 `Q8x32` for the 32-weight-block

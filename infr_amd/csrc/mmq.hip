@@ -966,6 +966,7 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
     __shared__ __attribute__((aligned(16))) float chain_l[64][4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r16 = lane & 15, kq = lane >> 4;
+    const int tok0 = (int)blockIdx.z * 16;  // batches beyond 16 tokens: one pass over the weights per 16
     const int rt = blockIdx.y * 16 + r16;  // row inside the 32-row tile
     const size_t in_f = (size_t)nb * 256;
     int wrow = blockIdx.x * 32 + rt;
@@ -1019,8 +1020,8 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
     v4i areg[MT / 4], bsreg = {0, 0, 0, 0};
     uint32_t aoff[MT / 4];
 #pragma unroll
-    for (int it = 0; it < MT / 4; ++it) aoff[it] = (uint32_t)min((lane >> 4) + 4 * it, m - 1) * (uint32_t)in_f + (lane & 15) * 16;
-    const uint32_t boff = (uint32_t)min(lane >> 1, m - 1) * (uint32_t)(nb * 32) + (lane & 1) * 16;
+    for (int it = 0; it < MT / 4; ++it) aoff[it] = (uint32_t)min(tok0 + (lane >> 4) + 4 * it, m - 1) * (uint32_t)in_f + (lane & 15) * 16;
+    const uint32_t boff = (uint32_t)min(tok0 + (lane >> 1), m - 1) * (uint32_t)(nb * 32) + (lane & 1) * 16;
     auto request_acts = [&](int b_) {
         const int b = min(b_, nb - 1);
         const int8_t* src = qs + (size_t)b * 256;
@@ -1063,11 +1064,11 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
 #pragma unroll
     for (int it = 0; it < (MT * BPW + 63) / 64; ++it) {
         const int i = lane + 64 * it;
-        dqoff[it] = (uint32_t)min(i / BPW, m - 1) * (uint32_t)nb + i % BPW;
+        dqoff[it] = (uint32_t)min(tok0 + i / BPW, m - 1) * (uint32_t)nb + i % BPW;
     }
     // per-32 activations: a pass's scales of a token are 8 BPW consecutive floats, four to a lane
     constexpr int kDqQuads = BPW * 2;  // 16-byte pieces per token and pass
-    const uint32_t dq32off = (uint32_t)min(lane / kDqQuads, m - 1) * (uint32_t)(nb * 8) + (lane % kDqQuads) * 4;
+    const uint32_t dq32off = (uint32_t)min(tok0 + lane / kDqQuads, m - 1) * (uint32_t)(nb * 8) + (lane % kDqQuads) * 4;
     static_assert(!F::kPer32Acts || MT * kDqQuads <= 64, "one 16-byte piece of scales per lane");
     request_rows(wave * BPW);
     request_acts(wave * BPW);
@@ -1109,7 +1110,7 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
             if (STAGES) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const int tok = 4 * kq + i;
+                    const int tok = tok0 + 4 * kq + i;
                     if (row_ok && tok < m && b0 + j < nb) {
                         if constexpr (kSub) {
 #pragma unroll
@@ -1159,7 +1160,7 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
     if (wave != NW - 1 || !row_ok) return;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const int tok = 4 * kq + i;
+        const int tok = tok0 + 4 * kq + i;
         if (tok < m) gstore<float>(y + (size_t)tok * out_f + wrow, acc[i]);
     }
 }
@@ -1169,31 +1170,52 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
 // (eight measured no faster, and four blocks per wave and pass - 576-byte, 64-byte-aligned runs per
 // row - measured 20-25 % slower: a wave then computes for longer before it asks for more).
 constexpr int kSkinny16Waves = 4, kSkinny16Blocks = 2;
-static bool skinny16_shape(int dtype, int nb, size_t m) {
-    if ((dtype != 12 && dtype != 13 && dtype != 14 && dtype != 8 && dtype != 42) || m > 16) return false;
-    // Q8_0: the dot4 batches stay ahead up to eight tokens on rows of one or two wave steps (4.2 / 3.8 /
-    // 4.8 against 3.8 / 3.3 / 4.2 TB/s at eight tokens on the 4096-column shapes, 5.1-5.9 at two to
-    // four); this kernel takes 9..16 tokens (one pass over the weights instead of two) and, from
-    // five tokens, rows of 8192 columns and more (4.4 against 3.95 TB/s at 4096 x 12288)
-    if (dtype == 8 && !(m > 8 || (m >= 5 && nb >= 32))) return false;
-    // Q2_0: 72 bytes a step make this kernel compute-bound (1.0-1.3 TB/s at any token count, what the
-    // dot4 batches reach at eight tokens): it takes 9..16 tokens, where they would need two passes
-    if (dtype == 42 && m <= 8) return false;
-    // the dot4 batch kernels, which unpack a weight once per two or four tokens, stay ahead at the
-    // bottom: Q5_K at two tokens (4.3-5.3 against 3.8-4.4 TB/s), Q6_K up to four (3.6-4.5 against 3.3-3.9)
-    if ((dtype == 13 && m < 3) || (dtype == 14 && m < 5)) return false;
-    return nb >= kSkinny16Blocks && nb % kSkinny16Blocks == 0;
+static bool skinny16_shape(int dtype, int nb, size_t m, size_t out_f) {
+    if (dtype != 12 && dtype != 13 && dtype != 14 && dtype != 8 && dtype != 42) return false;
+    if (nb < kSkinny16Blocks || nb % kSkinny16Blocks != 0) return false;
+    if (m <= 16) {
+        // the dot4 batch kernels, which unpack a weight once per two or four tokens, stay ahead at the
+        // bottom: Q5_K at two tokens (4.3-5.3 against 3.8-4.4 TB/s), Q6_K up to four (3.6-4.5 against 3.3-3.9)
+        if ((dtype == 13 && m < 3) || (dtype == 14 && m < 5)) return false;
+        // Q8_0: the dot4 batches stay ahead up to eight tokens on rows of one or two wave steps (4.2 / 3.8 /
+        // 4.8 against 3.8 / 3.3 / 4.2 TB/s at eight tokens on the 4096-column shapes, 5.1-5.9 at two to
+        // four); this kernel takes 9..16 tokens (one pass over the weights instead of two) and, from
+        // five tokens, rows of 8192 columns and more (4.4 against 3.95 TB/s at 4096 x 12288)
+        if (dtype == 8 && !(m > 8 || (m >= 5 && nb >= 32))) return false;
+        // Q2_0: 72 bytes a step make this kernel compute-bound (1.0-1.3 TB/s at any token count, what the
+        // dot4 batches reach at eight tokens): it takes 9 tokens and more, where they would need two passes
+        if (dtype == 42 && m <= 8) return false;
+        return true;
+    }
+    // Beyond 16 tokens the grid's third dimension walks the batch 16 tokens at a time (the weights
+    // then come once per 16 tokens, the later times from cache): taken while that beats what else
+    // the format has - dot4 passes of eight tokens up to 32 / 64 tokens, then a 128-token MFMA tile
+    // whose time is flat in the token count and has a floor of 26-42 us however small the matrix.
+    // Per op, us, at 12288 x 4096 / 4096 x 12288 / 4096 x 4096 / 1024 x 4096:
+    //   Q6_K  a 16-token pass 10.6 / 10.4 / 3.3 / 0.95; before: 68-114 at 17..32, then 61 / 102 / 40 / 40
+    //   Q5_K  9.2 / 8.8 / 2.9 / 0.8; 52-85, then 35 / 65 / 26 / 26
+    //   Q8_0  15.4 / 15.2 / 6.1 / 1.8; 51-71, then 46-50 / 73 / 30 / 28
+    //   Q2_0  12.5 / 10.7 / 4.1 / 1.2; 44-74 at 17..32, 79-144 at 33..64, then 51 / 120 / 42 / 41
+    // Q4_K has its own kernels there. out_f == 0: the caller has decided already.
+    if (dtype == 12) return false;
+    const bool long_rows = nb >= 32;                                          // 8192 columns and more
+    const bool small = out_f == 0 || out_f * (size_t)nb <= (size_t)4096 * 16;  // up to 4096 x 4096 weights
+    const size_t top = dtype == 13   ? (small || long_rows ? 96 : 48)
+                       : dtype == 14 ? (small || long_rows ? 128 : 80)
+                       : dtype == 8  ? (small || long_rows ? 64 : 32)
+                                     : (small || long_rows ? 128 : 64);
+    return m <= top;
 }
 
-bool mmq_skinny16_takes(int dtype, size_t m, size_t in_f) {
-    return in_f % 256 == 0 && skinny16_shape(dtype, (int)(in_f / 256), m);
+bool mmq_skinny16_takes(int dtype, size_t m, size_t in_f, size_t out_f) {
+    return in_f % 256 == 0 && skinny16_shape(dtype, (int)(in_f / 256), m, out_f);
 }
 
 template <typename F, bool STAGES>
 static void launch_mmq_skinny16_fmt(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, int nb,
                                     size_t out_f, size_t wgs, const IntStages& st, const BatchTile* tiles,
                                     hipStream_t stream) {
-    const dim3 grid((unsigned)wgs, 2), block(kSkinny16Waves * 64);
+    const dim3 grid((unsigned)wgs, 2, (unsigned)((m + 15) / 16)), block(kSkinny16Waves * 64);
     if (m <= 8)
         hipLaunchKernelGGL((mmq_skinny16_kernel<F, kSkinny16Waves, kSkinny16Blocks, 8, STAGES>), grid, block, 0, stream,
                            w, bpr, act.qs, act.d, act.bsums, y, (int)m, (int)out_f, nb, st.a, st.b, tiles);
@@ -1207,7 +1229,7 @@ static bool launch_mmq_skinny16(int dtype, const uint8_t* w, size_t bpr, const A
                                 size_t in_f, size_t out_f, size_t wgs, const IntStages& st, const BatchTile* tiles,
                                 hipStream_t stream) {
     const int nb = (int)(in_f / 256);
-    if (in_f % 256 != 0 || !skinny16_shape(dtype, nb, m)) return false;
+    if (in_f % 256 != 0 || !skinny16_shape(dtype, nb, m, out_f)) return false;
     if (dtype == 12)
         launch_mmq_skinny16_fmt<Skinny16Q4K, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     else if (dtype == 13)
@@ -1275,6 +1297,13 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
     // rows beyond the decode / small-batch kernels' length, when whole 256s, take the MFMA kernel of
     // their format at any token count (a 128-token tile for one token: slow, but exact and bounded)
     const bool long_row = gemv_row_too_long(dtype, in_f) && in_f % 256 == 0;
+    // the 16-token K-split kernel where it is ahead (for the formats other than Q4_K up to 32..64 tokens)
+    if (!long_row && dtype != 12 && mmq_skinny16_takes(dtype, m, in_f, out_f)) {
+        launch_quantize_q8(x, m, in_f, act_is_per32(dtype, in_f), act, stream);
+        const size_t wgs = (out_f + 31) / 32;
+        return st.a ? launch_mmq_skinny16<true>(dtype, w, bpr, act, y, m, in_f, out_f, wgs, st, nullptr, stream)
+                    : launch_mmq_skinny16<false>(dtype, w, bpr, act, y, m, in_f, out_f, wgs, st, nullptr, stream);
+    }
     if (dtype == 12 && (m >= 128 || long_row)) {
         launch_quantize_q8_tiled(x, m, in_f, act, stream);
         if (mmq_strip_q4k_takes(m, out_f)) {
@@ -1326,7 +1355,7 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
         return true;
     }
     launch_quantize_q8(x, m, in_f, act_is_per32(dtype, in_f), act, stream);
-    if (mmq_skinny16_takes(dtype, m, in_f)) {
+    if (mmq_skinny16_takes(dtype, m, in_f, out_f)) {
         const size_t wgs = (out_f + 31) / 32;
         return st.a ? launch_mmq_skinny16<true>(dtype, w, bpr, act, y, m, in_f, out_f, wgs, st, nullptr, stream)
                     : launch_mmq_skinny16<false>(dtype, w, bpr, act, y, m, in_f, out_f, wgs, st, nullptr, stream);

@@ -252,6 +252,29 @@ def test_q2_0_on_the_sixteen_token_mfma_kernel_is_bit_identical_to_oracle(be, m,
     assert np.array_equal(a, oa)
 
 
+@pytest.mark.parametrize("m", [17, 31, 33, 48, 64, 96, 128])
+@pytest.mark.parametrize("dtype", [DType.Q5K, DType.Q6K, DType.Q8_0, DType.Q2_0])
+def test_batches_beyond_sixteen_tokens_on_the_k_split_kernel(be, dtype, m):
+    """The 16-token K-split MFMA kernel walks larger batches 16 tokens at a time (up to 32..128
+    tokens by format, row length and matrix size): every output still equals the oracle's bit for
+    bit - the token tile a row falls into changes nothing about its arithmetic - and the per-block
+    integers are exact. A small matrix, which keeps the route for the longest, and a long-row one."""
+    if m > {DType.Q5K: 96, DType.Q6K: 128, DType.Q8_0: 64, DType.Q2_0: 128}[dtype]:
+        pytest.skip("beyond this format's range the 128-token MFMA tiles take over (their own tests)")
+    for in_f, out_f in ((1024, 70), (8192, 40)):
+        w = orc.synth_weight(dtype, in_f * out_f, 0x20E)
+        x = orc.gen_f32(m * in_f, 0x20E ^ 0x9E37)
+        x[in_f:2 * in_f] = 0.0                      # an all-zero token inside the first tile
+        y = run_linear(be, dtype, w, x, m, in_f, out_f)
+        want = orc.linear(dtype, w, x, m, in_f, out_f).reshape(m, out_f)
+        assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), f"not bit-identical at {in_f} x {out_f}"
+    a, b = be.linear_int_stages(dtype, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
+    oa, ob = orc.linear_int_stages(dtype, w, x, m, in_f, out_f)
+    assert np.array_equal(a, oa)
+    if dtype == DType.Q5K:
+        assert np.array_equal(b, ob)
+
+
 @pytest.mark.parametrize("m,in_f,out_f", [(6, 4608, 40), (13, 1024, 50)])
 @pytest.mark.parametrize("dtype,seed", [(DType.Q4K, 0x209), (DType.Q5K, 0x20A), (DType.Q6K, 0x20B)])
 def test_small_batch_kquant_mfma_int_stages_bit_exact(be, dtype, seed, m, in_f, out_f):
