@@ -267,11 +267,12 @@ static bool runs_alone(int dtype, size_t m, size_t in_f) {
 }
 
 // Ops that run in small-batch groups inside plans: the K-split MFMA kernels take Q4_K up to 32
-// rows and Q5_K up to 16 (rows of an even number of blocks), the dot4 batch kernel the other
+// rows, and Q4_K, Q5_K, Q6_K, Q8_0 and Q2_0 as far as their 16-token kernel is the route
+// (mmq_skinny16_takes: up to 32..128 rows by format and shape); the dot4 batch kernel the other
 // formats up to 8.
 static bool small_batch(const infr_hip_op_t& op) {
     if (op.m < 2 || is_plain(op.w_dtype) || infr::gemv_row_too_long(op.w_dtype, op.in_f)) return false;
-    if (op.w_dtype == INFR_DTYPE_Q4_K) return op.m <= 32;
+    if (op.w_dtype == INFR_DTYPE_Q4_K && op.m <= 32) return true;
     return op.m <= 8 || infr::mmq_skinny16_takes(op.w_dtype, op.m, op.in_f, op.out_f);
 }
 

@@ -1196,10 +1196,19 @@ static bool skinny16_shape(int dtype, int nb, size_t m, size_t out_f) {
     //   Q5_K  9.2 / 8.8 / 2.9 / 0.8; 52-85, then 35 / 65 / 26 / 26
     //   Q8_0  15.4 / 15.2 / 6.1 / 1.8; 51-71, then 46-50 / 73 / 30 / 28
     //   Q2_0  12.5 / 10.7 / 4.1 / 1.2; 44-74 at 17..32, 79-144 at 33..64, then 51 / 120 / 42 / 41
-    // Q4_K has its own kernels there. out_f == 0: the caller has decided already.
-    if (dtype == 12) return false;
+    // out_f == 0: the caller has decided already.
     const bool long_rows = nb >= 32;                                          // 8192 columns and more
     const bool small = out_f == 0 || out_f * (size_t)nb <= (size_t)4096 * 16;  // up to 4096 x 4096 weights
+    if (dtype == 12) {
+        // Q4_K keeps its 32-token K-split kernel up to 32 tokens (10.6-12.9 against 16 us at 12288 x 4096)
+        // and its 32-token tiles on large matrices of 4096-column rows (31 us flat from 33 to 127
+        // tokens; this kernel 29 at 33..48, 36 at 64). Those tiles cost 80 us on 4096 x 12288 and have a
+        // floor of 26 us on small matrices: there this kernel takes 33 tokens and up (4096 x 12288:
+        // 24 / 32 / 48 us at 33 / 64 / 96 tokens; 4096 x 4096: 7.6 / 9.8 / 14; 1024 x 4096: 2.7 / 3.3 / 4.4).
+        if (m <= 32) return false;
+        if (out_f == 0) return true;
+        return long_rows ? m <= 127 : (small && m <= 128);
+    }
     const size_t top = dtype == 13   ? (small || long_rows ? 96 : 48)
                        : dtype == 14 ? (small || long_rows ? 128 : 80)
                        : dtype == 8  ? (small || long_rows ? 64 : 32)
@@ -1297,8 +1306,8 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
     // rows beyond the decode / small-batch kernels' length, when whole 256s, take the MFMA kernel of
     // their format at any token count (a 128-token tile for one token: slow, but exact and bounded)
     const bool long_row = gemv_row_too_long(dtype, in_f) && in_f % 256 == 0;
-    // the 16-token K-split kernel where it is ahead (for the formats other than Q4_K up to 32..64 tokens)
-    if (!long_row && dtype != 12 && mmq_skinny16_takes(dtype, m, in_f, out_f)) {
+    // the 16-token K-split kernel where it is ahead beyond 16 tokens (up to 32..128 by format and shape)
+    if (!long_row && (dtype != 12 || m > 32) && mmq_skinny16_takes(dtype, m, in_f, out_f)) {
         launch_quantize_q8(x, m, in_f, act_is_per32(dtype, in_f), act, stream);
         const size_t wgs = (out_f + 31) / 32;
         return st.a ? launch_mmq_skinny16<true>(dtype, w, bpr, act, y, m, in_f, out_f, wgs, st, nullptr, stream)

@@ -253,13 +253,13 @@ def test_q2_0_on_the_sixteen_token_mfma_kernel_is_bit_identical_to_oracle(be, m,
 
 
 @pytest.mark.parametrize("m", [17, 31, 33, 48, 64, 96, 128])
-@pytest.mark.parametrize("dtype", [DType.Q5K, DType.Q6K, DType.Q8_0, DType.Q2_0])
+@pytest.mark.parametrize("dtype", [DType.Q4K, DType.Q5K, DType.Q6K, DType.Q8_0, DType.Q2_0])
 def test_batches_beyond_sixteen_tokens_on_the_k_split_kernel(be, dtype, m):
     """The 16-token K-split MFMA kernel walks larger batches 16 tokens at a time (up to 32..128
     tokens by format, row length and matrix size): every output still equals the oracle's bit for
     bit - the token tile a row falls into changes nothing about its arithmetic - and the per-block
     integers are exact. A small matrix, which keeps the route for the longest, and a long-row one."""
-    if m > {DType.Q5K: 96, DType.Q6K: 128, DType.Q8_0: 64, DType.Q2_0: 128}[dtype]:
+    if m > {DType.Q4K: 127, DType.Q5K: 96, DType.Q6K: 128, DType.Q8_0: 64, DType.Q2_0: 128}[dtype]:
         pytest.skip("beyond this format's range the 128-token MFMA tiles take over (their own tests)")
     for in_f, out_f in ((1024, 70), (8192, 40)):
         w = orc.synth_weight(dtype, in_f * out_f, 0x20E)
@@ -271,7 +271,7 @@ def test_batches_beyond_sixteen_tokens_on_the_k_split_kernel(be, dtype, m):
     a, b = be.linear_int_stages(dtype, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
     oa, ob = orc.linear_int_stages(dtype, w, x, m, in_f, out_f)
     assert np.array_equal(a, oa)
-    if dtype == DType.Q5K:
+    if dtype in (DType.Q4K, DType.Q5K):
         assert np.array_equal(b, ob)
 
 
