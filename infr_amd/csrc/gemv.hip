@@ -60,7 +60,7 @@ bool plan_batch_group(int dtype, size_t m, size_t in_f, const GemvOpDesc* ops, i
     BatchGroupPlan gp;
     size_t max_out_f = 0;
     for (int i = 0; i < n; ++i) max_out_f = std::max(max_out_f, (size_t)ops[i].out_f);
-    if ((dtype == 13 || dtype == 14 || dtype == 8 || dtype == 42 || (dtype == 12 && m > 32)) &&
+    if ((dtype != 12 || m > 32) &&
         mmq_skinny16_takes(dtype, m, in_f, max_out_f)) {  // the K-split MFMA kernel
         gp.kind = 1;
         gp.rows_per_wg = 32;

@@ -28,6 +28,7 @@
 #include <cstdlib>
 
 #include "device_common.hpp"
+#include "gemv_formats.hpp"
 #include "kernels.hpp"
 #include "mmq_tiles.hpp"
 
@@ -942,6 +943,103 @@ struct Skinny16Q2_0 {
     }
 };
 
+// Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL (32-weight blocks of 18..24 bytes; crates/infr-cpu/src/kernels.rs
+// vec_dot_*_32_batch, restated in the oracle's orc_vec_dot_blk32) against the per-32 activation: a
+// 256-element step is eight blocks. Byte j of a block's 16 holds element j in its low nibble and
+// element 16 + j in its high one, so the lane that supplies elements 8 kq .. 8 kq + 7 reads eight
+// bytes and takes one nibble of each (plus, for the Q5 kinds, eight bits of the mask spread to bit 4;
+// IQ4_NL's nibbles go through its table); one v_mfma_i32_16x16x32_i8 per block gives the exact
+// iprod, and the lane forms the CPU's f32 term at once - `(d * q8.d) * (iprod - 8 or 16 * bsum)`,
+// `(d * q8.d) * iprod` for IQ4_NL, `q8.d * (d * iprod + m * bsum)` for the affine kinds - for the
+// wave-to-wave chain to add in block order: infr-cpu's bits. Blocks of 18 and 22 bytes start two
+// bytes off a word boundary every other block: read as aligned words and shifted.
+template <Nib32 K>
+struct Skinny16Nib32 {
+    typedef int v2i __attribute__((ext_vector_type(2)));
+    static constexpr bool kAffine = K == Nib32::Q4_1 || K == Nib32::Q5_1;
+    static constexpr bool kFive = K == Nib32::Q5_0 || K == Nib32::Q5_1;
+    static constexpr bool kSubScales = true, kPer32Acts = true, kTranspose16 = false;
+    static constexpr int kB = 18 + (kAffine ? 2 : 0) + (kFive ? 4 : 0);  // bytes of a 32-weight block
+    static constexpr int kBlockBytes = 8 * kB;
+    static constexpr int kRowStride = 2 * kBlockBytes + 16;  // (stride / 4) mod 32 = 12, 20, 28, 4: eight rows' 16-byte reads cover all banks
+    // a word at `off` bytes into the row's stage, where off is 0 or 2 mod 4 (`odd`: known at compile time)
+    template <bool ODD>
+    __device__ static uint32_t word_at(const uint8_t* p) {
+        if (!ODD) return *reinterpret_cast<const uint32_t*>(p);
+        const uint32_t w0 = *reinterpret_cast<const uint32_t*>(p - 2), w1 = *reinterpret_cast<const uint32_t*>(p + 2);
+        return __builtin_amdgcn_alignbyte(w1, w0, 2);
+    }
+    template <int MT, int DQ_STRIDE>
+    __device__ static void block(const uint8_t* wrow, int jj, const uint8_t* arow, const uint8_t* bs_base,
+                                 const float* dq_base, int kq, int (&ip)[32], int (&raw)[32]) {
+        const uint8_t* blk = wrow + jj * kBlockBytes;
+        v4f dq[4][2];
+        v4i bs[4][2];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int tok = (4 * kq + i) & (MT - 1);
+            dq[i][0] = *reinterpret_cast<const v4f*>(dq_base + tok * DQ_STRIDE + jj * 8);
+            dq[i][1] = *reinterpret_cast<const v4f*>(dq_base + tok * DQ_STRIDE + jj * 8 + 4);
+            bs[i][0] = *reinterpret_cast<const v4i*>(bs_base + tok * 32);
+            bs[i][1] = *reinterpret_cast<const v4i*>(bs_base + tok * 32 + 16);
+        }
+        constexpr int kQhOff = 2 + (kAffine ? 2 : 0), kQsOff = kQhOff + (kFive ? 4 : 0);
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const uint8_t* sb = blk + s * kB;
+            // (s * kB + kQsOff) mod 4 is 2 for the even blocks of the 18- and 22-byte kinds, else 0
+            constexpr bool kOddStride = kB % 4 == 2;
+            const uint8_t* qp = sb + kQsOff + 8 * (kq & 1);
+            uint32_t c0, c1;
+            if (kOddStride && (s & 1) == 0) {
+                const uint32_t w0 = *reinterpret_cast<const uint32_t*>(qp - 2), w1 = *reinterpret_cast<const uint32_t*>(qp + 2);
+                const uint32_t w2 = *reinterpret_cast<const uint32_t*>(qp + 6);
+                c0 = __builtin_amdgcn_alignbyte(w1, w0, 2);
+                c1 = __builtin_amdgcn_alignbyte(w2, w1, 2);
+            } else {
+                c0 = *reinterpret_cast<const uint32_t*>(qp);
+                c1 = *reinterpret_cast<const uint32_t*>(qp + 4);
+            }
+            const int sh = 4 * (kq >> 1);
+            c0 = (c0 >> sh) & 0x0F0F0F0Fu;
+            c1 = (c1 >> sh) & 0x0F0F0F0Fu;
+            if (K == Nib32::IQ4_NL) {
+                c0 = (uint32_t)iq4nl_lookup(c0);
+                c1 = (uint32_t)iq4nl_lookup(c1);
+            }
+            if (kFive) {
+                const uint32_t qh = (kOddStride && (s & 1) == 0) ? word_at<true>(sb + kQhOff) : word_at<false>(sb + kQhOff);
+                const uint32_t h = qh >> (8 * kq);
+                c0 |= spread4_to_bit4(h);
+                c1 |= spread4_to_bit4(h >> 4);
+            }
+            const v2i b = {(int)c0, (int)c1};
+            const v2i a = *reinterpret_cast<const v2i*>(arow + s * 32 + 8 * kq);
+            const v4i r = __builtin_amdgcn_mfma_i32_16x16x32_i8(__builtin_bit_cast(long, a), __builtin_bit_cast(long, b),
+                                                                v4i{0, 0, 0, 0}, 0, 0, 0);
+            const float d = f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(sb));
+            const float mw = kAffine ? f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(sb + 2)) : 0.0f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                raw[4 * s + i] = r[i];
+                const float d8 = dq[i][s >> 2][s & 3];
+                const int bsum = bs[i][s >> 2][s & 3];
+                float term;
+                if (kAffine) term = d8 * (d * (float)r[i] + mw * (float)bsum);
+                else if (K == Nib32::IQ4_NL) term = (d * d8) * (float)r[i];
+                else term = (d * d8) * (float)(r[i] - (kFive ? 16 : 8) * bsum);  // both integers and the difference are exact in f32
+                ip[4 * s + i] = __builtin_bit_cast(int, term);
+            }
+        }
+    }
+    __device__ static void accumulate(float (&acc)[4], const float (&)[4], const uint32_t (&)[4], const int (&ip)[32]) {
+#pragma unroll
+        for (int s = 0; s < 8; ++s)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] += __builtin_bit_cast(float, ip[4 * s + i]);
+    }
+};
+
 template <typename F, int NW, int BPW, int MT, bool STAGES>
 __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
     const uint8_t* __restrict__ w, size_t bpr, const int8_t* __restrict__ qs,
@@ -1165,13 +1263,14 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
     }
 }
 
-// Which batches the 16-token K-split kernel takes: Q4_K, Q5_K, Q6_K, Q8_0 and Q2_0 rows of an even number of
+// Which batches the 16-token K-split kernel takes: rows (of any quantized format) of an even number of
 // 256-blocks (weights are staged two blocks at a time), up to 16 tokens. Four waves per workgroup;
 // (eight measured no faster, and four blocks per wave and pass - 576-byte, 64-byte-aligned runs per
 // row - measured 20-25 % slower: a wave then computes for longer before it asks for more).
 constexpr int kSkinny16Waves = 4, kSkinny16Blocks = 2;
 static bool skinny16_shape(int dtype, int nb, size_t m, size_t out_f) {
-    if (dtype != 12 && dtype != 13 && dtype != 14 && dtype != 8 && dtype != 42) return false;
+    const bool nib32 = dtype == 2 || dtype == 3 || dtype == 6 || dtype == 7 || dtype == 20;
+    if (dtype != 12 && dtype != 13 && dtype != 14 && dtype != 8 && dtype != 42 && !nib32) return false;
     if (nb < kSkinny16Blocks || nb % kSkinny16Blocks != 0) return false;
     if (m <= 16) {
         // the dot4 batch kernels, which unpack a weight once per two or four tokens, stay ahead at the
@@ -1185,6 +1284,8 @@ static bool skinny16_shape(int dtype, int nb, size_t m, size_t out_f) {
         // Q2_0: 72 bytes a step make this kernel compute-bound (1.0-1.3 TB/s at any token count, what the
         // dot4 batches reach at eight tokens): it takes 9 tokens and more, where they would need two passes
         if (dtype == 42 && m <= 8) return false;
+        // the 32-weight-block formats: as Q2_0 (12288 x 4096 at eight tokens: 10-12 us on the dot4 batches, 14-15 here)
+        if (nib32 && m <= 8) return false;
         return true;
     }
     // Beyond 16 tokens the grid's third dimension walks the batch 16 tokens at a time (the weights
@@ -1209,6 +1310,9 @@ static bool skinny16_shape(int dtype, int nb, size_t m, size_t out_f) {
         if (out_f == 0) return true;
         return long_rows ? m <= 127 : (small && m <= 128);
     }
+    //   Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL  14-16 / 12-14 / 5.0-5.7; before: 41 at 16 tokens, 76 at 32, 147 at 64,
+    //         then 59-71 / 130-180 / 50-64
+    if (nib32) return m <= (small || long_rows ? 128 : 64);
     const size_t top = dtype == 13   ? (small || long_rows ? 96 : 48)
                        : dtype == 14 ? (small || long_rows ? 128 : 80)
                        : dtype == 8  ? (small || long_rows ? 64 : 32)
@@ -1247,6 +1351,16 @@ static bool launch_mmq_skinny16(int dtype, const uint8_t* w, size_t bpr, const A
         launch_mmq_skinny16_fmt<Skinny16Q8_0, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     else if (dtype == 42)
         launch_mmq_skinny16_fmt<Skinny16Q2_0, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
+    else if (dtype == 2)
+        launch_mmq_skinny16_fmt<Skinny16Nib32<Nib32::Q4_0>, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
+    else if (dtype == 3)
+        launch_mmq_skinny16_fmt<Skinny16Nib32<Nib32::Q4_1>, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
+    else if (dtype == 6)
+        launch_mmq_skinny16_fmt<Skinny16Nib32<Nib32::Q5_0>, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
+    else if (dtype == 7)
+        launch_mmq_skinny16_fmt<Skinny16Nib32<Nib32::Q5_1>, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
+    else if (dtype == 20)
+        launch_mmq_skinny16_fmt<Skinny16Nib32<Nib32::IQ4_NL>, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     else
         launch_mmq_skinny16_fmt<Skinny16Q6K, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     return true;

@@ -81,6 +81,26 @@ def test_batches_vs_oracle(be, dtype, m):
         assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), "not bit-identical"
 
 
+@pytest.mark.parametrize("dtype", BLK32, ids=ids)
+@pytest.mark.parametrize("m", [9, 16, 17, 40, 64, 100, 128])
+def test_nine_tokens_and_up_on_the_k_split_kernel_are_bit_identical(be, dtype, m):
+    """From nine tokens the 32-weight-block formats take the 16-token K-split MFMA kernel (16 tokens
+    at a time beyond that): one exact iprod per block and the CPU's f32 term per block, added in
+    block order by the wave-to-wave chain (oracle orc_vec_dot_blk32 = infr-cpu's
+    vec_dot_*_32_batch_scalar) - so, unlike the dot4 batches and the 128-token tiles, these outputs
+    equal the scalar kernel's bits. Full-range payloads; a small matrix and one of long rows."""
+    for in_f, out_f in ((1024, 70), (8192, 40)):
+        w = orc.synth_weight(dtype, in_f * out_f, 0x30A)
+        x = orc.gen_f32(m * in_f, 0x30A ^ 0x9E37)
+        x[in_f:2 * in_f] = 0.0
+        y = run_linear(be, dtype, w, x, m, in_f, out_f)
+        want = orc.linear(dtype, w, x, m, in_f, out_f).reshape(m, out_f)
+        assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), f"not bit-identical at {in_f} x {out_f}"
+    a, _ = be.linear_int_stages(dtype, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
+    oa, _ = orc.linear_int_stages(dtype, w, x, m, in_f, out_f)
+    assert np.array_equal(a, oa)
+
+
 def test_q5_0_one_token_is_the_f32_path_not_the_int8_one(be):
     in_f, out_f = 2048, 64
     w = synth_weight(DType.Q5_0, 31, out_f, in_f)
