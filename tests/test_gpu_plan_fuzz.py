@@ -181,7 +181,8 @@ def describe(prog):
 
 
 @pytest.mark.parametrize("m,seed", [(1, s) for s in range(16)] + [(3, s) for s in range(100, 106)] +
-                         [(8, s) for s in range(200, 203)])
+                         [(8, s) for s in range(200, 203)] + [(20, s) for s in range(300, 303)] +
+                         [(48, s) for s in range(400, 402)])
 def test_scheduled_plan_equals_the_ops_run_one_by_one(be, m, seed):
     rng = np.random.default_rng(seed)
     prog = random_program(rng, int(rng.integers(6, 15)))
