@@ -64,7 +64,7 @@ bool plan_batch_group(int dtype, size_t m, size_t in_f, const GemvOpDesc* ops, i
         mmq_skinny16_takes(dtype, m, in_f, max_out_f)) {  // the K-split MFMA kernel
         gp.kind = 1;
         gp.rows_per_wg = 32;
-    } else if (dtype == 12) {  // Q4_K: the K-split MFMA kernels, 32 rows per workgroup
+    } else if (dtype == 12 && m > 2) {  // Q4_K from three tokens: the K-split MFMA kernels, 32 rows per workgroup
         if (in_f % 256 != 0 || m > 32) return false;
         gp.kind = 1;
         gp.rows_per_wg = 32;

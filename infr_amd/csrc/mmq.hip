@@ -1274,8 +1274,10 @@ static bool skinny16_shape(int dtype, int nb, size_t m, size_t out_f) {
     if (nb < kSkinny16Blocks || nb % kSkinny16Blocks != 0) return false;
     if (m <= 16) {
         // the dot4 batch kernels, which unpack a weight once per two or four tokens, stay ahead at the
-        // bottom: Q5_K at two tokens (4.3-5.3 against 3.8-4.4 TB/s), Q6_K up to four (3.6-4.5 against 3.3-3.9)
-        if ((dtype == 13 && m < 3) || (dtype == 14 && m < 5)) return false;
+        // bottom: Q4_K at two tokens (4.3 / 4.0 / 5.5 / 5.6 against 3.7 / 3.4 / 4.2 / 4.2 TB/s on the four
+        // layer shapes; level from three), Q5_K at two (4.3-5.3 against 3.8-4.4), Q6_K up to four
+        // (3.6-4.5 against 3.3-3.9)
+        if ((dtype == 12 && m < 3) || (dtype == 13 && m < 3) || (dtype == 14 && m < 5)) return false;
         // Q8_0: the dot4 batches stay ahead up to eight tokens on rows of one or two wave steps (4.2 / 3.8 /
         // 4.8 against 3.8 / 3.3 / 4.2 TB/s at eight tokens on the 4096-column shapes, 5.1-5.9 at two to
         // four); this kernel takes 9..16 tokens (one pass over the weights instead of two) and, from
@@ -1483,7 +1485,7 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
         return st.a ? launch_mmq_skinny16<true>(dtype, w, bpr, act, y, m, in_f, out_f, wgs, st, nullptr, stream)
                     : launch_mmq_skinny16<false>(dtype, w, bpr, act, y, m, in_f, out_f, wgs, st, nullptr, stream);
     }
-    if (dtype != 12) return launch_gemv_batch(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
+    if (dtype != 12 || m == 2) return launch_gemv_batch(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
     if (m <= 32) {
         // four blocks per round; eight for long rows or when four would leave most SIMDs without a wave
         const size_t wgs = (out_f + 31) / 32 * ((m + 31) / 32);
