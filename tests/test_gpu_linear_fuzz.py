@@ -68,3 +68,12 @@ def test_linear_on_a_random_shape_matches_the_oracle(be, seed):
         rel = np.linalg.norm(g - t) / max(np.linalg.norm(t), 1e-30)
         mx = np.abs(g - t).max() / max(np.abs(t).max(), 1e-30)
         assert rel <= 1e-4 and mx <= 1e-3, f"rel-L2 {rel:.2e} max-abs {mx:.2e}: {case}"
+    # every fourth quantized case: the per-block integers behind those outputs, exact on every route
+    # (one token of Q5_0 multiplies f32 activations: it has no integer stage, as on the CPU)
+    if seed % 4 == 1 and dtype not in PLAIN and not (dtype == DType.Q5_0 and m == 1):
+        a, b = be.linear_int_stages(dtype, be.upload_new(w), be.upload_new(x), m, in_f, out_f, w_numel=rows * in_f,
+                                    w_off=before * in_f)
+        oa, ob = orc.linear_int_stages(dtype, w, x, m, in_f, out_f, w_numel=rows * in_f, w_off=before * in_f)
+        assert np.array_equal(a, oa), f"first integer stage differs: {case}"
+        if dtype in (DType.Q4K, DType.Q5K):
+            assert np.array_equal(b, ob), f"second integer stage differs: {case}"
