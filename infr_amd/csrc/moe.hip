@@ -643,10 +643,10 @@ __global__ __launch_bounds__(256) void moe_gate_up_f32_kernel(
     const uint8_t* __restrict__ gate, const uint8_t* __restrict__ up, size_t gate_stride,
     size_t up_stride, const float* __restrict__ logits, int n_expert, int n_used, float scale,
     int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, const float* __restrict__ x,
-    float* __restrict__ act, int ne, int nff) {
+    float* __restrict__ act, int ne, int nff, int S, int chunks) {
     __shared__ __attribute__((aligned(16))) SelectLds sel;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int S = ne / 64, rps = 64 / S;  // lanes per weight row, rows per wave step
+    const int rps = 64 / S;  // S lanes per weight row (each on `chunks` units of it), rows per wave step
     const int seg = lane / S, u = lane % S;
     const bool lane_ok = seg < rps;
     const int slot = blockIdx.y;
@@ -666,20 +666,33 @@ __global__ __launch_bounds__(256) void moe_gate_up_f32_kernel(
     const size_t bpr = (size_t)(ne / 256) * P::kBlockBytes;
     const uint8_t* gw = gate + (size_t)e * gate_stride;
     const uint8_t* uw = up + (size_t)e * up_stride;
-    typename P::Row g[SPW], up_r[SPW];
+    float gp[SPW], upp[SPW];
 #pragma unroll
-    for (int i = 0; i < SPW; ++i) {
-        const int o = (st0 + i) * rps + seg;
-        const bool ok = lane_ok && o < nff;
-        P::load_row(g[i], gw + (size_t)(ok ? o : 0) * bpr, u, ok);
-        P::load_row(up_r[i], uw + (size_t)(ok ? o : 0) * bpr, u, ok);
+    for (int i = 0; i < SPW; ++i) gp[i] = upp[i] = 0.0f;
+    // rows longer than 64 lanes x 64 weights: unit c * S + u in round c, the partial sums added per lane
+    for (int c = 0; c < chunks; ++c) {
+        const int uc = c * S + u;
+        if (c) P::load_x(xa, x, uc, lane_ok);
+        typename P::Row g[SPW], up_r[SPW];
+#pragma unroll
+        for (int i = 0; i < SPW; ++i) {
+            const int o = (st0 + i) * rps + seg;
+            const bool ok = lane_ok && o < nff;
+            P::load_row(g[i], gw + (size_t)(ok ? o : 0) * bpr, uc, ok);
+            P::load_row(up_r[i], uw + (size_t)(ok ? o : 0) * bpr, uc, ok);
+        }
+#pragma unroll
+        for (int i = 0; i < SPW; ++i) {
+            gp[i] += P::partial(g[i], xa, uc);
+            upp[i] += P::partial(up_r[i], xa, uc);
+        }
     }
 #pragma unroll
     for (int i = 0; i < SPW; ++i) {
         const int o = (st0 + i) * rps + seg;
         const bool ok = lane_ok && o < nff;
-        const float gs = seg_sum(P::partial(g[i], xa, u), seg * S, S / 4);
-        const float us = seg_sum(P::partial(up_r[i], xa, u), seg * S, S / 4);
+        const float gs = seg_sum(gp[i], seg * S, S / 4);
+        const float us = seg_sum(upp[i], seg * S, S / 4);
         if (ok && u == 0) act[(size_t)slot * nff + o] = gs / (1.0f + expf(-gs)) * us;
     }
 }
@@ -695,10 +708,10 @@ template <typename P, int STEPS>
 __global__ __launch_bounds__(1024) void moe_down_f32_kernel(
     const uint8_t* __restrict__ down, size_t down_stride, const int32_t* __restrict__ ids,
     const float* __restrict__ wts, const float* __restrict__ act, float* __restrict__ out,
-    const float* add_b, float* add_dst, int nff, int ne, int n_used) {
+    const float* add_b, float* add_dst, int nff, int ne, int n_used, int S, int chunks) {
     __shared__ float ys[kDownMaxSteps][kDownMaxWaves][16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
-    const int S = nff / 64, rps = 64 / S;
+    const int rps = 64 / S;
     const int seg = lane / S, u = lane % S;
     const bool lane_ok = seg < rps;
     const size_t bpr = (size_t)(nff / 256) * P::kBlockBytes;
@@ -711,18 +724,26 @@ __global__ __launch_bounds__(1024) void moe_down_f32_kernel(
         if (k0) __syncthreads();
         if (k < n_used) {
             const uint8_t* dw = down + (size_t)ids[k] * down_stride;
-            typename P::Row row[STEPS];
+            float part[STEPS];
 #pragma unroll
-            for (int s = 0; s < STEPS; ++s) {
-                const int o = (st0 + s) * rps + seg;
-                const bool ok = lane_ok && o < ne;
-                P::load_row(row[s], dw + (size_t)(ok ? o : 0) * bpr, u, ok);
+            for (int s = 0; s < STEPS; ++s) part[s] = 0.0f;
+            for (int c = 0; c < chunks; ++c) {
+                const int uc = c * S + u;
+                typename P::Row row[STEPS];
+#pragma unroll
+                for (int s = 0; s < STEPS; ++s) {
+                    const int o = (st0 + s) * rps + seg;
+                    const bool ok = lane_ok && o < ne;
+                    P::load_row(row[s], dw + (size_t)(ok ? o : 0) * bpr, uc, ok);
+                }
+                typename P::X xa;
+                P::load_x(xa, act + (size_t)k * nff, uc, lane_ok);
+#pragma unroll
+                for (int s = 0; s < STEPS; ++s) part[s] += P::partial(row[s], xa, uc);
             }
-            typename P::X xa;
-            P::load_x(xa, act + (size_t)k * nff, u, lane_ok);
 #pragma unroll
             for (int s = 0; s < STEPS; ++s) {
-                const float yk = seg_sum(P::partial(row[s], xa, u), seg * S, S / 4);
+                const float yk = seg_sum(part[s], seg * S, S / 4);
                 if (lane_ok && u == 0) ys[s][wave][seg] = yk;
             }
         }
@@ -1235,8 +1256,7 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     // One row in the formats of the factored kernels: the gate / up kernel selects in its own
     // prologue, so the router only leaves the logits - one expert per workgroup, nothing to wait for.
     auto raw_ok = [](int dt) { return dt == 12 || dt == 13 || dt == 14 || dt == 8; };
-    const bool fast1 = s.rows == 1 && raw_ok(s.gate_dtype) && s.up_dtype == s.gate_dtype && raw_ok(s.down_dtype) &&
-                       s.ne <= 4096 && s.n_ff <= 4096;
+    const bool fast1 = s.rows == 1 && raw_ok(s.gate_dtype) && s.up_dtype == s.gate_dtype && raw_ok(s.down_dtype);
     switch (s.router_dtype) {
     case 0: launch_row_dots<0>(b.router, b.router_x, logits, s.ne, s.n_expert, s.rows, fast1, tickets, sel_idx, sel_w, s.n_used, s.scale, b.norm_w, b.norm_dst, b.norm_eps, stream); break;
     case 1: launch_row_dots<1>(b.router, b.router_x, logits, s.ne, s.n_expert, s.rows, fast1, tickets, sel_idx, sel_w, s.n_used, s.scale, b.norm_w, b.norm_dst, b.norm_eps, stream); break;
@@ -1290,8 +1310,7 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     if (s.rows == 1) {
         // ActsKind::Raw for every bank (lib.rs:2359: int8_ok = rows >= 2)
         if (!fast1) {
-            // other formats, mixed gate / up formats, rows too long for the factored kernels'
-            // registers: the decode-and-dot form of every stage
+            // other formats, mixed gate / up formats: the decode-and-dot form of every stage
             launch_raw(s.gate_dtype, b.gate, b.gate_stride, gbpr, b.x, s.n_used, s.ne, gbuf, s.n_ff);
             launch_raw(s.up_dtype, b.up, b.up_stride, ubpr, b.x, s.n_used, s.ne, ubuf, s.n_ff);
             const size_t n_act1 = pairs * s.n_ff;
@@ -1304,13 +1323,23 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
         }
         // row steps per wave: amortise the 64 activation registers while keeping >= ~1024 waves
         auto steps_per_wave = [](int wave_steps) { return std::max(1, std::min(4, wave_steps / kMoeWavesWanted)); };
-        const int rps_g = 64 / (s.ne / 64);
+        // lanes per weight row: every 64-weight unit its own lane up to 4096 columns; longer rows
+        // in rounds of the widest lane count that divides the units and leaves at most 8 lanes idle
+        auto row_lanes = [](int units) {
+            if (units <= 64) return units;
+            int l = 64;
+            while (units % l != 0 || 64 / l * l < 56) l -= 4;
+            return l;
+        };
+        const int lanes_g = row_lanes(s.ne / 64), chunks_g = s.ne / 64 / lanes_g;
+        const int rps_g = 64 / lanes_g;
         const int steps_g = (s.n_ff + rps_g - 1) / rps_g;
         const int spw = steps_per_wave(steps_g * s.n_used);
         const dim3 grid_g((unsigned)((steps_g + 4 * spw - 1) / (4 * spw)), (unsigned)s.n_used);
 #define INFR_GATE_UP_N(P, N)                                                                                  \
     hipLaunchKernelGGL((moe_gate_up_f32_kernel<P, N>), grid_g, dim3(256), 0, stream, b.gate, b.up, b.gate_stride, \
-                       b.up_stride, logits, s.n_expert, s.n_used, s.scale, sel_idx, sel_w, b.x, gbuf, s.ne, s.n_ff)
+                       b.up_stride, logits, s.n_expert, s.n_used, s.scale, sel_idx, sel_w, b.x, gbuf, s.ne, s.n_ff, \
+                       lanes_g, chunks_g)
 #define INFR_GATE_UP(P)                 \
     switch (spw) {                      \
     case 1: INFR_GATE_UP_N(P, 1); break; \
@@ -1325,14 +1354,16 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
 #undef INFR_GATE_UP
 #undef INFR_GATE_UP_N
         export_selection();
-        const int rps_d = 64 / (s.n_ff / 64);
+        const int lanes_d = row_lanes(s.n_ff / 64), chunks_d = s.n_ff / 64 / lanes_d;
+        const int rps_d = 64 / lanes_d;
         const int steps_d = (s.ne + rps_d - 1) / rps_d;
         const int spw_d = std::min(kDownMaxSteps, steps_per_wave(steps_d * s.n_used));
         const int nw_d = std::min(s.n_used, kDownMaxWaves);
         const dim3 grid_d((unsigned)((steps_d + spw_d - 1) / spw_d));
 #define INFR_DOWN_N(P, N)                                                                                   \
     hipLaunchKernelGGL((moe_down_f32_kernel<P, N>), grid_d, dim3((unsigned)(64 * nw_d)), 0, stream, b.down,   \
-                       b.down_stride, sel_idx, sel_w, gbuf, b.dst, b.add_b, b.add_dst, s.n_ff, s.ne, s.n_used)
+                       b.down_stride, sel_idx, sel_w, gbuf, b.dst, b.add_b, b.add_dst, s.n_ff, s.ne, s.n_used, \
+                       lanes_d, chunks_d)
 #define INFR_DOWN(P)                 \
     switch (spw_d) {                 \
     case 1: INFR_DOWN_N(P, 1); break; \

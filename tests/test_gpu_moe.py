@@ -362,14 +362,30 @@ def test_moe_banks_of_three_different_kinds(be, rows):
 @pytest.mark.parametrize("rows", [1, 3])
 @pytest.mark.parametrize("dtype", [DType.Q4K, DType.Q6K])
 def test_moe_hidden_size_above_4096(be, dtype, rows):
-    """The factored one-token kernels keep a row's activations in registers (up to 4096 of them);
-    longer single rows take the decode-and-dot form of the same Raw arithmetic. Two rows and more
-    run the id-gathered int8 GEMVs at any length their wave steps reach."""
+    """One token: a lane of the factored kernels keeps 64 activations of a row in registers, rows of
+    more than 4096 columns go round by round. Two rows and more run the id-gathered int8 GEMVs at any
+    length their wave steps reach."""
     ne, n_expert, n_used, nff = 8192, 4, 2, 512
     gate, up, down = banks(400, ne, n_expert, nff, dtype, sigma=0.03)
     x = synth_normal_f32(401, rows * ne)
     router = synth_normal_f32(402, n_expert * ne, sigma=0.02)
     got = run_moe(be, x, router, gate, up, down, rows, ne, n_expert, n_used, nff, 1.0, dtype)
+    want = orc.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
+                       gate_dtype=int(dtype), up_dtype=int(dtype), down_dtype=int(dtype))
+    check(*got, *want)
+
+
+@pytest.mark.parametrize("dtype", [DType.Q4K, DType.Q5K, DType.Q6K, DType.Q8_0])
+@pytest.mark.parametrize("ne,nff", [(5120, 256), (6144, 1024), (7168, 768), (256, 14336), (512, 4352), (768, 12288), (8192, 8192)])
+def test_moe_one_token_rows_in_several_rounds(be, dtype, ne, nff):
+    """Hidden sizes and expert widths beyond 4096 at one token (5120 x 8192, 6144 x 16384, 7168 x 2048,
+    4096 x 14336 in files): 80, 96, 112, 224, 68, 192 and 128 units of 64 weights per row run as 4 x 20,
+    3 x 32, 2 x 56, 4 x 56, 17 x 4, 3 x 64 and 2 x 64 lanes."""
+    n_expert, n_used = 3, 2
+    gate, up, down = banks(410, ne, n_expert, nff, dtype, sigma=0.03)
+    x = synth_normal_f32(411, ne)
+    router = synth_normal_f32(412, n_expert * ne, sigma=0.02)
+    got = run_moe(be, x, router, gate, up, down, 1, ne, n_expert, n_used, nff, 1.0, dtype)
     want = orc.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
                        gate_dtype=int(dtype), up_dtype=int(dtype), down_dtype=int(dtype))
     check(*got, *want)
