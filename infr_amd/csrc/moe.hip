@@ -401,6 +401,13 @@ __global__ __launch_bounds__(kRtThreads) void moe_router_tile_kernel(const void*
 //   X   / load_x(x, activation row, u, ok)     its activation floats and the group sums it needs
 //   partial(r, x, u)                           sum over the lane's 64 weights of w * x
 
+// Keeps a masked dword whole in the compiler's eyes: byte k of it then converts with one
+// v_cvt_f32_ubyte<k>, where a mask folded into each byte's extraction costs a bit-field extract more.
+__device__ __forceinline__ uint32_t whole_dword(uint32_t v) {
+    asm("" : "+v"(v));
+    return v;
+}
+
 // Q4_K: unit u = (block u/4, nibble pair u%4): sub-block 2p in the low nibbles of the pair's
 // 32 bytes, 2p+1 in the high ones. w = (d*sc)*code - dmin*m.
 struct RawQ4K {
@@ -452,7 +459,7 @@ struct RawQ4K {
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
             const uint32_t w = (uint32_t)wq[k];
-            const uint32_t l = w & 0x0F0F0F0Fu, h = (w >> 4) & 0x0F0F0F0Fu;
+            const uint32_t l = whole_dword(w & 0x0F0F0F0Fu), h = whole_dword((w >> 4) & 0x0F0F0F0Fu);
             lo0 = __builtin_fmaf((float)(l & 0xFF), a.x[4 * k + 0], lo0);
             lo1 = __builtin_fmaf((float)((l >> 8) & 0xFF), a.x[4 * k + 1], lo1);
             lo0 = __builtin_fmaf((float)((l >> 16) & 0xFF), a.x[4 * k + 2], lo0);
@@ -626,11 +633,15 @@ struct RawQ8_0 {
 };
 
 // Sum over the S lanes (a multiple of 4) of a row segment; every lane of the segment gets the total.
-__device__ __forceinline__ float seg_sum(float v, int seg_base, int quads) {
+__device__ __forceinline__ float seg_sum(float v, int seg_base, int S) {
     v += __builtin_bit_cast(float, quad_xor1(__builtin_bit_cast(int, v)));
     v += __builtin_bit_cast(float, quad_xor2(__builtin_bit_cast(int, v)));
+    if ((S & (S - 1)) == 0) {  // a power of two: the rest of the butterfly
+        for (int o = 4; o < S; o <<= 1) v += __shfl_xor(v, o, kWave);
+        return v;
+    }
     float s = 0.0f;
-    for (int i = 0; i < quads; ++i) s += __shfl(v, seg_base + 4 * i, kWave);
+    for (int i = 0; i < S / 4; ++i) s += __shfl(v, seg_base + 4 * i, kWave);
     return s;
 }
 
@@ -653,8 +664,10 @@ __global__ __launch_bounds__(256) void moe_gate_up_f32_kernel(
     const int steps_total = (nff + rps - 1) / rps;
     const int st0 = (blockIdx.x * 4 + wave) * SPW;
     // the activation does not depend on the routing: requested first, it arrives under the selection
+    // (every lane loads: idle lanes and rows past the end sit on valid units of row 0 and drop
+    // their results, which keeps branches and zero fills out of the load sequence)
     typename P::X xa;
-    P::load_x(xa, x, u, lane_ok);
+    P::load_x(xa, x, u, true);
     // Every workgroup selects for itself from the router's logits (a few hundred bytes and a few
     // barriers) instead of waiting for a selection kernel in between; the first one also leaves
     // the ranked experts and weights for the down kernel.
@@ -672,14 +685,14 @@ __global__ __launch_bounds__(256) void moe_gate_up_f32_kernel(
     // rows longer than 64 lanes x 64 weights: unit c * S + u in round c, the partial sums added per lane
     for (int c = 0; c < chunks; ++c) {
         const int uc = c * S + u;
-        if (c) P::load_x(xa, x, uc, lane_ok);
+        if (c) P::load_x(xa, x, uc, true);
         typename P::Row g[SPW], up_r[SPW];
 #pragma unroll
         for (int i = 0; i < SPW; ++i) {
             const int o = (st0 + i) * rps + seg;
             const bool ok = lane_ok && o < nff;
-            P::load_row(g[i], gw + (size_t)(ok ? o : 0) * bpr, uc, ok);
-            P::load_row(up_r[i], uw + (size_t)(ok ? o : 0) * bpr, uc, ok);
+            P::load_row(g[i], gw + (size_t)(ok ? o : 0) * bpr, uc, true);
+            P::load_row(up_r[i], uw + (size_t)(ok ? o : 0) * bpr, uc, true);
         }
 #pragma unroll
         for (int i = 0; i < SPW; ++i) {
@@ -691,21 +704,22 @@ __global__ __launch_bounds__(256) void moe_gate_up_f32_kernel(
     for (int i = 0; i < SPW; ++i) {
         const int o = (st0 + i) * rps + seg;
         const bool ok = lane_ok && o < nff;
-        const float gs = seg_sum(gp[i], seg * S, S / 4);
-        const float us = seg_sum(upp[i], seg * S, S / 4);
+        const float gs = seg_sum(gp[i], seg * S, S);
+        const float us = seg_sum(upp[i], seg * S, S);
         if (ok && u == 0) act[(size_t)slot * nff + o] = gs / (1.0f + expf(-gs)) * us;
     }
 }
 
 // down + accumulate at one token: out[o] = sum_k w_k * (down_{ids[k]}[o] . act[k]), k in rank
-// order. One wave per selected expert (up to 16 at a time), every wave of a workgroup on the same
-// STEPS row steps, all requested up front; the per-expert results meet in LDS and are added in rank
-// order with a separate multiply and add, as the CPU's `*o += w_e * yv`.
-constexpr int kDownMaxSteps = 4, kDownMaxWaves = 16;
+// order. One wave per selected expert (up to eight at a time: 512 threads leave every wave the 256
+// registers that four row steps in flight need), every wave of a workgroup on the same STEPS row
+// steps, all requested up front; the per-expert results meet in LDS and are added in rank order
+// with a separate multiply and add, as the CPU's `*o += w_e * yv`.
+constexpr int kDownMaxSteps = 4, kDownMaxWaves = 8;
 constexpr int kMoeWavesWanted = 1024;
 
 template <typename P, int STEPS>
-__global__ __launch_bounds__(1024) void moe_down_f32_kernel(
+__global__ __launch_bounds__(64 * kDownMaxWaves) void moe_down_f32_kernel(
     const uint8_t* __restrict__ down, size_t down_stride, const int32_t* __restrict__ ids,
     const float* __restrict__ wts, const float* __restrict__ act, float* __restrict__ out,
     const float* add_b, float* add_dst, int nff, int ne, int n_used, int S, int chunks) {
@@ -734,16 +748,16 @@ __global__ __launch_bounds__(1024) void moe_down_f32_kernel(
                 for (int s = 0; s < STEPS; ++s) {
                     const int o = (st0 + s) * rps + seg;
                     const bool ok = lane_ok && o < ne;
-                    P::load_row(row[s], dw + (size_t)(ok ? o : 0) * bpr, uc, ok);
+                    P::load_row(row[s], dw + (size_t)(ok ? o : 0) * bpr, uc, true);
                 }
                 typename P::X xa;
-                P::load_x(xa, act + (size_t)k * nff, uc, lane_ok);
+                P::load_x(xa, act + (size_t)k * nff, uc, true);
 #pragma unroll
                 for (int s = 0; s < STEPS; ++s) part[s] += P::partial(row[s], xa, uc);
             }
 #pragma unroll
             for (int s = 0; s < STEPS; ++s) {
-                const float yk = seg_sum(part[s], seg * S, S / 4);
+                const float yk = seg_sum(part[s], seg * S, S);
                 if (lane_ok && u == 0) ys[s][wave][seg] = yk;
             }
         }
