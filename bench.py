@@ -399,6 +399,52 @@ def moe_bench(be, n_layers=6):
     return out
 
 
+def moe_shapes_bench(be):
+    """One token of Op::MoeFfn at the expert shapes of other MoE files (hidden x expert FFN, experts,
+    top-k): Mixtral 8x7B, a 7168 x 2048 top-8 layer (32 experts standing in for 256), a 5120 x 8192
+    top-1 layer and Qwen3-235B-A22B's. Q4_K banks (one synthetic expert repeated), direct calls
+    that rotate over enough copies of the banks that the selected experts (71-198 MB) come from HBM.
+    Bytes = the selected experts' gate + up + down."""
+    from infr_amd import BufferUsage, DType, synth_normal_f32, synth_weight
+    out = {}
+    for name, ne, n_expert, n_used, nff in (("mixtral_8x7b", 4096, 8, 2, 14336), ("h7168_ff2048_top8", 7168, 32, 8, 2048),
+                                            ("h5120_ff8192_top1", 5120, 16, 1, 8192), ("qwen3_235b", 4096, 128, 8, 1536)):
+        protos = []
+        for i in range(3):
+            one = synth_weight(DType.Q4K, 90 + i, nff if i < 2 else ne, ne if i < 2 else nff)
+            protos.append(be.upload_new(np.tile(one, n_expert), BufferUsage.Weights))
+        active = n_used * 3 * nff * ne * 144 // 256
+        copies = max(2, -(-600_000_000 // active))
+        banks = [protos]
+        for _ in range(copies - 1):
+            layer = []
+            for proto in protos:
+                wb = be.alloc_uninit(proto.len_bytes(), BufferUsage.Weights)
+                be.copy_buffer(proto, wb, proto.len_bytes())
+                layer.append(wb)
+            banks.append(layer)
+        router = be.upload_new(synth_normal_f32(95, n_expert * ne, sigma=0.03))
+        x, y = be.upload_new(synth_normal_f32(96, ne)), be.alloc(ne * 4)
+        kw = dict(rows=1, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff, scale=1.0)
+        best = 1e30
+        for rep in range(4):
+            be.timer_begin()
+            for g, u, d in banks:
+                be.moe_ffn(x, router, g, u, d, y, **kw)
+            t = be.timer_end()
+            if rep:
+                best = min(best, t)
+        us = best * 1e3 / copies
+        out[f"moe_q4k_t1_{name}_us_per_layer"] = round(us, 1)
+        out[f"moe_q4k_t1_{name}_selected_expert_GBs"] = round(active / (us * 1e-6) / 1e9, 1)
+        for layer in banks:
+            for b in layer:
+                b.free()
+        for b in (router, x, y):
+            b.free()
+    return out
+
+
 def load_bench(be, n_layers=8):
     """A synthetic checkpoint of `n_layers` Qwen3-8B layers (Q4_K projections, Q6_K down) written
     as a GGUF file, then opened and uploaded tensor by tensor through the reader: page cache ->
@@ -465,7 +511,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-parity", action="store_true", help="skip the untimed oracle checks of the timed outputs")
     ap.add_argument("--sections", default="shapes,formats,mmq,chain,layer,ternary,moe,load",
-                    help="comma list of secondary sections: shapes, formats, mmq, chain, layer, ternary, moe, load; mmq_scaling (off by default)")
+                    help="comma list of secondary sections: shapes, formats, mmq, chain, layer, ternary, moe, load; mmq_scaling and moe_shapes (off by default)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
@@ -617,6 +663,8 @@ def main():
         tern.free()
     if "moe" in sections:
         extra.update(moe_bench(be))
+    if "moe_shapes" in sections:
+        extra.update(moe_shapes_bench(be))
     if "load" in sections:
         open_ms, up_ms, nb = load_bench(be)
         extra["gguf_open_ms"] = round(open_ms, 2)

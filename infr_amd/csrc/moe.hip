@@ -37,6 +37,21 @@ struct SelectLds {
     float red[8];
 };
 
+// Quad-major activation rows, [quad][unit][4]: unit = the 64 weights of a row that one lane of the
+// one-token expert kernels owns, quad q = the floats in its registers 4q .. 4q+3, so consecutive
+// lanes read consecutive 16 bytes. Unit and quad of the quad that starts at element e (a multiple
+// of 4): 64 consecutive elements per unit for Q4_K, Q5_K and Q8_0; for Q6_K a unit is four groups
+// of 16, 32 apart, of one half of a 256-block (the decode GEMV's mapping).
+__device__ __forceinline__ void quad_place_linear(int e, int& u, int& q) {
+    u = e >> 6;
+    q = (e & 63) >> 2;
+}
+__device__ __forceinline__ void quad_place_q6k(int e, int& u, int& q) {
+    const int r = e & 255, r2 = r & 127, r3 = r2 & 31;
+    u = (e >> 8) * 4 + (r >> 7) * 2 + (r3 >> 4);
+    q = 4 * (r2 >> 5) + ((r3 & 15) >> 2);
+}
+
 // Softmax + stable top-n_used + renormalised weights for one row, run by a whole 256-thread
 // workgroup. n_expert <= 1024, n_used <= 64. Order-sensitive parts follow the CPU: probabilities
 // are summed in index order by one thread, the stable descending sort is realised by counting
@@ -210,7 +225,7 @@ __global__ __launch_bounds__(256) void moe_router_kernel(
     const void* __restrict__ router, const float* __restrict__ rx, float* __restrict__ logits,
     int* __restrict__ tickets, int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, int ne,
     int n_expert, int rows, int n_used, float scale, int kc, int epw, int tpw, const float* __restrict__ norm_w,
-    float* __restrict__ norm_dst, float norm_eps) {
+    float* __restrict__ norm_dst, float norm_eps, float* __restrict__ xt, int xt_q6k) {
     extern __shared__ __attribute__((aligned(16))) float rl[];  // [epw] rows | [32 / epw] rows
     __shared__ __attribute__((aligned(16))) SelectLds sel;
     __shared__ int s_last;
@@ -261,6 +276,14 @@ __global__ __launch_bounds__(256) void moe_router_kernel(
                         tmp[u] = v4f{tmp[u].x * nscale * wv.x, tmp[u].y * nscale * wv.y, tmp[u].z * nscale * wv.z,
                                      tmp[u].w * nscale * wv.w};
                         if (norm_dst && blockIdx.x == 0) reinterpret_cast<v4f*>(norm_dst + k0)[q] = tmp[u];
+                    }
+                    // a single row for the one-token expert kernels: the first workgroup leaves it
+                    // quad-major, [quad][unit][4] of the gate / up format's lane mapping
+                    if (xt && row >= n_e && blockIdx.x == 0) {
+                        int xu, xq;
+                        if (xt_q6k) quad_place_q6k(k0 + 4 * q, xu, xq);
+                        else quad_place_linear(k0 + 4 * q, xu, xq);
+                        *reinterpret_cast<v4f*>(xt + ((size_t)xq * (ne / 64) + xu) * 4) = tmp[u];
                     }
                 }
             }
@@ -398,8 +421,34 @@ __global__ __launch_bounds__(kRtThreads) void moe_router_tile_kernel(const void*
 // (one conversion and one FMA per weight), which moves the result by f32 rounding only - orders
 // of magnitude inside the 1e-4 relative bound this path is held to. One policy per bank format:
 //   Row / load_row(r, row pointer, u, ok)      the lane's bytes of a weight row
-//   X   / load_x(x, activation row, u, ok)     its activation floats and the group sums it needs
+//   X   / load_x(x, source, u)                 its activation floats and the group sums it needs
 //   partial(r, x, u)                           sum over the lane's 64 weights of w * x
+
+// Where a lane's 64 activation floats come from, four at a time: quad q (0..15) of unit u is the
+// four floats from element `e` of the row on.
+//   XLinear    the row as the caller holds it: a lane's quads are 256 bytes apart from its
+//              neighbour's, so one load instruction touches 64 cache lines
+//   XLds       a round of the row staged in LDS by the whole workgroup (coalesced), four floats of
+//              padding per 64 so that the lanes' 16-byte reads spread over the banks
+//   XByQuad    a row stored quad-major, [q][unit][4]: consecutive lanes read consecutive 16 bytes.
+//              The gate / up kernel writes the activations in this order for the down kernel.
+struct XLinear {
+    const float* x;
+    __device__ v4f get(int, int, int e) const { return *reinterpret_cast<const v4f*>(x + e); }
+};
+struct XLds {
+    const float* xs;
+    int e0;  // first element of the staged round
+    __device__ static int pad(int i) { return i + (i >> 6) * 4; }
+    __device__ v4f get(int, int, int e) const { return *reinterpret_cast<const v4f*>(xs + pad(e - e0)); }
+};
+struct XByQuad {
+    const float* xt;
+    int n_units;
+    __device__ v4f get(int u, int q, int) const {
+        return *reinterpret_cast<const v4f*>(xt + ((size_t)q * n_units + u) * 4);
+    }
+};
 
 // Keeps a masked dword whole in the compiler's eyes: byte k of it then converts with one
 // v_cvt_f32_ubyte<k>, where a mask folded into each byte's extraction costs a bit-field extract more.
@@ -430,13 +479,14 @@ struct RawQ4K {
             r.hdr = r.qa = r.qb = v4i{0, 0, 0, 0};
         }
     }
-    __device__ static void load_x(X& a, const float* xrow, int u, bool ok) {
-        const float* src = xrow + (size_t)u * 64;
+    // element of the row that quad q of unit u starts at (quad_place_linear is the way back)
+    __device__ static int quad_elem(int u, int q) { return u * 64 + q * 4; }
+    template <typename Src>
+    __device__ static void load_x(X& a, const Src& src, int u) {
         float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
 #pragma unroll
         for (int k = 0; k < 16; ++k) {
-            v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
-            if (ok) v = *reinterpret_cast<const v4f*>(src + 4 * k);
+            const v4f v = src.get(u, k, quad_elem(u, k));
             a.x[4 * k + 0] = v.x; a.x[4 * k + 1] = v.y; a.x[4 * k + 2] = v.z; a.x[4 * k + 3] = v.w;
             if (k < 8) { s0 += v.x + v.y; s1 += v.z + v.w; } else { s2 += v.x + v.y; s3 += v.z + v.w; }
         }
@@ -498,7 +548,9 @@ struct RawQ5K {
             r.qb = v4i{0, 0, 0, 0};
         }
     }
-    __device__ static void load_x(X& a, const float* xrow, int u, bool ok) { RawQ4K::load_x(a, xrow, u, ok); }
+    __device__ static int quad_elem(int u, int q) { return RawQ4K::quad_elem(u, q); }
+    template <typename Src>
+    __device__ static void load_x(X& a, const Src& src, int u) { RawQ4K::load_x(a, src, u); }
     __device__ static float partial(const Row& r, const X& a, int u) {
         const int p = u & 3;
         uint32_t sc8[2], mn8[2];
@@ -544,16 +596,18 @@ struct RawQ6K {
     __device__ static void load_row(Row& r, const uint8_t* rowp, int u, bool ok) {
         FmtQ6K::load_row(r, rowp, 0, u, ok);
     }
-    __device__ static void load_x(X& a, const float* xrow, int u, bool ok) {
+    __device__ static int quad_elem(int u, int q) {
         const int h = (u >> 1) & 1, c = u & 1;
-        const float* src = xrow + (size_t)(u >> 2) * 256 + h * 128 + c * 16;
+        return (u >> 2) * 256 + h * 128 + c * 16 + 32 * (q >> 2) + 4 * (q & 3);
+    }
+    template <typename Src>
+    __device__ static void load_x(X& a, const Src& src, int u) {
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             float s0 = 0.0f, s1 = 0.0f;
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
-                if (ok) v = *reinterpret_cast<const v4f*>(src + 32 * k + 4 * q);
+                const v4f v = src.get(u, 4 * k + q, quad_elem(u, 4 * k + q));
                 a.x[16 * k + 4 * q + 0] = v.x; a.x[16 * k + 4 * q + 1] = v.y;
                 a.x[16 * k + 4 * q + 2] = v.z; a.x[16 * k + 4 * q + 3] = v.w;
                 s0 += v.x + v.y;
@@ -606,12 +660,12 @@ struct RawQ8_0 {
         FmtQ8_0::load_row(r.b0, rowp, 0, 2 * u, ok);
         FmtQ8_0::load_row(r.b1, rowp, 0, 2 * u + 1, ok);
     }
-    __device__ static void load_x(X& a, const float* xrow, int u, bool ok) {
-        const float* src = xrow + (size_t)u * 64;
+    __device__ static int quad_elem(int u, int q) { return RawQ4K::quad_elem(u, q); }
+    template <typename Src>
+    __device__ static void load_x(X& a, const Src& src, int u) {
 #pragma unroll
         for (int k = 0; k < 16; ++k) {
-            v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
-            if (ok) v = *reinterpret_cast<const v4f*>(src + 4 * k);
+            const v4f v = src.get(u, k, quad_elem(u, k));
             a.x[4 * k + 0] = v.x; a.x[4 * k + 1] = v.y; a.x[4 * k + 2] = v.z; a.x[4 * k + 3] = v.w;
         }
     }
@@ -654,7 +708,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_f32_kernel(
     const uint8_t* __restrict__ gate, const uint8_t* __restrict__ up, size_t gate_stride,
     size_t up_stride, const float* __restrict__ logits, int n_expert, int n_used, float scale,
     int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, const float* __restrict__ x,
-    float* __restrict__ act, int ne, int nff, int S, int chunks) {
+    float* __restrict__ act, int ne, int nff, int S, int chunks, int down_q6k) {
     __shared__ __attribute__((aligned(16))) SelectLds sel;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int rps = 64 / S;  // S lanes per weight row (each on `chunks` units of it), rows per wave step
@@ -666,8 +720,11 @@ __global__ __launch_bounds__(256) void moe_gate_up_f32_kernel(
     // the activation does not depend on the routing: requested first, it arrives under the selection
     // (every lane loads: idle lanes and rows past the end sit on valid units of row 0 and drop
     // their results, which keeps branches and zero fills out of the load sequence)
+    // `x` is the row in quad-major order (the router kernel leaves it so): consecutive lanes read
+    // consecutive 16 bytes
+    const XByQuad xsrc{x, ne / 64};
     typename P::X xa;
-    P::load_x(xa, x, u, true);
+    P::load_x(xa, xsrc, u);
     // Every workgroup selects for itself from the router's logits (a few hundred bytes and a few
     // barriers) instead of waiting for a selection kernel in between; the first one also leaves
     // the ranked experts and weights for the down kernel.
@@ -685,7 +742,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_f32_kernel(
     // rows longer than 64 lanes x 64 weights: unit c * S + u in round c, the partial sums added per lane
     for (int c = 0; c < chunks; ++c) {
         const int uc = c * S + u;
-        if (c) P::load_x(xa, x, uc, true);
+        if (c) P::load_x(xa, xsrc, uc);
         typename P::Row g[SPW], up_r[SPW];
 #pragma unroll
         for (int i = 0; i < SPW; ++i) {
@@ -706,7 +763,13 @@ __global__ __launch_bounds__(256) void moe_gate_up_f32_kernel(
         const bool ok = lane_ok && o < nff;
         const float gs = seg_sum(gp[i], seg * S, S);
         const float us = seg_sum(upp[i], seg * S, S);
-        if (ok && u == 0) act[(size_t)slot * nff + o] = gs / (1.0f + expf(-gs)) * us;
+        if (ok && u == 0) {
+            // stored in the order the down kernel's lanes read: [quad][unit][4] of its format
+            int du, dq;
+            if (down_q6k) quad_place_q6k(o, du, dq);
+            else quad_place_linear(o, du, dq);
+            act[(size_t)slot * nff + ((size_t)dq * (nff / 64) + du) * 4 + (o & 3)] = gs / (1.0f + expf(-gs)) * us;
+        }
     }
 }
 
@@ -751,7 +814,7 @@ __global__ __launch_bounds__(64 * kDownMaxWaves) void moe_down_f32_kernel(
                     P::load_row(row[s], dw + (size_t)(ok ? o : 0) * bpr, uc, true);
                 }
                 typename P::X xa;
-                P::load_x(xa, act + (size_t)k * nff, uc, true);
+                P::load_x(xa, XByQuad{act + (size_t)k * nff, nff / 64}, uc);
 #pragma unroll
                 for (int s = 0; s < STEPS; ++s) part[s] += P::partial(row[s], xa, uc);
             }
@@ -1140,7 +1203,8 @@ static bool launch_moe_down_fused(int dtype, const uint8_t* bank, size_t stride,
 template <int WT>
 static void launch_row_dots(const void* w, const float* x, float* logits, int ne, int n_rows_w, int rows,
                             bool logits_only, int* tickets, int32_t* sel_idx, float* sel_w, int n_used, float scale,
-                            const float* norm_w, float* norm_dst, float norm_eps, hipStream_t stream) {
+                            const float* norm_w, float* norm_dst, float norm_eps, float* xt, int xt_q6k,
+                            hipStream_t stream) {
     // One weight row per workgroup when only logits are wanted of a single row (nothing to wait
     // for); eight at a single row that ends in the selection (few tickets), four once rows fill the
     // pairs; whole rows in one chunk when they fit the LDS a workgroup may have, else kRouterChunk
@@ -1173,19 +1237,19 @@ static void launch_row_dots(const void* w, const float* x, float* logits, int ne
     else if (rows == 1)
         hipLaunchKernelGGL((moe_router_kernel<24, WT>), dim3((unsigned)((n_rows_w + epw - 1) / epw), 1), dim3(256), router_lds,
                            stream, w, x, logits, logits_only ? (int*)nullptr : tickets, sel_idx, sel_w, ne,
-                           n_rows_w, rows, n_used, scale, kc, epw, tpw, norm_w, norm_dst, norm_eps);
+                           n_rows_w, rows, n_used, scale, kc, epw, tpw, norm_w, norm_dst, norm_eps, xt, xt_q6k);
     else if (whole_rows && router_lds > 64 * 1024)
         hipLaunchKernelGGL((moe_router_kernel<24, WT>),
                            dim3((unsigned)((n_rows_w + epw - 1) / epw), (unsigned)((rows + tpw - 1) / tpw)),
                            dim3(256), router_lds, stream, w, x, logits, (int*)nullptr, sel_idx, sel_w,
                            ne, n_rows_w, rows, n_used, scale, kc, epw, tpw, (const float*)nullptr, (float*)nullptr,
-                           0.0f);
+                           0.0f, (float*)nullptr, 0);
     else
         hipLaunchKernelGGL((moe_router_kernel<8, WT>),
                            dim3((unsigned)((n_rows_w + epw - 1) / epw), (unsigned)((rows + tpw - 1) / tpw)),
                            dim3(256), router_lds, stream, w, x, logits, (int*)nullptr, sel_idx, sel_w,
                            ne, n_rows_w, rows, n_used, scale, kc, epw, tpw, (const float*)nullptr, (float*)nullptr,
-                           0.0f);
+                           0.0f, (float*)nullptr, 0);
 }
 
 // Op::Linear over plain f32 / f16 / bf16 weight rows (crates/infr-cpu/src/lib.rs:1162-1165,
@@ -1194,12 +1258,23 @@ bool launch_linear_plain_rows(int dtype, const void* w, const float* x, float* y
                               hipStream_t stream) {
     if (in_f % 32 != 0 || in_f > (size_t)1 << 30 || out_f > (size_t)1 << 30 || m > (size_t)1 << 30) return false;
     switch (dtype) {
-    case 0: launch_row_dots<0>(w, x, y, (int)in_f, (int)out_f, (int)m, true, nullptr, nullptr, nullptr, 0, 0.0f, nullptr, nullptr, 0.0f, stream); break;
-    case 1: launch_row_dots<1>(w, x, y, (int)in_f, (int)out_f, (int)m, true, nullptr, nullptr, nullptr, 0, 0.0f, nullptr, nullptr, 0.0f, stream); break;
-    case 30: launch_row_dots<30>(w, x, y, (int)in_f, (int)out_f, (int)m, true, nullptr, nullptr, nullptr, 0, 0.0f, nullptr, nullptr, 0.0f, stream); break;
+    case 0: launch_row_dots<0>(w, x, y, (int)in_f, (int)out_f, (int)m, true, nullptr, nullptr, nullptr, 0, 0.0f, nullptr, nullptr, 0.0f, nullptr, 0, stream); break;
+    case 1: launch_row_dots<1>(w, x, y, (int)in_f, (int)out_f, (int)m, true, nullptr, nullptr, nullptr, 0, 0.0f, nullptr, nullptr, 0.0f, nullptr, 0, stream); break;
+    case 30: launch_row_dots<30>(w, x, y, (int)in_f, (int)out_f, (int)m, true, nullptr, nullptr, nullptr, 0, 0.0f, nullptr, nullptr, 0.0f, nullptr, 0, stream); break;
     default: return false;
     }
     return hipGetLastError() == hipSuccess;
+}
+
+// A row into quad-major order (the expert input when it is not the row the router reads).
+__global__ __launch_bounds__(256) void moe_quad_major_kernel(const float* __restrict__ x, float* __restrict__ xt, int ne,
+                                                            int q6k) {
+    const int e = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (e >= ne) return;
+    int u, q;
+    if (q6k) quad_place_q6k(e, u, q);
+    else quad_place_linear(e, u, q);
+    *reinterpret_cast<v4f*>(xt + ((size_t)q * (ne / 64) + u) * 4) = *reinterpret_cast<const v4f*>(x + e);
 }
 
 size_t moe_workspace_bytes(const MoeShape& s) {
@@ -1271,10 +1346,18 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     // prologue, so the router only leaves the logits - one expert per workgroup, nothing to wait for.
     auto raw_ok = [](int dt) { return dt == 12 || dt == 13 || dt == 14 || dt == 8; };
     const bool fast1 = s.rows == 1 && raw_ok(s.gate_dtype) && s.up_dtype == s.gate_dtype && raw_ok(s.down_dtype);
+    // (one token on the factored kernels: the router's first workgroup also leaves the row
+    // quad-major for them, in the space of the per-pair down outputs that path does not use)
+    float* xt = fast1 ? yp : nullptr;
+    const bool router_row_is_x = b.x == b.router_x || b.norm_w;
+    if (fast1 && !router_row_is_x)
+        hipLaunchKernelGGL(moe_quad_major_kernel, dim3((unsigned)((s.ne / 4 + 255) / 256)), dim3(256), 0, stream, b.x, xt,
+                           s.ne, s.gate_dtype == 14 ? 1 : 0);
+    float* router_xt = router_row_is_x ? xt : nullptr;
     switch (s.router_dtype) {
-    case 0: launch_row_dots<0>(b.router, b.router_x, logits, s.ne, s.n_expert, s.rows, fast1, tickets, sel_idx, sel_w, s.n_used, s.scale, b.norm_w, b.norm_dst, b.norm_eps, stream); break;
-    case 1: launch_row_dots<1>(b.router, b.router_x, logits, s.ne, s.n_expert, s.rows, fast1, tickets, sel_idx, sel_w, s.n_used, s.scale, b.norm_w, b.norm_dst, b.norm_eps, stream); break;
-    default: launch_row_dots<30>(b.router, b.router_x, logits, s.ne, s.n_expert, s.rows, fast1, tickets, sel_idx, sel_w, s.n_used, s.scale, b.norm_w, b.norm_dst, b.norm_eps, stream); break;
+    case 0: launch_row_dots<0>(b.router, b.router_x, logits, s.ne, s.n_expert, s.rows, fast1, tickets, sel_idx, sel_w, s.n_used, s.scale, b.norm_w, b.norm_dst, b.norm_eps, router_xt, s.gate_dtype == 14 ? 1 : 0, stream); break;
+    case 1: launch_row_dots<1>(b.router, b.router_x, logits, s.ne, s.n_expert, s.rows, fast1, tickets, sel_idx, sel_w, s.n_used, s.scale, b.norm_w, b.norm_dst, b.norm_eps, router_xt, s.gate_dtype == 14 ? 1 : 0, stream); break;
+    default: launch_row_dots<30>(b.router, b.router_x, logits, s.ne, s.n_expert, s.rows, fast1, tickets, sel_idx, sel_w, s.n_used, s.scale, b.norm_w, b.norm_dst, b.norm_eps, router_xt, s.gate_dtype == 14 ? 1 : 0, stream); break;
     }
     auto bytes_per_row = [](int dtype, size_t in_f) -> size_t {
         switch (dtype) {
@@ -1352,8 +1435,8 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
         const dim3 grid_g((unsigned)((steps_g + 4 * spw - 1) / (4 * spw)), (unsigned)s.n_used);
 #define INFR_GATE_UP_N(P, N)                                                                                  \
     hipLaunchKernelGGL((moe_gate_up_f32_kernel<P, N>), grid_g, dim3(256), 0, stream, b.gate, b.up, b.gate_stride, \
-                       b.up_stride, logits, s.n_expert, s.n_used, s.scale, sel_idx, sel_w, b.x, gbuf, s.ne, s.n_ff, \
-                       lanes_g, chunks_g)
+                       b.up_stride, logits, s.n_expert, s.n_used, s.scale, sel_idx, sel_w, xt, gbuf, s.ne, s.n_ff, \
+                       lanes_g, chunks_g, s.down_dtype == 14 ? 1 : 0)
 #define INFR_GATE_UP(P)                 \
     switch (spw) {                      \
     case 1: INFR_GATE_UP_N(P, 1); break; \

@@ -389,3 +389,26 @@ def test_moe_one_token_rows_in_several_rounds(be, dtype, ne, nff):
     want = orc.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
                        gate_dtype=int(dtype), up_dtype=int(dtype), down_dtype=int(dtype))
     check(*got, *want)
+
+
+@pytest.mark.parametrize("rows", [1, 4])
+@pytest.mark.parametrize("dtype", [DType.Q4K, DType.Q6K])
+def test_moe_router_reads_another_row_than_the_experts(be, dtype, rows):
+    """`router_x` distinct from `x`: the selection comes from one tensor, the expert inputs from
+    another (at one token the expert kernels read their row in an order of their own, which the
+    router kernel cannot leave for them when its row is a different one)."""
+    ne, n_expert, n_used, nff = 1024, 8, 2, 512
+    gate, up, down = banks(420, ne, n_expert, nff, dtype, sigma=0.03)
+    x = synth_normal_f32(421, rows * ne)
+    rx = synth_normal_f32(422, rows * ne)
+    router = synth_normal_f32(423, n_expert * ne, sigma=0.05)
+    xb, rxb, rb = be.upload_new(x), be.upload_new(rx), be.upload_new(router)
+    gb, ub, db = be.upload_new(gate), be.upload_new(up), be.upload_new(down)
+    yb, ib, wb = be.alloc(rows * ne * 4), be.alloc(rows * n_used * 4), be.alloc(rows * n_used * 4)
+    be.moe_ffn(xb, rb, gb, ub, db, yb, rows=rows, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff, scale=1.0,
+               gate_dtype=dtype, up_dtype=dtype, down_dtype=dtype, router_x=rxb, sel_idx=ib, sel_w=wb)
+    got = (be.download(yb, np.empty((rows, ne), np.float32)), be.download(ib, np.empty((rows, n_used), np.int32)),
+           be.download(wb, np.empty((rows, n_used), np.float32)))
+    want = orc.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
+                       gate_dtype=int(dtype), up_dtype=int(dtype), down_dtype=int(dtype), router_x=rx)
+    check(*got, *want)
