@@ -1431,7 +1431,10 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
         const int lanes_g = row_lanes(s.ne / 64), chunks_g = s.ne / 64 / lanes_g;
         const int rps_g = 64 / lanes_g;
         const int steps_g = (s.n_ff + rps_g - 1) / rps_g;
-        const int spw = steps_per_wave(steps_g * s.n_used);
+        // (Q8_0 rows are 1.9x the bytes of Q4_K's: four steps of gate and up rows in flight leave
+        // one wave per SIMD, two steps three)
+        int spw = std::min(s.gate_dtype == 8 ? 2 : 4, steps_per_wave(steps_g * s.n_used));
+        if (s.gate_dtype == 14 && spw == 3) spw = 2;  // (three steps of Q6_K rows compile to one wave per SIMD, two to three)
         const dim3 grid_g((unsigned)((steps_g + 4 * spw - 1) / (4 * spw)), (unsigned)s.n_used);
 #define INFR_GATE_UP_N(P, N)                                                                                  \
     hipLaunchKernelGGL((moe_gate_up_f32_kernel<P, N>), grid_g, dim3(256), 0, stream, b.gate, b.up, b.gate_stride, \
