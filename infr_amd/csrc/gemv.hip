@@ -60,8 +60,10 @@ bool plan_batch_group(int dtype, size_t m, size_t in_f, const GemvOpDesc* ops, i
     BatchGroupPlan gp;
     size_t max_out_f = 0;
     for (int i = 0; i < n; ++i) max_out_f = std::max(max_out_f, (size_t)ops[i].out_f);
+    // (Q8_0 at 5..8 tokens on rows of 8192 columns and more: only when the group fills the device twice over)
+    const bool q8_0_long = dtype == 8 && m >= 5 && m <= 8 && in_f % 256 == 0 && in_f >= 8192 && total_rows >= 8192;
     if ((dtype != 12 || m > 32) &&
-        mmq_skinny16_takes(dtype, m, in_f, max_out_f)) {  // the K-split MFMA kernel
+        (q8_0_long || mmq_skinny16_takes(dtype, m, in_f, max_out_f))) {  // the K-split MFMA kernel
         gp.kind = 1;
         gp.rows_per_wg = 32;
     } else if (dtype == 12 && m > 2) {  // Q4_K from three tokens: the K-split MFMA kernels, 32 rows per workgroup

@@ -142,8 +142,9 @@ bool launch_gemv_batch_group(int dtype, size_t m, size_t in_f, const BatchTile* 
                              const BatchGroupPlan& plan, const ActQ8& act, hipStream_t stream);
 void launch_mmq_skinny_group(int dtype, size_t m, size_t in_f, const BatchTile* tiles_dev,
                              const BatchGroupPlan& plan, const ActQ8& act, hipStream_t stream);
-// Q4_K / Q5_K batches of 2..16 tokens on rows of an even number of 256-blocks: the K-split MFMA
-// kernel with 16 x 16 tiles (mmq.hip) takes them, alone or as a plan's group of 32-row tiles.
+// Small and middle batches on rows of whole 256-blocks (an even number of them for Q6_K and Q2_0):
+// whether the K-split MFMA kernel with 16 x 16 tiles (mmq.hip) takes them, alone or as a plan's
+// group of 32-row tiles; the thresholds are per format, row length and matrix size.
 bool mmq_skinny16_takes(int dtype, size_t m, size_t in_f, size_t out_f);
 
 // Which activation quantizer infr-cpu's dispatch pairs with a weight format

@@ -1174,6 +1174,10 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
     for (int pass = 0; pass < n_pass; ++pass) {
         const int b0 = (pass * NW + wave) * BPW;
         const int b0_next = b0 + NW * BPW;  // next pass (past the end: clamped, never used)
+        // A row of an odd number of blocks ends in a stage of one block: that stage starts a block
+        // early (request_rows), so block b0 + j sits in slot (j + 1) % BPW of the weight tile and of
+        // the scales; the slot that holds the block before is never summed (b0 + j < nb below).
+        const int slot0 = BPW == 2 && b0 == nb - 1 ? 1 : 0;
         // the activation scales of the wave's blocks: dq_l[token][j]
         if constexpr (F::kPer32Acts) {
             if (lane < MT * kDqQuads)
@@ -1201,10 +1205,11 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
             }
             wave_sync();
             int raw[kSub && F::kPer32Acts ? 32 : 1];  // the integers behind a policy's f32 terms (stage outputs)
+            const int slot = (j + slot0) % kPh;
             if constexpr (kSub && F::kPer32Acts)
-                F::template block<MT, kDq>(wfrag, j % kPh, afrag, tile + kBsOff, &dq_l[wave][0][0], kq, sd[j], raw);
-            else if constexpr (kSub) F::block(wfrag, j % kPh, afrag, kq, sd[j], ddm[j]);
-            else F::block(wfrag, j % kPh, afrag, zrow, bsfrag, kq, sd[j], sm[j], ddm[j][0]);
+                F::template block<MT, kDq>(wfrag, slot, afrag, tile + kBsOff, &dq_l[wave][0][0], kq, sd[j], raw);
+            else if constexpr (kSub) F::block(wfrag, slot, afrag, kq, sd[j], ddm[j]);
+            else F::block(wfrag, slot, afrag, zrow, bsfrag, kq, sd[j], sm[j], ddm[j][0]);
             if (STAGES) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
@@ -1240,12 +1245,12 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
                         if constexpr (kSub) {
                             float dqv[4];
 #pragma unroll
-                            for (int i = 0; i < 4; ++i) dqv[i] = dq_l[wave][(4 * kq + i) & (MT - 1)][j];
+                            for (int i = 0; i < 4; ++i) dqv[i] = dq_l[wave][(4 * kq + i) & (MT - 1)][(j + slot0) % BPW];
                             F::accumulate(acc, dqv, ddm[j], sd[j]);
                         } else {
 #pragma unroll
                             for (int i = 0; i < 4; ++i)
-                                acc[i] = F::accumulate(acc[i], dq_l[wave][(4 * kq + i) & (MT - 1)][j], ddm[j][0], sd[j][i], sm[j][i]);
+                                acc[i] = F::accumulate(acc[i], dq_l[wave][(4 * kq + i) & (MT - 1)][(j + slot0) % BPW], ddm[j][0], sd[j][i], sm[j][i]);
                         }
                     }
                 }
@@ -1263,26 +1268,30 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
     }
 }
 
-// Which batches the 16-token K-split kernel takes: rows (of any quantized format) of an even number of
-// 256-blocks (weights are staged two blocks at a time), up to 16 tokens. Four waves per workgroup;
+// Which batches the 16-token K-split kernel takes: rows (of any quantized format) of two 256-blocks
+// and more. Weights are staged two blocks at a time; a row of an odd number ends in a stage that starts
+// a block early, which needs every block 16-byte aligned in every row - not so for Q6_K (210 bytes) and
+// Q2_0 (72): their rows must be an even number of blocks. Four waves per workgroup;
 // (eight measured no faster, and four blocks per wave and pass - 576-byte, 64-byte-aligned runs per
 // row - measured 20-25 % slower: a wave then computes for longer before it asks for more).
 constexpr int kSkinny16Waves = 4, kSkinny16Blocks = 2;
 static bool skinny16_shape(int dtype, int nb, size_t m, size_t out_f) {
     const bool nib32 = dtype == 2 || dtype == 3 || dtype == 6 || dtype == 7 || dtype == 20;
     if (dtype != 12 && dtype != 13 && dtype != 14 && dtype != 8 && dtype != 42 && !nib32) return false;
-    if (nb < kSkinny16Blocks || nb % kSkinny16Blocks != 0) return false;
+    if (nb < kSkinny16Blocks || (nb % kSkinny16Blocks != 0 && (dtype == 14 || dtype == 42))) return false;
     if (m <= 16) {
         // the dot4 batch kernels, which unpack a weight once per two or four tokens, stay ahead at the
         // bottom: Q4_K at two tokens (4.3 / 4.0 / 5.5 / 5.6 against 3.7 / 3.4 / 4.2 / 4.2 TB/s on the four
         // layer shapes; level from three), Q5_K at two (4.3-5.3 against 3.8-4.4), Q6_K up to four
         // (3.6-4.5 against 3.3-3.9)
         if ((dtype == 12 && m < 3) || (dtype == 13 && m < 3) || (dtype == 14 && m < 5)) return false;
-        // Q8_0: the dot4 batches stay ahead up to eight tokens on rows of one or two wave steps (4.2 / 3.8 /
-        // 4.8 against 3.8 / 3.3 / 4.2 TB/s at eight tokens on the 4096-column shapes, 5.1-5.9 at two to
-        // four); this kernel takes 9..16 tokens (one pass over the weights instead of two) and, from
-        // five tokens, rows of 8192 columns and more (4.4 against 3.95 TB/s at 4096 x 12288)
-        if (dtype == 8 && !(m > 8 || (m >= 5 && nb >= 32))) return false;
+        // Q8_0: the dot4 batches stay ahead up to eight tokens (4.2 / 3.8 / 4.8 against 3.8 / 3.3 / 4.2 TB/s
+        // at eight tokens on the 4096-column shapes, 5.1-5.9 at two to four; on rows of 8192 columns and
+        // more this kernel is ahead by a tenth when forty such ops share a launch, 4.4 against 3.95 TB/s,
+        // but a single 4096 x 12288 op - what a layer has - takes 29 us here against 19 there: a plan's
+        // group of 8192 rows and more comes here from five tokens, out_f == 0); this kernel takes
+        // 9..16 tokens (one pass over the weights instead of two)
+        if (dtype == 8 && m <= 8 && !(out_f == 0 && m >= 5 && nb >= 32)) return false;
         // Q2_0: 72 bytes a step make this kernel compute-bound (1.0-1.3 TB/s at any token count, what the
         // dot4 batches reach at eight tokens): it takes 9 tokens and more, where they would need two passes
         if (dtype == 42 && m <= 8) return false;
@@ -1331,6 +1340,22 @@ static void launch_mmq_skinny16_fmt(const uint8_t* w, size_t bpr, const ActQ8& a
                                     size_t out_f, size_t wgs, const IntStages& st, const BatchTile* tiles,
                                     hipStream_t stream) {
     const dim3 grid((unsigned)wgs, 2, (unsigned)((m + 15) / 16)), block(kSkinny16Waves * 64);
+    // At most one workgroup per compute unit (one op of up to 4096 rows and 16 tokens: a down
+    // projection on its own level of a plan) and long rows: eight waves share a row's blocks
+    // instead of four, twice the requests in flight (4096 x 12288 at 8 tokens, per call with its
+    // quantizer: Q4_K 17.4 -> 15.3 us, Q8_0 at 16 tokens 29.2 -> 27.3). With more workgroups than
+    // that the four-wave form is as fast or faster (512 workgroups: 33 against 49 us).
+    if constexpr (!STAGES) {
+        if (wgs * 2 * grid.z <= 256 && nb >= 32) {
+            if (m <= 8)
+                hipLaunchKernelGGL((mmq_skinny16_kernel<F, 8, kSkinny16Blocks, 8, false>), grid, dim3(512), 0, stream,
+                                   w, bpr, act.qs, act.d, act.bsums, y, (int)m, (int)out_f, nb, st.a, st.b, tiles);
+            else
+                hipLaunchKernelGGL((mmq_skinny16_kernel<F, 8, kSkinny16Blocks, 16, false>), grid, dim3(512), 0, stream,
+                                   w, bpr, act.qs, act.d, act.bsums, y, (int)m, (int)out_f, nb, st.a, st.b, tiles);
+            return;
+        }
+    }
     if (m <= 8)
         hipLaunchKernelGGL((mmq_skinny16_kernel<F, kSkinny16Waves, kSkinny16Blocks, 8, STAGES>), grid, block, 0, stream,
                            w, bpr, act.qs, act.d, act.bsums, y, (int)m, (int)out_f, nb, st.a, st.b, tiles);

@@ -220,10 +220,10 @@ def test_small_batch_kquant_mfma_is_bit_identical_to_oracle(be, dtype, m, in_f, 
     assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), "not bit-identical"
 
 
-@pytest.mark.parametrize("m,in_f,out_f", [(9, 4096, 48), (13, 512, 40), (16, 5632, 24), (12, 1024, 70), (6, 8192, 40),
-                                          (5, 12288, 33)])
+@pytest.mark.parametrize("m,in_f,out_f", [(9, 4096, 48), (13, 512, 40), (16, 5632, 24), (12, 1024, 70), (10, 8192, 40),
+                                          (15, 12288, 33)])
 def test_q8_0_on_the_sixteen_token_mfma_kernel_is_bit_identical_to_oracle(be, m, in_f, out_f):
-    """9..16 tokens of Q8_0 (and 5..8 on rows of 8192 columns up) take the K-split MFMA kernel: one
+    """9..16 tokens of Q8_0 take the K-split MFMA kernel (eight waves per workgroup on the two long-row shapes): one
     exact iprod per 34-byte block and the CPU's chain `sumf += (q8.d * d_w) * iprod` block by block
     (crates/infr-cpu/src/kernels.rs:1170-1187) handed from wave to wave, so unlike the dot4 batches
     these outputs equal the scalar kernel's bits; the per-block integers are exact as everywhere."""
@@ -273,6 +273,29 @@ def test_batches_beyond_sixteen_tokens_on_the_k_split_kernel(be, dtype, m):
     assert np.array_equal(a, oa)
     if dtype in (DType.Q4K, DType.Q5K):
         assert np.array_equal(b, ob)
+
+
+@pytest.mark.parametrize("m", [3, 8, 16, 24, 40, 64])
+@pytest.mark.parametrize("dtype", [DType.Q4K, DType.Q5K, DType.Q8_0, DType.Q4_0, DType.Q5_1])
+def test_k_split_kernel_on_rows_of_an_odd_number_of_blocks(be, dtype, m):
+    """Rows of 3, 9 and 43 blocks of 256 (768, 2304 and 11008 columns: Llama-2-7B's and Qwen2.5's
+    down projections are such rows): the kernel stages weights two blocks at a time and the last,
+    single block of a row arrives in a stage that starts a block early. Outputs bit-identical to the
+    oracle's scalar kernels, the per-block integers exact (the last block's included)."""
+    if dtype in (DType.Q8_0, DType.Q4_0, DType.Q5_1) and m <= 8:
+        pytest.skip("these formats take the dot4 batches up to eight tokens")
+    for in_f, out_f in ((768, 70), (2304, 33), (11008, 40)):
+        w = orc.synth_weight(dtype, in_f * out_f, 0x30D + in_f)
+        x = orc.gen_f32(m * in_f, 0x30D ^ 0x9E37)
+        x[in_f:2 * in_f] = 0.0
+        y = run_linear(be, dtype, w, x, m, in_f, out_f)
+        want = orc.linear(dtype, w, x, m, in_f, out_f).reshape(m, out_f)
+        assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), f"not bit-identical at {in_f} x {out_f}"
+        a, b = be.linear_int_stages(dtype, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
+        oa, ob = orc.linear_int_stages(dtype, w, x, m, in_f, out_f)
+        assert np.array_equal(a, oa), f"first integer stage at {in_f} x {out_f}"
+        if dtype in (DType.Q4K, DType.Q5K):
+            assert np.array_equal(b, ob), f"second integer stage at {in_f} x {out_f}"
 
 
 @pytest.mark.parametrize("m,in_f,out_f", [(6, 4608, 40), (13, 1024, 50)])
