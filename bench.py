@@ -216,11 +216,12 @@ def settle_clocks(be, plan, binds, seconds=0.03):
             break
 
 
-def layer_bench(be, n_layers, dtype=None):
+def layer_bench(be, n_layers, dtype=None, rows=1):
     """A decode step through `n_layers` Qwen3-8B-shaped decoder layers without attention:
     RmsNorm -> {q, k, v} -> o(q) -> Add -> RmsNorm -> {gate, up} -> GatedAct -> down -> Add, every op
     reading what the previous one wrote. The plan absorbs the norms, the gated activation and the
-    residual adds into the decode GEMVs (4 launches per layer instead of 9). Returns
+    residual adds into the decode GEMVs (4 launches per layer instead of 9) at one token; `rows`
+    tokens (a decode batch) run the ops as they are, Linears of a level grouped. Returns
     (ms per step, weight bytes, launches per step)."""
     from infr_amd import (Add, Bindings, BufferUsage, DType, GatedAct, Graph, Linear, RmsNorm, TensorDesc,
                           synth_normal_f32, synth_weight)
@@ -237,7 +238,8 @@ def layer_bench(be, n_layers, dtype=None):
         keep.append(b)
         binds.bind(t, b)
         return t
-    x = f32((1, H), synth_normal_f32(1, H))
+    R = rows
+    x = f32((R, H), synth_normal_f32(1, R * H))
     protos = {name: be.upload_new(synth_weight(dtype, i, out_f, in_f), BufferUsage.Weights)
               for i, (name, out_f, in_f) in enumerate(LAYER)}
     keep += list(protos.values())
@@ -255,20 +257,20 @@ def layer_bench(be, n_layers, dtype=None):
             binds.bind(w[name], wb)
             total += nb
         n1, n2 = (f32((H,), synth_normal_f32(2 + i, H, mean=1.0, sigma=0.1)) for i in range(2))
-        h1, q, k, v, o = (f32((1, d), out=True) for d in (H, H, KV, KV, H))
-        h2, gt, up, act, dn = (f32((1, d), out=True) for d in (H, FF, FF, FF, H))
-        g.push(RmsNorm(x, n1, h1, 1, H, 1e-6))
-        g.push(Linear(h1, w["q"], q, 1, H, H))
-        g.push(Linear(h1, w["k"], k, 1, H, KV))
-        g.push(Linear(h1, w["v"], v, 1, H, KV))
-        g.push(Linear(q, w["o"], o, 1, H, H))
-        g.push(Add(o, x, x, H))
-        g.push(RmsNorm(x, n2, h2, 1, H, 1e-6))
-        g.push(Linear(h2, w["gate"], gt, 1, H, FF))
-        g.push(Linear(h2, w["up"], up, 1, H, FF))
-        g.push(GatedAct(gt, up, act, 1, FF))
-        g.push(Linear(act, w["down"], dn, 1, FF, H))
-        g.push(Add(dn, x, x, H))
+        h1, q, k, v, o = (f32((R, d), out=True) for d in (H, H, KV, KV, H))
+        h2, gt, up, act, dn = (f32((R, d), out=True) for d in (H, FF, FF, FF, H))
+        g.push(RmsNorm(x, n1, h1, R, H, 1e-6))
+        g.push(Linear(h1, w["q"], q, R, H, H))
+        g.push(Linear(h1, w["k"], k, R, H, KV))
+        g.push(Linear(h1, w["v"], v, R, H, KV))
+        g.push(Linear(q, w["o"], o, R, H, H))
+        g.push(Add(o, x, x, R * H))
+        g.push(RmsNorm(x, n2, h2, R, H, 1e-6))
+        g.push(Linear(h2, w["gate"], gt, R, H, FF))
+        g.push(Linear(h2, w["up"], up, R, H, FF))
+        g.push(GatedAct(gt, up, act, R, FF))
+        g.push(Linear(act, w["down"], dn, R, FF, H))
+        g.push(Add(dn, x, x, R * H))
     be.sync()
     plan = be.compile(g)
     settle_clocks(be, plan, binds)
@@ -640,6 +642,10 @@ def main():
         extra["decode_layer_Q4_K_GBs"] = round(nb / (ms * 1e-3) / 1e9, 1)
         extra["decode_layer_us_per_layer"] = round(ms * 1e3 / args.layers, 2)
         extra["decode_layer_launches_per_step"] = launches
+        for rows in (8, 16):
+            ms, nb, launches = layer_bench(be, args.layers, rows=rows)
+            extra[f"decode_layer_m{rows}_us_per_layer"] = round(ms * 1e3 / args.layers, 2)
+            extra[f"decode_layer_m{rows}_launches_per_step"] = launches
         if os.environ.get("INFR_HIP_FUSE", "1") != "0":
             # the same plan with the absorption switched off (a fresh process: the switch is read once)
             import subprocess

@@ -1152,15 +1152,91 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
         }
     }
 
-    int max_level = 0;
-    for (size_t i = 0; i < n; ++i) {
-        if (absorbed[i]) continue;
-        for (size_t j = 0; j < i; ++j) {
-            if (absorbed[j]) continue;
-            if (any_overlap(wr[j], rd[i]) || any_overlap(wr[j], wr[i]) || any_overlap(rd[j], wr[i]))
-                level[i] = std::max(level[i], level[j] + 1);
+    // Two rows and more: a RmsNorm or a gated activation whose output only feeds small-batch
+    // Linears of the same shape is evaluated by those Linears' quantizer launch (a workgroup
+    // applies the op to the floats it is about to quantize, with the stand-alone kernel's
+    // arithmetic, and stores them): one launch less per op, same bits. The users must end up on
+    // one level - the quantizers of a level all run before anything later - which is checked once
+    // the levels are known; a fold that fails the check is undone.
+    struct QuantFold {
+        size_t k;
+        std::vector<size_t> users;
+        std::vector<std::vector<Span>> users_rd;
+        std::vector<Span> front_wr;
+    };
+    std::vector<QuantFold> folds;
+    std::vector<int> qpre(n, -1);
+    for (size_t k = 0; env_fuse && k < n; ++k) {
+        const auto& p = plan->ops[k];
+        const bool gated = (p.kind == INFR_OP_GATED_ACT && p.gate_block_width == 0) || p.kind == INFR_OP_GATED_ACT_FUSED;
+        if (!(gated || p.kind == INFR_OP_RMS_NORM) || p.m < 2 || p.in_f % 256 != 0 || absorbed[k]) continue;
+        if (p.kind == INFR_OP_GATED_ACT && (p.up_off % 4 != 0 || p.up_stride % 4 != 0 || p.gate_stride % 4 != 0)) continue;
+        if (any_overlap(wr[k], rd[k])) continue;
+        size_t end = n - 1;
+        for (size_t j = k + 1; j < n; ++j) {
+            if (!any_overlap(wr[j], wr[k])) continue;
+            bool covers = false;
+            for (const auto& w : wr[j]) covers = covers || (w.lo <= wr[k][0].lo && w.hi >= wr[k][0].hi);
+            if (covers) end = j;
+            break;
         }
-        max_level = std::max(max_level, level[i]);
+        std::vector<size_t> users;
+        bool ok = true;
+        for (size_t i = k + 1; ok && i <= end; ++i) {
+            if (!any_overlap(rd[i], wr[k])) continue;
+            const auto& u = plan->ops[i];
+            ok = u.kind == INFR_OP_LINEAR && small_batch(u) && u.m == p.m && u.in_f == p.in_f && !self_alias(i) &&
+                 qpre[i] < 0 && static_cast<const float*>(bindings[u.x]->ptr) == ea[k].dst;
+            if (ok) users.push_back(i);
+        }
+        if (!ok || users.empty()) continue;
+        for (size_t j = k + 1; ok && j <= users.back(); ++j)
+            ok = !any_overlap(wr[j], rd[k]) && !any_overlap(wr[j], wr[k]);
+        if (!ok) continue;
+        QuantFold f;
+        f.k = k;
+        f.users = users;
+        for (size_t u : users) f.users_rd.push_back(rd[u]);
+        f.front_wr = wr[users.front()];
+        absorbed[k] = 1;
+        for (size_t u : users) {
+            qpre[u] = (int)k;
+            rd[u][0] = rd[k][0];
+            for (size_t q = 1; q < rd[k].size(); ++q) rd[u].push_back(rd[k][q]);
+        }
+        wr[users.front()].push_back(wr[k][0]);
+        folds.push_back(std::move(f));
+    }
+
+    int max_level = 0;
+    for (;;) {
+        max_level = 0;
+        std::fill(level.begin(), level.end(), 0);
+        for (size_t i = 0; i < n; ++i) {
+            if (absorbed[i]) continue;
+            for (size_t j = 0; j < i; ++j) {
+                if (absorbed[j]) continue;
+                if (any_overlap(wr[j], rd[i]) || any_overlap(wr[j], wr[i]) || any_overlap(rd[j], wr[i]))
+                    level[i] = std::max(level[i], level[j] + 1);
+            }
+            max_level = std::max(max_level, level[i]);
+        }
+        bool undone = false;
+        for (auto& f : folds) {
+            if (f.users.empty()) continue;
+            bool same = true;
+            for (size_t u : f.users) same = same && level[u] == level[f.users.front()];
+            if (same) continue;
+            absorbed[f.k] = 0;
+            for (size_t q = 0; q < f.users.size(); ++q) {
+                rd[f.users[q]] = f.users_rd[q];
+                qpre[f.users[q]] = -1;
+            }
+            wr[f.users.front()] = f.front_wr;
+            f.users.clear();
+            undone = true;
+        }
+        if (!undone) break;
     }
     auto fusion_of = [&](size_t k) {
         infr::GemvFusion f;
@@ -1206,6 +1282,7 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
                 st.m = op.m;
                 st.first = (int)plan->descs.size();
                 std::vector<const float*> xs;
+                std::vector<int> xs_pre;  // per activation tensor: the op folded into its quantizer tiles (-1: none)
                 std::vector<uint32_t> elem0;
                 const size_t x_elems = ((size_t)op.m * op.in_f + 255) / 256 * 256;
                 for (size_t k = i; k < n; ++k) {
@@ -1217,7 +1294,10 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
                     const float* x = static_cast<const float*>(bindings[o2.x]->ptr);
                     size_t xi = 0;
                     while (xi < xs.size() && xs[xi] != x) ++xi;
-                    if (xi == xs.size()) xs.push_back(x);
+                    if (xi == xs.size()) {
+                        xs.push_back(x);
+                        xs_pre.push_back(qpre[k]);
+                    }
                     elem0.push_back((uint32_t)(xi * x_elems));
                     plan->descs.push_back(infr::GemvOpDesc{la[k].wrows, x, static_cast<float*>(bindings[o2.dst]->ptr),
                                                            la[k].bpr, (int32_t)o2.out_f});
@@ -1234,10 +1314,44 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
                 infr::fill_batch_tiles(&plan->descs[st.first], elem0.data(), st.n, st.bp, &plan->btiles[st.tile_first]);
                 st.qtile_first = plan->qtiles.size();
                 const size_t n_elems = (size_t)op.m * op.in_f;
-                for (size_t xi = 0; xi < xs.size(); ++xi)
-                    for (size_t e = 0; e < n_elems; e += 1024)
-                        plan->qtiles.push_back(infr::QuantTile{xs[xi] + e, (uint32_t)((xi * x_elems + e) / 256),
-                                                               (uint32_t)std::min<size_t>(1024, n_elems - e)});
+                for (size_t xi = 0; xi < xs.size(); ++xi) {
+                    if (xs_pre[xi] < 0) {
+                        for (size_t e = 0; e < n_elems; e += 1024)
+                            plan->qtiles.push_back(infr::QuantTile{xs[xi] + e, (uint32_t)((xi * x_elems + e) / 256),
+                                                                   (uint32_t)std::min<size_t>(1024, n_elems - e)});
+                        continue;
+                    }
+                    // the folded op's rows, tiles inside a row (in_f is whole 256s here)
+                    const auto& p = plan->ops[xs_pre[xi]];
+                    const ElementwiseArgs& e = ea[xs_pre[xi]];
+                    for (size_t r = 0; r < op.m; ++r) {
+                        const float *src, *src2;
+                        if (p.kind == INFR_OP_RMS_NORM) {
+                            src = e.x + r * op.in_f;
+                            src2 = e.aux;
+                        } else if (p.kind == INFR_OP_GATED_ACT_FUSED) {
+                            src = e.x + r * 2 * op.in_f;
+                            src2 = src + op.in_f;
+                        } else {
+                            src = e.x + r * (p.gate_stride > 0 ? (size_t)p.gate_stride : op.in_f);
+                            src2 = e.aux + r * (p.up_stride > 0 ? (size_t)p.up_stride : op.in_f) + p.up_off;
+                        }
+                        for (size_t c = 0; c < op.in_f; c += 1024) {
+                            infr::QuantTile t{src + c, (uint32_t)((xi * x_elems + r * op.in_f + c) / 256),
+                                              (uint32_t)std::min<size_t>(1024, op.in_f - c)};
+                            t.pre = p.kind == INFR_OP_RMS_NORM ? 2 : 1;
+                            t.x2 = src2 + c;
+                            t.pre_dst = e.dst + r * op.in_f + c;
+                            t.row = src;
+                            t.dim = (uint32_t)op.in_f;
+                            t.eps = p.eps;
+                            t.act = p.act;
+                            t.has_clamp = p.has_clamp;
+                            t.clamp = p.clamp;
+                            plan->qtiles.push_back(t);
+                        }
+                    }
+                }
                 st.qtile_n = plan->qtiles.size() - st.qtile_first;
                 plan->steps.push_back(st);
                 continue;

@@ -27,6 +27,19 @@ struct QuantTile {
     const float* x;      // first float of the workgroup's chunks
     uint32_t chunk0;     // destination chunk index
     uint32_t n_elems;    // floats to quantize (<= 1024; a per-32 input may end inside a chunk)
+    // An op of two rows and more that a plan folded into the quantizer of the Linears reading it
+    // (tiles then stay inside one row): the workgroup evaluates the op on its floats with the
+    // stand-alone kernel's arithmetic, stores them to `pre_dst` and quantizes them.
+    //   1  gated activation: act(x[e]) * x2[e]
+    //   2  RmsNorm of the row `row` (dim floats): x[e] * scale * x2[e], x2 = the weight from the tile's first column on
+    uint32_t pre = 0;
+    const float* x2 = nullptr;
+    float* pre_dst = nullptr;
+    const float* row = nullptr;
+    uint32_t dim = 0;
+    float eps = 0.0f;
+    int32_t act = 0, has_clamp = 0;
+    float clamp = 0.0f;
 };
 void launch_quantize_q8_group(const QuantTile* tiles_dev, size_t n_tiles, bool per32, const ActQ8& out,
                               hipStream_t stream);

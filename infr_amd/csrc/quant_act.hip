@@ -3,6 +3,7 @@
 //
 // Layout: one wavefront handles 256 consecutive floats (one float4 per lane). HBM traffic is
 // 4 B read + ~1.2 B written per element; the kernel is a pure stream.
+#include "elementwise_fn.hpp"
 #include "kernels.hpp"
 #include "quant_chunk.hpp"
 
@@ -162,12 +163,39 @@ __global__ __launch_bounds__(256) void quantize_q8_group_kernel(const QuantTile*
                                                                 float* __restrict__ d,
                                                                 int32_t* __restrict__ bsums,
                                                                 int32_t* __restrict__ bsums16) {
+    __shared__ float part[4];
     const QuantTile t = tiles[blockIdx.x];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float scale = 0.0f;
+    if (t.pre == 2) {
+        // rms_norm_kernel's reduction over the whole row (stride-256 partial sums, wave sums,
+        // ((p0 + p1) + (p2 + p3))): the same scale, so the same floats and the same codes
+        float s = 0.0f;
+        for (uint32_t i = threadIdx.x; i < t.dim; i += 256) s += t.row[i] * t.row[i];
+        s = wave_sum_f(s);
+        if (lane == 0) part[wave] = s;
+        __syncthreads();
+        const float ss = ((part[0] + part[1]) + (part[2] + part[3])) / (float)t.dim;
+        scale = 1.0f / sqrtf(ss + t.eps);
+    }
     if ((uint32_t)wave * 256 >= t.n_elems) return;  // wave-uniform
     const bool live = (uint32_t)wave * 256 + (uint32_t)lane * 4 < t.n_elems;
     v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (live) v = *reinterpret_cast<const v4f*>(t.x + wave * 256 + lane * 4);
+    if (live) {
+        const int e = wave * 256 + lane * 4;
+        v = *reinterpret_cast<const v4f*>(t.x + e);
+        if (t.pre) {
+            const v4f u = *reinterpret_cast<const v4f*>(t.x2 + e);
+            if (t.pre == 1)
+                v = v4f{gated_act_fn(t.act, t.has_clamp != 0, t.clamp, v.x, u.x),
+                        gated_act_fn(t.act, t.has_clamp != 0, t.clamp, v.y, u.y),
+                        gated_act_fn(t.act, t.has_clamp != 0, t.clamp, v.z, u.z),
+                        gated_act_fn(t.act, t.has_clamp != 0, t.clamp, v.w, u.w)};
+            else
+                v = v4f{v.x * scale * u.x, v.y * scale * u.y, v.z * scale * u.z, v.w * scale * u.w};
+            *reinterpret_cast<v4f*>(t.pre_dst + e) = v;
+        }
+    }
     quantize_chunk<PER32>(v, live, lane, (size_t)t.chunk0 + wave, qs, d, bsums, bsums16);
 }
 
