@@ -595,3 +595,58 @@ def test_single_row_rms_norm_rides_in_the_moe_router_kernel(be):
         assert _rel(y1, want.ravel()) < 1e-4
         assert np.array_equal(bits(h1), bits(h0 + y1))
     assert fused[0].launches() == 3 and plain[0].launches() == 5
+
+
+@pytest.mark.parametrize("m", [2, 8, 16, 24])
+def test_norm_and_gated_activation_ride_in_the_small_batch_quantizer(be, m):
+    """A decode batch through RmsNorm -> {q (Q4_K), v (Q6_K)} and GatedAct -> down: the norm and the
+    activation are evaluated by the quantizer launches of the Linears that read them (stand-alone
+    arithmetic, so the same bits), their outputs are still stored, and the plan is four launches
+    shorter than one per op - two quantizers (one per weight format) compute the norm, which is
+    allowed because they sit on one level."""
+    from infr_amd import GatedAct, RmsNorm
+    H, FF = 1024, 1536
+    wq, wv = synth_weight(DType.Q4K, 1, H, H, 0.05), synth_weight(DType.Q6K, 2, 256, H, 0.05)
+    wd = synth_weight(DType.Q4K, 3, H, FF, 0.05)
+    nw = synth_normal_f32(4, H, mean=1.0, sigma=0.1)
+    g, binds = Graph(), Bindings()
+    x, gt, up = (g.input(TensorDesc((m, d), DType.F32)) for d in (H, FF, FF))
+    nwid = g.input(TensorDesc((H,), DType.F32))
+    h, q, v, act, dn = (g.output(TensorDesc((m, d), DType.F32)) for d in (H, H, 256, FF, H))
+    bufs = {t: be.alloc(m * d * 4) for t, d in ((x, H), (gt, FF), (up, FF), (h, H), (q, H), (v, 256), (act, FF), (dn, H))}
+    for t, b in bufs.items():
+        binds.bind(t, b)
+    binds.bind(nwid, be.upload_new(nw))
+    wqid, wvid, wdid = (g.weight(TensorDesc(s, dt)) for s, dt in (((H, H), DType.Q4K), ((256, H), DType.Q6K),
+                                                                 ((H, FF), DType.Q4K)))
+    binds.bind(wqid, be.upload_new(wq)).bind(wvid, be.upload_new(wv)).bind(wdid, be.upload_new(wd))
+    g.push(RmsNorm(x, nwid, h, m, H, 1e-6))
+    g.push(Linear(h, wqid, q, m, H, H))
+    g.push(Linear(h, wvid, v, m, H, 256))
+    g.push(GatedAct(gt, up, act, m, FF))
+    g.push(Linear(act, wdid, dn, m, FF, H))
+    plan = be.compile(g)
+    for seed in (10, 20):                                   # the second is a replay
+        x0, g0, u0 = synth_normal_f32(seed, m * H), synth_normal_f32(seed + 1, m * FF), synth_normal_f32(seed + 2, m * FF)
+        be.upload(bufs[x], x0)
+        be.upload(bufs[gt], g0)
+        be.upload(bufs[up], u0)
+        be.execute(plan, binds)
+        got_h = be.download(bufs[h], np.empty(m * H, np.float32))
+        got_act = be.download(bufs[act], np.empty(m * FF, np.float32))
+        # the folded ops' own outputs: the stand-alone kernels' values (each op alone in a plan)
+        alone = Graph()
+        ax, aw, ah = alone.input(TensorDesc((m, H), DType.F32)), alone.input(TensorDesc((H,), DType.F32)), alone.output(TensorDesc((m, H), DType.F32))
+        alone.push(RmsNorm(ax, aw, ah, m, H, 1e-6))
+        hb = be.alloc(m * H * 4)
+        be.execute(be.compile(alone), Bindings().bind(ax, bufs[x]).bind(aw, binds.get(nwid)).bind(ah, hb))
+        assert np.array_equal(bits(got_h), bits(be.download(hb, np.empty(m * H, np.float32))))
+        assert _rel(got_h, orc.rms_norm(x0, nw, m, H, 1e-6).ravel()) < 1e-6
+        assert _rel(got_act, orc.gated_act(g0, u0, m, FF).ravel()) < 1e-6
+        # the Linears multiply exactly those stored rows
+        for buf, w, dt, src, k, n in ((q, wq, DType.Q4K, got_h, H, H), (v, wv, DType.Q6K, got_h, H, 256),
+                                      (dn, wd, DType.Q4K, got_act, FF, H)):
+            got = be.download(bufs[buf], np.empty((m, n), np.float32))
+            assert np.array_equal(bits(got), bits(orc.linear(dt, w, src, m, k, n).reshape(m, n)))
+    # quantize + GEMM for each of the three (format, row length) groups; the norm and the activation add none
+    assert plan.launches() == 6
