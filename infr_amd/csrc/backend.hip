@@ -1123,7 +1123,10 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
         // or the producer's dst (the sum is produced at the producer's place in the order)
         for (size_t i = 0; i < k; ++i) {
             const auto& pr = plan->ops[i];
-            const bool lin = decode_linear(i) && pr.out_f == n_add;
+            // (a small-batch Linear's grouped launch stores the sum with each output as well)
+            const bool lin = (decode_linear(i) && pr.out_f == n_add) ||
+                             (pr.kind == INFR_OP_LINEAR && pr.m >= 2 && small_batch(pr) && !self_alias(i) &&
+                              (size_t)pr.m * pr.out_f == n_add);
             const bool moe = pr.kind == INFR_OP_MOE_FFN && (size_t)pr.moe.rows * pr.moe.ne == n_add;
             if ((!lin && !moe) || post[i] >= 0) continue;
             const float* pdst = static_cast<const float*>(bindings[pr.dst]->ptr);
@@ -1299,8 +1302,13 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
                         xs_pre.push_back(qpre[k]);
                     }
                     elem0.push_back((uint32_t)(xi * x_elems));
-                    plan->descs.push_back(infr::GemvOpDesc{la[k].wrows, x, static_cast<float*>(bindings[o2.dst]->ptr),
-                                                           la[k].bpr, (int32_t)o2.out_f});
+                    infr::GemvOpDesc desc{la[k].wrows, x, static_cast<float*>(bindings[o2.dst]->ptr), la[k].bpr,
+                                          (int32_t)o2.out_f};
+                    if (post[k] >= 0) {  // an Op::Add on this output rides in the launch
+                        desc.fus.add_b = resid[k];
+                        desc.fus.add_dst = ea[post[k]].dst;
+                    }
+                    plan->descs.push_back(desc);
                 }
                 st.n = (int)plan->descs.size() - st.first;
                 if (xs.size() * x_elems > be->act_cap_elems)

@@ -179,4 +179,16 @@ __device__ __forceinline__ void k4_all(uint32_t s0, uint32_t s1, uint32_t s2, ui
     mn8[1] = ((s2 >> 4) & 0x0F0F0F0Fu) | ((s1 >> 2) & 0x30303030u);
 }
 
+// Output (token, row) of a small-batch kernel, with the Op::Add a plan folded into the launch: the
+// sum goes to `add_dst` (which may be the residual `add_b` itself, or y: then only the sum is
+// stored); every output index is written by exactly one thread.
+struct BatchAdd {
+    const float* b = nullptr;
+    float* dst = nullptr;
+};
+__device__ __forceinline__ void store_batch_out(float* y, const BatchAdd& a, size_t idx, float v) {
+    if (y != a.dst) gstore<float>(y + idx, v);
+    if (a.dst) gstore<float>(a.dst + idx, v + a.b[idx]);
+}
+
 }  // namespace infr

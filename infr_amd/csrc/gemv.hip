@@ -102,10 +102,16 @@ void fill_batch_tiles(const GemvOpDesc* ops, const uint32_t* act_elem0, int n, c
                       BatchTile* out) {
     size_t k = 0;
     for (int i = 0; i < n; ++i)
-        for (int r0 = 0; r0 < ops[i].out_f; r0 += plan.rows_per_wg)
-            out[k++] = BatchTile{ops[i].w + (size_t)r0 * ops[i].bpr, ops[i].y + r0, act_elem0[i],
-                                 (uint32_t)ops[i].out_f, (uint32_t)std::min(plan.rows_per_wg, ops[i].out_f - r0),
-                                 (uint32_t)ops[i].bpr};
+        for (int r0 = 0; r0 < ops[i].out_f; r0 += plan.rows_per_wg) {
+            BatchTile t{ops[i].w + (size_t)r0 * ops[i].bpr, ops[i].y + r0, act_elem0[i],
+                        (uint32_t)ops[i].out_f, (uint32_t)std::min(plan.rows_per_wg, ops[i].out_f - r0),
+                        (uint32_t)ops[i].bpr};
+            if (ops[i].fus.add_dst) {  // an Op::Add folded into the launch
+                t.add_b = ops[i].fus.add_b + r0;
+                t.add_dst = ops[i].fus.add_dst + r0;
+            }
+            out[k++] = t;
+        }
 }
 
 bool launch_gemv_batch(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,

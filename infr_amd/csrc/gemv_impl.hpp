@@ -19,13 +19,14 @@ namespace infr {
 template <typename F, int STEPS, int MB, bool STAGES>
 __global__ __launch_bounds__(256) void gemv_batch_kernel(const uint8_t* __restrict__ w, size_t bpr,
                                                          ActPtrs act, int m_valid, int in_f,
-                                                         float* __restrict__ y, int out_f,
+                                                         float* y, int out_f,
                                                          int rows_per_wave, StagePtrs st,
                                                          const BatchTile* __restrict__ tiles) {
     const int lane = threadIdx.x & 63;
     int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
     int n_rows = out_f;
     size_t act_elem0 = 0;
+    BatchAdd add;
     if (tiles) {
         const BatchTile t = tiles[blockIdx.x];
         const int pass = blockIdx.y;
@@ -34,6 +35,7 @@ __global__ __launch_bounds__(256) void gemv_batch_kernel(const uint8_t* __restri
         out_f = (int)t.out_f;
         n_rows = (int)t.rows;
         y = t.y + (size_t)pass * MB * out_f;
+        if (t.add_dst) add = BatchAdd{t.add_b + (size_t)pass * MB * out_f, t.add_dst + (size_t)pass * MB * out_f};
         act_elem0 = (size_t)t.act_elem0 + (size_t)pass * MB * in_f;
         m_valid = min(MB, m_valid - pass * MB);
         wave = threadIdx.x >> 6;
@@ -61,7 +63,7 @@ __global__ __launch_bounds__(256) void gemv_batch_kernel(const uint8_t* __restri
     const size_t st_stride = (size_t)out_f * (F::kBlockElems == 64 ? 2 * n_units : n_units);
     gemv_rows_batch<F, STEPS, MB, STAGES>(
         w, bpr, first, acts, ok, y, (size_t)out_f, m_valid, n_units, row0, row_end, lane, st, st_stride,
-        osum + (threadIdx.x >> 6) * (F::kOrdered ? OrderedSum<STEPS>::kFloatsPerWave : 0));
+        osum + (threadIdx.x >> 6) * (F::kOrdered ? OrderedSum<STEPS>::kFloatsPerWave : 0), add);
 }
 
 // Small batch over rows longer than one wave step: K split over the waves of a workgroup. Wave w
@@ -86,13 +88,14 @@ struct BatchKs {
 template <typename F, int MB, bool STAGES>
 __global__ __launch_bounds__(512) void gemv_batch_ks_kernel(const uint8_t* __restrict__ w, size_t bpr,
                                                             ActPtrs act, int m_valid, int in_f,
-                                                            float* __restrict__ y, int out_f,
+                                                            float* y, int out_f,
                                                             int rows_per_wg, StagePtrs st,
                                                             const BatchTile* __restrict__ tiles) {
     extern __shared__ __attribute__((aligned(16))) float ks_lds[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     int row0 = blockIdx.x * rows_per_wg, n_rows = out_f;
     size_t act_elem0 = 0;
+    BatchAdd add;
     if (tiles) {
         const BatchTile t = tiles[blockIdx.x];
         const int pass = blockIdx.y;
@@ -101,6 +104,7 @@ __global__ __launch_bounds__(512) void gemv_batch_ks_kernel(const uint8_t* __res
         out_f = (int)t.out_f;
         n_rows = (int)t.rows;
         y = t.y + (size_t)pass * MB * out_f;
+        if (t.add_dst) add = BatchAdd{t.add_b + (size_t)pass * MB * out_f, t.add_dst + (size_t)pass * MB * out_f};
         act_elem0 = (size_t)t.act_elem0 + (size_t)pass * MB * in_f;
         m_valid = min(MB, m_valid - pass * MB);
         row0 = 0;
@@ -177,7 +181,7 @@ __global__ __launch_bounds__(512) void gemv_batch_ks_kernel(const uint8_t* __res
                 for (int k = 0; k < 4 * nw; ++k) acc += tr[k];
             }
             const int mi = task % MB;
-            if (mi < m_valid) gstore<float>(y + (size_t)mi * out_f + batch0 + task / MB, acc);
+            if (mi < m_valid) store_batch_out(y, add, (size_t)mi * out_f + batch0 + task / MB, acc);
         }
     }
 }

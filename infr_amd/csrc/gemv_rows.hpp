@@ -275,10 +275,10 @@ template <typename F, int STEPS, int MB, bool STAGES>
 __device__ __forceinline__ void gemv_rows_batch(const uint8_t* __restrict__ w, size_t bpr,
                                                 const typename F::Row& first,
                                                 const typename F::Acts (&acts)[MB][STEPS],
-                                                const bool (&ok)[STEPS], float* __restrict__ y,
+                                                const bool (&ok)[STEPS], float* y,
                                                 size_t y_stride, int m_valid, int n_units, int row0,
                                                 int row_end, int lane, const StagePtrs& st,
-                                                size_t st_stride, float* osum) {
+                                                size_t st_stride, float* osum, const BatchAdd& add = BatchAdd{}) {
     constexpr int LS = OrderedSum<STEPS>::kRowStride;
     constexpr int RB = 16 / MB;  // weight rows per ordered-sum flush
     typename F::Row cur = first;
@@ -322,7 +322,7 @@ __device__ __forceinline__ void gemv_rows_batch(const uint8_t* __restrict__ w, s
                         acc += v.w;
                     }
                     const int mi = lane % MB;
-                    if (mi < m_valid) gstore<float>(y + (size_t)mi * y_stride + batch_row0 + lane / MB, acc);
+                    if (mi < m_valid) store_batch_out(y, add, (size_t)mi * y_stride + batch_row0 + lane / MB, acc);
                 }
                 batch_row0 = row + 1;
                 in_batch = 0;
@@ -334,12 +334,12 @@ __device__ __forceinline__ void gemv_rows_batch(const uint8_t* __restrict__ w, s
                 float part = row16_transpose_sum<MB>(s, lane);
                 part += __shfl_xor(part, 16, kWave);
                 part += __shfl_xor(part, 32, kWave);
-                if (lane < MB && lane < m_valid) gstore<float>(y + (size_t)lane * y_stride + row, part);
+                if (lane < MB && lane < m_valid) store_batch_out(y, add, (size_t)lane * y_stride + row, part);
             } else {
 #pragma unroll
                 for (int mi = 0; mi < MB; ++mi) {
                     const float tot = wave_sum_f(s[mi]);
-                    if (lane == 0 && mi < m_valid) gstore<float>(y + (size_t)mi * y_stride + row, tot);
+                    if (lane == 0 && mi < m_valid) store_batch_out(y, add, (size_t)mi * y_stride + row, tot);
                 }
             }
         }

@@ -140,6 +140,10 @@ struct BatchTile {
     uint32_t out_f;      // row stride of y
     uint32_t rows;       // weight rows in this tile
     uint32_t bpr;
+    // an Op::Add on the op's output that the plan folded into this launch (both at the tile's
+    // first row, strided like y): add_dst = y + add_b; null: none
+    const float* add_b = nullptr;
+    float* add_dst = nullptr;
 };
 struct BatchGroupPlan {
     int kind = 0;          // 0: dot4 batch GEMV, 1: K-split MFMA kernel (Q4_K)

@@ -432,7 +432,7 @@ static void launch_mmq_shared_q4k(const uint8_t* w, size_t bpr, const ActQ8& act
 template <int NW, bool STAGES>
 __global__ __launch_bounds__(NW * 64) void mmq_skinny_q4k_kernel(
     const uint8_t* __restrict__ w, size_t bpr, const int8_t* __restrict__ qs,
-    const float* __restrict__ d8, const int32_t* __restrict__ bsums, float* __restrict__ y, int m,
+    const float* __restrict__ d8, const int32_t* __restrict__ bsums, float* y, int m,
     int out_f, int nb, int32_t* __restrict__ st_sd, int32_t* __restrict__ st_sm,
     const BatchTile* __restrict__ tiles) {
     constexpr int RG = 16 / NW;  // accumulators per epilogue thread
@@ -449,11 +449,13 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny_q4k_kernel(
     // activation rows start at act_elem0 of the scratch) or computed from the single op.
     int wrow = blockIdx.x * 32 + col;  // output column relative to y
     bool row_ok = wrow < out_f;
+    BatchAdd add;
     if (tiles) {
         const BatchTile t = tiles[blockIdx.x];
         w = t.w;
         bpr = t.bpr;
         y = t.y;
+        add = BatchAdd{t.add_b, t.add_dst};
         out_f = (int)t.out_f;
         wrow = col;
         row_ok = col < (int)t.rows;
@@ -595,7 +597,7 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny_q4k_kernel(
     if (!row_ok) return;
 #pragma unroll
     for (int i = 0; i < RG; ++i)
-        if (etok[i] < m) gstore<float>(y + (size_t)etok[i] * out_f + wrow, acc[i]);
+        if (etok[i] < m) store_batch_out(y, add, (size_t)etok[i] * out_f + wrow, acc[i]);
 }
 
 template <int NW>
@@ -1043,7 +1045,7 @@ struct Skinny16Nib32 {
 template <typename F, int NW, int BPW, int MT, bool STAGES>
 __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
     const uint8_t* __restrict__ w, size_t bpr, const int8_t* __restrict__ qs,
-    const float* __restrict__ d8, const int32_t* __restrict__ bsums, float* __restrict__ y, int m,
+    const float* __restrict__ d8, const int32_t* __restrict__ bsums, float* y, int m,
     int out_f, int nb, int32_t* __restrict__ st_sd, int32_t* __restrict__ st_sm,
     const BatchTile* __restrict__ tiles) {
     constexpr int kBlk = F::kBlockBytes;
@@ -1070,11 +1072,13 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
     int wrow = blockIdx.x * 32 + rt;
     bool row_ok = wrow < out_f;
     bool any_row = (int)blockIdx.x * 32 + (int)blockIdx.y * 16 < out_f;
+    BatchAdd add;
     if (tiles) {
         const BatchTile t = tiles[blockIdx.x];
         w = t.w;
         bpr = t.bpr;
         y = t.y;
+        add = BatchAdd{t.add_b, t.add_dst};
         out_f = (int)t.out_f;
         wrow = rt;
         row_ok = rt < (int)t.rows;
@@ -1264,7 +1268,7 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int tok = tok0 + 4 * kq + i;
-        if (tok < m) gstore<float>(y + (size_t)tok * out_f + wrow, acc[i]);
+        if (tok < m) store_batch_out(y, add, (size_t)tok * out_f + wrow, acc[i]);
     }
 }
 

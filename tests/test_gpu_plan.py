@@ -650,3 +650,34 @@ def test_norm_and_gated_activation_ride_in_the_small_batch_quantizer(be, m):
             assert np.array_equal(bits(got), bits(orc.linear(dt, w, src, m, k, n).reshape(m, n)))
     # quantize + GEMM for each of the three (format, row length) groups; the norm and the activation add none
     assert plan.launches() == 6
+
+
+@pytest.mark.parametrize("m,in_f", [(4, 1024), (4, 8192), (12, 1024), (24, 1024), (40, 8192)])
+@pytest.mark.parametrize("dtype", [DType.Q4K, DType.Q8_0])
+def test_residual_add_rides_in_the_small_batch_launch(be, dtype, m, in_f):
+    """Linear (two rows and more) -> Add(residual), in place on the residual stream: every
+    small-batch kernel (the dot4 batches in their one-wave and K-split forms, the 16- and
+    32-token MFMA kernels) stores `y + residual` beside y, so the Add has no launch of its own;
+    the sum is the CPU's `a + b` on the stored y, bit for bit."""
+    from infr_amd import Add
+    out_f = 96
+    w = synth_weight(dtype, 5, out_f, in_f, 0.05)
+    g, binds = Graph(), Bindings()
+    x, h = g.input(TensorDesc((m, in_f), DType.F32)), g.input(TensorDesc((m, out_f), DType.F32))
+    y = g.output(TensorDesc((m, out_f), DType.F32))
+    xb, hb, yb = be.alloc(m * in_f * 4), be.alloc(m * out_f * 4), be.alloc(m * out_f * 4)
+    wid = g.weight(TensorDesc((out_f, in_f), dtype))
+    binds.bind(x, xb).bind(h, hb).bind(y, yb).bind(wid, be.upload_new(w))
+    g.push(Linear(x, wid, y, m, in_f, out_f))
+    g.push(Add(y, h, h, m * out_f))
+    plan = be.compile(g)
+    for seed in (10, 20):
+        x0, h0 = synth_normal_f32(seed, m * in_f), synth_normal_f32(seed + 1, m * out_f)
+        be.upload(xb, x0)
+        be.upload(hb, h0)
+        be.execute(plan, binds)
+        got_y = be.download(yb, np.empty(m * out_f, np.float32))
+        got_h = be.download(hb, np.empty(m * out_f, np.float32))
+        assert _rel(got_y, orc.linear(dtype, w, x0, m, in_f, out_f).ravel()) < 1e-5
+        assert np.array_equal(bits(got_h), bits(h0 + got_y))
+    assert plan.launches() == 2                             # the quantizer and the GEMM
