@@ -166,6 +166,14 @@ __global__ __launch_bounds__(256) void quantize_q8_group_kernel(const QuantTile*
     __shared__ float part[4];
     const QuantTile t = tiles[blockIdx.x];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int e = wave * 256 + lane * 4;
+    const bool live = (uint32_t)e < t.n_elems;
+    // the tile's own floats are requested before the row reduction of a folded norm, not behind it
+    v4f v = {0.0f, 0.0f, 0.0f, 0.0f}, u = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (live) {
+        v = *reinterpret_cast<const v4f*>(t.x + e);
+        if (t.pre) u = *reinterpret_cast<const v4f*>(t.x2 + e);
+    }
     float scale = 0.0f;
     if (t.pre == 2) {
         // rms_norm_kernel's reduction over the whole row (stride-256 partial sums, wave sums,
@@ -179,22 +187,15 @@ __global__ __launch_bounds__(256) void quantize_q8_group_kernel(const QuantTile*
         scale = 1.0f / sqrtf(ss + t.eps);
     }
     if ((uint32_t)wave * 256 >= t.n_elems) return;  // wave-uniform
-    const bool live = (uint32_t)wave * 256 + (uint32_t)lane * 4 < t.n_elems;
-    v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (live) {
-        const int e = wave * 256 + lane * 4;
-        v = *reinterpret_cast<const v4f*>(t.x + e);
-        if (t.pre) {
-            const v4f u = *reinterpret_cast<const v4f*>(t.x2 + e);
-            if (t.pre == 1)
-                v = v4f{gated_act_fn(t.act, t.has_clamp != 0, t.clamp, v.x, u.x),
-                        gated_act_fn(t.act, t.has_clamp != 0, t.clamp, v.y, u.y),
-                        gated_act_fn(t.act, t.has_clamp != 0, t.clamp, v.z, u.z),
-                        gated_act_fn(t.act, t.has_clamp != 0, t.clamp, v.w, u.w)};
-            else
-                v = v4f{v.x * scale * u.x, v.y * scale * u.y, v.z * scale * u.z, v.w * scale * u.w};
-            *reinterpret_cast<v4f*>(t.pre_dst + e) = v;
-        }
+    if (live && t.pre) {
+        if (t.pre == 1)
+            v = v4f{gated_act_fn(t.act, t.has_clamp != 0, t.clamp, v.x, u.x),
+                    gated_act_fn(t.act, t.has_clamp != 0, t.clamp, v.y, u.y),
+                    gated_act_fn(t.act, t.has_clamp != 0, t.clamp, v.z, u.z),
+                    gated_act_fn(t.act, t.has_clamp != 0, t.clamp, v.w, u.w)};
+        else
+            v = v4f{v.x * scale * u.x, v.y * scale * u.y, v.z * scale * u.z, v.w * scale * u.w};
+        *reinterpret_cast<v4f*>(t.pre_dst + e) = v;
     }
     quantize_chunk<PER32>(v, live, lane, (size_t)t.chunk0 + wave, qs, d, bsums, bsums16);
 }
