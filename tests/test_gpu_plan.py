@@ -681,3 +681,36 @@ def test_residual_add_rides_in_the_small_batch_launch(be, dtype, m, in_f):
         assert _rel(got_y, orc.linear(dtype, w, x0, m, in_f, out_f).ravel()) < 1e-5
         assert np.array_equal(bits(got_h), bits(h0 + got_y))
     assert plan.launches() == 2                             # the quantizer and the GEMM
+
+
+@pytest.mark.parametrize("m", [3, 16])
+def test_combined_gate_up_activation_rides_in_the_small_batch_quantizer(be, m):
+    """Op::GatedActFused on a [rows, 2 * nff] buffer (gate half first) in front of a small-batch
+    Linear, with a clamp and the GELU form: folded into that Linear's quantizer launch, same bits
+    as the op alone."""
+    from infr_amd import GatedActFused
+    FF, H = 1024, 512
+    wd = synth_weight(DType.Q5K, 3, H, FF, 0.05)
+    g, binds = Graph(), Bindings()
+    gu = g.input(TensorDesc((m, 2 * FF), DType.F32))
+    act, dn = g.output(TensorDesc((m, FF), DType.F32)), g.output(TensorDesc((m, H), DType.F32))
+    gub, actb, dnb = be.alloc(m * 2 * FF * 4), be.alloc(m * FF * 4), be.alloc(m * H * 4)
+    wid = g.weight(TensorDesc((H, FF), DType.Q5K))
+    binds.bind(gu, gub).bind(act, actb).bind(dn, dnb).bind(wid, be.upload_new(wd))
+    g.push(GatedActFused(gu, act, m, FF, act=1, swiglu_clamp=1.5))
+    g.push(Linear(act, wid, dn, m, FF, H))
+    plan = be.compile(g)
+    alone = Graph()
+    agu, aact = alone.input(TensorDesc((m, 2 * FF), DType.F32)), alone.output(TensorDesc((m, FF), DType.F32))
+    alone.push(GatedActFused(agu, aact, m, FF, act=1, swiglu_clamp=1.5))
+    alone_plan, alone_out = be.compile(alone), be.alloc(m * FF * 4)
+    for seed in (10, 20):
+        gu0 = synth_normal_f32(seed, m * 2 * FF) * np.float32(1.5)
+        be.upload(gub, gu0)
+        be.execute(plan, binds)
+        be.execute(alone_plan, Bindings().bind(agu, gub).bind(aact, alone_out))
+        got_act = be.download(actb, np.empty(m * FF, np.float32))
+        assert np.array_equal(bits(got_act), bits(be.download(alone_out, np.empty(m * FF, np.float32))))
+        got = be.download(dnb, np.empty((m, H), np.float32))
+        assert np.array_equal(bits(got), bits(orc.linear(DType.Q5K, wd, got_act, m, FF, H).reshape(m, H)))
+    assert plan.launches() == 2
