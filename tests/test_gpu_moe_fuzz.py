@@ -1,7 +1,8 @@
 """Op::MoeFfn on random shapes and bank formats against the CPU oracle: row counts on both sides of
 every route's threshold (one row; a few rows: per-pair kernels and the fused down launch; from an
 average of two or four pairs per expert the bucketed int8-MFMA tiles), every bank format in every
-position, hidden sizes and expert widths of one to several 256-blocks, up to 32 experts per token.
+position, hidden sizes and expert widths of one to several 256-blocks (one case in four beyond
+4096 columns, where the one-token kernels walk a row in rounds), up to 32 experts per token.
 
 Bars: the expert selection equals the oracle's, its weights agree to 1e-5 relative, outputs within
 rel-L2 <= 1e-4 and max-abs <= 1e-3 * max|y| (crates/infr-cpu/src/lib.rs:2334-2541, moe.rs:42-53).
@@ -45,6 +46,11 @@ def draw_case(rng):
     while True:
         ne = int(rng.choice([256, 512, 768, 1024, 1024, 2048, 4096]))
         nff = 256 * int(rng.integers(1, 4))
+        long_rows = int(rng.integers(8))        # one case in four: rows beyond 4096 columns on one side
+        if long_rows == 0:
+            ne = int(rng.choice([4352, 5120, 6144, 7168, 8192]))
+        elif long_rows == 1:
+            ne, nff = int(rng.choice([256, 512])), int(rng.choice([4352, 5120, 8192, 14336]))
         n_expert = int(rng.choice([2, 4, 8, 16, 32, 48, 72, 128]))
         if n_expert * nff * ne <= 1 << 24:      # banks of at most 16 M weights each
             break
