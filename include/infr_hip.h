@@ -177,27 +177,70 @@ int infr_hip_linear_int_stages(infr_hip_t *be, int dtype, const infr_hip_buffer_
                                size_t in_f, size_t out_f, infr_hip_buffer_t *a,
                                infr_hip_buffer_t *b);
 
-/* Op::MoeFfn as qwen3moe emits it (graph.rs:911-1011; crates/infr-llama/src/seam/runner.rs:3971-3997):
- * softmax gating, renormalised top-n_used weights x scale, split gate/up banks, SiLU, weights on
- * the expert output. Expert e of a bank is its e-th equal byte slice. */
+/* Activation (crates/infr-core/src/graph.rs:47-54; act_fn in crates/infr-cpu/src/kernels.rs:6578-6585) */
+typedef enum { INFR_ACT_SILU = 0, INFR_ACT_GELU = 1, INFR_ACT_SIGMOID = 2 } infr_activation;
+/* MoeGating (crates/infr-core/src/graph.rs:76-85) */
+typedef enum { INFR_GATING_SOFTMAX = 0, INFR_GATING_SIGMOID = 1, INFR_GATING_SQRT_SOFTPLUS = 2 } infr_moe_gating;
+
+/* Op::MoeFfn, every field of the op (graph.rs:918-1011). qwen3moe emits softmax gating, norm_w,
+ * weight on the expert output, split gate/up banks, SiLU and none of the optional operands
+ * (crates/infr-llama/src/seam/runner.rs:3971-3997): act = gating = 0, norm_w = 1, the rest zero.
+ * Expert e of a bank is its e-th equal byte slice. */
 typedef struct {
     uint32_t ne, n_expert, n_used, n_ff_exp, rows;
     float scale;
     int router_dtype; /* INFR_DTYPE_F32, _F16 or _BF16 */
     int gate_dtype, up_dtype, down_dtype; /* any INFR_DTYPE_* (quantized, or plain F32 / F16 / BF16 rows), each bank its own */
+    int act;            /* infr_activation: act(gate) * up per expert (graph.rs:948) */
+    int gating;         /* infr_moe_gating (graph.rs:956-958) */
+    int norm_w;         /* 1: w = p / max(sum of the selected p, 1e-20) * scale; 0: w = p * scale (graph.rs:959-962) */
+    int weight_before;  /* 1: the routing weight multiplies gate and up before the activation, not the
+                           expert output (llama4; graph.rs:963-967, CPU arm lib.rs:2833-2861, 2976) */
+    int fused_gate_up;  /* 1: gate_exps holds [gate rows | up rows] per expert, up_exps and up_dtype are
+                           not read (graph.rs:936-941) */
+    int has_clamp;      /* swiglu_clamp = Some(clamp): act(min(gate, clamp)) * clamp(up, -clamp, clamp)
+                           (graph.rs:949-955). As on the CPU (lib.rs:2293-2299) it is refused with
+                           INFR_ACT_SIGMOID or weight_before. */
+    float clamp;
+    uint32_t n_expert_groups, n_expert_groups_used; /* group-limited routing when groups > 1 and used > 0:
+                           a group's score is the sum of its two best selection values, the best `used`
+                           groups stay, the rest are masked out (graph.rs:983-987, lib.rs:2488-2526);
+                           n_expert a multiple of the groups, at most 64 groups */
+    /* which optional operands the op carries (infr_hip_moe_optional_t / the op's tensor ids) */
+    int has_down_scale;  /* down_scale: Some (graph.rs:932-935) */
+    int has_exp_probs_b; /* exp_probs_b: Some (graph.rs:979-982) */
+    int has_expert_ids;  /* expert_ids: Some (graph.rs:988-1010); refused together with exp_probs_b or
+                            groups > 1, as on the CPU (lib.rs:2303-2309) */
+    int has_ep_band;     /* ep_band: Some - an expert-parallel shard of the banks (graph.rs:968-978). This
+                            backend runs one GPU and returns INFR_HIP_ERR_UNSUPPORTED for it. */
 } infr_hip_moe_params_t;
+
+/* The optional operands of Op::MoeFfn; each must be set exactly when its has_* flag is. */
+typedef struct {
+    const infr_hip_buffer_t *down_scale;  /* f32 [n_expert]: the selected expert's down output times
+                                             down_scale[e] before the weighted sum (lib.rs:2932-2938) */
+    const infr_hip_buffer_t *exp_probs_b; /* f32 [n_expert]: added to the probabilities for the SELECTION
+                                             only; the weights use the unbiased ones (lib.rs:2476-2485) */
+    const infr_hip_buffer_t *expert_ids;  /* i32 [rows, n_used]: the selection, in this order; the weights
+                                             are the router's probabilities at these ids (lib.rs:2456-2472).
+                                             An id outside [0, n_expert) is a panic on the CPU; here it is
+                                             clamped into range and nothing is read out of bounds. */
+} infr_hip_moe_optional_t;
 
 /* CPU arm: crates/infr-cpu/src/lib.rs:2264-2984, crates/infr-cpu/src/moe.rs. As there, rows == 1
  * multiplies decoded f32 weights with the unquantized activation; rows >= 2 takes, per bank
  * (expert_acts_kind, moe.rs:42-53), per-256 int8 activations (Q4_K, Q5_K, Q6_K, Q8_0), per-32 int8
  * activations (Q5_0), or the same f32 arm (every other format). ne and n_ff_exp are multiples of 256.
- * Only the selected experts' blocks are read. sel_idx (i32) / sel_w (f32), [rows, n_used], are
- * optional outputs of the routing in descending-probability order. */
+ * Only the selected experts' blocks are read. `opt` may be NULL when the op has no optional operand;
+ * up_exps may be NULL with fused_gate_up. sel_idx (i32) / sel_w (f32), [rows, n_used], are
+ * optional outputs of the routing in descending-probability order (the supplied order with expert_ids).
+ * Every combination of the fields above that the kernels do not implement returns
+ * INFR_HIP_ERR_UNSUPPORTED; none is silently read as another. */
 int infr_hip_moe_ffn(infr_hip_t *be, const infr_hip_moe_params_t *p, const infr_hip_buffer_t *x,
                      const infr_hip_buffer_t *router_x, const infr_hip_buffer_t *router,
                      const infr_hip_buffer_t *gate_exps, const infr_hip_buffer_t *up_exps,
-                     const infr_hip_buffer_t *down_exps, infr_hip_buffer_t *dst,
-                     infr_hip_buffer_t *sel_idx, infr_hip_buffer_t *sel_w);
+                     const infr_hip_buffer_t *down_exps, const infr_hip_moe_optional_t *opt,
+                     infr_hip_buffer_t *dst, infr_hip_buffer_t *sel_idx, infr_hip_buffer_t *sel_w);
 
 /* Op::EmbedGather (crates/infr-core/src/graph.rs:853-865; CPU arm crates/infr-cpu/src/lib.rs:2084-2111):
  * dst[r, :] = decode(table[ids[r], :]) * scale for `rows` rows of `ne` elements. `table` holds
@@ -222,9 +265,6 @@ typedef enum {
     INFR_OP_EMBED_GATHER = 8     /* Op::EmbedGather, graph.rs:853-865; lib.rs:2084-2111 */
 } infr_hip_op_kind;
 
-/* Activation (crates/infr-core/src/graph.rs, act_fn in crates/infr-cpu/src/kernels.rs:6578-6585) */
-typedef enum { INFR_ACT_SILU = 0, INFR_ACT_GELU = 1, INFR_ACT_SIGMOID = 2 } infr_activation;
-
 typedef struct {
     int kind;      /* infr_hip_op_kind */
     /* Op::Linear: tensor ids (indices into the bindings array) and shape */
@@ -233,8 +273,9 @@ typedef struct {
     uint64_t w_off;
     uint64_t w_numel;
     int w_dtype;
-    /* Op::MoeFfn */
+    /* Op::MoeFfn; down_scale / exp_probs_b / expert_ids are read when moe.has_* says so */
     uint32_t router_x, router, gate_exps, up_exps, down_exps;
+    uint32_t down_scale, exp_probs_b, expert_ids;
     infr_hip_moe_params_t moe;
     /* Elementwise ops, all f32. They reuse the fields above:
      *   RmsNorm / RmsNormAdd   x, weight (f32 [dim]), dst, m = rows, in_f = dim, eps

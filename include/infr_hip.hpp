@@ -119,15 +119,27 @@ struct TensorDesc {
 
 // crates/infr-core/src/graph.rs Activation; act_fn, crates/infr-cpu/src/kernels.rs:6578-6585
 enum class Activation : int { Silu = INFR_ACT_SILU, Gelu = INFR_ACT_GELU, Sigmoid = INFR_ACT_SIGMOID };
+// crates/infr-core/src/graph.rs:76-85
+enum class MoeGating : int { Softmax = INFR_GATING_SOFTMAX, Sigmoid = INFR_GATING_SIGMOID, SqrtSoftplus = INFR_GATING_SQRT_SOFTPLUS };
 
 namespace op {
 // graph.rs:177-191
 struct Linear { TensorId x, weight, dst; uint32_t m, in_f, out_f; uint64_t w_off = 0; };
-// graph.rs:911-1011, as qwen3moe emits it (softmax gating, renormalised weights, split banks, SiLU)
+// graph.rs:911-1011, every field under the reference's name; the defaults after `scale` are what
+// qwen3moe emits (softmax gating, renormalised weights on the output, split banks, SiLU)
 struct MoeFfn {
     TensorId x, router_x, router, gate_exps, up_exps, down_exps, dst;
     uint32_t ne, n_expert, n_used, n_ff_exp;
     float scale = 1.0f;
+    Activation act = Activation::Silu;
+    MoeGating gating = MoeGating::Softmax;
+    bool norm_w = true;
+    bool weight_before = false;
+    bool fused_gate_up = false;
+    std::optional<float> swiglu_clamp;
+    std::optional<TensorId> down_scale, exp_probs_b, expert_ids;
+    uint32_t n_expert_groups = 0, n_expert_groups_used = 0;
+    std::optional<std::pair<uint32_t, uint32_t>> ep_band;
 };
 // graph.rs:139-148 / 149-158
 struct RmsNorm { TensorId x, weight, dst; uint32_t rows, dim; float eps; };
@@ -324,6 +336,14 @@ private:
         c.moe.gate_dtype = (int)g.desc(v.gate_exps).dtype;
         c.moe.up_dtype = (int)g.desc(v.up_exps).dtype;
         c.moe.down_dtype = (int)g.desc(v.down_exps).dtype;
+        c.moe.act = (int)v.act; c.moe.gating = (int)v.gating;
+        c.moe.norm_w = v.norm_w; c.moe.weight_before = v.weight_before; c.moe.fused_gate_up = v.fused_gate_up;
+        c.moe.has_clamp = v.swiglu_clamp.has_value(); c.moe.clamp = v.swiglu_clamp.value_or(0.0f);
+        c.moe.n_expert_groups = v.n_expert_groups; c.moe.n_expert_groups_used = v.n_expert_groups_used;
+        c.moe.has_down_scale = v.down_scale.has_value(); c.down_scale = v.down_scale ? v.down_scale->v : 0;
+        c.moe.has_exp_probs_b = v.exp_probs_b.has_value(); c.exp_probs_b = v.exp_probs_b ? v.exp_probs_b->v : 0;
+        c.moe.has_expert_ids = v.expert_ids.has_value(); c.expert_ids = v.expert_ids ? v.expert_ids->v : 0;
+        c.moe.has_ep_band = v.ep_band.has_value();
     }
     static void fill(const Graph&, const op::RmsNorm& v, infr_hip_op_t& c) {
         c.kind = INFR_OP_RMS_NORM;

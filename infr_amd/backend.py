@@ -72,7 +72,26 @@ class _MoeParams(C.Structure):
     _fields_ = [("ne", C.c_uint32), ("n_expert", C.c_uint32), ("n_used", C.c_uint32),
                 ("n_ff_exp", C.c_uint32), ("rows", C.c_uint32), ("scale", C.c_float),
                 ("router_dtype", C.c_int), ("gate_dtype", C.c_int), ("up_dtype", C.c_int),
-                ("down_dtype", C.c_int)]
+                ("down_dtype", C.c_int),
+                ("act", C.c_int), ("gating", C.c_int), ("norm_w", C.c_int), ("weight_before", C.c_int),
+                ("fused_gate_up", C.c_int), ("has_clamp", C.c_int), ("clamp", C.c_float),
+                ("n_expert_groups", C.c_uint32), ("n_expert_groups_used", C.c_uint32),
+                ("has_down_scale", C.c_int), ("has_exp_probs_b", C.c_int), ("has_expert_ids", C.c_int),
+                ("has_ep_band", C.c_int)]
+
+
+class _MoeOptional(C.Structure):
+    _fields_ = [("down_scale", C.c_void_p), ("exp_probs_b", C.c_void_p), ("expert_ids", C.c_void_p)]
+
+
+def _moe_params(ne, n_expert, n_used, n_ff_exp, rows, scale, router_dtype, gate_dtype, up_dtype, down_dtype, act,
+                gating, norm_w, weight_before, fused_gate_up, swiglu_clamp, n_expert_groups, n_expert_groups_used,
+                has_down_scale, has_exp_probs_b, has_expert_ids, has_ep_band) -> "_MoeParams":
+    return _MoeParams(ne, n_expert, n_used, n_ff_exp, rows, scale, router_dtype, gate_dtype, up_dtype, down_dtype,
+                      int(act), int(gating), int(bool(norm_w)), int(bool(weight_before)), int(bool(fused_gate_up)),
+                      int(swiglu_clamp is not None), float(swiglu_clamp or 0.0), n_expert_groups,
+                      n_expert_groups_used, int(has_down_scale), int(has_exp_probs_b), int(has_expert_ids),
+                      int(has_ep_band))
 
 
 class _Op(C.Structure):
@@ -80,7 +99,9 @@ class _Op(C.Structure):
                 ("m", C.c_uint32), ("in_f", C.c_uint32), ("out_f", C.c_uint32),
                 ("w_off", C.c_uint64), ("w_numel", C.c_uint64), ("w_dtype", C.c_int),
                 ("router_x", C.c_uint32), ("router", C.c_uint32), ("gate_exps", C.c_uint32),
-                ("up_exps", C.c_uint32), ("down_exps", C.c_uint32), ("moe", _MoeParams),
+                ("up_exps", C.c_uint32), ("down_exps", C.c_uint32),
+                ("down_scale", C.c_uint32), ("exp_probs_b", C.c_uint32), ("expert_ids", C.c_uint32),
+                ("moe", _MoeParams),
                 ("aux", C.c_uint32), ("eps", C.c_float), ("act", C.c_int), ("up_off", C.c_uint32),
                 ("up_stride", C.c_uint32), ("gate_stride", C.c_uint32), ("gate_block_width", C.c_uint32),
                 ("has_clamp", C.c_int), ("clamp", C.c_float), ("scale", C.c_float)]
@@ -124,8 +145,8 @@ SYMBOLS = {
     "infr_hip_quantize_q8_32": (C.c_int, [_vp, _vp, C.c_size_t, C.c_size_t, _vp, _vp, _vp]),
     "infr_hip_linear_int_stages": (C.c_int, [_vp, C.c_int, _vp, C.c_size_t, C.c_size_t, _vp,
                                              C.c_size_t, C.c_size_t, C.c_size_t, _vp, _vp]),
-    "infr_hip_moe_ffn": (C.c_int, [_vp, C.POINTER(_MoeParams), _vp, _vp, _vp, _vp, _vp, _vp, _vp,
-                                   _vp, _vp]),
+    "infr_hip_moe_ffn": (C.c_int, [_vp, C.POINTER(_MoeParams), _vp, _vp, _vp, _vp, _vp, _vp,
+                                   C.POINTER(_MoeOptional), _vp, _vp, _vp]),
     "infr_hip_embed_gather": (C.c_int, [_vp, C.c_int, _vp, C.c_size_t, _vp, C.c_size_t, C.c_size_t, C.c_float, _vp]),
     "infr_hip_compile": (C.c_int, [_vp, C.POINTER(_Op), C.c_size_t, C.POINTER(_vp)]),
     "infr_hip_plan_free": (None, [_vp, _vp]),
@@ -260,9 +281,24 @@ class Linear:
     w_off: int = 0
 
 
+class Activation(IntEnum):
+    """crates/infr-core/src/graph.rs Activation; act_fn, crates/infr-cpu/src/kernels.rs:6578-6585."""
+    Silu = 0
+    Gelu = 1
+    Sigmoid = 2
+
+
+class MoeGating(IntEnum):
+    """crates/infr-core/src/graph.rs:76-85."""
+    Softmax = 0
+    Sigmoid = 1
+    SqrtSoftplus = 2
+
+
 @dataclass
 class MoeFfn:
-    """Op::MoeFfn as qwen3moe emits it (graph.rs:911-1011)."""
+    """Op::MoeFfn (graph.rs:911-1011), every field under the reference's name; the defaults are what
+    qwen3moe emits (crates/infr-llama/src/seam/runner.rs:3971-3997)."""
     x: TensorId
     router_x: TensorId
     router: TensorId
@@ -275,13 +311,18 @@ class MoeFfn:
     n_used: int
     n_ff_exp: int
     scale: float = 1.0
-
-
-class Activation(IntEnum):
-    """crates/infr-core/src/graph.rs Activation; act_fn, crates/infr-cpu/src/kernels.rs:6578-6585."""
-    Silu = 0
-    Gelu = 1
-    Sigmoid = 2
+    act: Activation = Activation.Silu
+    gating: MoeGating = MoeGating.Softmax
+    norm_w: bool = True
+    weight_before: bool = False
+    fused_gate_up: bool = False
+    swiglu_clamp: float | None = None
+    down_scale: TensorId | None = None
+    exp_probs_b: TensorId | None = None
+    n_expert_groups: int = 0
+    n_expert_groups_used: int = 0
+    expert_ids: TensorId | None = None
+    ep_band: tuple | None = None
 
 
 @dataclass
@@ -524,9 +565,15 @@ class HipBackend:
                 o.router_x, o.router = op.router_x.id, op.router.id
                 o.gate_exps, o.up_exps, o.down_exps = op.gate_exps.id, op.up_exps.id, op.down_exps.id
                 rows = g.desc(op.x).numel() // op.ne
-                o.moe = _MoeParams(op.ne, op.n_expert, op.n_used, op.n_ff_exp, rows, op.scale,
-                                   int(g.desc(op.router).dtype), int(g.desc(op.gate_exps).dtype),
-                                   int(g.desc(op.up_exps).dtype), int(g.desc(op.down_exps).dtype))
+                o.moe = _moe_params(op.ne, op.n_expert, op.n_used, op.n_ff_exp, rows, op.scale,
+                                    int(g.desc(op.router).dtype), int(g.desc(op.gate_exps).dtype),
+                                    int(g.desc(op.up_exps).dtype), int(g.desc(op.down_exps).dtype), op.act,
+                                    op.gating, op.norm_w, op.weight_before, op.fused_gate_up, op.swiglu_clamp,
+                                    op.n_expert_groups, op.n_expert_groups_used, op.down_scale is not None,
+                                    op.exp_probs_b is not None, op.expert_ids is not None, op.ep_band is not None)
+                o.down_scale = op.down_scale.id if op.down_scale is not None else 0
+                o.exp_probs_b = op.exp_probs_b.id if op.exp_probs_b is not None else 0
+                o.expert_ids = op.expert_ids.id if op.expert_ids is not None else 0
             elif isinstance(op, (RmsNorm, RmsNormAdd)):
                 o.kind = 3 if isinstance(op, RmsNorm) else 4
                 o.x, o.weight, o.dst = op.x.id, op.weight.id, op.dst.id
@@ -626,13 +673,24 @@ class HipBackend:
                 dst: Buffer, *, rows: int, ne: int, n_expert: int, n_used: int, n_ff_exp: int,
                 scale: float = 1.0, router_dtype: int = DType.F32, gate_dtype: int = DType.Q4K,
                 up_dtype: int = DType.Q4K, down_dtype: int = DType.Q4K, router_x: Buffer | None = None,
-                sel_idx: Buffer | None = None, sel_w: Buffer | None = None) -> None:
-        p = _MoeParams(ne, n_expert, n_used, n_ff_exp, rows, scale, int(router_dtype),
-                       int(gate_dtype), int(up_dtype), int(down_dtype))
+                sel_idx: Buffer | None = None, sel_w: Buffer | None = None,
+                act: int = Activation.Silu, gating: int = MoeGating.Softmax, norm_w: bool = True,
+                weight_before: bool = False, fused_gate_up: bool = False, swiglu_clamp: float | None = None,
+                n_expert_groups: int = 0, n_expert_groups_used: int = 0, down_scale: Buffer | None = None,
+                exp_probs_b: Buffer | None = None, expert_ids: Buffer | None = None,
+                ep_band: tuple | None = None) -> None:
+        """Op::MoeFfn; the keyword defaults are qwen3moe's setting. With ``fused_gate_up`` the ``gate``
+        bank holds gate rows then up rows per expert and ``up`` may be None."""
+        p = _moe_params(ne, n_expert, n_used, n_ff_exp, rows, scale, int(router_dtype), int(gate_dtype),
+                        int(up_dtype), int(down_dtype), act, gating, norm_w, weight_before, fused_gate_up,
+                        swiglu_clamp, n_expert_groups, n_expert_groups_used, down_scale is not None,
+                        exp_probs_b is not None, expert_ids is not None, ep_band is not None)
+        opt = _MoeOptional(down_scale._h if down_scale else None, exp_probs_b._h if exp_probs_b else None,
+                           expert_ids._h if expert_ids else None)
         rx = router_x if router_x is not None else x
         self._check(self._lib.infr_hip_moe_ffn(
-            self._h, C.byref(p), x._h, rx._h, router._h, gate._h, up._h, down._h, dst._h,
-            sel_idx._h if sel_idx else None, sel_w._h if sel_w else None))
+            self._h, C.byref(p), x._h, rx._h, router._h, gate._h, up._h if up is not None else None, down._h,
+            C.byref(opt), dst._h, sel_idx._h if sel_idx else None, sel_w._h if sel_w else None))
 
     # -- measurement --
     def stream_read_gbs(self, buf: Buffer, nbytes: int | None = None, reps: int = 10) -> float:

@@ -798,47 +798,96 @@ static size_t expert_bank_bytes(int dtype, size_t rows, size_t in_f) {
     return rows * (in_f / (size_t)qpb) * (size_t)bpb;
 }
 
-// Validates an Op::MoeFfn and fills the launch structures.
+// Validates an Op::MoeFfn and fills the launch structures. Every field of the op is either carried
+// into the launch or refused here: none is read as another setting.
 static int check_moe(infr_hip_t* be, const infr_hip_moe_params_t* p, const infr_hip_buffer_t* x,
                      const infr_hip_buffer_t* router_x, const infr_hip_buffer_t* router,
                      const infr_hip_buffer_t* gate, const infr_hip_buffer_t* up,
-                     const infr_hip_buffer_t* down, infr_hip_buffer_t* dst,
+                     const infr_hip_buffer_t* down, const infr_hip_moe_optional_t* opt, infr_hip_buffer_t* dst,
                      infr_hip_buffer_t* sel_idx, infr_hip_buffer_t* sel_w, infr::MoeShape* s,
                      infr::MoeBuffers* b) {
-    if (!p || !x || !router_x || !router || !gate || !up || !down || !dst)
+    if (!p) return fail(be, INFR_HIP_ERR_INVALID, "moe_ffn: null parameters");
+    const bool fused = p->fused_gate_up != 0;
+    if (!x || !router_x || !router || !gate || (!up && !fused) || !down || !dst)
         return fail(be, INFR_HIP_ERR_INVALID, "moe_ffn: unbound buffer");
     if (!p->ne || !p->n_expert || !p->n_used || !p->n_ff_exp || !p->rows || p->n_used > p->n_expert)
         return fail(be, INFR_HIP_ERR_INVALID, "moe_ffn: empty or inconsistent shape");
-    const size_t gb = expert_bank_bytes(p->gate_dtype, (size_t)p->n_expert * p->n_ff_exp, p->ne);
-    const size_t ub = expert_bank_bytes(p->up_dtype, (size_t)p->n_expert * p->n_ff_exp, p->ne);
+    if (p->has_ep_band)
+        return fail(be, INFR_HIP_ERR_UNSUPPORTED, "moe_ffn: ep_band (an expert-parallel shard) needs more than one GPU");
+    if (p->act < INFR_ACT_SILU || p->act > INFR_ACT_SIGMOID || p->gating < INFR_GATING_SOFTMAX ||
+        p->gating > INFR_GATING_SQRT_SOFTPLUS)
+        return fail(be, INFR_HIP_ERR_UNSUPPORTED, "moe_ffn: unknown activation or gating");
+    // the two combinations the CPU arm asserts against (lib.rs:2293-2309)
+    if (p->has_clamp && (p->act == INFR_ACT_SIGMOID || p->weight_before))
+        return fail(be, INFR_HIP_ERR_UNSUPPORTED, "moe_ffn: swiglu_clamp is defined for SiLU / GELU with output-side weighting only");
+    if (p->has_expert_ids && (p->has_exp_probs_b || p->n_expert_groups > 1))
+        return fail(be, INFR_HIP_ERR_UNSUPPORTED, "moe_ffn: expert_ids supplies the selection; exp_probs_b and expert groups must be absent");
+    const bool grouped = p->n_expert_groups > 1 && p->n_expert_groups_used > 0;
+    if (grouped && (p->n_expert_groups > 64 || p->n_expert % p->n_expert_groups != 0 ||
+                    p->n_expert_groups_used > p->n_expert_groups ||
+                    (uint64_t)p->n_expert / p->n_expert_groups * p->n_expert_groups_used < p->n_used))
+        return fail(be, INFR_HIP_ERR_UNSUPPORTED, "moe_ffn: expert groups must divide n_expert (at most 64 groups) and keep at least n_used experts");
+    const infr_hip_buffer_t* down_scale = opt ? opt->down_scale : nullptr;
+    const infr_hip_buffer_t* exp_probs_b = opt ? opt->exp_probs_b : nullptr;
+    const infr_hip_buffer_t* expert_ids = opt ? opt->expert_ids : nullptr;
+    if ((p->has_down_scale != 0) != (down_scale != nullptr) || (p->has_exp_probs_b != 0) != (exp_probs_b != nullptr) ||
+        (p->has_expert_ids != 0) != (expert_ids != nullptr))
+        return fail(be, INFR_HIP_ERR_INVALID, "moe_ffn: an optional operand does not match its has_* flag");
+    const int up_dtype = fused ? p->gate_dtype : p->up_dtype;
+    const size_t gb = expert_bank_bytes(p->gate_dtype, (size_t)p->n_expert * p->n_ff_exp * (fused ? 2 : 1), p->ne);
+    const size_t ub = fused ? gb : expert_bank_bytes(up_dtype, (size_t)p->n_expert * p->n_ff_exp, p->ne);
     const size_t db = expert_bank_bytes(p->down_dtype, (size_t)p->n_expert * p->ne, p->n_ff_exp);
-    if (!gb || !ub || !db || !is_moe_quant(p->gate_dtype) || !is_moe_quant(p->up_dtype) ||
+    if (!gb || !ub || !db || !is_moe_quant(p->gate_dtype) || !is_moe_quant(up_dtype) ||
         !is_moe_quant(p->down_dtype) || !is_plain(p->router_dtype))
         return fail(be, INFR_HIP_ERR_UNSUPPORTED, "moe_ffn: expert bank dtype/shape has no kernel");
     const size_t act_bytes = (size_t)p->rows * p->ne * sizeof(float);
-    if (gate->len < gb || up->len < ub || down->len < db ||
+    if (gate->len < gb || (!fused && up->len < ub) || down->len < db ||
         router->len < (size_t)p->n_expert * p->ne * (p->router_dtype == INFR_DTYPE_F32 ? 4 : 2) || x->len < act_bytes ||
         router_x->len < act_bytes || dst->len < act_bytes)
         return fail(be, INFR_HIP_ERR_INVALID, "moe_ffn: a buffer is smaller than its declared shape");
     const size_t sel_bytes = (size_t)p->rows * p->n_used * 4;
     if ((sel_idx && sel_idx->len < sel_bytes) || (sel_w && sel_w->len < sel_bytes))
         return fail(be, INFR_HIP_ERR_INVALID, "moe_ffn: selection output buffer too small");
+    if ((down_scale && down_scale->len < (size_t)p->n_expert * 4) || (exp_probs_b && exp_probs_b->len < (size_t)p->n_expert * 4) ||
+        (expert_ids && expert_ids->len < sel_bytes))
+        return fail(be, INFR_HIP_ERR_INVALID, "moe_ffn: an optional operand is smaller than its declared shape");
     *s = infr::MoeShape{(int)p->ne, (int)p->n_expert, (int)p->n_used, (int)p->n_ff_exp, (int)p->rows,
-                        p->scale, p->router_dtype, p->gate_dtype, p->up_dtype, p->down_dtype};
+                        p->scale, p->router_dtype, p->gate_dtype, up_dtype, p->down_dtype};
+    s->route.gating = p->gating;
+    s->route.norm_w = p->norm_w != 0;
+    s->route.n_groups = grouped ? (int)p->n_expert_groups : 0;
+    s->route.n_groups_used = grouped ? (int)p->n_expert_groups_used : 0;
+    s->route.bias = exp_probs_b ? static_cast<const float*>(exp_probs_b->ptr) : nullptr;
+    s->route.ids = expert_ids ? static_cast<const int32_t*>(expert_ids->ptr) : nullptr;
+    s->act.act = p->act;
+    s->act.has_clamp = p->has_clamp != 0;
+    s->act.clamp = p->clamp;
+    s->act.weight_before = p->weight_before != 0;
+    s->fused_gate_up = fused;
     b->x = static_cast<const float*>(x->ptr);
     b->router_x = static_cast<const float*>(router_x->ptr);
     b->router = static_cast<const float*>(router->ptr);
     b->gate = static_cast<const uint8_t*>(gate->ptr);
-    b->up = static_cast<const uint8_t*>(up->ptr);
+    b->up = fused ? b->gate : static_cast<const uint8_t*>(up->ptr);
     b->down = static_cast<const uint8_t*>(down->ptr);
     // expert e = the e-th equal byte slice of the bound bank (lib.rs:2345-2347)
     b->gate_stride = gate->len / p->n_expert;
-    b->up_stride = up->len / p->n_expert;
+    b->up_stride = fused ? b->gate_stride : up->len / p->n_expert;
     b->down_stride = down->len / p->n_expert;
     b->dst = static_cast<float*>(dst->ptr);
     b->sel_idx = sel_idx ? static_cast<int32_t*>(sel_idx->ptr) : nullptr;
     b->sel_w = sel_w ? static_cast<float*>(sel_w->ptr) : nullptr;
+    b->down_scale = down_scale ? static_cast<const float*>(down_scale->ptr) : nullptr;
     return INFR_HIP_OK;
+}
+
+// The optional operands of a plan's MoeFfn op, from the bindings.
+static infr_hip_moe_optional_t moe_optional(const infr_hip_op_t& op, infr_hip_buffer_t* const* bindings) {
+    infr_hip_moe_optional_t o{nullptr, nullptr, nullptr};
+    if (op.moe.has_down_scale) o.down_scale = bindings[op.down_scale];
+    if (op.moe.has_exp_probs_b) o.exp_probs_b = bindings[op.exp_probs_b];
+    if (op.moe.has_expert_ids) o.expert_ids = bindings[op.expert_ids];
+    return o;
 }
 
 static int enqueue_moe(infr_hip_t* be, const infr::MoeShape& s, const infr::MoeBuffers& b) {
@@ -851,13 +900,13 @@ static int enqueue_moe(infr_hip_t* be, const infr::MoeShape& s, const infr::MoeB
 int infr_hip_moe_ffn(infr_hip_t* be, const infr_hip_moe_params_t* p, const infr_hip_buffer_t* x,
                      const infr_hip_buffer_t* router_x, const infr_hip_buffer_t* router,
                      const infr_hip_buffer_t* gate_exps, const infr_hip_buffer_t* up_exps,
-                     const infr_hip_buffer_t* down_exps, infr_hip_buffer_t* dst,
+                     const infr_hip_buffer_t* down_exps, const infr_hip_moe_optional_t* opt, infr_hip_buffer_t* dst,
                      infr_hip_buffer_t* sel_idx, infr_hip_buffer_t* sel_w) {
     if (!be) return INFR_HIP_ERR_INVALID;
     if (int rc = check_latch(be)) return rc;
     infr::MoeShape s;
     infr::MoeBuffers b;
-    if (int rc = check_moe(be, p, x, router_x, router, gate_exps, up_exps, down_exps, dst, sel_idx, sel_w, &s, &b))
+    if (int rc = check_moe(be, p, x, router_x, router, gate_exps, up_exps, down_exps, opt, dst, sel_idx, sel_w, &s, &b))
         return rc;
     if (int rc = ensure_moe_ws(be, infr::moe_workspace_bytes(s))) return rc;
     return enqueue_moe(be, s, b);
@@ -871,7 +920,9 @@ int infr_hip_compile(infr_hip_t* be, const infr_hip_op_t* ops, size_t n_ops, inf
     infr_hip_plan_t* p = new (std::nothrow) infr_hip_plan();
     if (!p) return fail(be, INFR_HIP_ERR_OTHER, "compile: out of host memory");
     p->ops.assign(ops, ops + n_ops);
-    size_t act_need = 0, moe_need = 0, batch_need = 0;  // batch_need: every small-batch op in one level
+    // batch_need: one small-batch op's activations; a group of several distinct activation tensors
+    // grows the scratch when it is scheduled (the levels depend on the bound addresses)
+    size_t act_need = 0, moe_need = 0, batch_need = 0;
     for (const auto& op : p->ops) {
         if (op.kind == INFR_OP_LINEAR) {
             if ((!is_quant(op.w_dtype) && !is_plain(op.w_dtype)) || op.m == 0 || op.in_f == 0 || op.out_f == 0 ||
@@ -882,7 +933,7 @@ int infr_hip_compile(infr_hip_t* be, const infr_hip_op_t* ops, size_t n_ops, inf
             }
             p->max_tensor = std::max({p->max_tensor, op.x, op.weight, op.dst});
             act_need = std::max(act_need, linear_scratch_elems(op.w_dtype, op.m, op.in_f));
-            if (small_batch(op)) batch_need += ((size_t)op.m * op.in_f + 255) / 256 * 256;
+            if (small_batch(op)) batch_need = std::max(batch_need, ((size_t)op.m * op.in_f + 255) / 256 * 256);
         } else if (op.kind == INFR_OP_MOE_FFN) {
             const auto& mp = op.moe;
             if (!mp.ne || !mp.n_expert || !mp.n_used || !mp.n_ff_exp || !mp.rows) {
@@ -890,7 +941,9 @@ int infr_hip_compile(infr_hip_t* be, const infr_hip_op_t* ops, size_t n_ops, inf
                 return fail(be, INFR_HIP_ERR_UNSUPPORTED, "compile: MoeFfn op with empty shape");
             }
             p->max_tensor = std::max({p->max_tensor, op.x, op.dst, op.router_x, op.router,
-                                      op.gate_exps, op.up_exps, op.down_exps});
+                                      op.gate_exps, mp.fused_gate_up ? op.gate_exps : op.up_exps, op.down_exps,
+                                      mp.has_down_scale ? op.down_scale : 0u, mp.has_exp_probs_b ? op.exp_probs_b : 0u,
+                                      mp.has_expert_ids ? op.expert_ids : 0u});
             const infr::MoeShape ms{(int)mp.ne, (int)mp.n_expert, (int)mp.n_used, (int)mp.n_ff_exp,
                                     (int)mp.rows, mp.scale, mp.router_dtype, mp.gate_dtype,
                                     mp.up_dtype, mp.down_dtype};
@@ -990,12 +1043,16 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
         if (op.kind == INFR_OP_MOE_FFN) {
             infr::MoeShape ms;
             infr::MoeBuffers mb;
+            const infr_hip_moe_optional_t mo = moe_optional(op, bindings);
             if (int rc = check_moe(be, &op.moe, bindings[op.x], bindings[op.router_x], bindings[op.router],
-                                   bindings[op.gate_exps], bindings[op.up_exps], bindings[op.down_exps],
-                                   bindings[op.dst], nullptr, nullptr, &ms, &mb))
+                                   bindings[op.gate_exps], op.moe.fused_gate_up ? nullptr : bindings[op.up_exps],
+                                   bindings[op.down_exps], &mo, bindings[op.dst], nullptr, nullptr, &ms, &mb))
                 return rc;
             const size_t abytes = (size_t)ms.rows * ms.ne * sizeof(float);
             rd[i] = {span(bindings[op.x], abytes), span(bindings[op.router_x], abytes)};
+            if (mo.expert_ids) rd[i].push_back(span(mo.expert_ids, (size_t)ms.rows * ms.n_used * 4));
+            if (mo.down_scale) rd[i].push_back(span(mo.down_scale, (size_t)ms.n_expert * 4));
+            if (mo.exp_probs_b) rd[i].push_back(span(mo.exp_probs_b, (size_t)ms.n_expert * 4));
             wr[i] = {span(bindings[op.dst], abytes)};
         } else if (op.kind == INFR_OP_EMBED_GATHER) {
             EmbedArgs eg;
@@ -1290,8 +1347,10 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
                 const size_t x_elems = ((size_t)op.m * op.in_f + 255) / 256 * 256;
                 for (size_t k = i; k < n; ++k) {
                     const auto& o2 = plan->ops[k];
-                    if (level[k] != lv || taken[k] || o2.kind != INFR_OP_LINEAR || o2.m != op.m ||
-                        o2.w_dtype != op.w_dtype || o2.in_f != op.in_f)
+                    // (small_batch depends on out_f too: an op of the same dtype, rows and row length that
+                    // is not a small batch runs alone, as it does when it comes first)
+                    if (level[k] != lv || taken[k] || absorbed[k] || o2.kind != INFR_OP_LINEAR || o2.m != op.m ||
+                        o2.w_dtype != op.w_dtype || o2.in_f != op.in_f || !small_batch(o2))
                         continue;
                     taken[k] = 1;
                     const float* x = static_cast<const float*>(bindings[o2.x]->ptr);
@@ -1311,8 +1370,9 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
                     plan->descs.push_back(desc);
                 }
                 st.n = (int)plan->descs.size() - st.first;
-                if (xs.size() * x_elems > be->act_cap_elems)
-                    return fail(be, INFR_HIP_ERR_OTHER, "execute: activation scratch smaller than the plan needs");
+                // the group's distinct activation tensors side by side in the scratch (a regrow here is
+                // before anything of this schedule is recorded; it bumps the scratch epoch for other plans)
+                if (int rc = ensure_act(be, xs.size() * x_elems)) return rc;
                 if (!infr::plan_batch_group(st.dtype, st.m, st.in_f, &plan->descs[st.first], st.n, &st.bp))
                     return fail(be, INFR_HIP_ERR_UNSUPPORTED,
                                 "execute: no small-batch kernel for dtype " + std::to_string(st.dtype) +
@@ -1410,9 +1470,10 @@ static int enqueue_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t
             const auto& op = plan->ops[st.op];
             infr::MoeShape ms;
             infr::MoeBuffers mb;
+            const infr_hip_moe_optional_t mo = moe_optional(op, bindings);
             if (int rc = check_moe(be, &op.moe, bindings[op.x], bindings[op.router_x], bindings[op.router],
-                                   bindings[op.gate_exps], bindings[op.up_exps], bindings[op.down_exps],
-                                   bindings[op.dst], nullptr, nullptr, &ms, &mb))
+                                   bindings[op.gate_exps], op.moe.fused_gate_up ? nullptr : bindings[op.up_exps],
+                                   bindings[op.down_exps], &mo, bindings[op.dst], nullptr, nullptr, &ms, &mb))
                 return rc;
             if (plan->moe_norm[st.op] >= 0) {
                 const auto& nop = plan->ops[plan->moe_norm[st.op]];

@@ -14,8 +14,9 @@
 
 namespace infr {
 
-// One workgroup per row.
-__global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__ x,
+// One workgroup per row. `out` may alias `x` (in-place RmsNorm / RmsNormAdd), so neither carries
+// __restrict__.
+__global__ __launch_bounds__(256) void rms_norm_kernel(const float* x,
                                                        const float* __restrict__ w, float* out,
                                                        int dim, float eps, int accumulate) {
     __shared__ float part[4];
@@ -39,7 +40,7 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__
 // round trip per 256 elements of the row (10.6 us for 16 rows of 4096) - where this form requests all
 // of a thread's elements at once.
 template <int VPT>
-__global__ __launch_bounds__(256) void rms_norm_regs_kernel(const float* __restrict__ x,
+__global__ __launch_bounds__(256) void rms_norm_regs_kernel(const float* x,
                                                             const float* __restrict__ w, float* out,
                                                             int dim, float eps, int accumulate) {
     __shared__ float part[4];

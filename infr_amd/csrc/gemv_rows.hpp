@@ -34,11 +34,21 @@ struct LaneSums {
     static constexpr int kRows = 8, kRowStride = 68;
     static constexpr int kFloatsPerWave = kRows * kRowStride;
 };
+// Per-wave LDS scratch of the one-block-per-lane formats (Q8_0, the 32-weight-block formats) when
+// their per-block terms must be added in ascending block order as infr-cpu's scalar kernels add them
+// (kernels.rs:1170-1187: `sumf += d8 * d_w * iprod` block by block): every lane parks its block's
+// term, 8 rows x (64 * STEPS terms + 4 pad) floats, and lane i then adds row i's terms in order.
+template <int STEPS>
+struct LaneOrderedSum {
+    static constexpr int kRows = 8, kRowStride = 64 * STEPS + 4;
+    static constexpr int kFloatsPerWave = kRows * kRowStride;
+};
 // What gemv_rows needs per wave, by format.
-template <typename F, int STEPS>
+template <typename F, int STEPS, bool LANE_ORDERED = false>
 struct RowSumScratch {
     static constexpr int kFloatsPerWave =
-        F::kOrdered ? OrderedSum<STEPS>::kFloatsPerWave : (F::kLaneSums ? LaneSums::kFloatsPerWave : 1);
+        F::kOrdered ? OrderedSum<STEPS>::kFloatsPerWave
+                    : (LANE_ORDERED ? LaneOrderedSum<STEPS>::kFloatsPerWave : (F::kLaneSums ? LaneSums::kFloatsPerWave : 1));
 };
 
 // Step 0 of a row known to be readable, through the format's unpredicated loader where it has one.
@@ -63,7 +73,14 @@ __device__ __forceinline__ void load_row_clamped(typename F::Row& r, const uint8
 //
 // `add_first` is add_b[row0 + lane], requested by the caller ahead of its prologue (an absorbed
 // Op::Add); rows 64 and up of a wave read add_b when they are stored.
-template <typename F, int STEPS, bool STAGES, bool FIRST_WHOLE = false>
+//
+// LANE_ORDERED (formats that are not kOrdered, one block per lane): instead of a tree over the lanes,
+// every lane parks its block's term in LDS (LaneOrderedSum) and every eight rows lane i adds row i's
+// 64 * STEPS terms in ascending block order - the scalar CPU kernel's `sumf +=` chain, so the output
+// equals its bit for bit. Lanes past a row's last block park +0.0. The routed-expert GEMVs take this
+// form: their outputs are re-quantized to int8 for the down bank, where a last-bit difference in one
+// activation can flip a code.
+template <typename F, int STEPS, bool STAGES, bool FIRST_WHOLE = false, bool LANE_ORDERED = false>
 __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t bpr,
                                           const typename F::Row (&first)[FIRST_WHOLE ? STEPS : 1],
                                           const typename F::Acts (&acts)[STEPS],
@@ -82,17 +99,41 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
     // then only the sum is stored, through add_dst alone.
     const bool plain_y = y != add_dst;
     constexpr int LS = OrderedSum<STEPS>::kRowStride;
+    constexpr int LSO = LaneOrderedSum<STEPS>::kRowStride;
+    static_assert(!(LANE_ORDERED && F::kOrdered), "the ordered formats already add their blocks in order");
     int in_batch = 0, batch_row0 = row0;
     // A row's step-t term: parked for the ordered sum, or added to the lane's partial sum.
     auto take_term = [&](int t, float term, float& s) {
-        if (F::kOrdered) {
+        if (LANE_ORDERED) {
+            osum[in_batch * LSO + t * 64 + lane] = term;
+        } else if (F::kOrdered) {
             if ((lane & 3) == 0) osum[in_batch * LS + t * 16 + (lane >> 2)] = term;
         } else {
             s += term;
         }
     };
     auto finish_row = [&](int row, float s) {
-        if (F::kOrdered) {
+        if (LANE_ORDERED) {
+            if (++in_batch == LaneOrderedSum<STEPS>::kRows || row + 1 == row_end) {
+                const float resid = add_dst ? residual(batch_row0 + lane, lane < in_batch) : 0.0f;
+                if (lane < in_batch) {
+                    const v4f* tr = reinterpret_cast<const v4f*>(osum + lane * LSO);
+                    float acc = 0.0f;
+#pragma unroll 4
+                    for (int k = 0; k < 16 * STEPS; ++k) {
+                        const v4f v = tr[k];
+                        acc += v.x;
+                        acc += v.y;
+                        acc += v.z;
+                        acc += v.w;
+                    }
+                    if (plain_y) gstore<float>(y + batch_row0 + lane, acc);
+                    if (add_dst) gstore<float>(add_dst + batch_row0 + lane, acc + resid);
+                }
+                batch_row0 = row + 1;
+                in_batch = 0;
+            }
+        } else if (F::kOrdered) {
             if (++in_batch == 16 || row + 1 == row_end) {
                 const float resid = add_dst ? residual(batch_row0 + lane, lane < in_batch) : 0.0f;
                 if (lane < in_batch) {

@@ -236,11 +236,30 @@ void launch_gated_act(const float* gate, const float* up, float* out, const Gate
                       hipStream_t stream);
 void launch_add(const float* a, const float* b, float* out, size_t n, hipStream_t stream);
 
-// Op::MoeFfn (qwen3moe form). Expert e of a bank starts at bank + e * stride.
+// Op::MoeFfn. Expert e of a bank starts at bank + e * stride.
+// Routing (crates/infr-core/src/graph.rs:956-1010): how logits become probabilities, what the
+// selection ranks, how the selected probabilities become weights.
+struct MoeRoute {
+    int gating = 0;  // 0 softmax, 1 sigmoid, 2 sqrt(softplus)
+    int norm_w = 1;  // w = p / max(sum_sel p, 1e-20) * scale, else p * scale
+    int n_groups = 0, n_groups_used = 0;  // group-limited routing when n_groups > 1 and n_groups_used > 0
+    const float* bias = nullptr;          // exp_probs_b [n_expert]: added for the selection only
+    const int32_t* ids = nullptr;         // expert_ids [rows, n_used]: the selection itself
+};
+// The experts' gated activation (graph.rs:948-967).
+struct MoeAct {
+    int act = 0;  // 0 SiLU, 1 GELU (tanh form), 2 sigmoid
+    int has_clamp = 0;
+    float clamp = 0.0f;
+    int weight_before = 0;  // the routing weight on gate / up in front of the activation, not on the output
+};
 struct MoeShape {
     int ne, n_expert, n_used, n_ff, rows;
     float scale;
     int router_dtype, gate_dtype, up_dtype, down_dtype;
+    MoeRoute route;
+    MoeAct act;
+    int fused_gate_up = 0;  // `gate` holds [gate rows | up rows] per expert; `up` is not read
 };
 struct MoeBuffers {
     const float* x;         // [rows, ne]
@@ -253,6 +272,7 @@ struct MoeBuffers {
     float* dst;             // [rows, ne]
     int32_t* sel_idx;       // optional [rows, n_used]
     float* sel_w;           // optional [rows, n_used]
+    const float* down_scale = nullptr;  // optional f32 [n_expert]: y_e * down_scale[e] before the weighted sum
     // absorbed Op::Add (fusion.rs:155-200): add_dst[i] = dst[i] + add_b[i] from the kernel that
     // produces dst; add_dst may be add_b (each element is read and written by one thread)
     const float* add_b = nullptr;

@@ -7,8 +7,8 @@
 // the activation tile (row-major per-256 quantized rows, gathered through `perm`) sits in
 // double-buffered LDS. One policy per format supplies the bytes to load, the operands and what a
 // step adds to the 16 accumulators; integers, f32 expressions and block order are those of the
-// formats' dense prefill kernels (mmq_q5k.hip, mmq_q6k.hip, mmq_q8_0.hip), so Q5_K and Q6_K pairs
-// equal the per-pair GEMV bit for bit and Q8_0 pairs agree to rounding.
+// formats' dense prefill kernels (mmq_q5k.hip, mmq_q6k.hip) and, for Q8_0, of the scalar CPU kernel, so every
+// pair equals the per-pair GEMV bit for bit.
 #include "device_common.hpp"
 #include "kernels.hpp"
 #include "mmq_tiles.hpp"
@@ -138,7 +138,10 @@ struct GatherQ5K {
     }
 };
 
-// Q8_0 (eight 34-byte blocks per step): the stored codes are the operand; d8 * sum_blocks d_w * iprod.
+// Q8_0 (eight 34-byte blocks per step): the stored codes are the operand; every 32-block adds
+// (d8 * d_w) * (f32)iprod to the output, blocks ascending and without FMA - the scalar CPU kernel's
+// `sumf += d8 * d_w * iprod as f32` (kernels.rs:1170-1187) - so a pair's gate / up outputs, and with
+// them the int8 codes of its gated activation, equal the CPU's bit for bit.
 struct GatherQ8_0 {
     static constexpr int kStepBytes = 8 * 34;
     struct Raw {
@@ -154,22 +157,19 @@ struct GatherQ8_0 {
     }
     __device__ static void step(const Raw& cur, const GatherCtx& c, float (&acc)[16]) {
         const v16i zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        float part[16];
+        float dq[16];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) part[i] = 0.0f;
+        for (int j = 0; j < 4; ++j) {
+            const v4f q = *reinterpret_cast<const v4f*>(c.dtile + 8 * j);
+            dq[4 * j + 0] = q.x; dq[4 * j + 1] = q.y; dq[4 * j + 2] = q.z; dq[4 * j + 3] = q.w;
+        }
 #pragma unroll
         for (int sb = 0; sb < 8; ++sb) {
             const v4i a = *reinterpret_cast<const v4i*>(c.arow + sb * 32);
             const v16i r = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, cur.q[sb], zi, 0, 0, 0);
             const float dw = f16_bits_to_f32(cur.d[sb]);
 #pragma unroll
-            for (int i = 0; i < 16; ++i) part[i] = __builtin_fmaf(dw, (float)r[i], part[i]);
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const v4f dq = *reinterpret_cast<const v4f*>(c.dtile + 8 * j);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) acc[4 * j + i] = __builtin_fmaf(dq[i], part[4 * j + i], acc[4 * j + i]);
+            for (int i = 0; i < 16; ++i) acc[i] += (dq[i] * dw) * (float)r[i];
         }
     }
 };

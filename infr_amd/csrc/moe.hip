@@ -1,6 +1,8 @@
-// Op::MoeFfn on the device, as qwen3moe emits it (softmax gating, renormalised top-k, split
-// gate/up banks, SiLU, weights applied to the expert outputs). Mirrors infr-cpu's staged
-// pipeline (crates/infr-cpu/src/lib.rs:2264-2984, crates/infr-cpu/src/moe.rs):
+// Op::MoeFfn on the device. Mirrors infr-cpu's staged pipeline (crates/infr-cpu/src/lib.rs:2264-2984,
+// crates/infr-cpu/src/moe.rs); the list below is qwen3moe's setting (softmax gating, renormalised
+// top-k, split gate/up banks, SiLU, weights on the expert outputs), the op's other fields - gating
+// function, selection bias, group-limited routing, supplied expert ids, activation and clamp, the
+// weight on the expert input, fused gate|up banks, per-expert down scale - are MoeRoute / MoeAct below:
 //
 //   router   f32 router rows . router_x with infr-cpu's `dot` (8 FMA accumulators by index mod 8,
 //            summed in order, kernels.rs:6557-6573), evaluated in that exact order so the logits -
@@ -22,18 +24,24 @@
 #include "gemv_rows.hpp"
 #include "kernels.hpp"
 #include "decode_element.hpp"
+#include "elementwise_fn.hpp"
 #include "quant_chunk.hpp"
 
 namespace infr {
 
 // ───────────────────────────── router + selection ─────────────────────────────
 
-// LDS of one selection: probabilities, their ranks, the ranked winners, reduction slots.
+// LDS of one selection: probabilities, the values the selection ranks (the probabilities plus an
+// optional bias, masked by group), their ranks, the ranked winners with their weights, reduction slots.
 struct SelectLds {
     float p[1024];
+    float sv[1024];
     int rank[1024];
     float top_p[64];
+    float top_w[64];
     int top_e[64];
+    float gscore[64];
+    int gkeep[64];
     float red[8];
 };
 
@@ -52,19 +60,27 @@ __device__ __forceinline__ void quad_place_q6k(int e, int& u, int& q) {
     q = 4 * (r2 >> 5) + ((r3 & 15) >> 2);
 }
 
-// Softmax + stable top-n_used + renormalised weights for one row, run by a whole 256-thread
-// workgroup. n_expert <= 1024, n_used <= 64. Order-sensitive parts follow the CPU: probabilities
-// are summed in index order by one thread, the stable descending sort is realised by counting
-// rank(e) = #{j : p[j] > p[e] or (p[j] == p[e] and j < e)} on the NORMALISED probabilities
-// (normalising can create ties that the raw exponentials do not have), and the selected
-// probabilities are summed in rank order.
+// Gating probabilities, selection and weights of one row (lib.rs:2421-2543), run by a whole
+// 256-thread workgroup. n_expert <= 1024, n_used <= 64, at most 64 groups.
+//   probabilities  softmax with max-subtraction, summed in index order by one thread; or a per-expert
+//                  sigmoid; or sqrt(softplus) with the CPU's v > 20 shortcut
+//   selection      on a copy: + bias (exp_probs_b), then group-limited routing - a group's score is the
+//                  sum of its two best values, the best `n_groups_used` groups (ties to the lower group)
+//                  keep their values, the others become -inf - then the stable descending sort,
+//                  realised by counting rank(e) = #{j : v[j] > v[e] or (v[j] == v[e] and j < e)} (for
+//                  softmax on the NORMALISED probabilities: normalising can create ties that the raw
+//                  exponentials do not have). Supplied ids replace all of it, in their own order.
+//   weights        from the unbiased probabilities, summed in rank order:
+//                  norm_w ? p / max(sum, 1e-20) * scale : p * scale
+// Leaves s.top_e / s.top_p / s.top_w (all threads may read them on return) and stores the ranked
+// experts and weights when out_idx is given.
 // COHERENT: the logits were written by other workgroups of the same launch (with device-scope
 // stores) and are read past this compute unit's and this die's caches.
 template <bool COHERENT = false>
 __device__ __forceinline__ void moe_select_block(const float* __restrict__ l, SelectLds& s,
                                                  int n_expert, int n_used, float scale, int tid,
                                                  int32_t* __restrict__ out_idx,
-                                                 float* __restrict__ out_w) {
+                                                 float* __restrict__ out_w, const MoeRoute& rt, size_t row) {
     const int lane = tid & 63, wave = tid >> 6;
     float lv[4];
     float mx = -INFINITY;
@@ -76,82 +92,139 @@ __device__ __forceinline__ void moe_select_block(const float* __restrict__ l, Se
                              : l[e];
         mx = __builtin_fmaxf(mx, lv[i]);
     }
+    if (rt.gating == 0) {
 #pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) mx = __builtin_fmaxf(mx, __shfl_xor(mx, off, kWave));
-    if (lane == 0) s.red[wave] = mx;
-    __syncthreads();
-    mx = __builtin_fmaxf(__builtin_fmaxf(s.red[0], s.red[1]), __builtin_fmaxf(s.red[2], s.red[3]));
+        for (int off = 32; off >= 1; off >>= 1) mx = __builtin_fmaxf(mx, __shfl_xor(mx, off, kWave));
+        if (lane == 0) s.red[wave] = mx;
+        __syncthreads();
+        mx = __builtin_fmaxf(__builtin_fmaxf(s.red[0], s.red[1]), __builtin_fmaxf(s.red[2], s.red[3]));
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int e = tid + 256 * i;
-        if (e < n_expert) {
-            lv[i] = expf(lv[i] - mx);
-            s.p[e] = lv[i];
-            s.rank[e] = 0;
-        }
-    }
-    __syncthreads();
-    if (tid == 0) {  // `p.iter().sum()`: index order; 32 LDS values per wait
-        float sum = 0.0f;
-        int e = 0;
-        for (; e + 32 <= n_expert; e += 32) {
-            v4f q[8];
-#pragma unroll
-            for (int k = 0; k < 8; ++k) q[k] = *reinterpret_cast<const v4f*>(s.p + e + 4 * k);
-#pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                sum += q[k].x; sum += q[k].y; sum += q[k].z; sum += q[k].w;
+        for (int i = 0; i < 4; ++i) {
+            const int e = tid + 256 * i;
+            if (e < n_expert) {
+                lv[i] = expf(lv[i] - mx);
+                s.p[e] = lv[i];
+                s.rank[e] = 0;
             }
         }
-        for (; e < n_expert; ++e) sum += s.p[e];
-        s.red[4] = sum;
-    }
-    __syncthreads();
-    const float psum = s.red[4];
+        __syncthreads();
+        if (tid == 0) {  // `p.iter().sum()`: index order; 32 LDS values per wait
+            float sum = 0.0f;
+            int e = 0;
+            for (; e + 32 <= n_expert; e += 32) {
+                v4f q[8];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int e = tid + 256 * i;
-        if (e < n_expert) s.p[e] = lv[i] / psum;
-    }
-    __syncthreads();
-    // rank by counting: `parts` threads share an expert when n_expert < 256
-    const int parts = n_expert <= 128 ? 256 / n_expert : 1;
-    const int span = ((n_expert + parts - 1) / parts + 3) & ~3;
-    for (int item = tid; item < n_expert * parts; item += 256) {
-        const int e = item % n_expert, part = item / n_expert;
-        const float v = s.p[e];
-        const int j0 = part * span, j1 = min(n_expert, j0 + span);
-        int cnt = 0, j = j0;
-        for (; j + 4 <= j1; j += 4) {
-            const v4f q = *reinterpret_cast<const v4f*>(s.p + j);
-            cnt += (q.x > v ? 1 : 0) + ((q.x == v && j + 0 < e) ? 1 : 0);
-            cnt += (q.y > v ? 1 : 0) + ((q.y == v && j + 1 < e) ? 1 : 0);
-            cnt += (q.z > v ? 1 : 0) + ((q.z == v && j + 2 < e) ? 1 : 0);
-            cnt += (q.w > v ? 1 : 0) + ((q.w == v && j + 3 < e) ? 1 : 0);
+                for (int k = 0; k < 8; ++k) q[k] = *reinterpret_cast<const v4f*>(s.p + e + 4 * k);
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    sum += q[k].x; sum += q[k].y; sum += q[k].z; sum += q[k].w;
+                }
+            }
+            for (; e < n_expert; ++e) sum += s.p[e];
+            s.red[4] = sum;
         }
-        for (; j < j1; ++j) {
-            const float q = s.p[j];
-            cnt += (q > v ? 1 : 0) + ((q == v && j < e) ? 1 : 0);
+        __syncthreads();
+        const float psum = s.red[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int e = tid + 256 * i;
+            if (e < n_expert) s.p[e] = lv[i] / psum;
         }
-        if (parts > 1) atomicAdd(&s.rank[e], cnt);
-        else s.rank[e] = cnt;
-    }
-    __syncthreads();
-    for (int e = tid; e < n_expert; e += 256) {
-        const int r = s.rank[e];
-        if (r < n_used) {
-            s.top_e[r] = e;
-            s.top_p[r] = s.p[e];
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int e = tid + 256 * i;
+            if (e < n_expert) {
+                const float v = lv[i];
+                s.p[e] = rt.gating == 1 ? 1.0f / (1.0f + expf(-v)) : sqrtf(v > 20.0f ? v : logf(1.0f + expf(v)));
+                s.rank[e] = 0;
+            }
         }
     }
     __syncthreads();
-    if (out_idx && tid < n_used) {  // (without outputs the caller reads s.top_e)
+    if (rt.ids) {  // the selection is given; the weights still come from the probabilities
+        if (tid < n_used) {
+            const int e = min(max(rt.ids[row * n_used + tid], 0), n_expert - 1);
+            s.top_e[tid] = e;
+            s.top_p[tid] = s.p[e];
+        }
+    } else {
+        const float* v = s.p;  // what the selection ranks
+        const bool grouped = rt.n_groups > 1 && rt.n_groups_used > 0;
+        if (rt.bias || grouped) {
+            for (int e = tid; e < n_expert; e += 256) s.sv[e] = rt.bias ? s.p[e] + rt.bias[e] : s.p[e];
+            __syncthreads();
+            if (grouped) {
+                const int per = n_expert / rt.n_groups;
+                if (tid < rt.n_groups) {
+                    float b0 = -INFINITY, b1 = -INFINITY;
+                    for (int i = 0; i < per; ++i) {
+                        const float x = s.sv[tid * per + i];
+                        if (x > b0) { b1 = b0; b0 = x; } else if (x > b1) { b1 = x; }
+                    }
+                    s.gscore[tid] = b0 + b1;
+                }
+                __syncthreads();
+                if (tid < rt.n_groups) {
+                    const float g = s.gscore[tid];
+                    int cnt = 0;
+                    for (int j = 0; j < rt.n_groups; ++j) {
+                        const float q = s.gscore[j];
+                        cnt += (q > g ? 1 : 0) + ((q == g && j < tid) ? 1 : 0);
+                    }
+                    s.gkeep[tid] = cnt < rt.n_groups_used;
+                }
+                __syncthreads();
+                for (int e = tid; e < n_expert; e += 256)
+                    if (!s.gkeep[e / per]) s.sv[e] = -INFINITY;
+                __syncthreads();
+            }
+            v = s.sv;
+        }
+        // rank by counting: `parts` threads share an expert when n_expert < 256
+        const int parts = n_expert <= 128 ? 256 / n_expert : 1;
+        const int span = ((n_expert + parts - 1) / parts + 3) & ~3;
+        for (int item = tid; item < n_expert * parts; item += 256) {
+            const int e = item % n_expert, part = item / n_expert;
+            const float ve = v[e];
+            const int j0 = part * span, j1 = min(n_expert, j0 + span);
+            int cnt = 0, j = j0;
+            for (; j + 4 <= j1; j += 4) {
+                const v4f q = *reinterpret_cast<const v4f*>(v + j);
+                cnt += (q.x > ve ? 1 : 0) + ((q.x == ve && j + 0 < e) ? 1 : 0);
+                cnt += (q.y > ve ? 1 : 0) + ((q.y == ve && j + 1 < e) ? 1 : 0);
+                cnt += (q.z > ve ? 1 : 0) + ((q.z == ve && j + 2 < e) ? 1 : 0);
+                cnt += (q.w > ve ? 1 : 0) + ((q.w == ve && j + 3 < e) ? 1 : 0);
+            }
+            for (; j < j1; ++j) {
+                const float q = v[j];
+                cnt += (q > ve ? 1 : 0) + ((q == ve && j < e) ? 1 : 0);
+            }
+            if (parts > 1) atomicAdd(&s.rank[e], cnt);
+            else s.rank[e] = cnt;
+        }
+        __syncthreads();
+        for (int e = tid; e < n_expert; e += 256) {
+            const int r = s.rank[e];
+            if (r < n_used) {
+                s.top_e[r] = e;
+                s.top_p[r] = s.p[e];
+            }
+        }
+    }
+    __syncthreads();
+    if (tid < n_used) {
         float wsum = 0.0f;  // summed in rank order, as the CPU sums its selection
         for (int k = 0; k < n_used; ++k) wsum += s.top_p[k];
         wsum = __builtin_fmaxf(wsum, 1e-20f);
-        out_idx[tid] = s.top_e[tid];
-        out_w[tid] = s.top_p[tid] / wsum * scale;
+        const float w = rt.norm_w ? s.top_p[tid] / wsum * scale : s.top_p[tid] * scale;
+        s.top_w[tid] = w;
+        if (out_idx) {
+            out_idx[tid] = s.top_e[tid];
+            out_w[tid] = w;
+        }
     }
+    __syncthreads();
 }
 
 // One workgroup per row (used when there are several rows; a single row is selected by the
@@ -165,7 +238,7 @@ __global__ __launch_bounds__(256) void moe_select_kernel(const float* __restrict
                                                          const float* __restrict__ x, int ne,
                                                          int8_t* __restrict__ qs, float* __restrict__ qd,
                                                          int32_t* __restrict__ bsums,
-                                                         int32_t* __restrict__ bsums16) {
+                                                         int32_t* __restrict__ bsums16, MoeRoute rt) {
     __shared__ __attribute__((aligned(16))) SelectLds s;
     const size_t r = blockIdx.x;
     if (x) {
@@ -177,7 +250,7 @@ __global__ __launch_bounds__(256) void moe_select_kernel(const float* __restrict
         }
     }
     moe_select_block(logits + r * n_expert, s, n_expert, n_used, scale, threadIdx.x, sel_idx + r * n_used,
-                     sel_w + r * n_used);
+                     sel_w + r * n_used, rt, r);
 }
 
 // infr-cpu's `dot` keeps 8 FMA accumulators (element i goes to accumulator i mod 8) and adds them
@@ -225,7 +298,7 @@ __global__ __launch_bounds__(256) void moe_router_kernel(
     const void* __restrict__ router, const float* __restrict__ rx, float* __restrict__ logits,
     int* __restrict__ tickets, int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, int ne,
     int n_expert, int rows, int n_used, float scale, int kc, int epw, int tpw, const float* __restrict__ norm_w,
-    float* __restrict__ norm_dst, float norm_eps, float* __restrict__ xt, int xt_q6k) {
+    float* __restrict__ norm_dst, float norm_eps, float* __restrict__ xt, int xt_q6k, MoeRoute rt) {
     extern __shared__ __attribute__((aligned(16))) float rl[];  // [epw] rows | [32 / epw] rows
     __shared__ __attribute__((aligned(16))) SelectLds sel;
     __shared__ int s_last;
@@ -329,7 +402,7 @@ __global__ __launch_bounds__(256) void moe_router_kernel(
     if (tid == 0) s_last = atomicAdd(tickets, 1) == (int)gridDim.x - 1;
     __syncthreads();
     if (!s_last) return;
-    moe_select_block<true>(logits, sel, n_expert, n_used, scale, tid, sel_idx, sel_w);
+    moe_select_block<true>(logits, sel, n_expert, n_used, scale, tid, sel_idx, sel_w, rt, 0);
     if (tid == 0) *tickets = 0;
 }
 
@@ -708,7 +781,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_f32_kernel(
     const uint8_t* __restrict__ gate, const uint8_t* __restrict__ up, size_t gate_stride,
     size_t up_stride, const float* __restrict__ logits, int n_expert, int n_used, float scale,
     int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, const float* __restrict__ x,
-    float* __restrict__ act, int ne, int nff, int S, int chunks, int down_q6k) {
+    float* __restrict__ act, int ne, int nff, int S, int chunks, int down_q6k, MoeRoute rt, MoeAct ma) {
     __shared__ __attribute__((aligned(16))) SelectLds sel;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int rps = 64 / S;  // S lanes per weight row (each on `chunks` units of it), rows per wave step
@@ -730,9 +803,12 @@ __global__ __launch_bounds__(256) void moe_gate_up_f32_kernel(
     // the ranked experts and weights for the down kernel.
     const bool first = blockIdx.x == 0 && blockIdx.y == 0;
     moe_select_block(logits, sel, n_expert, n_used, scale, threadIdx.x, first ? sel_idx : nullptr,
-                     first ? sel_w : nullptr);
+                     first ? sel_w : nullptr, rt, 0);
     if (st0 >= steps_total) return;
     const int e = sel.top_e[slot];
+    // the routing weight on the expert input (`weight_before`): gate and up are linear in x, so it
+    // multiplies their outputs in front of the activation (lib.rs:2833-2857)
+    const float wp = ma.weight_before ? sel.top_w[slot] : 1.0f;
     const size_t bpr = (size_t)(ne / 256) * P::kBlockBytes;
     const uint8_t* gw = gate + (size_t)e * gate_stride;
     const uint8_t* uw = up + (size_t)e * up_stride;
@@ -768,7 +844,8 @@ __global__ __launch_bounds__(256) void moe_gate_up_f32_kernel(
             int du, dq;
             if (down_q6k) quad_place_q6k(o, du, dq);
             else quad_place_linear(o, du, dq);
-            act[(size_t)slot * nff + ((size_t)dq * (nff / 64) + du) * 4 + (o & 3)] = gs / (1.0f + expf(-gs)) * us;
+            act[(size_t)slot * nff + ((size_t)dq * (nff / 64) + du) * 4 + (o & 3)] =
+                gated_act_fn(ma.act, ma.has_clamp != 0, ma.clamp, wp * gs, wp * us);
         }
     }
 }
@@ -785,7 +862,8 @@ template <typename P, int STEPS>
 __global__ __launch_bounds__(64 * kDownMaxWaves) void moe_down_f32_kernel(
     const uint8_t* __restrict__ down, size_t down_stride, const int32_t* __restrict__ ids,
     const float* __restrict__ wts, const float* __restrict__ act, float* __restrict__ out,
-    const float* add_b, float* add_dst, int nff, int ne, int n_used, int S, int chunks) {
+    const float* add_b, float* add_dst, int nff, int ne, int n_used, int S, int chunks, int unit_w,
+    const float* __restrict__ down_scale) {
     __shared__ float ys[kDownMaxSteps][kDownMaxWaves][16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     const int rps = 64 / S;
@@ -801,6 +879,7 @@ __global__ __launch_bounds__(64 * kDownMaxWaves) void moe_down_f32_kernel(
         if (k0) __syncthreads();
         if (k < n_used) {
             const uint8_t* dw = down + (size_t)ids[k] * down_stride;
+            const float ds = down_scale ? down_scale[ids[k]] : 1.0f;  // `y = raw * s_e` (lib.rs:2932-2938)
             float part[STEPS];
 #pragma unroll
             for (int s = 0; s < STEPS; ++s) part[s] = 0.0f;
@@ -821,13 +900,14 @@ __global__ __launch_bounds__(64 * kDownMaxWaves) void moe_down_f32_kernel(
 #pragma unroll
             for (int s = 0; s < STEPS; ++s) {
                 const float yk = seg_sum(part[s], seg * S, S);
-                if (lane_ok && u == 0) ys[s][wave][seg] = yk;
+                if (lane_ok && u == 0) ys[s][wave][seg] = down_scale ? yk * ds : yk;
             }
         }
         __syncthreads();
         if (owner) {
             const int kn = min(nw, n_used - k0);
-            for (int j = 0; j < kn; ++j) acc += wts[k0 + j] * ys[own_s][j][own_seg];
+            // (`weight_before`: the weight is inside the activation already, w_e = 1.0, lib.rs:2976)
+            for (int j = 0; j < kn; ++j) acc += (unit_w ? 1.0f : wts[k0 + j]) * ys[own_s][j][own_seg];
         }
     }
     if (owner) {
@@ -840,6 +920,14 @@ __global__ __launch_bounds__(64 * kDownMaxWaves) void moe_down_f32_kernel(
 }
 
 // ───────────────────────────── rows >= 2: int8 path ─────────────────────────────
+
+// gated_act_fn(act, clamp, wp * gate, wp * up) for four elements (lib.rs:2836-2857): wp is the pair's
+// routing weight under `weight_before`, else 1.0 (an exact identity).
+__device__ __forceinline__ v4f moe_gated4(const MoeAct& ma, float wp, const v4f& g, const v4f& u) {
+    const bool c = ma.has_clamp != 0;
+    return v4f{gated_act_fn(ma.act, c, ma.clamp, wp * g.x, wp * u.x), gated_act_fn(ma.act, c, ma.clamp, wp * g.y, wp * u.y),
+               gated_act_fn(ma.act, c, ma.clamp, wp * g.z, wp * u.z), gated_act_fn(ma.act, c, ma.clamp, wp * g.w, wp * u.w)};
+}
 
 // id-gathered decode GEMV over pre-quantized activation rows: pair = blockIdx.y,
 // weights = bank + ids[pair] * expert_stride, activation row = pair / n_used.
@@ -870,11 +958,16 @@ __global__ __launch_bounds__(256) void gemv_id_kernel(const uint8_t* __restrict_
     F::load_row(first[0], w + (size_t)row0 * bpr, 0, lane, ok[0]);
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) F::load_acts(acts[t], a, t, lane, ok[t]);
-    // same body as the decode GEMV: per-block exact integers, CPU-ordered f32 sum
-    __shared__ __attribute__((aligned(16))) float osum[4 * RowSumScratch<F, STEPS>::kFloatsPerWave];
-    gemv_rows<F, STEPS, false>(w, bpr, first, acts, ok, y + (size_t)pair * out_f, n_units, row0, row_end,
-                               lane, StagePtrs{nullptr, nullptr},
-                               osum + (threadIdx.x >> 6) * RowSumScratch<F, STEPS>::kFloatsPerWave);
+    // same body as the decode GEMV: per-block exact integers, and the f32 terms added in ascending
+    // block order for every format (the one-block-per-lane formats through LANE_ORDERED), so each
+    // output equals the scalar CPU kernel's bit for bit and the int8 codes of the gated activation
+    // that the down bank multiplies equal the CPU's
+    constexpr bool kLaneOrdered = !F::kOrdered;
+    __shared__ __attribute__((aligned(16))) float osum[4 * RowSumScratch<F, STEPS, kLaneOrdered>::kFloatsPerWave];
+    gemv_rows<F, STEPS, false, false, kLaneOrdered>(w, bpr, first, acts, ok, y + (size_t)pair * out_f, n_units, row0,
+                                                    row_end, lane, StagePtrs{nullptr, nullptr},
+                                                    osum + (threadIdx.x >> 6) *
+                                                               RowSumScratch<F, STEPS, kLaneOrdered>::kFloatsPerWave);
 }
 
 // The same for short rows (in_f <= 2048) of Q4_K / Q6_K banks: 16 / nb rows per wave step.
@@ -921,17 +1014,15 @@ __global__ __launch_bounds__(256) void moe_act_quant_kernel(const float* __restr
                                                             float* __restrict__ d,
                                                             int32_t* __restrict__ bsums,
                                                             int32_t* __restrict__ bsums16,
-                                                            size_t n_elems) {
+                                                            size_t n_elems, int nff, MoeAct ma,
+                                                            const float* __restrict__ pair_w) {
     const int lane = threadIdx.x & 63;
     const size_t chunk = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (chunk * 256 >= n_elems) return;
     const v4f gv = *reinterpret_cast<const v4f*>(g + chunk * 256 + (size_t)lane * 4);
     const v4f uv = *reinterpret_cast<const v4f*>(u + chunk * 256 + (size_t)lane * 4);
-    v4f a;
-    a.x = gv.x / (1.0f + expf(-gv.x)) * uv.x;
-    a.y = gv.y / (1.0f + expf(-gv.y)) * uv.y;
-    a.z = gv.z / (1.0f + expf(-gv.z)) * uv.z;
-    a.w = gv.w / (1.0f + expf(-gv.w)) * uv.w;
+    const float wp = ma.weight_before ? pair_w[chunk * 256 / (size_t)nff] : 1.0f;
+    const v4f a = moe_gated4(ma, wp, gv, uv);
     quantize_chunk<PER32>(a, true, lane, chunk, qs, d, bsums, PER32 ? nullptr : bsums16);
 }
 
@@ -954,7 +1045,8 @@ template <typename F>
 __global__ __launch_bounds__(1024) void moe_down_fused_kernel(
     const uint8_t* __restrict__ bank, size_t expert_stride, size_t bpr, const int32_t* __restrict__ ids,
     const float* __restrict__ wts, const float* __restrict__ g, const float* __restrict__ u,
-    float* __restrict__ out, const float* add_b, float* add_dst, int nff, int ne, int n_used, int rows_per_wg) {
+    float* __restrict__ out, const float* add_b, float* add_dst, int nff, int ne, int n_used, int rows_per_wg,
+    MoeAct ma, const float* __restrict__ down_scale) {
     extern __shared__ __attribute__((aligned(16))) uint8_t dlds[];
     const int lane = threadIdx.x & 63, k = threadIdx.x >> 6;
     const int token = blockIdx.y, pair = token * n_used + k;
@@ -973,14 +1065,11 @@ __global__ __launch_bounds__(1024) void moe_down_fused_kernel(
     const int q = lane >> 2, rq = q / nb;
     typename F::Row first;
     F::load_row(first, w + (size_t)row0 * bpr, 0, lane, rq < 16 / nb && row0 + rq < row_end);
+    const float wp = ma.weight_before ? wts[pair] : 1.0f;
     for (int c = 0; c < nb; ++c) {
         const v4f gv = *reinterpret_cast<const v4f*>(g + (size_t)pair * nff + c * 256 + lane * 4);
         const v4f uv = *reinterpret_cast<const v4f*>(u + (size_t)pair * nff + c * 256 + lane * 4);
-        v4f a;
-        a.x = gv.x / (1.0f + expf(-gv.x)) * uv.x;
-        a.y = gv.y / (1.0f + expf(-gv.y)) * uv.y;
-        a.z = gv.z / (1.0f + expf(-gv.z)) * uv.z;
-        a.w = gv.w / (1.0f + expf(-gv.w)) * uv.w;
+        const v4f a = moe_gated4(ma, wp, gv, uv);
         quantize_chunk<false>(a, true, lane, (size_t)c, qs, d, bsums, bsums16);
     }
     __syncthreads();
@@ -998,7 +1087,8 @@ __global__ __launch_bounds__(1024) void moe_down_fused_kernel(
         float acc = 0.0f;
         for (int j = 0; j < n_used; ++j) {
             const float* yj = reinterpret_cast<const float*>(dlds + (size_t)j * wave_bytes + y_off);
-            acc += wts[token * n_used + j] * yj[o];
+            const float yv = down_scale ? yj[o] * down_scale[ids[token * n_used + j]] : yj[o];
+            acc += (ma.weight_before ? 1.0f : wts[token * n_used + j]) * yv;
         }
         const size_t i = (size_t)token * ne + row0 + o;
         if (out != add_dst) out[i] = acc;  // an Add in place on this op's dst stores the sum only
@@ -1008,16 +1098,13 @@ __global__ __launch_bounds__(1024) void moe_down_fused_kernel(
 
 // The same activation kept in f32 (in place over g) for a down bank that multiplies raw rows.
 __global__ __launch_bounds__(256) void moe_act_f32_kernel(float* __restrict__ g, const float* __restrict__ u,
-                                                          size_t n_elems) {
+                                                          size_t n_elems, int nff, MoeAct ma,
+                                                          const float* __restrict__ pair_w) {
     const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= n_elems) return;
     const v4f gv = *reinterpret_cast<const v4f*>(g + i), uv = *reinterpret_cast<const v4f*>(u + i);
-    v4f a;
-    a.x = gv.x / (1.0f + expf(-gv.x)) * uv.x;
-    a.y = gv.y / (1.0f + expf(-gv.y)) * uv.y;
-    a.z = gv.z / (1.0f + expf(-gv.z)) * uv.z;
-    a.w = gv.w / (1.0f + expf(-gv.w)) * uv.w;
-    *reinterpret_cast<v4f*>(g + i) = a;
+    const float wp = ma.weight_before ? pair_w[i / (size_t)nff] : 1.0f;
+    *reinterpret_cast<v4f*>(g + i) = moe_gated4(ma, wp, gv, uv);
 }
 
 // `ActsKind::Raw` for any bank format (crates/infr-cpu/src/moe.rs:143-172): the weight row is decoded
@@ -1050,13 +1137,18 @@ __global__ __launch_bounds__(256) void moe_accumulate_kernel(const float* __rest
                                                              const float* __restrict__ wts,
                                                              float* __restrict__ out,
                                                              const float* add_b, float* add_dst,
-                                                             int ne, int n_used, int rows) {
+                                                             int ne, int n_used, int rows, int unit_w,
+                                                             const float* __restrict__ down_scale,
+                                                             const int32_t* __restrict__ ids) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= (size_t)rows * ne) return;
     const size_t r = i / ne, o = i % ne;
     float acc = 0.0f;
-    for (int k = 0; k < n_used; ++k)
-        acc += wts[r * n_used + k] * yp[(r * n_used + k) * ne + o];
+    for (int k = 0; k < n_used; ++k) {
+        // `y = raw * s_e` per pair (lib.rs:2932-2938), then `*o += w_e * y`, w_e = 1.0 under weight_before
+        const float yv = yp[(r * n_used + k) * ne + o];
+        acc += (unit_w ? 1.0f : wts[r * n_used + k]) * (down_scale ? yv * down_scale[ids[r * n_used + k]] : yv);
+    }
     if (out != add_dst) out[i] = acc;  // an Add in place on this op's dst stores the sum only
     if (add_dst) add_dst[i] = acc + add_b[i];
 }
@@ -1171,7 +1263,7 @@ template <typename F>
 static bool launch_moe_down_fused_fmt(const uint8_t* bank, size_t stride, size_t bpr, const int32_t* ids,
                                       const float* wts, const float* g, const float* u, float* out,
                                       const float* add_b, float* add_dst, int nff, int ne, int n_used, int rows,
-                                      hipStream_t stream) {
+                                      const MoeAct& ma, const float* down_scale, hipStream_t stream) {
     const int rps = 16 / (nff / 256);
     int wave_steps = 8;  // rows per workgroup: enough waves in all (as the id-gathered launches size theirs)
     while (wave_steps > 1 && (size_t)((ne + rps * wave_steps - 1) / (rps * wave_steps)) * rows * n_used < 4096)
@@ -1181,17 +1273,18 @@ static bool launch_moe_down_fused_fmt(const uint8_t* bank, size_t stride, size_t
     if (lds > 64 * 1024) return false;
     hipLaunchKernelGGL((moe_down_fused_kernel<F>), dim3((unsigned)((ne + rows_per_wg - 1) / rows_per_wg), (unsigned)rows),
                        dim3((unsigned)(64 * n_used)), lds, stream, bank, stride, bpr, ids, wts, g, u, out, add_b, add_dst,
-                       nff, ne, n_used, rows_per_wg);
+                       nff, ne, n_used, rows_per_wg, ma, down_scale);
     return true;
 }
 static bool launch_moe_down_fused(int dtype, const uint8_t* bank, size_t stride, size_t bpr, const int32_t* ids,
                                   const float* wts, const float* g, const float* u, float* out, const float* add_b,
-                                  float* add_dst, int nff, int ne, int n_used, int rows, hipStream_t stream) {
+                                  float* add_dst, int nff, int ne, int n_used, int rows, const MoeAct& ma,
+                                  const float* down_scale, hipStream_t stream) {
     if (nff > 2048 || nff % 256 != 0 || n_used > 16 || rows > 65535) return false;
     switch (dtype) {
-    case 12: return launch_moe_down_fused_fmt<FmtQ4K>(bank, stride, bpr, ids, wts, g, u, out, add_b, add_dst, nff, ne, n_used, rows, stream);
-    case 13: return launch_moe_down_fused_fmt<FmtQ5K>(bank, stride, bpr, ids, wts, g, u, out, add_b, add_dst, nff, ne, n_used, rows, stream);
-    case 14: return launch_moe_down_fused_fmt<FmtQ6K>(bank, stride, bpr, ids, wts, g, u, out, add_b, add_dst, nff, ne, n_used, rows, stream);
+    case 12: return launch_moe_down_fused_fmt<FmtQ4K>(bank, stride, bpr, ids, wts, g, u, out, add_b, add_dst, nff, ne, n_used, rows, ma, down_scale, stream);
+    case 13: return launch_moe_down_fused_fmt<FmtQ5K>(bank, stride, bpr, ids, wts, g, u, out, add_b, add_dst, nff, ne, n_used, rows, ma, down_scale, stream);
+    case 14: return launch_moe_down_fused_fmt<FmtQ6K>(bank, stride, bpr, ids, wts, g, u, out, add_b, add_dst, nff, ne, n_used, rows, ma, down_scale, stream);
     default: return false;
     }
 }
@@ -1204,7 +1297,7 @@ template <int WT>
 static void launch_row_dots(const void* w, const float* x, float* logits, int ne, int n_rows_w, int rows,
                             bool logits_only, int* tickets, int32_t* sel_idx, float* sel_w, int n_used, float scale,
                             const float* norm_w, float* norm_dst, float norm_eps, float* xt, int xt_q6k,
-                            hipStream_t stream) {
+                            const MoeRoute& rt, hipStream_t stream) {
     // One weight row per workgroup when only logits are wanted of a single row (nothing to wait
     // for); eight at a single row that ends in the selection (few tickets), four once rows fill the
     // pairs; whole rows in one chunk when they fit the LDS a workgroup may have, else kRouterChunk
@@ -1237,19 +1330,19 @@ static void launch_row_dots(const void* w, const float* x, float* logits, int ne
     else if (rows == 1)
         hipLaunchKernelGGL((moe_router_kernel<24, WT>), dim3((unsigned)((n_rows_w + epw - 1) / epw), 1), dim3(256), router_lds,
                            stream, w, x, logits, logits_only ? (int*)nullptr : tickets, sel_idx, sel_w, ne,
-                           n_rows_w, rows, n_used, scale, kc, epw, tpw, norm_w, norm_dst, norm_eps, xt, xt_q6k);
+                           n_rows_w, rows, n_used, scale, kc, epw, tpw, norm_w, norm_dst, norm_eps, xt, xt_q6k, rt);
     else if (whole_rows && router_lds > 64 * 1024)
         hipLaunchKernelGGL((moe_router_kernel<24, WT>),
                            dim3((unsigned)((n_rows_w + epw - 1) / epw), (unsigned)((rows + tpw - 1) / tpw)),
                            dim3(256), router_lds, stream, w, x, logits, (int*)nullptr, sel_idx, sel_w,
                            ne, n_rows_w, rows, n_used, scale, kc, epw, tpw, (const float*)nullptr, (float*)nullptr,
-                           0.0f, (float*)nullptr, 0);
+                           0.0f, (float*)nullptr, 0, rt);
     else
         hipLaunchKernelGGL((moe_router_kernel<8, WT>),
                            dim3((unsigned)((n_rows_w + epw - 1) / epw), (unsigned)((rows + tpw - 1) / tpw)),
                            dim3(256), router_lds, stream, w, x, logits, (int*)nullptr, sel_idx, sel_w,
                            ne, n_rows_w, rows, n_used, scale, kc, epw, tpw, (const float*)nullptr, (float*)nullptr,
-                           0.0f, (float*)nullptr, 0);
+                           0.0f, (float*)nullptr, 0, rt);
 }
 
 // Op::Linear over plain f32 / f16 / bf16 weight rows (crates/infr-cpu/src/lib.rs:1162-1165,
@@ -1258,9 +1351,9 @@ bool launch_linear_plain_rows(int dtype, const void* w, const float* x, float* y
                               hipStream_t stream) {
     if (in_f % 32 != 0 || in_f > (size_t)1 << 30 || out_f > (size_t)1 << 30 || m > (size_t)1 << 30) return false;
     switch (dtype) {
-    case 0: launch_row_dots<0>(w, x, y, (int)in_f, (int)out_f, (int)m, true, nullptr, nullptr, nullptr, 0, 0.0f, nullptr, nullptr, 0.0f, nullptr, 0, stream); break;
-    case 1: launch_row_dots<1>(w, x, y, (int)in_f, (int)out_f, (int)m, true, nullptr, nullptr, nullptr, 0, 0.0f, nullptr, nullptr, 0.0f, nullptr, 0, stream); break;
-    case 30: launch_row_dots<30>(w, x, y, (int)in_f, (int)out_f, (int)m, true, nullptr, nullptr, nullptr, 0, 0.0f, nullptr, nullptr, 0.0f, nullptr, 0, stream); break;
+    case 0: launch_row_dots<0>(w, x, y, (int)in_f, (int)out_f, (int)m, true, nullptr, nullptr, nullptr, 0, 0.0f, nullptr, nullptr, 0.0f, nullptr, 0, MoeRoute{}, stream); break;
+    case 1: launch_row_dots<1>(w, x, y, (int)in_f, (int)out_f, (int)m, true, nullptr, nullptr, nullptr, 0, 0.0f, nullptr, nullptr, 0.0f, nullptr, 0, MoeRoute{}, stream); break;
+    case 30: launch_row_dots<30>(w, x, y, (int)in_f, (int)out_f, (int)m, true, nullptr, nullptr, nullptr, 0, 0.0f, nullptr, nullptr, 0.0f, nullptr, 0, MoeRoute{}, stream); break;
     default: return false;
     }
     return hipGetLastError() == hipSuccess;
@@ -1305,7 +1398,23 @@ size_t moe_workspace_bytes(const MoeShape& s) {
     return n;
 }
 
-const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hipStream_t stream) {
+const char* launch_moe_ffn(const MoeShape& shape, const MoeBuffers& bufs, void* ws, hipStream_t stream) {
+    MoeShape s = shape;
+    MoeBuffers b = bufs;
+    const MoeRoute& rt = s.route;
+    const MoeAct& ma = s.act;
+    if (s.fused_gate_up) {
+        // [gate rows | up rows] inside each expert's slice (graph.rs:936-941): the up bank is the
+        // gate bank from row n_ff of every slice on, same format and expert stride
+        s.up_dtype = s.gate_dtype;
+        b.up_stride = b.gate_stride;
+    }
+    if (ma.act < 0 || ma.act > 2 || rt.gating < 0 || rt.gating > 2) return "unknown activation or gating";
+    if (ma.has_clamp && (ma.act == 2 || ma.weight_before)) return "swiglu_clamp with Sigmoid or weight_before (the CPU arm asserts against it)";
+    if (rt.ids && (rt.bias || rt.n_groups > 1)) return "expert_ids with exp_probs_b or expert groups (the CPU arm asserts against it)";
+    if (rt.n_groups > 1 && rt.n_groups_used > 0 &&
+        (rt.n_groups > 64 || s.n_expert % rt.n_groups != 0 || rt.n_groups_used > rt.n_groups))
+        return "expert groups: n_expert must be a multiple of at most 64 groups, groups_used <= groups";
     if (s.router_dtype != 0 && s.router_dtype != 1 && s.router_dtype != 30) return "router dtype must be F32, F16 or BF16";
     if (b.norm_w && (s.rows != 1 || b.x != b.norm_dst)) return "an absorbed RmsNorm needs a single row read from its dst";
     if (s.n_used > 64 || s.n_expert > 1024 || s.n_used > s.n_expert) return "n_used <= 64 and n_expert <= 1024 required";
@@ -1355,9 +1464,9 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
                            s.ne, s.gate_dtype == 14 ? 1 : 0);
     float* router_xt = router_row_is_x ? xt : nullptr;
     switch (s.router_dtype) {
-    case 0: launch_row_dots<0>(b.router, b.router_x, logits, s.ne, s.n_expert, s.rows, fast1, tickets, sel_idx, sel_w, s.n_used, s.scale, b.norm_w, b.norm_dst, b.norm_eps, router_xt, s.gate_dtype == 14 ? 1 : 0, stream); break;
-    case 1: launch_row_dots<1>(b.router, b.router_x, logits, s.ne, s.n_expert, s.rows, fast1, tickets, sel_idx, sel_w, s.n_used, s.scale, b.norm_w, b.norm_dst, b.norm_eps, router_xt, s.gate_dtype == 14 ? 1 : 0, stream); break;
-    default: launch_row_dots<30>(b.router, b.router_x, logits, s.ne, s.n_expert, s.rows, fast1, tickets, sel_idx, sel_w, s.n_used, s.scale, b.norm_w, b.norm_dst, b.norm_eps, router_xt, s.gate_dtype == 14 ? 1 : 0, stream); break;
+    case 0: launch_row_dots<0>(b.router, b.router_x, logits, s.ne, s.n_expert, s.rows, fast1, tickets, sel_idx, sel_w, s.n_used, s.scale, b.norm_w, b.norm_dst, b.norm_eps, router_xt, s.gate_dtype == 14 ? 1 : 0, rt, stream); break;
+    case 1: launch_row_dots<1>(b.router, b.router_x, logits, s.ne, s.n_expert, s.rows, fast1, tickets, sel_idx, sel_w, s.n_used, s.scale, b.norm_w, b.norm_dst, b.norm_eps, router_xt, s.gate_dtype == 14 ? 1 : 0, rt, stream); break;
+    default: launch_row_dots<30>(b.router, b.router_x, logits, s.ne, s.n_expert, s.rows, fast1, tickets, sel_idx, sel_w, s.n_used, s.scale, b.norm_w, b.norm_dst, b.norm_eps, router_xt, s.gate_dtype == 14 ? 1 : 0, rt, stream); break;
     }
     auto bytes_per_row = [](int dtype, size_t in_f) -> size_t {
         switch (dtype) {
@@ -1378,6 +1487,8 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     const size_t gbpr = bytes_per_row(s.gate_dtype, s.ne), ubpr = bytes_per_row(s.up_dtype, s.ne);
     const size_t dbpr = bytes_per_row(s.down_dtype, s.n_ff);
     if (!gbpr || !ubpr || !dbpr) return "expert bank format has no kernel";
+    if (s.fused_gate_up) b.up = b.gate + (size_t)s.n_ff * gbpr;
+    const int unit_w = ma.weight_before ? 1 : 0;
     // expert_acts_kind (moe.rs:42-53) with whole-256 rows: per-256 int8 activations (Super) for the
     // K-quants and Q8_0, per-32 (Blk32) for Q5_0, f32 rows (Raw) for everything else - and for
     // every bank when there is a single row (int8_ok = rows >= 2, lib.rs:2359).
@@ -1397,7 +1508,7 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     if (s.rows > 1)
         hipLaunchKernelGGL(moe_select_kernel, dim3((unsigned)s.rows), dim3(256), 0, stream, logits, sel_idx,
                            sel_w, s.n_expert, s.n_used, s.scale, quant_in_select ? b.x : (const float*)nullptr,
-                           s.ne, aq.qs, aq.d, aq.bsums, aq.bsums16);
+                           s.ne, aq.qs, aq.d, aq.bsums, aq.bsums16, rt);
     auto export_selection = [&] {
         if (b.sel_idx) (void)hipMemcpyAsync(b.sel_idx, sel_idx, pairs * 4, hipMemcpyDeviceToDevice, stream);
         if (b.sel_w) (void)hipMemcpyAsync(b.sel_w, sel_w, pairs * 4, hipMemcpyDeviceToDevice, stream);
@@ -1412,10 +1523,10 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
             launch_raw(s.up_dtype, b.up, b.up_stride, ubpr, b.x, s.n_used, s.ne, ubuf, s.n_ff);
             const size_t n_act1 = pairs * s.n_ff;
             hipLaunchKernelGGL(moe_act_f32_kernel, dim3((unsigned)((n_act1 / 4 + 255) / 256)), dim3(256), 0, stream,
-                               gbuf, ubuf, n_act1);
+                               gbuf, ubuf, n_act1, s.n_ff, ma, sel_w);
             launch_raw(s.down_dtype, b.down, b.down_stride, dbpr, gbuf, 1, s.n_ff, yp, s.ne);
             hipLaunchKernelGGL(moe_accumulate_kernel, dim3((unsigned)((s.ne + 255) / 256)), dim3(256), 0, stream, yp,
-                               sel_w, b.dst, b.add_b, b.add_dst, s.ne, s.n_used, s.rows);
+                               sel_w, b.dst, b.add_b, b.add_dst, s.ne, s.n_used, s.rows, unit_w, b.down_scale, sel_idx);
             return hipGetLastError() == hipSuccess ? nullptr : "kernel launch failed";
         }
         // row steps per wave: amortise the 64 activation registers while keeping >= ~1024 waves
@@ -1439,7 +1550,7 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
 #define INFR_GATE_UP_N(P, N)                                                                                  \
     hipLaunchKernelGGL((moe_gate_up_f32_kernel<P, N>), grid_g, dim3(256), 0, stream, b.gate, b.up, b.gate_stride, \
                        b.up_stride, logits, s.n_expert, s.n_used, s.scale, sel_idx, sel_w, xt, gbuf, s.ne, s.n_ff, \
-                       lanes_g, chunks_g, s.down_dtype == 14 ? 1 : 0)
+                       lanes_g, chunks_g, s.down_dtype == 14 ? 1 : 0, rt, ma)
 #define INFR_GATE_UP(P)                 \
     switch (spw) {                      \
     case 1: INFR_GATE_UP_N(P, 1); break; \
@@ -1463,7 +1574,7 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
 #define INFR_DOWN_N(P, N)                                                                                   \
     hipLaunchKernelGGL((moe_down_f32_kernel<P, N>), grid_d, dim3((unsigned)(64 * nw_d)), 0, stream, b.down,   \
                        b.down_stride, sel_idx, sel_w, gbuf, b.dst, b.add_b, b.add_dst, s.n_ff, s.ne, s.n_used, \
-                       lanes_d, chunks_d)
+                       lanes_d, chunks_d, unit_w, b.down_scale)
 #define INFR_DOWN(P)                 \
     switch (spw_d) {                 \
     case 1: INFR_DOWN_N(P, 1); break; \
@@ -1531,18 +1642,18 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
     // a few rows: activation, down projection and the sum over a token's experts in one launch
     if (kd == kSuper && !(bucketed && has_mfma(s.down_dtype)) &&
         launch_moe_down_fused(s.down_dtype, b.down, b.down_stride, dbpr, sel_idx, sel_w, gbuf, ubuf, b.dst, b.add_b,
-                              b.add_dst, s.n_ff, s.ne, s.n_used, s.rows, stream))
+                              b.add_dst, s.n_ff, s.ne, s.n_used, s.rows, ma, b.down_scale, stream))
         return hipGetLastError() == hipSuccess ? nullptr : "kernel launch failed";
     // act = silu(g) * u in the form the down bank multiplies: per-256 codes, per-32 codes, or f32
     if (kd == kSuper)
         hipLaunchKernelGGL(moe_act_quant_kernel<false>, dim3((unsigned)((n_act / 256 + 3) / 4)), dim3(256), 0, stream,
-                           gbuf, ubuf, aq.qs, aq.d, aq.bsums, aq.bsums16, n_act);
+                           gbuf, ubuf, aq.qs, aq.d, aq.bsums, aq.bsums16, n_act, s.n_ff, ma, sel_w);
     else if (kd == kBlk32)
         hipLaunchKernelGGL(moe_act_quant_kernel<true>, dim3((unsigned)((n_act / 256 + 3) / 4)), dim3(256), 0, stream,
-                           gbuf, ubuf, aq32.qs, aq32.d, aq32.bsums, (int32_t*)nullptr, n_act);
+                           gbuf, ubuf, aq32.qs, aq32.d, aq32.bsums, (int32_t*)nullptr, n_act, s.n_ff, ma, sel_w);
     else
         hipLaunchKernelGGL(moe_act_f32_kernel, dim3((unsigned)((n_act / 4 + 255) / 256)), dim3(256), 0, stream, gbuf,
-                           ubuf, n_act);
+                           ubuf, n_act, s.n_ff, ma, sel_w);
     // the down projection's activation row is the pair itself: n_used = 1
     if (kd == kRaw)
         launch_raw(s.down_dtype, b.down, b.down_stride, dbpr, gbuf, 1, s.n_ff, yp, s.ne);
@@ -1552,7 +1663,7 @@ const char* launch_moe_ffn(const MoeShape& s, const MoeBuffers& b, void* ws, hip
                              (int)pairs, yp, s.ne, stream))
         return "no id-gathered kernel for this down shape";
     hipLaunchKernelGGL(moe_accumulate_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, stream,
-                       yp, sel_w, b.dst, b.add_b, b.add_dst, s.ne, s.n_used, s.rows);
+                       yp, sel_w, b.dst, b.add_b, b.add_dst, s.ne, s.n_used, s.rows, unit_w, b.down_scale, sel_idx);
     return hipGetLastError() == hipSuccess ? nullptr : "kernel launch failed";
 }
 

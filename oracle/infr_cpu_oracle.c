@@ -947,13 +947,35 @@ static int expert_gemm(const uint8_t *wbytes, size_t wlen, int dt, size_t in_f, 
     return -1;
 }
 
+/* Stable descending order of v[0..n): `idx.sort_by(|a, b| v[b].partial_cmp(&v[a]).unwrap())`
+ * (lib.rs:2509, 2528) — ties keep the lower index first. Selection sort over the first `take`. */
+static void top_desc_stable(const float *v, size_t n, size_t take, size_t *out, char *taken) {
+    memset(taken, 0, n);
+    for (size_t k = 0; k < take; k++) {
+        size_t best = n;
+        for (size_t e = 0; e < n; e++) {
+            if (taken[e]) continue;
+            if (best == n || v[e] > v[best]) best = e;
+        }
+        taken[best] = 1;
+        out[k] = best;
+    }
+}
+
 int orc_moe_ffn(const orc_moe_params *p, const float *x, const float *router_x,
                 const uint8_t *router, size_t router_bytes, const uint8_t *gate, size_t gate_bytes,
                 const uint8_t *up, size_t up_bytes, const uint8_t *down, size_t down_bytes,
-                float *y, int32_t *sel_idx, float *sel_w, int threads) {
+                float *y, int32_t *sel_idx, float *sel_w, int threads, const float *down_scale,
+                const float *exp_probs_b, const int32_t *expert_ids) {
     size_t ne = p->ne, n_expert = p->n_expert, n_used = p->n_used, nffx = p->n_ff_exp;
     size_t rows = p->rows;
     if (!ne || !n_expert || !n_used || !nffx || !rows || n_used > n_expert) return -2;
+    /* the two assertions in front of the arm (lib.rs:2293-2309) */
+    if (p->has_clamp && (p->act == ORC_ACT_SIGMOID || p->weight_before)) return -3;
+    if (expert_ids && (exp_probs_b || p->n_expert_groups > 1)) return -3;
+    if (p->n_expert_groups > 1 && p->n_expert_groups_used > 0 &&
+        (n_expert % p->n_expert_groups != 0 || p->n_expert_groups_used > p->n_expert_groups))
+        return -2;
 #ifdef _OPENMP
     int nt = threads > 0 ? threads : omp_get_max_threads();
 #else
@@ -961,7 +983,11 @@ int orc_moe_ffn(const orc_moe_params *p, const float *x, const float *router_x,
     (void)threads;
 #endif
     (void)nt;
-    size_t gst = gate_bytes / n_expert, ust = up_bytes / n_expert, dst_ = down_bytes / n_expert;
+    /* lib.rs:2340-2348: fused banks hold gate rows then up rows inside each expert's slice */
+    size_t gst = gate_bytes / n_expert, dst_ = down_bytes / n_expert;
+    size_t ust = p->fused_gate_up ? 0 : up_bytes / n_expert;
+    int udt = p->fused_gate_up ? p->gate_dtype : p->up_dtype;
+    size_t out_gu = p->fused_gate_up ? 2 * nffx : nffx;
     /* lib.rs:2359 */
     int int8_ok = rows >= 2 && !p->reference_mode;
     int rc = 0;
@@ -974,51 +1000,101 @@ int orc_moe_ffn(const orc_moe_params *p, const float *x, const float *router_x,
         return -1;
     }
 
-    /* Per-row softmax + stable top-k + renormalised weights (lib.rs:2421-2543). */
+    /* Per-row gating + selection + weights (lib.rs:2421-2543). */
     size_t *idx = (size_t *)malloc(sizeof(size_t) * rows * n_used);
     float *wts = (float *)malloc(sizeof(float) * rows * n_used);
     float *probs = (float *)malloc(sizeof(float) * n_expert);
+    float *selp = (float *)malloc(sizeof(float) * n_expert);
     char *taken = (char *)malloc(n_expert);
-    for (size_t r = 0; r < rows; r++) {
-        float maxl = -INFINITY;
-        for (size_t e = 0; e < n_expert; e++) {
-            float v = lt[e * rows + r];
-            maxl = v > maxl ? v : maxl;
-        }
-        float psum = 0.0f;
-        for (size_t e = 0; e < n_expert; e++) {
-            probs[e] = expf(lt[e * rows + r] - maxl);
-        }
-        for (size_t e = 0; e < n_expert; e++) psum += probs[e];
-        for (size_t e = 0; e < n_expert; e++) probs[e] /= psum;
-        /* stable descending sort, truncated: ties keep the lower expert index first */
-        memset(taken, 0, n_expert);
-        for (size_t k = 0; k < n_used; k++) {
-            size_t best = n_expert;
+    for (size_t r = 0; r < rows && rc == 0; r++) {
+        if (p->gating == ORC_GATING_SIGMOID) { /* :2437-2439 */
+            for (size_t e = 0; e < n_expert; e++) probs[e] = 1.0f / (1.0f + expf(-lt[e * rows + r]));
+        } else if (p->gating == ORC_GATING_SQRT_SOFTPLUS) { /* :2440-2454 */
             for (size_t e = 0; e < n_expert; e++) {
-                if (taken[e]) continue;
-                if (best == n_expert || probs[e] > probs[best]) best = e;
+                float v = lt[e * rows + r];
+                float sp = v > 20.0f ? v : logf(1.0f + expf(v));
+                probs[e] = sqrtf(sp);
             }
-            taken[best] = 1;
-            idx[r * n_used + k] = best;
+        } else { /* softmax, :2427-2436 */
+            float maxl = -INFINITY;
+            for (size_t e = 0; e < n_expert; e++) {
+                float v = lt[e * rows + r];
+                maxl = v > maxl ? v : maxl;
+            }
+            float psum = 0.0f;
+            for (size_t e = 0; e < n_expert; e++) probs[e] = expf(lt[e * rows + r] - maxl);
+            for (size_t e = 0; e < n_expert; e++) psum += probs[e];
+            for (size_t e = 0; e < n_expert; e++) probs[e] /= psum;
         }
+        if (expert_ids) { /* hash routing: the ids are the selection, in their own order (:2456-2472) */
+            for (size_t k = 0; k < n_used; k++) {
+                int32_t e = expert_ids[r * n_used + k];
+                if (e < 0 || (size_t)e >= n_expert) {
+                    rc = -4;
+                    break;
+                }
+                idx[r * n_used + k] = (size_t)e;
+            }
+            if (rc) break;
+        } else {
+            /* selection-only copy: bias (:2476-2485), then group masking (:2488-2526) */
+            for (size_t e = 0; e < n_expert; e++) selp[e] = exp_probs_b ? probs[e] + exp_probs_b[e] : probs[e];
+            if (p->n_expert_groups > 1 && p->n_expert_groups_used > 0) {
+                size_t ng = p->n_expert_groups, per = n_expert / ng, ng_used = p->n_expert_groups_used;
+                float *gscores = (float *)malloc(sizeof(float) * ng);
+                size_t *gidx = (size_t *)malloc(sizeof(size_t) * ng);
+                char *gtaken = (char *)malloc(ng);
+                for (size_t g = 0; g < ng; g++) {
+                    float best0 = -INFINITY, best1 = -INFINITY;
+                    for (size_t i = 0; i < per; i++) {
+                        float sv = selp[g * per + i];
+                        if (sv > best0) {
+                            best1 = best0;
+                            best0 = sv;
+                        } else if (sv > best1) {
+                            best1 = sv;
+                        }
+                    }
+                    gscores[g] = best0 + best1;
+                }
+                top_desc_stable(gscores, ng, ng_used, gidx, gtaken);
+                memset(gtaken, 0, ng);
+                for (size_t k = 0; k < ng_used; k++) gtaken[gidx[k]] = 1;
+                for (size_t g = 0; g < ng; g++)
+                    if (!gtaken[g])
+                        for (size_t i = 0; i < per; i++) selp[g * per + i] = -INFINITY;
+                free(gscores);
+                free(gidx);
+                free(gtaken);
+            }
+            top_desc_stable(selp, n_expert, n_used, idx + r * n_used, taken);
+        }
+        /* weights from the unbiased probs (:2536-2541) */
         float wsum = 0.0f;
         for (size_t k = 0; k < n_used; k++) wsum += probs[idx[r * n_used + k]];
         wsum = wsum > 1e-20f ? wsum : 1e-20f;
         for (size_t k = 0; k < n_used; k++) {
-            wts[r * n_used + k] = probs[idx[r * n_used + k]] / wsum * p->scale;
+            float pe = probs[idx[r * n_used + k]];
+            wts[r * n_used + k] = p->norm_w ? pe / wsum * p->scale : pe * p->scale;
             if (sel_idx) sel_idx[r * n_used + k] = (int32_t)idx[r * n_used + k];
             if (sel_w) sel_w[r * n_used + k] = wts[r * n_used + k];
         }
     }
     free(probs);
+    free(selp);
     free(taken);
     free(lt);
+    if (rc) {
+        free(idx);
+        free(wts);
+        return rc;
+    }
 
     /* Buckets: (row -> expert) pairs grouped by expert, rows ascending inside a bucket
-     * (lib.rs:2554-2587). */
+     * (lib.rs:2554-2587). pair_w = the pair's routing weight (weight_before folds it into stage C). */
     size_t n_pairs = rows * n_used;
     size_t *pair_row = (size_t *)malloc(sizeof(size_t) * n_pairs);
+    float *pair_w = (float *)malloc(sizeof(float) * n_pairs);
     size_t *slot_pair = (size_t *)malloc(sizeof(size_t) * n_pairs); /* [r][rank] */
     size_t *bucket_e = (size_t *)malloc(sizeof(size_t) * n_expert);
     size_t *bucket_p0 = (size_t *)malloc(sizeof(size_t) * (n_expert + 1));
@@ -1029,6 +1105,7 @@ int orc_moe_ffn(const orc_moe_params *p, const float *x, const float *router_x,
             for (size_t k = 0; k < n_used; k++)
                 if (idx[r * n_used + k] == e) {
                     slot_pair[r * n_used + k] = np;
+                    pair_w[np] = wts[r * n_used + k];
                     pair_row[np++] = r;
                 }
         if (np > p0) {
@@ -1040,7 +1117,7 @@ int orc_moe_ffn(const orc_moe_params *p, const float *x, const float *router_x,
     bucket_p0[n_buckets] = np;
 
     int g_kind = orc_expert_acts_kind(p->gate_dtype, ne, int8_ok);
-    int u_kind = orc_expert_acts_kind(p->up_dtype, ne, int8_ok);
+    int u_kind = p->fused_gate_up ? g_kind : orc_expert_acts_kind(udt, ne, int8_ok);
     int d_kind = orc_expert_acts_kind(p->down_dtype, nffx, int8_ok);
     float *y_pairs = (float *)calloc(n_pairs * ne, sizeof(float));
 
@@ -1052,42 +1129,50 @@ int orc_moe_ffn(const orc_moe_params *p, const float *x, const float *router_x,
         float *xin = (float *)malloc(sizeof(float) * count * ne);
         for (size_t i = 0; i < count; i++)
             memcpy(xin + i * ne, x + pair_row[p0 + i] * ne, sizeof(float) * ne);
-        float *gt = (float *)malloc(sizeof(float) * nffx * count);
-        float *ut = (float *)malloc(sizeof(float) * nffx * count);
+        float *gt = (float *)malloc(sizeof(float) * out_gu * count);
+        float *ut = p->fused_gate_up ? gt + nffx * count : (float *)malloc(sizeof(float) * nffx * count);
         float *act = (float *)malloc(sizeof(float) * count * nffx);
         float *dt_ = (float *)malloc(sizeof(float) * ne * count);
-        int e1 = expert_gemm(gate + e * gst, gst, p->gate_dtype, ne, nffx, g_kind, xin, count, gt);
-        int e2 = expert_gemm(up + e * ust, ust, p->up_dtype, ne, nffx, u_kind, xin, count, ut);
-        /* Stage C (lib.rs:2824-2892): gated_act_fn(Silu, None, 1.0*g, 1.0*u) */
-        for (size_t i = 0; i < count; i++)
+        int e1 = expert_gemm(gate + e * gst, gst, p->gate_dtype, ne, out_gu, g_kind, xin, count, gt);
+        int e2 = p->fused_gate_up ? 0 : expert_gemm(up + e * ust, ust, udt, ne, nffx, u_kind, xin, count, ut);
+        /* Stage C (lib.rs:2824-2861): gated_act_fn(act, clamp, wp * g, wp * u), wp = the pair's
+         * routing weight under weight_before, else 1.0 */
+        for (size_t i = 0; i < count; i++) {
+            float wp = p->weight_before ? pair_w[p0 + i] : 1.0f;
             for (size_t f = 0; f < nffx; f++)
-                act[i * nffx + f] = orc_silu(gt[f * count + i]) * ut[f * count + i];
+                act[i * nffx + f] = orc_gated_act(p->act, p->has_clamp, p->clamp, wp * gt[f * count + i],
+                                                  wp * ut[f * count + i]);
+        }
         int e3 = expert_gemm(down + e * dst_, dst_, p->down_dtype, nffx, ne, d_kind, act, count, dt_);
         if (e1 || e2 || e3) {
 #pragma omp atomic write
             rc = -1;
         }
+        /* un-transpose with the per-expert down_scale folded in (lib.rs:2926-2945) */
         for (size_t i = 0; i < count; i++)
-            for (size_t d = 0; d < ne; d++) y_pairs[(p0 + i) * ne + d] = dt_[d * count + i];
+            for (size_t d = 0; d < ne; d++)
+                y_pairs[(p0 + i) * ne + d] = down_scale ? dt_[d * count + i] * down_scale[e] : dt_[d * count + i];
         free(xin);
         free(gt);
-        free(ut);
+        if (!p->fused_gate_up) free(ut);
         free(act);
         free(dt_);
     }
 
-    /* Stage E (lib.rs:2967-2983): rank order, `*o += w_e * yv` (separate multiply and add). */
+    /* Stage E (lib.rs:2967-2983): rank order, `*o += w_e * yv` (separate multiply and add);
+     * under weight_before the weight is already inside the activation and w_e = 1.0. */
     for (size_t r = 0; r < rows; r++) {
         float *orow = y + r * ne;
         for (size_t d = 0; d < ne; d++) orow[d] = 0.0f;
         for (size_t k = 0; k < n_used; k++) {
-            float w_e = wts[r * n_used + k];
+            float w_e = p->weight_before ? 1.0f : wts[r * n_used + k];
             const float *yp = y_pairs + slot_pair[r * n_used + k] * ne;
             for (size_t d = 0; d < ne; d++) orow[d] += w_e * yp[d];
         }
     }
     free(y_pairs);
     free(pair_row);
+    free(pair_w);
     free(slot_pair);
     free(bucket_e);
     free(bucket_p0);

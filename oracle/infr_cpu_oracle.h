@@ -175,22 +175,39 @@ void orc_ref_linear_f64(const float *x, const float *w, size_t m, size_t in_f, s
 /* crates/infr-cpu/src/moe.rs:42-53 */
 int orc_expert_acts_kind(int dtype, size_t in_f, int int8_ok);
 
-/* Op::MoeFfn as qwen3moe builds it (crates/infr-llama/src/seam/runner.rs:3971-3997): softmax
- * gating, norm_w, weight on the output side, split gate/up banks, SiLU, no clamp/bias/groups. */
+/* Op::MoeFfn with every field of the op (crates/infr-core/src/graph.rs:918-1011). qwen3moe builds it
+ * with softmax gating, norm_w, weight on the output side, split gate/up banks, SiLU and none of the
+ * optional operands (crates/infr-llama/src/seam/runner.rs:3971-3997); a zeroed tail plus norm_w = 1
+ * is that setting. ep_band is not restated: the CPU arm ignores it (lib.rs:2283). */
+#define ORC_GATING_SOFTMAX 0
+#define ORC_GATING_SIGMOID 1
+#define ORC_GATING_SQRT_SOFTPLUS 2
 typedef struct {
     uint32_t ne, n_expert, n_used, n_ff_exp, rows;
     float scale;
     int router_dtype, gate_dtype, up_dtype, down_dtype;
     int reference_mode;
+    int act;            /* ORC_ACT_* */
+    int gating;         /* ORC_GATING_* */
+    int norm_w;         /* 1: w = p / max(sum_sel p, 1e-20) * scale; 0: w = p * scale */
+    int weight_before;  /* 1: the routing weight multiplies gate and up before the activation */
+    int fused_gate_up;  /* 1: `gate` holds [gate rows | up rows] per expert; `up` is not read */
+    int has_clamp;      /* swiglu_clamp = Some(clamp) */
+    float clamp;
+    uint32_t n_expert_groups, n_expert_groups_used;
 } orc_moe_params;
 
 /* crates/infr-cpu/src/lib.rs:2264-2984. x, router_x: [rows, ne] f32. Banks: expert e is the e-th
  * equal byte slice. y[rows*ne]. sel_idx/sel_w (optional, [rows*n_used]) receive the routing
- * (descending-probability order). Returns 0 or negative on unsupported input. */
+ * (descending-probability order, or the supplied ids' order). Optional operands, NULL when the op
+ * has None: down_scale f32 [n_expert], exp_probs_b f32 [n_expert], expert_ids i32 [rows*n_used].
+ * Returns 0, or negative on unsupported input and on the combinations the CPU arm asserts against
+ * (a clamp with Sigmoid or weight_before; expert_ids with a bias or groups; an id >= n_expert). */
 int orc_moe_ffn(const orc_moe_params *p, const float *x, const float *router_x,
                 const uint8_t *router, size_t router_bytes, const uint8_t *gate, size_t gate_bytes,
                 const uint8_t *up, size_t up_bytes, const uint8_t *down, size_t down_bytes,
-                float *y, int32_t *sel_idx, float *sel_w, int threads);
+                float *y, int32_t *sel_idx, float *sel_w, int threads, const float *down_scale,
+                const float *exp_probs_b, const int32_t *expert_ids);
 
 /* Test-input recipes the reference's own tests use (inputs only; it stores no expected outputs).
  * crates/infr-testkit/src/lib.rs:49-56 */

@@ -90,11 +90,16 @@ class _MoeParams(C.Structure):
     _fields_ = [("ne", C.c_uint32), ("n_expert", C.c_uint32), ("n_used", C.c_uint32),
                 ("n_ff_exp", C.c_uint32), ("rows", C.c_uint32), ("scale", C.c_float),
                 ("router_dtype", C.c_int), ("gate_dtype", C.c_int), ("up_dtype", C.c_int),
-                ("down_dtype", C.c_int), ("reference_mode", C.c_int)]
+                ("down_dtype", C.c_int), ("reference_mode", C.c_int),
+                ("act", C.c_int), ("gating", C.c_int), ("norm_w", C.c_int), ("weight_before", C.c_int),
+                ("fused_gate_up", C.c_int), ("has_clamp", C.c_int), ("clamp", C.c_float),
+                ("n_expert_groups", C.c_uint32), ("n_expert_groups_used", C.c_uint32)]
 
+
+GATING_SOFTMAX, GATING_SIGMOID, GATING_SQRT_SOFTPLUS = 0, 1, 2
 
 _moe = _sig("orc_moe_ffn", C.c_int, C.POINTER(_MoeParams), _f32p, _f32p, _u8p, C.c_size_t, _u8p,
-            C.c_size_t, _u8p, C.c_size_t, _u8p, C.c_size_t, _f32p, _i32p, _f32p, C.c_int)
+            C.c_size_t, _u8p, C.c_size_t, _u8p, C.c_size_t, _f32p, _i32p, _f32p, C.c_int, _f32p, _f32p, _i32p)
 
 
 def _c(a, dt):
@@ -339,7 +344,12 @@ def expert_acts_kind(dtype: int, in_f: int, int8_ok: bool) -> int:
 def moe_ffn(x, router, gate, up, down, *, ne: int, n_expert: int, n_used: int, n_ff_exp: int,
             scale: float = 1.0, router_dtype: int = F32, gate_dtype: int = Q4_K,
             up_dtype: int = Q4_K, down_dtype: int = Q4_K, router_x=None,
-            reference_mode: bool = False, threads: int = 0):
+            reference_mode: bool = False, threads: int = 0, act: int = 0, gating: int = 0,
+            norm_w: bool = True, weight_before: bool = False, fused_gate_up: bool = False,
+            swiglu_clamp=None, n_expert_groups: int = 0, n_expert_groups_used: int = 0,
+            down_scale=None, exp_probs_b=None, expert_ids=None):
+    """Op::MoeFfn on the CPU oracle; the keyword defaults are qwen3moe's setting. With
+    ``fused_gate_up`` the ``gate`` bank holds gate rows then up rows per expert and ``up`` is ignored."""
     x = _c(x, np.float32).ravel()
     rows = x.size // ne
     rx = x if router_x is None else _c(router_x, np.float32).ravel()
@@ -347,15 +357,21 @@ def moe_ffn(x, router, gate, up, down, *, ne: int, n_expert: int, n_used: int, n
         a = np.ascontiguousarray(a)
         return a.view(np.uint8).ravel()
 
-    router, gate, up, down = raw(router), raw(gate), raw(up), raw(down)
+    router, gate, down = raw(router), raw(gate), raw(down)
+    up = gate if fused_gate_up or up is None else raw(up)
     p = _MoeParams(ne, n_expert, n_used, n_ff_exp, rows, scale, router_dtype, gate_dtype, up_dtype,
-                   down_dtype, int(reference_mode))
+                   down_dtype, int(reference_mode), act, gating, int(norm_w), int(weight_before),
+                   int(fused_gate_up), int(swiglu_clamp is not None), float(swiglu_clamp or 0.0),
+                   n_expert_groups, n_expert_groups_used)
+    ds = None if down_scale is None else _c(down_scale, np.float32).ravel()
+    eb = None if exp_probs_b is None else _c(exp_probs_b, np.float32).ravel()
+    ids = None if expert_ids is None else _c(expert_ids, np.int32).ravel()
     y = np.empty(rows * ne, np.float32)
     idx = np.empty(rows * n_used, np.int32)
     w = np.empty(rows * n_used, np.float32)
     rc = _moe(C.byref(p), _p(x, _f32p), _p(rx, _f32p), _p(router, _u8p), router.size,
               _p(gate, _u8p), gate.size, _p(up, _u8p), up.size, _p(down, _u8p), down.size,
-              _p(y, _f32p), _p(idx, _i32p), _p(w, _f32p), threads)
+              _p(y, _f32p), _p(idx, _i32p), _p(w, _f32p), threads, _p(ds, _f32p), _p(eb, _f32p), _p(ids, _i32p))
     if rc != 0:
         raise ValueError(f"oracle moe_ffn failed rc={rc}")
     return y.reshape(rows, ne), idx.reshape(rows, n_used), w.reshape(rows, n_used)

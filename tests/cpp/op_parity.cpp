@@ -258,17 +258,45 @@ static void hip_moe_ffn_matches_the_cpu_arm(HipBackend& be) {
         const TensorId uid = g.weight({{n_expert, nff, ne}, DType::Q4K});
         const TensorId did = g.weight({{n_expert, ne, nff}, DType::Q6K});
         const TensorId dst = g.output({{rows, ne}, DType::F32});
-        g.push(op::MoeFfn{xid, xid, rid, gid, uid, did, dst, ne, n_expert, n_used, nff, 1.0f});
-        const std::vector<float> got = run_graph(
-            be, g, {{xid, f32_bytes(x)}, {rid, f32_bytes(router)}, {gid, gate_w}, {uid, up_w}, {did, down_w}}, dst,
-            (size_t)rows * ne);
-        orc_moe_params p{ne, n_expert, n_used, nff, rows, 1.0f, 0, 12, 12, 14, 0};
-        std::vector<float> want((size_t)rows * ne);
-        const int rc = orc_moe_ffn(&p, x.data(), x.data(), (const uint8_t*)router.data(), router.size() * 4,
-                                   gate_w.data(), gate_w.size(), up_w.data(), up_w.size(), down_w.data(),
-                                   down_w.size(), want.data(), nullptr, nullptr, 0);
-        EXPECT(rc == 0, "oracle MoeFfn rc %d", rc);
-        gate(rows == 1 ? "MoeFfn rows=1" : "MoeFfn rows=4", got, want);
+        // qwen3moe's setting, then llama4's (sigmoid gating, raw weights, weight on the expert input;
+        // graph.rs:956-967) with a GELU expert
+        for (int variant = 0; variant < 2; ++variant) {
+            op::MoeFfn moe{xid, xid, rid, gid, uid, did, dst, ne, n_expert, n_used, nff, 1.0f};
+            orc_moe_params p{};
+            p.ne = ne; p.n_expert = n_expert; p.n_used = n_used; p.n_ff_exp = nff; p.rows = rows; p.scale = 1.0f;
+            p.router_dtype = 0; p.gate_dtype = 12; p.up_dtype = 12; p.down_dtype = 14; p.norm_w = 1;
+            if (variant == 1) {
+                moe.gating = MoeGating::Sigmoid; moe.norm_w = false; moe.weight_before = true; moe.act = Activation::Gelu;
+                p.gating = ORC_GATING_SIGMOID; p.norm_w = 0; p.weight_before = 1; p.act = ORC_ACT_GELU;
+            }
+            Graph gv = g;
+            gv.push(moe);
+            const std::vector<float> got = run_graph(
+                be, gv, {{xid, f32_bytes(x)}, {rid, f32_bytes(router)}, {gid, gate_w}, {uid, up_w}, {did, down_w}}, dst,
+                (size_t)rows * ne);
+            std::vector<float> want((size_t)rows * ne);
+            const int rc = orc_moe_ffn(&p, x.data(), x.data(), (const uint8_t*)router.data(), router.size() * 4,
+                                       gate_w.data(), gate_w.size(), up_w.data(), up_w.size(), down_w.data(),
+                                       down_w.size(), want.data(), nullptr, nullptr, 0, nullptr, nullptr, nullptr);
+            EXPECT(rc == 0, "oracle MoeFfn rc %d", rc);
+            gate(variant ? (rows == 1 ? "MoeFfn llama4-style rows=1" : "MoeFfn llama4-style rows=4")
+                         : (rows == 1 ? "MoeFfn rows=1" : "MoeFfn rows=4"), got, want);
+        }
+        // an expert-parallel band is another GPU's business: refused, never read as the whole bank
+        {
+            op::MoeFfn moe{xid, xid, rid, gid, uid, did, dst, ne, n_expert, n_used, nff, 1.0f};
+            moe.ep_band = std::make_pair(0u, 8u);
+            Graph gv = g;
+            gv.push(moe);
+            bool refused = false;
+            try {
+                (void)run_graph(be, gv, {{xid, f32_bytes(x)}, {rid, f32_bytes(router)}, {gid, gate_w}, {uid, up_w}, {did, down_w}},
+                                dst, (size_t)rows * ne);
+            } catch (const Error& e) {
+                refused = e.kind == ErrorKind::Unsupported;
+            }
+            EXPECT(refused, "MoeFfn with ep_band must be Unsupported");
+        }
     }
 }
 

@@ -714,3 +714,41 @@ def test_combined_gate_up_activation_rides_in_the_small_batch_quantizer(be, m):
         got = be.download(dnb, np.empty((m, H), np.float32))
         assert np.array_equal(bits(got), bits(orc.linear(DType.Q5K, wd, got_act, m, FF, H).reshape(m, H)))
     assert plan.launches() == 2
+
+
+@pytest.mark.parametrize("wide_first", [False, True])
+@pytest.mark.parametrize("shared_x", [True, False])
+def test_small_and_large_batch_ops_of_one_shape_class_on_one_level(be, wide_first, shared_x):
+    """Whether a batch counts as small depends on out_f as well (Q4_K at 33..128 tokens: a 1024-row matrix
+    takes the 16-token K-split kernel, a 12288-row one the 32-token tiles). Two such Linears of one dtype,
+    row length and token count on one level: the narrow one runs in a small-batch group, the wide one alone,
+    whichever comes first; with distinct activations the group's scratch is sized when it is scheduled."""
+    m, in_f = 48, 4096
+    shapes = [(1024, 70), (12288, 71)]
+    if wide_first:
+        shapes.reverse()
+    g, binds = Graph(), Bindings()
+    xs, ws, ybs = [], [], []
+    for i, (out_f, seed) in enumerate(shapes):
+        if i == 0 or not shared_x:
+            x = synth_normal_f32(80 + i, m * in_f)
+            xid = g.input(TensorDesc((m, in_f), DType.F32))
+            binds.bind(xid, be.upload_new(x))
+        xs.append(x)
+        w = synth_weight(DType.Q4K, seed, out_f, in_f)
+        ws.append(w)
+        wid = g.weight(TensorDesc((out_f, in_f), DType.Q4K))
+        yid = g.output(TensorDesc((m, out_f), DType.F32))
+        yb = be.alloc(m * out_f * 4)
+        ybs.append(yb)
+        binds.bind(wid, be.upload_new(w)).bind(yid, yb)
+        g.push(Linear(xid, wid, yid, m, in_f, out_f))
+    plan = be.compile(g)
+    for _ in range(2):
+        be.execute(plan, binds)
+        for (out_f, _), x, w, yb in zip(shapes, xs, ws, ybs):
+            got = be.download(yb, np.empty((m, out_f), np.float32))
+            rows = 64                                                # sampled weight rows against the oracle
+            for row0 in (0, out_f - rows):
+                want = orc.linear(DType.Q4K, w[row0 * 2304:(row0 + rows) * 2304], x, m, in_f, rows)
+                assert np.array_equal(bits(got[:, row0:row0 + rows]), bits(want)), (out_f, row0)

@@ -165,3 +165,28 @@ def test_rust_mirror_structs_match_the_c_header(tmp_path, rust, ctype):
     ct = {"HipOp": B._Op, "HipMoe": B._MoeParams, "HipCaps": B._Caps}[rust]
     assert [f[0] for f in ct._fields_] == list(offsets)
     assert ctypes.sizeof(ct) == size
+
+
+def test_shim_moe_arm_names_every_field_of_the_op():
+    """The shim's `Op::MoeFfn { .. }` pattern must bind every field of the reference's op
+    (crates/infr-core/src/graph.rs:918-1011) and carry each into `HipMoe` or a tensor id: a `..` in the
+    pattern would let a field that changes the arithmetic (gating, weight_before, act, ...) vanish on the
+    way to the library, which can only refuse what it is told about."""
+    import re
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    m = re.search(r"Op::MoeFfn \{([^}]*)\} => ops\.push\(HipOp \{(.*?)\.\.Default::default\(\) \}\),", text, re.S)
+    assert m, "INTEGRATION.md no longer holds the MoeFfn arm"
+    pattern, body = m.group(1), m.group(2)
+    assert ".." not in pattern, "the MoeFfn pattern skips fields with `..`"
+    bound = {f.strip().split(":")[0].strip() for f in pattern.split(",") if f.strip()}
+    op_fields = {"x", "router_x", "router", "gate_exps", "up_exps", "down_exps", "down_scale", "fused_gate_up", "dst",
+                 "ne", "n_expert", "n_used", "n_ff_exp", "scale", "act", "swiglu_clamp", "gating", "norm_w",
+                 "weight_before", "ep_band", "exp_probs_b", "n_expert_groups", "n_expert_groups_used", "expert_ids"}
+    assert bound == op_fields
+    for f in op_fields:                          # and each one is used on the right-hand side
+        assert re.search(rf"\b{f}\b", body), f"{f} is bound but not passed on"
+    # the header documents what each flag means and that unsupported settings are refused
+    header = open(os.path.join(ROOT, "include", "infr_hip.h")).read()
+    for f in ("act", "gating", "norm_w", "weight_before", "fused_gate_up", "has_clamp", "n_expert_groups",
+              "n_expert_groups_used", "has_down_scale", "has_exp_probs_b", "has_expert_ids", "has_ep_band"):
+        assert re.search(rf"\b{f}\b", header), f

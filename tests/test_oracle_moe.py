@@ -7,20 +7,60 @@ import pytest
 from oracle import oracle as orc
 
 
-def moe_ref(x, router, gate, up, down, ne, n_expert, n_used, n_ff, scale):
-    """Softmax gating, stable descending top-k, renormalised weights, silu(gate.x)*(up.x), down."""
+def _act(kind, g):
+    if kind == orc.GELU:
+        return 0.5 * g * (1.0 + np.tanh(0.7978846 * (g + 0.044715 * g ** 3)))
+    if kind == orc.SIGMOID:
+        return 1.0 / (1.0 + np.exp(-g))
+    return g / (1.0 + np.exp(-g))
+
+
+def moe_ref(x, router, gate, up, down, ne, n_expert, n_used, n_ff, scale, *, gating=0, bias=None, groups=0,
+            groups_used=0, act=0, norm_w=True, weight_before=False, clamp=None, down_scale=None, ids=None):
+    """Textbook MoE of one row: gating probabilities, optional selection bias and group masking,
+    stable descending top-k (or the supplied ids), weights from the unbiased probabilities,
+    act(gate.x) * (up.x) with the weight on either side, down, weighted sum. `up` may be None when
+    `gate` holds [gate rows | up rows] per expert."""
     f = np.float32
     logits = (router.reshape(n_expert, ne) @ x).astype(f)
-    p = np.exp(logits - logits.max()).astype(f)
-    p = (p / p.sum(dtype=f)).astype(f)
-    idx = sorted(range(n_expert), key=lambda e: -p[e])[:n_used]      # sorted() is stable
+    if gating == orc.GATING_SIGMOID:
+        p = (1.0 / (1.0 + np.exp(-logits))).astype(f)
+    elif gating == orc.GATING_SQRT_SOFTPLUS:
+        p = np.sqrt(np.where(logits > 20, logits, np.log1p(np.exp(np.minimum(logits, 30))))).astype(f)
+    else:
+        p = np.exp(logits - logits.max()).astype(f)
+        p = (p / p.sum(dtype=f)).astype(f)
+    if ids is None:
+        sel = p.copy() if bias is None else (p + bias).astype(f)
+        if groups > 1 and groups_used > 0:
+            per = n_expert // groups
+            score = [float(np.sort(sel[g * per:(g + 1) * per])[-2:].sum(dtype=f)) for g in range(groups)]
+            keep = sorted(range(groups), key=lambda g: -score[g])[:groups_used]
+            for g in range(groups):
+                if g not in keep:
+                    sel[g * per:(g + 1) * per] = -np.inf
+        idx = sorted(range(n_expert), key=lambda e: -sel[e])[:n_used]      # sorted() is stable
+    else:
+        idx = [int(e) for e in ids]
     wsum = max(f(sum(p[e] for e in idx)), f(1e-20))
     out = np.zeros(ne, f)
     for e in idx:
-        g = gate.reshape(n_expert, n_ff, ne)[e] @ x
-        u = up.reshape(n_expert, n_ff, ne)[e] @ x
-        act = (g / (1.0 + np.exp(-g)) * u).astype(f)
-        out += (p[e] / wsum * scale) * (down.reshape(n_expert, ne, n_ff)[e] @ act)
+        w = f(p[e] / wsum * scale) if norm_w else f(p[e] * scale)
+        if up is None:
+            gu = gate.reshape(n_expert, 2 * n_ff, ne)[e] @ x
+            g, u = gu[:n_ff], gu[n_ff:]
+        else:
+            g = gate.reshape(n_expert, n_ff, ne)[e] @ x
+            u = up.reshape(n_expert, n_ff, ne)[e] @ x
+        if weight_before:
+            g, u = w * g, w * u
+        if clamp is not None:
+            g, u = np.minimum(g, clamp), np.clip(u, -clamp, clamp)
+        a = (_act(act, g.astype(np.float64)) * u).astype(f)
+        yk = down.reshape(n_expert, ne, n_ff)[e] @ a
+        if down_scale is not None:
+            yk = yk * down_scale[e]
+        out += yk if weight_before else w * yk
     return out, idx
 
 
@@ -127,3 +167,140 @@ def test_32_block_bank_formats_against_textbook(dtype, int8):
         assert np.abs(yref[r] - want).max() < 1e-4
         assert np.abs(y[r] - want).max() < (2e-2 * np.abs(want).max() if int8 else 1e-4)
     assert np.array_equal(y, yref) != int8
+
+
+# ---- the rest of Op::MoeFfn's fields (graph.rs:932-1010; CPU arm lib.rs:2293-2309, 2426-2543, 2833-2861,
+# 2932-2945, 2976), each against the textbook form above. The reference's own moe_ref covers gating,
+# bias and groups at rows == 1 (seam_op_parity.rs:1224-1322); act, norm_w, weight_before, clamp,
+# down_scale, fused banks and supplied ids follow the op's documentation. ----
+
+def _case(seed, ne=256, n_expert=8, n_used=2, n_ff=256, dtype=None, rows=1, fused=False):
+    dtype = orc.Q4_K if dtype is None else dtype
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal(rows * ne).astype(np.float32)
+    router = (rng.standard_normal(n_expert * ne) * 0.1).astype(np.float32)
+    from infr_amd import synth_weight
+    if fused:
+        gate = synth_weight(dtype, seed, n_expert * 2 * n_ff, ne, sigma=0.05)
+        up = None
+    else:
+        gate = synth_weight(dtype, seed, n_expert * n_ff, ne, sigma=0.05)
+        up = synth_weight(dtype, seed + 1, n_expert * n_ff, ne, sigma=0.05)
+    down = synth_weight(dtype, seed + 2, n_expert * ne, n_ff, sigma=0.05)
+    return x, router, gate, up, down, dict(ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=n_ff, gate_dtype=dtype,
+                                           up_dtype=dtype, down_dtype=dtype)
+
+
+def _check(x, router, gate, up, down, kw, scale=1.0, tol=1e-4, **opts):
+    """Runs the oracle with `opts` and compares every row with the textbook form."""
+    ref_names = dict(gating="gating", exp_probs_b="bias", n_expert_groups="groups", n_expert_groups_used="groups_used",
+                     act="act", norm_w="norm_w", weight_before="weight_before", swiglu_clamp="clamp",
+                     down_scale="down_scale")
+    y, idx, w = orc.moe_ffn(x, router, gate, up, down, scale=scale, fused_gate_up=up is None, **kw, **opts)
+    dt, ne = kw["gate_dtype"], kw["ne"]
+    gf, df = orc.dequant_block(dt, gate), orc.dequant_block(dt, down)
+    uf = None if up is None else orc.dequant_block(dt, up)
+    ropts = {ref_names[k]: v for k, v in opts.items() if k in ref_names}
+    ids = opts.get("expert_ids")
+    for r in range(x.size // ne):
+        want, want_idx = moe_ref(x[r * ne:(r + 1) * ne], router, gf, uf, df, ne, kw["n_expert"], kw["n_used"],
+                                 kw["n_ff_exp"], np.float32(scale),
+                                 ids=None if ids is None else np.asarray(ids).reshape(-1, kw["n_used"])[r], **ropts)
+        assert list(idx[r]) == want_idx
+        assert np.abs(y[r] - want).max() < tol * max(1.0, np.abs(want).max())
+    return y, idx, w
+
+
+@pytest.mark.parametrize("gating", [orc.GATING_SIGMOID, orc.GATING_SQRT_SOFTPLUS])
+@pytest.mark.parametrize("norm_w", [True, False])
+def test_gating_and_norm_w(gating, norm_w):
+    x, router, gate, up, down, kw = _case(60)
+    y, idx, w = _check(x, router, gate, up, down, kw, scale=2.0, gating=gating, norm_w=norm_w)
+    logits = router.reshape(kw["n_expert"], -1) @ x
+    if gating == orc.GATING_SIGMOID:            # closed form of the weights themselves
+        p = 1 / (1 + np.exp(-logits[idx[0]].astype(np.float64)))
+    else:
+        p = np.sqrt(np.log1p(np.exp(logits[idx[0]].astype(np.float64))))
+    want_w = p / p.sum() * 2.0 if norm_w else p * 2.0
+    assert np.allclose(w[0], want_w, rtol=1e-5)
+
+
+def test_sqrt_softplus_shortcut_above_20():
+    # lib.rs:2446-2450: v > 20 -> softplus(v) = v exactly
+    x, router, gate, up, down, kw = _case(61)
+    router = router.reshape(kw["n_expert"], -1).copy()
+    router[3] = x * (25.0 / float(x @ x))       # logit 25 for expert 3
+    _, idx, w = _check(x, router, gate, up, down, kw, gating=orc.GATING_SQRT_SOFTPLUS, norm_w=False)
+    assert idx[0][0] == 3 and abs(w[0][0] - np.sqrt(np.float32(router[3] @ x))) < 1e-5
+
+
+def test_llama4_style_weight_before_sigmoid_top1():
+    # llama4: sigmoid gating, top-1, no renormalisation, weight on the expert input (graph.rs:956-967)
+    x, router, gate, up, down, kw = _case(62, n_used=1)
+    y, _, _ = _check(x, router, gate, up, down, kw, gating=orc.GATING_SIGMOID, norm_w=False, weight_before=True)
+    y_after = orc.moe_ffn(x, router, gate, up, down, gating=orc.GATING_SIGMOID, norm_w=False, **kw)[0]
+    assert np.abs(y - y_after).max() > 1e-3 * np.abs(y).max()      # the two sides of the SiLU differ
+
+
+@pytest.mark.parametrize("act", [orc.GELU, orc.SIGMOID])
+def test_expert_activation(act):
+    x, router, gate, up, down, kw = _case(63)
+    _check(x, router, gate, up, down, kw, act=act)
+
+
+def test_swiglu_clamp_and_the_combinations_the_cpu_arm_asserts_against():
+    x, router, gate, up, down, kw = _case(64)
+    y = _check(x, router, gate, up, down, kw, swiglu_clamp=0.05)[0]
+    assert not np.array_equal(y, orc.moe_ffn(x, router, gate, up, down, **kw)[0])    # the clamp bit
+    for bad in (dict(act=orc.SIGMOID), dict(weight_before=True)):                     # lib.rs:2293-2299
+        with pytest.raises(ValueError):
+            orc.moe_ffn(x, router, gate, up, down, swiglu_clamp=1.0, **bad, **kw)
+
+
+def test_fused_gate_up_bank_equals_split_banks():
+    # graph.rs:936-941: gate rows first, up rows second inside each expert's slice
+    x, router, gate, up, down, kw = _case(65)
+    ne, n_expert, n_ff = kw["ne"], kw["n_expert"], kw["n_ff_exp"]
+    per = n_ff * ne // 256 * 144
+    fused = np.concatenate([np.concatenate([gate[e * per:(e + 1) * per], up[e * per:(e + 1) * per]])
+                            for e in range(n_expert)])
+    a = orc.moe_ffn(x, router, gate, up, down, **kw)[0]
+    b = orc.moe_ffn(x, router, fused, None, down, fused_gate_up=True, **kw)[0]
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    _check(x, router, fused, None, down, kw)
+
+
+def test_down_scale():
+    x, router, gate, up, down, kw = _case(66)
+    ds = np.linspace(0.5, 2.0, kw["n_expert"]).astype(np.float32)
+    _check(x, router, gate, up, down, kw, down_scale=ds)
+
+
+def test_selection_bias_moves_the_selection_but_not_the_weights():
+    x, router, gate, up, down, kw = _case(67)
+    base_idx = orc.moe_ffn(x, router, gate, up, down, **kw)[1][0]
+    bias = np.zeros(kw["n_expert"], np.float32)
+    loser = [e for e in range(kw["n_expert"]) if e not in base_idx][0]
+    bias[loser] = 10.0
+    _, idx, w = _check(x, router, gate, up, down, kw, exp_probs_b=bias)
+    assert idx[0][0] == loser and abs(float(w[0].sum()) - 1.0) < 1e-5      # weights from the unbiased probs
+
+
+def test_group_limited_routing():
+    x, router, gate, up, down, kw = _case(68, n_expert=16, n_used=4)
+    _, idx, _ = _check(x, router, gate, up, down, kw, n_expert_groups=4, n_expert_groups_used=2)
+    assert len({int(e) // 4 for e in idx[0]}) <= 2
+    # one group wins outright when only one is kept
+    _, idx1, _ = _check(x, router, gate, up, down, kw, n_expert_groups=4, n_expert_groups_used=1)
+    assert len({int(e) // 4 for e in idx1[0]}) == 1
+
+
+def test_supplied_expert_ids_keep_their_order_and_take_router_weights():
+    x, router, gate, up, down, kw = _case(69, rows=2)
+    ids = np.array([[5, 1], [0, 7]], np.int32)
+    _, idx, w = _check(x, router, gate, up, down, kw, expert_ids=ids, reference_mode=True)
+    assert np.array_equal(idx, ids) and np.allclose(w.sum(axis=1), 1.0, atol=1e-5)
+    with pytest.raises(ValueError):                                   # lib.rs:2303-2309
+        orc.moe_ffn(x, router, gate, up, down, expert_ids=ids, exp_probs_b=np.zeros(8, np.float32), **kw)
+    with pytest.raises(ValueError):                                   # lib.rs:2464-2469
+        orc.moe_ffn(x, router, gate, up, down, expert_ids=np.array([[5, 8], [0, 7]], np.int32), **kw)

@@ -64,3 +64,31 @@ def test_noalloc_rejects_what_the_static_scratch_cannot_hold(be):
         be.linear_noalloc(DType.Q4K, w, x, y, m_big, in_f, out_f)
     assert e.value.status == Status.Unsupported and "static scratch" in e.value.msg
     be.sync()
+
+
+def _free_device_bytes():
+    """hipMemGetInfo through the HIP runtime the library itself is linked against."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    free, total = ctypes.c_size_t(), ctypes.c_size_t()
+    assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+    return free.value
+
+
+def test_noalloc_leaves_free_device_memory_unchanged(be):
+    """A call far larger than any before it on this route must not take device memory: the grow-on-demand
+    scratch of infr_hip_linear would have to grow by several MB for it (and does, in the control below)."""
+    in_f, out_f = 4096, 64
+    w = be.upload_new(synth_weight(DType.Q4K, 2, out_f, in_f))
+    m_small, m_big = 128, 1000
+    x = be.upload_new(synth_normal_f32(3, m_big * in_f))
+    y = be.alloc(m_big * out_f * 4)
+    be.linear_noalloc(DType.Q4K, w, x, y, m_small, in_f, out_f)    # the route's kernels are loaded now
+    be.sync()
+    before = _free_device_bytes()
+    be.linear_noalloc(DType.Q4K, w, x, y, m_big, in_f, out_f)
+    be.sync()
+    assert _free_device_bytes() == before
+    got = be.download(y, np.empty((m_big, out_f), np.float32))
+    want = orc.linear(DType.Q4K, synth_weight(DType.Q4K, 2, out_f, in_f), synth_normal_f32(3, m_big * in_f)[:2 * in_f], 2, in_f, out_f)
+    assert np.array_equal(bits(got[:2]), bits(want))
