@@ -367,8 +367,11 @@ static bool floats_overlap(const float* a, size_t na, const float* b, size_t nb)
 }
 
 int enqueue_linear(infr_hip_t* be, int dtype, const LinearArgs& la, const float* x, float* y,
-                   size_t m, size_t in_f, size_t out_f, const infr::IntStages& st, const infr::ActQ8& act) {
+                   size_t m, size_t in_f, size_t out_f, const infr::IntStages& st, const infr::ActQ8& act,
+                   infr::QuantCache* qc = nullptr) {
     bool ok;
+    // (the branches that do not quantize may park a copy of x in the scratch)
+    if (qc && (is_plain(dtype) || infr::gemv_takes_f32_activations(dtype, m))) *qc = infr::QuantCache{};
     if (is_plain(dtype)) {
         if (st.a) return fail(be, INFR_HIP_ERR_UNSUPPORTED, "int_stages: unquantized weights have no integer stage");
         if (floats_overlap(x, m * in_f, y, m * out_f)) {
@@ -391,7 +394,8 @@ int enqueue_linear(infr_hip_t* be, int dtype, const LinearArgs& la, const float*
         ok = infr::launch_gemv_f32act(dtype, la.wrows, la.bpr, x, y, in_f, out_f, be->stream);
     } else {
         // quantizes x into the scratch in the layout its kernel reads, then multiplies
-        ok = infr::launch_mmq(dtype, la.wrows, la.bpr, x, act, y, m, in_f, out_f, st, be->stream);
+        ok = infr::launch_mmq(dtype, la.wrows, la.bpr, x, act, y, m, in_f, out_f, st, be->props.multiProcessorCount, be->stream, qc);
+        if (qc && floats_overlap(x, m * in_f, y, m * out_f)) *qc = infr::QuantCache{};  // x is overwritten
     }
     if (!ok)
         return fail(be, INFR_HIP_ERR_UNSUPPORTED,
@@ -1465,7 +1469,15 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
 
 // Enqueues the scheduled launches (this is what gets recorded for replay: kernels only).
 static int enqueue_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t* const* bindings) {
+    // Linears of one level that multiply the same activation tensor (q / k / v, gate / up of a prefill
+    // chunk) quantize it once: the scratch keeps it until the level ends or another step writes the
+    // scratch. (Ops of one level neither write what another reads nor each other's outputs.)
+    infr::QuantCache qc;
+    int qc_level = -1;
     for (const auto& st : plan->steps) {
+        const bool lone_linear = st.op >= 0 && plan->ops[st.op].kind == INFR_OP_LINEAR;
+        if (!lone_linear || st.level != qc_level) qc = infr::QuantCache{};
+        qc_level = st.level;
         if (st.op >= 0 && plan->ops[st.op].kind == INFR_OP_MOE_FFN) {
             const auto& op = plan->ops[st.op];
             infr::MoeShape ms;
@@ -1513,7 +1525,7 @@ static int enqueue_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t
                 return rc;
             if (int rc = enqueue_linear(be, op.w_dtype, la, static_cast<const float*>(bindings[op.x]->ptr),
                                         static_cast<float*>(bindings[op.dst]->ptr), op.m, op.in_f,
-                                        op.out_f, infr::IntStages{}, be->act))
+                                        op.out_f, infr::IntStages{}, be->act, &qc))
                 return rc;
         } else if (st.m > 1) {
             infr::launch_quantize_q8_group(plan->qtiles_dev + st.qtile_first, st.qtile_n, act_per32(st.dtype, st.in_f),

@@ -37,10 +37,10 @@ struct LaneSums {
 // Per-wave LDS scratch of the one-block-per-lane formats (Q8_0, the 32-weight-block formats) when
 // their per-block terms must be added in ascending block order as infr-cpu's scalar kernels add them
 // (kernels.rs:1170-1187: `sumf += d8 * d_w * iprod` block by block): every lane parks its block's
-// term, 8 rows x (64 * STEPS terms + 4 pad) floats, and lane i then adds row i's terms in order.
+// term, 8 (long rows: 4) rows x (64 * STEPS terms + 4 pad) floats, and lane i then adds row i's terms in order.
 template <int STEPS>
 struct LaneOrderedSum {
-    static constexpr int kRows = 8, kRowStride = 64 * STEPS + 4;
+    static constexpr int kRows = STEPS > 4 ? 4 : 8, kRowStride = 64 * STEPS + 4;  // (at most 33 KB for four waves)
     static constexpr int kFloatsPerWave = kRows * kRowStride;
 };
 // What gemv_rows needs per wave, by format.

@@ -127,8 +127,19 @@ bool launch_gemv_fused(int dtype, size_t in_f, const GemvOpDesc* ops, int n, con
 // m >= 2: GEMM over on-device quantized activations. y is [m][out_f] row-major.
 // m >= 2: quantizes x [m, in_f] into `act` (sized for m rounded up to 32 rows) in the layout the
 // chosen kernel reads, then multiplies.
+// `cus`: the device's compute units (the prefill kernels size their grids in rounds of them).
+// What the activation scratch currently holds: the quantization of the m x in_f floats at `x` in
+// `layout` (0: nothing known). A caller that runs several Linears over one activation tensor with
+// nothing in between that writes the scratch or x (q / k / v, gate / up of a prefill chunk) passes
+// the same QuantCache to each: the quantizer then runs once.
+struct QuantCache {
+    const float* x = nullptr;
+    size_t m = 0, in_f = 0;
+    int layout = 0;  // 1 row-major per-256, 2 row-major per-32, 3 tiled per-256, 4 tiled per-32, 5 tiled per-32 transposed
+};
 bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const ActQ8& act, float* y,
-                size_t m, size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream);
+                size_t m, size_t in_f, size_t out_f, const IntStages& st, int cus, hipStream_t stream,
+                QuantCache* qc = nullptr);
 
 // Small-batch ops of one dependency level that share (dtype, in_f, m), as ONE launch: the
 // workgroups index a tile table. `act_elem0` is where the op's quantized activation rows start
@@ -299,11 +310,13 @@ void launch_mmq_shared_q5k(const uint8_t* w, size_t bpr, const ActQ8& act, float
 // iprod per (token, row, 32-element block).
 bool launch_mmq_shared_nib32(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m,
                              size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream);
-// Q4_K strip form (mmq_q4k_strip.hip): 256 tokens x 96 rows per workgroup, activations in the tiled
-// quantizer's layout. `takes` says whether the grid fills the device well enough to prefer it.
-bool mmq_strip_q4k_takes(size_t m, size_t out_f);
+// Q4_K strip form (mmq_q4k_strip.hip): 256 tokens x (32 * tiles) rows per workgroup, activations in
+// the tiled quantizer's layout. mmq_strip_q4k_tiles picks the strip height (1..3 row tiles) for a device
+// of `cus` compute units.
+// exact: the f32 epilogue as infr-cpu writes it (y bit-identical) instead of the contracted one.
+int mmq_strip_q4k_tiles(size_t m, size_t out_f, size_t in_f, int cus);
 void launch_mmq_strip_q4k(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
-                          size_t out_f, const IntStages& st, hipStream_t stream);
+                          size_t out_f, const IntStages& st, int tiles, bool exact, hipStream_t stream);
 // Routed pairs bucketed by expert, in tiles of at most 32 pairs of one expert each (device arrays;
 // `*n_tiles` of the `max_tiles` entries exist). `perm` lists the pairs expert by expert.
 struct MoeTileTable {

@@ -1323,7 +1323,12 @@ static bool skinny16_shape(int dtype, int nb, size_t m, size_t out_f) {
         // 24 / 32 / 48 us at 33 / 64 / 96 tokens; 4096 x 4096: 7.6 / 9.8 / 14; 1024 x 4096: 2.7 / 3.3 / 4.4).
         if (m <= 32) return false;
         if (out_f == 0) return true;
-        return long_rows ? m <= 127 : (small && m <= 128);
+        // Beyond that this kernel runs at ~225 TOP/s whatever the shape (it unpacks a block once per
+        // 16 tokens), while the tiled kernels have a floor: a workgroup walks a whole row, ~1.6 us per
+        // 256-block, however few workgroups there are. The two meet at about 640 K outputs (measured at
+        // 1024 / 2048 / 4096 x 4096 and 4096 x 12288, 128 to 1024 tokens: 1024 x 4096 at 512 tokens takes
+        // 19 us here and 27 on the tiles, 4096 x 4096 at 192 tokens 29 against 25).
+        return m * out_f <= (size_t)640 * 1024;
     }
     //   Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL  14-16 / 12-14 / 5.0-5.7; before: 41 at 16 tokens, 76 at 32, 147 at 64,
     //         then 59-71 / 130-180 / 50-64
@@ -1438,7 +1443,23 @@ void launch_mmq_q4k_gathered(const uint8_t* bank, size_t expert_stride, size_t b
 }
 
 bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const ActQ8& act, float* y,
-                size_t m, size_t in_f, size_t out_f, const IntStages& st, hipStream_t stream) {
+                size_t m, size_t in_f, size_t out_f, const IntStages& st, int cus, hipStream_t stream,
+                QuantCache* qc) {
+    // the activation quantizers, skipped when the scratch already holds this tensor in this layout
+    auto have = [&](int layout) {
+        if (qc && qc->x == x && qc->m == m && qc->in_f == in_f && qc->layout == layout) return true;
+        if (qc) *qc = QuantCache{x, m, in_f, layout};
+        return false;
+    };
+    auto quantize_rows = [&](bool per32) {
+        if (!have(per32 ? 2 : 1)) launch_quantize_q8(x, m, in_f, per32, act, stream);
+    };
+    auto quantize_tiled = [&] {
+        if (!have(3)) launch_quantize_q8_tiled(x, m, in_f, act, stream);
+    };
+    auto quantize_32_tiled = [&](bool transposed16) {
+        if (!have(transposed16 ? 5 : 4)) launch_quantize_q8_32_tiled(x, m, in_f, transposed16, act, stream);
+    };
     // Q4_K routes by token count (thresholds from sweeps at K = 4096, N = 12288):
     //   2..32      skinny kernel, K split over the waves of a workgroup
     //   33..127    tiled kernel, 32 tokens x 128 rows per workgroup (most workgroups for few tokens)
@@ -1453,27 +1474,20 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
     const bool long_row = gemv_row_too_long(dtype, in_f) && in_f % 256 == 0;
     // the 16-token K-split kernel where it is ahead beyond 16 tokens (up to 32..128 by format and shape)
     if (!long_row && (dtype != 12 || m > 32) && mmq_skinny16_takes(dtype, m, in_f, out_f)) {
-        launch_quantize_q8(x, m, in_f, act_is_per32(dtype, in_f), act, stream);
+        quantize_rows(act_is_per32(dtype, in_f));
         const size_t wgs = (out_f + 31) / 32;
         return st.a ? launch_mmq_skinny16<true>(dtype, w, bpr, act, y, m, in_f, out_f, wgs, st, nullptr, stream)
                     : launch_mmq_skinny16<false>(dtype, w, bpr, act, y, m, in_f, out_f, wgs, st, nullptr, stream);
     }
     if (dtype == 12 && (m >= 128 || long_row)) {
-        launch_quantize_q8_tiled(x, m, in_f, act, stream);
-        if (mmq_strip_q4k_takes(m, out_f)) {
-            launch_mmq_strip_q4k(w, bpr, act, y, m, in_f, out_f, st, stream);
-            return true;
-        }
-        // (896 / 1000 tokens at 12288 x 4096: 658 / 730 against 622 / 627 TOPS; at 768 and below the
-        // 32-row form is ahead)
-        // 256-token tiles pad up to 128 tokens more than 128-token tiles do: taken when both pad alike,
-        // or when that padding is small against the batch
-        const size_t pad_w = (m + 255) / 256 * 256, pad_n = (m + 127) / 128 * 128;
-        const bool wide = m > 768 && (pad_w == pad_n || pad_w >= 2048);
-        // two row tiles: eight waves (256 tokens) per workgroup, each unpacking one tile's nibble pair -
-        // half the unpack work and row loads per output tile; 729 / 763 / 766 against 669 / 719 / 731
-        // TOPS at 1024 / 2048 / 4096 tokens (12288 x 4096)
-        if (wide) launch_mmq_shared_q4k<2, 8>(w, bpr, act, y, m, in_f, out_f, st, stream);
+        quantize_tiled();
+        // From 128 tokens up y is held to 1e-4 of infr-cpu, not to its bits (the integers stay exact):
+        // the strip kernel contracts the f32 epilogue. The integer-stage entry point keeps the exact form.
+        // Strips are 256 tokens wide: a batch that fills less than ~0.6 of its 256-token groups (128..153,
+        // 257..307 tokens) takes the 128-token tiles of the shared-operand kernel instead.
+        const size_t groups256 = (m + 255) / 256;
+        const int tiles = (double)m >= 0.6 * (double)(groups256 * 256) ? mmq_strip_q4k_tiles(m, out_f, in_f, cus) : 0;
+        if (tiles > 0) launch_mmq_strip_q4k(w, bpr, act, y, m, in_f, out_f, st, tiles, st.a != nullptr, stream);
         else launch_mmq_shared_q4k<1>(w, bpr, act, y, m, in_f, out_f, st, stream);
         return true;
     }
@@ -1481,12 +1495,12 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
     // 4096 x 12288, 1024 x 4096) and the dot4 batches cost ~3.5 / 3.2 / 1.1 us per token there, so
     // it takes over from 33 tokens
     if (dtype == 14 && (m >= 33 || long_row)) {
-        launch_quantize_q8_tiled(x, m, in_f, act, stream);
+        quantize_tiled();
         launch_mmq_shared_q6k(w, bpr, act, y, m, in_f, out_f, st, stream);
         return true;
     }
     if (dtype == 13 && (m >= 33 || long_row)) {
-        launch_quantize_q8_tiled(x, m, in_f, act, stream);
+        quantize_tiled();
         launch_mmq_shared_q5k(w, bpr, act, y, m, in_f, out_f, st, stream);
         return true;
     }
@@ -1496,19 +1510,19 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
     // multiply the per-32 activation like these formats, crates/infr-cpu/src/lib.rs:1037-1042)
     if ((dtype == 2 || dtype == 3 || dtype == 6 || dtype == 7 || dtype == 20 || (dtype == 8 && in_f % 256 != 0)) &&
         in_f % 32 == 0 && (m >= 65 || long_row)) {
-        launch_quantize_q8_32_tiled(x, m, in_f, false, act, stream);
+        quantize_32_tiled(false);
         return launch_mmq_shared_nib32(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
     }
     if (dtype == 42 && in_f % 64 == 0 && (m >= 65 || long_row)) {
-        launch_quantize_q8_32_tiled(x, m, in_f, true, act, stream);
+        quantize_32_tiled(true);
         return launch_mmq_shared_nib32(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
     }
     if (dtype == 8 && in_f % 256 == 0 && (m >= 33 || long_row)) {
-        launch_quantize_q8_tiled(x, m, in_f, act, stream);
+        quantize_tiled();
         launch_mmq_shared_q8_0(w, bpr, act, y, m, in_f, out_f, st, stream);
         return true;
     }
-    launch_quantize_q8(x, m, in_f, act_is_per32(dtype, in_f), act, stream);
+    quantize_rows(act_is_per32(dtype, in_f));
     if (mmq_skinny16_takes(dtype, m, in_f, out_f)) {
         const size_t wgs = (out_f + 31) / 32;
         return st.a ? launch_mmq_skinny16<true>(dtype, w, bpr, act, y, m, in_f, out_f, wgs, st, nullptr, stream)

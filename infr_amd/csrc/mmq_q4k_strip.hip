@@ -1,17 +1,23 @@
-// Q4_K prefill GEMM, strip form: 256 tokens x 96 weight rows per workgroup of eight waves.
+// Q4_K prefill GEMM, strip form: 256 tokens x 32 / 64 / 96 weight rows per workgroup of eight waves.
 //
 // Arithmetic is that of mmq.hip (crates/infr-cpu/src/kernels.rs:151-184 per block and output):
 //     sd = sum_s sc_s * (sum_l q4 * q8)   on the int8 matrix cores, the 6-bit scale split into two
 //                                         3-bit digits so that q4 * digit is an int8 operand
 //     sm = sum_s m_s * bsum_s             one K = 16 f16 MFMA over the split per-32 sums (exact)
-//     y += q8.d[b] * (d * (f32)sd - dmin * (f32)sm)     separate multiplies and adds, blocks ascending
-// so y is bit-identical to infr-cpu's batch kernel and to the other routes of this library.
+//     y += q8.d[b] * (d * (f32)sd - dmin * (f32)sm)     blocks ascending
+// sd and sm are exact in every form. The f32 line has two forms: EXACT evaluates it with separate
+// multiplies and adds, as infr-cpu writes it, so y is bit-identical to its batch kernel and to the
+// other routes of this library (the integer-stage entry point runs that form); the form Op::Linear
+// takes from 128 tokens up contracts it into fused multiply-adds - five vector instructions per output
+// and block instead of seven, y within ~1e-7 relative of infr-cpu's.
 //
 // What differs from the other Q4_K kernels is the shape of the work: every workgroup fills a compute
-// unit, so a grid is taken when it comes out at (nearly) whole rounds of one workgroup per unit.
-//  - A workgroup owns a strip of 96 weight rows (three 32-row tiles) and 256 tokens. Wave w owns
-//    tokens 32w .. 32w+31 for all 96 rows: three accumulator tiles per wave. At 512 tokens x 12288
-//    rows that is 256 workgroups - one per compute unit, two waves per SIMD, no second round.
+// unit (or half of one), so the strip height is chosen for the grid to come out at whole rounds of
+// the device's compute units.
+//  - A workgroup owns a strip of KT 32-row tiles (KT = 1, 2 or 3) and 256 tokens. Wave w owns
+//    tokens 32w .. 32w+31 for all the strip's rows: KT accumulator tiles per wave. At 512 tokens x 12288
+//    rows and KT = 3 that is 256 workgroups - one per compute unit, two waves per SIMD, no second round;
+//    4096 rows take KT = 1 for the same 256 workgroups.
 //  - Weights: the 12 (row tile, nibble pair) pieces of a block are unpacked by the waves into MFMA
 //    B-operand order in LDS (two digit planes, 48 KB per block, double-buffered), one block ahead of
 //    the multiplication, from raw bytes requested two blocks ahead. One barrier per block.
@@ -34,11 +40,10 @@ namespace {
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-constexpr int kT = 3;             // 32-row tiles per strip
 constexpr int kNW = 8;            // waves per workgroup, 32 tokens each
-constexpr int kStripRows = 32 * kT;
 constexpr int kStripTokens = 32 * kNW;
 
+template <int kT>  // 32-row tiles per strip
 struct StripLds {
     static constexpr int frag = 1024;                    // one B fragment: 64 lanes x 16 B
     static constexpr int b_bytes = 8 * 2 * kT * frag;    // [sub-block][digit plane][row tile]
@@ -95,12 +100,17 @@ struct ActFrags {
     float d;
 };
 
-template <bool STAGES>
+// EXACT: the f32 epilogue with infr-cpu's separate multiplies and adds (y bit-identical); STAGES (implies
+// EXACT) also stores sd / sm per block.
+template <int kT, bool STAGES, bool EXACT>
 __global__ __launch_bounds__(kNW * 64) void mmq_strip_q4k_kernel(
     const uint8_t* __restrict__ w, size_t bpr, const int8_t* __restrict__ qs, const float* __restrict__ d8,
     const _Float16* __restrict__ bsh, float* __restrict__ y, int m, int out_f, int nb, int nx, int ny,
     int32_t* __restrict__ st_sd, int32_t* __restrict__ st_sm) {
-    typedef StripLds L;
+    static_assert(!STAGES || EXACT, "the integer-stage form is the exact form");
+    static_assert(kT >= 1 && kT <= 3, "one to three row tiles");
+    typedef StripLds<kT> L;
+    constexpr int kStripRows = 32 * kT;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: branches on it are scalar
@@ -114,14 +124,18 @@ __global__ __launch_bounds__(kNW * 64) void mmq_strip_q4k_kernel(
     const int row0 = strip * kStripRows;
     const int tok0 = ty * kStripTokens + wave * 32;
 
-    // ---- the unpack pieces of this wave. Waves w and w + 4 share a SIMD: the lower four take
-    // (row tiles 0 and 1, nibble pair w) and unpack before they multiply, the upper four take
-    // (row tile 2, nibble pair w - 4) and unpack after, so each SIMD carries three pieces and its two
-    // waves are out of phase ----
-    constexpr int NU = 2;
-    const bool two = wave < 4;
-    const int ut[NU] = {two ? 0 : 2, 1};
-    const int up[NU] = {wave & 3, wave & 3};
+    // ---- the unpack pieces of this wave: (row tile, nibble pair) of a block, 4 * kT in all. Waves w
+    // and w + 4 share a SIMD. Three tiles: the lower four take (tiles 0 and 1, pair w) and unpack before
+    // they multiply, the upper four take (tile 2, pair w - 4) and unpack after, so each SIMD carries
+    // three pieces and its two waves are out of phase. Two tiles: one piece each, (tile w / 4, pair
+    // w % 4). One tile: the lower four waves one piece each, the upper four none. ----
+    constexpr int NU = kT == 3 ? 2 : 1;
+    const bool two = wave < 4;                  // the waves that unpack before they multiply
+    const int ut[2] = {two ? 0 : kT - 1, 1};
+    const int up[2] = {wave & 3, wave & 3};
+    // (one tile: waves w and w + 4 share pair w's piece, one sub-block of it each - both read the
+    // piece's raw bytes - so that all eight waves carry the same unpack work)
+    const int e_first = kT == 1 ? wave >> 2 : 0, e_last = kT == 1 ? wave >> 2 : 1;
     const uint8_t* urow[NU];
 #pragma unroll
     for (int u = 0; u < NU; ++u) {
@@ -151,6 +165,7 @@ __global__ __launch_bounds__(kNW * 64) void mmq_strip_q4k_kernel(
                 const int qw[4] = {qv[u].x, qv[u].y, qv[u].z, qv[u].w};
 #pragma unroll
                 for (int e = 0; e < 2; ++e) {  // e = 0: sub-block 2p (low nibbles), 1: 2p+1 (high)
+                    if (e < e_first || e > e_last) continue;
                     const uint32_t sc = (scw >> (sh + 8 * e)) & 0xFFu;
                     const uint32_t lo3 = sc & 7u, hi3 = sc >> 3;
                     v4i blo, bhi;
@@ -164,7 +179,7 @@ __global__ __launch_bounds__(kNW * 64) void mmq_strip_q4k_kernel(
                     *reinterpret_cast<v4i*>(dst) = blo;
                     *reinterpret_cast<v4i*>(dst + kT * L::frag) = bhi;
                 }
-                if (h == 0) {
+                if (h == 0 && e_first == 0) {
                     // the two mins of this pair as f16, k-slots 2p and 2p+1 of the row's eight
                     typedef _Float16 h2 __attribute__((ext_vector_type(2)));
                     const h2 mn = {(_Float16)(int)((mnw >> sh) & 0xFFu), (_Float16)(int)((mnw >> (sh + 8)) & 0xFFu)};
@@ -220,7 +235,8 @@ __global__ __launch_bounds__(kNW * 64) void mmq_strip_q4k_kernel(
                 st_sm[((size_t)tok * out_f + wrow) * nb + b] = (int)sm_prev[r];
             }
         }
-        acc[t][r] += dq[r] * (d_prev * (float)sd - dmin_prev * sm_prev[r]);
+        if (EXACT) acc[t][r] += dq[r] * (d_prev * (float)sd - dmin_prev * sm_prev[r]);
+        else acc[t][r] = __builtin_fmaf(dq[r], __builtin_fmaf(d_prev, (float)sd, -(dmin_prev * sm_prev[r])), acc[t][r]);
     };
 
     // One block. Between two barriers a wave unpacks the next block's weights into the other
@@ -234,8 +250,12 @@ __global__ __launch_bounds__(kNW * 64) void mmq_strip_q4k_kernel(
     // t = 0) is cut into its 16 accumulators, one behind each MFMA, so that the matrix core and the
     // vector ALU work at the same time inside one wave; each activation fragment is requested
     // again, for the next block, right after its last use.
-    ActFrags f;
-    auto multiply = [&](int b) {
+    //
+    // One and two row tiles: a block is too short to cover those requests (an L2 round trip against
+    // half a block's MFMAs), so the fragments are double-buffered instead - `fn` receives the next
+    // block's at the start of this one - which the three-tile form has no registers for.
+    constexpr bool kTwoSets = kT <= 2;
+    auto multiply = [&](int b, ActFrags& f, ActFrags& fn) {
         const uint8_t* buf = lds + (b & 1) * L::bytes;
         const size_t gb_next = g * nb + min(b + 1, nb - 1);
         const int8_t* ap_next = qs + gb_next * (8 * 1024) + lane * 16;
@@ -243,8 +263,12 @@ __global__ __launch_bounds__(kNW * 64) void mmq_strip_q4k_kernel(
         dql_b[col] = f.d;  // both halves of the wave hold the token's scale: same value, same address
         const v8h bs_cur = f.bs;
         // the next block's scales and sums: a whole block ahead
-        f.bs = gload<v8h>(bsh + (gb_next * 64 + lane) * 8);
-        f.d = gload<float>(d8 + gb_next * 32 + col);
+        fn.bs = gload<v8h>(bsh + (gb_next * 64 + lane) * 8);
+        fn.d = gload<float>(d8 + gb_next * 32 + col);
+        if constexpr (kTwoSets) {
+#pragma unroll
+            for (int sb = 0; sb < 8; ++sb) fn.a[sb] = gload<v4i>(ap_next + sb * 1024);
+        }
         const v16i zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         const v16f zf = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         const uint32_t bl = (uint32_t)(uintptr_t)(buf + lane * 16);  // LDS address of the lane's piece of fragment 0
@@ -270,8 +294,8 @@ __global__ __launch_bounds__(kNW * 64) void mmq_strip_q4k_kernel(
             else
                 lo = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.a[sb], bop, k == 1 ? zi : lo, 0, 0, 0);
             // the last use of this activation fragment in the block: ask for the next block's
-            if constexpr (t == kT - 1 && (k & 1)) {
-                f.a[sb] = gload<v4i>(ap_next + sb * 1024);
+            if constexpr (!kTwoSets && t == kT - 1 && (k & 1)) {
+                fn.a[sb] = gload<v4i>(ap_next + sb * 1024);  // (fn is f itself in this form)
             }
             epilogue_one(t == 0 ? kT - 1 : t - 1, k, t == 0 ? b - 1 : b);
             if constexpr (k == 15) {
@@ -297,16 +321,17 @@ __global__ __launch_bounds__(kNW * 64) void mmq_strip_q4k_kernel(
 #pragma unroll
         for (int t = 0; t < kT; ++t) asm volatile("" : "+v"(acc[t]));
         if (!STAGES) {
-            // issue order of the block: per slot the MFMA and seven vector instructions (one
-            // accumulator's epilogue)
+            // issue order of the block: per slot the MFMA and the vector instructions of one
+            // accumulator's epilogue (seven, five in the contracted form)
             constexpr int kMfma = 0x008, kValu = 0x002, kVmemRead = 0x020;
+            constexpr int kEpi = EXACT ? 7 : 5;
 #pragma unroll
             for (int t = 0; t < kT; ++t) {
 #pragma unroll
                 for (int k = 0; k < 16; ++k) {
                     __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
-                    if (t == kT - 1 && (k & 1)) __builtin_amdgcn_sched_group_barrier(kVmemRead, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(kValu, 7, 0);
+                    if (!kTwoSets && t == kT - 1 && (k & 1)) __builtin_amdgcn_sched_group_barrier(kVmemRead, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(kValu, kEpi, 0);
                 }
                 __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
             }
@@ -315,23 +340,34 @@ __global__ __launch_bounds__(kNW * 64) void mmq_strip_q4k_kernel(
 
     // Requests past the last block are clamped to it (redundant loads, never consumed), so the
     // loop body is straight-line code.
+    ActFrags f0, f1;
     request_rows(0);
-    request_acts(f, 0);
+    request_acts(f0, 0);
     unpack_to(lds);
     request_rows(min(1, nb - 1));
     __syncthreads();
-    for (int b = 0; b < nb; ++b) {
+    auto block = [&](int b, ActFrags& f, ActFrags& fn) {
         uint8_t* other = lds + ((b + 1) & 1) * L::bytes;
         if (two) {
             unpack_to(other);
             request_rows(min(b + 2, nb - 1));
         }
-        multiply(b);
+        multiply(b, f, fn);
         if (!two) {
             unpack_to(other);
             request_rows(min(b + 2, nb - 1));
         }
         __syncthreads();
+    };
+    if constexpr (kTwoSets) {
+        int b = 0;
+        for (; b + 2 <= nb; b += 2) {
+            block(b, f0, f1);
+            block(b + 1, f1, f0);
+        }
+        if (b < nb) block(b, f0, f1);
+    } else {
+        for (int b = 0; b < nb; ++b) block(b, f0, f0);
     }
     // the last block's last row tile
 #pragma unroll
@@ -351,35 +387,57 @@ __global__ __launch_bounds__(kNW * 64) void mmq_strip_q4k_kernel(
 
 }  // namespace
 
-bool mmq_strip_q4k_takes(size_t m, size_t out_f) {
-    // One workgroup fills a compute unit (104 KB of LDS, two waves per SIMD) for the whole of K, so
-    // the grid runs in rounds of 256 workgroups: taken when at least nine tenths of the tokens x rows
-    // those rounds could hold are real. 512 tokens x 12288 rows is exactly one round. Measured at
-    // K = 4096, N = 12288 against the 32-row shared-operand kernel: 69 against 85 us at 512 tokens,
-    // 208 against 222 at 1536, 276 against 290 at 2048; half-filled rounds lose (117 against 108 us
-    // at 640 tokens).
-    const size_t wgs = ((out_f + kStripRows - 1) / kStripRows) * ((m + kStripTokens - 1) / kStripTokens);
-    const size_t rounds = (wgs + 255) / 256;
-    return (double)m * (double)out_f >= 0.9 * (double)(rounds * 256 * kStripRows * kStripTokens);
+// Strip height for `m` tokens x `out_f` rows of `in_f` columns on `cus` compute units: the number of
+// 32-row tiles (1..3) whose grid takes the least time, a taller strip winning ties. A workgroup
+// walks its whole row; a round of one workgroup per compute unit costs, per 256-block, ~1.6 / 2.3 /
+// 3.6 us at one / two / three tiles (measured at 4096 and 12288 columns, 256 to 2048 tokens: two tiles
+// have double-buffered activation fragments and an even unpack, three have neither for want of
+// registers, one spends most of a block on what does not depend on the height), and the grid runs in
+// whole rounds: 512 tokens x 12288 rows are one round at three tiles (58 us) against two at two (74);
+// 512 x 4096 one round at one tile (26) against one at two on half the units (37).
+int mmq_strip_q4k_tiles(size_t m, size_t out_f, size_t in_f, int cus) {
+    if (cus <= 0) cus = 256;
+    static const double per_block_us[4] = {0.0, 1.6, 2.3, 3.6};
+    const size_t ny = (m + kStripTokens - 1) / kStripTokens, nb = in_f / 256;
+    int best = 1;
+    double best_cost = 0.0;
+    for (int kt = 3; kt >= 1; --kt) {
+        const size_t rows = 32 * (size_t)kt;
+        const size_t wgs = ((out_f + rows - 1) / rows) * ny;
+        const size_t rounds = (wgs + cus - 1) / cus;
+        const double cost = (double)rounds * (double)nb * per_block_us[kt];
+        if (kt == 3 || cost < best_cost) best = kt, best_cost = cost;
+    }
+    return best;
 }
 
-void launch_mmq_strip_q4k(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
-                          size_t out_f, const IntStages& st, hipStream_t stream) {
-    const int nx = (int)((out_f + kStripRows - 1) / kStripRows), ny = (int)((m + kStripTokens - 1) / kStripTokens);
+template <int KT>
+static void launch_strip(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
+                         size_t out_f, const IntStages& st, bool exact, hipStream_t stream) {
+    const int nx = (int)((out_f + 32 * KT - 1) / (32 * KT)), ny = (int)((m + kStripTokens - 1) / kStripTokens);
     const dim3 grid((unsigned)(8 * ((nx + 7) / 8) * ny)), block(kNW * 64);
     const int nb = (int)(in_f / 256);
     const auto* bsh = reinterpret_cast<const _Float16*>(act.bsums);
-    if (st.a) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&mmq_strip_q4k_kernel<true>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, StripLds::total);
-        hipLaunchKernelGGL((mmq_strip_q4k_kernel<true>), grid, block, StripLds::total, stream, w, bpr, act.qs, act.d,
-                           bsh, y, (int)m, (int)out_f, nb, nx, ny, st.a, st.b);
-    } else {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&mmq_strip_q4k_kernel<false>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, StripLds::total);
-        hipLaunchKernelGGL((mmq_strip_q4k_kernel<false>), grid, block, StripLds::total, stream, w, bpr, act.qs, act.d,
-                           bsh, y, (int)m, (int)out_f, nb, nx, ny, (int32_t*)nullptr, (int32_t*)nullptr);
-    }
+    constexpr int lds = StripLds<KT>::total;
+#define INFR_STRIP(STAGES, EXACT, A, B)                                                                              \
+    do {                                                                                                             \
+        if (lds > 64 * 1024)                                                                                         \
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&mmq_strip_q4k_kernel<KT, STAGES, EXACT>),      \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, lds);                              \
+        hipLaunchKernelGGL((mmq_strip_q4k_kernel<KT, STAGES, EXACT>), grid, block, lds, stream, w, bpr, act.qs, act.d, \
+                           bsh, y, (int)m, (int)out_f, nb, nx, ny, A, B);                                            \
+    } while (0)
+    if (st.a) INFR_STRIP(true, true, st.a, st.b);
+    else if (exact) INFR_STRIP(false, true, (int32_t*)nullptr, (int32_t*)nullptr);
+    else INFR_STRIP(false, false, (int32_t*)nullptr, (int32_t*)nullptr);
+#undef INFR_STRIP
+}
+
+void launch_mmq_strip_q4k(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
+                          size_t out_f, const IntStages& st, int tiles, bool exact, hipStream_t stream) {
+    if (tiles == 3) launch_strip<3>(w, bpr, act, y, m, in_f, out_f, st, exact, stream);
+    else if (tiles == 2) launch_strip<2>(w, bpr, act, y, m, in_f, out_f, st, exact, stream);
+    else launch_strip<1>(w, bpr, act, y, m, in_f, out_f, st, exact, stream);
 }
 
 }  // namespace infr

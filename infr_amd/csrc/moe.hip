@@ -1238,8 +1238,17 @@ static bool launch_gemv_id_fmt(const uint8_t* bank, size_t expert_stride, size_t
         return true;
     switch (steps) {
         INFR_CASE(1) INFR_CASE(2) INFR_CASE(3) INFR_CASE(4)
-    default: return false;
+    default: break;
     }
+    // rows of five to eight wave steps of the one-block-per-lane formats (2048 columns a step: up to
+    // 16384, Mixtral's 14336-wide experts); the K-quants' four steps already reach 16384
+    if constexpr (!F::kOrdered) {
+        switch (steps) {
+            INFR_CASE(5) INFR_CASE(6) INFR_CASE(7) INFR_CASE(8)
+        default: break;
+        }
+    }
+    return false;
 #undef INFR_CASE
 }
 

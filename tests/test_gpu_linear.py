@@ -25,6 +25,15 @@ def gate(y, want):
     return rel, mx
 
 
+def close(got, want, rel_bar=2e-6, mx_bar=1e-5):
+    """The bar of the contracted Q4_K prefill epilogue (128 tokens and more on the strip kernel): fused
+    multiply-adds where infr-cpu rounds every product, ~1e-7 relative; exact integers either way."""
+    g, t = np.asarray(got, np.float64).ravel(), np.asarray(want, np.float64).ravel()
+    rel = np.linalg.norm(g - t) / np.linalg.norm(t)
+    mx = np.abs(g - t).max() / np.abs(t).max()
+    assert rel <= rel_bar and mx <= mx_bar, f"rel-L2 {rel:.3e} max-abs/|y|inf {mx:.3e}"
+
+
 def run_linear(be, dtype, w, x, m, in_f, out_f, w_off=0, w_numel=None):
     wb, xb = be.upload_new(w), be.upload_new(x)
     yb = be.alloc(m * out_f * 4)
@@ -185,14 +194,17 @@ def test_w_off_selects_rows_of_a_concatenated_weight(be):
 
 # ───────────── prefill (m >= 2): int8 MFMA path for Q4_K ─────────────
 
-# above 768 tokens: 64 rows x 256 tokens on eight waves where the padding allows (ragged last tiles in both
-# directions), else the 32-row form
+# from 128 tokens: the 16-token K-split kernel (rows of two blocks and more, up to 640 K outputs), the
+# 128-token tiles (batches that fill little of their 256-token groups) or the strips (ragged last tiles in
+# both directions)
 PREFILL_SHAPES = [(2, 256, 8), (8, 1024, 96), (33, 512, 200), (64, 1024, 256), (130, 768, 130), (257, 2048, 384),
                   (800, 256, 64), (900, 256, 64), (1024, 256, 64), (1200, 512, 72), (2100, 256, 40)]
 
 
 @pytest.mark.parametrize("m,in_f,out_f", PREFILL_SHAPES)
-def test_prefill_q4k_is_bit_identical_to_oracle(be, m, in_f, out_f):
+def test_prefill_q4k_matches_the_oracle(be, m, in_f, out_f):
+    """Bit-identical below 128 tokens; from 128 on the route may be the strips, whose contracted f32
+    epilogue is held to 2e-6 (the integers behind it are checked exactly elsewhere)."""
     w = synth_weight(DType.Q4K, 300 + m, out_f, in_f)
     x = synth_normal_f32(400 + m, m * in_f)
     x[:in_f] *= 37.0            # rows with very different scales
@@ -201,7 +213,10 @@ def test_prefill_q4k_is_bit_identical_to_oracle(be, m, in_f, out_f):
     y = run_linear(be, DType.Q4K, w, x, m, in_f, out_f)
     want = orc.linear(DType.Q4K, w, x, m, in_f, out_f)
     gate(y, want)
-    assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), "not bit-identical"
+    if m < 128:
+        assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), "not bit-identical"
+    else:
+        close(y, want)
 
 
 # 2..16 tokens on rows of an even number of blocks: 16 x 16 MFMA tiles, K split over the waves of a
@@ -530,9 +545,10 @@ def test_full_size_decode_rows_vs_oracle(be, dtype, in_f, out_f):
 @pytest.mark.parametrize("m", [8, 64, 512, 1024, 1100, 2048])
 def test_full_size_prefill_q4k(be, m):
     """K = 4096 -> N = 12288 at the benchmark's token counts (every Q4_K kernel route; 512, 1024 and
-    2048 tokens fill whole rounds of the 96-row strip kernel, 1100 takes the 32-row shared-operand
-    form): sampled rows bit-identical to the oracle, and every token's row equal to its own m = 1
-    result."""
+    2048 tokens fill whole rounds of 96-row strips, 1100 takes 64-row strips): sampled rows against the
+    oracle and every token's row against its own m = 1 result - bit-identical below 128 tokens, within
+    the contracted epilogue's 2e-6 from there on (the per-block integers of those routes are checked
+    exactly in the strip tests below)."""
     in_f, out_f = 4096, 12288
     w = synth_weight(DType.Q4K, 910, out_f, in_f)
     x = synth_normal_f32(911 + m, m * in_f)
@@ -545,19 +561,27 @@ def test_full_size_prefill_q4k(be, m):
         want = _oracle_rows(DType.Q4K, w, x[np.concatenate([np.arange(t * in_f, (t + 1) * in_f) for t in toks])],
                             len(toks), in_f, out_f, row0, 32)
         got = y[toks, row0:row0 + 32]
-        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), "not bit-identical"
+        if m < 128:
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), "not bit-identical"
+        else:
+            close(got, want)
     y1 = be.alloc(out_f * 4)
     for t in toks:
         be.linear(DType.Q4K, wb, be.upload_new(x[t * in_f:(t + 1) * in_f]), y1, 1, in_f, out_f)
         single = be.download(y1, np.empty((1, out_f), np.float32))
-        assert np.array_equal(single[0].view(np.uint32), y[t].view(np.uint32)), "batch != single"
+        if m < 128:
+            assert np.array_equal(single[0].view(np.uint32), y[t].view(np.uint32)), "batch != single"
+        else:
+            close(y[t], single[0])
 
 
-@pytest.mark.parametrize("m,in_f,out_f", [(2560, 256, 2304), (2400, 768, 2300), (512, 512, 12288)])
+@pytest.mark.parametrize("m,in_f,out_f", [(2560, 256, 2304), (2400, 768, 2300), (512, 512, 12288), (512, 1024, 4096),
+                                          (700, 512, 3000), (1024, 768, 4100), (300, 2304, 2500)])
 def test_q4k_strip_route_is_exact(be, m, in_f, out_f):
-    """Grids of (nearly) whole rounds of 256 workgroups take the strip kernel (256 tokens x 96 rows
-    per workgroup): ragged last strip and token group, one and several blocks per row. Per-block
-    sd / sm exact and y bit-identical on sampled tokens, full-range payloads."""
+    """The prefill strips (256 tokens x 32, 64 or 96 rows per workgroup, the height chosen for the grid):
+    ragged last strip and token group, one and several blocks per row, odd block counts (the two lower
+    heights unroll their block loop by two). Per-block sd / sm exact on sampled tokens and y within the
+    contracted epilogue's bar, full-range payloads."""
     w = orc.synth_weight(DType.Q4K, in_f * out_f, 0x300 + in_f)      # full-range payload bytes
     x = synth_normal_f32(778 + m, m * in_f) * np.float32(3.0)
     x[in_f:2 * in_f] = 1e4      # saturates every code to +127: bsums reach +4064
@@ -569,16 +593,15 @@ def test_q4k_strip_route_is_exact(be, m, in_f, out_f):
     toks = sorted({0, 1, 2, 31, 32, 255, 256, m // 2 + 3, m - 33, m - 1})
     xs = x.reshape(m, in_f)[toks].ravel()
     want = orc.linear(DType.Q4K, w, xs, len(toks), in_f, out_f)
-    assert np.array_equal(y[toks].view(np.uint32), want.view(np.uint32)), "not bit-identical"
+    close(y[toks], want)
     sd, sm = be.linear_int_stages(DType.Q4K, wb, xb, m, in_f, out_f)
     osd, osm = orc.linear_int_stages(DType.Q4K, w, xs, len(toks), in_f, out_f)
     assert np.array_equal(sd[toks], osd) and np.array_equal(sm[toks], osm)
 
 
-def test_q4k_eight_wave_form_at_sixteen_blocks(be):
-    """1280 tokens x 4096 rows pads alike in 128- and 256-token tiles and does not fill the strip
-    kernel's rounds: the eight-wave 64-row x 256-token form, here with 16 blocks per row (its
-    double-buffered block loop at the benchmark's K)."""
+def test_q4k_strips_at_sixteen_blocks_on_4096_rows(be):
+    """1280 tokens x 4096 rows: five token groups of 64- or 32-row strips, 16 blocks per row (the
+    double-buffered activation fragments at the benchmark's K)."""
     m, in_f, out_f = 1280, 4096, 4096
     w = synth_weight(DType.Q4K, 930, out_f, in_f)
     x = synth_normal_f32(931, m * in_f)
@@ -586,7 +609,7 @@ def test_q4k_eight_wave_form_at_sixteen_blocks(be):
     toks = [0, 255, 256, 640, 1279]
     for row0 in (0, 2040, out_f - 32):
         want = _oracle_rows(DType.Q4K, w, x.reshape(m, in_f)[toks].ravel(), len(toks), in_f, out_f, row0, 32)
-        assert np.array_equal(y[toks, row0:row0 + 32].view(np.uint32), want.view(np.uint32)), "not bit-identical"
+        close(y[toks, row0:row0 + 32], want)
 
 
 @pytest.mark.parametrize("dtype", [DType.Q6K, DType.Q8_0])

@@ -6,7 +6,10 @@ The directed tests pin each kernel at the sizes it was written for; this one is 
 between them: a threshold off by one, a tile that assumes a multiple it is not given, a row window
 that starts inside a tile. Bars are the path's: K-quant outputs bit-identical to the oracle
 (same per-block expression, same order), the other formats within rel-L2 <= 1e-4 and
-max-abs <= 1e-3 * max|y|.
+max-abs <= 1e-3 * max|y|. One K-quant route is not bit-identical by design: Q4_K from 128 tokens up may
+take the prefill strips, whose f32 epilogue is contracted into fused
+multiply-adds (the integers stay exact); it is held to rel-L2 <= 2e-6, fifty times inside the path's bar
+and far from what a wrong block, scale or row would give.
 """
 import numpy as np
 import pytest
@@ -34,6 +37,9 @@ def draw_case(rng):
         in_f = 256 * int(rng.integers(1, 10))
     m = int(TOKENS[rng.integers(len(TOKENS))])
     out_f = int(rng.choice([1, 7, 16, 31, 32, 33, 64, 96, 100, 128, 130, 257, 384]))
+    if dtype == DType.Q4K and m >= 128 and rng.integers(2):
+        out_f = int(rng.choice([2304, 2600, 5100, 6144]))        # enough outputs for the prefill strips
+        in_f = 256 * int(rng.integers(1, 5))
     extra_before, extra_after = (int(rng.integers(0, 40)) if rng.integers(2) else 0 for _ in range(2))
     return dtype, m, in_f, out_f, extra_before, extra_after
 
@@ -61,7 +67,12 @@ def test_linear_on_a_random_shape_matches_the_oracle(be, seed):
     got = be.download(yb, np.empty((m, out_f), np.float32))
     want = orc.linear(dtype, w, x, m, in_f, out_f, w_numel=rows * in_f, w_off=before * in_f).reshape(m, out_f)
     assert np.isfinite(want).all(), case
-    if dtype in BIT_IDENTICAL:
+    contracted = dtype == DType.Q4K and m >= 128        # (the routes that are still bit-identical pass this bar too)
+    if contracted:
+        g, t = got.astype(np.float64), want.astype(np.float64)
+        rel = np.linalg.norm(g - t) / max(np.linalg.norm(t), 1e-30)
+        assert rel <= 2e-6 and np.abs(g - t).max() <= 1e-5 * np.abs(t).max(), f"rel-L2 {rel:.2e}: {case}"
+    elif dtype in BIT_IDENTICAL:
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), f"not bit-identical: {case}"
     else:
         g, t = got.astype(np.float64), want.astype(np.float64)

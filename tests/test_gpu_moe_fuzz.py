@@ -14,7 +14,8 @@ every output of that pair, 1e-4..7e-4 of the whole output. The device therefore 
 terms of every int8 bank format in the scalar CPU kernel's order (ascending blocks, kernels.rs:1170-1187):
 K-quants through their ordered sums, Q8_0 and Q5_0 through a per-lane ordered sum in the per-pair
 kernels and block-by-block accumulation in the bucketed tiles. The directed seeds below are cases of
-a 1200-seed sweep that sat at 1.1e-4..6.5e-4 while Q8_0 / Q5_0 terms were added in a tree.
+a sweep of seeds 80..4300 that sat at 1.0e-4..8.6e-4 while Q8_0 / Q5_0 terms were added in a tree
+(twenty of 460 such cases; none of 1015 up to seed 9000 with the ordered sums).
 """
 import numpy as np
 import pytest
@@ -64,7 +65,9 @@ def draw_case(rng):
 
 
 # seeds of the wide sweep whose Q8_0 / Q5_0 gate / up sums used to flip an activation code (see above)
-DIRECTED_SEEDS = ()
+DIRECTED_SEEDS = (207, 524, 750, 841, 1103, 1929, 2027, 2242, 2462, 2564, 2588, 2834, 3113, 3188, 3513, 3549, 3764, 3816,
+                  4108, 4205,
+                  4219, 5853, 5940)     # and three with 14336-wide Q8_0 / Q5_0 down rows (seven wave steps per row)
 
 
 @pytest.mark.parametrize("seed", list(range(80)) + list(DIRECTED_SEEDS))

@@ -752,3 +752,40 @@ def test_small_and_large_batch_ops_of_one_shape_class_on_one_level(be, wide_firs
             for row0 in (0, out_f - rows):
                 want = orc.linear(DType.Q4K, w[row0 * 2304:(row0 + rows) * 2304], x, m, in_f, rows)
                 assert np.array_equal(bits(got[:, row0:row0 + rows]), bits(want)), (out_f, row0)
+
+
+def test_prefill_linears_of_one_level_share_the_activation_quantization(be):
+    """q / k / v of a prefill chunk multiply one activation tensor: the plan quantizes it once per layout
+    and level. Five Linears over one x at 300 tokens - Q4_K strips, a Q6_K tile kernel (same tiled layout:
+    shared), a narrow Q4_K matrix on the 16-token kernel (row-major layout: quantized again), then strips
+    again (tiled once more) and a Linear over another tensor - each against the oracle on sampled rows,
+    on the recording execute and on a replay with new activations."""
+    m, in_f = 300, 1024
+    specs = [(DType.Q4K, 2304, 0), (DType.Q6K, 640, 0), (DType.Q4K, 512, 0), (DType.Q4K, 2600, 0), (DType.Q4K, 2304, 1)]
+    g, binds = Graph(), Bindings()
+    xids, xbs = [], []
+    for i in range(2):
+        xids.append(g.input(TensorDesc((m, in_f), DType.F32)))
+        xbs.append(be.alloc(m * in_f * 4))
+        binds.bind(xids[i], xbs[i])
+    ws, ybs = [], []
+    for i, (dt, out_f, xi) in enumerate(specs):
+        w = synth_weight(dt, 600 + i, out_f, in_f, 0.05)
+        ws.append(w)
+        wid = g.weight(TensorDesc((out_f, in_f), dt))
+        yid = g.output(TensorDesc((m, out_f), DType.F32))
+        ybs.append(be.alloc(m * out_f * 4))
+        binds.bind(wid, be.upload_new(w)).bind(yid, ybs[i])
+        g.push(Linear(xids[xi], wid, yid, m, in_f, out_f))
+    plan = be.compile(g)
+    for rep in range(2):
+        xs = [synth_normal_f32(610 + 2 * rep + i, m * in_f) for i in range(2)]
+        for xb, x in zip(xbs, xs):
+            be.upload(xb, x)
+        be.execute(plan, binds)
+        toks = [0, 37, 255, 256, m - 1]
+        for (dt, out_f, xi), w, yb in zip(specs, ws, ybs):
+            got = be.download(yb, np.empty((m, out_f), np.float32))[toks]
+            want = orc.linear(dt, w, xs[xi].reshape(m, in_f)[toks].ravel(), len(toks), in_f, out_f)
+            rel = np.linalg.norm(got.astype(np.float64) - want) / np.linalg.norm(want)
+            assert rel <= 2e-6, (rep, int(dt), out_f, rel)
