@@ -41,7 +41,7 @@ __global__ __launch_bounds__(256) void quantize_q8_kernel(const float* __restric
 // contiguous 16-byte stores - a wave that
 // wrote its own token's codes in place would scatter every store over sixteen 128-byte lines.
 // Tokens past m quantize zeros (their slots hold d = 0 and zero codes).
-constexpr int kTiledQuantWaves = 16, kTiledQuantPerWave = 32 / kTiledQuantWaves;
+template <int kTiledQuantWaves>
 __global__ __launch_bounds__(kTiledQuantWaves * 64) void quantize_q8_tiled_kernel(const float* __restrict__ x,
                                                                 int8_t* __restrict__ qs,
                                                                 float* __restrict__ d,
@@ -57,7 +57,7 @@ __global__ __launch_bounds__(kTiledQuantWaves * 64) void quantize_q8_tiled_kerne
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int b = blockIdx.x, g = blockIdx.y;
     const size_t in_f = (size_t)nb * 256;
-    constexpr int PW = kTiledQuantPerWave;
+    constexpr int PW = 32 / kTiledQuantWaves;
     v4f v[PW];
 #pragma unroll
     for (int i = 0; i < PW; ++i) {
@@ -83,8 +83,7 @@ __global__ __launch_bounds__(kTiledQuantWaves * 64) void quantize_q8_tiled_kerne
     }
     __syncthreads();
     const size_t gb = (size_t)g * nb + b;
-    if (tid < 512) {
-        const int piece = tid;  // 16-byte piece of the tile: [sub-block][lane]
+    for (int piece = tid; piece < 512; piece += kTiledQuantWaves * 64) {  // 16-byte pieces of the tile: [sub-block][lane]
         const v4i c = *reinterpret_cast<const v4i*>(tile + (piece >> 6) * kSbStride + (piece & 63) * 16);
         gstore<v4i>(qs + gb * (8 * 1024) + (size_t)piece * 16, c);
     }
@@ -94,8 +93,10 @@ __global__ __launch_bounds__(kTiledQuantWaves * 64) void quantize_q8_tiled_kerne
 
 void launch_quantize_q8_tiled(const float* x, size_t m, size_t k, const ActQ8& out, hipStream_t stream) {
     if (m == 0 || k < 256) return;
-    hipLaunchKernelGGL(quantize_q8_tiled_kernel, dim3((unsigned)(k / 256), (unsigned)((m + 31) / 32)),
-                       dim3(kTiledQuantWaves * 64), 0, stream, x, out.qs, out.d, reinterpret_cast<_Float16*>(out.bsums), (int)m, (int)(k / 256));
+    const dim3 grid((unsigned)(k / 256), (unsigned)((m + 31) / 32));
+    // (sixteen waves of two tokens each; eight and four waves a workgroup measured 5-15 % slower)
+    hipLaunchKernelGGL(quantize_q8_tiled_kernel<16>, grid, dim3(1024), 0, stream, x, out.qs, out.d,
+                       reinterpret_cast<_Float16*>(out.bsums), (int)m, (int)(k / 256));
 }
 
 // The per-32 quantizer (quantize_q8_32, crates/infr-cpu/src/quant.rs:97-117) in the same tiled code
