@@ -1572,7 +1572,7 @@ int infr_hip_execute(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t* c
         // elementwise ops name their second operand per kind; check_elementwise validates it
         if (!bindings[op.x] || !bindings[op.dst] || ((op.kind == INFR_OP_LINEAR || op.kind == INFR_OP_EMBED_GATHER) && !bindings[op.weight]) ||
             (moe && (!bindings[op.router_x] || !bindings[op.router] || !bindings[op.gate_exps] ||
-                     !bindings[op.up_exps] || !bindings[op.down_exps])))
+                     (!op.moe.fused_gate_up && !bindings[op.up_exps]) || !bindings[op.down_exps])))
             return fail(be, INFR_HIP_ERR_INVALID, "execute: unbound tensor");
     }
     if (int rc = schedule_plan(be, plan, bindings)) return rc;
