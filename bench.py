@@ -30,7 +30,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
 # algorithmic bytes per launch -> measured HBM bytes per launch (profiles/gemv_q4k_decode_sweep.md); the
 # figure holds for that launch shape only, so it is looked up by the bytes the timed launch really moved
-MEASURED_TRAFFIC = {2887778304: 2896067761}
+MEASURED_TRAFFIC = {2887778304: 2905303356}
 # prefill Op::Linear (quantizer + strip kernel) at M = 512, K = 4096, N = 12288: HBM bytes per op from the
 # FETCH_SIZE / WRITE_SIZE runs in profiles/mmq_q4k_prefill.md, keyed by the op's integer operations
 MEASURED_TRAFFIC_MMQ = {}
@@ -636,7 +636,7 @@ def main():
     bytes_per_launch = sw.bytes_4096 // k_launches
     achieved = bytes_per_launch / (avg_launch_us * 1e-6) / 1e9
     # HBM bytes per launch of that kernel at the default 36-layer sweep, from two rocprofv3 --pmc
-    # runs of this command (FETCH_SIZE x 1.99786 and WRITE_SIZE x 1.0, the factors a plain
+    # runs of this command (FETCH_SIZE x 1.99788 and WRITE_SIZE x 1.0, the factors a plain
     # 28,311,552-byte device copy in the same runs gives); null for any other launch shape.
     traffic = MEASURED_TRAFFIC.get(bytes_per_launch)
     if traffic is None:
@@ -644,7 +644,8 @@ def main():
               f"algorithmic bytes (MEASURED_TRAFFIC holds {sorted(MEASURED_TRAFFIC)})", file=sys.stderr)
     # what a kernel that only fetches reaches here: a read-only streaming pass over 2 GiB, same run
     probe = be.alloc_uninit(2 << 30)
-    stream_read = be.stream_read_gbs(probe, reps=10)
+    stream_read_plain = be.stream_read_gbs(probe, reps=10)
+    stream_read = be.stream_read_gbs(probe, reps=10, nontemporal=True)  # as the streamed GEMV fetches
     probe.free()
     parity = "skipped (--no-parity)" if args.no_parity else parity_gate_sweep(be, sw, DType.Q4K)
     out = {
@@ -661,11 +662,12 @@ def main():
                    "device": caps["device_name"], "compute_units": caps["compute_units"]},
         "pct_of_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "launches_per_step": n_launch,
-        "roofline": {"bound": "hbm", "kernel": "gemv_fused_kernel<FmtQ4K, 1, 8> (in_f 4096 group)",
+        "roofline": {"bound": "hbm", "kernel": "gemv_fused_kernel<FmtQ4K, 1, 8, false, true> (in_f 4096 group, rows streamed through LDS rings)",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "avg_launch_us": round(avg_launch_us, 3), "bytes_per_launch": bytes_per_launch,
                      "stream_read_GBs": round(stream_read, 1),
+                     "stream_read_plain_loads_GBs": round(stream_read_plain, 1),
                      "frac_of_stream_read": round(achieved / stream_read, 4)},
     }
     sw.free()

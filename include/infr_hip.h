@@ -322,10 +322,12 @@ void infr_hip_reset_shutdown(void); /* tests only: the reference's latch is mono
 int infr_hip_timer_begin(infr_hip_t *be);
 int infr_hip_timer_end(infr_hip_t *be, float *elapsed_ms); /* synchronises */
 /* Measurement aid with no counterpart in the reference: reads the first `bytes` of `src` `reps`
- * times with a plain streaming kernel (16-byte loads, no arithmetic) and reports the device time of
- * those passes - the read bandwidth this device gives a kernel that only fetches, which the
- * HBM-bound GEMVs are compared with. Synchronises. */
-int infr_hip_stream_read(infr_hip_t *be, const infr_hip_buffer_t *src, size_t bytes, int reps, float *elapsed_ms);
+ * times with a plain streaming kernel (16-byte loads, whole lines per instruction, no arithmetic)
+ * and reports the device time of those passes - the read bandwidth this device gives a kernel that
+ * only fetches, which the HBM-bound GEMVs are compared with. `nontemporal` != 0 issues the loads
+ * non-temporally, as the streamed decode GEMV fetches its weights. Synchronises. */
+int infr_hip_stream_read(infr_hip_t *be, const infr_hip_buffer_t *src, size_t bytes, int reps, int nontemporal,
+                         float *elapsed_ms);
 /* Measurement aid with no counterpart in the reference: `iters` rounds of four independent
  * v_mfma_i32_32x32x32_i8 per wave, `waves_per_simd` (1..8) waves on every SIMD, operands in registers
  * (small constants, or pseudo-random bytes when random_data != 0). Reports the device time of one

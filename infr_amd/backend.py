@@ -158,7 +158,7 @@ SYMBOLS = {
     "infr_hip_reset_shutdown": (None, []),
     "infr_hip_timer_begin": (C.c_int, [_vp]),
     "infr_hip_timer_end": (C.c_int, [_vp, C.POINTER(C.c_float)]),
-    "infr_hip_stream_read": (C.c_int, [_vp, _vp, C.c_size_t, C.c_int, C.POINTER(C.c_float)]),
+    "infr_hip_stream_read": (C.c_int, [_vp, _vp, C.c_size_t, C.c_int, C.c_int, C.POINTER(C.c_float)]),
     "infr_hip_mfma_i8_peak": (C.c_int, [_vp, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_double)]),
     "infr_synth_normal_f32": (None, [C.c_uint64, C.c_float, C.c_float, C.c_size_t, _vp]),
     "infr_synth_weight": (C.c_size_t, [C.c_int, C.c_uint64, C.c_float, C.c_size_t, C.c_size_t, _vp]),
@@ -693,11 +693,12 @@ class HipBackend:
             C.byref(opt), dst._h, sel_idx._h if sel_idx else None, sel_w._h if sel_w else None))
 
     # -- measurement --
-    def stream_read_gbs(self, buf: Buffer, nbytes: int | None = None, reps: int = 10) -> float:
-        """GB/s of a plain read-only streaming kernel over ``buf`` (what fetching alone reaches)."""
+    def stream_read_gbs(self, buf: Buffer, nbytes: int | None = None, reps: int = 10, nontemporal: bool = False) -> float:
+        """GB/s of a read-only streaming kernel over ``buf`` (what fetching alone reaches), with plain
+        or non-temporal loads."""
         n = buf.len_bytes() if nbytes is None else nbytes
         ms = C.c_float()
-        self._check(self._lib.infr_hip_stream_read(self._h, buf._h, n, reps, C.byref(ms)))
+        self._check(self._lib.infr_hip_stream_read(self._h, buf._h, n, reps, 1 if nontemporal else 0, C.byref(ms)))
         return n * reps / (ms.value * 1e-3) / 1e9
 
     def mfma_i8_peak_tops(self, waves_per_simd: int = 4, iters: int = 4096, random_data: bool = True) -> float:

@@ -1626,16 +1626,18 @@ int infr_hip_timer_end(infr_hip_t* be, float* elapsed_ms) {
     return INFR_HIP_OK;
 }
 
-int infr_hip_stream_read(infr_hip_t* be, const infr_hip_buffer_t* src, size_t bytes, int reps, float* elapsed_ms) {
+int infr_hip_stream_read(infr_hip_t* be, const infr_hip_buffer_t* src, size_t bytes, int reps, int nontemporal,
+                         float* elapsed_ms) {
     if (!be || !src || !elapsed_ms || reps <= 0) return fail(be, INFR_HIP_ERR_INVALID, "stream_read: bad argument");
     if (bytes > src->len || bytes < 16) return fail(be, INFR_HIP_ERR_INVALID, "stream_read: size outside the buffer");
     if (int rc = check_latch(be)) return rc;
     const int wgs = std::max(1, be->props.multiProcessorCount) * 64;
     int* out = nullptr;
     HIP_TRY(be, hipMalloc((void**)&out, sizeof(int) * (size_t)wgs));
-    infr::launch_stream_read(src->ptr, bytes, out, wgs, be->stream);  // untimed first pass
+    infr::launch_stream_read(src->ptr, bytes, out, wgs, nontemporal != 0, be->stream);  // untimed first pass
     hipError_t e = hipEventRecord(be->ev0, be->stream);
-    for (int r = 0; r < reps && e == hipSuccess; ++r) infr::launch_stream_read(src->ptr, bytes, out, wgs, be->stream);
+    for (int r = 0; r < reps && e == hipSuccess; ++r)
+        infr::launch_stream_read(src->ptr, bytes, out, wgs, nontemporal != 0, be->stream);
     if (e == hipSuccess) e = hipEventRecord(be->ev1, be->stream);
     if (e == hipSuccess) e = hipEventSynchronize(be->ev1);
     if (e == hipSuccess) e = hipEventElapsedTime(elapsed_ms, be->ev0, be->ev1);

@@ -125,9 +125,10 @@ void launch_add(const float* a, const float* b, float* out, size_t n, hipStream_
 }
 
 // Measurement aid: a read-only streaming pass over `bytes` of device memory with nothing but
-// 16-byte loads and a xor, i.e. what a kernel that only had to fetch the weights could reach on
-// this device. Each workgroup walks 16 KB chunks grid-stride; one word per workgroup is written so
+// 16-byte loads (plain or non-temporal) and a xor, i.e. what a kernel that only had to fetch the
+// weights could reach on this device. Each workgroup walks 16 KB chunks grid-stride; one word per workgroup is written so
 // the loads cannot be dropped.
+template <bool NT>
 __global__ __launch_bounds__(256) void stream_read_kernel(const v4i* __restrict__ src, size_t n_vec,
                                                           int* __restrict__ out) {
     const size_t chunk = 1024;  // v4i per workgroup per iteration: 4 per thread
@@ -137,7 +138,7 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const v4i* __restrict_
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             const size_t i = base + k * 256 + threadIdx.x;
-            v[k] = i < n_vec ? gload<v4i>(src + i) : v4i{0, 0, 0, 0};
+            v[k] = i < n_vec ? (NT ? gload_stream<v4i>(src + i) : gload<v4i>(src + i)) : v4i{0, 0, 0, 0};
         }
 #pragma unroll
         for (int k = 0; k < 4; ++k) acc ^= v[k];
@@ -146,10 +147,14 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const v4i* __restrict_
     if (threadIdx.x == 0 || r == 0x5EEDF00D) out[blockIdx.x] = r;
 }
 
-void launch_stream_read(const void* src, size_t bytes, int* out, int workgroups, hipStream_t stream) {
+void launch_stream_read(const void* src, size_t bytes, int* out, int workgroups, bool nontemporal, hipStream_t stream) {
     if (bytes < 16 || workgroups <= 0) return;
-    hipLaunchKernelGGL(stream_read_kernel, dim3((unsigned)workgroups), dim3(256), 0, stream,
-                       static_cast<const v4i*>(src), bytes / 16, out);
+    if (nontemporal)
+        hipLaunchKernelGGL(stream_read_kernel<true>, dim3((unsigned)workgroups), dim3(256), 0, stream,
+                           static_cast<const v4i*>(src), bytes / 16, out);
+    else
+        hipLaunchKernelGGL(stream_read_kernel<false>, dim3((unsigned)workgroups), dim3(256), 0, stream,
+                           static_cast<const v4i*>(src), bytes / 16, out);
 }
 
 // Measurement aid: nothing but v_mfma_i32_32x32x32_i8 on four independent accumulator tiles per

@@ -82,6 +82,26 @@ struct FmtQ4K {
             r.hdr = r.qa = r.qb = v4i{0, 0, 0, 0};
         }
     }
+    // The same pieces out of a wave's LDS ring of the weight bytes: `pos` is the ring position of the
+    // step's first byte (below `ring_bytes`). Blocks are whole 16-byte pieces at 16-byte boundaries
+    // and the ring is a whole number of pieces, so no piece straddles the wrap.
+    static constexpr uint32_t kStepBytes = 16 * 144;
+    __device__ static void load_row_ring(Row& r, const uint8_t* ring, uint32_t pos, uint32_t ring_bytes, int lane, bool ok) {
+        const int p = lane & 3;
+        uint32_t o0 = pos + (uint32_t)(lane >> 2) * 144;
+        uint32_t o1 = o0 + 16 + p * 32, o2 = o0 + 32 + p * 32;
+        o0 = o0 >= ring_bytes ? o0 - ring_bytes : o0;
+        o1 = o1 >= ring_bytes ? o1 - ring_bytes : o1;
+        o2 = o2 >= ring_bytes ? o2 - ring_bytes : o2;
+        const v4i hdr = *reinterpret_cast<const v4i*>(ring + o0);
+        const v4i qa = *reinterpret_cast<const v4i*>(ring + o1);
+        const v4i qb = *reinterpret_cast<const v4i*>(ring + o2);
+        // a lane without a block: d = dmin = 0 makes its term +0.0 whatever the other bytes are
+        r.hdr = hdr;
+        r.hdr.x = ok ? hdr.x : 0;
+        r.qa = qa;
+        r.qb = qb;
+    }
     __device__ static void load_acts(Acts& a, const ActPtrs& s, int t, int lane, bool ok) {
         if (ok) {
             const int b = t * 16 + (lane >> 2), p = lane & 3;
@@ -519,6 +539,25 @@ struct FmtQ5K {
         } else {
             r.hdr = r.ha = r.hb = r.qa = r.qb = v4i{0, 0, 0, 0};
         }
+    }
+    // The same pieces out of a wave's LDS ring (see FmtQ4K::load_row_ring).
+    static constexpr uint32_t kStepBytes = 16 * 176;
+    __device__ static void load_row_ring(Row& r, const uint8_t* ring, uint32_t pos, uint32_t ring_bytes, int lane, bool ok) {
+        const int p = lane & 3;
+        uint32_t o[5];
+        o[0] = pos + (uint32_t)(lane >> 2) * 176;
+        o[1] = o[0] + 16;
+        o[2] = o[0] + 32;
+        o[3] = o[0] + 48 + p * 32;
+        o[4] = o[0] + 64 + p * 32;
+#pragma unroll
+        for (int i = 0; i < 5; ++i) o[i] = o[i] >= ring_bytes ? o[i] - ring_bytes : o[i];
+        r.hdr = *reinterpret_cast<const v4i*>(ring + o[0]);
+        r.ha = *reinterpret_cast<const v4i*>(ring + o[1]);
+        r.hb = *reinterpret_cast<const v4i*>(ring + o[2]);
+        r.qa = *reinterpret_cast<const v4i*>(ring + o[3]);
+        r.qb = *reinterpret_cast<const v4i*>(ring + o[4]);
+        r.hdr.x = ok ? r.hdr.x : 0;  // d = dmin = 0: a lane without a block contributes +0.0
     }
     __device__ static void load_acts(Acts& a, const ActPtrs& s, int t, int lane, bool ok) {
         FmtQ4K::load_acts(a, s, t, lane, ok);

@@ -214,13 +214,17 @@ __device__ __forceinline__ float fused_gated_act(int act, bool has_clamp, float 
 // Fused + grouped form. LDS: qs[in_f] | d[in_f/32] | bsums[in_f/32] | bsums16[in_f/16] | per-wave
 // ordered-sum scratch.
 // STAGES: the per-block integers of every row also go to single.st_a / st_b (single-op launches only).
-template <typename F, int STEPS, int NW, bool STAGES>
+// STREAMED: the weight rows go through per-wave LDS rings (gemv_rows_streamed). LDS is then
+// rings[NW] | per-wave ordered-sum scratch, and the activation arrays lie over the start of the
+// rings: they are dead once every wave holds its activation registers (a second barrier).
+template <typename F, int STEPS, int NW, bool STAGES, bool STREAMED = false>
 __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, int single_rows,
                                                              const GemvTile* __restrict__ tiles,
                                                              int in_f) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    // (STREAMED: as a scalar, so that the row and chunk bookkeeping runs on the scalar unit)
+    const int wave = STREAMED ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : (int)(threadIdx.x >> 6);
 
     // This workgroup's rows: one table entry, or computed from the single op's descriptor.
     GemvTile tile;
@@ -286,7 +290,15 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, 
     bool ok[STEPS];
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) ok[t] = has_rows && F::valid(t, lane, n_units);
-    F::load_row(first[0], tile.w + (size_t)row0 * tile.bpr, 0, lane, ok[0]);
+    // STREAMED: the image of this wave's rows starts at the line that holds their first byte
+    const uint8_t* span = tile.w + (size_t)row0 * tile.bpr;
+    const uint32_t head = (uint32_t)(reinterpret_cast<uintptr_t>(span) & 127);
+    const uint32_t total = has_rows ? (head + (uint32_t)(row_end - row0) * tile.bpr + 127) & ~127u : 0;
+    RingChunk chunks_ahead;
+    if constexpr (STREAMED) {
+        if (has_rows) ring_issue(span - head, 0, total, lane, chunks_ahead.v);  // (wave-uniform)
+    }
+    else F::load_row(first[0], tile.w + (size_t)row0 * tile.bpr, 0, lane, ok[0]);
     // An absorbed producer of x (workgroup-uniform branch): every workgroup recomputes the vector
     // from the producer's inputs - cheaper than a launch of its own - and the op's first
     // workgroup stores it where the producer would have.
@@ -327,7 +339,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, 
             }
         }
     }
-    if constexpr (kFirstWhole) {
+    if constexpr (kFirstWhole && !STREAMED) {
         asm volatile("" ::: "memory");  // not before the loads above have been waited for
 #pragma unroll
         for (int t = 1; t < STEPS; ++t) F::load_row(first[t], tile.w + (size_t)row0 * tile.bpr, t, lane, ok[t]);
@@ -340,20 +352,28 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, 
                                       l_bs, F::kPer32 ? nullptr : l_bs16);
     }
     __syncthreads();
-    if (!has_rows) {
-            return;
-    }
+    if (!STREAMED && !has_rows) return;
 
     ActPtrs act{l_qs, l_d, l_bs, l_bs16};
     typename F::Acts acts[STEPS];
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) F::load_acts(acts[t], act, t, lane, ok[t]);
-    float* osum = reinterpret_cast<float*>(lds + in_f + in_f / 2) + wave * RowSumScratch<F, STEPS>::kFloatsPerWave;
     // stage outputs are indexed by the op's row: offset them to the tile's first
     const size_t st_off = (size_t)first_row * (F::kBlockElems == 64 ? 2 * n_units : n_units);
     const StagePtrs st{STAGES ? single.st_a + st_off : nullptr, STAGES && single.st_b ? single.st_b + st_off : nullptr};
-    gemv_rows<F, STEPS, STAGES, kFirstWhole>(tile.w, tile.bpr, first, acts, ok, tile.y, n_units, row0, row_end, lane,
-                                             st, osum, tile.fus.add_b, tile.fus.add_dst, add_first);
+    if constexpr (STREAMED) {
+        __syncthreads();  // the rings lie over the activation arrays
+        if (!has_rows) return;
+        float* osum = reinterpret_cast<float*>(lds + (size_t)NW * WeightRingOf<F>::kBytes) +
+                      wave * RowSumScratch<F, STEPS>::kFloatsPerWave;
+        gemv_rows_streamed<F, STEPS, STAGES>(span - head, head, total, tile.bpr, chunks_ahead,
+                                             lds + (size_t)wave * WeightRingOf<F>::kBytes, acts, ok, tile.y, n_units,
+                                             row0, row_end, lane, st, osum, tile.fus.add_dst, add_first);
+    } else {
+        float* osum = reinterpret_cast<float*>(lds + in_f + in_f / 2) + wave * RowSumScratch<F, STEPS>::kFloatsPerWave;
+        gemv_rows<F, STEPS, STAGES, kFirstWhole>(tile.w, tile.bpr, first, acts, ok, tile.y, n_units, row0, row_end, lane,
+                                                 st, osum, tile.fus.add_b, tile.fus.add_dst, add_first);
+    }
 }
 
 // ───────────────────────────────────── launch ─────────────────────────────────────
@@ -577,12 +597,33 @@ static bool plan_group_fmt(size_t in_f, const GemvOpDesc* ops, int n, GemvGroupP
         wg = 0;
         for (int i = 0; i < n; ++i) wg += (int)(((size_t)ops[i].out_f + rows_per_wg - 1) / rows_per_wg);
     }
+    const size_t sum_scratch =
+        (size_t)nw * (F::kOrdered ? 16 * (16 * steps + 4) : (F::kLaneSums ? LaneSums::kFloatsPerWave : 0)) * sizeof(float);
     plan->total_wgs = wg;
     plan->waves_per_wg = nw;
     plan->rows_per_wg = (int)rows_per_wg;
     // qs + d + bsums + bsums16, then the ordered-sum scratch of every wave
-    plan->lds_bytes = in_f + in_f / 2 +
-                      (size_t)nw * (F::kOrdered ? 16 * (16 * steps + 4) : (F::kLaneSums ? LaneSums::kFloatsPerWave : 0)) * sizeof(float);
+    plan->lds_bytes = in_f + in_f / 2 + sum_scratch;
+    // Many rounds of workgroups: the weight bytes go through per-wave LDS rings as whole lines,
+    // non-temporally (gemv_rows_streamed), 64 rows per eight-wave workgroup. Launches of a few rounds
+    // measured slower that way - the ring adds a trip through LDS to every wave's start-up - and keep
+    // the direct loads.
+    plan->streamed = false;
+    if constexpr (HasRingLoads<F>::value) {
+        bool aligned = true;  // the ring's 16-byte pieces need 16-byte-aligned rows
+        for (int i = 0; i < n; ++i)
+            aligned = aligned && reinterpret_cast<uintptr_t>(ops[i].w) % 16 == 0 && ops[i].bpr % 16 == 0 && ops[i].st_a == nullptr;
+        // (measured crossover: 139264 rows of 4096 columns, 98304 rows of 12288)
+        const size_t wg64 = wgs_at(64);
+        if (aligned && steps <= 3 && cus > 0 && wg64 > (size_t)8 * cus &&
+            in_f + in_f / 2 <= (size_t)8 * WeightRingOf<F>::kBytes) {
+            plan->streamed = true;
+            plan->waves_per_wg = 8;
+            plan->rows_per_wg = 64;
+            plan->total_wgs = (int)wg64;
+            plan->lds_bytes = (size_t)8 * WeightRingOf<F>::kBytes + (size_t)8 * 16 * (16 * steps + 4) * sizeof(float);
+        }
+    }
     return true;
 }
 
@@ -613,6 +654,27 @@ template <typename F>
 static bool launch_fused_fmt(size_t in_f, const GemvOpDesc& op, const GemvTile* tiles_dev,
                              const GemvGroupPlan& plan, hipStream_t stream) {
     const int steps = (int)((in_f + F::kElemsPerStep - 1) / F::kElemsPerStep);
+    if constexpr (HasRingLoads<F>::value) {
+        if (plan.streamed) {
+            if (plan.waves_per_wg != 8 || steps > 3 || op.st_a != nullptr || plan.lds_bytes > 64 * 1024) return false;
+            const dim3 grid((unsigned)plan.total_wgs), block(512);
+            switch (steps) {
+            case 1:
+                hipLaunchKernelGGL((gemv_fused_kernel<F, 1, 8, false, true>), grid, block, plan.lds_bytes, stream, op,
+                                   plan.rows_per_wg, tiles_dev, (int)in_f);
+                break;
+            case 2:
+                hipLaunchKernelGGL((gemv_fused_kernel<F, 2, 8, false, true>), grid, block, plan.lds_bytes, stream, op,
+                                   plan.rows_per_wg, tiles_dev, (int)in_f);
+                break;
+            default:
+                hipLaunchKernelGGL((gemv_fused_kernel<F, 3, 8, false, true>), grid, block, plan.lds_bytes, stream, op,
+                                   plan.rows_per_wg, tiles_dev, (int)in_f);
+                break;
+            }
+            return true;
+        }
+    }
     if (op.st_a != nullptr) {
         // the integer-stage outputs: the same kernel, single-op launches only
         if (tiles_dev != nullptr) return false;

@@ -253,6 +253,131 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
     }
 }
 
+// ───────────────────────────── rows streamed through LDS ─────────────────────────────
+// A wave's rows [row0, row_end) are one contiguous span of the weight matrix. gemv_rows reads it the
+// way the lanes consume it - 16 bytes of a block header here, 32 bytes of nibbles there - so every
+// load instruction touches a part of many 128-byte lines and every line is touched by three or more
+// instructions. That access pattern must not be non-temporal (a line is dropped after its first
+// touch and fetched again: 4.9 TB/s measured), and plain loads stop at 6.2-6.5 TB/s on this device.
+// Here the span is instead fetched as it lies in memory: whole lines, 1024 contiguous bytes per load
+// instruction, non-temporal (7.1-7.3 TB/s measured for this shape of kernel), in chunks of a few
+// instructions into a ring in LDS that belongs to the wave alone; the lanes then pick their block
+// pieces out of the ring with the format's load_row_ring. One chunk is in flight in registers while
+// the previous one is consumed. No barrier is involved: a wave's LDS operations execute in order.
+//
+// The image in the ring starts at `origin`, the 128-byte line that holds the span's first byte
+// (`head` bytes into it), and ends with the line that holds its last byte (`total` bytes in all):
+// bytes outside the span but inside those two lines are fetched and never looked at (a line never
+// crosses a page, so they are readable). Ring offsets are image offsets modulo the ring size: a chunk
+// is written when less than one wave step of older bytes is still to be consumed, so a ring of a step
+// plus a chunk never overwrites bytes that are still wanted.
+struct WeightRing {
+    // 1024-byte load instructions per chunk: two and three measured alike (6.74 TB/s on 216 matrices
+    // of 4096 columns) and four 6 % slower at 64 rows per workgroup; two keeps the ring smallest
+    static constexpr int kInstr = 2;
+    static constexpr uint32_t kChunk = kInstr * 1024;
+};
+template <typename F, typename = void>
+struct HasRingLoads : std::false_type {};
+template <typename F>
+struct HasRingLoads<F, std::void_t<decltype(&F::load_row_ring)>> : std::true_type {};
+// Ring bytes per wave: a chunk is written only when less than one wave step of older bytes is still
+// to be consumed, so a step plus a chunk always fit.
+template <typename F>
+struct WeightRingOf {
+    static constexpr uint32_t kBytes = F::kStepBytes + WeightRing::kChunk;
+    static_assert(kBytes % 16 == 0, "pieces are 16 bytes");
+};
+struct RingChunk {
+    v4i v[WeightRing::kInstr];
+};
+
+// Chunk `c` of the image: lane l takes bytes [16 l, 16 l + 16) of each of its 1024-byte pieces.
+// Pieces past the image's end read its last piece again instead of being masked off (total >= 128):
+// with every load unconditional the compiler can count how many are in flight and wait for the
+// oldest chunk alone; behind a per-lane branch it waits for all of them.
+__device__ __forceinline__ void ring_issue(const uint8_t* origin, uint32_t c, uint32_t total, int lane,
+                                           v4i (&v)[WeightRing::kInstr]) {
+#pragma unroll
+    for (int k = 0; k < WeightRing::kInstr; ++k) {
+        const uint32_t o = c * WeightRing::kChunk + k * 1024 + lane * 16;
+        v[k] = gload_stream<v4i>(origin + (o < total ? o : total - 16));
+    }
+}
+// gemv_rows for an ordered format with load_row_ring, fed from the ring. `rc` holds chunk 0 of the
+// image (the caller requests it ahead of its prologue). A chunk's registers are written to the ring
+// and at once reloaded with the next chunk, which is then in flight while the rows that the ring now
+// holds are computed (a second register set would have to be copied into the first, and a copy
+// waits for the load it reads). row0, row_end, head and total must be wave-uniform scalars.
+// Every output equals gemv_rows' bit for bit: the per-block terms and the order in which they are
+// added are the same code.
+template <typename F, int STEPS, bool STAGES>
+__device__ __forceinline__ void gemv_rows_streamed(const uint8_t* origin, uint32_t head, uint32_t total, size_t bpr,
+                                                   RingChunk& rc, uint8_t* ring,
+                                                   const typename F::Acts (&acts)[STEPS], const bool (&ok)[STEPS],
+                                                   float* __restrict__ y, int n_units, int row0, int row_end,
+                                                   int lane, const StagePtrs& st, float* osum,
+                                                   float* add_dst = nullptr, float add_first = 0.0f) {
+    static_assert(F::kOrdered, "the streamed loop adds per-block terms in block order");
+    // (a wave has at most 64 rows here: every residual is among the lanes' prefetched values, and
+    // the loop holds no load but the chunks' - one more would be waited for together with them)
+    auto residual = [&](int r) { return __shfl(add_first, (r - row0) & 63, kWave); };
+    const bool plain_y = y != add_dst;
+    constexpr int LS = OrderedSum<STEPS>::kRowStride;
+    constexpr uint32_t kRing = WeightRingOf<F>::kBytes;
+    uint32_t chunks = 0;  // chunks of the image written to the ring so far
+    uint32_t wpos = 0;    // ring position of the next chunk (image offset modulo the ring size)
+    auto advance = [&]() {
+#pragma unroll
+        for (int k = 0; k < WeightRing::kInstr; ++k) {
+            uint32_t o = wpos + k * 1024 + lane * 16;
+            o = o >= kRing ? o - kRing : o;
+            *reinterpret_cast<v4i*>(ring + o) = rc.v[k];
+        }
+        ++chunks;
+        ring_issue(origin, chunks, total, lane, rc.v);
+        wpos += WeightRing::kChunk;
+        wpos = wpos >= kRing ? wpos - kRing : wpos;
+    };
+    int in_batch = 0, batch_row0 = row0;
+    uint32_t rpos = head;  // ring position of the current row's first byte
+    for (int row = row0; row < row_end; ++row) {
+        const uint32_t roff = head + (uint32_t)(row - row0) * (uint32_t)bpr;
+#pragma unroll
+        for (int t = 0; t < STEPS; ++t) {
+            const uint32_t step_end = (uint32_t)(t + 1) * F::kStepBytes < (uint32_t)bpr ? (uint32_t)(t + 1) * F::kStepBytes : (uint32_t)bpr;
+            while (chunks * WeightRing::kChunk < roff + step_end) advance();
+            typename F::Row r;
+            uint32_t spos = rpos + (uint32_t)t * (F::kStepBytes % kRing);
+            while (spos >= kRing) spos -= kRing;
+            F::load_row_ring(r, ring, spos, kRing, lane, ok[t]);
+            const float term = F::template term<STAGES>(r, acts[t], t, lane, ok[t], st, (size_t)row * n_units);
+            if ((lane & 3) == 0) osum[in_batch * LS + t * 16 + (lane >> 2)] = term;
+        }
+        rpos += (uint32_t)(bpr % kRing);
+        rpos = rpos >= kRing ? rpos - kRing : rpos;
+        if (++in_batch == 16 || row + 1 == row_end) {
+            const float resid = add_dst ? residual(batch_row0 + lane) : 0.0f;
+            if (lane < in_batch) {
+                const v4f* tr = reinterpret_cast<const v4f*>(osum + lane * LS);
+                float acc = 0.0f;
+#pragma unroll
+                for (int k = 0; k < 4 * STEPS; ++k) {
+                    const v4f v = tr[k];
+                    acc += v.x;
+                    acc += v.y;
+                    acc += v.z;
+                    acc += v.w;
+                }
+                if (plain_y) gstore<float>(y + batch_row0 + lane, acc);
+                if (add_dst) gstore<float>(add_dst + batch_row0 + lane, acc + resid);
+            }
+            batch_row0 = row + 1;
+            in_batch = 0;
+        }
+    }
+}
+
 // Folded form for short rows of the 16-blocks-per-step formats (Q4_K, Q6_K) with nb <= 8 blocks
 // per row: consecutive weight rows are contiguous in memory, so one wave step takes
 // rps = 16 / nb whole rows at once (block slot q = lane / 4 -> row q / nb, block q % nb) instead of

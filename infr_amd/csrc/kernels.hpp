@@ -112,6 +112,7 @@ struct GemvGroupPlan {
     int waves_per_wg = 0;
     int rows_per_wg = 0;
     size_t lds_bytes = 0;
+    bool streamed = false;  // the weight bytes go through per-wave LDS rings (gemv_rows_streamed)
 };
 
 // Chooses workgroup shape and rows per wave for a group. false = no kernel for (dtype, in_f).
@@ -197,7 +198,7 @@ void launch_embed_gather(int dtype, const uint8_t* table, size_t bpr, size_t tot
                          size_t rows, size_t ne, float scale, float* dst, hipStream_t stream);
 
 // Read-only streaming pass (measurement aid): `out` holds one int per workgroup.
-void launch_stream_read(const void* src, size_t bytes, int* out, int workgroups, hipStream_t stream);
+void launch_stream_read(const void* src, size_t bytes, int* out, int workgroups, bool nontemporal, hipStream_t stream);
 void launch_mfma_i8_peak(int* out, int workgroups, int iters, int random_data, hipStream_t stream);
 
 // The decode-GEMV launchers of one weight format. Each format's kernels are instantiated in one

@@ -138,6 +138,7 @@ def test_measurement_probes_report_sane_rates(be):
     with pytest.raises(InfrError):
         be.mfma_i8_peak_tops(2, 0, True)
     buf = be.alloc(64 << 20)
-    gbs = be.stream_read_gbs(buf, reps=3)
+    for nt in (False, True):
+        gbs = be.stream_read_gbs(buf, reps=3, nontemporal=nt)
+        assert 100.0 < gbs < 8200.0, (nt, gbs)
     buf.free()
-    assert 100.0 < gbs < 8200.0, gbs

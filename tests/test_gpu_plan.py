@@ -789,3 +789,41 @@ def test_prefill_linears_of_one_level_share_the_activation_quantization(be):
             want = orc.linear(dt, w, xs[xi].reshape(m, in_f)[toks].ravel(), len(toks), in_f, out_f)
             rel = np.linalg.norm(got.astype(np.float64) - want) / np.linalg.norm(want)
             assert rel <= 2e-6, (rep, int(dt), out_f, rel)
+
+
+@pytest.mark.parametrize("dtype,in_f", [(DType.Q4K, 1024), (DType.Q4K, 1536), (DType.Q4K, 4096), (DType.Q4K, 5120),
+                                        (DType.Q4K, 8192), (DType.Q4K, 12288), (DType.Q5K, 1536), (DType.Q5K, 4096),
+                                        (DType.Q5K, 12288)])
+def test_many_round_decode_groups_stream_their_rows_through_lds(be, dtype, in_f):
+    # A level of one-token Q4_K / Q5_K Linears with enough rows for many rounds of workgroups (over 131072)
+    # takes the form whose waves fetch their rows as whole lines into LDS rings. Row counts that are
+    # not multiples of the tile height, rows of 4.5 and 6.75 lines (waves start mid-line), rows
+    # shorter than a wave step, rows of two and three wave steps with a short last step; two
+    # activations. Ordered sums: every output equals the oracle's bits.
+    rows_each = [16387, 20011, 9001] if in_f <= 4096 else [6007, 4001, 3003]
+    reps = -(-140000 // sum(rows_each))
+    g, binds = Graph(), Bindings()
+    xs = [synth_normal_f32(31 + i, in_f) for i in range(2)]
+    xids = [g.input(TensorDesc((1, in_f), DType.F32)) for _ in xs]
+    for xid, x in zip(xids, xs):
+        binds.bind(xid, be.upload_new(x))
+    ws = [synth_weight(dtype, 500 + i, r, in_f) for i, r in enumerate(rows_each)]
+    wbufs = [be.upload_new(w) for w in ws]
+    cases = []
+    for rep in range(reps):
+        for i, r in enumerate(rows_each):
+            wid = g.weight(TensorDesc((r, in_f), dtype))
+            yid = g.output(TensorDesc((1, r), DType.F32))
+            yb = be.alloc(r * 4)
+            binds.bind(wid, wbufs[i]).bind(yid, yb)
+            xi = (rep + i) % 2
+            g.push(Linear(xids[xi], wid, yid, 1, in_f, r))
+            cases.append((i, xi, yb))
+    plan = be.compile(g)
+    want = {(i, xi): orc.linear(dtype, ws[i], xs[xi], 1, in_f, rows_each[i]).ravel()
+            for i in range(len(ws)) for xi in range(2)}
+    for _ in range(2):  # record, then replay
+        be.execute(plan, binds)
+        for i, xi, yb in cases:
+            got = be.download(yb, np.empty(rows_each[i], np.float32))
+            assert np.array_equal(bits(got), bits(want[(i, xi)])), (i, xi)
