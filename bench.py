@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
 MEASURED_TRAFFIC = {2887778304: 2905303356}
 # prefill Op::Linear (quantizer + strip kernel) at M = 512, K = 4096, N = 12288: HBM bytes per op from the
 # FETCH_SIZE / WRITE_SIZE runs in profiles/mmq_q4k_prefill.md, keyed by the op's integer operations
-MEASURED_TRAFFIC_MMQ = {}
+MEASURED_TRAFFIC_MMQ = {51539607552: 83607984}
 INT8_PEAK_TOPS = 5000.0    # MI355X dense int8 MFMA, published
 
 # (name, out_f, in_f) of one Qwen3-8B decoder layer

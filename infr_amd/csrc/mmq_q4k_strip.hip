@@ -68,7 +68,12 @@ __device__ __forceinline__ int scale_codes4(uint32_t codes, uint32_t digit) {
 // a block; so the read and its wait are written out. The compiler does not count these reads in
 // its own lgkmcnt bookkeeping: LDS accesses complete in order, so its waits can only cover more than
 // they need to, never less, and lds_wait<N> is exact when nothing else was issued in between and
-// stricter otherwise.
+// stricter otherwise. That argument holds for LDS traffic only: scalar memory loads share lgkmcnt
+// and return out of order, so a scalar load issued between an ahead-read and its lds_wait<N> could
+// let the wait pass with the LDS read still outstanding. The block loop therefore has no scalar
+// operand that is not in a register before it starts (kernel arguments, strides and table entries
+// are all read in the prologue), and the strip route's bit-identity tests at 512 / 1024 / 2048
+// tokens would show a stale fragment.
 template <int OFFSET>
 __device__ __forceinline__ v4i lds_read16_ahead(uint32_t addr) {
     v4i r;
