@@ -294,7 +294,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, 
     const uint8_t* span = tile.w + (size_t)row0 * tile.bpr;
     const uint32_t head = (uint32_t)(reinterpret_cast<uintptr_t>(span) & 127);
     const uint32_t total = has_rows ? (head + (uint32_t)(row_end - row0) * tile.bpr + 127) & ~127u : 0;
-    RingChunk chunks_ahead;
+    RingChunk<WeightRing::instr(STEPS)> chunks_ahead;
     if constexpr (STREAMED) {
         if (has_rows) ring_issue(span - head, 0, total, lane, chunks_ahead.v);  // (wave-uniform)
     }
@@ -364,10 +364,10 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, 
     if constexpr (STREAMED) {
         __syncthreads();  // the rings lie over the activation arrays
         if (!has_rows) return;
-        float* osum = reinterpret_cast<float*>(lds + (size_t)NW * WeightRingOf<F>::kBytes) +
+        float* osum = reinterpret_cast<float*>(lds + (size_t)NW * WeightRingOf<F, STEPS>::kBytes) +
                       wave * RowSumScratch<F, STEPS>::kFloatsPerWave;
         gemv_rows_streamed<F, STEPS, STAGES>(span - head, head, total, tile.bpr, chunks_ahead,
-                                             lds + (size_t)wave * WeightRingOf<F>::kBytes, acts, ok, tile.y, n_units,
+                                             lds + (size_t)wave * WeightRingOf<F, STEPS>::kBytes, acts, ok, tile.y, n_units,
                                              row0, row_end, lane, st, osum, tile.fus.add_dst, add_first);
     } else {
         float* osum = reinterpret_cast<float*>(lds + in_f + in_f / 2) + wave * RowSumScratch<F, STEPS>::kFloatsPerWave;
@@ -615,13 +615,14 @@ static bool plan_group_fmt(size_t in_f, const GemvOpDesc* ops, int n, GemvGroupP
             aligned = aligned && reinterpret_cast<uintptr_t>(ops[i].w) % 16 == 0 && ops[i].bpr % 16 == 0 && ops[i].st_a == nullptr;
         // (measured crossover: 139264 rows of 4096 columns, 98304 rows of 12288)
         const size_t wg64 = wgs_at(64);
+        const size_t ring_bytes = steps == 1 ? WeightRingOf<F, 1>::kBytes : WeightRingOf<F, 2>::kBytes;
         if (aligned && steps <= 3 && cus > 0 && wg64 > (size_t)8 * cus &&
-            in_f + in_f / 2 <= (size_t)8 * WeightRingOf<F>::kBytes) {
+            in_f + in_f / 2 <= (size_t)8 * ring_bytes) {
             plan->streamed = true;
             plan->waves_per_wg = 8;
             plan->rows_per_wg = 64;
             plan->total_wgs = (int)wg64;
-            plan->lds_bytes = (size_t)8 * WeightRingOf<F>::kBytes + (size_t)8 * 16 * (16 * steps + 4) * sizeof(float);
+            plan->lds_bytes = (size_t)8 * ring_bytes + (size_t)8 * 16 * (16 * steps + 4) * sizeof(float);
         }
     }
     return true;
@@ -656,22 +657,20 @@ static bool launch_fused_fmt(size_t in_f, const GemvOpDesc& op, const GemvTile* 
     const int steps = (int)((in_f + F::kElemsPerStep - 1) / F::kElemsPerStep);
     if constexpr (HasRingLoads<F>::value) {
         if (plan.streamed) {
-            if (plan.waves_per_wg != 8 || steps > 3 || op.st_a != nullptr || plan.lds_bytes > 64 * 1024) return false;
+            if (plan.waves_per_wg != 8 || steps > 3 || op.st_a != nullptr) return false;
             const dim3 grid((unsigned)plan.total_wgs), block(512);
-            switch (steps) {
-            case 1:
-                hipLaunchKernelGGL((gemv_fused_kernel<F, 1, 8, false, true>), grid, block, plan.lds_bytes, stream, op,
-                                   plan.rows_per_wg, tiles_dev, (int)in_f);
-                break;
-            case 2:
-                hipLaunchKernelGGL((gemv_fused_kernel<F, 2, 8, false, true>), grid, block, plan.lds_bytes, stream, op,
-                                   plan.rows_per_wg, tiles_dev, (int)in_f);
-                break;
-            default:
-                hipLaunchKernelGGL((gemv_fused_kernel<F, 3, 8, false, true>), grid, block, plan.lds_bytes, stream, op,
-                                   plan.rows_per_wg, tiles_dev, (int)in_f);
-                break;
-            }
+#define INFR_STREAMED(N)                                                                                          \
+    do {                                                                                                          \
+        if (plan.lds_bytes > 64 * 1024)                                                                           \
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_fused_kernel<F, N, 8, false, true>),    \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan.lds_bytes);           \
+        hipLaunchKernelGGL((gemv_fused_kernel<F, N, 8, false, true>), grid, block, plan.lds_bytes, stream, op,    \
+                           plan.rows_per_wg, tiles_dev, (int)in_f);                                               \
+    } while (0)
+            if (steps == 1) INFR_STREAMED(1);
+            else if (steps == 2) INFR_STREAMED(2);
+            else INFR_STREAMED(3);
+#undef INFR_STREAMED
             return true;
         }
     }

@@ -272,10 +272,12 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
 // is written when less than one wave step of older bytes is still to be consumed, so a ring of a step
 // plus a chunk never overwrites bytes that are still wanted.
 struct WeightRing {
-    // 1024-byte load instructions per chunk: two and three measured alike (6.74 TB/s on 216 matrices
-    // of 4096 columns) and four 6 % slower at 64 rows per workgroup; two keeps the ring smallest
-    static constexpr int kInstr = 2;
-    static constexpr uint32_t kChunk = kInstr * 1024;
+    // 1024-byte load instructions per chunk. One-step rows: two and three measured alike (6.74 TB/s on
+    // 216 matrices of 4096 columns) and four 6 % slower at 64 rows per workgroup; two keeps the ring
+    // smallest (three workgroups per compute unit). Longer rows hold more activation registers and fit
+    // two workgroups per compute unit, which leaves too few bytes in flight at two instructions: 36
+    // matrices of 4096 x 12288 ran at 5.61 / 5.72 / 5.82 TB/s with two / three / four.
+    __host__ __device__ static constexpr int instr(int steps) { return steps == 1 ? 2 : 4; }
 };
 template <typename F, typename = void>
 struct HasRingLoads : std::false_type {};
@@ -283,24 +285,27 @@ template <typename F>
 struct HasRingLoads<F, std::void_t<decltype(&F::load_row_ring)>> : std::true_type {};
 // Ring bytes per wave: a chunk is written only when less than one wave step of older bytes is still
 // to be consumed, so a step plus a chunk always fit.
-template <typename F>
+template <typename F, int STEPS>
 struct WeightRingOf {
-    static constexpr uint32_t kBytes = F::kStepBytes + WeightRing::kChunk;
+    static constexpr int kInstr = WeightRing::instr(STEPS);
+    static constexpr uint32_t kChunk = kInstr * 1024;
+    static constexpr uint32_t kBytes = F::kStepBytes + kChunk;
     static_assert(kBytes % 16 == 0, "pieces are 16 bytes");
 };
+template <int INSTR>
 struct RingChunk {
-    v4i v[WeightRing::kInstr];
+    v4i v[INSTR];
 };
 
 // Chunk `c` of the image: lane l takes bytes [16 l, 16 l + 16) of each of its 1024-byte pieces.
 // Pieces past the image's end read its last piece again instead of being masked off (total >= 128):
 // with every load unconditional the compiler can count how many are in flight and wait for the
 // oldest chunk alone; behind a per-lane branch it waits for all of them.
-__device__ __forceinline__ void ring_issue(const uint8_t* origin, uint32_t c, uint32_t total, int lane,
-                                           v4i (&v)[WeightRing::kInstr]) {
+template <int INSTR>
+__device__ __forceinline__ void ring_issue(const uint8_t* origin, uint32_t c, uint32_t total, int lane, v4i (&v)[INSTR]) {
 #pragma unroll
-    for (int k = 0; k < WeightRing::kInstr; ++k) {
-        const uint32_t o = c * WeightRing::kChunk + k * 1024 + lane * 16;
+    for (int k = 0; k < INSTR; ++k) {
+        const uint32_t o = c * (INSTR * 1024) + k * 1024 + lane * 16;
         v[k] = gload_stream<v4i>(origin + (o < total ? o : total - 16));
     }
 }
@@ -313,7 +318,7 @@ __device__ __forceinline__ void ring_issue(const uint8_t* origin, uint32_t c, ui
 // added are the same code.
 template <typename F, int STEPS, bool STAGES>
 __device__ __forceinline__ void gemv_rows_streamed(const uint8_t* origin, uint32_t head, uint32_t total, size_t bpr,
-                                                   RingChunk& rc, uint8_t* ring,
+                                                   RingChunk<WeightRing::instr(STEPS)>& rc, uint8_t* ring,
                                                    const typename F::Acts (&acts)[STEPS], const bool (&ok)[STEPS],
                                                    float* __restrict__ y, int n_units, int row0, int row_end,
                                                    int lane, const StagePtrs& st, float* osum,
@@ -324,19 +329,21 @@ __device__ __forceinline__ void gemv_rows_streamed(const uint8_t* origin, uint32
     auto residual = [&](int r) { return __shfl(add_first, (r - row0) & 63, kWave); };
     const bool plain_y = y != add_dst;
     constexpr int LS = OrderedSum<STEPS>::kRowStride;
-    constexpr uint32_t kRing = WeightRingOf<F>::kBytes;
+    constexpr uint32_t kRing = WeightRingOf<F, STEPS>::kBytes;
+    constexpr int kInstr = WeightRingOf<F, STEPS>::kInstr;
+    constexpr uint32_t kChunk = WeightRingOf<F, STEPS>::kChunk;
     uint32_t chunks = 0;  // chunks of the image written to the ring so far
     uint32_t wpos = 0;    // ring position of the next chunk (image offset modulo the ring size)
     auto advance = [&]() {
 #pragma unroll
-        for (int k = 0; k < WeightRing::kInstr; ++k) {
+        for (int k = 0; k < kInstr; ++k) {
             uint32_t o = wpos + k * 1024 + lane * 16;
             o = o >= kRing ? o - kRing : o;
             *reinterpret_cast<v4i*>(ring + o) = rc.v[k];
         }
         ++chunks;
         ring_issue(origin, chunks, total, lane, rc.v);
-        wpos += WeightRing::kChunk;
+        wpos += kChunk;
         wpos = wpos >= kRing ? wpos - kRing : wpos;
     };
     int in_batch = 0, batch_row0 = row0;
@@ -346,7 +353,7 @@ __device__ __forceinline__ void gemv_rows_streamed(const uint8_t* origin, uint32
 #pragma unroll
         for (int t = 0; t < STEPS; ++t) {
             const uint32_t step_end = (uint32_t)(t + 1) * F::kStepBytes < (uint32_t)bpr ? (uint32_t)(t + 1) * F::kStepBytes : (uint32_t)bpr;
-            while (chunks * WeightRing::kChunk < roff + step_end) advance();
+            while (chunks * kChunk < roff + step_end) advance();
             typename F::Row r;
             uint32_t spos = rpos + (uint32_t)t * (F::kStepBytes % kRing);
             while (spos >= kRing) spos -= kRing;
