@@ -302,10 +302,13 @@ def single_shape(be, dtype, m, in_f, out_f, reps=40, rotate_bytes=768 << 20, dis
     quantizer (a plan quantizes a tensor once for all the Linears of a level that read it)."""
     from infr_amd import Bindings, BufferUsage, DType, Graph, Linear, TensorDesc, synth_normal_f32, synth_weight
     nb = weight_bytes(dtype, out_f, in_f)
-    # small matrices: enough ops that a plan moves ~384 MB, so the fixed cost of one graph launch
-    # (~8 us against a 20 us kernel for forty 1024 x 4096 matrices) does not pass for bandwidth
+    # decode shapes: enough ops over distinct copies that a plan moves ~1.5 GB - the fixed cost of one
+    # graph launch (~8 us) is then a few percent of the launch, and the 256 MB memory-side cache holds
+    # a sixth of the weights at most when the plan runs again (at 384 MB per plan it held most of
+    # them, and the launch cost was a fifth of a 1024 x 4096 group's time)
     if rotate_bytes > 1 and m <= 8:
-        reps = max(reps, -(-(384 << 20) // nb))
+        reps = max(reps, -(-(1536 << 20) // nb))
+        rotate_bytes = max(rotate_bytes, reps * nb)
     copies = max(2, min(reps, -(-rotate_bytes // nb)))
     g, binds, keep = Graph(), Bindings(), []
     xid = g.input(TensorDesc((m, in_f), DType.F32))
