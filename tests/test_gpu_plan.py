@@ -791,13 +791,14 @@ def test_prefill_linears_of_one_level_share_the_activation_quantization(be):
             assert rel <= 2e-6, (rep, int(dt), out_f, rel)
 
 
-@pytest.mark.parametrize("dtype,in_f", [(DType.Q4K, 1024), (DType.Q4K, 1536), (DType.Q4K, 4096), (DType.Q4K, 5120),
+@pytest.mark.parametrize("dtype,in_f", [(DType.Q4K, 256), (DType.Q4K, 768), (DType.Q4K, 1024), (DType.Q4K, 1536), (DType.Q4K, 4096), (DType.Q4K, 5120),
                                         (DType.Q4K, 8192), (DType.Q4K, 12288), (DType.Q5K, 1536), (DType.Q5K, 4096),
                                         (DType.Q5K, 12288)])
 def test_many_round_decode_groups_stream_their_rows_through_lds(be, dtype, in_f):
     # A level of one-token Q4_K / Q5_K Linears with enough rows for many rounds of workgroups (over 131072)
     # takes the form whose waves fetch their rows as whole lines into LDS rings. Row counts that are
-    # not multiples of the tile height, rows of 4.5 and 6.75 lines (waves start mid-line), rows
+    # not multiples of the tile height, rows of 1.125, 3.375, 4.5 and 6.75 lines (waves start at every
+    # 16-byte offset of a line), rows
     # shorter than a wave step, rows of two and three wave steps with a short last step; two
     # activations. Ordered sums: every output equals the oracle's bits.
     rows_each = [16387, 20011, 9001] if in_f <= 4096 else [6007, 4001, 3003]
@@ -827,3 +828,48 @@ def test_many_round_decode_groups_stream_their_rows_through_lds(be, dtype, in_f)
         for i, xi, yb in cases:
             got = be.download(yb, np.empty(rows_each[i], np.float32))
             assert np.array_equal(bits(got), bits(want[(i, xi)])), (i, xi)
+
+
+def test_streamed_decode_group_with_an_absorbed_norm_and_absorbed_adds(be):
+    # RmsNorm -> many one-token Q4_K Linears on one level (enough rows for the streamed form), each
+    # followed by a residual Add: the norm runs in every workgroup's prologue, the adds in the row
+    # flush (residuals of a wave's rows prefetched by its lanes). Row counts leave partial tiles.
+    from infr_amd import Add, RmsNorm
+    H, n_ops = 2048, 12
+    rows_each = [12291, 11777, 12800]
+    g, binds = Graph(), Bindings()
+    x = synth_normal_f32(77, H)
+    nw = synth_normal_f32(78, H) * np.float32(0.1) + np.float32(1.0)
+    xid, nwid = g.input(TensorDesc((1, H), DType.F32)), g.input(TensorDesc((H,), DType.F32))
+    hid = g.output(TensorDesc((1, H), DType.F32))
+    hb = be.alloc(H * 4)
+    binds.bind(xid, be.upload_new(x)).bind(nwid, be.upload_new(nw)).bind(hid, hb)
+    g.push(RmsNorm(xid, nwid, hid, 1, H, 1e-6))
+    ws = [synth_weight(DType.Q4K, 600 + i, r, H) for i, r in enumerate(rows_each)]
+    wbufs = [be.upload_new(w) for w in ws]
+    cases = []
+    for k in range(n_ops):
+        i = k % len(rows_each)
+        r = rows_each[i]
+        wid = g.weight(TensorDesc((r, H), DType.Q4K))
+        yid, zid = g.output(TensorDesc((1, r), DType.F32)), g.output(TensorDesc((1, r), DType.F32))
+        resid = synth_normal_f32(900 + k, r)
+        rid = g.input(TensorDesc((1, r), DType.F32))
+        yb, zb = be.alloc(r * 4), be.alloc(r * 4)
+        binds.bind(wid, wbufs[i]).bind(yid, yb).bind(zid, zb).bind(rid, be.upload_new(resid))
+        g.push(Linear(hid, wid, yid, 1, H, r))
+        g.push(Add(yid, rid, zid, r))
+        cases.append((i, resid, yb, zb))
+    assert sum(rows_each[k % 3] for k in range(n_ops)) > 139264
+    plan = be.compile(g)
+    for _ in range(2):
+        be.execute(plan, binds)
+        assert plan.launches() == 1, plan.launches()
+        h = be.download(hb, np.empty(H, np.float32))
+        assert _rel(h, orc.rms_norm(x, nw, 1, H, 1e-6)) < 1e-6
+        want = [orc.linear(DType.Q4K, w, h, 1, H, r).ravel() for w, r in zip(ws, rows_each)]
+        for i, resid, yb, zb in cases:
+            y = be.download(yb, np.empty(rows_each[i], np.float32))
+            z = be.download(zb, np.empty(rows_each[i], np.float32))
+            assert np.array_equal(bits(y), bits(want[i]))
+            assert np.array_equal(bits(z), bits(orc.add(y, resid)))
