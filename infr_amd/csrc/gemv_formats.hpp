@@ -86,6 +86,7 @@ struct FmtQ4K {
     // step's first byte (below `ring_bytes`). Blocks are whole 16-byte pieces at 16-byte boundaries
     // and the ring is a whole number of pieces, so no piece straddles the wrap.
     static constexpr uint32_t kStepBytes = 16 * 144;
+    static constexpr int kRingMaxSteps = 3, kRingLongInstr = 4;
     __device__ static void load_row_ring(Row& r, const uint8_t* ring, uint32_t pos, uint32_t ring_bytes, int lane, bool ok) {
         const int p = lane & 3;
         uint32_t o0 = pos + (uint32_t)(lane >> 2) * 144;
@@ -542,6 +543,7 @@ struct FmtQ5K {
     }
     // The same pieces out of a wave's LDS ring (see FmtQ4K::load_row_ring).
     static constexpr uint32_t kStepBytes = 16 * 176;
+    static constexpr int kRingMaxSteps = 3, kRingLongInstr = 3;  // (two: 5.79 TB/s, three: 5.83, four: one workgroup per compute unit, 5.21)
     __device__ static void load_row_ring(Row& r, const uint8_t* ring, uint32_t pos, uint32_t ring_bytes, int lane, bool ok) {
         const int p = lane & 3;
         uint32_t o[5];

@@ -294,7 +294,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, 
     const uint8_t* span = tile.w + (size_t)row0 * tile.bpr;
     const uint32_t head = (uint32_t)(reinterpret_cast<uintptr_t>(span) & 127);
     const uint32_t total = has_rows ? (head + (uint32_t)(row_end - row0) * tile.bpr + 127) & ~127u : 0;
-    RingChunk<WeightRing::instr(STEPS)> chunks_ahead;
+    typename std::conditional<STREAMED, RingChunk<ring_instr<F, STEPS, STREAMED>()>, int>::type chunks_ahead;
     if constexpr (STREAMED) {
         if (has_rows) ring_issue(span - head, 0, total, lane, chunks_ahead.v);  // (wave-uniform)
     }
@@ -615,8 +615,8 @@ static bool plan_group_fmt(size_t in_f, const GemvOpDesc* ops, int n, GemvGroupP
             aligned = aligned && reinterpret_cast<uintptr_t>(ops[i].w) % 16 == 0 && ops[i].bpr % 16 == 0 && ops[i].st_a == nullptr;
         // (measured crossover: 139264 rows of 4096 columns, 98304 rows of 12288)
         const size_t wg64 = wgs_at(64);
-        const size_t ring_bytes = steps == 1 ? WeightRingOf<F, 1>::kBytes : WeightRingOf<F, 2>::kBytes;
-        if (aligned && steps <= 3 && cus > 0 && wg64 > (size_t)8 * cus &&
+        const size_t ring_bytes = ring_alloc_bytes<F>(steps);
+        if (aligned && steps <= F::kRingMaxSteps && cus > 0 && wg64 > (size_t)8 * cus &&
             in_f + in_f / 2 <= (size_t)8 * ring_bytes) {
             plan->streamed = true;
             plan->waves_per_wg = 8;
@@ -657,7 +657,7 @@ static bool launch_fused_fmt(size_t in_f, const GemvOpDesc& op, const GemvTile* 
     const int steps = (int)((in_f + F::kElemsPerStep - 1) / F::kElemsPerStep);
     if constexpr (HasRingLoads<F>::value) {
         if (plan.streamed) {
-            if (plan.waves_per_wg != 8 || steps > 3 || op.st_a != nullptr) return false;
+            if (plan.waves_per_wg != 8 || steps > F::kRingMaxSteps || op.st_a != nullptr) return false;
             const dim3 grid((unsigned)plan.total_wgs), block(512);
 #define INFR_STREAMED(N)                                                                                          \
     do {                                                                                                          \
@@ -668,8 +668,10 @@ static bool launch_fused_fmt(size_t in_f, const GemvOpDesc& op, const GemvTile* 
                            plan.rows_per_wg, tiles_dev, (int)in_f);                                               \
     } while (0)
             if (steps == 1) INFR_STREAMED(1);
-            else if (steps == 2) INFR_STREAMED(2);
-            else INFR_STREAMED(3);
+            if constexpr (F::kRingMaxSteps >= 3) {
+                if (steps == 2) INFR_STREAMED(2);
+                if (steps == 3) INFR_STREAMED(3);
+            }
 #undef INFR_STREAMED
             return true;
         }

@@ -271,27 +271,41 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
 // crosses a page, so they are readable). Ring offsets are image offsets modulo the ring size: a chunk
 // is written when less than one wave step of older bytes is still to be consumed, so a ring of a step
 // plus a chunk never overwrites bytes that are still wanted.
-struct WeightRing {
-    // 1024-byte load instructions per chunk. One-step rows: two and three measured alike (6.74 TB/s on
-    // 216 matrices of 4096 columns) and four 6 % slower at 64 rows per workgroup; two keeps the ring
-    // smallest (three workgroups per compute unit). Longer rows hold more activation registers and fit
-    // two workgroups per compute unit, which leaves too few bytes in flight at two instructions: 36
-    // matrices of 4096 x 12288 ran at 5.61 / 5.72 / 5.82 TB/s with two / three / four.
-    __host__ __device__ static constexpr int instr(int steps) { return steps == 1 ? 2 : 4; }
-};
 template <typename F, typename = void>
 struct HasRingLoads : std::false_type {};
 template <typename F>
 struct HasRingLoads<F, std::void_t<decltype(&F::load_row_ring)>> : std::true_type {};
-// Ring bytes per wave: a chunk is written only when less than one wave step of older bytes is still
-// to be consumed, so a step plus a chunk always fit.
+// Ring geometry of a format at a row length of STEPS wave steps.
+// kInstr: 1024-byte load instructions per chunk. One-step rows: two and three measured alike (6.74 TB/s
+// on 216 Q4_K matrices of 4096 columns) and four 6 % slower at 64 rows per workgroup; two keeps the ring
+// smallest (three workgroups per compute unit). Longer rows hold more activation registers and fit two
+// workgroups per compute unit, which leaves too few bytes in flight at two instructions: 36 Q4_K
+// matrices of 4096 x 12288 ran at 5.61 / 5.72 / 5.82 TB/s with two / three / four; the format says how
+// many its ring can afford there (F::kRingLongInstr: two workgroups must still fit the LDS).
+// kBytes: a chunk is written only when less than one wave step of older bytes is still to be consumed,
+// so a step plus a chunk always fit. The lanes' pieces must be 16-byte aligned in the row (Q4_K's and
+// Q5_K's are): a ring of whole pieces then never splits one at its end. Q6_K's pieces sit at any even
+// offset; a form that kept a second copy of the ring's first 16 bytes behind its end and read the
+// pieces with misaligned 16-byte LDS loads gave the right bits and ran 7-9 % slower than the direct
+// loads (5.28 against 5.67 TB/s at 4096 x 4096), and is not kept.
 template <typename F, int STEPS>
 struct WeightRingOf {
-    static constexpr int kInstr = WeightRing::instr(STEPS);
+    static constexpr int kInstr = STEPS == 1 ? 2 : F::kRingLongInstr;
     static constexpr uint32_t kChunk = kInstr * 1024;
     static constexpr uint32_t kBytes = F::kStepBytes + kChunk;
-    static_assert(kBytes % 16 == 0, "pieces are 16 bytes");
+    static_assert(kBytes % 16 == 0, "chunk pieces are 16 bytes");
 };
+// The ring of a row of `steps` wave steps, for host code that sizes LDS by the step count.
+template <typename F>
+inline size_t ring_alloc_bytes(int steps) {
+    return steps == 1 ? WeightRingOf<F, 1>::kBytes : WeightRingOf<F, 2>::kBytes;
+}
+// (kInstr for a kernel that may be instantiated for formats without ring loads)
+template <typename F, int STEPS, bool STREAMED>
+constexpr int ring_instr() {
+    if constexpr (STREAMED) return WeightRingOf<F, STEPS>::kInstr;
+    else return 1;
+}
 template <int INSTR>
 struct RingChunk {
     v4i v[INSTR];
@@ -318,7 +332,7 @@ __device__ __forceinline__ void ring_issue(const uint8_t* origin, uint32_t c, ui
 // added are the same code.
 template <typename F, int STEPS, bool STAGES>
 __device__ __forceinline__ void gemv_rows_streamed(const uint8_t* origin, uint32_t head, uint32_t total, size_t bpr,
-                                                   RingChunk<WeightRing::instr(STEPS)>& rc, uint8_t* ring,
+                                                   RingChunk<WeightRingOf<F, STEPS>::kInstr>& rc, uint8_t* ring,
                                                    const typename F::Acts (&acts)[STEPS], const bool (&ok)[STEPS],
                                                    float* __restrict__ y, int n_units, int row0, int row_end,
                                                    int lane, const StagePtrs& st, float* osum,

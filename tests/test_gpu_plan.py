@@ -793,9 +793,9 @@ def test_prefill_linears_of_one_level_share_the_activation_quantization(be):
 
 @pytest.mark.parametrize("dtype,in_f", [(DType.Q4K, 256), (DType.Q4K, 768), (DType.Q4K, 1024), (DType.Q4K, 1536), (DType.Q4K, 4096), (DType.Q4K, 5120),
                                         (DType.Q4K, 8192), (DType.Q4K, 12288), (DType.Q5K, 1536), (DType.Q5K, 4096),
-                                        (DType.Q5K, 12288)])
+                                        (DType.Q5K, 12288), (DType.Q6K, 4096)])
 def test_many_round_decode_groups_stream_their_rows_through_lds(be, dtype, in_f):
-    # A level of one-token Q4_K / Q5_K Linears with enough rows for many rounds of workgroups (over 131072)
+    # A level of one-token Q4_K / Q5_K Linears (and Q6_K, which keeps the direct loads) with enough rows for many rounds of workgroups (over 131072)
     # takes the form whose waves fetch their rows as whole lines into LDS rings. Row counts that are
     # not multiples of the tile height, rows of 1.125, 3.375, 4.5 and 6.75 lines (waves start at every
     # 16-byte offset of a line), rows
