@@ -873,3 +873,41 @@ def test_streamed_decode_group_with_an_absorbed_norm_and_absorbed_adds(be):
             z = be.download(zb, np.empty(rows_each[i], np.float32))
             assert np.array_equal(bits(y), bits(want[i]))
             assert np.array_equal(bits(z), bits(orc.add(y, resid)))
+
+
+def test_streamed_decode_group_of_two_step_rows_behind_an_absorbed_gated_activation(be):
+    # GatedAct -> many one-token Q4_K Linears over 8192 columns (two wave steps a row, chunks of four
+    # load instructions) on one level: the activation is evaluated and quantized in every workgroup's
+    # prologue, over the LDS that the rings take afterwards.
+    from infr_amd import GatedAct
+    FF, n_ops = 8192, 18
+    rows_each = [9001, 8000, 7203]
+    g, binds = Graph(), Bindings()
+    gate, up = synth_normal_f32(41, FF), synth_normal_f32(42, FF)
+    gid, uid = g.input(TensorDesc((1, FF), DType.F32)), g.input(TensorDesc((1, FF), DType.F32))
+    aid = g.output(TensorDesc((1, FF), DType.F32))
+    ab = be.alloc(FF * 4)
+    binds.bind(gid, be.upload_new(gate)).bind(uid, be.upload_new(up)).bind(aid, ab)
+    g.push(GatedAct(gid, uid, aid, 1, FF))
+    ws = [synth_weight(DType.Q4K, 700 + i, r, FF) for i, r in enumerate(rows_each)]
+    wbufs = [be.upload_new(w) for w in ws]
+    cases = []
+    for k in range(n_ops):
+        i = k % len(rows_each)
+        wid = g.weight(TensorDesc((rows_each[i], FF), DType.Q4K))
+        yid = g.output(TensorDesc((1, rows_each[i]), DType.F32))
+        yb = be.alloc(rows_each[i] * 4)
+        binds.bind(wid, wbufs[i]).bind(yid, yb)
+        g.push(Linear(aid, wid, yid, 1, FF, rows_each[i]))
+        cases.append((i, yb))
+    assert sum(rows_each[k % 3] for k in range(n_ops)) > 139264
+    plan = be.compile(g)
+    for _ in range(2):
+        be.execute(plan, binds)
+        assert plan.launches() == 1, plan.launches()
+        act = be.download(ab, np.empty(FF, np.float32))
+        assert _rel(act, orc.gated_act(gate, up, 1, FF)) < 1e-6
+        want = [orc.linear(DType.Q4K, w, act, 1, FF, r).ravel() for w, r in zip(ws, rows_each)]
+        for i, yb in cases:
+            y = be.download(yb, np.empty(rows_each[i], np.float32))
+            assert np.array_equal(bits(y), bits(want[i]))
