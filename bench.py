@@ -344,8 +344,8 @@ def single_shape(be, dtype, m, in_f, out_f, reps=40, rotate_bytes=768 << 20, dis
         g.push(Linear(xids[i % len(xids)], wids[i % copies], yid, m, in_f, out_f))
     plan = be.compile(g)
     settle_clocks(be, plan, binds)
-    # three executes back to back per timing: the host side of an execute (binding checks of up to
-    # 2000 tensors, the graph launch) then runs while the device is busy with the execute before
+    # three executes back to back per timing: the start-up of an execute (host-side checks, the graph
+    # launch reaching an idle device) then overlaps the execute before
     best = 1e30
     for _ in range(4):
         be.timer_begin()
