@@ -97,14 +97,16 @@ def test_synth_q2_0_codes_are_ternary():
     assert all(abs(f - 1 / 3) < 0.02 for f in frac)
 
 
-# ---- the Rust mirror in INTEGRATION.md against the C header's layout ----
+# ---- the Rust mirror in the binding notes against the C header's layout ----
+
+BINDING_NOTES = "INTEGRATION.md"  # the file that holds the reference-side shim's source text
 
 _RUST_TYPES = {"i32": (4, 4), "u32": (4, 4), "f32": (4, 4), "u64": (8, 8), "i64": (8, 8), "usize": (8, 8)}
 
 
 def _rust_repr_c_structs():
-    """name -> [(field, size, align)] for every `#[repr(C)] ... pub struct` in INTEGRATION.md."""
-    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    """name -> [(field, size, align)] for every `#[repr(C)] ... pub struct` of the shim's source text."""
+    text = open(os.path.join(ROOT, BINDING_NOTES)).read()
     out = {}
     for name, body in re.findall(r"#\[repr\(C\)\][^{;]*?pub struct (\w+)\s*\{(.*?)\}", text, flags=re.S):
         body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
@@ -156,7 +158,7 @@ def test_rust_mirror_structs_match_the_c_header(tmp_path, rust, ctype):
     """The `impl Backend for HipBackend` shim cannot be compiled here (no Rust toolchain); what can be
     checked is that its #[repr(C)] structs still describe the header's structs field by field."""
     structs = _rust_repr_c_structs()
-    assert rust in structs, f"INTEGRATION.md no longer declares {rust}"
+    assert rust in structs, f"{BINDING_NOTES} no longer declares {rust}"
     offsets, size, _ = _repr_c_layout(structs, rust)
     c = _c_layout(tmp_path, ctype, list(offsets))          # a field the header lacks fails to compile
     assert c.pop("sizeof") == size, f"{rust} and {ctype} differ in size"
@@ -173,9 +175,9 @@ def test_shim_moe_arm_names_every_field_of_the_op():
     pattern would let a field that changes the arithmetic (gating, weight_before, act, ...) vanish on the
     way to the library, which can only refuse what it is told about."""
     import re
-    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    text = open(os.path.join(ROOT, BINDING_NOTES)).read()
     m = re.search(r"Op::MoeFfn \{([^}]*)\} => ops\.push\(HipOp \{(.*?)\.\.Default::default\(\) \}\),", text, re.S)
-    assert m, "INTEGRATION.md no longer holds the MoeFfn arm"
+    assert m, f"{BINDING_NOTES} no longer holds the MoeFfn arm"
     pattern, body = m.group(1), m.group(2)
     assert ".." not in pattern, "the MoeFfn pattern skips fields with `..`"
     bound = {f.strip().split(":")[0].strip() for f in pattern.split(",") if f.strip()}
