@@ -143,6 +143,23 @@ def test_decode_gemv_vs_oracle(be, dtype, in_f, out_f):
         assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), "not bit-identical"
 
 
+@pytest.mark.parametrize("dtype,in_f", [(DType.Q4K, 1024), (DType.Q5K, 768), (DType.Q4K, 2560)])
+@pytest.mark.parametrize("noalloc", [False, True])
+def test_one_token_over_an_output_head_sized_matrix(be, dtype, in_f, noalloc):
+    """A single one-token op with a vocabulary's worth of rows (Qwen3's 151936) is many rounds of
+    workgroups by itself and takes the streamed-row form of the decode GEMV through the direct entry
+    points (no tile table: the descriptor travels as a kernel argument); the last tile is partial.
+    The integer-stage entry point keeps the direct-load form: same bits."""
+    out_f = 151936 + 5
+    w = orc.synth_weight(dtype, out_f * in_f, 0x77 + in_f)
+    x = synth_normal_f32(0x78, in_f)
+    yb = be.alloc(out_f * 4)
+    (be.linear_noalloc if noalloc else be.linear)(dtype, be.upload_new(w), be.upload_new(x), yb, 1, in_f, out_f)
+    got = be.download(yb, np.empty(out_f, np.float32))
+    want = orc.linear(dtype, w, x, 1, in_f, out_f).ravel()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
 @pytest.mark.parametrize("dtype", [DType.Q4K, DType.Q6K, DType.Q8_0, DType.Q2_0])
 def test_decode_int_stages_bit_exact(be, dtype):
     in_f, out_f = 1024, 24
