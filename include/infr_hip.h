@@ -131,7 +131,9 @@ int infr_hip_sync(infr_hip_t *be);
  *   x        f32 [m, in_f]; dst f32 [m, out_f], row-major.
  * Activations are quantized on the device exactly as infr-cpu does (per-256 int8 + f32 scale for
  * Q4_K/Q6_K/Q8_0, crates/infr-cpu/src/quant.rs:27-58; per-32 for Q2_0, quant.rs:97-117), the
- * integer dot is exact, and the f32 epilogue follows the CPU kernels' expression per block.
+ * integer dot is exact, and the f32 epilogue follows the CPU kernels' expression per block
+ * (Q4_K from 128 tokens up fuses each block's products into its adds: y within 2e-6 relative of
+ * infr-cpu instead of equal to it; the integers are exact there too).
  * in_f must be a whole number of weight blocks (256 for the K-quants, 64 for Q2_0, 32 otherwise): a
  * shorter tail is rejected, never truncated. in_f above 32768 (Q8_0, Q4_1, Q5_1: 16384) must be a
  * multiple of 256 (it then runs the prefill kernels at any m), else INFR_HIP_ERR_UNSUPPORTED.
