@@ -223,8 +223,8 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, 
                                                              int in_f) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int lane = threadIdx.x & 63;
-    // (STREAMED: as a scalar, so that the row and chunk bookkeeping runs on the scalar unit)
-    const int wave = STREAMED ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : (int)(threadIdx.x >> 6);
+    // (as a scalar, so that the row, tile and chunk bookkeeping runs on the scalar unit)
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 
     // This workgroup's rows: one table entry, or computed from the single op's descriptor.
     GemvTile tile;
