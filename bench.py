@@ -693,7 +693,8 @@ def main():
             extra[f"gemv_Q4_K_m1_{out_f}x{in_f}_warm_cache_resident_GBs"] = round(nb / (t * 1e-3) / 1e9, 1)
     if "formats" in sections:
         for name, dt in (("Q5_K", DType.Q5K), ("Q4_0", DType.Q4_0), ("Q4_1", DType.Q4_1), ("Q5_0", DType.Q5_0),
-                         ("Q5_1", DType.Q5_1), ("IQ4_NL", DType.IQ4NL), ("Q2_0", DType.Q2_0)):
+                         ("Q5_1", DType.Q5_1), ("IQ4_NL", DType.IQ4NL), ("Q2_0", DType.Q2_0), ("Q2_K", DType.Q2K),
+                         ("Q3_K", DType.Q3K)):
             for m in (1, 8):
                 for (out_f, in_f) in ((4096, 4096), (12288, 4096), (4096, 12288)):
                     t, nb = single_shape(be, dt, m, in_f, out_f)

@@ -46,6 +46,8 @@ typedef enum {
     INFR_DTYPE_Q5_0 = 6,  /* 32 / 22 B:  [f16 d][u32 qh][u8 qs[16]]     w = d*(q-16)       :315-316 */
     INFR_DTYPE_Q5_1 = 7,  /* 32 / 24 B:  [f16 d][f16 m][u32 qh][u8 qs[16]]  w = d*q+m      :317-318 */
     INFR_DTYPE_Q8_0 = 8,  /* 32 elems / 34 B:  [f16 d][i8 qs[32]]            decode_spec.rs:319-320 */
+    INFR_DTYPE_Q2_K = 10, /* 256 / 84 B:  [u8 scales[16]][u8 qs[64]][f16 d][f16 dmin]     :322-323 */
+    INFR_DTYPE_Q3_K = 11, /* 256 / 110 B: [u8 hmask[32]][u8 qs[64]][u8 scales[12]][f16 d] :324-325 */
     INFR_DTYPE_Q4_K = 12, /* 256 / 144 B: [f16 d][f16 dmin][u8 sc[12]][u8 qs[128]]        :326-327 */
     INFR_DTYPE_Q5_K = 13, /* 256 / 176 B: [f16 d][f16 dmin][u8 sc[12]][u8 qh[32]][u8 qs[128]] :328-329 */
     INFR_DTYPE_Q6_K = 14, /* 256 / 210 B: [u8 ql[128]][u8 qh[64]][i8 sc[16]][f16 d]       :330-331 */

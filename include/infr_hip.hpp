@@ -43,7 +43,8 @@ namespace infr {
 // crates/infr-core/src/tensor.rs:7-57; numbered as GGML type ids.
 enum class DType : int {
     F32 = INFR_DTYPE_F32, F16 = INFR_DTYPE_F16, Q4_0 = INFR_DTYPE_Q4_0, Q4_1 = INFR_DTYPE_Q4_1,
-    Q5_0 = INFR_DTYPE_Q5_0, Q5_1 = INFR_DTYPE_Q5_1, Q8_0 = INFR_DTYPE_Q8_0, Q4K = INFR_DTYPE_Q4_K,
+    Q5_0 = INFR_DTYPE_Q5_0, Q5_1 = INFR_DTYPE_Q5_1, Q8_0 = INFR_DTYPE_Q8_0, Q2K = INFR_DTYPE_Q2_K,
+    Q3K = INFR_DTYPE_Q3_K, Q4K = INFR_DTYPE_Q4_K,
     Q5K = INFR_DTYPE_Q5_K, Q6K = INFR_DTYPE_Q6_K, IQ4NL = INFR_DTYPE_IQ4_NL, I32 = 26,
     BF16 = INFR_DTYPE_BF16, Q2_0 = INFR_DTYPE_Q2_0,
 };
@@ -57,6 +58,8 @@ inline const char* dtype_name(DType d) {
     case DType::Q5_0: return "Q5_0";
     case DType::Q5_1: return "Q5_1";
     case DType::Q8_0: return "Q8_0";
+    case DType::Q2K: return "Q2K";
+    case DType::Q3K: return "Q3K";
     case DType::Q4K: return "Q4K";
     case DType::Q5K: return "Q5K";
     case DType::Q6K: return "Q6K";

@@ -28,6 +28,8 @@ class DType(IntEnum):
     Q5_0 = 6
     Q5_1 = 7
     Q8_0 = 8
+    Q2K = 10
+    Q3K = 11
     Q4K = 12
     Q5K = 13
     Q6K = 14
@@ -636,9 +638,9 @@ class HipBackend:
         if w_numel is None:
             e, b = block_layout(dtype)
             w_numel = w.len_bytes() // b * e
-        blocks = in_f // 256 if dtype in (DType.Q4K, DType.Q5K, DType.Q6K) else in_f // 32
+        blocks = in_f // 256 if dtype in (DType.Q4K, DType.Q5K, DType.Q6K, DType.Q2K, DType.Q3K) else in_f // 32
         a = self.alloc(m * out_f * blocks * 4)
-        b_ = self.alloc(m * out_f * blocks * 4) if dtype in (DType.Q4K, DType.Q5K) else None
+        b_ = self.alloc(m * out_f * blocks * 4) if dtype in (DType.Q4K, DType.Q5K, DType.Q2K) else None
         self._check(self._lib.infr_hip_linear_int_stages(
             self._h, int(dtype), w._h, w_numel, w_off, x._h, m, in_f, out_f, a._h,
             b_._h if b_ else None))

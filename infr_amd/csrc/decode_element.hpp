@@ -65,6 +65,24 @@ __device__ inline float decode_element(int dtype, const uint8_t* rowp, int e) {
         const float fs = ldf16(blk) * (float)sc, fm = ldf16(blk + 2) * (float)(-m);
         return fs * (float)code + fm;
     }
+    case 10: {  // Q2_K: (d * scale) * code + dmin * (-min), sub-block i / 16 (dequant.rs:220-247)
+        const uint8_t* blk = rowp + (size_t)(e >> 8) * 84;
+        const int i = e & 255, n = i >> 7, j = (i >> 5) & 3, half = (i >> 4) & 1, l = i & 15;
+        const uint32_t sb = ld8(blk + (i >> 4));
+        const uint32_t code = (ld8(blk + 16 + 32 * n + 16 * half + l) >> (2 * j)) & 3u;
+        return (ldf16(blk + 80) * (float)(int)(sb & 15u)) * (float)code + ldf16(blk + 82) * (float)(-(int)(sb >> 4));
+    }
+    case 11: {  // Q3_K: (d * s) * code + d * (-4 s), s = sc6 - 32 (dequant.rs:248-298)
+        const uint8_t* blk = rowp + (size_t)(e >> 8) * 110;
+        const int i = e & 255, n = i >> 7, j = (i >> 5) & 3, half = (i >> 4) & 1, l = i & 15, is = i >> 4;
+        const uint32_t low2 = (ld8(blk + 32 + 32 * n + 16 * half + l) >> (2 * j)) & 3u;
+        const uint32_t high = (ld8(blk + 16 * half + l) >> (4 * n + j)) & 1u;
+        const uint32_t lo4 = (ld8(blk + 96 + (is & 7)) >> (4 * (is >> 3))) & 15u;
+        const uint32_t hi2 = (ld8(blk + 104 + (is & 3)) >> (2 * (is >> 2))) & 3u;
+        const int s = (int)(lo4 | (hi2 << 4)) - 32;
+        const float d = ldf16(blk + 108);
+        return (d * (float)s) * (float)(low2 | (high << 2)) + d * (float)(-4 * s);
+    }
     case 14: {  // Q6_K
         const uint8_t* blk = rowp + (size_t)(e >> 8) * 210;
         const int i = e & 255, half = i >> 7, r = i & 127, col = r >> 5, l = r & 31;

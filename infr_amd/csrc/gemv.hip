@@ -34,6 +34,8 @@ static const GemvFormatOps* format_ops(int dtype, size_t in_f) {
     case 8: return in_f % 256 == 0 ? &gemv_ops_q8_0() : (in_f % 64 == 0 ? &gemv_ops_q8_0_32_aligned() : &gemv_ops_q8_0_32());
     case 42: return in_f % 128 == 0 ? &gemv_ops_q2_0_aligned() : &gemv_ops_q2_0();
     case 13: return &gemv_ops_q5k();
+    case 10: return &gemv_ops_q2k();
+    case 11: return &gemv_ops_q3k();
     case 2: return in_f % 64 == 0 ? &gemv_ops_q4_0_pair() : &gemv_ops_q4_0();
     case 3: return &gemv_ops_q4_1();
     case 6: return in_f % 64 == 0 ? &gemv_ops_q5_0_pair() : &gemv_ops_q5_0();

@@ -3,7 +3,7 @@
 // Each format follows infr-cpu's scalar kernel for one block:
 //   Q4_K  crates/infr-cpu/src/kernels.rs:151-184     Q6_K  kernels.rs:487-526
 //   Q8_0  kernels.rs:1170-1187                       Q2_0  kernels.rs:5641-5668
-//   Q5_K  kernels.rs:1286-1327
+//   Q5_K  kernels.rs:1286-1327                      Q2_K  kernels.rs:315-361    Q3_K  :764-852
 //   Q4_0  kernels.rs:5496-5520   Q4_1  :5793-5822    Q5_0  :5350-5377   Q5_1  :5948-5980
 //   IQ4_NL  kernels.rs:6128-6152
 //
@@ -596,6 +596,146 @@ struct FmtQ5K {
         const float dmin = f16_bits_to_f32((uint32_t)r.hdr.x >> 16);
         // sumf += q8.d[b] * (d * sd as f32 - dmin * sm as f32)
         return a.dact * (d * (float)sd - dmin * (float)sm);
+    }
+};
+
+// ───────────────────────────────────── Q2_K / Q3_K ─────────────────────────────────────
+// Both keep a block's 2-bit fields in qs[64]: element 128 n + 32 j + 16 half + l is field j of byte
+// qs[32 n + 16 half + l], and its 16-element sub-block 8 n + 2 j + half has a scale of its own. Lane l:
+// block-in-step q = l/4, p = l%4 = 2 n + half: the lane owns the 16 bytes qs[16 p ..], i.e. the four
+// sub-blocks 8 n + half + 2 j, and their 64 activation bytes (FmtQ6K's activation mapping: groups of
+// 16 at 128 n + 16 half + 32 j, per-16 sums at 8 n + half + 2 j). 16 blocks per wave step.
+//
+// Q2_K (84-byte block, 4-byte aligned: [u8 scales[16]][u8 qs[64]][f16 d][f16 dmin]): a scale byte is a
+// 4-bit scale (low) and a 4-bit min (high); sd = sum scale * (q2 . q8), sm = sum min * bsum16, and the
+// CPU's term q8.d[b] * (d * sd - dmin * sm) (kernels.rs:315-361), blocks in ascending order.
+struct FmtQ2K {
+    static constexpr int kElemsPerStep = 4096;
+    static constexpr bool kPer32 = false;
+    static constexpr bool kOrdered = true;
+    static constexpr int kBlockBytes = 84, kBlockElems = 256;
+    static constexpr int kWide16Steps = 3;
+    static constexpr bool kClampedLoads = false;
+    static constexpr bool kLaneSums = true;
+    static constexpr bool kRowAhead = false;
+    struct Row {
+        v4i q;
+        v2i sc;       // scales[8 n .. 8 n + 8)
+        uint32_t dm;  // d | dmin << 16
+    };
+    typedef FmtQ6K::Acts Acts;
+    __device__ static int units(int in_f) { return in_f / 256; }
+    __device__ static bool valid(int t, int lane, int n) { return t * 16 + (lane >> 2) < n; }
+    __device__ static void load_row(Row& r, const uint8_t* rowp, int t, int lane, bool ok) {
+        if (ok) {
+            const uint8_t* blk = rowp + (size_t)(t * 16 + (lane >> 2)) * 84;
+            const int p = lane & 3;
+            r.q = load16_a4(blk + 16 + 16 * p);
+            r.sc = gload<v2i_a4>(blk + 8 * (p >> 1));
+            r.dm = (uint32_t)load_u32(blk + 80);
+        } else {
+            r.q = v4i{0, 0, 0, 0};
+            r.sc = v2i{0, 0};
+            r.dm = 0;
+        }
+    }
+    __device__ static void load_acts(Acts& a, const ActPtrs& s, int t, int lane, bool ok) {
+        FmtQ6K::load_acts(a, s, t, lane, ok);
+    }
+    template <bool STAGES>
+    __device__ static float term(const Row& r, const Acts& a, int t, int lane, bool ok,
+                                 const StagePtrs& st, size_t row_units) {
+        const int half = lane & 1;
+        const int qw[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
+        int pd = 0, pm = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            int ip = 0;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) ip = dot4((int)(((uint32_t)qw[k] >> (2 * j)) & 0x03030303u), a.xa[4 * j + k], ip);
+            // sub-block 8 n + half + 2 j: byte half + 2 j of the eight scale bytes
+            const uint32_t sb = ((uint32_t)(j < 2 ? r.sc.x : r.sc.y) >> (8 * (half + 2 * (j & 1)))) & 0xFFu;
+            pd += __mul24((int)(sb & 15u), ip);  // |ip| <= 16 * 3 * 127: the 24-bit multiply is exact
+            pm += __mul24((int)(sb >> 4), a.bs16[j]);
+        }
+        const int sd = quad_sum(pd), sm = quad_sum(pm);
+        if (STAGES && ok && (lane & 3) == 0) {
+            st.a[row_units + t * 16 + (lane >> 2)] = sd;
+            st.b[row_units + t * 16 + (lane >> 2)] = sm;
+        }
+        const float d = f16_bits_to_f32(r.dm & 0xFFFFu), dmin = f16_bits_to_f32(r.dm >> 16);
+        // sumf += q8.d[b] * (d * sd as f32 - dmin * sm as f32)
+        return a.dact * (d * (float)sd - dmin * (float)sm);
+    }
+};
+
+// Q3_K (110-byte block, 2-byte aligned: [u8 hmask[32]][u8 qs[64]][u8 scales[12]][f16 d]): a code is
+// the 2-bit field plus bit 4 n + j of hmask[16 half + l] as its third bit; sixteen 6-bit scales are
+// packed as low nibbles, high nibbles and a word of top bit pairs (q3k_scales, kernels.rs:764-783),
+// and enter as sc6 - 32. isum = sum (sc6 - 32) * (q3 . q8 - 4 bsum16), term d * q8.d[b] * isum
+// (kernels.rs:812-852), blocks in ascending order.
+struct FmtQ3K {
+    static constexpr int kElemsPerStep = 4096;
+    static constexpr bool kPer32 = false;
+    static constexpr bool kOrdered = true;
+    static constexpr int kBlockBytes = 110, kBlockElems = 256;
+    static constexpr int kWide16Steps = 2;
+    static constexpr bool kClampedLoads = false;
+    static constexpr bool kLaneSums = true;
+    static constexpr bool kRowAhead = false;
+    struct Row {
+        v4i q, hm;
+        v3i sc;      // the 12 scale bytes
+        uint32_t d;
+    };
+    typedef FmtQ6K::Acts Acts;
+    __device__ static int units(int in_f) { return in_f / 256; }
+    __device__ static bool valid(int t, int lane, int n) { return t * 16 + (lane >> 2) < n; }
+    __device__ static void load_row(Row& r, const uint8_t* rowp, int t, int lane, bool ok) {
+        if (ok) {
+            const uint8_t* blk = rowp + (size_t)(t * 16 + (lane >> 2)) * 110;
+            const int p = lane & 3;
+            r.hm = load16_a2(blk + 16 * (p & 1));
+            r.q = load16_a2(blk + 32 + 16 * p);
+            r.sc = gload<v3i_a2>(blk + 96);
+            r.d = load_u16(blk + 108);
+        } else {
+            r.q = r.hm = v4i{0, 0, 0, 0};
+            r.sc = v3i{0, 0, 0};
+            r.d = 0;
+        }
+    }
+    __device__ static void load_acts(Acts& a, const ActPtrs& s, int t, int lane, bool ok) {
+        FmtQ6K::load_acts(a, s, t, lane, ok);
+    }
+    template <bool STAGES>
+    __device__ static float term(const Row& r, const Acts& a, int t, int lane, bool ok,
+                                 const StagePtrs& st, size_t row_units) {
+        const int n = (lane >> 1) & 1, half = lane & 1;
+        const int qw[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
+        const int hw[4] = {r.hm.x, r.hm.y, r.hm.z, r.hm.w};
+        // scales 8 n .. 8 n + 7 as two words of bytes: nibbles of the first eight bytes (low for
+        // n = 0, high for n = 1) with two more bits each from the last four
+        const uint32_t k1 = 0x03030303u, k2 = 0x0F0F0F0Fu, tt = (uint32_t)r.sc.z >> (4 * n);
+        const uint32_t w0 = (((uint32_t)r.sc.x >> (4 * n)) & k2) | ((tt & k1) << 4);
+        const uint32_t w1 = (((uint32_t)r.sc.y >> (4 * n)) & k2) | (((tt >> 2) & k1) << 4);
+        int part = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            int ip = 0;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t low2 = ((uint32_t)qw[k] >> (2 * j)) & 0x03030303u;
+                const uint32_t high = (((uint32_t)hw[k] >> (4 * n + j)) & 0x01010101u) << 2;
+                ip = dot4((int)(low2 | high), a.xa[4 * j + k], ip);
+            }
+            const int s = (int)(((j < 2 ? w0 : w1) >> (8 * (half + 2 * (j & 1)))) & 0xFFu) - 32;
+            part += __mul24(s, ip - 4 * a.bs16[j]);  // |.| <= 16 * 11 * 127: the 24-bit multiply is exact
+        }
+        const int isum = quad_sum(part);
+        if (STAGES && ok && (lane & 3) == 0) st.a[row_units + t * 16 + (lane >> 2)] = isum;
+        // sumf += d * q8.d[b] * isum as f32
+        return f16_bits_to_f32(r.d) * a.dact * (float)isum;
     }
 };
 

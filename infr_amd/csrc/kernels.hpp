@@ -224,6 +224,8 @@ const GemvFormatOps& gemv_ops_q8_0_32_aligned();  // rows of whole 64s
 const GemvFormatOps& gemv_ops_q2_0();
 const GemvFormatOps& gemv_ops_q2_0_aligned();  // rows of whole 128s
 const GemvFormatOps& gemv_ops_q5k();
+const GemvFormatOps& gemv_ops_q2k();
+const GemvFormatOps& gemv_ops_q3k();
 const GemvFormatOps& gemv_ops_q4_0();
 const GemvFormatOps& gemv_ops_q4_1();
 const GemvFormatOps& gemv_ops_q5_0();  // batch launchers only: one token takes the f32 kernel

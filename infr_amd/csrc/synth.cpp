@@ -255,6 +255,75 @@ void encode_q5k(const float* x, uint8_t* blk) {
     }
 }
 
+// 256 floats -> one 84-byte Q2_K block (scales[16] | qs[64] | d | dmin): per 16-weight sub-block an
+// affine 2-bit grid [min(0, min x), max x]; 4-bit sub-block scales (low nibble) and mins (high
+// nibble) against f16 super scales. Sub-block s = 8n + 2j + h holds elements 16s..16s+15; their
+// codes sit at bit 2j of qs[32n + 16h ..] (crates/infr-gguf/src/dequant.rs, Q2_K).
+void encode_q2k(const float* x, uint8_t* blk) {
+    float scale[16], minv[16];
+    float max_scale = 0.0f, max_min = 0.0f;
+    for (int s = 0; s < 16; ++s) {
+        float lo = 0.0f, hi = 0.0f;
+        for (int l = 0; l < 16; ++l) {
+            lo = std::min(lo, x[s * 16 + l]);
+            hi = std::max(hi, x[s * 16 + l]);
+        }
+        scale[s] = (hi - lo) / 3.0f;
+        minv[s] = -lo;
+        max_scale = std::max(max_scale, scale[s]);
+        max_min = std::max(max_min, minv[s]);
+    }
+    put_f16(blk + 80, max_scale / 15.0f);
+    put_f16(blk + 82, max_min / 15.0f);
+    const float d = f16_to_f32((uint16_t)(blk[80] | (blk[81] << 8)));
+    const float dmin = f16_to_f32((uint16_t)(blk[82] | (blk[83] << 8)));
+    std::memset(blk + 16, 0, 64);
+    for (int s = 0; s < 16; ++s) {
+        const int sc = d > 0.0f ? clampi((int)std::lround(scale[s] / d), 0, 15) : 0;
+        const int mn = dmin > 0.0f ? clampi((int)std::lround(minv[s] / dmin), 0, 15) : 0;
+        blk[s] = (uint8_t)(sc | (mn << 4));
+        const float ws = d * (float)sc, wm = dmin * (float)mn;
+        const int n = s / 8, j = (s % 8) / 2, h = s & 1;
+        for (int l = 0; l < 16; ++l) {
+            const int q = ws > 0.0f ? clampi((int)std::lround((x[s * 16 + l] + wm) / ws), 0, 3) : 0;
+            blk[16 + 32 * n + 16 * h + l] |= (uint8_t)(q << (2 * j));
+        }
+    }
+}
+
+// 256 floats -> one 110-byte Q3_K block (hmask[32] | qs[64] | scales[12] | d): per 16-weight
+// sub-block a 3-bit grid (code - 4) whose signed scale puts the element of largest magnitude on
+// code 0 (= -4), so sub-block scales take both signs; stored as 6-bit fields with a bias of 32
+// against one f16 super scale. Codes: low two bits as in Q2_K, the third in bit 4n + j of
+// hmask[16h + l]. Scale field i (group g = i / 4, byte k = i % 4): low nibble in the low (g < 2) or
+// high nibble of scales[4 (g & 1) + k], top two bits at bit 2g of scales[8 + k].
+void encode_q3k(const float* x, uint8_t* blk) {
+    float scale[16], max_scale = 0.0f;
+    for (int s = 0; s < 16; ++s) {
+        float peak = 0.0f;
+        for (int l = 0; l < 16; ++l)
+            if (std::fabs(x[s * 16 + l]) > std::fabs(peak)) peak = x[s * 16 + l];
+        scale[s] = -peak / 4.0f;
+        max_scale = std::max(max_scale, std::fabs(scale[s]));
+    }
+    put_f16(blk + 108, max_scale / 31.0f);
+    const float d = f16_to_f32((uint16_t)(blk[108] | (blk[109] << 8)));
+    std::memset(blk, 0, 108);
+    for (int s = 0; s < 16; ++s) {
+        const int sc = d > 0.0f ? clampi((int)std::lround(scale[s] / d), -31, 31) : 0;
+        const int field = sc + 32, g = s / 4, k = s % 4;
+        blk[96 + 4 * (g & 1) + k] |= (uint8_t)((field & 0xF) << (g < 2 ? 0 : 4));
+        blk[96 + 8 + k] |= (uint8_t)((field >> 4) << (2 * g));
+        const float ws = d * (float)sc;
+        const int n = s / 8, j = (s % 8) / 2, h = s & 1;
+        for (int l = 0; l < 16; ++l) {
+            const int c = ws != 0.0f ? clampi((int)std::lround(x[s * 16 + l] / ws) + 4, 0, 7) : 4;
+            blk[32 + 32 * n + 16 * h + l] |= (uint8_t)((c & 3) << (2 * j));
+            blk[16 * h + l] |= (uint8_t)((c >> 2) << (4 * n + j));
+        }
+    }
+}
+
 // The 16-entry codebook of IQ4_NL (crates/infr-gguf/src/dequant.rs:439-441).
 const int kIq4nl[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
 
@@ -345,6 +414,8 @@ int infr_block_layout(int dtype, int* elems, int* bytes) {
     case INFR_DTYPE_Q5_0: e = 32; b = 22; break;
     case INFR_DTYPE_Q5_1: e = 32; b = 24; break;
     case INFR_DTYPE_Q5_K: e = 256; b = 176; break;
+    case INFR_DTYPE_Q2_K: e = 256; b = 84; break;
+    case INFR_DTYPE_Q3_K: e = 256; b = 110; break;
     case INFR_DTYPE_IQ4_NL: e = 32; b = 18; break;
     default: return 0;
     }
@@ -392,6 +463,8 @@ size_t infr_synth_weight(int dtype, uint64_t seed, float sigma, size_t rows, siz
             if (dtype == INFR_DTYPE_Q4_K) encode_q4k(x.data(), blk);
             else if (dtype == INFR_DTYPE_Q5_K) encode_q5k(x.data(), blk);
             else if (dtype == INFR_DTYPE_Q6_K) encode_q6k(x.data(), blk);
+            else if (dtype == INFR_DTYPE_Q2_K) encode_q2k(x.data(), blk);
+            else if (dtype == INFR_DTYPE_Q3_K) encode_q3k(x.data(), blk);
             else if (dtype == INFR_DTYPE_Q8_0) encode_q8_0(x.data(), blk);
             else encode_blk32(dtype, x.data(), blk);
         }

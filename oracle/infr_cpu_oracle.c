@@ -30,6 +30,8 @@ int orc_block_layout(int dtype, int *elems, int *bytes) {
     case ORC_IQ4_NL: e = 32; b = 18; break;
     case ORC_Q8_0: e = 32; b = 34; break;
     case ORC_Q5_K: e = 256; b = 176; break;
+    case ORC_Q2_K: e = 256; b = 84; break;
+    case ORC_Q3_K: e = 256; b = 110; break;
     case ORC_Q4_K: e = 256; b = 144; break;
     case ORC_Q6_K: e = 256; b = 210; break;
     case ORC_Q2_0: e = 64; b = 18; break;
@@ -257,6 +259,53 @@ int orc_dequant_block(int dtype, const uint8_t *bytes, size_t nbytes, float *out
                     o[j * 64 + 32 + l] = fs2 * (float)c2 + fm2;
                 }
             }
+        }
+        return 0;
+    case ORC_Q2_K:
+        /* dequant.rs:220-247: [u8 scales[16]][u8 qs[64]][f16 d][f16 dmin]; sub-block `is` (16
+         * elements, output order) = 8n + 2j + half reads qs[32n + 16half + l] >> 2j; its scale byte
+         * holds the 4-bit scale (low) and the 4-bit min (high). y = (d*scale)*code + dmin*(-min). */
+        for (size_t b = 0; b < nblk; b++) {
+            const uint8_t *blk = bytes + b * 84;
+            const uint8_t *scales = blk, *qs = blk + 16;
+            float d = orc_rdf16(blk + 80), dmin = orc_rdf16(blk + 82);
+            float *o = out + b * 256;
+            int is = 0;
+            for (int n = 0; n < 2; n++)
+                for (int j = 0; j < 4; j++)
+                    for (int half = 0; half < 2; half++, is++) {
+                        float fs = d * (float)(int16_t)(scales[is] & 0xF);
+                        float fm = dmin * (float)(int16_t)(-(int16_t)(scales[is] >> 4));
+                        for (int l = 0; l < 16; l++) {
+                            uint8_t c = (uint8_t)((qs[32 * n + 16 * half + l] >> (2 * j)) & 3);
+                            o[is * 16 + l] = fs * (float)c + fm;
+                        }
+                    }
+        }
+        return 0;
+    case ORC_Q3_K:
+        /* dequant.rs:248-298: [u8 hmask[32]][u8 qs[64]][u8 scales[12]][f16 d]; the code's low two
+         * bits are laid out as Q2_K's, its third bit is bit 4n + j of hmask[16half + l]; scale
+         * s = sc6 - 32 per 16 elements, min -4s, both against d: y = (d*s)*code + d*(-4s). */
+        for (size_t b = 0; b < nblk; b++) {
+            const uint8_t *blk = bytes + b * 110;
+            const uint8_t *hmask = blk, *qs = blk + 32;
+            int16_t sc[16];
+            orc_q3k_scales(blk + 96, sc);
+            float d = orc_rdf16(blk + 108);
+            float *o = out + b * 256;
+            int is = 0;
+            for (int n = 0; n < 2; n++)
+                for (int j = 0; j < 4; j++)
+                    for (int half = 0; half < 2; half++, is++) {
+                        float fs = d * (float)sc[is];
+                        float fm = d * (float)(int16_t)(-4 * sc[is]);
+                        for (int l = 0; l < 16; l++) {
+                            uint8_t low2 = (uint8_t)((qs[32 * n + 16 * half + l] >> (2 * j)) & 3);
+                            uint8_t high = (uint8_t)((hmask[16 * half + l] >> (4 * n + j)) & 1);
+                            o[is * 16 + l] = fs * (float)(uint8_t)(low2 | (high << 2)) + fm;
+                        }
+                    }
         }
         return 0;
     case ORC_IQ4_NL:
@@ -526,6 +575,85 @@ float orc_vec_dot_q5k(const uint8_t *row, const int8_t *qs8, const float *d8, co
     return sumf;
 }
 
+/* crates/infr-cpu/src/kernels.rs:764-783 (q3k_scales): the 12 scale bytes as three little-endian
+ * words a0, a1, t; sixteen 6-bit fields = low nibbles of a0, a1, high nibbles of a0, a1, each with
+ * two more bits from t (t, t >> 2, t >> 4, t >> 6); minus 32. */
+void orc_q3k_scales(const uint8_t *r, int16_t out[16]) {
+    uint32_t a0 = (uint32_t)r[0] | ((uint32_t)r[1] << 8) | ((uint32_t)r[2] << 16) | ((uint32_t)r[3] << 24);
+    uint32_t a1 = (uint32_t)r[4] | ((uint32_t)r[5] << 8) | ((uint32_t)r[6] << 16) | ((uint32_t)r[7] << 24);
+    uint32_t t = (uint32_t)r[8] | ((uint32_t)r[9] << 8) | ((uint32_t)r[10] << 16) | ((uint32_t)r[11] << 24);
+    const uint32_t k1 = 0x03030303u, k2 = 0x0f0f0f0fu;
+    uint32_t aux[4];
+    aux[0] = (a0 & k2) | ((t & k1) << 4);
+    aux[1] = (a1 & k2) | (((t >> 2) & k1) << 4);
+    aux[2] = ((a0 >> 4) & k2) | (((t >> 4) & k1) << 4);
+    aux[3] = ((a1 >> 4) & k2) | (((t >> 6) & k1) << 4);
+    for (int i = 0; i < 16; i++)
+        out[i] = (int16_t)((int16_t)(int8_t)(uint8_t)((aux[i / 4] >> ((i % 4) * 8)) & 0xFF) - 32);
+}
+
+/* crates/infr-cpu/src/kernels.rs:315-361 (vec_dot_q2k_scalar). */
+float orc_vec_dot_q2k(const uint8_t *row, const int8_t *qs8, const float *d8, const int32_t *bsums16,
+                      size_t in_f, int32_t *sd_out, int32_t *sm_out) {
+    size_t nb = in_f / 256;
+    float sumf = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * 84;
+        const uint8_t *scales = blk, *qs = blk + 16;
+        float d = orc_rdf16(blk + 80), dmin = orc_rdf16(blk + 82);
+        const int8_t *q8b = qs8 + b * 256;
+        int32_t sd = 0, sm = 0;
+        int is = 0;
+        for (int n = 0; n < 2; n++)
+            for (int j = 0; j < 4; j++)
+                for (int half = 0; half < 2; half++, is++) {
+                    int32_t scale = scales[is] & 0xF, minv = scales[is] >> 4;
+                    const uint8_t *qb = qs + 32 * n + 16 * half;
+                    int32_t iprod = 0;
+                    for (int l = 0; l < 16; l++)
+                        iprod += (int32_t)((qb[l] >> (2 * j)) & 3) * (int32_t)q8b[is * 16 + l];
+                    sd += scale * iprod;
+                    sm += minv * bsums16[b * 16 + is];
+                }
+        if (sd_out) sd_out[b] = sd;
+        if (sm_out) sm_out[b] = sm;
+        sumf += d8[b] * (d * (float)sd - dmin * (float)sm);
+    }
+    return sumf;
+}
+
+/* crates/infr-cpu/src/kernels.rs:812-852 (vec_dot_q3k_scalar). */
+float orc_vec_dot_q3k(const uint8_t *row, const int8_t *qs8, const float *d8, const int32_t *bsums16,
+                      size_t in_f, int32_t *isum_out) {
+    size_t nb = in_f / 256;
+    float sumf = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * 110;
+        const uint8_t *hmask = blk, *qs = blk + 32;
+        int16_t sc[16];
+        orc_q3k_scales(blk + 96, sc);
+        float d = orc_rdf16(blk + 108);
+        const int8_t *q8b = qs8 + b * 256;
+        int32_t isum = 0;
+        int is = 0;
+        for (int n = 0; n < 2; n++)
+            for (int j = 0; j < 4; j++)
+                for (int half = 0; half < 2; half++, is++) {
+                    const uint8_t *qb = qs + 32 * n + 16 * half, *hb = hmask + 16 * half;
+                    int32_t iprod = 0;
+                    for (int l = 0; l < 16; l++) {
+                        int32_t low2 = (qb[l] >> (2 * j)) & 3;
+                        int32_t high = ((hb[l] >> (4 * n + j)) & 1) ? 4 : 0;
+                        iprod += (low2 | high) * (int32_t)q8b[is * 16 + l];
+                    }
+                    isum += (int32_t)sc[is] * (iprod - 4 * bsums16[b * 16 + is]);
+                }
+        if (isum_out) isum_out[b] = isum;
+        sumf += d * d8[b] * (float)isum;
+    }
+    return sumf;
+}
+
 /* The 32-weight-block formats against the per-32 activation, one activation row of the batch
  * scalars: Q4_0 kernels.rs:5496-5520, Q4_1 :5793-5822, Q5_0 :5350-5377, Q5_1 :5948-5980,
  * IQ4_NL :6128-6152. Element j of a block takes the low nibble of qs[j], element j+16 the high
@@ -697,7 +825,7 @@ typedef struct {
 /* lib.rs:1037-1062: per-256 `Q8` for the 256-block formats and for Q8_0 rows of whole 256s;
  * a Q8_0 row that is a multiple of 32 only takes the per-32 `Q8x32` (q8_0_blk32). */
 static int is_q8_super(int dtype, size_t in_f) {
-    return dtype == ORC_Q4_K || dtype == ORC_Q5_K || dtype == ORC_Q6_K ||
+    return dtype == ORC_Q4_K || dtype == ORC_Q5_K || dtype == ORC_Q6_K || dtype == ORC_Q2_K || dtype == ORC_Q3_K ||
            (dtype == ORC_Q8_0 && in_f % 256 == 0);
 }
 
@@ -761,6 +889,14 @@ static float row_dot(int dtype, const uint8_t *row, const acts_t *a, size_t r, s
         return orc_vec_dot_q5k(row, a->qs + r * in_f, a->d + r * nb, a->bsums + r * nb * 8, in_f,
                                ia, ib);
     }
+    case ORC_Q2_K: {
+        size_t nb = in_f / 256;
+        return orc_vec_dot_q2k(row, a->qs + r * in_f, a->d + r * nb, a->bsums16 + r * nb * 16, in_f, ia, ib);
+    }
+    case ORC_Q3_K: {
+        size_t nb = in_f / 256;
+        return orc_vec_dot_q3k(row, a->qs + r * in_f, a->d + r * nb, a->bsums16 + r * nb * 16, in_f, ia);
+    }
     case ORC_Q4_0:
     case ORC_Q4_1:
     case ORC_Q5_0:
@@ -782,6 +918,8 @@ static int linear_shape_ok(int dtype, size_t in_f) {
     switch (dtype) {
     case ORC_Q4_K:
     case ORC_Q5_K:
+    case ORC_Q2_K:
+    case ORC_Q3_K:
     case ORC_Q6_K: return in_f % 256 == 0;
     case ORC_Q4_0:
     case ORC_Q4_1:
@@ -878,7 +1016,7 @@ int orc_linear_int_stages(int dtype, const uint8_t *w, size_t wbytes, size_t w_n
     size_t row0 = w_off / in_f;
     if (row0 + out_f > total_rows) return -2;
     const uint8_t *wb = w + row0 * bpr;
-    size_t blocks = (dtype == ORC_Q4_K || dtype == ORC_Q5_K || dtype == ORC_Q6_K) ? in_f / 256 : in_f / 32;
+    size_t blocks = (dtype == ORC_Q4_K || dtype == ORC_Q5_K || dtype == ORC_Q6_K || dtype == ORC_Q2_K || dtype == ORC_Q3_K) ? in_f / 256 : in_f / 32;
     acts_t a;
     acts_build(dtype, x, m, in_f, &a);
 #pragma omp parallel for schedule(dynamic, 8)
@@ -1226,6 +1364,11 @@ size_t orc_synth_weight(int dtype, size_t n_elem, uint32_t seed, uint8_t *out) {
             put_f16(blk, 0.05f);
             put_f16(blk + 2, 0.10f);
             break;
+        case ORC_Q2_K: /* d@80, dmin@82 (decode_spec.rs:323) */
+            put_f16(blk + 80, 0.05f);
+            put_f16(blk + 82, 0.10f);
+            break;
+        case ORC_Q3_K: put_f16(blk + 108, 0.03f); break; /* d@108 (decode_spec.rs:325) */
         case ORC_Q4_0:
         case ORC_Q5_0: put_f16(blk, 0.04f); break;
         case ORC_Q4_1:

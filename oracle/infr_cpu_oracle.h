@@ -24,6 +24,11 @@
  *                                 the reference's five single-block known answers; hand blocks for
  *                                 the 5th code bit; independent numpy decoders bit for bit; int64
  *                                 brute-force stages; per-block f32 terms re-evaluated in numpy f32
+ *   Q2_K / Q3_K (dequant, orc_vec_dot_q2k, orc_vec_dot_q3k, orc_q3k_scales)
+ *                                 the reference's q2k_single_block / q3k_single_block known answers;
+ *                                 hand blocks (each shift position, the hmask bit, a split scale
+ *                                 field); independent numpy decoders bit for bit; int64 brute-force
+ *                                 stages; per-superblock f32 terms re-evaluated in numpy f32
  *   orc_vec_dot_q8_0_32           brute-force int64 dots; hand-derived known answer
  *   orc_rms_norm / orc_gated_act* / orc_add / orc_act
  *                                 closed forms at hand-picked points; layouts against written-out
@@ -55,6 +60,8 @@ enum {
     ORC_Q5_0 = 6,
     ORC_Q5_1 = 7,
     ORC_Q8_0 = 8,
+    ORC_Q2_K = 10,
+    ORC_Q3_K = 11,
     ORC_Q4_K = 12,
     ORC_Q5_K = 13,
     ORC_Q6_K = 14,
@@ -110,6 +117,14 @@ float orc_vec_dot_q2_0(const uint8_t *row, const int8_t *qs, const float *d, con
 /* Q5_K: kernels.rs:1286-1327 — sd[nb], sm[nb] like Q4_K. */
 float orc_vec_dot_q5k(const uint8_t *row, const int8_t *qs, const float *d, const int32_t *bsums,
                       size_t in_f, int32_t *sd_out, int32_t *sm_out);
+/* Q2_K: kernels.rs:315-361 (vec_dot_q2k_scalar) - sd[nb], sm[nb]; the min term reads the per-16 sums. */
+float orc_vec_dot_q2k(const uint8_t *row, const int8_t *qs, const float *d, const int32_t *bsums16,
+                      size_t in_f, int32_t *sd_out, int32_t *sm_out);
+/* Q3_K: kernels.rs:812-852 (vec_dot_q3k_scalar), scales by kernels.rs:764-783 (q3k_scales) - isum[nb]. */
+float orc_vec_dot_q3k(const uint8_t *row, const int8_t *qs, const float *d, const int32_t *bsums16,
+                      size_t in_f, int32_t *isum_out);
+/* Q3_K's sixteen signed scales (sc6 - 32) of one block from its 12 scale bytes (kernels.rs:764-783). */
+void orc_q3k_scales(const uint8_t *scales_raw, int16_t out[16]);
 /* Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL against the per-32 activation: kernels.rs:5496-5520,
  * 5793-5822, 5350-5377, 5948-5980, 6128-6152 — iprod[in_f/32] (raw codes; IQ4_NL: codebook values). */
 float orc_vec_dot_blk32(int dtype, const uint8_t *row, const int8_t *qs, const float *d,

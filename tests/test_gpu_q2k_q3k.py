@@ -1,0 +1,156 @@
+"""GPU parity of Q2_K and Q3_K weights against the CPU oracle, through the C ABI: Op::Linear (one
+token and batches), Op::EmbedGather tables and Op::MoeFfn expert banks.
+
+infr-cpu multiplies both formats with a per-256 int8 activation (crates/infr-cpu/src/lib.rs:1093-1124,
+vec_dot_q2k / vec_dot_q3k in crates/infr-cpu/src/quant.rs): the integer stages must be equal and,
+since the device adds the per-superblock f32 terms in block order like the CPU, every output must
+be bit-identical. Weights are the oracle's full-range payloads (every 2-/3-bit code, all 6-bit
+scale patterns); the synthesiser behind the C ABI has no encoder for these two formats."""
+import numpy as np
+import pytest
+
+from infr_amd import Bindings, DType, Graph, InfrError, Linear, Status, TensorDesc, synth_normal_f32
+from oracle import oracle as orc
+from tests.test_gpu_linear import _oracle_rows, gate, run_linear
+from tests.test_gpu_moe import check, run_moe
+
+pytestmark = pytest.mark.gpu
+
+BOTH = [DType.Q2K, DType.Q3K]
+ids = lambda d: DType(d).name
+
+
+def bits(a):
+    return np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
+@pytest.mark.parametrize("dtype", BOTH, ids=ids)
+@pytest.mark.parametrize("in_f,out_f", [(256, 8), (768, 37), (2048, 100), (4096, 256), (5120, 64), (12288, 96),
+                                        (32768, 20), (1280, 1)])
+def test_decode_is_bit_identical_to_the_oracle(be, dtype, in_f, out_f):
+    w = orc.synth_weight(dtype, in_f * out_f, 0x51 + in_f)
+    x = synth_normal_f32(200 + out_f, in_f)
+    y = run_linear(be, dtype, w, x, 1, in_f, out_f)
+    want = orc.linear(dtype, w, x, 1, in_f, out_f)
+    gate(y, want)
+    assert np.array_equal(bits(y).ravel(), bits(want).ravel()), f"not bit-identical at {in_f} x {out_f}"
+
+
+@pytest.mark.parametrize("dtype", BOTH, ids=ids)
+@pytest.mark.parametrize("m", [1, 3, 8, 19])
+def test_int_stages_bit_exact(be, dtype, m):
+    in_f, out_f = 1024, 24
+    w = orc.synth_weight(dtype, in_f * out_f, 0x301 + dtype)
+    x = orc.gen_f32(m * in_f, 0x9E37 + dtype)
+    a, b = be.linear_int_stages(dtype, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
+    oa, ob = orc.linear_int_stages(dtype, w, x, m, in_f, out_f)
+    assert np.array_equal(a, oa)
+    if dtype == DType.Q2K:
+        assert np.array_equal(b, ob)         # the dmin stage: sum of (scale >> 4) * bsums16
+
+
+@pytest.mark.parametrize("dtype", BOTH, ids=ids)
+@pytest.mark.parametrize("m", [2, 5, 8, 9, 19, 40, 130])
+def test_batches_are_bit_identical_to_the_oracle(be, dtype, m):
+    """Up to eight tokens share one pass over the weights (activations in registers); beyond that the
+    weights are streamed once per eight tokens. Every token's value is the one-token value."""
+    in_f, out_f = 1024, 96
+    w = orc.synth_weight(dtype, in_f * out_f, 0x77 + m)
+    x = synth_normal_f32(8 + m, m * in_f)
+    x[:in_f] *= 29.0
+    x[in_f:2 * in_f] = 0.0           # an all-zero row
+    y = run_linear(be, dtype, w, x, m, in_f, out_f)
+    want = orc.linear(dtype, w, x, m, in_f, out_f).reshape(m, out_f)
+    assert np.all(y[1] == 0.0)
+    gate(y, want)
+    assert np.array_equal(bits(y), bits(want)), "not bit-identical"
+
+
+@pytest.mark.parametrize("dtype", BOTH, ids=ids)
+def test_batch_on_long_rows_and_many_rows(be, dtype):
+    for m, in_f, out_f in ((4, 8192, 40), (7, 4096, 1031), (3, 256, 5)):
+        w = orc.synth_weight(dtype, in_f * out_f, 0x99 + m)
+        x = orc.gen_f32(m * in_f, 0x1234 + m)
+        y = run_linear(be, dtype, w, x, m, in_f, out_f)
+        want = orc.linear(dtype, w, x, m, in_f, out_f).reshape(m, out_f)
+        assert np.array_equal(bits(y), bits(want)), f"not bit-identical at m {m}, {in_f} x {out_f}"
+
+
+@pytest.mark.parametrize("dtype", BOTH, ids=ids)
+def test_full_size_rows_vs_oracle(be, dtype):
+    in_f, out_f = 4096, 12288
+    w = orc.synth_weight(dtype, in_f * out_f, 900 + int(dtype))
+    x = synth_normal_f32(901, in_f)
+    y = run_linear(be, dtype, w, x, 1, in_f, out_f)
+    for row0 in (0, out_f // 2 - 7, out_f - 48):
+        want = _oracle_rows(dtype, w, x, 1, in_f, out_f, row0, 48)
+        got = y[:, row0:row0 + 48]
+        gate(got, want)
+        assert np.array_equal(bits(got), bits(want)), "not bit-identical"
+
+
+@pytest.mark.parametrize("dtype", BOTH, ids=ids)
+def test_w_off_selects_rows_of_a_concatenated_weight(be, dtype):
+    """Q2_K rows are 84 bytes per 256 weights, Q3_K rows 110: row starts fall on 4- and 2-byte
+    boundaries only."""
+    in_f, rows = 768, 40
+    w = orc.synth_weight(dtype, in_f * rows, 3)
+    x = synth_normal_f32(4, in_f)
+    for row0, n in ((0, 40), (7, 16), (33, 7)):
+        y = run_linear(be, dtype, w, x, 1, in_f, n, w_off=row0 * in_f, w_numel=rows * in_f)
+        want = orc.linear(dtype, w, x, 1, in_f, n, w_numel=rows * in_f, w_off=row0 * in_f)
+        assert np.array_equal(bits(y).ravel(), bits(want).ravel())
+
+
+@pytest.mark.parametrize("dtype", BOTH, ids=ids)
+def test_rows_that_are_not_whole_superblocks_are_refused(be, dtype):
+    in_f, out_f = 256 + 32, 4
+    w = np.zeros(2 * out_f * orc.block_layout(dtype)[1], np.uint8)
+    with pytest.raises(InfrError) as e:
+        run_linear(be, dtype, w, np.zeros(in_f, np.float32), 1, in_f, out_f)
+    assert e.value.status == Status.Unsupported
+
+
+def test_a_plan_mixes_them_with_other_formats(be):
+    """One decode step's worth of Linears over one activation, each in its own format: the plan
+    groups by (format, in_f) and every output equals the single-op value."""
+    in_f = 2048
+    outs = [(DType.Q2K, 96), (DType.Q3K, 80), (DType.Q4K, 64), (DType.Q2K, 33), (DType.Q3K, 130)]
+    g = Graph()
+    x = g.input(TensorDesc((1, in_f), DType.F32))
+    ws, ys = [], []
+    for dt, out_f in outs:
+        ws.append(g.weight(TensorDesc((out_f, in_f), dt)))
+        ys.append(g.output(TensorDesc((1, out_f), DType.F32)))
+        g.push(Linear(x, ws[-1], ys[-1], 1, in_f, out_f))
+    xv = synth_normal_f32(77, in_f)
+    wv = [orc.synth_weight(dt, in_f * out_f, 0x600 + i) for i, (dt, out_f) in enumerate(outs)]
+    binds = Bindings().bind(x, be.upload_new(xv))
+    ybs = []
+    for i, (dt, out_f) in enumerate(outs):
+        ybs.append(be.alloc(out_f * 4))
+        binds.bind(ws[i], be.upload_new(wv[i])).bind(ys[i], ybs[-1])
+    plan = be.compile(g)
+    for _ in range(2):
+        be.execute(plan, binds)
+        for i, (dt, out_f) in enumerate(outs):
+            got = be.download(ybs[i], np.empty(out_f, np.float32))
+            want = orc.linear(dt, wv[i], xv, 1, in_f, out_f)
+            assert np.array_equal(bits(got), bits(want).ravel()), f"op {i} ({DType(dt).name}) differs"
+
+
+@pytest.mark.parametrize("rows", [1, 5])
+@pytest.mark.parametrize("dtype", BOTH, ids=ids)
+def test_moe_banks(be, dtype, rows):
+    """expert_acts_kind (crates/infr-cpu/src/moe.rs:42-53) has no int8 arm for these two formats:
+    their expert rows are decoded and multiplied with the raw activation row at every row count."""
+    ne, n_expert, n_used, nff = 512, 8, 2, 256
+    gate_w = orc.synth_weight(dtype, n_expert * nff * ne, 0x700)
+    up_w = orc.synth_weight(dtype, n_expert * nff * ne, 0x701)
+    down_w = orc.synth_weight(dtype, n_expert * ne * nff, 0x702)
+    x = synth_normal_f32(230 + rows, rows * ne)
+    router = synth_normal_f32(231, n_expert * ne, sigma=0.05)
+    got = run_moe(be, x, router, gate_w, up_w, down_w, rows, ne, n_expert, n_used, nff, 1.0, dtype)
+    want = orc.moe_ffn(x, router, gate_w, up_w, down_w, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
+                       gate_dtype=int(dtype), up_dtype=int(dtype), down_dtype=int(dtype))
+    check(*got, *want)
