@@ -826,6 +826,132 @@ struct Skinny16Q6K {
     }
 };
 
+// Q2_K (84-byte block: scales[16] (scale | min << 4 per 16 weights), qs[64], d, dmin;
+// crates/infr-cpu/src/kernels.rs:315-361): sd = sum_g sc_g * (q . q8)_g, sm = sum_g mn_g * bsum16_g,
+// y += q8.d[b] * (d * sd - dmin * sm). Lane (., kq = 2 n + half) owns bytes qs[16 kq .. 16 kq + 15]:
+// their bit pairs j = 0..3 are elements 128 n + 32 j + 16 half .. + 15, sub-block 8 n + 2 j + half,
+// so a K = 64 step takes bit pair j of every lane's 16 bytes and each lane's 16 K-slots are one
+// sub-block. A 2-bit code times a 4-bit scale fits a byte: the scaled codes are the operand and
+// four steps chain into sd; a second chain against bytes that all hold the sub-block's min sums
+// min * q8 over the sub-block - mn_g * bsum16_g without the sums. Exact integers either way.
+struct Skinny16Q2K {
+    static constexpr bool kPer32Acts = false, kTranspose16 = false;
+    static constexpr bool kSubScales = false;
+    static constexpr int kBlockBytes = 84;
+    static constexpr int kRowStride = 176;  // two blocks (168 bytes) padded: 44 words, eight rows' 16-byte reads cover all banks
+    __device__ static float accumulate(float acc, float dq, uint32_t ddm, int sd, float sm) {
+        return Skinny16Q4K::accumulate(acc, dq, ddm, sd, sm);
+    }
+    __device__ static void block(const uint8_t* wrow, int jj, const uint8_t* arow, const uint8_t*, const uint8_t*,
+                                 int kq, int (&sd)[4], float (&sm)[4], uint32_t& ddm) {
+        const uint8_t* wblk = wrow + jj * kBlockBytes;  // blocks are word-aligned, not 16-byte aligned
+        const int n = kq >> 1, half = kq & 1;
+        const int* qp = reinterpret_cast<const int*>(wblk + 16 + 16 * kq);
+        const int qw[4] = {qp[0], qp[1], qp[2], qp[3]};
+        const int* sp = reinterpret_cast<const int*>(wblk + 8 * n);
+        const uint32_t scw[2] = {(uint32_t)sp[0] >> (8 * half), (uint32_t)sp[1] >> (8 * half)};
+        ddm = *reinterpret_cast<const uint32_t*>(wblk + 80);
+        v4i ad = {0, 0, 0, 0}, am = {0, 0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t sb = (scw[j >> 1] >> (16 * (j & 1))) & 0xFFu;  // byte half + 2 j of scales[8 n ..]
+            const uint32_t s4 = sb & 15u;
+            const int mw = (int)((sb >> 4) * 0x01010101u);
+            v4i b;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) b[k] = scale_codes(((uint32_t)qw[k] >> (2 * j)) & 0x03030303u, s4);
+            const v4i a = *reinterpret_cast<const v4i*>(arow + 128 * n + 32 * j + 16 * half);
+            ad = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, ad, 0, 0, 0);
+            am = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, v4i{mw, mw, mw, mw}, am, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            sd[i] = ad[i];
+            sm[i] = (float)am[i];  // |sm| <= 15 * 127 * 256: exact
+        }
+    }
+};
+
+// Q3_K (110-byte block: hmask[32], qs[64], scales[12], d; crates/infr-cpu/src/kernels.rs:812-852,
+// scales by :764-783): isum = sum_g (sc6_g - 32) * sum (code - 4) * q8, y += (d * q8.d[b]) * isum.
+// Lanes own bytes and sub-blocks as for Q2_K; the third code bit of bit pair j is bit 4 n + j of
+// hmask[16 half + l]. (4 - code) * (sc6 - 32) lies in [-128, 124]: the lane builds that product's
+// eight values for its sub-block as a byte table - (4 - v) u - 32 (4 - v) for v < 4 and
+// (v - 4) (64 - u) - 32 (v - 4) above, u = sc6, each a packed multiply and a byte-wise subtract -
+// and one v_perm_b32 per word looks four codes up in it. Four K = 64 steps chain into -isum. A
+// stage of two blocks is 220 bytes: the second block sits 2 bytes off a word boundary in LDS and is
+// read as aligned words and shifted; rows are an even number of blocks.
+struct Skinny16Q3K {
+    static constexpr bool kPer32Acts = false, kTranspose16 = false;
+    static constexpr bool kSubScales = false;
+    static constexpr int kBlockBytes = 110;
+    static constexpr int kRowStride = 240;  // 220 rounded up: 60 words, eight rows' 16-byte reads cover all banks
+    __device__ static float accumulate(float acc, float dq, uint32_t ddm, int sd, float) {
+        return acc + (f16_bits_to_f32(ddm) * dq) * (float)sd;
+    }
+    template <bool ODD, int N>
+    __device__ static void words(const uint8_t* blk, int o, uint32_t (&out)[N]) {
+        if (!ODD) {
+#pragma unroll
+            for (int i = 0; i < N; ++i) out[i] = *reinterpret_cast<const uint32_t*>(blk + o + 4 * i);
+        } else {
+            uint32_t w[N + 1];
+#pragma unroll
+            for (int i = 0; i <= N; ++i) w[i] = *reinterpret_cast<const uint32_t*>(blk - 2 + o + 4 * i);
+#pragma unroll
+            for (int i = 0; i < N; ++i) out[i] = __builtin_amdgcn_alignbyte(w[i + 1], w[i], 2);
+        }
+    }
+    // x - y on each byte, modulo 256, without borrows between bytes
+    __device__ static uint32_t sub_bytes(uint32_t x, uint32_t y_low7, uint32_t not_y_top) {
+        return ((x | 0x80808080u) - y_low7) ^ (x & 0x80808080u) ^ not_y_top;
+    }
+    __device__ static uint32_t mul_bytes(uint32_t halves, uint32_t f) {
+        typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+        const us2 s = {(unsigned short)f, (unsigned short)f};
+        return __builtin_bit_cast(uint32_t, (us2)(__builtin_bit_cast(us2, halves) * s));
+    }
+    template <bool ODD>
+    __device__ static void block_at(const uint8_t* blk, const uint8_t* arow, int kq, int (&sd)[4], uint32_t& ddm) {
+        const int n = kq >> 1, half = kq & 1;
+        uint32_t qw[4], hw[4], scw[3];
+        words<ODD, 4>(blk, 32 + 16 * kq, qw);
+        words<ODD, 4>(blk, 16 * half, hw);
+        words<ODD, 3>(blk, 96, scw);
+        ddm = *reinterpret_cast<const uint16_t*>(blk + 108);
+        // field 8 n + 2 j + half: low nibble in nibble n of byte 2 j + half of the first eight, top
+        // two bits at bit 4 n + 2 (j / 2) of byte 8 + 2 (j % 2) + half
+        const int sh = 8 * half + 4 * n;
+        const uint32_t a0 = scw[0] >> sh, a1 = scw[1] >> sh, tt = scw[2] >> sh;
+        v4i acc = {0, 0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t u = (((j < 2 ? a0 : a1) >> (16 * (j & 1))) & 15u) | (((tt >> (16 * (j & 1) + 2 * (j >> 1))) & 3u) << 4);
+            // table[v] = (4 - v) * (u - 32) as int8, v = 0..3 in t_lo, 4..7 in t_hi
+            const uint32_t t_lo = sub_bytes(mul_bytes(0x01020304u, u), 0x20406000u, 0x80808000u);
+            const uint32_t t_hi = sub_bytes(mul_bytes(0x03020100u, 64u - u), 0x60402000u, 0x80808080u);
+            v4i b;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t low2 = (qw[k] >> (2 * j)) & 0x03030303u;
+                const uint32_t high = (hw[k] >> (4 * n + j)) & 0x01010101u;
+                b[k] = (int)__builtin_amdgcn_perm(t_hi, t_lo, low2 | (high << 2));
+            }
+            const v4i a = *reinterpret_cast<const v4i*>(arow + 128 * n + 32 * j + 16 * half);
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sd[i] = -acc[i];
+    }
+    __device__ static void block(const uint8_t* wrow, int jj, const uint8_t* arow, const uint8_t*, const uint8_t*,
+                                 int kq, int (&sd)[4], float (&sm)[4], uint32_t& ddm) {
+        if (jj & 1) block_at<true>(wrow + jj * kBlockBytes, arow, kq, sd, ddm);
+        else block_at<false>(wrow + jj * kBlockBytes, arow, kq, sd, ddm);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sm[i] = 0.0f;
+    }
+};
+
 // Q8_0 (34-byte blocks: f16 d, 32 int8 codes; crates/infr-cpu/src/kernels.rs:1170-1187): a 256-element
 // step is eight blocks, 272 bytes, each with a scale of its own. The stored codes are the operand:
 // one v_mfma_i32_16x16x32_i8 per block gives its exact iprod, and the f32 side is the CPU's chain
@@ -1055,9 +1181,9 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
     constexpr int kTileBytes = kZeroOff + 256;
     constexpr int kPh = BPW;                        // blocks of weights staged at a time: the wave's share of a pass
     constexpr int kRowStride = BPW == 2 ? F::kRowStride : kPh * kBlk + 16;
-    // a row's stage in 16-byte pieces, and a last piece of one word (Q6_K: 420 = 26 x 16 + 4)
+    // a row's stage in 16-byte pieces, and a last piece of one to three words (Q6_K: 420 = 26 x 16 + 4)
     constexpr int kFull = kPh * kBlk / 16, kTail = kPh * kBlk % 16;
-    static_assert(kTail == 0 || kTail == 4, "a stage is whole 16-byte pieces plus at most one word");
+    static_assert(kTail % 4 == 0, "a stage is whole 16-byte pieces plus at most three words");
     constexpr int kPieces = kFull + (kTail ? 1 : 0), kIt = (kPieces + 3) / 4;
     __shared__ __attribute__((aligned(16))) uint8_t w_l[NW][16 * kRowStride];
     __shared__ __attribute__((aligned(16))) uint8_t act_l[NW][kTileBytes];
@@ -1105,7 +1231,11 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
 #pragma unroll
         for (int it = 0; it < kIt; ++it) {
             if (pq + 4 * it < kFull) wreg[it] = kBlk % 16 == 0 ? load16(src + goff + 64 * it) : load16_a4(src + goff + 64 * it);
-            else if (kTail && pq + 4 * it == kFull) wreg[it].x = load_u32(src + goff + 64 * it);
+            else if (kTail && pq + 4 * it == kFull) {
+                wreg[it].x = load_u32(src + goff + 64 * it);
+                if (kTail >= 8) wreg[it].y = load_u32(src + goff + 64 * it + 4);
+                if (kTail >= 12) wreg[it].z = load_u32(src + goff + 64 * it + 8);
+            }
         }
     };
     uint8_t* wl = w_l[wave];
@@ -1113,7 +1243,12 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
 #pragma unroll
         for (int it = 0; it < kIt; ++it) {
             if (pq + 4 * it < kFull) *reinterpret_cast<v4i*>(wl + loff + 64 * it) = wreg[it];
-            else if (kTail && pq + 4 * it == kFull) *reinterpret_cast<int*>(wl + loff + 64 * it) = wreg[it].x;
+            else if (kTail && pq + 4 * it == kFull) {
+                int* dst = reinterpret_cast<int*>(wl + loff + 64 * it);
+                dst[0] = wreg[it].x;
+                if (kTail >= 8) dst[1] = wreg[it].y;
+                if (kTail >= 12) dst[2] = wreg[it].z;
+            }
         }
     };
     const uint8_t* wfrag = wl + r16 * kRowStride;
@@ -1281,8 +1416,11 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
 constexpr int kSkinny16Waves = 4, kSkinny16Blocks = 2;
 static bool skinny16_shape(int dtype, int nb, size_t m, size_t out_f) {
     const bool nib32 = dtype == 2 || dtype == 3 || dtype == 6 || dtype == 7 || dtype == 20;
-    if (dtype != 12 && dtype != 13 && dtype != 14 && dtype != 8 && dtype != 42 && !nib32) return false;
-    if (nb < kSkinny16Blocks || (nb % kSkinny16Blocks != 0 && (dtype == 14 || dtype == 42))) return false;
+    if (dtype != 12 && dtype != 13 && dtype != 14 && dtype != 8 && dtype != 42 && dtype != 10 && dtype != 11 && !nib32)
+        return false;
+    if (nb < kSkinny16Blocks || (nb % kSkinny16Blocks != 0 && (dtype == 14 || dtype == 42 || dtype == 11))) return false;
+    // Q2_K, Q3_K: the dot4 batches are the only other kernel, eight tokens per pass over the weights
+    if (dtype == 10 || dtype == 11) return m >= 3;
     if (m <= 16) {
         // the dot4 batch kernels, which unpack a weight once per two or four tokens, stay ahead at the
         // bottom: Q4_K at two tokens (4.3 / 4.0 / 5.5 / 5.6 against 3.7 / 3.4 / 4.2 / 4.2 TB/s on the four
@@ -1397,6 +1535,10 @@ static bool launch_mmq_skinny16(int dtype, const uint8_t* w, size_t bpr, const A
         launch_mmq_skinny16_fmt<Skinny16Nib32<Nib32::Q5_1>, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     else if (dtype == 20)
         launch_mmq_skinny16_fmt<Skinny16Nib32<Nib32::IQ4_NL>, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
+    else if (dtype == 10)
+        launch_mmq_skinny16_fmt<Skinny16Q2K, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
+    else if (dtype == 11)
+        launch_mmq_skinny16_fmt<Skinny16Q3K, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     else
         launch_mmq_skinny16_fmt<Skinny16Q6K, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     return true;

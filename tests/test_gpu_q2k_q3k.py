@@ -5,7 +5,7 @@ infr-cpu multiplies both formats with a per-256 int8 activation (crates/infr-cpu
 vec_dot_q2k / vec_dot_q3k in crates/infr-cpu/src/quant.rs): the integer stages must be equal and,
 since the device adds the per-superblock f32 terms in block order like the CPU, every output must
 be bit-identical. Weights are the oracle's full-range payloads (every 2-/3-bit code, all 6-bit
-scale patterns); the synthesiser behind the C ABI has no encoder for these two formats."""
+scale patterns, both signs of the Q3_K scales)."""
 import numpy as np
 import pytest
 
@@ -52,8 +52,10 @@ def test_int_stages_bit_exact(be, dtype, m):
 @pytest.mark.parametrize("dtype", BOTH, ids=ids)
 @pytest.mark.parametrize("m", [2, 5, 8, 9, 19, 40, 130])
 def test_batches_are_bit_identical_to_the_oracle(be, dtype, m):
-    """Up to eight tokens share one pass over the weights (activations in registers); beyond that the
-    weights are streamed once per eight tokens. Every token's value is the one-token value."""
+    """Two tokens share one pass of the dot4 kernel over the weights; from three the 16-token K-split
+    MFMA kernel takes rows of two superblocks and more (an even number of them for Q3_K), 16 tokens
+    at a time; other rows keep the dot4 kernel, eight tokens per pass. Every token's value is the
+    one-token value."""
     in_f, out_f = 1024, 96
     w = orc.synth_weight(dtype, in_f * out_f, 0x77 + m)
     x = synth_normal_f32(8 + m, m * in_f)
@@ -68,7 +70,7 @@ def test_batches_are_bit_identical_to_the_oracle(be, dtype, m):
 
 @pytest.mark.parametrize("dtype", BOTH, ids=ids)
 def test_batch_on_long_rows_and_many_rows(be, dtype):
-    for m, in_f, out_f in ((4, 8192, 40), (7, 4096, 1031), (3, 256, 5)):
+    for m, in_f, out_f in ((4, 8192, 40), (7, 4096, 1031), (3, 256, 5), (5, 768, 33), (16, 1280, 50), (12, 2048, 17)):
         w = orc.synth_weight(dtype, in_f * out_f, 0x99 + m)
         x = orc.gen_f32(m * in_f, 0x1234 + m)
         y = run_linear(be, dtype, w, x, m, in_f, out_f)
@@ -137,6 +139,35 @@ def test_a_plan_mixes_them_with_other_formats(be):
             got = be.download(ybs[i], np.empty(out_f, np.float32))
             want = orc.linear(dt, wv[i], xv, 1, in_f, out_f)
             assert np.array_equal(bits(got), bits(want).ravel()), f"op {i} ({DType(dt).name}) differs"
+
+
+@pytest.mark.parametrize("m", [6, 24])
+def test_a_batch_plan_groups_them(be, m):
+    """Linears of one level over one activation tensor at several tokens: the plan shares one
+    quantized activation and one launch per (format, in_f) group."""
+    in_f = 2048
+    outs = [(DType.Q2K, 96), (DType.Q2K, 40), (DType.Q3K, 80), (DType.Q3K, 33), (DType.Q4K, 64)]
+    g = Graph()
+    x = g.input(TensorDesc((m, in_f), DType.F32))
+    ws, ys = [], []
+    for dt, out_f in outs:
+        ws.append(g.weight(TensorDesc((out_f, in_f), dt)))
+        ys.append(g.output(TensorDesc((m, out_f), DType.F32)))
+        g.push(Linear(x, ws[-1], ys[-1], m, in_f, out_f))
+    xv = synth_normal_f32(78, m * in_f)
+    wv = [orc.synth_weight(dt, in_f * out_f, 0x610 + i) for i, (dt, out_f) in enumerate(outs)]
+    binds = Bindings().bind(x, be.upload_new(xv))
+    ybs = []
+    for i, (dt, out_f) in enumerate(outs):
+        ybs.append(be.alloc(m * out_f * 4))
+        binds.bind(ws[i], be.upload_new(wv[i])).bind(ys[i], ybs[-1])
+    plan = be.compile(g)
+    for _ in range(2):
+        be.execute(plan, binds)
+        for i, (dt, out_f) in enumerate(outs):
+            got = be.download(ybs[i], np.empty((m, out_f), np.float32))
+            want = orc.linear(dt, wv[i], xv, m, in_f, out_f).reshape(m, out_f)
+            assert np.array_equal(bits(got), bits(want)), f"op {i} ({DType(dt).name}) differs"
 
 
 @pytest.mark.parametrize("rows", [1, 5])
