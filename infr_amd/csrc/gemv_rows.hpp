@@ -57,6 +57,13 @@ __device__ __forceinline__ void load_row_clamped(typename F::Row& r, const uint8
     if constexpr (F::kClampedLoads) F::load_row_clamped(r, rowp, 0, lane, ok);
     else F::load_row(r, rowp, 0, lane, ok);
 }
+// Whether the loop that runs one step ahead uses the unpredicated loader too (the loop that runs a
+// whole row ahead always does): a format says kClampedOneAhead = false when its predicated loads
+// measured faster there.
+template <typename F, typename = void>
+struct ClampedOneAhead : std::integral_constant<bool, F::kClampedLoads> {};
+template <typename F>
+struct ClampedOneAhead<F, std::void_t<decltype(F::kClampedOneAhead)>> : std::integral_constant<bool, F::kClampedOneAhead> {};
 
 // Rows [row0, row_end) of one weight matrix against activation registers `acts`. `first` already
 // holds step 0 of row0 - every step of it when FIRST_WHOLE - (the caller issues those loads as
@@ -223,7 +230,7 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
         for (int t = 0; t < STEPS; ++t) {
             typename F::Row nxt;
             if (t + 1 < STEPS) F::load_row(nxt, rowp, t + 1, lane, ok[t + 1 < STEPS ? t + 1 : 0]);
-            else if (F::kClampedLoads)  // the wave's last row prefetches itself again: no predicate
+            else if (ClampedOneAhead<F>::value)  // the wave's last row prefetches itself again: no predicate
                 load_row_clamped<F>(next0, row + 1 < row_end ? rowp + bpr : rowp, lane, ok[0]);
             else F::load_row(next0, rowp + bpr, 0, lane, ok[0] && row + 1 < row_end);
             take_term(t, F::template term<STAGES>(cur, acts[t], t, lane, ok[t], st, (size_t)row * n_units), s);
@@ -236,7 +243,7 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
     if constexpr (FIRST_WHOLE && STEPS > 1) {
         if (row < row_end) {  // every step of the first row is here already
             const uint8_t* rowp = w + (size_t)row * bpr;
-            if (F::kClampedLoads) load_row_clamped<F>(cur, row + 1 < row_end ? rowp + bpr : rowp, lane, ok[0]);
+            if (ClampedOneAhead<F>::value) load_row_clamped<F>(cur, row + 1 < row_end ? rowp + bpr : rowp, lane, ok[0]);
             else F::load_row(cur, rowp + bpr, 0, lane, ok[0] && row + 1 < row_end);
             float s = 0.0f;
 #pragma unroll
