@@ -34,6 +34,7 @@ class DType(IntEnum):
     Q5K = 13
     Q6K = 14
     IQ4NL = 20
+    IQ4XS = 23
     BF16 = 30    # plain rows, as F16
     I32 = 26     # token ids (never a weight here)
     Q2_0 = 42
@@ -638,7 +639,7 @@ class HipBackend:
         if w_numel is None:
             e, b = block_layout(dtype)
             w_numel = w.len_bytes() // b * e
-        blocks = in_f // 256 if dtype in (DType.Q4K, DType.Q5K, DType.Q6K, DType.Q2K, DType.Q3K) else in_f // 32
+        blocks = in_f // 256 if dtype in (DType.Q4K, DType.Q5K, DType.Q6K, DType.Q2K, DType.Q3K, DType.IQ4XS) else in_f // 32
         a = self.alloc(m * out_f * blocks * 4)
         b_ = self.alloc(m * out_f * blocks * 4) if dtype in (DType.Q4K, DType.Q5K, DType.Q2K) else None
         self._check(self._lib.infr_hip_linear_int_stages(

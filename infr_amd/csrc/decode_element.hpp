@@ -83,6 +83,15 @@ __device__ inline float decode_element(int dtype, const uint8_t* rowp, int e) {
         const float d = ldf16(blk + 108);
         return (d * (float)s) * (float)(low2 | (high << 2)) + d * (float)(-4 * s);
     }
+    case 23: {  // IQ4_XS: (d * (ls - 32)) * table[nibble] (dequant.rs:517-550)
+        const uint8_t* blk = rowp + (size_t)(e >> 8) * 136;
+        const int i = e & 255, ib = i >> 5, j = i & 15;
+        const uint32_t sh = ld8(blk + 2) | (ld8(blk + 3) << 8);
+        const int ls = (int)(((ld8(blk + 4 + (ib >> 1)) >> (4 * (ib & 1))) & 15u) | (((sh >> (2 * ib)) & 3u) << 4)) - 32;
+        const uint32_t nib = (ld8(blk + 8 + 16 * ib + j) >> (4 * ((i >> 4) & 1))) & 15u;
+        const int kv[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+        return (ldf16(blk) * (float)ls) * (float)kv[nib];
+    }
     case 14: {  // Q6_K
         const uint8_t* blk = rowp + (size_t)(e >> 8) * 210;
         const int i = e & 255, half = i >> 7, r = i & 127, col = r >> 5, l = r & 31;

@@ -1,4 +1,4 @@
-// Instantiates the decode GEMV templates for: FmtQ2K, FmtQ3K.
+// Instantiates the decode GEMV templates for: FmtQ2K, FmtQ3K, FmtIQ4XS.
 #include "gemv_impl.hpp"
 
 namespace infr {
@@ -9,6 +9,10 @@ const GemvFormatOps& gemv_ops_q2k() {
 }
 const GemvFormatOps& gemv_ops_q3k() {
     static const GemvFormatOps ops = make_gemv_format_ops<FmtQ3K>();
+    return ops;
+}
+const GemvFormatOps& gemv_ops_iq4xs() {
+    static const GemvFormatOps ops = make_gemv_format_ops<FmtIQ4XS>();
     return ops;
 }
 

@@ -795,6 +795,71 @@ __device__ __forceinline__ int iq4nl_lookup(uint32_t nib) {
     return (int)((hi & pick) | (lo & ~pick));
 }
 
+// ───────────────────────────────────── IQ4_XS ─────────────────────────────────────
+// 136-byte block, 8-byte aligned: [f16 d][u16 scales_h][u8 scales_l[4]][u8 qs[128]]. Sub-block ib
+// (32 weights) is 16 bytes - low nibbles elements 0..15, high nibbles 16..31 - of indices into
+// IQ4_NL's signed table, with a 6-bit scale ls (nibble ib of scales_l, two more bits from
+// scales_h), entering as ls - 32: isum = sum_ib (ls - 32) * (table[q] . q8), term
+// (d * q8.d[b]) * isum (crates/infr-cpu/src/kernels.rs:995-1036), blocks in ascending order.
+// Lanes as for Q4_K: block-in-step q = l / 4, lane p = l % 4 owns qs[32 p .. 32 p + 31] - sub-blocks
+// 2 p and 2 p + 1 - against 64 consecutive activation bytes.
+struct FmtIQ4XS {
+    static constexpr int kElemsPerStep = 4096;
+    static constexpr bool kPer32 = false;
+    static constexpr bool kOrdered = true;
+    static constexpr int kBlockBytes = 136, kBlockElems = 256;
+    static constexpr int kWide16Steps = 3;
+    static constexpr bool kClampedLoads = false;
+    static constexpr bool kLaneSums = true;
+    static constexpr bool kRowAhead = false;
+    struct Row {
+        v2i hdr;  // d | scales_h << 16, scales_l
+        v4i qa, qb;
+    };
+    typedef FmtQ4K::Acts Acts;
+    __device__ static int units(int in_f) { return in_f / 256; }
+    __device__ static bool valid(int t, int lane, int n) { return t * 16 + (lane >> 2) < n; }
+    __device__ static void load_row(Row& r, const uint8_t* rowp, int t, int lane, bool ok) {
+        if (ok) {
+            const uint8_t* blk = rowp + (size_t)(t * 16 + (lane >> 2)) * 136;
+            const int p = lane & 3;
+            r.hdr = gload<v2i_a4>(blk);
+            r.qa = load16_a4(blk + 8 + p * 32);
+            r.qb = load16_a4(blk + 24 + p * 32);
+        } else {
+            r.hdr = v2i{0, 0};
+            r.qa = r.qb = v4i{0, 0, 0, 0};
+        }
+    }
+    __device__ static void load_acts(Acts& a, const ActPtrs& s, int t, int lane, bool ok) {
+        FmtQ4K::load_acts(a, s, t, lane, ok);
+    }
+    template <bool STAGES>
+    __device__ static float term(const Row& r, const Acts& a, int t, int lane, bool ok,
+                                 const StagePtrs& st, size_t row_units) {
+        const int p = lane & 3;
+        const uint32_t m4 = 0x0F0F0F0Fu;
+        const int wa[4] = {r.qa.x, r.qa.y, r.qa.z, r.qa.w}, wb[4] = {r.qb.x, r.qb.y, r.qb.z, r.qb.w};
+        int ip_e = 0, ip_o = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            ip_e = dot4(iq4nl_lookup((uint32_t)wa[k] & m4), a.xa[k], ip_e);
+            ip_e = dot4(iq4nl_lookup(((uint32_t)wa[k] >> 4) & m4), a.xa[4 + k], ip_e);
+            ip_o = dot4(iq4nl_lookup((uint32_t)wb[k] & m4), a.xa[8 + k], ip_o);
+            ip_o = dot4(iq4nl_lookup(((uint32_t)wb[k] >> 4) & m4), a.xa[12 + k], ip_o);
+        }
+        // sub-blocks 2 p, 2 p + 1: nibbles 2 p, 2 p + 1 of scales_l, bits 4 p .. 4 p + 3 of scales_h
+        const uint32_t lo = (uint32_t)r.hdr.y >> (8 * p), hi = (uint32_t)r.hdr.x >> (16 + 4 * p);
+        const int ls_e = (int)((lo & 15u) | ((hi & 3u) << 4)) - 32;
+        const int ls_o = (int)(((lo >> 4) & 15u) | (((hi >> 2) & 3u) << 4)) - 32;
+        // |ip| <= 32 * 127 * 127: the 24-bit multiplies are exact
+        const int isum = quad_sum(__mul24(ls_e, ip_e) + __mul24(ls_o, ip_o));
+        if (STAGES && ok && p == 0) st.a[row_units + t * 16 + (lane >> 2)] = isum;
+        // sumf += d * q8.d[b] * isum as f32
+        return f16_bits_to_f32((uint32_t)r.hdr.x & 0xFFFFu) * a.dact * (float)isum;
+    }
+};
+
 template <Nib32 K>
 struct FmtNib32 {
     static constexpr bool kAffine = K == Nib32::Q4_1 || K == Nib32::Q5_1;

@@ -226,6 +226,7 @@ const GemvFormatOps& gemv_ops_q2_0_aligned();  // rows of whole 128s
 const GemvFormatOps& gemv_ops_q5k();
 const GemvFormatOps& gemv_ops_q2k();
 const GemvFormatOps& gemv_ops_q3k();
+const GemvFormatOps& gemv_ops_iq4xs();
 const GemvFormatOps& gemv_ops_q4_0();
 const GemvFormatOps& gemv_ops_q4_1();
 const GemvFormatOps& gemv_ops_q5_0();  // batch launchers only: one token takes the f32 kernel

@@ -952,6 +952,55 @@ struct Skinny16Q3K {
     }
 };
 
+// IQ4_XS (136-byte block: d, scales_h, scales_l[4], qs[128]; crates/infr-cpu/src/kernels.rs:995-1036):
+// isum = sum_ib (ls_ib - 32) * (table[q] . q8) over eight sub-blocks of 32, y += (d * q8.d[b]) * isum.
+// A table value times a 6-bit scale does not fit a byte, so a sub-block is one
+// v_mfma_i32_16x16x32_i8 (lane (., kq): elements 8 kq .. 8 kq + 7 - nibble kq / 2 of bytes
+// 8 (kq % 2) .. + 7 of the sub-block's 16, looked up in IQ4_NL's table) scaled into isum by a 24-bit
+// multiply-add. Blocks are 8-byte aligned; a stage of two is 272 bytes.
+struct Skinny16IQ4XS {
+    typedef int v2i __attribute__((ext_vector_type(2)));
+    static constexpr bool kPer32Acts = false, kTranspose16 = false;
+    static constexpr bool kSubScales = false;
+    static constexpr int kBlockBytes = 136;
+    static constexpr int kRowStride = 2 * kBlockBytes + 16;
+    __device__ static float accumulate(float acc, float dq, uint32_t ddm, int sd, float) {
+        return acc + (f16_bits_to_f32(ddm & 0xFFFFu) * dq) * (float)sd;
+    }
+    __device__ static int lookup(uint32_t nib) {  // IQ4_NL's table (crates/infr-gguf/src/dequant.rs:439-441)
+        const uint32_t sel = nib & 0x07070707u;
+        const uint32_t lo = __builtin_amdgcn_perm(0xF6EADDCFu, 0xBFAD9881u, sel);
+        const uint32_t hi = __builtin_amdgcn_perm(0x71594535u, 0x26190D01u, sel);
+        const uint32_t pick = ((nib >> 3) & 0x01010101u) * 0xFFu;
+        return (int)((hi & pick) | (lo & ~pick));
+    }
+    __device__ static void block(const uint8_t* wrow, int jj, const uint8_t* arow, const uint8_t*, const uint8_t*,
+                                 int kq, int (&sd)[4], float (&sm)[4], uint32_t& ddm) {
+        const uint8_t* wblk = wrow + jj * kBlockBytes;
+        const v2i hdr = *reinterpret_cast<const v2i*>(wblk);
+        ddm = (uint32_t)hdr.x;
+        const uint32_t sl = (uint32_t)hdr.y, sh = (uint32_t)hdr.x >> 16;
+        const int shift = 4 * (kq >> 1);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sd[i] = 0;
+#pragma unroll
+        for (int ib = 0; ib < 8; ++ib) {
+            const v2i q = *reinterpret_cast<const v2i*>(wblk + 8 + 16 * ib + 8 * (kq & 1));
+            v2i b;
+            b.x = lookup(((uint32_t)q.x >> shift) & 0x0F0F0F0Fu);
+            b.y = lookup(((uint32_t)q.y >> shift) & 0x0F0F0F0Fu);
+            const v2i a = *reinterpret_cast<const v2i*>(arow + ib * 32 + 8 * kq);
+            const v4i r = __builtin_amdgcn_mfma_i32_16x16x32_i8(__builtin_bit_cast(long, a), __builtin_bit_cast(long, b),
+                                                                v4i{0, 0, 0, 0}, 0, 0, 0);
+            const int ls = (int)(((sl >> (4 * ib)) & 15u) | (((sh >> (2 * ib)) & 3u) << 4)) - 32;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sd[i] += __mul24(r[i], ls);  // |r| <= 32 * 127 * 127
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sm[i] = 0.0f;
+    }
+};
+
 // Q8_0 (34-byte blocks: f16 d, 32 int8 codes; crates/infr-cpu/src/kernels.rs:1170-1187): a 256-element
 // step is eight blocks, 272 bytes, each with a scale of its own. The stored codes are the operand:
 // one v_mfma_i32_16x16x32_i8 per block gives its exact iprod, and the f32 side is the CPU's chain
@@ -1416,11 +1465,11 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
 constexpr int kSkinny16Waves = 4, kSkinny16Blocks = 2;
 static bool skinny16_shape(int dtype, int nb, size_t m, size_t out_f) {
     const bool nib32 = dtype == 2 || dtype == 3 || dtype == 6 || dtype == 7 || dtype == 20;
-    if (dtype != 12 && dtype != 13 && dtype != 14 && dtype != 8 && dtype != 42 && dtype != 10 && dtype != 11 && !nib32)
+    if (dtype != 12 && dtype != 13 && dtype != 14 && dtype != 8 && dtype != 42 && dtype != 10 && dtype != 11 && dtype != 23 && !nib32)
         return false;
     if (nb < kSkinny16Blocks || (nb % kSkinny16Blocks != 0 && (dtype == 14 || dtype == 42 || dtype == 11))) return false;
-    // Q2_K, Q3_K: the dot4 batches are the only other kernel, eight tokens per pass over the weights
-    if (dtype == 10 || dtype == 11) return m >= 3;
+    // Q2_K, Q3_K, IQ4_XS: the dot4 batches are the only other kernel, eight tokens per pass over the weights
+    if (dtype == 10 || dtype == 11 || dtype == 23) return m >= 3;
     if (m <= 16) {
         // the dot4 batch kernels, which unpack a weight once per two or four tokens, stay ahead at the
         // bottom: Q4_K at two tokens (4.3 / 4.0 / 5.5 / 5.6 against 3.7 / 3.4 / 4.2 / 4.2 TB/s on the four
@@ -1539,6 +1588,8 @@ static bool launch_mmq_skinny16(int dtype, const uint8_t* w, size_t bpr, const A
         launch_mmq_skinny16_fmt<Skinny16Q2K, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     else if (dtype == 11)
         launch_mmq_skinny16_fmt<Skinny16Q3K, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
+    else if (dtype == 23)
+        launch_mmq_skinny16_fmt<Skinny16IQ4XS, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     else
         launch_mmq_skinny16_fmt<Skinny16Q6K, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     return true;

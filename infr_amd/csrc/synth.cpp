@@ -327,6 +327,42 @@ void encode_q3k(const float* x, uint8_t* blk) {
 // The 16-entry codebook of IQ4_NL (crates/infr-gguf/src/dequant.rs:439-441).
 const int kIq4nl[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
 
+// 256 floats -> one 136-byte IQ4_XS block (d | scales_h | scales_l[4] | qs[128]): per 32-weight
+// sub-block the table value nearest to x / (d * (ls - 32)). A sub-block's scale is signed so that
+// its element of largest magnitude lands on the table's end value -127; ls - 32 in -31..31 against
+// one f16 super scale.
+void encode_iq4xs(const float* x, uint8_t* blk) {
+    float scale[8], max_scale = 0.0f;
+    for (int s = 0; s < 8; ++s) {
+        float peak = 0.0f;
+        for (int l = 0; l < 32; ++l)
+            if (std::fabs(x[s * 32 + l]) > std::fabs(peak)) peak = x[s * 32 + l];
+        scale[s] = -peak / 127.0f;
+        max_scale = std::max(max_scale, std::fabs(scale[s]));
+    }
+    put_f16(blk, max_scale / 31.0f);
+    const float d = f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+    std::memset(blk + 2, 0, 134);
+    uint32_t scales_h = 0;
+    for (int s = 0; s < 8; ++s) {
+        int sc = d > 0.0f ? clampi((int)std::lround(scale[s] / d), -31, 31) : 0;
+        if (sc == 0) sc = scale[s] < 0.0f ? -1 : 1;
+        const int ls = sc + 32;
+        blk[4 + s / 2] |= (uint8_t)((ls & 0xF) << (4 * (s & 1)));
+        scales_h |= (uint32_t)(ls >> 4) << (2 * s);
+        const float ws = d * (float)sc;
+        for (int l = 0; l < 32; ++l) {
+            const float v = ws != 0.0f ? x[s * 32 + l] / ws : 0.0f;
+            int best = 0;
+            for (int c = 1; c < 16; ++c)
+                if (std::fabs(v - (float)kIq4nl[c]) < std::fabs(v - (float)kIq4nl[best])) best = c;
+            blk[8 + 16 * s + (l & 15)] |= (uint8_t)(best << (4 * (l >> 4)));
+        }
+    }
+    blk[2] = (uint8_t)(scales_h & 0xFF);
+    blk[3] = (uint8_t)(scales_h >> 8);
+}
+
 // 32 floats -> one block of a 32-weight format. Element j's code goes to the low nibble of qs[j],
 // element j+16's to the high nibble; the 5-bit formats put the 5th bit of element e in bit e of qh.
 //   Q4_0 [d][qs]: symmetric, code = round(x/d) + 8        Q5_0 [d][qh][qs]: ... + 16
@@ -416,6 +452,7 @@ int infr_block_layout(int dtype, int* elems, int* bytes) {
     case INFR_DTYPE_Q5_K: e = 256; b = 176; break;
     case INFR_DTYPE_Q2_K: e = 256; b = 84; break;
     case INFR_DTYPE_Q3_K: e = 256; b = 110; break;
+    case INFR_DTYPE_IQ4_XS: e = 256; b = 136; break;
     case INFR_DTYPE_IQ4_NL: e = 32; b = 18; break;
     default: return 0;
     }
@@ -465,6 +502,7 @@ size_t infr_synth_weight(int dtype, uint64_t seed, float sigma, size_t rows, siz
             else if (dtype == INFR_DTYPE_Q6_K) encode_q6k(x.data(), blk);
             else if (dtype == INFR_DTYPE_Q2_K) encode_q2k(x.data(), blk);
             else if (dtype == INFR_DTYPE_Q3_K) encode_q3k(x.data(), blk);
+            else if (dtype == INFR_DTYPE_IQ4_XS) encode_iq4xs(x.data(), blk);
             else if (dtype == INFR_DTYPE_Q8_0) encode_q8_0(x.data(), blk);
             else encode_blk32(dtype, x.data(), blk);
         }

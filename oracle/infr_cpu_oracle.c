@@ -32,6 +32,7 @@ int orc_block_layout(int dtype, int *elems, int *bytes) {
     case ORC_Q5_K: e = 256; b = 176; break;
     case ORC_Q2_K: e = 256; b = 84; break;
     case ORC_Q3_K: e = 256; b = 110; break;
+    case ORC_IQ4_XS: e = 256; b = 136; break;
     case ORC_Q4_K: e = 256; b = 144; break;
     case ORC_Q6_K: e = 256; b = 210; break;
     case ORC_Q2_0: e = 64; b = 18; break;
@@ -316,6 +317,24 @@ int orc_dequant_block(int dtype, const uint8_t *bytes, size_t nbytes, float *out
             for (int j = 0; j < 16; j++) {
                 out[b * 32 + j] = d * (float)orc_kvalues_iq4nl[blk[2 + j] & 0xF];
                 out[b * 32 + j + 16] = d * (float)orc_kvalues_iq4nl[blk[2 + j] >> 4];
+            }
+        }
+        return 0;
+    case ORC_IQ4_XS:
+        /* dequant.rs:517-550: [f16 d][u16 scales_h][u8 scales_l[4]][u8 qs[128]]; eight sub-blocks of
+         * 32, ls = nibble ib of scales_l | two bits of scales_h << 4; y = (d * (ls - 32)) * codebook,
+         * low nibble of qs[16 ib + j] -> element 32 ib + j, high nibble -> 32 ib + j + 16. */
+        for (size_t b = 0; b < nblk; b++) {
+            const uint8_t *blk = bytes + b * 136;
+            float d = orc_rdf16(blk);
+            uint32_t scales_h = (uint32_t)blk[2] | ((uint32_t)blk[3] << 8);
+            for (int ib = 0; ib < 8; ib++) {
+                float dl = d * (float)orc_iq4xs_scale(scales_h, blk + 4, ib);
+                const uint8_t *qs = blk + 8 + 16 * ib;
+                for (int j = 0; j < 16; j++) {
+                    out[b * 256 + ib * 32 + j] = dl * (float)orc_kvalues_iq4nl[qs[j] & 0xF];
+                    out[b * 256 + ib * 32 + j + 16] = dl * (float)orc_kvalues_iq4nl[qs[j] >> 4];
+                }
             }
         }
         return 0;
@@ -654,6 +673,40 @@ float orc_vec_dot_q3k(const uint8_t *row, const int8_t *qs8, const float *d8, co
     return sumf;
 }
 
+/* crates/infr-cpu/src/kernels.rs:995-1002 (iq4xs_ls_minus_32): sub-block ib's 6-bit scale, minus 32. */
+int orc_iq4xs_scale(uint32_t scales_h, const uint8_t *scales_l, int ib) {
+    int lo = (scales_l[ib / 2] >> (4 * (ib % 2))) & 0xF;
+    int hi = (int)((scales_h >> (2 * ib)) & 3u);
+    return (lo | (hi << 4)) - 32;
+}
+
+/* crates/infr-cpu/src/kernels.rs:1008-1036 (vec_dot_iq4xs_scalar): per sub-block of 32 the signed
+ * codebook dot with the activation codes, weighted by (ls - 32) in i32; one f32 step per superblock. */
+float orc_vec_dot_iq4xs(const uint8_t *row, const int8_t *qs8, const float *d8, size_t in_f, int32_t *isum_out) {
+    size_t nb = in_f / 256;
+    float sumf = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * 136;
+        float d = orc_rdf16(blk);
+        uint32_t scales_h = (uint32_t)blk[2] | ((uint32_t)blk[3] << 8);
+        const int8_t *q8b = qs8 + b * 256;
+        int32_t isum = 0;
+        for (int ib = 0; ib < 8; ib++) {
+            const uint8_t *qsb = blk + 8 + 16 * ib;
+            const int8_t *a = q8b + 32 * ib;
+            int32_t dot = 0;
+            for (int j = 0; j < 16; j++) {
+                dot += (int32_t)orc_kvalues_iq4nl[qsb[j] & 0xF] * (int32_t)a[j];
+                dot += (int32_t)orc_kvalues_iq4nl[qsb[j] >> 4] * (int32_t)a[j + 16];
+            }
+            isum += orc_iq4xs_scale(scales_h, blk + 4, ib) * dot;
+        }
+        if (isum_out) isum_out[b] = isum;
+        sumf += d * d8[b] * (float)isum;
+    }
+    return sumf;
+}
+
 /* The 32-weight-block formats against the per-32 activation, one activation row of the batch
  * scalars: Q4_0 kernels.rs:5496-5520, Q4_1 :5793-5822, Q5_0 :5350-5377, Q5_1 :5948-5980,
  * IQ4_NL :6128-6152. Element j of a block takes the low nibble of qs[j], element j+16 the high
@@ -826,7 +879,7 @@ typedef struct {
  * a Q8_0 row that is a multiple of 32 only takes the per-32 `Q8x32` (q8_0_blk32). */
 static int is_q8_super(int dtype, size_t in_f) {
     return dtype == ORC_Q4_K || dtype == ORC_Q5_K || dtype == ORC_Q6_K || dtype == ORC_Q2_K || dtype == ORC_Q3_K ||
-           (dtype == ORC_Q8_0 && in_f % 256 == 0);
+           dtype == ORC_IQ4_XS || (dtype == ORC_Q8_0 && in_f % 256 == 0);
 }
 
 static void acts_free(acts_t *a) {
@@ -897,6 +950,7 @@ static float row_dot(int dtype, const uint8_t *row, const acts_t *a, size_t r, s
         size_t nb = in_f / 256;
         return orc_vec_dot_q3k(row, a->qs + r * in_f, a->d + r * nb, a->bsums16 + r * nb * 16, in_f, ia);
     }
+    case ORC_IQ4_XS: return orc_vec_dot_iq4xs(row, a->qs + r * in_f, a->d + r * (in_f / 256), in_f, ia);
     case ORC_Q4_0:
     case ORC_Q4_1:
     case ORC_Q5_0:
@@ -920,6 +974,7 @@ static int linear_shape_ok(int dtype, size_t in_f) {
     case ORC_Q5_K:
     case ORC_Q2_K:
     case ORC_Q3_K:
+    case ORC_IQ4_XS:
     case ORC_Q6_K: return in_f % 256 == 0;
     case ORC_Q4_0:
     case ORC_Q4_1:
@@ -1016,7 +1071,7 @@ int orc_linear_int_stages(int dtype, const uint8_t *w, size_t wbytes, size_t w_n
     size_t row0 = w_off / in_f;
     if (row0 + out_f > total_rows) return -2;
     const uint8_t *wb = w + row0 * bpr;
-    size_t blocks = (dtype == ORC_Q4_K || dtype == ORC_Q5_K || dtype == ORC_Q6_K || dtype == ORC_Q2_K || dtype == ORC_Q3_K) ? in_f / 256 : in_f / 32;
+    size_t blocks = (dtype == ORC_Q4_K || dtype == ORC_Q5_K || dtype == ORC_Q6_K || dtype == ORC_Q2_K || dtype == ORC_Q3_K || dtype == ORC_IQ4_XS) ? in_f / 256 : in_f / 32;
     acts_t a;
     acts_build(dtype, x, m, in_f, &a);
 #pragma omp parallel for schedule(dynamic, 8)
@@ -1369,6 +1424,7 @@ size_t orc_synth_weight(int dtype, size_t n_elem, uint32_t seed, uint8_t *out) {
             put_f16(blk + 82, 0.10f);
             break;
         case ORC_Q3_K: put_f16(blk + 108, 0.03f); break; /* d@108 (decode_spec.rs:325) */
+        case ORC_IQ4_XS: put_f16(blk, 0.06f); break;      /* d@0 (decode_spec.rs:351) */
         case ORC_Q4_0:
         case ORC_Q5_0: put_f16(blk, 0.04f); break;
         case ORC_Q4_1:

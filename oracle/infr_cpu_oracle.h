@@ -29,6 +29,9 @@
  *                                 hand blocks (each shift position, the hmask bit, a split scale
  *                                 field); independent numpy decoders bit for bit; int64 brute-force
  *                                 stages; per-superblock f32 terms re-evaluated in numpy f32
+ *   IQ4_XS (dequant, orc_vec_dot_iq4xs, orc_iq4xs_scale)
+ *                                 the reference's iq4xs_single_block known answer; a hand block with a
+ *                                 scale per sub-block and a code per nibble position; the rest as above
  *   orc_vec_dot_q8_0_32           brute-force int64 dots; hand-derived known answer
  *   orc_rms_norm / orc_gated_act* / orc_add / orc_act
  *                                 closed forms at hand-picked points; layouts against written-out
@@ -62,6 +65,7 @@ enum {
     ORC_Q8_0 = 8,
     ORC_Q2_K = 10,
     ORC_Q3_K = 11,
+    ORC_IQ4_XS = 23,
     ORC_Q4_K = 12,
     ORC_Q5_K = 13,
     ORC_Q6_K = 14,
@@ -123,6 +127,9 @@ float orc_vec_dot_q2k(const uint8_t *row, const int8_t *qs, const float *d, cons
 /* Q3_K: kernels.rs:812-852 (vec_dot_q3k_scalar), scales by kernels.rs:764-783 (q3k_scales) - isum[nb]. */
 float orc_vec_dot_q3k(const uint8_t *row, const int8_t *qs, const float *d, const int32_t *bsums16,
                       size_t in_f, int32_t *isum_out);
+/* IQ4_XS: kernels.rs:1008-1036 (vec_dot_iq4xs_scalar), scale by kernels.rs:995-1002 - isum[nb]. */
+float orc_vec_dot_iq4xs(const uint8_t *row, const int8_t *qs, const float *d, size_t in_f, int32_t *isum_out);
+int orc_iq4xs_scale(uint32_t scales_h, const uint8_t *scales_l, int ib);
 /* Q3_K's sixteen signed scales (sc6 - 32) of one block from its 12 scale bytes (kernels.rs:764-783). */
 void orc_q3k_scales(const uint8_t *scales_raw, int16_t out[16]);
 /* Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL against the per-32 activation: kernels.rs:5496-5520,

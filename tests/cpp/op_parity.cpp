@@ -63,7 +63,7 @@ static void hip_linear_all_weight_quants_match_the_host_oracle(HipBackend& be) {
         const auto cases = weight_quant_cases(m, 256, 8);
         const SweepReport r = sweep_linear_on("hip Linear m=" + std::to_string(m), be, cases,
                                               [](const LinearCase&) { return CPU_INT8_ACT_TOL; });
-        EXPECT(r.cases.size() == 12, "expected the twelve formats of this backend, got %zu", r.cases.size());
+        EXPECT(r.cases.size() == 13, "expected the thirteen formats of this backend, got %zu", r.cases.size());
         EXPECT(r.failures() == 0, "cases outside %.0e of the host decode oracle", CPU_INT8_ACT_TOL);
     }
 }
@@ -82,14 +82,14 @@ static void hip_linear_matches_the_cpu_production_arm(HipBackend& be) {
                 std::snprintf(what, sizeof what, "%s m=%zu %zux%zu", dtype_name(c.dtype), m, s[0], s[1]);
                 gate(what, got, want);
                 const bool ordered = c.dtype == DType::Q4K || c.dtype == DType::Q5K || c.dtype == DType::Q6K ||
-                                     c.dtype == DType::Q2K || c.dtype == DType::Q3K;
+                                     c.dtype == DType::Q2K || c.dtype == DType::Q3K || c.dtype == DType::IQ4XS;
                 if (ordered && m <= 8) EXPECT(same_bits(got, want), "%s: not bit-identical to infr-cpu", what);
             }
 }
 
 // batch == single, bit for bit (crates/infr-cpu/src/kernels.rs:9297-9405 holds the CPU to the same)
 static void hip_linear_batch_rows_equal_single_rows(HipBackend& be) {
-    for (DType dt : {DType::Q4K, DType::Q5K, DType::Q6K, DType::Q2K, DType::Q3K}) {
+    for (DType dt : {DType::Q4K, DType::Q5K, DType::Q6K, DType::Q2K, DType::Q3K, DType::IQ4XS}) {
         const LinearCase c{dt, 6, 1024, 40};
         auto [w, x] = case_inputs(c);
         const std::vector<float> batch = run_linear(be, c);
@@ -362,13 +362,13 @@ static void hip_backend_honours_the_seam_contract(HipBackend& be) {
     EXPECT(threw, "execute with an unbound weight did not report Invalid");
     // a format outside this backend is Unsupported at compile, never a wrong answer
     Graph g2;
-    const TensorId w2 = g2.weight({{8, 256}, (DType)23 /* IQ4_XS */});
+    const TensorId w2 = g2.weight({{8, 256}, (DType)39 /* MXFP4 */});
     const TensorId x2 = g2.input({{1, 256}, DType::F32});
     const TensorId d2 = g2.output({{1, 8}, DType::F32});
     g2.push(op::Linear{x2, w2, d2, 1, 256, 8, 0});
     threw = false;
     try { Plan p2 = be.compile(g2); } catch (const Error& e) { threw = e.kind == ErrorKind::Unsupported; }
-    EXPECT(threw, "IQ4_XS Linear did not report Unsupported");
+    EXPECT(threw, "MXFP4 Linear did not report Unsupported");
     // a ragged row is refused, not truncated
     Graph g3;
     const TensorId w3 = g3.weight({{8, 128}, DType::Q4K});

@@ -1,8 +1,8 @@
-"""GPU parity of Q2_K and Q3_K weights against the CPU oracle, through the C ABI: Op::Linear (one
-token and batches), Op::EmbedGather tables and Op::MoeFfn expert banks.
+"""GPU parity of Q2_K, Q3_K and IQ4_XS weights against the CPU oracle, through the C ABI: Op::Linear
+(one token and batches), Op::EmbedGather tables and Op::MoeFfn expert banks.
 
-infr-cpu multiplies both formats with a per-256 int8 activation (crates/infr-cpu/src/lib.rs:1093-1124,
-vec_dot_q2k / vec_dot_q3k in crates/infr-cpu/src/quant.rs): the integer stages must be equal and,
+infr-cpu multiplies these formats with a per-256 int8 activation (crates/infr-cpu/src/lib.rs:1043-1124,
+vec_dot_q2k / vec_dot_q3k / vec_dot_iq4xs in crates/infr-cpu/src/kernels.rs): the integer stages must be equal and,
 since the device adds the per-superblock f32 terms in block order like the CPU, every output must
 be bit-identical. Weights are the oracle's full-range payloads (every 2-/3-bit code, all 6-bit
 scale patterns, both signs of the Q3_K scales)."""
@@ -16,7 +16,7 @@ from tests.test_gpu_moe import check, run_moe
 
 pytestmark = pytest.mark.gpu
 
-BOTH = [DType.Q2K, DType.Q3K]
+BOTH = [DType.Q2K, DType.Q3K, DType.IQ4XS]
 ids = lambda d: DType(d).name
 
 
@@ -93,8 +93,8 @@ def test_full_size_rows_vs_oracle(be, dtype):
 
 @pytest.mark.parametrize("dtype", BOTH, ids=ids)
 def test_w_off_selects_rows_of_a_concatenated_weight(be, dtype):
-    """Q2_K rows are 84 bytes per 256 weights, Q3_K rows 110: row starts fall on 4- and 2-byte
-    boundaries only."""
+    """Q2_K rows are 84 bytes per 256 weights, Q3_K rows 110, IQ4_XS rows 136: row starts fall on
+    4-, 2- and 8-byte boundaries only."""
     in_f, rows = 768, 40
     w = orc.synth_weight(dtype, in_f * rows, 3)
     x = synth_normal_f32(4, in_f)
@@ -117,7 +117,8 @@ def test_a_plan_mixes_them_with_other_formats(be):
     """One decode step's worth of Linears over one activation, each in its own format: the plan
     groups by (format, in_f) and every output equals the single-op value."""
     in_f = 2048
-    outs = [(DType.Q2K, 96), (DType.Q3K, 80), (DType.Q4K, 64), (DType.Q2K, 33), (DType.Q3K, 130)]
+    outs = [(DType.Q2K, 96), (DType.Q3K, 80), (DType.Q4K, 64), (DType.Q2K, 33), (DType.Q3K, 130), (DType.IQ4XS, 70),
+            (DType.IQ4XS, 9)]
     g = Graph()
     x = g.input(TensorDesc((1, in_f), DType.F32))
     ws, ys = [], []
@@ -146,7 +147,8 @@ def test_a_batch_plan_groups_them(be, m):
     """Linears of one level over one activation tensor at several tokens: the plan shares one
     quantized activation and one launch per (format, in_f) group."""
     in_f = 2048
-    outs = [(DType.Q2K, 96), (DType.Q2K, 40), (DType.Q3K, 80), (DType.Q3K, 33), (DType.Q4K, 64)]
+    outs = [(DType.Q2K, 96), (DType.Q2K, 40), (DType.Q3K, 80), (DType.Q3K, 33), (DType.Q4K, 64), (DType.IQ4XS, 50),
+            (DType.IQ4XS, 31)]
     g = Graph()
     x = g.input(TensorDesc((m, in_f), DType.F32))
     ws, ys = [], []
@@ -173,7 +175,7 @@ def test_a_batch_plan_groups_them(be, m):
 @pytest.mark.parametrize("rows", [1, 5])
 @pytest.mark.parametrize("dtype", BOTH, ids=ids)
 def test_moe_banks(be, dtype, rows):
-    """expert_acts_kind (crates/infr-cpu/src/moe.rs:42-53) has no int8 arm for these two formats:
+    """expert_acts_kind (crates/infr-cpu/src/moe.rs:42-53) has no int8 arm for these formats:
     their expert rows are decoded and multiplied with the raw activation row at every row count."""
     ne, n_expert, n_used, nff = 512, 8, 2, 256
     gate_w = orc.synth_weight(dtype, n_expert * nff * ne, 0x700)
