@@ -35,6 +35,8 @@ class DType(IntEnum):
     Q6K = 14
     IQ4NL = 20
     IQ4XS = 23
+    MXFP4 = 39
+    NVFP4 = 40
     BF16 = 30    # plain rows, as F16
     I32 = 26     # token ids (never a weight here)
     Q2_0 = 42

@@ -138,7 +138,7 @@ bool is_quant(int dt) {
     switch (dt) {
     case INFR_DTYPE_Q4_0: case INFR_DTYPE_Q4_1: case INFR_DTYPE_Q5_0: case INFR_DTYPE_Q5_1:
     case INFR_DTYPE_Q8_0: case INFR_DTYPE_Q4_K: case INFR_DTYPE_Q5_K: case INFR_DTYPE_Q6_K:
-    case INFR_DTYPE_Q2_K: case INFR_DTYPE_Q3_K: case INFR_DTYPE_IQ4_XS:
+    case INFR_DTYPE_Q2_K: case INFR_DTYPE_Q3_K: case INFR_DTYPE_IQ4_XS: case INFR_DTYPE_MXFP4: case INFR_DTYPE_NVFP4:
     case INFR_DTYPE_IQ4_NL: case INFR_DTYPE_Q2_0: return true;
     default: return false;
     }
@@ -150,7 +150,7 @@ bool is_moe_quant(int dt) {
     case INFR_DTYPE_Q4_K: case INFR_DTYPE_Q5_K: case INFR_DTYPE_Q6_K: case INFR_DTYPE_Q8_0:
     case INFR_DTYPE_Q4_0: case INFR_DTYPE_Q4_1: case INFR_DTYPE_Q5_0: case INFR_DTYPE_Q5_1:
     case INFR_DTYPE_IQ4_NL: case INFR_DTYPE_Q2_0: case INFR_DTYPE_Q2_K: case INFR_DTYPE_Q3_K:
-    case INFR_DTYPE_IQ4_XS:
+    case INFR_DTYPE_IQ4_XS: case INFR_DTYPE_MXFP4: case INFR_DTYPE_NVFP4:
     case INFR_DTYPE_F32: case INFR_DTYPE_F16: case INFR_DTYPE_BF16:
         return true;
     default: return false;
@@ -357,7 +357,8 @@ int check_linear(infr_hip_t* be, int dtype, const infr_hip_buffer_t* w, size_t w
     out->bpr = bpr;
     // The kernels fetch blocks with 2-, 4- or 16-byte loads according to the block stride and
     // assume the first row starts where a row stride of that alignment would put it.
-    const uintptr_t align = bpr % 16 == 0 ? 16 : (bpr % 4 == 0 ? 4 : 2);
+    // (MXFP4's 17-byte blocks sit at any byte: its kernels fetch the aligned dwords around a block)
+    const uintptr_t align = dtype == INFR_DTYPE_MXFP4 ? 1 : (bpr % 16 == 0 ? 16 : (bpr % 4 == 0 ? 4 : 2));
     if (reinterpret_cast<uintptr_t>(out->wrows) % align != 0)
         return fail(be, INFR_HIP_ERR_INVALID,
                     "linear: weight rows start at an address that is not " + std::to_string(align) + "-byte aligned");
@@ -725,6 +726,8 @@ int infr_hip_linear_int_stages(infr_hip_t* be, int dtype, const infr_hip_buffer_
     if (int rc = check_latch(be)) return rc;
     LinearArgs la;
     if (int rc = check_linear(be, dtype, w, w_numel, w_off, x, m, in_f, out_f, &la)) return rc;
+    if (dtype == INFR_DTYPE_NVFP4)
+        return fail(be, INFR_HIP_ERR_UNSUPPORTED, "int_stages: NVFP4 has four integers per block, not one");
     const size_t blocks = stage_blocks(dtype, in_f);
     const size_t need = m * out_f * blocks * sizeof(int32_t);
     if (!a || a->len < need) return fail(be, INFR_HIP_ERR_INVALID, "int_stages: buffer a too small");

@@ -92,6 +92,24 @@ __device__ inline float decode_element(int dtype, const uint8_t* rowp, int e) {
         const int kv[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
         return (ldf16(blk) * (float)ls) * (float)kv[nib];
     }
+    case 39: {  // MXFP4: table[nibble] * 2^(e - 128) (dequant.rs:1024-1042)
+        const int kv[16] = {0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12};
+        const uint8_t* blk = rowp + (size_t)(e >> 5) * 17;
+        const int i = e & 31;
+        const uint32_t x = ld8(blk), b = ld8(blk + 1 + (i & 15));
+        const float d = __builtin_bit_cast(float, x < 2u ? 0x00200000u << x : (x - 1u) << 23);
+        return (float)kv[i < 16 ? (b & 0xF) : (b >> 4)] * d;
+    }
+    case 40: {  // NVFP4: table[nibble] * ue4m3(d[sub-block]) (dequant.rs:1050-1072, 423-435)
+        const int kv[16] = {0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12};
+        const uint8_t* blk = rowp + (size_t)(e >> 6) * 36;
+        const int i = e & 63, sb = i >> 4, j = i & 7;
+        const uint32_t x = ld8(blk + sb), b = ld8(blk + 4 + 8 * sb + j);
+        const uint32_t exp = (x >> 3) & 15u, man = x & 7u;
+        float d = exp ? __builtin_bit_cast(float, ((exp + 119u) << 23) | (man << 20)) : (float)man * 0.0009765625f;
+        if (x == 0u || x == 0x7Fu) d = 0.0f;
+        return (float)kv[(i & 8) ? (b >> 4) : (b & 0xF)] * d;
+    }
     case 14: {  // Q6_K
         const uint8_t* blk = rowp + (size_t)(e >> 8) * 210;
         const int i = e & 255, half = i >> 7, r = i & 127, col = r >> 5, l = r & 31;

@@ -1,4 +1,4 @@
-// Instantiates the decode GEMV templates for: FmtQ2K, FmtQ3K, FmtIQ4XS.
+// Instantiates the decode GEMV templates for: FmtQ2K, FmtQ3K, FmtIQ4XS, FmtMXFP4, FmtNVFP4.
 #include "gemv_impl.hpp"
 
 namespace infr {
@@ -13,6 +13,14 @@ const GemvFormatOps& gemv_ops_q3k() {
 }
 const GemvFormatOps& gemv_ops_iq4xs() {
     static const GemvFormatOps ops = make_gemv_format_ops<FmtIQ4XS>();
+    return ops;
+}
+const GemvFormatOps& gemv_ops_mxfp4() {
+    static const GemvFormatOps ops = make_gemv_format_ops<FmtMXFP4>();
+    return ops;
+}
+const GemvFormatOps& gemv_ops_nvfp4() {
+    static const GemvFormatOps ops = make_gemv_format_ops<FmtNVFP4>();
     return ops;
 }
 

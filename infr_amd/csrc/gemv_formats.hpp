@@ -976,6 +976,158 @@ using FmtQ5_0 = FmtNib32<Nib32::Q5_0>;
 using FmtQ5_1 = FmtNib32<Nib32::Q5_1>;
 using FmtIQ4NL = FmtNib32<Nib32::IQ4_NL>;
 
+// ───────────────────────────── MXFP4 / NVFP4: E2M1 codes ─────────────────────────────
+// KVALUES_MXFP4 (crates/infr-gguf/src/dequant.rs:405): 0 1 2 3 4 6 8 12 and their negatives - the
+// E2M1 values doubled - looked up like IQ4_NL's table.
+__device__ __forceinline__ int mxfp4_lookup(uint32_t nib) {
+    const uint32_t sel = nib & 0x07070707u;
+    const uint32_t lo = __builtin_amdgcn_perm(0x0C080604u, 0x03020100u, sel);  // entries 0..7
+    const uint32_t hi = __builtin_amdgcn_perm(0xF4F8FAFCu, 0xFDFEFF00u, sel);  // entries 8..15
+    const uint32_t pick = ((nib >> 3) & 0x01010101u) * 0xFFu;                  // 0xFF where nibble >= 8
+    return (int)((hi & pick) | (lo & ~pick));
+}
+// e8m0_to_fp32_half (dequant.rs:411-417): 2^(x - 128), the two lowest codes subnormal.
+__device__ __forceinline__ float e8m0_half(uint32_t x) {
+    return __builtin_bit_cast(float, x < 2u ? 0x00200000u << x : (x - 1u) << 23);
+}
+// ue4m3_to_fp32 (dequant.rs:423-435): 4 exponent bits (bias 7), 3 mantissa bits, halved; 0 and 0x7F
+// are 0. (8 + man) * 2^(exp - 11) for exp > 0, man * 2^-10 below: both exact.
+__device__ __forceinline__ float ue4m3_half(uint32_t x) {
+    const uint32_t exp = (x >> 3) & 15u, man = x & 7u;
+    const float v = exp ? __builtin_bit_cast(float, ((exp + 119u) << 23) | (man << 20)) : (float)man * 0.0009765625f;
+    return (x == 0u || x == 0x7Fu) ? 0.0f : v;
+}
+
+// MXFP4 (17-byte block [u8 e][u8 qs[16]], any byte alignment; crates/infr-cpu/src/kernels.rs:6303-6327):
+// a lane owns block t * 64 + l against the per-32 activation, sumf += d * q8.d[b] * iprod. The 16
+// code bytes are fetched as the five aligned dwords that cover them and shifted into place; when
+// the codes happen to start on a dword the fifth load repeats the fourth (nothing beyond the
+// block's last byte's dword is ever read).
+struct FmtMXFP4 {
+    static constexpr int kElemsPerStep = 2048;
+    static constexpr bool kPer32 = true;
+    static constexpr bool kOrdered = false;
+    static constexpr int kBlockBytes = 17, kBlockElems = 32;
+    static constexpr int kWide16Steps = 4;
+    static constexpr bool kClampedLoads = false;
+    static constexpr bool kLaneSums = true;
+    static constexpr bool kRowAhead = false;
+    struct Row {
+        v4i qs;
+        uint32_t e;
+    };
+    typedef FmtNib32<Nib32::IQ4_NL>::Acts Acts;
+    __device__ static int units(int in_f) { return in_f / 32; }
+    __device__ static bool valid(int t, int lane, int n) { return t * 64 + lane < n; }
+    __device__ static void load_row(Row& r, const uint8_t* rowp, int t, int lane, bool ok) {
+        if (!ok) {
+            r.qs = v4i{0, 0, 0, 0};
+            r.e = 0;
+            return;
+        }
+        const uint8_t* blk = rowp + (size_t)(t * 64 + lane) * 17;
+        r.e = gload<uint8_t>(blk);
+        const uint32_t sh = (uint32_t)(reinterpret_cast<uintptr_t>(blk + 1) & 3);
+        const uint8_t* a = blk + 1 - sh;
+        const v4i lo = load16_a4(a);
+        const uint32_t w4 = (uint32_t)load_u32(a + (sh ? 16 : 12));
+        r.qs = v4i{(int)__builtin_amdgcn_alignbyte((uint32_t)lo.y, (uint32_t)lo.x, sh),
+                   (int)__builtin_amdgcn_alignbyte((uint32_t)lo.z, (uint32_t)lo.y, sh),
+                   (int)__builtin_amdgcn_alignbyte((uint32_t)lo.w, (uint32_t)lo.z, sh),
+                   (int)__builtin_amdgcn_alignbyte(w4, (uint32_t)lo.w, sh)};
+    }
+    __device__ static void load_acts(Acts& a, const ActPtrs& s, int t, int lane, bool ok) {
+        FmtNib32<Nib32::IQ4_NL>::load_acts(a, s, t, lane, ok);
+    }
+    template <bool STAGES>
+    __device__ static float term(const Row& r, const Acts& a, int t, int lane, bool ok,
+                                 const StagePtrs& st, size_t row_units) {
+        const uint32_t m4 = 0x0F0F0F0Fu;
+        const int qw[4] = {r.qs.x, r.qs.y, r.qs.z, r.qs.w};
+        int ip = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            ip = dot4(mxfp4_lookup((uint32_t)qw[k] & m4), a.xa[k], ip);
+            ip = dot4(mxfp4_lookup(((uint32_t)qw[k] >> 4) & m4), a.xa[4 + k], ip);
+        }
+        if (STAGES && ok) st.a[row_units + t * 64 + lane] = ip;
+        return e8m0_half(r.e) * a.dact * (float)ip;  // d * q8.d[b] * iprod as f32
+    }
+};
+
+// NVFP4 (36-byte block [u8 d[4]][u8 qs[32]], 64 weights; crates/infr-cpu/src/kernels.rs:6472-6500):
+// sub-block s (16 weights, UE4M3 scale d[s]) reads qs[8 s .. 8 s + 7] - low nibbles elements 0..7,
+// high nibbles 8..15 - and meets half of activation block 2 b + s / 2:
+// sumf += d_s * q8.d[2 b + s / 2] * iprod_s. A lane owns block t * 64 + l (two activation blocks).
+struct FmtNVFP4 {
+    static constexpr int kElemsPerStep = 4096;
+    static constexpr bool kPer32 = true;
+    static constexpr bool kOrdered = false;
+    static constexpr int kBlockBytes = 36, kBlockElems = 64;
+    static constexpr int kWide16Steps = 3;
+    static constexpr bool kClampedLoads = false;
+    static constexpr bool kLaneSums = true;
+    static constexpr bool kRowAhead = false;
+    struct Row {
+        v4i qa, qb;
+        uint32_t d4;
+    };
+    struct Acts {
+        int xa[16];
+        float dact0, dact1;
+    };
+    __device__ static int units(int in_f) { return in_f / 64; }
+    __device__ static bool valid(int t, int lane, int n) { return t * 64 + lane < n; }
+    __device__ static void load_row(Row& r, const uint8_t* rowp, int t, int lane, bool ok) {
+        if (ok) {
+            const uint8_t* blk = rowp + (size_t)(t * 64 + lane) * 36;
+            r.d4 = (uint32_t)load_u32(blk);
+            r.qa = load16_a4(blk + 4);
+            r.qb = load16_a4(blk + 20);
+        } else {
+            r.qa = r.qb = v4i{0, 0, 0, 0};
+            r.d4 = 0;
+        }
+    }
+    __device__ static void load_acts(Acts& a, const ActPtrs& s, int t, int lane, bool ok) {
+        if (ok) {
+            const int b = t * 64 + lane;
+            const v4i* xp = reinterpret_cast<const v4i*>(s.qs + (size_t)b * 64);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const v4i v = xp[k];
+                a.xa[4 * k + 0] = v.x;
+                a.xa[4 * k + 1] = v.y;
+                a.xa[4 * k + 2] = v.z;
+                a.xa[4 * k + 3] = v.w;
+            }
+            a.dact0 = s.d[2 * b];
+            a.dact1 = s.d[2 * b + 1];
+        } else {
+#pragma unroll
+            for (int k = 0; k < 16; ++k) a.xa[k] = 0;
+            a.dact0 = a.dact1 = 0.0f;
+        }
+    }
+    // (no stage outputs: a block has four integers, one per sub-block)
+    template <bool STAGES>
+    __device__ static float term(const Row& r, const Acts& a, int, int, bool, const StagePtrs&, size_t) {
+        const uint32_t m4 = 0x0F0F0F0Fu;
+        const int qw[8] = {r.qa.x, r.qa.y, r.qa.z, r.qa.w, r.qb.x, r.qb.y, r.qb.z, r.qb.w};
+        float sum = 0.0f;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const uint32_t w0 = (uint32_t)qw[2 * s], w1 = (uint32_t)qw[2 * s + 1];
+            int ip = dot4(mxfp4_lookup(w0 & m4), a.xa[4 * s], 0);
+            ip = dot4(mxfp4_lookup(w1 & m4), a.xa[4 * s + 1], ip);
+            ip = dot4(mxfp4_lookup((w0 >> 4) & m4), a.xa[4 * s + 2], ip);
+            ip = dot4(mxfp4_lookup((w1 >> 4) & m4), a.xa[4 * s + 3], ip);
+            sum += ue4m3_half((r.d4 >> (8 * s)) & 0xFFu) * (s < 2 ? a.dact0 : a.dact1) * (float)ip;
+        }
+        return sum;
+    }
+};
+
 // Pair form of the formats whose block stride is 2 mod 4 (Q4_0 / IQ4_NL 18 B, Q5_0 22 B), for rows
 // of whole 64s: two consecutive blocks are 36 / 44 bytes, a whole number of dwords, and every row
 // starts on a dword. Lane l owns the pair t*64 + l (64 weights): three dword-aligned loads fetch it

@@ -181,7 +181,7 @@ bool mmq_skinny16_takes(int dtype, size_t m, size_t in_f, size_t out_f);
 // formats and Q2_0, and for Q8_0 rows that are not whole 256s; per-256 `Q8` otherwise.
 inline bool act_is_per32(int dtype, size_t in_f) {
     switch (dtype) {
-    case 2: case 3: case 6: case 7: case 20: case 42: return true;
+    case 2: case 3: case 6: case 7: case 20: case 42: case 39: case 40: return true;
     case 8: return in_f % 256 != 0;
     default: return false;
     }
@@ -227,6 +227,8 @@ const GemvFormatOps& gemv_ops_q5k();
 const GemvFormatOps& gemv_ops_q2k();
 const GemvFormatOps& gemv_ops_q3k();
 const GemvFormatOps& gemv_ops_iq4xs();
+const GemvFormatOps& gemv_ops_mxfp4();
+const GemvFormatOps& gemv_ops_nvfp4();
 const GemvFormatOps& gemv_ops_q4_0();
 const GemvFormatOps& gemv_ops_q4_1();
 const GemvFormatOps& gemv_ops_q5_0();  // batch launchers only: one token takes the f32 kernel

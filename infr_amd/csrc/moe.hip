@@ -1486,6 +1486,8 @@ const char* launch_moe_ffn(const MoeShape& shape, const MoeBuffers& bufs, void* 
         case 10: return in_f / 256 * 84;
         case 11: return in_f / 256 * 110;
         case 23: return in_f / 256 * 136;
+        case 39: return in_f / 32 * 17;
+        case 40: return in_f / 64 * 36;
         case 14: return in_f / 256 * 210;
         case 8: return in_f / 32 * 34;
         case 2: case 20: return in_f / 32 * 18;

@@ -363,6 +363,51 @@ void encode_iq4xs(const float* x, uint8_t* blk) {
     blk[3] = (uint8_t)(scales_h >> 8);
 }
 
+// The E2M1 values, doubled (crates/infr-gguf/src/dequant.rs:405).
+const int kFp4[16] = {0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12};
+int nearest_fp4(float v) {
+    int best = 0;
+    for (int c = 1; c < 16; ++c)
+        if (c != 8 && std::fabs(v - (float)kFp4[c]) < std::fabs(v - (float)kFp4[best])) best = c;
+    return best;
+}
+// 32 floats -> one 17-byte MXFP4 block [u8 e][u8 qs[16]]: the smallest power of two d = 2^(e - 128)
+// with 12 d >= max |x|, codes the nearest table values of x / d.
+void encode_mxfp4(const float* x, uint8_t* blk) {
+    float amax = 0.0f;
+    for (int i = 0; i < 32; ++i) amax = std::max(amax, std::fabs(x[i]));
+    int e = amax > 0.0f ? (int)std::ceil(std::log2(amax / 12.0f)) + 128 : 2;
+    e = clampi(e, 2, 254);
+    const float d = std::ldexp(1.0f, e - 128);
+    blk[0] = (uint8_t)e;
+    for (int j = 0; j < 16; ++j)
+        blk[1 + j] = (uint8_t)(nearest_fp4(x[j] / d) | (nearest_fp4(x[j + 16] / d) << 4));
+}
+// 64 floats -> one 36-byte NVFP4 block [u8 d[4]][u8 qs[32]]: per 16-weight sub-block the UE4M3 code
+// (exponent bias 7, three mantissa bits, decoded halved) whose value is the smallest one with
+// 12 d >= max |x|; codes the nearest table values of x / d, low nibbles elements 0..7, high 8..15.
+void encode_nvfp4(const float* x, uint8_t* blk) {
+    for (int s = 0; s < 4; ++s) {
+        float amax = 0.0f;
+        for (int i = 0; i < 16; ++i) amax = std::max(amax, std::fabs(x[16 * s + i]));
+        int code = 0x7E;
+        float d = 0.0f;
+        for (int c = 1; c <= 0x7E; ++c) {  // values ascend with the code
+            const int ex = c >> 3, man = c & 7;
+            const float v = 0.5f * (ex == 0 ? (float)man / 8.0f * std::ldexp(1.0f, -6) : (1.0f + (float)man / 8.0f) * std::ldexp(1.0f, ex - 7));
+            if (12.0f * v >= amax) {
+                code = c;
+                d = v;
+                break;
+            }
+            d = v;
+        }
+        blk[s] = (uint8_t)code;
+        for (int j = 0; j < 8; ++j)
+            blk[4 + 8 * s + j] = (uint8_t)(nearest_fp4(x[16 * s + j] / d) | (nearest_fp4(x[16 * s + 8 + j] / d) << 4));
+    }
+}
+
 // 32 floats -> one block of a 32-weight format. Element j's code goes to the low nibble of qs[j],
 // element j+16's to the high nibble; the 5-bit formats put the 5th bit of element e in bit e of qh.
 //   Q4_0 [d][qs]: symmetric, code = round(x/d) + 8        Q5_0 [d][qh][qs]: ... + 16
@@ -453,6 +498,8 @@ int infr_block_layout(int dtype, int* elems, int* bytes) {
     case INFR_DTYPE_Q2_K: e = 256; b = 84; break;
     case INFR_DTYPE_Q3_K: e = 256; b = 110; break;
     case INFR_DTYPE_IQ4_XS: e = 256; b = 136; break;
+    case INFR_DTYPE_MXFP4: e = 32; b = 17; break;
+    case INFR_DTYPE_NVFP4: e = 64; b = 36; break;
     case INFR_DTYPE_IQ4_NL: e = 32; b = 18; break;
     default: return 0;
     }
@@ -503,6 +550,8 @@ size_t infr_synth_weight(int dtype, uint64_t seed, float sigma, size_t rows, siz
             else if (dtype == INFR_DTYPE_Q2_K) encode_q2k(x.data(), blk);
             else if (dtype == INFR_DTYPE_Q3_K) encode_q3k(x.data(), blk);
             else if (dtype == INFR_DTYPE_IQ4_XS) encode_iq4xs(x.data(), blk);
+            else if (dtype == INFR_DTYPE_MXFP4) encode_mxfp4(x.data(), blk);
+            else if (dtype == INFR_DTYPE_NVFP4) encode_nvfp4(x.data(), blk);
             else if (dtype == INFR_DTYPE_Q8_0) encode_q8_0(x.data(), blk);
             else encode_blk32(dtype, x.data(), blk);
         }

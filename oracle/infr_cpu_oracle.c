@@ -33,6 +33,8 @@ int orc_block_layout(int dtype, int *elems, int *bytes) {
     case ORC_Q2_K: e = 256; b = 84; break;
     case ORC_Q3_K: e = 256; b = 110; break;
     case ORC_IQ4_XS: e = 256; b = 136; break;
+    case ORC_MXFP4: e = 32; b = 17; break;
+    case ORC_NVFP4: e = 64; b = 36; break;
     case ORC_Q4_K: e = 256; b = 144; break;
     case ORC_Q6_K: e = 256; b = 210; break;
     case ORC_Q2_0: e = 64; b = 18; break;
@@ -123,6 +125,28 @@ void orc_k4(int j, const uint8_t *q, uint32_t *sc, uint32_t *m) {
 /* ───────────────────────────── host decode ───────────────────────────── */
 
 /* crates/infr-gguf/src/dequant.rs:439-441 */
+/* crates/infr-gguf/src/dequant.rs:405 (KVALUES_MXFP4: the E2M1 values, doubled). */
+const int8_t orc_kvalues_mxfp4[16] = {0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12};
+
+/* crates/infr-gguf/src/dequant.rs:411-417 (e8m0_to_fp32_half): 2^(x - 128); the two lowest codes
+ * are f32 subnormals. */
+float orc_e8m0_half(uint8_t x) {
+    uint32_t bits = x < 2 ? (0x00200000u << x) : (((uint32_t)x - 1u) << 23);
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+
+/* crates/infr-gguf/src/dequant.rs:423-435 (ue4m3_to_fp32): unsigned, 4 exponent bits (bias 7), 3
+ * mantissa bits, halved; 0 and 0x7F decode to 0. */
+float orc_ue4m3_half(uint8_t x) {
+    if (x == 0 || x == 0x7F) return 0.0f;
+    int exp = (x >> 3) & 0xF;
+    float man = (float)(x & 0x7);
+    float raw = exp == 0 ? man * ldexpf(1.0f, -9) : (1.0f + man / 8.0f) * ldexpf(1.0f, exp - 7);
+    return raw * 0.5f;
+}
+
 const int8_t orc_kvalues_iq4nl[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
 
 /* crates/infr-gguf/src/dequant.rs:11-51: for affine quants the factored form is expanded as
@@ -334,6 +358,31 @@ int orc_dequant_block(int dtype, const uint8_t *bytes, size_t nbytes, float *out
                 for (int j = 0; j < 16; j++) {
                     out[b * 256 + ib * 32 + j] = dl * (float)orc_kvalues_iq4nl[qs[j] & 0xF];
                     out[b * 256 + ib * 32 + j + 16] = dl * (float)orc_kvalues_iq4nl[qs[j] >> 4];
+                }
+            }
+        }
+        return 0;
+    case ORC_MXFP4:
+        /* dequant.rs:1024-1042: [u8 e][u8 qs[16]]; y[j] = table[low nibble] * d, y[j + 16] = table[high] * d. */
+        for (size_t b = 0; b < nblk; b++) {
+            const uint8_t *blk = bytes + b * 17;
+            float d = orc_e8m0_half(blk[0]);
+            for (int j = 0; j < 16; j++) {
+                out[b * 32 + j] = (float)orc_kvalues_mxfp4[blk[1 + j] & 0xF] * d;
+                out[b * 32 + j + 16] = (float)orc_kvalues_mxfp4[blk[1 + j] >> 4] * d;
+            }
+        }
+        return 0;
+    case ORC_NVFP4:
+        /* dequant.rs:1050-1072: [u8 d[4]][u8 qs[32]]; sub-block s (16 elements) reads qs[8s .. 8s + 7]:
+         * low nibbles elements 0..7, high nibbles 8..15, each times the sub-block's UE4M3 scale. */
+        for (size_t b = 0; b < nblk; b++) {
+            const uint8_t *blk = bytes + b * 36;
+            for (int sb = 0; sb < 4; sb++) {
+                float d = orc_ue4m3_half(blk[sb]);
+                for (int j = 0; j < 8; j++) {
+                    out[b * 64 + sb * 16 + j] = (float)orc_kvalues_mxfp4[blk[4 + sb * 8 + j] & 0xF] * d;
+                    out[b * 64 + sb * 16 + j + 8] = (float)orc_kvalues_mxfp4[blk[4 + sb * 8 + j] >> 4] * d;
                 }
             }
         }
@@ -707,6 +756,47 @@ float orc_vec_dot_iq4xs(const uint8_t *row, const int8_t *qs8, const float *d8, 
     return sumf;
 }
 
+/* crates/infr-cpu/src/kernels.rs:6303-6327 (vec_dot_mxfp4_32_batch_scalar), one activation row:
+ * per 32-block the table dot with the per-32 activation codes, sumf += d * q8.d[b] * iprod. */
+float orc_vec_dot_mxfp4(const uint8_t *row, const int8_t *qs8, const float *d8, size_t in_f, int32_t *iprod_out) {
+    size_t nb = in_f / 32;
+    float sumf = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * 17;
+        const int8_t *a = qs8 + b * 32;
+        int32_t iprod = 0;
+        for (int j = 0; j < 16; j++)
+            iprod += (int32_t)orc_kvalues_mxfp4[blk[1 + j] & 0xF] * (int32_t)a[j] +
+                     (int32_t)orc_kvalues_mxfp4[blk[1 + j] >> 4] * (int32_t)a[j + 16];
+        if (iprod_out) iprod_out[b] = iprod;
+        sumf += orc_e8m0_half(blk[0]) * d8[b] * (float)iprod;
+    }
+    return sumf;
+}
+
+/* crates/infr-cpu/src/kernels.rs:6472-6500 (vec_dot_nvfp4_batch_scalar), one activation row: the
+ * 64-weight block meets activation blocks 2b and 2b + 1; per 16-element sub-block s,
+ * sumf += d_s * q8.d[2b + s/2] * iprod_s. iprod_out holds in_f / 16 integers. */
+float orc_vec_dot_nvfp4(const uint8_t *row, const int8_t *qs8, const float *d8, size_t in_f, int32_t *iprod_out) {
+    size_t nb = in_f / 64;
+    float sumf = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * 36;
+        for (int sb = 0; sb < 4; sb++) {
+            size_t t = 2 * b + (size_t)sb / 2;
+            const int8_t *a = qs8 + t * 32 + (sb % 2) * 16;
+            const uint8_t *code = blk + 4 + sb * 8;
+            int32_t iprod = 0;
+            for (int j = 0; j < 8; j++)
+                iprod += (int32_t)orc_kvalues_mxfp4[code[j] & 0xF] * (int32_t)a[j] +
+                         (int32_t)orc_kvalues_mxfp4[code[j] >> 4] * (int32_t)a[j + 8];
+            if (iprod_out) iprod_out[b * 4 + sb] = iprod;
+            sumf += orc_ue4m3_half(blk[sb]) * d8[t] * (float)iprod;
+        }
+    }
+    return sumf;
+}
+
 /* The 32-weight-block formats against the per-32 activation, one activation row of the batch
  * scalars: Q4_0 kernels.rs:5496-5520, Q4_1 :5793-5822, Q5_0 :5350-5377, Q5_1 :5948-5980,
  * IQ4_NL :6128-6152. Element j of a block takes the low nibble of qs[j], element j+16 the high
@@ -959,6 +1049,8 @@ static float row_dot(int dtype, const uint8_t *row, const acts_t *a, size_t r, s
         size_t nb = in_f / 32;
         return orc_vec_dot_blk32(dtype, row, a->qs + r * in_f, a->d + r * nb, a->bsums + r * nb, in_f, ia);
     }
+    case ORC_MXFP4: return orc_vec_dot_mxfp4(row, a->qs + r * in_f, a->d + r * (in_f / 32), in_f, ia);
+    case ORC_NVFP4: return orc_vec_dot_nvfp4(row, a->qs + r * in_f, a->d + r * (in_f / 32), in_f, ia);
     default:
         return 0.0f;
     }
@@ -981,7 +1073,9 @@ static int linear_shape_ok(int dtype, size_t in_f) {
     case ORC_Q5_0:
     case ORC_Q5_1:
     case ORC_IQ4_NL:
+    case ORC_MXFP4:
     case ORC_Q8_0: return in_f % 32 == 0;
+    case ORC_NVFP4:
     case ORC_Q2_0: return in_f % 64 == 0;
     case ORC_F32:
     case ORC_F16:
@@ -1071,7 +1165,7 @@ int orc_linear_int_stages(int dtype, const uint8_t *w, size_t wbytes, size_t w_n
     size_t row0 = w_off / in_f;
     if (row0 + out_f > total_rows) return -2;
     const uint8_t *wb = w + row0 * bpr;
-    size_t blocks = (dtype == ORC_Q4_K || dtype == ORC_Q5_K || dtype == ORC_Q6_K || dtype == ORC_Q2_K || dtype == ORC_Q3_K || dtype == ORC_IQ4_XS) ? in_f / 256 : in_f / 32;
+    size_t blocks = (dtype == ORC_Q4_K || dtype == ORC_Q5_K || dtype == ORC_Q6_K || dtype == ORC_Q2_K || dtype == ORC_Q3_K || dtype == ORC_IQ4_XS) ? in_f / 256 : (dtype == ORC_NVFP4 ? in_f / 16 : in_f / 32);
     acts_t a;
     acts_build(dtype, x, m, in_f, &a);
 #pragma omp parallel for schedule(dynamic, 8)
@@ -1425,6 +1519,10 @@ size_t orc_synth_weight(int dtype, size_t n_elem, uint32_t seed, uint8_t *out) {
             break;
         case ORC_Q3_K: put_f16(blk + 108, 0.03f); break; /* d@108 (decode_spec.rs:325) */
         case ORC_IQ4_XS: put_f16(blk, 0.06f); break;      /* d@0 (decode_spec.rs:351) */
+        case ORC_MXFP4: blk[0] = 125; break;              /* E8M0 nearest 0.25 in log space: 2^(125 - 127) (decode_spec.rs:191, 216-219) */
+        case ORC_NVFP4:                                   /* UE4M3 nearest 0.5 * (0.625 + 0.125 i) (decode_spec.rs:192-198, 223-245) */
+            blk[0] = 42, blk[1] = 44, blk[2] = 46, blk[3] = 48;
+            break;
         case ORC_Q4_0:
         case ORC_Q5_0: put_f16(blk, 0.04f); break;
         case ORC_Q4_1:

@@ -66,6 +66,8 @@ enum {
     ORC_Q2_K = 10,
     ORC_Q3_K = 11,
     ORC_IQ4_XS = 23,
+    ORC_MXFP4 = 39,
+    ORC_NVFP4 = 40,
     ORC_Q4_K = 12,
     ORC_Q5_K = 13,
     ORC_Q6_K = 14,
@@ -130,6 +132,12 @@ float orc_vec_dot_q3k(const uint8_t *row, const int8_t *qs, const float *d, cons
 /* IQ4_XS: kernels.rs:1008-1036 (vec_dot_iq4xs_scalar), scale by kernels.rs:995-1002 - isum[nb]. */
 float orc_vec_dot_iq4xs(const uint8_t *row, const int8_t *qs, const float *d, size_t in_f, int32_t *isum_out);
 int orc_iq4xs_scale(uint32_t scales_h, const uint8_t *scales_l, int ib);
+/* MXFP4: kernels.rs:6303-6327 - iprod[in_f/32]; NVFP4: kernels.rs:6472-6500 - iprod[in_f/16]. Both
+ * against the per-32 activation; scale decoders dequant.rs:411-435. */
+float orc_vec_dot_mxfp4(const uint8_t *row, const int8_t *qs, const float *d, size_t in_f, int32_t *iprod_out);
+float orc_vec_dot_nvfp4(const uint8_t *row, const int8_t *qs, const float *d, size_t in_f, int32_t *iprod_out);
+float orc_e8m0_half(uint8_t x);
+float orc_ue4m3_half(uint8_t x);
 /* Q3_K's sixteen signed scales (sc6 - 32) of one block from its 12 scale bytes (kernels.rs:764-783). */
 void orc_q3k_scales(const uint8_t *scales_raw, int16_t out[16]);
 /* Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL against the per-32 activation: kernels.rs:5496-5520,

@@ -63,7 +63,7 @@ static void hip_linear_all_weight_quants_match_the_host_oracle(HipBackend& be) {
         const auto cases = weight_quant_cases(m, 256, 8);
         const SweepReport r = sweep_linear_on("hip Linear m=" + std::to_string(m), be, cases,
                                               [](const LinearCase&) { return CPU_INT8_ACT_TOL; });
-        EXPECT(r.cases.size() == 13, "expected the thirteen formats of this backend, got %zu", r.cases.size());
+        EXPECT(r.cases.size() == 15, "expected the fifteen formats of this backend, got %zu", r.cases.size());
         EXPECT(r.failures() == 0, "cases outside %.0e of the host decode oracle", CPU_INT8_ACT_TOL);
     }
 }
@@ -362,13 +362,13 @@ static void hip_backend_honours_the_seam_contract(HipBackend& be) {
     EXPECT(threw, "execute with an unbound weight did not report Invalid");
     // a format outside this backend is Unsupported at compile, never a wrong answer
     Graph g2;
-    const TensorId w2 = g2.weight({{8, 256}, (DType)39 /* MXFP4 */});
+    const TensorId w2 = g2.weight({{8, 256}, (DType)16 /* IQ2_XXS */});
     const TensorId x2 = g2.input({{1, 256}, DType::F32});
     const TensorId d2 = g2.output({{1, 8}, DType::F32});
     g2.push(op::Linear{x2, w2, d2, 1, 256, 8, 0});
     threw = false;
     try { Plan p2 = be.compile(g2); } catch (const Error& e) { threw = e.kind == ErrorKind::Unsupported; }
-    EXPECT(threw, "MXFP4 Linear did not report Unsupported");
+    EXPECT(threw, "IQ2_XXS Linear did not report Unsupported");
     // a ragged row is refused, not truncated
     Graph g3;
     const TensorId w3 = g3.weight({{8, 128}, DType::Q4K});

@@ -78,7 +78,8 @@ def test_synth_is_deterministic_and_thread_count_independent():
 
 
 @pytest.mark.parametrize("dtype,tol", [(B.DType.Q4K, 0.09), (B.DType.Q6K, 0.03), (B.DType.Q8_0, 0.01),
-                                       (B.DType.Q2K, 0.06), (B.DType.Q3K, 0.02), (B.DType.IQ4XS, 0.03)])
+                                       (B.DType.Q2K, 0.06), (B.DType.Q3K, 0.02), (B.DType.IQ4XS, 0.03),
+                                       (B.DType.MXFP4, 0.08), (B.DType.NVFP4, 0.06)])
 def test_synth_encoders_reproduce_their_input_distribution(dtype, tol):
     """The encoders are nearest-code quantizers of N(0, 0.02^2): decoding (with the CPU oracle's
     host decode) must give that distribution back within the format's step size."""
