@@ -53,6 +53,7 @@ typedef enum {
     INFR_DTYPE_Q6_K = 14, /* 256 / 210 B: [u8 ql[128]][u8 qh[64]][i8 sc[16]][f16 d]       :330-331 */
     INFR_DTYPE_IQ4_NL = 20, /* 32 / 18 B: [f16 d][u8 qs[16]]  w = d*codebook[q]           :349-350 */
     INFR_DTYPE_IQ4_XS = 23, /* 256 / 136 B: [f16 d][u16 scales_h][u8 scales_l[4]][u8 qs[128]] :351 */
+    INFR_DTYPE_TQ2_0 = 35,  /* 256 / 66 B: [u8 qs[64]][f16 d]  w = d*(q-1), 2-bit ternary codes         :356 */
     INFR_DTYPE_MXFP4 = 39,  /* 32 / 17 B: [u8 e][u8 qs[16]]  w = table[q] * 2^(e-128)             :361 */
     INFR_DTYPE_NVFP4 = 40,  /* 64 / 36 B: [u8 d[4]][u8 qs[32]]  w = table[q] * ue4m3(d[i/16]) / 2     :363 */
     INFR_DTYPE_BF16 = 30, /* plain rows, as F16 */

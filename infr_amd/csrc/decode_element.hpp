@@ -92,6 +92,12 @@ __device__ inline float decode_element(int dtype, const uint8_t* rowp, int e) {
         const int kv[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
         return (ldf16(blk) * (float)ls) * (float)kv[nib];
     }
+    case 35: {  // TQ2_0: (q - 1) * d (dequant.rs:968-996)
+        const uint8_t* blk = rowp + (size_t)(e >> 8) * 66;
+        const int i = e & 255;
+        const int q = (int)((ld8(blk + 32 * (i >> 7) + (i & 31)) >> (2 * ((i >> 5) & 3))) & 3u);
+        return (float)(q - 1) * ldf16(blk + 64);
+    }
     case 39: {  // MXFP4: table[nibble] * 2^(e - 128) (dequant.rs:1024-1042)
         const int kv[16] = {0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12};
         const uint8_t* blk = rowp + (size_t)(e >> 5) * 17;

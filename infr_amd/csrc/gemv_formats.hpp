@@ -681,6 +681,61 @@ struct FmtQ2K {
     }
 };
 
+// TQ2_0 (66-byte block, 2-byte aligned: [u8 qs[64]][f16 d]): the bit pairs are laid out as Q2_K's, a
+// code q is the ternary weight q - 1 with one scale per superblock: iprod = sum (q - 1) * q8 =
+// sum q * q8 - (the activation's code sum), term d * q8.d[b] * iprod
+// (crates/infr-cpu/src/kernels.rs:3066-3126), blocks in ascending order. Lanes as for Q2_K.
+struct FmtTQ2_0 {
+    static constexpr int kElemsPerStep = 4096;
+    static constexpr bool kPer32 = false;
+    static constexpr bool kOrdered = true;
+    static constexpr int kBlockBytes = 66, kBlockElems = 256;
+    static constexpr int kWide16Steps = 3;
+    static constexpr bool kClampedLoads = false;
+    static constexpr bool kLaneSums = true;
+    static constexpr bool kRowAhead = false;
+    struct Row {
+        v4i q;
+        uint32_t d;
+    };
+    typedef FmtQ6K::Acts Acts;
+    __device__ static int units(int in_f) { return in_f / 256; }
+    __device__ static bool valid(int t, int lane, int n) { return t * 16 + (lane >> 2) < n; }
+    __device__ static void load_row(Row& r, const uint8_t* rowp, int t, int lane, bool ok) {
+        if (ok) {
+            const uint8_t* blk = rowp + (size_t)(t * 16 + (lane >> 2)) * 66;
+            r.q = load16_a2(blk + 16 * (lane & 3));
+            r.d = load_u16(blk + 64);
+        } else {
+            r.q = v4i{0, 0, 0, 0};
+            r.d = 0;
+        }
+    }
+    __device__ static void load_acts(Acts& a, const ActPtrs& s, int t, int lane, bool ok) {
+        FmtQ6K::load_acts(a, s, t, lane, ok);
+    }
+    template <bool STAGES>
+    __device__ static float term(const Row& r, const Acts& a, int t, int lane, bool ok,
+                                 const StagePtrs& st, size_t row_units) {
+        const int qw[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
+        int part = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            int ip = 0;  // (bit pairs 1 and 2 multiplied where they sit, as for Q2_K)
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t c = j == 3 ? ((uint32_t)qw[k] >> 6) & 0x03030303u : (uint32_t)qw[k] & (0x03030303u << (2 * j));
+                ip = dot4((int)c, a.xa[4 * j + k], ip);
+            }
+            if (j == 1 || j == 2) ip >>= 2 * j;
+            part += ip - a.bs16[j];
+        }
+        const int iprod = quad_sum(part);
+        if (STAGES && ok && (lane & 3) == 0) st.a[row_units + t * 16 + (lane >> 2)] = iprod;
+        return f16_bits_to_f32(r.d) * a.dact * (float)iprod;  // sumf += d * q8.d[b] * iprod as f32
+    }
+};
+
 // Q3_K (110-byte block, 2-byte aligned: [u8 hmask[32]][u8 qs[64]][u8 scales[12]][f16 d]): a code is
 // the 2-bit field plus bit 4 n + j of hmask[16 half + l] as its third bit; sixteen 6-bit scales are
 // packed as low nibbles, high nibbles and a word of top bit pairs (q3k_scales, kernels.rs:764-783),

@@ -952,6 +952,45 @@ struct Skinny16Q3K {
     }
 };
 
+// TQ2_0 (66-byte block: qs[64], d; crates/infr-cpu/src/kernels.rs:3066-3126): the ternary weights
+// q - 1 are the operand as they are - lanes and bit pairs as for Q2_K, four K = 64 steps chain into
+// the block's iprod - and y += (d * q8.d[b]) * iprod. A stage of two blocks is 132 bytes: the second
+// sits 2 bytes off a word boundary in LDS (read as aligned words and shifted); rows are an even
+// number of blocks.
+struct Skinny16TQ2_0 {
+    static constexpr bool kPer32Acts = false, kTranspose16 = false;
+    static constexpr bool kSubScales = false;
+    static constexpr int kBlockBytes = 66;
+    static constexpr int kRowStride = 144;  // 132 rounded up: 36 words, eight rows' 16-byte reads cover all banks
+    __device__ static float accumulate(float acc, float dq, uint32_t ddm, int sd, float) {
+        return acc + (f16_bits_to_f32(ddm) * dq) * (float)sd;
+    }
+    __device__ static void block(const uint8_t* wrow, int jj, const uint8_t* arow, const uint8_t*, const uint8_t*,
+                                 int kq, int (&sd)[4], float (&sm)[4], uint32_t& ddm) {
+        const uint8_t* blk = wrow + jj * kBlockBytes;
+        const int n = kq >> 1, half = kq & 1;
+        uint32_t qw[4];
+        if (jj & 1) Skinny16Q3K::words<true, 4>(blk, 16 * kq, qw);
+        else Skinny16Q3K::words<false, 4>(blk, 16 * kq, qw);
+        ddm = *reinterpret_cast<const uint16_t*>(blk + 64);
+        v4i acc = {0, 0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            v4i b;
+#pragma unroll
+            for (int k = 0; k < 4; ++k)  // q - 1 on every byte: q + 0x7F stays inside the byte, flipping bit 7 gives q - 1
+                b[k] = (int)((((qw[k] >> (2 * j)) & 0x03030303u) + 0x7F7F7F7Fu) ^ 0x80808080u);
+            const v4i a = *reinterpret_cast<const v4i*>(arow + 128 * n + 32 * j + 16 * half);
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            sd[i] = acc[i];
+            sm[i] = 0.0f;
+        }
+    }
+};
+
 // IQ4_XS (136-byte block: d, scales_h, scales_l[4], qs[128]; crates/infr-cpu/src/kernels.rs:995-1036):
 // isum = sum_ib (ls_ib - 32) * (table[q] . q8) over eight sub-blocks of 32, y += (d * q8.d[b]) * isum.
 // A table value times a 6-bit scale does not fit a byte, so a sub-block is one
@@ -1465,11 +1504,11 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
 constexpr int kSkinny16Waves = 4, kSkinny16Blocks = 2;
 static bool skinny16_shape(int dtype, int nb, size_t m, size_t out_f) {
     const bool nib32 = dtype == 2 || dtype == 3 || dtype == 6 || dtype == 7 || dtype == 20;
-    if (dtype != 12 && dtype != 13 && dtype != 14 && dtype != 8 && dtype != 42 && dtype != 10 && dtype != 11 && dtype != 23 && !nib32)
+    if (dtype != 12 && dtype != 13 && dtype != 14 && dtype != 8 && dtype != 42 && dtype != 10 && dtype != 11 && dtype != 23 && dtype != 35 && !nib32)
         return false;
-    if (nb < kSkinny16Blocks || (nb % kSkinny16Blocks != 0 && (dtype == 14 || dtype == 42 || dtype == 11))) return false;
-    // Q2_K, Q3_K, IQ4_XS: the dot4 batches are the only other kernel, eight tokens per pass over the weights
-    if (dtype == 10 || dtype == 11 || dtype == 23) return m >= 3;
+    if (nb < kSkinny16Blocks || (nb % kSkinny16Blocks != 0 && (dtype == 14 || dtype == 42 || dtype == 11 || dtype == 35))) return false;
+    // Q2_K, Q3_K, IQ4_XS, TQ2_0: the dot4 batches are the only other kernel, eight tokens per pass over the weights
+    if (dtype == 10 || dtype == 11 || dtype == 23 || dtype == 35) return m >= 3;
     if (m <= 16) {
         // the dot4 batch kernels, which unpack a weight once per two or four tokens, stay ahead at the
         // bottom: Q4_K at two tokens (4.3 / 4.0 / 5.5 / 5.6 against 3.7 / 3.4 / 4.2 / 4.2 TB/s on the four
@@ -1590,6 +1629,8 @@ static bool launch_mmq_skinny16(int dtype, const uint8_t* w, size_t bpr, const A
         launch_mmq_skinny16_fmt<Skinny16Q3K, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     else if (dtype == 23)
         launch_mmq_skinny16_fmt<Skinny16IQ4XS, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
+    else if (dtype == 35)
+        launch_mmq_skinny16_fmt<Skinny16TQ2_0, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     else
         launch_mmq_skinny16_fmt<Skinny16Q6K, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     return true;

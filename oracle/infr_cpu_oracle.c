@@ -33,6 +33,7 @@ int orc_block_layout(int dtype, int *elems, int *bytes) {
     case ORC_Q2_K: e = 256; b = 84; break;
     case ORC_Q3_K: e = 256; b = 110; break;
     case ORC_IQ4_XS: e = 256; b = 136; break;
+    case ORC_TQ2_0: e = 256; b = 66; break;
     case ORC_MXFP4: e = 32; b = 17; break;
     case ORC_NVFP4: e = 64; b = 36; break;
     case ORC_Q4_K: e = 256; b = 144; break;
@@ -360,6 +361,20 @@ int orc_dequant_block(int dtype, const uint8_t *bytes, size_t nbytes, float *out
                     out[b * 256 + ib * 32 + j + 16] = dl * (float)orc_kvalues_iq4nl[qs[j] >> 4];
                 }
             }
+        }
+        return 0;
+    case ORC_TQ2_0:
+        /* dequant.rs:968-996: [u8 qs[64]][f16 d]; element 128 chunk + 32 l + m reads bit pair l of
+         * qs[32 chunk + m]; y = (q - 1) * d. */
+        for (size_t b = 0; b < nblk; b++) {
+            const uint8_t *blk = bytes + b * 66;
+            float d = orc_rdf16(blk + 64);
+            for (int chunk = 0; chunk < 2; chunk++)
+                for (int l = 0; l < 4; l++)
+                    for (int mm = 0; mm < 32; mm++) {
+                        int q = (blk[32 * chunk + mm] >> (2 * l)) & 3;
+                        out[b * 256 + chunk * 128 + l * 32 + mm] = (float)(q - 1) * d;
+                    }
         }
         return 0;
     case ORC_MXFP4:
@@ -756,6 +771,25 @@ float orc_vec_dot_iq4xs(const uint8_t *row, const int8_t *qs8, const float *d8, 
     return sumf;
 }
 
+/* crates/infr-cpu/src/kernels.rs:3066-3126 (tq2_0_expand_row, vec_dot_tq2_0): the ternary row as
+ * q - 1 in {-1, 0, 1, 2}, one integer dot per superblock, sumf += d * q8.d[b] * iprod. */
+float orc_vec_dot_tq2_0(const uint8_t *row, const int8_t *qs8, const float *d8, size_t in_f, int32_t *iprod_out) {
+    size_t nb = in_f / 256;
+    float sumf = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * 66;
+        const int8_t *a = qs8 + b * 256;
+        int32_t iprod = 0;
+        for (int chunk = 0; chunk < 2; chunk++)
+            for (int l = 0; l < 4; l++)
+                for (int mm = 0; mm < 32; mm++)
+                    iprod += (((blk[32 * chunk + mm] >> (2 * l)) & 3) - 1) * (int32_t)a[chunk * 128 + l * 32 + mm];
+        if (iprod_out) iprod_out[b] = iprod;
+        sumf += orc_rdf16(blk + 64) * d8[b] * (float)iprod;
+    }
+    return sumf;
+}
+
 /* crates/infr-cpu/src/kernels.rs:6303-6327 (vec_dot_mxfp4_32_batch_scalar), one activation row:
  * per 32-block the table dot with the per-32 activation codes, sumf += d * q8.d[b] * iprod. */
 float orc_vec_dot_mxfp4(const uint8_t *row, const int8_t *qs8, const float *d8, size_t in_f, int32_t *iprod_out) {
@@ -969,7 +1003,7 @@ typedef struct {
  * a Q8_0 row that is a multiple of 32 only takes the per-32 `Q8x32` (q8_0_blk32). */
 static int is_q8_super(int dtype, size_t in_f) {
     return dtype == ORC_Q4_K || dtype == ORC_Q5_K || dtype == ORC_Q6_K || dtype == ORC_Q2_K || dtype == ORC_Q3_K ||
-           dtype == ORC_IQ4_XS || (dtype == ORC_Q8_0 && in_f % 256 == 0);
+           dtype == ORC_IQ4_XS || dtype == ORC_TQ2_0 || (dtype == ORC_Q8_0 && in_f % 256 == 0);
 }
 
 static void acts_free(acts_t *a) {
@@ -1041,6 +1075,7 @@ static float row_dot(int dtype, const uint8_t *row, const acts_t *a, size_t r, s
         return orc_vec_dot_q3k(row, a->qs + r * in_f, a->d + r * nb, a->bsums16 + r * nb * 16, in_f, ia);
     }
     case ORC_IQ4_XS: return orc_vec_dot_iq4xs(row, a->qs + r * in_f, a->d + r * (in_f / 256), in_f, ia);
+    case ORC_TQ2_0: return orc_vec_dot_tq2_0(row, a->qs + r * in_f, a->d + r * (in_f / 256), in_f, ia);
     case ORC_Q4_0:
     case ORC_Q4_1:
     case ORC_Q5_0:
@@ -1067,6 +1102,7 @@ static int linear_shape_ok(int dtype, size_t in_f) {
     case ORC_Q2_K:
     case ORC_Q3_K:
     case ORC_IQ4_XS:
+    case ORC_TQ2_0:
     case ORC_Q6_K: return in_f % 256 == 0;
     case ORC_Q4_0:
     case ORC_Q4_1:
@@ -1165,7 +1201,7 @@ int orc_linear_int_stages(int dtype, const uint8_t *w, size_t wbytes, size_t w_n
     size_t row0 = w_off / in_f;
     if (row0 + out_f > total_rows) return -2;
     const uint8_t *wb = w + row0 * bpr;
-    size_t blocks = (dtype == ORC_Q4_K || dtype == ORC_Q5_K || dtype == ORC_Q6_K || dtype == ORC_Q2_K || dtype == ORC_Q3_K || dtype == ORC_IQ4_XS) ? in_f / 256 : (dtype == ORC_NVFP4 ? in_f / 16 : in_f / 32);
+    size_t blocks = (dtype == ORC_Q4_K || dtype == ORC_Q5_K || dtype == ORC_Q6_K || dtype == ORC_Q2_K || dtype == ORC_Q3_K || dtype == ORC_IQ4_XS || dtype == ORC_TQ2_0) ? in_f / 256 : (dtype == ORC_NVFP4 ? in_f / 16 : in_f / 32);
     acts_t a;
     acts_build(dtype, x, m, in_f, &a);
 #pragma omp parallel for schedule(dynamic, 8)
@@ -1519,6 +1555,7 @@ size_t orc_synth_weight(int dtype, size_t n_elem, uint32_t seed, uint8_t *out) {
             break;
         case ORC_Q3_K: put_f16(blk + 108, 0.03f); break; /* d@108 (decode_spec.rs:325) */
         case ORC_IQ4_XS: put_f16(blk, 0.06f); break;      /* d@0 (decode_spec.rs:351) */
+        case ORC_TQ2_0: put_f16(blk + 64, 0.05f); break;  /* d@64 (decode_spec.rs:356) */
         case ORC_MXFP4: blk[0] = 125; break;              /* E8M0 nearest 0.25 in log space: 2^(125 - 127) (decode_spec.rs:191, 216-219) */
         case ORC_NVFP4:                                   /* UE4M3 nearest 0.5 * (0.625 + 0.125 i) (decode_spec.rs:192-198, 223-245) */
             blk[0] = 42, blk[1] = 44, blk[2] = 46, blk[3] = 48;

@@ -1,8 +1,8 @@
-"""GPU parity of Q2_K, Q3_K and IQ4_XS weights against the CPU oracle, through the C ABI: Op::Linear
+"""GPU parity of Q2_K, Q3_K, IQ4_XS and TQ2_0 weights against the CPU oracle, through the C ABI: Op::Linear
 (one token and batches), Op::EmbedGather tables and Op::MoeFfn expert banks.
 
 infr-cpu multiplies these formats with a per-256 int8 activation (crates/infr-cpu/src/lib.rs:1043-1124,
-vec_dot_q2k / vec_dot_q3k / vec_dot_iq4xs in crates/infr-cpu/src/kernels.rs): the integer stages must be equal and,
+vec_dot_q2k / vec_dot_q3k / vec_dot_iq4xs / vec_dot_tq2_0 in crates/infr-cpu/src/kernels.rs): the integer stages must be equal and,
 since the device adds the per-superblock f32 terms in block order like the CPU, every output must
 be bit-identical. Weights are the oracle's full-range payloads (every 2-/3-bit code, all 6-bit
 scale patterns, both signs of the Q3_K scales)."""
@@ -16,7 +16,7 @@ from tests.test_gpu_moe import check, run_moe
 
 pytestmark = pytest.mark.gpu
 
-BOTH = [DType.Q2K, DType.Q3K, DType.IQ4XS]
+BOTH = [DType.Q2K, DType.Q3K, DType.IQ4XS, DType.TQ2_0]
 ids = lambda d: DType(d).name
 
 
@@ -118,7 +118,7 @@ def test_a_plan_mixes_them_with_other_formats(be):
     groups by (format, in_f) and every output equals the single-op value."""
     in_f = 2048
     outs = [(DType.Q2K, 96), (DType.Q3K, 80), (DType.Q4K, 64), (DType.Q2K, 33), (DType.Q3K, 130), (DType.IQ4XS, 70),
-            (DType.IQ4XS, 9)]
+            (DType.IQ4XS, 9), (DType.TQ2_0, 45)]
     g = Graph()
     x = g.input(TensorDesc((1, in_f), DType.F32))
     ws, ys = [], []
@@ -148,7 +148,7 @@ def test_a_batch_plan_groups_them(be, m):
     quantized activation and one launch per (format, in_f) group."""
     in_f = 2048
     outs = [(DType.Q2K, 96), (DType.Q2K, 40), (DType.Q3K, 80), (DType.Q3K, 33), (DType.Q4K, 64), (DType.IQ4XS, 50),
-            (DType.IQ4XS, 31)]
+            (DType.IQ4XS, 31), (DType.TQ2_0, 45), (DType.TQ2_0, 8)]
     g = Graph()
     x = g.input(TensorDesc((m, in_f), DType.F32))
     ws, ys = [], []

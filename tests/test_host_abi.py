@@ -91,9 +91,11 @@ def test_synth_encoders_reproduce_their_input_distribution(dtype, tol):
     assert np.isfinite(f).all()
 
 
-def test_synth_q2_0_codes_are_ternary():
-    w = infr_amd.synth_weight(B.DType.Q2_0, 5, 16, 1024).reshape(-1, 18)
-    codes = np.stack([(w[:, 2:] >> s) & 3 for s in (0, 2, 4, 6)])
+@pytest.mark.parametrize("dtype", [B.DType.Q2_0, B.DType.TQ2_0])
+def test_synth_ternary_codes(dtype):
+    w = infr_amd.synth_weight(dtype, 5, 16, 1024)
+    w = w.reshape(-1, 18)[:, 2:] if dtype == B.DType.Q2_0 else w.reshape(-1, 66)[:, :64]
+    codes = np.stack([(w >> s) & 3 for s in (0, 2, 4, 6)])
     assert codes.max() == 2 and set(np.unique(codes)) == {0, 1, 2}
     frac = [(codes == v).mean() for v in (0, 1, 2)]
     assert all(abs(f - 1 / 3) < 0.02 for f in frac)
