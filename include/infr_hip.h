@@ -178,8 +178,12 @@ int infr_hip_quantize_q8_32(infr_hip_t *be, const infr_hip_buffer_t *x, size_t m
 /* Per-block integer stages of Op::Linear for every (row r, output o), i32 [m][out_f][blocks]:
  *   Q4_K: a = sd, b = sm per 256-block (crates/infr-cpu/src/kernels.rs:162-181);
  *   Q6_K: a = isum per 256-block (kernels.rs:519-522);
- *   Q8_0: a = iprod per 32-block (kernels.rs:1182); Q2_0: a = iprod per 32 sub-block (:5657-5662).
- * b may be NULL unless dtype is Q4_K. Uses the same device code as infr_hip_linear. */
+ *   Q8_0: a = iprod per 32-block (kernels.rs:1182); Q2_0: a = iprod per 32 sub-block (:5657-5662);
+ *   Q5_K: a = sd, b = sm; Q2_K: a = sd, b = sm (kernels.rs:315-361); Q3_K, IQ4_XS: a = isum (:812-852,
+ *   :1008-1036); TQ2_0: a = iprod per 256-block (:3108-3126); the 32-weight-block formats and MXFP4:
+ *   a = iprod per block. NVFP4 (four integers per block) and one token of Q5_0 (f32 activations)
+ *   return Unsupported.
+ * b may be NULL unless dtype is Q4_K, Q5_K or Q2_K. Uses the same device code as infr_hip_linear. */
 int infr_hip_linear_int_stages(infr_hip_t *be, int dtype, const infr_hip_buffer_t *w,
                                size_t w_numel, size_t w_off, const infr_hip_buffer_t *x, size_t m,
                                size_t in_f, size_t out_f, infr_hip_buffer_t *a,
