@@ -20,9 +20,10 @@ from oracle import oracle as orc
 pytestmark = pytest.mark.gpu
 
 FORMATS = (DType.Q4K, DType.Q5K, DType.Q6K, DType.Q8_0, DType.Q2_0, DType.Q4_0, DType.Q4_1, DType.Q5_0, DType.Q5_1,
-           DType.IQ4NL, DType.F32, DType.F16, DType.BF16)
+           DType.IQ4NL, DType.F32, DType.F16, DType.BF16, DType.Q2K, DType.Q3K, DType.IQ4XS, DType.TQ2_0, DType.MXFP4,
+           DType.NVFP4)
 PLAIN = (DType.F32, DType.F16, DType.BF16)
-BIT_IDENTICAL = (DType.Q4K, DType.Q5K, DType.Q6K) + PLAIN
+BIT_IDENTICAL = (DType.Q4K, DType.Q5K, DType.Q6K, DType.Q2K, DType.Q3K, DType.IQ4XS, DType.TQ2_0) + PLAIN
 TOKENS = (1, 1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 24, 31, 32, 33, 40, 63, 64, 65, 66, 96, 127, 128, 129, 130, 200,
           255, 256, 257, 300)
 
@@ -44,7 +45,7 @@ def draw_case(rng):
     return dtype, m, in_f, out_f, extra_before, extra_after
 
 
-@pytest.mark.parametrize("seed", range(160))
+@pytest.mark.parametrize("seed", range(240))
 def test_linear_on_a_random_shape_matches_the_oracle(be, seed):
     rng = np.random.default_rng(0xF00D + seed)
     dtype, m, in_f, out_f, before, after = draw_case(rng)
@@ -80,11 +81,12 @@ def test_linear_on_a_random_shape_matches_the_oracle(be, seed):
         mx = np.abs(g - t).max() / max(np.abs(t).max(), 1e-30)
         assert rel <= 1e-4 and mx <= 1e-3, f"rel-L2 {rel:.2e} max-abs {mx:.2e}: {case}"
     # every fourth quantized case: the per-block integers behind those outputs, exact on every route
-    # (one token of Q5_0 multiplies f32 activations: it has no integer stage, as on the CPU)
-    if seed % 4 == 1 and dtype not in PLAIN and not (dtype == DType.Q5_0 and m == 1):
+    # (one token of Q5_0 multiplies f32 activations: it has no integer stage, as on the CPU; NVFP4 has
+    # four integers per block and no stage entry)
+    if seed % 4 == 1 and dtype not in PLAIN and dtype != DType.NVFP4 and not (dtype == DType.Q5_0 and m == 1):
         a, b = be.linear_int_stages(dtype, be.upload_new(w), be.upload_new(x), m, in_f, out_f, w_numel=rows * in_f,
                                     w_off=before * in_f)
         oa, ob = orc.linear_int_stages(dtype, w, x, m, in_f, out_f, w_numel=rows * in_f, w_off=before * in_f)
         assert np.array_equal(a, oa), f"first integer stage differs: {case}"
-        if dtype in (DType.Q4K, DType.Q5K):
+        if dtype in (DType.Q4K, DType.Q5K, DType.Q2K):
             assert np.array_equal(b, ob), f"second integer stage differs: {case}"

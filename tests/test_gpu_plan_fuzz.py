@@ -25,7 +25,8 @@ pytestmark = pytest.mark.gpu
 
 WIDTHS = (256, 512, 1024)
 PER_WIDTH = 3
-LINEAR_DTYPES = (DType.Q4K, DType.Q4K, DType.Q6K, DType.Q8_0, DType.Q5_0, DType.Q2_0)
+LINEAR_DTYPES = (DType.Q4K, DType.Q4K, DType.Q6K, DType.Q8_0, DType.Q5_0, DType.Q2_0, DType.Q2K, DType.Q3K, DType.IQ4XS,
+                 DType.TQ2_0, DType.MXFP4, DType.NVFP4)
 MOE = dict(ne=512, n_expert=8, n_used=2, nff=256)
 
 
@@ -180,8 +181,8 @@ def describe(prog):
     return "\n".join(f"  {i:2d}: {op}" for i, op in enumerate(prog))
 
 
-@pytest.mark.parametrize("m,seed", [(1, s) for s in range(16)] + [(3, s) for s in range(100, 106)] +
-                         [(8, s) for s in range(200, 203)] + [(20, s) for s in range(300, 303)] +
+@pytest.mark.parametrize("m,seed", [(1, s) for s in range(24)] + [(3, s) for s in range(100, 108)] +
+                         [(8, s) for s in range(200, 204)] + [(20, s) for s in range(300, 303)] +
                          [(48, s) for s in range(400, 402)])
 def test_scheduled_plan_equals_the_ops_run_one_by_one(be, m, seed):
     rng = np.random.default_rng(seed)
