@@ -145,3 +145,24 @@ def test_moe_banks(be, dtype, rows):
     want = orc.moe_ffn(x, router, gate_w, up_w, down_w, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
                        gate_dtype=int(dtype), up_dtype=int(dtype), down_dtype=int(dtype))
     check(*got, *want)
+
+
+@pytest.mark.parametrize("rows", [1, 9, 40])
+@pytest.mark.parametrize("dts", [(DType.MXFP4, DType.MXFP4, DType.Q4K), (DType.Q2K, DType.Q3K, DType.IQ4XS),
+                                 (DType.Q4K, DType.Q4K, DType.NVFP4), (DType.TQ2_0, DType.TQ2_0, DType.TQ2_0)],
+                         ids=lambda d: "-".join(DType(x).name for x in d))
+def test_moe_banks_mixed_with_the_int8_formats(be, dts, rows):
+    """Each bank of an op takes its own kind (expert_acts_kind, crates/infr-cpu/src/moe.rs:42-53):
+    per-256 int8 activations for a Q4_K bank from two rows up, decoded rows for the others; rows
+    beyond the bucketing thresholds too."""
+    from tests.test_gpu_moe import run_moe_mixed
+    ne, n_expert, n_used, nff = 1024, 16, 4, 512
+    gate_w = synth_weight(dts[0], 0x710, n_expert * nff, ne, 0.05)
+    up_w = synth_weight(dts[1], 0x711, n_expert * nff, ne, 0.05)
+    down_w = synth_weight(dts[2], 0x712, n_expert * ne, nff, 0.05)
+    x = synth_normal_f32(240 + rows, rows * ne)
+    router = synth_normal_f32(241, n_expert * ne, sigma=0.05)
+    got = run_moe_mixed(be, x, router, gate_w, up_w, down_w, rows, ne, n_expert, n_used, nff, dts)
+    want = orc.moe_ffn(x, router, gate_w, up_w, down_w, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
+                       gate_dtype=int(dts[0]), up_dtype=int(dts[1]), down_dtype=int(dts[2]))
+    check(*got, *want)
