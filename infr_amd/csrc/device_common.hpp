@@ -46,6 +46,7 @@ typedef v2i v2i_a2 __attribute__((aligned(2)));
 typedef int v3i __attribute__((ext_vector_type(3)));
 typedef v3i v3i_a4 __attribute__((aligned(4)));
 typedef v3i v3i_a2 __attribute__((aligned(2)));
+typedef int int_a2 __attribute__((aligned(2)));
 typedef v2i v2i_a4 __attribute__((aligned(4)));
 
 // 16-byte load from an address that is only 2-byte aligned (Q6_K / Q8_0 / Q2_0 block strides

@@ -753,10 +753,14 @@ struct FmtQ3K {
     static constexpr bool kClampedOneAhead = false;
     static constexpr bool kLaneSums = true;
     static constexpr bool kRowAhead = true;
+    // A quad's lanes split the fields they all need and exchange them in registers (term): lane p
+    // fetches hmask bytes 8 p .. 8 p + 7 and one word of the block's last 16 bytes - scale words 0..2
+    // for p < 3, the word at byte 106 (two scale bytes and d) for p = 3 - so a block's 110 bytes are
+    // requested once (112 with the overlap) instead of 184 over the quad.
     struct Row {
-        v4i q, hm;
-        v3i sc;      // the 12 scale bytes
-        uint32_t d;
+        v4i q;
+        v2i hm8;
+        uint32_t tail;
     };
     typedef FmtQ6K::Acts Acts;
     __device__ static int units(int in_f) { return in_f / 256; }
@@ -765,18 +769,17 @@ struct FmtQ3K {
     __device__ static void load_row_clamped(Row& r, const uint8_t* rowp, int t, int lane, bool ok) {
         const uint8_t* blk = rowp + (size_t)(ok ? t * 16 + (lane >> 2) : 0) * 110;
         const int p = lane & 3;
-        r.hm = load16_a2(blk + 16 * (p & 1));
+        r.hm8 = gload<v2i_a2>(blk + 8 * p);
         r.q = load16_a2(blk + 32 + 16 * p);
-        r.sc = gload<v3i_a2>(blk + 96);
-        r.d = load_u16(blk + 108);
+        r.tail = (uint32_t)gload<int_a2>(blk + (p < 3 ? 96 + 4 * p : 106));
     }
     __device__ static void load_row(Row& r, const uint8_t* rowp, int t, int lane, bool ok) {
         if (ok) {
             load_row_clamped(r, rowp, t, lane, true);
         } else {
-            r.q = r.hm = v4i{0, 0, 0, 0};
-            r.sc = v3i{0, 0, 0};
-            r.d = 0;
+            r.q = v4i{0, 0, 0, 0};
+            r.hm8 = v2i{0, 0};
+            r.tail = 0;
         }
     }
     __device__ static void load_acts(Acts& a, const ActPtrs& s, int t, int lane, bool ok) {
@@ -787,12 +790,20 @@ struct FmtQ3K {
                                  const StagePtrs& st, size_t row_units) {
         const int n = (lane >> 1) & 1, half = lane & 1;
         const int qw[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
-        const int hw[4] = {r.hm.x, r.hm.y, r.hm.z, r.hm.w};
+        // hmask[16 half ..]: the two words of lane 2 half, then those of lane 2 half + 1
+        const int hw[4] = {__builtin_amdgcn_mov_dpp(r.hm8.x, 0x88, 0xF, 0xF, true),   // quad_perm [0,2,0,2]
+                           __builtin_amdgcn_mov_dpp(r.hm8.y, 0x88, 0xF, 0xF, true),
+                           __builtin_amdgcn_mov_dpp(r.hm8.x, 0xDD, 0xF, 0xF, true),   // quad_perm [1,3,1,3]
+                           __builtin_amdgcn_mov_dpp(r.hm8.y, 0xDD, 0xF, 0xF, true)};
+        const uint32_t sc_x = (uint32_t)__builtin_amdgcn_mov_dpp((int)r.tail, 0x00, 0xF, 0xF, true);  // lane 0's word
+        const uint32_t sc_y = (uint32_t)__builtin_amdgcn_mov_dpp((int)r.tail, 0x55, 0xF, 0xF, true);  // lane 1's
+        const uint32_t sc_z = (uint32_t)__builtin_amdgcn_mov_dpp((int)r.tail, 0xAA, 0xF, 0xF, true);  // lane 2's
+        const uint32_t d16 = (uint32_t)__builtin_amdgcn_mov_dpp((int)r.tail, 0xFF, 0xF, 0xF, true) >> 16;  // lane 3's: d on top
         // scales 8 n .. 8 n + 7 as two words of bytes: nibbles of the first eight bytes (low for
         // n = 0, high for n = 1) with two more bits each from the last four
-        const uint32_t k1 = 0x03030303u, k2 = 0x0F0F0F0Fu, tt = (uint32_t)r.sc.z >> (4 * n);
-        const uint32_t w0 = (((uint32_t)r.sc.x >> (4 * n)) & k2) | ((tt & k1) << 4);
-        const uint32_t w1 = (((uint32_t)r.sc.y >> (4 * n)) & k2) | (((tt >> 2) & k1) << 4);
+        const uint32_t k1 = 0x03030303u, k2 = 0x0F0F0F0Fu, tt = sc_z >> (4 * n);
+        const uint32_t w0 = ((sc_x >> (4 * n)) & k2) | ((tt & k1) << 4);
+        const uint32_t w1 = ((sc_y >> (4 * n)) & k2) | (((tt >> 2) & k1) << 4);
         // hmask bits 4 n .. 4 n + 3 of every byte moved to bits 2 .. 5: bit pair j's third bit then
         // sits 2 + j above bit 0
         uint32_t hs[4];
@@ -820,7 +831,7 @@ struct FmtQ3K {
         const int isum = quad_sum(part);
         if (STAGES && ok && (lane & 3) == 0) st.a[row_units + t * 16 + (lane >> 2)] = isum;
         // sumf += d * q8.d[b] * isum as f32
-        return f16_bits_to_f32(r.d) * a.dact * (float)isum;
+        return f16_bits_to_f32(d16) * a.dact * (float)isum;
     }
 };
 
