@@ -1065,10 +1065,9 @@ __device__ __forceinline__ float ue4m3_half(uint32_t x) {
 }
 
 // MXFP4 (17-byte block [u8 e][u8 qs[16]], any byte alignment; crates/infr-cpu/src/kernels.rs:6303-6327):
-// a lane owns block t * 64 + l against the per-32 activation, sumf += d * q8.d[b] * iprod. The 16
-// code bytes are fetched as the five aligned dwords that cover them and shifted into place; when
-// the codes happen to start on a dword the fifth load repeats the fourth (nothing beyond the
-// block's last byte's dword is ever read).
+// a lane owns block t * 64 + l against the per-32 activation, sumf += d * q8.d[b] * iprod. The
+// block is fetched as the five aligned dwords that hold it - two loads - and shifted into place
+// (nothing beyond the dword of the block's last byte is read).
 struct FmtMXFP4 {
     static constexpr int kElemsPerStep = 2048;
     static constexpr bool kPer32 = true;
@@ -1092,15 +1091,21 @@ struct FmtMXFP4 {
             return;
         }
         const uint8_t* blk = rowp + (size_t)(t * 64 + lane) * 17;
-        r.e = gload<uint8_t>(blk);
-        const uint32_t sh = (uint32_t)(reinterpret_cast<uintptr_t>(blk + 1) & 3);
-        const uint8_t* a = blk + 1 - sh;
+        // the five aligned words that hold the block: e is byte `off` of the first, the codes start
+        // off + 1 bytes in (a whole word further when off == 3)
+        const uint32_t off = (uint32_t)(reinterpret_cast<uintptr_t>(blk) & 3);
+        const uint8_t* a = blk - off;
         const v4i lo = load16_a4(a);
-        const uint32_t w4 = (uint32_t)load_u32(a + (sh ? 16 : 12));
-        r.qs = v4i{(int)__builtin_amdgcn_alignbyte((uint32_t)lo.y, (uint32_t)lo.x, sh),
-                   (int)__builtin_amdgcn_alignbyte((uint32_t)lo.z, (uint32_t)lo.y, sh),
-                   (int)__builtin_amdgcn_alignbyte((uint32_t)lo.w, (uint32_t)lo.z, sh),
-                   (int)__builtin_amdgcn_alignbyte(w4, (uint32_t)lo.w, sh)};
+        const uint32_t w4 = (uint32_t)load_u32(a + 16);
+        r.e = ((uint32_t)lo.x >> (8 * off)) & 0xFFu;
+        const uint32_t sh = off + 1;  // v_alignbyte_b32 takes the shift modulo 4: 4 selects the next word
+        const uint32_t c0 = __builtin_amdgcn_alignbyte((uint32_t)lo.y, (uint32_t)lo.x, sh);
+        const uint32_t c1 = __builtin_amdgcn_alignbyte((uint32_t)lo.z, (uint32_t)lo.y, sh);
+        const uint32_t c2 = __builtin_amdgcn_alignbyte((uint32_t)lo.w, (uint32_t)lo.z, sh);
+        const uint32_t c3 = __builtin_amdgcn_alignbyte(w4, (uint32_t)lo.w, sh);
+        const bool whole = off == 3;
+        r.qs = v4i{(int)(whole ? (uint32_t)lo.y : c0), (int)(whole ? (uint32_t)lo.z : c1),
+                   (int)(whole ? (uint32_t)lo.w : c2), (int)(whole ? w4 : c3)};
     }
     __device__ static void load_acts(Acts& a, const ActPtrs& s, int t, int lane, bool ok) {
         FmtNib32<Nib32::IQ4_NL>::load_acts(a, s, t, lane, ok);
