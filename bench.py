@@ -695,7 +695,7 @@ def main():
         for name, dt in (("Q5_K", DType.Q5K), ("Q4_0", DType.Q4_0), ("Q4_1", DType.Q4_1), ("Q5_0", DType.Q5_0),
                          ("Q5_1", DType.Q5_1), ("IQ4_NL", DType.IQ4NL), ("Q2_0", DType.Q2_0), ("Q2_K", DType.Q2K),
                          ("Q3_K", DType.Q3K), ("IQ4_XS", DType.IQ4XS), ("MXFP4", DType.MXFP4), ("NVFP4", DType.NVFP4),
-                         ("TQ2_0", DType.TQ2_0)):
+                         ("TQ2_0", DType.TQ2_0), ("TQ1_0", DType.TQ1_0)):
             for m in (1, 8):
                 for (out_f, in_f) in ((4096, 4096), (12288, 4096), (4096, 12288)):
                     t, nb = single_shape(be, dt, m, in_f, out_f)

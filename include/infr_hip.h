@@ -53,6 +53,7 @@ typedef enum {
     INFR_DTYPE_Q6_K = 14, /* 256 / 210 B: [u8 ql[128]][u8 qh[64]][i8 sc[16]][f16 d]       :330-331 */
     INFR_DTYPE_IQ4_NL = 20, /* 32 / 18 B: [f16 d][u8 qs[16]]  w = d*codebook[q]           :349-350 */
     INFR_DTYPE_IQ4_XS = 23, /* 256 / 136 B: [f16 d][u16 scales_h][u8 scales_l[4]][u8 qs[128]] :351 */
+    INFR_DTYPE_TQ1_0 = 34,  /* 256 / 54 B: [u8 qs[48]][u8 qh[4]][f16 d]  w = d*(digit-1), base-3 packed ternary :354 */
     INFR_DTYPE_TQ2_0 = 35,  /* 256 / 66 B: [u8 qs[64]][f16 d]  w = d*(q-1), 2-bit ternary codes         :356 */
     INFR_DTYPE_MXFP4 = 39,  /* 32 / 17 B: [u8 e][u8 qs[16]]  w = table[q] * 2^(e-128)             :361 */
     INFR_DTYPE_NVFP4 = 40,  /* 64 / 36 B: [u8 d[4]][u8 qs[32]]  w = table[q] * ue4m3(d[i/16]) / 2     :363 */
@@ -180,7 +181,7 @@ int infr_hip_quantize_q8_32(infr_hip_t *be, const infr_hip_buffer_t *x, size_t m
  *   Q6_K: a = isum per 256-block (kernels.rs:519-522);
  *   Q8_0: a = iprod per 32-block (kernels.rs:1182); Q2_0: a = iprod per 32 sub-block (:5657-5662);
  *   Q5_K: a = sd, b = sm; Q2_K: a = sd, b = sm (kernels.rs:315-361); Q3_K, IQ4_XS: a = isum (:812-852,
- *   :1008-1036); TQ2_0: a = iprod per 256-block (:3108-3126); the 32-weight-block formats and MXFP4:
+ *   :1008-1036); TQ1_0, TQ2_0: a = iprod per 256-block (:3218-3240, :3108-3126); the 32-weight-block formats and MXFP4:
  *   a = iprod per block. NVFP4 (four integers per block) and one token of Q5_0 (f32 activations)
  *   return Unsupported.
  * b may be NULL unless dtype is Q4_K, Q5_K or Q2_K. Uses the same device code as infr_hip_linear. */

@@ -45,7 +45,7 @@ enum class DType : int {
     F32 = INFR_DTYPE_F32, F16 = INFR_DTYPE_F16, Q4_0 = INFR_DTYPE_Q4_0, Q4_1 = INFR_DTYPE_Q4_1,
     Q5_0 = INFR_DTYPE_Q5_0, Q5_1 = INFR_DTYPE_Q5_1, Q8_0 = INFR_DTYPE_Q8_0, Q2K = INFR_DTYPE_Q2_K,
     Q3K = INFR_DTYPE_Q3_K, Q4K = INFR_DTYPE_Q4_K,
-    Q5K = INFR_DTYPE_Q5_K, Q6K = INFR_DTYPE_Q6_K, IQ4NL = INFR_DTYPE_IQ4_NL, IQ4XS = INFR_DTYPE_IQ4_XS, TQ2_0 = INFR_DTYPE_TQ2_0, MXFP4 = INFR_DTYPE_MXFP4, NVFP4 = INFR_DTYPE_NVFP4, I32 = 26,
+    Q5K = INFR_DTYPE_Q5_K, Q6K = INFR_DTYPE_Q6_K, IQ4NL = INFR_DTYPE_IQ4_NL, IQ4XS = INFR_DTYPE_IQ4_XS, TQ1_0 = INFR_DTYPE_TQ1_0, TQ2_0 = INFR_DTYPE_TQ2_0, MXFP4 = INFR_DTYPE_MXFP4, NVFP4 = INFR_DTYPE_NVFP4, I32 = 26,
     BF16 = INFR_DTYPE_BF16, Q2_0 = INFR_DTYPE_Q2_0,
 };
 
@@ -65,6 +65,7 @@ inline const char* dtype_name(DType d) {
     case DType::Q6K: return "Q6K";
     case DType::IQ4NL: return "IQ4NL";
     case DType::IQ4XS: return "IQ4XS";
+    case DType::TQ1_0: return "TQ1_0";
     case DType::TQ2_0: return "TQ2_0";
     case DType::MXFP4: return "MXFP4";
     case DType::NVFP4: return "NVFP4";

@@ -35,6 +35,7 @@ class DType(IntEnum):
     Q6K = 14
     IQ4NL = 20
     IQ4XS = 23
+    TQ1_0 = 34
     TQ2_0 = 35
     MXFP4 = 39
     NVFP4 = 40
@@ -642,7 +643,7 @@ class HipBackend:
         if w_numel is None:
             e, b = block_layout(dtype)
             w_numel = w.len_bytes() // b * e
-        blocks = in_f // 256 if dtype in (DType.Q4K, DType.Q5K, DType.Q6K, DType.Q2K, DType.Q3K, DType.IQ4XS, DType.TQ2_0) else in_f // 32
+        blocks = in_f // 256 if dtype in (DType.Q4K, DType.Q5K, DType.Q6K, DType.Q2K, DType.Q3K, DType.IQ4XS, DType.TQ2_0, DType.TQ1_0) else in_f // 32
         a = self.alloc(m * out_f * blocks * 4)
         b_ = self.alloc(m * out_f * blocks * 4) if dtype in (DType.Q4K, DType.Q5K, DType.Q2K) else None
         self._check(self._lib.infr_hip_linear_int_stages(

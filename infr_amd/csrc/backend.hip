@@ -139,7 +139,7 @@ bool is_quant(int dt) {
     case INFR_DTYPE_Q4_0: case INFR_DTYPE_Q4_1: case INFR_DTYPE_Q5_0: case INFR_DTYPE_Q5_1:
     case INFR_DTYPE_Q8_0: case INFR_DTYPE_Q4_K: case INFR_DTYPE_Q5_K: case INFR_DTYPE_Q6_K:
     case INFR_DTYPE_Q2_K: case INFR_DTYPE_Q3_K: case INFR_DTYPE_IQ4_XS: case INFR_DTYPE_MXFP4: case INFR_DTYPE_NVFP4:
-    case INFR_DTYPE_TQ2_0: case INFR_DTYPE_IQ4_NL: case INFR_DTYPE_Q2_0: return true;
+    case INFR_DTYPE_TQ1_0: case INFR_DTYPE_TQ2_0: case INFR_DTYPE_IQ4_NL: case INFR_DTYPE_Q2_0: return true;
     default: return false;
     }
 }
@@ -151,6 +151,7 @@ bool is_moe_quant(int dt) {
     case INFR_DTYPE_Q4_0: case INFR_DTYPE_Q4_1: case INFR_DTYPE_Q5_0: case INFR_DTYPE_Q5_1:
     case INFR_DTYPE_IQ4_NL: case INFR_DTYPE_Q2_0: case INFR_DTYPE_Q2_K: case INFR_DTYPE_Q3_K:
     case INFR_DTYPE_IQ4_XS: case INFR_DTYPE_MXFP4: case INFR_DTYPE_NVFP4: case INFR_DTYPE_TQ2_0:
+    case INFR_DTYPE_TQ1_0:
     case INFR_DTYPE_F32: case INFR_DTYPE_F16: case INFR_DTYPE_BF16:
         return true;
     default: return false;
@@ -169,7 +170,7 @@ size_t in_f_multiple(int dt) {
 // Blocks per row of the per-block integer stage outputs: per 256 for the K-quants, per 32 otherwise.
 size_t stage_blocks(int dt, size_t in_f) {
     return (dt == INFR_DTYPE_Q4_K || dt == INFR_DTYPE_Q5_K || dt == INFR_DTYPE_Q6_K || dt == INFR_DTYPE_Q2_K ||
-            dt == INFR_DTYPE_Q3_K || dt == INFR_DTYPE_IQ4_XS || dt == INFR_DTYPE_TQ2_0)
+            dt == INFR_DTYPE_Q3_K || dt == INFR_DTYPE_IQ4_XS || dt == INFR_DTYPE_TQ2_0 || dt == INFR_DTYPE_TQ1_0)
                ? in_f / 256
                : in_f / 32;
 }

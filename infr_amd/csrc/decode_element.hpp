@@ -92,6 +92,17 @@ __device__ inline float decode_element(int dtype, const uint8_t* rowp, int e) {
         const int kv[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
         return (ldf16(blk) * (float)ls) * (float)kv[nib];
     }
+    case 34: {  // TQ1_0: (digit - 1) * d, digit n of a byte = high byte of 3 * (byte * 3^n mod 256) (dequant.rs:922-967)
+        const uint8_t* blk = rowp + (size_t)(e >> 8) * 54;
+        const int i = e & 255;
+        int n, at;
+        if (i < 160) { n = i >> 5; at = i & 31; }
+        else if (i < 240) { n = (i - 160) >> 4; at = 32 + ((i - 160) & 15); }
+        else { n = (i - 240) >> 2; at = 48 + ((i - 240) & 3); }
+        uint32_t q = ld8(blk + at);
+        for (int k = 0; k < n; ++k) q = (q * 3u) & 0xFFu;
+        return (float)((int)((q * 3u) >> 8) - 1) * ldf16(blk + 52);
+    }
     case 35: {  // TQ2_0: (q - 1) * d (dequant.rs:968-996)
         const uint8_t* blk = rowp + (size_t)(e >> 8) * 66;
         const int i = e & 255;

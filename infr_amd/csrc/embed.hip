@@ -31,7 +31,7 @@ __global__ __launch_bounds__(256) void embed_gather_kernel(int dtype, const uint
 bool embed_gather_supported(int dtype) {
     switch (dtype) {
     case 0: case 1: case 30: case 2: case 3: case 6: case 7: case 8: case 10: case 11: case 12: case 13: case 14: case 20:
-    case 23: case 35: case 39: case 40: case 42:
+    case 23: case 34: case 35: case 39: case 40: case 42:
         return true;
     default: return false;
     }

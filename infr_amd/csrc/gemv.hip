@@ -37,6 +37,7 @@ static const GemvFormatOps* format_ops(int dtype, size_t in_f) {
     case 10: return &gemv_ops_q2k();
     case 11: return &gemv_ops_q3k();
     case 23: return &gemv_ops_iq4xs();
+    case 34: return &gemv_ops_tq1_0();
     case 35: return &gemv_ops_tq2_0();
     case 39: return &gemv_ops_mxfp4();
     case 40: return &gemv_ops_nvfp4();

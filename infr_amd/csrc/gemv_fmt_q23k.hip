@@ -1,4 +1,4 @@
-// Instantiates the decode GEMV templates for: FmtQ2K, FmtQ3K, FmtTQ2_0, FmtIQ4XS, FmtMXFP4, FmtNVFP4.
+// Instantiates the decode GEMV templates for: FmtQ2K, FmtQ3K, FmtTQ1_0, FmtTQ2_0, FmtIQ4XS, FmtMXFP4, FmtNVFP4.
 #include "gemv_impl.hpp"
 
 namespace infr {
@@ -13,6 +13,10 @@ const GemvFormatOps& gemv_ops_q3k() {
 }
 const GemvFormatOps& gemv_ops_iq4xs() {
     static const GemvFormatOps ops = make_gemv_format_ops<FmtIQ4XS>();
+    return ops;
+}
+const GemvFormatOps& gemv_ops_tq1_0() {
+    static const GemvFormatOps ops = make_gemv_format_ops<FmtTQ1_0>();
     return ops;
 }
 const GemvFormatOps& gemv_ops_tq2_0() {

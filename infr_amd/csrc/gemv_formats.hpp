@@ -681,6 +681,115 @@ struct FmtQ2K {
     }
 };
 
+// TQ1_0 (54-byte block, 2-byte aligned: [u8 qs[48]][u8 qh[4]][f16 d]): base-3 packed ternary. A byte
+// holds five digits (qh: four): digit n is the high byte of three times (byte * 3^n mod 256), i.e.
+// repeated "times three, take the carry". Elements come in three runs - qs[0..32) x 5 digits ->
+// 32 n + m, qs[32..48) x 5 -> 160 + 16 n + m, qh[0..4) x 4 -> 240 + 4 n + j - and a weight is
+// (digit - 1) d: iprod = sum digit * q8 - (the activation's code sum), term d * q8.d[b] * iprod
+// (crates/infr-cpu/src/kernels.rs:3167-3240), blocks in ascending order. Lane p of a block's four owns
+// qs[8 p .. 8 p + 8), qs[32 + 4 p .. + 4) and qh[p]: 64 weights, whose activations are gathered to
+// match (digit n of word k of the first run meets bytes 32 n + 8 p + 4 k .. + 3). Four bytes are
+// unpacked at a time, even and odd bytes in the two halves of a word (three times a byte fits 16 bits).
+struct FmtTQ1_0 {
+    static constexpr int kElemsPerStep = 4096;
+    static constexpr bool kPer32 = false;
+    static constexpr bool kOrdered = true;
+    static constexpr int kBlockBytes = 54, kBlockElems = 256;
+    static constexpr int kWide16Steps = 3;
+    static constexpr bool kClampedLoads = false;
+    static constexpr bool kLaneSums = true;
+    static constexpr bool kRowAhead = false;
+    struct Row {
+        v2i a;       // qs[8 p .. 8 p + 8)
+        uint32_t b;  // qs[32 + 4 p .. + 4)
+        v2i tail;    // bytes 46 .. 53: qs[46], qs[47], qh[0..4), d
+    };
+    struct Acts {
+        int xa[16];  // 2 n + k: first run, digit n, word k; 10 + n: second run, digit n; 15: third run
+        int bs;      // code sum of the 64 activations this lane's index p stands for (two per-32 sums)
+        float dact;
+    };
+    __device__ static int units(int in_f) { return in_f / 256; }
+    __device__ static bool valid(int t, int lane, int n) { return t * 16 + (lane >> 2) < n; }
+    __device__ static void load_row(Row& r, const uint8_t* rowp, int t, int lane, bool ok) {
+        if (ok) {
+            const uint8_t* blk = rowp + (size_t)(t * 16 + (lane >> 2)) * 54;
+            const int p = lane & 3;
+            r.a = gload<v2i_a2>(blk + 8 * p);
+            r.b = (uint32_t)gload<int_a2>(blk + 32 + 4 * p);
+            r.tail = gload<v2i_a2>(blk + 46);
+        } else {
+            r.a = r.tail = v2i{0, 0};
+            r.b = 0;
+        }
+    }
+    __device__ static void load_acts(Acts& a, const ActPtrs& s, int t, int lane, bool ok) {
+        if (ok) {
+            const int b = t * 16 + (lane >> 2), p = lane & 3;
+            const int8_t* base = s.qs + (size_t)b * 256;
+#pragma unroll
+            for (int n = 0; n < 5; ++n) {
+                const v2i v = *reinterpret_cast<const v2i*>(base + 32 * n + 8 * p);
+                a.xa[2 * n] = v.x;
+                a.xa[2 * n + 1] = v.y;
+                a.xa[10 + n] = *reinterpret_cast<const int*>(base + 160 + 16 * n + 4 * p);
+            }
+            // elements 240 + 4 n + p: byte p of each of the last four words
+            const v4i last = *reinterpret_cast<const v4i*>(base + 240);
+            const int sh = 8 * p;
+            a.xa[15] = (int)((((uint32_t)last.x >> sh) & 0xFFu) | ((((uint32_t)last.y >> sh) & 0xFFu) << 8) |
+                             ((((uint32_t)last.z >> sh) & 0xFFu) << 16) | ((((uint32_t)last.w >> sh) & 0xFFu) << 24));
+            a.bs = s.bsums[(size_t)b * 8 + 2 * p] + s.bsums[(size_t)b * 8 + 2 * p + 1];
+            a.dact = s.d[b];
+        } else {
+#pragma unroll
+            for (int k = 0; k < 16; ++k) a.xa[k] = 0;
+            a.bs = 0;
+            a.dact = 0.0f;
+        }
+    }
+    // The five digits of each of a word's four bytes: out[n] holds digit n of byte k in byte k.
+    __device__ static void digits5(uint32_t w, uint32_t (&out)[5]) {
+        uint32_t e = w & 0x00FF00FFu, o = (w >> 8) & 0x00FF00FFu;
+#pragma unroll
+        for (int n = 0; n < 5; ++n) {
+            const uint32_t te = e * 3u, to = o * 3u;  // per 16-bit half: at most 765
+            out[n] = ((te >> 8) & 0x00FF00FFu) | (to & 0xFF00FF00u);
+            e = te & 0x00FF00FFu;
+            o = to & 0x00FF00FFu;
+        }
+    }
+    template <bool STAGES>
+    __device__ static float term(const Row& r, const Acts& a, int t, int lane, bool ok,
+                                 const StagePtrs& st, size_t row_units) {
+        const int p = lane & 3;
+        uint32_t d0[5], d1[5], d2[5];
+        digits5((uint32_t)r.a.x, d0);
+        digits5((uint32_t)r.a.y, d1);
+        digits5(r.b, d2);
+        int ip = 0;
+#pragma unroll
+        for (int n = 0; n < 5; ++n) {
+            ip = dot4((int)d0[n], a.xa[2 * n], ip);
+            ip = dot4((int)d1[n], a.xa[2 * n + 1], ip);
+            ip = dot4((int)d2[n], a.xa[10 + n], ip);
+        }
+        // qh[p]: four digits, digit n to byte n
+        const uint32_t qh = ((uint32_t)r.tail.x >> 16) | ((uint32_t)r.tail.y << 16);
+        uint32_t q = (qh >> (8 * p)) & 0xFFu, dq = 0;
+#pragma unroll
+        for (int n = 0; n < 4; ++n) {
+            const uint32_t tq = q * 3u;
+            dq |= (tq >> 8) << (8 * n);
+            q = tq & 0xFFu;
+        }
+        ip = dot4((int)dq, a.xa[15], ip);
+        const int iprod = quad_sum(ip - a.bs);
+        if (STAGES && ok && p == 0) st.a[row_units + t * 16 + (lane >> 2)] = iprod;
+        return f16_bits_to_f32((uint32_t)r.tail.y >> 16) * a.dact * (float)iprod;  // sumf += d * q8.d[b] * iprod as f32
+    }
+};
+
 // TQ2_0 (66-byte block, 2-byte aligned: [u8 qs[64]][f16 d]): the bit pairs are laid out as Q2_K's, a
 // code q is the ternary weight q - 1 with one scale per superblock: iprod = sum (q - 1) * q8 =
 // sum q * q8 - (the activation's code sum), term d * q8.d[b] * iprod

@@ -227,6 +227,7 @@ const GemvFormatOps& gemv_ops_q5k();
 const GemvFormatOps& gemv_ops_q2k();
 const GemvFormatOps& gemv_ops_q3k();
 const GemvFormatOps& gemv_ops_iq4xs();
+const GemvFormatOps& gemv_ops_tq1_0();
 const GemvFormatOps& gemv_ops_tq2_0();
 const GemvFormatOps& gemv_ops_mxfp4();
 const GemvFormatOps& gemv_ops_nvfp4();

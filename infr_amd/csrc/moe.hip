@@ -1486,6 +1486,7 @@ const char* launch_moe_ffn(const MoeShape& shape, const MoeBuffers& bufs, void* 
         case 10: return in_f / 256 * 84;
         case 11: return in_f / 256 * 110;
         case 23: return in_f / 256 * 136;
+        case 34: return in_f / 256 * 54;
         case 35: return in_f / 256 * 66;
         case 39: return in_f / 32 * 17;
         case 40: return in_f / 64 * 36;

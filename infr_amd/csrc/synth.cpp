@@ -498,6 +498,7 @@ int infr_block_layout(int dtype, int* elems, int* bytes) {
     case INFR_DTYPE_Q2_K: e = 256; b = 84; break;
     case INFR_DTYPE_Q3_K: e = 256; b = 110; break;
     case INFR_DTYPE_IQ4_XS: e = 256; b = 136; break;
+    case INFR_DTYPE_TQ1_0: e = 256; b = 54; break;
     case INFR_DTYPE_TQ2_0: e = 256; b = 66; break;
     case INFR_DTYPE_MXFP4: e = 32; b = 17; break;
     case INFR_DTYPE_NVFP4: e = 64; b = 36; break;
@@ -537,6 +538,20 @@ size_t infr_synth_weight(int dtype, uint64_t seed, float sigma, size_t rows, siz
                     uint8_t byte = 0;
                     for (int k = 0; k < 4; ++k) byte |= (uint8_t)((g.rng.next() % 3) << (2 * k));
                     blk[2 + i] = byte;
+                }
+            }
+            return;
+        }
+        if (dtype == INFR_DTYPE_TQ1_0) {
+            // digits i.i.d. uniform over {0,1,2}, five to a byte as ceil(v * 256 / 243) with the first digit
+            // most significant (qh: four digits and a zero), scale |N(0, sigma^2)| per block
+            for (size_t b = 0; b < in_f / 256; ++b) {
+                uint8_t* blk = row + b * 54;
+                put_f16(blk + 52, std::fabs(sigma * (float)g.next()));
+                for (int i = 0; i < 52; ++i) {
+                    uint32_t v = 0;
+                    for (int k = 0; k < 5; ++k) v = v * 3 + (k == 4 && i >= 48 ? 0u : (uint32_t)(g.rng.next() % 3));
+                    blk[i] = (uint8_t)((v * 256 + 242) / 243);
                 }
             }
             return;

@@ -33,6 +33,7 @@ int orc_block_layout(int dtype, int *elems, int *bytes) {
     case ORC_Q2_K: e = 256; b = 84; break;
     case ORC_Q3_K: e = 256; b = 110; break;
     case ORC_IQ4_XS: e = 256; b = 136; break;
+    case ORC_TQ1_0: e = 256; b = 54; break;
     case ORC_TQ2_0: e = 256; b = 66; break;
     case ORC_MXFP4: e = 32; b = 17; break;
     case ORC_NVFP4: e = 64; b = 36; break;
@@ -361,6 +362,16 @@ int orc_dequant_block(int dtype, const uint8_t *bytes, size_t nbytes, float *out
                     out[b * 256 + ib * 32 + j + 16] = dl * (float)orc_kvalues_iq4nl[qs[j] >> 4];
                 }
             }
+        }
+        return 0;
+    case ORC_TQ1_0:
+        /* dequant.rs:922-967: [u8 qs[48]][u8 qh[4]][f16 d]; y = (digit - 1) * d in three runs:
+         * qs[0..32) x 5 digits -> elements 32 n + m, qs[32..48) x 5 -> 160 + 16 n + m,
+         * qh[0..4) x 4 -> 240 + 4 n + j. */
+        for (size_t b = 0; b < nblk; b++) {
+            const uint8_t *blk = bytes + b * 54;
+            float d = orc_rdf16(blk + 52);
+            for (int i = 0; i < 256; i++) out[b * 256 + i] = (float)(orc_tq1_0_digit(blk, i) - 1) * d;
         }
         return 0;
     case ORC_TQ2_0:
@@ -771,6 +782,35 @@ float orc_vec_dot_iq4xs(const uint8_t *row, const int8_t *qs8, const float *d8, 
     return sumf;
 }
 
+/* Ternary digit (0..2) of element i of a TQ1_0 block: byte * 3^n modulo 256, times three, high byte
+ * (crates/infr-cpu/src/kernels.rs:3167-3216, tq1_0_expand_row; dequant.rs:926-962). */
+int orc_tq1_0_digit(const uint8_t *blk, int i) {
+    static const uint8_t pow3[5] = {1, 3, 9, 27, 81};
+    uint8_t byte;
+    int n;
+    if (i < 160) { n = i / 32; byte = blk[i % 32]; }
+    else if (i < 240) { n = (i - 160) / 16; byte = blk[32 + (i - 160) % 16]; }
+    else { n = (i - 240) / 4; byte = blk[48 + (i - 240) % 4]; }
+    uint8_t q = (uint8_t)(byte * pow3[n]);
+    return (int)(((uint16_t)q * 3) >> 8);
+}
+
+/* crates/infr-cpu/src/kernels.rs:3218-3240 (vec_dot_tq1_0): the row as digit - 1, one integer dot per
+ * superblock, sumf += d * q8.d[b] * iprod. */
+float orc_vec_dot_tq1_0(const uint8_t *row, const int8_t *qs8, const float *d8, size_t in_f, int32_t *iprod_out) {
+    size_t nb = in_f / 256;
+    float sumf = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * 54;
+        const int8_t *a = qs8 + b * 256;
+        int32_t iprod = 0;
+        for (int i = 0; i < 256; i++) iprod += (orc_tq1_0_digit(blk, i) - 1) * (int32_t)a[i];
+        if (iprod_out) iprod_out[b] = iprod;
+        sumf += orc_rdf16(blk + 52) * d8[b] * (float)iprod;
+    }
+    return sumf;
+}
+
 /* crates/infr-cpu/src/kernels.rs:3066-3126 (tq2_0_expand_row, vec_dot_tq2_0): the ternary row as
  * q - 1 in {-1, 0, 1, 2}, one integer dot per superblock, sumf += d * q8.d[b] * iprod. */
 float orc_vec_dot_tq2_0(const uint8_t *row, const int8_t *qs8, const float *d8, size_t in_f, int32_t *iprod_out) {
@@ -1003,7 +1043,7 @@ typedef struct {
  * a Q8_0 row that is a multiple of 32 only takes the per-32 `Q8x32` (q8_0_blk32). */
 static int is_q8_super(int dtype, size_t in_f) {
     return dtype == ORC_Q4_K || dtype == ORC_Q5_K || dtype == ORC_Q6_K || dtype == ORC_Q2_K || dtype == ORC_Q3_K ||
-           dtype == ORC_IQ4_XS || dtype == ORC_TQ2_0 || (dtype == ORC_Q8_0 && in_f % 256 == 0);
+           dtype == ORC_IQ4_XS || dtype == ORC_TQ2_0 || dtype == ORC_TQ1_0 || (dtype == ORC_Q8_0 && in_f % 256 == 0);
 }
 
 static void acts_free(acts_t *a) {
@@ -1076,6 +1116,7 @@ static float row_dot(int dtype, const uint8_t *row, const acts_t *a, size_t r, s
     }
     case ORC_IQ4_XS: return orc_vec_dot_iq4xs(row, a->qs + r * in_f, a->d + r * (in_f / 256), in_f, ia);
     case ORC_TQ2_0: return orc_vec_dot_tq2_0(row, a->qs + r * in_f, a->d + r * (in_f / 256), in_f, ia);
+    case ORC_TQ1_0: return orc_vec_dot_tq1_0(row, a->qs + r * in_f, a->d + r * (in_f / 256), in_f, ia);
     case ORC_Q4_0:
     case ORC_Q4_1:
     case ORC_Q5_0:
@@ -1103,6 +1144,7 @@ static int linear_shape_ok(int dtype, size_t in_f) {
     case ORC_Q3_K:
     case ORC_IQ4_XS:
     case ORC_TQ2_0:
+    case ORC_TQ1_0:
     case ORC_Q6_K: return in_f % 256 == 0;
     case ORC_Q4_0:
     case ORC_Q4_1:
@@ -1201,7 +1243,7 @@ int orc_linear_int_stages(int dtype, const uint8_t *w, size_t wbytes, size_t w_n
     size_t row0 = w_off / in_f;
     if (row0 + out_f > total_rows) return -2;
     const uint8_t *wb = w + row0 * bpr;
-    size_t blocks = (dtype == ORC_Q4_K || dtype == ORC_Q5_K || dtype == ORC_Q6_K || dtype == ORC_Q2_K || dtype == ORC_Q3_K || dtype == ORC_IQ4_XS || dtype == ORC_TQ2_0) ? in_f / 256 : (dtype == ORC_NVFP4 ? in_f / 16 : in_f / 32);
+    size_t blocks = (dtype == ORC_Q4_K || dtype == ORC_Q5_K || dtype == ORC_Q6_K || dtype == ORC_Q2_K || dtype == ORC_Q3_K || dtype == ORC_IQ4_XS || dtype == ORC_TQ2_0 || dtype == ORC_TQ1_0) ? in_f / 256 : (dtype == ORC_NVFP4 ? in_f / 16 : in_f / 32);
     acts_t a;
     acts_build(dtype, x, m, in_f, &a);
 #pragma omp parallel for schedule(dynamic, 8)
@@ -1555,6 +1597,7 @@ size_t orc_synth_weight(int dtype, size_t n_elem, uint32_t seed, uint8_t *out) {
             break;
         case ORC_Q3_K: put_f16(blk + 108, 0.03f); break; /* d@108 (decode_spec.rs:325) */
         case ORC_IQ4_XS: put_f16(blk, 0.06f); break;      /* d@0 (decode_spec.rs:351) */
+        case ORC_TQ1_0: put_f16(blk + 52, 0.05f); break;  /* d@52 (decode_spec.rs:354) */
         case ORC_TQ2_0: put_f16(blk + 64, 0.05f); break;  /* d@64 (decode_spec.rs:356) */
         case ORC_MXFP4: blk[0] = 125; break;              /* E8M0 nearest 0.25 in log space: 2^(125 - 127) (decode_spec.rs:191, 216-219) */
         case ORC_NVFP4:                                   /* UE4M3 nearest 0.5 * (0.625 + 0.125 i) (decode_spec.rs:192-198, 223-245) */

@@ -29,6 +29,9 @@
  *                                 hand blocks (each shift position, the hmask bit, a split scale
  *                                 field); independent numpy decoders bit for bit; int64 brute-force
  *                                 stages; per-superblock f32 terms re-evaluated in numpy f32
+ *   TQ1_0 (dequant, orc_tq1_0_digit, orc_vec_dot_tq1_0)
+ *                                 the reference's tq1_0_single_block known answer; all 243 five-digit
+ *                                 strings packed by the format's rule come back; the element order
  *   TQ2_0 / MXFP4 / NVFP4 (dequant, orc_vec_dot_tq2_0, orc_vec_dot_mxfp4, orc_vec_dot_nvfp4, scale decoders)
  *                                 the reference's three single-block known answers; every E8M0 and
  *                                 UE4M3 byte against its definition; hand blocks; the rest as above
@@ -69,6 +72,7 @@ enum {
     ORC_Q2_K = 10,
     ORC_Q3_K = 11,
     ORC_IQ4_XS = 23,
+    ORC_TQ1_0 = 34,
     ORC_TQ2_0 = 35,
     ORC_MXFP4 = 39,
     ORC_NVFP4 = 40,
@@ -136,6 +140,9 @@ float orc_vec_dot_q3k(const uint8_t *row, const int8_t *qs, const float *d, cons
 /* IQ4_XS: kernels.rs:1008-1036 (vec_dot_iq4xs_scalar), scale by kernels.rs:995-1002 - isum[nb]. */
 float orc_vec_dot_iq4xs(const uint8_t *row, const int8_t *qs, const float *d, size_t in_f, int32_t *isum_out);
 int orc_iq4xs_scale(uint32_t scales_h, const uint8_t *scales_l, int ib);
+/* TQ1_0: kernels.rs:3167-3240 (tq1_0_expand_row + vec_dot_tq1_0) - iprod[nb]; digit of element i of a block. */
+float orc_vec_dot_tq1_0(const uint8_t *row, const int8_t *qs, const float *d, size_t in_f, int32_t *iprod_out);
+int orc_tq1_0_digit(const uint8_t *blk, int i);
 /* TQ2_0: kernels.rs:3066-3126 (tq2_0_expand_row + vec_dot_tq2_0) - iprod[nb]. */
 float orc_vec_dot_tq2_0(const uint8_t *row, const int8_t *qs, const float *d, size_t in_f, int32_t *iprod_out);
 /* MXFP4: kernels.rs:6303-6327 - iprod[in_f/32]; NVFP4: kernels.rs:6472-6500 - iprod[in_f/16]. Both

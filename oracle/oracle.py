@@ -22,7 +22,7 @@ Q4_0, Q4_1, Q5_0, Q5_1, Q5_K, IQ4_NL = 2, 3, 6, 7, 13, 20
 Q2_K, Q3_K = 10, 11
 IQ4_XS = 23
 MXFP4, NVFP4 = 39, 40
-TQ2_0 = 35
+TQ1_0, TQ2_0 = 34, 35
 BF16 = 30
 KVALUES_IQ4NL = (-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113)
 ACTS_SUPER, ACTS_BLK32, ACTS_RAW = 0, 1, 2
@@ -76,6 +76,8 @@ _vd_q3k = _sig("orc_vec_dot_q3k", C.c_float, _u8p, _i8p, _f32p, _i32p, C.c_size_
 _q3k_scales = _sig("orc_q3k_scales", None, _u8p, C.POINTER(C.c_int16))
 _vd_iq4xs = _sig("orc_vec_dot_iq4xs", C.c_float, _u8p, _i8p, _f32p, C.c_size_t, _i32p)
 _iq4xs_scale = _sig("orc_iq4xs_scale", C.c_int, C.c_uint32, _u8p, C.c_int)
+_vd_tq1_0 = _sig("orc_vec_dot_tq1_0", C.c_float, _u8p, _i8p, _f32p, C.c_size_t, _i32p)
+_tq1_digit = _sig("orc_tq1_0_digit", C.c_int, _u8p, C.c_int)
 _vd_tq2_0 = _sig("orc_vec_dot_tq2_0", C.c_float, _u8p, _i8p, _f32p, C.c_size_t, _i32p)
 _vd_mxfp4 = _sig("orc_vec_dot_mxfp4", C.c_float, _u8p, _i8p, _f32p, C.c_size_t, _i32p)
 _vd_nvfp4 = _sig("orc_vec_dot_nvfp4", C.c_float, _u8p, _i8p, _f32p, C.c_size_t, _i32p)
@@ -252,6 +254,17 @@ def vec_dot_iq4xs(row, q8: Q8, in_f: int, stages: bool = False):
     return (np.float32(y), isum) if stages else np.float32(y)
 
 
+def vec_dot_tq1_0(row, q8: Q8, in_f: int, stages: bool = False):
+    row = _c(row, np.uint8)
+    ip = np.empty(in_f // 256, np.int32) if stages else None
+    y = _vd_tq1_0(_p(row, _u8p), _p(q8.qs, _i8p), _p(q8.d, _f32p), in_f, _p(ip, _i32p))
+    return (np.float32(y), ip) if stages else np.float32(y)
+
+
+def tq1_0_digit(blk, i: int) -> int:
+    return int(_tq1_digit(_p(_c(blk, np.uint8), _u8p), i))
+
+
 def vec_dot_tq2_0(row, q8: Q8, in_f: int, stages: bool = False):
     row = _c(row, np.uint8)
     ip = np.empty(in_f // 256, np.int32) if stages else None
@@ -395,7 +408,7 @@ def linear_int_stages(dtype: int, w, x, m: int, in_f: int, out_f: int, *,
     if w_numel is None:
         e, b = block_layout(dtype)
         w_numel = w.size // b * e
-    blocks = in_f // 256 if dtype in (Q4_K, Q5_K, Q6_K, Q2_K, Q3_K, IQ4_XS, TQ2_0) else (in_f // 16 if dtype == NVFP4 else in_f // 32)
+    blocks = in_f // 256 if dtype in (Q4_K, Q5_K, Q6_K, Q2_K, Q3_K, IQ4_XS, TQ2_0, TQ1_0) else (in_f // 16 if dtype == NVFP4 else in_f // 32)
     a = np.empty((m, out_f, blocks), np.int32)
     b_ = np.empty((m, out_f, blocks), np.int32) if dtype in (Q4_K, Q5_K, Q2_K) else None
     rc = _linear_int(dtype, _p(w, _u8p), w.size, w_numel, w_off, _p(x, _f32p), m, in_f, out_f,

@@ -63,7 +63,7 @@ static void hip_linear_all_weight_quants_match_the_host_oracle(HipBackend& be) {
         const auto cases = weight_quant_cases(m, 256, 8);
         const SweepReport r = sweep_linear_on("hip Linear m=" + std::to_string(m), be, cases,
                                               [](const LinearCase&) { return CPU_INT8_ACT_TOL; });
-        EXPECT(r.cases.size() == 16, "expected the sixteen formats of this backend, got %zu", r.cases.size());
+        EXPECT(r.cases.size() == 17, "expected the seventeen formats of this backend, got %zu", r.cases.size());
         EXPECT(r.failures() == 0, "cases outside %.0e of the host decode oracle", CPU_INT8_ACT_TOL);
     }
 }
@@ -83,7 +83,7 @@ static void hip_linear_matches_the_cpu_production_arm(HipBackend& be) {
                 gate(what, got, want);
                 const bool ordered = c.dtype == DType::Q4K || c.dtype == DType::Q5K || c.dtype == DType::Q6K ||
                                      c.dtype == DType::Q2K || c.dtype == DType::Q3K || c.dtype == DType::IQ4XS ||
-                                     c.dtype == DType::TQ2_0;
+                                     c.dtype == DType::TQ2_0 || c.dtype == DType::TQ1_0;
                 if (ordered && m <= 8) EXPECT(same_bits(got, want), "%s: not bit-identical to infr-cpu", what);
             }
 }

@@ -150,7 +150,7 @@ inline const std::vector<RosterEntry>& weight_quants() {
     static const std::vector<RosterEntry> r = {
         {"Q4_0", 2}, {"Q4_1", 3}, {"Q5_0", 6}, {"Q5_1", 7}, {"Q8_0", 8}, {"Q2K", 10}, {"Q3K", 11}, {"Q4K", 12},
         {"Q5K", 13}, {"Q6K", 14}, {"Iq1S", -1}, {"Iq1M", -1}, {"Iq2Xxs", -1}, {"Iq2Xs", -1}, {"Iq2S", -1},
-        {"Iq3Xxs", -1}, {"Iq3S", -1}, {"Iq4Nl", 20}, {"Iq4Xs", 23}, {"Tq1_0", -1}, {"Tq2_0", 35}, {"Q2_0", 42},
+        {"Iq3Xxs", -1}, {"Iq3S", -1}, {"Iq4Nl", 20}, {"Iq4Xs", 23}, {"Tq1_0", 34}, {"Tq2_0", 35}, {"Q2_0", 42},
         {"Mxfp4", 39}, {"Nvfp4", 40}};
     return r;
 }

@@ -8,7 +8,7 @@ import pytest
 from oracle import oracle as orc
 
 FORMATS = [orc.F32, orc.F16, orc.BF16, orc.Q8_0, orc.Q4_0, orc.Q4_1, orc.Q5_0, orc.Q5_1, orc.Q4_K, orc.Q5_K,
-           orc.Q6_K, orc.IQ4_NL, orc.Q2_0, orc.Q2_K, orc.Q3_K, orc.IQ4_XS, orc.MXFP4, orc.NVFP4, orc.TQ2_0]
+           orc.Q6_K, orc.IQ4_NL, orc.Q2_0, orc.Q2_K, orc.Q3_K, orc.IQ4_XS, orc.MXFP4, orc.NVFP4, orc.TQ2_0, orc.TQ1_0]
 
 
 def table_bytes(dtype, rows, ne, seed):

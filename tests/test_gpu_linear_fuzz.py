@@ -21,9 +21,9 @@ pytestmark = pytest.mark.gpu
 
 FORMATS = (DType.Q4K, DType.Q5K, DType.Q6K, DType.Q8_0, DType.Q2_0, DType.Q4_0, DType.Q4_1, DType.Q5_0, DType.Q5_1,
            DType.IQ4NL, DType.F32, DType.F16, DType.BF16, DType.Q2K, DType.Q3K, DType.IQ4XS, DType.TQ2_0, DType.MXFP4,
-           DType.NVFP4)
+           DType.NVFP4, DType.TQ1_0)
 PLAIN = (DType.F32, DType.F16, DType.BF16)
-BIT_IDENTICAL = (DType.Q4K, DType.Q5K, DType.Q6K, DType.Q2K, DType.Q3K, DType.IQ4XS, DType.TQ2_0) + PLAIN
+BIT_IDENTICAL = (DType.Q4K, DType.Q5K, DType.Q6K, DType.Q2K, DType.Q3K, DType.IQ4XS, DType.TQ2_0, DType.TQ1_0) + PLAIN
 TOKENS = (1, 1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 24, 31, 32, 33, 40, 63, 64, 65, 66, 96, 127, 128, 129, 130, 200,
           255, 256, 257, 300)
 

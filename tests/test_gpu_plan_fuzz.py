@@ -26,7 +26,7 @@ pytestmark = pytest.mark.gpu
 WIDTHS = (256, 512, 1024)
 PER_WIDTH = 3
 LINEAR_DTYPES = (DType.Q4K, DType.Q4K, DType.Q6K, DType.Q8_0, DType.Q5_0, DType.Q2_0, DType.Q2K, DType.Q3K, DType.IQ4XS,
-                 DType.TQ2_0, DType.MXFP4, DType.NVFP4)
+                 DType.TQ2_0, DType.MXFP4, DType.NVFP4, DType.TQ1_0)
 MOE = dict(ne=512, n_expert=8, n_used=2, nff=256)
 
 

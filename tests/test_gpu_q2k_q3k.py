@@ -1,4 +1,4 @@
-"""GPU parity of Q2_K, Q3_K, IQ4_XS and TQ2_0 weights against the CPU oracle, through the C ABI: Op::Linear
+"""GPU parity of Q2_K, Q3_K, IQ4_XS, TQ2_0 and TQ1_0 weights against the CPU oracle, through the C ABI: Op::Linear
 (one token and batches), Op::EmbedGather tables and Op::MoeFfn expert banks.
 
 infr-cpu multiplies these formats with a per-256 int8 activation (crates/infr-cpu/src/lib.rs:1043-1124,
@@ -16,7 +16,7 @@ from tests.test_gpu_moe import check, run_moe
 
 pytestmark = pytest.mark.gpu
 
-BOTH = [DType.Q2K, DType.Q3K, DType.IQ4XS, DType.TQ2_0]
+BOTH = [DType.Q2K, DType.Q3K, DType.IQ4XS, DType.TQ2_0, DType.TQ1_0]
 ids = lambda d: DType(d).name
 
 
@@ -53,9 +53,9 @@ def test_int_stages_bit_exact(be, dtype, m):
 @pytest.mark.parametrize("m", [2, 5, 8, 9, 19, 40, 130])
 def test_batches_are_bit_identical_to_the_oracle(be, dtype, m):
     """Two tokens share one pass of the dot4 kernel over the weights; from three the 16-token K-split
-    MFMA kernel takes rows of two superblocks and more (an even number of them for Q3_K), 16 tokens
-    at a time; other rows keep the dot4 kernel, eight tokens per pass. Every token's value is the
-    one-token value."""
+    MFMA kernel takes rows of two superblocks and more (an even number of them for Q3_K and TQ2_0),
+    16 tokens at a time; other rows, and TQ1_0 at every token count, keep the dot4 kernel, eight
+    tokens per pass. Every token's value is the one-token value."""
     in_f, out_f = 1024, 96
     w = orc.synth_weight(dtype, in_f * out_f, 0x77 + m)
     x = synth_normal_f32(8 + m, m * in_f)
@@ -118,7 +118,7 @@ def test_a_plan_mixes_them_with_other_formats(be):
     groups by (format, in_f) and every output equals the single-op value."""
     in_f = 2048
     outs = [(DType.Q2K, 96), (DType.Q3K, 80), (DType.Q4K, 64), (DType.Q2K, 33), (DType.Q3K, 130), (DType.IQ4XS, 70),
-            (DType.IQ4XS, 9), (DType.TQ2_0, 45)]
+            (DType.IQ4XS, 9), (DType.TQ2_0, 45), (DType.TQ1_0, 77)]
     g = Graph()
     x = g.input(TensorDesc((1, in_f), DType.F32))
     ws, ys = [], []
@@ -148,7 +148,7 @@ def test_a_batch_plan_groups_them(be, m):
     quantized activation and one launch per (format, in_f) group."""
     in_f = 2048
     outs = [(DType.Q2K, 96), (DType.Q2K, 40), (DType.Q3K, 80), (DType.Q3K, 33), (DType.Q4K, 64), (DType.IQ4XS, 50),
-            (DType.IQ4XS, 31), (DType.TQ2_0, 45), (DType.TQ2_0, 8)]
+            (DType.IQ4XS, 31), (DType.TQ2_0, 45), (DType.TQ2_0, 8), (DType.TQ1_0, 21)]
     g = Graph()
     x = g.input(TensorDesc((m, in_f), DType.F32))
     ws, ys = [], []

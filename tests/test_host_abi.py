@@ -91,6 +91,16 @@ def test_synth_encoders_reproduce_their_input_distribution(dtype, tol):
     assert np.isfinite(f).all()
 
 
+def test_synth_tq1_0_digits_are_uniform():
+    from oracle import oracle as orc
+    w = infr_amd.synth_weight(B.DType.TQ1_0, 5, 16, 1024)
+    f = orc.dequant_block(orc.TQ1_0, w).reshape(-1, 256)
+    d = np.abs(f).max(axis=1, keepdims=True)
+    digits = np.rint(f / d).astype(int) + 1
+    assert set(np.unique(digits)) == {0, 1, 2}
+    assert all(abs((digits == v).mean() - 1 / 3) < 0.02 for v in (0, 1, 2))
+
+
 @pytest.mark.parametrize("dtype", [B.DType.Q2_0, B.DType.TQ2_0])
 def test_synth_ternary_codes(dtype):
     w = infr_amd.synth_weight(dtype, 5, 16, 1024)
