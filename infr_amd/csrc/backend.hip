@@ -1112,6 +1112,52 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
         return plan->ops[i].kind == INFR_OP_LINEAR && plan->ops[i].m == 1 &&
                !runs_alone(plan->ops[i].w_dtype, 1, plan->ops[i].in_f) && !self_alias(i);
     };
+    // pair_act[i] >= 0: Linear i is the gate projection of gated activation pair_act[i], evaluated by
+    // the workgroups that produce its operands; pair_up[i] is the up projection (i itself when one
+    // Linear writes [gate | up]) and pair_follower marks an up projection that rides in i's tiles.
+    std::vector<int> pair_act(n, -1), pair_up(n, -1);
+    std::vector<char> pair_follower(n, 0);
+    struct PairUndo {
+        size_t k, gate, up;
+        std::vector<Span> gate_wr;
+    };
+    std::vector<PairUndo> pairs;
+    // INFR_HIP_PAIR=0: gated activations go into their consumer's prologue only
+    static const int env_pair = getenv("INFR_HIP_PAIR") ? atoi(getenv("INFR_HIP_PAIR")) : 1;
+    auto try_pair = [&](size_t k) {
+        const auto& p = plan->ops[k];
+        const size_t nff = p.in_f;
+        const bool one = p.kind == INFR_OP_GATED_ACT_FUSED;
+        const float* G = ea[k].x;
+        const float* U = one ? ea[k].x + nff : ea[k].aux + p.up_off;
+        const std::vector<Span> gs{fspan(G, nff)}, us{fspan(U, nff)};
+        int ig = -1, iu = -1;  // the last writers of the two operands
+        for (size_t j = 0; j < k; ++j) {
+            if (any_overlap(wr[j], gs)) ig = (int)j;
+            if (any_overlap(wr[j], us)) iu = (int)j;
+        }
+        if (ig < 0 || iu < 0 || (ig == iu) != one) return false;
+        const auto &og = plan->ops[ig], &ou = plan->ops[iu];
+        if (!decode_linear(ig) || !decode_linear(iu) || absorbed[ig] || absorbed[iu]) return false;
+        if (pair_act[ig] >= 0 || pair_act[iu] >= 0 || pair_follower[ig] || pair_follower[iu]) return false;
+        if (static_cast<const float*>(bindings[og.dst]->ptr) != G || og.out_f != (one ? 2 * nff : nff)) return false;
+        if (!one && (static_cast<const float*>(bindings[ou.dst]->ptr) != U || ou.out_f != nff ||
+                     ou.w_dtype != og.w_dtype || ou.in_f != og.in_f || la[iu].bpr != la[ig].bpr ||
+                     bindings[ou.x]->ptr != bindings[og.x]->ptr || pre[iu] != pre[ig]))
+            return false;
+        if (pre[ig] >= 0 && plan->ops[pre[ig]].kind != INFR_OP_RMS_NORM) return false;
+        // dst is stored where the operands are produced: nothing from there up to the activation
+        // may touch it, and the producers' own inputs must not lie in it
+        for (size_t j = (size_t)std::min(ig, iu); j < k; ++j)
+            if (any_overlap(wr[j], wr[k]) || any_overlap(rd[j], wr[k])) return false;
+        pairs.push_back(PairUndo{k, (size_t)ig, (size_t)iu, wr[ig]});
+        pair_act[ig] = (int)k;
+        pair_up[ig] = iu;
+        if (!one) pair_follower[iu] = 1;
+        absorbed[k] = 1;
+        wr[ig].push_back(wr[k][0]);
+        return true;
+    };
     for (size_t k = 0; env_fuse && k < n; ++k) {
         const auto& p = plan->ops[k];
         const bool gated = (p.kind == INFR_OP_GATED_ACT && p.gate_block_width == 0) || p.kind == INFR_OP_GATED_ACT_FUSED;
@@ -1120,6 +1166,7 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
         // every workgroup of the consumer re-reads the producer's inputs while the first one
         // stores dst, so later workgroups would apply the op to its own result.
         if (any_overlap(wr[k], rd[k])) continue;
+        if (gated && env_pair && try_pair(k)) continue;
         // The definition's live range ends at the next op that overwrites dst (scratch tensors
         // are reused from layer to layer, graph.rs:10-14): readers beyond it see that op's value.
         // An op that overwrites only part of dst keeps the whole plan as the range.
@@ -1198,7 +1245,7 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
                              (pr.kind == INFR_OP_LINEAR && pr.m >= 2 && small_batch(pr) && !self_alias(i) &&
                               (size_t)pr.m * pr.out_f == n_add);
             const bool moe = pr.kind == INFR_OP_MOE_FFN && (size_t)pr.moe.rows * pr.moe.ne == n_add;
-            if ((!lin && !moe) || post[i] >= 0) continue;
+            if ((!lin && !moe) || post[i] >= 0 || pair_act[i] >= 0 || pair_follower[i]) continue;
             const float* pdst = static_cast<const float*>(bindings[pr.dst]->ptr);
             if (pdst != ea[k].x && pdst != ea[k].aux) continue;
             const bool resid_is_a = pdst == ea[k].aux;
@@ -1309,10 +1356,30 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
             f.users.clear();
             undone = true;
         }
+        // a pair's two projections share one launch: they must have come out on one level
+        for (auto& pr : pairs) {
+            if (pair_act[pr.gate] < 0 || level[pr.gate] == level[pr.up]) continue;
+            pair_act[pr.gate] = pair_up[pr.gate] = -1;
+            pair_follower[pr.up] = 0;
+            absorbed[pr.k] = 0;
+            wr[pr.gate] = pr.gate_wr;
+            undone = true;
+        }
         if (!undone) break;
     }
     auto fusion_of = [&](size_t k) {
         infr::GemvFusion f;
+        if (pair_act[k] >= 0) {
+            const auto& p = plan->ops[pair_act[k]];
+            const ElementwiseArgs& e = ea[pair_act[k]];
+            const bool one = (size_t)pair_up[k] == k;
+            f.pair_w = one ? la[k].wrows + (size_t)p.in_f * la[k].bpr : la[pair_up[k]].wrows;
+            f.pair_y = const_cast<float*>(one ? e.x + p.in_f : e.aux + p.up_off);
+            f.pair_dst = e.dst;
+            f.act = p.act;
+            f.has_clamp = p.has_clamp;
+            f.clamp = p.clamp;
+        }
         if (pre[k] >= 0) {
             const auto& p = plan->ops[pre[k]];
             const ElementwiseArgs& e = ea[pre[k]];
@@ -1327,7 +1394,9 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
                 f.has_clamp = p.has_clamp;
                 f.clamp = p.clamp;
             }
-            f.pre_dst = publishes[k] ? e.dst : nullptr;
+            // (a paired up projection that was to publish the vector hands that to its gate's tiles)
+            const bool pub = publishes[k] || (pair_act[k] >= 0 && publishes[pair_up[k]]);
+            f.pre_dst = pub ? e.dst : nullptr;
         }
         if (post[k] >= 0) {
             f.add_b = resid[k];
@@ -1453,10 +1522,13 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
                     (op.w_dtype == INFR_DTYPE_Q8_0 && (o2.in_f % 256 == 0) != (op.in_f % 256 == 0)))
                     continue;
                 taken[k] = 1;
+                if (pair_follower[k]) continue;  // its rows ride in the gate projection's tiles
                 // with an absorbed producer the GEMV starts from the producer's first input
                 const float* xsrc = pre[k] >= 0 ? ea[pre[k]].x : static_cast<const float*>(bindings[o2.x]->ptr);
+                // (one Linear onto [gate | up]: the op's rows are the gate half, the pair the other)
+                const size_t rows = pair_act[k] >= 0 && (size_t)pair_up[k] == k ? o2.out_f / 2 : o2.out_f;
                 plan->descs.push_back(infr::GemvOpDesc{la[k].wrows, xsrc, static_cast<float*>(bindings[o2.dst]->ptr),
-                                                       la[k].bpr, (int32_t)o2.out_f, fusion_of(k)});
+                                                       la[k].bpr, (int32_t)rows, fusion_of(k)});
             }
             st.n = (int)plan->descs.size() - st.first;
             if (!infr::plan_gemv_group(st.dtype, st.in_f, &plan->descs[st.first], st.n, &st.gp))

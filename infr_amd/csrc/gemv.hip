@@ -135,9 +135,10 @@ bool plan_gemv_group(int dtype, size_t in_f, const GemvOpDesc* ops, int n, GemvG
 }
 
 void fill_gemv_tiles(const GemvOpDesc* ops, int n, const GemvGroupPlan& plan, GemvTile* tiles) {
-    const int per_wg = plan.rows_per_wg;
     int t = 0;
-    for (int i = 0; i < n; ++i)
+    for (int i = 0; i < n; ++i) {
+        // a paired op's workgroup takes half of its rows from each of the two matrices
+        const int per_wg = ops[i].fus.pair_w ? plan.rows_per_wg / 2 : plan.rows_per_wg;
         for (int r = 0; r < ops[i].out_f; r += per_wg) {
             GemvTile& tl = tiles[t++];
             tl.w = ops[i].w + (size_t)r * ops[i].bpr;
@@ -150,14 +151,23 @@ void fill_gemv_tiles(const GemvOpDesc* ops, int n, const GemvGroupPlan& plan, Ge
                 tl.fus.add_b += r;
                 tl.fus.add_dst += r;
             }
+            if (tl.fus.pair_w) {
+                tl.fus.pair_w += (size_t)r * ops[i].bpr;
+                tl.fus.pair_y += r;
+                tl.fus.pair_dst += r;
+            }
             if (r != 0) tl.fus.pre_dst = nullptr;
         }
+    }
 }
 
 bool launch_gemv_fused(int dtype, size_t in_f, const GemvOpDesc* ops, int n, const GemvTile* tiles_dev,
                        const GemvGroupPlan& plan, hipStream_t stream) {
     if (n <= 0 || plan.total_wgs <= 0) return n == 0;
     if (n > 1 && tiles_dev == nullptr) return false;
+    for (int i = 0; i < n; ++i)  // paired ops need the table, and carry neither an Add nor a gated producer
+        if (ops[i].fus.pair_w && (tiles_dev == nullptr || ops[i].fus.add_dst || ops[i].fus.pre == 1 || ops[i].st_a))
+            return false;
     if (bpr_too_big(ops, n)) return false;
     const GemvFormatOps* f = format_ops(dtype, in_f);
     return f && f->fused && f->fused(in_f, ops[0], tiles_dev, plan, stream);

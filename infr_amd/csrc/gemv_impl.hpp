@@ -186,6 +186,9 @@ __global__ __launch_bounds__(512) void gemv_batch_ks_kernel(const uint8_t* __res
     }
 }
 
+// Rows per side of a paired tile at most (the workgroup keeps both sides' outputs in LDS).
+constexpr int kPairRows = 128;
+
 // act(gate) * up with the optional clamp, as Op::GatedAct evaluates one element
 // (gated_act_fn, crates/infr-cpu/src/kernels.rs:6591-6597).
 __device__ __forceinline__ float fused_gated_act(int act, bool has_clamp, float l, float gate, float up) {
@@ -246,9 +249,18 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, 
         }
         if (blockIdx.x != 0) tile.fus.pre_dst = nullptr;
     }
-    const int rpw = (tile.rows + NW - 1) / NW;
+    // A paired tile (workgroup-uniform): the second half of the waves takes the same rows of the up matrix.
+    const bool paired = tile.fus.pair_w != nullptr;
+    const bool second = paired && wave >= NW / 2;
+    const int side_waves = paired ? NW / 2 : NW;
+    const uint8_t* const wrows = second ? tile.fus.pair_w : tile.w;
+    float* const yrows = second ? tile.fus.pair_y : tile.y;
+    // the two halves' outputs, kept for the gated activation at the end (a side has at most kPairRows rows)
+    __shared__ float pair_out[2][kPairRows];
+    float* const pair_lds = paired ? pair_out[second ? 1 : 0] : nullptr;
+    const int rpw = (tile.rows + side_waves - 1) / side_waves;
     const int n_units = F::units(in_f);
-    const int row0 = wave * rpw;
+    const int row0 = (second ? wave - NW / 2 : wave) * rpw;
     const int row_end = min(row0 + rpw, tile.rows);
 
     int8_t* l_qs = reinterpret_cast<int8_t*>(lds);
@@ -291,14 +303,14 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, 
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) ok[t] = has_rows && F::valid(t, lane, n_units);
     // STREAMED: the image of this wave's rows starts at the line that holds their first byte
-    const uint8_t* span = tile.w + (size_t)row0 * tile.bpr;
+    const uint8_t* span = wrows + (size_t)row0 * tile.bpr;
     const uint32_t head = (uint32_t)(reinterpret_cast<uintptr_t>(span) & 127);
     const uint32_t total = has_rows ? (head + (uint32_t)(row_end - row0) * tile.bpr + 127) & ~127u : 0;
     typename std::conditional<STREAMED, RingChunk<ring_instr<F, STEPS, STREAMED>()>, int>::type chunks_ahead;
     if constexpr (STREAMED) {
         if (has_rows) ring_issue(span - head, 0, total, lane, chunks_ahead.v);  // (wave-uniform)
     }
-    else F::load_row(first[0], tile.w + (size_t)row0 * tile.bpr, 0, lane, ok[0]);
+    else F::load_row(first[0], wrows + (size_t)row0 * tile.bpr, 0, lane, ok[0]);
     // An absorbed producer of x (workgroup-uniform branch): every workgroup recomputes the vector
     // from the producer's inputs - cheaper than a launch of its own - and the op's first
     // workgroup stores it where the producer would have.
@@ -342,7 +354,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, 
     if constexpr (kFirstWhole && !STREAMED) {
         asm volatile("" ::: "memory");  // not before the loads above have been waited for
 #pragma unroll
-        for (int t = 1; t < STEPS; ++t) F::load_row(first[t], tile.w + (size_t)row0 * tile.bpr, t, lane, ok[t]);
+        for (int t = 1; t < STEPS; ++t) F::load_row(first[t], wrows + (size_t)row0 * tile.bpr, t, lane, ok[t]);
     }
 #pragma unroll
     for (int i = 0; i < kMaxChunks; ++i) {
@@ -352,7 +364,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, 
                                       l_bs, F::kPer32 ? nullptr : l_bs16);
     }
     __syncthreads();
-    if (!STREAMED && !has_rows) return;
+    if (!STREAMED && !has_rows && !paired) return;
 
     ActPtrs act{l_qs, l_d, l_bs, l_bs16};
     typename F::Acts acts[STEPS];
@@ -363,16 +375,27 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(GemvOpDesc single, 
     const StagePtrs st{STAGES ? single.st_a + st_off : nullptr, STAGES && single.st_b ? single.st_b + st_off : nullptr};
     if constexpr (STREAMED) {
         __syncthreads();  // the rings lie over the activation arrays
-        if (!has_rows) return;
+        if (!has_rows && !paired) return;
         float* osum = reinterpret_cast<float*>(lds + (size_t)NW * WeightRingOf<F, STEPS>::kBytes) +
                       wave * RowSumScratch<F, STEPS>::kFloatsPerWave;
-        gemv_rows_streamed<F, STEPS, STAGES>(span - head, head, total, tile.bpr, chunks_ahead,
-                                             lds + (size_t)wave * WeightRingOf<F, STEPS>::kBytes, acts, ok, tile.y, n_units,
-                                             row0, row_end, lane, st, osum, tile.fus.add_dst, add_first);
+        if (has_rows)
+            gemv_rows_streamed<F, STEPS, STAGES>(span - head, head, total, tile.bpr, chunks_ahead,
+                                                 lds + (size_t)wave * WeightRingOf<F, STEPS>::kBytes, acts, ok, yrows, n_units,
+                                                 row0, row_end, lane, st, osum, tile.fus.add_dst, add_first,
+                                                 pair_lds);
     } else {
         float* osum = reinterpret_cast<float*>(lds + in_f + in_f / 2) + wave * RowSumScratch<F, STEPS>::kFloatsPerWave;
-        gemv_rows<F, STEPS, STAGES, kFirstWhole>(tile.w, tile.bpr, first, acts, ok, tile.y, n_units, row0, row_end, lane,
-                                                 st, osum, tile.fus.add_b, tile.fus.add_dst, add_first);
+        if (has_rows)
+            gemv_rows<F, STEPS, STAGES, kFirstWhole>(wrows, tile.bpr, first, acts, ok, yrows, n_units, row0, row_end, lane,
+                                                     st, osum, tile.fus.add_b, tile.fus.add_dst, add_first, pair_lds);
+    }
+    if (paired) {
+        // Both halves' outputs of this tile are in LDS once every wave is here: one gated activation per row.
+        __syncthreads();
+        const bool hc = tile.fus.has_clamp != 0;
+        for (int i = (int)threadIdx.x; i < tile.rows; i += NW * 64)
+            gstore<float>(tile.fus.pair_dst + i,
+                          fused_gated_act(tile.fus.act, hc, tile.fus.clamp, pair_out[0][i], pair_out[1][i]));
     }
 }
 
@@ -532,8 +555,9 @@ template <typename F>
 static bool plan_group_fmt(size_t in_f, const GemvOpDesc* ops, int n, GemvGroupPlan* plan) {
     const int steps = (int)((in_f + F::kElemsPerStep - 1) / F::kElemsPerStep);
     if (steps < 1 || steps > 8) return false;
+    // (a paired op stands for the rows of two matrices: its workgroups take rows_per_wg / 2 of each)
     size_t total_rows = 0;
-    for (int i = 0; i < n; ++i) total_rows += (size_t)ops[i].out_f;
+    for (int i = 0; i < n; ++i) total_rows += (size_t)ops[i].out_f * (ops[i].fus.pair_w ? 2 : 1);
     // Every workgroup re-quantizes x (about the arithmetic of eleven weight rows at in_f 4096), so
     // big groups take up to 128 rows per workgroup (more than that loses to the uneven tail);
     // small ones keep at least ~512 workgroups in flight. The workgroup is always as wide as the register budget allows, so that the
@@ -560,7 +584,10 @@ static bool plan_group_fmt(size_t in_f, const GemvOpDesc* ops, int n, GemvGroupP
         fixed = std::max(fixed, ops[i].fus.pre == 1 ? 32.0 : (ops[i].fus.pre == 2 ? 15.0 : 11.0));
     auto wgs_at = [&](size_t r) {
         size_t w = 0;
-        for (int i = 0; i < n; ++i) w += ((size_t)ops[i].out_f + r - 1) / r;
+        for (int i = 0; i < n; ++i) {
+            const size_t per = ops[i].fus.pair_w ? r / 2 : r;
+            w += ((size_t)ops[i].out_f + per - 1) / per;
+        }
         return w;
     };
     if (resident > 0 && wgs_at(rows_per_wg) < (size_t)resident * 4) {
@@ -577,8 +604,7 @@ static bool plan_group_fmt(size_t in_f, const GemvOpDesc* ops, int n, GemvGroupP
         }
         rows_per_wg = best_r;
     }
-    int wg = 0;
-    for (int i = 0; i < n; ++i) wg += (int)(((size_t)ops[i].out_f + rows_per_wg - 1) / rows_per_wg);
+    int wg = (int)wgs_at(rows_per_wg);
     // A single round of workgroups: nothing else on the compute unit covers the prologue, so it is
     // spread over the widest workgroup that fits the registers (18.1 -> 15.4 us for a 4096 x 12288
     // Q4_K matrix behind an absorbed gated activation).
@@ -594,11 +620,12 @@ static bool plan_group_fmt(size_t in_f, const GemvOpDesc* ops, int n, GemvGroupP
         // its sweep runs at 5.3 TB/s so, 4.9 with 64)
         const size_t cap = std::max<size_t>(64, (size_t)147456 / std::max<size_t>(1, ops[0].bpr));
         rows_per_wg = std::min<size_t>(rows_per_wg, cap);
-        wg = 0;
-        for (int i = 0; i < n; ++i) wg += (int)(((size_t)ops[i].out_f + rows_per_wg - 1) / rows_per_wg);
+        wg = (int)wgs_at(rows_per_wg);
     }
     const size_t sum_scratch =
         (size_t)nw * (F::kOrdered ? 16 * (16 * steps + 4) : (F::kLaneSums ? LaneSums::kFloatsPerWave : 0)) * sizeof(float);
+    for (int i = 0; i < n; ++i)
+        if (ops[i].fus.pair_w && rows_per_wg / 2 > (size_t)kPairRows) return false;
     plan->total_wgs = wg;
     plan->waves_per_wg = nw;
     plan->rows_per_wg = (int)rows_per_wg;

@@ -94,7 +94,9 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
                                           const bool (&ok)[STEPS], float* __restrict__ y, int n_units,
                                           int row0, int row_end, int lane, const StagePtrs& st,
                                           float* osum, const float* add_b = nullptr,
-                                          float* add_dst = nullptr, float add_first = 0.0f) {
+                                          float* add_dst = nullptr, float add_first = 0.0f,
+                                          float* y_lds = nullptr) {
+    // y_lds: an LDS image of y (same row index) for a workgroup that reads its outputs back.
     // The residual of row r for an absorbed Add, from the lanes' prefetched values while
     // r - row0 < 64 (every lane of the wave must call this; `wanted` guards the late read).
     auto residual = [&](int r, bool wanted) {
@@ -135,6 +137,7 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
                         acc += v.w;
                     }
                     if (plain_y) gstore<float>(y + batch_row0 + lane, acc);
+                    if (y_lds) y_lds[batch_row0 + lane] = acc;
                     if (add_dst) gstore<float>(add_dst + batch_row0 + lane, acc + resid);
                 }
                 batch_row0 = row + 1;
@@ -155,6 +158,7 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
                         acc += v.w;
                     }
                     if (plain_y) gstore<float>(y + batch_row0 + lane, acc);
+                    if (y_lds) y_lds[batch_row0 + lane] = acc;
                     // an absorbed Op::Add: dst = a + b with a = this output
                     if (add_dst) gstore<float>(add_dst + batch_row0 + lane, acc + resid);
                 }
@@ -166,6 +170,7 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
             const float resid = add_dst ? residual(row, lane == 0) : 0.0f;
             if (lane == 0) {
                 if (plain_y) gstore<float>(y + row, s);
+                if (y_lds) y_lds[row] = s;
                 if (add_dst) gstore<float>(add_dst + row, s + resid);
             }
         } else {
@@ -183,6 +188,7 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
                 const float resid = add_dst ? residual(batch_row0 + lane, lane < in_batch) : 0.0f;
                 if (lane < in_batch) {
                     if (plain_y) gstore<float>(y + batch_row0 + lane, acc);
+                    if (y_lds) y_lds[batch_row0 + lane] = acc;
                     if (add_dst) gstore<float>(add_dst + batch_row0 + lane, acc + resid);
                 }
                 batch_row0 = row + 1;
@@ -343,7 +349,8 @@ __device__ __forceinline__ void gemv_rows_streamed(const uint8_t* origin, uint32
                                                    const typename F::Acts (&acts)[STEPS], const bool (&ok)[STEPS],
                                                    float* __restrict__ y, int n_units, int row0, int row_end,
                                                    int lane, const StagePtrs& st, float* osum,
-                                                   float* add_dst = nullptr, float add_first = 0.0f) {
+                                                   float* add_dst = nullptr, float add_first = 0.0f,
+                                                   float* y_lds = nullptr) {
     static_assert(F::kOrdered, "the streamed loop adds per-block terms in block order");
     // (a wave has at most 64 rows here: every residual is among the lanes' prefetched values, and
     // the loop holds no load but the chunks' - one more would be waited for together with them)
@@ -398,6 +405,7 @@ __device__ __forceinline__ void gemv_rows_streamed(const uint8_t* origin, uint32
                     acc += v.w;
                 }
                 if (plain_y) gstore<float>(y + batch_row0 + lane, acc);
+                if (y_lds) y_lds[batch_row0 + lane] = acc;
                 if (add_dst) gstore<float>(add_dst + batch_row0 + lane, acc + resid);
             }
             batch_row0 = row + 1;

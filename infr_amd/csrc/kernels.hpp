@@ -70,13 +70,20 @@ bool launch_gemv_batch(int dtype, const uint8_t* w, size_t bpr, const ActQ8& act
 //           (Op::RmsNorm), computed by every workgroup in its quantization prologue; the first
 //           workgroup of the op also stores that f32 vector to `pre_dst` (the absorbed op's dst)
 //   after:  add_dst[row] = y[row] + add_b[row] (Op::Add), next to the plain y store
+//   paired: the op is the gate projection of a gated activation whose up projection has the same
+//           shape and input; a workgroup computes the same rows of both matrices (half of its
+//           waves each) and then also stores pair_dst[row] = act(y[row]) * pair_y[row]
+//           (Op::GatedAct / GatedActFused evaluated where its operands are produced)
 struct GemvFusion {
     const float* x2 = nullptr;   // GatedAct: up; RmsNorm: weight
     float* pre_dst = nullptr;    // nullptr: computed but not stored
     const float* add_b = nullptr;
     float* add_dst = nullptr;    // nullptr: no Add
+    const uint8_t* pair_w = nullptr;  // first row of the up matrix; nullptr: not paired
+    float* pair_y = nullptr;          // the up projection's output
+    float* pair_dst = nullptr;        // the gated activation's output
     int32_t pre = 0;             // 0 none, 1 gated activation, 2 RmsNorm
-    int32_t act = 0;             // gated activation kind (0 SiLU, 1 GELU, 2 sigmoid)
+    int32_t act = 0;             // gated activation kind (0 SiLU, 1 GELU, 2 sigmoid), of pre == 1 or of the pair
     int32_t has_clamp = 0;
     float clamp = 0.0f;
     float eps = 0.0f;

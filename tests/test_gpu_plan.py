@@ -911,3 +911,149 @@ def test_streamed_decode_group_of_two_step_rows_behind_an_absorbed_gated_activat
         for i, yb in cases:
             y = be.download(yb, np.empty(rows_each[i], np.float32))
             assert np.array_equal(bits(y), bits(want[i]))
+
+
+def _gated_ffn(be, dt, H, FF, *, combined, up_first=False, act=0, clamp=None, norm=False, reader_between=False,
+               down_dt=None, seed=0):
+    """x [-> RmsNorm] -> gate / up (or one Linear onto [gate | up]) -> GatedAct -> down. Returns
+    (plan, run) where run(x) executes and returns every tensor of the chain from the device."""
+    from infr_amd import Add, GatedAct, GatedActFused, RmsNorm
+    down_dt = dt if down_dt is None else down_dt
+    g, binds, bufs, host = Graph(), Bindings(), {}, {}
+
+    def tensor(name, n, data=None):
+        t = g.output(TensorDesc((1, n), DType.F32)) if data is None else g.input(TensorDesc((1, n), DType.F32))
+        bufs[name] = be.upload_new(data) if data is not None else be.alloc(n * 4)
+        binds.bind(t, bufs[name])
+        return t
+
+    def weight(name, d, out_f, in_f, s):
+        host[name] = synth_weight(d, s, out_f, in_f, 0.05)
+        t = g.weight(TensorDesc((out_f, in_f), d))
+        binds.bind(t, be.upload_new(host[name]))
+        return t
+
+    x = tensor("x", H, np.zeros(H, np.float32))
+    h = x
+    if norm:
+        host["nw"] = synth_normal_f32(seed + 3, H) * np.float32(0.1) + np.float32(1.0)
+        nw = tensor("nw", H, host["nw"])
+        h = tensor("h", H)
+        g.push(RmsNorm(x, nw, h, 1, H, 1e-6))
+    a = tensor("act", FF)
+    if combined:
+        wgu, gu = weight("wgu", dt, 2 * FF, H, seed + 10), tensor("gu", 2 * FF)
+        g.push(Linear(h, wgu, gu, 1, H, 2 * FF))
+        g.push(GatedActFused(gu, a, 1, FF, act=act, swiglu_clamp=clamp))
+    else:
+        wg, wu = weight("wg", dt, FF, H, seed + 10), weight("wu", dt, FF, H, seed + 11)
+        gt, up = tensor("gate", FF), tensor("up", FF)
+        lin = [Linear(h, wg, gt, 1, H, FF), Linear(h, wu, up, 1, H, FF)]
+        for op in (reversed(lin) if up_first else lin):
+            g.push(op)
+        if reader_between:   # someone still reads the activation's dst after the projections
+            zero, cp = tensor("zero", FF, np.zeros(FF, np.float32)), tensor("copy", FF)
+            g.push(Add(a, zero, cp, FF))
+        g.push(GatedAct(gt, up, a, 1, FF, act=act, swiglu_clamp=clamp))
+    if FF % 256 == 0:    # (the narrow cases end at the activation)
+        wd, y = weight("wd", down_dt, H, FF, seed + 12), tensor("y", H)
+        g.push(Linear(a, wd, y, 1, FF, H))
+    plan = be.compile(g)
+
+    def run(xv, act_before=None):
+        be.upload(bufs["x"], xv)
+        if act_before is not None:
+            be.upload(bufs["act"], act_before)
+        be.execute(plan, binds)
+        return {nm: be.download(b, np.empty(b.len_bytes() // 4, np.float32)) for nm, b in bufs.items()}
+    return plan, run, host
+
+
+@pytest.mark.parametrize("dt", [DType.Q4K, DType.Q6K, DType.Q8_0, DType.Q4_0, DType.Q3K, DType.MXFP4],
+                         ids=lambda d: DType(d).name)
+@pytest.mark.parametrize("combined", [False, True])
+@pytest.mark.parametrize("H,FF", [(512, 100), (1024, 2816), (4096, 1000), (256, 4)])
+def test_gated_activation_is_evaluated_where_gate_and_up_are_produced(be, dt, combined, H, FF):
+    """Op::GatedAct / GatedActFused behind one-token gate and up projections of one shape: the
+    workgroups that produce a row of both also store act(gate) * up, so the chain is two launches
+    and the down projection (where the test has one) starts from the finished vector. Gate, up and the activation equal
+    what the ops give one by one: the projections bit for bit where the format's decode is
+    bit-identical, the activation within 1e-6 of the CPU's expf form."""
+    plan, run, host = _gated_ffn(be, dt, H, FF, combined=combined, norm=H >= 1024, seed=H + FF)
+    exact = dt in (DType.Q4K, DType.Q6K, DType.Q3K)
+    for rep in range(2):
+        xv = synth_normal_f32(50 + rep, H)
+        d = run(xv)
+        assert plan.launches() == (2 if "y" in d else 1), plan.launches()
+        h = d["h"] if "h" in d else xv
+        if "h" in d:
+            assert _rel(h, orc.rms_norm(xv, host["nw"], 1, H, 1e-6)) < 1e-6
+        if combined:
+            gu = orc.linear(dt, host["wgu"], h, 1, H, 2 * FF).ravel()
+            want_g, want_u, got_g, got_u = gu[:FF], gu[FF:], d["gu"][:FF], d["gu"][FF:]
+        else:
+            want_g = orc.linear(dt, host["wg"], h, 1, H, FF).ravel()
+            want_u = orc.linear(dt, host["wu"], h, 1, H, FF).ravel()
+            got_g, got_u = d["gate"], d["up"]
+        if exact and "h" not in d:
+            assert np.array_equal(bits(got_g), bits(want_g)) and np.array_equal(bits(got_u), bits(want_u))
+        else:
+            assert _rel(got_g, want_g) < 1e-4 and _rel(got_u, want_u) < 1e-4
+        assert _rel(d["act"], orc.gated_act(got_g, got_u, 1, FF)) < 1e-6
+        if "y" not in d:
+            continue
+        y_want = orc.linear(dt, host["wd"], d["act"], 1, FF, H).ravel()
+        if exact:
+            assert np.array_equal(bits(d["y"]), bits(y_want))       # down sees the stored vector itself
+        else:
+            assert _rel(d["y"], y_want) < 1e-4
+
+
+@pytest.mark.parametrize("act,clamp", [(1, None), (2, None), (0, 0.75), (1, 1.5)])
+def test_paired_gated_activation_kinds_and_clamp(be, act, clamp):
+    """GELU, sigmoid and the clamped forms through the paired launch, with the up projection first
+    in program order behind an absorbed RmsNorm (whose vector the pair's tiles must still store)."""
+    H, FF = 1024, 1536
+    plan, run, host = _gated_ffn(be, DType.Q4K, H, FF, combined=False, up_first=True, act=act, clamp=clamp, norm=True,
+                                 down_dt=DType.Q6K, seed=7)
+    xv = synth_normal_f32(61, H) * np.float32(3.0)
+    d = run(xv)
+    assert plan.launches() == 2
+    assert _rel(d["h"], orc.rms_norm(xv, host["nw"], 1, H, 1e-6)) < 1e-6
+    assert _rel(d["gate"], orc.linear(DType.Q4K, host["wg"], d["h"], 1, H, FF)) < 1e-4
+    assert _rel(d["act"], orc.gated_act(d["gate"], d["up"], 1, FF, act, clamp=clamp)) < 1e-6
+    assert np.array_equal(bits(d["y"]), bits(orc.linear(DType.Q6K, host["wd"], d["act"], 1, FF, H).ravel()))
+
+
+def test_pairing_is_refused_when_the_activations_dst_is_still_read(be):
+    """An op between the projections and the GatedAct reads the activation's dst (its previous
+    contents): the activation may not be stored early, and it goes into the down projection's
+    prologue instead."""
+    H, FF = 512, 768
+    plan, run, host = _gated_ffn(be, DType.Q4K, H, FF, combined=False, reader_between=True, seed=9)
+    before = synth_normal_f32(71, FF)
+    d = run(synth_normal_f32(70, H), act_before=before)
+    assert np.array_equal(bits(d["copy"]), bits(before))            # the reader saw the old contents
+    assert _rel(d["act"], orc.gated_act(d["gate"], d["up"], 1, FF)) < 1e-6
+    assert _rel(d["y"], orc.linear(DType.Q4K, host["wd"], d["act"], 1, FF, H)) < 1e-4
+
+
+@pytest.mark.parametrize("combined", [False, True])
+@pytest.mark.parametrize("H", [1024, 5120])
+def test_paired_gated_activation_in_a_many_round_group(be, combined, H):
+    """66,000 gate rows and as many up rows: the group is many rounds of workgroups, whose rows go
+    through the per-wave LDS rings; a paired tile's two wave sets stream their own matrix each."""
+    FF = 66000
+    plan, run, host = _gated_ffn(be, DType.Q4K, H, FF, combined=combined, seed=31)
+    xv = synth_normal_f32(90, H)
+    d = run(xv)
+    assert plan.launches() == 1
+    if combined:
+        gu = orc.linear(DType.Q4K, host["wgu"], xv, 1, H, 2 * FF).ravel()
+        want_g, want_u, got_g, got_u = gu[:FF], gu[FF:], d["gu"][:FF], d["gu"][FF:]
+    else:
+        want_g = orc.linear(DType.Q4K, host["wg"], xv, 1, H, FF).ravel()
+        want_u = orc.linear(DType.Q4K, host["wu"], xv, 1, H, FF).ravel()
+        got_g, got_u = d["gate"], d["up"]
+    assert np.array_equal(bits(got_g), bits(want_g)) and np.array_equal(bits(got_u), bits(want_u))
+    assert _rel(d["act"], orc.gated_act(got_g, got_u, 1, FF)) < 1e-6
