@@ -54,7 +54,8 @@ def random_program(rng, n_ops):
 
     while len(prog) < n_ops:
         kind = rng.choice(["linear", "norm", "add", "gated", "norm_add", "moe",
-                           "norm>linears", "gated>linear", "linear>add", "moe>add", "norm>moe>add", "layer"])
+                           "norm>linears", "gated>linear", "linear>add", "moe>add", "norm>moe>add", "layer",
+                           "gate/up>gated"])
         if kind == "linear":
             prog.append(linear(t(width()), t(width())))          # equal widths may pick dst == x
         elif kind in ("norm", "norm_add"):
@@ -92,6 +93,19 @@ def random_program(rng, n_ops):
             prog.append(("norm", t(MOE["ne"]), h, int(rng.integers(2))))
             prog.append(("moe", h, y, int(rng.integers(2))))
             prog.append(add_behind(y))
+        elif kind == "gate/up>gated":
+            # two projections of one format over one input, sometimes an op in between, then the
+            # gated activation of their outputs; the tensors may collide in every way
+            w, ff = width(), width()
+            h, g, u, a = t(w), t(ff), t(ff), t(ff)
+            lg = linear(h, g)
+            lu = ("linear", h, u, lg[3], int(rng.integers(4)))
+            prog += [lu, lg] if rng.integers(2) else [lg, lu]
+            if rng.integers(3) == 0:
+                prog.append(("add", t(ff), t(ff), t(ff)))
+            prog.append(("gated", g, u, a))
+            if rng.integers(2):
+                prog.append(linear(a, t(width())))
         else:  # norm -> two projections -> gated -> down -> residual add
             w, ff = width(), width()
             x, h, g, u, a, y = t(w), t(w), t(ff), t(ff), t(ff), t(w)
@@ -181,7 +195,7 @@ def describe(prog):
     return "\n".join(f"  {i:2d}: {op}" for i, op in enumerate(prog))
 
 
-@pytest.mark.parametrize("m,seed", [(1, s) for s in range(24)] + [(3, s) for s in range(100, 108)] +
+@pytest.mark.parametrize("m,seed", [(1, s) for s in range(160)] + [(3, s) for s in range(100, 108)] +
                          [(8, s) for s in range(200, 204)] + [(20, s) for s in range(300, 303)] +
                          [(48, s) for s in range(400, 402)])
 def test_scheduled_plan_equals_the_ops_run_one_by_one(be, m, seed):
