@@ -39,6 +39,7 @@ struct infr_hip_plan {
         int dtype = 0;            // group
         size_t in_f = 0;
         size_t m = 1;             // 1: decode group; 2..32: small-batch group
+        bool f32act = false;      // decode group of the f32-activation kernel (Q5_0 at one token)
         int first = 0, n = 0;     // slice of descs
         size_t tile_first = 0;    // slice of tiles (decode) / btiles (small batch)
         infr::GemvGroupPlan gp;
@@ -1506,6 +1507,53 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
                 plan->steps.push_back(st);
                 continue;
             }
+            // One token of a format that multiplies f32 activations: the level's ops of one row
+            // length share a launch (no absorbed neighbours: decode_linear() excludes them).
+            auto f32act_op = [&](size_t k) {
+                const auto& o2 = plan->ops[k];
+                return o2.kind == INFR_OP_LINEAR && o2.m == 1 && infr::gemv_takes_f32_activations(o2.w_dtype, 1) &&
+                       infr::gemv_f32act_groups(o2.w_dtype, o2.in_f) && !self_alias(k);
+            };
+            if (f32act_op(i)) {
+                st.dtype = op.w_dtype;
+                st.in_f = op.in_f;
+                st.f32act = true;
+                st.first = (int)plan->descs.size();
+                size_t total_rows = 0;
+                for (size_t k = i; k < n; ++k) {
+                    const auto& o2 = plan->ops[k];
+                    if (level[k] != lv || taken[k] || absorbed[k] || !f32act_op(k) || o2.w_dtype != op.w_dtype ||
+                        o2.in_f != op.in_f || la[k].bpr > 0xFFFFFFFFull)
+                        continue;
+                    taken[k] = 1;
+                    plan->descs.push_back(infr::GemvOpDesc{la[k].wrows, static_cast<const float*>(bindings[o2.x]->ptr),
+                                                           static_cast<float*>(bindings[o2.dst]->ptr), la[k].bpr,
+                                                           (int32_t)o2.out_f, infr::GemvFusion{}});
+                    total_rows += o2.out_f;
+                }
+                st.n = (int)plan->descs.size() - st.first;
+                if (st.n > 0) {
+                    st.gp.rows_per_wg = infr::gemv_f32act_group_rows(total_rows, op.in_f);
+                    st.tile_first = plan->tiles.size();
+                    for (int q = st.first; q < st.first + st.n; ++q) {
+                        const auto& d = plan->descs[q];
+                        for (int r = 0; r < d.out_f; r += st.gp.rows_per_wg) {
+                            infr::GemvTile tl{};
+                            tl.w = d.w + (size_t)r * d.bpr;
+                            tl.x = d.x;
+                            tl.y = d.y + r;
+                            tl.bpr = (uint32_t)d.bpr;
+                            tl.rows = std::min(st.gp.rows_per_wg, d.out_f - r);
+                            plan->tiles.push_back(tl);
+                        }
+                    }
+                    st.gp.total_wgs = (int)(plan->tiles.size() - st.tile_first);
+                    plan->steps.push_back(st);
+                    continue;
+                }
+                st = infr_hip_plan::Step{};   // (a row too long for the table: the op runs alone below)
+                st.level = lv;
+            }
             if (op.kind != INFR_OP_LINEAR || op.m != 1 || runs_alone(op.w_dtype, op.m, op.in_f) || self_alias(i)) {
                 st.op = (int)i;
                 taken[i] = 1;
@@ -1617,6 +1665,11 @@ static int enqueue_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t
             else if (!infr::launch_gemv_batch_group(st.dtype, st.m, st.in_f, plan->btiles_dev + st.tile_first,
                                                     st.bp, be->act, be->stream))
                 return fail(be, INFR_HIP_ERR_UNSUPPORTED, "execute: small-batch launch rejected");
+            HIP_TRY(be, hipGetLastError());
+        } else if (st.f32act) {
+            if (!infr::launch_gemv_f32act_group(st.dtype, st.in_f, plan->tiles_dev + st.tile_first, st.gp.total_wgs,
+                                                be->stream))
+                return fail(be, INFR_HIP_ERR_UNSUPPORTED, "execute: f32-activation decode launch rejected");
             HIP_TRY(be, hipGetLastError());
         } else {
             if (!infr::launch_gemv_fused(st.dtype, st.in_f, &plan->descs[st.first], st.n,

@@ -198,6 +198,11 @@ inline bool act_is_per32(int dtype, size_t in_f) {
 bool gemv_takes_f32_activations(int dtype, size_t m);
 bool launch_gemv_f32act(int dtype, const uint8_t* w, size_t bpr, const float* x, float* y, size_t in_f,
                         size_t out_f, hipStream_t stream);
+// Plans: the one-token Linears of a level that take this kernel and share (dtype, in_f) run as one
+// launch over a tile table (GemvTile: w, x, y, bpr, rows; no fusion fields are read).
+bool gemv_f32act_groups(int dtype, size_t in_f);
+int gemv_f32act_group_rows(size_t total_rows, size_t in_f);
+bool launch_gemv_f32act_group(int dtype, size_t in_f, const GemvTile* tiles_dev, int n_tiles, hipStream_t stream);
 
 // Op::EmbedGather: dst[r, :] = decode(table[ids[r], :]) * scale, rows decoded from the raw blocks.
 bool embed_gather_supported(int dtype);

@@ -301,3 +301,49 @@ def test_prefill_mfma_rows_that_are_not_whole_256s(be, dtype):
     oa, _ = orc.linear_int_stages(dtype, w, x, m, in_f, out_f)
     assert np.array_equal(a, oa)
     gate(run_linear(be, dtype, w, x, m, in_f, out_f), orc.linear(dtype, w, x, m, in_f, out_f))
+
+
+def test_q5_0_one_token_linears_of_a_level_share_a_launch(be):
+    """One-token Q5_0 Linears multiply f32 activations (no int8 arm on the CPU): inside a plan the
+    ops of a level run as one launch per row length - sixteen-wave workgroups from 8192 columns -
+    over distinct activations, ragged row counts and a w_off slice, each within 1e-4 of decode + dot;
+    a second level reads the first one's output."""
+    spec = [(4096, 100, "x0"), (4096, 37, "x0"), (4096, 1, "x1"), (12288, 130, "x2"), (12288, 16, "x2"),
+            (256, 9, "x3"), (13824, 21, "x4")]
+    g, binds = Graph(), Bindings()
+    xs, host = {}, {}
+    for name, n in (("x0", 4096), ("x1", 4096), ("x2", 12288), ("x3", 256), ("x4", 13824)):
+        xs[name] = g.input(TensorDesc((1, n), DType.F32))
+        host[name] = synth_normal_f32(len(xs) + 500, n)
+        binds.bind(xs[name], be.upload_new(host[name]))
+    outs = []
+    for i, (in_f, out_f, xn) in enumerate(spec):
+        rows = out_f + 5                                  # the op takes rows 3 .. 3 + out_f of a taller weight
+        w = synth_weight(DType.Q5_0, 300 + i, rows, in_f)
+        wid = g.weight(TensorDesc((rows, in_f), DType.Q5_0))
+        binds.bind(wid, be.upload_new(w))
+        y = g.output(TensorDesc((1, out_f), DType.F32))
+        yb = be.alloc(out_f * 4)
+        binds.bind(y, yb)
+        g.push(Linear(xs[xn], wid, y, 1, in_f, out_f, w_off=3 * in_f))
+        outs.append((w, in_f, out_f, xn, yb, rows, y))
+    # and a chain over two levels: x3 -> [256 x 256] -> [64 x 256]
+    w1, w2 = synth_weight(DType.Q5_0, 400, 256, 256), synth_weight(DType.Q5_0, 401, 64, 256)
+    a, b = g.weight(TensorDesc((256, 256), DType.Q5_0)), g.weight(TensorDesc((64, 256), DType.Q5_0))
+    binds.bind(a, be.upload_new(w1)).bind(b, be.upload_new(w2))
+    h, z = g.output(TensorDesc((1, 256), DType.F32)), g.output(TensorDesc((1, 64), DType.F32))
+    hb, zb = be.alloc(256 * 4), be.alloc(64 * 4)
+    binds.bind(h, hb).bind(z, zb)
+    g.push(Linear(xs["x3"], a, h, 1, 256, 256))
+    g.push(Linear(h, b, z, 1, 256, 64))
+    plan = be.compile(g)
+    for rep in range(2):
+        be.execute(plan, binds)
+        assert plan.launches() == 5, plan.launches()      # 4096, 12288, 256, 13824 on the first level; 256 on the second
+        for w, in_f, out_f, xn, yb, rows, _ in outs:
+            got = be.download(yb, np.empty((1, out_f), np.float32))
+            gate(got, orc.linear(DType.Q5_0, w, host[xn], 1, in_f, out_f, w_numel=rows * in_f, w_off=3 * in_f,
+                                 reference_mode=True))
+        hv = be.download(hb, np.empty((1, 256), np.float32))
+        gate(hv, orc.linear(DType.Q5_0, w1, host["x3"], 1, 256, 256, reference_mode=True))
+        gate(be.download(zb, np.empty((1, 64), np.float32)), orc.linear(DType.Q5_0, w2, hv, 1, 256, 64, reference_mode=True))
