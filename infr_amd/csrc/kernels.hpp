@@ -325,6 +325,9 @@ void launch_mmq_shared_q8_0(const uint8_t* w, size_t bpr, const ActQ8& act, floa
 // The same for Q5_K; st.a / st.b receive sd / sm per (token, row, 256-block).
 void launch_mmq_shared_q5k(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
                            size_t out_f, const IntStages& st, hipStream_t stream);
+// The same for IQ4_XS; st.a receives isum per (token, row, 256-block).
+void launch_mmq_shared_iq4xs(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
+                             size_t out_f, const IntStages& st, hipStream_t stream);
 // The same for Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL (and Q2_0: transposed16 activations) rows that are whole
 // 256s, against the per-32 activation in the tiled order (launch_quantize_q8_32_tiled); st.a receives
 // iprod per (token, row, 32-element block).

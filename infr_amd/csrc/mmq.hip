@@ -1508,6 +1508,10 @@ static bool skinny16_shape(int dtype, int nb, size_t m, size_t out_f) {
         return false;
     if (nb < kSkinny16Blocks || (nb % kSkinny16Blocks != 0 && (dtype == 14 || dtype == 42 || dtype == 11 || dtype == 35))) return false;
     // Q2_K, Q3_K, IQ4_XS, TQ2_0: the dot4 batches are the only other kernel, eight tokens per pass over the weights
+    // IQ4_XS has a 128-token tile kernel whose time is flat up to 128 tokens (30 / 59 / 22 us at 12288 x 4096,
+    // 4096 x 12288, 4096 x 4096) where a 16-token pass here costs 8.2 / 8.0 / 2.8: it takes over at 49 tokens
+    // on large matrices of 4096-column rows, at 113 on long rows and small matrices
+    if (dtype == 23 && m > 16) return m <= ((out_f == 0 || out_f * (size_t)nb <= (size_t)4096 * 16 || nb >= 32) ? 112u : 48u);
     if (dtype == 10 || dtype == 11 || dtype == 23 || dtype == 35) return m >= 3;
     if (m <= 16) {
         // the dot4 batch kernels, which unpack a weight once per two or four tokens, stay ahead at the
@@ -1736,6 +1740,11 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
     if (dtype == 13 && (m >= 33 || long_row)) {
         quantize_tiled();
         launch_mmq_shared_q5k(w, bpr, act, y, m, in_f, out_f, st, stream);
+        return true;
+    }
+    if (dtype == 23 && in_f % 256 == 0 && (m >= 17 || long_row)) {  // (what the 16-token kernel left: 49 / 113 tokens and up)
+        quantize_tiled();
+        launch_mmq_shared_iq4xs(w, bpr, act, y, m, in_f, out_f, st, stream);
         return true;
     }
     // (their kernel's flat time up to 128 tokens, ~145 us at 4096 x 12288, meets the dot4 batches'
