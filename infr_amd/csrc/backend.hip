@@ -40,6 +40,8 @@ struct infr_hip_plan {
         size_t in_f = 0;
         size_t m = 1;             // 1: decode group; 2..32: small-batch group
         bool f32act = false;      // decode group of the f32-activation kernel (Q5_0 at one token)
+        bool strips = false;      // prefill group: Q4_K Linears over one activation tensor, one strip launch
+        const float* x = nullptr; // strips: the shared activation tensor
         int first = 0, n = 0;     // slice of descs
         size_t tile_first = 0;    // slice of tiles (decode) / btiles (small batch)
         infr::GemvGroupPlan gp;
@@ -58,6 +60,10 @@ struct infr_hip_plan {
     std::vector<infr::GemvTile> tiles;
     infr::GemvTile* tiles_dev = nullptr;
     size_t tiles_cap = 0;
+    // prefill strip groups: one entry per strip (tile_first per step)
+    std::vector<infr::StripSeg> ssegs;
+    infr::StripSeg* ssegs_dev = nullptr;
+    size_t ssegs_cap = 0;
     // small-batch groups: quantizer and GEMM tile tables
     std::vector<infr::QuantTile> qtiles;
     std::vector<infr::BatchTile> btiles;
@@ -1021,6 +1027,7 @@ void infr_hip_plan_free(infr_hip_t* be, infr_hip_plan_t* plan) {
     if (be && be->stream) (void)hipStreamSynchronize(be->stream);
     if (plan->exec) (void)hipGraphExecDestroy(plan->exec);
     if (plan->tiles_dev) (void)hipFree(plan->tiles_dev);
+    if (plan->ssegs_dev) (void)hipFree(plan->ssegs_dev);
     if (plan->qtiles_dev) (void)hipFree(plan->qtiles_dev);
     if (plan->btiles_dev) (void)hipFree(plan->btiles_dev);
     delete plan;
@@ -1408,6 +1415,7 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
     plan->steps.clear();
     plan->descs.clear();
     plan->tiles.clear();
+    plan->ssegs.clear();
     plan->qtiles.clear();
     plan->btiles.clear();
     for (int lv = 0; lv <= max_level; ++lv) {
@@ -1417,6 +1425,46 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
             const auto& op = plan->ops[i];
             infr_hip_plan::Step st;
             st.level = lv;
+            // Q4_K Linears of a prefill chunk that read one activation tensor (q / k / v, gate / up):
+            // one quantization and one strip launch over all their rows, so that a narrow projection
+            // (k, v) shares the grid instead of running on a fraction of the machine.
+            auto strip_op = [&](size_t k) {
+                const auto& o2 = plan->ops[k];
+                return o2.kind == INFR_OP_LINEAR && o2.w_dtype == INFR_DTYPE_Q4_K && o2.m == op.m && o2.in_f == op.in_f &&
+                       bindings[o2.x]->ptr == bindings[op.x]->ptr && !self_alias(k) && la[k].bpr == la[i].bpr;
+            };
+            if (op.kind == INFR_OP_LINEAR && op.w_dtype == INFR_DTYPE_Q4_K && op.m >= 128 && !self_alias(i)) {
+                size_t total = 0, count = 0;
+                for (size_t k = i; k < n; ++k)
+                    if (level[k] == lv && !taken[k] && !absorbed[k] && strip_op(k)) total += plan->ops[k].out_f, ++count;
+                if (count >= 2 && infr::mmq_q4k_strip_group_takes(op.m, op.in_f, total)) {
+                    st.dtype = op.w_dtype;
+                    st.in_f = op.in_f;
+                    st.m = op.m;
+                    st.strips = true;
+                    st.x = static_cast<const float*>(bindings[op.x]->ptr);
+                    st.first = (int)plan->descs.size();
+                    const int tiles = infr::mmq_strip_q4k_tiles(op.m, total, op.in_f, be->props.multiProcessorCount);
+                    const int rows = infr::mmq_strip_q4k_rows(tiles);
+                    st.gp.rows_per_wg = tiles;
+                    st.tile_first = plan->ssegs.size();
+                    for (size_t k = i; k < n; ++k) {
+                        if (level[k] != lv || taken[k] || absorbed[k] || !strip_op(k)) continue;
+                        taken[k] = 1;
+                        const auto& o2 = plan->ops[k];
+                        float* yk = static_cast<float*>(bindings[o2.dst]->ptr);
+                        plan->descs.push_back(infr::GemvOpDesc{la[k].wrows, st.x, yk, la[k].bpr, (int32_t)o2.out_f,
+                                                               infr::GemvFusion{}});
+                        for (size_t r = 0; r < o2.out_f; r += (size_t)rows)
+                            plan->ssegs.push_back(infr::StripSeg{la[k].wrows + r * la[k].bpr, yk + r, (int32_t)o2.out_f,
+                                                                 (int32_t)std::min<size_t>((size_t)rows, o2.out_f - r)});
+                    }
+                    st.n = (int)plan->descs.size() - st.first;
+                    st.gp.total_wgs = (int)(plan->ssegs.size() - st.tile_first);
+                    plan->steps.push_back(st);
+                    continue;
+                }
+            }
             if (op.kind == INFR_OP_LINEAR && small_batch(op)) {
                 // small-batch group: same (dtype, in_f, m) in this level -> one quantize launch over
                 // the distinct activation tensors + one GEMM launch over a tile table
@@ -1590,6 +1638,7 @@ static int schedule_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_
         }
     }
     if (int rc = upload_table(be, plan->tiles, &plan->tiles_dev, &plan->tiles_cap)) return rc;
+    if (int rc = upload_table(be, plan->ssegs, &plan->ssegs_dev, &plan->ssegs_cap)) return rc;
     if (int rc = upload_table(be, plan->qtiles, &plan->qtiles_dev, &plan->qtiles_cap)) return rc;
     if (int rc = upload_table(be, plan->btiles, &plan->btiles_dev, &plan->btiles_cap)) return rc;
     HIP_TRY(be, hipStreamSynchronize(be->stream));
@@ -1656,6 +1705,11 @@ static int enqueue_plan(infr_hip_t* be, infr_hip_plan_t* plan, infr_hip_buffer_t
                                         static_cast<float*>(bindings[op.dst]->ptr), op.m, op.in_f,
                                         op.out_f, infr::IntStages{}, be->act, &qc))
                 return rc;
+        } else if (st.strips) {
+            infr::launch_quantize_q8_tiled(st.x, st.m, st.in_f, be->act, be->stream);
+            infr::launch_mmq_strip_q4k_group(plan->descs[st.first].bpr, be->act, st.m, st.in_f, st.gp.rows_per_wg,
+                                             plan->ssegs_dev + st.tile_first, st.gp.total_wgs, be->stream);
+            HIP_TRY(be, hipGetLastError());
         } else if (st.m > 1) {
             infr::launch_quantize_q8_group(plan->qtiles_dev + st.qtile_first, st.qtile_n, act_per32(st.dtype, st.in_f),
                                            be->act, be->stream);

@@ -337,7 +337,20 @@ bool launch_mmq_shared_nib32(int dtype, const uint8_t* w, size_t bpr, const ActQ
 // the tiled quantizer's layout. mmq_strip_q4k_tiles picks the strip height (1..3 row tiles) for a device
 // of `cus` compute units.
 // exact: the f32 epilogue as infr-cpu writes it (y bit-identical) instead of the contracted one.
+// One strip of a grouped launch: `rows` (at most the strip height) rows of one op, whose outputs
+// go to y[token * ldy + row].
+struct StripSeg {
+    const uint8_t* w;  // the strip's first weight row
+    float* y;          // the op's output at the strip's first row
+    int32_t ldy;       // the op's out_f
+    int32_t rows;
+};
 int mmq_strip_q4k_tiles(size_t m, size_t out_f, size_t in_f, int cus);
+int mmq_strip_q4k_rows(int tiles);
+bool mmq_q4k_strip_group_takes(size_t m, size_t in_f, size_t total_out_f);
+// Several Q4_K Linears over one quantized activation tensor as one launch (the 1e-4 form).
+void launch_mmq_strip_q4k_group(size_t bpr, const ActQ8& act, size_t m, size_t in_f, int tiles, const StripSeg* segs_dev,
+                                int n_segs, hipStream_t stream);
 void launch_mmq_strip_q4k(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
                           size_t out_f, const IntStages& st, int tiles, bool exact, hipStream_t stream);
 // Routed pairs bucketed by expert, in tiles of at most 32 pairs of one expert each (device arrays;

@@ -1680,6 +1680,16 @@ void launch_mmq_q4k_gathered(const uint8_t* bank, size_t expert_stride, size_t b
                        (int32_t*)nullptr);
 }
 
+// Whether Q4_K Linears of `m` tokens over one activation tensor, `total_out_f` rows between them, run
+// as one grouped strip launch inside a plan: the token counts launch_mmq sends to the strip kernel,
+// on rows the decode mapping covers, when the rows together are past the 16-token kernel's reach.
+bool mmq_q4k_strip_group_takes(size_t m, size_t in_f, size_t total_out_f) {
+    if (in_f % 256 != 0 || gemv_row_too_long(12, in_f) || m < 128) return false;
+    const size_t groups256 = (m + 255) / 256;
+    if ((double)m < 0.6 * (double)(groups256 * 256)) return false;
+    return !mmq_skinny16_takes(12, m, in_f, total_out_f);
+}
+
 bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const ActQ8& act, float* y,
                 size_t m, size_t in_f, size_t out_f, const IntStages& st, int cus, hipStream_t stream,
                 QuantCache* qc) {

@@ -111,7 +111,7 @@ template <int kT, bool STAGES, bool EXACT>
 __global__ __launch_bounds__(kNW * 64) void mmq_strip_q4k_kernel(
     const uint8_t* __restrict__ w, size_t bpr, const int8_t* __restrict__ qs, const float* __restrict__ d8,
     const _Float16* __restrict__ bsh, float* __restrict__ y, int m, int out_f, int nb, int nx, int ny,
-    int32_t* __restrict__ st_sd, int32_t* __restrict__ st_sm) {
+    int32_t* __restrict__ st_sd, int32_t* __restrict__ st_sm, const StripSeg* __restrict__ segs) {
     static_assert(!STAGES || EXACT, "the integer-stage form is the exact form");
     static_assert(kT >= 1 && kT <= 3, "one to three row tiles");
     typedef StripLds<kT> L;
@@ -126,8 +126,18 @@ __global__ __launch_bounds__(kNW * 64) void mmq_strip_q4k_kernel(
     const int xcd = blockIdx.x & 7, chunk = blockIdx.x >> 3;
     const int strip = xcd + 8 * (chunk / ny), ty = chunk % ny;
     if (strip >= nx) return;  // uniform over the workgroup, before any barrier
-    const int row0 = strip * kStripRows;
+    int row0 = strip * kStripRows, ldy = out_f;
     const int tok0 = ty * kStripTokens + wave * 32;
+    // A grouped launch (several Linears over one activation tensor, plans): the strip is an entry
+    // of a table - some rows of one of the ops - and `out_f` below is that entry's.
+    if (segs != nullptr) {
+        const StripSeg sg = segs[strip];
+        w = sg.w;
+        y = sg.y;
+        out_f = sg.rows;
+        row0 = 0;
+        ldy = sg.ldy;
+    }
 
     // ---- the unpack pieces of this wave: (row tile, nibble pair) of a block, 4 * kT in all. Waves w
     // and w + 4 share a SIMD. Three tiles: the lower four take (tiles 0 and 1, pair w) and unpack before
@@ -385,7 +395,7 @@ __global__ __launch_bounds__(kNW * 64) void mmq_strip_q4k_kernel(
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int tok = tok0 + 8 * (r >> 2) + 4 * h + (r & 3);
-            if (tok < m) gstore<float>(y + (size_t)tok * out_f + wrow, acc[t][r]);
+            if (tok < m) gstore<float>(y + (size_t)tok * ldy + wrow, acc[t][r]);
         }
     }
 }
@@ -418,8 +428,9 @@ int mmq_strip_q4k_tiles(size_t m, size_t out_f, size_t in_f, int cus) {
 
 template <int KT>
 static void launch_strip(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
-                         size_t out_f, const IntStages& st, bool exact, hipStream_t stream) {
-    const int nx = (int)((out_f + 32 * KT - 1) / (32 * KT)), ny = (int)((m + kStripTokens - 1) / kStripTokens);
+                         size_t out_f, const IntStages& st, bool exact, hipStream_t stream,
+                         const StripSeg* segs = nullptr, int n_segs = 0) {
+    const int nx = segs ? n_segs : (int)((out_f + 32 * KT - 1) / (32 * KT)), ny = (int)((m + kStripTokens - 1) / kStripTokens);
     const dim3 grid((unsigned)(8 * ((nx + 7) / 8) * ny)), block(kNW * 64);
     const int nb = (int)(in_f / 256);
     const auto* bsh = reinterpret_cast<const _Float16*>(act.bsums);
@@ -430,7 +441,7 @@ static void launch_strip(const uint8_t* w, size_t bpr, const ActQ8& act, float* 
             (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&mmq_strip_q4k_kernel<KT, STAGES, EXACT>),      \
                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);                              \
         hipLaunchKernelGGL((mmq_strip_q4k_kernel<KT, STAGES, EXACT>), grid, block, lds, stream, w, bpr, act.qs, act.d, \
-                           bsh, y, (int)m, (int)out_f, nb, nx, ny, A, B);                                            \
+                           bsh, y, (int)m, (int)out_f, nb, nx, ny, A, B, segs);                                      \
     } while (0)
     if (st.a) INFR_STRIP(true, true, st.a, st.b);
     else if (exact) INFR_STRIP(false, true, (int32_t*)nullptr, (int32_t*)nullptr);
@@ -443,6 +454,17 @@ void launch_mmq_strip_q4k(const uint8_t* w, size_t bpr, const ActQ8& act, float*
     if (tiles == 3) launch_strip<3>(w, bpr, act, y, m, in_f, out_f, st, exact, stream);
     else if (tiles == 2) launch_strip<2>(w, bpr, act, y, m, in_f, out_f, st, exact, stream);
     else launch_strip<1>(w, bpr, act, y, m, in_f, out_f, st, exact, stream);
+}
+
+int mmq_strip_q4k_rows(int tiles) { return 32 * tiles; }
+
+void launch_mmq_strip_q4k_group(size_t bpr, const ActQ8& act, size_t m, size_t in_f, int tiles, const StripSeg* segs_dev,
+                                int n_segs, hipStream_t stream) {
+    if (n_segs <= 0) return;
+    const IntStages none{};
+    if (tiles == 3) launch_strip<3>(nullptr, bpr, act, nullptr, m, in_f, 0, none, false, stream, segs_dev, n_segs);
+    else if (tiles == 2) launch_strip<2>(nullptr, bpr, act, nullptr, m, in_f, 0, none, false, stream, segs_dev, n_segs);
+    else launch_strip<1>(nullptr, bpr, act, nullptr, m, in_f, 0, none, false, stream, segs_dev, n_segs);
 }
 
 }  // namespace infr

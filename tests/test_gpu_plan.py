@@ -1057,3 +1057,53 @@ def test_paired_gated_activation_in_a_many_round_group(be, combined, H):
         got_g, got_u = d["gate"], d["up"]
     assert np.array_equal(bits(got_g), bits(want_g)) and np.array_equal(bits(got_u), bits(want_u))
     assert _rel(d["act"], orc.gated_act(got_g, got_u, 1, FF)) < 1e-6
+
+
+@pytest.mark.parametrize("m", [130, 200, 512, 700])
+def test_q4k_prefill_linears_over_one_tensor_run_as_one_strip_launch(be, m):
+    """q / k / v of a prefill chunk: Q4_K Linears of a level that read one activation tensor are one
+    quantization plus one strip launch over all their rows (a 256-row k or v on its own would fill
+    a fraction of the machine), from the token counts the strip kernel takes, when the rows together
+    are past the 16-token kernel's reach. Every output equals the same op run alone - same kernel, same per-row
+    arithmetic - and the oracle within the route's 1e-4; a Linear over another tensor and a Q6_K
+    one over the same tensor stay out of the group."""
+    in_f = 1024
+    specs = [(DType.Q4K, 1024, 0), (DType.Q4K, 256, 0), (DType.Q4K, 300, 0), (DType.Q6K, 256, 0), (DType.Q4K, 1100, 1)]
+    g, binds = Graph(), Bindings()
+    xids, xbs = [], []
+    for i in range(2):
+        xids.append(g.input(TensorDesc((m, in_f), DType.F32)))
+        xbs.append(be.alloc(m * in_f * 4))
+        binds.bind(xids[i], xbs[i])
+    ws, wbs, ybs = [], [], []
+    for i, (dt, out_f, xi) in enumerate(specs):
+        w = synth_weight(dt, 640 + i, out_f, in_f, 0.05)
+        ws.append(w)
+        wbs.append(be.upload_new(w))
+        wid = g.weight(TensorDesc((out_f, in_f), dt))
+        yid = g.output(TensorDesc((m, out_f), DType.F32))
+        ybs.append(be.alloc(m * out_f * 4))
+        binds.bind(wid, wbs[i]).bind(yid, ybs[i])
+        g.push(Linear(xids[xi], wid, yid, m, in_f, out_f))
+    plan = be.compile(g)
+    grouped = m >= 512      # (130: under 0.6 of a 256-token group; 200: the three are within the 16-token kernel's reach)
+    for rep in range(2):
+        xs = [synth_normal_f32(650 + 2 * rep + i, m * in_f) for i in range(2)]
+        for xb, x in zip(xbs, xs):
+            be.upload(xb, x)
+        be.execute(plan, binds)
+        if rep == 0:
+            # grouped: (quantize + strips) + Q6_K's (quantize + tiles) + the other tensor's (quantize + GEMM)
+            assert not grouped or plan.launches() == 6, plan.launches()
+        toks = [0, 37, m // 2, m - 1]
+        alone = be.alloc(m * 1100 * 4)
+        for (dt, out_f, xi), w, wb, yb in zip(specs, ws, wbs, ybs):
+            got = be.download(yb, np.empty((m, out_f), np.float32))
+            be.linear(dt, wb, xbs[xi], alone, m, in_f, out_f)
+            one = be.download(alone, np.empty((m, out_f), np.float32))
+            # (alone, a narrow op may take the 16-token kernel, whose y is infr-cpu's bit for bit; the
+            # strips contract the f32 epilogue: the route's 1e-4, in practice ~1e-7)
+            assert _rel(got, one) <= 1e-6, (rep, int(dt), out_f)
+            want = orc.linear(dt, w, xs[xi].reshape(m, in_f)[toks].ravel(), len(toks), in_f, out_f)
+            assert _rel(got[toks], want) <= 2e-6, (rep, int(dt), out_f)
+        alone.free()
