@@ -1511,6 +1511,21 @@ static bool skinny16_shape(int dtype, int nb, size_t m, size_t out_f) {
     // IQ4_XS has a 128-token tile kernel whose time is flat up to 128 tokens (30 / 59 / 22 us at 12288 x 4096,
     // 4096 x 12288, 4096 x 4096) where a 16-token pass here costs 8.2 / 8.0 / 2.8: it takes over at 49 tokens
     // on large matrices of 4096-column rows, at 113 on long rows and small matrices
+    // Narrow matrices at any token count: a 128-token tile kernel walks a whole row per workgroup,
+    // so its time has a floor however few rows there are (26-29 us at 4096 columns for Q5_K, Q8_0 and
+    // IQ4_XS, 41 for Q6_K: a 1024-row projection at 128..512 tokens is 32..128 workgroups), while a
+    // pass here costs its share of the outputs. The two meet at about 700 K outputs for Q5_K, 1 M for
+    // Q6_K, 600 K for IQ4_XS, 640 K for Q8_0 (1024 x 4096 at 128 / 256 / 512 tokens: Q5_K 26.7 / 27.8 /
+    // 29.5 us on the tiles, 5.7 / 10.2 / 19.0 here; Q6_K 7.9 / 41.4 / 43.1 and 7.8 / 9.5 / 17.6), 768 K for
+    // the 32-weight-block formats (Q4_0 at 256 / 512 tokens: 62 / 65 us on the tiles), 600 K for Q2_0 (44 / 47). Independent of the row length: both scale with it.
+    if (m > 16 && out_f == 0 && dtype != 12) return true;  // (a plan's group: its ops were taken one by one)
+    if (m > 16) {
+        const size_t outputs = m * out_f;
+        if ((dtype == 13 && outputs <= (size_t)700 * 1024) || (dtype == 14 && outputs <= (size_t)1024 * 1024) ||
+            (dtype == 23 && outputs <= (size_t)600 * 1024) || (dtype == 8 && outputs <= (size_t)640 * 1024) ||
+            (nib32 && outputs <= (size_t)768 * 1024) || (dtype == 42 && outputs <= (size_t)600 * 1024))
+            return true;
+    }
     if (dtype == 23 && m > 16) return m <= ((out_f == 0 || out_f * (size_t)nb <= (size_t)4096 * 16 || nb >= 32) ? 112u : 48u);
     if (dtype == 10 || dtype == 11 || dtype == 23 || dtype == 35) return m >= 3;
     if (m <= 16) {

@@ -347,3 +347,25 @@ def test_q5_0_one_token_linears_of_a_level_share_a_launch(be):
         hv = be.download(hb, np.empty((1, 256), np.float32))
         gate(hv, orc.linear(DType.Q5_0, w1, host["x3"], 1, 256, 256, reference_mode=True))
         gate(be.download(zb, np.empty((1, 64), np.float32)), orc.linear(DType.Q5_0, w2, hv, 1, 256, 64, reference_mode=True))
+
+
+@pytest.mark.parametrize("dtype", [DType.Q5K, DType.Q6K, DType.Q8_0, DType.IQ4XS, DType.Q4_0, DType.Q5_1, DType.IQ4NL, DType.Q2_0],
+                         ids=lambda d: DType(d).name)
+@pytest.mark.parametrize("m,out_f", [(300, 200), (512, 1024), (1000, 96)])
+def test_narrow_matrices_keep_the_16_token_kernel_at_any_token_count(be, dtype, m, out_f):
+    """A 128-token tile kernel walks whole rows per workgroup and has a floor however few rows there
+    are, so matrices with few outputs (tokens x rows) stay on the 16-token K-split kernel, 16 tokens
+    per pass, beyond its usual token range. Same integers and block order as at 16 tokens: the
+    super-block formats and Q8_0 bit-identical to the oracle, the others within the path's 1e-4."""
+    in_f = 1024
+    w = synth_weight(dtype, 0x510 + int(dtype), out_f, in_f, 0.05)
+    x = synth_normal_f32(0x520 + m, m * in_f)
+    x[in_f:2 * in_f] = 0.0
+    y = run_linear(be, dtype, w, x, m, in_f, out_f)
+    toks = np.unique(np.r_[0, 1, 15, 16, m // 2, m - 17, m - 1])
+    want = orc.linear(dtype, w, x.reshape(m, in_f)[toks].ravel(), len(toks), in_f, out_f).reshape(len(toks), out_f)
+    if dtype in (DType.Q5K, DType.Q6K, DType.Q8_0, DType.IQ4XS):
+        assert np.array_equal(y[toks].view(np.uint32), want.view(np.uint32))
+    else:
+        gate(y[toks], want)
+    assert np.all(y[1] == 0.0)
