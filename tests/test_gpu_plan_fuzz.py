@@ -197,7 +197,8 @@ def describe(prog):
 
 @pytest.mark.parametrize("m,seed", [(1, s) for s in range(160)] + [(3, s) for s in range(100, 108)] +
                          [(8, s) for s in range(200, 204)] + [(20, s) for s in range(300, 303)] +
-                         [(48, s) for s in range(400, 402)])
+                         [(48, s) for s in range(400, 402)] + [(300, s) for s in range(500, 504)] +
+                         [(700, s) for s in range(600, 606)])
 def test_scheduled_plan_equals_the_ops_run_one_by_one(be, m, seed):
     rng = np.random.default_rng(seed)
     prog = random_program(rng, int(rng.integers(6, 15)))
