@@ -5,9 +5,14 @@
 //     y   += (d * q8.d[b]) * (f32)isum
 // with an int8 scale sc_g per group. q - 32 (in -32..31) is an int8 operand as it is, so
 // sum_l (q - 32) * q8 comes straight out of the matrix cores; what cannot is the scale: (q - 32) *
-// sc_g needs 13 bits. A group is therefore multiplied on its own - one v_mfma_i32_32x32x32_i8 per
-// group whose other 16 K-slots meet a zero operand - and scaled into the block's isum with one
-// 24-bit multiply-add per output. isum is the CPU's integer, the f32 epilogue is the CPU's expression
+// sc_g needs 13 bits. A group is therefore multiplied on its own - one v_mfma_i32_32x32x16_i8 per
+// group (the K = 16 form takes half the passes of the K = 32 one, which a group would only half
+// fill) - and scaled into the block's isum with one 24-bit multiply-add per output. The tiled
+// activation layout gives lane (token, h) elements 16h..16h+15 of a 32-element sub-block, i.e. the
+// whole of group h, where the K = 16 operand wants bytes 8h..8h+7 of one group: two
+// v_permlane32_swap per sub-block exchange the upper dwords of the h = 0 lanes with the lower
+// dwords of the h = 1 lanes, after which a lane's first eight bytes are its share of the even
+// group and its last eight of the odd one. isum is the CPU's integer, the f32 epilogue is the CPU's expression
 // and the blocks are added in ascending order, so y equals infr-cpu's batch kernel (and this
 // library's m == 1 GEMV) bit for bit.
 //
@@ -24,12 +29,12 @@ namespace infr {
 
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-// LDS of one block: B operands [sub-block][lane] x 16 B | group scales [row][16] | d [row] | 16 zero bytes
+// LDS of one block: B operands [sub-block][lane] x (8 B of the even group | 8 B of the odd group) |
+// group scales [row][16] | d [row]
 struct Q6kLds {
     static constexpr int sc_off = 8 * 1024;
     static constexpr int d_off = sc_off + 32 * 16;
-    static constexpr int zero_off = d_off + 32 * 4;
-    static constexpr int bytes = zero_off + 16;
+    static constexpr int bytes = d_off + 32 * 4;
 };
 
 template <bool STAGES>
@@ -81,13 +86,16 @@ __global__ __launch_bounds__(256) void mmq_shared_q6k_kernel(
                 // q - 32 for q >= 32 and 256 + q - 32 below
                 out[k] = (int)((q + 0x60606060u) ^ 0x80808080u);
             }
-            *reinterpret_cast<v4i*>(buf + (size_t)(2 * p + e) * 1024 + lane * 16) = out;
+            // this lane holds elements 16h..16h+15 of the sub-block = group 2s + h whole: bytes 0..7
+            // are the operand of reader lane (col, 0), bytes 8..15 of reader lane (col, 1), in slot h
+            uint8_t* dst = buf + (size_t)(2 * p + e) * 1024 + col * 16 + 8 * h;
+            *reinterpret_cast<v2i*>(dst) = v2i{out[0], out[1]};
+            *reinterpret_cast<v2i*>(dst + 32 * 16) = v2i{out[2], out[3]};
         }
         if (p == 0 && h == 0) {
             *reinterpret_cast<v4i*>(buf + Q6kLds::sc_off + col * 16) = r.sc;
             reinterpret_cast<float*>(buf + Q6kLds::d_off)[col] = f16_bits_to_f32(r.d);
         }
-        if (tid < 4) reinterpret_cast<int*>(buf + Q6kLds::zero_off)[tid] = 0;
     };
     // activation fragments in the tiled quantizer's order: every load is a contiguous kilobyte
     v4i a[8];
@@ -120,16 +128,18 @@ __global__ __launch_bounds__(256) void mmq_shared_q6k_kernel(
         const v16i zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
         for (int i = 0; i < 16; ++i) isum[i] = 0;
-        // group 2s lives in the K-slots of the h = 0 lanes, group 2s+1 in those of the h = 1 lanes:
-        // the other half reads the zero bytes
-        const uint8_t* zero = cur + Q6kLds::zero_off;
 #pragma unroll
         for (int sb = 0; sb < 8; ++sb) {
-            const uint8_t* src = cur + (size_t)sb * 1024 + lane * 16;
-            const v4i b0 = *reinterpret_cast<const v4i*>(h == 0 ? src : zero);
-            const v4i b1 = *reinterpret_cast<const v4i*>(h == 1 ? src : zero);
-            const v16i r0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[sb], b0, zi, 0, 0, 0);
-            const v16i r1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[sb], b1, zi, 0, 0, 0);
+            // (lane (tok, 0): x y = group 2sb bytes 0..7, z w = bytes 8..15; lane (tok, 1) the same of
+            // group 2sb+1) -> x y = the lane's K-slots of group 2sb, z w = of group 2sb+1
+            // (the swap exchanges lanes 32..63 of its first operand with lanes 0..31 of its second)
+            const auto s0 = __builtin_amdgcn_permlane32_swap(a[sb].x, a[sb].z, false, false);
+            const auto s1 = __builtin_amdgcn_permlane32_swap(a[sb].y, a[sb].w, false, false);
+            const v2i a0 = {(int)s0[0], (int)s1[0]}, a1 = {(int)s0[1], (int)s1[1]};
+            const v4i bf = *reinterpret_cast<const v4i*>(cur + (size_t)sb * 1024 + lane * 16);
+            const v2i b0 = {bf.x, bf.y}, b1 = {bf.z, bf.w};
+            const v16i r0 = __builtin_amdgcn_mfma_i32_32x32x16_i8(__builtin_bit_cast(long, a0), __builtin_bit_cast(long, b0), zi, 0, 0, 0);
+            const v16i r1 = __builtin_amdgcn_mfma_i32_32x32x16_i8(__builtin_bit_cast(long, a1), __builtin_bit_cast(long, b1), zi, 0, 0, 0);
             const int g0 = 2 * sb, g1 = 2 * sb + 1;
             const int sc0 = __builtin_amdgcn_sbfe(scw[g0 >> 2], 8 * (g0 & 3), 8);
             const int sc1 = __builtin_amdgcn_sbfe(scw[g1 >> 2], 8 * (g1 & 3), 8);
