@@ -1044,10 +1044,14 @@ def test_paired_gated_activation_in_a_many_round_group(be, combined, H):
     """66,000 gate rows and as many up rows: the group is many rounds of workgroups, whose rows go
     through the per-wave LDS rings; a paired tile's two wave sets stream their own matrix each."""
     FF = 66000
-    plan, run, host = _gated_ffn(be, DType.Q4K, H, FF, combined=combined, seed=31)
+    norm = H == 5120 and not combined          # one case also behind an absorbed RmsNorm
+    plan, run, host = _gated_ffn(be, DType.Q4K, H, FF, combined=combined, norm=norm, seed=31)
     xv = synth_normal_f32(90, H)
     d = run(xv)
     assert plan.launches() == 1
+    if norm:
+        assert _rel(d["h"], orc.rms_norm(xv, host["nw"], 1, H, 1e-6)) < 1e-6
+        xv = d["h"]
     if combined:
         gu = orc.linear(DType.Q4K, host["wgu"], xv, 1, H, 2 * FF).ravel()
         want_g, want_u, got_g, got_u = gu[:FF], gu[FF:], d["gu"][:FF], d["gu"][FF:]
@@ -1055,7 +1059,10 @@ def test_paired_gated_activation_in_a_many_round_group(be, combined, H):
         want_g = orc.linear(DType.Q4K, host["wg"], xv, 1, H, FF).ravel()
         want_u = orc.linear(DType.Q4K, host["wu"], xv, 1, H, FF).ravel()
         got_g, got_u = d["gate"], d["up"]
-    assert np.array_equal(bits(got_g), bits(want_g)) and np.array_equal(bits(got_u), bits(want_u))
+    if norm:       # (the device normalises in registers; its stored vector is what the oracle multiplies)
+        assert _rel(got_g, want_g) < 1e-4 and _rel(got_u, want_u) < 1e-4
+    else:
+        assert np.array_equal(bits(got_g), bits(want_g)) and np.array_equal(bits(got_u), bits(want_u))
     assert _rel(d["act"], orc.gated_act(got_g, got_u, 1, FF)) < 1e-6
 
 
