@@ -17,7 +17,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libinfr_hip.so")
 OBJ = os.path.join(HERE, "build")
 
-SOURCES = ["backend.hip", "quant_act.hip", "gemv.hip", "gemv_fmt_kquant.hip", "gemv_fmt_blk32.hip", "gemv_fmt_q5k.hip", "gemv_fmt_q23k.hip", "gemv_fmt_tq.hip", "gemv_fmt_iq4xs_fp4.hip", "gemv_fmt_nib4.hip", "gemv_fmt_nib5.hip", "gemv_fmt_pair.hip", "gemv_f32act.hip", "mmq.hip", "mmq_q4k_strip.hip", "mmq_q5k.hip", "mmq_iq4xs.hip", "mmq_q6k.hip", "mmq_q8_0.hip", "mmq_nib32.hip", "mmq_gathered.hip", "moe.hip", "elementwise.hip", "embed.hip", "synth.cpp", "gguf.cpp"]
+SOURCES = ["backend.hip", "quant_act.hip", "gemv.hip", "gemv_fmt_kquant.hip", "gemv_fmt_blk32.hip", "gemv_fmt_q5k.hip", "gemv_fmt_q23k.hip", "gemv_fmt_tq.hip", "gemv_fmt_iq4xs_fp4.hip", "gemv_fmt_nib4.hip", "gemv_fmt_nib5.hip", "gemv_fmt_pair.hip", "gemv_f32act.hip", "mmq.hip", "mmq_q4k_strip.hip", "mmq_q5k.hip", "mmq_iq4xs.hip", "mmq_q2k.hip", "mmq_q3k.hip", "mmq_q6k.hip", "mmq_q8_0.hip", "mmq_nib32.hip", "mmq_gathered.hip", "moe.hip", "elementwise.hip", "embed.hip", "synth.cpp", "gguf.cpp"]
 
 # -ffp-contract=off: the f32 epilogues restate infr-cpu's expressions, which never fuse a multiply
 # into an add; -packed-fp32-ops off: packed FP32 forms are not used on this hardware pool.

@@ -1507,7 +1507,8 @@ static bool skinny16_shape(int dtype, int nb, size_t m, size_t out_f) {
     if (dtype != 12 && dtype != 13 && dtype != 14 && dtype != 8 && dtype != 42 && dtype != 10 && dtype != 11 && dtype != 23 && dtype != 35 && !nib32)
         return false;
     if (nb < kSkinny16Blocks || (nb % kSkinny16Blocks != 0 && (dtype == 14 || dtype == 42 || dtype == 11 || dtype == 35))) return false;
-    // Q2_K, Q3_K, IQ4_XS, TQ2_0: the dot4 batches are the only other kernel, eight tokens per pass over the weights
+    // Q2_K, Q3_K, IQ4_XS, TQ2_0 up to 16 tokens: the dot4 batches are the only other kernel there, eight tokens per
+    // pass over the weights; beyond, their 128-token tile kernels take over as measured below
     // IQ4_XS has a 128-token tile kernel whose time is flat up to 128 tokens (30 / 59 / 22 us at 12288 x 4096,
     // 4096 x 12288, 4096 x 4096) where a 16-token pass here costs 8.2 / 8.0 / 2.8: it takes over at 49 tokens
     // on large matrices of 4096-column rows, at 113 on long rows and small matrices
@@ -1515,17 +1516,27 @@ static bool skinny16_shape(int dtype, int nb, size_t m, size_t out_f) {
     // so its time has a floor however few rows there are (26-29 us at 4096 columns for Q5_K, Q8_0 and
     // IQ4_XS, 41 for Q6_K: a 1024-row projection at 128..512 tokens is 32..128 workgroups), while a
     // pass here costs its share of the outputs. The two meet at about 700 K outputs for Q5_K, 1 M for
-    // Q6_K, 600 K for IQ4_XS, 640 K for Q8_0 (1024 x 4096 at 128 / 256 / 512 tokens: Q5_K 26.7 / 27.8 /
+    // Q6_K, 600 K for IQ4_XS and Q2_K, 700 K for Q3_K and TQ2_0, 640 K for Q8_0 (1024 x 4096 at 128 / 256 / 512 tokens: Q5_K 26.7 / 27.8 /
     // 29.5 us on the tiles, 5.7 / 10.2 / 19.0 here; Q6_K 7.9 / 41.4 / 43.1 and 7.8 / 9.5 / 17.6), 768 K for
     // the 32-weight-block formats (Q4_0 at 256 / 512 tokens: 62 / 65 us on the tiles), 600 K for Q2_0 (44 / 47). Independent of the row length: both scale with it.
     if (m > 16 && out_f == 0 && dtype != 12) return true;  // (a plan's group: its ops were taken one by one)
     if (m > 16) {
         const size_t outputs = m * out_f;
         if ((dtype == 13 && outputs <= (size_t)700 * 1024) || (dtype == 14 && outputs <= (size_t)1024 * 1024) ||
-            (dtype == 23 && outputs <= (size_t)600 * 1024) || (dtype == 8 && outputs <= (size_t)640 * 1024) ||
+            ((dtype == 23 || dtype == 10) && outputs <= (size_t)600 * 1024) ||
+            ((dtype == 11 || dtype == 35) && nb % kSkinny16Blocks == 0 && outputs <= (size_t)700 * 1024) || (dtype == 8 && outputs <= (size_t)640 * 1024) ||
             (nib32 && outputs <= (size_t)768 * 1024) || (dtype == 42 && outputs <= (size_t)600 * 1024))
             return true;
     }
+    // Q2_K's 128-token tiles (mmq_q2k.hip) are flat up to 128 tokens at 23 / 45 / 18 us (12288 x 4096, 4096 x 12288,
+    // 4096 x 4096) where a 16-token pass here costs 5.8 / 5.4 / 2.0: they take over at 65 tokens on large matrices
+    // of 4096-column rows, at 129 on long rows and small matrices
+    // Q3_K and TQ2_0 (mmq_q3k.hip): tiles flat at 36 / 70 / 25 us and 23 / 44 / 17 us up to 128 tokens, a 16-token
+    // pass here 6.6 / 6.3 / 2.3 and 4.4 / 4.4 / 1.6: from 97 (Q3_K) and 81 (TQ2_0) tokens on large matrices of
+    // 4096-column rows, from 161 on long rows and small matrices
+    if ((dtype == 11 || dtype == 35) && m > 16)
+        return m <= ((out_f == 0 || out_f * (size_t)nb <= (size_t)4096 * 16 || nb >= 32) ? 160u : (dtype == 11 ? 96u : 80u));
+    if (dtype == 10 && m > 16) return m <= ((out_f == 0 || out_f * (size_t)nb <= (size_t)4096 * 16 || nb >= 32) ? 128u : 64u);
     if (dtype == 23 && m > 16) return m <= ((out_f == 0 || out_f * (size_t)nb <= (size_t)4096 * 16 || nb >= 32) ? 112u : 48u);
     if (dtype == 10 || dtype == 11 || dtype == 23 || dtype == 35) return m >= 3;
     if (m <= 16) {
@@ -1765,6 +1776,17 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
     if (dtype == 13 && (m >= 33 || long_row)) {
         quantize_tiled();
         launch_mmq_shared_q5k(w, bpr, act, y, m, in_f, out_f, st, stream);
+        return true;
+    }
+    if (dtype == 10 && in_f % 256 == 0 && (m >= 17 || long_row)) {  // (what the 16-token kernel left)
+        quantize_tiled();
+        launch_mmq_shared_q2k(w, bpr, act, y, m, in_f, out_f, st, stream);
+        return true;
+    }
+    if ((dtype == 11 || dtype == 35) && in_f % 256 == 0 && (m >= 17 || long_row)) {  // (what the 16-token kernel left)
+        quantize_tiled();
+        if (dtype == 11) launch_mmq_shared_q3k(w, bpr, act, y, m, in_f, out_f, st, stream);
+        else launch_mmq_shared_tq2_0(w, bpr, act, y, m, in_f, out_f, st, stream);
         return true;
     }
     if (dtype == 23 && in_f % 256 == 0 && (m >= 17 || long_row)) {  // (what the 16-token kernel left: 49 / 113 tokens and up)

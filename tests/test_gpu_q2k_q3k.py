@@ -189,29 +189,38 @@ def test_moe_banks(be, dtype, rows):
     check(*got, *want)
 
 
-@pytest.mark.parametrize("m,in_f,out_f", [(49, 4096, 4128), (113, 1024, 96), (130, 2048, 70), (200, 768, 33), (512, 4096, 64),
-                                          (300, 256, 1), (128, 8192, 40)])
-def test_iq4xs_prefill_tiles_are_bit_identical_to_the_oracle(be, m, in_f, out_f):
-    """Beyond the 16-token kernel's reach (49 tokens on large matrices, 113 elsewhere) IQ4_XS takes
-    128-token x 32-row tiles on the int8 matrix cores, a product per 32-weight sub-block scaled by
-    ls - 32 in integers: the same per-block integer and f32 expression as the one-token kernel,
-    blocks in ascending order - every output bit-identical; ragged token and row counts included."""
-    w = orc.synth_weight(DType.IQ4XS, in_f * out_f, 0x4A + m)
+TILED = [DType.Q2K, DType.Q3K, DType.IQ4XS, DType.TQ2_0]
+
+
+@pytest.mark.parametrize("dtype", TILED, ids=ids)
+@pytest.mark.parametrize("m,in_f,out_f", [(97, 4096, 8224), (161, 1024, 96), (200, 2048, 70), (300, 768, 33), (512, 4096, 64),
+                                          (300, 256, 1), (170, 8192, 40), (190, 1280, 50)])
+def test_prefill_tiles_are_bit_identical_to_the_oracle(be, dtype, m, in_f, out_f):
+    """Beyond the 16-token kernel's reach these formats take 128-token x 32-row tiles on the int8
+    matrix cores: IQ4_XS a product per 32-weight sub-block scaled by ls - 32 in integers; Q2_K, Q3_K
+    and TQ2_0 scaled codes (code x scale fits a byte), so a block is one chain of eight MFMAs, Q2_K's
+    mins an f16 MFMA against per-16 sums formed in the kernel. Same per-block integers and f32
+    expression as the one-token kernels, blocks in ascending order - every output bit-identical;
+    ragged token and row counts and an odd number of blocks per row included."""
+    w = orc.synth_weight(dtype, in_f * out_f, 0x4A + m)
     x = synth_normal_f32(30 + m, m * in_f)
     x[:in_f] *= 17.0
     x[in_f:2 * in_f] = 0.0
-    y = run_linear(be, DType.IQ4XS, w, x, m, in_f, out_f)
+    y = run_linear(be, dtype, w, x, m, in_f, out_f)
     rows = np.unique(np.r_[0, 1, m // 2, m - 1, np.arange(0, m, max(1, m // 9))])
     for r in rows:                                    # (a sample of tokens keeps the oracle's time down at the large case)
-        want = orc.linear(DType.IQ4XS, w, x[r * in_f:(r + 1) * in_f], 1, in_f, out_f).ravel()
+        want = orc.linear(dtype, w, x[r * in_f:(r + 1) * in_f], 1, in_f, out_f).ravel()
         assert np.array_equal(bits(y[r]), bits(want)), f"token {r} differs"
     assert np.all(y[1] == 0.0)
 
 
-def test_iq4xs_prefill_int_stage_is_exact(be):
-    m, in_f, out_f = 150, 1024, 40
-    w = orc.synth_weight(DType.IQ4XS, in_f * out_f, 0x4B)
+@pytest.mark.parametrize("dtype", TILED, ids=ids)
+def test_prefill_tiles_int_stages_are_exact(be, dtype):
+    m, in_f, out_f = 200, 1024, 40
+    w = orc.synth_weight(dtype, in_f * out_f, 0x4B)
     x = orc.gen_f32(m * in_f, 0x77AA)
-    a, _ = be.linear_int_stages(DType.IQ4XS, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
-    oa, _ = orc.linear_int_stages(DType.IQ4XS, w, x, m, in_f, out_f)
+    a, b = be.linear_int_stages(dtype, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
+    oa, ob = orc.linear_int_stages(dtype, w, x, m, in_f, out_f)
     assert np.array_equal(a, oa)
+    if dtype == DType.Q2K:
+        assert np.array_equal(b, ob)
