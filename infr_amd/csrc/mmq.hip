@@ -1519,6 +1519,7 @@ static bool skinny16_shape(int dtype, int nb, size_t m, size_t out_f) {
     // Q6_K, 600 K for IQ4_XS and Q2_K, 700 K for Q3_K and TQ2_0, 640 K for Q8_0 (1024 x 4096 at 128 / 256 / 512 tokens: Q5_K 26.7 / 27.8 /
     // 29.5 us on the tiles, 5.7 / 10.2 / 19.0 here; Q6_K 7.9 / 41.4 / 43.1 and 7.8 / 9.5 / 17.6), 768 K for
     // the 32-weight-block formats (Q4_0 at 256 / 512 tokens: 62 / 65 us on the tiles), 600 K for Q2_0 (44 / 47). Independent of the row length: both scale with it.
+    if (m > (size_t)16 * 65535) return false;  // (the grid's third dimension walks the batch 16 tokens at a time)
     if (m > 16 && out_f == 0 && dtype != 12) return true;  // (a plan's group: its ops were taken one by one)
     if (m > 16) {
         const size_t outputs = m * out_f;
