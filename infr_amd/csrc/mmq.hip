@@ -1761,7 +1761,11 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
         // Strips are 256 tokens wide: a batch that fills less than ~0.6 of its 256-token groups (128..153,
         // 257..307 tokens) takes the 128-token tiles of the shared-operand kernel instead.
         const size_t groups256 = (m + 255) / 256;
-        const int tiles = (double)m >= 0.6 * (double)(groups256 * 256) ? mmq_strip_q4k_tiles(m, out_f, in_f, cus) : 0;
+        int tiles = (double)m >= 0.6 * (double)(groups256 * 256) ? mmq_strip_q4k_tiles(m, out_f, in_f, cus) : 0;
+        // One-tile strips that cover at most half of the compute units (4096 rows at up to 256 tokens): the
+        // 128-token tiles are twice the workgroups (4096 x 12288 at 200 / 256 tokens: 64 / 66 us against 78 / 79;
+        // 4096 x 4096: 26 against 30).
+        if (tiles == 1 && ((out_f + 31) / 32) * groups256 * 2 <= (size_t)(cus > 0 ? cus : 256)) tiles = 0;
         if (tiles > 0) launch_mmq_strip_q4k(w, bpr, act, y, m, in_f, out_f, st, tiles, st.a != nullptr, stream);
         else launch_mmq_shared_q4k<1>(w, bpr, act, y, m, in_f, out_f, st, stream);
         return true;
