@@ -10,7 +10,8 @@ bytes / wall time of the timed steps (inputs resident in HBM), the reference's G
 
 The same JSON line carries `roofline` for the dominant kernel (the Q4_K GEMV; achieved = weight
 bytes per launch / average launch duration from HIP events on the backend's stream), the
-`cpu_baseline` (the C restatement of infr-cpu's scalar kernels on the host cores, bounded sample)
+`cpu_baseline` (the C restatement of infr-cpu's scalar kernels on the host cores, bounded sample;
+`cpu_baseline_mmq` and `cpu_baseline_moe` for the prefill half and the routed-expert path)
 and `extra` with the secondary figures of the benchmark's other configurations: Q6_K / Q8_0 GEMV, batch 8, prefill
 mmq int8 TOPS at M in {64, 512, 2048}, the ternary Q2_0 sweep and the MoE routed-expert GEMV.
 """
@@ -603,6 +604,32 @@ def cpu_baseline_mmq(m=512, in_f=4096, rows=512):
                       f"batch kernel, OpenMP over output rows"}
 
 
+def cpu_baseline_moe(n_expert=16):
+    """The routed-expert path on the CPU oracle: one token of Op::MoeFfn at the Qwen3-30B-A3B expert
+    shape (hidden 2048, expert FFN 768, top-8, Q4_K banks; a token touches eight experts whatever the
+    bank holds, so the sample's bank has `n_expert` of the 128 experts), every thread, best of at
+    least 3 passes within ~1.5 s. The same unit as `moe_q4k_t1_us_per_layer`."""
+    from infr_amd import DType, synth_normal_f32, synth_weight
+    from oracle import oracle as orc
+    threads = orc.max_threads()
+    ne, n_used, nff = 2048, 8, 768
+    banks = [synth_weight(DType.Q4K, 70 + i, n_expert * (nff if i < 2 else ne), ne if i < 2 else nff) for i in range(3)]
+    router = synth_normal_f32(80, n_expert * ne, sigma=0.03)
+    x = synth_normal_f32(81, ne)
+    call = lambda: orc.moe_ffn(x, router, banks[0], banks[1], banks[2], ne=ne, n_expert=n_expert, n_used=n_used,
+                               n_ff_exp=nff, threads=threads)
+    call()  # warm-up
+    best, passes, t_start = 1e30, 0, time.perf_counter()
+    while passes < 3 or (time.perf_counter() - t_start < 1.5 and passes < 2000):
+        t0 = time.perf_counter()
+        call()
+        best = min(best, time.perf_counter() - t0)
+        passes += 1
+    return {"value": round(best * 1e6, 1), "unit": "us per layer (1 token)", "cores": threads, "kind": "port",
+            "sample": f"Op::MoeFfn, one token, hidden {ne}, expert FFN {nff}, top-{n_used} of a {n_expert}-expert Q4_K bank "
+                      f"(8 experts touched as with 128), best of {passes} passes; C restatement of infr-cpu's MoeFfn arm"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -804,6 +831,7 @@ def main():
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline()
         out["cpu_baseline_mmq"] = cpu_baseline_mmq()
+        out["cpu_baseline_moe"] = cpu_baseline_moe()
     print(json.dumps(out))
 
 
