@@ -42,6 +42,7 @@ __device__ __forceinline__ void gstore(void* p, T v) {
 
 typedef v4i v4i_a4 __attribute__((aligned(4)));
 typedef v4i v4i_a2 __attribute__((aligned(2)));
+typedef v4i v4i_a1 __attribute__((aligned(1)));
 typedef v2i v2i_a2 __attribute__((aligned(2)));
 typedef int v3i __attribute__((ext_vector_type(3)));
 typedef v3i v3i_a4 __attribute__((aligned(4)));

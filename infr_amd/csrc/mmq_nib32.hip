@@ -1,5 +1,5 @@
-// Prefill GEMM (65 tokens and up) of the 32-weight-block formats Q4_0, Q4_1, Q5_0, Q5_1 and IQ4_NL on
-// the int8 matrix cores, and of Q8_0 rows that are not whole 256s (which infr-cpu multiplies against
+// Prefill GEMM (65 tokens and up) of the 32-weight-block formats Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL and MXFP4
+// on the int8 matrix cores, and of Q8_0 rows that are not whole 256s (which infr-cpu multiplies against
 // the per-32 activation as well: `q8_0_blk32`, crates/infr-cpu/src/lib.rs:1037-1042, d*d8 * iprod per
 // block, kernels.rs:1170-1187). A row may end inside a 256-element step: the quantizer pads the
 // activation with zero codes, scales and sums up to the step, and the blocks past the row's end
@@ -11,6 +11,7 @@
 //     Q4_0   d*d8 * (iprod - 8*bsum)        Q5_0   d*d8 * (iprod - 16*bsum)
 //     Q4_1   d8 * (d*iprod + m*bsum)        Q5_1   d8 * (d*iprod + m*bsum)
 //     IQ4_NL d*d8 * iprod                   (iprod over the signed codebook values)
+//     MXFP4  d*d8 * iprod                   (d the E8M0 scale halved, iprod over doubled E2M1 values)
 // The codes (0..15, 0..31, or the codebook's int8) are int8 operands, so iprod is one
 // v_mfma_i32_32x32x32_i8 per block, exact. Every format's term is d8 * (A * iprod + B * bsum) with
 // two per-block constants (A = d; B = -8d, -16d, m or 0), evaluated with one conversion, one
@@ -38,7 +39,7 @@ struct Nib32Lds {
 };
 
 // The formats of this kernel: the five nibble formats and Q8_0 against per-32 activations.
-enum class Blk32 { Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, Q8_0 };
+enum class Blk32 { Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, Q8_0, MXFP4 };
 
 // nb: 256-element steps (the last one may be partly past the row); nblk: 32-weight blocks of a row
 template <Blk32 K, bool STAGES>
@@ -49,7 +50,10 @@ __global__ __launch_bounds__(256) void mmq_shared_nib32_kernel(
     constexpr bool kAffine = K == Blk32::Q4_1 || K == Blk32::Q5_1;
     constexpr bool kFive = K == Blk32::Q5_0 || K == Blk32::Q5_1;
     constexpr bool kBytes = K == Blk32::Q8_0;  // codes are whole bytes: 32 of them per block
-    constexpr int kBlockBytes = kBytes ? 34 : 18 + (kAffine ? 2 : 0) + (kFive ? 4 : 0);
+    // MXFP4: [E8M0 scale][16 code bytes], 17 bytes at any byte alignment; the codes index a signed
+    // table of doubled E2M1 values and the scale decodes halved (crates/infr-cpu/src/lib.rs:1394-1432)
+    constexpr bool kMx = K == Blk32::MXFP4;
+    constexpr int kBlockBytes = kMx ? 17 : (kBytes ? 34 : 18 + (kAffine ? 2 : 0) + (kFive ? 4 : 0));
     constexpr int kQhOff = kAffine ? 4 : 2, kQsOff = kBytes ? 2 : kBlockBytes - 16;
     __shared__ __attribute__((aligned(16))) uint8_t lds[2 * Nib32Lds::bytes];
     __shared__ __attribute__((aligned(16))) float dql[4][8][32], bql[4][8][32];  // per wave: [block][token]
@@ -75,8 +79,8 @@ __global__ __launch_bounds__(256) void mmq_shared_nib32_kernel(
             const int bi = b * 8 + 2 * p + e;
             const bool in_row = bi < nblk;  // wave-uniform; past the row's end: block 0 again, scale 0
             const uint8_t* blk = wrowp + (size_t)(in_row ? bi : 0) * kBlockBytes;  // 2-byte aligned
-            r.q[e] = load16_a2(blk + kQsOff + (kBytes ? 16 * h : 0));
-            r.d[e] = in_row ? load_u16(blk) : 0u;
+            r.q[e] = kMx ? gload<v4i_a1>(blk + kQsOff) : load16_a2(blk + kQsOff + (kBytes ? 16 * h : 0));
+            r.d[e] = in_row ? (kMx ? (uint32_t)gload<uint8_t>(blk) : load_u16(blk)) : (kMx ? 0x100u : 0u);
             r.mw[e] = kAffine && in_row ? load_u16(blk + 2) : 0u;
             r.qh[e] = kFive ? (load_u16(blk + kQhOff) | (load_u16(blk + kQhOff + 2) << 16)) : 0u;
         }
@@ -90,14 +94,16 @@ __global__ __launch_bounds__(256) void mmq_shared_nib32_kernel(
                 uint32_t c = (uint32_t)r.q[e][k];
                 if (!kBytes) c = (c >> (4 * h)) & 0x0F0F0F0Fu;
                 if (K == Blk32::IQ4_NL) c = (uint32_t)iq4nl_lookup(c);
+                if (kMx) c = (uint32_t)mxfp4_lookup(c);
                 if (kFive) c |= spread4_to_bit4(r.qh[e] >> (16 * h + 4 * k));
                 out[k] = (int)c;
             }
             *reinterpret_cast<v4i*>(buf + (size_t)(2 * p + e) * 1024 + lane * 16) = out;
             if (h == 0) {
-                const float d = f16_bits_to_f32(r.d[e]);
+                // (MXFP4: a block past the row's end carries the marker 0x100 instead of a scale byte)
+                const float d = kMx ? (r.d[e] < 0x100u ? e8m0_half(r.d[e]) : 0.0f) : f16_bits_to_f32(r.d[e]);
                 const float bb = kAffine ? f16_bits_to_f32(r.mw[e])
-                                         : (K == Blk32::IQ4_NL || kBytes ? 0.0f : (kFive ? -16.0f : -8.0f) * d);
+                                         : (K == Blk32::IQ4_NL || kBytes || kMx ? 0.0f : (kFive ? -16.0f : -8.0f) * d);
                 reinterpret_cast<float*>(buf + Nib32Lds::a_off)[col * 8 + 2 * p + e] = d;
                 reinterpret_cast<float*>(buf + Nib32Lds::b_off)[col * 8 + 2 * p + e] = bb;
             }
@@ -331,6 +337,7 @@ bool launch_mmq_shared_nib32(int dtype, const uint8_t* w, size_t bpr, const ActQ
     case 6: launch_nib32<Blk32::Q5_0>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
     case 7: launch_nib32<Blk32::Q5_1>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
     case 20: launch_nib32<Blk32::IQ4_NL>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
+    case 39: launch_nib32<Blk32::MXFP4>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
     case 8: launch_nib32<Blk32::Q8_0>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
     case 42: {
         const dim3 grid((unsigned)((out_f + 31) / 32), (unsigned)((m + 127) / 128)), block(256);

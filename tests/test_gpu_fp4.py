@@ -166,3 +166,25 @@ def test_moe_banks_mixed_with_the_int8_formats(be, dts, rows):
     want = orc.moe_ffn(x, router, gate_w, up_w, down_w, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=nff,
                        gate_dtype=int(dts[0]), up_dtype=int(dts[1]), down_dtype=int(dts[2]))
     check(*got, *want)
+
+
+@pytest.mark.parametrize("m,in_f,out_f", [(41, 1024, 96), (64, 4096, 8200), (130, 2048, 70), (300, 288, 33), (200, 1280, 50),
+                                          (70, 8192, 40), (512, 4096, 64)])
+def test_mxfp4_prefill_tiles(be, m, in_f, out_f):
+    """From 33..65 tokens (by shape) MXFP4 takes the 32-weight-block formats' 128-token tiles on the
+    int8 matrix cores: one MFMA per block over the doubled E2M1 table values, scaled by the halved
+    E8M0 scale and the per-32 activation scale - per-block integers equal to the oracle's, y within
+    the path's 1e-4 (another association of the same f32 terms); rows that are not whole 256s and
+    17-byte blocks at every byte alignment included."""
+    w = orc.synth_weight(DType.MXFP4, in_f * out_f, 0x5A + m)
+    x = synth_normal_f32(40 + m, m * in_f)
+    x[in_f:2 * in_f] = 0.0
+    y = run_linear(be, DType.MXFP4, w, x, m, in_f, out_f)
+    toks = np.unique(np.r_[0, 1, 31, 32, m // 2, m - 1])
+    want = orc.linear(DType.MXFP4, w, x.reshape(m, in_f)[toks].ravel(), len(toks), in_f, out_f)
+    gate(y[toks], want)
+    assert np.all(y[1] == 0.0)
+    if out_f <= 96:
+        a, _ = be.linear_int_stages(DType.MXFP4, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
+        oa, _ = orc.linear_int_stages(DType.MXFP4, w, x, m, in_f, out_f)
+        assert np.array_equal(a, oa)
