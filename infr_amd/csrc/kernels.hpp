@@ -328,10 +328,12 @@ void launch_mmq_shared_q5k(const uint8_t* w, size_t bpr, const ActQ8& act, float
 // The same for Q2_K; st.a / st.b receive sd / sm per (token, row, 256-block).
 void launch_mmq_shared_q2k(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
                            size_t out_f, const IntStages& st, hipStream_t stream);
-// The same for Q3_K and TQ2_0; st.a receives isum / iprod per (token, row, 256-block).
+// The same for Q3_K, TQ2_0 and TQ1_0; st.a receives isum / iprod per (token, row, 256-block).
 void launch_mmq_shared_q3k(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
                            size_t out_f, const IntStages& st, hipStream_t stream);
 void launch_mmq_shared_tq2_0(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
+                             size_t out_f, const IntStages& st, hipStream_t stream);
+void launch_mmq_shared_tq1_0(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
                              size_t out_f, const IntStages& st, hipStream_t stream);
 // The same for IQ4_XS; st.a receives isum per (token, row, 256-block).
 void launch_mmq_shared_iq4xs(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,

@@ -1788,6 +1788,14 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
         launch_mmq_shared_q2k(w, bpr, act, y, m, in_f, out_f, st, stream);
         return true;
     }
+    // TQ1_0 has no 16-token kernel: its dot4 batches cost 2.6 / 2.3 / 1.3 us per token (12288 x 4096, 4096 x 12288,
+    // 4096 x 4096), the tiles - whose unpack takes the base-3 digits out - a flat 44 / 106 / 39 us up to 128 tokens
+    const size_t tq1_tile_tokens = in_f < 8192 && out_f * in_f >= ((size_t)32 << 20) ? 17 : 33;
+    if (dtype == 34 && in_f % 256 == 0 && (m >= tq1_tile_tokens || long_row)) {
+        quantize_tiled();
+        launch_mmq_shared_tq1_0(w, bpr, act, y, m, in_f, out_f, st, stream);
+        return true;
+    }
     if ((dtype == 11 || dtype == 35) && in_f % 256 == 0 && (m >= 17 || long_row)) {  // (what the 16-token kernel left)
         quantize_tiled();
         if (dtype == 11) launch_mmq_shared_q3k(w, bpr, act, y, m, in_f, out_f, st, stream);

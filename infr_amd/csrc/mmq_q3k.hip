@@ -1,5 +1,5 @@
-// Prefill GEMM of Q3_K and TQ2_0 weights on the int8 matrix cores, 128 tokens x 32 weight rows per
-// workgroup. Both formats keep 2-bit fields in the Q2_K arrangement - element 32 sb + 16 h + l of a
+// Prefill GEMM of Q3_K, TQ2_0 and TQ1_0 weights on the int8 matrix cores, 128 tokens x 32 weight rows
+// per workgroup. Q3_K and TQ2_0 keep 2-bit fields in the Q2_K arrangement - element 32 sb + 16 h + l of a
 // block is bit pair sb % 4 of byte qs[32 (sb / 4) + 16 h + l] - and both reduce a block to ONE
 // chain of eight v_mfma_i32_32x32x32_i8 (the accumulators carry from sub-block to sub-block), with
 // nothing per group left to do on the outputs:
@@ -94,6 +94,63 @@ struct TileTQ2_0 {
 #pragma unroll
         for (int k = 0; k < 4; ++k)  // q - 1 per byte: q + 0x7F stays inside the byte, flipping bit 7 gives q - 1
             out[k] = (int)(((((uint32_t)r.q[k] >> sh) & 0x03030303u) + 0x7F7F7F7Fu) ^ 0x80808080u);
+        return out;
+    }
+};
+
+// TQ1_0 (54-byte block: qs[48], qh[4], d; kernels.rs:3167-3240): base-3 packed ternary digits, weight
+// (digit - 1) d. Digit n of a byte is the high byte of three times (byte * 3^n mod 256). Elements
+// come in three runs - qs[0..32) x 5 digits -> 32 n + m, qs[32..48) x 5 -> 160 + 16 n + m, qh[0..4) x 4
+// -> 240 + 4 n + j - so the 16 elements 32 sb + 16 h .. of lane (row, h) are digit sb of
+// qs[16 h .. 16 h + 15] for sb < 5; digit 2 (sb - 5) + h of qs[32..47] for sb = 5, 6; digit 4 of
+// qs[32..47] (h = 0) or digits 0..3 of the four qh bytes (h = 1) for sb = 7. The digits are taken
+// out once per 128 tokens; digit - 1 is the operand and the block one chain, as for TQ2_0.
+struct TileTQ1_0 {
+    static constexpr int kBlockBytes = 54;
+    static constexpr bool kNegate = false;
+    struct Raw {
+        v4i qa, qb;
+        uint32_t qh, d;
+    };
+    __device__ static void load(Raw& r, const uint8_t* blk, int, int h) {  // 2-byte aligned
+        r.qa = load16_a2(blk + 16 * h);
+        r.qb = load16_a2(blk + 32);
+        r.qh = (uint32_t)gload<int_a2>(blk + 48);
+        r.d = load_u16(blk + 52);
+    }
+    // The five digits of each of a word's four bytes: out[n] holds digit n of byte k in byte k
+    // (even and odd bytes in the two halves of a word: three times a byte fits 16 bits).
+    __device__ static void digits5(uint32_t w, uint32_t (&out)[5]) {
+        uint32_t e = w & 0x00FF00FFu, o = (w >> 8) & 0x00FF00FFu;
+#pragma unroll
+        for (int n = 0; n < 5; ++n) {
+            const uint32_t te = e * 3u, to = o * 3u;  // per 16-bit half: at most 765
+            out[n] = ((te >> 8) & 0x00FF00FFu) | (to & 0xFF00FF00u);
+            e = te & 0x00FF00FFu;
+            o = to & 0x00FF00FFu;
+        }
+    }
+    __device__ static uint32_t pick(const uint32_t (&dg)[5], int n) {
+        return n == 0 ? dg[0] : (n == 1 ? dg[1] : (n == 2 ? dg[2] : (n == 3 ? dg[3] : dg[4])));
+    }
+    __device__ static v4i operand(const Raw& r, int p, int e, int h) {
+        const int sb = 2 * p + e;
+        const v4i src = sb < 5 ? r.qa : r.qb;
+        const int n = sb < 5 ? sb : (sb == 7 ? 4 : 2 * (sb - 5) + h);
+        uint32_t dg[5];
+        v4i out;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            digits5((uint32_t)src[k], dg);
+            out[k] = (int)pick(dg, n);
+        }
+        if (sb == 7 && h == 1) {  // the last 16 elements: digit k of the four qh bytes
+            digits5(r.qh, dg);
+            out = v4i{(int)dg[0], (int)dg[1], (int)dg[2], (int)dg[3]};
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k)  // digit - 1 per byte
+            out[k] = (int)(((uint32_t)out[k] + 0x7F7F7F7Fu) ^ 0x80808080u);
         return out;
     }
 };
@@ -203,6 +260,11 @@ void launch_mmq_shared_q3k(const uint8_t* w, size_t bpr, const ActQ8& act, float
 void launch_mmq_shared_tq2_0(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
                              size_t out_f, const IntStages& st, hipStream_t stream) {
     launch_chain<TileTQ2_0>(w, bpr, act, y, m, in_f, out_f, st, stream);
+}
+
+void launch_mmq_shared_tq1_0(const uint8_t* w, size_t bpr, const ActQ8& act, float* y, size_t m, size_t in_f,
+                             size_t out_f, const IntStages& st, hipStream_t stream) {
+    launch_chain<TileTQ1_0>(w, bpr, act, y, m, in_f, out_f, st, stream);
 }
 
 }  // namespace infr

@@ -189,7 +189,7 @@ def test_moe_banks(be, dtype, rows):
     check(*got, *want)
 
 
-TILED = [DType.Q2K, DType.Q3K, DType.IQ4XS, DType.TQ2_0]
+TILED = [DType.Q2K, DType.Q3K, DType.IQ4XS, DType.TQ2_0, DType.TQ1_0]
 
 
 @pytest.mark.parametrize("dtype", TILED, ids=ids)
@@ -199,7 +199,8 @@ def test_prefill_tiles_are_bit_identical_to_the_oracle(be, dtype, m, in_f, out_f
     """Beyond the 16-token kernel's reach these formats take 128-token x 32-row tiles on the int8
     matrix cores: IQ4_XS a product per 32-weight sub-block scaled by ls - 32 in integers; Q2_K, Q3_K
     and TQ2_0 scaled codes (code x scale fits a byte), so a block is one chain of eight MFMAs, Q2_K's
-    mins an f16 MFMA against per-16 sums formed in the kernel. Same per-block integers and f32
+    mins an f16 MFMA against per-16 sums formed in the kernel; TQ1_0 the same chain over its base-3
+    digits minus one. Same per-block integers and f32
     expression as the one-token kernels, blocks in ascending order - every output bit-identical;
     ragged token and row counts and an odd number of blocks per row included."""
     w = orc.synth_weight(dtype, in_f * out_f, 0x4A + m)
