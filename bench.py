@@ -770,7 +770,8 @@ def main():
         # in a Q4_K_M file)
         for name, dt in (("Q6_K", DType.Q6K), ("Q5_K", DType.Q5K), ("Q8_0", DType.Q8_0), ("Q4_0", DType.Q4_0),
                          ("Q2_0", DType.Q2_0), ("IQ4_XS", DType.IQ4XS), ("Q2_K", DType.Q2K),
-                         ("Q3_K", DType.Q3K), ("TQ2_0", DType.TQ2_0), ("TQ1_0", DType.TQ1_0), ("MXFP4", DType.MXFP4)):
+                         ("Q3_K", DType.Q3K), ("TQ2_0", DType.TQ2_0), ("TQ1_0", DType.TQ1_0), ("MXFP4", DType.MXFP4),
+                         ("NVFP4", DType.NVFP4)):
             for M in (64, 512, 2048):
                 t, nb = single_shape(be, dt, M, 12288, 4096, reps=10, distinct_x=True)
                 extra[f"mmq_{name}_M{M}_TOPS"] = round(2.0 * M * 12288 * 4096 / (t * 1e-3) / 1e12, 2)

@@ -1810,13 +1810,16 @@ bool launch_mmq(int dtype, const uint8_t* w, size_t bpr, const float* x, const A
     // MXFP4 has no 16-token kernel: its dot4 batches cost 2.1 / 2.2 / 1.3 us per token (12288 x 4096, 4096 x 12288,
     // 4096 x 4096) against the tiles' flat 61 / 149 / 51 us
     const size_t mxfp4_tile_tokens = in_f >= 8192 ? 65 : (out_f * in_f >= ((size_t)32 << 20) ? 33 : 41);
+    // NVFP4 likewise: 4.5 / 4.5 / 2.3 us per token against a flat 69 / 165 / 55 us
+    const size_t nvfp4_tile_tokens = in_f >= 8192 ? 41 : (out_f * in_f >= ((size_t)32 << 20) ? 9 : 25);
     // (their kernel's flat time up to 128 tokens, ~145 us at 4096 x 12288, meets the dot4 batches'
     // ~2.1 us per token at 64 tokens)
     // (rows that are not whole 256s included: the kernel pads the last step; Q8_0 rows of that kind
     // multiply the per-32 activation like these formats, crates/infr-cpu/src/lib.rs:1037-1042)
     if ((dtype == 2 || dtype == 3 || dtype == 6 || dtype == 7 || dtype == 20 || (dtype == 8 && in_f % 256 != 0) ||
-         (dtype == 39 && m >= mxfp4_tile_tokens)) &&
-        in_f % 32 == 0 && (m >= 65 || long_row || dtype == 39)) {
+         (dtype == 39 && m >= mxfp4_tile_tokens) ||
+         (dtype == 40 && st.a == nullptr && in_f % 64 == 0 && m >= nvfp4_tile_tokens)) &&
+        in_f % 32 == 0 && (m >= 65 || long_row || dtype == 39 || dtype == 40)) {
         quantize_32_tiled(false);
         return launch_mmq_shared_nib32(dtype, w, bpr, act, y, m, in_f, out_f, st, stream);
     }

@@ -1,5 +1,5 @@
-// Prefill GEMM (65 tokens and up) of the 32-weight-block formats Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL and MXFP4
-// on the int8 matrix cores, and of Q8_0 rows that are not whole 256s (which infr-cpu multiplies against
+// Prefill GEMM (65 tokens and up) of the 32-weight-block formats Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, MXFP4 and
+// NVFP4 on the int8 matrix cores, and of Q8_0 rows that are not whole 256s (which infr-cpu multiplies against
 // the per-32 activation as well: `q8_0_blk32`, crates/infr-cpu/src/lib.rs:1037-1042, d*d8 * iprod per
 // block, kernels.rs:1170-1187). A row may end inside a 256-element step: the quantizer pads the
 // activation with zero codes, scales and sums up to the step, and the blocks past the row's end
@@ -12,6 +12,7 @@
 //     Q4_1   d8 * (d*iprod + m*bsum)        Q5_1   d8 * (d*iprod + m*bsum)
 //     IQ4_NL d*d8 * iprod                   (iprod over the signed codebook values)
 //     MXFP4  d*d8 * iprod                   (d the E8M0 scale halved, iprod over doubled E2M1 values)
+//     NVFP4  d_s*d8 * iprod_s               (per 16 weights: a UE4M3 scale, halved, and a K = 16 MFMA each)
 // The codes (0..15, 0..31, or the codebook's int8) are int8 operands, so iprod is one
 // v_mfma_i32_32x32x32_i8 per block, exact. Every format's term is d8 * (A * iprod + B * bsum) with
 // two per-block constants (A = d; B = -8d, -16d, m or 0), evaluated with one conversion, one
@@ -39,7 +40,7 @@ struct Nib32Lds {
 };
 
 // The formats of this kernel: the five nibble formats and Q8_0 against per-32 activations.
-enum class Blk32 { Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, Q8_0, MXFP4 };
+enum class Blk32 { Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, Q8_0, MXFP4, NVFP4 };
 
 // nb: 256-element steps (the last one may be partly past the row); nblk: 32-weight blocks of a row
 template <Blk32 K, bool STAGES>
@@ -53,6 +54,12 @@ __global__ __launch_bounds__(256) void mmq_shared_nib32_kernel(
     // MXFP4: [E8M0 scale][16 code bytes], 17 bytes at any byte alignment; the codes index a signed
     // table of doubled E2M1 values and the scale decodes halved (crates/infr-cpu/src/lib.rs:1394-1432)
     constexpr bool kMx = K == Blk32::MXFP4;
+    // NVFP4: 36-byte blocks of 64 weights [UE4M3 d[4]][qs[32]]; a 32-element "block" of this kernel is half
+    // of one - sub-blocks 2 hf, 2 hf + 1 of 16 weights (qs[8 s .. 8 s + 7]: low nibbles elements 0..7, high
+    // nibbles 8..15), each with its own scale against the half's one activation scale
+    // (crates/infr-cpu/src/kernels.rs:6472-6500). A sub-block is one K = 16 MFMA; the A constant is the
+    // first sub-block's scale and the B constant, which the format does not need, the second's.
+    constexpr bool kNv = K == Blk32::NVFP4;
     constexpr int kBlockBytes = kMx ? 17 : (kBytes ? 34 : 18 + (kAffine ? 2 : 0) + (kFive ? 4 : 0));
     constexpr int kQhOff = kAffine ? 4 : 2, kQsOff = kBytes ? 2 : kBlockBytes - 16;
     __shared__ __attribute__((aligned(16))) uint8_t lds[2 * Nib32Lds::bytes];
@@ -78,6 +85,15 @@ __global__ __launch_bounds__(256) void mmq_shared_nib32_kernel(
         for (int e = 0; e < 2; ++e) {
             const int bi = b * 8 + 2 * p + e;
             const bool in_row = bi < nblk;  // wave-uniform; past the row's end: block 0 again, scale 0
+            if (kNv) {
+                const uint8_t* nv = wrowp + (size_t)((in_row ? bi : 0) >> 1) * 36;  // 4-byte aligned
+                const int hf = (in_row ? bi : 0) & 1;
+                r.q[e] = load16_a4(nv + 4 + 16 * hf);
+                // the half's two scale bytes; past the row's end both 0 (which decodes to 0)
+                r.d[e] = in_row ? ((uint32_t)load_u32(nv) >> (16 * hf)) & 0xFFFFu : 0u;
+                r.mw[e] = r.qh[e] = 0u;
+                continue;
+            }
             const uint8_t* blk = wrowp + (size_t)(in_row ? bi : 0) * kBlockBytes;  // 2-byte aligned
             r.q[e] = kMx ? gload<v4i_a1>(blk + kQsOff) : load16_a2(blk + kQsOff + (kBytes ? 16 * h : 0));
             r.d[e] = in_row ? (kMx ? (uint32_t)gload<uint8_t>(blk) : load_u16(blk)) : (kMx ? 0x100u : 0u);
@@ -94,16 +110,18 @@ __global__ __launch_bounds__(256) void mmq_shared_nib32_kernel(
                 uint32_t c = (uint32_t)r.q[e][k];
                 if (!kBytes) c = (c >> (4 * h)) & 0x0F0F0F0Fu;
                 if (K == Blk32::IQ4_NL) c = (uint32_t)iq4nl_lookup(c);
-                if (kMx) c = (uint32_t)mxfp4_lookup(c);
+                if (kMx || kNv) c = (uint32_t)mxfp4_lookup(c);  // (NVFP4: dwords 0, 1 sub-block 0's K slots 8h .., 2, 3 sub-block 1's)
                 if (kFive) c |= spread4_to_bit4(r.qh[e] >> (16 * h + 4 * k));
                 out[k] = (int)c;
             }
             *reinterpret_cast<v4i*>(buf + (size_t)(2 * p + e) * 1024 + lane * 16) = out;
             if (h == 0) {
                 // (MXFP4: a block past the row's end carries the marker 0x100 instead of a scale byte)
-                const float d = kMx ? (r.d[e] < 0x100u ? e8m0_half(r.d[e]) : 0.0f) : f16_bits_to_f32(r.d[e]);
-                const float bb = kAffine ? f16_bits_to_f32(r.mw[e])
-                                         : (K == Blk32::IQ4_NL || kBytes || kMx ? 0.0f : (kFive ? -16.0f : -8.0f) * d);
+                const float d = kNv ? ue4m3_half(r.d[e] & 0xFFu)
+                                    : (kMx ? (r.d[e] < 0x100u ? e8m0_half(r.d[e]) : 0.0f) : f16_bits_to_f32(r.d[e]));
+                const float bb = kNv ? ue4m3_half(r.d[e] >> 8)
+                                     : (kAffine ? f16_bits_to_f32(r.mw[e])
+                                                : (K == Blk32::IQ4_NL || kBytes || kMx ? 0.0f : (kFive ? -16.0f : -8.0f) * d));
                 reinterpret_cast<float*>(buf + Nib32Lds::a_off)[col * 8 + 2 * p + e] = d;
                 reinterpret_cast<float*>(buf + Nib32Lds::b_off)[col * 8 + 2 * p + e] = bb;
             }
@@ -157,6 +175,29 @@ __global__ __launch_bounds__(256) void mmq_shared_nib32_kernel(
 #pragma unroll
         for (int sb = 0; sb < 8; ++sb) {
             const v4i bf = *reinterpret_cast<const v4i*>(cur + (size_t)sb * 1024 + lane * 16);
+            if constexpr (kNv) {
+                // lane (token, h) holds sub-block h of the 32 whole; the K = 16 operand wants bytes 8h .. 8h + 7
+                // of one sub-block: the swap exchanges lanes 32..63 of its first operand with lanes 0..31 of
+                // its second, after which x y are the lane's K slots of sub-block 0 and z w of sub-block 1
+                typedef int v2i_ __attribute__((ext_vector_type(2)));
+                const auto s0 = __builtin_amdgcn_permlane32_swap(a[sb].x, a[sb].z, false, false);
+                const auto s1 = __builtin_amdgcn_permlane32_swap(a[sb].y, a[sb].w, false, false);
+                const v2i_ a0 = {(int)s0[0], (int)s1[0]}, a1 = {(int)s0[1], (int)s1[1]}, b0 = {bf.x, bf.y}, b1 = {bf.z, bf.w};
+                const v16i r0 = __builtin_amdgcn_mfma_i32_32x32x16_i8(__builtin_bit_cast(long, a0), __builtin_bit_cast(long, b0), zi, 0, 0, 0);
+                const v16i r1 = __builtin_amdgcn_mfma_i32_32x32x16_i8(__builtin_bit_cast(long, a1), __builtin_bit_cast(long, b1), zi, 0, 0, 0);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const v4f dq = *reinterpret_cast<const v4f*>(&dql[wave][sb][8 * j + 4 * h]);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int ri = 4 * j + i;
+                        // d8 * (d_0 * iprod_0 + d_1 * iprod_1)
+                        const float t = __builtin_fmaf(cb[sb], (float)r1[ri], ca[sb] * (float)r0[ri]);
+                        acc[ri] = __builtin_fmaf(dq[i], t, acc[ri]);
+                    }
+                }
+                continue;
+            }
             const v16i r = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[sb], bf, zi, 0, 0, 0);
             // accumulator i of this lane is token 8*(i/4) + 4*h + i%4 of the wave's 32
 #pragma unroll
@@ -338,6 +379,10 @@ bool launch_mmq_shared_nib32(int dtype, const uint8_t* w, size_t bpr, const ActQ
     case 7: launch_nib32<Blk32::Q5_1>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
     case 20: launch_nib32<Blk32::IQ4_NL>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
     case 39: launch_nib32<Blk32::MXFP4>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
+    case 40:
+        if (st.a || in_f % 64 != 0) return false;  // (no integer-stage form: four integers per block)
+        launch_nib32<Blk32::NVFP4>(w, bpr, act, y, m, in_f, out_f, st, stream);
+        return true;
     case 8: launch_nib32<Blk32::Q8_0>(w, bpr, act, y, m, in_f, out_f, st, stream); return true;
     case 42: {
         const dim3 grid((unsigned)((out_f + 31) / 32), (unsigned)((m + 127) / 128)), block(256);

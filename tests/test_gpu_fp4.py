@@ -188,3 +188,20 @@ def test_mxfp4_prefill_tiles(be, m, in_f, out_f):
         a, _ = be.linear_int_stages(DType.MXFP4, be.upload_new(w), be.upload_new(x), m, in_f, out_f)
         oa, _ = orc.linear_int_stages(DType.MXFP4, w, x, m, in_f, out_f)
         assert np.array_equal(a, oa)
+
+
+@pytest.mark.parametrize("m,in_f,out_f", [(25, 1024, 96), (9, 4096, 8200), (130, 2048, 70), (300, 320, 33), (200, 1280, 50),
+                                          (70, 8192, 40), (512, 4096, 64)])
+def test_nvfp4_prefill_tiles(be, m, in_f, out_f):
+    """From 9..41 tokens (by shape) NVFP4 takes the same tiles with a K = 16 MFMA per 16-weight
+    sub-block (lane swaps put the activation halves in operand order), each scaled by its halved
+    UE4M3 scale and the per-32 activation scale: y within the path's 1e-4 of the oracle; rows that
+    are not whole 256s included."""
+    w = orc.synth_weight(DType.NVFP4, in_f * out_f, 0x5B + m)
+    x = synth_normal_f32(50 + m, m * in_f)
+    x[in_f:2 * in_f] = 0.0
+    y = run_linear(be, DType.NVFP4, w, x, m, in_f, out_f)
+    toks = np.unique(np.r_[0, 1, m // 2, m - 1, min(31, m - 1), min(32, m - 1)])
+    want = orc.linear(DType.NVFP4, w, x.reshape(m, in_f)[toks].ravel(), len(toks), in_f, out_f)
+    gate(y[toks], want)
+    assert np.all(y[1] == 0.0)
