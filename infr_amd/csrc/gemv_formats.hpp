@@ -802,7 +802,10 @@ struct FmtTQ2_0 {
     static constexpr int kWide16Steps = 3;
     static constexpr bool kClampedLoads = false;
     static constexpr bool kLaneSums = true;
-    static constexpr bool kRowAhead = false;
+    // rows of two and three wave steps run a whole row ahead (4096 x 12288: 4.4 -> 4.8 TB/s, 1024 x 12288:
+    // 4.2 -> 4.6; 8192 columns the same); four steps lose a fifth that way (two sets of four rows' registers)
+    static constexpr bool kRowAhead = true;
+    static constexpr int kRowAheadMaxSteps = 3;
     struct Row {
         v4i q;
         uint32_t d;

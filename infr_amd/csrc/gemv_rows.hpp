@@ -65,6 +65,13 @@ struct ClampedOneAhead : std::integral_constant<bool, F::kClampedLoads> {};
 template <typename F>
 struct ClampedOneAhead<F, std::void_t<decltype(F::kClampedOneAhead)>> : std::integral_constant<bool, F::kClampedOneAhead> {};
 
+// The longest rows (in wave steps) that the loop running a whole row ahead takes: a format says
+// kRowAheadMaxSteps when two register sets of longer rows cost it more than the lead buys.
+template <typename F, typename = void>
+struct RowAheadMaxSteps : std::integral_constant<int, 8> {};
+template <typename F>
+struct RowAheadMaxSteps<F, std::void_t<decltype(F::kRowAheadMaxSteps)>> : std::integral_constant<int, F::kRowAheadMaxSteps> {};
+
 // Rows [row0, row_end) of one weight matrix against activation registers `acts`. `first` already
 // holds step 0 of row0 - every step of it when FIRST_WHOLE - (the caller issues those loads as
 // early as it can). The loads run one wave
@@ -196,7 +203,7 @@ __device__ __forceinline__ void gemv_rows(const uint8_t* __restrict__ w, size_t 
             }
         }
     };
-    if constexpr (STEPS > 1 && F::kRowAhead) {
+    if constexpr (STEPS > 1 && F::kRowAhead && STEPS <= RowAheadMaxSteps<F>::value) {
         // Long rows run in eight-wave workgroups, where one step ahead is too few bytes in flight:
         // the loads run a whole row ahead - step t of the next row is requested before step t of
         // this one is computed.
