@@ -174,7 +174,8 @@ struct FmtQ6K {
     static constexpr int kWide16Steps = 1;
     static constexpr bool kClampedLoads = false;
     static constexpr bool kLaneSums = true;
-    static constexpr bool kRowAhead = false;
+    static constexpr bool kRowAhead = true;  // rows of two and three wave steps run a whole row ahead: 4096 x 12288 5.28 -> 5.57 TB/s,
+    static constexpr int kRowAheadMaxSteps = 3;  // 1024 x 12288 5.20 -> 5.48, 8192 columns +2.5 %; four steps lose 1.6 %
     struct Row {
         v4i qla, qlb, qh;
         v2i sc;
