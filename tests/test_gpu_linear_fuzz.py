@@ -41,11 +41,14 @@ def draw_case(rng):
     if dtype == DType.Q4K and m >= 128 and rng.integers(2):
         out_f = int(rng.choice([2304, 2600, 5100, 6144]))        # enough outputs for the prefill strips
         in_f = 256 * int(rng.integers(1, 5))
+    if dtype in (DType.Q2K, DType.Q3K, DType.IQ4XS, DType.TQ2_0, DType.Q5K, DType.Q6K) and m >= 96 and rng.integers(2):
+        out_f = int(rng.choice([2304, 2600, 5100]))              # enough outputs for the 128-token tiles
+        in_f = 256 * int(rng.integers(1, 5))
     extra_before, extra_after = (int(rng.integers(0, 40)) if rng.integers(2) else 0 for _ in range(2))
     return dtype, m, in_f, out_f, extra_before, extra_after
 
 
-@pytest.mark.parametrize("seed", range(240))
+@pytest.mark.parametrize("seed", range(320))
 def test_linear_on_a_random_shape_matches_the_oracle(be, seed):
     rng = np.random.default_rng(0xF00D + seed)
     dtype, m, in_f, out_f, before, after = draw_case(rng)
