@@ -1256,6 +1256,63 @@ struct Skinny16Nib32 {
     }
 };
 
+// NVFP4 (36-byte blocks of 64 weights [UE4M3 d[4]][qs[32]], four to a 256-element step: 144 bytes, like
+// Q4_K's; crates/infr-cpu/src/kernels.rs:6472-6500): sub-block sb of a block (16 weights: the low
+// nibbles of qs[8 sb .. 8 sb + 7] elements 0..7, the high nibbles 8..15) has its own halved UE4M3
+// scale and meets half of a per-32 activation block, term d_sb * q8.d * iprod_sb. The K = 32 step of
+// a 32-element activation block therefore runs twice, once with the operand bytes of the second
+// sub-block zeroed and once with the first's: lanes kq = 0, 1 hold the first sub-block's K slots,
+// kq = 2, 3 the second's. The two terms of a 32 are added before they join the chain.
+struct Skinny16NVFP4 {
+    typedef int v2i __attribute__((ext_vector_type(2)));
+    static constexpr bool kSubScales = true, kPer32Acts = true, kTranspose16 = false;
+    static constexpr int kBlockBytes = 144;
+    static constexpr int kRowStride = 2 * kBlockBytes + 16;  // 76 words: eight rows' 16-byte reads cover all banks
+    template <int MT, int DQ_STRIDE>
+    __device__ static void block(const uint8_t* wrow, int jj, const uint8_t* arow, const uint8_t*,
+                                 const float* dq_base, int kq, int (&ip)[32], int (&raw)[32]) {
+        const uint8_t* blk = wrow + jj * kBlockBytes;
+        v4f dq[4][2];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int tok = (4 * kq + i) & (MT - 1);
+            dq[i][0] = *reinterpret_cast<const v4f*>(dq_base + tok * DQ_STRIDE + jj * 8);
+            dq[i][1] = *reinterpret_cast<const v4f*>(dq_base + tok * DQ_STRIDE + jj * 8 + 4);
+        }
+        const bool second = kq >= 2;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const uint8_t* nv = blk + 36 * (s >> 1);
+            const int sb0 = 2 * (s & 1);  // the 32's sub-blocks sb0, sb0 + 1; this lane's own: sb0 + (kq >> 1)
+            const uint8_t* qp = nv + 4 + 8 * (sb0 + (kq >> 1));
+            const int sh = 4 * (kq & 1);
+            const uint32_t c0 = (uint32_t)mxfp4_lookup((*reinterpret_cast<const uint32_t*>(qp) >> sh) & 0x0F0F0F0Fu);
+            const uint32_t c1 = (uint32_t)mxfp4_lookup((*reinterpret_cast<const uint32_t*>(qp + 4) >> sh) & 0x0F0F0F0Fu);
+            const v2i b0 = {second ? 0 : (int)c0, second ? 0 : (int)c1}, b1 = {second ? (int)c0 : 0, second ? (int)c1 : 0};
+            const v2i a = *reinterpret_cast<const v2i*>(arow + s * 32 + 8 * kq);
+            const v4i r0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(__builtin_bit_cast(long, a), __builtin_bit_cast(long, b0),
+                                                                 v4i{0, 0, 0, 0}, 0, 0, 0);
+            const v4i r1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(__builtin_bit_cast(long, a), __builtin_bit_cast(long, b1),
+                                                                 v4i{0, 0, 0, 0}, 0, 0, 0);
+            const uint32_t dw = *reinterpret_cast<const uint32_t*>(nv);
+            const float w0 = ue4m3_half((dw >> (8 * sb0)) & 0xFFu), w1 = ue4m3_half((dw >> (8 * sb0 + 8)) & 0xFFu);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                raw[4 * s + i] = r0[i];
+                const float d8 = dq[i][s >> 2][s & 3];
+                const float term = (w0 * d8) * (float)r0[i] + (w1 * d8) * (float)r1[i];
+                ip[4 * s + i] = __builtin_bit_cast(int, term);
+            }
+        }
+    }
+    __device__ static void accumulate(float (&acc)[4], const float (&)[4], const uint32_t (&)[4], const int (&ip)[32]) {
+#pragma unroll
+        for (int s = 0; s < 8; ++s)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] += __builtin_bit_cast(float, ip[4 * s + i]);
+    }
+};
+
 template <typename F, int NW, int BPW, int MT, bool STAGES>
 __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
     const uint8_t* __restrict__ w, size_t bpr, const int8_t* __restrict__ qs,
@@ -1504,7 +1561,7 @@ __global__ __launch_bounds__(NW * 64) void mmq_skinny16_kernel(
 constexpr int kSkinny16Waves = 4, kSkinny16Blocks = 2;
 static bool skinny16_shape(int dtype, int nb, size_t m, size_t out_f) {
     const bool nib32 = dtype == 2 || dtype == 3 || dtype == 6 || dtype == 7 || dtype == 20;
-    if (dtype != 12 && dtype != 13 && dtype != 14 && dtype != 8 && dtype != 42 && dtype != 10 && dtype != 11 && dtype != 23 && dtype != 35 && !nib32)
+    if (dtype != 12 && dtype != 13 && dtype != 14 && dtype != 8 && dtype != 42 && dtype != 10 && dtype != 11 && dtype != 23 && dtype != 35 && dtype != 40 && !nib32)
         return false;
     if (nb < kSkinny16Blocks || (nb % kSkinny16Blocks != 0 && (dtype == 14 || dtype == 42 || dtype == 11 || dtype == 35))) return false;
     // Q2_K, Q3_K, IQ4_XS, TQ2_0 up to 16 tokens: the dot4 batches are the only other kernel there, eight tokens per
@@ -1520,6 +1577,11 @@ static bool skinny16_shape(int dtype, int nb, size_t m, size_t out_f) {
     // 29.5 us on the tiles, 5.7 / 10.2 / 19.0 here; Q6_K 7.9 / 41.4 / 43.1 and 7.8 / 9.5 / 17.6), 768 K for
     // the 32-weight-block formats (Q4_0 at 256 / 512 tokens: 62 / 65 us on the tiles), 600 K for Q2_0 (44 / 47). Independent of the row length: both scale with it.
     if (m > (size_t)16 * 65535) return false;  // (the grid's third dimension walks the batch 16 tokens at a time)
+    // NVFP4: from nine tokens (the dot4 batches take eight a pass) up to where its tiles take over - a 16-token
+    // pass costs 34 / 31 / 12 us (12288 x 4096, 4096 x 12288, 4096 x 4096: two half-empty MFMAs per 32 weights),
+    // the tiles a flat 69 / 166 / 55
+    if (dtype == 40)
+        return m >= 9 && (out_f == 0 || m <= ((out_f * (size_t)nb <= (size_t)4096 * 16 || nb >= 32) ? 80u : 32u));
     if (m > 16 && out_f == 0 && dtype != 12) return true;  // (a plan's group: its ops were taken one by one)
     if (m > 16) {
         const size_t outputs = m * out_f;
@@ -1654,6 +1716,8 @@ static bool launch_mmq_skinny16(int dtype, const uint8_t* w, size_t bpr, const A
         launch_mmq_skinny16_fmt<Skinny16Nib32<Nib32::Q5_1>, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     else if (dtype == 20)
         launch_mmq_skinny16_fmt<Skinny16Nib32<Nib32::IQ4_NL>, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
+    else if (dtype == 40)
+        launch_mmq_skinny16_fmt<Skinny16NVFP4, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     else if (dtype == 10)
         launch_mmq_skinny16_fmt<Skinny16Q2K, STAGES>(w, bpr, act, y, m, nb, out_f, wgs, st, tiles, stream);
     else if (dtype == 11)
